@@ -1,0 +1,195 @@
+/*
+ * flhip.h — C ABI of the MI355X (gfx950) kernels behind Flashlight's
+ * AutogradExtension operator interface.
+ *
+ * The reference has no C ABI for this path: its extension point is the C++
+ * abstract class fl::AutogradExtension
+ * (flashlight/fl/autograd/tensor/AutogradExtension.h:46-180).  Each entry point
+ * below is what one virtual of that class lowers to once tensors have been
+ * reduced to raw device pointers, and names the virtual it serves.
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer into memory owned by the caller.
+ *   - Layout: Flashlight column-major [W,H,C,N] == row-major N,C,H,W; weights
+ *     [kx,ky,Cin/groups,Cout] == row-major Cout,Cin/groups,KH,KW
+ *     (flashlight/fl/autograd/tensor/backend/onednn/Conv2D.cpp:69-93,171-178).
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Work
+ *     is enqueued; no entry point synchronises the device.
+ *   - Return value: FLHIP_OK, FLHIP_INVALID_ARGUMENT (host maps it to
+ *     std::invalid_argument) or FLHIP_RUNTIME_ERROR (std::runtime_error), the two
+ *     exception kinds of the reference boundary
+ *     (flashlight/fl/autograd/tensor/backend/cudnn/CudnnUtils.cpp:88-99).
+ *     flhip_last_error() returns the message of the calling thread's last failure.
+ *   - The library allocates nothing: scratch comes in through `ws`/`ws_bytes`
+ *     (size from the matching *_workspace_bytes query).
+ */
+#ifndef FLHIP_H
+#define FLHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  FLHIP_OK = 0,
+  FLHIP_INVALID_ARGUMENT = 1,
+  FLHIP_RUNTIME_ERROR = 2
+};
+
+/* Storage type of activations.  Reductions and accumulators are always fp32.
+ * Flashlight has no bf16 dtype (flashlight/fl/tensor/Types.h:17-30); FLHIP_BF16
+ * is this library's private tag for bf16 storage with fp32 accumulate. */
+enum {
+  FLHIP_F32 = 0,
+  FLHIP_BF16 = 1
+};
+
+/* fl::PoolingMode, same numeric values (flashlight/fl/common/Defines.h:53-64). */
+enum {
+  FLHIP_POOL_MAX = 0,
+  FLHIP_POOL_AVG_INCLUDE_PADDING = 1,
+  FLHIP_POOL_AVG_EXCLUDE_PADDING = 2
+};
+
+/* Which convolution pass a workspace query is for. */
+enum {
+  FLHIP_CONV_FWD = 0,
+  FLHIP_CONV_BWD_DATA = 1,
+  FLHIP_CONV_BWD_FILTER = 2
+};
+
+/* Convolution geometry.  x is [N,C,H,W], w is [K,C/groups,KH,KW], y is
+ * [N,K,OH,OW] with OH = 1 + (H + 2*py - (1 + (KH-1)*dil_y)) / sy (integer
+ * division), likewise OW (onednn/Conv2D.cpp:179-188).  Dilation uses
+ * Flashlight's convention (1 = dense).  dtype = FLHIP_F32: every buffer fp32.
+ * dtype = FLHIP_BF16: x, w, y, dy, dx are bf16; bias, dw, db stay fp32. */
+typedef struct flhip_conv_desc {
+  int32_t N, C, H, W;
+  int32_t K, KH, KW;
+  int32_t sy, sx;
+  int32_t py, px;
+  int32_t dil_y, dil_x;
+  int32_t groups;
+  int32_t dtype;
+} flhip_conv_desc;
+
+/* Pooling geometry.  x is [N,C,H,W]; y is [N,C,OH,OW], OH = 1 + (H + 2*py - wy)/sy
+ * (onednn/Pool2D.cpp:100-102).  Padding is symmetric and must be smaller than the
+ * window.  dtype tags x, y, dy and dx. */
+typedef struct flhip_pool_desc {
+  int32_t N, C, H, W;
+  int32_t wy, wx;
+  int32_t sy, sx;
+  int32_t py, px;
+  int32_t mode;
+  int32_t dtype;
+} flhip_pool_desc;
+
+/* Batch-norm view, as the oneDNN extension derives it from the feature axes
+ * (onednn/BatchNorm.cpp:40-71): element (o, c, i) lives at (o*C + c)*inner + i.
+ * Spatial mode (axes do not include dim 0): outer = product of dims after the
+ * last feature axis, inner = product of dims before the first.  Per-activation
+ * mode (axes start at dim 0): inner = 1, outer = elements / C.
+ * dtype tags x, y, dy, dx; gamma, beta, statistics and their gradients are fp32. */
+typedef struct flhip_bn_desc {
+  int64_t outer;
+  int64_t C;
+  int64_t inner;
+  int32_t dtype;
+} flhip_bn_desc;
+
+const char* flhip_last_error(void);
+
+/* Library version, and the gfx architecture the kernels were compiled for. */
+int flhip_version(void);
+const char* flhip_arch(void);
+
+/* Output extents of the geometries above; return FLHIP_INVALID_ARGUMENT when the
+ * geometry is not valid (non-positive sizes, window larger than padded input…). */
+int flhip_conv2d_out_dims(const flhip_conv_desc* d, int32_t* OH, int32_t* OW);
+int flhip_pool2d_out_dims(const flhip_pool_desc* d, int32_t* OH, int32_t* OW);
+
+/* Scratch a convolution pass needs (0 is possible). */
+size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pass);
+
+/* AutogradExtension::conv2d (AutogradExtension.h:58-69; oneDNN peer
+ * onednn/Conv2D.cpp:155-270): y = cross-correlation(x, w) + bias.  bias may be
+ * NULL (the reference's "bias.elements() == 0"). */
+int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const void* w,
+                     const float* bias, void* y, void* ws, size_t ws_bytes,
+                     void* stream);
+
+/* AutogradExtension::conv2dBackwardData (AutogradExtension.h:110-122; oneDNN
+ * peer onednn/Conv2D.cpp:272-375): dx = d(loss)/d(x) from dy and w. */
+int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy,
+                          const void* w, void* dx, void* ws, size_t ws_bytes,
+                          void* stream);
+
+/* AutogradExtension::conv2dBackwardFilterBias (AutogradExtension.h:124-138;
+ * oneDNN peer onednn/Conv2D.cpp:377-507): dw (fp32, weight shape) and, when db
+ * is not NULL, db[k] = sum of dy over n, oh, ow (fp32).  dw may be NULL to get
+ * the bias gradient alone. */
+int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x,
+                            const void* dy, float* dw, float* db, void* ws,
+                            size_t ws_bytes, void* stream);
+
+/* AutogradExtension::pool2d (AutogradExtension.h:71-80; oneDNN peer
+ * onednn/Pool2D.cpp:78-176).  For FLHIP_POOL_MAX with argmax != NULL the kernel
+ * also writes one byte per output: the window-relative index kh*wx + kw of the
+ * first maximum in (kh outer, kw inner) scan order under strict '>', padded
+ * positions skipped — the workspace the reference keeps in its payload
+ * (onednn/Pool2D.cpp:150-161).  Needs wy*wx <= 256 when argmax is requested. */
+int flhip_pool2d_fwd(const flhip_pool_desc* d, const void* x, void* y,
+                     uint8_t* argmax, void* stream);
+
+/* AutogradExtension::pool2dBackward (AutogradExtension.h:141-152; oneDNN peer
+ * onednn/Pool2D.cpp:178-247).  MAX needs the argmax bytes of the forward call;
+ * the average modes ignore it.  Every element of dx is written (no pre-zeroing). */
+int flhip_pool2d_bwd(const flhip_pool_desc* d, const void* dy,
+                     const uint8_t* argmax, void* dx, void* stream);
+
+/* Scratch for the batch-norm passes below (partial sums). */
+size_t flhip_bn_workspace_bytes(const flhip_bn_desc* d);
+
+/* AutogradExtension::batchnorm with train = true (AutogradExtension.h:82-94;
+ * oneDNN peer onednn/BatchNorm.cpp:88-200; cuDNN peer cudnn/BatchNorm.cpp:145-162).
+ * Batch mean and biased variance per feature; y = gamma*(x-mean)*invstd + beta.
+ * gamma/beta NULL = ones/zeros.  save_mean/save_invstd (fp32[C]) receive the
+ * batch mean and 1/sqrt(var+eps) for the backward pass.  When run_mean/run_var
+ * are not NULL they are updated in place: momentum == 0 stores the batch mean
+ * and biased variance (what the oneDNN extension does, BatchNorm.cpp:154-157);
+ * momentum != 0 blends r = (1-momentum)*r + momentum*batch with the unbiased
+ * batch variance (cuDNN semantics). */
+int flhip_bn_fwd_train(const flhip_bn_desc* d, const void* x,
+                       const float* gamma, const float* beta, void* y,
+                       float* save_mean, float* save_invstd, float* run_mean,
+                       float* run_var, double momentum, double eps, void* ws,
+                       size_t ws_bytes, void* stream);
+
+/* AutogradExtension::batchnorm with train = false (use_global_stats,
+ * onednn/BatchNorm.cpp:171-175): y = gamma*(x-run_mean)/sqrt(run_var+eps)+beta. */
+int flhip_bn_fwd_infer(const flhip_bn_desc* d, const void* x,
+                       const float* gamma, const float* beta,
+                       const float* run_mean, const float* run_var, double eps,
+                       void* y, void* stream);
+
+/* AutogradExtension::batchnormBackward (AutogradExtension.h:155-164; oneDNN peer
+ * onednn/BatchNorm.cpp:202-279): dbeta = sum dy, dgamma = sum dy*xhat,
+ * dx = gamma*invstd*(dy - dbeta/M - xhat*dgamma/M), M = outer*inner. */
+int flhip_bn_bwd(const flhip_bn_desc* d, const void* x, const void* dy,
+                 const float* gamma, const float* save_mean,
+                 const float* save_invstd, void* dx, float* dgamma,
+                 float* dbeta, void* ws, size_t ws_bytes, void* stream);
+
+/* Plain device-to-device copy kernel of `bytes` bytes (multiple of 16).  Not part
+ * of the operator interface: it is the known-size kernel that hardware byte
+ * counters are calibrated against when measuring the kernels above. */
+int flhip_copy_bytes(const void* src, void* dst, size_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLHIP_H */

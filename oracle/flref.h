@@ -1,0 +1,95 @@
+/*
+ * flref — CPU restatement of the arithmetic behind Flashlight's oneDNN
+ * AutogradExtension (conv2d, pool2d, batchnorm and their backward passes).
+ *
+ * TEST INFRASTRUCTURE ONLY.  This is the checker the HIP kernels are compared
+ * with; nothing in the shipped library or its host layer calls it.
+ *
+ * The reference delegates the arithmetic to oneDNN (un-vendored, not pinned:
+ * find_package(DNNL), flashlight/fl/tensor/backend/onednn/CMakeLists.txt:6), so
+ * each function restates the published definition of the primitive the
+ * reference requests, with the shapes, flags and quirks of the reference's own
+ * call site (cited per function).  Layout is the reference's: row-major
+ * N,C,H,W == Flashlight column-major [W,H,C,N].
+ *
+ * How each function is pinned (tests/test_oracle_*.py):
+ *   conv fwd / bwd-data / bwd-filter+bias: brute-force definition in numpy on
+ *     tiny cases, adjoint identities, 1x1-conv == GEMM, batching invariance, the
+ *     shapes of the reference's own Jacobian tests, and PyTorch-CPU's library
+ *     routines (oneDNN v3.7.1 inside) on seeded cases.
+ *   pool fwd / bwd (max, avg include/exclude padding): brute force with ties on
+ *     a 1/8 grid, sum(dx) == sum(dy), library routines.
+ *   batchnorm train / infer / backward: the closed forms of the reference's
+ *     tests (AutogradNormalizationTest.cpp:37-226), invariants sum(dx) == 0 and
+ *     sum(dx*xhat) == 0, finite differences, library routines.
+ * Not pinned by anything the reference holds ("parity unpinned" there, fixed
+ * here by the definition above and checked against oneDNN through PyTorch):
+ * the max-pool tie order and the running-statistics update for momentum != 0.
+ */
+#ifndef FLREF_H
+#define FLREF_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct flref_conv {
+  int32_t N, C, H, W;
+  int32_t K, KH, KW;
+  int32_t sy, sx, py, px, dil_y, dil_x, groups;
+} flref_conv;
+
+typedef struct flref_pool {
+  int32_t N, C, H, W;
+  int32_t wy, wx, sy, sx, py, px;
+  int32_t mode; /* 0 max, 1 avg include padding, 2 avg exclude padding */
+} flref_pool;
+
+int flref_conv_out(const flref_conv* d, int32_t* OH, int32_t* OW);
+int flref_pool_out(const flref_pool* d, int32_t* OH, int32_t* OW);
+
+/* onednn/Conv2D.cpp:155-270 */
+void flref_conv2d_fwd(const flref_conv* d, const float* x, const float* w,
+                      const float* bias, float* y);
+/* onednn/Conv2D.cpp:272-375 */
+void flref_conv2d_bwd_data(const flref_conv* d, const float* dy, const float* w,
+                           float* dx);
+/* onednn/Conv2D.cpp:377-507 */
+void flref_conv2d_bwd_filter(const flref_conv* d, const float* x,
+                             const float* dy, float* dw, float* db);
+
+/* onednn/Pool2D.cpp:78-176.  argmax (may be NULL) gets kh*wx+kw per output. */
+void flref_pool2d_fwd(const flref_pool* d, const float* x, float* y,
+                      uint8_t* argmax);
+/* onednn/Pool2D.cpp:178-247 */
+void flref_pool2d_bwd(const flref_pool* d, const float* dy,
+                      const uint8_t* argmax, float* dx);
+
+/* onednn/BatchNorm.cpp:88-200; element (o,c,i) at (o*C + c)*inner + i. */
+void flref_bn_fwd_train(int64_t outer, int64_t C, int64_t inner, const float* x,
+                        const float* gamma, const float* beta, double eps,
+                        float* y, float* mean, float* var);
+void flref_bn_fwd_infer(int64_t outer, int64_t C, int64_t inner, const float* x,
+                        const float* gamma, const float* beta,
+                        const float* mean, const float* var, double eps,
+                        float* y);
+/* onednn/BatchNorm.cpp:202-279 */
+void flref_bn_bwd(int64_t outer, int64_t C, int64_t inner, const float* x,
+                  const float* dy, const float* gamma, const float* mean,
+                  const float* var, double eps, float* dx, float* dgamma,
+                  float* dbeta);
+
+/* Running-statistics update.  momentum == 0: overwrite with batch mean and
+ * biased variance (onednn/BatchNorm.cpp:154-157 binds the running buffers as the
+ * primitive's mean/variance outputs).  Otherwise r = (1-m)*r + m*batch with the
+ * unbiased variance var*M/(M-1) (cudnnBatchNormalizationForwardTraining, called
+ * at cudnn/BatchNorm.cpp:145-162). */
+void flref_bn_running_update(int64_t C, int64_t M, const float* mean,
+                             const float* var, double momentum, float* run_mean,
+                             float* run_var);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

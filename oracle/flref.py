@@ -1,0 +1,181 @@
+"""ctypes binding of the CPU checker (libflref.so).
+
+Test infrastructure only: imported by tests/, by the smoke check and by the
+CPU-baseline leg of bench.py — never by the flashlight_amd package.
+Arrays are numpy float32, C-contiguous, in the reference's layout (row-major
+N,C,H,W == Flashlight [W,H,C,N]).
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "N", "C", "H", "W", "K", "KH", "KW", "sy", "sx", "py", "px",
+        "dil_y", "dil_x", "groups")]
+
+
+class PoolDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "N", "C", "H", "W", "wy", "wx", "sy", "sx", "py", "px", "mode")]
+
+
+def build(force=False):
+    so = os.path.join(_HERE, "libflref.so")
+    if force or not os.path.exists(so):
+        subprocess.check_call(["make", "-B", "-C", _HERE, "libflref.so"],
+                              stdout=subprocess.DEVNULL)
+    return so
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        _LIB = C.CDLL(build())
+    return _LIB
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _f32(a):
+    return None if a is None else np.ascontiguousarray(a, dtype=np.float32)
+
+
+def conv_desc(x_shape, w_shape, stride=(1, 1), pad=(0, 0), dil=(1, 1), groups=1):
+    """stride/pad/dil are (y, x)."""
+    N, Cc, H, W = x_shape
+    K, Cg, KH, KW = w_shape
+    assert Cg * groups == Cc, (x_shape, w_shape, groups)
+    return ConvDesc(N, Cc, H, W, K, KH, KW, stride[0], stride[1], pad[0], pad[1],
+                    dil[0], dil[1], groups)
+
+
+def conv_out(d):
+    oh, ow = C.c_int32(), C.c_int32()
+    if lib().flref_conv_out(C.byref(d), C.byref(oh), C.byref(ow)):
+        raise ValueError("invalid conv geometry")
+    return oh.value, ow.value
+
+
+def conv2d_fwd(d, x, w, b=None):
+    x, w, b = _f32(x), _f32(w), _f32(b)
+    oh, ow = conv_out(d)
+    y = np.empty((d.N, d.K, oh, ow), np.float32)
+    lib().flref_conv2d_fwd(C.byref(d), _p(x), _p(w), _p(b), _p(y))
+    return y
+
+
+def conv2d_bwd_data(d, dy, w):
+    dy, w = _f32(dy), _f32(w)
+    dx = np.empty((d.N, d.C, d.H, d.W), np.float32)
+    lib().flref_conv2d_bwd_data(C.byref(d), _p(dy), _p(w), _p(dx))
+    return dx
+
+
+def conv2d_bwd_filter(d, x, dy, want_bias=True):
+    x, dy = _f32(x), _f32(dy)
+    dw = np.empty((d.K, d.C // d.groups, d.KH, d.KW), np.float32)
+    db = np.empty((d.K,), np.float32) if want_bias else None
+    lib().flref_conv2d_bwd_filter(C.byref(d), _p(x), _p(dy), _p(dw), _p(db))
+    return dw, db
+
+
+def pool_desc(x_shape, window, stride, pad, mode):
+    """window/stride/pad are (y, x); mode 0 max, 1 avg-include, 2 avg-exclude."""
+    N, Cc, H, W = x_shape
+    return PoolDesc(N, Cc, H, W, window[0], window[1], stride[0], stride[1],
+                    pad[0], pad[1], mode)
+
+
+def pool_out(d):
+    oh, ow = C.c_int32(), C.c_int32()
+    if lib().flref_pool_out(C.byref(d), C.byref(oh), C.byref(ow)):
+        raise ValueError("invalid pool geometry")
+    return oh.value, ow.value
+
+
+def pool2d_fwd(d, x):
+    x = _f32(x)
+    oh, ow = pool_out(d)
+    y = np.empty((d.N, d.C, oh, ow), np.float32)
+    am = np.zeros((d.N, d.C, oh, ow), np.uint8) if d.mode == 0 else None
+    lib().flref_pool2d_fwd(C.byref(d), _p(x), _p(y), _p(am))
+    return y, am
+
+
+def pool2d_bwd(d, dy, argmax=None):
+    dy = _f32(dy)
+    if argmax is not None:
+        argmax = np.ascontiguousarray(argmax, dtype=np.uint8)
+    dx = np.empty((d.N, d.C, d.H, d.W), np.float32)
+    lib().flref_pool2d_bwd(C.byref(d), _p(dy), _p(argmax), _p(dx))
+    return dx
+
+
+def _i64(v):
+    return C.c_int64(int(v))
+
+
+def bn_fwd_train(outer, Cc, inner, x, gamma, beta, eps):
+    x, gamma, beta = _f32(x), _f32(gamma), _f32(beta)
+    y = np.empty_like(x)
+    mean = np.empty((Cc,), np.float32)
+    var = np.empty((Cc,), np.float32)
+    lib().flref_bn_fwd_train(_i64(outer), _i64(Cc), _i64(inner), _p(x), _p(gamma),
+                             _p(beta), C.c_double(eps), _p(y), _p(mean), _p(var))
+    return y, mean, var
+
+
+def bn_fwd_infer(outer, Cc, inner, x, gamma, beta, mean, var, eps):
+    x, gamma, beta, mean, var = map(_f32, (x, gamma, beta, mean, var))
+    y = np.empty_like(x)
+    lib().flref_bn_fwd_infer(_i64(outer), _i64(Cc), _i64(inner), _p(x), _p(gamma),
+                             _p(beta), _p(mean), _p(var), C.c_double(eps), _p(y))
+    return y
+
+
+def bn_bwd(outer, Cc, inner, x, dy, gamma, mean, var, eps):
+    x, dy, gamma, mean, var = map(_f32, (x, dy, gamma, mean, var))
+    dx = np.empty_like(x)
+    dg = np.empty((Cc,), np.float32)
+    db = np.empty((Cc,), np.float32)
+    lib().flref_bn_bwd(_i64(outer), _i64(Cc), _i64(inner), _p(x), _p(dy), _p(gamma),
+                       _p(mean), _p(var), C.c_double(eps), _p(dx), _p(dg), _p(db))
+    return dx, dg, db
+
+
+def bn_running_update(M, mean, var, momentum, run_mean, run_var):
+    mean, var = _f32(mean), _f32(var)
+    rm, rv = _f32(run_mean).copy(), _f32(run_var).copy()
+    lib().flref_bn_running_update(_i64(mean.size), _i64(M), _p(mean), _p(var),
+                                  C.c_double(momentum), _p(rm), _p(rv))
+    return rm, rv
+
+
+def bn_view(shape_whcn, axes):
+    """(outer, C, inner) of the view the oneDNN extension builds from a Flashlight
+    shape [d0,d1,...] (column-major) and feature axes
+    (flashlight/fl/autograd/tensor/backend/onednn/BatchNorm.cpp:40-71,124-130)."""
+    axes = sorted(axes)
+    if axes != list(range(axes[0], axes[-1] + 1)):
+        raise ValueError("axis array should be continuous")
+    nfeat = 1
+    for a in axes:
+        nfeat *= shape_whcn[a]
+    total = 1
+    for s in shape_whcn:
+        total *= s
+    if axes[0] == 0:
+        return total // nfeat, nfeat, 1
+    outer = 1
+    for s in shape_whcn[axes[-1] + 1:]:
+        outer *= s
+    return outer, nfeat, total // (nfeat * outer)
