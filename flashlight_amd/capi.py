@@ -1,0 +1,80 @@
+"""ctypes declarations of include/flhip.h."""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libflhip.so")
+
+OK, INVALID_ARGUMENT, RUNTIME_ERROR = 0, 1, 2
+F32, BF16 = 0, 1
+CONV_FWD, CONV_BWD_DATA, CONV_BWD_FILTER = 0, 1, 2
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "N", "C", "H", "W", "K", "KH", "KW", "sy", "sx", "py", "px",
+        "dil_y", "dil_x", "groups", "dtype")]
+
+
+class PoolDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "N", "C", "H", "W", "wy", "wx", "sy", "sx", "py", "px", "mode", "dtype")]
+
+
+class BnDesc(C.Structure):
+    _fields_ = [("outer", C.c_int64), ("C", C.c_int64), ("inner", C.c_int64),
+                ("dtype", C.c_int32)]
+
+
+# every symbol include/flhip.h declares: name -> (restype, argtypes)
+_VP, _SZ, _I32P = C.c_void_p, C.c_size_t, C.POINTER(C.c_int32)
+SYMBOLS = {
+    "flhip_last_error": (C.c_char_p, []),
+    "flhip_version": (C.c_int, []),
+    "flhip_arch": (C.c_char_p, []),
+    "flhip_conv2d_out_dims": (C.c_int, [C.POINTER(ConvDesc), _I32P, _I32P]),
+    "flhip_pool2d_out_dims": (C.c_int, [C.POINTER(PoolDesc), _I32P, _I32P]),
+    "flhip_conv2d_workspace_bytes": (_SZ, [C.POINTER(ConvDesc), C.c_int]),
+    "flhip_conv2d_fwd": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
+    "flhip_conv2d_bwd_data": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _SZ, _VP]),
+    "flhip_conv2d_bwd_filter": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
+    "flhip_pool2d_fwd": (C.c_int, [C.POINTER(PoolDesc), _VP, _VP, _VP, _VP]),
+    "flhip_pool2d_bwd": (C.c_int, [C.POINTER(PoolDesc), _VP, _VP, _VP, _VP]),
+    "flhip_bn_workspace_bytes": (_SZ, [C.POINTER(BnDesc)]),
+    "flhip_bn_fwd_train": (C.c_int, [C.POINTER(BnDesc), _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
+                                      C.c_double, C.c_double, _VP, _SZ, _VP]),
+    "flhip_bn_fwd_infer": (C.c_int, [C.POINTER(BnDesc), _VP, _VP, _VP, _VP, _VP, C.c_double,
+                                      _VP, _VP]),
+    "flhip_bn_bwd": (C.c_int, [C.POINTER(BnDesc), _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
+                                _SZ, _VP]),
+    "flhip_copy_bytes": (C.c_int, [_VP, _VP, _SZ, _VP]),
+}
+
+_lib = None
+
+
+def lib():
+    """Loads libflhip.so; there is no fallback when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "flashlight_amd: %s is missing; build it with "
+                "`python -m flashlight_amd.build` (needs hipcc)" % LIB_PATH)
+        h = C.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            f = getattr(h, name)
+            f.restype = res
+            f.argtypes = args
+        _lib = h
+    return _lib
+
+
+def check(rc):
+    """Maps a status to the exception kinds of the reference boundary."""
+    if rc == OK:
+        return
+    msg = lib().flhip_last_error().decode()
+    if rc == INVALID_ARGUMENT:
+        raise ValueError(msg)      # std::invalid_argument
+    raise RuntimeError(msg)        # std::runtime_error

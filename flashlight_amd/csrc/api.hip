@@ -1,0 +1,76 @@
+// Error state, version and the calibration copy kernel of the C ABI.
+#include "common.h"
+
+namespace flhip {
+
+static thread_local std::string g_last_error;
+
+void set_error(const std::string& msg) { g_last_error = msg; }
+int fail(int code, const std::string& msg) {
+  g_last_error = msg;
+  return code;
+}
+
+__global__ void __launch_bounds__(256) copy16_kernel(const uint4* __restrict__ src,
+                                                      uint4* __restrict__ dst,
+                                                      size_t n16) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
+    dst[i] = src[i];
+}
+
+}  // namespace flhip
+
+using namespace flhip;
+
+extern "C" const char* flhip_last_error(void) { return g_last_error.c_str(); }
+extern "C" int flhip_version(void) { return 100; }
+extern "C" const char* flhip_arch(void) { return "gfx950"; }
+
+extern "C" int flhip_conv2d_out_dims(const flhip_conv_desc* d, int32_t* OH, int32_t* OW) {
+  FLHIP_REQUIRE(d && OH && OW, "conv2d_out_dims: null argument");
+  FLHIP_REQUIRE(d->N > 0 && d->C > 0 && d->H > 0 && d->W > 0 && d->K > 0 &&
+                    d->KH > 0 && d->KW > 0,
+                "conv2d: sizes must be positive");
+  FLHIP_REQUIRE(d->sy > 0 && d->sx > 0 && d->dil_y > 0 && d->dil_x > 0,
+                "conv2d: stride and dilation must be positive");
+  FLHIP_REQUIRE(d->py >= 0 && d->px >= 0, "conv2d: padding must be non-negative");
+  FLHIP_REQUIRE(d->groups > 0 && d->C % d->groups == 0 && d->K % d->groups == 0,
+                "conv2d: groups must divide input and output channels");
+  FLHIP_REQUIRE(dtype_ok(d->dtype), "conv2d: unknown dtype");
+  const int eh = 1 + (d->KH - 1) * d->dil_y, ew = 1 + (d->KW - 1) * d->dil_x;
+  FLHIP_REQUIRE(d->H + 2 * d->py >= eh && d->W + 2 * d->px >= ew,
+                "conv2d: kernel larger than padded input");
+  *OH = 1 + (d->H + 2 * d->py - eh) / d->sy;
+  *OW = 1 + (d->W + 2 * d->px - ew) / d->sx;
+  return FLHIP_OK;
+}
+
+extern "C" int flhip_pool2d_out_dims(const flhip_pool_desc* d, int32_t* OH, int32_t* OW) {
+  FLHIP_REQUIRE(d && OH && OW, "pool2d_out_dims: null argument");
+  FLHIP_REQUIRE(d->N > 0 && d->C > 0 && d->H > 0 && d->W > 0 && d->wy > 0 && d->wx > 0,
+                "pool2d: sizes must be positive");
+  FLHIP_REQUIRE(d->sy > 0 && d->sx > 0, "pool2d: stride must be positive");
+  FLHIP_REQUIRE(d->py >= 0 && d->px >= 0 && d->py < d->wy && d->px < d->wx,
+                "pool2d: padding must be non-negative and smaller than the window");
+  FLHIP_REQUIRE(d->mode >= FLHIP_POOL_MAX && d->mode <= FLHIP_POOL_AVG_EXCLUDE_PADDING,
+                "pool2d: unknown pooling mode");
+  FLHIP_REQUIRE(dtype_ok(d->dtype), "pool2d: unknown dtype");
+  FLHIP_REQUIRE(d->H + 2 * d->py >= d->wy && d->W + 2 * d->px >= d->wx,
+                "pool2d: window larger than padded input");
+  *OH = 1 + (d->H + 2 * d->py - d->wy) / d->sy;
+  *OW = 1 + (d->W + 2 * d->px - d->wx) / d->sx;
+  return FLHIP_OK;
+}
+
+extern "C" int flhip_copy_bytes(const void* src, void* dst, size_t bytes, void* stream) {
+  FLHIP_REQUIRE(src && dst, "copy_bytes: null pointer");
+  FLHIP_REQUIRE(bytes % 16 == 0, "copy_bytes: size must be a multiple of 16");
+  if (bytes == 0) return FLHIP_OK;
+  const size_t n16 = bytes / 16;
+  size_t blocks = (n16 + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                     reinterpret_cast<const uint4*>(src), reinterpret_cast<uint4*>(dst), n16);
+  return check_launch("copy_bytes");
+}

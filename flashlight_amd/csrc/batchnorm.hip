@@ -1,0 +1,529 @@
+// batchnorm (train / inference) and batchnormBackward.
+//
+// View: element (o, c, i) at (o*C + c)*inner + i.  Two kernels per pass:
+//   1. partial per-feature sums over S slices of the (o, i) domain, written to
+//      the workspace as ws[(c*S + s)*2 + {0,1}];
+//   2. an elementwise kernel whose prologue folds the S partials of its feature
+//      (in double) and then streams the tensor once more.
+// inner > 1 ("segment" kernels): every feature owns `outer` contiguous runs of
+// `inner` elements; threads stream them with 4-wide loads when inner % 4 == 0.
+// inner == 1 ("column" kernels, per-activation mode): features are contiguous, a
+// wave covers 64 features and rows are strided by C.
+#include "common.h"
+
+namespace flhip {
+
+struct BnGeom {
+  long long outer, C, inner;
+  int S;            // slices per feature
+  long long units;  // seg: outer * inner / VEC   col: outer
+  long long ups;    // units per slice
+  int step_o, step_i;  // seg: 256 = step_o * (inner/VEC) + step_i
+};
+
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// Folds the S (<= 64) partial pairs of feature c; valid in wave 0.
+__device__ __forceinline__ void fold_partials(const float* __restrict__ ws, long long c, int S,
+                                              double* a, double* b) {
+  const int lane = threadIdx.x & 63;
+  double p0 = 0.0, p1 = 0.0;
+  if (lane < S) {
+    p0 = (double)ws[(c * S + lane) * 2 + 0];
+    p1 = (double)ws[(c * S + lane) * 2 + 1];
+  }
+  *a = wave_sum_f64(p0);
+  *b = wave_sum_f64(p1);
+}
+
+template <typename T, int VEC>
+struct Vec;
+template <typename T>
+struct Vec<T, 1> {
+  float v[1];
+  __device__ __forceinline__ void load(const T* p, size_t i) { v[0] = ld(p, i); }
+  __device__ __forceinline__ void store(T* p, size_t i) const { st(p, i, v[0]); }
+};
+template <typename T>
+struct Vec<T, 4> {
+  float v[4];
+  __device__ __forceinline__ void load(const T* p, size_t i) {
+    const float4 f = ld4(p, i);
+    v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
+  }
+  __device__ __forceinline__ void store(T* p, size_t i) const {
+    st4(p, i, make_float4(v[0], v[1], v[2], v[3]));
+  }
+};
+
+// Iterates the units [u0, u1) of slice blockIdx.x of feature blockIdx.y.
+#define BN_SEG_LOOP_BEGIN(g)                                                   \
+  const long long c = blockIdx.y;                                              \
+  const long long innerV = (g).inner / VEC;                                    \
+  const long long u0 = (long long)blockIdx.x * (g).ups;                        \
+  const long long u1 = min(u0 + (g).ups, (g).units);                           \
+  long long u = u0 + threadIdx.x;                                              \
+  long long o = u / innerV;                                                    \
+  long long i = u - o * innerV;                                                \
+  for (; u < u1; u += 256) {                                                   \
+    const size_t off = (size_t)((o * (g).C + c) * (g).inner + i * VEC);
+#define BN_SEG_LOOP_END(g)                                                     \
+    o += (g).step_o;                                                           \
+    i += (g).step_i;                                                           \
+    if (i >= innerV) {                                                         \
+      i -= innerV;                                                             \
+      ++o;                                                                     \
+    }                                                                          \
+  }
+
+// ---- forward, segment mode -------------------------------------------------
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+bn_stats_seg(BnGeom g, const T* __restrict__ x, float* __restrict__ ws) {
+  __shared__ float red[8];
+  float s1 = 0.f, s2 = 0.f;
+  const float shift = ld(x, (size_t)(blockIdx.y * g.inner));
+  BN_SEG_LOOP_BEGIN(g)
+    Vec<T, VEC> a;
+    a.load(x, off);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      const float t = a.v[k] - shift;
+      s1 += t;
+      s2 += t * t;
+    }
+  BN_SEG_LOOP_END(g)
+  s1 = block_sum(s1, red);
+  s2 = block_sum(s2, red);
+  if (threadIdx.x == 0) {
+    ws[(c * g.S + blockIdx.x) * 2 + 0] = s1;
+    ws[(c * g.S + blockIdx.x) * 2 + 1] = s2;
+  }
+}
+
+struct BnTrainArgs {
+  const float* gamma;
+  const float* beta;
+  float* save_mean;
+  float* save_invstd;
+  float* run_mean;
+  float* run_var;
+  double momentum, eps;
+};
+
+// Mean / inverse std of feature c from the folded shifted sums; lane 0 of wave 0
+// of slice 0 also publishes the statistics.
+__device__ __forceinline__ void finish_stats(const BnGeom& g, const BnTrainArgs& a, long long c,
+                                             float shift, double p0, double p1, bool publish,
+                                             float* sh /* [2] */) {
+  if (threadIdx.x == 0) {
+    const double M = (double)g.outer * (double)g.inner;
+    const double m1 = p0 / M;
+    double var = p1 / M - m1 * m1;
+    if (var < 0.0) var = 0.0;
+    const double mean = (double)shift + m1;
+    const double invstd = 1.0 / sqrt(var + a.eps);
+    sh[0] = (float)mean;
+    sh[1] = (float)invstd;
+    if (publish) {
+      if (a.save_mean) a.save_mean[c] = (float)mean;
+      if (a.save_invstd) a.save_invstd[c] = (float)invstd;
+      if (a.run_mean && a.run_var) {
+        if (a.momentum == 0.0) {
+          a.run_mean[c] = (float)mean;
+          a.run_var[c] = (float)var;
+        } else {
+          const double unb = M > 1.0 ? var * M / (M - 1.0) : var;
+          a.run_mean[c] = (float)((1.0 - a.momentum) * (double)a.run_mean[c] + a.momentum * mean);
+          a.run_var[c] = (float)((1.0 - a.momentum) * (double)a.run_var[c] + a.momentum * unb);
+        }
+      }
+    }
+  }
+}
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+bn_train_apply_seg(BnGeom g, const T* __restrict__ x, T* __restrict__ y,
+                   const float* __restrict__ ws, BnTrainArgs a) {
+  __shared__ float sh[2];
+  if (threadIdx.x < 64) {
+    double p0, p1;
+    fold_partials(ws, blockIdx.y, g.S, &p0, &p1);
+    finish_stats(g, a, blockIdx.y, ld(x, (size_t)(blockIdx.y * g.inner)), p0, p1,
+                 blockIdx.x == 0, sh);
+  }
+  __syncthreads();
+  const float mean = sh[0];
+  const float gm = a.gamma ? a.gamma[blockIdx.y] : 1.f;
+  const float scale = gm * sh[1];
+  const float bt = a.beta ? a.beta[blockIdx.y] : 0.f;
+  BN_SEG_LOOP_BEGIN(g)
+    Vec<T, VEC> v;
+    v.load(x, off);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) v.v[k] = (v.v[k] - mean) * scale + bt;
+    v.store(y, off);
+  BN_SEG_LOOP_END(g)
+}
+
+// ---- backward, segment mode ------------------------------------------------
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+bn_bwd_stats_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
+                 const float* __restrict__ save_mean, float* __restrict__ ws) {
+  __shared__ float red[8];
+  float s1 = 0.f, s2 = 0.f;
+  const float mean = save_mean[blockIdx.y];
+  BN_SEG_LOOP_BEGIN(g)
+    Vec<T, VEC> a, b;
+    a.load(x, off);
+    b.load(dy, off);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      s1 += b.v[k];
+      s2 += b.v[k] * (a.v[k] - mean);
+    }
+  BN_SEG_LOOP_END(g)
+  s1 = block_sum(s1, red);
+  s2 = block_sum(s2, red);
+  if (threadIdx.x == 0) {
+    ws[(c * g.S + blockIdx.x) * 2 + 0] = s1;
+    ws[(c * g.S + blockIdx.x) * 2 + 1] = s2;
+  }
+}
+
+struct BnBwdArgs {
+  const float* gamma;
+  const float* save_mean;
+  const float* save_invstd;
+  float* dgamma;
+  float* dbeta;
+};
+
+// dx = k_dy*dy + k_x*(x-mean) + k_0 for feature c; publishes dgamma/dbeta.
+__device__ __forceinline__ void finish_bwd(const BnGeom& g, const BnBwdArgs& a, long long c,
+                                           double p0, double p1, bool publish, float* sh /*[4]*/) {
+  if (threadIdx.x == 0) {
+    const double M = (double)g.outer * (double)g.inner;
+    const double is = (double)a.save_invstd[c];
+    const double gm = a.gamma ? (double)a.gamma[c] : 1.0;
+    sh[0] = a.save_mean[c];
+    sh[1] = (float)(gm * is);                    // k_dy
+    sh[2] = (float)(-gm * is * is * is * p1 / M);  // k_x
+    sh[3] = (float)(-gm * is * p0 / M);          // k_0
+    if (publish) {
+      if (a.dgamma) a.dgamma[c] = (float)(p1 * is);
+      if (a.dbeta) a.dbeta[c] = (float)p0;
+    }
+  }
+}
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+bn_bwd_apply_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
+                 T* __restrict__ dx, const float* __restrict__ ws, BnBwdArgs a) {
+  __shared__ float sh[4];
+  if (threadIdx.x < 64) {
+    double p0, p1;
+    fold_partials(ws, blockIdx.y, g.S, &p0, &p1);
+    finish_bwd(g, a, blockIdx.y, p0, p1, blockIdx.x == 0, sh);
+  }
+  __syncthreads();
+  const float mean = sh[0], kdy = sh[1], kx = sh[2], k0 = sh[3];
+  BN_SEG_LOOP_BEGIN(g)
+    Vec<T, VEC> v, w;
+    v.load(x, off);
+    w.load(dy, off);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) v.v[k] = kdy * w.v[k] + (kx * (v.v[k] - mean) + k0);
+    v.store(dx, off);
+  BN_SEG_LOOP_END(g)
+}
+
+// ---- column mode (inner == 1) ----------------------------------------------
+// block = 64 features x 4 row lanes; grid = (ceil(C/64), S); slice s owns rows
+// [s*ups, (s+1)*ups).
+template <typename T, bool BWD>
+__global__ void __launch_bounds__(256)
+bn_stats_col(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
+             const float* __restrict__ save_mean, float* __restrict__ ws) {
+  __shared__ float red[2][4][64];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const long long c = (long long)blockIdx.x * 64 + tx;
+  const long long r0 = (long long)blockIdx.y * g.ups, r1 = min(r0 + g.ups, g.outer);
+  float s1 = 0.f, s2 = 0.f;
+  if (c < g.C) {
+    const float ref = BWD ? save_mean[c] : ld(x, (size_t)c);
+    for (long long r = r0 + ty; r < r1; r += 4) {
+      const size_t off = (size_t)(r * g.C + c);
+      if (BWD) {
+        const float d = ld(dy, off);
+        s1 += d;
+        s2 += d * (ld(x, off) - ref);
+      } else {
+        const float t = ld(x, off) - ref;
+        s1 += t;
+        s2 += t * t;
+      }
+    }
+  }
+  red[0][ty][tx] = s1;
+  red[1][ty][tx] = s2;
+  __syncthreads();
+  if (ty == 0 && c < g.C) {
+    ws[(c * g.S + blockIdx.y) * 2 + 0] = (red[0][0][tx] + red[0][1][tx]) + (red[0][2][tx] + red[0][3][tx]);
+    ws[(c * g.S + blockIdx.y) * 2 + 1] = (red[1][0][tx] + red[1][1][tx]) + (red[1][2][tx] + red[1][3][tx]);
+  }
+}
+
+// Per-feature coefficients for the column apply kernels: out = k1*in1 + k2*(x-mean) + k0.
+// One thread per feature folds the partials serially (S is small).
+template <typename T>
+__global__ void __launch_bounds__(256)
+bn_train_apply_col(BnGeom g, const T* __restrict__ x, T* __restrict__ y,
+                   const float* __restrict__ ws, BnTrainArgs a) {
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const long long c = (long long)blockIdx.x * 64 + tx;
+  if (c >= g.C) return;
+  double p0 = 0.0, p1 = 0.0;
+  for (int s = 0; s < g.S; ++s) {
+    p0 += (double)ws[(c * g.S + s) * 2 + 0];
+    p1 += (double)ws[(c * g.S + s) * 2 + 1];
+  }
+  const double M = (double)g.outer;
+  const double m1 = p0 / M;
+  double var = p1 / M - m1 * m1;
+  if (var < 0.0) var = 0.0;
+  const double mean = (double)ld(x, (size_t)c) + m1;
+  const double invstd = 1.0 / sqrt(var + a.eps);
+  if (blockIdx.y == 0 && ty == 0) {
+    if (a.save_mean) a.save_mean[c] = (float)mean;
+    if (a.save_invstd) a.save_invstd[c] = (float)invstd;
+    if (a.run_mean && a.run_var) {
+      if (a.momentum == 0.0) {
+        a.run_mean[c] = (float)mean;
+        a.run_var[c] = (float)var;
+      } else {
+        const double unb = M > 1.0 ? var * M / (M - 1.0) : var;
+        a.run_mean[c] = (float)((1.0 - a.momentum) * (double)a.run_mean[c] + a.momentum * mean);
+        a.run_var[c] = (float)((1.0 - a.momentum) * (double)a.run_var[c] + a.momentum * unb);
+      }
+    }
+  }
+  const float fm = (float)mean;
+  const float scale = (a.gamma ? a.gamma[c] : 1.f) * (float)invstd;
+  const float bt = a.beta ? a.beta[c] : 0.f;
+  const long long r0 = (long long)blockIdx.y * g.ups, r1 = min(r0 + g.ups, g.outer);
+  for (long long r = r0 + ty; r < r1; r += 4) {
+    const size_t off = (size_t)(r * g.C + c);
+    st(y, off, (ld(x, off) - fm) * scale + bt);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+bn_bwd_apply_col(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
+                 T* __restrict__ dx, const float* __restrict__ ws, BnBwdArgs a) {
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const long long c = (long long)blockIdx.x * 64 + tx;
+  if (c >= g.C) return;
+  double p0 = 0.0, p1 = 0.0;
+  for (int s = 0; s < g.S; ++s) {
+    p0 += (double)ws[(c * g.S + s) * 2 + 0];
+    p1 += (double)ws[(c * g.S + s) * 2 + 1];
+  }
+  const double M = (double)g.outer;
+  const double is = (double)a.save_invstd[c];
+  const double gm = a.gamma ? (double)a.gamma[c] : 1.0;
+  const float mean = a.save_mean[c];
+  const float kdy = (float)(gm * is), kx = (float)(-gm * is * is * is * p1 / M),
+              k0 = (float)(-gm * is * p0 / M);
+  if (blockIdx.y == 0 && ty == 0) {
+    if (a.dgamma) a.dgamma[c] = (float)(p1 * is);
+    if (a.dbeta) a.dbeta[c] = (float)p0;
+  }
+  const long long r0 = (long long)blockIdx.y * g.ups, r1 = min(r0 + g.ups, g.outer);
+  for (long long r = r0 + ty; r < r1; r += 4) {
+    const size_t off = (size_t)(r * g.C + c);
+    st(dx, off, kdy * ld(dy, off) + (kx * (ld(x, off) - mean) + k0));
+  }
+}
+
+// ---- inference ---------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+bn_infer_kernel(BnGeom g, const T* __restrict__ x, T* __restrict__ y,
+                const float* __restrict__ gamma, const float* __restrict__ beta,
+                const float* __restrict__ mean, const float* __restrict__ var, float eps,
+                size_t total) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+    const long long c = (long long)((e / (size_t)g.inner) % (size_t)g.C);
+    const float is = 1.0f / sqrtf(var[c] + eps);
+    const float gm = gamma ? gamma[c] : 1.f, bt = beta ? beta[c] : 0.f;
+    st(y, e, (ld(x, e) - mean[c]) * (gm * is) + bt);
+  }
+}
+
+// ---- host side ---------------------------------------------------------------
+static int make_geom(const flhip_bn_desc* d, BnGeom* g, int* vec) {
+  FLHIP_REQUIRE(d, "batchnorm: null descriptor");
+  FLHIP_REQUIRE(d->outer > 0 && d->C > 0 && d->inner > 0, "batchnorm: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(d->dtype), "batchnorm: unknown dtype");
+  g->outer = d->outer;
+  g->C = d->C;
+  g->inner = d->inner;
+  if (d->inner == 1) {
+    *vec = 0;
+    const long long cb = (d->C + 63) / 64;
+    FLHIP_REQUIRE(cb <= 0x7fffffffLL, "batchnorm: too many features");
+    long long S = 4096 / cb;
+    const long long maxS = (d->outer + 3) / 4;
+    if (S > maxS) S = maxS;
+    if (S > 64) S = 64;
+    if (S < 1) S = 1;
+    g->S = (int)S;
+    g->units = d->outer;
+    g->ups = (g->units + S - 1) / S;
+    g->step_o = g->step_i = 0;
+  } else {
+    FLHIP_REQUIRE(d->C <= 65535, "batchnorm: spatial mode supports at most 65535 features");
+    *vec = (d->inner % 4 == 0) ? 4 : 1;
+    const long long innerV = d->inner / *vec;
+    g->units = d->outer * innerV;
+    long long S = 4096 / d->C;
+    const long long maxS = (g->units + 511) / 512;
+    if (S > maxS) S = maxS;
+    if (S > 64) S = 64;
+    if (S < 1) S = 1;
+    g->S = (int)S;
+    g->ups = (g->units + S - 1) / S;
+    g->step_o = (int)(256 / innerV);
+    g->step_i = (int)(256 % innerV);
+  }
+  return FLHIP_OK;
+}
+
+template <typename T>
+static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws,
+                     const BnTrainArgs& a, hipStream_t s) {
+  const T* xp = static_cast<const T*>(x);
+  T* yp = static_cast<T*>(y);
+  if (vec == 0) {
+    const dim3 grid((unsigned)((g.C + 63) / 64), g.S);
+    hipLaunchKernelGGL((bn_stats_col<T, false>), grid, dim3(256), 0, s, g, xp, (const T*)nullptr,
+                       (const float*)nullptr, ws);
+    hipLaunchKernelGGL((bn_train_apply_col<T>), grid, dim3(256), 0, s, g, xp, yp, ws, a);
+  } else {
+    const dim3 grid(g.S, (unsigned)g.C);
+    if (vec == 4) {
+      hipLaunchKernelGGL((bn_stats_seg<T, 4>), grid, dim3(256), 0, s, g, xp, ws);
+      hipLaunchKernelGGL((bn_train_apply_seg<T, 4>), grid, dim3(256), 0, s, g, xp, yp, ws, a);
+    } else {
+      hipLaunchKernelGGL((bn_stats_seg<T, 1>), grid, dim3(256), 0, s, g, xp, ws);
+      hipLaunchKernelGGL((bn_train_apply_seg<T, 1>), grid, dim3(256), 0, s, g, xp, yp, ws, a);
+    }
+  }
+  return check_launch("bn_fwd_train");
+}
+
+template <typename T>
+static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void* dx, float* ws,
+                   const BnBwdArgs& a, hipStream_t s) {
+  const T* xp = static_cast<const T*>(x);
+  const T* dyp = static_cast<const T*>(dy);
+  T* dxp = static_cast<T*>(dx);
+  if (vec == 0) {
+    const dim3 grid((unsigned)((g.C + 63) / 64), g.S);
+    hipLaunchKernelGGL((bn_stats_col<T, true>), grid, dim3(256), 0, s, g, xp, dyp, a.save_mean, ws);
+    hipLaunchKernelGGL((bn_bwd_apply_col<T>), grid, dim3(256), 0, s, g, xp, dyp, dxp, ws, a);
+  } else {
+    const dim3 grid(g.S, (unsigned)g.C);
+    if (vec == 4) {
+      hipLaunchKernelGGL((bn_bwd_stats_seg<T, 4>), grid, dim3(256), 0, s, g, xp, dyp, a.save_mean, ws);
+      hipLaunchKernelGGL((bn_bwd_apply_seg<T, 4>), grid, dim3(256), 0, s, g, xp, dyp, dxp, ws, a);
+    } else {
+      hipLaunchKernelGGL((bn_bwd_stats_seg<T, 1>), grid, dim3(256), 0, s, g, xp, dyp, a.save_mean, ws);
+      hipLaunchKernelGGL((bn_bwd_apply_seg<T, 1>), grid, dim3(256), 0, s, g, xp, dyp, dxp, ws, a);
+    }
+  }
+  return check_launch("bn_bwd");
+}
+
+}  // namespace flhip
+
+using namespace flhip;
+
+extern "C" size_t flhip_bn_workspace_bytes(const flhip_bn_desc* d) {
+  BnGeom g;
+  int vec;
+  if (make_geom(d, &g, &vec) != FLHIP_OK) return 0;
+  return (size_t)g.C * g.S * 2 * sizeof(float);
+}
+
+extern "C" int flhip_bn_fwd_train(const flhip_bn_desc* d, const void* x, const float* gamma,
+                                  const float* beta, void* y, float* save_mean,
+                                  float* save_invstd, float* run_mean, float* run_var,
+                                  double momentum, double eps, void* ws, size_t ws_bytes,
+                                  void* stream) {
+  BnGeom g;
+  int vec;
+  const int rc = make_geom(d, &g, &vec);
+  if (rc != FLHIP_OK) return rc;
+  FLHIP_REQUIRE(x && y, "bn_fwd_train: null tensor");
+  FLHIP_REQUIRE((run_mean == nullptr) == (run_var == nullptr),
+                "bn_fwd_train: running mean and variance must be given together");
+  FLHIP_REQUIRE(momentum >= 0.0 && momentum <= 1.0, "bn_fwd_train: momentum must lie in [0, 1]");
+  FLHIP_REQUIRE(eps >= 0.0, "bn_fwd_train: epsilon must be non-negative");
+  FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_fwd_train: workspace too small");
+  const BnTrainArgs a{gamma, beta, save_mean, save_invstd, run_mean, run_var, momentum, eps};
+  return d->dtype == FLHIP_F32
+             ? run_train<float>(g, vec, x, y, static_cast<float*>(ws), a, as_stream(stream))
+             : run_train<bf16_t>(g, vec, x, y, static_cast<float*>(ws), a, as_stream(stream));
+}
+
+extern "C" int flhip_bn_fwd_infer(const flhip_bn_desc* d, const void* x, const float* gamma,
+                                  const float* beta, const float* run_mean, const float* run_var,
+                                  double eps, void* y, void* stream) {
+  BnGeom g;
+  int vec;
+  const int rc = make_geom(d, &g, &vec);
+  if (rc != FLHIP_OK) return rc;
+  FLHIP_REQUIRE(x && y && run_mean && run_var, "bn_fwd_infer: null tensor");
+  const size_t total = (size_t)g.outer * g.C * g.inner;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  if (d->dtype == FLHIP_F32)
+    hipLaunchKernelGGL((bn_infer_kernel<float>), dim3((unsigned)blocks), dim3(256), 0,
+                       as_stream(stream), g, static_cast<const float*>(x), static_cast<float*>(y),
+                       gamma, beta, run_mean, run_var, (float)eps, total);
+  else
+    hipLaunchKernelGGL((bn_infer_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0,
+                       as_stream(stream), g, static_cast<const bf16_t*>(x),
+                       static_cast<bf16_t*>(y), gamma, beta, run_mean, run_var, (float)eps, total);
+  return check_launch("bn_fwd_infer");
+}
+
+extern "C" int flhip_bn_bwd(const flhip_bn_desc* d, const void* x, const void* dy,
+                            const float* gamma, const float* save_mean, const float* save_invstd,
+                            void* dx, float* dgamma, float* dbeta, void* ws, size_t ws_bytes,
+                            void* stream) {
+  BnGeom g;
+  int vec;
+  const int rc = make_geom(d, &g, &vec);
+  if (rc != FLHIP_OK) return rc;
+  FLHIP_REQUIRE(x && dy && dx, "bn_bwd: null tensor");
+  // the reference throws std::invalid_argument without the forward payload
+  // (onednn/BatchNorm.cpp:212-215)
+  FLHIP_REQUIRE(save_mean && save_invstd, "bn_bwd: needs the saved statistics of the forward pass");
+  FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_bwd: workspace too small");
+  const BnBwdArgs a{gamma, save_mean, save_invstd, dgamma, dbeta};
+  return d->dtype == FLHIP_F32
+             ? run_bwd<float>(g, vec, x, dy, dx, static_cast<float*>(ws), a, as_stream(stream))
+             : run_bwd<bf16_t>(g, vec, x, dy, dx, static_cast<float*>(ws), a, as_stream(stream));
+}

@@ -1,0 +1,100 @@
+// Shared device/host helpers for the gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "flhip.h"
+
+namespace flhip {
+
+// ---- errors ---------------------------------------------------------------
+void set_error(const std::string& msg);
+int fail(int code, const std::string& msg);
+
+#define FLHIP_REQUIRE(cond, msg)                                    \
+  do {                                                              \
+    if (!(cond)) return ::flhip::fail(FLHIP_INVALID_ARGUMENT, msg); \
+  } while (0)
+
+// Checks the launch itself; execution errors surface at the caller's next sync.
+inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess)
+    return fail(FLHIP_RUNTIME_ERROR,
+                std::string(what) + ": " + hipGetErrorString(e));
+  return FLHIP_OK;
+}
+
+// ---- storage types --------------------------------------------------------
+typedef uint16_t bf16_t;  // raw bits
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+  return __uint_as_float(((uint32_t)v) << 16);
+}
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float ld(const float* p, size_t i) { return p[i]; }
+__device__ __forceinline__ float ld(const bf16_t* p, size_t i) {
+  return bf16_to_f32(p[i]);
+}
+__device__ __forceinline__ void st(float* p, size_t i, float v) { p[i] = v; }
+__device__ __forceinline__ void st(bf16_t* p, size_t i, float v) {
+  p[i] = f32_to_bf16(v);
+}
+
+// four consecutive elements, 16-byte (f32) / 8-byte (bf16) aligned
+__device__ __forceinline__ float4 ld4(const float* p, size_t i) {
+  return *reinterpret_cast<const float4*>(p + i);
+}
+__device__ __forceinline__ float4 ld4(const bf16_t* p, size_t i) {
+  uint2 r = *reinterpret_cast<const uint2*>(p + i);
+  return make_float4(__uint_as_float(r.x << 16),
+                     __uint_as_float(r.x & 0xffff0000u),
+                     __uint_as_float(r.y << 16),
+                     __uint_as_float(r.y & 0xffff0000u));
+}
+__device__ __forceinline__ void st4(float* p, size_t i, float4 v) {
+  *reinterpret_cast<float4*>(p + i) = v;
+}
+__device__ __forceinline__ void st4(bf16_t* p, size_t i, float4 v) {
+  uint2 r;
+  r.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
+  r.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+  *reinterpret_cast<uint2*>(p + i) = r;
+}
+
+// ---- reductions -----------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// Sum of `v` over the block; result valid in every thread.  `smem` holds at
+// least blockDim.x/64 floats and may be reused after the call returns.
+__device__ __forceinline__ float block_sum(float v, float* smem) {
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int nw = (blockDim.x + 63) >> 6;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) smem[wid] = v;
+  __syncthreads();
+  float r = 0.f;
+  for (int i = 0; i < nw; ++i) r += smem[i];
+  return r;
+}
+
+inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline bool dtype_ok(int32_t dt) { return dt == FLHIP_F32 || dt == FLHIP_BF16; }
+
+}  // namespace flhip

@@ -1,0 +1,24 @@
+// Internal interface between the convolution entry points and their kernels.
+#pragma once
+#include "common.h"
+
+namespace flhip {
+
+struct ConvGeom {
+  int N, C, H, W, K, KH, KW, OH, OW;
+  int sy, sx, py, px, dly, dlx, groups;
+  int Cg, Kg;  // channels per group
+};
+
+// Implicit-GEMM MFMA kernels (conv2d_mfma.hip).  Each returns FLHIP_OK after
+// enqueueing, or -1 when the shape is outside what the kernel handles (the
+// caller then uses the direct kernels).
+int mfma_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w, const float* bias,
+                  void* y, hipStream_t s);
+int mfma_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
+                       hipStream_t s);
+int mfma_conv_bwd_filter(const ConvGeom& g, int dtype, const void* x, const void* dy, float* dw,
+                         float* db, void* ws, size_t ws_bytes, hipStream_t s);
+size_t mfma_conv_bwd_filter_ws(const ConvGeom& g, int dtype);
+
+}  // namespace flhip

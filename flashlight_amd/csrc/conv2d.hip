@@ -1,0 +1,240 @@
+// conv2d / conv2dBackwardData / conv2dBackwardFilterBias entry points, and the
+// direct (one thread per result) kernels that cover every geometry.  The MFMA
+// implicit-GEMM kernels in conv2d_mfma.hip are used whenever they accept the
+// shape; FLHIP_CONV_ALGO=direct in the environment forces the kernels here.
+#include <stdlib.h>
+#include <string.h>
+
+#include "conv2d.h"
+
+namespace flhip {
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+conv_fwd_direct(ConvGeom g, const T* __restrict__ x, const T* __restrict__ w,
+                const float* __restrict__ bias, T* __restrict__ y, size_t total) {
+  const size_t o = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (o >= total) return;
+  const int ow = (int)(o % g.OW);
+  size_t t = o / g.OW;
+  const int oh = (int)(t % g.OH);
+  t /= g.OH;
+  const int k = (int)(t % g.K);
+  const int n = (int)(t / g.K);
+  const int grp = k / g.Kg;
+  float acc = bias ? bias[k] : 0.f;
+  for (int c = 0; c < g.Cg; ++c) {
+    const T* xp = x + ((size_t)n * g.C + grp * g.Cg + c) * g.H * g.W;
+    const T* wp = w + ((size_t)k * g.Cg + c) * g.KH * g.KW;
+    for (int kh = 0; kh < g.KH; ++kh) {
+      const int ih = oh * g.sy - g.py + kh * g.dly;
+      if (ih < 0 || ih >= g.H) continue;
+      for (int kw = 0; kw < g.KW; ++kw) {
+        const int iw = ow * g.sx - g.px + kw * g.dlx;
+        if (iw < 0 || iw >= g.W) continue;
+        acc += ld(xp, (size_t)ih * g.W + iw) * ld(wp, kh * g.KW + kw);
+      }
+    }
+  }
+  st(y, o, acc);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+conv_bwd_data_direct(ConvGeom g, const T* __restrict__ dy, const T* __restrict__ w,
+                     T* __restrict__ dx, size_t total) {
+  const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int iw = (int)(e % g.W);
+  size_t t = e / g.W;
+  const int ih = (int)(t % g.H);
+  t /= g.H;
+  const int ci = (int)(t % g.C);
+  const int n = (int)(t / g.C);
+  const int grp = ci / g.Cg, c = ci % g.Cg;
+  float acc = 0.f;
+  for (int kk = 0; kk < g.Kg; ++kk) {
+    const int k = grp * g.Kg + kk;
+    const T* dyp = dy + ((size_t)n * g.K + k) * g.OH * g.OW;
+    const T* wp = w + ((size_t)k * g.Cg + c) * g.KH * g.KW;
+    for (int kh = 0; kh < g.KH; ++kh) {
+      const int th = ih + g.py - kh * g.dly;
+      if (th < 0 || th % g.sy != 0) continue;
+      const int oh = th / g.sy;
+      if (oh >= g.OH) continue;
+      for (int kw = 0; kw < g.KW; ++kw) {
+        const int tw = iw + g.px - kw * g.dlx;
+        if (tw < 0 || tw % g.sx != 0) continue;
+        const int ow = tw / g.sx;
+        if (ow >= g.OW) continue;
+        acc += ld(dyp, (size_t)oh * g.OW + ow) * ld(wp, kh * g.KW + kw);
+      }
+    }
+  }
+  st(dx, e, acc);
+}
+
+// one block per filter element
+template <typename T>
+__global__ void __launch_bounds__(256)
+conv_bwd_filter_direct(ConvGeom g, const T* __restrict__ x, const T* __restrict__ dy,
+                       float* __restrict__ dw) {
+  __shared__ float red[8];
+  const int e = blockIdx.x;
+  const int kw = e % g.KW;
+  int t = e / g.KW;
+  const int kh = t % g.KH;
+  t /= g.KH;
+  const int c = t % g.Cg;
+  const int k = t / g.Cg;
+  const int grp = k / g.Kg;
+  const int P = g.OH * g.OW;
+  float acc = 0.f;
+  for (int n = 0; n < g.N; ++n) {
+    const T* xp = x + ((size_t)n * g.C + grp * g.Cg + c) * g.H * g.W;
+    const T* dyp = dy + ((size_t)n * g.K + k) * P;
+    for (int p = threadIdx.x; p < P; p += 256) {
+      const int oh = p / g.OW, ow = p % g.OW;
+      const int ih = oh * g.sy - g.py + kh * g.dly, iw = ow * g.sx - g.px + kw * g.dlx;
+      if (ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
+        acc += ld(dyp, p) * ld(xp, (size_t)ih * g.W + iw);
+    }
+  }
+  acc = block_sum(acc, red);
+  if (threadIdx.x == 0) dw[e] = acc;
+}
+
+// db[k] = sum over n and pixels of dy; one block per output channel
+template <typename T>
+__global__ void __launch_bounds__(256)
+conv_bwd_bias_kernel(ConvGeom g, const T* __restrict__ dy, float* __restrict__ db) {
+  __shared__ float red[8];
+  const int k = blockIdx.x;
+  const int P = g.OH * g.OW;
+  float acc = 0.f;
+  for (int n = 0; n < g.N; ++n) {
+    const T* dyp = dy + ((size_t)n * g.K + k) * P;
+    for (int p = threadIdx.x; p < P; p += 256) acc += ld(dyp, p);
+  }
+  acc = block_sum(acc, red);
+  if (threadIdx.x == 0) db[k] = acc;
+}
+
+static bool force_direct() {
+  const char* e = getenv("FLHIP_CONV_ALGO");
+  return e && strcmp(e, "direct") == 0;
+}
+
+static int make_geom(const flhip_conv_desc* d, ConvGeom* g) {
+  int32_t OH, OW;
+  const int rc = flhip_conv2d_out_dims(d, &OH, &OW);
+  if (rc != FLHIP_OK) return rc;
+  *g = ConvGeom{d->N, d->C, d->H, d->W, d->K, d->KH, d->KW, OH, OW,
+                d->sy, d->sx, d->py, d->px, d->dil_y, d->dil_x, d->groups,
+                d->C / d->groups, d->K / d->groups};
+  FLHIP_REQUIRE((size_t)d->N * d->C * d->H * d->W < (1ull << 31) &&
+                    (size_t)d->N * d->K * OH * OW < (1ull << 31),
+                "conv2d: tensors of 2^31 elements or more are not supported");
+  return FLHIP_OK;
+}
+
+}  // namespace flhip
+
+using namespace flhip;
+
+extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pass) {
+  ConvGeom g;
+  if (make_geom(d, &g) != FLHIP_OK) return 0;
+  if (pass == FLHIP_CONV_BWD_FILTER) return mfma_conv_bwd_filter_ws(g, d->dtype);
+  return 0;
+}
+
+extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const void* w,
+                                const float* bias, void* y, void* ws, size_t ws_bytes,
+                                void* stream) {
+  (void)ws;
+  (void)ws_bytes;
+  FLHIP_REQUIRE(d && x && w && y, "conv2d_fwd: null argument");
+  ConvGeom g;
+  const int rc = make_geom(d, &g);
+  if (rc != FLHIP_OK) return rc;
+  hipStream_t s = as_stream(stream);
+  if (!force_direct()) {
+    const int r = mfma_conv_fwd(g, d->dtype, x, w, bias, y, s);
+    if (r >= 0) return r;
+  }
+  const size_t total = (size_t)g.N * g.K * g.OH * g.OW;
+  const dim3 grid((unsigned)((total + 255) / 256));
+  if (d->dtype == FLHIP_F32)
+    hipLaunchKernelGGL((conv_fwd_direct<float>), grid, dim3(256), 0, s, g,
+                       static_cast<const float*>(x), static_cast<const float*>(w), bias,
+                       static_cast<float*>(y), total);
+  else
+    hipLaunchKernelGGL((conv_fwd_direct<bf16_t>), grid, dim3(256), 0, s, g,
+                       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), bias,
+                       static_cast<bf16_t*>(y), total);
+  return check_launch("conv2d_fwd");
+}
+
+extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, const void* w,
+                                     void* dx, void* ws, size_t ws_bytes, void* stream) {
+  (void)ws;
+  (void)ws_bytes;
+  FLHIP_REQUIRE(d && dy && w && dx, "conv2d_bwd_data: null argument");
+  ConvGeom g;
+  const int rc = make_geom(d, &g);
+  if (rc != FLHIP_OK) return rc;
+  hipStream_t s = as_stream(stream);
+  if (!force_direct()) {
+    const int r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s);
+    if (r >= 0) return r;
+  }
+  const size_t total = (size_t)g.N * g.C * g.H * g.W;
+  const dim3 grid((unsigned)((total + 255) / 256));
+  if (d->dtype == FLHIP_F32)
+    hipLaunchKernelGGL((conv_bwd_data_direct<float>), grid, dim3(256), 0, s, g,
+                       static_cast<const float*>(dy), static_cast<const float*>(w),
+                       static_cast<float*>(dx), total);
+  else
+    hipLaunchKernelGGL((conv_bwd_data_direct<bf16_t>), grid, dim3(256), 0, s, g,
+                       static_cast<const bf16_t*>(dy), static_cast<const bf16_t*>(w),
+                       static_cast<bf16_t*>(dx), total);
+  return check_launch("conv2d_bwd_data");
+}
+
+extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, const void* dy,
+                                       float* dw, float* db, void* ws, size_t ws_bytes,
+                                       void* stream) {
+  FLHIP_REQUIRE(d && dy, "conv2d_bwd_filter: null argument");
+  FLHIP_REQUIRE(dw || db, "conv2d_bwd_filter: nothing to compute");
+  FLHIP_REQUIRE(!dw || x, "conv2d_bwd_filter: filter gradient needs the input");
+  ConvGeom g;
+  const int rc = make_geom(d, &g);
+  if (rc != FLHIP_OK) return rc;
+  hipStream_t s = as_stream(stream);
+  if (!force_direct()) {
+    FLHIP_REQUIRE(ws_bytes >= mfma_conv_bwd_filter_ws(g, d->dtype) &&
+                      (ws || mfma_conv_bwd_filter_ws(g, d->dtype) == 0),
+                  "conv2d_bwd_filter: workspace too small");
+    const int r = mfma_conv_bwd_filter(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
+    if (r >= 0) return r;
+  }
+  if (dw) {
+    const dim3 grid((unsigned)(g.K * g.Cg * g.KH * g.KW));
+    if (d->dtype == FLHIP_F32)
+      hipLaunchKernelGGL((conv_bwd_filter_direct<float>), grid, dim3(256), 0, s, g,
+                         static_cast<const float*>(x), static_cast<const float*>(dy), dw);
+    else
+      hipLaunchKernelGGL((conv_bwd_filter_direct<bf16_t>), grid, dim3(256), 0, s, g,
+                         static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), dw);
+  }
+  if (db) {
+    if (d->dtype == FLHIP_F32)
+      hipLaunchKernelGGL((conv_bwd_bias_kernel<float>), dim3(g.K), dim3(256), 0, s, g,
+                         static_cast<const float*>(dy), db);
+    else
+      hipLaunchKernelGGL((conv_bwd_bias_kernel<bf16_t>), dim3(g.K), dim3(256), 0, s, g,
+                         static_cast<const bf16_t*>(dy), db);
+  }
+  return check_launch("conv2d_bwd_filter");
+}

@@ -1,0 +1,263 @@
+"""Operator-level binding over torch device tensors.
+
+Argument order and meaning follow fl::AutogradExtension
+(flashlight/fl/autograd/tensor/AutogradExtension.h:58-164): ints in x-then-y
+order, `axes` as Flashlight dimension indices of the column-major shape
+[W,H,C,N].  A contiguous torch tensor of shape (N,C,H,W) is byte-identical to
+that Flashlight tensor, so torch is used here only as the owner of device
+memory and of the stream.
+"""
+import ctypes as C
+import enum
+
+import torch
+
+from . import capi
+
+
+class PoolingMode(enum.IntEnum):
+    """fl::PoolingMode (flashlight/fl/common/Defines.h:53-64)."""
+    MAX = 0
+    AVG_INCLUDE_PADDING = 1
+    AVG_EXCLUDE_PADDING = 2
+
+
+def derive_padding(in_size, filter_size, stride, pad, dilation=1):
+    """fl::derivePadding (flashlight/fl/nn/Utils.cpp:87-100); pad == -1 is SAME."""
+    if pad == -1:
+        rem = in_size % stride
+        p = ((filter_size - 1) * dilation - (stride if rem == 0 else rem) + 1 + 1) // 2
+        return max(p, 0)
+    return pad
+
+
+def _dtype_tag(t):
+    if t.dtype == torch.float32:
+        return capi.F32
+    if t.dtype == torch.bfloat16:
+        return capi.BF16
+    raise RuntimeError("flashlight_amd: unsupported dtype %s" % t.dtype)
+
+
+def _dev(t, name):
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise ValueError("%s must live on the GPU" % name)
+    if not t.is_contiguous():
+        # fl::DevicePtr refuses non-contiguous tensors (flashlight/fl/common/DevicePtr.cpp:16-33)
+        raise ValueError("%s must be contiguous" % name)
+    return t
+
+
+def _ptr(t):
+    return None if t is None or t.numel() == 0 else C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _as4(t):
+    """Missing trailing Flashlight dims count as 1 (onednn/Pool2D.cpp:95-98);
+    in row-major terms: missing LEADING dims."""
+    if t.dim() > 4:
+        raise ValueError("at most 4 dimensions")
+    return (1,) * (4 - t.dim()) + tuple(t.shape)
+
+
+def _conv_desc(x_shape, w_shape, sx, sy, px, py, dx, dy, groups, tag):
+    N, Cc, H, W = x_shape
+    K, Cg, KH, KW = w_shape
+    if Cg * groups != Cc:
+        raise ValueError("conv2d: weight/input channel mismatch")
+    return capi.ConvDesc(N, Cc, H, W, K, KH, KW, sy, sx, py, px, dy, dx, groups, tag)
+
+
+def _ws(nbytes, device):
+    return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
+
+
+def conv2d(input, weights, bias, sx=1, sy=1, px=0, py=0, dx=1, dy=1, groups=1):
+    """AutogradExtension::conv2d.  bias may be None or empty."""
+    x, w = _dev(input, "input"), _dev(weights, "weights")
+    if x.dim() != 4 or w.dim() != 4:
+        raise ValueError("conv2d: input and weights must have 4 dimensions")
+    if x.dtype != w.dtype:
+        raise ValueError("conv2d: input and weights must have the same type")
+    tag = _dtype_tag(x)
+    d = _conv_desc(x.shape, w.shape, sx, sy, px, py, dx, dy, groups, tag)
+    oh, ow = C.c_int32(), C.c_int32()
+    capi.check(capi.lib().flhip_conv2d_out_dims(C.byref(d), C.byref(oh), C.byref(ow)))
+    b = None
+    if bias is not None and bias.numel() > 0:
+        if bias.numel() != d.K:
+            raise ValueError("conv2d: bias must have one element per output channel")
+        b = _dev(bias, "bias").float().contiguous()
+    y = torch.empty((d.N, d.K, oh.value, ow.value), dtype=x.dtype, device=x.device)
+    nws = capi.lib().flhip_conv2d_workspace_bytes(C.byref(d), capi.CONV_FWD)
+    ws = _ws(nws, x.device)
+    capi.check(capi.lib().flhip_conv2d_fwd(C.byref(d), _ptr(x), _ptr(w), _ptr(b), _ptr(y),
+                                           _ptr(ws), nws, _stream()))
+    return y
+
+
+def conv2d_backward_data(grad_output, input_shape, weights, sx=1, sy=1, px=0, py=0, dx=1, dy=1,
+                         groups=1):
+    """AutogradExtension::conv2dBackwardData; only the input's shape is needed
+    (onednn/Conv2D.cpp:285)."""
+    g, w = _dev(grad_output, "gradOutput"), _dev(weights, "weights")
+    tag = _dtype_tag(g)
+    d = _conv_desc(tuple(input_shape), w.shape, sx, sy, px, py, dx, dy, groups, tag)
+    oh, ow = C.c_int32(), C.c_int32()
+    capi.check(capi.lib().flhip_conv2d_out_dims(C.byref(d), C.byref(oh), C.byref(ow)))
+    if tuple(g.shape) != (d.N, d.K, oh.value, ow.value):
+        raise ValueError("conv2dBackwardData: gradOutput shape does not match the geometry")
+    out = torch.empty(tuple(input_shape), dtype=g.dtype, device=g.device)
+    nws = capi.lib().flhip_conv2d_workspace_bytes(C.byref(d), capi.CONV_BWD_DATA)
+    ws = _ws(nws, g.device)
+    capi.check(capi.lib().flhip_conv2d_bwd_data(C.byref(d), _ptr(g), _ptr(w), _ptr(out),
+                                                _ptr(ws), nws, _stream()))
+    return out
+
+
+def conv2d_backward_filter_bias(grad_output, input, weights_shape, want_bias, sx=1, sy=1, px=0,
+                                py=0, dx=1, dy=1, groups=1):
+    """AutogradExtension::conv2dBackwardFilterBias -> (gradWeights, gradBias or None).
+    Gradients are fp32 (the master-weight precision) for both storage types."""
+    g, x = _dev(grad_output, "gradOutput"), _dev(input, "input")
+    tag = _dtype_tag(x)
+    d = _conv_desc(x.shape, tuple(weights_shape), sx, sy, px, py, dx, dy, groups, tag)
+    oh, ow = C.c_int32(), C.c_int32()
+    capi.check(capi.lib().flhip_conv2d_out_dims(C.byref(d), C.byref(oh), C.byref(ow)))
+    if tuple(g.shape) != (d.N, d.K, oh.value, ow.value):
+        raise ValueError("conv2dBackwardFilterBias: gradOutput shape does not match the geometry")
+    dw = torch.empty(tuple(weights_shape), dtype=torch.float32, device=x.device)
+    db = torch.empty((d.K,), dtype=torch.float32, device=x.device) if want_bias else None
+    nws = capi.lib().flhip_conv2d_workspace_bytes(C.byref(d), capi.CONV_BWD_FILTER)
+    ws = _ws(nws, x.device)
+    capi.check(capi.lib().flhip_conv2d_bwd_filter(C.byref(d), _ptr(x), _ptr(g), _ptr(dw), _ptr(db),
+                                                  _ptr(ws), nws, _stream()))
+    return dw, db
+
+
+def _pool_desc(x_shape4, wx, wy, sx, sy, px, py, mode, tag):
+    N, Cc, H, W = x_shape4
+    return capi.PoolDesc(N, Cc, H, W, wy, wx, sy, sx, py, px, int(mode), tag)
+
+
+def pool2d(input, wx, wy, sx, sy, px, py, mode=PoolingMode.MAX, train=True):
+    """AutogradExtension::pool2d -> (output, argmax).  argmax (uint8, one
+    window-relative index per output) is returned for MAX when train is set —
+    the reference keeps the equivalent oneDNN workspace in its payload only when
+    a payload exists (onednn/Pool2D.cpp:88-92,150-161)."""
+    x = _dev(input, "input")
+    s4 = _as4(x)
+    d = _pool_desc(s4, wx, wy, sx, sy, px, py, mode, _dtype_tag(x))
+    oh, ow = C.c_int32(), C.c_int32()
+    capi.check(capi.lib().flhip_pool2d_out_dims(C.byref(d), C.byref(oh), C.byref(ow)))
+    oshape = (s4[0], s4[1], oh.value, ow.value)
+    y = torch.empty(oshape, dtype=x.dtype, device=x.device)
+    am = None
+    if train and int(mode) == PoolingMode.MAX:
+        am = torch.empty(oshape, dtype=torch.uint8, device=x.device)
+    capi.check(capi.lib().flhip_pool2d_fwd(C.byref(d), _ptr(x), _ptr(y), _ptr(am), _stream()))
+    return y, am
+
+
+def pool2d_backward(grad_output, input_shape, argmax, wx, wy, sx, sy, px, py,
+                    mode=PoolingMode.MAX):
+    """AutogradExtension::pool2dBackward.  The result has the type of
+    gradOutput."""
+    g = _dev(grad_output, "gradOutput")
+    s4 = (1,) * (4 - len(input_shape)) + tuple(input_shape)
+    d = _pool_desc(s4, wx, wy, sx, sy, px, py, mode, _dtype_tag(g))
+    if int(mode) == PoolingMode.MAX and argmax is None:
+        raise ValueError("pool2dBackward: max pooling needs the forward payload")
+    am = _dev(argmax, "argmax") if argmax is not None else None
+    out = torch.empty(s4, dtype=g.dtype, device=g.device)
+    capi.check(capi.lib().flhip_pool2d_bwd(C.byref(d), _ptr(g), _ptr(am), _ptr(out), _stream()))
+    return out
+
+
+def bn_view(shape_nchw, axes):
+    """(outer, C, inner) from Flashlight feature axes; the rule of
+    onednn/BatchNorm.cpp:40-71 and the contiguity check of :124-130."""
+    whcn = list(shape_nchw)[::-1]
+    axes = sorted(int(a) for a in axes)
+    if not axes or axes != list(range(axes[0], axes[-1] + 1)) or axes[-1] >= len(whcn):
+        raise ValueError("axis array should be continuous")
+    nfeat = 1
+    for a in axes:
+        nfeat *= whcn[a]
+    total = 1
+    for s in whcn:
+        total *= s
+    if axes[0] == 0:
+        return total // nfeat, nfeat, 1
+    outer = 1
+    for s in whcn[axes[-1] + 1:]:
+        outer *= s
+    return outer, nfeat, total // (nfeat * outer)
+
+
+def _f32vec(t, n, name):
+    if t is None or t.numel() == 0:
+        return None
+    if t.numel() != n:
+        raise ValueError("batchnorm: %s must have one element per feature" % name)
+    t = _dev(t, name)
+    return t if t.dtype == torch.float32 else t.float()
+
+
+def batchnorm(input, weight, bias, running_mean, running_var, axes, train, momentum, epsilon):
+    """AutogradExtension::batchnorm -> (output, saveMean, saveInvStd).
+
+    Train mode: batch statistics; running_mean/running_var (fp32, updated in
+    place) follow the rule documented at flhip_bn_fwd_train.  Inference: uses the
+    running statistics and returns (output, None, None)."""
+    x = _dev(input, "input")
+    outer, Cc, inner = bn_view(x.shape, axes)
+    d = capi.BnDesc(outer, Cc, inner, _dtype_tag(x))
+    g, b = _f32vec(weight, Cc, "weight"), _f32vec(bias, Cc, "bias")
+    y = torch.empty_like(x)
+    if not train:
+        if running_mean is None or running_var is None:
+            raise ValueError("batchnorm: inference needs running statistics")
+        rm, rv = _f32vec(running_mean, Cc, "runningMean"), _f32vec(running_var, Cc, "runningVar")
+        capi.check(capi.lib().flhip_bn_fwd_infer(C.byref(d), _ptr(x), _ptr(g), _ptr(b), _ptr(rm),
+                                                 _ptr(rv), float(epsilon), _ptr(y), _stream()))
+        return y, None, None
+    for t, name in ((running_mean, "runningMean"), (running_var, "runningVar")):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != Cc):
+            raise ValueError("batchnorm: %s must be fp32 with one element per feature" % name)
+    sm = torch.empty((Cc,), dtype=torch.float32, device=x.device)
+    si = torch.empty((Cc,), dtype=torch.float32, device=x.device)
+    nws = capi.lib().flhip_bn_workspace_bytes(C.byref(d))
+    ws = _ws(nws, x.device)
+    capi.check(capi.lib().flhip_bn_fwd_train(
+        C.byref(d), _ptr(x), _ptr(g), _ptr(b), _ptr(y), _ptr(sm), _ptr(si),
+        _ptr(_dev(running_mean, "runningMean")), _ptr(_dev(running_var, "runningVar")),
+        float(momentum), float(epsilon), _ptr(ws), nws, _stream()))
+    return y, sm, si
+
+
+def batchnorm_backward(grad_output, input, weight, save_mean, save_invstd, axes):
+    """AutogradExtension::batchnormBackward -> (gradInput, gradWeight, gradBias)."""
+    g, x = _dev(grad_output, "gradOutput"), _dev(input, "input")
+    if g.dtype != x.dtype or g.shape != x.shape:
+        raise ValueError("batchnormBackward: gradOutput must match the input")
+    if save_mean is None or save_invstd is None:
+        raise ValueError("batchnormBackward: needs the forward payload")
+    outer, Cc, inner = bn_view(x.shape, axes)
+    d = capi.BnDesc(outer, Cc, inner, _dtype_tag(x))
+    w = _f32vec(weight, Cc, "weight")
+    dx = torch.empty_like(x)
+    dg = torch.empty((Cc,), dtype=torch.float32, device=x.device)
+    db = torch.empty((Cc,), dtype=torch.float32, device=x.device)
+    nws = capi.lib().flhip_bn_workspace_bytes(C.byref(d))
+    ws = _ws(nws, x.device)
+    capi.check(capi.lib().flhip_bn_bwd(C.byref(d), _ptr(x), _ptr(g), _ptr(w), _ptr(save_mean),
+                                       _ptr(save_invstd), _ptr(dx), _ptr(dg), _ptr(db), _ptr(ws),
+                                       nws, _stream()))
+    return dx, dg, db

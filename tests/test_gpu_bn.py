@@ -1,0 +1,133 @@
+"""GPU parity: batchnorm / batchnormBackward through the C ABI against the CPU
+checker (fp32 relative L2 <= 1e-4; bf16 storage <= 2e-2)."""
+import numpy as np
+import pytest
+import torch
+
+import flashlight_amd as fa
+from gpu_util import bf16_round, dev, host
+from oracle import flref
+from refmath import rel_l2
+
+pytestmark = pytest.mark.gpu
+
+# (row-major shape N,C,H,W ; Flashlight feature axes)
+CASES = [
+    ((8, 3, 13, 13), [2]),          # AutogradNormalizationTest.cpp:158-189
+    ((8, 4, 13, 13), [0, 1, 2]),    # :191-226 per-activation
+    ((4, 16, 14, 14), [2]),         # inner % 4 == 0
+    ((2, 5, 3, 7), [1, 2]),         # features over (H,C)
+    ((1, 7, 5, 6), [0, 1, 2, 3]),   # LayerNorm-style: every element its own feature
+    ((16, 250, 1, 75), [2]),        # speech stack shape [T,1,250,B]
+    ((6, 300, 2, 2), [2]),          # many features, tiny inner
+    ((64, 10), [0]),                # 2-D, per-activation
+    ((3, 2, 56, 56), [2]),          # long rows
+]
+
+
+def _data(shape, axes, seed, dtype):
+    rng = np.random.default_rng(seed)
+    outer, C, inner = flref.bn_view(list(shape[::-1]), axes)
+    x = (rng.standard_normal(shape) * np.sqrt(2) + 0.5).astype(np.float32)
+    dy = rng.standard_normal(shape).astype(np.float32)
+    if dtype == torch.bfloat16:
+        x, dy = bf16_round(x), bf16_round(dy)
+    g = (1 + 0.1 * rng.standard_normal(C)).astype(np.float32)
+    b = rng.standard_normal(C).astype(np.float32)
+    return outer, C, inner, x, dy, g, b
+
+
+@pytest.mark.parametrize("shape,axes", CASES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_train_forward_backward(shape, axes, dtype):
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    outer, C, inner, x, dy, g, b = _data(shape, axes, 50, dtype)
+    y_ref, mean, var = flref.bn_fwd_train(outer, C, inner, x, g, b, 1e-5)
+    dx_ref, dg_ref, db_ref = flref.bn_bwd(outer, C, inner, x, dy, g, mean, var, 1e-5)
+    rm, rv = dev(np.zeros(C, np.float32)), dev(np.ones(C, np.float32))
+    xd, dyd = dev(x, dtype), dev(dy, dtype)
+    y, sm, si = fa.batchnorm(xd, dev(g), dev(b), rm, rv, axes, True, 0.1, 1e-5)
+    dx, dg, db = fa.batchnorm_backward(dyd, xd, dev(g), sm, si, axes)
+    assert rel_l2(host(y), y_ref) <= tol
+    assert np.allclose(host(sm), mean, rtol=1e-5, atol=1e-6)
+    assert np.allclose(host(si), 1 / np.sqrt(var.astype(np.float64) + 1e-5), rtol=1e-4)
+    rm_ref, rv_ref = flref.bn_running_update(outer * inner, mean, var, 0.1, np.zeros(C), np.ones(C))
+    assert np.allclose(host(rm), rm_ref, rtol=1e-5, atol=1e-6)
+    assert np.allclose(host(rv), rv_ref, rtol=1e-4, atol=1e-6)
+    assert rel_l2(host(dx), dx_ref) <= tol
+    # with bf16 storage the checker sees the same rounded inputs; parameter
+    # gradients are fp32 sums
+    assert rel_l2(host(dg), dg_ref) <= 1e-4 and rel_l2(host(db), db_ref) <= 1e-4
+
+
+def test_momentum_zero_overwrites_running_stats_like_onednn():
+    # onednn/BatchNorm.cpp:154-157
+    shape, axes = CASES[0]
+    outer, C, inner, x, _, g, b = _data(shape, axes, 51, torch.float32)
+    _, mean, var = flref.bn_fwd_train(outer, C, inner, x, g, b, 1e-5)
+    rm, rv = dev(np.full(C, 7, np.float32)), dev(np.full(C, 9, np.float32))
+    fa.batchnorm(dev(x), dev(g), dev(b), rm, rv, axes, True, 0.0, 1e-5)
+    assert np.allclose(host(rm), mean, rtol=1e-5, atol=1e-6)
+    assert np.allclose(host(rv), var, rtol=1e-4, atol=1e-6)
+
+
+def test_no_affine_and_no_running_stats():
+    shape, axes = CASES[2]
+    outer, C, inner, x, dy, _, _ = _data(shape, axes, 52, torch.float32)
+    y_ref, mean, var = flref.bn_fwd_train(outer, C, inner, x, None, None, 1e-5)
+    y, sm, si = fa.batchnorm(dev(x), None, None, None, None, axes, True, 0.0, 1e-5)
+    assert rel_l2(host(y), y_ref) <= 1e-4
+    dx_ref, _, _ = flref.bn_bwd(outer, C, inner, x, dy, None, mean, var, 1e-5)
+    dx, _, _ = fa.batchnorm_backward(dev(dy), dev(x), None, sm, si, axes)
+    assert rel_l2(host(dx), dx_ref) <= 1e-4
+
+
+@pytest.mark.parametrize("shape,axes", CASES[:3])
+def test_inference(shape, axes):
+    # AutogradNormalizationTest.cpp:37-156
+    outer, C, inner, x, _, g, b = _data(shape, axes, 53, torch.float32)
+    rng = np.random.default_rng(54)
+    rm, rv = rng.random(C).astype(np.float32), rng.random(C).astype(np.float32)
+    y_ref = flref.bn_fwd_infer(outer, C, inner, x, g, b, rm, rv, 1e-5)
+    y, sm, si = fa.batchnorm(dev(x), dev(g), dev(b), dev(rm), dev(rv), axes, False, 0.0, 1e-5)
+    assert sm is None and si is None
+    assert np.allclose(host(y), y_ref, atol=1e-5, rtol=1e-5)
+
+
+def test_large_mean_small_variance():
+    # a shifted-sum variance must survive mean >> std
+    rng = np.random.default_rng(55)
+    x = (1000.0 + 0.01 * rng.standard_normal((4, 8, 16, 16))).astype(np.float32)
+    y_ref, mean, var = flref.bn_fwd_train(4, 8, 256, x, None, None, 1e-5)
+    y, sm, si = fa.batchnorm(dev(x), None, None, None, None, [2], True, 0.0, 1e-5)
+    assert rel_l2(host(y), y_ref) <= 1e-3
+    assert np.allclose(host(sm), mean, rtol=1e-6)
+
+
+def test_errors():
+    x = torch.zeros((2, 3, 4, 4), device="cuda")
+    with pytest.raises(ValueError):
+        fa.batchnorm(x, None, None, None, None, [0, 2], True, 0.0, 1e-5)   # axes not contiguous
+    with pytest.raises(ValueError):
+        fa.batchnorm_backward(x, x, None, None, None, [2])                 # no payload
+    with pytest.raises(ValueError):
+        fa.batchnorm(x, torch.zeros(5, device="cuda"), None, None, None, [2], True, 0.0, 1e-5)
+
+
+def test_full_size_invariants():
+    # cfg-3 shape: per-feature sums of dx and of dx*xhat vanish; y has zero mean
+    # and unit variance per feature.
+    g = torch.Generator(device="cuda").manual_seed(56)
+    x = torch.randn((32, 256, 56, 56), device="cuda", generator=g) * (2 ** 0.5) + 0.5
+    dy = torch.randn((32, 256, 56, 56), device="cuda", generator=g)
+    gamma = 1 + 0.1 * torch.randn(256, device="cuda", generator=g)
+    y, sm, si = fa.batchnorm(x, gamma, None, None, None, [2], True, 0.1, 1e-5)
+    ym = y.double().mean(dim=(0, 2, 3)); yv = y.double().var(dim=(0, 2, 3), unbiased=False)
+    assert ym.abs().max().item() < 1e-4
+    assert torch.allclose(yv, gamma.double() ** 2, rtol=1e-3)
+    dx, dg, db = fa.batchnorm_backward(dy, x, gamma, sm, si, [2])
+    assert torch.allclose(db.double(), dy.double().sum(dim=(0, 2, 3)), rtol=1e-4, atol=1e-2)
+    s = dx.double().sum(dim=(0, 2, 3)).abs().max().item()
+    assert s < 1e-1, s     # 1e5 elements per feature of magnitude ~1
+    xh = (x.double() - sm.double().view(1, -1, 1, 1)) * si.double().view(1, -1, 1, 1)
+    assert (dx.double() * xh).sum(dim=(0, 2, 3)).abs().max().item() < 1.0

@@ -1,0 +1,115 @@
+"""GPU parity: conv2d / conv2dBackwardData / conv2dBackwardFilterBias through the
+C ABI against the CPU checker.  Tolerances: fp32 relative L2 <= 1e-4, bf16
+storage with fp32 accumulate <= 2e-2 against the fp32 checker on the same
+bf16-rounded inputs."""
+import numpy as np
+import pytest
+import torch
+
+import flashlight_amd as fa
+from gpu_util import bf16_round, dev, host
+from oracle import flref
+from refmath import rel_l2
+from test_oracle_conv import CASES, LIB_CASES
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL, BF16_TOL = 1e-4, 2e-2
+
+MORE = [
+    ((2, 64, 14, 14), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),      # ResNet 3x3
+    ((2, 3, 32, 32), (16, 3, 7, 7), (2, 2), (3, 3), (1, 1), 1),         # stem 7x7 s2
+    ((2, 32, 14, 14), (48, 32, 1, 1), (1, 1), (0, 0), (1, 1), 1),       # 1x1
+    ((2, 32, 14, 14), (48, 32, 1, 1), (2, 2), (0, 0), (1, 1), 1),       # 1x1 s2 downsample
+    ((2, 16, 15, 15), (32, 16, 3, 3), (2, 2), (1, 1), (1, 1), 1),       # 3x3 s2
+    ((2, 1, 28, 28), (32, 1, 5, 5), (1, 1), (2, 2), (1, 1), 1),         # MNIST conv1
+    ((2, 80, 1, 100), (250, 80, 1, 21), (1, 1), (0, 10), (1, 1), 1),    # speech 21x1
+    ((2, 80, 1, 100), (250, 80, 1, 21), (1, 2), (0, 10), (1, 1), 1),    # speech stride 2
+    ((3, 30, 17, 20), (50, 30, 7, 9), (3, 2), (2, 3), (1, 1), 1),       # ModuleTest.cpp:338-353
+    ((1, 130, 9, 9), (70, 130, 3, 3), (1, 1), (1, 1), (1, 1), 1),       # ragged channel counts
+    ((2, 8, 6, 500), (8, 4, 3, 3), (1, 1), (1, 1), (1, 1), 2),          # wide rows, groups
+]
+ALL = LIB_CASES + MORE
+
+
+def _run(case, seed, dtype):
+    xs, ws, st, pd, dl, g = case
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal(xs).astype(np.float32)
+    w = (rng.standard_normal(ws) / np.sqrt(ws[1] * ws[2] * ws[3])).astype(np.float32)
+    b = rng.uniform(-1, 1, ws[0]).astype(np.float32)
+    if dtype == torch.bfloat16:
+        x, w = bf16_round(x), bf16_round(w)
+    d = flref.conv_desc(xs, ws, st, pd, dl, g)
+    y_ref = flref.conv2d_fwd(d, x, w, b)
+    dy = rng.standard_normal(y_ref.shape).astype(np.float32)
+    if dtype == torch.bfloat16:
+        dy = bf16_round(dy)
+    dx_ref = flref.conv2d_bwd_data(d, dy, w)
+    dw_ref, db_ref = flref.conv2d_bwd_filter(d, x, dy)
+    kw = dict(sx=st[1], sy=st[0], px=pd[1], py=pd[0], dx=dl[1], dy=dl[0], groups=g)
+    xd, wd, bd, dyd = dev(x, dtype), dev(w, dtype), dev(b), dev(dy, dtype)
+    y = fa.conv2d(xd, wd, bd, **kw)
+    dxg = fa.conv2d_backward_data(dyd, xs, wd, **kw)
+    dw, db = fa.conv2d_backward_filter_bias(dyd, xd, ws, True, **kw)
+    y_nb = fa.conv2d(xd, wd, None, **kw)
+    torch.cuda.synchronize()
+    return dict(y=(host(y), y_ref), dx=(host(dxg), dx_ref), dw=(host(dw), dw_ref),
+                db=(host(db), db_ref),
+                y_nobias=(host(y_nb), y_ref - b.reshape(1, -1, 1, 1)))
+
+
+@pytest.mark.parametrize("case", ALL)
+def test_conv_f32(case):
+    for name, (got, ref) in _run(case, 30, torch.float32).items():
+        assert got.shape == ref.shape, name
+        assert rel_l2(got, ref) <= F32_TOL, (name, rel_l2(got, ref))
+
+
+@pytest.mark.parametrize("case", ALL)
+def test_conv_bf16(case):
+    for name, (got, ref) in _run(case, 31, torch.bfloat16).items():
+        assert rel_l2(got, ref) <= BF16_TOL, (name, rel_l2(got, ref))
+
+
+def test_bias_gradient_alone_and_empty_bias():
+    # the caller passes an empty bias when its gradient is not needed
+    # (flashlight/fl/autograd/Functions.cpp:1391-1395)
+    case = ALL[0]
+    xs, ws, st, pd, dl, g = case
+    rng = np.random.default_rng(32)
+    x = rng.standard_normal(xs).astype(np.float32)
+    d = flref.conv_desc(xs, ws, st, pd, dl, g)
+    oh, ow = flref.conv_out(d)
+    dy = rng.standard_normal((xs[0], ws[0], oh, ow)).astype(np.float32)
+    kw = dict(sx=st[1], sy=st[0], px=pd[1], py=pd[0], dx=dl[1], dy=dl[0], groups=g)
+    dw, db = fa.conv2d_backward_filter_bias(dev(dy), dev(x), ws, False, **kw)
+    assert db is None
+    dw_ref, _ = flref.conv2d_bwd_filter(d, x, dy, want_bias=False)
+    assert rel_l2(host(dw), dw_ref) <= F32_TOL
+
+
+def test_batching_invariance_on_device():
+    # flashlight/fl/test/nn/ModuleTest.cpp:338-353 (tolerance 1e-5 there)
+    rng = np.random.default_rng(33)
+    x = rng.standard_normal((4, 30, 17, 20)).astype(np.float32)
+    w = (rng.standard_normal((50, 30, 7, 9)) / 40).astype(np.float32)
+    b = rng.standard_normal(50).astype(np.float32)
+    kw = dict(sx=2, sy=3, px=3, py=2)
+    y = host(fa.conv2d(dev(x), dev(w), dev(b), **kw))
+    for n in range(4):
+        y1 = host(fa.conv2d(dev(x[n:n + 1]), dev(w), dev(b), **kw))
+        assert np.allclose(y1[0], y[n], atol=1e-5, rtol=0)
+
+
+def test_invalid_arguments_raise():
+    x = torch.zeros((1, 4, 8, 8), device="cuda")
+    w = torch.zeros((4, 3, 3, 3), device="cuda")
+    with pytest.raises(ValueError):
+        fa.conv2d(x, w, None)                       # channel mismatch
+    with pytest.raises(ValueError):
+        fa.conv2d(x, torch.zeros((4, 4, 3, 3), device="cuda", dtype=torch.bfloat16), None)
+    with pytest.raises(ValueError):
+        fa.conv2d(x, torch.zeros((4, 4, 9, 9), device="cuda"), None)   # kernel > input
+    with pytest.raises(RuntimeError):
+        fa.conv2d(x.double(), torch.zeros((4, 4, 3, 3), device="cuda").double(), None)

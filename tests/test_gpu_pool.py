@@ -1,0 +1,102 @@
+"""GPU parity: pool2d / pool2dBackward through the C ABI against the CPU
+checker.  fp32 results, argmax bytes and gradients are compared bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+import flashlight_amd as fa
+from gpu_util import bf16_round, dev, host
+from oracle import flref
+from test_oracle_pool import GEOMS
+
+pytestmark = pytest.mark.gpu
+
+MORE = [
+    ((2, 5, 112, 112), (3, 3), (2, 2), (1, 1)),   # ResNet stem pool (W % 4 == 0)
+    ((3, 4, 28, 28), (2, 2), (2, 2), (0, 0)),     # MNIST pools
+    ((2, 3, 14, 14), (2, 2), (2, 2), (0, 0)),
+    ((2, 3, 9, 7), (7, 9), (1, 1), (3, 4)),       # ModuleTest.cpp:398-413: 9x7 SAME stride 1
+    ((1, 2, 30, 50), (3, 3), (2, 2), (1, 1)),     # W % 4 != 0
+    ((1, 3, 33, 36), (3, 3), (2, 2), (1, 1)),     # odd height
+    ((2, 6, 7, 7), (7, 7), (1, 1), (0, 0)),
+    ((1, 2, 1, 40), (1, 4), (1, 3), (0, 1)),      # 1-D
+]
+ALL = GEOMS + MORE
+
+
+def _x(shape, seed):
+    return (np.round(np.random.default_rng(seed).standard_normal(shape) * 8) / 8).astype(np.float32)
+
+
+@pytest.mark.parametrize("geom", ALL)
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_pool_f32_bit_exact(geom, mode):
+    xs, win, st, pd = geom
+    x = _x(xs, 40)
+    d = flref.pool_desc(xs, win, st, pd, mode)
+    y_ref, am_ref = flref.pool2d_fwd(d, x)
+    dy = np.random.default_rng(41).standard_normal(y_ref.shape).astype(np.float32)
+    dx_ref = flref.pool2d_bwd(d, dy, am_ref)
+    args = (win[1], win[0], st[1], st[0], pd[1], pd[0])
+    y, am = fa.pool2d(dev(x), *args, mode=mode, train=True)
+    dx = fa.pool2d_backward(dev(dy), xs, am, *args, mode=mode)
+    assert np.array_equal(host(y), y_ref)
+    if mode == 0:
+        assert am.dtype == torch.uint8 and np.array_equal(am.cpu().numpy(), am_ref)
+    else:
+        assert am is None
+    assert np.array_equal(host(dx), dx_ref)
+    # inference (no payload): same values, no argmax
+    y2, am2 = fa.pool2d(dev(x), *args, mode=mode, train=False)
+    assert am2 is None and np.array_equal(host(y2), y_ref)
+
+
+@pytest.mark.parametrize("geom", [ALL[0], MORE[0], MORE[1]])
+@pytest.mark.parametrize("mode", [0, 2])
+def test_pool_bf16(geom, mode):
+    xs, win, st, pd = geom
+    x = bf16_round(_x(xs, 42))
+    d = flref.pool_desc(xs, win, st, pd, mode)
+    y_ref, am_ref = flref.pool2d_fwd(d, x)
+    dy = bf16_round(np.random.default_rng(43).standard_normal(y_ref.shape))
+    dx_ref = flref.pool2d_bwd(d, dy, am_ref)
+    args = (win[1], win[0], st[1], st[0], pd[1], pd[0])
+    y, am = fa.pool2d(dev(x, torch.bfloat16), *args, mode=mode)
+    dx = fa.pool2d_backward(dev(dy, torch.bfloat16), xs, am, *args, mode=mode)
+    if mode == 0:   # selection only: exact
+        assert np.array_equal(host(y), y_ref) and np.array_equal(am.cpu().numpy(), am_ref)
+    else:
+        assert np.allclose(host(y), y_ref, rtol=1e-2, atol=1e-2)
+    assert np.allclose(host(dx), dx_ref, rtol=1e-2, atol=1e-2)
+
+
+def test_missing_trailing_dims_count_as_one():
+    # onednn/Pool2D.cpp:95-98: a [W,H] tensor pools as [W,H,1,1]
+    x = _x((6, 8), 44)
+    y, _ = fa.pool2d(dev(x), 2, 2, 2, 2, 0, 0)
+    d = flref.pool_desc((1, 1, 6, 8), (2, 2), (2, 2), (0, 0), 0)
+    assert np.array_equal(host(y)[0, 0], flref.pool2d_fwd(d, x)[0][0, 0])
+
+
+def test_backward_without_payload_raises():
+    dy = torch.zeros((1, 1, 4, 4), device="cuda")
+    with pytest.raises(ValueError):
+        fa.pool2d_backward(dy, (1, 1, 8, 8), None, 2, 2, 2, 2, 0, 0, mode=0)
+
+
+def test_full_size_properties():
+    # cfg-3 size: gradient mass is conserved and idempotence of max over its
+    # own output positions; sizes the CPU checker would take too long on are
+    # covered by these size-independent properties.
+    g = torch.Generator(device="cuda").manual_seed(45)
+    x = torch.round(torch.randn((32, 64, 112, 112), device="cuda", generator=g) * 8) / 8
+    dy = torch.randn((32, 64, 56, 56), device="cuda", generator=g)
+    for mode in (0, 2):
+        y, am = fa.pool2d(x, 3, 3, 2, 2, 1, 1, mode=mode)
+        dx = fa.pool2d_backward(dy, x.shape, am, 3, 3, 2, 2, 1, 1, mode=mode)
+        assert abs(dx.double().sum().item() - dy.double().sum().item()) < 1e-2
+        if mode == 0:
+            # routing dy = y through the argmax and reading x there returns y
+            probe = fa.pool2d_backward(torch.ones_like(y), x.shape, am, 3, 3, 2, 2, 1, 1, mode=0)
+            assert probe.sum().item() == y.numel()
+            assert (x[probe > 0].max() == y.max()).item()
