@@ -54,10 +54,12 @@ def test_train_forward_backward(shape, axes, dtype):
     rm_ref, rv_ref = flref.bn_running_update(outer * inner, mean, var, 0.1, np.zeros(C), np.ones(C))
     assert np.allclose(host(rm), rm_ref, rtol=1e-5, atol=1e-6)
     assert np.allclose(host(rv), rv_ref, rtol=1e-4, atol=1e-6)
-    assert rel_l2(host(dx), dx_ref) <= tol
+    # (a feature with a single sample has dx == 0 exactly: absolute check there)
+    assert rel_l2(host(dx), dx_ref) <= tol or np.abs(host(dx) - dx_ref).max() <= 1e-4
     # with bf16 storage the checker sees the same rounded inputs; parameter
     # gradients are fp32 sums
-    assert rel_l2(host(dg), dg_ref) <= 1e-4 and rel_l2(host(db), db_ref) <= 1e-4
+    assert rel_l2(host(dg), dg_ref) <= 1e-4 or np.abs(host(dg) - dg_ref).max() <= 1e-4
+    assert rel_l2(host(db), db_ref) <= 1e-4
 
 
 def test_momentum_zero_overwrites_running_stats_like_onednn():
@@ -100,8 +102,10 @@ def test_large_mean_small_variance():
     x = (1000.0 + 0.01 * rng.standard_normal((4, 8, 16, 16))).astype(np.float32)
     y_ref, mean, var = flref.bn_fwd_train(4, 8, 256, x, None, None, 1e-5)
     y, sm, si = fa.batchnorm(dev(x), None, None, None, None, [2], True, 0.0, 1e-5)
-    assert rel_l2(host(y), y_ref) <= 1e-3
+    # the fp32 mean itself is only known to 6e-5 here (ulp of 1000), 0.6% of the std
+    assert rel_l2(host(y), y_ref) <= 1e-2
     assert np.allclose(host(sm), mean, rtol=1e-6)
+    assert np.allclose(host(si), 1 / np.sqrt(var.astype(np.float64) + 1e-5), rtol=1e-3)
 
 
 def test_errors():
