@@ -1,0 +1,299 @@
+#!/usr/bin/env python3
+"""Benchmark of the AutogradExtension hot path on one MI355X.
+
+A step is one conv2dBackwardData + conv2dBackwardFilterBias at the ResNet-50
+stage-2 3x3 shape (input 56x56x64, batch 32, 64 filters, stride 1, pad 1); the
+headline value is the pair's TFLOP/s over exactly --steps steps.  The
+bandwidth-bound half of the metric (batchnormBackward at 56x56x256x32,
+pool2dBackward max/avg 3x3 s2 p1 at 112x112x64x32) is timed the same way in
+its own loops and reported in `ops`, with buffer sets rotated so that no call
+finds its operands in the 256 MB memory-side cache.
+
+All inputs are resident in HBM before any timed region starts.  Timing uses HIP
+events on the stream the kernels are launched on (torch's current stream, whose
+handle is passed through the C ABI).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK = {"hbm_GBps": 8000.0, "f32_TFLOPs": 157.3, "bf16_TFLOPs": 2500.0}
+CONV_FLOP = 2 * 32 * 64 * 56 * 56 * 64 * 9          # one pass, 7.398752256e9
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by
+# the same counters on the library's copy kernel (see profiles/); None = not measured.
+MEASURED_TRAFFIC = {"conv2d_bwd_data_f32": None}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--dtype", choices=["f32", "bf16"], default="f32")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--only", default="", help="comma list of ops to time (debugging/profiling)")
+    return ap.parse_args()
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        sys.stderr.write("bench.py: this build runs on one GPU; --gpus %d is not supported "
+                         "(no collectives or sharding are part of it)\n" % a.gpus)
+        return 2
+    import torch
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py: no GPU visible\n")
+        return 1
+    import flashlight_amd as fa
+    fa.capi.lib()                      # fails loudly when the HIP library is missing
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    tdt = torch.float32 if a.dtype == "f32" else torch.bfloat16
+    gen = torch.Generator(device=dev).manual_seed(0)
+
+    def randn(*shape, scale=1.0, shift=0.0):
+        return torch.randn(shape, device=dev, generator=gen) * scale + shift
+
+    def timed(fn, steps, warmup):
+        """Average seconds per call over exactly `steps` calls."""
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for i in range(steps):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        return e0.elapsed_time(e1) * 1e-3 / steps, wall / steps
+
+    only = set(x for x in a.only.split(",") if x)
+    want = lambda name: not only or name in only
+    ops = []
+
+    # The timed loops call the C ABI directly on preallocated outputs and
+    # workspaces (a few microseconds of host time per call), so the GPU never
+    # waits for Python.
+    import ctypes as C
+    from flashlight_amd import capi
+    L = capi.lib()
+    S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: C.c_void_p(t.data_ptr())
+
+    def checked(fn):
+        """Runs fn once and raises on a non-zero status; returns fn."""
+        capi.check(fn(0))
+        return fn
+
+    # ---- conv pair at cfg 2 --------------------------------------------------
+    tag = capi.F32 if a.dtype == "f32" else capi.BF16
+    x = randn(32, 64, 56, 56).to(tdt)
+    w = randn(64, 64, 3, 3, scale=1.0 / 24.0).to(tdt)          # Kaiming normal, fan-in 576
+    b = randn(64)
+    dy = randn(32, 64, 56, 56).to(tdt)
+    y, dx = torch.empty_like(x), torch.empty_like(x)
+    dw = torch.empty((64, 64, 3, 3), device=dev)
+    db = torch.empty(64, device=dev)
+    cd = capi.ConvDesc(32, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, tag)
+    nws = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_BWD_FILTER)
+    ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=dev)
+    peak_mfma = PEAK["f32_TFLOPs"] if a.dtype == "f32" else PEAK["bf16_TFLOPs"]
+    cdp, xp, wp, bp, dyp, yp, dxp, dwp, dbp, wsp = (C.byref(cd), P(x), P(w), P(b), P(dy), P(y),
+                                                     P(dx), P(dw), P(db), P(ws))
+    f_fwd = checked(lambda _: L.flhip_conv2d_fwd(cdp, xp, wp, bp, yp, None, 0, S))
+    f_bwd_data = checked(lambda _: L.flhip_conv2d_bwd_data(cdp, dyp, wp, dxp, None, 0, S))
+    f_bwd_filter = checked(lambda _: L.flhip_conv2d_bwd_filter(cdp, xp, dyp, dwp, dbp, wsp, nws, S))
+
+    def conv_pair(i):
+        f_bwd_data(i)
+        f_bwd_filter(i)
+
+    pair_s = pair_wall = None
+    if want("conv_pair"):
+        pair_s, pair_wall = timed(conv_pair, a.steps, a.warmup)
+    for name, fn in (("conv2d_fwd", f_fwd), ("conv2d_bwd_data", f_bwd_data),
+                     ("conv2d_bwd_filter_bias", f_bwd_filter)):
+        if not want(name):
+            continue
+        s, _ = timed(fn, a.steps, a.warmup)
+        ach = CONV_FLOP / s / 1e12
+        ops.append({"op": name, "workload": "32x64x56x56, 64 filters 3x3 s1 p1", "dtype": a.dtype,
+                    "us": s * 1e6, "bound": "mfma", "achieved": ach, "peak": peak_mfma,
+                    "unit": "TFLOP/s", "frac": ach / peak_mfma})
+    del x, w, dy, y, dx, ws
+
+    # ---- bandwidth ops at cfg 3 (fp32) ----------------------------------------
+    def bw_op(name, workload, nbytes, fn, nsets):
+        if not want(name):
+            return
+        checked(fn)
+        s, _ = timed(fn, a.steps, a.warmup)
+        ach = nbytes / s / 1e9
+        ops.append({"op": name, "workload": workload, "dtype": "f32", "us": s * 1e6,
+                    "bound": "hbm", "achieved": ach, "peak": PEAK["hbm_GBps"], "unit": "GB/s",
+                    "frac": ach / PEAK["hbm_GBps"], "algorithmic_bytes": nbytes,
+                    "buffer_sets_rotated": nsets})
+
+    if want("batchnorm_bwd") or want("batchnorm_fwd_train"):
+        nsets = 2
+        bx = [randn(32, 256, 56, 56, scale=2 ** 0.5, shift=0.5) for _ in range(nsets)]
+        bdy = [randn(32, 256, 56, 56) for _ in range(nsets)]
+        bout = torch.empty_like(bx[0])
+        gamma = randn(256, scale=0.1, shift=1.0)
+        beta = torch.zeros(256, device=dev)
+        rm, rv = torch.zeros(256, device=dev), torch.ones(256, device=dev)
+        dg, dbt = torch.empty(256, device=dev), torch.empty(256, device=dev)
+        T = bx[0].numel() * 4
+        bd = capi.BnDesc(32, 256, 56 * 56, capi.F32)
+        bnws = L.flhip_bn_workspace_bytes(C.byref(bd))
+        bws = torch.empty(max(bnws, 16), dtype=torch.uint8, device=dev)
+        sm = [torch.empty(256, device=dev) for _ in range(nsets)]
+        si = [torch.empty(256, device=dev) for _ in range(nsets)]
+        bdp, boutp, bwsp = C.byref(bd), P(bout), P(bws)
+        bxp, bdyp = [P(t) for t in bx], [P(t) for t in bdy]
+        smp, sip = [P(t) for t in sm], [P(t) for t in si]
+        gp, btp, rmp, rvp, dgp, dbtp = P(gamma), P(beta), P(rm), P(rv), P(dg), P(dbt)
+        f_bn_fwd = lambda i: L.flhip_bn_fwd_train(bdp, bxp[i % nsets], gp, btp, boutp,
+                                                  smp[i % nsets], sip[i % nsets], rmp, rvp,
+                                                  0.1, 1e-5, bwsp, bnws, S)
+        for i in range(nsets):
+            capi.check(f_bn_fwd(i))
+        bw_op("batchnorm_fwd_train", "56x56x256x32, axes {2}", 2 * T, f_bn_fwd, nsets)
+        bw_op("batchnorm_bwd", "56x56x256x32, axes {2}", 3 * T,
+              lambda i: L.flhip_bn_bwd(bdp, bxp[i % nsets], bdyp[i % nsets], gp, smp[i % nsets],
+                                       sip[i % nsets], boutp, dgp, dbtp, bwsp, bnws, S), nsets)
+        del bx, bdy, bout
+
+    if any(want(n) for n in ("pool2d_max_fwd", "pool2d_max_bwd", "pool2d_avg_fwd", "pool2d_avg_bwd")):
+        nsets = 3
+        px_ = [torch.round(randn(32, 64, 112, 112) * 8) / 8 for _ in range(nsets)]
+        pdy = [randn(32, 64, 56, 56) for _ in range(nsets)]
+        pam = [torch.empty((32, 64, 56, 56), dtype=torch.uint8, device=dev) for _ in range(nsets)]
+        pyo = torch.empty((32, 64, 56, 56), device=dev)
+        pdx = torch.empty((32, 64, 112, 112), device=dev)
+        pdm = capi.PoolDesc(32, 64, 112, 112, 3, 3, 2, 2, 1, 1, 0, capi.F32)
+        pda = capi.PoolDesc(32, 64, 112, 112, 3, 3, 2, 2, 1, 1, 2, capi.F32)
+        pdmp, pdap, pyop, pdxp = C.byref(pdm), C.byref(pda), P(pyo), P(pdx)
+        pxp, pdyp, pamp = [P(t) for t in px_], [P(t) for t in pdy], [P(t) for t in pam]
+        f_max_fwd = lambda i: L.flhip_pool2d_fwd(pdmp, pxp[i % nsets], pyop, pamp[i % nsets], S)
+        for i in range(nsets):
+            capi.check(f_max_fwd(i))
+        nx, ny = px_[0].numel() * 4, pdy[0].numel() * 4
+        wl = "112x112x64x32, 3x3 s2 p1"
+        bw_op("pool2d_max_fwd", wl, nx + ny + ny // 4, f_max_fwd, nsets)
+        bw_op("pool2d_max_bwd", wl, nx + ny + ny // 4,
+              lambda i: L.flhip_pool2d_bwd(pdmp, pdyp[i % nsets], pamp[i % nsets], pdxp, S), nsets)
+        bw_op("pool2d_avg_fwd", wl, nx + ny,
+              lambda i: L.flhip_pool2d_fwd(pdap, pxp[i % nsets], pyop, None, S), nsets)
+        bw_op("pool2d_avg_bwd", wl, nx + ny,
+              lambda i: L.flhip_pool2d_bwd(pdap, pdyp[i % nsets], None, pdxp, S), nsets)
+        del px_, pdy, pam, pyo, pdx
+
+    torch.cuda.synchronize()
+    by = {o["op"]: o for o in ops}
+
+    # ---- CPU baselines (rank 0, bounded sample) --------------------------------
+    cpu_baseline = cpu_onednn = None
+    if not a.no_cpu and not only:
+        cpu_baseline, cpu_onednn = cpu_legs()
+
+    out = {
+        "metric": "TFLOP/s conv2dBackwardData+Filter (ResNet-50 3x3) + GB/s BN/pool backward, 1 GPU",
+        "value": (2 * CONV_FLOP / pair_s / 1e12) if pair_s else None,
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": pair_s * 1e3 if pair_s else None,
+        "wall_ms_per_step": pair_wall * 1e3 if pair_wall else None,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": a.dtype, "data": "synthetic",
+        "config": {"workload": "configs[1]: conv2dBackwardData + conv2dBackwardFilterBias, input "
+                               "56x56x64 batch 32, 64 filters 3x3 stride 1 pad 1, bias on"},
+        "bn_bwd_GBps": by.get("batchnorm_bwd", {}).get("achieved"),
+        "pool_max_bwd_GBps": by.get("pool2d_max_bwd", {}).get("achieved"),
+        "pool_avg_bwd_GBps": by.get("pool2d_avg_bwd", {}).get("achieved"),
+    }
+    if "conv2d_bwd_data" in by:
+        o = by["conv2d_bwd_data"]
+        out["roofline"] = {
+            "kernel": "gather_conv_kernel (conv2dBackwardData, one launch per call)",
+            "bound": "mfma", "achieved": o["achieved"], "peak": o["peak"], "unit": "TFLOP/s",
+            "frac": o["frac"], "avg_launch_us": o["us"],
+            "traffic": MEASURED_TRAFFIC.get("conv2d_bwd_data_" + a.dtype)}
+    out["ops"] = ops
+    out["cpu_baseline"] = cpu_baseline
+    out["cpu_onednn"] = cpu_onednn
+    print(json.dumps(out))
+    return 0
+
+
+def cpu_legs():
+    """(1) the C restatement in oracle/ on a bounded sample of the conv pair;
+    (2) the same oneDNN primitives the reference requests, reached through
+    PyTorch-CPU, on the full batch.  Both on this host's cores."""
+    import numpy as np
+    import torch
+    from oracle import flref
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+    rng = np.random.default_rng(0)
+    nb = 32                                             # the full batch
+    x = rng.standard_normal((nb, 64, 56, 56)).astype(np.float32)
+    w = (rng.standard_normal((64, 64, 3, 3)) / 24).astype(np.float32)
+    dy = rng.standard_normal((nb, 64, 56, 56)).astype(np.float32)
+    d = flref.conv_desc(x.shape, w.shape, (1, 1), (1, 1))
+    flref.conv2d_bwd_data(d, dy[:1], w)                 # warm-up (thread pool, page faults)
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        flref.conv2d_bwd_data(d, dy, w)
+        flref.conv2d_bwd_filter(d, x, dy)
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > 12.0:
+            break
+    flop = 2 * CONV_FLOP * nb / 32 * reps
+    port = {"value": flop / el / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": "%d repetitions of the pair on the full batch of %d, oracle/flref.c with "
+                      "OpenMP, %.1f s" % (reps, nb, el)}
+
+    torch.set_num_threads(threads)
+    xt = torch.from_numpy(rng.standard_normal((32, 64, 56, 56)).astype(np.float32))
+    wt = torch.from_numpy(w)
+    dyt = torch.from_numpy(rng.standard_normal((32, 64, 56, 56)).astype(np.float32))
+    conv_bw = torch.ops.aten.convolution_backward
+
+    def pair():
+        conv_bw(dyt, xt, wt, [64], [1, 1], [1, 1], [1, 1], False, [0, 0], 1, [True, False, False])
+        conv_bw(dyt, xt, wt, [64], [1, 1], [1, 1], [1, 1], False, [0, 0], 1, [False, True, True])
+
+    for _ in range(3):
+        pair()
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        pair()
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > 8.0:
+            break
+    onednn = {"value": 2 * CONV_FLOP * reps / el / 1e12, "unit": "TFLOP/s", "cores": threads,
+              "kind": "oneDNN %s via PyTorch-CPU aten::convolution_backward (the primitives the "
+                      "reference's oneDNN extension requests), full batch 32" % _onednn_version(),
+              "sample": "%d repetitions, %.1f s" % (reps, el)}
+    return port, onednn
+
+
+def _onednn_version():
+    import re
+    import torch
+    m = re.search(r"MKL-DNN (v[0-9.]+)", torch.__config__.show())
+    return m.group(1) if m else "?"
+
+
+if __name__ == "__main__":
+    sys.exit(main())
