@@ -11,7 +11,7 @@ LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "_obj")
 LIB = os.path.join(LIBDIR, "libflhip.so")
 
-SOURCES = ["api.hip", "pool2d.hip", "batchnorm.hip", "conv2d.hip", "conv2d_mfma.hip"]
+SOURCES = ["api.hip", "pool2d.hip", "batchnorm.hip", "conv2d.hip", "conv2d_mfma_gather.hip", "conv2d_mfma_wgrad.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

@@ -72,6 +72,19 @@ __device__ __forceinline__ void st4(bf16_t* p, size_t i, float4 v) {
   *reinterpret_cast<uint2*>(p + i) = r;
 }
 
+// ---- buffer loads ------------------------------------------------------------
+// Raw buffer descriptor over `bytes` bytes at p: loads at a byte offset at or
+// past `bytes` return zero, which is how the gathers fetch padding.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ float buf_ld(__amdgpu_buffer_rsrc_t r, int byte_off, const float*) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, 0));
+}
+__device__ __forceinline__ float buf_ld(__amdgpu_buffer_rsrc_t r, int byte_off, const bf16_t*) {
+  return bf16_to_f32((bf16_t)__builtin_amdgcn_raw_buffer_load_b16(r, byte_off, 0, 0));
+}
+
 // ---- reductions -----------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

@@ -1,0 +1,396 @@
+// Implicit-GEMM convolution on the gfx950 matrix cores: forward and
+// backward-data.
+//
+// Both are one "gather" kernel.  The result tensor D [N, DC, DH, DW] is a GEMM
+//   D[m, P] = sum_kk A[m, kk] * B[kk, P]
+//   m  = result channel inside its group,
+//   P  = flattened result position (n, h, w),
+//   kk = (source channel, kh, kw) in the weights' own memory order,
+//   A  = weights, read in place (no reordering pass),
+//   B  = source values gathered on the fly (im2col never exists in memory).
+// A workgroup of 4 waves owns a 64 x (16*NB) tile of D, two workgroups share a CU
+// (so that one computes while the other loads).  K is walked in chunks
+// of 16 rows through a double-buffered LDS tile: while the matrix cores work on
+// chunk c, every thread gathers its result position's 16 values of chunk c+1
+// into registers (coalesced along W, branch-free: out-of-image taps become
+// out-of-range buffer loads, which return zero), stores them to the other
+// buffer and meets the others at the single barrier of the iteration.  What a K
+// row means (channel offset, window shift) is decoded once per kernel into an
+// LDS table that is read 16 rows at a time, so the per-element cost is two adds,
+// a bounds test, a select and the load.
+// Waves are arranged 2 (M) x 2 (N); wave (wm, wn) owns 32 x (16*nt) of the tile
+// with nt = floor or ceil of NB/2, and the inner loop is compiled for each nt
+// so that it is straight-line code: all LDS fragments of a chunk are read up
+// front, then the chunk's MFMAs issue back to back.  NB is chosen per launch so
+// that the tile count fills 2 slots per CU with as little tail as possible
+// (NB = 13 for 32x64x56x56: 483 workgroups on 512 slots).
+//
+// v_mfma_f32_16x16x4_f32 operand layout (lane l of 64):
+//   A operand: A[i = l%16][k = l/16]     B operand: B[k = l/16][j = l%16]
+//   result   : D[i = 4*(l/16) + r][j = l%16], r = 0..3
+#include "conv2d_mfma.h"
+
+namespace flhip {
+
+static int g_num_cus = 0;
+int mfma_num_cus() {
+  if (g_num_cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      g_num_cus = n;
+    else
+      g_num_cus = 256;
+  }
+  return g_num_cus;
+}
+
+bool mfma_allow_lds(const void* func, size_t bytes) {
+  if (bytes <= 64 * 1024) return true;
+  if (bytes > 160 * 1024) return false;
+  return hipFuncSetAttribute(func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) ==
+         hipSuccess;
+}
+
+namespace {
+
+constexpr int KC = 16;        // K rows per chunk
+constexpr int BM = MFMA_BM;
+constexpr int APITCH = 80;    // LDS pitch of the A tile (== 16 mod 32 banks)
+constexpr int NT_MAX = 8;     // 16-wide position blocks per wave
+constexpr int NB_MAX = 2 * NT_MAX;
+constexpr int THREADS = 256;  // 4 waves
+constexpr int AROWS = BM * KC / THREADS;   // A elements per thread and chunk
+
+enum { MODE_FWD = 0, MODE_BWD_S1 = 1, MODE_BWD_GEN = 2 };
+
+struct GatherParams {
+  int N, SC, SH, SW, DC, DH, DW;  // source [N,SC,SH,SW], result [N,DC,DH,DW]
+  int KH, KW, KHW;
+  int sy, sx, py, px, dly, dlx;
+  int groups, SCg, DCg;
+  int Ktot;             // SCg*KH*KW
+  int nchunks;          // ceil(Ktot / KC)
+  int a_mstride;        // weight stride between result channels
+  int w_group_stride;   // weight stride between groups
+  int a_bwd_kstride;    // bwd: weight stride between source channels (Cg*KHW)
+  int q16, r16;         // KC = q16*KHW + r16
+  int NB;               // position blocks per workgroup
+  int BNP;              // LDS pitch of the B tile
+  int mtiles;
+  int Ptotal;           // N*DH*DW
+  int DHW, SHW;
+  unsigned src_bytes, wgt_bytes;
+};
+
+// K-row table in LDS: tabA[kk] = {byte offset contributed by the row (channel and
+// window shift), dh}, tabB[kk] = dw; dh = -2^20 marks a row past Ktot.
+constexpr int ROW_INVALID = -(1 << 20);
+
+template <typename T, int MODE>
+__global__ void __launch_bounds__(THREADS, 2)
+gather_conv_kernel(GatherParams p, const T* __restrict__ src, const T* __restrict__ wgt,
+                   const float* __restrict__ bias, T* __restrict__ dst) {
+  extern __shared__ float lds[];
+  const int bstride = KC * p.BNP, astride = KC * APITCH;
+  float* Bs = lds;                                   // [2][KC][BNP]
+  float* As = lds + 2 * bstride;                     // [2][KC][APITCH]
+  const int nrows = p.nchunks * KC;
+  int2* tabA = reinterpret_cast<int2*>(As + 2 * astride);   // [nrows]
+  int* tabB = reinterpret_cast<int*>(tabA + nrows);           // [nrows]
+  const int esz = (int)sizeof(T);
+  const __amdgpu_buffer_rsrc_t srsrc = make_rsrc(src, p.src_bytes);
+  const __amdgpu_buffer_rsrc_t wrsrc = make_rsrc(wgt, p.wgt_bytes);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave & 1, wn = wave >> 1;
+  const int grp = blockIdx.y / p.mtiles, mtile = blockIdx.y % p.mtiles;
+  const int BN = p.NB * 16;
+  const int tile_p0 = blockIdx.x * BN;
+
+  // this wave's share of the NB position blocks
+  const int base = p.NB >> 1, rem = p.NB & 1;
+  const int nt = base + (wn < rem ? 1 : 0);
+  const int nb0 = wn * base + min(wn, rem);
+
+  // ---- K-row table, once per kernel -------------------------------------------
+  for (int kk = tid; kk < nrows; kk += THREADS) {
+    int2 ra = make_int2(0, ROW_INVALID);
+    int rb = 0;
+    if (kk < p.Ktot) {
+      const int c = kk / p.KHW, t = kk - c * p.KHW;
+      const int kh = t / p.KW, kw = t - kh * p.KW;
+      const int dh = (MODE == MODE_FWD ? kh : -kh) * p.dly;
+      const int dw = (MODE == MODE_FWD ? kw : -kw) * p.dlx;
+      ra.x = (c * p.SHW + (MODE != MODE_BWD_GEN ? dh * p.SW + dw : 0)) * esz;
+      ra.y = dh;
+      rb = dw;
+    }
+    tabA[kk] = ra;
+    tabB[kk] = rb;
+  }
+
+  // ---- per-thread gather position (one result position per thread) ----------
+  const bool loader = tid < BN;
+  const int P = tile_p0 + tid;
+  const bool pvalid = loader && P < p.Ptotal;
+  int hb, wb, pixbase;
+  {
+    const int Pc = pvalid ? P : 0;
+    const int n = Pc / p.DHW, q = Pc - n * p.DHW;
+    const int h = q / p.DW, w = q - h * p.DW;
+    if (MODE == MODE_FWD) {
+      hb = h * p.sy - p.py;
+      wb = w * p.sx - p.px;
+    } else {
+      hb = h + p.py;
+      wb = w + p.px;
+    }
+    pixbase = (n * p.SC + grp * p.SCg) * p.SHW;
+    if (MODE != MODE_BWD_GEN) pixbase += hb * p.SW + wb;
+    pixbase *= esz;                                  // byte offset
+    if (!pvalid) hb = 4 * ROW_INVALID;               // every tap fails the bounds test
+  }
+
+  // ---- per-thread share of the A tile: row ar = tid%16, m = tid/16 + 16*i ------
+  const int ar = tid & 15, am = tid >> 4;
+  const int m_lim = p.DCg - mtile * BM;               // valid result channels in the tile
+  const int wbase = grp * p.w_group_stride + mtile * BM * p.a_mstride;   // elements
+  int a_kk = ar, a_c = 0, a_t = ar;                   // row of the chunk being loaded
+  if (MODE != MODE_FWD) {
+    a_c = ar / p.KHW;
+    a_t = ar - a_c * p.KHW;
+  }
+
+  float breg[KC];
+  float areg[AROWS];
+
+  auto load_chunk = [&](int chunk) {
+    // the 16 rows' table entries first (broadcast LDS reads, 12 instructions)
+    int goff[KC], dh[KC], dw[KC];
+    {
+      const int4* ta = reinterpret_cast<const int4*>(tabA + chunk * KC);
+      const int4* tb = reinterpret_cast<const int4*>(tabB + chunk * KC);
+#pragma unroll
+      for (int i = 0; i < KC / 2; ++i) {
+        const int4 v = ta[i];
+        goff[2 * i] = v.x; dh[2 * i] = v.y; goff[2 * i + 1] = v.z; dh[2 * i + 1] = v.w;
+      }
+#pragma unroll
+      for (int i = 0; i < KC / 4; ++i) {
+        const int4 v = tb[i];
+        dw[4 * i] = v.x; dw[4 * i + 1] = v.y; dw[4 * i + 2] = v.z; dw[4 * i + 3] = v.w;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < KC; ++r) {
+      bool ok;
+      int off;
+      if (MODE == MODE_BWD_GEN) {
+        const int th = hb + dh[r], tw = wb + dw[r];
+        const int ih = th / p.sy, iw = tw / p.sx;
+        ok = (th >= 0) & (tw >= 0) & (ih * p.sy == th) & (iw * p.sx == tw) & (ih < p.SH) &
+             (iw < p.SW);
+        off = pixbase + goff[r] + (ih * p.SW + iw) * esz;
+      } else {
+        const int ih = hb + dh[r], iw = wb + dw[r];
+        ok = ((unsigned)ih < (unsigned)p.SH) & ((unsigned)iw < (unsigned)p.SW);
+        off = pixbase + goff[r];
+      }
+      breg[r] = buf_ld(srsrc, ok ? off : -1, src);
+    }
+    const bool kok = a_kk < p.Ktot;
+    const int arow = wbase + (MODE == MODE_FWD ? a_kk : a_c * p.a_bwd_kstride + a_t);
+#pragma unroll
+    for (int i = 0; i < AROWS; ++i) {
+      const int m = am + 16 * i;
+      const bool ok = kok & (m < m_lim);
+      areg[i] = buf_ld(wrsrc, ok ? (m * p.a_mstride + arow) * esz : -1, wgt);
+    }
+    a_kk += KC;
+    if (MODE != MODE_FWD) {
+      a_c += p.q16;
+      a_t += p.r16;
+      if (a_t >= p.KHW) {
+        a_t -= p.KHW;
+        ++a_c;
+      }
+    }
+  };
+
+  auto store_chunk = [&](int buf) {
+    float* bs = Bs + buf * bstride;
+    float* as = As + buf * astride;
+    if (loader) {
+#pragma unroll
+      for (int r = 0; r < KC; ++r) bs[r * p.BNP + tid] = breg[r];
+    }
+#pragma unroll
+    for (int i = 0; i < AROWS; ++i) as[ar * APITCH + am + 16 * i] = areg[i];
+  };
+
+  __syncthreads();                                    // table visible
+  load_chunk(0);
+  store_chunk(0);
+  __syncthreads();
+
+  const int fr = lane & 15, fk = lane >> 4;
+
+  auto run = [&](auto ntc) {
+    constexpr int NT = decltype(ntc)::value;
+    floatx4 acc[2][NT];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    for (int c = 0; c < p.nchunks; ++c) {
+      const bool more = c + 1 < p.nchunks;
+      if (more) load_chunk(c + 1);
+      const float* as = As + (c & 1) * astride + wm * 32 + fr;
+      const float* bs = Bs + (c & 1) * bstride + nb0 * 16 + fr;
+      float a[KC / 4][2], b[KC / 4][NT];
+#pragma unroll
+      for (int ks = 0; ks < KC / 4; ++ks) {
+        const int krow = ks * 4 + fk;
+        a[ks][0] = as[krow * APITCH];
+        a[ks][1] = as[krow * APITCH + 16];
+#pragma unroll
+        for (int j = 0; j < NT; ++j) b[ks][j] = bs[krow * p.BNP + j * 16];
+      }
+#pragma unroll
+      for (int ks = 0; ks < KC / 4; ++ks) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[ks][0], b[ks][j], acc[0][j], 0, 0, 0);
+          acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[ks][1], b[ks][j], acc[1][j], 0, 0, 0);
+        }
+      }
+      if (more) store_chunk((c + 1) & 1);
+      __syncthreads();
+    }
+
+    // ---- epilogue: bias and store ---------------------------------------------
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int Pj = tile_p0 + (nb0 + j) * 16 + fr;
+      if (Pj < p.Ptotal) {
+        const int n = Pj / p.DHW, q = Pj - n * p.DHW;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int m = wm * 32 + i * 16 + fk * 4 + r;
+            if (m < m_lim) {
+              const int ch = grp * p.DCg + mtile * BM + m;
+              float v = acc[i][j][r];
+              if (bias) v += bias[ch];
+              st(dst, (size_t)(n * p.DC + ch) * p.DHW + q, v);
+            }
+          }
+        }
+      }
+    }
+  };
+
+  switch (nt) {
+    case 4: run(std::integral_constant<int, 4>{}); break;
+    case 5: run(std::integral_constant<int, 5>{}); break;
+    case 6: run(std::integral_constant<int, 6>{}); break;
+    case 7: run(std::integral_constant<int, 7>{}); break;
+    default: run(std::integral_constant<int, 8>{}); break;
+  }
+}
+
+// Chooses the number of 16-position blocks per workgroup so that the tile count
+// wastes as little of the last round over the CUs as possible.
+int choose_nb(long long pblocks, int mtiles_total, int slots) {
+  int best = 8;
+  double best_cost = 1e30;
+  for (int nb = 8; nb <= NB_MAX; ++nb) {
+    const long long tiles = ((pblocks + nb - 1) / nb) * mtiles_total;
+    const long long rounds = (tiles + slots - 1) / slots;
+    // time ~ rounds * nb (+ a small fixed cost per round for prologue/epilogue)
+    const double cost = (double)rounds * (nb + 1.0);
+    if (cost < best_cost - 1e-9 || (cost < best_cost + 1e-9 && nb > best)) {
+      best_cost = cost;
+      best = nb;
+    }
+  }
+  return best;
+}
+
+template <typename T, int MODE>
+int launch_gather(const GatherParams& p0, const void* src, const void* wgt, const float* bias,
+                  void* dst, hipStream_t s) {
+  GatherParams p = p0;
+  // byte offsets are 32-bit; rows past Ktot rely on |shift| < 2^20
+  const long long sbytes = (long long)p.N * p.SC * p.SHW * (long long)sizeof(T);
+  const long long wbytes = (long long)p.groups * p.w_group_stride * (long long)sizeof(T);
+  const int hmax = MODE == MODE_FWD ? p.DH * p.sy : p.DH + p.py;
+  if (sbytes >= (1ll << 31) || wbytes >= (1ll << 31) || hmax >= (1 << 19) ||
+      (p.KH - 1) * p.dly >= (1 << 19))
+    return -1;
+  p.src_bytes = (unsigned)sbytes;
+  p.wgt_bytes = (unsigned)wbytes;
+  p.nchunks = (p.Ktot + KC - 1) / KC;
+  p.q16 = KC / p.KHW;
+  p.r16 = KC % p.KHW;
+  const long long pblocks = ((long long)p.Ptotal + 15) / 16;
+  p.NB = choose_nb(pblocks, p.mtiles * p.groups, 2 * mfma_num_cus());
+  const int BN = p.NB * 16;
+  p.BNP = BN + ((16 - BN % 32) + 32) % 32;   // == 16 mod 32
+  const size_t shmem = (size_t)2 * (KC * p.BNP + KC * APITCH) * sizeof(float) +
+                       (size_t)p.nchunks * KC * 3 * sizeof(int);
+  auto kernel = gather_conv_kernel<T, MODE>;
+  if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
+  const dim3 grid((unsigned)((pblocks + p.NB - 1) / p.NB), (unsigned)(p.mtiles * p.groups));
+  hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const T*>(src),
+                     static_cast<const T*>(wgt), bias, static_cast<T*>(dst));
+  return check_launch("conv2d (mfma)");
+}
+
+}  // namespace
+
+int mfma_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w, const float* bias,
+                  void* y, hipStream_t s) {
+  GatherParams p{};
+  p.N = g.N; p.SC = g.C; p.SH = g.H; p.SW = g.W; p.DC = g.K; p.DH = g.OH; p.DW = g.OW;
+  p.KH = g.KH; p.KW = g.KW; p.KHW = g.KH * g.KW;
+  p.sy = g.sy; p.sx = g.sx; p.py = g.py; p.px = g.px; p.dly = g.dly; p.dlx = g.dlx;
+  p.groups = g.groups; p.SCg = g.Cg; p.DCg = g.Kg;
+  p.Ktot = g.Cg * p.KHW;
+  p.a_mstride = p.Ktot;
+  p.w_group_stride = g.Kg * p.Ktot;
+  p.a_bwd_kstride = 0;
+  p.mtiles = (g.Kg + BM - 1) / BM;
+  p.Ptotal = g.N * g.OH * g.OW;
+  p.DHW = g.OH * g.OW; p.SHW = g.H * g.W;
+  return dtype == FLHIP_F32 ? launch_gather<float, MODE_FWD>(p, x, w, bias, y, s)
+                            : launch_gather<bf16_t, MODE_FWD>(p, x, w, bias, y, s);
+}
+
+int mfma_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
+                       hipStream_t s) {
+  GatherParams p{};
+  p.N = g.N; p.SC = g.K; p.SH = g.OH; p.SW = g.OW; p.DC = g.C; p.DH = g.H; p.DW = g.W;
+  p.KH = g.KH; p.KW = g.KW; p.KHW = g.KH * g.KW;
+  p.sy = g.sy; p.sx = g.sx; p.py = g.py; p.px = g.px; p.dly = g.dly; p.dlx = g.dlx;
+  p.groups = g.groups; p.SCg = g.Kg; p.DCg = g.Cg;
+  p.Ktot = g.Kg * p.KHW;
+  p.a_mstride = p.KHW;
+  p.w_group_stride = g.Kg * g.Cg * p.KHW;
+  p.a_bwd_kstride = g.Cg * p.KHW;
+  p.mtiles = (g.Cg + BM - 1) / BM;
+  p.Ptotal = g.N * g.H * g.W;
+  p.DHW = g.H * g.W; p.SHW = g.OH * g.OW;
+  const bool s1 = g.sy == 1 && g.sx == 1;
+  if (dtype == FLHIP_F32)
+    return s1 ? launch_gather<float, MODE_BWD_S1>(p, dy, w, nullptr, dx, s)
+              : launch_gather<float, MODE_BWD_GEN>(p, dy, w, nullptr, dx, s);
+  return s1 ? launch_gather<bf16_t, MODE_BWD_S1>(p, dy, w, nullptr, dx, s)
+            : launch_gather<bf16_t, MODE_BWD_GEN>(p, dy, w, nullptr, dx, s);
+}
+
+}  // namespace flhip
