@@ -8,22 +8,24 @@
 //   kk = (source channel, kh, kw) in the weights' own memory order,
 //   A  = weights, read in place (no reordering pass),
 //   B  = source values gathered on the fly (im2col never exists in memory).
-// A workgroup of 4 waves owns a 64 x (16*NB) tile of D, two workgroups share a CU
-// (so that one computes while the other loads).  K is walked in chunks
-// of 16 rows through a double-buffered LDS tile: while the matrix cores work on
-// chunk c, every thread gathers its result position's 16 values of chunk c+1
-// into registers (coalesced along W, branch-free: out-of-image taps become
-// out-of-range buffer loads, which return zero), stores them to the other
-// buffer and meets the others at the single barrier of the iteration.  What a K
-// row means (channel offset, window shift) is decoded once per kernel into an
-// LDS table that is read 16 rows at a time, so the per-element cost is two adds,
-// a bounds test, a select and the load.
-// Waves are arranged 2 (M) x 2 (N); wave (wm, wn) owns 32 x (16*nt) of the tile
-// with nt = floor or ceil of NB/2, and the inner loop is compiled for each nt
-// so that it is straight-line code: all LDS fragments of a chunk are read up
-// front, then the chunk's MFMAs issue back to back.  NB is chosen per launch so
-// that the tile count fills 2 slots per CU with as little tail as possible
-// (NB = 13 for 32x64x56x56: 483 workgroups on 512 slots).
+// A workgroup owns a 64 x (16*NB) tile of D and has 8 waves with two roles:
+//   waves 0-3 ("gather"): one result position per thread; per K-chunk of 16 rows
+//     each thread fetches its position's 16 values (coalesced along W,
+//     branch-free: out-of-image taps become out-of-range buffer loads, which
+//     return zero) plus its share of the weight tile, two chunks ahead of the
+//     matrix cores, and stores the chunk that arrived into the LDS buffer the
+//     MFMA waves are not reading;
+//   waves 4-7 ("mfma"): arranged 2 (M) x 2 (N); wave (wm, wn) owns 32 x (16*nt)
+//     of the tile, nt = floor or ceil of NB/2, reads its LDS fragments and issues
+//     the chunk's MFMAs back to back (the loop is compiled per nt so that it is
+//     straight-line code).
+// Wave w and wave w+4 sit on the same SIMD, so the hardware overlaps address
+// arithmetic, loads and LDS stores of one with the MFMAs of the other; the two
+// roles meet at one barrier per chunk (double-buffered LDS).  Two workgroups
+// share a CU.  What a K row means (channel offset, window shift) is decoded once
+// per kernel into an LDS table that the gather waves read 16 rows at a time.
+// NB is chosen per launch so that the tile count fills 2 slots per CU with as
+// little tail as possible (NB = 13 for 32x64x56x56: 483 workgroups, 512 slots).
 //
 // v_mfma_f32_16x16x4_f32 operand layout (lane l of 64):
 //   A operand: A[i = l%16][k = l/16]     B operand: B[k = l/16][j = l%16]
@@ -59,8 +61,9 @@ constexpr int BM = MFMA_BM;
 constexpr int APITCH = 80;    // LDS pitch of the A tile (== 16 mod 32 banks)
 constexpr int NT_MAX = 8;     // 16-wide position blocks per wave
 constexpr int NB_MAX = 2 * NT_MAX;
-constexpr int THREADS = 256;  // 4 waves
-constexpr int AROWS = BM * KC / THREADS;   // A elements per thread and chunk
+constexpr int GTHREADS = 256;              // gather threads (waves 0-3)
+constexpr int THREADS = 2 * GTHREADS;      // plus the four MFMA waves
+constexpr int AROWS = BM * KC / GTHREADS;  // A elements per gather thread and chunk
 
 enum { MODE_FWD = 0, MODE_BWD_S1 = 1, MODE_BWD_GEN = 2 };
 
@@ -83,19 +86,24 @@ struct GatherParams {
   unsigned src_bytes, wgt_bytes;
 };
 
-// K-row table in LDS: tabA[kk] = {byte offset contributed by the row (channel and
-// window shift), dh}, tabB[kk] = dw; dh = -2^20 marks a row past Ktot.
+// K-row table in LDS, tabA[kk] = {x, y}, tabB[kk] = z:
+//   stride-1 modes: x = byte offset contributed by the row (channel and window
+//     shift), y / z = low / high word of (1 << tap).  Whether a tap falls inside
+//     the image depends on the position only, so every gather thread keeps a
+//     64-bit validity mask over the taps and tests one bit per element;
+//   general backward mode: x = byte offset of the channel, y = dh, z = dw
+//     (dh = -2^20 marks a row past Ktot) and validity is computed per element.
 constexpr int ROW_INVALID = -(1 << 20);
 
 template <typename T, int MODE>
-__global__ void __launch_bounds__(THREADS, 2)
+__global__ void __launch_bounds__(THREADS, 4)
 gather_conv_kernel(GatherParams p, const T* __restrict__ src, const T* __restrict__ wgt,
                    const float* __restrict__ bias, T* __restrict__ dst) {
   extern __shared__ float lds[];
   const int bstride = KC * p.BNP, astride = KC * APITCH;
   float* Bs = lds;                                   // [2][KC][BNP]
   float* As = lds + 2 * bstride;                     // [2][KC][APITCH]
-  const int nrows = p.nchunks * KC;
+  const int nrows = (p.nchunks + 2) * KC;              // two chunks of padding rows
   int2* tabA = reinterpret_cast<int2*>(As + 2 * astride);   // [nrows]
   int* tabB = reinterpret_cast<int*>(tabA + nrows);           // [nrows]
   const int esz = (int)sizeof(T);
@@ -104,15 +112,11 @@ gather_conv_kernel(GatherParams p, const T* __restrict__ src, const T* __restric
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave & 1, wn = wave >> 1;
   const int grp = blockIdx.y / p.mtiles, mtile = blockIdx.y % p.mtiles;
   const int BN = p.NB * 16;
   const int tile_p0 = blockIdx.x * BN;
-
-  // this wave's share of the NB position blocks
-  const int base = p.NB >> 1, rem = p.NB & 1;
-  const int nt = base + (wn < rem ? 1 : 0);
-  const int nb0 = wn * base + min(wn, rem);
+  const int m_lim = p.DCg - mtile * BM;               // valid result channels in the tile
+  const int n = p.nchunks;
 
   // ---- K-row table, once per kernel -------------------------------------------
   for (int kk = tid; kk < nrows; kk += THREADS) {
@@ -123,118 +127,156 @@ gather_conv_kernel(GatherParams p, const T* __restrict__ src, const T* __restric
       const int kh = t / p.KW, kw = t - kh * p.KW;
       const int dh = (MODE == MODE_FWD ? kh : -kh) * p.dly;
       const int dw = (MODE == MODE_FWD ? kw : -kw) * p.dlx;
-      ra.x = (c * p.SHW + (MODE != MODE_BWD_GEN ? dh * p.SW + dw : 0)) * esz;
-      ra.y = dh;
-      rb = dw;
+      if (MODE == MODE_BWD_GEN) {
+        ra.x = c * p.SHW * esz;
+        ra.y = dh;
+        rb = dw;
+      } else {
+        ra.x = (c * p.SHW + dh * p.SW + dw) * esz;
+        ra.y = t < 32 ? (int)(1u << t) : 0;
+        rb = t >= 32 ? (int)(1u << (t - 32)) : 0;
+      }
+    } else if (MODE != MODE_BWD_GEN) {
+      ra.y = 0;
     }
     tabA[kk] = ra;
     tabB[kk] = rb;
   }
-
-  // ---- per-thread gather position (one result position per thread) ----------
-  const bool loader = tid < BN;
-  const int P = tile_p0 + tid;
-  const bool pvalid = loader && P < p.Ptotal;
-  int hb, wb, pixbase;
-  {
-    const int Pc = pvalid ? P : 0;
-    const int n = Pc / p.DHW, q = Pc - n * p.DHW;
-    const int h = q / p.DW, w = q - h * p.DW;
-    if (MODE == MODE_FWD) {
-      hb = h * p.sy - p.py;
-      wb = w * p.sx - p.px;
-    } else {
-      hb = h + p.py;
-      wb = w + p.px;
-    }
-    pixbase = (n * p.SC + grp * p.SCg) * p.SHW;
-    if (MODE != MODE_BWD_GEN) pixbase += hb * p.SW + wb;
-    pixbase *= esz;                                  // byte offset
-    if (!pvalid) hb = 4 * ROW_INVALID;               // every tap fails the bounds test
-  }
-
-  // ---- per-thread share of the A tile: row ar = tid%16, m = tid/16 + 16*i ------
-  const int ar = tid & 15, am = tid >> 4;
-  const int m_lim = p.DCg - mtile * BM;               // valid result channels in the tile
-  const int wbase = grp * p.w_group_stride + mtile * BM * p.a_mstride;   // elements
-  int a_kk = ar, a_c = 0, a_t = ar;                   // row of the chunk being loaded
-  if (MODE != MODE_FWD) {
-    a_c = ar / p.KHW;
-    a_t = ar - a_c * p.KHW;
-  }
-
-  float breg[KC];
-  float areg[AROWS];
-
-  auto load_chunk = [&](int chunk) {
-    // the 16 rows' table entries first (broadcast LDS reads, 12 instructions)
-    int goff[KC], dh[KC], dw[KC];
-    {
-      const int4* ta = reinterpret_cast<const int4*>(tabA + chunk * KC);
-      const int4* tb = reinterpret_cast<const int4*>(tabB + chunk * KC);
-#pragma unroll
-      for (int i = 0; i < KC / 2; ++i) {
-        const int4 v = ta[i];
-        goff[2 * i] = v.x; dh[2 * i] = v.y; goff[2 * i + 1] = v.z; dh[2 * i + 1] = v.w;
-      }
-#pragma unroll
-      for (int i = 0; i < KC / 4; ++i) {
-        const int4 v = tb[i];
-        dw[4 * i] = v.x; dw[4 * i + 1] = v.y; dw[4 * i + 2] = v.z; dw[4 * i + 3] = v.w;
-      }
-    }
-#pragma unroll
-    for (int r = 0; r < KC; ++r) {
-      bool ok;
-      int off;
-      if (MODE == MODE_BWD_GEN) {
-        const int th = hb + dh[r], tw = wb + dw[r];
-        const int ih = th / p.sy, iw = tw / p.sx;
-        ok = (th >= 0) & (tw >= 0) & (ih * p.sy == th) & (iw * p.sx == tw) & (ih < p.SH) &
-             (iw < p.SW);
-        off = pixbase + goff[r] + (ih * p.SW + iw) * esz;
-      } else {
-        const int ih = hb + dh[r], iw = wb + dw[r];
-        ok = ((unsigned)ih < (unsigned)p.SH) & ((unsigned)iw < (unsigned)p.SW);
-        off = pixbase + goff[r];
-      }
-      breg[r] = buf_ld(srsrc, ok ? off : -1, src);
-    }
-    const bool kok = a_kk < p.Ktot;
-    const int arow = wbase + (MODE == MODE_FWD ? a_kk : a_c * p.a_bwd_kstride + a_t);
-#pragma unroll
-    for (int i = 0; i < AROWS; ++i) {
-      const int m = am + 16 * i;
-      const bool ok = kok & (m < m_lim);
-      areg[i] = buf_ld(wrsrc, ok ? (m * p.a_mstride + arow) * esz : -1, wgt);
-    }
-    a_kk += KC;
-    if (MODE != MODE_FWD) {
-      a_c += p.q16;
-      a_t += p.r16;
-      if (a_t >= p.KHW) {
-        a_t -= p.KHW;
-        ++a_c;
-      }
-    }
-  };
-
-  auto store_chunk = [&](int buf) {
-    float* bs = Bs + buf * bstride;
-    float* as = As + buf * astride;
-    if (loader) {
-#pragma unroll
-      for (int r = 0; r < KC; ++r) bs[r * p.BNP + tid] = breg[r];
-    }
-#pragma unroll
-    for (int i = 0; i < AROWS; ++i) as[ar * APITCH + am + 16 * i] = areg[i];
-  };
-
-  __syncthreads();                                    // table visible
-  load_chunk(0);
-  store_chunk(0);
   __syncthreads();
 
+  if (wave < 4) {
+    // =========================== gather waves ==================================
+    const int P = tile_p0 + tid;
+    const bool pvalid = tid < BN && P < p.Ptotal;
+    int hb, wb, pixbase;
+    {
+      const int Pc = pvalid ? P : 0;
+      const int ni = Pc / p.DHW, q = Pc - ni * p.DHW;
+      const int h = q / p.DW, w = q - h * p.DW;
+      if (MODE == MODE_FWD) {
+        hb = h * p.sy - p.py;
+        wb = w * p.sx - p.px;
+      } else {
+        hb = h + p.py;
+        wb = w + p.px;
+      }
+      pixbase = (ni * p.SC + grp * p.SCg) * p.SHW;
+      if (MODE != MODE_BWD_GEN) pixbase += hb * p.SW + wb;
+      pixbase *= esz;                                  // byte offset
+      if (!pvalid) hb = 4 * ROW_INVALID;               // every tap fails the bounds test
+    }
+    unsigned mask_lo = 0, mask_hi = 0;                 // taps that fall inside the image
+    if (MODE != MODE_BWD_GEN) {
+      for (int t = 0; t < p.KHW; ++t) {
+        const int kh = t / p.KW, kw = t - kh * p.KW;
+        const int ih = hb + (MODE == MODE_FWD ? kh : -kh) * p.dly;
+        const int iw = wb + (MODE == MODE_FWD ? kw : -kw) * p.dlx;
+        const unsigned ok = ((unsigned)ih < (unsigned)p.SH) & ((unsigned)iw < (unsigned)p.SW);
+        if (t < 32)
+          mask_lo |= ok << t;
+        else
+          mask_hi |= ok << (t - 32);
+      }
+    }
+    const bool taps64 = p.KHW > 32;
+    // share of the A tile: row ar = tid%16, m = tid/16 + 16*i
+    const int ar = tid & 15, am = tid >> 4;
+    const int wbase = grp * p.w_group_stride + mtile * BM * p.a_mstride;   // elements
+    int a_kk = ar, a_c = 0, a_t = ar;                  // row of the chunk being fetched
+    if (MODE != MODE_FWD) {
+      a_c = ar / p.KHW;
+      a_t = ar - a_c * p.KHW;
+    }
+
+    auto load_chunk = [&](int chunk, float (&breg)[KC], float (&areg)[AROWS]) {
+      int goff[KC], dh[KC], dw[KC];
+      {
+        const int4* ta = reinterpret_cast<const int4*>(tabA + chunk * KC);
+        const int4* tb = reinterpret_cast<const int4*>(tabB + chunk * KC);
+#pragma unroll
+        for (int i = 0; i < KC / 2; ++i) {
+          const int4 v = ta[i];
+          goff[2 * i] = v.x; dh[2 * i] = v.y; goff[2 * i + 1] = v.z; dh[2 * i + 1] = v.w;
+        }
+        if (MODE == MODE_BWD_GEN || taps64) {
+#pragma unroll
+          for (int i = 0; i < KC / 4; ++i) {
+            const int4 v = tb[i];
+            dw[4 * i] = v.x; dw[4 * i + 1] = v.y; dw[4 * i + 2] = v.z; dw[4 * i + 3] = v.w;
+          }
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < KC; ++r) {
+        bool ok;
+        int off;
+        if (MODE == MODE_BWD_GEN) {
+          const int th = hb + dh[r], tw = wb + dw[r];
+          const int ih = th / p.sy, iw = tw / p.sx;
+          ok = (th >= 0) & (tw >= 0) & (ih * p.sy == th) & (iw * p.sx == tw) & (ih < p.SH) &
+               (iw < p.SW);
+          off = pixbase + goff[r] + (ih * p.SW + iw) * esz;
+        } else {
+          unsigned m = mask_lo & (unsigned)dh[r];
+          if (taps64) m |= mask_hi & (unsigned)dw[r];
+          ok = m != 0;
+          off = pixbase + goff[r];
+        }
+        breg[r] = buf_ld(srsrc, ok ? off : -1, src);
+      }
+      const int arow = wbase + (MODE == MODE_FWD ? a_kk : a_c * p.a_bwd_kstride + a_t);
+      const bool kok = a_kk < p.Ktot;
+#pragma unroll
+      for (int i = 0; i < AROWS; ++i) {
+        const int m = am + 16 * i;
+        const bool ok = kok & (m < m_lim);
+        areg[i] = buf_ld(wrsrc, ok ? (m * p.a_mstride + arow) * esz : -1, wgt);
+      }
+      a_kk += KC;
+      if (MODE != MODE_FWD) {
+        a_c += p.q16;
+        a_t += p.r16;
+        if (a_t >= p.KHW) {
+          a_t -= p.KHW;
+          ++a_c;
+        }
+      }
+    };
+    auto store_chunk = [&](int buf, const float (&breg)[KC], const float (&areg)[AROWS]) {
+      float* bs = Bs + buf * bstride;
+      float* as = As + buf * astride;
+#pragma unroll
+      for (int r = 0; r < KC; ++r) bs[r * p.BNP + tid] = breg[r];
+#pragma unroll
+      for (int i = 0; i < AROWS; ++i) as[ar * APITCH + am + 16 * i] = areg[i];
+    };
+
+    // Two register sets: chunk c+1 waits in one while chunk c+2 is being fetched
+    // into the other, so a fetch has two MFMA phases to come back from HBM.  The
+    // table has two chunks of padding rows, so fetching past the end is harmless.
+    float bregA[KC], aregA[AROWS], bregB[KC], aregB[AROWS];
+    load_chunk(0, bregA, aregA);
+    store_chunk(0, bregA, aregA);
+    load_chunk(1, bregB, aregB);
+    __syncthreads();
+    for (int c = 0; c < n; c += 2) {
+      load_chunk(c + 2, bregA, aregA);
+      store_chunk(1, bregB, aregB);              // chunk c+1
+      __syncthreads();
+      if (c + 1 >= n) break;
+      load_chunk(c + 3, bregB, aregB);
+      store_chunk(0, bregA, aregA);              // chunk c+2
+      __syncthreads();
+    }
+    return;
+  }
+
+  // ============================= MFMA waves ====================================
+  const int cw = wave - 4;
+  const int wm = cw & 1, wn = cw >> 1;
+  const int base = p.NB >> 1, rem = p.NB & 1;
+  const int nt = base + (wn < rem ? 1 : 0);
+  const int nb0 = wn * base + min(wn, rem);
   const int fr = lane & 15, fk = lane >> 4;
 
   auto run = [&](auto ntc) {
@@ -245,9 +287,8 @@ gather_conv_kernel(GatherParams p, const T* __restrict__ src, const T* __restric
 #pragma unroll
       for (int j = 0; j < NT; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    for (int c = 0; c < p.nchunks; ++c) {
-      const bool more = c + 1 < p.nchunks;
-      if (more) load_chunk(c + 1);
+    __syncthreads();                             // chunk 0 is in LDS buffer 0
+    for (int c = 0; c < n; ++c) {
       const float* as = As + (c & 1) * astride + wm * 32 + fr;
       const float* bs = Bs + (c & 1) * bstride + nb0 * 16 + fr;
       float a[KC / 4][2], b[KC / 4][NT];
@@ -259,6 +300,7 @@ gather_conv_kernel(GatherParams p, const T* __restrict__ src, const T* __restric
 #pragma unroll
         for (int j = 0; j < NT; ++j) b[ks][j] = bs[krow * p.BNP + j * 16];
       }
+      __builtin_amdgcn_sched_barrier(0);         // all fragment reads ahead of the MFMAs
 #pragma unroll
       for (int ks = 0; ks < KC / 4; ++ks) {
 #pragma unroll
@@ -267,7 +309,6 @@ gather_conv_kernel(GatherParams p, const T* __restrict__ src, const T* __restric
           acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[ks][1], b[ks][j], acc[1][j], 0, 0, 0);
         }
       }
-      if (more) store_chunk((c + 1) & 1);
       __syncthreads();
     }
 
@@ -276,7 +317,7 @@ gather_conv_kernel(GatherParams p, const T* __restrict__ src, const T* __restric
     for (int j = 0; j < NT; ++j) {
       const int Pj = tile_p0 + (nb0 + j) * 16 + fr;
       if (Pj < p.Ptotal) {
-        const int n = Pj / p.DHW, q = Pj - n * p.DHW;
+        const int ni = Pj / p.DHW, q = Pj - ni * p.DHW;
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
 #pragma unroll
@@ -286,7 +327,7 @@ gather_conv_kernel(GatherParams p, const T* __restrict__ src, const T* __restric
               const int ch = grp * p.DCg + mtile * BM + m;
               float v = acc[i][j][r];
               if (bias) v += bias[ch];
-              st(dst, (size_t)(n * p.DC + ch) * p.DHW + q, v);
+              st(dst, (size_t)(ni * p.DC + ch) * p.DHW + q, v);
             }
           }
         }
@@ -330,7 +371,7 @@ int launch_gather(const GatherParams& p0, const void* src, const void* wgt, cons
   const long long wbytes = (long long)p.groups * p.w_group_stride * (long long)sizeof(T);
   const int hmax = MODE == MODE_FWD ? p.DH * p.sy : p.DH + p.py;
   if (sbytes >= (1ll << 31) || wbytes >= (1ll << 31) || hmax >= (1 << 19) ||
-      (p.KH - 1) * p.dly >= (1 << 19))
+      (p.KH - 1) * p.dly >= (1 << 19) || (MODE != MODE_BWD_GEN && p.KHW > 64))
     return -1;
   p.src_bytes = (unsigned)sbytes;
   p.wgt_bytes = (unsigned)wbytes;
@@ -340,9 +381,10 @@ int launch_gather(const GatherParams& p0, const void* src, const void* wgt, cons
   const long long pblocks = ((long long)p.Ptotal + 15) / 16;
   p.NB = choose_nb(pblocks, p.mtiles * p.groups, 2 * mfma_num_cus());
   const int BN = p.NB * 16;
-  p.BNP = BN + ((16 - BN % 32) + 32) % 32;   // == 16 mod 32
+  (void)BN;
+  p.BNP = GTHREADS + 16;                     // every gather thread owns a column; == 16 mod 32
   const size_t shmem = (size_t)2 * (KC * p.BNP + KC * APITCH) * sizeof(float) +
-                       (size_t)p.nchunks * KC * 3 * sizeof(int);
+                       (size_t)(p.nchunks + 2) * KC * 3 * sizeof(int);
   auto kernel = gather_conv_kernel<T, MODE>;
   if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
   const dim3 grid((unsigned)((pblocks + p.NB - 1) / p.NB), (unsigned)(p.mtiles * p.groups));

@@ -103,10 +103,10 @@ wgrad_kernel(WgradParams p, const T* __restrict__ x, const T* __restrict__ dy,
     ld_ow = q - ld_oh * p.OW;
   }
 
-  float breg[WCL_MAX];
-  float areg[WAR];
+  // two register sets: chunk c+1 waits in one while chunk c+2 is being fetched
+  float bregA[WCL_MAX], aregA[WAR], bregB[WCL_MAX], aregB[WAR];
 
-  auto load_chunk = [&]() {
+  auto load_chunk = [&](float (&breg)[WCL_MAX], float (&areg)[WAR]) {
     const bool pv = ld_P < P_end;
     const int ihb = pv ? ld_oh * p.sy - p.py : 4 * COL_INVALID, iwb = ld_ow * p.sx - p.px;
     const int xbase = ((ld_n * p.C + grp * p.Cg) * p.HW + ihb * p.W + iwb) * esz;
@@ -138,7 +138,7 @@ wgrad_kernel(WgradParams p, const T* __restrict__ x, const T* __restrict__ dy,
     }
   };
 
-  auto store_chunk = [&](int buf) {
+  auto store_chunk = [&](int buf, const float (&breg)[WCL_MAX], const float (&areg)[WAR]) {
     float* bs = Bs + buf * bstride;
     float* as = As + buf * astride;
 #pragma unroll
@@ -148,8 +148,9 @@ wgrad_kernel(WgradParams p, const T* __restrict__ x, const T* __restrict__ dy,
     for (int i = 0; i < WAR; ++i) as[(cl + 16 * i) * WKP + pl] = areg[i];
   };
 
-  load_chunk();
-  store_chunk(0);
+  load_chunk(bregA, aregA);
+  store_chunk(0, bregA, aregA);
+  if (nchunks > 1) load_chunk(bregB, aregB);
   __syncthreads();
 
   const int fr = lane & 15, fk = lane >> 4;
@@ -165,9 +166,7 @@ wgrad_kernel(WgradParams p, const T* __restrict__ x, const T* __restrict__ dy,
 #pragma unroll
       for (int j = 0; j < NT; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    for (int c = 0; c < nchunks; ++c) {
-      const bool more = c + 1 < nchunks;
-      if (more) load_chunk();
+    auto compute = [&](int c) {
       const float* as = As + (c & 1) * astride + (wm * 32 + fr) * WKP + fk;
       const float* bs = Bs + (c & 1) * bstride + (nb0 * 16 + fr) * WKP + fk;
       float a[WKC / 4][2], b[WKC / 4][NT];
@@ -178,6 +177,7 @@ wgrad_kernel(WgradParams p, const T* __restrict__ x, const T* __restrict__ dy,
 #pragma unroll
         for (int j = 0; j < NT; ++j) b[ks][j] = bs[j * 16 * WKP + ks * 4];
       }
+      __builtin_amdgcn_sched_barrier(0);   // keep the fragment reads ahead of the MFMAs
 #pragma unroll
       for (int ks = 0; ks < WKC / 4; ++ks) {
 #pragma unroll
@@ -193,7 +193,18 @@ wgrad_kernel(WgradParams p, const T* __restrict__ x, const T* __restrict__ dy,
         for (int k = 0; k < WKC; ++k) s += ar[k];
         dbacc += s;
       }
-      if (more) store_chunk((c + 1) & 1);
+    };
+
+    const int n = nchunks;
+    for (int c = 0; c < n; c += 2) {
+      if (c + 2 < n) load_chunk(bregA, aregA);
+      compute(c);
+      if (c + 1 < n) store_chunk(1, bregB, aregB);
+      __syncthreads();
+      if (c + 1 >= n) break;
+      if (c + 3 < n) load_chunk(bregB, aregB);
+      compute(c + 1);
+      if (c + 2 < n) store_chunk(0, bregA, aregA);
       __syncthreads();
     }
 
