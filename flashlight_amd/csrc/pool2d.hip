@@ -101,6 +101,255 @@ pool_bwd_direct(PoolGeom g, const T* __restrict__ dy,
   st(dx, e, acc);
 }
 
+// ---------------------------------------------------------------------------
+// Fast path: 3x3 window, stride 2, padding 1, W % 4 == 0 (the ResNet stem pool).
+// A thread owns four input columns [4*tq, 4*tq+3] = two output columns of a
+// strip of POOL_OHB output rows and walks down the strip, so that every input
+// row is fetched once as one 16-byte load per lane; the column left of the
+// quad comes from the neighbouring lane.  Rows are visited in window order,
+// which keeps the first-maximum tie rule and the fp32 summation order of the
+// generic kernels.
+// ---------------------------------------------------------------------------
+constexpr int POOL_OHB = 8;
+
+struct PoolRow {
+  float l;      // column 4*tq - 1 (meaningful when tq > 0)
+  float4 v;     // columns 4*tq .. 4*tq + 3
+  bool ok;      // row inside the image
+};
+
+template <typename T>
+__device__ __forceinline__ PoolRow pool_load_row(const T* xq, int W, int ih, bool ok, int tq,
+                                                 int lane) {
+  PoolRow r;
+  r.ok = ok;
+  r.v = ok ? ld4(xq, (size_t)ih * W) : make_float4(0.f, 0.f, 0.f, 0.f);
+  float up = __shfl_up(r.v.w, 1, 64);
+  if (lane == 0 && tq > 0 && ok) up = ld(xq, (size_t)ih * W - 1);
+  r.l = up;
+  return r;
+}
+
+template <int MODE>
+__device__ __forceinline__ void pool_scan3(const PoolRow& r, int kh, bool has_left, float a,
+                                           float b, float c, float& best, int& idx, float& sum,
+                                           int& cnt, bool first_col) {
+  // one window row: candidates (kw = 0, 1, 2) = (a, b, c); for the first output
+  // column of the thread, a is the neighbour's value and may be padding
+  if (!r.ok) return;
+  if (!first_col || has_left) {
+    if (MODE == FLHIP_POOL_MAX) {
+      if (a > best) { best = a; idx = kh * 3; }
+    } else {
+      sum += a; ++cnt;
+    }
+  }
+  if (MODE == FLHIP_POOL_MAX) {
+    if (b > best) { best = b; idx = kh * 3 + 1; }
+    if (c > best) { best = c; idx = kh * 3 + 2; }
+  } else {
+    sum += b; sum += c; cnt += 2;
+  }
+}
+
+__device__ __forceinline__ void st2(float* p, size_t i, float a, float b) {
+  *reinterpret_cast<float2*>(p + i) = make_float2(a, b);
+}
+__device__ __forceinline__ void st2(bf16_t* p, size_t i, float a, float b) {
+  *reinterpret_cast<uint32_t*>(p + i) = (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+}
+__device__ __forceinline__ float2 ld2(const float* p, size_t i) {
+  return *reinterpret_cast<const float2*>(p + i);
+}
+__device__ __forceinline__ float2 ld2(const bf16_t* p, size_t i) {
+  const uint32_t r = *reinterpret_cast<const uint32_t*>(p + i);
+  return make_float2(__uint_as_float(r << 16), __uint_as_float(r & 0xffff0000u));
+}
+
+template <typename T, int MODE>
+__global__ void __launch_bounds__(256)
+pool_w3s2_fwd(PoolGeom g, const T* __restrict__ x, T* __restrict__ y,
+              uint8_t* __restrict__ argmax, int TQ, int nstrips, size_t items) {
+  const size_t item0 = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const bool active = item0 < items;
+  const size_t item = active ? item0 : items - 1;
+  const int lane = threadIdx.x & 63;
+  const int tq = (int)(item % TQ);
+  const size_t t = item / TQ;
+  const int oh0 = (int)(t % nstrips) * POOL_OHB;
+  const size_t plane = t / nstrips;
+  const T* xq = x + plane * (size_t)g.H * g.W + 4 * tq;
+  const size_t obase = plane * (size_t)g.OH * g.OW + 2 * tq;
+  const bool has_left = tq > 0;
+
+  PoolRow r0 = pool_load_row(xq, g.W, 2 * oh0 - 1, oh0 > 0, tq, lane);
+#pragma unroll 2
+  for (int k = 0; k < POOL_OHB; ++k) {
+    const int oh = oh0 + k;
+    const bool ok = oh < g.OH;
+    const PoolRow r1 = pool_load_row(xq, g.W, 2 * oh, ok && 2 * oh < g.H, tq, lane);
+    const PoolRow r2 = pool_load_row(xq, g.W, 2 * oh + 1, ok && 2 * oh + 1 < g.H, tq, lane);
+    float b0 = -FLT_MAX, b1 = -FLT_MAX, s0 = 0.f, s1 = 0.f;
+    int i0 = 0, i1 = 0, c0 = 0, c1 = 0;
+    pool_scan3<MODE>(r0, 0, has_left, r0.l, r0.v.x, r0.v.y, b0, i0, s0, c0, true);
+    pool_scan3<MODE>(r1, 1, has_left, r1.l, r1.v.x, r1.v.y, b0, i0, s0, c0, true);
+    pool_scan3<MODE>(r2, 2, has_left, r2.l, r2.v.x, r2.v.y, b0, i0, s0, c0, true);
+    pool_scan3<MODE>(r0, 0, true, r0.v.y, r0.v.z, r0.v.w, b1, i1, s1, c1, false);
+    pool_scan3<MODE>(r1, 1, true, r1.v.y, r1.v.z, r1.v.w, b1, i1, s1, c1, false);
+    pool_scan3<MODE>(r2, 2, true, r2.v.y, r2.v.z, r2.v.w, b1, i1, s1, c1, false);
+    if (active && ok) {
+      const size_t o = obase + (size_t)oh * g.OW;
+      if (MODE == FLHIP_POOL_MAX) {
+        st2(y, o, b0, b1);
+        if (argmax) *reinterpret_cast<uint16_t*>(argmax + o) = (uint16_t)(i0 | (i1 << 8));
+      } else if (MODE == FLHIP_POOL_AVG_INCLUDE_PADDING) {
+        st2(y, o, s0 / 9.f, s1 / 9.f);
+      } else {
+        st2(y, o, s0 / (float)c0, s1 / (float)c1);
+      }
+    }
+    r0 = r2;
+  }
+}
+
+// Backward for the same geometry.  A thread owns the same four input columns
+// and strip; it reads dy / argmax of its two output columns (plus the next one
+// from the neighbouring lane) row by row and accumulates the three input rows
+// each output row touches, carrying the shared odd row to the next output row so
+// that the additions happen in ascending (oh, ow) order.
+struct PoolGrad {
+  float g0, g1, g2;   // dy (already divided for the average modes) at ow = 2tq, 2tq+1, 2tq+2
+  int a0, a1, a2;     // argmax bytes (max mode)
+  bool ok;            // output row exists
+};
+
+template <typename T, int MODE>
+__device__ __forceinline__ PoolGrad pool_load_grad(const PoolGeom& g, const T* dyq,
+                                                   const uint8_t* amq, int oh, bool ok, int tq,
+                                                   int TQ, int lane) {
+  PoolGrad r;
+  r.ok = ok;
+  float2 d = make_float2(0.f, 0.f);
+  int a0 = 255, a1 = 255;
+  if (ok) {
+    d = ld2(dyq, (size_t)oh * g.OW);
+    if (MODE == FLHIP_POOL_MAX) {
+      const uint16_t a = *reinterpret_cast<const uint16_t*>(amq + (size_t)oh * g.OW);
+      a0 = a & 0xff;
+      a1 = a >> 8;
+    } else if (MODE == FLHIP_POOL_AVG_INCLUDE_PADDING) {
+      d.x = d.x / 9.f;
+      d.y = d.y / 9.f;
+    } else {
+      // in-bounds count of window (oh, ow): rows 2oh-1..2oh+1, cols 2ow-1..2ow+1
+      const int rows = min(2 * oh + 2, g.H) - max(2 * oh - 1, 0);
+      const int cw0 = min(4 * tq + 2, g.W) - max(4 * tq - 1, 0);
+      const int cw1 = min(4 * tq + 4, g.W) - (4 * tq + 1);
+      d.x = d.x / (float)(rows * cw0);
+      d.y = d.y / (float)(rows * cw1);
+    }
+  }
+  r.g0 = d.x; r.g1 = d.y; r.a0 = a0; r.a1 = a1;
+  // the next output column belongs to the next lane
+  float g2 = __shfl_down(d.x, 1, 64);
+  int a2 = __shfl_down(a0, 1, 64);
+  const bool has_right = tq + 1 < TQ;
+  if (lane == 63 && has_right && ok) {
+    if (MODE == FLHIP_POOL_MAX) {
+      g2 = ld(dyq, (size_t)oh * g.OW + 2);
+      a2 = amq[(size_t)oh * g.OW + 2];
+    } else {
+      float v = ld(dyq, (size_t)oh * g.OW + 2);
+      if (MODE == FLHIP_POOL_AVG_INCLUDE_PADDING) {
+        v = v / 9.f;
+      } else {
+        const int rows = min(2 * oh + 2, g.H) - max(2 * oh - 1, 0);
+        const int cw2 = min(4 * tq + 6, g.W) - (4 * tq + 3);
+        v = v / (float)(rows * cw2);
+      }
+      g2 = v;
+    }
+  }
+  r.g2 = (has_right && ok) ? g2 : 0.f;
+  r.a2 = has_right ? a2 : 255;
+  return r;
+}
+
+// adds the contributions of output row `q` through window row kh to the four columns
+template <int MODE>
+__device__ __forceinline__ void pool_bwd_row(const PoolGrad& q, int kh, float4& acc) {
+  if (!q.ok) return;
+  if (MODE == FLHIP_POOL_MAX) {
+    acc.x += (q.a0 == kh * 3 + 1) ? q.g0 : 0.f;
+    acc.y += (q.a0 == kh * 3 + 2) ? q.g0 : 0.f;
+    acc.y += (q.a1 == kh * 3 + 0) ? q.g1 : 0.f;
+    acc.z += (q.a1 == kh * 3 + 1) ? q.g1 : 0.f;
+    acc.w += (q.a1 == kh * 3 + 2) ? q.g1 : 0.f;
+    acc.w += (q.a2 == kh * 3 + 0) ? q.g2 : 0.f;
+  } else {
+    acc.x += q.g0;
+    acc.y += q.g0;
+    acc.y += q.g1;
+    acc.z += q.g1;
+    acc.w += q.g1;
+    acc.w += q.g2;
+  }
+}
+
+template <typename T, int MODE>
+__global__ void __launch_bounds__(256)
+pool_w3s2_bwd(PoolGeom g, const T* __restrict__ dy, const uint8_t* __restrict__ argmax,
+              T* __restrict__ dx, int TQ, int nstrips, size_t items) {
+  const size_t item0 = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const bool active = item0 < items;
+  const size_t item = active ? item0 : items - 1;
+  const int lane = threadIdx.x & 63;
+  const int tq = (int)(item % TQ);
+  const size_t t = item / TQ;
+  const int strip = (int)(t % nstrips);
+  const int oh0 = strip * POOL_OHB;
+  const size_t plane = t / nstrips;
+  const T* dyq = dy + plane * (size_t)g.OH * g.OW + 2 * tq;
+  const uint8_t* amq = MODE == FLHIP_POOL_MAX ? argmax + plane * (size_t)g.OH * g.OW + 2 * tq : nullptr;
+  T* dxq = dx + plane * (size_t)g.H * g.W + 4 * tq;
+
+  // the strip owns input rows 2*oh0-1 .. 2*oh_end-2 (and 2*oh_end-1 when it is the
+  // last strip); row 2*oh0-1 also receives from output row oh0-1
+  float4 odd = make_float4(0.f, 0.f, 0.f, 0.f);   // accumulates row 2*oh-1
+  {
+    const PoolGrad q = pool_load_grad<T, MODE>(g, dyq, amq, oh0 - 1, oh0 > 0, tq, TQ, lane);
+    pool_bwd_row<MODE>(q, 2, odd);
+  }
+#pragma unroll 2
+  for (int k = 0; k < POOL_OHB; ++k) {
+    const int oh = oh0 + k;
+    const bool ok = oh < g.OH;
+    const PoolGrad q = pool_load_grad<T, MODE>(g, dyq, amq, oh, ok, tq, TQ, lane);
+    pool_bwd_row<MODE>(q, 0, odd);
+    float4 even = make_float4(0.f, 0.f, 0.f, 0.f);
+    pool_bwd_row<MODE>(q, 1, even);
+    if (active && ok) {
+      if (2 * oh - 1 >= 0) st4(dxq, (size_t)(2 * oh - 1) * g.W, odd);
+      if (2 * oh < g.H) st4(dxq, (size_t)(2 * oh) * g.W, even);
+    }
+    odd = make_float4(0.f, 0.f, 0.f, 0.f);
+    pool_bwd_row<MODE>(q, 2, odd);
+    // last output row of the image: nothing below adds to row 2*oh+1
+    if (active && ok && oh == g.OH - 1) {
+      for (int r = 2 * oh + 1; r < g.H; ++r) {
+        st4(dxq, (size_t)r * g.W, odd);
+        odd = make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    }
+  }
+}
+
+static bool w3s2_applies(const PoolGeom& g, const void* a, const void* b, const void* am) {
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b);
+  return g.wy == 3 && g.wx == 3 && g.sy == 2 && g.sx == 2 && g.py == 1 && g.px == 1 &&
+         g.W % 4 == 0 && g.H >= 2 && bits % 16 == 0 && reinterpret_cast<uintptr_t>(am) % 2 == 0;
+}
+
 template <typename T>
 static int launch_fwd(const PoolGeom& g, int mode, const void* x, void* y,
                       uint8_t* argmax, hipStream_t s) {
@@ -108,6 +357,22 @@ static int launch_fwd(const PoolGeom& g, int mode, const void* x, void* y,
   const dim3 grid((unsigned)((total + 255) / 256)), block(256);
   const T* xp = static_cast<const T*>(x);
   T* yp = static_cast<T*>(y);
+  if (w3s2_applies(g, x, y, argmax)) {
+    const int TQ = g.W / 4, nstrips = (g.OH + POOL_OHB - 1) / POOL_OHB;
+    const size_t items = (size_t)g.N * g.C * nstrips * TQ;
+    const dim3 fgrid((unsigned)((items + 255) / 256));
+    switch (mode) {
+      case FLHIP_POOL_MAX:
+        hipLaunchKernelGGL((pool_w3s2_fwd<T, FLHIP_POOL_MAX>), fgrid, block, 0, s, g, xp, yp, argmax, TQ, nstrips, items);
+        break;
+      case FLHIP_POOL_AVG_INCLUDE_PADDING:
+        hipLaunchKernelGGL((pool_w3s2_fwd<T, FLHIP_POOL_AVG_INCLUDE_PADDING>), fgrid, block, 0, s, g, xp, yp, argmax, TQ, nstrips, items);
+        break;
+      default:
+        hipLaunchKernelGGL((pool_w3s2_fwd<T, FLHIP_POOL_AVG_EXCLUDE_PADDING>), fgrid, block, 0, s, g, xp, yp, argmax, TQ, nstrips, items);
+    }
+    return check_launch("pool2d_fwd");
+  }
   switch (mode) {
     case FLHIP_POOL_MAX:
       hipLaunchKernelGGL((pool_fwd_direct<T, FLHIP_POOL_MAX>), grid, block, 0, s, g, xp, yp, argmax, total);
@@ -128,6 +393,22 @@ static int launch_bwd(const PoolGeom& g, int mode, const void* dy,
   const dim3 grid((unsigned)((total + 255) / 256)), block(256);
   const T* dyp = static_cast<const T*>(dy);
   T* dxp = static_cast<T*>(dx);
+  if (w3s2_applies(g, dy, dx, argmax)) {
+    const int TQ = g.W / 4, nstrips = (g.OH + POOL_OHB - 1) / POOL_OHB;
+    const size_t items = (size_t)g.N * g.C * nstrips * TQ;
+    const dim3 fgrid((unsigned)((items + 255) / 256));
+    switch (mode) {
+      case FLHIP_POOL_MAX:
+        hipLaunchKernelGGL((pool_w3s2_bwd<T, FLHIP_POOL_MAX>), fgrid, block, 0, s, g, dyp, argmax, dxp, TQ, nstrips, items);
+        break;
+      case FLHIP_POOL_AVG_INCLUDE_PADDING:
+        hipLaunchKernelGGL((pool_w3s2_bwd<T, FLHIP_POOL_AVG_INCLUDE_PADDING>), fgrid, block, 0, s, g, dyp, argmax, dxp, TQ, nstrips, items);
+        break;
+      default:
+        hipLaunchKernelGGL((pool_w3s2_bwd<T, FLHIP_POOL_AVG_EXCLUDE_PADDING>), fgrid, block, 0, s, g, dyp, argmax, dxp, TQ, nstrips, items);
+    }
+    return check_launch("pool2d_bwd");
+  }
   switch (mode) {
     case FLHIP_POOL_MAX:
       hipLaunchKernelGGL((pool_bwd_direct<T, FLHIP_POOL_MAX>), grid, block, 0, s, g, dyp, argmax, dxp, total);

@@ -20,6 +20,10 @@ MORE = [
     ((1, 3, 33, 36), (3, 3), (2, 2), (1, 1)),     # odd height
     ((2, 6, 7, 7), (7, 7), (1, 1), (0, 0)),
     ((1, 2, 1, 40), (1, 4), (1, 3), (0, 1)),      # 1-D
+    ((3, 7, 56, 280), (3, 3), (2, 2), (1, 1)),    # fast path, rows wider than a wave
+    ((2, 3, 37, 24), (3, 3), (2, 2), (1, 1)),     # fast path, odd height, short last strip
+    ((5, 3, 2, 4), (3, 3), (2, 2), (1, 1)),       # fast path, tiny planes
+    ((1, 2, 18, 8), (3, 3), (2, 2), (1, 1)),
 ]
 ALL = GEOMS + MORE
 
