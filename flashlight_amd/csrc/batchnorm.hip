@@ -56,29 +56,52 @@ struct Vec<T, 4> {
     v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
   }
   __device__ __forceinline__ void store(T* p, size_t i) const {
-    st4(p, i, make_float4(v[0], v[1], v[2], v[3]));
+    st4_stream(p, i, make_float4(v[0], v[1], v[2], v[3]));
   }
 };
 
-// Iterates the units [u0, u1) of slice blockIdx.x of feature blockIdx.y.
-#define BN_SEG_LOOP_BEGIN(g)                                                   \
-  const long long c = blockIdx.y;                                              \
-  const long long innerV = (g).inner / VEC;                                    \
-  const long long u0 = (long long)blockIdx.x * (g).ups;                        \
-  const long long u1 = min(u0 + (g).ups, (g).units);                           \
-  long long u = u0 + threadIdx.x;                                              \
-  long long o = u / innerV;                                                    \
-  long long i = u - o * innerV;                                                \
-  for (; u < u1; u += 256) {                                                   \
-    const size_t off = (size_t)((o * (g).C + c) * (g).inner + i * VEC);
-#define BN_SEG_LOOP_END(g)                                                     \
-    o += (g).step_o;                                                           \
-    i += (g).step_i;                                                           \
-    if (i >= innerV) {                                                         \
-      i -= innerV;                                                             \
-      ++o;                                                                     \
-    }                                                                          \
+// Visits the units [u0, u1) of slice blockIdx.y of feature blockIdx.x, BN_UN at a
+// time per thread: f(off, n) gets BN_UN element offsets of which the first n are
+// in range (the others repeat a valid offset so loads need no branch).  Issuing
+// BN_UN independent 16-byte loads per thread is what keeps enough bytes in flight
+// to cover HBM latency.  The feature index is the fast grid dimension:
+// workgroups that run together then read neighbouring segments of the same
+// outer slice, i.e. one contiguous region of memory, which is what HBM likes.
+constexpr int BN_UN = 4;
+
+template <int VEC, bool REVERSE, typename F>
+__device__ __forceinline__ void bn_seg_visit(const BnGeom& g, F&& f) {
+  // REVERSE: slices are taken from the end of the tensor first.  The second
+  // kernel of a pass uses it so that it starts with what the first kernel read
+  // last and is most likely still cached.
+  const long long c = blockIdx.x;
+  const long long innerV = g.inner / VEC;
+  const long long slice = REVERSE ? (long long)(gridDim.y - 1 - blockIdx.y) : (long long)blockIdx.y;
+  const long long u0 = slice * g.ups;
+  const long long u1 = min(u0 + g.ups, g.units);
+  long long u = u0 + threadIdx.x;
+  long long o = u / innerV;
+  long long i = u - o * innerV;
+  while (u < u1) {
+    size_t off[BN_UN];
+    int n = 0;
+#pragma unroll
+    for (int k = 0; k < BN_UN; ++k) {
+      const size_t here = (size_t)((o * g.C + c) * g.inner + i * VEC);
+      const bool in = u < u1;
+      off[k] = in ? here : off[0];
+      n += in ? 1 : 0;
+      u += 256;
+      o += g.step_o;
+      i += g.step_i;
+      if (i >= innerV) {
+        i -= innerV;
+        ++o;
+      }
+    }
+    f(off, n);
   }
+}
 
 // ---- forward, segment mode -------------------------------------------------
 template <typename T, int VEC>
@@ -86,22 +109,32 @@ __global__ void __launch_bounds__(256)
 bn_stats_seg(BnGeom g, const T* __restrict__ x, float* __restrict__ ws) {
   __shared__ float red[8];
   float s1 = 0.f, s2 = 0.f;
-  const float shift = ld(x, (size_t)(blockIdx.y * g.inner));
-  BN_SEG_LOOP_BEGIN(g)
-    Vec<T, VEC> a;
-    a.load(x, off);
+  const long long c = blockIdx.x;
+  const float shift = ld(x, (size_t)(c * g.inner));
+  bn_seg_visit<VEC, false>(g, [&](const size_t (&off)[BN_UN], int n) {
+    Vec<T, VEC> a[BN_UN];
 #pragma unroll
-    for (int k = 0; k < VEC; ++k) {
-      const float t = a.v[k] - shift;
-      s1 += t;
-      s2 += t * t;
+    for (int k = 0; k < BN_UN; ++k) a[k].load(x, off[k]);
+#pragma unroll
+    for (int k = 0; k < BN_UN; ++k) {
+      float p1 = 0.f, p2 = 0.f;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        const float t = a[k].v[e] - shift;
+        p1 += t;
+        p2 += t * t;
+      }
+      if (k < n) {
+        s1 += p1;
+        s2 += p2;
+      }
     }
-  BN_SEG_LOOP_END(g)
+  });
   s1 = block_sum(s1, red);
   s2 = block_sum(s2, red);
   if (threadIdx.x == 0) {
-    ws[(c * g.S + blockIdx.x) * 2 + 0] = s1;
-    ws[(c * g.S + blockIdx.x) * 2 + 1] = s2;
+    ws[(c * g.S + blockIdx.y) * 2 + 0] = s1;
+    ws[(c * g.S + blockIdx.y) * 2 + 1] = s2;
   }
 }
 
@@ -153,22 +186,26 @@ bn_train_apply_seg(BnGeom g, const T* __restrict__ x, T* __restrict__ y,
   __shared__ float sh[2];
   if (threadIdx.x < 64) {
     double p0, p1;
-    fold_partials(ws, blockIdx.y, g.S, &p0, &p1);
-    finish_stats(g, a, blockIdx.y, ld(x, (size_t)(blockIdx.y * g.inner)), p0, p1,
-                 blockIdx.x == 0, sh);
+    fold_partials(ws, blockIdx.x, g.S, &p0, &p1);
+    finish_stats(g, a, blockIdx.x, ld(x, (size_t)(blockIdx.x * g.inner)), p0, p1,
+                 blockIdx.y == 0, sh);
   }
   __syncthreads();
   const float mean = sh[0];
-  const float gm = a.gamma ? a.gamma[blockIdx.y] : 1.f;
+  const float gm = a.gamma ? a.gamma[blockIdx.x] : 1.f;
   const float scale = gm * sh[1];
-  const float bt = a.beta ? a.beta[blockIdx.y] : 0.f;
-  BN_SEG_LOOP_BEGIN(g)
-    Vec<T, VEC> v;
-    v.load(x, off);
+  const float bt = a.beta ? a.beta[blockIdx.x] : 0.f;
+  bn_seg_visit<VEC, true>(g, [&](const size_t (&off)[BN_UN], int n) {
+    Vec<T, VEC> v[BN_UN];
 #pragma unroll
-    for (int k = 0; k < VEC; ++k) v.v[k] = (v.v[k] - mean) * scale + bt;
-    v.store(y, off);
-  BN_SEG_LOOP_END(g)
+    for (int k = 0; k < BN_UN; ++k) v[k].load(x, off[k]);
+#pragma unroll
+    for (int k = 0; k < BN_UN; ++k) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v[k].v[e] = (v[k].v[e] - mean) * scale + bt;
+      if (k < n) v[k].store(y, off[k]);
+    }
+  });
 }
 
 // ---- backward, segment mode ------------------------------------------------
@@ -178,22 +215,34 @@ bn_bwd_stats_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
                  const float* __restrict__ save_mean, float* __restrict__ ws) {
   __shared__ float red[8];
   float s1 = 0.f, s2 = 0.f;
-  const float mean = save_mean[blockIdx.y];
-  BN_SEG_LOOP_BEGIN(g)
-    Vec<T, VEC> a, b;
-    a.load(x, off);
-    b.load(dy, off);
+  const long long c = blockIdx.x;
+  const float mean = save_mean[c];
+  bn_seg_visit<VEC, false>(g, [&](const size_t (&off)[BN_UN], int n) {
+    Vec<T, VEC> a[BN_UN], b[BN_UN];
 #pragma unroll
-    for (int k = 0; k < VEC; ++k) {
-      s1 += b.v[k];
-      s2 += b.v[k] * (a.v[k] - mean);
+    for (int k = 0; k < BN_UN; ++k) {
+      a[k].load(x, off[k]);
+      b[k].load(dy, off[k]);
     }
-  BN_SEG_LOOP_END(g)
+#pragma unroll
+    for (int k = 0; k < BN_UN; ++k) {
+      float p1 = 0.f, p2 = 0.f;
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        p1 += b[k].v[e];
+        p2 += b[k].v[e] * (a[k].v[e] - mean);
+      }
+      if (k < n) {
+        s1 += p1;
+        s2 += p2;
+      }
+    }
+  });
   s1 = block_sum(s1, red);
   s2 = block_sum(s2, red);
   if (threadIdx.x == 0) {
-    ws[(c * g.S + blockIdx.x) * 2 + 0] = s1;
-    ws[(c * g.S + blockIdx.x) * 2 + 1] = s2;
+    ws[(c * g.S + blockIdx.y) * 2 + 0] = s1;
+    ws[(c * g.S + blockIdx.y) * 2 + 1] = s2;
   }
 }
 
@@ -230,19 +279,25 @@ bn_bwd_apply_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
   __shared__ float sh[4];
   if (threadIdx.x < 64) {
     double p0, p1;
-    fold_partials(ws, blockIdx.y, g.S, &p0, &p1);
-    finish_bwd(g, a, blockIdx.y, p0, p1, blockIdx.x == 0, sh);
+    fold_partials(ws, blockIdx.x, g.S, &p0, &p1);
+    finish_bwd(g, a, blockIdx.x, p0, p1, blockIdx.y == 0, sh);
   }
   __syncthreads();
   const float mean = sh[0], kdy = sh[1], kx = sh[2], k0 = sh[3];
-  BN_SEG_LOOP_BEGIN(g)
-    Vec<T, VEC> v, w;
-    v.load(x, off);
-    w.load(dy, off);
+  bn_seg_visit<VEC, true>(g, [&](const size_t (&off)[BN_UN], int n) {
+    Vec<T, VEC> v[BN_UN], w[BN_UN];
 #pragma unroll
-    for (int k = 0; k < VEC; ++k) v.v[k] = kdy * w.v[k] + (kx * (v.v[k] - mean) + k0);
-    v.store(dx, off);
-  BN_SEG_LOOP_END(g)
+    for (int k = 0; k < BN_UN; ++k) {
+      v[k].load(x, off[k]);
+      w[k].load(dy, off[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < BN_UN; ++k) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v[k].v[e] = kdy * w[k].v[e] + (kx * (v[k].v[e] - mean) + k0);
+      if (k < n) v[k].store(dx, off[k]);
+    }
+  });
 }
 
 // ---- column mode (inner == 1) ----------------------------------------------
@@ -392,11 +447,11 @@ static int make_geom(const flhip_bn_desc* d, BnGeom* g, int* vec) {
     g->ups = (g->units + S - 1) / S;
     g->step_o = g->step_i = 0;
   } else {
-    FLHIP_REQUIRE(d->C <= 65535, "batchnorm: spatial mode supports at most 65535 features");
+    FLHIP_REQUIRE(d->C <= 0x7fffffffLL, "batchnorm: too many features");
     *vec = (d->inner % 4 == 0) ? 4 : 1;
     const long long innerV = d->inner / *vec;
     g->units = d->outer * innerV;
-    long long S = 4096 / d->C;
+    long long S = 8192 / d->C;
     const long long maxS = (g->units + 511) / 512;
     if (S > maxS) S = maxS;
     if (S > 64) S = 64;
@@ -420,7 +475,7 @@ static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws
                        (const float*)nullptr, ws);
     hipLaunchKernelGGL((bn_train_apply_col<T>), grid, dim3(256), 0, s, g, xp, yp, ws, a);
   } else {
-    const dim3 grid(g.S, (unsigned)g.C);
+    const dim3 grid((unsigned)g.C, g.S);
     if (vec == 4) {
       hipLaunchKernelGGL((bn_stats_seg<T, 4>), grid, dim3(256), 0, s, g, xp, ws);
       hipLaunchKernelGGL((bn_train_apply_seg<T, 4>), grid, dim3(256), 0, s, g, xp, yp, ws, a);
@@ -443,7 +498,7 @@ static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void
     hipLaunchKernelGGL((bn_stats_col<T, true>), grid, dim3(256), 0, s, g, xp, dyp, a.save_mean, ws);
     hipLaunchKernelGGL((bn_bwd_apply_col<T>), grid, dim3(256), 0, s, g, xp, dyp, dxp, ws, a);
   } else {
-    const dim3 grid(g.S, (unsigned)g.C);
+    const dim3 grid((unsigned)g.C, g.S);
     if (vec == 4) {
       hipLaunchKernelGGL((bn_bwd_stats_seg<T, 4>), grid, dim3(256), 0, s, g, xp, dyp, a.save_mean, ws);
       hipLaunchKernelGGL((bn_bwd_apply_seg<T, 4>), grid, dim3(256), 0, s, g, xp, dyp, dxp, ws, a);

@@ -72,6 +72,20 @@ __device__ __forceinline__ void st4(bf16_t* p, size_t i, float4 v) {
   *reinterpret_cast<uint2*>(p + i) = r;
 }
 
+// Streaming stores: the result is not read again by the kernel that writes it, so
+// it should not displace re-used input lines from the caches.
+typedef float floatx4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uintx2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void st4_stream(float* p, size_t i, float4 v) {
+  const floatx4_t t = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(t, reinterpret_cast<floatx4_t*>(p + i));
+}
+__device__ __forceinline__ void st4_stream(bf16_t* p, size_t i, float4 v) {
+  const uintx2_t t = {(uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16),
+                      (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16)};
+  __builtin_nontemporal_store(t, reinterpret_cast<uintx2_t*>(p + i));
+}
+
 // ---- buffer loads ------------------------------------------------------------
 // Raw buffer descriptor over `bytes` bytes at p: loads at a byte offset at or
 // past `bytes` return zero, which is how the gathers fetch padding.

@@ -329,15 +329,15 @@ pool_w3s2_bwd(PoolGeom g, const T* __restrict__ dy, const uint8_t* __restrict__ 
     float4 even = make_float4(0.f, 0.f, 0.f, 0.f);
     pool_bwd_row<MODE>(q, 1, even);
     if (active && ok) {
-      if (2 * oh - 1 >= 0) st4(dxq, (size_t)(2 * oh - 1) * g.W, odd);
-      if (2 * oh < g.H) st4(dxq, (size_t)(2 * oh) * g.W, even);
+      if (2 * oh - 1 >= 0) st4_stream(dxq, (size_t)(2 * oh - 1) * g.W, odd);
+      if (2 * oh < g.H) st4_stream(dxq, (size_t)(2 * oh) * g.W, even);
     }
     odd = make_float4(0.f, 0.f, 0.f, 0.f);
     pool_bwd_row<MODE>(q, 2, odd);
     // last output row of the image: nothing below adds to row 2*oh+1
     if (active && ok && oh == g.OH - 1) {
       for (int r = 2 * oh + 1; r < g.H; ++r) {
-        st4(dxq, (size_t)r * g.W, odd);
+        st4_stream(dxq, (size_t)r * g.W, odd);
         odd = make_float4(0.f, 0.f, 0.f, 0.f);
       }
     }
