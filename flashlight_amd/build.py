@@ -36,6 +36,38 @@ def _compile(src):
     return obj
 
 
+HOST = os.path.join(HERE, "host")
+HOST_LIB = os.path.join(LIBDIR, "libflhip_host.so")
+HOST_SOURCES = ["HipTensor.cpp", "HipAutogradExtension.cpp", "Functions.cpp"]
+HOST_TEST_SRC = os.path.join(ROOT, "tests", "cpp", "test_host_extension.cpp")
+HOST_TEST_BIN = os.path.join(ROOT, "tests", "cpp", "bin", "test_host_extension")
+
+
+def build_host(verbose=True):
+    """The C++ host layer (HipTensor, HipAutogradExtension, caller closures) and its
+    test program; both link libflhip.so, the test also links the CPU checker."""
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cxx = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-Wall", "-D__HIP_PLATFORM_AMD__",
+           "-I" + os.path.join(rocm, "include"), "-I" + os.path.join(ROOT, "include"), "-I" + HOST]
+    hiplibs = ["-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(rocm, "lib")]
+    cmd = cxx + ["-fPIC", "-shared", "-o", HOST_LIB]
+    cmd += [os.path.join(HOST, f) for f in HOST_SOURCES]
+    cmd += ["-L" + LIBDIR, "-lflhip", "-Wl,-rpath,$ORIGIN"] + hiplibs
+    subprocess.check_call(cmd)
+    if os.path.exists(HOST_TEST_SRC):
+        os.makedirs(os.path.dirname(HOST_TEST_BIN), exist_ok=True)
+        oracle = os.path.join(ROOT, "oracle")
+        subprocess.check_call(["make", "-C", oracle, "libflref.so"], stdout=subprocess.DEVNULL)
+        cmd = cxx + ["-I" + oracle, "-o", HOST_TEST_BIN, HOST_TEST_SRC,
+                     "-L" + LIBDIR, "-lflhip_host", "-lflhip", "-L" + oracle, "-lflref",
+                     "-Wl,-rpath,$ORIGIN/../../../flashlight_amd/lib",
+                     "-Wl,-rpath,$ORIGIN/../../../oracle"] + hiplibs
+        subprocess.check_call(cmd)
+    if verbose:
+        print("built", HOST_LIB)
+    return HOST_LIB
+
+
 def build(verbose=True):
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
@@ -45,6 +77,7 @@ def build(verbose=True):
     subprocess.check_call(cmd)
     if verbose:
         print("built", LIB)
+    build_host(verbose)
     return LIB
 
 

@@ -48,6 +48,8 @@ SYMBOLS = {
     "flhip_bn_bwd": (C.c_int, [C.POINTER(BnDesc), _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
                                 _SZ, _VP]),
     "flhip_copy_bytes": (C.c_int, [_VP, _VP, _SZ, _VP]),
+    "flhip_convert": (C.c_int, [_VP, C.c_int, _VP, C.c_int, _SZ, _VP]),
+    "flhip_add": (C.c_int, [_VP, _VP, _VP, _SZ, C.c_int, _VP]),
 }
 
 _lib = None

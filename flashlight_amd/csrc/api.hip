@@ -19,6 +19,21 @@ __global__ void __launch_bounds__(256) copy16_kernel(const uint4* __restrict__ s
     dst[i] = src[i];
 }
 
+template <typename S, typename D>
+__global__ void __launch_bounds__(256) convert_kernel(const S* __restrict__ src,
+                                                       D* __restrict__ dst, size_t n) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
+    st(dst, i, ld(src, i));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) add_kernel(const T* a, const T* b, T* out, size_t n) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
+    st(out, i, ld(a, i) + ld(b, i));
+}
+
 }  // namespace flhip
 
 using namespace flhip;
@@ -73,4 +88,40 @@ extern "C" int flhip_copy_bytes(const void* src, void* dst, size_t bytes, void* 
   hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
                      reinterpret_cast<const uint4*>(src), reinterpret_cast<uint4*>(dst), n16);
   return check_launch("copy_bytes");
+}
+
+extern "C" int flhip_convert(const void* src, int src_dtype, void* dst, int dst_dtype, size_t n,
+                             void* stream) {
+  FLHIP_REQUIRE(dtype_ok(src_dtype) && dtype_ok(dst_dtype), "convert: unknown dtype");
+  if (n == 0) return FLHIP_OK;
+  FLHIP_REQUIRE(src && dst, "convert: null pointer");
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  const dim3 grid((unsigned)blocks), block(256);
+  hipStream_t s = as_stream(stream);
+  if (src_dtype == FLHIP_F32 && dst_dtype == FLHIP_F32)
+    hipLaunchKernelGGL((convert_kernel<float, float>), grid, block, 0, s, (const float*)src, (float*)dst, n);
+  else if (src_dtype == FLHIP_F32)
+    hipLaunchKernelGGL((convert_kernel<float, bf16_t>), grid, block, 0, s, (const float*)src, (bf16_t*)dst, n);
+  else if (dst_dtype == FLHIP_F32)
+    hipLaunchKernelGGL((convert_kernel<bf16_t, float>), grid, block, 0, s, (const bf16_t*)src, (float*)dst, n);
+  else
+    hipLaunchKernelGGL((convert_kernel<bf16_t, bf16_t>), grid, block, 0, s, (const bf16_t*)src, (bf16_t*)dst, n);
+  return check_launch("convert");
+}
+
+extern "C" int flhip_add(const void* a, const void* b, void* out, size_t n, int dtype,
+                         void* stream) {
+  FLHIP_REQUIRE(dtype_ok(dtype), "add: unknown dtype");
+  if (n == 0) return FLHIP_OK;
+  FLHIP_REQUIRE(a && b && out, "add: null pointer");
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  if (dtype == FLHIP_F32)
+    hipLaunchKernelGGL((add_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                       (const float*)a, (const float*)b, (float*)out, n);
+  else
+    hipLaunchKernelGGL((add_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0,
+                       as_stream(stream), (const bf16_t*)a, (const bf16_t*)b, (bf16_t*)out, n);
+  return check_launch("add");
 }

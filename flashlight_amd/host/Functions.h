@@ -1,0 +1,61 @@
+// The caller side of the boundary: a minimal autograd Variable and the three
+// differentiable functions whose closures drive the extension, with the control
+// flow of flashlight/fl/autograd/Functions.cpp:1327-1565 (dtype checks, payload
+// creation, which backward op runs when) and the reverse-topological backward of
+// flashlight/fl/autograd/Variable.cpp:235-294.  Only what is needed to exercise
+// the extension the way Flashlight does is provided.
+#pragma once
+
+#include <functional>
+#include <memory>
+#include <vector>
+
+#include "AutogradExtension.h"
+
+namespace fl {
+
+class Variable {
+ public:
+  using GradFunc = std::function<void(std::vector<Variable>& inputs, const Variable& gradOutput)>;
+
+  Variable() : data_(std::make_shared<Tensor>()), grad_(std::make_shared<SharedGrad>()) {}
+  Variable(Tensor data, bool calcGrad);
+  Variable(Tensor data, std::vector<Variable> inputs, GradFunc gradFunc);
+
+  Tensor& tensor() const { return *data_; }
+  const Shape& shape() const { return data_->shape(); }
+  dtype type() const { return data_->type(); }
+  bool isEmpty() const { return data_->isEmpty(); }
+  bool isCalcGrad() const { return grad_->calcGrad; }
+  bool isGradAvailable() const { return grad_->grad != nullptr; }
+  Variable& grad() const;
+  void addGrad(const Variable& childGrad);
+  void zeroGrad() { grad_->grad.reset(); }
+  void backward(const Variable& grad, bool retainGraph = false);
+
+ private:
+  struct SharedGrad {
+    bool calcGrad = false;
+    std::vector<Variable> inputs;
+    std::unique_ptr<Variable> grad;
+    GradFunc gradFunc;
+  };
+  std::vector<Variable> build() const;   // nodes in topological order
+  std::shared_ptr<Tensor> data_;
+  std::shared_ptr<SharedGrad> grad_;
+};
+
+// fl::derivePadding (flashlight/fl/nn/Utils.cpp:87-100); pad == -1 is SAME
+int derivePadding(int inSz, int filterSz, int stride, int pad, int dilation);
+
+Variable conv2d(const Variable& input, const Variable& weights, const Variable& bias, int sx = 1,
+                int sy = 1, int px = 0, int py = 0, int dx = 1, int dy = 1, int groups = 1);
+Variable conv2d(const Variable& input, const Variable& weights, int sx = 1, int sy = 1,
+                int px = 0, int py = 0, int dx = 1, int dy = 1, int groups = 1);
+Variable pool2d(const Variable& input, int wx, int wy, int sx = 1, int sy = 1, int px = 0,
+                int py = 0, PoolingMode mode = PoolingMode::MAX);
+Variable batchnorm(const Variable& input, const Variable& weight, const Variable& bias,
+                   Variable& runningMean, Variable& runningVar, const std::vector<int>& axes,
+                   bool train, double momentum, double epsilon);
+
+}  // namespace fl

@@ -1,0 +1,364 @@
+#include "HipAutogradExtension.h"
+
+#include <algorithm>
+#include <map>
+#include <mutex>
+
+#include "flhip.h"
+
+namespace fl {
+
+// ---- registry ---------------------------------------------------------------
+namespace detail {
+namespace {
+struct Registry {
+  std::mutex m;
+  std::map<TensorBackendType, AutogradExtensionFactory> factories;
+  std::map<TensorBackendType, std::unique_ptr<AutogradExtension>> instances;
+};
+Registry& registry() {
+  static Registry r;
+  return r;
+}
+}  // namespace
+
+bool registerAutogradExtension(TensorBackendType backend, AutogradExtensionFactory f) {
+  Registry& r = registry();
+  std::lock_guard<std::mutex> lock(r.m);
+  // try_emplace semantics: the first registration for a backend stays
+  return r.factories.emplace(backend, std::move(f)).second;
+}
+}  // namespace detail
+
+AutogradExtension& getAutogradExtension(TensorBackendType backend) {
+  auto& r = detail::registry();
+  std::lock_guard<std::mutex> lock(r.m);
+  auto it = r.instances.find(backend);
+  if (it == r.instances.end()) {
+    auto f = r.factories.find(backend);
+    if (f == r.factories.end())
+      throw std::invalid_argument("no AutogradExtension registered for this tensor backend");
+    it = r.instances.emplace(backend, f->second()).first;
+  }
+  return *it->second;
+}
+
+// registers next to the cuDNN / oneDNN extensions of
+// flashlight/fl/autograd/tensor/AutogradExtensionBackends.h:28-42
+FL_REGISTER_AUTOGRAD_EXTENSION(HipAutogradExtension, Hip);
+
+// ---- helpers ----------------------------------------------------------------
+namespace {
+
+// status of the C ABI -> the exception kinds of the reference boundary
+// (flashlight/fl/autograd/tensor/backend/cudnn/CudnnUtils.cpp:88-99)
+void check(int rc) {
+  if (rc == FLHIP_OK) return;
+  if (rc == FLHIP_INVALID_ARGUMENT) throw std::invalid_argument(flhip_last_error());
+  throw std::runtime_error(flhip_last_error());
+}
+
+int dtypeTag(dtype t, const char* op) {
+  if (t == dtype::f32) return FLHIP_F32;
+  if (t == dtype::bf16) return FLHIP_BF16;
+  throw std::runtime_error(std::string(op) + ": data type not supported by the HIP autograd extension");
+}
+
+// fp32 view of a small parameter vector (bias, gamma, beta, statistics)
+Tensor asF32(const Tensor& t) { return (t.isEmpty() || t.type() == dtype::f32) ? t : t.astype(dtype::f32); }
+
+struct HipPool2DPayload : detail::AutogradPayloadData {
+  Tensor argmax;   // one byte per output: first maximum, window-relative index
+};
+struct HipBatchNormPayload : detail::AutogradPayloadData {
+  Tensor saveMean, saveInvStd;   // fp32 per feature
+};
+
+flhip_conv_desc convDesc(const Shape& in, const Tensor& weights, int sx, int sy, int px, int py,
+                         int dx, int dy, int groups, int tag, const char* op) {
+  if (in.ndim() != 4 || weights.ndim() != 4)
+    throw std::invalid_argument(std::string(op) + ": input and weights must have 4 dimensions");
+  flhip_conv_desc d{};
+  d.W = (int)in.dim(0); d.H = (int)in.dim(1); d.C = (int)in.dim(2); d.N = (int)in.dim(3);
+  d.KW = (int)weights.dim(0); d.KH = (int)weights.dim(1); d.K = (int)weights.dim(3);
+  d.sx = sx; d.sy = sy; d.px = px; d.py = py; d.dil_x = dx; d.dil_y = dy;
+  d.groups = groups; d.dtype = tag;
+  if (groups <= 0 || weights.dim(2) * groups != in.dim(2))
+    throw std::invalid_argument(std::string(op) + ": weights do not match the input channels");
+  return d;
+}
+
+// (outer, C, inner) of the view of onednn/BatchNorm.cpp:40-71 with the axis
+// check of :124-130
+flhip_bn_desc bnDesc(const Tensor& input, const std::vector<int>& axes, int tag) {
+  if (axes.empty()) throw std::invalid_argument("batchnorm: no feature axes");
+  const int maxAxis = *std::max_element(axes.begin(), axes.end());
+  const int minAxis = *std::min_element(axes.begin(), axes.end());
+  if ((int)axes.size() != maxAxis - minAxis + 1 || minAxis < 0 || maxAxis >= input.ndim())
+    throw std::invalid_argument("axis array should be continuous");
+  long long nfeat = 1;
+  for (int ax : axes) nfeat *= input.dim(ax);
+  flhip_bn_desc d{};
+  d.C = nfeat;
+  d.dtype = tag;
+  if (minAxis == 0) {
+    d.inner = 1;
+    d.outer = input.elements() / nfeat;
+  } else {
+    long long batch = 1;
+    for (int i = maxAxis + 1; i < input.ndim(); ++i) batch *= input.dim(i);
+    d.outer = batch;
+    d.inner = input.elements() / (nfeat * batch);
+  }
+  return d;
+}
+
+}  // namespace
+
+Tensor HipAutogradExtension::workspace(size_t bytes) {
+  if (bytes == 0) return Tensor();
+  if (ws_.bytes() < bytes) ws_ = Tensor({(Dim)bytes}, dtype::u8);
+  return ws_;
+}
+
+bool HipAutogradExtension::isDataTypeSupported(const dtype& type) const {
+  return type == dtype::f32 || type == dtype::bf16;
+}
+
+// ---- conv2d -------------------------------------------------------------------
+Tensor HipAutogradExtension::conv2d(const Tensor& input, const Tensor& weights, const Tensor& bias,
+                                    const int sx, const int sy, const int px, const int py,
+                                    const int dx, const int dy, const int groups,
+                                    std::shared_ptr<detail::AutogradPayload>) {
+  if (input.type() != weights.type())
+    throw std::invalid_argument("conv2d: input and weights must have the same type");
+  const int tag = dtypeTag(input.type(), "conv2d");
+  flhip_conv_desc d = convDesc(input.shape(), weights, sx, sy, px, py, dx, dy, groups, tag, "conv2d");
+  int32_t OH = 0, OW = 0;
+  check(flhip_conv2d_out_dims(&d, &OH, &OW));
+  const bool hasBias = bias.elements() > 0;       // onednn/Conv2D.cpp:71,189
+  if (hasBias && bias.elements() != d.K)
+    throw std::invalid_argument("conv2d: bias must have one element per output channel");
+  const Tensor b = asF32(bias);
+  Tensor output({OW, OH, d.K, d.N}, input.type());
+  const size_t wsBytes = flhip_conv2d_workspace_bytes(&d, FLHIP_CONV_FWD);
+  Tensor ws = workspace(wsBytes);
+  DevicePtr xp(input), wp(weights), bp(b), yp(output), wsp(ws);
+  check(flhip_conv2d_fwd(&d, xp.get(), wp.get(), static_cast<const float*>(bp.get()), yp.get(),
+                         wsp.get(), wsBytes, hipBackendStream()));
+  return output;
+}
+
+Tensor HipAutogradExtension::conv2dBackwardData(const Tensor& gradOutput, const Tensor& input,
+                                                const Tensor& weight, const int sx, const int sy,
+                                                const int px, const int py, const int dx,
+                                                const int dy, const int groups,
+                                                std::shared_ptr<DynamicBenchmark>,
+                                                std::shared_ptr<detail::AutogradPayload>) {
+  if (gradOutput.type() != weight.type())
+    throw std::invalid_argument("conv2dBackwardData: gradOutput and weights must have the same type");
+  const int tag = dtypeTag(gradOutput.type(), "conv2dBackwardData");
+  flhip_conv_desc d =
+      convDesc(input.shape(), weight, sx, sy, px, py, dx, dy, groups, tag, "conv2dBackwardData");
+  int32_t OH = 0, OW = 0;
+  check(flhip_conv2d_out_dims(&d, &OH, &OW));
+  if (gradOutput.shape() != Shape({OW, OH, d.K, d.N}))
+    throw std::invalid_argument("conv2dBackwardData: gradOutput shape does not match the geometry");
+  Tensor gradInput(input.shape(), gradOutput.type());   // onednn/Conv2D.cpp:285
+  const size_t wsBytes = flhip_conv2d_workspace_bytes(&d, FLHIP_CONV_BWD_DATA);
+  Tensor ws = workspace(wsBytes);
+  DevicePtr gp(gradOutput), wp(weight), op(gradInput), wsp(ws);
+  check(flhip_conv2d_bwd_data(&d, gp.get(), wp.get(), op.get(), wsp.get(), wsBytes,
+                              hipBackendStream()));
+  return gradInput;
+}
+
+std::pair<Tensor, Tensor> HipAutogradExtension::conv2dBackwardFilterBias(
+    const Tensor& gradOutput, const Tensor& input, const Tensor& weights, const Tensor& bias,
+    const int sx, const int sy, const int px, const int py, const int dx, const int dy,
+    const int groups, std::shared_ptr<DynamicBenchmark>, std::shared_ptr<DynamicBenchmark>,
+    std::shared_ptr<detail::AutogradPayload>) {
+  if (gradOutput.type() != input.type())
+    throw std::invalid_argument("conv2dBackwardFilterBias: gradOutput and input must have the same type");
+  const int tag = dtypeTag(input.type(), "conv2dBackwardFilterBias");
+  flhip_conv_desc d = convDesc(input.shape(), weights, sx, sy, px, py, dx, dy, groups, tag,
+                               "conv2dBackwardFilterBias");
+  int32_t OH = 0, OW = 0;
+  check(flhip_conv2d_out_dims(&d, &OH, &OW));
+  if (gradOutput.shape() != Shape({OW, OH, d.K, d.N}))
+    throw std::invalid_argument("conv2dBackwardFilterBias: gradOutput shape does not match the geometry");
+  // gradients are produced in fp32 (for bf16 storage: the master-weight precision)
+  Tensor gradWeights(weights.shape(), dtype::f32);
+  // the bias gradient comes from the same pass iff a bias was passed
+  // (onednn/Conv2D.cpp:411-415); the caller passes an empty one when it is not
+  // needed (flashlight/fl/autograd/Functions.cpp:1391-1395)
+  Tensor gradBias;
+  if (!bias.isEmpty()) gradBias = Tensor(bias.shape(), dtype::f32);
+  const size_t wsBytes = flhip_conv2d_workspace_bytes(&d, FLHIP_CONV_BWD_FILTER);
+  Tensor ws = workspace(wsBytes);
+  DevicePtr xp(input), gp(gradOutput), dwp(gradWeights), dbp(gradBias), wsp(ws);
+  check(flhip_conv2d_bwd_filter(&d, xp.get(), gp.get(), static_cast<float*>(dwp.get()),
+                                static_cast<float*>(dbp.get()), wsp.get(), wsBytes,
+                                hipBackendStream()));
+  return {gradWeights, gradBias};
+}
+
+// ---- pool2d -------------------------------------------------------------------
+namespace {
+flhip_pool_desc poolDesc(const Shape& in, int wx, int wy, int sx, int sy, int px, int py,
+                         PoolingMode mode, int tag) {
+  // missing trailing dimensions count as 1 (onednn/Pool2D.cpp:95-98)
+  flhip_pool_desc d{};
+  d.W = (int)in.dim(0);
+  d.H = in.ndim() > 1 ? (int)in.dim(1) : 1;
+  d.C = in.ndim() > 2 ? (int)in.dim(2) : 1;
+  d.N = in.ndim() > 3 ? (int)in.dim(3) : 1;
+  d.wx = wx; d.wy = wy; d.sx = sx; d.sy = sy; d.px = px; d.py = py;
+  d.mode = (int)mode;
+  d.dtype = tag;
+  return d;
+}
+}  // namespace
+
+Tensor HipAutogradExtension::pool2d(const Tensor& input, const int wx, const int wy, const int sx,
+                                    const int sy, const int px, const int py,
+                                    const PoolingMode mode,
+                                    std::shared_ptr<detail::AutogradPayload> autogradPayload) {
+  if (input.ndim() < 1 || input.ndim() > 4)
+    throw std::invalid_argument("pool2d: input must have 1 to 4 dimensions");
+  const bool train = autogradPayload != nullptr;    // onednn/Pool2D.cpp:88
+  flhip_pool_desc d = poolDesc(input.shape(), wx, wy, sx, sy, px, py, mode, dtypeTag(input.type(), "pool2d"));
+  int32_t OH = 0, OW = 0;
+  check(flhip_pool2d_out_dims(&d, &OH, &OW));
+  Tensor output({OW, OH, d.C, d.N}, input.type());
+  auto payload = std::make_shared<HipPool2DPayload>();
+  if (train && mode == PoolingMode::MAX) payload->argmax = Tensor({OW, OH, d.C, d.N}, dtype::u8);
+  if (train) autogradPayload->data = payload;
+  DevicePtr xp(input), yp(output), ap(payload->argmax);
+  check(flhip_pool2d_fwd(&d, xp.get(), yp.get(), static_cast<uint8_t*>(ap.get()), hipBackendStream()));
+  return output;
+}
+
+Tensor HipAutogradExtension::pool2dBackward(const Tensor& gradOutput, const Tensor& input,
+                                            const Tensor&, const int wx, const int wy,
+                                            const int sx, const int sy, const int px, const int py,
+                                            const PoolingMode mode,
+                                            std::shared_ptr<detail::AutogradPayload> autogradPayload) {
+  if (!autogradPayload || !autogradPayload->data)   // onednn/Pool2D.cpp:190-193
+    throw std::invalid_argument("HipAutogradExtension::pool2dBackward given null or empty payload");
+  auto payload = std::dynamic_pointer_cast<HipPool2DPayload>(autogradPayload->data);
+  if (!payload) throw std::invalid_argument("pool2dBackward: payload of another operation");
+  flhip_pool_desc d =
+      poolDesc(input.shape(), wx, wy, sx, sy, px, py, mode, dtypeTag(gradOutput.type(), "pool2dBackward"));
+  int32_t OH = 0, OW = 0;
+  check(flhip_pool2d_out_dims(&d, &OH, &OW));
+  if (gradOutput.elements() != (Dim)OW * OH * d.C * d.N)
+    throw std::invalid_argument("pool2dBackward: gradOutput shape does not match the geometry");
+  // the reference allocates f32 whatever the input type (onednn/Pool2D.cpp:197),
+  // which its own caller cannot add to a non-f32 gradient; here the gradient has
+  // the type of gradOutput
+  Tensor gradInput(input.shape(), gradOutput.type());
+  DevicePtr gp(gradOutput), ap(payload->argmax), op(gradInput);
+  check(flhip_pool2d_bwd(&d, gp.get(), static_cast<const uint8_t*>(ap.get()), op.get(),
+                         hipBackendStream()));
+  return gradInput;
+}
+
+// ---- batchnorm ------------------------------------------------------------------
+Tensor HipAutogradExtension::batchnorm(Tensor& saveMean, Tensor& saveVar, const Tensor& input,
+                                       const Tensor& weight, const Tensor& bias,
+                                       Tensor& runningMean, Tensor& runningVar,
+                                       const std::vector<int>& axes, const bool train,
+                                       const double momentum, const double epsilon,
+                                       std::shared_ptr<detail::AutogradPayload> autogradPayload) {
+  const int tag = dtypeTag(input.type(), "batchnorm");
+  flhip_bn_desc d = bnDesc(input, axes, tag);
+  const Dim nfeat = (Dim)d.C;
+  for (const Tensor* t : {&weight, &bias, static_cast<const Tensor*>(&runningMean),
+                          static_cast<const Tensor*>(&runningVar)})
+    if (!t->isEmpty() && t->elements() != nfeat)
+      throw std::invalid_argument("batchnorm: parameters must have one element per feature");
+  // empty running statistics are created (onednn/BatchNorm.cpp:116-122); they stay fp32
+  if (runningVar.isEmpty()) runningVar = Tensor::full({nfeat}, 1., dtype::f32);
+  if (runningMean.isEmpty()) runningMean = Tensor::full({nfeat}, 0., dtype::f32);
+  if (runningMean.type() != dtype::f32 || runningVar.type() != dtype::f32)
+    throw std::invalid_argument("batchnorm: running statistics must be f32");
+  const Tensor gamma = asF32(weight), beta = asF32(bias);   // empty = no affine (:136-139)
+  Tensor output(input.shape(), input.type());
+  DevicePtr xp(input), gp(gamma), bp(beta), yp(output), rmp(runningMean), rvp(runningVar);
+  if (!train) {
+    check(flhip_bn_fwd_infer(&d, xp.get(), static_cast<const float*>(gp.get()),
+                             static_cast<const float*>(bp.get()),
+                             static_cast<const float*>(rmp.get()),
+                             static_cast<const float*>(rvp.get()), epsilon, yp.get(),
+                             hipBackendStream()));
+    return output;
+  }
+  // like the cuDNN extension (cudnn/BatchNorm.cpp:138-162): saveMean holds the batch
+  // mean, saveVar the inverse standard deviation, both f32
+  saveMean = Tensor({nfeat}, dtype::f32);
+  saveVar = Tensor({nfeat}, dtype::f32);
+  const size_t wsBytes = flhip_bn_workspace_bytes(&d);
+  Tensor ws = workspace(wsBytes);
+  DevicePtr smp(saveMean), sip(saveVar), wsp(ws);
+  check(flhip_bn_fwd_train(&d, xp.get(), static_cast<const float*>(gp.get()),
+                           static_cast<const float*>(bp.get()), yp.get(),
+                           static_cast<float*>(smp.get()), static_cast<float*>(sip.get()),
+                           static_cast<float*>(rmp.get()), static_cast<float*>(rvp.get()), momentum,
+                           epsilon, wsp.get(), wsBytes, hipBackendStream()));
+  if (autogradPayload) {
+    auto payload = std::make_shared<HipBatchNormPayload>();
+    payload->saveMean = saveMean;
+    payload->saveInvStd = saveVar;
+    autogradPayload->data = payload;
+  }
+  return output;
+}
+
+std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::batchnormBackward(
+    const Tensor& gradOutput, const Tensor& saveMean, const Tensor& saveVar, const Tensor& input,
+    const Tensor& weight, const std::vector<int>& axes, const bool train, const float,
+    std::shared_ptr<detail::AutogradPayload> autogradPayload) {
+  if (!train)   // cudnn/BatchNorm.cpp:196-199
+    throw std::logic_error("HipAutogradExtension::batchnormBackward: only train mode has a backward pass");
+  Tensor mean = saveMean, invstd = saveVar;
+  if (autogradPayload && autogradPayload->data) {
+    auto payload = std::dynamic_pointer_cast<HipBatchNormPayload>(autogradPayload->data);
+    if (!payload) throw std::invalid_argument("batchnormBackward: payload of another operation");
+    mean = payload->saveMean;
+    invstd = payload->saveInvStd;
+  }
+  if (mean.isEmpty() || invstd.isEmpty())   // onednn/BatchNorm.cpp:212-215
+    throw std::invalid_argument("HipAutogradExtension::batchnormBackward given null or empty payload");
+  if (gradOutput.type() != input.type() || gradOutput.shape() != input.shape())
+    throw std::invalid_argument("batchnormBackward: gradOutput must match the input");
+  flhip_bn_desc d = bnDesc(input, axes, dtypeTag(input.type(), "batchnormBackward"));
+  const Dim nfeat = (Dim)d.C;
+  const Tensor gamma = asF32(weight);
+  Tensor gradInput(input.shape(), input.type());
+  Tensor gradWeight({nfeat}, dtype::f32), gradBias({nfeat}, dtype::f32);
+  const size_t wsBytes = flhip_bn_workspace_bytes(&d);
+  Tensor ws = workspace(wsBytes);
+  DevicePtr xp(input), dyp(gradOutput), gp(gamma), mp(mean), ip(invstd), dxp(gradInput),
+      dgp(gradWeight), dbp(gradBias), wsp(ws);
+  check(flhip_bn_bwd(&d, xp.get(), dyp.get(), static_cast<const float*>(gp.get()),
+                     static_cast<const float*>(mp.get()), static_cast<const float*>(ip.get()),
+                     dxp.get(), static_cast<float*>(dgp.get()), static_cast<float*>(dbp.get()),
+                     wsp.get(), wsBytes, hipBackendStream()));
+  return std::make_tuple(gradInput, gradWeight, gradBias);   // always all three (:278)
+}
+
+// ---- rnn: not part of this backend ------------------------------------------------
+std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::rnn(
+    const Tensor&, const Tensor&, const Tensor&, const Tensor&, const int, const int, const RnnMode,
+    const bool, const float, std::shared_ptr<detail::AutogradPayload>) {
+  throw std::runtime_error("HipAutogradExtension::rnn is not implemented");
+}
+std::tuple<Tensor, Tensor, Tensor, Tensor> HipAutogradExtension::rnnBackward(
+    const Tensor&, const Tensor&, const Tensor&, const Tensor&,
+    const std::shared_ptr<detail::RNNGradData>, const Tensor&, const int, const int, const RnnMode,
+    const bool, const float, std::shared_ptr<detail::AutogradPayload>) {
+  throw std::runtime_error("HipAutogradExtension::rnnBackward is not implemented");
+}
+
+}  // namespace fl

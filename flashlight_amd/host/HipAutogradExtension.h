@@ -1,0 +1,60 @@
+// AutogradExtension for MI355X: every op lowers to one C ABI call of libflhip on
+// device-resident tensors.  Peer of OneDnnAutogradExtension / CudnnAutogradExtension
+// (flashlight/fl/autograd/tensor/backend/{onednn,cudnn}).
+#pragma once
+
+#include "AutogradExtension.h"
+
+namespace fl {
+
+class HipAutogradExtension : public AutogradExtension {
+ public:
+  // f32 and the private bf16 tag; the oneDNN extension supports everything but f16
+  // (onednn/OneDnnAutogradExtension.cpp:12-16), the cuDNN one f16/f32/f64.
+  bool isDataTypeSupported(const dtype& type) const override;
+
+  Tensor conv2d(const Tensor& input, const Tensor& weights, const Tensor& bias, const int sx,
+                const int sy, const int px, const int py, const int dx, const int dy,
+                const int groups, std::shared_ptr<detail::AutogradPayload> payload) override;
+  Tensor pool2d(const Tensor& input, const int wx, const int wy, const int sx, const int sy,
+                const int px, const int py, const PoolingMode mode,
+                std::shared_ptr<detail::AutogradPayload> payload) override;
+  Tensor batchnorm(Tensor& saveMean, Tensor& saveVar, const Tensor& input, const Tensor& weight,
+                   const Tensor& bias, Tensor& runningMean, Tensor& runningVar,
+                   const std::vector<int>& axes, const bool train, const double momentum,
+                   const double epsilon, std::shared_ptr<detail::AutogradPayload> payload) override;
+  std::tuple<Tensor, Tensor, Tensor> rnn(const Tensor&, const Tensor&, const Tensor&,
+                                         const Tensor&, const int, const int, const RnnMode,
+                                         const bool, const float,
+                                         std::shared_ptr<detail::AutogradPayload>) override;
+
+  Tensor conv2dBackwardData(const Tensor& gradOutput, const Tensor& input, const Tensor& weight,
+                            const int sx, const int sy, const int px, const int py, const int dx,
+                            const int dy, const int groups,
+                            std::shared_ptr<DynamicBenchmark> dataGradBenchmark,
+                            std::shared_ptr<detail::AutogradPayload> payload) override;
+  std::pair<Tensor, Tensor> conv2dBackwardFilterBias(
+      const Tensor& gradOutput, const Tensor& input, const Tensor& weights, const Tensor& bias,
+      const int sx, const int sy, const int px, const int py, const int dx, const int dy,
+      const int groups, std::shared_ptr<DynamicBenchmark> filterBench,
+      std::shared_ptr<DynamicBenchmark> biasBench,
+      std::shared_ptr<detail::AutogradPayload> autogradPayload) override;
+  Tensor pool2dBackward(const Tensor& gradOutput, const Tensor& input, const Tensor& poolOutput,
+                        const int wx, const int wy, const int sx, const int sy, const int px,
+                        const int py, const PoolingMode mode,
+                        std::shared_ptr<detail::AutogradPayload> payload) override;
+  std::tuple<Tensor, Tensor, Tensor> batchnormBackward(
+      const Tensor& gradOutput, const Tensor& saveMean, const Tensor& saveVar, const Tensor& input,
+      const Tensor& weight, const std::vector<int>& axes, const bool train, const float epsilon,
+      std::shared_ptr<detail::AutogradPayload> payload) override;
+  std::tuple<Tensor, Tensor, Tensor, Tensor> rnnBackward(
+      const Tensor&, const Tensor&, const Tensor&, const Tensor&,
+      const std::shared_ptr<detail::RNNGradData>, const Tensor&, const int, const int,
+      const RnnMode, const bool, const float, std::shared_ptr<detail::AutogradPayload>) override;
+
+ private:
+  Tensor workspace(size_t bytes);   // grown on demand, reused across calls
+  Tensor ws_;
+};
+
+}  // namespace fl

@@ -184,6 +184,18 @@ int flhip_bn_bwd(const flhip_bn_desc* d, const void* x, const void* dy,
                  const float* save_invstd, void* dx, float* dgamma,
                  float* dbeta, void* ws, size_t ws_bytes, void* stream);
 
+/* Storage conversion between FLHIP_F32 and FLHIP_BF16 (round to nearest even) of n
+ * elements; same dtype = copy.  Serves the casts the caller closures make around
+ * the extension (Tensor::astype in flashlight/fl/autograd/Functions.cpp:1558-1561
+ * and FL_ADJUST_INPUT_TYPE, flashlight/fl/autograd/Functions.h:57-82). */
+int flhip_convert(const void* src, int src_dtype, void* dst, int dst_dtype,
+                  size_t n, void* stream);
+
+/* out = a + b over n elements of `dtype` (out may alias a or b): the gradient
+ * accumulation of Variable::addGrad (flashlight/fl/autograd/Variable.cpp:185-218). */
+int flhip_add(const void* a, const void* b, void* out, size_t n, int dtype,
+              void* stream);
+
 /* Plain device-to-device copy kernel of `bytes` bytes (multiple of 16).  Not part
  * of the operator interface: it is the known-size kernel that hardware byte
  * counters are calibrated against when measuring the kernels above. */

@@ -1,0 +1,291 @@
+// GPU test of the C++ host layer: tensors, registration, HipAutogradExtension and
+// the caller closures, checked against the CPU checker (oracle/flref.c).  The
+// cases re-express the reference's own tests for this path:
+//   flashlight/fl/test/tensor/TensorExtensionTest.cpp:24-68 (extension reachable),
+//   flashlight/fl/test/autograd/AutogradConv2DTest.cpp:21-74,137-162 (shapes),
+//   flashlight/fl/test/autograd/AutogradTest.cpp:65-81,333-337 (dtype errors, pool),
+//   flashlight/fl/test/autograd/AutogradNormalizationTest.cpp:158-189 (batchnorm),
+//   flashlight/fl/test/nn/ModuleTest.cpp:338-353 (batching invariance).
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "Functions.h"
+#include "HipAutogradExtension.h"
+#include "flref.h"
+
+using namespace fl;
+
+static int g_fail = 0;
+#define CHECK(cond)                                                          \
+  do {                                                                       \
+    if (!(cond)) {                                                           \
+      std::printf("  FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);        \
+      ++g_fail;                                                              \
+    }                                                                        \
+  } while (0)
+
+static std::vector<float> randn(size_t n, unsigned seed, float scale = 1.f, float shift = 0.f) {
+  std::mt19937 gen(seed);
+  std::normal_distribution<float> d(0.f, 1.f);
+  std::vector<float> v(n);
+  for (auto& x : v) x = d(gen) * scale + shift;
+  return v;
+}
+static double relL2(const std::vector<float>& a, const std::vector<float>& b) {
+  double num = 0, den = 0;
+  if (a.size() != b.size()) return 1e30;
+  for (size_t i = 0; i < a.size(); ++i) {
+    num += ((double)a[i] - b[i]) * ((double)a[i] - b[i]);
+    den += (double)b[i] * b[i];
+  }
+  return den > 0 ? std::sqrt(num / den) : std::sqrt(num);
+}
+static float bf16round(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  u &= 0xffff0000u;
+  std::memcpy(&f, &u, 4);
+  return f;
+}
+template <typename E>
+static bool throws(const std::function<void()>& f) {
+  try {
+    f();
+  } catch (const E&) {
+    return true;
+  } catch (...) {
+    return false;
+  }
+  return false;
+}
+
+static void testRegistration() {
+  std::printf("registration\n");
+  AutogradExtension& e = getAutogradExtension(TensorBackendType::Hip);
+  CHECK(dynamic_cast<HipAutogradExtension*>(&e) != nullptr);
+  CHECK(&e == &getAutogradExtension(TensorBackendType::Hip));       // one instance per backend
+  CHECK(e.isDataTypeSupported(dtype::f32) && e.isDataTypeSupported(dtype::bf16));
+  CHECK(!e.isDataTypeSupported(dtype::f16) && !e.isDataTypeSupported(dtype::f64));
+  CHECK(e.createBenchmarkOptions() == nullptr);
+  // a second registration for the same backend is ignored (TensorExtension.cpp:27-29)
+  CHECK(!detail::registerAutogradExtension(TensorBackendType::Hip, [] {
+    return std::unique_ptr<AutogradExtension>(new HipAutogradExtension());
+  }));
+  CHECK(throws<std::invalid_argument>([] { getAutogradExtension(TensorBackendType::Stub); }));
+  CHECK(throws<std::runtime_error>([&] {
+    Tensor t;
+    e.rnn(t, t, t, t, 1, 1, RnnMode::LSTM, false, 0.f, nullptr);
+  }));
+}
+
+static void testConv(dtype dt, int groups, double tol) {
+  std::printf("conv2d %s groups=%d\n", dt == dtype::f32 ? "f32" : "bf16", groups);
+  // input [10,9,8,7], weights [4,3,8/groups,6], px=2, py=1
+  const int W = 10, H = 9, C = 8, N = 7, KW = 4, KH = 3, K = 6, px = 2, py = 1;
+  flref_conv d{N, C, H, W, K, KH, KW, 1, 1, py, px, 1, 1, groups};
+  int32_t OH, OW;
+  flref_conv_out(&d, &OH, &OW);
+  auto x = randn((size_t)N * C * H * W, 1), w = randn((size_t)K * (C / groups) * KH * KW, 2, 0.2f);
+  auto b = randn(K, 3), dy = randn((size_t)N * K * OH * OW, 4);
+  if (dt == dtype::bf16) {
+    for (auto* v : {&x, &w, &b, &dy})
+      for (auto& f : *v) f = bf16round(f);
+  }
+  std::vector<float> y(dy.size()), dx(x.size()), dw(w.size()), db(K);
+  flref_conv2d_fwd(&d, x.data(), w.data(), b.data(), y.data());
+  flref_conv2d_bwd_data(&d, dy.data(), w.data(), dx.data());
+  flref_conv2d_bwd_filter(&d, x.data(), dy.data(), dw.data(), db.data());
+
+  Variable in(Tensor::fromVector({W, H, C, N}, x).astype(dt), true);
+  Variable wt(Tensor::fromVector({KW, KH, C / groups, K}, w).astype(dt), true);
+  Variable bs(Tensor::fromVector({1, 1, K, 1}, b).astype(dt), true);
+  Variable out = conv2d(in, wt, bs, 1, 1, px, py, 1, 1, groups);
+  CHECK(out.shape() == Shape({OW, OH, K, N}));
+  CHECK(out.type() == dt);
+  CHECK(relL2(out.tensor().toHostVector(), y) <= tol);
+  out.backward(Variable(Tensor::fromVector(out.shape(), dy).astype(dt), false));
+  CHECK(relL2(in.grad().tensor().toHostVector(), dx) <= tol);
+  CHECK(relL2(wt.grad().tensor().toHostVector(), dw) <= tol);
+  CHECK(relL2(bs.grad().tensor().toHostVector(), db) <= tol);
+  CHECK(in.grad().type() == dt && wt.grad().type() == dt && bs.grad().shape() == bs.shape());
+
+  // an input without gradient: backward-data is skipped (Functions.cpp:1407)
+  Variable in2(in.tensor(), false), wt2(wt.tensor(), true);
+  Variable out2 = conv2d(in2, wt2, 1, 1, px, py, 1, 1, groups);
+  out2.backward(Variable(Tensor::fromVector(out2.shape(), dy).astype(dt), false));
+  CHECK(!in2.isGradAvailable() && wt2.isGradAvailable());
+  CHECK(relL2(wt2.grad().tensor().toHostVector(), dw) <= tol);
+}
+
+static void testConvErrors() {
+  std::printf("conv2d errors\n");
+  Variable in(Tensor({8, 8, 4, 1}, dtype::f32), false);
+  Variable wbf(Tensor({3, 3, 4, 4}, dtype::bf16), false);
+  // mixed types are rejected before the boundary (AutogradTest.cpp:75-81)
+  CHECK(throws<std::invalid_argument>([&] { conv2d(in, wbf); }));
+  Variable wbad(Tensor({3, 3, 3, 4}, dtype::f32), false);
+  CHECK(throws<std::invalid_argument>([&] { conv2d(in, wbad); }));
+  Variable wbig(Tensor({9, 9, 4, 4}, dtype::f32), false);
+  CHECK(throws<std::invalid_argument>([&] { conv2d(in, wbig); }));
+  Variable f64(Tensor({8, 8, 4, 1}, dtype::f64), false), w64(Tensor({3, 3, 4, 4}, dtype::f64), false);
+  CHECK(throws<std::runtime_error>([&] { conv2d(f64, w64); }));
+}
+
+static void testBatchingInvariance() {
+  std::printf("conv2d batching invariance\n");
+  // 30 -> 50 channels, 9x7 kernel, stride 2x3, padding 3x2 (ModuleTest.cpp:338-353)
+  const int W = 20, H = 17, C = 30, N = 4, K = 50;
+  auto x = randn((size_t)N * C * H * W, 5), w = randn((size_t)K * C * 7 * 9, 6, 0.03f);
+  Variable wt(Tensor::fromVector({9, 7, C, K}, w), false);
+  auto full = conv2d(Variable(Tensor::fromVector({W, H, C, N}, x), false), wt, 2, 3, 3, 2)
+                  .tensor().toHostVector();
+  const size_t per = full.size() / N;
+  for (int n = 0; n < N; ++n) {
+    std::vector<float> xi(x.begin() + (size_t)n * C * H * W, x.begin() + (size_t)(n + 1) * C * H * W);
+    auto one = conv2d(Variable(Tensor::fromVector({W, H, C, 1}, xi), false), wt, 2, 3, 3, 2)
+                   .tensor().toHostVector();
+    double worst = 0;
+    for (size_t i = 0; i < per; ++i) worst = std::max(worst, (double)std::fabs(one[i] - full[n * per + i]));
+    CHECK(worst <= 1e-5);
+  }
+}
+
+static void testPool() {
+  std::printf("pool2d\n");
+  const int W = 12, H = 10, C = 3, N = 2;
+  auto x = randn((size_t)N * C * H * W, 7);
+  for (auto& v : x) v = std::round(v * 8.f) / 8.f;   // ties
+  for (int mode = 0; mode < 3; ++mode) {
+    flref_pool d{N, C, H, W, 3, 3, 2, 2, 1, 1, mode};
+    int32_t OH, OW;
+    flref_pool_out(&d, &OH, &OW);
+    std::vector<float> y((size_t)N * C * OH * OW), dx(x.size());
+    std::vector<uint8_t> am(y.size());
+    auto dy = randn(y.size(), 8);
+    flref_pool2d_fwd(&d, x.data(), y.data(), am.data());
+    flref_pool2d_bwd(&d, dy.data(), am.data(), dx.data());
+    Variable in(Tensor::fromVector({W, H, C, N}, x), true);
+    Variable out = pool2d(in, 3, 3, 2, 2, 1, 1, (PoolingMode)mode);
+    CHECK(out.shape() == Shape({OW, OH, C, N}));
+    CHECK(out.tensor().toHostVector() == y);               // bit-exact
+    out.backward(Variable(Tensor::fromVector(out.shape(), dy), false));
+    CHECK(in.grad().tensor().toHostVector() == dx);        // bit-exact, tie routing included
+  }
+  // AutogradTest.cpp:333-337: 3x3x1x1 input, 2x2 window, stride 1
+  Variable small(Tensor::fromVector({3, 3, 1, 1}, randn(9, 9)), true);
+  CHECK(pool2d(small, 2, 2, 1, 1).shape() == Shape({2, 2, 1, 1}));
+  // missing trailing dimensions count as 1 (onednn/Pool2D.cpp:95-98)
+  Variable two(Tensor::fromVector({8, 6}, randn(48, 10)), false);
+  CHECK(pool2d(two, 2, 2, 2, 2).shape() == Shape({4, 3, 1, 1}));
+  // backward without the forward payload (onednn/Pool2D.cpp:190-193)
+  AutogradExtension& e = getAutogradExtension(TensorBackendType::Hip);
+  Tensor t({4, 4, 1, 1}, dtype::f32), g({2, 2, 1, 1}, dtype::f32);
+  CHECK(throws<std::invalid_argument>(
+      [&] { e.pool2dBackward(g, t, g, 2, 2, 2, 2, 0, 0, PoolingMode::MAX, nullptr); }));
+  CHECK(throws<std::invalid_argument>([&] { pool2d(small, 2, 2, 1, 1, 2, 2); }));   // pad >= window
+}
+
+static void testBatchnorm() {
+  std::printf("batchnorm\n");
+  const int W = 13, H = 13, C = 3, N = 8;
+  auto x = randn((size_t)N * C * H * W, 11, 1.4f, 0.5f), g = randn(C, 12, 0.1f, 1.f), b = randn(C, 13);
+  auto dy = randn(x.size(), 14);
+  std::vector<float> y(x.size()), mean(C), var(C), dx(x.size()), dg(C), db(C);
+  flref_bn_fwd_train(N, C, (int64_t)H * W, x.data(), g.data(), b.data(), 1e-5, y.data(), mean.data(), var.data());
+  flref_bn_bwd(N, C, (int64_t)H * W, x.data(), dy.data(), g.data(), mean.data(), var.data(), 1e-5,
+               dx.data(), dg.data(), db.data());
+  Variable in(Tensor::fromVector({W, H, C, N}, x), true);
+  Variable wt(Tensor::fromVector({C}, g), true), bs(Tensor::fromVector({C}, b), true);
+  Variable rm, rv;   // empty: created by the op (onednn/BatchNorm.cpp:116-122)
+  Variable out = batchnorm(in, wt, bs, rm, rv, {2}, true, 0.0, 1e-5);
+  CHECK(relL2(out.tensor().toHostVector(), y) <= 1e-4);
+  // momentum 0: running buffers hold the batch statistics (onednn/BatchNorm.cpp:154-157)
+  CHECK(relL2(rm.tensor().toHostVector(), mean) <= 1e-5);
+  CHECK(relL2(rv.tensor().toHostVector(), var) <= 1e-4);
+  out.backward(Variable(Tensor::fromVector(out.shape(), dy), false));
+  CHECK(relL2(in.grad().tensor().toHostVector(), dx) <= 1e-4);
+  CHECK(relL2(wt.grad().tensor().toHostVector(), dg) <= 1e-4);
+  CHECK(relL2(bs.grad().tensor().toHostVector(), db) <= 1e-4);
+
+  // momentum 0.1: r = 0.9 r + 0.1 batch with the unbiased variance
+  Variable rm2(Tensor::full({C}, 0., dtype::f32), false), rv2(Tensor::full({C}, 1., dtype::f32), false);
+  batchnorm(in, wt, bs, rm2, rv2, {2}, true, 0.1, 1e-5);
+  std::vector<float> erm(C, 0.f), erv(C, 1.f);
+  flref_bn_running_update(C, (int64_t)N * H * W, mean.data(), var.data(), 0.1, erm.data(), erv.data());
+  CHECK(relL2(rm2.tensor().toHostVector(), erm) <= 1e-5);
+  CHECK(relL2(rv2.tensor().toHostVector(), erv) <= 1e-4);
+
+  // inference with running statistics, with and without affine parameters
+  std::vector<float> yi(x.size());
+  flref_bn_fwd_infer(N, C, (int64_t)H * W, x.data(), g.data(), b.data(), erm.data(), erv.data(), 1e-5, yi.data());
+  Variable nograd(in.tensor(), false);
+  Variable wng(wt.tensor(), false), bng(bs.tensor(), false);
+  CHECK(relL2(batchnorm(nograd, wng, bng, rm2, rv2, {2}, false, 0.0, 1e-5).tensor().toHostVector(), yi) <= 1e-5);
+  flref_bn_fwd_infer(N, C, (int64_t)H * W, x.data(), nullptr, nullptr, erm.data(), erv.data(), 1e-5, yi.data());
+  Variable none1, none2;
+  CHECK(relL2(batchnorm(nograd, none1, none2, rm2, rv2, {2}, false, 0.0, 1e-5).tensor().toHostVector(), yi) <= 1e-5);
+
+  // per-activation mode, axes {0,1,2} (AutogradNormalizationTest.cpp:191-226)
+  const int64_t nf = (int64_t)W * H * C;
+  auto g3 = randn(nf, 15, 0.1f, 1.f), b3 = randn(nf, 16);
+  std::vector<float> y3(x.size()), m3(nf), v3(nf);
+  flref_bn_fwd_train(N, nf, 1, x.data(), g3.data(), b3.data(), 1e-5, y3.data(), m3.data(), v3.data());
+  Variable w3(Tensor::fromVector({(Dim)nf}, g3), false), bb3(Tensor::fromVector({(Dim)nf}, b3), false);
+  Variable rm3, rv3;
+  CHECK(relL2(batchnorm(nograd, w3, bb3, rm3, rv3, {0, 1, 2}, true, 0.0, 1e-5).tensor().toHostVector(), y3) <= 1e-4);
+
+  // errors: non-contiguous axes (onednn/BatchNorm.cpp:124-130), mixed types, missing payload
+  CHECK(throws<std::invalid_argument>([&] { batchnorm(nograd, none1, none2, rm3, rv3, {0, 2}, true, 0.0, 1e-5); }));
+  Variable wbf(wt.tensor().astype(dtype::bf16), false);
+  CHECK(throws<std::invalid_argument>([&] { batchnorm(nograd, wbf, none2, rm2, rv2, {2}, true, 0.0, 1e-5); }));
+  AutogradExtension& e = getAutogradExtension(TensorBackendType::Hip);
+  Tensor empty;
+  CHECK(throws<std::invalid_argument>(
+      [&] { e.batchnormBackward(in.tensor(), empty, empty, in.tensor(), wt.tensor(), {2}, true, 1e-5f, nullptr); }));
+}
+
+static void testGradAccumulation() {
+  std::printf("gradient accumulation\n");
+  // one input feeding two pools: the gradients add (Variable.cpp:185-218)
+  const int W = 8, H = 8;
+  auto x = randn(64, 17);
+  Variable in(Tensor::fromVector({W, H, 1, 1}, x), true);
+  Variable a = pool2d(in, 2, 2, 2, 2, 0, 0, PoolingMode::AVG_INCLUDE_PADDING);
+  std::vector<float> ones(16, 1.f);
+  a.backward(Variable(Tensor::fromVector(a.shape(), ones), false));
+  Variable b = pool2d(in, 2, 2, 2, 2, 0, 0, PoolingMode::AVG_INCLUDE_PADDING);
+  b.backward(Variable(Tensor::fromVector(b.shape(), ones), false));
+  auto g = in.grad().tensor().toHostVector();
+  bool ok = true;
+  for (float v : g) ok = ok && v == 0.5f;
+  CHECK(ok);
+}
+
+int main() {
+  try {
+    CHECK(derivePadding(56, 3, 1, -1, 1) == 1 && derivePadding(224, 7, 2, -1, 1) == 3 &&
+          derivePadding(56, 1, 2, -1, 1) == 0 && derivePadding(1500, 21, 2, -1, 1) == 10 &&
+          derivePadding(9, 3, 1, 4, 1) == 4);
+    testRegistration();
+    testConv(dtype::f32, 1, 1e-4);
+    testConv(dtype::f32, 2, 1e-4);
+    testConv(dtype::bf16, 1, 2e-2);
+    testConvErrors();
+    testBatchingInvariance();
+    testPool();
+    testBatchnorm();
+    testGradAccumulation();
+    fl::sync();
+  } catch (const std::exception& e) {
+    std::printf("unexpected exception: %s\n", e.what());
+    return 2;
+  }
+  std::printf(g_fail ? "%d check(s) FAILED\n" : "all host extension checks passed\n", g_fail);
+  return g_fail ? 1 : 0;
+}

@@ -1,0 +1,30 @@
+"""Runs the C++ test program of the host layer (HipTensor, registration,
+HipAutogradExtension, caller closures) on the GPU."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "tests", "cpp", "bin", "test_host_extension")
+
+
+@pytest.mark.gpu
+def test_host_extension_program():
+    assert os.path.exists(BIN), "build it with `python -m flashlight_amd.build`"
+    r = subprocess.run([BIN], capture_output=True, text=True, timeout=110)
+    print(r.stdout)
+    print(r.stderr)
+    assert r.returncode == 0, r.stdout[-3000:]
+    assert "all host extension checks passed" in r.stdout
+
+
+def test_host_library_is_built_and_links_the_c_abi():
+    lib = os.path.join(ROOT, "flashlight_amd", "lib", "libflhip_host.so")
+    assert os.path.exists(lib)
+    out = subprocess.run(["nm", "-D", "--defined-only", lib], capture_output=True, text=True).stdout
+    for sym in ("HipAutogradExtension", "getAutogradExtension", "conv2dBackwardFilterBias",
+                "batchnormBackward", "pool2dBackward"):
+        assert sym in out, sym
+    und = subprocess.run(["nm", "-D", "--undefined-only", lib], capture_output=True, text=True).stdout
+    assert "flhip_conv2d_bwd_filter" in und and "flhip_bn_bwd" in und
