@@ -26,7 +26,7 @@ PEAK = {"hbm_GBps": 8000.0, "f32_TFLOPs": 157.3, "bf16_TFLOPs": 2500.0}
 CONV_FLOP = 2 * 32 * 64 * 56 * 56 * 64 * 9          # one pass, 7.398752256e9
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by
 # the same counters on the library's copy kernel (see profiles/); None = not measured.
-MEASURED_TRAFFIC = {"conv2d_bwd_data_f32": None}
+MEASURED_TRAFFIC = {"conv2d_bwd_data_f32": 76.3e6}
 
 
 def parse():
@@ -196,6 +196,14 @@ def main():
         bw_op("pool2d_avg_bwd", wl, nx + ny,
               lambda i: L.flhip_pool2d_bwd(pdap, pdyp[i % nsets], None, pdxp, S), nsets)
         del px_, pdy, pam, pyo, pdx
+
+    if "copy" in only:
+        # known-size kernel for calibrating hardware byte counters (never part of the default run)
+        ca = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        cb = torch.empty_like(ca)
+        cap, cbp = P(ca), P(cb)
+        bw_op("copy", "flhip_copy_bytes 256 MiB", 2 * (256 << 20),
+              lambda i: L.flhip_copy_bytes(cap, cbp, 256 << 20, S), 1)
 
     torch.cuda.synchronize()
     by = {o["op"]: o for o in ops}
