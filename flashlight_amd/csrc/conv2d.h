@@ -21,4 +21,11 @@ int mfma_conv_bwd_filter(const ConvGeom& g, int dtype, const void* x, const void
                          float* db, void* ws, size_t ws_bytes, hipStream_t s);
 size_t mfma_conv_bwd_filter_ws(const ConvGeom& g, int dtype);
 
+// LDS-resident-slab kernels for stride-1 convolutions with small windows
+// (conv2d_mfma_slab.hip); same return convention.
+int mfma_slab_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w,
+                       const float* bias, void* y, hipStream_t s);
+int mfma_slab_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
+                            hipStream_t s);
+
 }  // namespace flhip

@@ -120,10 +120,13 @@ conv_bwd_bias_kernel(ConvGeom g, const T* __restrict__ dy, float* __restrict__ d
   if (threadIdx.x == 0) db[k] = acc;
 }
 
-static bool force_direct() {
+// FLHIP_CONV_ALGO: "direct" = one-thread-per-result kernels, "gather" = skip the
+// LDS-slab kernels; anything else = fastest applicable.
+static bool algo_is(const char* name) {
   const char* e = getenv("FLHIP_CONV_ALGO");
-  return e && strcmp(e, "direct") == 0;
+  return e && strcmp(e, name) == 0;
 }
+static bool force_direct() { return algo_is("direct"); }
 
 static int make_geom(const flhip_conv_desc* d, ConvGeom* g) {
   int32_t OH, OW;
@@ -160,7 +163,8 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
   if (rc != FLHIP_OK) return rc;
   hipStream_t s = as_stream(stream);
   if (!force_direct()) {
-    const int r = mfma_conv_fwd(g, d->dtype, x, w, bias, y, s);
+    int r = algo_is("gather") ? -1 : mfma_slab_conv_fwd(g, d->dtype, x, w, bias, y, s);
+    if (r < 0) r = mfma_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r >= 0) return r;
   }
   const size_t total = (size_t)g.N * g.K * g.OH * g.OW;
@@ -186,7 +190,8 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
   if (rc != FLHIP_OK) return rc;
   hipStream_t s = as_stream(stream);
   if (!force_direct()) {
-    const int r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s);
+    int r = algo_is("gather") ? -1 : mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s);
+    if (r < 0) r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r >= 0) return r;
   }
   const size_t total = (size_t)g.N * g.C * g.H * g.W;
