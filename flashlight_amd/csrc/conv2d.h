@@ -25,6 +25,10 @@ size_t mfma_conv_bwd_filter_ws(const ConvGeom& g, int dtype);
 // (conv2d_mfma_slab.hip); same return convention.
 int mfma_slab_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w,
                        const float* bias, void* y, hipStream_t s);
+int mfma_slab_wgrad(const ConvGeom& g, int dtype, const void* x, const void* dy, float* dw,
+                    float* db, void* ws, size_t ws_bytes, hipStream_t s);
+size_t mfma_slab_wgrad_ws(const ConvGeom& g, int dtype);
+bool mfma_slab_wgrad_applies(const ConvGeom& g);
 int mfma_slab_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
                             hipStream_t s);
 

@@ -148,7 +148,11 @@ using namespace flhip;
 extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pass) {
   ConvGeom g;
   if (make_geom(d, &g) != FLHIP_OK) return 0;
-  if (pass == FLHIP_CONV_BWD_FILTER) return mfma_conv_bwd_filter_ws(g, d->dtype);
+  if (pass == FLHIP_CONV_BWD_FILTER) {
+    // the larger of the two filter-gradient plans, so either kernel can run
+    const size_t a = mfma_conv_bwd_filter_ws(g, d->dtype), b = mfma_slab_wgrad_ws(g, d->dtype);
+    return a > b ? a : b;
+  }
   return 0;
 }
 
@@ -218,10 +222,10 @@ extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, 
   if (rc != FLHIP_OK) return rc;
   hipStream_t s = as_stream(stream);
   if (!force_direct()) {
-    FLHIP_REQUIRE(ws_bytes >= mfma_conv_bwd_filter_ws(g, d->dtype) &&
-                      (ws || mfma_conv_bwd_filter_ws(g, d->dtype) == 0),
-                  "conv2d_bwd_filter: workspace too small");
-    const int r = mfma_conv_bwd_filter(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
+    const size_t need = flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER);
+    FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter: workspace too small");
+    int r = algo_is("gather") ? -1 : mfma_slab_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
+    if (r < 0) r = mfma_conv_bwd_filter(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
     if (r >= 0) return r;
   }
   if (dw) {

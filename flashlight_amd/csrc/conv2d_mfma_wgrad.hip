@@ -323,6 +323,13 @@ bool wgrad_split(WgradParams* p, const ConvGeom& g) {
 
 }  // namespace
 
+void wgrad_reduce_launch(const float* part, int nsplit, int E, int K, int want_db, float* dw,
+                         float* db, hipStream_t s) {
+  const int total = E + (want_db ? K : 0);
+  hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((total + 63) / 64), dim3(256), 0, s, part, nsplit, E,
+                     K, want_db, dw, db);
+}
+
 size_t mfma_conv_bwd_filter_ws(const ConvGeom& g, int) {
   WgradParams p{};
   if (!wgrad_plan(g, &p) || !wgrad_split(&p, g)) return 0;

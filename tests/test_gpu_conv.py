@@ -28,6 +28,11 @@ MORE = [
     ((3, 30, 17, 20), (50, 30, 7, 9), (3, 2), (2, 3), (1, 1), 1),       # ModuleTest.cpp:338-353
     ((1, 130, 9, 9), (70, 130, 3, 3), (1, 1), (1, 1), (1, 1), 1),       # ragged channel counts
     ((2, 8, 6, 500), (8, 4, 3, 3), (1, 1), (1, 1), (1, 1), 2),          # wide rows, groups
+    ((2, 64, 28, 28), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),       # LDS-slab kernels (all three passes)
+    ((3, 32, 9, 12), (40, 32, 3, 3), (1, 1), (2, 2), (2, 2), 1),        # slab, dilation 2, ragged K, odd rows
+    ((2, 64, 10, 16), (96, 32, 3, 3), (1, 1), (1, 1), (1, 1), 2),       # slab, groups, two column halves... per group 32
+    ((1, 20, 12, 20), (24, 20, 3, 3), (1, 1), (0, 1), (1, 1), 1),       # slab fwd/bwd-data with a channel tail
+    ((2, 64, 7, 8), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),         # few rows per split
 ]
 ALL = LIB_CASES + MORE
 
