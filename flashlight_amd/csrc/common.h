@@ -99,6 +99,25 @@ __device__ __forceinline__ float buf_ld(__amdgpu_buffer_rsrc_t r, int byte_off, 
   return bf16_to_f32((bf16_t)__builtin_amdgcn_raw_buffer_load_b16(r, byte_off, 0, 0));
 }
 
+// ---- small-integer division ------------------------------------------------------
+// e / d for 0 <= e < 2^22 with inv = 1.0f / d: a float estimate corrected to the
+// exact quotient (a handful of VALU operations instead of the ~30 of an integer
+// division).  *rem receives e - q*d.
+__device__ __forceinline__ int fast_div(int e, int d, float inv, int* rem) {
+  int q = (int)((float)e * inv);
+  int r = e - q * d;
+  if (r < 0) {
+    --q;
+    r += d;
+  }
+  if (r >= d) {
+    ++q;
+    r -= d;
+  }
+  *rem = r;
+  return q;
+}
+
 // ---- reductions -----------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

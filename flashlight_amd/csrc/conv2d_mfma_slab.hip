@@ -10,7 +10,7 @@
 // innermost with an odd pitch (9 words): the k index of an MFMA fragment is then
 // a compile-time immediate offset and consecutive lanes hit distinct banks.
 //   slab   xs[position (row-major rows x cols)][9]   (8 channels + pad)
-//   weights as[64 result channels][tap][9]           (8 channels + pad)
+//   weights as[64 result channels][9 tap slots][9]   (8 channels + pad)
 // 8 waves, two roles (wave w and w+4 share a SIMD):
 //   waves 0-3 load chunk c+1 (global -> registers -> the LDS buffer not in use);
 //     what each thread loads is the same every chunk, so offsets are computed
@@ -79,6 +79,8 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
     // after the chunk offset is added, so its buffer load returns zero.
     constexpr int OOB = (int)0x80000000;
     const int slab_pos = p.RS * p.WS;
+    const float inv_slab = 1.0f / (float)slab_pos, inv_ws = 1.0f / (float)p.WS;
+    const float inv_khw = 1.0f / (float)p.KHW;
     const int nex = (CK * slab_pos + GTHREADS - 1) / GTHREADS;
     const int xdummy = p.slab_words - 1, adummy = p.a_words - 1;   // spare words of each buffer
     int xg[NEX_MAX], xl[NEX_MAX];                // global byte offset, LDS word offset
@@ -90,8 +92,9 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
       xg[i] = OOB;
       xl[i] = xdummy;
       if (i < nex && e < CK * slab_pos) {
-        const int c = e / slab_pos, q = e - c * slab_pos;
-        const int rs = q / p.WS, ws = q - rs * p.WS;
+        int q, ws;
+        const int c = fast_div(e, slab_pos, inv_slab, &q);
+        const int rs = fast_div(q, p.WS, inv_ws, &ws);
         const int sr = r0 + p.min_sh + rs, sc = p.min_sw + ws;
         xl[i] = q * PP + c;
         if ((unsigned)sr < (unsigned)p.SH && (unsigned)sc < (unsigned)p.SW)
@@ -112,19 +115,15 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
       al[i] = adummy;
       ac[i] = 0;
       if (i < nea && e < BM * per_m) {
-        int m, c, tap;
+        int m, c, tap, q;
         if (!BWD) {        // w[m][c][tap]: (c, tap) contiguous per m
-          m = e / per_m;
-          const int q = e - m * per_m;
-          c = q / p.KHW;
-          tap = q - c * p.KHW;
+          m = fast_div(e, per_m, 1.0f / (float)per_m, &q);
+          c = fast_div(q, p.KHW, inv_khw, &tap);
         } else {           // w[c][m][tap]: (m, tap) contiguous per c
-          c = e / (BM * p.KHW);
-          const int q = e - c * (BM * p.KHW);
-          m = q / p.KHW;
-          tap = q - m * p.KHW;
+          c = fast_div(e, BM * p.KHW, 1.0f / (float)(BM * p.KHW), &q);
+          m = fast_div(q, p.KHW, inv_khw, &tap);
         }
-        al[i] = (m * p.KHW + tap) * PP + c;
+        al[i] = (m * KHW_MAX + tap) * PP + c;
         ac[i] = c;
         if (m < m_lim) ag[i] = (w_base + m * p.a_mstride + c * p.a_cstride + tap) * esz;
       }
@@ -137,35 +136,31 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
       const int c0 = chunk * CK;
       const int xbase = c0 * chan_bytes, abase = c0 * p.a_cstride * esz;
       if (c0 + CK <= p.SCg) {
+        // unused slots carry the out-of-range offset: no branch, no memory access
 #pragma unroll
-        for (int i = 0; i < NEX_MAX; ++i)
-          if (i < nex) xv[i] = buf_ld(srsrc, xg[i] + xbase, src);
+        for (int i = 0; i < NEX_MAX; ++i) xv[i] = buf_ld(srsrc, xg[i] + xbase, src);
 #pragma unroll
-        for (int i = 0; i < NEA_MAX; ++i)
-          if (i < nea) av[i] = buf_ld(wrsrc, ag[i] + abase, wgt);
+        for (int i = 0; i < NEA_MAX; ++i) av[i] = buf_ld(wrsrc, ag[i] + abase, wgt);
       } else {
         // last chunk of a channel count that is not a multiple of 8: channels past
         // the end read zero
 #pragma unroll
-        for (int i = 0; i < NEX_MAX; ++i)
-          if (i < nex) {
-            const int c = xl[i] - (xl[i] / PP) * PP;
-            xv[i] = buf_ld(srsrc, c0 + c < p.SCg ? xg[i] + xbase : OOB, src);
-          }
+        for (int i = 0; i < NEX_MAX; ++i) {
+          const int c = xl[i] - (xl[i] / PP) * PP;
+          xv[i] = buf_ld(srsrc, c0 + c < p.SCg ? xg[i] + xbase : OOB, src);
+        }
 #pragma unroll
         for (int i = 0; i < NEA_MAX; ++i)
-          if (i < nea) av[i] = buf_ld(wrsrc, c0 + ac[i] < p.SCg ? ag[i] + abase : OOB, wgt);
+          av[i] = buf_ld(wrsrc, c0 + ac[i] < p.SCg ? ag[i] + abase : OOB, wgt);
       }
     };
     auto store_chunk = [&](int buf) {
       float* xs = Xs + buf * p.slab_words;
       float* as = As + buf * p.a_words;
 #pragma unroll
-      for (int i = 0; i < NEX_MAX; ++i)
-        if (i < nex) xs[xl[i]] = xv[i];
+      for (int i = 0; i < NEX_MAX; ++i) xs[xl[i]] = xv[i];
 #pragma unroll
-      for (int i = 0; i < NEA_MAX; ++i)
-        if (i < nea) as[al[i]] = av[i];
+      for (int i = 0; i < NEA_MAX; ++i) as[al[i]] = av[i];
     };
 
     load_chunk(0);
@@ -199,47 +194,83 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
       for (int j = 0; j < NT; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     // slab word offset of this lane's position in block j (tap shift excluded)
+    const float inv_dw = 1.0f / (float)p.DW;
     int pbase[NT];
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
       int pos = (nb0 + j) * 16 + fr;
       if (pos >= npos) pos = 0;                  // padding lanes compute a discarded column
-      const int r = pos / p.DW, w = pos - r * p.DW;
+      int w;
+      const int r = fast_div(pos, p.DW, inv_dw, &w);
       pbase[j] = (r * p.WS + w) * PP + fk;
     }
-    const int abase0 = (wm * 32 + fr) * p.KHW * PP + fk;
+    const int abase0 = (wm * 32 + fr) * KHW_MAX * PP + fk;
+
+    // One tap: 2 k-steps of (2 A + NT B fragment reads, 2*NT MFMAs); every offset
+    // inside is a compile-time immediate on top of the per-block address ba[j].
+    auto tap_mma = [&](const float* at, const int (&ba)[NT], const float* xs, int boff) {
+#pragma unroll
+      for (int ks = 0; ks < CK / 4; ++ks) {
+        const float a0 = at[ks * 4];
+        const float a1 = at[16 * KHW_MAX * PP + ks * 4];
+        float b[NT];
+#pragma unroll
+        for (int j = 0; j < NT; ++j) b[j] = xs[ba[j] + boff + ks * 4];
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b[j], acc[0][j], 0, 0, 0);
+          acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b[j], acc[1][j], 0, 0, 0);
+        }
+      }
+    };
+    const int row_step = p.shs * p.WS * PP, col_step = p.sws * PP;   // window row / column
+    const int origin = ((p.sh0 - p.min_sh) * p.WS + (p.sw0 - p.min_sw)) * PP;   // tap (0,0)
+    // three taps per window row one column apart: their offsets become immediates
+    // (forward walks kw upwards, backward-data downwards)
+    const bool unit_cols = p.KW == 3 && (p.sws == 1 || p.sws == -1);
+    const int kw_first = p.sws == 1 ? 0 : 2, kw_dir = p.sws == 1 ? 1 : -1;
 
     __syncthreads();                             // chunk 0 is in buffer 0
     for (int c = 0; c < n; ++c) {
       const float* xs = Xs + (c & 1) * p.slab_words;
       const float* as = As + (c & 1) * p.a_words + abase0;
-      int tap = 0;
-      for (int kh = 0; kh < p.KH; ++kh) {
-        for (int kw = 0; kw < p.KW; ++kw, ++tap) {
-          const int toff = ((p.sh0 + kh * p.shs - p.min_sh) * p.WS + (p.sw0 + kw * p.sws - p.min_sw)) * PP;
-          const float* at = as + tap * PP;
-          const float* bp[NT];
+      int ba[NT];
 #pragma unroll
-          for (int j = 0; j < NT; ++j) bp[j] = xs + pbase[j] + toff;
+      for (int j = 0; j < NT; ++j) ba[j] = pbase[j] + origin + (unit_cols ? kw_first * col_step : 0);
+      if (unit_cols) {
+        for (int kh = 0; kh < p.KH; ++kh) {
+          const float* at = as + (kh * 3 + kw_first) * PP;
+          tap_mma(at, ba, xs, 0);
+          tap_mma(at + kw_dir * PP, ba, xs, PP);
+          tap_mma(at + 2 * kw_dir * PP, ba, xs, 2 * PP);
 #pragma unroll
-          for (int ks = 0; ks < CK / 4; ++ks) {
-            const float a0 = at[ks * 4];
-            const float a1 = at[16 * p.KHW * PP + ks * 4];
-            float b[NT];
+          for (int j = 0; j < NT; ++j) ba[j] += row_step;
+        }
+      } else {
+        int tap = 0;
+        for (int kh = 0; kh < p.KH; ++kh) {
+          for (int kw = 0; kw < p.KW; ++kw, ++tap) {
+            tap_mma(as + tap * PP, ba, xs, 0);
 #pragma unroll
-            for (int j = 0; j < NT; ++j) b[j] = bp[j][ks * 4];
-#pragma unroll
-            for (int j = 0; j < NT; ++j) {
-              acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b[j], acc[0][j], 0, 0, 0);
-              acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b[j], acc[1][j], 0, 0, 0);
-            }
+            for (int j = 0; j < NT; ++j) ba[j] += col_step;
           }
+#pragma unroll
+          for (int j = 0; j < NT; ++j) ba[j] += row_step - p.KW * col_step;
         }
       }
       __syncthreads();
     }
 
     // ---- epilogue ----------------------------------------------------------------
+    // this lane's eight result channels and their bias
+    float bv[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = wm * 32 + i * 16 + fk * 4 + r;
+        bv[i][r] = (bias && m < m_lim) ? bias[grp * p.DCg + mtile * BM + m] : 0.f;
+      }
     const size_t out_base = (size_t)img * p.DC * p.DH * p.DW + (size_t)r0 * p.DW;
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
@@ -252,9 +283,7 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
             const int m = wm * 32 + i * 16 + fk * 4 + r;
             if (m < m_lim) {
               const int ch = grp * p.DCg + mtile * BM + m;
-              float v = acc[i][j][r];
-              if (bias) v += bias[ch];
-              st(dst, out_base + (size_t)ch * p.DH * p.DW + pos, v);
+              st(dst, out_base + (size_t)ch * p.DH * p.DW + pos, acc[i][j][r] + bv[i][r]);
             }
           }
       }
@@ -290,7 +319,7 @@ bool plan(SlabParams* p, size_t* shmem) {
   double best_cost = 1e30;
   for (int R = 1; R <= p->DH && R * p->DW <= max_pos; ++R) {
     const int RS = R + (p->KH - 1) * p->dly, WS = p->DW + (p->KW - 1) * p->dlx;
-    const int slab_words = RS * WS * PP + 8, a_words = p->KHW * BM * PP + 8;
+    const int slab_words = RS * WS * PP + 8, a_words = KHW_MAX * BM * PP + 8;
     const size_t bytes = (size_t)2 * (slab_words + a_words) * sizeof(float);
     if (bytes > 150 * 1024) break;
     if ((CK * RS * WS + GTHREADS - 1) / GTHREADS > NEX_MAX) break;
@@ -313,7 +342,7 @@ bool plan(SlabParams* p, size_t* shmem) {
   p->NB = (best_r * p->DW + 15) / 16;
   p->nchunks = (p->SCg + CK - 1) / CK;
   p->slab_words = p->RS * p->WS * PP + 8;   // + spare words for out-of-slab loader lanes
-  p->a_words = p->KHW * BM * PP + 8;
+  p->a_words = KHW_MAX * BM * PP + 8;
   *shmem = (size_t)2 * (p->slab_words + p->a_words) * sizeof(float);
   // a tile with few positions would leave the matrix cores idle: not worth it
   return best_r * p->DW >= 64;

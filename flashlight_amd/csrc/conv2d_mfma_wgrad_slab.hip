@@ -70,7 +70,7 @@ wgrad_slab_kernel(WSlabParams p, const T* __restrict__ x, const T* __restrict__ 
     for (int i = 0; i < NXE; ++i) {
       const int e = tid + GTHREADS * i;
       xg[i] = OOB;
-      xl[i] = p.xs_words - 1;                 // spare word
+      xl[i] = CB * p.CP;                      // spare words past the tile (kh*WS is added)
       if (i < nxe && e < CB * p.WS) {
         const int c = e / p.WS, ws = e - c * p.WS;
         const int iw = ws - p.px;
@@ -102,8 +102,7 @@ wgrad_slab_kernel(WSlabParams p, const T* __restrict__ x, const T* __restrict__ 
         const int rb = (img * p.C * HW + ih * p.W) * esz;
         if ((unsigned)ih < (unsigned)p.H) {           // uniform: the whole window row exists
 #pragma unroll
-          for (int i = 0; i < NXE; ++i)
-            if (i < nxe) xv[kh][i] = buf_ld(xrsrc, xg[i] + rb, x);
+          for (int i = 0; i < NXE; ++i) xv[kh][i] = buf_ld(xrsrc, xg[i] + rb, x);
         } else {
 #pragma unroll
           for (int i = 0; i < NXE; ++i) xv[kh][i] = 0.f;
@@ -111,8 +110,7 @@ wgrad_slab_kernel(WSlabParams p, const T* __restrict__ x, const T* __restrict__ 
       }
       const int yb = (img * p.K * OHW + oh * p.OW) * esz;
 #pragma unroll
-      for (int i = 0; i < NDE; ++i)
-        if (i < nde) yv[i] = buf_ld(yrsrc, yg[i] + yb, dy);
+      for (int i = 0; i < NDE; ++i) yv[i] = buf_ld(yrsrc, yg[i] + yb, dy);
     };
     auto store_row = [&](int buf, const float (&xv)[3][NXE], const float (&yv)[NDE]) {
       float* xs = Xs + buf * p.xs_words;
@@ -120,11 +118,9 @@ wgrad_slab_kernel(WSlabParams p, const T* __restrict__ x, const T* __restrict__ 
 #pragma unroll
       for (int kh = 0; kh < 3; ++kh)
 #pragma unroll
-        for (int i = 0; i < NXE; ++i)
-          if (i < nxe) xs[xl[i] + kh * p.WS] = xv[kh][i];
+        for (int i = 0; i < NXE; ++i) xs[xl[i] + kh * p.WS] = xv[kh][i];
 #pragma unroll
-      for (int i = 0; i < NDE; ++i)
-        if (i < nde) ds[yl[i]] = yv[i];
+      for (int i = 0; i < NDE; ++i) ds[yl[i]] = yv[i];
     };
 
     const bool do_db = p.want_db && half == 0 && tid < BM;
@@ -251,8 +247,8 @@ bool plan(const ConvGeom& g, WSlabParams* p) {
   if ((BM * g.OW + GTHREADS - 1) / GTHREADS > NDE) return false;
   p->CP = 3 * p->WS + 1;
   if (p->CP % 2 == 0) ++p->CP;                     // odd channel pitch spreads the banks
-  p->DP = g.OW + ((4 - g.OW % 32) + 32) % 32;      // == 4 mod 32
-  p->xs_words = CB * p->CP + 8;
+  p->DP = g.OW + ((2 - g.OW % 32) + 32) % 32;      // == 2 mod 32: dy fragments conflict-free
+  p->xs_words = CB * p->CP + 2 * p->WS + 8;   // + spare words for unused loader slots
   p->ds_words = BM * p->DP + 8;
   p->nhalves = g.Cg / CB;
   p->mtiles = (g.Kg + BM - 1) / BM;
