@@ -37,6 +37,7 @@ constexpr int NEA_MAX = 20;      // weight elements per loader thread and chunk
 constexpr int KHW_MAX = 9;
 
 struct SlabParams {
+  int stage_ok;          // result rows are 16-byte aligned and a half tile fits in LDS
   int N, SC, SH, SW, DC, DH, DW;
   int KH, KW, KHW, dly, dlx;
   int sh0, sw0;          // window shift of tap (0,0): fwd -py,-px ; bwd +py,+px
@@ -68,6 +69,29 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
   const int m_lim = p.DCg - mtile * BM;
   const int rows = min(p.R, p.DH - r0);          // result rows of this tile
   const int n = p.nchunks;
+  const int npos = rows * p.DW;
+
+  // Epilogue through LDS (when rows are 16-byte aligned): the MFMA waves of one
+  // channel half park their accumulators as stage[32 channels][npos] in the LDS
+  // that held the operands, then all 512 threads write each channel's run of
+  // npos results with 16-byte stores.
+  const int SP = ((npos + 3) & ~3) + 4;                       // stage pitch (words)
+  const bool staged = p.stage_ok && (npos & 3) == 0;
+  auto coop_store = [&](int h) {
+    const int q4 = npos >> 2;
+    const size_t out_base = (size_t)img * p.DC * p.DH * p.DW + (size_t)r0 * p.DW;
+    for (int idx = tid; idx < 32 * q4; idx += THREADS) {
+      const int ch_l = idx / q4, q = idx - ch_l * q4;
+      const int m = h * 32 + ch_l;
+      if (m < m_lim) {
+        const int ch = grp * p.DCg + mtile * BM + m;
+        const float b = bias ? bias[ch] : 0.f;
+        float4 v = *reinterpret_cast<const float4*>(lds + ch_l * SP + 4 * q);
+        v.x += b; v.y += b; v.z += b; v.w += b;
+        st4_stream(dst, out_base + (size_t)ch * p.DH * p.DW + 4 * q, v);
+      }
+    }
+  };
 
   if (wave < 4) {
     // ============================ loader waves ===================================
@@ -106,14 +130,12 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
     const int per_m = CK * p.KHW;
     const int nea = (BM * per_m + GTHREADS - 1) / GTHREADS;
     int ag[NEA_MAX], al[NEA_MAX];                // global byte offset, LDS word offset
-    int ac[NEA_MAX];                             // chunk channel (for the last, partial chunk)
     const int w_base = grp * p.w_group_stride + mtile * BM * p.a_mstride;
 #pragma unroll
     for (int i = 0; i < NEA_MAX; ++i) {
       const int e = tid + GTHREADS * i;
       ag[i] = OOB;
       al[i] = adummy;
-      ac[i] = 0;
       if (i < nea && e < BM * per_m) {
         int m, c, tap, q;
         if (!BWD) {        // w[m][c][tap]: (c, tap) contiguous per m
@@ -124,7 +146,6 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
           m = fast_div(q, p.KHW, inv_khw, &tap);
         }
         al[i] = (m * KHW_MAX + tap) * PP + c;
-        ac[i] = c;
         if (m < m_lim) ag[i] = (w_base + m * p.a_mstride + c * p.a_cstride + tap) * esz;
       }
     }
@@ -151,7 +172,7 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
         }
 #pragma unroll
         for (int i = 0; i < NEA_MAX; ++i)
-          av[i] = buf_ld(wrsrc, c0 + ac[i] < p.SCg ? ag[i] + abase : OOB, wgt);
+          av[i] = buf_ld(wrsrc, c0 + (al[i] - (al[i] / PP) * PP) < p.SCg ? ag[i] + abase : OOB, wgt);
       }
     };
     auto store_chunk = [&](int buf) {
@@ -173,6 +194,13 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
       }
       __syncthreads();
     }
+    if (staged) {
+      for (int h = 0; h < 2; ++h) {
+        __syncthreads();        // half h is staged
+        coop_store(h);
+        __syncthreads();        // stage may be overwritten
+      }
+    }
     return;
   }
 
@@ -183,8 +211,6 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
   const int nt = base + (wn < rem ? 1 : 0);
   const int nb0 = wn * base + min(wn, rem);
   const int fr = lane & 15, fk = lane >> 4;
-  const int npos = rows * p.DW;
-
   auto run = [&](auto ntc) {
     constexpr int NT = decltype(ntc)::value;
     floatx4 acc[2][NT];
@@ -206,51 +232,80 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
     }
     const int abase0 = (wm * 32 + fr) * KHW_MAX * PP + fk;
 
-    // One tap: 2 k-steps of (2 A + NT B fragment reads, 2*NT MFMAs); every offset
-    // inside is a compile-time immediate on top of the per-block address ba[j].
-    auto tap_mma = [&](const float* at, const int (&ba)[NT], const float* xs, int boff) {
+    // Fragments of one tap: 2 k-steps x (2 A + NT B).  Every offset inside is a
+    // compile-time immediate on top of the per-block address ba[j].
+    struct Frag {
+      float a[CK / 4][2];
+      float b[CK / 4][NT];
+    };
+    auto read_frags = [&](Frag& f, const float* at, const int (&ba)[NT], const float* xs, int boff) {
 #pragma unroll
       for (int ks = 0; ks < CK / 4; ++ks) {
-        const float a0 = at[ks * 4];
-        const float a1 = at[16 * KHW_MAX * PP + ks * 4];
-        float b[NT];
+        f.a[ks][0] = at[ks * 4];
+        f.a[ks][1] = at[16 * KHW_MAX * PP + ks * 4];
 #pragma unroll
-        for (int j = 0; j < NT; ++j) b[j] = xs[ba[j] + boff + ks * 4];
+        for (int j = 0; j < NT; ++j) f.b[ks][j] = xs[ba[j] + boff + ks * 4];
+      }
+    };
+    auto mma = [&](const Frag& f) {
+#pragma unroll
+      for (int ks = 0; ks < CK / 4; ++ks)
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
-          acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b[j], acc[0][j], 0, 0, 0);
-          acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b[j], acc[1][j], 0, 0, 0);
+          acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(f.a[ks][0], f.b[ks][j], acc[0][j], 0, 0, 0);
+          acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(f.a[ks][1], f.b[ks][j], acc[1][j], 0, 0, 0);
         }
-      }
     };
     const int row_step = p.shs * p.WS * PP, col_step = p.sws * PP;   // window row / column
     const int origin = ((p.sh0 - p.min_sh) * p.WS + (p.sw0 - p.min_sw)) * PP;   // tap (0,0)
-    // three taps per window row one column apart: their offsets become immediates
-    // (forward walks kw upwards, backward-data downwards)
-    const bool unit_cols = p.KW == 3 && (p.sws == 1 || p.sws == -1);
+    // 3x3 window whose columns are one apart: the nine taps are straight-line code,
+    // the three taps of a window row differ by immediate offsets (forward walks kw
+    // upwards, backward-data downwards), and the fragments of tap t+1 are read
+    // while the MFMAs of tap t run.
+    const bool static33 = p.KH == 3 && p.KW == 3 && (p.sws == 1 || p.sws == -1);
     const int kw_first = p.sws == 1 ? 0 : 2, kw_dir = p.sws == 1 ? 1 : -1;
 
     __syncthreads();                             // chunk 0 is in buffer 0
     for (int c = 0; c < n; ++c) {
       const float* xs = Xs + (c & 1) * p.slab_words;
       const float* as = As + (c & 1) * p.a_words + abase0;
-      int ba[NT];
+      if (static33) {
+        int ba[NT];
 #pragma unroll
-      for (int j = 0; j < NT; ++j) ba[j] = pbase[j] + origin + (unit_cols ? kw_first * col_step : 0);
-      if (unit_cols) {
-        for (int kh = 0; kh < p.KH; ++kh) {
-          const float* at = as + (kh * 3 + kw_first) * PP;
-          tap_mma(at, ba, xs, 0);
-          tap_mma(at + kw_dir * PP, ba, xs, PP);
-          tap_mma(at + 2 * kw_dir * PP, ba, xs, 2 * PP);
-#pragma unroll
-          for (int j = 0; j < NT; ++j) ba[j] += row_step;
-        }
+        for (int j = 0; j < NT; ++j) ba[j] = pbase[j] + origin + kw_first * col_step;
+        const float* a0 = as + kw_first * PP;
+        const int ad = kw_dir * PP;
+        Frag f0, f1;
+        read_frags(f0, a0, ba, xs, 0);
+#define FLHIP_TAP(CUR, NXT, AT, BA, BOFF)        \
+  read_frags(NXT, AT, BA, xs, BOFF);             \
+  __builtin_amdgcn_sched_barrier(0);             \
+  mma(CUR);                                      \
+  __builtin_amdgcn_sched_barrier(0);
+#define FLHIP_NEXT_ROW _Pragma("unroll") for (int j = 0; j < NT; ++j) ba[j] += row_step;
+        FLHIP_TAP(f0, f1, a0 + ad, ba, PP)
+        FLHIP_TAP(f1, f0, a0 + 2 * ad, ba, 2 * PP)
+        FLHIP_NEXT_ROW
+        FLHIP_TAP(f0, f1, a0 + 3 * PP, ba, 0)
+        FLHIP_TAP(f1, f0, a0 + 3 * PP + ad, ba, PP)
+        FLHIP_TAP(f0, f1, a0 + 3 * PP + 2 * ad, ba, 2 * PP)
+        FLHIP_NEXT_ROW
+        FLHIP_TAP(f1, f0, a0 + 6 * PP, ba, 0)
+        FLHIP_TAP(f0, f1, a0 + 6 * PP + ad, ba, PP)
+        FLHIP_TAP(f1, f0, a0 + 6 * PP + 2 * ad, ba, 2 * PP)
+#undef FLHIP_NEXT_ROW
+#undef FLHIP_TAP
+        mma(f0);
       } else {
+        int ba[NT];
+#pragma unroll
+        for (int j = 0; j < NT; ++j) ba[j] = pbase[j] + origin;
         int tap = 0;
         for (int kh = 0; kh < p.KH; ++kh) {
           for (int kw = 0; kw < p.KW; ++kw, ++tap) {
-            tap_mma(as + tap * PP, ba, xs, 0);
+            Frag f;
+            read_frags(f, as + tap * PP, ba, xs, 0);
+            mma(f);
 #pragma unroll
             for (int j = 0; j < NT; ++j) ba[j] += col_step;
           }
@@ -262,6 +317,26 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
     }
 
     // ---- epilogue ----------------------------------------------------------------
+    if (staged) {
+      for (int h = 0; h < 2; ++h) {
+        if (wm == h) {
+#pragma unroll
+          for (int j = 0; j < NT; ++j) {
+            const int pos = (nb0 + j) * 16 + fr;
+            if (pos < npos) {
+#pragma unroll
+              for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) lds[(i * 16 + fk * 4 + r) * SP + pos] = acc[i][j][r];
+            }
+          }
+        }
+        __syncthreads();
+        coop_store(h);
+        __syncthreads();
+      }
+      return;
+    }
     // this lane's eight result channels and their bias
     float bv[2][4];
 #pragma unroll
@@ -344,6 +419,10 @@ bool plan(SlabParams* p, size_t* shmem) {
   p->slab_words = p->RS * p->WS * PP + 8;   // + spare words for out-of-slab loader lanes
   p->a_words = KHW_MAX * BM * PP + 8;
   *shmem = (size_t)2 * (p->slab_words + p->a_words) * sizeof(float);
+  {
+    const int npos = best_r * p->DW, sp = ((npos + 3) & ~3) + 4;
+    p->stage_ok = p->DW % 4 == 0 && (size_t)32 * sp * sizeof(float) <= *shmem;
+  }
   // a tile with few positions would leave the matrix cores idle: not worth it
   return best_r * p->DW >= 64;
 }
@@ -358,6 +437,7 @@ int launch(SlabParams& p, const void* src, const void* wgt, const float* bias, v
   p.wgt_bytes = (unsigned)wbytes;
   size_t shmem = 0;
   if (!plan(&p, &shmem)) return -1;
+  if (reinterpret_cast<uintptr_t>(dst) % 16 != 0) p.stage_ok = 0;
   auto kernel = slab_conv_kernel<T, BWD>;
   if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
   const dim3 grid((unsigned)(p.N * p.tiles_per_image), (unsigned)(p.mtiles * p.groups));
