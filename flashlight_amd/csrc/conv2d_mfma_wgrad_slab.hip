@@ -185,37 +185,65 @@ wgrad_slab_kernel(WSlabParams p, const T* __restrict__ x, const T* __restrict__ 
   const int abase = (wm * 32 + fr) * p.DP + fk;
   const int ksteps = p.OW / 4;
 
+  // Fragments of two k-steps (8 positions): 2x2 dy values and 2xNTW x values.
+  struct Frag {
+    float a[2][2];
+    float b[2][NTW];
+  };
+  const float* ds_row;
+  const float* bp[NTW];
+  auto read_frags = [&](Frag& f, int ks) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      f.a[u][0] = ds_row[(ks + u) * 4];
+      f.a[u][1] = ds_row[16 * p.DP + (ks + u) * 4];
+#pragma unroll
+      for (int j = 0; j < NTW; ++j) f.b[u][j] = bp[j][(ks + u) * 4];
+    }
+  };
+  auto mma = [&](const Frag& f) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int j = 0; j < NTW; ++j) {
+        acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(f.a[u][0], f.b[u][j], acc[0][j], 0, 0, 0);
+        acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(f.a[u][1], f.b[u][j], acc[1][j], 0, 0, 0);
+      }
+  };
+
   __syncthreads();
   for (int r = 0; r < nrows; ++r) {
     const float* xs = Xs + (r & 1) * p.xs_words;
-    const float* ds = Ds + (r & 1) * p.ds_words + abase;
-    const float* bp[NTW];
+    ds_row = Ds + (r & 1) * p.ds_words + abase;
 #pragma unroll
     for (int j = 0; j < NTW; ++j) bp[j] = xs + colbase[j];
-    int ks = 0;
-    for (; ks + 2 <= ksteps; ks += 2) {
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const float a0 = ds[(ks + u) * 4];
-        const float a1 = ds[16 * p.DP + (ks + u) * 4];
-        float b[NTW];
-#pragma unroll
-        for (int j = 0; j < NTW; ++j) b[j] = bp[j][(ks + u) * 4];
+    if ((ksteps & 1) == 0) {
+      // pairs of k-steps, fragments of the next pair read while this pair's MFMAs
+      // run.  The read past the last pair stays inside the LDS tile and is unused.
+      Frag f0, f1;
+      read_frags(f0, 0);
+      int ks = 0;
+      for (; ks + 4 <= ksteps; ks += 4) {
+        read_frags(f1, ks + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(f0);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(f0, ks + 4);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(f1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if (ks < ksteps) mma(f0);      // ksteps == 2 (mod 4)
+    } else {
+      for (int ks = 0; ks < ksteps; ++ks) {
+        const float a0 = ds_row[ks * 4];
+        const float a1 = ds_row[16 * p.DP + ks * 4];
 #pragma unroll
         for (int j = 0; j < NTW; ++j) {
-          acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b[j], acc[0][j], 0, 0, 0);
-          acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b[j], acc[1][j], 0, 0, 0);
+          const float b = bp[j][ks * 4];
+          acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b, acc[0][j], 0, 0, 0);
+          acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b, acc[1][j], 0, 0, 0);
         }
-      }
-    }
-    if (ks < ksteps) {
-      const float a0 = ds[ks * 4];
-      const float a1 = ds[16 * p.DP + ks * 4];
-#pragma unroll
-      for (int j = 0; j < NTW; ++j) {
-        const float b = bp[j][ks * 4];
-        acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b, acc[0][j], 0, 0, 0);
-        acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b, acc[1][j], 0, 0, 0);
       }
     }
     __syncthreads();
@@ -249,7 +277,7 @@ bool plan(const ConvGeom& g, WSlabParams* p) {
   if (p->CP % 2 == 0) ++p->CP;                     // odd channel pitch spreads the banks
   p->DP = g.OW + ((2 - g.OW % 32) + 32) % 32;      // == 2 mod 32: dy fragments conflict-free
   p->xs_words = CB * p->CP + 2 * p->WS + 8;   // + spare words for unused loader slots
-  p->ds_words = BM * p->DP + 8;
+  p->ds_words = BM * p->DP + 16;
   p->nhalves = g.Cg / CB;
   p->mtiles = (g.Kg + BM - 1) / BM;
   p->total_rows = g.N * g.OH;
