@@ -277,10 +277,17 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
         const int ad = kw_dir * PP;
         Frag f0, f1;
         read_frags(f0, a0, ba, xs, 0);
-#define FLHIP_TAP(CUR, NXT, AT, BA, BOFF)        \
-  read_frags(NXT, AT, BA, xs, BOFF);             \
-  __builtin_amdgcn_sched_barrier(0);             \
-  mma(CUR);                                      \
+        // One LDS read is slotted behind each of the first MFMAs of the tap, so the
+        // reads issue in the shadow of the matrix pipe instead of ahead of it.
+#define FLHIP_TAP(CUR, NXT, AT, BA, BOFF)                     \
+  __builtin_amdgcn_sched_barrier(0);                          \
+  read_frags(NXT, AT, BA, xs, BOFF);                          \
+  mma(CUR);                                                   \
+  _Pragma("unroll") for (int q = 0; q < (CK / 4) * (2 + NT); ++q) { \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        \
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);        \
+  }                                                           \
+  __builtin_amdgcn_sched_group_barrier(0x008, (CK / 4) * (2 * NT - 2), 0); \
   __builtin_amdgcn_sched_barrier(0);
 #define FLHIP_NEXT_ROW _Pragma("unroll") for (int j = 0; j < NT; ++j) ba[j] += row_step;
         FLHIP_TAP(f0, f1, a0 + ad, ba, PP)
