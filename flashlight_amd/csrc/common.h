@@ -99,6 +99,28 @@ __device__ __forceinline__ float buf_ld(__amdgpu_buffer_rsrc_t r, int byte_off, 
   return bf16_to_f32((bf16_t)__builtin_amdgcn_raw_buffer_load_b16(r, byte_off, 0, 0));
 }
 
+// four consecutive elements at a byte offset (16-byte aligned for float, 8 for bf16)
+typedef unsigned uintx4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 buf_ld4(__amdgpu_buffer_rsrc_t r, int byte_off, const float*) {
+  const uintx4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
+  return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z),
+                     __uint_as_float(v.w));
+}
+__device__ __forceinline__ float4 buf_ld4(__amdgpu_buffer_rsrc_t r, int byte_off, const bf16_t*) {
+  const uintx2_t v = __builtin_amdgcn_raw_buffer_load_b64(r, byte_off, 0, 0);
+  return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u),
+                     __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
+}
+
+// pointers into LDS (the host pass of the compiler only parses the kernels)
+#if defined(__HIP_DEVICE_COMPILE__)
+typedef __attribute__((address_space(3))) const float2* lds_f2;
+typedef __attribute__((address_space(3))) const float* lds_f1;
+#else
+typedef const float2* lds_f2;
+typedef const float* lds_f1;
+#endif
+
 // ---- small-integer division ------------------------------------------------------
 // e / d for 0 <= e < 2^22 with inv = 1.0f / d: a float estimate corrected to the
 // exact quotient (a handful of VALU operations instead of the ~30 of an integer

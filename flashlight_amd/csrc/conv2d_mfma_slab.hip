@@ -70,29 +70,6 @@ struct SlabParams {
   unsigned src_bytes, wgt_bytes;
 };
 
-// pointers into LDS (the host pass of the compiler only parses the kernel)
-#if defined(__HIP_DEVICE_COMPILE__)
-typedef __attribute__((address_space(3))) const float2* lds_f2;
-typedef __attribute__((address_space(3))) const float* lds_f1;
-#else
-typedef const float2* lds_f2;
-typedef const float* lds_f1;
-#endif
-typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
-typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
-
-// four consecutive elements at a byte offset (16-byte aligned for float, 8 for bf16)
-__device__ __forceinline__ float4 buf_ld4(__amdgpu_buffer_rsrc_t r, int byte_off, const float*) {
-  const uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
-  return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z),
-                     __uint_as_float(v.w));
-}
-__device__ __forceinline__ float4 buf_ld4(__amdgpu_buffer_rsrc_t r, int byte_off, const bf16_t*) {
-  const uintx2 v = __builtin_amdgcn_raw_buffer_load_b64(r, byte_off, 0, 0);
-  return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u),
-                     __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
-}
-
 template <typename T, bool BWD>
 __global__ void __launch_bounds__(THREADS, 2)
 slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ wgt,
