@@ -307,8 +307,7 @@ wgrad_slab_kernel(WSlabParams p, const T* __restrict__ x, const T* __restrict__ 
     for (int j = 0; j < NTW; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   const int ksteps = p.OW >> 2;
-  const bool pairs = (ksteps & 1) == 0;     // groups of 8 positions, 2 per lane
-  const int fmul = pairs ? 2 : 1;
+  const int ngroups = ksteps >> 1;          // groups of 8 positions, 2 per lane
   // this lane's column in block j: local column -> (channel, kh, kw) -> LDS address
   lds_f1 bp[NTW];
 #pragma unroll
@@ -316,9 +315,9 @@ wgrad_slab_kernel(WSlabParams p, const T* __restrict__ x, const T* __restrict__ 
     const int col = (wn * NTW + j) * 16 + fr;
     const int c = col / 9, t = col - c * 9;
     const int kh = t / 3, kw = t - kh * 3;
-    bp[j] = (lds_f1)Xs + (c * p.CP + kh * p.WS + kw * p.dlx + p.XOFF - p.px + fmul * fk);
+    bp[j] = (lds_f1)Xs + (c * p.CP + kh * p.WS + kw * p.dlx + p.XOFF - p.px + 2 * fk);
   }
-  lds_f1 ap0 = (lds_f1)Ds + ((wm * 32 + fr) * p.DP + fmul * fk);
+  lds_f1 ap0 = (lds_f1)Ds + ((wm * 32 + fr) * p.DP + 2 * fk);
   lds_f1 ap1 = ap0 + 16 * p.DP;
 
   // Fragments of a group of 8 positions: .x and .y are the two k-steps.
@@ -354,11 +353,10 @@ wgrad_slab_kernel(WSlabParams p, const T* __restrict__ x, const T* __restrict__ 
   __syncthreads();
   for (int r = 0; r < nrows; ++r) {
     int walked = 0;
-    if (pairs) {
+    if (ngroups > 0) {
       // Fragments of the next group are read while this group's MFMAs run, one LDS
       // read slotted behind each of the first MFMAs.  The read past the last group
       // stays inside the LDS tile and is not used.
-      const int ngroups = ksteps >> 1;
       Frag f0, f1;
       read_frags(f0, 0);
 #define FLHIP_GROUP(CUR, NXT, OFF)                                    \
@@ -380,16 +378,18 @@ wgrad_slab_kernel(WSlabParams p, const T* __restrict__ x, const T* __restrict__ 
       }
 #undef FLHIP_GROUP
       if (g < ngroups) mma(f0);
-    } else {
-      for (int ks = 0; ks < ksteps; ++ks) {
-        const float a0 = ap0[ks * 4];
-        const float a1 = ap1[ks * 4];
+    }
+    if (ksteps & 1) {
+      // last four positions of a row whose length is not a multiple of 8: one
+      // k-step, lane fk takes position 8*ngroups + fk
+      const int off = 8 * ngroups - walked - fk;
+      const float a0 = ap0[off];
+      const float a1 = ap1[off];
 #pragma unroll
-        for (int j = 0; j < NTW; ++j) {
-          const float b = bp[j][ks * 4];
-          acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b, acc[0][j], 0, 0, 0);
-          acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b, acc[1][j], 0, 0, 0);
-        }
+      for (int j = 0; j < NTW; ++j) {
+        const float b = bp[j][off];
+        acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0, b, acc[0][j], 0, 0, 0);
+        acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a1, b, acc[1][j], 0, 0, 0);
       }
     }
     // back to the row start, in the other buffer

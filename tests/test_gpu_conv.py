@@ -33,6 +33,9 @@ MORE = [
     ((2, 64, 10, 16), (96, 32, 3, 3), (1, 1), (1, 1), (1, 1), 2),       # slab, groups, two column halves... per group 32
     ((1, 20, 12, 20), (24, 20, 3, 3), (1, 1), (0, 1), (1, 1), 1),       # slab fwd/bwd-data with a channel tail
     ((2, 64, 7, 8), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),         # few rows per split
+    ((1, 32, 5, 24), (64, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),        # slab, rows of 3 groups of 8
+    ((1, 32, 6, 18), (70, 32, 3, 3), (1, 1), (0, 0), (1, 1), 1),        # slab, rows not 16-byte aligned
+    ((2, 32, 9, 20), (64, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),        # slab, row length 4 (mod 8)
 ]
 ALL = LIB_CASES + MORE
 
