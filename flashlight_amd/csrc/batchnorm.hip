@@ -9,6 +9,9 @@
 // `inner` elements; threads stream them with 4-wide loads when inner % 4 == 0.
 // inner == 1 ("column" kernels, per-activation mode): features are contiguous, a
 // wave covers 64 features and rows are strided by C.
+#include <stdlib.h>
+#include <string.h>
+
 #include "common.h"
 
 namespace flhip {
@@ -300,6 +303,148 @@ bn_bwd_apply_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
   });
 }
 
+// ---- resident kernels (segment mode, 4-wide) ------------------------------------
+// One workgroup of 1024 threads owns a whole feature and keeps its x values in
+// registers between the reduction and the elementwise pass (K 16-byte vectors per
+// thread), so x is read from memory once.  The backward kernel also parks the
+// first KL vectors of dy per thread in LDS and re-reads only the rest.  Used when
+// a feature fits (outer*inner <= 4096*K) and there are enough features to fill
+// the machine; no workspace, no second launch.
+constexpr int RES_THREADS = 1024;
+constexpr int RES_KMAX = 25;
+constexpr int RES_KL = 9;             // dy vectors per thread parked in LDS (9 x 16 KiB)
+constexpr int RES_MIN_C = 128;        // fewer features leave too many CUs idle
+
+// Walks this thread's vectors q = tid + 1024*k: f(k, byte offset, in range).  The
+// offset is relative to the tensor base and goes through a buffer descriptor; slots
+// past the feature get an offset past the descriptor's range, so their loads return
+// zero and their stores are dropped without a branch.
+template <int K, int ESZ, int FENCE, typename F>
+__device__ __forceinline__ void res_visit(const BnGeom& g, F&& f) {
+  constexpr int OOB = (int)0x80000000;
+  const int innerV = (int)(g.inner >> 2);
+  const int c = blockIdx.x;
+  int q = threadIdx.x;
+  int o = q / innerV, i = q - o * innerV;
+  const int so = RES_THREADS / innerV, si = RES_THREADS - so * innerV;
+  const int row = (int)(g.C * g.inner) * ESZ;                 // bytes between outer slices
+  int off = ((o * (int)g.C + c) * (int)g.inner + i * 4) * ESZ;
+  const int step = so * row + si * 4 * ESZ;
+  const int wrap = row - (int)g.inner * ESZ;
+  // Each walk recomputes its offsets (two or three adds per vector): keeping the K
+  // offsets of the first walk alive for the next one would cost K registers.
+  asm volatile("" : "+v"(off), "+v"(i), "+v"(q));
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const bool in = q < (int)g.units;
+    f(k, in ? off : OOB, in);
+    // FENCE > 0: finish each group of FENCE vectors before starting the next, or the
+    // scheduler overlaps the temporaries of all K vectors and runs out of registers
+    if (FENCE > 0 && k % (FENCE > 0 ? FENCE : 1) == (FENCE > 0 ? FENCE : 1) - 1)
+      __builtin_amdgcn_sched_barrier(0);
+    q += RES_THREADS;
+    off += step;
+    i += si;
+    if (i >= innerV) {
+      i -= innerV;
+      off += wrap;
+    }
+  }
+}
+
+// 16-byte (float) / 8-byte (bf16) buffer store of four values, streaming
+__device__ __forceinline__ void buf_st4(__amdgpu_buffer_rsrc_t r, int byte_off, float4 v, float*) {
+  const uintx4_t t = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z),
+                      __float_as_uint(v.w)};
+  __builtin_amdgcn_raw_buffer_store_b128(t, r, byte_off, 0, 2);
+}
+__device__ __forceinline__ void buf_st4(__amdgpu_buffer_rsrc_t r, int byte_off, float4 v, bf16_t*) {
+  const uintx2_t t = {(uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16),
+                      (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16)};
+  __builtin_amdgcn_raw_buffer_store_b64(t, r, byte_off, 0, 2);
+}
+
+template <typename T, int K>
+__global__ void __launch_bounds__(RES_THREADS)
+bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restrict__ y,
+                  BnTrainArgs a) {
+  __shared__ float red[16];
+  __shared__ float sh[2];
+  constexpr int ESZ = (int)sizeof(T);
+  const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
+  const long long c = blockIdx.x;
+  const float shift = ld(x, (size_t)(c * g.inner));
+  float4 xr[K];
+  float s1 = 0.f, s2 = 0.f;
+  res_visit<K, ESZ, 0>(g, [&](int k, int off, bool in) { xr[k] = buf_ld4(xr_, off, x); });
+  res_visit<K, ESZ, 1>(g, [&](int k, int, bool in) {
+    const float t0 = xr[k].x - shift, t1 = xr[k].y - shift, t2 = xr[k].z - shift,
+                t3 = xr[k].w - shift;
+    const float p1 = (t0 + t1) + (t2 + t3);
+    const float p2 = (t0 * t0 + t1 * t1) + (t2 * t2 + t3 * t3);
+    s1 += in ? p1 : 0.f;
+    s2 += in ? p2 : 0.f;
+    // both sums are finished per vector: otherwise the second one is sunk below the
+    // first block reduction and drags every vector's temporaries along
+    asm volatile("" : "+v"(s1), "+v"(s2));
+  });
+  s1 = block_sum(s1, red);
+  s2 = block_sum(s2, red);
+  finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh);
+  __syncthreads();
+  const float mean = sh[0];
+  const float scale = (a.gamma ? a.gamma[c] : 1.f) * sh[1];
+  const float bt = a.beta ? a.beta[c] : 0.f;
+  res_visit<K, ESZ, 1>(g, [&](int k, int off, bool) {
+    const float4 v = make_float4((xr[k].x - mean) * scale + bt, (xr[k].y - mean) * scale + bt,
+                                 (xr[k].z - mean) * scale + bt, (xr[k].w - mean) * scale + bt);
+    buf_st4(yr_, off, v, y);
+  });
+}
+
+template <typename T, int K>
+__global__ void __launch_bounds__(RES_THREADS)
+bn_bwd_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, const T* __restrict__ dy,
+                T* __restrict__ dx, BnBwdArgs a) {
+  extern __shared__ float4 dyl[];           // [min(K, RES_KL)][1024]
+  __shared__ float red[16];
+  __shared__ float sh[4];
+  constexpr int ESZ = (int)sizeof(T);
+  constexpr int KL = K < RES_KL ? K : RES_KL;
+  const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes),
+                               dxr_ = make_rsrc(dx, bytes);
+  const long long c = blockIdx.x;
+  const float mean = a.save_mean[c];
+  float4 xr[K];
+  float s1 = 0.f, s2 = 0.f;
+  res_visit<K, ESZ, 0>(g, [&](int k, int off, bool in) { xr[k] = buf_ld4(xr_, off, x); });
+  res_visit<K, ESZ, 4>(g, [&](int k, int off, bool in) {
+    const float4 d = buf_ld4(dyr_, off, dy);
+    if (k < KL) dyl[k * RES_THREADS + threadIdx.x] = d;
+    const float p1 = (d.x + d.y) + (d.z + d.w);
+    const float p2 = (d.x * (xr[k].x - mean) + d.y * (xr[k].y - mean)) +
+                     (d.z * (xr[k].z - mean) + d.w * (xr[k].w - mean));
+    s1 += in ? p1 : 0.f;
+    s2 += in ? p2 : 0.f;
+    // both sums are finished per vector: otherwise the second one is sunk below the
+    // first block reduction and drags every vector's temporaries along
+    asm volatile("" : "+v"(s1), "+v"(s2));
+  });
+  s1 = block_sum(s1, red);
+  s2 = block_sum(s2, red);
+  finish_bwd(g, a, c, (double)s1, (double)s2, true, sh);
+  __syncthreads();
+  const float kdy = sh[1], kx = sh[2], k0 = sh[3];
+  res_visit<K, ESZ, 4>(g, [&](int k, int off, bool) {
+    const float4 d = k < KL ? dyl[k * RES_THREADS + threadIdx.x] : buf_ld4(dyr_, off, dy);
+    const float4 v = make_float4(kdy * d.x + (kx * (xr[k].x - mean) + k0),
+                                 kdy * d.y + (kx * (xr[k].y - mean) + k0),
+                                 kdy * d.z + (kx * (xr[k].z - mean) + k0),
+                                 kdy * d.w + (kx * (xr[k].w - mean) + k0));
+    buf_st4(dxr_, off, v, dx);
+  });
+}
+
 // ---- column mode (inner == 1) ----------------------------------------------
 // block = 64 features x 4 row lanes; grid = (ceil(C/64), S); slice s owns rows
 // [s*ups, (s+1)*ups).
@@ -464,11 +609,60 @@ static int make_geom(const flhip_bn_desc* d, BnGeom* g, int* vec) {
   return FLHIP_OK;
 }
 
+// Vectors per thread of the resident kernels for this geometry, 0 when they do not
+// apply.  FLHIP_BN_ALGO=split forces the two-kernel path, =resident lifts the
+// feature-count threshold (measurement aids).
+static int resident_k(const BnGeom& g, int vec) {
+  static const int mode = [] {
+    const char* e = getenv("FLHIP_BN_ALGO");
+    if (e && !strcmp(e, "split")) return 1;
+    if (e && !strcmp(e, "resident")) return 2;
+    return 0;
+  }();
+  if (mode == 1 || vec != 4) return 0;
+  if (g.units > (long long)RES_KMAX * RES_THREADS) return 0;
+  if (g.outer * g.C * g.inner * 4 >= (1ll << 31)) return 0;   // 32-bit buffer offsets
+  if (mode != 2 && g.C < RES_MIN_C) return 0;
+  const int need = (int)((g.units + RES_THREADS - 1) / RES_THREADS);
+  return need <= 8 ? 8 : need <= 16 ? 16 : RES_KMAX;
+}
+
+template <typename T, int K>
+static int launch_train_resident(const BnGeom& g, const T* x, T* y, const BnTrainArgs& a,
+                                 hipStream_t s) {
+  const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
+  hipLaunchKernelGGL((bn_train_resident<T, K>), dim3((unsigned)g.C), dim3(RES_THREADS), 0, s, g,
+                     bytes, x, y, a);
+  return check_launch("bn_fwd_train (resident)");
+}
+
+template <typename T, int K>
+static int launch_bwd_resident(const BnGeom& g, const T* x, const T* dy, T* dx, const BnBwdArgs& a,
+                               hipStream_t s) {
+  constexpr int KL = K < RES_KL ? K : RES_KL;
+  constexpr size_t shmem = (size_t)KL * RES_THREADS * sizeof(float4);
+  auto kernel = bn_bwd_resident<T, K>;
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+  if (attr != hipSuccess)
+    return fail(FLHIP_RUNTIME_ERROR, std::string("bn_bwd: LDS limit: ") + hipGetErrorString(attr));
+  const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
+  hipLaunchKernelGGL(kernel, dim3((unsigned)g.C), dim3(RES_THREADS), shmem, s, g, bytes, x, dy, dx,
+                     a);
+  return check_launch("bn_bwd (resident)");
+}
+
 template <typename T>
 static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws,
                      const BnTrainArgs& a, hipStream_t s) {
   const T* xp = static_cast<const T*>(x);
   T* yp = static_cast<T*>(y);
+  switch (resident_k(g, vec)) {
+    case 8: return launch_train_resident<T, 8>(g, xp, yp, a, s);
+    case 16: return launch_train_resident<T, 16>(g, xp, yp, a, s);
+    case RES_KMAX: return launch_train_resident<T, RES_KMAX>(g, xp, yp, a, s);
+    default: break;
+  }
   if (vec == 0) {
     const dim3 grid((unsigned)((g.C + 63) / 64), g.S);
     hipLaunchKernelGGL((bn_stats_col<T, false>), grid, dim3(256), 0, s, g, xp, (const T*)nullptr,
@@ -493,6 +687,12 @@ static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void
   const T* xp = static_cast<const T*>(x);
   const T* dyp = static_cast<const T*>(dy);
   T* dxp = static_cast<T*>(dx);
+  switch (resident_k(g, vec)) {
+    case 8: return launch_bwd_resident<T, 8>(g, xp, dyp, dxp, a, s);
+    case 16: return launch_bwd_resident<T, 16>(g, xp, dyp, dxp, a, s);
+    case RES_KMAX: return launch_bwd_resident<T, RES_KMAX>(g, xp, dyp, dxp, a, s);
+    default: break;
+  }
   if (vec == 0) {
     const dim3 grid((unsigned)((g.C + 63) / 64), g.S);
     hipLaunchKernelGGL((bn_stats_col<T, true>), grid, dim3(256), 0, s, g, xp, dyp, a.save_mean, ws);

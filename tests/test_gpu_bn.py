@@ -22,6 +22,10 @@ CASES = [
     ((6, 300, 2, 2), [2]),          # many features, tiny inner
     ((64, 10), [0]),                # 2-D, per-activation
     ((3, 2, 56, 56), [2]),          # long rows
+    ((8, 8, 130, 3), [2]),          # one workgroup per feature, mostly idle lanes
+    ((28, 28, 128, 9), [2]),        # one workgroup per feature, 8 vectors per thread
+    ((56, 56, 128, 11), [2]),       # ... 16 vectors per thread
+    ((56, 56, 128, 22), [2]),       # ... 25 vectors per thread, part of dy re-read
 ]
 
 
