@@ -304,22 +304,22 @@ bn_bwd_apply_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
 }
 
 // ---- resident kernels (segment mode, 4-wide) ------------------------------------
-// One workgroup of 1024 threads owns a whole feature and keeps its x values in
+// One workgroup (1024 threads, 256 for small features) owns a whole feature and keeps its x values in
 // registers between the reduction and the elementwise pass (K 16-byte vectors per
 // thread), so x is read from memory once.  The backward kernel also parks the
 // first KL vectors of dy per thread in LDS and re-reads only the rest.  Used when
 // a feature fits (outer*inner <= 4096*K) and there are enough features to fill
 // the machine; no workspace, no second launch.
-constexpr int RES_THREADS = 1024;
 constexpr int RES_KMAX = 25;
 constexpr int RES_KL = 9;             // dy vectors per thread parked in LDS (9 x 16 KiB)
-constexpr int RES_MIN_C = 128;        // fewer features leave too many CUs idle
+constexpr int RES_MIN_C_FWD = 64;     // fewer features leave too many CUs idle
+constexpr int RES_MIN_C_BWD = 128;
 
 // Walks this thread's vectors q = tid + 1024*k: f(k, byte offset, in range).  The
 // offset is relative to the tensor base and goes through a buffer descriptor; slots
 // past the feature get an offset past the descriptor's range, so their loads return
 // zero and their stores are dropped without a branch.
-template <int K, int ESZ, int FENCE, typename F>
+template <int RES_THREADS, int K, int ESZ, int FENCE, typename F>
 __device__ __forceinline__ void res_visit(const BnGeom& g, F&& f) {
   constexpr int OOB = (int)0x80000000;
   const int innerV = (int)(g.inner >> 2);
@@ -364,11 +364,11 @@ __device__ __forceinline__ void buf_st4(__amdgpu_buffer_rsrc_t r, int byte_off, 
   __builtin_amdgcn_raw_buffer_store_b64(t, r, byte_off, 0, 2);
 }
 
-template <typename T, int K>
+template <typename T, int RES_THREADS, int K>
 __global__ void __launch_bounds__(RES_THREADS)
 bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restrict__ y,
                   BnTrainArgs a) {
-  __shared__ float red[16];
+  __shared__ float red[RES_THREADS / 64];
   __shared__ float sh[2];
   constexpr int ESZ = (int)sizeof(T);
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
@@ -376,8 +376,8 @@ bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restri
   const float shift = ld(x, (size_t)(c * g.inner));
   float4 xr[K];
   float s1 = 0.f, s2 = 0.f;
-  res_visit<K, ESZ, 0>(g, [&](int k, int off, bool in) { xr[k] = buf_ld4(xr_, off, x); });
-  res_visit<K, ESZ, 1>(g, [&](int k, int, bool in) {
+  res_visit<RES_THREADS, K, ESZ, 0>(g, [&](int k, int off, bool in) { xr[k] = buf_ld4(xr_, off, x); });
+  res_visit<RES_THREADS, K, ESZ, 1>(g, [&](int k, int, bool in) {
     const float t0 = xr[k].x - shift, t1 = xr[k].y - shift, t2 = xr[k].z - shift,
                 t3 = xr[k].w - shift;
     const float p1 = (t0 + t1) + (t2 + t3);
@@ -395,32 +395,31 @@ bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restri
   const float mean = sh[0];
   const float scale = (a.gamma ? a.gamma[c] : 1.f) * sh[1];
   const float bt = a.beta ? a.beta[c] : 0.f;
-  res_visit<K, ESZ, 1>(g, [&](int k, int off, bool) {
+  res_visit<RES_THREADS, K, ESZ, 1>(g, [&](int k, int off, bool) {
     const float4 v = make_float4((xr[k].x - mean) * scale + bt, (xr[k].y - mean) * scale + bt,
                                  (xr[k].z - mean) * scale + bt, (xr[k].w - mean) * scale + bt);
     buf_st4(yr_, off, v, y);
   });
 }
 
-template <typename T, int K>
+template <typename T, int RES_THREADS, int K>
 __global__ void __launch_bounds__(RES_THREADS)
-bn_bwd_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, const T* __restrict__ dy,
+bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, const T* __restrict__ dy,
                 T* __restrict__ dx, BnBwdArgs a) {
-  extern __shared__ float4 dyl[];           // [min(K, RES_KL)][1024]
-  __shared__ float red[16];
+  extern __shared__ float4 dyl[];           // [klim][threads], klim <= min(K, RES_KL)
+  __shared__ float red[RES_THREADS / 64];
   __shared__ float sh[4];
   constexpr int ESZ = (int)sizeof(T);
-  constexpr int KL = K < RES_KL ? K : RES_KL;
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes),
                                dxr_ = make_rsrc(dx, bytes);
   const long long c = blockIdx.x;
   const float mean = a.save_mean[c];
   float4 xr[K];
   float s1 = 0.f, s2 = 0.f;
-  res_visit<K, ESZ, 0>(g, [&](int k, int off, bool in) { xr[k] = buf_ld4(xr_, off, x); });
-  res_visit<K, ESZ, 4>(g, [&](int k, int off, bool in) {
+  res_visit<RES_THREADS, K, ESZ, 0>(g, [&](int k, int off, bool in) { xr[k] = buf_ld4(xr_, off, x); });
+  res_visit<RES_THREADS, K, ESZ, 4>(g, [&](int k, int off, bool in) {
     const float4 d = buf_ld4(dyr_, off, dy);
-    if (k < KL) dyl[k * RES_THREADS + threadIdx.x] = d;
+    if (k < klim) dyl[k * RES_THREADS + threadIdx.x] = d;
     const float p1 = (d.x + d.y) + (d.z + d.w);
     const float p2 = (d.x * (xr[k].x - mean) + d.y * (xr[k].y - mean)) +
                      (d.z * (xr[k].z - mean) + d.w * (xr[k].w - mean));
@@ -435,8 +434,8 @@ bn_bwd_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, const T* __re
   finish_bwd(g, a, c, (double)s1, (double)s2, true, sh);
   __syncthreads();
   const float kdy = sh[1], kx = sh[2], k0 = sh[3];
-  res_visit<K, ESZ, 4>(g, [&](int k, int off, bool) {
-    const float4 d = k < KL ? dyl[k * RES_THREADS + threadIdx.x] : buf_ld4(dyr_, off, dy);
+  res_visit<RES_THREADS, K, ESZ, 4>(g, [&](int k, int off, bool) {
+    const float4 d = k < klim ? dyl[k * RES_THREADS + threadIdx.x] : buf_ld4(dyr_, off, dy);
     const float4 v = make_float4(kdy * d.x + (kx * (xr[k].x - mean) + k0),
                                  kdy * d.y + (kx * (xr[k].y - mean) + k0),
                                  kdy * d.z + (kx * (xr[k].z - mean) + k0),
@@ -609,46 +608,63 @@ static int make_geom(const flhip_bn_desc* d, BnGeom* g, int* vec) {
   return FLHIP_OK;
 }
 
-// Vectors per thread of the resident kernels for this geometry, 0 when they do not
-// apply.  FLHIP_BN_ALGO=split forces the two-kernel path, =resident lifts the
-// feature-count threshold (measurement aids).
-static int resident_k(const BnGeom& g, int vec) {
+// Shape of the resident kernels for this geometry: threads per workgroup and
+// vectors per thread; threads = 0 when they do not apply.  FLHIP_BN_ALGO=split
+// forces the two-kernel path, =resident lifts the feature-count threshold
+// (measurement aids).
+struct ResPlan {
+  int threads, k, need;
+};
+static ResPlan resident_plan(const BnGeom& g, int vec, int min_c) {
   static const int mode = [] {
     const char* e = getenv("FLHIP_BN_ALGO");
     if (e && !strcmp(e, "split")) return 1;
     if (e && !strcmp(e, "resident")) return 2;
     return 0;
   }();
-  if (mode == 1 || vec != 4) return 0;
-  if (g.units > (long long)RES_KMAX * RES_THREADS) return 0;
-  if (g.outer * g.C * g.inner * 4 >= (1ll << 31)) return 0;   // 32-bit buffer offsets
-  if (mode != 2 && g.C < RES_MIN_C) return 0;
-  const int need = (int)((g.units + RES_THREADS - 1) / RES_THREADS);
-  return need <= 8 ? 8 : need <= 16 ? 16 : RES_KMAX;
+  ResPlan r{0, 0, 0};
+  if (mode == 1 || vec != 4) return r;
+  if (g.units > (long long)RES_KMAX * 1024) return r;
+  if (g.outer * g.C * g.inner * 4 >= (1ll << 31)) return r;   // 32-bit buffer offsets
+  if (mode != 2 && g.C < min_c) return r;
+  if (g.units <= 8 * 256) {
+    r.threads = 256;
+    r.k = 8;
+  } else {
+    r.threads = 1024;
+    const int need = (int)((g.units + 1023) / 1024);
+    r.k = need <= 8 ? 8 : need <= 16 ? 16 : RES_KMAX;
+  }
+  r.need = (int)((g.units + r.threads - 1) / r.threads);
+  return r;
 }
 
-template <typename T, int K>
+template <typename T, int THREADS, int K>
 static int launch_train_resident(const BnGeom& g, const T* x, T* y, const BnTrainArgs& a,
                                  hipStream_t s) {
   const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
-  hipLaunchKernelGGL((bn_train_resident<T, K>), dim3((unsigned)g.C), dim3(RES_THREADS), 0, s, g,
-                     bytes, x, y, a);
+  hipLaunchKernelGGL((bn_train_resident<T, THREADS, K>), dim3((unsigned)g.C), dim3(THREADS), 0, s,
+                     g, bytes, x, y, a);
   return check_launch("bn_fwd_train (resident)");
 }
 
-template <typename T, int K>
-static int launch_bwd_resident(const BnGeom& g, const T* x, const T* dy, T* dx, const BnBwdArgs& a,
-                               hipStream_t s) {
+template <typename T, int THREADS, int K>
+static int launch_bwd_resident(const BnGeom& g, int need, const T* x, const T* dy, T* dx,
+                               const BnBwdArgs& a, hipStream_t s) {
   constexpr int KL = K < RES_KL ? K : RES_KL;
-  constexpr size_t shmem = (size_t)KL * RES_THREADS * sizeof(float4);
-  auto kernel = bn_bwd_resident<T, K>;
+  constexpr size_t max_shmem = (size_t)KL * THREADS * sizeof(float4);
+  auto kernel = bn_bwd_resident<T, THREADS, K>;
   static const hipError_t attr = hipFuncSetAttribute(
-      reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+      reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+      (int)max_shmem);
   if (attr != hipSuccess)
     return fail(FLHIP_RUNTIME_ERROR, std::string("bn_bwd: LDS limit: ") + hipGetErrorString(attr));
+  // dy vectors per thread parked in LDS: all of them when the feature is small
+  const int klim = need < KL ? need : KL;
+  const size_t shmem = (size_t)klim * THREADS * sizeof(float4);
   const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
-  hipLaunchKernelGGL(kernel, dim3((unsigned)g.C), dim3(RES_THREADS), shmem, s, g, bytes, x, dy, dx,
-                     a);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)g.C), dim3(THREADS), shmem, s, g, bytes, klim, x, dy,
+                     dx, a);
   return check_launch("bn_bwd (resident)");
 }
 
@@ -657,11 +673,14 @@ static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws
                      const BnTrainArgs& a, hipStream_t s) {
   const T* xp = static_cast<const T*>(x);
   T* yp = static_cast<T*>(y);
-  switch (resident_k(g, vec)) {
-    case 8: return launch_train_resident<T, 8>(g, xp, yp, a, s);
-    case 16: return launch_train_resident<T, 16>(g, xp, yp, a, s);
-    case RES_KMAX: return launch_train_resident<T, RES_KMAX>(g, xp, yp, a, s);
-    default: break;
+  {
+    const ResPlan r = resident_plan(g, vec, RES_MIN_C_FWD);
+    if (r.threads == 256) return launch_train_resident<T, 256, 8>(g, xp, yp, a, s);
+    if (r.threads == 1024) {
+      if (r.k == 8) return launch_train_resident<T, 1024, 8>(g, xp, yp, a, s);
+      if (r.k == 16) return launch_train_resident<T, 1024, 16>(g, xp, yp, a, s);
+      return launch_train_resident<T, 1024, RES_KMAX>(g, xp, yp, a, s);
+    }
   }
   if (vec == 0) {
     const dim3 grid((unsigned)((g.C + 63) / 64), g.S);
@@ -687,11 +706,14 @@ static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void
   const T* xp = static_cast<const T*>(x);
   const T* dyp = static_cast<const T*>(dy);
   T* dxp = static_cast<T*>(dx);
-  switch (resident_k(g, vec)) {
-    case 8: return launch_bwd_resident<T, 8>(g, xp, dyp, dxp, a, s);
-    case 16: return launch_bwd_resident<T, 16>(g, xp, dyp, dxp, a, s);
-    case RES_KMAX: return launch_bwd_resident<T, RES_KMAX>(g, xp, dyp, dxp, a, s);
-    default: break;
+  {
+    const ResPlan r = resident_plan(g, vec, RES_MIN_C_BWD);
+    if (r.threads == 256) return launch_bwd_resident<T, 256, 8>(g, r.need, xp, dyp, dxp, a, s);
+    if (r.threads == 1024) {
+      if (r.k == 8) return launch_bwd_resident<T, 1024, 8>(g, r.need, xp, dyp, dxp, a, s);
+      if (r.k == 16) return launch_bwd_resident<T, 1024, 16>(g, r.need, xp, dyp, dxp, a, s);
+      return launch_bwd_resident<T, 1024, RES_KMAX>(g, r.need, xp, dyp, dxp, a, s);
+    }
   }
   if (vec == 0) {
     const dim3 grid((unsigned)((g.C + 63) / 64), g.S);

@@ -23,7 +23,8 @@ CASES = [
     ((64, 10), [0]),                # 2-D, per-activation
     ((3, 2, 56, 56), [2]),          # long rows
     ((8, 8, 130, 3), [2]),          # one workgroup per feature, mostly idle lanes
-    ((28, 28, 128, 9), [2]),        # one workgroup per feature, 8 vectors per thread
+    ((28, 28, 128, 9), [2]),        # one workgroup of 256 threads per feature
+    ((28, 28, 128, 20), [2]),       # one workgroup of 1024 threads per feature, 8 vectors per thread
     ((56, 56, 128, 11), [2]),       # ... 16 vectors per thread
     ((56, 56, 128, 22), [2]),       # ... 25 vectors per thread, part of dy re-read
 ]
