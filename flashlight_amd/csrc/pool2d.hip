@@ -110,7 +110,7 @@ pool_bwd_direct(PoolGeom g, const T* __restrict__ dy,
 // which keeps the first-maximum tie rule and the fp32 summation order of the
 // generic kernels.
 // ---------------------------------------------------------------------------
-constexpr int POOL_OHB = 8;
+constexpr int POOL_OHB = 2;
 
 struct PoolRow {
   float l;      // column 4*tq - 1 (meaningful when tq > 0)
@@ -118,37 +118,28 @@ struct PoolRow {
   bool ok;      // row inside the image
 };
 
-template <typename T>
-__device__ __forceinline__ PoolRow pool_load_row(const T* xq, int W, int ih, bool ok, int tq,
-                                                 int lane) {
-  PoolRow r;
-  r.ok = ok;
-  r.v = ok ? ld4(xq, (size_t)ih * W) : make_float4(0.f, 0.f, 0.f, 0.f);
-  float up = __shfl_up(r.v.w, 1, 64);
-  if (lane == 0 && tq > 0 && ok) up = ld(xq, (size_t)ih * W - 1);
-  r.l = up;
-  return r;
-}
-
 template <int MODE>
 __device__ __forceinline__ void pool_scan3(const PoolRow& r, int kh, bool has_left, float a,
                                            float b, float c, float& best, int& idx, float& sum,
                                            int& cnt, bool first_col) {
   // one window row: candidates (kw = 0, 1, 2) = (a, b, c); for the first output
-  // column of the thread, a is the neighbour's value and may be padding
-  if (!r.ok) return;
-  if (!first_col || has_left) {
-    if (MODE == FLHIP_POOL_MAX) {
-      if (a > best) { best = a; idx = kh * 3; }
-    } else {
-      sum += a; ++cnt;
-    }
-  }
+  // column of the thread, a is the neighbour's value and may be padding.  Rows and
+  // columns outside the image are skipped by turning their candidates into values
+  // that change nothing (no branches: the strip is straight-line code).
+  const bool use_a = r.ok && (!first_col || has_left);
   if (MODE == FLHIP_POOL_MAX) {
-    if (b > best) { best = b; idx = kh * 3 + 1; }
-    if (c > best) { best = c; idx = kh * 3 + 2; }
+    const float ca = use_a ? a : -FLT_MAX, cb = r.ok ? b : -FLT_MAX, cc = r.ok ? c : -FLT_MAX;
+    if (ca > best) { best = ca; idx = kh * 3; }
+    if (cb > best) { best = cb; idx = kh * 3 + 1; }
+    if (cc > best) { best = cc; idx = kh * 3 + 2; }
   } else {
-    sum += b; sum += c; cnt += 2;
+    // same additions in the same order as the generic kernel; skipped terms add
+    // nothing because they are not added at all (a select keeps the old sum)
+    sum = use_a ? sum + a : sum;
+    cnt += use_a ? 1 : 0;
+    sum = r.ok ? sum + b : sum;
+    sum = r.ok ? sum + c : sum;
+    cnt += r.ok ? 2 : 0;
   }
 }
 
@@ -182,13 +173,39 @@ pool_w3s2_fwd(PoolGeom g, const T* __restrict__ x, T* __restrict__ y,
   const size_t obase = plane * (size_t)g.OH * g.OW + 2 * tq;
   const bool has_left = tq > 0;
 
-  PoolRow r0 = pool_load_row(xq, g.W, 2 * oh0 - 1, oh0 > 0, tq, lane);
-#pragma unroll 2
+  // All 2*POOL_OHB+1 input rows of the strip are requested before any is used: the
+  // 16-byte loads first, then (lane 0 of a wave only) the column left of the quad,
+  // which the other lanes get from their neighbour.
+  constexpr int NR = 2 * POOL_OHB + 1;
+  float4 rv[NR];
+  float rl[NR];
+#pragma unroll
+  for (int j = 0; j < NR; ++j) {
+    // row index clamped into the image (plane sizes are below 2^31 elements)
+    rv[j] = ld4(xq, (size_t)(min(max(2 * oh0 - 1 + j, 0), g.H - 1) * g.W));
+    rl[j] = 0.f;
+  }
+  if (lane == 0 && tq > 0) {
+#pragma unroll
+    for (int j = 0; j < NR; ++j)
+      rl[j] = ld(xq, (size_t)(min(max(2 * oh0 - 1 + j, 0), g.H - 1) * g.W - 1));
+  }
+  // row j of the strip with its left neighbour; `ok` says whether it lies in the image
+  auto row = [&](int j, bool ok) {
+    PoolRow r;
+    r.ok = ok;
+    r.v = rv[j];
+    const float up = __shfl_up(rv[j].w, 1, 64);
+    r.l = lane == 0 ? rl[j] : up;
+    return r;
+  };
+  PoolRow r0 = row(0, oh0 > 0);
+#pragma unroll
   for (int k = 0; k < POOL_OHB; ++k) {
     const int oh = oh0 + k;
     const bool ok = oh < g.OH;
-    const PoolRow r1 = pool_load_row(xq, g.W, 2 * oh, ok && 2 * oh < g.H, tq, lane);
-    const PoolRow r2 = pool_load_row(xq, g.W, 2 * oh + 1, ok && 2 * oh + 1 < g.H, tq, lane);
+    const PoolRow r1 = row(2 * k + 1, ok && 2 * oh < g.H);
+    const PoolRow r2 = row(2 * k + 2, ok && 2 * oh + 1 < g.H);
     float b0 = -FLT_MAX, b1 = -FLT_MAX, s0 = 0.f, s1 = 0.f;
     int i0 = 0, i1 = 0, c0 = 0, c1 = 0;
     pool_scan3<MODE>(r0, 0, has_left, r0.l, r0.v.x, r0.v.y, b0, i0, s0, c0, true);
