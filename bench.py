@@ -26,7 +26,7 @@ PEAK = {"hbm_GBps": 8000.0, "f32_TFLOPs": 157.3, "bf16_TFLOPs": 2500.0}
 CONV_FLOP = 2 * 32 * 64 * 56 * 56 * 64 * 9          # one pass, 7.398752256e9
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by
 # the same counters on the library's copy kernel (see profiles/); None = not measured.
-MEASURED_TRAFFIC = {"conv2d_bwd_data_f32": 76.3e6}
+MEASURED_TRAFFIC = {"conv2d_bwd_data_f32": 61.8e6}
 
 
 def parse():
@@ -231,7 +231,7 @@ def main():
     if "conv2d_bwd_data" in by:
         o = by["conv2d_bwd_data"]
         out["roofline"] = {
-            "kernel": "gather_conv_kernel (conv2dBackwardData, one launch per call)",
+            "kernel": "slab_conv_kernel<float, true> (conv2dBackwardData, one launch per call)",
             "bound": "mfma", "achieved": o["achieved"], "peak": o["peak"], "unit": "TFLOP/s",
             "frac": o["frac"], "avg_launch_us": o["us"],
             "traffic": MEASURED_TRAFFIC.get("conv2d_bwd_data_" + a.dtype)}
