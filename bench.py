@@ -105,11 +105,16 @@ def main():
     cd = capi.ConvDesc(32, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, tag)
     nws = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_BWD_FILTER)
     ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=dev)
+    nws_f = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_FWD)
+    nws_d = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_BWD_DATA)
+    ws_f = torch.empty(max(nws_f, 16), dtype=torch.uint8, device=dev)
+    ws_d = torch.empty(max(nws_d, 16), dtype=torch.uint8, device=dev)
     peak_mfma = PEAK["f32_TFLOPs"] if a.dtype == "f32" else PEAK["bf16_TFLOPs"]
     cdp, xp, wp, bp, dyp, yp, dxp, dwp, dbp, wsp = (C.byref(cd), P(x), P(w), P(b), P(dy), P(y),
                                                      P(dx), P(dw), P(db), P(ws))
-    f_fwd = checked(lambda _: L.flhip_conv2d_fwd(cdp, xp, wp, bp, yp, None, 0, S))
-    f_bwd_data = checked(lambda _: L.flhip_conv2d_bwd_data(cdp, dyp, wp, dxp, None, 0, S))
+    wsfp, wsdp = P(ws_f), P(ws_d)
+    f_fwd = checked(lambda _: L.flhip_conv2d_fwd(cdp, xp, wp, bp, yp, wsfp, nws_f, S))
+    f_bwd_data = checked(lambda _: L.flhip_conv2d_bwd_data(cdp, dyp, wp, dxp, wsdp, nws_d, S))
     f_bwd_filter = checked(lambda _: L.flhip_conv2d_bwd_filter(cdp, xp, dyp, dwp, dbp, wsp, nws, S))
 
     def conv_pair(i):
@@ -128,7 +133,7 @@ def main():
         ops.append({"op": name, "workload": "32x64x56x56, 64 filters 3x3 s1 p1", "dtype": a.dtype,
                     "us": s * 1e6, "bound": "mfma", "achieved": ach, "peak": peak_mfma,
                     "unit": "TFLOP/s", "frac": ach / peak_mfma})
-    del x, w, dy, y, dx, ws
+    del x, w, dy, y, dx, ws, ws_f, ws_d
 
     # ---- bandwidth ops at cfg 3 (fp32) ----------------------------------------
     def bw_op(name, workload, nbytes, fn, nsets):

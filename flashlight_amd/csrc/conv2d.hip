@@ -121,7 +121,8 @@ conv_bwd_bias_kernel(ConvGeom g, const T* __restrict__ dy, float* __restrict__ d
 }
 
 // FLHIP_CONV_ALGO: "direct" = one-thread-per-result kernels, "gather" = skip the
-// LDS-slab kernels; anything else = fastest applicable.
+// LDS-slab kernels, "convert" = skip the bf16 matrix-core kernels (bf16 storage is
+// then converted on load and multiplied in fp32); anything else = fastest applicable.
 static bool algo_is(const char* name) {
   const char* e = getenv("FLHIP_CONV_ALGO");
   return e && strcmp(e, name) == 0;
@@ -153,21 +154,26 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
     const size_t a = mfma_conv_bwd_filter_ws(g, d->dtype), b = mfma_slab_wgrad_ws(g, d->dtype);
     return a > b ? a : b;
   }
+  // bf16 forward / backward-data: room for the weights in matrix-core order (the
+  // passes run without it, on the slower converting kernels)
+  if (d->dtype == FLHIP_BF16 && (pass == FLHIP_CONV_FWD || pass == FLHIP_CONV_BWD_DATA))
+    return mfma_slab16_ws(g, pass == FLHIP_CONV_BWD_DATA);
   return 0;
 }
 
 extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const void* w,
                                 const float* bias, void* y, void* ws, size_t ws_bytes,
                                 void* stream) {
-  (void)ws;
-  (void)ws_bytes;
   FLHIP_REQUIRE(d && x && w && y, "conv2d_fwd: null argument");
   ConvGeom g;
   const int rc = make_geom(d, &g);
   if (rc != FLHIP_OK) return rc;
   hipStream_t s = as_stream(stream);
   if (!force_direct()) {
-    int r = algo_is("gather") ? -1 : mfma_slab_conv_fwd(g, d->dtype, x, w, bias, y, s);
+    int r = -1;
+    if (d->dtype == FLHIP_BF16 && !algo_is("gather") && !algo_is("convert"))
+      r = mfma_slab16_conv_fwd(g, x, w, bias, y, ws, ws_bytes, s);
+    if (r < 0 && !algo_is("gather")) r = mfma_slab_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r < 0) r = mfma_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r >= 0) return r;
   }
@@ -186,15 +192,16 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
 
 extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, const void* w,
                                      void* dx, void* ws, size_t ws_bytes, void* stream) {
-  (void)ws;
-  (void)ws_bytes;
   FLHIP_REQUIRE(d && dy && w && dx, "conv2d_bwd_data: null argument");
   ConvGeom g;
   const int rc = make_geom(d, &g);
   if (rc != FLHIP_OK) return rc;
   hipStream_t s = as_stream(stream);
   if (!force_direct()) {
-    int r = algo_is("gather") ? -1 : mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s);
+    int r = -1;
+    if (d->dtype == FLHIP_BF16 && !algo_is("gather") && !algo_is("convert"))
+      r = mfma_slab16_conv_bwd_data(g, dy, w, dx, ws, ws_bytes, s);
+    if (r < 0 && !algo_is("gather")) r = mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0) r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r >= 0) return r;
   }

@@ -1,0 +1,536 @@
+// Stride-1 convolution (forward and backward-data) for small windows in bf16
+// storage on the bf16 matrix cores (v_mfma_f32_16x16x32_bf16, fp32 accumulate).
+//
+// Same tiling as the fp32 slab kernel: a workgroup owns R whole result rows of one
+// image x 64 result channels; per chunk of 32 source channels the source rows
+// those results need are put in LDS once and every window tap reads them at a
+// shifted address.  What differs is the operand format: an MFMA lane needs eight
+// consecutive source channels of one position (16 bytes), while memory is
+// channel-major.
+//   slab     xs[4 channel groups][slab rows x WSP columns] of 16-byte cells (8
+//            channels of one position).  A loader thread reads eight 16-byte row
+//            pieces (8 channels x 8 columns), transposes them in registers
+//            (v_perm_b32) and stores eight cells.  WSP = 4 (mod 16) and the plane
+//            pitch = 1 (mod 16) put the 16 stores of a quarter wave in 16 distinct
+//            bank groups; the 16 positions of a fragment read are contiguous.
+//   weights  as[4 channel groups][64 result channels x taps] cells.  Memory order is
+//            (channel, tap) or (channel, result channel, tap), so a small kernel
+//            rewrites the weights once per call into that cell order (workspace)
+//            and the main kernel copies cells.
+// 8 waves, two roles as in the fp32 kernel.  The B fragments of tap t+1 are read
+// into the registers tap t has just finished with (one read behind each pair of
+// MFMAs), so one set of fragment registers is enough.
+#include <algorithm>
+
+#include "conv2d_mfma.h"
+
+namespace flhip {
+namespace {
+
+constexpr int CKB = 32;          // source channels per chunk (= K of one MFMA)
+constexpr int CG = CKB / 8;      // channel groups of 8
+constexpr int BM = MFMA_BM;
+constexpr int GTHREADS = 256;
+constexpr int THREADS = 512;
+constexpr int NT_MAX = 13;       // 16-position blocks per MFMA wave
+constexpr int NXU_MAX = 3;       // slab units (8 channels x 8 columns) per loader thread and chunk
+constexpr int NAU_MAX = 9;       // weight cells per loader thread and chunk
+constexpr int KHW_MAX = 9;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+#if defined(__HIP_DEVICE_COMPILE__)
+typedef __attribute__((address_space(3))) const uint4* lds_cell;
+#else
+typedef const uint4* lds_cell;
+#endif
+
+struct Slab16Params {
+  int stage_ok;          // result rows are 16-byte aligned and a half tile fits in LDS
+  int N, SC, SH, SW, DC, DH, DW;
+  int KH, KW, KHW, dly, dlx;
+  int sh0, sw0;          // window shift of tap (0,0): fwd -py,-px ; bwd +py,+px
+  int shs, sws;          // shift step per kh / kw: fwd +dly,+dlx ; bwd -dly,-dlx
+  int min_sh, min_sw;    // smallest shifts (slab origin relative to the result origin)
+  int groups, SCg, DCg;
+  int a_mstride, a_cstride, w_group_stride;
+  int R, RS;             // result rows per tile, slab rows
+  int WSP, XOFF;         // slab row pitch (positions), slab column of image column 0
+  int XPL, APL;          // plane pitches in cells: slab, weights
+  int tiles_per_image, mtiles;
+  int NB;                // ceil(R*DW / 16)
+  int nchunks;           // ceil(SCg / 32)
+  int x_cells, a_cells;  // per buffer, spare cells for idle loader lanes included
+  unsigned src_bytes, wt_bytes;
+};
+
+// Weights in cell order: cell (grp, mtile, chunk, channel group, m, tap) holds the 8
+// source channels chunk*32 + cg*8 .. +7 of result channel mtile*64 + m; channels or
+// result channels past the end are zero.
+__global__ void __launch_bounds__(256)
+slab16_weight_cells(Slab16Params p, const bf16_t* __restrict__ w, uint4* __restrict__ out,
+                    int ncells) {
+  const int cell = blockIdx.x * 256 + threadIdx.x;
+  if (cell >= ncells) return;
+  int t = cell;
+  const int tap = t % p.KHW; t /= p.KHW;
+  const int m = t % BM; t /= BM;
+  const int cg = t % CG; t /= CG;
+  const int chunk = t % p.nchunks; t /= p.nchunks;
+  const int mtile = t % p.mtiles;
+  const int grp = t / p.mtiles;
+  const int c0 = chunk * CKB + cg * 8;
+  const bool m_ok = mtile * BM + m < p.DCg;
+  const int base = grp * p.w_group_stride + (mtile * BM + m) * p.a_mstride + tap;
+  unsigned h[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    h[i] = (m_ok && c0 + i < p.SCg) ? (unsigned)w[base + (c0 + i) * p.a_cstride] : 0u;
+  out[cell] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16),
+                         h[6] | (h[7] << 16));
+}
+
+template <bool BWD>
+__global__ void __launch_bounds__(THREADS, 2)
+slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const uint4* __restrict__ wcells,
+                   const float* __restrict__ bias, bf16_t* __restrict__ dst) {
+  extern __shared__ uint4 lds16[];
+  uint4* Xs = lds16;                            // [2][x_cells]
+  uint4* As = lds16 + 2 * p.x_cells;            // [2][a_cells]
+  float* lds = reinterpret_cast<float*>(lds16);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int img = blockIdx.x / p.tiles_per_image;
+  const int r0 = (blockIdx.x % p.tiles_per_image) * p.R;
+  const int grp = blockIdx.y / p.mtiles, mtile = blockIdx.y % p.mtiles;
+  const int m_lim = p.DCg - mtile * BM;
+  const int rows = min(p.R, p.DH - r0);          // result rows of this tile
+  const int n = p.nchunks;
+  const int npos = rows * p.DW;
+
+  // Halo columns of both slab buffers are never written by a chunk: zero them once.
+  for (int i = tid; i < 2 * p.x_cells; i += THREADS) Xs[i] = make_uint4(0u, 0u, 0u, 0u);
+  __syncthreads();
+
+  // Epilogue through LDS (when rows are 16-byte aligned): the MFMA waves of one
+  // channel half park their accumulators as stage[32 channels][npos] floats, then
+  // all 512 threads write each channel's run of npos results, 4 at a time.
+  const int SP = ((npos + 3) & ~3) + 4;                       // stage pitch (words)
+  const bool staged = p.stage_ok && (npos & 3) == 0;
+  auto coop_store = [&](int h) {
+    const int q4 = npos >> 2;
+    const size_t out_base = (size_t)img * p.DC * p.DH * p.DW + (size_t)r0 * p.DW;
+    for (int idx = tid; idx < 32 * q4; idx += THREADS) {
+      const int ch_l = idx / q4, q = idx - ch_l * q4;
+      const int m = h * 32 + ch_l;
+      if (m < m_lim) {
+        const int ch = grp * p.DCg + mtile * BM + m;
+        const float b = bias ? bias[ch] : 0.f;
+        float4 v = *reinterpret_cast<const float4*>(lds + ch_l * SP + 4 * q);
+        v.x += b; v.y += b; v.z += b; v.w += b;
+        st4_stream(dst, out_base + (size_t)ch * p.DH * p.DW + 4 * q, v);
+      }
+    }
+  };
+
+  if (wave < 4) {
+    // ============================ loader waves ===================================
+    const __amdgpu_buffer_rsrc_t srsrc = make_rsrc(src, p.src_bytes);
+    const __amdgpu_buffer_rsrc_t wrsrc = make_rsrc(wcells, p.wt_bytes);
+    constexpr int OOB = (int)0x80000000;
+    const int chan_bytes = p.SH * p.SW * 2;
+    const int img_base = (img * p.SC + grp * p.SCg) * p.SH * p.SW;
+    // slab unit u: bits 0-1 channel group, bits 2-3 low bits of the slab row, then the
+    // group of 8 image columns, then the high bits of the row (see the bank note above)
+    const int qrow = p.SW >> 3, rs_hi = (p.RS + 3) >> 2;
+    const int n_units = CG * 4 * qrow * rs_hi;
+    int xg[NXU_MAX], xl[NXU_MAX];                // global byte offset of channel 0 of the group, LDS cell
+    int xc[NXU_MAX];                             // first channel of the unit within the chunk
+#pragma unroll
+    for (int i = 0; i < NXU_MAX; ++i) {
+      const int u = tid + GTHREADS * i;
+      xg[i] = OOB;
+      xl[i] = p.x_cells - 8;
+      xc[i] = 0;
+      if (u < n_units) {
+        const int cg = u & 3, rl = (u >> 2) & 3;
+        const int t = u >> 4;
+        const int q = t % qrow, rh = t / qrow;
+        const int rs = rh * 4 + rl;
+        const int sr = r0 + p.min_sh + rs;
+        xc[i] = cg * 8;
+        if (rs < p.RS) {
+          xl[i] = cg * p.XPL + rs * p.WSP + p.XOFF + 8 * q;
+          if ((unsigned)sr < (unsigned)p.SH) xg[i] = (img_base + (cg * 8 * p.SH + sr) * p.SW + 8 * q) * 2;
+        }
+      }
+    }
+    // weight cells of this tile and chunk are contiguous in the workspace
+    const int chunk_cells = CG * p.APL;
+    const int wt_base = ((grp * p.mtiles + mtile) * n) * chunk_cells;
+    const int nau = (chunk_cells + GTHREADS - 1) / GTHREADS;
+
+    uint4 xv[NXU_MAX][8], av[NAU_MAX];
+    auto load_chunk = [&](int chunk) {
+      const int c0 = chunk * CKB;
+      const int xbase = c0 * chan_bytes;
+#pragma unroll
+      for (int i = 0; i < NXU_MAX; ++i)
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          // channels past the end of the group read zero
+          const int off = (c0 + xc[i] + k < p.SCg) ? xg[i] + xbase + k * chan_bytes : OOB;
+          const uintx4_t v = __builtin_amdgcn_raw_buffer_load_b128(srsrc, off, 0, 0);
+          xv[i][k] = make_uint4(v.x, v.y, v.z, v.w);
+        }
+#pragma unroll
+      for (int i = 0; i < NAU_MAX; ++i) {
+        const int cell = tid + GTHREADS * i;
+        const int off = (i < nau && cell < chunk_cells) ? (wt_base + chunk * chunk_cells + cell) * 16 : OOB;
+        const uintx4_t v = __builtin_amdgcn_raw_buffer_load_b128(wrsrc, off, 0, 0);
+        av[i] = make_uint4(v.x, v.y, v.z, v.w);
+      }
+    };
+    auto store_chunk = [&](int buf) {
+      uint4* xs = Xs + buf * p.x_cells;
+      uint4* as = As + buf * p.a_cells;
+#pragma unroll
+      for (int i = 0; i < NXU_MAX; ++i) {
+        // 8x8 transpose of 16-bit values: column 2t+s of channels 2k, 2k+1 is the low
+        // (s = 0) or high (s = 1) half of dword t of the two rows
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          unsigned lo[4], hi[4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const unsigned e = t == 0 ? xv[i][2 * k].x : t == 1 ? xv[i][2 * k].y : t == 2 ? xv[i][2 * k].z : xv[i][2 * k].w;
+            const unsigned o = t == 0 ? xv[i][2 * k + 1].x : t == 1 ? xv[i][2 * k + 1].y : t == 2 ? xv[i][2 * k + 1].z : xv[i][2 * k + 1].w;
+            lo[k] = __builtin_amdgcn_perm(o, e, 0x05040100u);
+            hi[k] = __builtin_amdgcn_perm(o, e, 0x07060302u);
+          }
+          xs[xl[i] + 2 * t] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+          xs[xl[i] + 2 * t + 1] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < NAU_MAX; ++i) {
+        const int cell = tid + GTHREADS * i;
+        as[(i < nau && cell < chunk_cells) ? cell : p.a_cells - 1] = av[i];
+      }
+    };
+    load_chunk(0);
+    store_chunk(0);
+    __syncthreads();
+    for (int c = 0; c < n; ++c) {
+      if (c + 1 < n) {
+        load_chunk(c + 1);
+        store_chunk((c + 1) & 1);
+      }
+      __syncthreads();
+    }
+    if (staged) {
+      for (int h = 0; h < 2; ++h) {
+        __syncthreads();        // half h is staged
+        coop_store(h);
+        __syncthreads();        // stage may be overwritten
+      }
+    }
+    return;
+  }
+
+  // =============================== MFMA waves ====================================
+  const int cw = wave - 4;
+  const int wm = cw & 1, wn = cw >> 1;
+  const int base = p.NB >> 1, rem = p.NB & 1;
+  const int nt = base + (wn < rem ? 1 : 0);
+  const int nb0 = wn * base + min(wn, rem);
+  const int fr = lane & 15, fk = lane >> 4;
+  auto run = [&](auto ntc) {
+    constexpr int NT = decltype(ntc)::value;
+    floatx4 acc[2][NT];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const int row_step = p.shs * p.WSP, col_step = p.sws;            // window row / column
+    const int origin = (p.sh0 - p.min_sh) * p.WSP + p.sw0;           // tap (0,0)
+    // 3x3 window with adjacent columns: straight-line taps, a window row walked
+    // towards larger slab columns (forward kw = 0,1,2, backward kw = 2,1,0)
+    const bool static33 = p.KH == 3 && p.KW == 3 && p.dlx == 1;
+    const int first = origin + (static33 ? (BWD ? 2 : 0) * col_step : 0);
+    const float inv_dw = 1.0f / (float)p.DW;
+    lds_cell bp[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      int pos = (nb0 + j) * 16 + fr;
+      if (pos >= npos) pos = 0;                  // padding lanes compute a discarded column
+      int w;
+      const int r = fast_div(pos, p.DW, inv_dw, &w);
+      bp[j] = (lds_cell)Xs + (fk * p.XPL + r * p.WSP + w + p.XOFF + first);
+    }
+    lds_cell ap = (lds_cell)As + (fk * p.APL + (wm * 32 + fr) * p.KHW);
+
+    auto frag = [](uint4 v) { return __builtin_bit_cast(bf16x8, v); };
+    auto mma2 = [&](int j, uint4 a0, uint4 a1, uint4 b) {
+      acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(a0), frag(b), acc[0][j], 0, 0, 0);
+      acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(a1), frag(b), acc[1][j], 0, 0, 0);
+    };
+
+    __syncthreads();                             // chunk 0 is in buffer 0
+    for (int c = 0; c < n; ++c) {
+      if (static33) {
+        constexpr int T0 = BWD ? 2 : 0, TD = BWD ? -1 : 1;   // kw of the first tap, kw step
+        uint4 b[NT], a0, a1;
+        a0 = ap[T0];
+        a1 = ap[16 * 9 + T0];
+#pragma unroll
+        for (int j = 0; j < NT; ++j) b[j] = bp[j][0];
+        // tap t: MFMAs on (a0, a1, b); behind each pair the fragment of tap t+1 is read
+        // into the b register just used
+#define FLHIP_TAP16(NEXT_TAP, NEXT_OFF)                                  \
+  {                                                                      \
+    __builtin_amdgcn_sched_barrier(0);                                   \
+    const uint4 n0 = ap[NEXT_TAP], n1 = ap[16 * 9 + (NEXT_TAP)];         \
+    _Pragma("unroll") for (int j = 0; j < NT; ++j) {                     \
+      mma2(j, a0, a1, b[j]);                                             \
+      b[j] = bp[j][NEXT_OFF];                                            \
+    }                                                                    \
+    a0 = n0;                                                             \
+    a1 = n1;                                                             \
+    _Pragma("unroll") for (int q = 0; q < NT + 2; ++q) {                 \
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                 \
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                 \
+    }                                                                    \
+    __builtin_amdgcn_sched_barrier(0);                                   \
+  }
+#define FLHIP_NEXT_ROW16 _Pragma("unroll") for (int j = 0; j < NT; ++j) bp[j] += row_step;
+        FLHIP_TAP16(T0 + TD, 1)
+        FLHIP_TAP16(T0 + 2 * TD, 2)
+        FLHIP_NEXT_ROW16
+        FLHIP_TAP16(3 + T0, 0)
+        FLHIP_TAP16(3 + T0 + TD, 1)
+        FLHIP_TAP16(3 + T0 + 2 * TD, 2)
+        FLHIP_NEXT_ROW16
+        FLHIP_TAP16(6 + T0, 0)
+        FLHIP_TAP16(6 + T0 + TD, 1)
+        FLHIP_TAP16(6 + T0 + 2 * TD, 2)
+#undef FLHIP_NEXT_ROW16
+#undef FLHIP_TAP16
+#pragma unroll
+        for (int j = 0; j < NT; ++j) mma2(j, a0, a1, b[j]);
+      } else {
+        int tap = 0;
+        for (int kh = 0; kh < p.KH; ++kh) {
+          for (int kw = 0; kw < p.KW; ++kw, ++tap) {
+            const uint4 a0 = ap[tap], a1 = ap[16 * p.KHW + tap];
+#pragma unroll
+            for (int j = 0; j < NT; ++j) mma2(j, a0, a1, bp[j][0]);
+#pragma unroll
+            for (int j = 0; j < NT; ++j) bp[j] += col_step;
+          }
+#pragma unroll
+          for (int j = 0; j < NT; ++j) bp[j] += row_step - p.KW * col_step;
+        }
+      }
+      // back to the first tap, in the other buffer
+      {
+        const int sign = (c & 1) ? -1 : 1;
+        const int xd = sign * p.x_cells - (p.KH - 1) * row_step - (static33 ? 0 : row_step);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) bp[j] += xd;
+        ap += sign * p.a_cells;
+      }
+      __syncthreads();
+    }
+
+    // ---- epilogue ----------------------------------------------------------------
+    if (staged) {
+      for (int h = 0; h < 2; ++h) {
+        if (wm == h) {
+#pragma unroll
+          for (int j = 0; j < NT; ++j) {
+            const int pos = (nb0 + j) * 16 + fr;
+            if (pos < npos) {
+#pragma unroll
+              for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) lds[(i * 16 + fk * 4 + r) * SP + pos] = acc[i][j][r];
+            }
+          }
+        }
+        __syncthreads();
+        coop_store(h);
+        __syncthreads();
+      }
+      return;
+    }
+    float bv[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = wm * 32 + i * 16 + fk * 4 + r;
+        bv[i][r] = (bias && m < m_lim) ? bias[grp * p.DCg + mtile * BM + m] : 0.f;
+      }
+    const size_t out_base = (size_t)img * p.DC * p.DH * p.DW + (size_t)r0 * p.DW;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int pos = (nb0 + j) * 16 + fr;
+      if (pos < npos) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int m = wm * 32 + i * 16 + fk * 4 + r;
+            if (m < m_lim) {
+              const int ch = grp * p.DCg + mtile * BM + m;
+              st(dst, out_base + (size_t)ch * p.DH * p.DW + pos, acc[i][j][r] + bv[i][r]);
+            }
+          }
+      }
+    }
+  };
+
+  switch (nt) {
+    case 0: case 1: run(std::integral_constant<int, 1>{}); break;
+    case 2: run(std::integral_constant<int, 2>{}); break;
+    case 3: run(std::integral_constant<int, 3>{}); break;
+    case 4: run(std::integral_constant<int, 4>{}); break;
+    case 5: run(std::integral_constant<int, 5>{}); break;
+    case 6: run(std::integral_constant<int, 6>{}); break;
+    case 7: run(std::integral_constant<int, 7>{}); break;
+    case 8: run(std::integral_constant<int, 8>{}); break;
+    case 9: run(std::integral_constant<int, 9>{}); break;
+    case 10: run(std::integral_constant<int, 10>{}); break;
+    case 11: run(std::integral_constant<int, 11>{}); break;
+    case 12: run(std::integral_constant<int, 12>{}); break;
+    default: run(std::integral_constant<int, 13>{}); break;
+  }
+}
+
+// smallest value >= v that is congruent to r modulo m
+inline int round_to_residue(int v, int r, int m) { return v + ((r - v) % m + m) % m; }
+
+void layout(Slab16Params* p, int R) {
+  p->R = R;
+  p->RS = R + (p->KH - 1) * p->dly;
+  p->XOFF = std::max(0, -p->min_sw);
+  const int max_sc = p->min_sw + p->DW - 1 + (p->KW - 1) * p->dlx;   // last source column read
+  p->WSP = round_to_residue(p->XOFF + std::max(max_sc + 1, p->SW), 4, 16);
+  p->XPL = round_to_residue(p->RS * p->WSP, 1, 16);
+  p->x_cells = CG * p->XPL + 8;
+  p->APL = BM * p->KHW;
+  p->a_cells = CG * p->APL + 1;
+}
+
+bool plan(Slab16Params* p, size_t* shmem) {
+  if (p->KHW > KHW_MAX) return false;
+  if (p->SW % 8 != 0) return false;              // rows are read 16 bytes at a time
+  const int max_pos = 2 * NT_MAX * 16;
+  if (p->DW > max_pos) return false;
+  const int cus = mfma_num_cus();
+  int best_r = 0;
+  double best_cost = 1e30;
+  for (int R = 1; R <= p->DH && R * p->DW <= max_pos; ++R) {
+    layout(p, R);
+    const size_t bytes = (size_t)2 * (p->x_cells + p->a_cells) * 16;
+    if (bytes > 156 * 1024) break;
+    if (CG * 4 * (p->SW / 8) * ((p->RS + 3) / 4) > GTHREADS * NXU_MAX) break;
+    const long long tiles = (long long)p->N * ((p->DH + R - 1) / R) * p->mtiles * p->groups;
+    const long long rounds = (tiles + cus - 1) / cus;
+    const int nb = (R * p->DW + 15) / 16;
+    const double cost = (double)rounds * ((nb + 1) / 2 + 0.5);
+    if (cost < best_cost - 1e-9) {
+      best_cost = cost;
+      best_r = R;
+    }
+  }
+  if (best_r == 0) return false;
+  layout(p, best_r);
+  if ((CG * p->APL + GTHREADS - 1) / GTHREADS > NAU_MAX) return false;
+  p->tiles_per_image = (p->DH + best_r - 1) / best_r;
+  p->NB = (best_r * p->DW + 15) / 16;
+  p->nchunks = (p->SCg + CKB - 1) / CKB;
+  *shmem = (size_t)2 * (p->x_cells + p->a_cells) * 16;
+  {
+    const int npos = best_r * p->DW, sp = ((npos + 3) & ~3) + 4;
+    p->stage_ok = p->DW % 4 == 0 && (size_t)32 * sp * sizeof(float) <= *shmem;
+  }
+  return best_r * p->DW >= 64;
+}
+
+size_t cells_of(const Slab16Params& p) {
+  return (size_t)p.groups * p.mtiles * p.nchunks * CG * p.APL;
+}
+
+template <bool BWD>
+int launch(Slab16Params& p, const void* src, const void* wgt, const float* bias, void* dst,
+           void* ws, size_t ws_bytes, hipStream_t s) {
+  const long long sbytes = (long long)p.N * p.SC * p.SH * p.SW * 2;
+  if (sbytes >= (1ll << 31)) return -1;
+  if (reinterpret_cast<uintptr_t>(src) % 16 != 0 || reinterpret_cast<uintptr_t>(ws) % 16 != 0) return -1;
+  p.src_bytes = (unsigned)sbytes;
+  size_t shmem = 0;
+  if (!plan(&p, &shmem)) return -1;
+  const size_t ncells = cells_of(p);
+  if (!ws || ws_bytes < ncells * 16 || ncells * 16 >= (1ull << 31)) return -1;
+  p.wt_bytes = (unsigned)(ncells * 16);
+  if (reinterpret_cast<uintptr_t>(dst) % 8 != 0) p.stage_ok = 0;
+  auto kernel = slab16_conv_kernel<BWD>;
+  if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
+  hipLaunchKernelGGL(slab16_weight_cells, dim3((unsigned)((ncells + 255) / 256)), dim3(256), 0, s, p,
+                     static_cast<const bf16_t*>(wgt), static_cast<uint4*>(ws), (int)ncells);
+  const dim3 grid((unsigned)(p.N * p.tiles_per_image), (unsigned)(p.mtiles * p.groups));
+  hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const bf16_t*>(src),
+                     static_cast<const uint4*>(ws), bias, static_cast<bf16_t*>(dst));
+  return check_launch("conv2d (bf16 mfma slab)");
+}
+
+void fill_fwd(const ConvGeom& g, Slab16Params* p) {
+  p->N = g.N; p->SC = g.C; p->SH = g.H; p->SW = g.W; p->DC = g.K; p->DH = g.OH; p->DW = g.OW;
+  p->KH = g.KH; p->KW = g.KW; p->KHW = g.KH * g.KW; p->dly = g.dly; p->dlx = g.dlx;
+  p->sh0 = -g.py; p->sw0 = -g.px; p->shs = g.dly; p->sws = g.dlx;
+  p->min_sh = -g.py; p->min_sw = -g.px;
+  p->groups = g.groups; p->SCg = g.Cg; p->DCg = g.Kg;
+  p->a_mstride = g.Cg * p->KHW; p->a_cstride = p->KHW; p->w_group_stride = g.Kg * g.Cg * p->KHW;
+  p->mtiles = (g.Kg + BM - 1) / BM;
+}
+
+void fill_bwd(const ConvGeom& g, Slab16Params* p) {
+  p->N = g.N; p->SC = g.K; p->SH = g.OH; p->SW = g.OW; p->DC = g.C; p->DH = g.H; p->DW = g.W;
+  p->KH = g.KH; p->KW = g.KW; p->KHW = g.KH * g.KW; p->dly = g.dly; p->dlx = g.dlx;
+  p->sh0 = g.py; p->sw0 = g.px; p->shs = -g.dly; p->sws = -g.dlx;
+  p->min_sh = g.py - (g.KH - 1) * g.dly; p->min_sw = g.px - (g.KW - 1) * g.dlx;
+  p->groups = g.groups; p->SCg = g.Kg; p->DCg = g.Cg;
+  p->a_mstride = p->KHW; p->a_cstride = g.Cg * p->KHW; p->w_group_stride = g.Kg * g.Cg * p->KHW;
+  p->mtiles = (g.Cg + BM - 1) / BM;
+}
+
+}  // namespace
+
+size_t mfma_slab16_ws(const ConvGeom& g, bool bwd) {
+  if (g.sy != 1 || g.sx != 1) return 0;
+  Slab16Params p{};
+  if (bwd) fill_bwd(g, &p); else fill_fwd(g, &p);
+  size_t shmem = 0;
+  if (!plan(&p, &shmem)) return 0;
+  return cells_of(p) * 16;
+}
+
+int mfma_slab16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
+                         void* ws, size_t ws_bytes, hipStream_t s) {
+  if (g.sy != 1 || g.sx != 1) return -1;
+  Slab16Params p{};
+  fill_fwd(g, &p);
+  return launch<false>(p, x, w, bias, y, ws, ws_bytes, s);
+}
+
+int mfma_slab16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, void* ws,
+                              size_t ws_bytes, hipStream_t s) {
+  if (g.sy != 1 || g.sx != 1) return -1;
+  Slab16Params p{};
+  fill_bwd(g, &p);
+  return launch<true>(p, dy, w, nullptr, dx, ws, ws_bytes, s);
+}
+
+}  // namespace flhip

@@ -36,6 +36,9 @@ MORE = [
     ((1, 32, 5, 24), (64, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),        # slab, rows of 3 groups of 8
     ((1, 32, 6, 18), (70, 32, 3, 3), (1, 1), (0, 0), (1, 1), 1),        # slab, rows not 16-byte aligned
     ((2, 32, 9, 20), (64, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),        # slab, row length 4 (mod 8)
+    ((1, 64, 20, 56), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),       # ResNet row length, two 32-channel chunks
+    ((2, 40, 6, 16), (72, 40, 3, 3), (1, 1), (1, 1), (1, 1), 1),        # channel tails on both sides (bf16 matrix-core path)
+    ((1, 96, 5, 8), (32, 48, 2, 3), (1, 1), (1, 1), (1, 1), 2),         # groups, 2x3 window (bf16 generic tap loop)
 ]
 ALL = LIB_CASES + MORE
 
