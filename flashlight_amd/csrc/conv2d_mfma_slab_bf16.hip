@@ -99,9 +99,12 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const uint4* 
   float* lds = reinterpret_cast<float*>(lds16);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int img = blockIdx.x / p.tiles_per_image;
-  const int r0 = (blockIdx.x % p.tiles_per_image) * p.R;
-  const int grp = blockIdx.y / p.mtiles, mtile = blockIdx.y % p.mtiles;
+  // workgroup-uniform values go through readfirstlane: integer division runs on the
+  // vector ALU, and without it everything derived from these lives in (spilled) VGPRs
+  const int img = __builtin_amdgcn_readfirstlane(blockIdx.x / p.tiles_per_image);
+  const int r0 = __builtin_amdgcn_readfirstlane((blockIdx.x % p.tiles_per_image) * p.R);
+  const int grp = __builtin_amdgcn_readfirstlane(blockIdx.y / p.mtiles);
+  const int mtile = __builtin_amdgcn_readfirstlane(blockIdx.y % p.mtiles);
   const int m_lim = p.DCg - mtile * BM;
   const int rows = min(p.R, p.DH - r0);          // result rows of this tile
   const int n = p.nchunks;
@@ -109,6 +112,10 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const uint4* 
 
   // Halo columns of both slab buffers are never written by a chunk: zero them once.
   for (int i = tid; i < 2 * p.x_cells; i += THREADS) Xs[i] = make_uint4(0u, 0u, 0u, 0u);
+  // bias of the tile's 64 result channels, behind the operand buffers (the epilogue
+  // then needs no global loads)
+  float* bias_lds = lds + 8 * (p.x_cells + p.a_cells);
+  if (tid < BM) bias_lds[tid] = (bias && tid < m_lim) ? bias[grp * p.DCg + mtile * BM + tid] : 0.f;
   __syncthreads();
 
   // Epilogue through LDS (when rows are 16-byte aligned): the MFMA waves of one
@@ -118,17 +125,17 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const uint4* 
   const bool staged = p.stage_ok && (npos & 3) == 0;
   auto coop_store = [&](int h) {
     const int q4 = npos >> 2;
+    const float inv_q4 = 1.0f / (float)q4;
     const size_t out_base = (size_t)img * p.DC * p.DH * p.DW + (size_t)r0 * p.DW;
-    for (int idx = tid; idx < 32 * q4; idx += THREADS) {
-      const int ch_l = idx / q4, q = idx - ch_l * q4;
-      const int m = h * 32 + ch_l;
-      if (m < m_lim) {
-        const int ch = grp * p.DCg + mtile * BM + m;
-        const float b = bias ? bias[ch] : 0.f;
-        float4 v = *reinterpret_cast<const float4*>(lds + ch_l * SP + 4 * q);
-        v.x += b; v.y += b; v.z += b; v.w += b;
-        st4_stream(dst, out_base + (size_t)ch * p.DH * p.DW + 4 * q, v);
-      }
+    const int ch0 = grp * p.DCg + mtile * BM + h * 32;
+    const int lim = min(32, m_lim - h * 32) * q4;
+    for (int idx = tid; idx < lim; idx += THREADS) {
+      int q;
+      const int ch_l = fast_div(idx, q4, inv_q4, &q);
+      float4 v = *reinterpret_cast<const float4*>(lds + ch_l * SP + 4 * q);
+      const float b = bias_lds[h * 32 + ch_l];
+      v.x += b; v.y += b; v.z += b; v.w += b;
+      st4_stream(dst, out_base + (size_t)(ch0 + ch_l) * p.DH * p.DW + 4 * q, v);
     }
   };
 
@@ -368,10 +375,7 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const uint4* 
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int m = wm * 32 + i * 16 + fk * 4 + r;
-        bv[i][r] = (bias && m < m_lim) ? bias[grp * p.DCg + mtile * BM + m] : 0.f;
-      }
+      for (int r = 0; r < 4; ++r) bv[i][r] = bias_lds[wm * 32 + i * 16 + fk * 4 + r];
     const size_t out_base = (size_t)img * p.DC * p.DH * p.DW + (size_t)r0 * p.DW;
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
@@ -451,10 +455,10 @@ bool plan(Slab16Params* p, size_t* shmem) {
   p->tiles_per_image = (p->DH + best_r - 1) / best_r;
   p->NB = (best_r * p->DW + 15) / 16;
   p->nchunks = (p->SCg + CKB - 1) / CKB;
-  *shmem = (size_t)2 * (p->x_cells + p->a_cells) * 16;
+  *shmem = (size_t)2 * (p->x_cells + p->a_cells) * 16 + BM * sizeof(float);
   {
     const int npos = best_r * p->DW, sp = ((npos + 3) & ~3) + 4;
-    p->stage_ok = p->DW % 4 == 0 && (size_t)32 * sp * sizeof(float) <= *shmem;
+    p->stage_ok = p->DW % 4 == 0 && (size_t)32 * sp * sizeof(float) <= *shmem - BM * sizeof(float);
   }
   return best_r * p->DW >= 64;
 }

@@ -63,7 +63,9 @@ wgrad_slab_kernel(WSlabParams p, const T* __restrict__ x, const T* __restrict__ 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int split = blockIdx.x;
-  const int half = blockIdx.y % p.nhalves, mtile = blockIdx.y / p.nhalves;
+  // readfirstlane: the division runs on the vector ALU, the results are uniform
+  const int half = __builtin_amdgcn_readfirstlane(blockIdx.y % p.nhalves);
+  const int mtile = __builtin_amdgcn_readfirstlane(blockIdx.y / p.nhalves);
   const int grp = blockIdx.z;
   const int m_lim = p.Kg - mtile * BM;
   const int row_begin = split * p.rps, row_end = min(row_begin + p.rps, p.total_rows);
