@@ -38,6 +38,9 @@ int mfma_slab_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const 
 size_t mfma_slab16_ws(const ConvGeom& g, bool bwd);
 int mfma_slab16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
                          void* ws, size_t ws_bytes, hipStream_t s);
+size_t mfma_wgrad16_ws(const ConvGeom& g);
+int mfma_wgrad16(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
+                 size_t ws_bytes, hipStream_t s);
 int mfma_slab16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, void* ws,
                               size_t ws_bytes, hipStream_t s);
 

@@ -151,8 +151,11 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
   if (make_geom(d, &g) != FLHIP_OK) return 0;
   if (pass == FLHIP_CONV_BWD_FILTER) {
     // the larger of the two filter-gradient plans, so either kernel can run
-    const size_t a = mfma_conv_bwd_filter_ws(g, d->dtype), b = mfma_slab_wgrad_ws(g, d->dtype);
-    return a > b ? a : b;
+    size_t a = mfma_conv_bwd_filter_ws(g, d->dtype);
+    const size_t b = mfma_slab_wgrad_ws(g, d->dtype);
+    const size_t c = d->dtype == FLHIP_BF16 ? mfma_wgrad16_ws(g) : 0;
+    if (b > a) a = b;
+    return c > a ? c : a;
   }
   // bf16 forward / backward-data: room for the weights in matrix-core order (the
   // passes run without it, on the slower converting kernels)
@@ -231,7 +234,10 @@ extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, 
   if (!force_direct()) {
     const size_t need = flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER);
     FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter: workspace too small");
-    int r = algo_is("gather") ? -1 : mfma_slab_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
+    int r = -1;
+    if (d->dtype == FLHIP_BF16 && !algo_is("gather") && !algo_is("convert"))
+      r = mfma_wgrad16(g, x, dy, dw, db, ws, ws_bytes, s);
+    if (r < 0 && !algo_is("gather")) r = mfma_slab_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0) r = mfma_conv_bwd_filter(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
     if (r >= 0) return r;
   }

@@ -1,0 +1,389 @@
+// Filter (and bias) gradient for 3x3 stride-1 pad-1 convolutions in bf16 storage on
+// the bf16 matrix cores (v_mfma_f32_16x16x32_bf16, fp32 accumulate and fp32 result).
+//
+// dw[m, (c,kh,kw)] = sum over positions of dy[m, pos] * x[c, pos + shift].  The
+// contraction index is the position, which is contiguous in memory for both
+// operands, so the fragments (8 consecutive positions per lane) need no transpose.
+// A workgroup owns 64 output channels x 32 input channels (288 columns) over a
+// range of (image, output row) pairs, as the fp32 row kernel does.  Per output row
+// LDS holds
+//   ds[64 output channels][OWp]            the dy row, zero past OW
+//   xs[288 columns = (c,kh,kw)][OWp]       input row ih(kh) of channel c shifted by
+//                                          kw-1 columns: x[p + kw - 1], zero outside
+// (bf16, OWp = OW rounded up to 32, row pitch OWp*2+16 bytes so that the 16 rows of a
+// fragment read fall on distinct banks).  The three shifted copies are made in
+// registers from one aligned 16-byte load per 8 columns: the neighbouring columns
+// come from the adjacent lanes, v_alignbit_b32 shifts by one element.
+// 8 waves, two roles: waves 0-3 keep four rows in flight in registers (a row of
+// MFMA work is far shorter than memory latency) and write row r+2 while waves 4-7
+// (2 along m x 2 along the columns, 32 x 144 each) work on row r out of three LDS
+// buffers; fragments of the next k-step - or of the next row, which is complete one
+// barrier earlier - are read into the registers just used.  One barrier per row.
+// Partial tiles go to the workspace and are added in a fixed order by
+// wgrad_reduce_kernel; the bias gradient is summed from the dy values as they pass
+// through the loader registers.
+#include <algorithm>
+
+#include "conv2d_mfma.h"
+
+namespace flhip {
+namespace {
+
+constexpr int BM = MFMA_BM;
+constexpr int CB = 32;           // input channels per workgroup
+constexpr int NCOL = CB * 9;     // columns of the tile
+constexpr int THREADS = 512;
+constexpr int NTW = 9;           // 16-column blocks per MFMA wave
+constexpr int NXI = 3;           // x units (one (c,kh) row piece of 8 columns) per loader thread and row
+constexpr int NDI = 2;           // dy units per loader thread and row
+constexpr int NSET = 4;          // rows in flight in loader registers
+constexpr int SPW = NCOL + 4;    // pitch of the parked result tile (words)
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+#if defined(__HIP_DEVICE_COMPILE__)
+typedef __attribute__((address_space(3))) const uint4* lds_cell;
+#else
+typedef const uint4* lds_cell;
+#endif
+
+struct W16Params {
+  int N, C, H, W, K, OH, OW;
+  int py, dly;
+  int groups, Cg, Kg;
+  int Q;               // 8-column groups per row
+  int RPW;             // rows per loader wave pass (64 / Q)
+  int nks;             // k-steps of 32 positions per row
+  int PB;              // LDS row pitch in bytes
+  int buf_cells;       // 16-byte cells per LDS buffer (xs then ds)
+  int nhalves, mtiles;
+  int nsplit, rps;     // K-splits, (image,row) pairs per split
+  int total_rows;
+  int E;               // K*Cg*9
+  int want_db;
+  unsigned x_bytes, dy_bytes;
+};
+
+__global__ void __launch_bounds__(THREADS, 2)
+wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy,
+               float* __restrict__ out, float* __restrict__ db_out) {
+  extern __shared__ uint4 lds16[];
+  float* lds = reinterpret_cast<float*>(lds16);
+  constexpr int OOB = (int)0x80000000;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int split = blockIdx.x;
+  const int half = __builtin_amdgcn_readfirstlane(blockIdx.y % p.nhalves);
+  const int mtile = __builtin_amdgcn_readfirstlane(blockIdx.y / p.nhalves);
+  const int grp = blockIdx.z;
+  const int m_lim = p.Kg - mtile * BM;
+  const int row_begin = split * p.rps, row_end = min(row_begin + p.rps, p.total_rows);
+  const int nrows = row_end - row_begin;
+  const int HW = p.H * p.W, OHW = p.OH * p.OW;
+  float* o = out + (p.nsplit > 1 ? (size_t)split * (p.E + p.K) : 0);
+  const int ncols = p.Cg * 9;
+  const int pcells = p.PB >> 4;             // row pitch in cells
+  const int ds_cell0 = NCOL * pcells;       // dy rows follow the 288 x rows of a buffer
+  float* stage = lds;                       // [BM][SPW] after the last row
+  float* dbpart = lds + BM * SPW;           // [BM][Q] bias partials
+
+  // Positions past OW and the columns outside the image are never written: zero all
+  // three buffers once.
+  for (int i = tid; i < 3 * p.buf_cells; i += THREADS) lds16[i] = make_uint4(0u, 0u, 0u, 0u);
+  __syncthreads();
+
+  auto store_tile = [&]() {
+    constexpr int QT = NCOL / 4;
+    for (int idx = tid; idx < BM * QT; idx += THREADS) {
+      const int m = idx / QT, q = idx - m * QT;
+      if (m < m_lim) {
+        const float4 v = *reinterpret_cast<const float4*>(stage + m * SPW + 4 * q);
+        *reinterpret_cast<float4*>(o + (size_t)(grp * p.Kg + mtile * BM + m) * ncols +
+                                   half * NCOL + 4 * q) = v;
+      }
+    }
+  };
+
+  if (wave < 4) {
+    // ============================== loader waves ================================
+    const __amdgpu_buffer_rsrc_t xrsrc = make_rsrc(x, p.x_bytes);
+    const __amdgpu_buffer_rsrc_t yrsrc = make_rsrc(dy, p.dy_bytes);
+    const bool do_db = p.want_db && half == 0;
+    // A wave pass covers RPW rows of Q units; lane = row_in_pass * Q + q, so the
+    // columns next to a unit's eight are in the adjacent lanes.
+    const int rl = lane / p.Q, q = lane - rl * p.Q;
+    const bool lane_ok = rl < p.RPW;
+    const bool first_q = q == 0, last_q = q == p.Q - 1;
+    // x rows: index xr = c*3 + kh (96 per tile); dy rows: m (64 per tile)
+    int xg[NXI], xl[NXI], xkh[NXI];
+#pragma unroll
+    for (int i = 0; i < NXI; ++i) {
+      const int xr = (i * 4 + wave) * p.RPW + rl;
+      xg[i] = OOB;
+      xl[i] = -1;
+      xkh[i] = 0;
+      if (lane_ok && xr < CB * 3) {
+        const int c = xr / 3, kh = xr - c * 3;
+        xkh[i] = kh;
+        xl[i] = xr * 3 * pcells + q;           // cell of the kw = 0 copy; kw copies are pcells apart
+        xg[i] = ((grp * p.Cg + half * CB + c) * HW + 8 * q) * 2;
+      }
+    }
+    int yg[NDI], yl[NDI];
+#pragma unroll
+    for (int i = 0; i < NDI; ++i) {
+      const int m = (i * 4 + wave) * p.RPW + rl;
+      yg[i] = OOB;
+      yl[i] = -1;
+      if (lane_ok && m < BM) {
+        yl[i] = ds_cell0 + m * pcells + q;
+        if (m < m_lim) yg[i] = ((grp * p.Kg + mtile * BM + m) * OHW + 8 * q) * 2;
+      }
+    }
+    float dbp[NDI];
+#pragma unroll
+    for (int i = 0; i < NDI; ++i) dbp[i] = 0.f;
+
+    struct RowRegs {
+      uintx4_t xv[NXI], yv[NDI];
+    };
+    auto load_row = [&](int row, RowRegs& r) {
+      const bool live = row < row_end;
+      const int img = row / p.OH, oh = row - img * p.OH;
+#pragma unroll
+      for (int i = 0; i < NXI; ++i) {
+        const int ih = oh - p.py + xkh[i] * p.dly;
+        const bool ok = live && (unsigned)ih < (unsigned)p.H;
+        r.xv[i] = __builtin_amdgcn_raw_buffer_load_b128(
+            xrsrc, ok ? xg[i] + (img * p.C * HW + ih * p.W) * 2 : OOB, 0, 0);
+      }
+      const int yb = (img * p.K * OHW + oh * p.OW) * 2;
+#pragma unroll
+      for (int i = 0; i < NDI; ++i)
+        r.yv[i] = __builtin_amdgcn_raw_buffer_load_b128(yrsrc, live ? yg[i] + yb : OOB, 0, 0);
+    };
+    auto store_row = [&](int buf, const RowRegs& r) {
+      uint4* b = lds16 + buf * p.buf_cells;
+#pragma unroll
+      for (int i = 0; i < NXI; ++i) {
+        const uintx4_t v = r.xv[i];
+        // element left of the eight (high half of the left lane's last dword) and
+        // right of them (low half of the right lane's first dword); zero at row ends
+        unsigned left = __shfl_up(v.w, 1, 64), right = __shfl_down(v.x, 1, 64);
+        left = first_q ? 0u : left;
+        right = last_q ? 0u : right;
+        const unsigned s1 = __builtin_amdgcn_alignbit(v.y, v.x, 16);
+        const unsigned s2 = __builtin_amdgcn_alignbit(v.z, v.y, 16);
+        const unsigned s3 = __builtin_amdgcn_alignbit(v.w, v.z, 16);
+        if (xl[i] >= 0) {
+          b[xl[i]] = make_uint4(__builtin_amdgcn_alignbit(v.x, left, 16), s1, s2, s3);   // x[p-1]
+          b[xl[i] + pcells] = make_uint4(v.x, v.y, v.z, v.w);                            // x[p]
+          b[xl[i] + 2 * pcells] =
+              make_uint4(s1, s2, s3, __builtin_amdgcn_alignbit(right, v.w, 16));         // x[p+1]
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < NDI; ++i) {
+        const uintx4_t v = r.yv[i];
+        if (yl[i] >= 0) b[yl[i]] = make_uint4(v.x, v.y, v.z, v.w);
+        float s = 0.f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const unsigned d = k == 0 ? v.x : k == 1 ? v.y : k == 2 ? v.z : v.w;
+          s += __uint_as_float(d << 16) + __uint_as_float(d & 0xffff0000u);
+        }
+        dbp[i] += s;
+      }
+    };
+
+    // rows r..r+1 in LDS before the first barrier, r+2..r+5 in registers
+    RowRegs set[NSET];
+#pragma unroll
+    for (int u = 0; u < NSET; ++u) load_row(row_begin + u, set[u]);
+    if (nrows > 0) store_row(0, set[0]);
+    load_row(row_begin + 4, set[0]);
+    if (nrows > 1) store_row(1, set[1]);
+    load_row(row_begin + 5, set[1]);
+    __syncthreads();
+    // iteration r: the MFMA waves work on row r; row r+2 (register set (r+2)%4) goes
+    // to buffer (r+2)%3 and the set is refilled with row r+6
+    for (int r4 = 0; r4 < nrows; r4 += NSET) {
+#pragma unroll
+      for (int u = 0; u < NSET; ++u) {
+        const int r = r4 + u;
+        if (r < nrows) {
+          if (r + 2 < nrows) store_row((r + 2) % 3, set[(u + 2) % NSET]);
+          load_row(row_begin + r + 6, set[(u + 2) % NSET]);
+          __syncthreads();
+        }
+      }
+    }
+    // bias: partials of a channel sit in Q consecutive slots behind the parked tile
+    if (do_db) {
+#pragma unroll
+      for (int i = 0; i < NDI; ++i) {
+        const int m = (i * 4 + wave) * p.RPW + rl;
+        if (lane_ok && m < BM) dbpart[m * p.Q + q] = dbp[i];
+      }
+    }
+    __syncthreads();                        // tile parked, partials written
+    if (do_db && tid < m_lim) {
+      float s = 0.f;
+      for (int k = 0; k < p.Q; ++k) s += dbpart[tid * p.Q + k];
+      const int ch = grp * p.Kg + mtile * BM + tid;
+      if (p.nsplit > 1)
+        o[p.E + ch] = s;
+      else
+        db_out[ch] = s;
+    }
+    store_tile();
+    return;
+  }
+
+  // ================================ MFMA waves ===================================
+  const int cw = wave - 4;
+  const int wm = cw & 1, wn = cw >> 1;
+  const int fr = lane & 15, fk = lane >> 4;
+  floatx4 acc[2][NTW];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < NTW; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  // cell addresses in buffer 0: a lane reads positions 8*fk .. 8*fk+7 of a k-step
+  lds_cell bp[NTW];
+#pragma unroll
+  for (int j = 0; j < NTW; ++j)
+    bp[j] = (lds_cell)lds16 + (((wn * NTW + j) * 16 + fr) * pcells + fk);
+  lds_cell ap0 = (lds_cell)lds16 + (ds_cell0 + (wm * 32 + fr) * pcells + fk);
+  lds_cell ap1 = ap0 + 16 * pcells;
+  auto advance = [&](int cells) {
+#pragma unroll
+    for (int j = 0; j < NTW; ++j) bp[j] += cells;
+    ap0 += cells;
+    ap1 += cells;
+  };
+  auto frag = [](uint4 v) { return __builtin_bit_cast(bf16x8, v); };
+
+  uint4 a0, a1, b[NTW];
+  // One k-step: MFMAs on the fragments in registers; behind each pair the fragment at
+  // cell offset OFF (next k-step of this row, or k-step 0 of the next row after the
+  // pointers moved) is read into the register just used.
+#define FLHIP_KSTEP(OFF)                                                 \
+  {                                                                      \
+    __builtin_amdgcn_sched_barrier(0);                                   \
+    const uint4 n0 = ap0[OFF], n1 = ap1[OFF];                            \
+    _Pragma("unroll") for (int j = 0; j < NTW; ++j) {                    \
+      acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(a0), frag(b[j]), acc[0][j], 0, 0, 0); \
+      acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(a1), frag(b[j]), acc[1][j], 0, 0, 0); \
+      b[j] = bp[j][OFF];                                                 \
+    }                                                                    \
+    a0 = n0;                                                             \
+    a1 = n1;                                                             \
+    _Pragma("unroll") for (int q = 0; q < NTW + 2; ++q) {                \
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                 \
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                 \
+    }                                                                    \
+    __builtin_amdgcn_sched_barrier(0);                                   \
+  }
+
+  __syncthreads();                          // rows 0 and 1 are in buffers 0 and 1
+  a0 = ap0[0];
+  a1 = ap1[0];
+#pragma unroll
+  for (int j = 0; j < NTW; ++j) b[j] = bp[j][0];
+  for (int r = 0; r < nrows; ++r) {
+    for (int ks = 0; ks + 1 < p.nks; ++ks) {
+      FLHIP_KSTEP(4)
+      advance(4);
+    }
+    // last k-step of the row: the next fragments are k-step 0 of row r+1, in the
+    // next buffer (written one barrier ago)
+    advance(((r % 3 == 2) ? -2 : 1) * p.buf_cells - 4 * (p.nks - 1));
+    FLHIP_KSTEP(0)
+    __syncthreads();
+  }
+#undef FLHIP_KSTEP
+
+#pragma unroll
+  for (int j = 0; j < NTW; ++j) {
+    const int col = (wn * NTW + j) * 16 + fr;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr)
+        stage[(wm * 32 + i * 16 + fk * 4 + rr) * SPW + col] = acc[i][j][rr];
+  }
+  __syncthreads();
+  store_tile();
+}
+
+bool plan(const ConvGeom& g, W16Params* p) {
+  if (g.KH != 3 || g.KW != 3 || g.sy != 1 || g.sx != 1 || g.px != 1 || g.dlx != 1) return false;
+  if (g.Cg % CB != 0 || g.OW % 8 != 0 || g.W != g.OW || g.OW > 64) return false;
+  p->N = g.N; p->C = g.C; p->H = g.H; p->W = g.W; p->K = g.K; p->OH = g.OH; p->OW = g.OW;
+  p->py = g.py; p->dly = g.dly;
+  p->groups = g.groups; p->Cg = g.Cg; p->Kg = g.Kg;
+  p->Q = g.OW / 8;
+  p->RPW = 64 / p->Q;
+  if (CB * 3 > NXI * 4 * p->RPW || BM > NDI * 4 * p->RPW) return false;
+  const int owp = (g.OW + 31) & ~31;
+  p->nks = owp / 32;
+  p->PB = owp * 2 + 16;
+  p->buf_cells = (NCOL + BM) * (p->PB / 16) + 1;   // + one cell: the read-ahead past the last row
+  if ((size_t)3 * p->buf_cells * 16 > 158 * 1024) return false;
+  if ((size_t)(BM * SPW + BM * p->Q) * sizeof(float) > (size_t)3 * p->buf_cells * 16) return false;
+  p->nhalves = g.Cg / CB;
+  p->mtiles = (g.Kg + BM - 1) / BM;
+  p->total_rows = g.N * g.OH;
+  p->E = g.K * g.Cg * 9;
+  const long long base_wgs = (long long)p->nhalves * p->mtiles * g.groups;
+  if (p->nhalves * p->mtiles > 65535 || g.groups > 65535) return false;
+  long long ns = mfma_num_cus() / base_wgs;
+  if (ns > p->total_rows) ns = p->total_rows;
+  if (ns < 1) ns = 1;
+  p->rps = (int)((p->total_rows + ns - 1) / ns);
+  p->nsplit = (p->total_rows + p->rps - 1) / p->rps;
+  return true;
+}
+
+}  // namespace
+
+// defined in conv2d_mfma_wgrad.hip
+void wgrad_reduce_launch(const float* part, int nsplit, int E, int K, int want_db, float* dw,
+                         float* db, hipStream_t s);
+
+size_t mfma_wgrad16_ws(const ConvGeom& g) {
+  W16Params p{};
+  if (!plan(g, &p)) return 0;
+  return p.nsplit > 1 ? (size_t)p.nsplit * (p.E + p.K) * sizeof(float) : 0;
+}
+
+int mfma_wgrad16(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
+                 size_t ws_bytes, hipStream_t s) {
+  if (!dw) return -1;
+  W16Params p{};
+  if (!plan(g, &p)) return -1;
+  if (reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(dy) % 16 != 0) return -1;
+  const long long xb = (long long)g.N * g.C * g.H * g.W * 2;
+  const long long yb = (long long)g.N * g.K * g.OH * g.OW * 2;
+  if (xb >= (1ll << 31) || yb >= (1ll << 31)) return -1;
+  p.x_bytes = (unsigned)xb;
+  p.dy_bytes = (unsigned)yb;
+  p.want_db = db != nullptr;
+  const size_t need = p.nsplit > 1 ? (size_t)p.nsplit * (p.E + p.K) * sizeof(float) : 0;
+  if (need && (!ws || ws_bytes < need))
+    return fail(FLHIP_INVALID_ARGUMENT, "conv2d_bwd_filter: workspace too small");
+  float* out = p.nsplit > 1 ? static_cast<float*>(ws) : dw;
+  if (reinterpret_cast<uintptr_t>(out) % 16 != 0) return -1;
+  const size_t shmem = (size_t)3 * p.buf_cells * 16;
+  auto kernel = wgrad16_kernel;
+  if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
+  const dim3 grid(p.nsplit, p.nhalves * p.mtiles, g.groups);
+  hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const bf16_t*>(x),
+                     static_cast<const bf16_t*>(dy), out, db);
+  if (p.nsplit > 1)
+    wgrad_reduce_launch(static_cast<const float*>(ws), p.nsplit, p.E, p.K, p.want_db, dw, db, s);
+  return check_launch("conv2d_bwd_filter (bf16 mfma)");
+}
+
+}  // namespace flhip
