@@ -32,8 +32,8 @@ MEASURED_TRAFFIC = {"conv2d_bwd_data_f32": 61.8e6}
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--dtype", choices=["f32", "bf16"], default="f32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--only", default="", help="comma list of ops to time (debugging/profiling)")
@@ -94,46 +94,56 @@ def main():
         return fn
 
     # ---- conv pair at cfg 2 --------------------------------------------------
-    tag = capi.F32 if a.dtype == "f32" else capi.BF16
-    x = randn(32, 64, 56, 56).to(tdt)
-    w = randn(64, 64, 3, 3, scale=1.0 / 24.0).to(tdt)          # Kaiming normal, fan-in 576
-    b = randn(64)
-    dy = randn(32, 64, 56, 56).to(tdt)
-    y, dx = torch.empty_like(x), torch.empty_like(x)
-    dw = torch.empty((64, 64, 3, 3), device=dev)
-    db = torch.empty(64, device=dev)
-    cd = capi.ConvDesc(32, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, tag)
-    nws = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_BWD_FILTER)
-    ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=dev)
-    nws_f = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_FWD)
-    nws_d = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_BWD_DATA)
-    ws_f = torch.empty(max(nws_f, 16), dtype=torch.uint8, device=dev)
-    ws_d = torch.empty(max(nws_d, 16), dtype=torch.uint8, device=dev)
-    peak_mfma = PEAK["f32_TFLOPs"] if a.dtype == "f32" else PEAK["bf16_TFLOPs"]
-    cdp, xp, wp, bp, dyp, yp, dxp, dwp, dbp, wsp = (C.byref(cd), P(x), P(w), P(b), P(dy), P(y),
-                                                     P(dx), P(dw), P(db), P(ws))
-    wsfp, wsdp = P(ws_f), P(ws_d)
-    f_fwd = checked(lambda _: L.flhip_conv2d_fwd(cdp, xp, wp, bp, yp, wsfp, nws_f, S))
-    f_bwd_data = checked(lambda _: L.flhip_conv2d_bwd_data(cdp, dyp, wp, dxp, wsdp, nws_d, S))
-    f_bwd_filter = checked(lambda _: L.flhip_conv2d_bwd_filter(cdp, xp, dyp, dwp, dbp, wsp, nws, S))
+    def conv_block(dname, with_pair):
+        """Times the conv ops of cfg 2 in storage type `dname`; returns the pair timing."""
+        tag = capi.F32 if dname == "f32" else capi.BF16
+        ttype = torch.float32 if dname == "f32" else torch.bfloat16
+        x = randn(32, 64, 56, 56).to(ttype)
+        w = randn(64, 64, 3, 3, scale=1.0 / 24.0).to(ttype)          # Kaiming normal, fan-in 576
+        b = randn(64)
+        dy = randn(32, 64, 56, 56).to(ttype)
+        y, dx = torch.empty_like(x), torch.empty_like(x)
+        dw = torch.empty((64, 64, 3, 3), device=dev)
+        db = torch.empty(64, device=dev)
+        cd = capi.ConvDesc(32, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, tag)
+        nws = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_BWD_FILTER)
+        nws_f = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_FWD)
+        nws_d = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_BWD_DATA)
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device=dev)
+        ws_f = torch.empty(max(nws_f, 16), dtype=torch.uint8, device=dev)
+        ws_d = torch.empty(max(nws_d, 16), dtype=torch.uint8, device=dev)
+        peak_mfma = PEAK["f32_TFLOPs"] if dname == "f32" else PEAK["bf16_TFLOPs"]
+        cdp, xp, wp, bp, dyp, yp, dxp, dwp, dbp, wsp = (C.byref(cd), P(x), P(w), P(b), P(dy), P(y),
+                                                         P(dx), P(dw), P(db), P(ws))
+        wsfp, wsdp = P(ws_f), P(ws_d)
+        f_fwd = checked(lambda _: L.flhip_conv2d_fwd(cdp, xp, wp, bp, yp, wsfp, nws_f, S))
+        f_bwd_data = checked(lambda _: L.flhip_conv2d_bwd_data(cdp, dyp, wp, dxp, wsdp, nws_d, S))
+        f_bwd_filter = checked(lambda _: L.flhip_conv2d_bwd_filter(cdp, xp, dyp, dwp, dbp, wsp, nws, S))
 
-    def conv_pair(i):
-        f_bwd_data(i)
-        f_bwd_filter(i)
+        def conv_pair(i):
+            f_bwd_data(i)
+            f_bwd_filter(i)
 
-    pair_s = pair_wall = None
-    if want("conv_pair"):
-        pair_s, pair_wall = timed(conv_pair, a.steps, a.warmup)
-    for name, fn in (("conv2d_fwd", f_fwd), ("conv2d_bwd_data", f_bwd_data),
-                     ("conv2d_bwd_filter_bias", f_bwd_filter)):
-        if not want(name):
-            continue
-        s, _ = timed(fn, a.steps, a.warmup)
-        ach = CONV_FLOP / s / 1e12
-        ops.append({"op": name, "workload": "32x64x56x56, 64 filters 3x3 s1 p1", "dtype": a.dtype,
-                    "us": s * 1e6, "bound": "mfma", "achieved": ach, "peak": peak_mfma,
-                    "unit": "TFLOP/s", "frac": ach / peak_mfma})
-    del x, w, dy, y, dx, ws, ws_f, ws_d
+        res = (None, None)
+        if with_pair and want("conv_pair"):
+            res = timed(conv_pair, a.steps, a.warmup)
+        for name, fn in (("conv2d_fwd", f_fwd), ("conv2d_bwd_data", f_bwd_data),
+                         ("conv2d_bwd_filter_bias", f_bwd_filter)):
+            if not want(name):
+                continue
+            s, _ = timed(fn, a.steps, a.warmup)
+            ach = CONV_FLOP / s / 1e12
+            ops.append({"op": name, "workload": "32x64x56x56, 64 filters 3x3 s1 p1", "dtype": dname,
+                        "us": s * 1e6, "bound": "mfma", "achieved": ach, "peak": peak_mfma,
+                        "unit": "TFLOP/s", "frac": ach / peak_mfma})
+        return res
+
+    pair_s, pair_wall = conv_block(a.dtype, True)
+    # the same ops in the other storage type (bf16 storage, fp32 accumulate, when the
+    # headline runs in fp32): listed under "ops", not part of `value`
+    other = "bf16" if a.dtype == "f32" else "f32"
+    if not only or "other_dtype" in only:
+        conv_block(other, False)
 
     # ---- bandwidth ops at cfg 3 (fp32) ----------------------------------------
     def bw_op(name, workload, nbytes, fn, nsets):
@@ -142,10 +152,14 @@ def main():
         checked(fn)
         s, _ = timed(fn, a.steps, a.warmup)
         ach = nbytes / s / 1e9
+        # the same call on one buffer set every time: operands may sit in the 256 MB
+        # memory-side cache (reported beside the cold figure, never as `achieved`)
+        warm, _ = timed(lambda i: fn(0), a.steps, a.warmup)
         ops.append({"op": name, "workload": workload, "dtype": "f32", "us": s * 1e6,
                     "bound": "hbm", "achieved": ach, "peak": PEAK["hbm_GBps"], "unit": "GB/s",
                     "frac": ach / PEAK["hbm_GBps"], "algorithmic_bytes": nbytes,
-                    "buffer_sets_rotated": nsets})
+                    "buffer_sets_rotated": nsets, "us_cache_warm": warm * 1e6,
+                    "GBps_cache_warm": nbytes / warm / 1e9})
 
     if want("batchnorm_bwd") or want("batchnorm_fwd_train"):
         nsets = 2
@@ -211,7 +225,10 @@ def main():
               lambda i: L.flhip_copy_bytes(cap, cbp, 256 << 20, S), 1)
 
     torch.cuda.synchronize()
-    by = {o["op"]: o for o in ops}
+    by = {}
+    for o in ops:
+        other_conv = o["op"].startswith("conv2d") and o["dtype"] != a.dtype
+        by.setdefault(o["op"] + "_" + o["dtype"] if other_conv else o["op"], o)
 
     # ---- CPU baselines (rank 0, bounded sample) --------------------------------
     cpu_baseline = cpu_onednn = None
