@@ -247,10 +247,60 @@ wgrad_kernel(WgradParams p, const T* __restrict__ x, const T* __restrict__ dy,
   }
 }
 
-// out[e] = sum over s of part[s][e]; elements past E go to db.
-__global__ void __launch_bounds__(256)
+// out[e] = sum over s of part[s][e]; elements past E go to db.  A block covers 64
+// groups of four consecutive elements with 16 threads each; a thread adds every 16th
+// partial, all of its 16-byte loads in flight together, and the 16 sums of a group
+// are added in a fixed order (deterministic).  (E + K) % 4 == 0 is required.
+constexpr int RED_TY = 16;
+__global__ void __launch_bounds__(64 * RED_TY)
 wgrad_reduce_kernel(const float* __restrict__ part, int nsplit, int E, int K, int want_db,
                     float* __restrict__ dw, float* __restrict__ db) {
+  __shared__ float4 red[RED_TY][64];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int e = (blockIdx.x * 64 + tx) * 4;
+  const int total = E + (want_db ? K : 0);
+  const size_t stride = (size_t)E + K;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (e < total) {
+    for (int s0 = ty; s0 < nsplit; s0 += 8 * RED_TY) {
+      float4 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int s = s0 + u * RED_TY;
+        v[u] = s < nsplit ? *reinterpret_cast<const float4*>(part + (size_t)s * stride + e)
+                          : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        acc.x += v[u].x; acc.y += v[u].y; acc.z += v[u].z; acc.w += v[u].w;
+      }
+    }
+  }
+  red[ty][tx] = acc;
+  __syncthreads();
+  if (ty == 0 && e < total) {
+    float4 r = red[0][tx];
+#pragma unroll
+    for (int k = 1; k < RED_TY; ++k) {
+      const float4 t = red[k][tx];
+      r.x += t.x; r.y += t.y; r.z += t.z; r.w += t.w;
+    }
+    const float rv[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int ek = e + k;
+      if (ek < E)
+        dw[ek] = rv[k];
+      else if (ek < total)
+        db[ek - E] = rv[k];
+    }
+  }
+}
+
+// element-wise variant for sizes that are not multiples of four
+__global__ void __launch_bounds__(256)
+wgrad_reduce_kernel1(const float* __restrict__ part, int nsplit, int E, int K, int want_db,
+                     float* __restrict__ dw, float* __restrict__ db) {
   __shared__ float red[4][64];
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   const int e = blockIdx.x * 64 + tx;
@@ -326,8 +376,12 @@ bool wgrad_split(WgradParams* p, const ConvGeom& g) {
 void wgrad_reduce_launch(const float* part, int nsplit, int E, int K, int want_db, float* dw,
                          float* db, hipStream_t s) {
   const int total = E + (want_db ? K : 0);
-  hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((total + 63) / 64), dim3(256), 0, s, part, nsplit, E,
-                     K, want_db, dw, db);
+  if ((E + K) % 4 == 0 && reinterpret_cast<uintptr_t>(part) % 16 == 0)
+    hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((total + 255) / 256), dim3(64 * RED_TY), 0, s, part,
+                       nsplit, E, K, want_db, dw, db);
+  else
+    hipLaunchKernelGGL(wgrad_reduce_kernel1, dim3((total + 63) / 64), dim3(256), 0, s, part, nsplit,
+                       E, K, want_db, dw, db);
 }
 
 size_t mfma_conv_bwd_filter_ws(const ConvGeom& g, int) {
@@ -360,11 +414,8 @@ int mfma_conv_bwd_filter(const ConvGeom& g, int dtype, const void* x, const void
     hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const bf16_t*>(x),
                        static_cast<const bf16_t*>(dy), out, db);
   }
-  if (p.nsplit > 1) {
-    const int total = p.E + (p.want_db ? p.K : 0);
-    hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((total + 63) / 64), dim3(256), 0, s,
-                       static_cast<const float*>(ws), p.nsplit, p.E, p.K, p.want_db, dw, db);
-  }
+  if (p.nsplit > 1)
+    wgrad_reduce_launch(static_cast<const float*>(ws), p.nsplit, p.E, p.K, p.want_db, dw, db, s);
   return check_launch("conv2d_bwd_filter (mfma)");
 }
 
