@@ -32,16 +32,14 @@ bool mfma_slab_wgrad_applies(const ConvGeom& g);
 int mfma_slab_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
                             hipStream_t s);
 
-// bf16-storage variants on the bf16 matrix cores (conv2d_mfma_slab_bf16.hip).  They
-// need a workspace of mfma_slab16_ws() bytes for the rearranged weights and
-// return -1 without one.
-size_t mfma_slab16_ws(const ConvGeom& g, bool bwd);
+// bf16-storage variants on the bf16 matrix cores (conv2d_mfma_slab_bf16.hip,
+// conv2d_mfma_wgrad_slab_bf16.hip); same return convention.
 int mfma_slab16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
-                         void* ws, size_t ws_bytes, hipStream_t s);
+                         hipStream_t s);
+int mfma_slab16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx,
+                              hipStream_t s);
 size_t mfma_wgrad16_ws(const ConvGeom& g);
 int mfma_wgrad16(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
                  size_t ws_bytes, hipStream_t s);
-int mfma_slab16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, void* ws,
-                              size_t ws_bytes, hipStream_t s);
 
 }  // namespace flhip

@@ -157,16 +157,14 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
     if (b > a) a = b;
     return c > a ? c : a;
   }
-  // bf16 forward / backward-data: room for the weights in matrix-core order (the
-  // passes run without it, on the slower converting kernels)
-  if (d->dtype == FLHIP_BF16 && (pass == FLHIP_CONV_FWD || pass == FLHIP_CONV_BWD_DATA))
-    return mfma_slab16_ws(g, pass == FLHIP_CONV_BWD_DATA);
   return 0;
 }
 
 extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const void* w,
                                 const float* bias, void* y, void* ws, size_t ws_bytes,
                                 void* stream) {
+  (void)ws;
+  (void)ws_bytes;
   FLHIP_REQUIRE(d && x && w && y, "conv2d_fwd: null argument");
   ConvGeom g;
   const int rc = make_geom(d, &g);
@@ -175,7 +173,7 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
   if (!force_direct()) {
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !algo_is("gather") && !algo_is("convert"))
-      r = mfma_slab16_conv_fwd(g, x, w, bias, y, ws, ws_bytes, s);
+      r = mfma_slab16_conv_fwd(g, x, w, bias, y, s);
     if (r < 0 && !algo_is("gather")) r = mfma_slab_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r < 0) r = mfma_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r >= 0) return r;
@@ -195,6 +193,8 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
 
 extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, const void* w,
                                      void* dx, void* ws, size_t ws_bytes, void* stream) {
+  (void)ws;
+  (void)ws_bytes;
   FLHIP_REQUIRE(d && dy && w && dx, "conv2d_bwd_data: null argument");
   ConvGeom g;
   const int rc = make_geom(d, &g);
@@ -203,7 +203,7 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
   if (!force_direct()) {
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !algo_is("gather") && !algo_is("convert"))
-      r = mfma_slab16_conv_bwd_data(g, dy, w, dx, ws, ws_bytes, s);
+      r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s);
     if (r < 0 && !algo_is("gather")) r = mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0) r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r >= 0) return r;

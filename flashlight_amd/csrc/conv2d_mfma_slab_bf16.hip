@@ -14,9 +14,13 @@
 //            pitch = 1 (mod 16) put the 16 stores of a quarter wave in 16 distinct
 //            bank groups; the 16 positions of a fragment read are contiguous.
 //   weights  as[4 channel groups][64 result channels x taps] cells.  Memory order is
-//            (channel, tap) or (channel, result channel, tap), so a small kernel
-//            rewrites the weights once per call into that cell order (workspace)
-//            and the main kernel copies cells.
+//            (channel, tap) per result channel (forward) or (result channel, tap)
+//            per channel (backward-data).  Forward: a thread reads the 72
+//            contiguous values of (result channel, 8 channels) with 16-byte loads
+//            and regroups them with v_perm_b32 (3x3 windows).  Backward-data: the
+//            weights look like the slab - channel-major with (result channel, tap)
+//            contiguous - and go through the same 8x8 transpose.  Other shapes
+//            gather a cell with eight 2-byte loads.
 // 8 waves, two roles as in the fp32 kernel.  The B fragments of tap t+1 are read
 // into the registers tap t has just finished with (one read behind each pair of
 // MFMAs), so one set of fragment registers is enough.
@@ -46,6 +50,7 @@ typedef const uint4* lds_cell;
 
 struct Slab16Params {
   int stage_ok;          // result rows are 16-byte aligned and a half tile fits in LDS
+  int wvec;              // weights are read 16 bytes at a time
   int N, SC, SH, SW, DC, DH, DW;
   int KH, KW, KHW, dly, dlx;
   int sh0, sw0;          // window shift of tap (0,0): fwd -py,-px ; bwd +py,+px
@@ -63,35 +68,9 @@ struct Slab16Params {
   unsigned src_bytes, wt_bytes;
 };
 
-// Weights in cell order: cell (grp, mtile, chunk, channel group, m, tap) holds the 8
-// source channels chunk*32 + cg*8 .. +7 of result channel mtile*64 + m; channels or
-// result channels past the end are zero.
-__global__ void __launch_bounds__(256)
-slab16_weight_cells(Slab16Params p, const bf16_t* __restrict__ w, uint4* __restrict__ out,
-                    int ncells) {
-  const int cell = blockIdx.x * 256 + threadIdx.x;
-  if (cell >= ncells) return;
-  int t = cell;
-  const int tap = t % p.KHW; t /= p.KHW;
-  const int m = t % BM; t /= BM;
-  const int cg = t % CG; t /= CG;
-  const int chunk = t % p.nchunks; t /= p.nchunks;
-  const int mtile = t % p.mtiles;
-  const int grp = t / p.mtiles;
-  const int c0 = chunk * CKB + cg * 8;
-  const bool m_ok = mtile * BM + m < p.DCg;
-  const int base = grp * p.w_group_stride + (mtile * BM + m) * p.a_mstride + tap;
-  unsigned h[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i)
-    h[i] = (m_ok && c0 + i < p.SCg) ? (unsigned)w[base + (c0 + i) * p.a_cstride] : 0u;
-  out[cell] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16),
-                         h[6] | (h[7] << 16));
-}
-
 template <bool BWD>
 __global__ void __launch_bounds__(THREADS, 2)
-slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const uint4* __restrict__ wcells,
+slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t* __restrict__ wgt,
                    const float* __restrict__ bias, bf16_t* __restrict__ dst) {
   extern __shared__ uint4 lds16[];
   uint4* Xs = lds16;                            // [2][x_cells]
@@ -142,7 +121,7 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const uint4* 
   if (wave < 4) {
     // ============================ loader waves ===================================
     const __amdgpu_buffer_rsrc_t srsrc = make_rsrc(src, p.src_bytes);
-    const __amdgpu_buffer_rsrc_t wrsrc = make_rsrc(wcells, p.wt_bytes);
+    const __amdgpu_buffer_rsrc_t wrsrc = make_rsrc(wgt, p.wt_bytes);
     constexpr int OOB = (int)0x80000000;
     const int chan_bytes = p.SH * p.SW * 2;
     const int img_base = (img * p.SC + grp * p.SCg) * p.SH * p.SW;
@@ -171,68 +150,168 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const uint4* 
         }
       }
     }
-    // weight cells of this tile and chunk are contiguous in the workspace
-    const int chunk_cells = CG * p.APL;
-    const int wt_base = ((grp * p.mtiles + mtile) * n) * chunk_cells;
-    const int nau = (chunk_cells + GTHREADS - 1) / GTHREADS;
+    const int APD = BM * p.KHW;                  // cells of a channel group (plane pitch is APL)
+    const int w_base = grp * p.w_group_stride + mtile * BM * p.a_mstride;
+    const int cstride_bytes = p.a_cstride * 2;
 
-    uint4 xv[NXU_MAX][8], av[NAU_MAX];
-    auto load_chunk = [&](int chunk) {
+    // 8x8 transpose of 16-bit values: in[k] = 8 consecutive positions of channel k;
+    // cell t = the 8 channels of position t.  Column 2t+s of channels 2k, 2k+1 is the
+    // low (s = 0) or high (s = 1) half of dword t of the two rows.
+    auto transpose_store = [&](const uint4 (&in)[8], uint4* dst) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        unsigned lo[4], hi[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const unsigned e = t == 0 ? in[2 * k].x : t == 1 ? in[2 * k].y : t == 2 ? in[2 * k].z : in[2 * k].w;
+          const unsigned o = t == 0 ? in[2 * k + 1].x : t == 1 ? in[2 * k + 1].y : t == 2 ? in[2 * k + 1].z : in[2 * k + 1].w;
+          lo[k] = __builtin_amdgcn_perm(o, e, 0x05040100u);
+          hi[k] = __builtin_amdgcn_perm(o, e, 0x07060302u);
+        }
+        dst[2 * t] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        dst[2 * t + 1] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+      }
+    };
+    auto ld16 = [&](__amdgpu_buffer_rsrc_t r, int off) {
+      const uintx4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+      return make_uint4(v.x, v.y, v.z, v.w);
+    };
+
+    uint4 xv[NXU_MAX][8];
+    auto load_x = [&](int chunk) {
       const int c0 = chunk * CKB;
       const int xbase = c0 * chan_bytes;
 #pragma unroll
       for (int i = 0; i < NXU_MAX; ++i)
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
-          // channels past the end of the group read zero
-          const int off = (c0 + xc[i] + k < p.SCg) ? xg[i] + xbase + k * chan_bytes : OOB;
-          const uintx4_t v = __builtin_amdgcn_raw_buffer_load_b128(srsrc, off, 0, 0);
-          xv[i][k] = make_uint4(v.x, v.y, v.z, v.w);
-        }
-#pragma unroll
-      for (int i = 0; i < NAU_MAX; ++i) {
-        const int cell = tid + GTHREADS * i;
-        const int off = (i < nau && cell < chunk_cells) ? (wt_base + chunk * chunk_cells + cell) * 16 : OOB;
-        const uintx4_t v = __builtin_amdgcn_raw_buffer_load_b128(wrsrc, off, 0, 0);
-        av[i] = make_uint4(v.x, v.y, v.z, v.w);
-      }
+        for (int k = 0; k < 8; ++k)   // channels past the end of the group read zero
+          xv[i][k] = ld16(srsrc, (c0 + xc[i] + k < p.SCg) ? xg[i] + xbase + k * chan_bytes : OOB);
     };
-    auto store_chunk = [&](int buf) {
+    auto store_x = [&](int buf) {
       uint4* xs = Xs + buf * p.x_cells;
-      uint4* as = As + buf * p.a_cells;
 #pragma unroll
-      for (int i = 0; i < NXU_MAX; ++i) {
-        // 8x8 transpose of 16-bit values: column 2t+s of channels 2k, 2k+1 is the low
-        // (s = 0) or high (s = 1) half of dword t of the two rows
+      for (int i = 0; i < NXU_MAX; ++i) transpose_store(xv[i], xs + xl[i]);
+    };
+    // runs the chunk pipeline with the given weight loader / storer
+    auto pipeline = [&](auto&& load_w, auto&& store_w) {
+      load_x(0);
+      load_w(0);
+      store_x(0);
+      store_w(0);
+      __syncthreads();
+      for (int c = 0; c < n; ++c) {
+        if (c + 1 < n) {
+          load_x(c + 1);
+          load_w(c + 1);
+          store_x((c + 1) & 1);
+          store_w((c + 1) & 1);
+        }
+        __syncthreads();
+      }
+    };
+
+    if (p.wvec && !BWD) {
+      // forward, 3x3: thread = (result channel m = lane, channel group = wave); the 72
+      // values (8 channels x 9 taps) are contiguous; cell `tap` takes value k*9 + tap
+      // of each channel k
+      const int m = lane, cg = wave;
+      const int wg = m < m_lim ? (w_base + m * p.a_mstride + cg * 8 * 9) * 2 : OOB;
+      const int wl = cg * p.APL + m * 9;
+      uint4 wv[9];
+      pipeline(
+          [&](int chunk) {
+            const int c0 = chunk * CKB;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          unsigned lo[4], hi[4];
+            for (int k = 0; k < 9; ++k)
+              wv[k] = ld16(wrsrc, (c0 + cg * 8 < p.SCg) ? wg + c0 * 18 + k * 16 : OOB);
+          },
+          [&](int buf) {
+            uint4* as = As + buf * p.a_cells + wl;
+            unsigned d[36];
 #pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            const unsigned e = t == 0 ? xv[i][2 * k].x : t == 1 ? xv[i][2 * k].y : t == 2 ? xv[i][2 * k].z : xv[i][2 * k].w;
-            const unsigned o = t == 0 ? xv[i][2 * k + 1].x : t == 1 ? xv[i][2 * k + 1].y : t == 2 ? xv[i][2 * k + 1].z : xv[i][2 * k + 1].w;
-            lo[k] = __builtin_amdgcn_perm(o, e, 0x05040100u);
-            hi[k] = __builtin_amdgcn_perm(o, e, 0x07060302u);
-          }
-          xs[xl[i] + 2 * t] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-          xs[xl[i] + 2 * t + 1] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+            for (int k = 0; k < 9; ++k) {
+              d[4 * k] = wv[k].x; d[4 * k + 1] = wv[k].y; d[4 * k + 2] = wv[k].z; d[4 * k + 3] = wv[k].w;
+            }
+#pragma unroll
+            for (int tap = 0; tap < 9; ++tap) {
+              unsigned o[4];
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                const int e0 = 2 * j * 9 + tap, e1 = (2 * j + 1) * 9 + tap;   // values of channels 2j, 2j+1
+                const unsigned sel = ((e0 & 1) ? 0x0302u : 0x0100u) | ((e1 & 1) ? 0x07060000u : 0x05040000u);
+                o[j] = __builtin_amdgcn_perm(d[e1 >> 1], d[e0 >> 1], sel);
+              }
+              as[tap] = make_uint4(o[0], o[1], o[2], o[3]);
+            }
+          });
+    } else if (p.wvec) {
+      // backward-data: unit = (channel group, 8 consecutive (result channel, tap) values)
+      constexpr int NWU = 2;
+      const int egroups = APD >> 3;
+      int wg[NWU], wl[NWU], wc[NWU];
+#pragma unroll
+      for (int i = 0; i < NWU; ++i) {
+        const int u = tid + GTHREADS * i;
+        const int cg = u & 3, eg = u >> 2;
+        wg[i] = OOB;
+        wl[i] = p.a_cells - 8;
+        wc[i] = cg * 8;
+        if (eg < egroups) {
+          wl[i] = cg * p.APL + 8 * eg;
+          wg[i] = (w_base + 8 * eg) * 2 + cg * 8 * cstride_bytes;
         }
       }
+      uint4 wv[NWU][8];
+      pipeline(
+          [&](int chunk) {
+            const int c0 = chunk * CKB;
+#pragma unroll
+            for (int i = 0; i < NWU; ++i)
+#pragma unroll
+              for (int k = 0; k < 8; ++k)
+                wv[i][k] = ld16(wrsrc, (c0 + wc[i] + k < p.SCg) ? wg[i] + (c0 + k) * cstride_bytes : OOB);
+          },
+          [&](int buf) {
+            uint4* as = As + buf * p.a_cells;
+#pragma unroll
+            for (int i = 0; i < NWU; ++i) transpose_store(wv[i], as + wl[i]);
+          });
+    } else {
+      // any layout: cell = (channel group, result channel m, tap), eight 2-byte loads
+      int wg[NAU_MAX], wc[NAU_MAX], wl[NAU_MAX];
 #pragma unroll
       for (int i = 0; i < NAU_MAX; ++i) {
         const int cell = tid + GTHREADS * i;
-        as[(i < nau && cell < chunk_cells) ? cell : p.a_cells - 1] = av[i];
+        wg[i] = OOB;
+        wc[i] = 0;
+        wl[i] = p.a_cells - 1;
+        if (cell < CG * APD) {
+          const int cg = cell / APD, rem = cell - cg * APD;
+          const int m = rem / p.KHW, tap = rem - m * p.KHW;
+          wl[i] = cg * p.APL + rem;
+          wc[i] = cg * 8;
+          if (m < m_lim) wg[i] = (w_base + m * p.a_mstride + tap) * 2 + cg * 8 * cstride_bytes;
+        }
       }
-    };
-    load_chunk(0);
-    store_chunk(0);
-    __syncthreads();
-    for (int c = 0; c < n; ++c) {
-      if (c + 1 < n) {
-        load_chunk(c + 1);
-        store_chunk((c + 1) & 1);
-      }
-      __syncthreads();
+      unsigned av[NAU_MAX][8];
+      pipeline(
+          [&](int chunk) {
+            const int c0 = chunk * CKB;
+#pragma unroll
+            for (int i = 0; i < NAU_MAX; ++i)
+#pragma unroll
+              for (int k = 0; k < 8; ++k) {
+                const int off = (c0 + wc[i] + k < p.SCg) ? wg[i] + (c0 + k) * cstride_bytes : OOB;
+                av[i][k] = (unsigned short)__builtin_amdgcn_raw_buffer_load_b16(wrsrc, off, 0, 0);
+              }
+          },
+          [&](int buf) {
+            uint4* as = As + buf * p.a_cells;
+#pragma unroll
+            for (int i = 0; i < NAU_MAX; ++i)
+              as[wl[i]] = make_uint4(av[i][0] | (av[i][1] << 16), av[i][2] | (av[i][3] << 16),
+                                     av[i][4] | (av[i][5] << 16), av[i][6] | (av[i][7] << 16));
+          });
     }
     if (staged) {
       for (int h = 0; h < 2; ++h) {
@@ -423,8 +502,10 @@ void layout(Slab16Params* p, int R) {
   p->WSP = round_to_residue(p->XOFF + std::max(max_sc + 1, p->SW), 4, 16);
   p->XPL = round_to_residue(p->RS * p->WSP, 1, 16);
   p->x_cells = CG * p->XPL + 8;
-  p->APL = BM * p->KHW;
-  p->a_cells = CG * p->APL + 1;
+  // plane pitch = 2 (mod 16): the cell stores of the backward-data transpose spread
+  // over the bank groups
+  p->APL = round_to_residue(BM * p->KHW, 2, 16);
+  p->a_cells = CG * p->APL + 8;
 }
 
 bool plan(Slab16Params* p, size_t* shmem) {
@@ -451,7 +532,7 @@ bool plan(Slab16Params* p, size_t* shmem) {
   }
   if (best_r == 0) return false;
   layout(p, best_r);
-  if ((CG * p->APL + GTHREADS - 1) / GTHREADS > NAU_MAX) return false;
+  if ((CG * BM * p->KHW + GTHREADS - 1) / GTHREADS > NAU_MAX) return false;
   p->tiles_per_image = (p->DH + best_r - 1) / best_r;
   p->NB = (best_r * p->DW + 15) / 16;
   p->nchunks = (p->SCg + CKB - 1) / CKB;
@@ -463,30 +544,29 @@ bool plan(Slab16Params* p, size_t* shmem) {
   return best_r * p->DW >= 64;
 }
 
-size_t cells_of(const Slab16Params& p) {
-  return (size_t)p.groups * p.mtiles * p.nchunks * CG * p.APL;
-}
-
 template <bool BWD>
 int launch(Slab16Params& p, const void* src, const void* wgt, const float* bias, void* dst,
-           void* ws, size_t ws_bytes, hipStream_t s) {
+           hipStream_t s) {
   const long long sbytes = (long long)p.N * p.SC * p.SH * p.SW * 2;
-  if (sbytes >= (1ll << 31)) return -1;
-  if (reinterpret_cast<uintptr_t>(src) % 16 != 0 || reinterpret_cast<uintptr_t>(ws) % 16 != 0) return -1;
+  const long long wbytes = (long long)p.groups * p.w_group_stride * 2;
+  if (sbytes >= (1ll << 31) || wbytes >= (1ll << 31)) return -1;
+  if (reinterpret_cast<uintptr_t>(src) % 16 != 0) return -1;
   p.src_bytes = (unsigned)sbytes;
+  p.wt_bytes = (unsigned)wbytes;
   size_t shmem = 0;
   if (!plan(&p, &shmem)) return -1;
-  const size_t ncells = cells_of(p);
-  if (!ws || ws_bytes < ncells * 16 || ncells * 16 >= (1ull << 31)) return -1;
-  p.wt_bytes = (unsigned)(ncells * 16);
   if (reinterpret_cast<uintptr_t>(dst) % 8 != 0) p.stage_ok = 0;
+  // 16-byte weight loads: rows of the weight tensor start on 16-byte boundaries
+  {
+    const bool al = reinterpret_cast<uintptr_t>(wgt) % 16 == 0 && p.w_group_stride % 8 == 0;
+    p.wvec = BWD ? (al && p.a_cstride % 8 == 0 && (BM * p.KHW) % 8 == 0 && (BM * p.a_mstride) % 8 == 0)
+                 : (al && p.KHW == 9 && p.a_mstride % 8 == 0 && p.SCg % 8 == 0);
+  }
   auto kernel = slab16_conv_kernel<BWD>;
   if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
-  hipLaunchKernelGGL(slab16_weight_cells, dim3((unsigned)((ncells + 255) / 256)), dim3(256), 0, s, p,
-                     static_cast<const bf16_t*>(wgt), static_cast<uint4*>(ws), (int)ncells);
   const dim3 grid((unsigned)(p.N * p.tiles_per_image), (unsigned)(p.mtiles * p.groups));
   hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const bf16_t*>(src),
-                     static_cast<const uint4*>(ws), bias, static_cast<bf16_t*>(dst));
+                     static_cast<const bf16_t*>(wgt), bias, static_cast<bf16_t*>(dst));
   return check_launch("conv2d (bf16 mfma slab)");
 }
 
@@ -512,29 +592,20 @@ void fill_bwd(const ConvGeom& g, Slab16Params* p) {
 
 }  // namespace
 
-size_t mfma_slab16_ws(const ConvGeom& g, bool bwd) {
-  if (g.sy != 1 || g.sx != 1) return 0;
-  Slab16Params p{};
-  if (bwd) fill_bwd(g, &p); else fill_fwd(g, &p);
-  size_t shmem = 0;
-  if (!plan(&p, &shmem)) return 0;
-  return cells_of(p) * 16;
-}
-
 int mfma_slab16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
-                         void* ws, size_t ws_bytes, hipStream_t s) {
+                         hipStream_t s) {
   if (g.sy != 1 || g.sx != 1) return -1;
   Slab16Params p{};
   fill_fwd(g, &p);
-  return launch<false>(p, x, w, bias, y, ws, ws_bytes, s);
+  return launch<false>(p, x, w, bias, y, s);
 }
 
-int mfma_slab16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, void* ws,
-                              size_t ws_bytes, hipStream_t s) {
+int mfma_slab16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx,
+                              hipStream_t s) {
   if (g.sy != 1 || g.sx != 1) return -1;
   Slab16Params p{};
   fill_bwd(g, &p);
-  return launch<true>(p, dy, w, nullptr, dx, ws, ws_bytes, s);
+  return launch<true>(p, dy, w, nullptr, dx, s);
 }
 
 }  // namespace flhip

@@ -39,6 +39,7 @@ MORE = [
     ((1, 64, 20, 56), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),       # ResNet row length, two 32-channel chunks
     ((2, 40, 6, 16), (72, 40, 3, 3), (1, 1), (1, 1), (1, 1), 1),        # channel tails on both sides (bf16 matrix-core path)
     ((1, 96, 5, 8), (32, 48, 2, 3), (1, 1), (1, 1), (1, 1), 2),         # groups, 2x3 window (bf16 generic tap loop)
+    ((1, 20, 6, 16), (24, 20, 3, 3), (1, 1), (1, 1), (1, 1), 1),        # bf16 matrix-core path, weights not 16-byte friendly
 ]
 ALL = LIB_CASES + MORE
 
