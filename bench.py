@@ -231,9 +231,10 @@ def main():
         by.setdefault(o["op"] + "_" + o["dtype"] if other_conv else o["op"], o)
 
     # ---- CPU baselines (rank 0, bounded sample) --------------------------------
-    cpu_baseline = cpu_onednn = None
+    cpu_baseline = cpu_onednn = cpu_bw = None
     if not a.no_cpu and not only:
         cpu_baseline, cpu_onednn = cpu_legs()
+        cpu_bw = cpu_bandwidth_legs()
 
     out = {
         "metric": "TFLOP/s conv2dBackwardData+Filter (ResNet-50 3x3) + GB/s BN/pool backward, 1 GPU",
@@ -260,6 +261,7 @@ def main():
     out["ops"] = ops
     out["cpu_baseline"] = cpu_baseline
     out["cpu_onednn"] = cpu_onednn
+    out["cpu_onednn_bandwidth_ops"] = cpu_bw
     print(json.dumps(out))
     return 0
 
@@ -316,6 +318,66 @@ def cpu_legs():
                       "reference's oneDNN extension requests), full batch 32" % _onednn_version(),
               "sample": "%d repetitions, %.1f s" % (reps, el)}
     return port, onednn
+
+
+def cpu_bandwidth_legs():
+    """The bandwidth-bound ops of cfg 3 on this host's cores through PyTorch-CPU with
+    oneDNN tensors (`to_mkldnn`: the pooling / batch-normalisation primitives the
+    reference's oneDNN extension requests); a few seconds each.  GB/s by the same
+    algorithmic bytes as the GPU figures."""
+    import torch
+    import torch.nn.functional as F
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(0)
+    out = []
+
+    def leg(name, nbytes, fn, budget=2.5):
+        try:
+            fn()
+            reps, t0 = 0, time.perf_counter()
+            while True:
+                fn()
+                reps += 1
+                el = time.perf_counter() - t0
+                if el > budget:
+                    break
+            out.append({"op": name, "ms": el / reps * 1e3, "GBps": nbytes * reps / el / 1e9,
+                        "cores": threads, "sample": "%d repetitions, %.1f s" % (reps, el)})
+        except Exception as e:      # a primitive PyTorch does not route to oneDNN on this host
+            out.append({"op": name, "error": str(e)[:200]})
+
+    T = 32 * 256 * 56 * 56 * 4
+    x = (torch.randn(32, 256, 56, 56, generator=g) * 2 ** 0.5 + 0.5).to_mkldnn()
+    dy = torch.randn(32, 256, 56, 56, generator=g).to_mkldnn()
+    gamma = torch.randn(256, generator=g) * 0.1 + 1
+    beta = torch.zeros(256)
+    leg("batchnorm_fwd_train", 2 * T,
+        lambda: torch.ops.aten.native_batch_norm(x, gamma, beta, None, None, True, 0.0, 1e-5))
+
+    def bn_fwd_bwd():
+        xr = x.to_dense().requires_grad_(True)
+        y = F.batch_norm(xr.to_mkldnn(), None, None, gamma, beta, True, 0.0, 1e-5)
+        y.backward(dy)
+    leg("batchnorm_fwd_train+bwd (autograd, includes layout conversions)", 5 * T, bn_fwd_bwd)
+    del x, dy
+
+    nx, ny = 32 * 64 * 112 * 112 * 4, 32 * 64 * 56 * 56 * 4
+    px = (torch.round(torch.randn(32, 64, 112, 112, generator=g) * 8) / 8).to_mkldnn()
+    leg("pool2d_max_fwd", nx + ny + ny // 4, lambda: torch.max_pool2d(px, 3, 2, 1))
+    leg("pool2d_avg_fwd", nx + ny, lambda: F.avg_pool2d(px, 3, 2, 1, count_include_pad=False))
+    pdy = torch.randn(32, 64, 56, 56, generator=g).to_mkldnn()
+
+    def pool_fwd_bwd(avg):
+        xr = px.to_dense().requires_grad_(True)
+        xm = xr.to_mkldnn()
+        y = F.avg_pool2d(xm, 3, 2, 1, count_include_pad=False) if avg else torch.max_pool2d(xm, 3, 2, 1)
+        y.backward(pdy)
+    leg("pool2d_max_fwd+bwd (autograd, includes layout conversions)", 2 * (nx + ny + ny // 4),
+        lambda: pool_fwd_bwd(False))
+    leg("pool2d_avg_fwd+bwd (autograd, includes layout conversions)", 2 * (nx + ny),
+        lambda: pool_fwd_bwd(True))
+    return out
 
 
 def _onednn_version():
