@@ -352,6 +352,19 @@ __device__ __forceinline__ void res_visit(const BnGeom& g, F&& f) {
   }
 }
 
+// 16-byte (float) / 8-byte (bf16) buffer loads marked non-temporal: data that is read
+// once should not displace what a later pass re-reads from the caches
+__device__ __forceinline__ float4 buf_ld4_stream(__amdgpu_buffer_rsrc_t r, int byte_off, const float*) {
+  const uintx4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 2);
+  return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z),
+                     __uint_as_float(v.w));
+}
+__device__ __forceinline__ float4 buf_ld4_stream(__amdgpu_buffer_rsrc_t r, int byte_off, const bf16_t*) {
+  const uintx2_t v = __builtin_amdgcn_raw_buffer_load_b64(r, byte_off, 0, 2);
+  return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u),
+                     __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
+}
+
 // 16-byte (float) / 8-byte (bf16) buffer store of four values, streaming
 __device__ __forceinline__ void buf_st4(__amdgpu_buffer_rsrc_t r, int byte_off, float4 v, float*) {
   const uintx4_t t = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z),
@@ -376,7 +389,7 @@ bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restri
   const float shift = ld(x, (size_t)(c * g.inner));
   float4 xr[K];
   float s1 = 0.f, s2 = 0.f;
-  res_visit<RES_THREADS, K, ESZ, 0>(g, [&](int k, int off, bool in) { xr[k] = buf_ld4(xr_, off, x); });
+  res_visit<RES_THREADS, K, ESZ, 0>(g, [&](int k, int off, bool in) { xr[k] = buf_ld4_stream(xr_, off, x); });
   res_visit<RES_THREADS, K, ESZ, 1>(g, [&](int k, int, bool in) {
     const float t0 = xr[k].x - shift, t1 = xr[k].y - shift, t2 = xr[k].z - shift,
                 t3 = xr[k].w - shift;
@@ -416,9 +429,10 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
   const float mean = a.save_mean[c];
   float4 xr[K];
   float s1 = 0.f, s2 = 0.f;
-  res_visit<RES_THREADS, K, ESZ, 0>(g, [&](int k, int off, bool in) { xr[k] = buf_ld4(xr_, off, x); });
+  res_visit<RES_THREADS, K, ESZ, 0>(g, [&](int k, int off, bool in) { xr[k] = buf_ld4_stream(xr_, off, x); });
   res_visit<RES_THREADS, K, ESZ, 4>(g, [&](int k, int off, bool in) {
-    const float4 d = buf_ld4(dyr_, off, dy);
+    // dy vectors that stay in LDS are read once; the others come back in the second walk
+    const float4 d = k < klim ? buf_ld4_stream(dyr_, off, dy) : buf_ld4(dyr_, off, dy);
     if (k < klim) dyl[k * RES_THREADS + threadIdx.x] = d;
     const float p1 = (d.x + d.y) + (d.z + d.w);
     const float p2 = (d.x * (xr[k].x - mean) + d.y * (xr[k].y - mean)) +
