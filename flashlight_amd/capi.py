@@ -50,6 +50,16 @@ SYMBOLS = {
     "flhip_copy_bytes": (C.c_int, [_VP, _VP, _SZ, _VP]),
     "flhip_convert": (C.c_int, [_VP, C.c_int, _VP, C.c_int, _SZ, _VP]),
     "flhip_add": (C.c_int, [_VP, _VP, _VP, _SZ, C.c_int, _VP]),
+    "flhip_relu_fwd": (C.c_int, [_VP, _VP, _SZ, C.c_int, _VP]),
+    "flhip_relu_bwd": (C.c_int, [_VP, _VP, _VP, _SZ, C.c_int, _VP]),
+    "flhip_matmul": (C.c_int, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int, C.c_int, _VP,
+                               C.c_int, _VP]),
+    "flhip_sum_columns": (C.c_int, [_VP, _VP, C.c_int32, C.c_int32, C.c_int, _VP]),
+    "flhip_logsoftmax_fwd": (C.c_int, [_VP, _VP, C.c_int32, C.c_int32, C.c_int, _VP]),
+    "flhip_logsoftmax_bwd": (C.c_int, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int, _VP]),
+    "flhip_cce_fwd": (C.c_int, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int, _VP]),
+    "flhip_cce_bwd": (C.c_int, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int, C.c_int32, C.c_int,
+                                _VP]),
 }
 
 _lib = None

@@ -1,0 +1,318 @@
+// Operations of the caller closures around the extension (flashlight/fl/autograd/
+// Functions.cpp) that a network built from conv / pool / batch-norm layers needs to
+// run end to end on device memory: ReLU, the matrix products of Linear, the bias
+// reduction, logSoftmax and categorical cross-entropy.  They are not the measured
+// path; the kernels are plain and bandwidth-shaped.
+//
+// Matrices are column-major like Flashlight tensors: element (r, c) of an R x C
+// matrix is at r + c*R.
+#include "common.h"
+
+namespace flhip {
+namespace {
+
+// ---- ReLU = max(x, 0) and its mask backward (Functions.cpp:329-338, 1787-1789) ----
+template <typename T>
+__global__ void __launch_bounds__(256) relu_fwd_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                       size_t n) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    const float v = ld(x, i);
+    st(y, i, v > 0.f ? v : 0.f);       // fl::maximum(x, 0): NaN compares false -> 0
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) relu_bwd_kernel(const T* __restrict__ dy,
+                                                       const T* __restrict__ x,
+                                                       T* __restrict__ dx, size_t n) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
+    st(dx, i, ld(x, i) > 0.f ? ld(dy, i) : 0.f);
+}
+
+// ---- C = op(A) op(B) (+ bias per row), 64 x 64 tiles, 256 threads, 4 x 4 per thread ----
+constexpr int GT = 64, GK = 16;
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+matmul_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int M, int N,
+              int K, int ta, int tb, const float* __restrict__ bias) {
+  __shared__ float As[GK][GT + 4];      // As[k][m]
+  __shared__ float Bs[GK][GT + 4];      // Bs[k][n]
+  const int tid = threadIdx.x;
+  const int m0 = blockIdx.x * GT, n0 = blockIdx.y * GT;
+  const int tm = (tid & 15) * 4, tn = (tid >> 4) * 4;
+  // op(A)(m, k) = ta ? A[k + m*K] : A[m + k*M];  op(B)(k, n) = tb ? B[n + k*N] : B[k + n*K]
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += GK) {
+    for (int e = tid; e < GT * GK; e += 256) {
+      // consecutive threads walk the contiguous dimension of each operand
+      const int am = ta ? e / GK : e % GT, ak = ta ? e % GK : e / GT;
+      const int gm = m0 + am, gk = k0 + ak;
+      As[ak][am] = (gm < M && gk < K) ? ld(A, ta ? (size_t)gk + (size_t)gm * K : (size_t)gm + (size_t)gk * M) : 0.f;
+      const int bn = tb ? e % GT : e / GK, bk = tb ? e / GT : e % GK;
+      const int gn = n0 + bn, gkb = k0 + bk;
+      Bs[bk][bn] = (gn < N && gkb < K) ? ld(B, tb ? (size_t)gn + (size_t)gkb * N : (size_t)gkb + (size_t)gn * K) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < GK; ++k) {
+      const float4 a = *reinterpret_cast<const float4*>(&As[k][tm]);
+      const float4 b = *reinterpret_cast<const float4*>(&Bs[k][tn]);
+      const float av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] += av[i] * bv[j];
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + tm + i, n = n0 + tn + j;
+      if (m < M && n < N) st(C, (size_t)m + (size_t)n * M, acc[i][j] + (bias ? bias[m] : 0.f));
+    }
+}
+
+// ---- out[r] = sum over columns of x[r, c]  (sumAs(gradOutput, bias), Functions.cpp:1287) ----
+template <typename T>
+__global__ void __launch_bounds__(256)
+sum_cols_kernel(const T* __restrict__ x, float* __restrict__ out, int R, int Cn) {
+  __shared__ float red[4][64];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int r = blockIdx.x * 64 + tx;
+  float s = 0.f;
+  if (r < R)
+    for (int c = ty; c < Cn; c += 4) s += ld(x, (size_t)r + (size_t)c * R);
+  red[ty][tx] = s;
+  __syncthreads();
+  if (ty == 0 && r < R) out[r] = (red[0][tx] + red[1][tx]) + (red[2][tx] + red[3][tx]);
+}
+
+// ---- logSoftmax over dimension 0 of a C x X matrix (Functions.cpp:1044-1070) ----
+// one wave per column
+template <typename T>
+__global__ void __launch_bounds__(256)
+logsoftmax_fwd_kernel(const T* __restrict__ x, T* __restrict__ y, int Cn, int X) {
+  const int col = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (col >= X) return;
+  const T* xc = x + (size_t)col * Cn;
+  float mx = -INFINITY;
+  for (int c = lane; c < Cn; c += 64) mx = fmaxf(mx, ld(xc, c));
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  float s = 0.f;
+  for (int c = lane; c < Cn; c += 64) s += expf(ld(xc, c) - mx);
+  s = wave_sum(s);
+  const float lse = logf(s) + mx;
+  for (int c = lane; c < Cn; c += 64) st(y + (size_t)col * Cn, c, ld(xc, c) - lse);
+}
+
+// dx = dy - exp(y) * sum_c dy
+template <typename T>
+__global__ void __launch_bounds__(256)
+logsoftmax_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ y, T* __restrict__ dx,
+                      int Cn, int X) {
+  const int col = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (col >= X) return;
+  const size_t o = (size_t)col * Cn;
+  float s = 0.f;
+  for (int c = lane; c < Cn; c += 64) s += ld(dy + o, c);
+  s = wave_sum(s);
+  for (int c = lane; c < Cn; c += 64) st(dx + o, c, ld(dy + o, c) - expf(ld(y + o, c)) * s);
+}
+
+// ---- categorical cross-entropy on log-probabilities (Functions.cpp:1078-1154) ----
+// stats[0] = sum over counted columns of -x[target, col], stats[1] = counted columns,
+// stats[2] = columns whose target is neither in [0, C) nor the ignore index,
+// stats[3] = stats[0] / stats[1] (the MEAN reduction).  One block; columns are added
+// in a fixed order.
+template <typename T>
+__global__ void __launch_bounds__(256)
+cce_fwd_kernel(const T* __restrict__ x, const int32_t* __restrict__ target, float* __restrict__ stats,
+               float* __restrict__ per_col, int Cn, int X, int ignore) {
+  __shared__ float red[4];
+  float s = 0.f, cnt = 0.f, bad = 0.f;
+  for (int i = threadIdx.x; i < X; i += 256) {
+    const int t = target[i];
+    float v = 0.f;
+    if (t == ignore) {
+    } else if (t < 0 || t >= Cn) {
+      bad += 1.f;
+    } else {
+      v = -ld(x, (size_t)i * Cn + t);
+      cnt += 1.f;
+    }
+    if (per_col) per_col[i] = v;
+    s += v;
+  }
+  s = block_sum(s, red);
+  cnt = block_sum(cnt, red);
+  bad = block_sum(bad, red);
+  if (threadIdx.x == 0) {
+    stats[0] = s;
+    stats[1] = cnt;
+    stats[2] = bad;
+    stats[3] = s / cnt;
+  }
+}
+
+// dx[c, col] = -(g_col) where c == target[col] and the column counts, else 0;
+// g_col = grad[0] / count (mean), grad[0] (sum) or grad[col] (none)
+template <typename T>
+__global__ void __launch_bounds__(256)
+cce_bwd_kernel(const float* __restrict__ grad, const int32_t* __restrict__ target,
+               const float* __restrict__ stats, T* __restrict__ dx, int Cn, int X, int reduction,
+               int ignore) {
+  const size_t total = (size_t)Cn * X;
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+    const int col = (int)(e / Cn), c = (int)(e - (size_t)col * Cn);
+    const int t = target[col];
+    float v = 0.f;
+    if (t != ignore && c == t) {
+      const float g = reduction == 0 ? grad[col] : reduction == 1 ? grad[0] / stats[1] : grad[0];
+      v = -g;
+    }
+    st(dx, e, v);
+  }
+}
+
+unsigned blocks_for(size_t n) {
+  size_t b = (n + 255) / 256;
+  if (b > 16384) b = 16384;
+  if (b < 1) b = 1;
+  return (unsigned)b;
+}
+
+}  // namespace
+}  // namespace flhip
+
+using namespace flhip;
+
+extern "C" int flhip_relu_fwd(const void* x, void* y, size_t n, int dtype, void* stream) {
+  FLHIP_REQUIRE((x && y) || n == 0, "relu: null argument");
+  FLHIP_REQUIRE(dtype_ok(dtype), "relu: unknown dtype");
+  if (n == 0) return FLHIP_OK;
+  if (dtype == FLHIP_F32)
+    hipLaunchKernelGGL((relu_fwd_kernel<float>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream),
+                       (const float*)x, (float*)y, n);
+  else
+    hipLaunchKernelGGL((relu_fwd_kernel<bf16_t>), dim3(blocks_for(n)), dim3(256), 0,
+                       as_stream(stream), (const bf16_t*)x, (bf16_t*)y, n);
+  return check_launch("relu");
+}
+
+extern "C" int flhip_relu_bwd(const void* dy, const void* x, void* dx, size_t n, int dtype,
+                              void* stream) {
+  FLHIP_REQUIRE((dy && x && dx) || n == 0, "relu_bwd: null argument");
+  FLHIP_REQUIRE(dtype_ok(dtype), "relu_bwd: unknown dtype");
+  if (n == 0) return FLHIP_OK;
+  if (dtype == FLHIP_F32)
+    hipLaunchKernelGGL((relu_bwd_kernel<float>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream),
+                       (const float*)dy, (const float*)x, (float*)dx, n);
+  else
+    hipLaunchKernelGGL((relu_bwd_kernel<bf16_t>), dim3(blocks_for(n)), dim3(256), 0,
+                       as_stream(stream), (const bf16_t*)dy, (const bf16_t*)x, (bf16_t*)dx, n);
+  return check_launch("relu_bwd");
+}
+
+extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, int32_t N, int32_t K,
+                            int trans_a, int trans_b, const float* bias_rows, int dtype,
+                            void* stream) {
+  FLHIP_REQUIRE(A && B && C, "matmul: null argument");
+  FLHIP_REQUIRE(M > 0 && N > 0 && K > 0, "matmul: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "matmul: unknown dtype");
+  const dim3 grid((unsigned)((M + GT - 1) / GT), (unsigned)((N + GT - 1) / GT));
+  FLHIP_REQUIRE(grid.y <= 65535, "matmul: too many columns");
+  if (dtype == FLHIP_F32)
+    hipLaunchKernelGGL((matmul_kernel<float>), grid, dim3(256), 0, as_stream(stream), (const float*)A,
+                       (const float*)B, (float*)C, M, N, K, trans_a, trans_b, bias_rows);
+  else
+    hipLaunchKernelGGL((matmul_kernel<bf16_t>), grid, dim3(256), 0, as_stream(stream),
+                       (const bf16_t*)A, (const bf16_t*)B, (bf16_t*)C, M, N, K, trans_a, trans_b,
+                       bias_rows);
+  return check_launch("matmul");
+}
+
+extern "C" int flhip_sum_columns(const void* x, float* out, int32_t rows, int32_t cols, int dtype,
+                                 void* stream) {
+  FLHIP_REQUIRE(x && out, "sum_columns: null argument");
+  FLHIP_REQUIRE(rows > 0 && cols > 0, "sum_columns: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "sum_columns: unknown dtype");
+  const dim3 grid((unsigned)((rows + 63) / 64));
+  if (dtype == FLHIP_F32)
+    hipLaunchKernelGGL((sum_cols_kernel<float>), grid, dim3(256), 0, as_stream(stream),
+                       (const float*)x, out, rows, cols);
+  else
+    hipLaunchKernelGGL((sum_cols_kernel<bf16_t>), grid, dim3(256), 0, as_stream(stream),
+                       (const bf16_t*)x, out, rows, cols);
+  return check_launch("sum_columns");
+}
+
+extern "C" int flhip_logsoftmax_fwd(const void* x, void* y, int32_t classes, int32_t cols, int dtype,
+                                    void* stream) {
+  FLHIP_REQUIRE(x && y, "logsoftmax: null argument");
+  FLHIP_REQUIRE(classes > 0 && cols > 0, "logsoftmax: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "logsoftmax: unknown dtype");
+  const dim3 grid((unsigned)((cols + 3) / 4));
+  if (dtype == FLHIP_F32)
+    hipLaunchKernelGGL((logsoftmax_fwd_kernel<float>), grid, dim3(256), 0, as_stream(stream),
+                       (const float*)x, (float*)y, classes, cols);
+  else
+    hipLaunchKernelGGL((logsoftmax_fwd_kernel<bf16_t>), grid, dim3(256), 0, as_stream(stream),
+                       (const bf16_t*)x, (bf16_t*)y, classes, cols);
+  return check_launch("logsoftmax");
+}
+
+extern "C" int flhip_logsoftmax_bwd(const void* dy, const void* y, void* dx, int32_t classes,
+                                    int32_t cols, int dtype, void* stream) {
+  FLHIP_REQUIRE(dy && y && dx, "logsoftmax_bwd: null argument");
+  FLHIP_REQUIRE(classes > 0 && cols > 0, "logsoftmax_bwd: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "logsoftmax_bwd: unknown dtype");
+  const dim3 grid((unsigned)((cols + 3) / 4));
+  if (dtype == FLHIP_F32)
+    hipLaunchKernelGGL((logsoftmax_bwd_kernel<float>), grid, dim3(256), 0, as_stream(stream),
+                       (const float*)dy, (const float*)y, (float*)dx, classes, cols);
+  else
+    hipLaunchKernelGGL((logsoftmax_bwd_kernel<bf16_t>), grid, dim3(256), 0, as_stream(stream),
+                       (const bf16_t*)dy, (const bf16_t*)y, (bf16_t*)dx, classes, cols);
+  return check_launch("logsoftmax_bwd");
+}
+
+extern "C" int flhip_cce_fwd(const void* logp, const int32_t* target, float* stats, float* per_column,
+                             int32_t classes, int32_t cols, int32_t ignore_index, int dtype,
+                             void* stream) {
+  FLHIP_REQUIRE(logp && target && stats, "cce: null argument");
+  FLHIP_REQUIRE(classes > 0 && cols > 0, "cce: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "cce: unknown dtype");
+  if (dtype == FLHIP_F32)
+    hipLaunchKernelGGL((cce_fwd_kernel<float>), dim3(1), dim3(256), 0, as_stream(stream),
+                       (const float*)logp, target, stats, per_column, classes, cols, ignore_index);
+  else
+    hipLaunchKernelGGL((cce_fwd_kernel<bf16_t>), dim3(1), dim3(256), 0, as_stream(stream),
+                       (const bf16_t*)logp, target, stats, per_column, classes, cols, ignore_index);
+  return check_launch("cce");
+}
+
+extern "C" int flhip_cce_bwd(const float* grad, const int32_t* target, const float* stats, void* dx,
+                             int32_t classes, int32_t cols, int reduction, int32_t ignore_index,
+                             int dtype, void* stream) {
+  FLHIP_REQUIRE(grad && target && stats && dx, "cce_bwd: null argument");
+  FLHIP_REQUIRE(classes > 0 && cols > 0, "cce_bwd: sizes must be positive");
+  FLHIP_REQUIRE(reduction >= 0 && reduction <= 2, "cce_bwd: unknown reduction");
+  FLHIP_REQUIRE(dtype_ok(dtype), "cce_bwd: unknown dtype");
+  const size_t total = (size_t)classes * cols;
+  if (dtype == FLHIP_F32)
+    hipLaunchKernelGGL((cce_bwd_kernel<float>), dim3(blocks_for(total)), dim3(256), 0,
+                       as_stream(stream), grad, target, stats, (float*)dx, classes, cols, reduction,
+                       ignore_index);
+  else
+    hipLaunchKernelGGL((cce_bwd_kernel<bf16_t>), dim3(blocks_for(total)), dim3(256), 0,
+                       as_stream(stream), grad, target, stats, (bf16_t*)dx, classes, cols, reduction,
+                       ignore_index);
+  return check_launch("cce_bwd");
+}

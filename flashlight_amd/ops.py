@@ -261,3 +261,119 @@ def batchnorm_backward(grad_output, input, weight, save_mean, save_invstd, axes)
                                        _ptr(save_invstd), _ptr(dx), _ptr(dg), _ptr(db), _ptr(ws),
                                        nws, _stream()))
     return dx, dg, db
+
+
+# ---- operations of the caller closures (flashlight/fl/autograd/Functions.cpp) -------
+# Shapes follow the rule of the rest of this module: a torch tensor's shape is the
+# Flashlight shape reversed (same memory).  A Flashlight [features, batch] matrix is a
+# torch [batch, features] tensor.
+
+def relu(input):
+    """fl::relu (Functions.cpp:1787-1789)."""
+    x = _dev(input, "input")
+    y = torch.empty_like(x)
+    capi.check(capi.lib().flhip_relu_fwd(_ptr(x), _ptr(y), x.numel(), _dtype_tag(x), _stream()))
+    return y
+
+
+def relu_backward(grad_output, input):
+    g, x = _dev(grad_output, "gradOutput"), _dev(input, "input")
+    if g.shape != x.shape or g.dtype != x.dtype:
+        raise ValueError("relu backward: gradOutput must match the input")
+    dx = torch.empty_like(x)
+    capi.check(capi.lib().flhip_relu_bwd(_ptr(g), _ptr(x), _ptr(dx), x.numel(), _dtype_tag(x),
+                                         _stream()))
+    return dx
+
+
+def linear(input, weight, bias=None):
+    """fl::linear (Functions.cpp:1255-1309): input [..., in] (Flashlight [in, ...]), weight
+    torch [in, out] (Flashlight [out, in]), bias [out] or None -> [..., out]."""
+    x, w = _dev(input, "input"), _dev(weight, "weight")
+    if w.dim() != 2 or x.shape[-1] != w.shape[0] or x.dtype != w.dtype:
+        raise ValueError("linear: input [.., in] and weight [in, out] of one type expected")
+    fin, fout = w.shape
+    frames = x.numel() // fin
+    b = None
+    if bias is not None and bias.numel() > 0:
+        if bias.numel() != fout:
+            raise ValueError("linear: bias must have one element per output feature")
+        b = _dev(bias, "bias").float().contiguous()
+    y = torch.empty(tuple(x.shape[:-1]) + (fout,), dtype=x.dtype, device=x.device)
+    capi.check(capi.lib().flhip_matmul(_ptr(w), _ptr(x), _ptr(y), fout, frames, fin, 0, 0, _ptr(b),
+                                       _dtype_tag(x), _stream()))
+    return y
+
+
+def linear_backward(grad_output, input, weight, want_bias=True):
+    """-> (gradInput, gradWeight, gradBias or None), the three branches of the gradient
+    closure of fl::linear (Functions.cpp:1276-1303)."""
+    g, x, w = _dev(grad_output, "gradOutput"), _dev(input, "input"), _dev(weight, "weight")
+    fin, fout = w.shape
+    frames = x.numel() // fin
+    tag = _dtype_tag(x)
+    dx = torch.empty_like(x)
+    capi.check(capi.lib().flhip_matmul(_ptr(w), _ptr(g), _ptr(dx), fin, frames, fout, 1, 0, None, tag,
+                                       _stream()))
+    dw = torch.empty_like(w)
+    capi.check(capi.lib().flhip_matmul(_ptr(g), _ptr(x), _ptr(dw), fout, fin, frames, 0, 1, None, tag,
+                                       _stream()))
+    db = None
+    if want_bias:
+        db = torch.empty((fout,), dtype=torch.float32, device=x.device)
+        capi.check(capi.lib().flhip_sum_columns(_ptr(g), _ptr(db), fout, frames, tag, _stream()))
+    return dx, dw, db
+
+
+def log_softmax(input):
+    """fl::logSoftmax over Flashlight dimension 0 (Functions.cpp:1044-1070): torch [..., classes]."""
+    x = _dev(input, "input")
+    y = torch.empty_like(x)
+    classes = x.shape[-1]
+    capi.check(capi.lib().flhip_logsoftmax_fwd(_ptr(x), _ptr(y), classes, x.numel() // classes,
+                                               _dtype_tag(x), _stream()))
+    return y
+
+
+def log_softmax_backward(grad_output, output):
+    g, y = _dev(grad_output, "gradOutput"), _dev(output, "output")
+    dx = torch.empty_like(y)
+    classes = y.shape[-1]
+    capi.check(capi.lib().flhip_logsoftmax_bwd(_ptr(g), _ptr(y), _ptr(dx), classes,
+                                               y.numel() // classes, _dtype_tag(y), _stream()))
+    return dx
+
+
+REDUCE_NONE, REDUCE_MEAN, REDUCE_SUM = 0, 1, 2
+
+
+def categorical_cross_entropy(input, targets, reduction=REDUCE_MEAN, ignore_index=-1):
+    """fl::categoricalCrossEntropy (Functions.cpp:1078-1154) on log-probabilities
+    [..., classes] and int32 targets [...] -> (loss, stats); stats feeds the backward.
+    Raises ValueError for targets outside [0, classes), as the reference throws."""
+    x, t = _dev(input, "input"), _dev(targets, "targets")
+    if t.dtype != torch.int32 or tuple(t.shape) != tuple(x.shape[:-1]):
+        raise ValueError("categoricalCrossEntropy: int32 targets with one dimension fewer expected")
+    classes = x.shape[-1]
+    cols = t.numel()
+    stats = torch.empty((4,), dtype=torch.float32, device=x.device)
+    per = torch.empty((cols,), dtype=torch.float32, device=x.device) if reduction == REDUCE_NONE else None
+    capi.check(capi.lib().flhip_cce_fwd(_ptr(x), _ptr(t), _ptr(stats), _ptr(per), classes, cols,
+                                        ignore_index, _dtype_tag(x), _stream()))
+    if float(stats[2].item()) != 0.0:
+        raise ValueError("target contains elements out of valid range [0, num_categories) "
+                         "in categorical cross entropy")
+    if reduction == REDUCE_NONE:
+        return per.reshape(t.shape), stats
+    return (stats[3:4] if reduction == REDUCE_MEAN else stats[0:1]), stats
+
+
+def categorical_cross_entropy_backward(grad_output, input_shape, dtype, targets, stats,
+                                       reduction=REDUCE_MEAN, ignore_index=-1):
+    g, t = _dev(grad_output, "gradOutput").float().contiguous(), _dev(targets, "targets")
+    dx = torch.empty(tuple(input_shape), dtype=dtype, device=t.device)
+    classes = input_shape[-1]
+    tag = capi.F32 if dtype == torch.float32 else capi.BF16
+    capi.check(capi.lib().flhip_cce_bwd(_ptr(g), _ptr(t), _ptr(stats), _ptr(dx), classes, t.numel(),
+                                        reduction, ignore_index, tag, _stream()))
+    return dx

@@ -196,6 +196,55 @@ int flhip_convert(const void* src, int src_dtype, void* dst, int dst_dtype,
 int flhip_add(const void* a, const void* b, void* out, size_t n, int dtype,
               void* stream);
 
+/* ---- operations of the caller closures (flashlight/fl/autograd/Functions.cpp) ----
+ * What a network of conv / pool / batch-norm layers needs besides the extension to
+ * run one training step on device memory.  Matrices are column-major like
+ * Flashlight tensors: element (r, c) of an R x C matrix is at r + c*R. */
+
+/* fl::relu = max(x, 0) (Functions.cpp:329-338, 1787-1789) and its backward
+ * dx = dy where x > 0, else 0. */
+int flhip_relu_fwd(const void* x, void* y, size_t n, int dtype, void* stream);
+int flhip_relu_bwd(const void* dy, const void* x, void* dx, size_t n, int dtype,
+                   void* stream);
+
+/* C (M x N) = op(A) (M x K) * op(B) (K x N), fp32 accumulate; trans_a: A is stored
+ * K x M, trans_b: B is stored N x K.  bias_rows (fp32[M], may be NULL) is added to
+ * every column.  Serves fl::linear (Functions.cpp:1255-1309): forward
+ * matmul(weight, input) + tile(bias), backward matmulTN(weight, gradOutput) and
+ * matmulNT(gradOutput, input). */
+int flhip_matmul(const void* A, const void* B, void* C, int32_t M, int32_t N,
+                 int32_t K, int trans_a, int trans_b, const float* bias_rows,
+                 int dtype, void* stream);
+
+/* out[r] (fp32) = sum over c of x[r, c] for a rows x cols matrix: the bias gradient
+ * sumAs(gradOutput, bias) of fl::linear (Functions.cpp:1285-1289). */
+int flhip_sum_columns(const void* x, float* out, int32_t rows, int32_t cols, int dtype,
+                      void* stream);
+
+/* fl::logSoftmax over dimension 0 of a classes x cols matrix (Functions.cpp:1044-1070)
+ * and its backward dx = dy - exp(y) * sum over classes of dy. */
+int flhip_logsoftmax_fwd(const void* x, void* y, int32_t classes, int32_t cols,
+                         int dtype, void* stream);
+int flhip_logsoftmax_bwd(const void* dy, const void* y, void* dx, int32_t classes,
+                         int32_t cols, int dtype, void* stream);
+
+/* fl::categoricalCrossEntropy on log-probabilities logp (classes x cols) and int32
+ * targets (Functions.cpp:1078-1154).  stats (fp32[4], device) receives: [0] the sum of
+ * -logp[target, col] over counted columns (ReduceMode::SUM), [1] the number of counted
+ * columns (target != ignore_index), [2] the number of columns whose target is outside
+ * [0, classes) and not ignore_index (the reference throws std::invalid_argument for
+ * those, :1100-1108: the host reads this entry), [3] = [0] / [1] (ReduceMode::MEAN).
+ * per_column (fp32[cols], may be NULL) receives the unreduced values (ReduceMode::NONE).
+ * Backward: dx[c, col] = -g where c == target[col] and the column counts, else 0, with
+ * g = grad[col] (reduction 0 = NONE), grad[0] / stats[1] (1 = MEAN) or grad[0] (2 = SUM);
+ * grad is fp32 on the device. */
+int flhip_cce_fwd(const void* logp, const int32_t* target, float* stats,
+                  float* per_column, int32_t classes, int32_t cols,
+                  int32_t ignore_index, int dtype, void* stream);
+int flhip_cce_bwd(const float* grad, const int32_t* target, const float* stats, void* dx,
+                  int32_t classes, int32_t cols, int reduction, int32_t ignore_index,
+                  int dtype, void* stream);
+
 /* Plain device-to-device copy kernel of `bytes` bytes (multiple of 16).  Not part
  * of the operator interface: it is the known-size kernel that hardware byte
  * counters are calibrated against when measuring the kernels above. */

@@ -388,3 +388,98 @@ void flref_bn_running_update(int64_t C, int64_t M, const float* mean,
     }
   }
 }
+
+/* ---- caller closures (flashlight/fl/autograd/Functions.cpp) ---------------------- */
+
+/* fl::maximum(x, 0) (:329-338): NaN > 0 is false, so NaN maps to 0 as in the mask */
+void flref_relu_fwd(int64_t n, const float* x, float* y) {
+  for (int64_t i = 0; i < n; ++i) y[i] = x[i] > 0.f ? x[i] : 0.f;
+}
+
+/* mask = (x > 0) (:333-335) */
+void flref_relu_bwd(int64_t n, const float* dy, const float* x, float* dx) {
+  for (int64_t i = 0; i < n; ++i) dx[i] = x[i] > 0.f ? dy[i] : 0.f;
+}
+
+/* fl::matmul / matmulTN / matmulNT as used by fl::linear (:1264-1265, 1292-1301) */
+void flref_matmul(int M, int N, int K, int ta, int tb, const float* A, const float* B,
+                  const float* bias, float* C) {
+#pragma omp parallel for
+  for (int n = 0; n < N; ++n)
+    for (int m = 0; m < M; ++m) {
+      double s = 0.0;
+      for (int k = 0; k < K; ++k) {
+        const double a = ta ? A[(size_t)k + (size_t)m * K] : A[(size_t)m + (size_t)k * M];
+        const double b = tb ? B[(size_t)n + (size_t)k * N] : B[(size_t)k + (size_t)n * K];
+        s += a * b;
+      }
+      C[(size_t)m + (size_t)n * M] = (float)(s + (bias ? (double)bias[m] : 0.0));
+    }
+}
+
+void flref_sum_columns(int rows, int cols, const float* x, float* out) {
+  for (int r = 0; r < rows; ++r) {
+    double s = 0.0;
+    for (int c = 0; c < cols; ++c) s += x[(size_t)r + (size_t)c * rows];
+    out[r] = (float)s;
+  }
+}
+
+/* x - (log(sum(exp(x - max))) + max) per column (:1046-1056) */
+void flref_logsoftmax_fwd(int classes, int cols, const float* x, float* y) {
+  for (int c = 0; c < cols; ++c) {
+    const float* xc = x + (size_t)c * classes;
+    double mx = xc[0];
+    for (int k = 1; k < classes; ++k) mx = xc[k] > mx ? xc[k] : mx;
+    double s = 0.0;
+    for (int k = 0; k < classes; ++k) s += exp((double)xc[k] - mx);
+    const double lse = log(s) + mx;
+    for (int k = 0; k < classes; ++k) y[(size_t)c * classes + k] = (float)((double)xc[k] - lse);
+  }
+}
+
+/* gradOutput - exp(result) * sum(gradOutput) (:1061-1066) */
+void flref_logsoftmax_bwd(int classes, int cols, const float* dy, const float* y, float* dx) {
+  for (int c = 0; c < cols; ++c) {
+    const size_t o = (size_t)c * classes;
+    double s = 0.0;
+    for (int k = 0; k < classes; ++k) s += dy[o + k];
+    for (int k = 0; k < classes; ++k) dx[o + k] = (float)((double)dy[o + k] - exp((double)y[o + k]) * s);
+  }
+}
+
+/* -x[target] per column, ignored columns 0; MEAN divides by the counted columns
+ * (:1112-1126) */
+int flref_cce_fwd(int classes, int cols, const float* logp, const int32_t* target, int ignore,
+                  float* per_column, float* loss, float* count) {
+  int bad = 0;
+  double s = 0.0, n = 0.0;
+  for (int c = 0; c < cols; ++c) {
+    const int t = target[c];
+    double v = 0.0;
+    if (t == ignore) {
+    } else if (t < 0 || t >= classes) {
+      ++bad;
+    } else {
+      v = -(double)logp[(size_t)c * classes + t];
+      n += 1.0;
+    }
+    if (per_column) per_column[c] = (float)v;
+    s += v;
+  }
+  loss[0] = (float)s;
+  loss[1] = (float)(s / n);
+  *count = (float)n;
+  return bad;
+}
+
+/* tile(grad) * mask with mask = -(class == target), ignored columns 0 (:1135-1150) */
+void flref_cce_bwd(int classes, int cols, const float* grad, const int32_t* target, int ignore,
+                   int reduction, float count, float* dx) {
+  for (int c = 0; c < cols; ++c) {
+    const int t = target[c];
+    const double g = reduction == 0 ? grad[c] : reduction == 1 ? (double)grad[0] / count : grad[0];
+    for (int k = 0; k < classes; ++k)
+      dx[(size_t)c * classes + k] = (t != ignore && k == t) ? (float)(-g) : 0.f;
+  }
+}

@@ -89,6 +89,27 @@ void flref_bn_running_update(int64_t C, int64_t M, const float* mean,
                              const float* var, double momentum, float* run_mean,
                              float* run_var);
 
+/* ---- caller closures (flashlight/fl/autograd/Functions.cpp); column-major matrices:
+ * element (r, c) of an R x C matrix at r + c*R ---- */
+/* max(x, 0) and its mask backward (:329-338, 1787-1789) */
+void flref_relu_fwd(int64_t n, const float* x, float* y);
+void flref_relu_bwd(int64_t n, const float* dy, const float* x, float* dx);
+/* C (M x N) = op(A) op(B) + bias[m]; ta: A stored K x M, tb: B stored N x K; double
+ * accumulate.  fl::linear (:1255-1309) = (W, X), backward (W^T, dY) and (dY, X^T). */
+void flref_matmul(int M, int N, int K, int ta, int tb, const float* A, const float* B,
+                  const float* bias, float* C);
+/* out[r] = sum_c x[r, c] (sumAs(gradOutput, bias), :1285-1289) */
+void flref_sum_columns(int rows, int cols, const float* x, float* out);
+/* logSoftmax over dimension 0 of a classes x cols matrix (:1044-1070) */
+void flref_logsoftmax_fwd(int classes, int cols, const float* x, float* y);
+void flref_logsoftmax_bwd(int classes, int cols, const float* dy, const float* y, float* dx);
+/* categoricalCrossEntropy (:1078-1154): returns the number of targets outside
+ * [0, classes) that are not ignore; loss[0] = SUM, loss[1] = MEAN, count = counted columns */
+int flref_cce_fwd(int classes, int cols, const float* logp, const int32_t* target, int ignore,
+                  float* per_column, float* loss, float* count);
+void flref_cce_bwd(int classes, int cols, const float* grad, const int32_t* target, int ignore,
+                   int reduction, float count, float* dx);
+
 #ifdef __cplusplus
 }
 #endif

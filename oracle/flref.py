@@ -179,3 +179,75 @@ def bn_view(shape_whcn, axes):
     for s in shape_whcn[axes[-1] + 1:]:
         outer *= s
     return outer, nfeat, total // (nfeat * outer)
+
+
+# ---- caller closures; matrices column-major (numpy: pass arrays whose reversed shape is
+# the Flashlight shape, i.e. [cols, rows] row-major) ----------------------------------------
+
+def relu_fwd(x):
+    x = _f32(x)
+    y = np.empty_like(x)
+    lib().flref_relu_fwd(_i64(x.size), _p(x), _p(y))
+    return y
+
+
+def relu_bwd(dy, x):
+    dy, x = _f32(dy), _f32(x)
+    dx = np.empty_like(x)
+    lib().flref_relu_bwd(_i64(x.size), _p(dy), _p(x), _p(dx))
+    return dx
+
+
+def matmul(M, N, K, A, B, ta=False, tb=False, bias=None):
+    """C (M x N, column-major, returned as a numpy [N, M] array)."""
+    A, B = _f32(A), _f32(B)
+    b = None if bias is None else _f32(bias)
+    out = np.empty((N, M), np.float32)
+    lib().flref_matmul(C.c_int(M), C.c_int(N), C.c_int(K), C.c_int(int(ta)), C.c_int(int(tb)), _p(A),
+                       _p(B), None if b is None else _p(b), _p(out))
+    return out
+
+
+def sum_columns(rows, cols, x):
+    x = _f32(x)
+    out = np.empty((rows,), np.float32)
+    lib().flref_sum_columns(C.c_int(rows), C.c_int(cols), _p(x), _p(out))
+    return out
+
+
+def logsoftmax_fwd(x):
+    """x: numpy [cols, classes] (Flashlight [classes, cols])."""
+    x = _f32(x)
+    y = np.empty_like(x)
+    lib().flref_logsoftmax_fwd(C.c_int(x.shape[-1]), C.c_int(x.size // x.shape[-1]), _p(x), _p(y))
+    return y
+
+
+def logsoftmax_bwd(dy, y):
+    dy, y = _f32(dy), _f32(y)
+    dx = np.empty_like(y)
+    lib().flref_logsoftmax_bwd(C.c_int(y.shape[-1]), C.c_int(y.size // y.shape[-1]), _p(dy), _p(y),
+                               _p(dx))
+    return dx
+
+
+def cce_fwd(logp, target, ignore=-1):
+    """-> (per_column, loss_sum, loss_mean, count, bad)."""
+    logp = _f32(logp)
+    t = np.ascontiguousarray(target, dtype=np.int32)
+    per = np.empty((t.size,), np.float32)
+    loss = np.empty((2,), np.float32)
+    cnt = C.c_float()
+    bad = lib().flref_cce_fwd(C.c_int(logp.shape[-1]), C.c_int(t.size), _p(logp),
+                              t.ctypes.data_as(C.c_void_p), C.c_int(ignore), _p(per), _p(loss),
+                              C.byref(cnt))
+    return per, float(loss[0]), float(loss[1]), cnt.value, bad
+
+
+def cce_bwd(shape, grad, target, count, reduction=1, ignore=-1):
+    g = _f32(np.atleast_1d(grad))
+    t = np.ascontiguousarray(target, dtype=np.int32)
+    dx = np.empty(shape, np.float32)
+    lib().flref_cce_bwd(C.c_int(shape[-1]), C.c_int(t.size), _p(g), t.ctypes.data_as(C.c_void_p),
+                        C.c_int(ignore), C.c_int(reduction), C.c_float(count), _p(dx))
+    return dx

@@ -1,0 +1,169 @@
+"""GPU parity of the caller-closure operations (ReLU, Linear's matrix products, bias
+reduction, logSoftmax, categorical cross-entropy) against oracle/flref.c, through the C
+ABI, and one training step of the README MNIST convnet (configs[0]) end to end."""
+import numpy as np
+import pytest
+import torch
+
+import flashlight_amd as fa
+from flashlight_amd import ops
+from gpu_util import bf16_round, dev, host
+from oracle import flref
+from refmath import rel_l2
+
+pytestmark = pytest.mark.gpu
+DT = [torch.float32, torch.bfloat16]
+
+
+def _tol(dtype):
+    return 1e-4 if dtype == torch.float32 else 2e-2
+
+
+def _round(a, dtype):
+    return a if dtype == torch.float32 else bf16_round(a)
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_relu(dtype):
+    rng = np.random.default_rng(60)
+    x = _round(rng.standard_normal(5000).astype(np.float32), dtype)
+    x[:4] = [0.0, -0.0, np.inf, -np.inf]
+    dy = _round(rng.standard_normal(5000).astype(np.float32), dtype)
+    assert np.array_equal(host(ops.relu(dev(x, dtype))), flref.relu_fwd(x))
+    assert np.array_equal(host(ops.relu_backward(dev(dy, dtype), dev(x, dtype))), flref.relu_bwd(dy, x))
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("fin,fout,batch", [(3136, 1024, 16), (1024, 10, 64), (37, 21, 9), (5, 130, 1), (200, 1, 70)])
+def test_linear(fin, fout, batch, dtype):
+    rng = np.random.default_rng(fin + fout + batch)
+    x = _round(rng.standard_normal((batch, fin)).astype(np.float32), dtype)
+    w = _round((rng.standard_normal((fin, fout)) / np.sqrt(fin)).astype(np.float32), dtype)
+    b = rng.standard_normal(fout).astype(np.float32)
+    dy = _round(rng.standard_normal((batch, fout)).astype(np.float32), dtype)
+    tol = _tol(dtype)
+    y = ops.linear(dev(x, dtype), dev(w, dtype), dev(b))
+    assert rel_l2(host(y), flref.matmul(fout, batch, fin, w, x, False, False, b)) <= tol
+    y0 = ops.linear(dev(x, dtype), dev(w, dtype), None)
+    assert rel_l2(host(y0), flref.matmul(fout, batch, fin, w, x)) <= tol
+    dx, dw, db = ops.linear_backward(dev(dy, dtype), dev(x, dtype), dev(w, dtype))
+    assert rel_l2(host(dx), flref.matmul(fin, batch, fout, w, dy, True, False)) <= tol
+    assert rel_l2(host(dw), flref.matmul(fout, fin, batch, dy, x, False, True)) <= tol
+    assert rel_l2(host(db), flref.sum_columns(fout, batch, dy)) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("classes,cols", [(10, 64), (1000, 7), (1, 5), (65, 3)])
+def test_logsoftmax(classes, cols, dtype):
+    rng = np.random.default_rng(classes + cols)
+    x = _round((rng.standard_normal((cols, classes)) * 4).astype(np.float32), dtype)
+    dy = _round(rng.standard_normal((cols, classes)).astype(np.float32), dtype)
+    y_ref = flref.logsoftmax_fwd(x)
+    y = ops.log_softmax(dev(x, dtype))
+    if dtype == torch.float32:
+        assert np.allclose(host(y), y_ref, atol=2e-6, rtol=1e-5)
+    else:
+        assert np.allclose(host(y), y_ref, atol=0.06, rtol=1e-2)
+    yq = _round(y_ref, dtype)
+    dx = ops.log_softmax_backward(dev(dy, dtype), dev(yq, dtype))
+    dx_ref = flref.logsoftmax_bwd(dy, yq)
+    assert np.allclose(host(dx), dx_ref, atol=_tol(dtype) * 10, rtol=_tol(dtype))
+
+
+@pytest.mark.parametrize("reduction", [ops.REDUCE_NONE, ops.REDUCE_MEAN, ops.REDUCE_SUM])
+def test_cross_entropy(reduction):
+    rng = np.random.default_rng(70 + reduction)
+    logp = np.log(rng.dirichlet(np.ones(10), size=300)).astype(np.float32)
+    target = rng.integers(0, 10, 300).astype(np.int32)
+    target[[5, 17, 200]] = -1
+    per, s, mean, count, bad = flref.cce_fwd(logp, target)
+    loss, stats = ops.categorical_cross_entropy(dev(logp), dev(target), reduction)
+    want = [per, np.float32(mean), np.float32(s)][reduction]
+    assert np.allclose(host(loss).reshape(np.shape(want)), want, rtol=1e-5, atol=1e-6)
+    g = rng.standard_normal(300 if reduction == ops.REDUCE_NONE else 1).astype(np.float32)
+    dx = ops.categorical_cross_entropy_backward(dev(g), logp.shape, torch.float32, dev(target), stats,
+                                                reduction)
+    assert np.allclose(host(dx), flref.cce_bwd(logp.shape, g, target, count, reduction), rtol=1e-6,
+                       atol=1e-7)
+    with pytest.raises(ValueError):
+        ops.categorical_cross_entropy(dev(logp), dev(np.full(300, 10, np.int32)))
+
+
+def _mnist_params(rng):
+    """Conv2D / Linear initialisation of the reference (nn/modules/Conv2D.cpp:177-194,
+    Linear.cpp:62-74): Kaiming-uniform weights, bias U(+-sqrt(1/fanIn))."""
+    def ku(shape, fan_in):
+        return rng.uniform(-np.sqrt(3.0 / fan_in), np.sqrt(3.0 / fan_in), shape).astype(np.float32)
+
+    def bu(n, fan_in):
+        return rng.uniform(-np.sqrt(1.0 / fan_in), np.sqrt(1.0 / fan_in), n).astype(np.float32)
+    return dict(w1=ku((32, 1, 5, 5), 25), b1=bu(32, 25), w2=ku((64, 32, 5, 5), 800), b2=bu(64, 800),
+                w3=ku((3136, 1024), 3136), b3=bu(1024, 3136), w4=ku((1024, 10), 1024), b4=bu(10, 1024))
+
+
+def test_mnist_convnet_training_step():
+    """configs[0]: View, Conv2D 1->32 5x5 SAME, ReLU, Pool2D max 2x2 s2, Conv2D 32->64 5x5
+    SAME, ReLU, Pool2D, View, Linear 3136->1024, ReLU, Linear 1024->10, LogSoftmax, then
+    categoricalCrossEntropy (reference README); dropout left out (it is a random mask, not
+    part of the path).  Forward and the gradient closures in tape order, device against
+    oracle, every parameter gradient compared."""
+    rng = np.random.default_rng(80)
+    B = 16
+    x = rng.standard_normal((B, 1, 28, 28)).astype(np.float32)
+    labels = rng.integers(0, 10, B).astype(np.int32)
+    P = _mnist_params(rng)
+    pad = fa.derive_padding(28, 5, 1, -1)          # SAME
+    assert pad == 2 and fa.derive_padding(14, 5, 1, -1) == 2
+    MAXP = fa.PoolingMode.MAX
+
+    # ---- oracle -----------------------------------------------------------------
+    d1 = flref.conv_desc(x.shape, P["w1"].shape, (1, 1), (2, 2))
+    a1 = flref.conv2d_fwd(d1, x, P["w1"], P["b1"]); r1 = flref.relu_fwd(a1)
+    pd1 = flref.pool_desc(r1.shape, (2, 2), (2, 2), (0, 0), 0); p1, am1 = flref.pool2d_fwd(pd1, r1)
+    d2 = flref.conv_desc(p1.shape, P["w2"].shape, (1, 1), (2, 2))
+    a2 = flref.conv2d_fwd(d2, p1, P["w2"], P["b2"]); r2 = flref.relu_fwd(a2)
+    pd2 = flref.pool_desc(r2.shape, (2, 2), (2, 2), (0, 0), 0); p2, am2 = flref.pool2d_fwd(pd2, r2)
+    f = p2.reshape(B, 3136)
+    a3 = flref.matmul(1024, B, 3136, P["w3"], f, False, False, P["b3"]); r3 = flref.relu_fwd(a3)
+    a4 = flref.matmul(10, B, 1024, P["w4"], r3, False, False, P["b4"])
+    lp = flref.logsoftmax_fwd(a4)
+    _, _, loss_ref, count, bad = flref.cce_fwd(lp, labels)
+    assert bad == 0
+    g = flref.cce_bwd(lp.shape, np.ones(1, np.float32), labels, count, 1)
+    g = flref.logsoftmax_bwd(g, lp)
+    R = {"b4": flref.sum_columns(10, B, g), "w4": flref.matmul(10, 1024, B, g, r3, False, True)}
+    g = flref.relu_bwd(flref.matmul(1024, B, 10, P["w4"], g, True, False), a3)
+    R["b3"] = flref.sum_columns(1024, B, g); R["w3"] = flref.matmul(1024, 3136, B, g, f, False, True)
+    g = flref.matmul(3136, B, 1024, P["w3"], g, True, False).reshape(p2.shape)
+    g = flref.relu_bwd(flref.pool2d_bwd(pd2, g, am2), a2)
+    R["w2"], R["b2"] = flref.conv2d_bwd_filter(d2, p1, g)
+    g = flref.relu_bwd(flref.pool2d_bwd(pd1, flref.conv2d_bwd_data(d2, g, P["w2"]), am1), a1)
+    R["w1"], R["b1"] = flref.conv2d_bwd_filter(d1, x, g)
+
+    # ---- device ------------------------------------------------------------------
+    D = {k: dev(v) for k, v in P.items()}
+    xd, ld = dev(x), dev(labels)
+    A1 = ops.conv2d(xd, D["w1"], D["b1"], 1, 1, 2, 2); R1 = ops.relu(A1)
+    P1, AM1 = ops.pool2d(R1, 2, 2, 2, 2, 0, 0, MAXP)
+    A2 = ops.conv2d(P1, D["w2"], D["b2"], 1, 1, 2, 2); R2 = ops.relu(A2)
+    P2, AM2 = ops.pool2d(R2, 2, 2, 2, 2, 0, 0, MAXP)
+    Fl = P2.reshape(B, 3136)
+    A3 = ops.linear(Fl, D["w3"], D["b3"]); R3 = ops.relu(A3)
+    A4 = ops.linear(R3, D["w4"], D["b4"])
+    LP = ops.log_softmax(A4)
+    loss, stats = ops.categorical_cross_entropy(LP, ld)
+    assert abs(float(loss.item()) - loss_ref) <= 1e-5 * max(1.0, abs(loss_ref))
+    G = ops.categorical_cross_entropy_backward(dev(np.ones(1, np.float32)), LP.shape, torch.float32, ld,
+                                               stats)
+    G = ops.log_softmax_backward(G, LP)
+    G, dw4, db4 = ops.linear_backward(G, R3, D["w4"])
+    G, dw3, db3 = ops.linear_backward(ops.relu_backward(G, A3), Fl, D["w3"])
+    G = ops.pool2d_backward(G.reshape(P2.shape), R2.shape, AM2, 2, 2, 2, 2, 0, 0, MAXP)
+    G = ops.relu_backward(G, A2)
+    dw2, db2 = ops.conv2d_backward_filter_bias(G, P1, D["w2"].shape, True, 1, 1, 2, 2)
+    G = ops.conv2d_backward_data(G, P1.shape, D["w2"], 1, 1, 2, 2)
+    G = ops.relu_backward(ops.pool2d_backward(G, R1.shape, AM1, 2, 2, 2, 2, 0, 0, MAXP), A1)
+    dw1, db1 = ops.conv2d_backward_filter_bias(G, xd, D["w1"].shape, True, 1, 1, 2, 2)
+    got = dict(w1=dw1, b1=db1, w2=dw2, b2=db2, w3=dw3, b3=db3, w4=dw4, b4=db4)
+    for k in sorted(R):
+        assert rel_l2(host(got[k]), R[k]) <= 1e-4, (k, rel_l2(host(got[k]), R[k]))

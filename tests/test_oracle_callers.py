@@ -1,0 +1,104 @@
+"""Pins the caller-closure functions of oracle/flref.c (ReLU, the matrix products of
+Linear, logSoftmax, categorical cross-entropy) against PyTorch-CPU library routines in
+float64 and against closed forms.  Arrays are row-major with the Flashlight shape
+reversed: a Flashlight [features, batch] matrix is a numpy [batch, features] array."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import flref
+from refmath import rel_l2
+
+
+def test_relu_and_mask():
+    # Functions.cpp:329-338, 1787-1789; AutogradTest checks relu by its Jacobian
+    x = np.array([-2.0, -0.0, 0.0, 1e-30, 3.5, np.nan, -np.inf, np.inf], np.float32)
+    y = flref.relu_fwd(x)
+    assert np.array_equal(y, np.array([0, 0, 0, 1e-30, 3.5, 0, 0, np.inf], np.float32))
+    dy = np.arange(1, 9, dtype=np.float32)
+    assert np.array_equal(flref.relu_bwd(dy, x), np.array([0, 0, 0, 4, 5, 0, 0, 8], np.float32))
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal(1000).astype(np.float32)
+    assert np.array_equal(flref.relu_fwd(x), F.relu(torch.from_numpy(x)).numpy())
+
+
+@pytest.mark.parametrize("M,N,K", [(5, 7, 3), (64, 64, 16), (70, 33, 129), (1, 9, 200), (10, 1, 1)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_matmul_against_float64(M, N, K, ta, tb):
+    rng = np.random.default_rng(M * 1000 + N * 10 + K)
+    opA = rng.standard_normal((M, K))          # mathematical op(A), op(B)
+    opB = rng.standard_normal((K, N))
+    bias = rng.standard_normal(M).astype(np.float32)
+    # storage: column-major M x K == numpy [K, M]; transposed storage K x M == numpy [M, K]
+    A = np.ascontiguousarray(opA if ta else opA.T, dtype=np.float32)
+    B = np.ascontiguousarray(opB if tb else opB.T, dtype=np.float32)
+    a64 = (A.astype(np.float64) if ta else A.astype(np.float64).T)
+    b64 = (B.astype(np.float64) if tb else B.astype(np.float64).T)
+    want = a64 @ b64 + bias[:, None]
+    got = flref.matmul(M, N, K, A, B, ta, tb, bias)          # numpy [N, M]
+    assert rel_l2(got.T, want) < 1e-6
+
+
+def test_linear_forward_backward_like_torch():
+    # fl::linear (Functions.cpp:1255-1309): y = W x + b; dX = W^T dY; dW = dY X^T; db = sum dY
+    rng = np.random.default_rng(3)
+    fin, fout, batch = 37, 21, 9
+    x = rng.standard_normal((batch, fin)).astype(np.float32)          # Flashlight [in, batch]
+    w = rng.standard_normal((fin, fout)).astype(np.float32)           # Flashlight [out, in]
+    b = rng.standard_normal(fout).astype(np.float32)
+    dy = rng.standard_normal((batch, fout)).astype(np.float32)
+    xt = torch.from_numpy(x).double().requires_grad_(True)
+    wt = torch.from_numpy(w).double().requires_grad_(True)            # [in, out]
+    bt = torch.from_numpy(b).double().requires_grad_(True)
+    yt = xt @ wt + bt
+    yt.backward(torch.from_numpy(dy).double())
+    y = flref.matmul(fout, batch, fin, w, x, False, False, b)
+    assert rel_l2(y, yt.detach().numpy()) < 1e-6
+    dx = flref.matmul(fin, batch, fout, w, dy, True, False)
+    assert rel_l2(dx, xt.grad.numpy()) < 1e-6
+    dw = flref.matmul(fout, fin, batch, dy, x, False, True)            # numpy [in, out]
+    assert rel_l2(dw, wt.grad.numpy()) < 1e-6
+    db = flref.sum_columns(fout, batch, dy)
+    assert rel_l2(db, bt.grad.numpy()) < 1e-6
+
+
+def test_logsoftmax_like_torch():
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal((13, 10)) * 5).astype(np.float32)
+    x[0, 3] = 80.0          # large logits: the max subtraction must keep this finite
+    dy = rng.standard_normal((13, 10)).astype(np.float32)
+    xt = torch.from_numpy(x).double().requires_grad_(True)
+    yt = torch.log_softmax(xt, dim=-1)
+    yt.backward(torch.from_numpy(dy).double())
+    y = flref.logsoftmax_fwd(x)
+    assert np.allclose(y, yt.detach().numpy(), atol=1e-5, rtol=1e-6)
+    assert np.allclose(np.exp(y.astype(np.float64)).sum(-1), 1.0, atol=1e-5)
+    dx = flref.logsoftmax_bwd(dy, y)
+    assert rel_l2(dx, xt.grad.numpy()) < 1e-5
+
+
+@pytest.mark.parametrize("reduction", [0, 1, 2])
+def test_cross_entropy_like_torch(reduction):
+    # Functions.cpp:1078-1154, ignoreIndex = -1 by default
+    rng = np.random.default_rng(5 + reduction)
+    logp = np.log(rng.dirichlet(np.ones(10), size=17)).astype(np.float32)
+    target = rng.integers(0, 10, 17).astype(np.int32)
+    target[[2, 11]] = -1                                   # ignored columns
+    per, s, mean, count, bad = flref.cce_fwd(logp, target)
+    assert bad == 0 and count == 15
+    lt = torch.from_numpy(logp).double().requires_grad_(True)
+    tt = torch.from_numpy(target).long()
+    mode = ["none", "mean", "sum"][reduction]
+    want = F.nll_loss(lt, tt, ignore_index=-1, reduction=mode)
+    got = [per, mean, s][reduction]
+    assert np.allclose(got, want.detach().numpy(), rtol=1e-6, atol=1e-6)
+    g = rng.standard_normal(17 if reduction == 0 else 1).astype(np.float32)
+    want.backward(torch.from_numpy(g).double() if reduction == 0 else torch.tensor(float(g[0]), dtype=torch.float64))
+    dx = flref.cce_bwd(logp.shape, g, target, count, reduction)
+    assert np.allclose(dx, lt.grad.numpy(), rtol=1e-6, atol=1e-7)
+
+
+def test_cross_entropy_flags_bad_targets():
+    logp = np.zeros((4, 3), np.float32)
+    assert flref.cce_fwd(logp, np.array([0, 3, 2, -2], np.int32))[4] == 2
