@@ -185,4 +185,173 @@ Variable batchnorm(const Variable& input, const Variable& weight, const Variable
   return Variable(output, {input, weight, bias}, gradFunc);
 }
 
+namespace {
+int tagOf(dtype t, const char* fn) {
+  if (t == dtype::f32) return FLHIP_F32;
+  if (t == dtype::bf16) return FLHIP_BF16;
+  throw std::runtime_error(std::string(fn) + ": f32 and bf16 only");
+}
+void check(int rc) {
+  if (rc == FLHIP_INVALID_ARGUMENT) throw std::invalid_argument(flhip_last_error());
+  if (rc != FLHIP_OK) throw std::runtime_error(flhip_last_error());
+}
+}  // namespace
+
+Variable relu(const Variable& input) {
+  Tensor out(input.shape(), input.type());
+  check(flhip_relu_fwd(input.tensor().device(), out.device(), (size_t)out.elements(),
+                       tagOf(input.type(), "relu"), hipBackendStream()));
+  auto gradFunc = [](std::vector<Variable>& inputs, const Variable& gradOutput) {
+    // mask = (input > 0) (Functions.cpp:333-335)
+    auto& in = inputs[0];
+    if (!in.isCalcGrad()) return;
+    Tensor g(in.shape(), gradOutput.type());
+    check(flhip_relu_bwd(gradOutput.tensor().device(), in.tensor().device(), g.device(),
+                         (size_t)g.elements(), tagOf(g.type(), "relu"), hipBackendStream()));
+    in.addGrad(Variable(g, false));
+  };
+  return Variable(out, {input}, gradFunc);
+}
+
+Variable moddims(const Variable& input, const Shape& dims) {
+  // one -1 is inferred from the element count (Functions.cpp:797-815)
+  std::vector<Dim> d = dims.get();
+  Dim known = 1;
+  int infer = -1;
+  for (size_t i = 0; i < d.size(); ++i) {
+    if (d[i] == -1) {
+      if (infer >= 0) throw std::invalid_argument("moddims: only one dimension may be -1");
+      infer = (int)i;
+    } else {
+      known *= d[i];
+    }
+  }
+  if (infer >= 0) d[infer] = known ? input.tensor().elements() / known : 0;
+  const Shape target(d);
+  if (target.elements() != input.tensor().elements())
+    throw std::invalid_argument("moddims: mismatched number of elements");
+  const Shape inShape = input.shape();
+  auto gradFunc = [inShape](std::vector<Variable>& inputs, const Variable& gradOutput) {
+    inputs[0].addGrad(Variable(gradOutput.tensor().reshaped(inShape), false));
+  };
+  return Variable(input.tensor().reshaped(target), {input}, gradFunc);
+}
+
+Variable linear(const Variable& input, const Variable& weight) {
+  return linear(input, weight, Variable());
+}
+
+Variable linear(const Variable& input, const Variable& weight, const Variable& bias) {
+  dtypesMatch("linear", {&input, &weight, &bias});
+  if (weight.tensor().ndim() != 2 || input.tensor().ndim() < 1 ||
+      input.tensor().dim(0) != weight.tensor().dim(1))
+    throw std::invalid_argument("linear: weight must be [out, in] and input [in, ...]");
+  const int tag = tagOf(input.type(), "linear");
+  const Dim out = weight.tensor().dim(0), in = weight.tensor().dim(1);
+  const Dim frames = input.tensor().elements() / in;
+  std::vector<Dim> oshape = input.shape().get();
+  oshape[0] = out;
+  const bool hasBias = bias.tensor().elements() > 0;
+  if (hasBias && bias.tensor().elements() != out)
+    throw std::invalid_argument("linear: bias must have one element per output feature");
+  // the tiled bias is added in fp32 inside the product (Functions.cpp:1267-1272)
+  const Tensor b32 = hasBias ? bias.tensor().astype(dtype::f32) : Tensor();
+  Tensor output(Shape(oshape), input.type());
+  check(flhip_matmul(weight.tensor().device(), input.tensor().device(), output.device(), (int32_t)out,
+                     (int32_t)frames, (int32_t)in, 0, 0, static_cast<const float*>(b32.device()), tag,
+                     hipBackendStream()));
+  auto gradFunc = [hasBias, tag, out, in, frames](std::vector<Variable>& inputs,
+                                                  const Variable& gradOutput) {
+    // Functions.cpp:1276-1303
+    auto& x = inputs[0];
+    auto& wt = inputs[1];
+    const void* g = gradOutput.tensor().device();
+    if (hasBias && inputs[2].isCalcGrad()) {
+      Tensor db(inputs[2].shape(), dtype::f32);
+      check(flhip_sum_columns(g, static_cast<float*>(db.device()), (int32_t)out, (int32_t)frames, tag,
+                              hipBackendStream()));
+      inputs[2].addGrad(Variable(db.astype(inputs[2].type()), false));
+    }
+    if (x.isCalcGrad()) {
+      Tensor dx(x.shape(), x.type());
+      check(flhip_matmul(wt.tensor().device(), g, dx.device(), (int32_t)in, (int32_t)frames,
+                         (int32_t)out, 1, 0, nullptr, tag, hipBackendStream()));
+      x.addGrad(Variable(dx, false));
+    }
+    if (wt.isCalcGrad()) {
+      Tensor dw(wt.shape(), wt.type());
+      check(flhip_matmul(g, x.tensor().device(), dw.device(), (int32_t)out, (int32_t)in,
+                         (int32_t)frames, 0, 1, nullptr, tag, hipBackendStream()));
+      wt.addGrad(Variable(dw, false));
+    }
+  };
+  if (hasBias) return Variable(output, {input, weight, bias}, gradFunc);
+  return Variable(output, {input, weight}, gradFunc);
+}
+
+Variable logSoftmax(const Variable& input, int dim) {
+  if (dim != 0) throw std::invalid_argument("logSoftmax: only dimension 0 is supported by this backend");
+  const int tag = tagOf(input.type(), "logSoftmax");
+  const Dim classes = input.tensor().dim(0), cols = input.tensor().elements() / classes;
+  Tensor result(input.shape(), input.type());
+  check(flhip_logsoftmax_fwd(input.tensor().device(), result.device(), (int32_t)classes, (int32_t)cols,
+                             tag, hipBackendStream()));
+  auto gradFunc = [result, tag, classes, cols](std::vector<Variable>& inputs,
+                                               const Variable& gradOutput) {
+    // gradOutput - exp(result) * sum(gradOutput) (Functions.cpp:1061-1066)
+    Tensor g(result.shape(), result.type());
+    check(flhip_logsoftmax_bwd(gradOutput.tensor().device(), result.device(), g.device(),
+                               (int32_t)classes, (int32_t)cols, tag, hipBackendStream()));
+    inputs[0].addGrad(Variable(g.astype(inputs[0].type()), false));
+  };
+  return Variable(result, {input}, gradFunc);
+}
+
+Variable categoricalCrossEntropy(const Variable& input, const Variable& targets, ReduceMode reduction,
+                                 int ignoreIndex) {
+  // Functions.cpp:1086-1098
+  if (input.tensor().ndim() != targets.tensor().ndim() + 1)
+    throw std::invalid_argument("dimension mismatch in categorical cross entropy: "
+                                "target must have one fewer dimension than input");
+  for (int i = 1; i < input.tensor().ndim(); ++i)
+    if (input.tensor().dim(i) != targets.tensor().dim(i - 1))
+      throw std::invalid_argument("dimension mismatch in categorical cross entropy");
+  if (targets.type() != dtype::s32)
+    throw std::invalid_argument("categoricalCrossEntropy: targets must be s32 on this backend");
+  const int tag = tagOf(input.type(), "categoricalCrossEntropy");
+  const Dim C = input.tensor().dim(0), X = targets.tensor().elements();
+  Tensor stats(Shape({4}), dtype::f32);
+  Tensor per = reduction == ReduceMode::NONE ? Tensor(targets.shape(), dtype::f32) : Tensor();
+  check(flhip_cce_fwd(input.tensor().device(), static_cast<const int32_t*>(targets.tensor().device()),
+                      static_cast<float*>(stats.device()), static_cast<float*>(per.device()),
+                      (int32_t)C, (int32_t)X, ignoreIndex, tag, hipBackendStream()));
+  // the reference reads a device scalar here too (:1100-1108)
+  const std::vector<float> st = stats.toHostVector();
+  if (st[2] != 0.f)
+    throw std::invalid_argument("target contains elements out of valid range [0, num_categories) "
+                                "in categorical cross entropy");
+  Tensor result;
+  if (reduction == ReduceMode::NONE) {
+    result = per;
+  } else {
+    const float v = reduction == ReduceMode::MEAN ? st[3] : st[0];
+    result = Tensor::fromHost(Shape({1}), dtype::f32, &v);
+  }
+  const Shape inShape = input.shape();
+  const dtype inType = input.type();
+  const Tensor tg = targets.tensor();
+  auto gradFunc = [stats, tg, inShape, inType, tag, C, X, reduction, ignoreIndex](
+                      std::vector<Variable>& inputs, const Variable& gradOutput) {
+    // tile(grad / denominator) * mask (Functions.cpp:1131-1150)
+    Tensor g(inShape, inType);
+    const Tensor go = gradOutput.tensor().astype(dtype::f32);
+    check(flhip_cce_bwd(static_cast<const float*>(go.device()),
+                        static_cast<const int32_t*>(tg.device()),
+                        static_cast<const float*>(stats.device()), g.device(), (int32_t)C, (int32_t)X,
+                        (int)reduction, ignoreIndex, tag, hipBackendStream()));
+    inputs[0].addGrad(Variable(g, false));
+  };
+  return Variable(result, {input, targets}, gradFunc);
+}
+
 }  // namespace fl

@@ -2,8 +2,10 @@
 // differentiable functions whose closures drive the extension, with the control
 // flow of flashlight/fl/autograd/Functions.cpp:1327-1565 (dtype checks, payload
 // creation, which backward op runs when) and the reverse-topological backward of
-// flashlight/fl/autograd/Variable.cpp:235-294.  Only what is needed to exercise
-// the extension the way Flashlight does is provided.
+// flashlight/fl/autograd/Variable.cpp:235-294; plus the few functions a network of
+// those layers needs to run a training step on the device (relu, linear, moddims,
+// logSoftmax, categoricalCrossEntropy).  Only what is needed to exercise the
+// extension the way Flashlight does is provided.
 #pragma once
 
 #include <functional>
@@ -57,5 +59,22 @@ Variable pool2d(const Variable& input, int wx, int wy, int sx = 1, int sy = 1, i
 Variable batchnorm(const Variable& input, const Variable& weight, const Variable& bias,
                    Variable& runningMean, Variable& runningVar, const std::vector<int>& axes,
                    bool train, double momentum, double epsilon);
+
+// flashlight/fl/common/Defines.h:83-87
+enum class ReduceMode { NONE = 0, MEAN = 1, SUM = 2 };
+
+// fl::relu = max(input, 0) (Functions.cpp:329-338, 1787-1789)
+Variable relu(const Variable& input);
+// fl::moddims / View: same data, new shape; one dimension may be -1 (Functions.cpp:790-829)
+Variable moddims(const Variable& input, const Shape& dims);
+// fl::linear (Functions.cpp:1255-1309): weight [out, in], input [in, ...], bias [out] or empty
+Variable linear(const Variable& input, const Variable& weight, const Variable& bias);
+Variable linear(const Variable& input, const Variable& weight);
+// fl::logSoftmax over dimension 0 (Functions.cpp:1044-1070; other dimensions throw here)
+Variable logSoftmax(const Variable& input, int dim);
+// fl::categoricalCrossEntropy (Functions.cpp:1078-1154): input [C, X...] log-probabilities,
+// targets [X...] of type s32
+Variable categoricalCrossEntropy(const Variable& input, const Variable& targets,
+                                 ReduceMode reduction = ReduceMode::MEAN, int ignoreIndex = -1);
 
 }  // namespace fl

@@ -5,7 +5,9 @@
 //   flashlight/fl/test/autograd/AutogradConv2DTest.cpp:21-74,137-162 (shapes),
 //   flashlight/fl/test/autograd/AutogradTest.cpp:65-81,333-337 (dtype errors, pool),
 //   flashlight/fl/test/autograd/AutogradNormalizationTest.cpp:158-189 (batchnorm),
-//   flashlight/fl/test/nn/ModuleTest.cpp:338-353 (batching invariance).
+//   flashlight/fl/test/nn/ModuleTest.cpp:338-353 (batching invariance),
+// and one training step of the README MNIST convnet (README.md:45-84) through the tape.
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -267,6 +269,103 @@ static void testGradAccumulation() {
   CHECK(ok);
 }
 
+static std::vector<float> uniformv(size_t n, unsigned seed, float bound) {
+  std::mt19937 gen(seed);
+  std::uniform_real_distribution<float> d(-bound, bound);
+  std::vector<float> v(n);
+  for (auto& x : v) x = d(gen);
+  return v;
+}
+
+// One forward + backward step of the README convnet (README.md:45-84; dropout left out):
+// View, Conv2D 1->32 5x5 SAME, ReLU, Pool2D 2x2 s2, Conv2D 32->64 5x5 SAME, ReLU, Pool2D,
+// View, Linear 3136->1024, ReLU, Linear 1024->10, LogSoftmax, categoricalCrossEntropy;
+// loss.backward() through the tape against the CPU checker run layer by layer.
+static void testMnistStep() {
+  std::printf("MNIST convnet training step\n");
+  const int B = 8;
+  auto x = randn((size_t)B * 28 * 28, 21);
+  std::vector<int32_t> labels(B);
+  for (int i = 0; i < B; ++i) labels[i] = (i * 7 + 3) % 10;
+  // Conv2D::initialize / Linear::initialize: Kaiming-uniform weights, bias U(+-sqrt(1/fanIn))
+  auto w1 = uniformv(32 * 25, 22, std::sqrt(3.f / 25)), b1 = uniformv(32, 23, std::sqrt(1.f / 25));
+  auto w2 = uniformv(64 * 32 * 25, 24, std::sqrt(3.f / 800)), b2 = uniformv(64, 25, std::sqrt(1.f / 800));
+  auto w3 = uniformv((size_t)1024 * 3136, 26, std::sqrt(3.f / 3136)), b3 = uniformv(1024, 27, std::sqrt(1.f / 3136));
+  auto w4 = uniformv(10 * 1024, 28, std::sqrt(3.f / 1024)), b4 = uniformv(10, 29, std::sqrt(1.f / 1024));
+  const int pad = derivePadding(28, 5, 1, -1, 1);
+  CHECK(pad == 2);
+
+  // ---- CPU checker ---------------------------------------------------------------
+  flref_conv d1{B, 1, 28, 28, 32, 5, 5, 1, 1, pad, pad, 1, 1, 1}, d2{B, 32, 14, 14, 64, 5, 5, 1, 1, pad, pad, 1, 1, 1};
+  flref_pool p1{B, 32, 28, 28, 2, 2, 2, 2, 0, 0, 0}, p2{B, 64, 14, 14, 2, 2, 2, 2, 0, 0, 0};
+  std::vector<float> a1((size_t)B * 32 * 784), r1(a1.size()), q1((size_t)B * 32 * 196);
+  std::vector<uint8_t> m1(q1.size());
+  std::vector<float> a2((size_t)B * 64 * 196), r2(a2.size()), q2((size_t)B * 64 * 49);
+  std::vector<uint8_t> m2(q2.size());
+  std::vector<float> a3((size_t)B * 1024), r3(a3.size()), a4((size_t)B * 10), lp(a4.size());
+  flref_conv2d_fwd(&d1, x.data(), w1.data(), b1.data(), a1.data());
+  flref_relu_fwd((int64_t)a1.size(), a1.data(), r1.data());
+  flref_pool2d_fwd(&p1, r1.data(), q1.data(), m1.data());
+  flref_conv2d_fwd(&d2, q1.data(), w2.data(), b2.data(), a2.data());
+  flref_relu_fwd((int64_t)a2.size(), a2.data(), r2.data());
+  flref_pool2d_fwd(&p2, r2.data(), q2.data(), m2.data());
+  flref_matmul(1024, B, 3136, 0, 0, w3.data(), q2.data(), b3.data(), a3.data());
+  flref_relu_fwd((int64_t)a3.size(), a3.data(), r3.data());
+  flref_matmul(10, B, 1024, 0, 0, w4.data(), r3.data(), b4.data(), a4.data());
+  flref_logsoftmax_fwd(10, B, a4.data(), lp.data());
+  float loss[2], count;
+  CHECK(flref_cce_fwd(10, B, lp.data(), labels.data(), -1, nullptr, loss, &count) == 0);
+  const float one = 1.f;
+  std::vector<float> g4(a4.size()), g4b(a4.size()), dw4(w4.size()), db4(10), g3(a3.size()), dw3(w3.size()), db3(1024);
+  std::vector<float> gq2(q2.size()), gr2(r2.size()), dw2(w2.size()), db2(64), gq1(q1.size()), gr1(r1.size()), dw1(w1.size()), db1(32);
+  flref_cce_bwd(10, B, &one, labels.data(), -1, 1, count, g4.data());
+  flref_logsoftmax_bwd(10, B, g4.data(), lp.data(), g4b.data());
+  flref_sum_columns(10, B, g4b.data(), db4.data());
+  flref_matmul(10, 1024, B, 0, 1, g4b.data(), r3.data(), nullptr, dw4.data());
+  flref_matmul(1024, B, 10, 1, 0, w4.data(), g4b.data(), nullptr, g3.data());
+  flref_relu_bwd((int64_t)g3.size(), g3.data(), a3.data(), g3.data());
+  flref_sum_columns(1024, B, g3.data(), db3.data());
+  flref_matmul(1024, 3136, B, 0, 1, g3.data(), q2.data(), nullptr, dw3.data());
+  flref_matmul(3136, B, 1024, 1, 0, w3.data(), g3.data(), nullptr, gq2.data());
+  flref_pool2d_bwd(&p2, gq2.data(), m2.data(), gr2.data());
+  flref_relu_bwd((int64_t)gr2.size(), gr2.data(), a2.data(), gr2.data());
+  flref_conv2d_bwd_filter(&d2, q1.data(), gr2.data(), dw2.data(), db2.data());
+  flref_conv2d_bwd_data(&d2, gr2.data(), w2.data(), gq1.data());
+  flref_pool2d_bwd(&p1, gq1.data(), m1.data(), gr1.data());
+  flref_relu_bwd((int64_t)gr1.size(), gr1.data(), a1.data(), gr1.data());
+  flref_conv2d_bwd_filter(&d1, x.data(), gr1.data(), dw1.data(), db1.data());
+
+  // ---- device, through the tape ---------------------------------------------------
+  Variable in(Tensor::fromVector({28 * 28, B}, x), false);
+  Variable W1(Tensor::fromVector({5, 5, 1, 32}, w1), true), B1(Tensor::fromVector({1, 1, 32, 1}, b1), true);
+  Variable W2(Tensor::fromVector({5, 5, 32, 64}, w2), true), B2(Tensor::fromVector({1, 1, 64, 1}, b2), true);
+  Variable W3(Tensor::fromVector({1024, 3136}, w3), true), B3(Tensor::fromVector({1024}, b3), true);
+  Variable W4(Tensor::fromVector({10, 1024}, w4), true), B4(Tensor::fromVector({10}, b4), true);
+  Variable tg(Tensor::fromHost(Shape({B}), dtype::s32, labels.data()), false);
+  Variable h = moddims(in, Shape({28, 28, 1, -1}));
+  h = pool2d(relu(conv2d(h, W1, B1, 1, 1, pad, pad)), 2, 2, 2, 2);
+  h = pool2d(relu(conv2d(h, W2, B2, 1, 1, pad, pad)), 2, 2, 2, 2);
+  CHECK(h.shape() == Shape({7, 7, 64, B}));
+  h = moddims(h, Shape({7 * 7 * 64, -1}));
+  h = relu(linear(h, W3, B3));
+  Variable out = logSoftmax(linear(h, W4, B4), 0);
+  CHECK(out.shape() == Shape({10, B}));
+  CHECK(relL2(out.tensor().toHostVector(), lp) <= 1e-4);
+  Variable L = categoricalCrossEntropy(out, tg);
+  CHECK(std::fabs(L.tensor().toHostVector()[0] - loss[1]) <= 1e-5f * std::max(1.f, std::fabs(loss[1])));
+  L.backward(Variable(Tensor::fromVector({1}, {1.f}), false));
+  CHECK(relL2(W4.grad().tensor().toHostVector(), dw4) <= 1e-4 && relL2(B4.grad().tensor().toHostVector(), db4) <= 1e-4);
+  CHECK(relL2(W3.grad().tensor().toHostVector(), dw3) <= 1e-4 && relL2(B3.grad().tensor().toHostVector(), db3) <= 1e-4);
+  CHECK(relL2(W2.grad().tensor().toHostVector(), dw2) <= 1e-4 && relL2(B2.grad().tensor().toHostVector(), db2) <= 1e-4);
+  CHECK(relL2(W1.grad().tensor().toHostVector(), dw1) <= 1e-4 && relL2(B1.grad().tensor().toHostVector(), db1) <= 1e-4);
+  CHECK(!in.isCalcGrad());
+  // targets outside [0, classes) throw like the reference (Functions.cpp:1100-1108)
+  std::vector<int32_t> badl(B, 10);
+  Variable bad(Tensor::fromHost(Shape({B}), dtype::s32, badl.data()), false);
+  CHECK(throws<std::invalid_argument>([&] { categoricalCrossEntropy(out, bad); }));
+  CHECK(throws<std::invalid_argument>([&] { moddims(in, Shape({5, -1})); }));
+}
+
 int main() {
   try {
     CHECK(derivePadding(56, 3, 1, -1, 1) == 1 && derivePadding(224, 7, 2, -1, 1) == 3 &&
@@ -281,6 +380,7 @@ int main() {
     testPool();
     testBatchnorm();
     testGradAccumulation();
+    testMnistStep();
     fl::sync();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
