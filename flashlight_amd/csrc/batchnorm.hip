@@ -319,12 +319,14 @@ constexpr int RES_MIN_C_BWD = 128;
 // offset is relative to the tensor base and goes through a buffer descriptor; slots
 // past the feature get an offset past the descriptor's range, so their loads return
 // zero and their stores are dropped without a branch.
-template <int RES_THREADS, int K, int ESZ, int FENCE, typename F>
+template <int RES_THREADS, int K, int ESZ, int FENCE, bool REV = false, typename F>
 __device__ __forceinline__ void res_visit(const BnGeom& g, F&& f) {
   constexpr int OOB = (int)0x80000000;
   const int innerV = (int)(g.inner >> 2);
   const int c = blockIdx.x;
-  int q = threadIdx.x;
+  // REV walks k = K-1 .. 0: what the previous walk loaded last is asked for first,
+  // while the caches still hold it
+  int q = threadIdx.x + (REV ? (K - 1) * RES_THREADS : 0);
   int o = q / innerV, i = q - o * innerV;
   const int so = RES_THREADS / innerV, si = RES_THREADS - so * innerV;
   const int row = (int)(g.C * g.inner) * ESZ;                 // bytes between outer slices
@@ -335,19 +337,30 @@ __device__ __forceinline__ void res_visit(const BnGeom& g, F&& f) {
   // offsets of the first walk alive for the next one would cost K registers.
   asm volatile("" : "+v"(off), "+v"(i), "+v"(q));
 #pragma unroll
-  for (int k = 0; k < K; ++k) {
+  for (int kk = 0; kk < K; ++kk) {
+    const int k = REV ? K - 1 - kk : kk;
     const bool in = q < (int)g.units;
     f(k, in ? off : OOB, in);
     // FENCE > 0: finish each group of FENCE vectors before starting the next, or the
     // scheduler overlaps the temporaries of all K vectors and runs out of registers
-    if (FENCE > 0 && k % (FENCE > 0 ? FENCE : 1) == (FENCE > 0 ? FENCE : 1) - 1)
+    if (FENCE > 0 && kk % (FENCE > 0 ? FENCE : 1) == (FENCE > 0 ? FENCE : 1) - 1)
       __builtin_amdgcn_sched_barrier(0);
-    q += RES_THREADS;
-    off += step;
-    i += si;
-    if (i >= innerV) {
-      i -= innerV;
-      off += wrap;
+    if (REV) {
+      q -= RES_THREADS;
+      off -= step;
+      i -= si;
+      if (i < 0) {
+        i += innerV;
+        off -= wrap;
+      }
+    } else {
+      q += RES_THREADS;
+      off += step;
+      i += si;
+      if (i >= innerV) {
+        i -= innerV;
+        off += wrap;
+      }
     }
   }
 }
@@ -448,7 +461,7 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
   finish_bwd(g, a, c, (double)s1, (double)s2, true, sh);
   __syncthreads();
   const float kdy = sh[1], kx = sh[2], k0 = sh[3];
-  res_visit<RES_THREADS, K, ESZ, 4>(g, [&](int k, int off, bool) {
+  res_visit<RES_THREADS, K, ESZ, 4, true>(g, [&](int k, int off, bool) {
     const float4 d = k < klim ? dyl[k * RES_THREADS + threadIdx.x] : buf_ld4(dyr_, off, dy);
     const float4 v = make_float4(kdy * d.x + (kx * (xr[k].x - mean) + k0),
                                  kdy * d.y + (kx * (xr[k].y - mean) + k0),
