@@ -60,6 +60,11 @@ SYMBOLS = {
     "flhip_cce_fwd": (C.c_int, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int, _VP]),
     "flhip_cce_bwd": (C.c_int, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int, C.c_int32, C.c_int,
                                 _VP]),
+    "flhip_affine_fwd": (C.c_int, [_VP, _VP, _VP, _VP, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int,
+                                   _VP]),
+    "flhip_affine_bwd_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int64, C.c_int64, C.c_int]),
+    "flhip_affine_bwd": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, C.c_int64, C.c_int64, C.c_int64, C.c_int,
+                                   C.c_int, _VP, C.c_size_t, _VP]),
 }
 
 _lib = None

@@ -188,6 +188,89 @@ unsigned blocks_for(size_t n) {
   return (unsigned)b;
 }
 
+// ---- broadcast scale and shift, y = w * x + b (the affine part of LayerNorm,
+// flashlight/fl/nn/modules/LayerNorm.cpp:110-128: tileAs(weight) * output + tileAs(bias)) ----
+// The tensor is viewed as [outer][mid][inner]; the parameters have one element per
+// mid index (pstride 1) or a single element (pstride 0).
+template <typename T>
+__global__ void __launch_bounds__(256)
+affine_fwd_kernel(const T* __restrict__ x, const T* __restrict__ w, const T* __restrict__ b,
+                  T* __restrict__ y, size_t n, long long mid, long long inner, int pstride) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += stride) {
+    const size_t m = (size_t)pstride * ((e / (size_t)inner) % (size_t)mid);
+    st(y, e, ld(w, m) * ld(x, e) + ld(b, m));
+  }
+}
+
+// Backward: dx = w * dy, and per parameter element the partial sums of dy * x and dy
+// over slice blockIdx.y of its elements: part[(m * S + s) * 2 + {0, 1}].
+template <typename T>
+__global__ void __launch_bounds__(256)
+affine_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ w,
+                  T* __restrict__ dx, float* __restrict__ part, long long per, long long chunk,
+                  long long mid, long long inner, int S) {
+  __shared__ float red[4];
+  const long long m = blockIdx.x, s = blockIdx.y;
+  const long long j0 = s * chunk, j1 = min(j0 + chunk, per);
+  const float wm = w ? ld(w, (size_t)m) : 0.f;
+  float s1 = 0.f, s2 = 0.f;
+  for (long long j = j0 + threadIdx.x; j < j1; j += 256) {
+    const long long o = j / inner, i = j - o * inner;
+    const size_t e = (size_t)((o * mid + m) * inner + i);
+    const float d = ld(dy, e);
+    if (part) {
+      s1 += d * ld(x, e);
+      s2 += d;
+    }
+    if (dx) st(dx, e, wm * d);
+  }
+  if (!part) return;
+  s1 = block_sum(s1, red);
+  s2 = block_sum(s2, red);
+  if (threadIdx.x == 0) {
+    part[(m * S + s) * 2 + 0] = s1;
+    part[(m * S + s) * 2 + 1] = s2;
+  }
+}
+
+__global__ void __launch_bounds__(256)
+affine_fold_kernel(const float* __restrict__ part, float* __restrict__ dw, float* __restrict__ db,
+                   long long nparam, int S) {
+  const long long m = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (m >= nparam) return;
+  double a = 0.0, b = 0.0;
+  for (int s = 0; s < S; ++s) {
+    a += (double)part[(m * S + s) * 2 + 0];
+    b += (double)part[(m * S + s) * 2 + 1];
+  }
+  if (dw) dw[m] = (float)a;
+  if (db) db[m] = (float)b;
+}
+
+// slices per parameter element: enough blocks to fill the machine, at least 2048
+// elements each
+struct AffinePlan {
+  long long nparam, per, mid, inner, chunk;
+  int S;
+};
+AffinePlan affine_plan(long long outer, long long mid, long long inner, int scalar) {
+  AffinePlan p;
+  if (scalar) {                        // one parameter element sees the whole tensor
+    p.nparam = 1; p.mid = 1; p.inner = outer * mid * inner; p.per = p.inner;
+  } else {
+    p.nparam = mid; p.mid = mid; p.inner = inner; p.per = outer * inner;
+  }
+  long long S = 4096 / p.nparam;
+  const long long maxS = (p.per + 2047) / 2048;
+  if (S > maxS) S = maxS;
+  if (S > 1024) S = 1024;
+  if (S < 1) S = 1;
+  p.S = (int)S;
+  p.chunk = (p.per + S - 1) / S;
+  return p;
+}
+
 }  // namespace
 }  // namespace flhip
 
@@ -315,4 +398,64 @@ extern "C" int flhip_cce_bwd(const float* grad, const int32_t* target, const flo
                        as_stream(stream), grad, target, stats, (bf16_t*)dx, classes, cols, reduction,
                        ignore_index);
   return check_launch("cce_bwd");
+}
+
+extern "C" int flhip_affine_fwd(const void* x, const void* w, const void* b, void* y, int64_t outer,
+                                int64_t mid, int64_t inner, int scalar_params, int dtype,
+                                void* stream) {
+  FLHIP_REQUIRE(x && w && b && y, "affine: null argument");
+  FLHIP_REQUIRE(outer > 0 && mid > 0 && inner > 0, "affine: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "affine: unknown dtype");
+  const size_t n = (size_t)outer * (size_t)mid * (size_t)inner;
+  if (dtype == FLHIP_F32)
+    hipLaunchKernelGGL((affine_fwd_kernel<float>), dim3(blocks_for(n)), dim3(256), 0,
+                       as_stream(stream), (const float*)x, (const float*)w, (const float*)b,
+                       (float*)y, n, (long long)mid, (long long)inner, scalar_params ? 0 : 1);
+  else
+    hipLaunchKernelGGL((affine_fwd_kernel<bf16_t>), dim3(blocks_for(n)), dim3(256), 0,
+                       as_stream(stream), (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)b,
+                       (bf16_t*)y, n, (long long)mid, (long long)inner, scalar_params ? 0 : 1);
+  return check_launch("affine");
+}
+
+extern "C" size_t flhip_affine_bwd_workspace_bytes(int64_t outer, int64_t mid, int64_t inner,
+                                                   int scalar_params) {
+  if (outer <= 0 || mid <= 0 || inner <= 0) return 0;
+  const AffinePlan p = affine_plan(outer, mid, inner, scalar_params);
+  return (size_t)p.nparam * (size_t)p.S * 2 * sizeof(float);
+}
+
+extern "C" int flhip_affine_bwd(const void* dy, const void* x, const void* w, void* dx, float* dw,
+                                float* db, int64_t outer, int64_t mid, int64_t inner,
+                                int scalar_params, int dtype, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+  FLHIP_REQUIRE(dy, "affine_bwd: null argument");
+  FLHIP_REQUIRE(outer > 0 && mid > 0 && inner > 0, "affine_bwd: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "affine_bwd: unknown dtype");
+  FLHIP_REQUIRE(!dx || w, "affine_bwd: dx needs the weight");
+  const bool sums = dw || db;
+  FLHIP_REQUIRE(!sums || x, "affine_bwd: the parameter gradients need x");
+  if (!dx && !sums) return FLHIP_OK;
+  const AffinePlan p = affine_plan(outer, mid, inner, scalar_params);
+  FLHIP_REQUIRE(p.nparam <= 0x7fffffffLL, "affine_bwd: too many parameter elements");
+  if (sums)
+    FLHIP_REQUIRE(workspace && workspace_bytes >= (size_t)p.nparam * (size_t)p.S * 2 * sizeof(float),
+                  "affine_bwd: workspace too small");
+  float* part = sums ? static_cast<float*>(workspace) : nullptr;
+  const dim3 grid((unsigned)p.nparam, (unsigned)p.S);
+  if (dtype == FLHIP_F32)
+    hipLaunchKernelGGL((affine_bwd_kernel<float>), grid, dim3(256), 0, as_stream(stream),
+                       (const float*)dy, (const float*)x, (const float*)w, (float*)dx, part, p.per,
+                       p.chunk, p.mid, p.inner, p.S);
+  else
+    hipLaunchKernelGGL((affine_bwd_kernel<bf16_t>), grid, dim3(256), 0, as_stream(stream),
+                       (const bf16_t*)dy, (const bf16_t*)x, (const bf16_t*)w, (bf16_t*)dx, part,
+                       p.per, p.chunk, p.mid, p.inner, p.S);
+  if (const int rc = check_launch("affine_bwd")) return rc;
+  if (sums) {
+    hipLaunchKernelGGL(affine_fold_kernel, dim3((unsigned)((p.nparam + 255) / 256)), dim3(256), 0,
+                       as_stream(stream), part, dw, db, p.nparam, p.S);
+    return check_launch("affine_bwd (fold)");
+  }
+  return FLHIP_OK;
 }

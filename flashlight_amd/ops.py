@@ -377,3 +377,97 @@ def categorical_cross_entropy_backward(grad_output, input_shape, dtype, targets,
     capi.check(capi.lib().flhip_cce_bwd(_ptr(g), _ptr(t), _ptr(stats), _ptr(dx), classes, t.numel(),
                                         reduction, ignore_index, tag, _stream()))
     return dx
+
+
+# ---- LayerNorm = batchnorm over the complement axes + broadcast scale and shift -------
+def _affine_view(whcn, norm_axes, nparam):
+    """(outer, mid, inner, scalar) of the parameter broadcast of LayerNorm.cpp:110-126:
+    one element, or one per position along the (contiguous) normalised axes."""
+    if nparam == 1:
+        return 1, 1, 1, True
+    axes = sorted(norm_axes)
+    if axes != list(range(axes[0], axes[-1] + 1)):
+        raise ValueError("LayerNorm: per-element parameters need contiguous normalised axes")
+    mid = inner = outer = 1
+    for d, s in enumerate(whcn):
+        if d < axes[0]:
+            inner *= s
+        elif d <= axes[-1]:
+            mid *= s
+        else:
+            outer *= s
+    if mid != nparam:
+        raise ValueError("[LayerNorm] Input size along the norm axis doesn't with axisSize.")
+    return outer, mid, inner, False
+
+
+def affine(input, weight, bias, view):
+    """y = tileAs(weight) * input + tileAs(bias) on the [outer][mid][inner] view."""
+    x = _dev(input, "input")
+    outer, mid, inner, scalar = view
+    if scalar:
+        outer, mid, inner = 1, 1, x.numel()
+    w, b = _dev(weight, "weight").to(x.dtype), _dev(bias, "bias").to(x.dtype)
+    y = torch.empty_like(x)
+    capi.check(capi.lib().flhip_affine_fwd(_ptr(x), _ptr(w), _ptr(b), _ptr(y), outer, mid, inner,
+                                           int(scalar), _dtype_tag(x), _stream()))
+    return y
+
+
+def affine_backward(grad_output, input, weight, view):
+    """-> (gradInput, gradWeight fp32, gradBias fp32) of `affine`."""
+    g, x = _dev(grad_output, "gradOutput"), _dev(input, "input")
+    outer, mid, inner, scalar = view
+    if scalar:
+        outer, mid, inner = 1, 1, x.numel()
+    w = _dev(weight, "weight").to(x.dtype)
+    n = 1 if scalar else mid
+    dx = torch.empty_like(x)
+    dw = torch.empty((n,), dtype=torch.float32, device=x.device)
+    db = torch.empty((n,), dtype=torch.float32, device=x.device)
+    nws = capi.lib().flhip_affine_bwd_workspace_bytes(outer, mid, inner, int(scalar))
+    ws = _ws(nws, x.device)
+    capi.check(capi.lib().flhip_affine_bwd(_ptr(g), _ptr(x), _ptr(w), _ptr(dx), _ptr(dw), _ptr(db),
+                                           outer, mid, inner, int(scalar), _dtype_tag(x), _ptr(ws),
+                                           nws, _stream()))
+    return dx, dw, db
+
+
+def _layer_norm_axes(shape, norm_axes):
+    whcn = list(shape)[::-1]
+    if len(whcn) > 4:
+        raise ValueError("LayerNorm::forward - input must be 4 or fewer dimensions.")
+    whcn += [1] * (4 - len(whcn))
+    norm = sorted(int(a) for a in norm_axes)
+    comp = [d for d in range(4) if d not in norm]
+    if not comp or comp != list(range(comp[0], comp[-1] + 1)):
+        raise ValueError("LayerNorm: a non-contiguous axis complement needs a reorder, "
+                         "which this backend does not provide")
+    return whcn, norm, comp
+
+
+def layer_norm(input, norm_axes, epsilon=1e-5, weight=None, bias=None):
+    """fl::LayerNorm::forward (nn/modules/LayerNorm.cpp:42-131): batchnorm in train mode
+    over the complement of the normalised axes with no parameters and no running
+    statistics, then the broadcast scale and shift.  -> (output, ctx for the backward)."""
+    x = _dev(input, "input")
+    whcn, norm, comp = _layer_norm_axes(x.shape, norm_axes)
+    x4 = x.reshape(whcn[::-1])
+    xhat, sm, si = batchnorm(x4, None, None, None, None, comp, True, 0.0, epsilon)
+    ctx = {"x4": x4, "xhat": xhat, "sm": sm, "si": si, "comp": comp, "view": None}
+    out = xhat
+    if weight is not None:
+        ctx["view"] = _affine_view(whcn, norm, weight.numel())
+        out = affine(xhat, weight, bias, ctx["view"])
+    return out.reshape(x.shape), ctx
+
+
+def layer_norm_backward(grad_output, ctx, weight=None):
+    """-> (gradInput, gradWeight, gradBias) of `layer_norm` (the last two None without
+    parameters)."""
+    g = _dev(grad_output, "gradOutput").reshape(ctx["x4"].shape)
+    dw = db = None
+    if ctx["view"] is not None:
+        g, dw, db = affine_backward(g, ctx["xhat"], weight, ctx["view"])
+    dx, _, _ = batchnorm_backward(g, ctx["x4"], None, ctx["sm"], ctx["si"], ctx["comp"])
+    return dx.reshape(grad_output.shape), dw, db

@@ -221,6 +221,25 @@ int flhip_matmul(const void* A, const void* B, void* C, int32_t M, int32_t N,
 int flhip_sum_columns(const void* x, float* out, int32_t rows, int32_t cols, int dtype,
                       void* stream);
 
+/* The affine part of fl::LayerNorm (flashlight/fl/nn/modules/LayerNorm.cpp:110-128),
+ * tileAs(weight, input) * output + tileAs(bias, input), on a tensor viewed as
+ * [outer][mid][inner] (inner fastest): y = w[m] * x + b[m] with one parameter element
+ * per mid index, or a single element when scalar_params != 0.  w and b have the
+ * tensor's dtype. */
+int flhip_affine_fwd(const void* x, const void* w, const void* b, void* y, int64_t outer,
+                     int64_t mid, int64_t inner, int scalar_params, int dtype,
+                     void* stream);
+/* Its backward: dx = w * dy (skipped when dx is NULL), dw[m] = sum of dy * x and
+ * db[m] = sum of dy over the elements that share parameter m (fp32, either may be
+ * NULL).  The sums are two-stage with a fixed order; the workspace holds the
+ * partials and is needed only when dw or db is asked for. */
+size_t flhip_affine_bwd_workspace_bytes(int64_t outer, int64_t mid, int64_t inner,
+                                        int scalar_params);
+int flhip_affine_bwd(const void* dy, const void* x, const void* w, void* dx, float* dw,
+                     float* db, int64_t outer, int64_t mid, int64_t inner,
+                     int scalar_params, int dtype, void* workspace,
+                     size_t workspace_bytes, void* stream);
+
 /* fl::logSoftmax over dimension 0 of a classes x cols matrix (Functions.cpp:1044-1070)
  * and its backward dx = dy - exp(y) * sum over classes of dy. */
 int flhip_logsoftmax_fwd(const void* x, void* y, int32_t classes, int32_t cols,

@@ -425,6 +425,36 @@ void flref_sum_columns(int rows, int cols, const float* x, float* out) {
   }
 }
 
+/* LayerNorm.cpp:110-128: the parameter element of (o, m, i) is m, or 0 when scalar */
+void flref_affine_fwd(int64_t outer, int64_t mid, int64_t inner, int scalar, const float* x,
+                      const float* w, const float* b, float* y) {
+  for (int64_t o = 0; o < outer; ++o)
+    for (int64_t m = 0; m < mid; ++m)
+      for (int64_t i = 0; i < inner; ++i) {
+        const int64_t e = (o * mid + m) * inner + i, pm = scalar ? 0 : m;
+        y[e] = (float)((double)w[pm] * x[e] + b[pm]);
+      }
+}
+
+void flref_affine_bwd(int64_t outer, int64_t mid, int64_t inner, int scalar, const float* dy,
+                      const float* x, const float* w, float* dx, float* dw, float* db) {
+  const int64_t np = scalar ? 1 : mid;
+  double* acc = (double*)calloc((size_t)np * 2, sizeof(double));
+  for (int64_t o = 0; o < outer; ++o)
+    for (int64_t m = 0; m < mid; ++m)
+      for (int64_t i = 0; i < inner; ++i) {
+        const int64_t e = (o * mid + m) * inner + i, pm = scalar ? 0 : m;
+        if (dx) dx[e] = w[pm] * dy[e];
+        acc[2 * pm] += (double)dy[e] * x[e];
+        acc[2 * pm + 1] += dy[e];
+      }
+  for (int64_t m = 0; m < np; ++m) {
+    if (dw) dw[m] = (float)acc[2 * m];
+    if (db) db[m] = (float)acc[2 * m + 1];
+  }
+  free(acc);
+}
+
 /* x - (log(sum(exp(x - max))) + max) per column (:1046-1056) */
 void flref_logsoftmax_fwd(int classes, int cols, const float* x, float* y) {
   for (int c = 0; c < cols; ++c) {

@@ -100,6 +100,16 @@ void flref_matmul(int M, int N, int K, int ta, int tb, const float* A, const flo
                   const float* bias, float* C);
 /* out[r] = sum_c x[r, c] (sumAs(gradOutput, bias), :1285-1289) */
 void flref_sum_columns(int rows, int cols, const float* x, float* out);
+
+/* Affine part of fl::LayerNorm (flashlight/fl/nn/modules/LayerNorm.cpp:110-128):
+ * y = tileAs(w) * x + tileAs(b) on a tensor viewed as [outer][mid][inner]; the
+ * parameters have `mid` elements, or one when scalar != 0.  Backward: dx = w * dy,
+ * dw = sum of dy * x and db = sum of dy over the tiled dimensions (the gradients of
+ * the broadcast multiply and add). */
+void flref_affine_fwd(int64_t outer, int64_t mid, int64_t inner, int scalar, const float* x,
+                      const float* w, const float* b, float* y);
+void flref_affine_bwd(int64_t outer, int64_t mid, int64_t inner, int scalar, const float* dy,
+                      const float* x, const float* w, float* dx, float* dw, float* db);
 /* logSoftmax over dimension 0 of a classes x cols matrix (:1044-1070) */
 void flref_logsoftmax_fwd(int classes, int cols, const float* x, float* y);
 void flref_logsoftmax_bwd(int classes, int cols, const float* dy, const float* y, float* dx);

@@ -215,6 +215,25 @@ def sum_columns(rows, cols, x):
     return out
 
 
+def affine_fwd(outer, mid, inner, scalar, x, w, b):
+    x, w, b = _f32(x), _f32(w), _f32(b)
+    y = np.empty_like(x)
+    lib().flref_affine_fwd(_i64(outer), _i64(mid), _i64(inner), C.c_int(int(scalar)), _p(x), _p(w),
+                           _p(b), _p(y))
+    return y
+
+
+def affine_bwd(outer, mid, inner, scalar, dy, x, w):
+    """-> (dx, dw, db)"""
+    dy, x, w = _f32(dy), _f32(x), _f32(w)
+    n = 1 if scalar else mid
+    dx = np.empty_like(x)
+    dw, db = np.empty((n,), np.float32), np.empty((n,), np.float32)
+    lib().flref_affine_bwd(_i64(outer), _i64(mid), _i64(inner), C.c_int(int(scalar)), _p(dy), _p(x),
+                           _p(w), _p(dx), _p(dw), _p(db))
+    return dx, dw, db
+
+
 def logsoftmax_fwd(x):
     """x: numpy [cols, classes] (Flashlight [classes, cols])."""
     x = _f32(x)
@@ -251,3 +270,45 @@ def cce_bwd(shape, grad, target, count, reduction=1, ignore=-1):
     lib().flref_cce_bwd(C.c_int(shape[-1]), C.c_int(t.size), _p(g), t.ctypes.data_as(C.c_void_p),
                         C.c_int(ignore), C.c_int(reduction), C.c_float(count), _p(dx))
     return dx
+
+
+# ---- fl::LayerNorm::forward (flashlight/fl/nn/modules/LayerNorm.cpp:42-131) restated on
+# the functions above: the shape is padded to 4 dimensions, batchnorm runs in train mode
+# over the complement of the normalised axes with no parameters, then the broadcast
+# scale and shift.  Only a contiguous complement is restated (the other case reorders).
+def layer_norm_plan(shape_whcn, norm_axes, nparam):
+    whcn = list(shape_whcn) + [1] * (4 - len(shape_whcn))
+    norm = sorted(norm_axes)
+    comp = [d for d in range(4) if d not in norm]
+    if comp != list(range(comp[0], comp[-1] + 1)):
+        raise ValueError("non-contiguous complement")
+    view = None
+    if nparam == 1:
+        view = (1, 1, int(np.prod(whcn)), True)
+    elif nparam:
+        inner = int(np.prod(whcn[:norm[0]]))
+        mid = int(np.prod(whcn[norm[0]:norm[-1] + 1]))
+        outer = int(np.prod(whcn[norm[-1] + 1:]))
+        assert mid == nparam and norm == list(range(norm[0], norm[-1] + 1))
+        view = (outer, mid, inner, False)
+    return bn_view(whcn, comp), view
+
+
+def layer_norm_fwd(x, shape_whcn, norm_axes, eps, w=None, b=None):
+    """-> (y, xhat, mean, var); x is the flat/any-shape array of the tensor's memory."""
+    bnv, view = layer_norm_plan(shape_whcn, norm_axes, 0 if w is None else np.size(w))
+    ones, zeros = np.ones(bnv[1], np.float32), np.zeros(bnv[1], np.float32)
+    xhat, mean, var = bn_fwd_train(*bnv, x, ones, zeros, eps)
+    y = xhat if w is None else affine_fwd(*view, xhat, w, b)
+    return y, xhat, mean, var
+
+
+def layer_norm_bwd(dy, x, xhat, mean, var, shape_whcn, norm_axes, eps, w=None):
+    """-> (dx, dw, db)"""
+    bnv, view = layer_norm_plan(shape_whcn, norm_axes, 0 if w is None else np.size(w))
+    dw = db = None
+    g = dy
+    if w is not None:
+        g, dw, db = affine_bwd(*view, dy, xhat, w)
+    dx, _, _ = bn_bwd(*bnv, x, g, np.ones(bnv[1], np.float32), mean, var, eps)
+    return dx, dw, db

@@ -101,6 +101,75 @@ def _mnist_params(rng):
                 w3=ku((3136, 1024), 3136), b3=bu(1024, 3136), w4=ku((1024, 10), 1024), b4=bu(10, 1024))
 
 
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("outer,mid,inner,scalar", [(3, 5, 7, False), (1, 600, 1, False), (40, 9, 1, False),
+                                                    (1, 8, 5000, False), (2, 3, 4, True),
+                                                    (1, 1, 300000, True), (64, 512, 1, False)])
+def test_affine(outer, mid, inner, scalar, dtype):
+    rng = np.random.default_rng(outer + mid + inner)
+    x = _round(rng.standard_normal((outer, mid, inner)).astype(np.float32), dtype)
+    dy = _round(rng.standard_normal((outer, mid, inner)).astype(np.float32), dtype)
+    n = 1 if scalar else mid
+    w = _round(rng.standard_normal(n).astype(np.float32), dtype)
+    b = _round(rng.standard_normal(n).astype(np.float32), dtype)
+    view = (outer, mid, inner, scalar)
+    tol = _tol(dtype)
+    y = ops.affine(dev(x, dtype), dev(w, dtype), dev(b, dtype), view)
+    assert rel_l2(host(y), flref.affine_fwd(outer, mid, inner, scalar, x, w, b)) <= tol
+    dx, dw, db = ops.affine_backward(dev(dy, dtype), dev(x, dtype), dev(w, dtype), view)
+    rdx, rdw, rdb = flref.affine_bwd(outer, mid, inner, scalar, dy, x, w)
+    assert rel_l2(host(dx), rdx) <= tol
+    # the sums accumulate in fp32 whatever the storage type
+    assert rel_l2(host(dw), rdw) <= 1e-4 and rel_l2(host(db), rdb) <= 1e-4
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("whcn,norm,params", [
+    ((6, 5, 4, 3), (0, 1, 2), "per"),        # LayerNorm over {0,1,2} of WHCN
+    ((6, 5, 4, 3), (0, 1, 2), "scalar"),
+    ((512, 50, 8), (0,), "per"),             # [C, T, B], normalise C
+    ((512, 50, 8), (0,), None),
+    ((20, 4, 3, 16), (3,), "per"),
+    ((56, 56, 64, 4), (0, 1, 2), "per"),
+])
+def test_layer_norm(whcn, norm, params, dtype):
+    # fl::LayerNorm::forward (nn/modules/LayerNorm.cpp:42-131) = the extension's batchnorm
+    # over the complement axes + the broadcast scale and shift
+    rng = np.random.default_rng(sum(whcn) + len(norm))
+    tshape = tuple(whcn[::-1])
+    x = _round((rng.standard_normal(tshape) * 2 + 0.5).astype(np.float32), dtype)
+    dy = _round(rng.standard_normal(tshape).astype(np.float32), dtype)
+    w = b = None
+    if params == "per":
+        n = int(np.prod([whcn[a] for a in norm]))
+        w = _round(rng.standard_normal(n).astype(np.float32), dtype)
+        b = _round(rng.standard_normal(n).astype(np.float32), dtype)
+    elif params == "scalar":
+        w, b = _round(np.array([1.7], np.float32), dtype), _round(np.array([-0.3], np.float32), dtype)
+    eps = 1e-5
+    ry, rxhat, rmean, rvar = flref.layer_norm_fwd(x, whcn, norm, eps, w, b)
+    rdx, rdw, rdb = flref.layer_norm_bwd(dy, x, rxhat, rmean, rvar, whcn, norm, eps, w)
+    dw_ = None if w is None else dev(w, dtype)
+    db_ = None if b is None else dev(b, dtype)
+    y, ctx = ops.layer_norm(dev(x, dtype), norm, eps, dw_, db_)
+    tol = _tol(dtype)
+    assert tuple(y.shape) == tshape
+    assert rel_l2(host(y), ry.reshape(tshape)) <= tol
+    dx, dw, db = ops.layer_norm_backward(dev(dy, dtype), ctx, dw_)
+    assert rel_l2(host(dx), rdx.reshape(tshape)) <= (1e-4 if dtype == torch.float32 else 3e-2)
+    if w is not None:
+        assert rel_l2(host(dw), rdw) <= tol and rel_l2(host(db), rdb) <= tol
+
+
+def test_layer_norm_needs_contiguous_complement():
+    x = dev(np.zeros((2, 3, 4, 5), np.float32))
+    with pytest.raises(ValueError):
+        ops.layer_norm(x, (0, 2))
+    with pytest.raises(ValueError):
+        ops.layer_norm(dev(np.zeros((2, 2, 2, 2, 2), np.float32)), (0,))
+
+
+
 def test_mnist_convnet_training_step():
     """configs[0]: View, Conv2D 1->32 5x5 SAME, ReLU, Pool2D max 2x2 s2, Conv2D 32->64 5x5
     SAME, ReLU, Pool2D, View, Linear 3136->1024, ReLU, Linear 1024->10, LogSoftmax, then

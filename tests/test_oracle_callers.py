@@ -102,3 +102,77 @@ def test_cross_entropy_like_torch(reduction):
 def test_cross_entropy_flags_bad_targets():
     logp = np.zeros((4, 3), np.float32)
     assert flref.cce_fwd(logp, np.array([0, 3, 2, -2], np.int32))[4] == 2
+
+
+@pytest.mark.parametrize("outer,mid,inner,scalar", [(3, 5, 7, False), (1, 6, 1, False), (4, 9, 1, False),
+                                                    (1, 8, 5, False), (2, 3, 4, True)])
+def test_affine_against_numpy_broadcast(outer, mid, inner, scalar):
+    # tileAs(weight) * x + tileAs(bias) and the gradients of the broadcasts
+    # (LayerNorm.cpp:110-128), written with numpy broadcasting in float64
+    rng = np.random.default_rng(outer * 100 + mid * 10 + inner)
+    x = rng.standard_normal((outer, mid, inner)).astype(np.float32)
+    dy = rng.standard_normal((outer, mid, inner)).astype(np.float32)
+    n = 1 if scalar else mid
+    w, b = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    wb = w.astype(np.float64).reshape(1, n, 1)
+    bb = b.astype(np.float64).reshape(1, n, 1)
+    y = flref.affine_fwd(outer, mid, inner, scalar, x, w, b)
+    assert rel_l2(y, wb * x + bb) < 1e-6
+    dx, dw, db = flref.affine_bwd(outer, mid, inner, scalar, dy, x, w)
+    assert rel_l2(dx, wb * dy) < 1e-6
+    red = (0, 1, 2) if scalar else (0, 2)
+    assert rel_l2(dw, (dy.astype(np.float64) * x).sum(axis=red).reshape(-1)) < 1e-6
+    assert rel_l2(db, dy.astype(np.float64).sum(axis=red).reshape(-1)) < 1e-6
+
+
+@pytest.mark.parametrize("whcn,norm,params", [
+    ((6, 5, 4, 3), (0, 1, 2), "per"),      # the reference's LayerNorm test: axes {0,1,2} of WHCN
+    ((6, 5, 4, 3), (0, 1, 2), "scalar"),
+    ((16, 7, 3), (0,), "per"),             # transformer use: [C, T, B], normalise C
+    ((16, 7, 3), (0,), None),
+    ((5, 4, 3, 2), (3,), "per"),
+    ((8, 3), (0, 1), "scalar"),
+])
+def test_layer_norm_restated_on_batchnorm_is_layer_norm(whcn, norm, params):
+    # LayerNorm.cpp:42-131 against torch.nn.functional.layer_norm (float64) and its autograd
+    rng = np.random.default_rng(sum(whcn) + len(norm))
+    tshape = tuple(whcn[::-1])                       # torch shape = reversed Flashlight shape
+    x = (rng.standard_normal(tshape) * 2 + 0.5).astype(np.float32)
+    dy = rng.standard_normal(tshape).astype(np.float32)
+    w = b = None
+    norm_t = sorted(len(whcn) - 1 - a for a in norm)    # torch dims that are normalised
+    nshape = [whcn[a] for a in sorted(norm)][::-1]
+    if params == "per":
+        w = rng.standard_normal(int(np.prod(nshape))).astype(np.float32)
+        b = rng.standard_normal(int(np.prod(nshape))).astype(np.float32)
+    elif params == "scalar":
+        w, b = np.array([1.7], np.float32), np.array([-0.3], np.float32)
+    eps = 1e-5
+    y, xhat, mean, var = flref.layer_norm_fwd(x, whcn, norm, eps, w, b)
+    dx, dw, db = flref.layer_norm_bwd(dy, x, xhat, mean, var, whcn, norm, eps, w)
+    # torch: move the normalised dims last (they are contiguous here), normalise, move back
+    xt = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+    keep = [d for d in range(len(tshape)) if d not in norm_t]
+    perm = keep + norm_t
+    xp = xt.permute(perm)
+    yp = F.layer_norm(xp, xp.shape[len(keep):], eps=eps)
+    inv = [perm.index(d) for d in range(len(tshape))]
+    yt = yp.permute(inv)
+    params_t = []
+    if params == "per":
+        bshape = [tshape[d] if d in norm_t else 1 for d in range(len(tshape))]
+        wt = torch.tensor(w, dtype=torch.float64, requires_grad=True)
+        bt = torch.tensor(b, dtype=torch.float64, requires_grad=True)
+        yt = yt * wt.reshape(bshape) + bt.reshape(bshape)
+        params_t = [wt, bt]
+    elif params == "scalar":
+        wt = torch.tensor(w, dtype=torch.float64, requires_grad=True)
+        bt = torch.tensor(b, dtype=torch.float64, requires_grad=True)
+        yt = yt * wt + bt
+        params_t = [wt, bt]
+    yt.backward(torch.tensor(dy, dtype=torch.float64))
+    assert rel_l2(y.reshape(tshape), yt.detach().numpy()) < 1e-5
+    assert rel_l2(dx.reshape(tshape), xt.grad.numpy()) < 1e-4
+    if params_t:
+        assert rel_l2(dw, params_t[0].grad.numpy().reshape(-1)) < 1e-5
+        assert rel_l2(db, params_t[1].grad.numpy().reshape(-1)) < 1e-5
