@@ -51,6 +51,24 @@ void Variable::addGrad(const Variable& childGrad) {
   grad_->grad.reset(new Variable(sum, false));
 }
 
+void Variable::setCalcGrad(bool calcGrad) {
+  grad_->calcGrad = calcGrad;
+  if (!calcGrad) {
+    grad_->gradFunc = nullptr;
+    grad_->inputs.clear();
+    grad_->grad.reset();
+  }
+}
+
+Variable Variable::astype(dtype newType) const {
+  if (newType == type()) return *this;
+  const dtype oldType = type();
+  auto gradFunc = [oldType](std::vector<Variable>& inputs, const Variable& gradOutput) {
+    inputs[0].addGrad(Variable(gradOutput.tensor().astype(oldType), false));
+  };
+  return Variable(tensor().astype(newType), {*this}, gradFunc);
+}
+
 std::vector<Variable> Variable::build() const {
   // depth-first post order = topological order (Variable.cpp:274-294)
   std::unordered_set<SharedGrad*> seen;
@@ -162,7 +180,11 @@ Variable pool2d(const Variable& input, int wx, int wy, int sx, int sy, int px, i
 Variable batchnorm(const Variable& input, const Variable& weight, const Variable& bias,
                    Variable& runningMean, Variable& runningVar, const std::vector<int>& axes,
                    bool train, double momentum, double epsilon) {
-  dtypesMatch("batchnorm", {&input, &weight, &bias});
+  // the BatchNorm and LayerNorm modules keep f32 parameters for 16-bit inputs
+  // (flashlight/fl/nn/modules/BatchNorm.cpp:86-88), so f32 is accepted beside the input type
+  for (const Variable* v : {&weight, &bias})
+    if (!v->isEmpty() && v->type() != input.type() && v->type() != dtype::f32)
+      throw std::invalid_argument("batchnorm: parameters must have the input's type or f32");
   auto payload = createPayload({&input, &weight, &bias});
   auto saveMean = std::make_shared<Tensor>();
   auto saveVar = std::make_shared<Tensor>();
@@ -196,6 +218,53 @@ void check(int rc) {
   if (rc != FLHIP_OK) throw std::runtime_error(flhip_last_error());
 }
 }  // namespace
+
+Variable add(const Variable& lhs, const Variable& rhs) {
+  dtypesMatch("add", {&lhs, &rhs});
+  if (lhs.shape() != rhs.shape())
+    throw std::invalid_argument("add: shapes must match (no broadcasting on this backend)");
+  const int tag = tagOf(lhs.type(), "add");
+  Tensor out(lhs.shape(), lhs.type());
+  check(flhip_add(lhs.tensor().device(), rhs.tensor().device(), out.device(), (size_t)out.elements(), tag,
+                  hipBackendStream()));
+  auto gradFunc = [](std::vector<Variable>& inputs, const Variable& gradOutput) {
+    inputs[0].addGrad(Variable(gradOutput.tensor(), false));
+    inputs[1].addGrad(Variable(gradOutput.tensor(), false));
+  };
+  return Variable(out, {lhs, rhs}, gradFunc);
+}
+
+Variable detail::affine(const Variable& input, const Variable& weight, const Variable& bias, Dim outer,
+                        Dim mid, Dim inner, bool scalar) {
+  dtypesMatch("affine", {&input, &weight, &bias});
+  if (outer * mid * inner != input.elements() || weight.elements() != (scalar ? 1 : mid) ||
+      bias.elements() != weight.elements())
+    throw std::invalid_argument("affine: the view or the parameters do not match the input");
+  const int tag = tagOf(input.type(), "affine");
+  Tensor out(input.shape(), input.type());
+  check(flhip_affine_fwd(input.tensor().device(), weight.tensor().device(), bias.tensor().device(),
+                         out.device(), outer, mid, inner, scalar ? 1 : 0, tag, hipBackendStream()));
+  auto gradFunc = [outer, mid, inner, scalar, tag](std::vector<Variable>& inputs,
+                                                   const Variable& gradOutput) {
+    auto& x = inputs[0];
+    auto& w = inputs[1];
+    auto& b = inputs[2];
+    const bool sums = w.isCalcGrad() || b.isCalcGrad();
+    Tensor dx = x.isCalcGrad() ? Tensor(x.shape(), x.type()) : Tensor();
+    Tensor dw = sums ? Tensor(w.shape(), dtype::f32) : Tensor();
+    Tensor db = sums ? Tensor(b.shape(), dtype::f32) : Tensor();
+    const size_t wsBytes = sums ? flhip_affine_bwd_workspace_bytes(outer, mid, inner, scalar ? 1 : 0) : 0;
+    Tensor ws = wsBytes ? Tensor({(Dim)wsBytes}, dtype::u8) : Tensor();
+    check(flhip_affine_bwd(gradOutput.tensor().device(), x.tensor().device(), w.tensor().device(),
+                           dx.device(), static_cast<float*>(dw.device()),
+                           static_cast<float*>(db.device()), outer, mid, inner, scalar ? 1 : 0, tag,
+                           ws.device(), wsBytes, hipBackendStream()));
+    if (x.isCalcGrad()) x.addGrad(Variable(dx, false));
+    if (w.isCalcGrad()) w.addGrad(Variable(dw.astype(w.type()), false));
+    if (b.isCalcGrad()) b.addGrad(Variable(db.astype(b.type()), false));
+  };
+  return Variable(out, {input, weight, bias}, gradFunc);
+}
 
 Variable relu(const Variable& input) {
   Tensor out(input.shape(), input.type());

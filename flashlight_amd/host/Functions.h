@@ -28,7 +28,14 @@ class Variable {
   const Shape& shape() const { return data_->shape(); }
   dtype type() const { return data_->type(); }
   bool isEmpty() const { return data_->isEmpty(); }
+  int ndim() const { return data_->ndim(); }
+  Dim dim(int i) const { return data_->dim(i); }
+  Dim elements() const { return data_->elements(); }
   bool isCalcGrad() const { return grad_->calcGrad; }
+  // flashlight/fl/autograd/Variable.cpp:155-163: switching off also drops the graph
+  void setCalcGrad(bool calcGrad);
+  // differentiable cast (Variable.cpp:100-108); f32 <-> bf16 here
+  Variable astype(dtype type) const;
   bool isGradAvailable() const { return grad_->grad != nullptr; }
   Variable& grad() const;
   void addGrad(const Variable& childGrad);
@@ -62,6 +69,17 @@ Variable batchnorm(const Variable& input, const Variable& weight, const Variable
 
 // flashlight/fl/common/Defines.h:83-87
 enum class ReduceMode { NONE = 0, MEAN = 1, SUM = 2 };
+
+// input + other, same shapes (the residual add; Functions.cpp:111-121)
+Variable add(const Variable& lhs, const Variable& rhs);
+inline Variable operator+(const Variable& lhs, const Variable& rhs) { return add(lhs, rhs); }
+namespace detail {
+// tileAs(weight, input) * input + tileAs(bias, input) on the [outer][mid][inner] view of
+// the input, one parameter element per mid index or a single one (scalar): the affine
+// part of LayerNorm (flashlight/fl/nn/modules/LayerNorm.cpp:110-128)
+Variable affine(const Variable& input, const Variable& weight, const Variable& bias, Dim outer,
+                Dim mid, Dim inner, bool scalar);
+}  // namespace detail
 
 // fl::relu = max(input, 0) (Functions.cpp:329-338, 1787-1789)
 Variable relu(const Variable& input);

@@ -1,0 +1,344 @@
+#include "Modules.h"
+
+#include <algorithm>
+#include <cmath>
+#include <random>
+#include <sstream>
+
+namespace fl {
+
+// ---- initialisation --------------------------------------------------------------------
+namespace {
+std::mt19937_64& generator() {
+  static std::mt19937_64 gen(0);
+  return gen;
+}
+Tensor fromFloats(const Shape& shape, dtype type, const std::vector<float>& v) {
+  if (type != dtype::f32 && type != dtype::bf16)
+    throw std::invalid_argument("initialisation: f32 and bf16 only");
+  Tensor t = Tensor::fromVector(shape, v);
+  return type == dtype::f32 ? t : t.astype(type);
+}
+}  // namespace
+
+void setSeed(unsigned long long seed) { generator().seed(seed); }
+
+Variable constant(double val, const Shape& shape, dtype type, bool calcGrad) {
+  return Variable(fromFloats(shape, type, std::vector<float>((size_t)shape.elements(), (float)val)),
+                  calcGrad);
+}
+
+Variable uniform(const Shape& shape, double min, double max, dtype type, bool calcGrad) {
+  // (max - min) * rand + min (Init.cpp:22-26)
+  std::uniform_real_distribution<double> d(0.0, 1.0);
+  std::vector<float> v((size_t)shape.elements());
+  for (auto& x : v) x = (float)((max - min) * d(generator()) + min);
+  return Variable(fromFloats(shape, type, v), calcGrad);
+}
+
+Variable kaimingUniform(const Shape& shape, int fanIn, dtype type, bool calcGrad) {
+  // Init.cpp:33-40
+  const double stdv = std::sqrt(1.0 / (double)fanIn);
+  const double limit = std::sqrt(3.0) * stdv;
+  return uniform(shape, -limit, limit, type, calcGrad);
+}
+
+// ---- Module ----------------------------------------------------------------------------
+Variable Module::param(int position) const {
+  if (!(position >= 0 && position < (int)params_.size()))
+    throw std::out_of_range("Module param index out of range");
+  return params_[position];
+}
+
+void Module::setParams(const Variable& var, int position) {
+  if (!(position >= 0 && position < (int)params_.size()))
+    throw std::out_of_range("Module param index out of range");
+  params_[position] = var;
+}
+
+void Module::train() {
+  train_ = true;
+  for (auto& p : params_) p.setCalcGrad(true);
+}
+
+void Module::eval() {
+  train_ = false;
+  for (auto& p : params_) p.setCalcGrad(false);
+}
+
+void Module::zeroGrad() {
+  for (auto& p : params_) p.zeroGrad();
+}
+
+std::vector<Variable> UnaryModule::forward(const std::vector<Variable>& inputs) {
+  if (inputs.size() != 1) throw std::invalid_argument("UnaryModule expects only one input");
+  return {forward(inputs[0])};
+}
+
+std::vector<Variable> BinaryModule::forward(const std::vector<Variable>& inputs) {
+  if (inputs.size() != 2) throw std::invalid_argument("BinaryModule expects two inputs");
+  return {forward(inputs[0], inputs[1])};
+}
+
+// ---- Container / Sequential ---------------------------------------------------------------
+void Container::train() {
+  train_ = true;
+  for (auto& m : modules_) m->train();
+}
+
+void Container::eval() {
+  train_ = false;
+  for (auto& m : modules_) m->eval();
+}
+
+void Container::setParams(const Variable& var, int position) {
+  Module::setParams(var, position);
+  for (const auto& c : childParamIdx_)
+    if (c.position == position) modules_[c.module]->setParams(var, c.index);
+}
+
+std::vector<Variable> Sequential::forward(const std::vector<Variable>& inputs) {
+  auto output = inputs;
+  for (auto& m : modules_) output = m->forward(output);
+  return output;
+}
+
+Variable Sequential::forward(const Variable& input) {
+  std::vector<Variable> output = {input};
+  for (auto& m : modules_) output = m->forward(output);
+  if (output.size() != 1) throw std::invalid_argument("Module output size is not 1");
+  return output.front();
+}
+
+std::string Sequential::prettyString() const {
+  std::ostringstream ss;
+  ss << "Sequential [input";
+  for (size_t i = 0; i < modules_.size(); ++i) ss << " -> (" << i << ")";
+  ss << " -> output]";
+  for (size_t i = 0; i < modules_.size(); ++i) ss << "\n\t(" << i << "): " << modules_[i]->prettyString();
+  return ss.str();
+}
+
+// ---- Conv2D ----------------------------------------------------------------------------
+Conv2D::Conv2D(int nin, int nout, int wx, int wy, int sx, int sy, IntOrPadMode px, IntOrPadMode py,
+               int dx, int dy, bool bias, int groups)
+    : nIn_(nin), nOut_(nout), xFilter_(wx), yFilter_(wy), xStride_(sx), yStride_(sy), xPad_(px.padVal),
+      yPad_(py.padVal), xDilation_(dx), yDilation_(dy), bias_(bias), groups_(groups) {
+  if (groups <= 0 || nin % groups != 0)
+    throw std::invalid_argument("Conv2D: input channels must divide into the groups");
+  const int fanIn = xFilter_ * yFilter_ * nIn_ / groups_;
+  auto wt = kaimingUniform(Shape({xFilter_, yFilter_, nIn_ / groups_, nOut_}), fanIn, dtype::f32, true);
+  if (bias_) {
+    const double bound = std::sqrt(1.0 / fanIn);
+    params_ = {wt, uniform(Shape({1, 1, nOut_, 1}), -bound, bound, dtype::f32, true)};
+  } else {
+    params_ = {wt};
+  }
+}
+
+Conv2D::Conv2D(const Variable& w, int sx, int sy, IntOrPadMode px, IntOrPadMode py, int dx, int dy,
+               int groups)
+    : UnaryModule({w}), nIn_((int)w.dim(2) * groups), nOut_((int)w.dim(3)), xFilter_((int)w.dim(0)),
+      yFilter_((int)w.dim(1)), xStride_(sx), yStride_(sy), xPad_(px.padVal), yPad_(py.padVal),
+      xDilation_(dx), yDilation_(dy), bias_(false), groups_(groups) {}
+
+Conv2D::Conv2D(const Variable& w, const Variable& b, int sx, int sy, IntOrPadMode px, IntOrPadMode py,
+               int dx, int dy, int groups)
+    : UnaryModule({w, b}), nIn_((int)w.dim(2) * groups), nOut_((int)w.dim(3)), xFilter_((int)w.dim(0)),
+      yFilter_((int)w.dim(1)), xStride_(sx), yStride_(sy), xPad_(px.padVal), yPad_(py.padVal),
+      xDilation_(dx), yDilation_(dy), bias_(true), groups_(groups) {
+  if (b.ndim() < 3 || b.dim(2) != w.dim(3))
+    throw std::invalid_argument("output channel dimension mismatch between Conv2D weight and bias");
+  if (b.elements() != b.dim(2))
+    throw std::invalid_argument("only 3rd dimension of Conv2D bias may be non-singleton");
+}
+
+Variable Conv2D::forward(const Variable& input) {
+  const int px = derivePadding((int)input.dim(0), xFilter_, xStride_, xPad_, xDilation_);
+  const int py = derivePadding((int)input.dim(1), yFilter_, yStride_, yPad_, yDilation_);
+  if (!(px >= 0 && py >= 0)) throw std::invalid_argument("invalid padding for Conv2D");
+  if (bias_)
+    return conv2d(input, params_[0].astype(input.type()), params_[1].astype(input.type()), xStride_,
+                  yStride_, px, py, xDilation_, yDilation_, groups_);
+  return conv2d(input, params_[0].astype(input.type()), xStride_, yStride_, px, py, xDilation_,
+                yDilation_, groups_);
+}
+
+namespace {
+std::string padString(int p) {
+  return p == static_cast<int>(PaddingMode::SAME) ? std::string("SAME") : std::to_string(p);
+}
+}  // namespace
+
+std::string Conv2D::prettyString() const {
+  std::ostringstream ss;
+  ss << "Conv2D (" << nIn_ << "->" << nOut_ << ", " << xFilter_ << "x" << yFilter_ << ", " << xStride_
+     << "," << yStride_ << ", " << padString(xPad_) << "," << padString(yPad_) << ", " << xDilation_
+     << ", " << yDilation_ << ")" << (bias_ ? " (with bias)" : " (without bias)");
+  return ss.str();
+}
+
+// ---- Pool2D ----------------------------------------------------------------------------
+Pool2D::Pool2D(int wx, int wy, int sx, int sy, IntOrPadMode px, IntOrPadMode py, PoolingMode mode)
+    : xFilter_(wx), yFilter_(wy), xStride_(sx), yStride_(sy), xPad_(px.padVal), yPad_(py.padVal),
+      mode_(mode) {}
+
+Variable Pool2D::forward(const Variable& input) {
+  const int px = derivePadding((int)input.dim(0), xFilter_, xStride_, xPad_, 1);
+  const int py = derivePadding((int)input.dim(1), yFilter_, yStride_, yPad_, 1);
+  if (!(px >= 0 && py >= 0)) throw std::invalid_argument("invalid padding for Pool2D");
+  return pool2d(input, xFilter_, yFilter_, xStride_, yStride_, px, py, mode_);
+}
+
+std::string Pool2D::prettyString() const {
+  std::ostringstream ss;
+  ss << "Pool2D"
+     << (mode_ == PoolingMode::MAX ? "-max"
+                                   : mode_ == PoolingMode::AVG_EXCLUDE_PADDING ? "-avg(without pad)"
+                                                                               : "-avg(with pad)")
+     << " (" << xFilter_ << "x" << yFilter_ << ", " << xStride_ << "," << yStride_ << ", "
+     << padString(xPad_) << "," << padString(yPad_) << ")";
+  return ss.str();
+}
+
+// ---- BatchNorm -------------------------------------------------------------------------
+BatchNorm::BatchNorm(int featAxis, int featSize, double momentum, double eps, bool affine,
+                     bool trackStats)
+    : BatchNorm(std::vector<int>(1, featAxis), featSize, momentum, eps, affine, trackStats) {}
+
+BatchNorm::BatchNorm(const std::vector<int>& featAxis, int featSize, double momentum, double eps,
+                     bool affine, bool trackStats)
+    : featAxis_(featAxis), featSize_(featSize), momentum_(momentum), epsilon_(eps), affine_(affine),
+      trackStats_(trackStats) {
+  // BatchNorm.cpp:100-112
+  if (trackStats_) {
+    runningMean_ = constant(0.0, Shape({featSize_}), dtype::f32, false);
+    runningVar_ = constant(1.0, Shape({featSize_}), dtype::f32, false);
+  }
+  if (affine_)
+    params_ = {uniform(Shape({featSize_}), 0.0, 1.0, dtype::f32, true),
+               constant(0.0, Shape({featSize_}), dtype::f32, true)};
+}
+
+Variable BatchNorm::forward(const Variable& input) {
+  // BatchNorm.cpp:74-98
+  double avgFactor = 0.0;
+  if (train_ && trackStats_) {
+    ++numBatchesTracked_;
+    avgFactor = momentum_ < 0 ? 1.0 / numBatchesTracked_ : momentum_;
+  }
+  // parameters stay f32 for 16-bit inputs (the reference does this for f16)
+  const Variable none(Tensor(), false);
+  return batchnorm(input, params_.empty() ? none : params_[0], params_.empty() ? none : params_[1],
+                   runningMean_, runningVar_, featAxis_, train_ || !trackStats_, avgFactor, epsilon_);
+}
+
+std::string BatchNorm::prettyString() const {
+  std::ostringstream ss;
+  ss << "BatchNorm ( axis : { ";
+  for (int a : featAxis_) ss << a << " ";
+  ss << "}, size : " << featSize_ << " )";
+  return ss.str();
+}
+
+// ---- LayerNorm -------------------------------------------------------------------------
+namespace {
+constexpr int kLnExpectedNumDims = 4;
+}
+
+LayerNorm::LayerNorm(int axis, double eps, bool affine, int axisSize)
+    : LayerNorm(std::vector<int>({axis}), eps, affine, axisSize) {}
+
+LayerNorm::LayerNorm(const std::vector<int>& axis, double eps, bool affine, int axisSize)
+    : axis_(axis), epsilon_(eps), affine_(affine), axisSize_(axisSize) {
+  for (int d = 0; d < kLnExpectedNumDims; ++d)
+    if (std::find(axis.begin(), axis.end(), d) == axis.end()) axisComplement_.push_back(d);
+  if (axisComplement_.empty()) throw std::invalid_argument("LayerNorm: no axis left to batch over");
+  std::sort(axis_.begin(), axis_.end());
+  if (affine_) {
+    const int paramDim = axisSize_ == kLnVariableAxisSize ? 1 : axisSize_;
+    params_ = {constant(1.0, Shape({paramDim}), dtype::f32, true),
+               constant(0.0, Shape({paramDim}), dtype::f32, true)};
+  }
+}
+
+Variable LayerNorm::forward(const Variable& in) {
+  // LayerNorm.cpp:42-131
+  Variable input = in;
+  if (input.ndim() < kLnExpectedNumDims) {
+    std::vector<Dim> s = in.shape().get();
+    while ((int)s.size() < kLnExpectedNumDims) s.push_back(1);
+    input = moddims(in, Shape(s));
+  } else if (input.ndim() > kLnExpectedNumDims) {
+    throw std::invalid_argument("LayerNorm::forward - input must be " +
+                                std::to_string(kLnExpectedNumDims) + " or fewer dimensions.");
+  }
+  const int maxAxis = *std::max_element(axisComplement_.begin(), axisComplement_.end());
+  const int minAxis = *std::min_element(axisComplement_.begin(), axisComplement_.end());
+  if ((int)axisComplement_.size() != maxAxis - minAxis + 1)
+    throw std::invalid_argument("LayerNorm: a non-contiguous axis complement needs a reorder, which "
+                                "this backend does not provide");
+  Variable dummyInMean, dummyInVar;
+  const Variable none(Tensor(), false);
+  Variable output = batchnorm(input, none, none, dummyInMean, dummyInVar, axisComplement_, true, 0.0,
+                              epsilon_);
+  if (affine_) {
+    const Variable weight = params_[0].astype(output.type());
+    const Variable bias = params_[1].astype(output.type());
+    if (axisSize_ == kLnVariableAxisSize) {
+      output = detail::affine(output, weight, bias, 1, 1, output.elements(), true);
+    } else {
+      // the parameters take the input's shape with the complement axes set to 1
+      if (axis_.empty() || axis_.back() - axis_.front() + 1 != (int)axis_.size())
+        throw std::invalid_argument("LayerNorm: per-element parameters need contiguous normalised axes");
+      Dim inner = 1, mid = 1, outer = 1;
+      for (int d = 0; d < input.ndim(); ++d)
+        (d < axis_.front() ? inner : d <= axis_.back() ? mid : outer) *= input.dim(d);
+      if (mid != axisSize_)
+        throw std::invalid_argument("[LayerNorm] Input size along the norm axis doesn't with axisSize.");
+      output = detail::affine(output, weight, bias, outer, mid, inner, false);
+    }
+  }
+  return moddims(output, in.shape());
+}
+
+std::string LayerNorm::prettyString() const {
+  std::ostringstream ss;
+  ss << "LayerNorm ( axis : { ";
+  for (int a : axis_) ss << a << " ";
+  ss << "} , size : " << axisSize_ << ")";
+  return ss.str();
+}
+
+// ---- Linear ----------------------------------------------------------------------------
+Linear::Linear(int inputSize, int outputSize, bool bias) : nIn_(inputSize), nOut_(outputSize), bias_(bias) {
+  // Linear.cpp:62-74
+  const int fanIn = nIn_;
+  auto w = kaimingUniform(Shape({nOut_, nIn_}), fanIn, dtype::f32, true);
+  if (bias_) {
+    const double bound = std::sqrt(1.0 / fanIn);
+    params_ = {w, uniform(Shape({nOut_}), -bound, bound, dtype::f32, true)};
+  } else {
+    params_ = {w};
+  }
+}
+
+Linear::Linear(const Variable& w) : UnaryModule({w}), nIn_((int)w.dim(1)), nOut_((int)w.dim(0)), bias_(false) {}
+
+Linear::Linear(const Variable& w, const Variable& b)
+    : UnaryModule({w, b}), nIn_((int)w.dim(1)), nOut_((int)w.dim(0)), bias_(true) {
+  if (b.dim(0) != w.dim(0)) throw std::invalid_argument("dimension mismatch between Linear weight and bias");
+}
+
+Variable Linear::forward(const Variable& input) {
+  if (bias_) return linear(input, params_[0].astype(input.type()), params_[1].astype(input.type()));
+  return linear(input, params_[0].astype(input.type()));
+}
+
+std::string Linear::prettyString() const {
+  std::ostringstream ss;
+  ss << "Linear (" << nIn_ << "->" << nOut_ << ")" << (bias_ ? " (with bias)" : " (without bias)");
+  return ss.str();
+}
+
+}  // namespace fl

@@ -1,0 +1,257 @@
+// nn-level wrappers over the differentiable functions of Functions.h, with the
+// constructor arguments, parameter layout, initialisation and train/eval behaviour
+// of the Flashlight modules they stand for (flashlight/fl/nn/modules/*.cpp), so that
+// a network description written for Flashlight (Sequential of Conv2D / BatchNorm /
+// ReLU / Pool2D / View / Linear / LogSoftmax, a ResNet bottleneck) reads the same
+// here.  Serialization, clone() and the modules that do not touch the extension's
+// operators are not provided.
+#pragma once
+
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "Functions.h"
+
+namespace fl {
+
+// ---- initialisation (flashlight/fl/nn/Init.cpp:21-48, 142-200) --------------------------
+// Values are drawn on the host from one process-wide generator and copied to the device.
+void setSeed(unsigned long long seed);
+Variable constant(double val, const Shape& shape, dtype type = dtype::f32, bool calcGrad = true);
+Variable uniform(const Shape& shape, double min = 0, double max = 1, dtype type = dtype::f32,
+                 bool calcGrad = true);
+Variable kaimingUniform(const Shape& shape, int fanIn, dtype type = dtype::f32, bool calcGrad = true);
+
+// ---- Module (flashlight/fl/nn/modules/Module.cpp:17-112) --------------------------------
+class Module {
+ public:
+  virtual ~Module() = default;
+  std::vector<Variable> params() const { return params_; }
+  int numParamTensors() const { return (int)params_.size(); }
+  Variable param(int position) const;
+  virtual void setParams(const Variable& var, int position);
+  virtual void train();
+  virtual void eval();
+  bool isTrain() const { return train_; }
+  void zeroGrad();
+  virtual std::vector<Variable> forward(const std::vector<Variable>& inputs) = 0;
+  std::vector<Variable> operator()(const std::vector<Variable>& inputs) { return forward(inputs); }
+  virtual std::string prettyString() const = 0;
+
+ protected:
+  Module() = default;
+  explicit Module(const std::vector<Variable>& params) : params_(params) {}
+  std::vector<Variable> params_;
+  bool train_ = true;
+};
+using ModulePtr = std::shared_ptr<Module>;
+
+class UnaryModule : public Module {
+ public:
+  using Module::forward;
+  std::vector<Variable> forward(const std::vector<Variable>& inputs) override;
+  virtual Variable forward(const Variable& input) = 0;
+  Variable operator()(const Variable& input) { return forward(input); }
+
+ protected:
+  UnaryModule() = default;
+  explicit UnaryModule(const std::vector<Variable>& params) : Module(params) {}
+};
+
+class BinaryModule : public Module {
+ public:
+  using Module::forward;
+  std::vector<Variable> forward(const std::vector<Variable>& inputs) override;
+  virtual Variable forward(const Variable& input1, const Variable& input2) = 0;
+  Variable operator()(const Variable& a, const Variable& b) { return forward(a, b); }
+};
+
+// ---- Container / Sequential (flashlight/fl/nn/modules/Container.{h,cpp}) ------------------
+class Container : public Module {
+ public:
+  template <typename T>
+  void add(std::shared_ptr<T> module) {
+    if (!module) throw std::invalid_argument("can't add null Module to Container");
+    for (int i = 0; i < module->numParamTensors(); ++i) {
+      childParamIdx_.push_back({(int)params_.size(), (int)modules_.size(), i});
+      params_.push_back(module->param(i));
+    }
+    modules_.emplace_back(std::move(module));
+  }
+  template <typename T, typename = std::enable_if_t<std::is_base_of_v<Module, std::decay_t<T>>>>
+  void add(T&& module) {
+    static_assert(!std::is_lvalue_reference_v<T>, "add() can only accept rvalues. Use std::move().");
+    add(std::make_shared<std::decay_t<T>>(std::forward<T>(module)));
+  }
+  ModulePtr module(int id) const { return modules_.at(id); }
+  std::vector<ModulePtr> modules() const { return modules_; }
+  void train() override;
+  void eval() override;
+  void setParams(const Variable& var, int position) override;
+
+ protected:
+  struct ChildParam {
+    int position, module, index;
+  };
+  std::vector<ModulePtr> modules_;
+  std::vector<ChildParam> childParamIdx_;
+};
+
+class Sequential : public Container {
+ public:
+  using Module::operator();
+  std::vector<Variable> forward(const std::vector<Variable>& inputs) override;
+  Variable forward(const Variable& input);
+  Variable operator()(const Variable& input) { return forward(input); }
+  std::string prettyString() const override;
+};
+
+// ---- layers ----------------------------------------------------------------------------
+// int or PaddingMode::SAME (flashlight/fl/nn/Utils.h:40-51)
+struct IntOrPadMode {
+  IntOrPadMode(int v) : padVal(v) {}
+  IntOrPadMode(PaddingMode m) : padVal(static_cast<int>(m)) {}
+  int padVal;
+};
+
+// flashlight/fl/nn/modules/Conv2D.cpp:22-227: weight [wx, wy, nin/groups, nout] Kaiming
+// uniform with fanIn = wx*wy*nin/groups, bias [1, 1, nout, 1] uniform(+-sqrt(1/fanIn))
+class Conv2D : public UnaryModule {
+ public:
+  Conv2D(int nin, int nout, int wx, int wy, int sx = 1, int sy = 1, IntOrPadMode px = 0,
+         IntOrPadMode py = 0, int dx = 1, int dy = 1, bool bias = true, int groups = 1);
+  explicit Conv2D(const Variable& w, int sx = 1, int sy = 1, IntOrPadMode px = 0, IntOrPadMode py = 0,
+                  int dx = 1, int dy = 1, int groups = 1);
+  Conv2D(const Variable& w, const Variable& b, int sx = 1, int sy = 1, IntOrPadMode px = 0,
+         IntOrPadMode py = 0, int dx = 1, int dy = 1, int groups = 1);
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override;
+  std::string prettyString() const override;
+
+ private:
+  int nIn_, nOut_, xFilter_, yFilter_, xStride_, yStride_, xPad_, yPad_, xDilation_, yDilation_;
+  bool bias_;
+  int groups_;
+};
+
+// flashlight/fl/nn/modules/Pool2D.cpp:19-52
+class Pool2D : public UnaryModule {
+ public:
+  Pool2D(int wx, int wy, int sx = 1, int sy = 1, IntOrPadMode px = 0, IntOrPadMode py = 0,
+         PoolingMode mode = PoolingMode::MAX);
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override;
+  std::string prettyString() const override;
+
+ private:
+  int xFilter_, yFilter_, xStride_, yStride_, xPad_, yPad_;
+  PoolingMode mode_;
+};
+
+// flashlight/fl/nn/modules/BatchNorm.cpp:20-128: momentum < 0 selects the cumulative
+// average 1 / numBatchesTracked; eval mode normalises with the running statistics when
+// they are tracked, with batch statistics otherwise
+class BatchNorm : public UnaryModule {
+ public:
+  BatchNorm(int featAxis, int featSize, double momentum = 0.1, double eps = 1e-5, bool affine = true,
+            bool trackStats = true);
+  BatchNorm(const std::vector<int>& featAxis, int featSize, double momentum = 0.1, double eps = 1e-5,
+            bool affine = true, bool trackStats = true);
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override;
+  std::string prettyString() const override;
+  Variable runningMean() const { return runningMean_; }
+  Variable runningVar() const { return runningVar_; }
+  int numBatchesTracked() const { return numBatchesTracked_; }
+
+ private:
+  std::vector<int> featAxis_;
+  int featSize_;
+  int numBatchesTracked_ = 0;
+  Variable runningMean_, runningVar_;
+  double momentum_, epsilon_;
+  bool affine_, trackStats_;
+};
+
+// flashlight/fl/nn/modules/LayerNorm.cpp:20-160: normalises over `axis` by calling
+// batchnorm over the complement axes; the complement must be contiguous here (the
+// other case needs a reorder, which this backend does not provide)
+constexpr int kLnVariableAxisSize = -1;
+class LayerNorm : public UnaryModule {
+ public:
+  explicit LayerNorm(int axis, double eps = 1e-5, bool affine = true, int axisSize = kLnVariableAxisSize);
+  explicit LayerNorm(const std::vector<int>& axis, double eps = 1e-5, bool affine = true,
+                     int axisSize = kLnVariableAxisSize);
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override;
+  std::string prettyString() const override;
+
+ private:
+  std::vector<int> axis_, axisComplement_;
+  double epsilon_;
+  bool affine_;
+  int axisSize_;
+};
+
+// flashlight/fl/nn/modules/Linear.cpp:18-92: weight [out, in] Kaiming uniform (fanIn = in)
+class Linear : public UnaryModule {
+ public:
+  Linear(int inputSize, int outputSize, bool bias = true);
+  explicit Linear(const Variable& w);
+  Linear(const Variable& w, const Variable& b);
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override;
+  std::string prettyString() const override;
+
+ private:
+  int nIn_, nOut_;
+  bool bias_;
+};
+
+class ReLU : public UnaryModule {          // Activations.cpp:58-70
+ public:
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return relu(input); }
+  std::string prettyString() const override { return "ReLU"; }
+};
+
+class LogSoftmax : public UnaryModule {    // Activations.cpp:180-192
+ public:
+  explicit LogSoftmax(int dim = 0) : dim_(dim) {}
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return logSoftmax(input, dim_); }
+  std::string prettyString() const override { return "LogSoftmax"; }
+
+ private:
+  int dim_;
+};
+
+class View : public UnaryModule {          // View.cpp:17-24
+ public:
+  explicit View(Shape dims) : dims_(std::move(dims)) {}
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return moddims(input, dims_); }
+  std::string prettyString() const override { return "View " + dims_.toString(); }
+
+ private:
+  Shape dims_;
+};
+
+// flashlight/fl/nn/modules/Loss.cpp (CategoricalCrossEntropy)
+class CategoricalCrossEntropy : public BinaryModule {
+ public:
+  explicit CategoricalCrossEntropy(ReduceMode reduction = ReduceMode::MEAN, int ignoreIndex = -1)
+      : reduction_(reduction), ignoreIndex_(ignoreIndex) {}
+  using BinaryModule::forward;
+  Variable forward(const Variable& inputs, const Variable& targets) override {
+    return categoricalCrossEntropy(inputs, targets, reduction_, ignoreIndex_);
+  }
+  std::string prettyString() const override { return "CategoricalCrossEntropy"; }
+
+ private:
+  ReduceMode reduction_;
+  int ignoreIndex_;
+};
+
+}  // namespace fl

@@ -6,7 +6,9 @@
 //   flashlight/fl/test/autograd/AutogradTest.cpp:65-81,333-337 (dtype errors, pool),
 //   flashlight/fl/test/autograd/AutogradNormalizationTest.cpp:158-189 (batchnorm),
 //   flashlight/fl/test/nn/ModuleTest.cpp:338-353 (batching invariance),
-// and one training step of the README MNIST convnet (README.md:45-84) through the tape.
+// one training step of the README MNIST convnet (README.md:45-84) through the tape, and
+// the nn modules over those functions (flashlight/fl/test/nn/ModuleTest.cpp:670-719 for
+// LayerNorm; Sequential, BatchNorm statistics, a ResNet bottleneck with its residual add).
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
@@ -17,6 +19,7 @@
 #include <vector>
 
 #include "Functions.h"
+#include "Modules.h"
 #include "HipAutogradExtension.h"
 #include "flref.h"
 
@@ -366,6 +369,268 @@ static void testMnistStep() {
   CHECK(throws<std::invalid_argument>([&] { moddims(in, Shape({5, -1})); }));
 }
 
+static std::vector<float> hostOf(const Variable& v) { return v.tensor().toHostVector(); }
+
+// The README network built from modules: same result as the functional chain on the
+// modules' own parameters, initialisation bounds, train/eval, zeroGrad, setParams.
+static void testSequentialMnist() {
+  std::printf("Sequential MNIST convnet\n");
+  const int B = 4;
+  setSeed(5);
+  Sequential model;
+  model.add(View(Shape({28, 28, 1, -1})));
+  model.add(Conv2D(1, 32, 5, 5, 1, 1, PaddingMode::SAME, PaddingMode::SAME));
+  model.add(ReLU());
+  model.add(Pool2D(2, 2, 2, 2));
+  model.add(Conv2D(32, 64, 5, 5, 1, 1, PaddingMode::SAME, PaddingMode::SAME));
+  model.add(ReLU());
+  model.add(Pool2D(2, 2, 2, 2));
+  model.add(View(Shape({7 * 7 * 64, -1})));
+  model.add(Linear(7 * 7 * 64, 1024));
+  model.add(ReLU());
+  model.add(Linear(1024, 10));
+  model.add(LogSoftmax());
+  CHECK(model.params().size() == 8 && model.modules().size() == 12);
+  CHECK(model.param(0).shape() == Shape({5, 5, 1, 32}) && model.param(1).shape() == Shape({1, 1, 32, 1}));
+  CHECK(model.param(4).shape() == Shape({1024, 3136}) && model.param(7).shape() == Shape({10}));
+  // Kaiming-uniform bounds: sqrt(3 / fanIn) for weights, sqrt(1 / fanIn) for biases
+  const double lim[8] = {std::sqrt(3. / 25), std::sqrt(1. / 25), std::sqrt(3. / 800), std::sqrt(1. / 800),
+                         std::sqrt(3. / 3136), std::sqrt(1. / 3136), std::sqrt(3. / 1024), std::sqrt(1. / 1024)};
+  for (int i = 0; i < 8; ++i) {
+    const auto v = hostOf(model.param(i));
+    float mx = 0.f;
+    double mean = 0;
+    for (float f : v) {
+      mx = std::max(mx, std::fabs(f));
+      mean += f;
+    }
+    CHECK(mx <= lim[i] * 1.0000001 && mx >= (v.size() >= 32 ? 0.8 : 0.3) * lim[i]);
+    if (v.size() > 10000) CHECK(std::fabs(mean / v.size()) < 0.02 * lim[i]);
+  }
+  CHECK(model.prettyString().find("Conv2D (32->64, 5x5, 1,1, SAME,SAME, 1, 1) (with bias)") != std::string::npos);
+
+  auto x = randn((size_t)B * 28 * 28, 31);
+  std::vector<int32_t> labels = {3, 1, 4, 1};
+  Variable in(Tensor::fromVector({28 * 28, B}, x), false);
+  Variable tg(Tensor::fromHost(Shape({B}), dtype::s32, labels.data()), false);
+  Variable out = model.forward(in);
+  CHECK(out.shape() == Shape({10, B}));
+  // the functional chain on the same parameters
+  auto P = model.params();
+  Variable h = moddims(in, Shape({28, 28, 1, -1}));
+  h = pool2d(relu(conv2d(h, P[0], P[1], 1, 1, 2, 2)), 2, 2, 2, 2);
+  h = pool2d(relu(conv2d(h, P[2], P[3], 1, 1, 2, 2)), 2, 2, 2, 2);
+  h = relu(linear(moddims(h, Shape({7 * 7 * 64, -1})), P[4], P[5]));
+  Variable ref = logSoftmax(linear(h, P[6], P[7]), 0);
+  CHECK(hostOf(out) == hostOf(ref));
+  CategoricalCrossEntropy criterion;
+  Variable loss = criterion(out, tg);
+  loss.backward(Variable(Tensor::fromVector({1}, {1.f}), false));
+  std::vector<std::vector<float>> grads;
+  for (auto& p : model.params()) {
+    CHECK(p.isGradAvailable());
+    grads.push_back(hostOf(p.grad()));
+  }
+  model.zeroGrad();
+  for (auto& p : model.params()) CHECK(!p.isGradAvailable());
+  Variable loss2 = categoricalCrossEntropy(ref, tg);
+  loss2.backward(Variable(Tensor::fromVector({1}, {1.f}), false));
+  for (int i = 0; i < 8; ++i) CHECK(hostOf(model.param(i).grad()) == grads[i]);
+  CHECK(hostOf(loss) == hostOf(loss2));
+
+  // eval(): parameters stop asking for gradients, in the children as well (Module.cpp:58-70)
+  model.eval();
+  CHECK(!model.isTrain() && !model.module(1)->isTrain());
+  for (auto& p : model.params()) CHECK(!p.isCalcGrad());
+  CHECK(!model.forward(in).isCalcGrad());
+  model.train();
+  for (auto& p : model.params()) CHECK(p.isCalcGrad());
+  // setParams reaches the child module (Container.cpp:85-93)
+  Variable zeroBias(Tensor::full({10}, 0., dtype::f32), true);
+  model.setParams(zeroBias, 7);
+  CHECK(hostOf(model.module(10)->param(1)) == std::vector<float>(10, 0.f));
+  CHECK(throws<std::out_of_range>([&] { model.param(8); }));
+  CHECK(throws<std::invalid_argument>([&] { model.forward(std::vector<Variable>{in, in}); }));
+  // bias shape rules of Conv2D(w, b) (Conv2D.cpp:88-96)
+  Variable w(Tensor::full({3, 3, 4, 6}, 0.1, dtype::f32), true), bad(Tensor::full({1, 1, 5, 1}, 0., dtype::f32), true);
+  CHECK(throws<std::invalid_argument>([&] { Conv2D(w, bad); }));
+}
+
+// BatchNorm module: exponential and cumulative running statistics over several
+// batches, eval mode, statistics not tracked (BatchNorm.cpp:74-112)
+static void testBatchNormModule() {
+  std::printf("BatchNorm module\n");
+  const int W = 6, H = 5, C = 4, N = 7;
+  const int64_t M = (int64_t)N * H * W;
+  setSeed(9);
+  BatchNorm bn(2, C), cum(2, C, -1.0), loose(2, C, 0.1, 1e-5, true, false);
+  CHECK(hostOf(bn.runningMean()) == std::vector<float>(C, 0.f) && hostOf(bn.runningVar()) == std::vector<float>(C, 1.f));
+  CHECK(hostOf(bn.param(1)) == std::vector<float>(C, 0.f));
+  for (float f : hostOf(bn.param(0))) CHECK(f >= 0.f && f <= 1.f);
+  std::vector<float> erm(C, 0.f), erv(C, 1.f), crm(C, 0.f), crv(C, 1.f);
+  std::vector<float> x, y(x.size()), mean(C), var(C);
+  const auto g = hostOf(bn.param(0)), b = hostOf(bn.param(1));
+  const auto gc = hostOf(cum.param(0)), bc = hostOf(cum.param(1));
+  for (int step = 1; step <= 3; ++step) {
+    x = randn((size_t)N * C * H * W, 40 + step, 1.f + 0.3f * step, 0.2f * step);
+    y.resize(x.size());
+    flref_bn_fwd_train(N, C, (int64_t)H * W, x.data(), g.data(), b.data(), 1e-5, y.data(), mean.data(), var.data());
+    flref_bn_running_update(C, M, mean.data(), var.data(), 0.1, erm.data(), erv.data());
+    flref_bn_running_update(C, M, mean.data(), var.data(), 1.0 / step, crm.data(), crv.data());
+    Variable in(Tensor::fromVector({W, H, C, N}, x), true);
+    CHECK(relL2(hostOf(bn.forward(in)), y) <= 1e-4);
+    cum.forward(in);
+    CHECK(bn.numBatchesTracked() == step);
+  }
+  CHECK(relL2(hostOf(bn.runningMean()), erm) <= 1e-5 && relL2(hostOf(bn.runningVar()), erv) <= 1e-4);
+  // momentum < 0: the running mean is the plain average of the batch means
+  CHECK(relL2(hostOf(cum.runningMean()), crm) <= 1e-5 && relL2(hostOf(cum.runningVar()), crv) <= 1e-4);
+  // eval: running statistics, no update, no gradient request
+  bn.eval();
+  Variable in(Tensor::fromVector({W, H, C, N}, x), false);
+  flref_bn_fwd_infer(N, C, (int64_t)H * W, x.data(), g.data(), b.data(), erm.data(), erv.data(), 1e-5, y.data());
+  Variable ye = bn.forward(in);
+  CHECK(relL2(hostOf(ye), y) <= 1e-5 && !ye.isCalcGrad() && bn.numBatchesTracked() == 3);
+  CHECK(relL2(hostOf(bn.runningMean()), erm) <= 1e-5);
+  // statistics not tracked: batch statistics also in eval mode
+  const auto gl = hostOf(loose.param(0)), bl = hostOf(loose.param(1));
+  loose.eval();
+  flref_bn_fwd_train(N, C, (int64_t)H * W, x.data(), gl.data(), bl.data(), 1e-5, y.data(), mean.data(), var.data());
+  CHECK(relL2(hostOf(loose.forward(in)), y) <= 1e-4 && loose.numBatchesTracked() == 0);
+  // bf16 input keeps f32 parameters (BatchNorm.cpp:86-88)
+  bn.train();
+  Variable in16(in.tensor().astype(dtype::bf16), true);
+  Variable y16 = bn.forward(in16);
+  CHECK(y16.type() == dtype::bf16);
+  y16.backward(Variable(Tensor::full(y16.shape(), 1., dtype::f32).astype(dtype::bf16), false));
+  CHECK(bn.param(0).grad().type() == dtype::f32 && in16.grad().type() == dtype::bf16);
+}
+
+// LayerNorm module on the reference test's shapes (ModuleTest.cpp:670-719) plus the
+// transformer use (normalise dimension 0 of [C, T, B]) with per-element parameters
+static void testLayerNormModule() {
+  std::printf("LayerNorm module\n");
+  const double eps = 1e-5;
+  const int F = 10, S = 4 * 4 * 3;
+  auto x = randn((size_t)S * F, 51, 1.f, 0.5f);
+  Variable input(Tensor::fromVector({4, 4, 3, F}, x), true);
+  // direct definition: mean and biased variance over axis 3
+  std::vector<float> want(x.size());
+  for (int s = 0; s < S; ++s) {
+    double m = 0, v = 0;
+    for (int f = 0; f < F; ++f) m += x[(size_t)f * S + s];
+    m /= F;
+    for (int f = 0; f < F; ++f) v += (x[(size_t)f * S + s] - m) * (x[(size_t)f * S + s] - m);
+    v /= F;
+    for (int f = 0; f < F; ++f) want[(size_t)f * S + s] = (float)((x[(size_t)f * S + s] - m) / std::sqrt(v + eps));
+  }
+  LayerNorm module1(std::vector<int>{3}, eps, false);
+  module1.train();
+  Variable out = module1.forward(input);
+  CHECK(relL2(hostOf(out), want) <= 1e-4 && out.type() == input.type());
+  module1.eval();
+  CHECK(relL2(hostOf(module1.forward(input)), want) <= 1e-4);
+  LayerNorm module2(std::vector<int>{3}, eps, true);
+  module2.train();
+  const auto outTrain = hostOf(module2.forward(input));
+  module2.eval();
+  CHECK(hostOf(module2.forward(input)) == outTrain && relL2(outTrain, want) <= 1e-4);
+  LayerNorm module3(std::vector<int>{3}, eps, true, F);
+  module3.setParams(Variable(Tensor::full({F}, 1.0, dtype::f32), false), 0);
+  module3.setParams(Variable(Tensor::full({F}, 0.0, dtype::f32), false), 1);
+  CHECK(relL2(hostOf(module3.forward(input)), outTrain) <= 1e-6);
+  Variable input3(Tensor::fromVector({4, 4, 3}, randn(48, 52)), true);
+  LayerNorm module4(std::vector<int>{0}, eps, false);
+  CHECK(module4.forward(input3).shape() == input3.shape());
+  // a complement that is not contiguous needs a reorder
+  LayerNorm module5(std::vector<int>{0, 2}, eps, false);
+  CHECK(throws<std::invalid_argument>([&] { module5.forward(input); }));
+  CHECK(throws<std::invalid_argument>([&] { LayerNorm(std::vector<int>{3}, eps, true, F + 1).forward(input); }));
+
+  // [C, T, B], normalise C with per-element scale and shift; forward and backward against
+  // the CPU checker (batchnorm over the complement, then the broadcast affine)
+  const int Cn = 24, T = 9, Bn = 5;
+  auto xt = randn((size_t)Cn * T * Bn, 53, 2.f, -0.3f), dyt = randn(xt.size(), 54);
+  auto w = randn(Cn, 55, 0.2f, 1.f), b = randn(Cn, 56);
+  std::vector<float> ones(T * Bn, 1.f), zeros(T * Bn, 0.f), xhat(xt.size()), mean(T * Bn), var(T * Bn), y(xt.size());
+  flref_bn_fwd_train(1, T * Bn, Cn, xt.data(), ones.data(), zeros.data(), eps, xhat.data(), mean.data(), var.data());
+  flref_affine_fwd(T * Bn, Cn, 1, 0, xhat.data(), w.data(), b.data(), y.data());
+  std::vector<float> g(xt.size()), dw(Cn), db(Cn), dx(xt.size()), dgam(T * Bn), dbet(T * Bn);
+  flref_affine_bwd(T * Bn, Cn, 1, 0, dyt.data(), xhat.data(), w.data(), g.data(), dw.data(), db.data());
+  flref_bn_bwd(1, T * Bn, Cn, xt.data(), g.data(), ones.data(), mean.data(), var.data(), eps, dx.data(),
+               dgam.data(), dbet.data());
+  LayerNorm ln(0, eps, true, Cn);
+  ln.setParams(Variable(Tensor::fromVector({Cn}, w), true), 0);
+  ln.setParams(Variable(Tensor::fromVector({Cn}, b), true), 1);
+  Variable vin(Tensor::fromVector({Cn, T, Bn}, xt), true);
+  Variable vout = ln.forward(vin);
+  CHECK(vout.shape() == Shape({Cn, T, Bn}) && relL2(hostOf(vout), y) <= 1e-4);
+  vout.backward(Variable(Tensor::fromVector({Cn, T, Bn}, dyt), false));
+  CHECK(relL2(hostOf(vin.grad()), dx) <= 1e-4);
+  CHECK(relL2(hostOf(ln.param(0).grad()), dw) <= 1e-4 && relL2(hostOf(ln.param(1).grad()), db) <= 1e-4);
+}
+
+// One ResNet bottleneck (pkg/vision/models/Resnet.cpp:38-87: 1x1 -> 3x3 -> 1x1, BatchNorm
+// after every convolution, ReLU, residual add, ReLU) from modules, forward and backward
+// against the CPU checker
+static void testBottleneck() {
+  std::printf("ResNet bottleneck from modules\n");
+  const int W = 14, H = 14, Cin = 16, Cm = 8, N = 4;
+  const int64_t HW = (int64_t)H * W;
+  setSeed(13);
+  Conv2D c1(Cin, Cm, 1, 1, 1, 1, 0, 0, 1, 1, false), c2(Cm, Cm, 3, 3, 1, 1, PaddingMode::SAME, PaddingMode::SAME, 1, 1, false),
+      c3(Cm, Cin, 1, 1, 1, 1, 0, 0, 1, 1, false);
+  BatchNorm b1(2, Cm), b2(2, Cm), b3(2, Cin);
+  auto x = randn((size_t)N * Cin * HW, 61), dy = randn((size_t)N * Cin * HW, 62);
+  Variable in(Tensor::fromVector({W, H, Cin, N}, x), true);
+  Variable t3 = b3(c3(relu(b2(c2(relu(b1(c1(in))))))));
+  Variable out = relu(t3 + in);
+  out.backward(Variable(Tensor::fromVector(out.shape(), dy), false));
+
+  // ---- CPU checker -------------------------------------------------------------------
+  const auto w1 = hostOf(c1.param(0)), w2 = hostOf(c2.param(0)), w3 = hostOf(c3.param(0));
+  const auto g1 = hostOf(b1.param(0)), g2 = hostOf(b2.param(0)), g3 = hostOf(b3.param(0));
+  const auto z1 = hostOf(b1.param(1)), z2 = hostOf(b2.param(1)), z3 = hostOf(b3.param(1));
+  flref_conv d1{N, Cin, H, W, Cm, 1, 1, 1, 1, 0, 0, 1, 1, 1}, d2{N, Cm, H, W, Cm, 3, 3, 1, 1, 1, 1, 1, 1, 1},
+      d3{N, Cm, H, W, Cin, 1, 1, 1, 1, 0, 0, 1, 1, 1};
+  const size_t nm = (size_t)N * Cm * HW, ni = (size_t)N * Cin * HW;
+  std::vector<float> a1(nm), n1(nm), r1(nm), a2(nm), n2(nm), r2(nm), a3(ni), n3(ni), s(ni), o(ni);
+  std::vector<float> m1(Cm), v1(Cm), m2(Cm), v2(Cm), m3(Cin), v3(Cin);
+  flref_conv2d_fwd(&d1, x.data(), w1.data(), nullptr, a1.data());
+  flref_bn_fwd_train(N, Cm, HW, a1.data(), g1.data(), z1.data(), 1e-5, n1.data(), m1.data(), v1.data());
+  flref_relu_fwd((int64_t)nm, n1.data(), r1.data());
+  flref_conv2d_fwd(&d2, r1.data(), w2.data(), nullptr, a2.data());
+  flref_bn_fwd_train(N, Cm, HW, a2.data(), g2.data(), z2.data(), 1e-5, n2.data(), m2.data(), v2.data());
+  flref_relu_fwd((int64_t)nm, n2.data(), r2.data());
+  flref_conv2d_fwd(&d3, r2.data(), w3.data(), nullptr, a3.data());
+  flref_bn_fwd_train(N, Cin, HW, a3.data(), g3.data(), z3.data(), 1e-5, n3.data(), m3.data(), v3.data());
+  for (size_t i = 0; i < ni; ++i) s[i] = n3[i] + x[i];
+  flref_relu_fwd((int64_t)ni, s.data(), o.data());
+  CHECK(relL2(hostOf(out), o) <= 1e-4);
+  std::vector<float> gs(ni), ga3(ni), dg3(Cin), db3(Cin), gr2(nm), dw3(w3.size()), gn2(nm), ga2(nm), dg2(Cm), db2(Cm),
+      gr1(nm), dw2(w2.size()), gn1(nm), ga1(nm), dg1(Cm), db1(Cm), gx(ni), dw1(w1.size());
+  flref_relu_bwd((int64_t)ni, dy.data(), s.data(), gs.data());
+  flref_bn_bwd(N, Cin, HW, a3.data(), gs.data(), g3.data(), m3.data(), v3.data(), 1e-5, ga3.data(), dg3.data(), db3.data());
+  flref_conv2d_bwd_filter(&d3, r2.data(), ga3.data(), dw3.data(), nullptr);
+  flref_conv2d_bwd_data(&d3, ga3.data(), w3.data(), gr2.data());
+  flref_relu_bwd((int64_t)nm, gr2.data(), n2.data(), gn2.data());
+  flref_bn_bwd(N, Cm, HW, a2.data(), gn2.data(), g2.data(), m2.data(), v2.data(), 1e-5, ga2.data(), dg2.data(), db2.data());
+  flref_conv2d_bwd_filter(&d2, r1.data(), ga2.data(), dw2.data(), nullptr);
+  flref_conv2d_bwd_data(&d2, ga2.data(), w2.data(), gr1.data());
+  flref_relu_bwd((int64_t)nm, gr1.data(), n1.data(), gn1.data());
+  flref_bn_bwd(N, Cm, HW, a1.data(), gn1.data(), g1.data(), m1.data(), v1.data(), 1e-5, ga1.data(), dg1.data(), db1.data());
+  flref_conv2d_bwd_filter(&d1, x.data(), ga1.data(), dw1.data(), nullptr);
+  flref_conv2d_bwd_data(&d1, ga1.data(), w1.data(), gx.data());
+  for (size_t i = 0; i < ni; ++i) gx[i] += gs[i];        // the residual branch
+  CHECK(relL2(hostOf(in.grad()), gx) <= 2e-4);
+  CHECK(relL2(hostOf(c1.param(0).grad()), dw1) <= 2e-4 && relL2(hostOf(c2.param(0).grad()), dw2) <= 2e-4 &&
+        relL2(hostOf(c3.param(0).grad()), dw3) <= 2e-4);
+  CHECK(relL2(hostOf(b1.param(0).grad()), dg1) <= 2e-4 && relL2(hostOf(b1.param(1).grad()), db1) <= 2e-4);
+  CHECK(relL2(hostOf(b2.param(0).grad()), dg2) <= 2e-4 && relL2(hostOf(b2.param(1).grad()), db2) <= 2e-4);
+  CHECK(relL2(hostOf(b3.param(0).grad()), dg3) <= 2e-4 && relL2(hostOf(b3.param(1).grad()), db3) <= 2e-4);
+  CHECK(throws<std::invalid_argument>([&] { t3 + c1(in); }));   // shapes differ
+}
+
 int main() {
   try {
     CHECK(derivePadding(56, 3, 1, -1, 1) == 1 && derivePadding(224, 7, 2, -1, 1) == 3 &&
@@ -381,6 +646,10 @@ int main() {
     testBatchnorm();
     testGradAccumulation();
     testMnistStep();
+    testSequentialMnist();
+    testBatchNormModule();
+    testLayerNormModule();
+    testBottleneck();
     fl::sync();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
