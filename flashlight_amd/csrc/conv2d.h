@@ -32,6 +32,21 @@ bool mfma_slab_wgrad_applies(const ConvGeom& g);
 int mfma_slab_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
                             hipStream_t s);
 
+// 1x1 convolutions without padding as GEMMs (conv2d_mfma_pointwise.hip); same return
+// convention.
+int mfma_pointwise_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w,
+                            const float* bias, void* y, hipStream_t s);
+int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w,
+                                 void* dx, hipStream_t s);
+size_t mfma_pointwise_wgrad_ws(const ConvGeom& g);
+int mfma_pointwise_wgrad(const ConvGeom& g, int dtype, const void* x, const void* dy, float* dw,
+                         float* db, void* ws, size_t ws_bytes, hipStream_t s);
+
+// Adds the slices of a split filter gradient in a fixed order (conv2d_mfma_wgrad.hip):
+// slice s holds E floats of dw followed by K floats of db at part + s * (E + K).
+void wgrad_reduce_launch(const float* part, int nsplit, int E, int K, int want_db, float* dw,
+                         float* db, hipStream_t s);
+
 // bf16-storage variants on the bf16 matrix cores (conv2d_mfma_slab_bf16.hip,
 // conv2d_mfma_wgrad_slab_bf16.hip); same return convention.
 int mfma_slab16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,

@@ -154,7 +154,9 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
     size_t a = mfma_conv_bwd_filter_ws(g, d->dtype);
     const size_t b = mfma_slab_wgrad_ws(g, d->dtype);
     const size_t c = d->dtype == FLHIP_BF16 ? mfma_wgrad16_ws(g) : 0;
+    const size_t e = mfma_pointwise_wgrad_ws(g);
     if (b > a) a = b;
+    if (e > a) a = e;
     return c > a ? c : a;
   }
   return 0;
@@ -174,6 +176,7 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !algo_is("gather") && !algo_is("convert"))
       r = mfma_slab16_conv_fwd(g, x, w, bias, y, s);
+    if (r < 0 && !algo_is("gather")) r = mfma_pointwise_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r < 0 && !algo_is("gather")) r = mfma_slab_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r < 0) r = mfma_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r >= 0) return r;
@@ -204,6 +207,7 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !algo_is("gather") && !algo_is("convert"))
       r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s);
+    if (r < 0 && !algo_is("gather")) r = mfma_pointwise_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0 && !algo_is("gather")) r = mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0) r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r >= 0) return r;
@@ -237,6 +241,7 @@ extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, 
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !algo_is("gather") && !algo_is("convert"))
       r = mfma_wgrad16(g, x, dy, dw, db, ws, ws_bytes, s);
+    if (r < 0 && !algo_is("gather")) r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0 && !algo_is("gather")) r = mfma_slab_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0) r = mfma_conv_bwd_filter(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
     if (r >= 0) return r;

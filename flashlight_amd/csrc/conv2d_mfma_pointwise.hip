@@ -1,0 +1,656 @@
+// 1x1 convolutions without padding as GEMMs on the gfx950 fp32 matrix cores:
+// forward and backward-data, any stride.
+//
+// With a 1x1 window the result is, per image n,
+//   D[n][m][map_d(q)] = sum_k A[m][k] * S[n][k][map_s(q)],   q = 0 .. P-1,
+//   forward : S = x, A = w [K][C] (k contiguous), P = OH*OW, map_s = the stride
+//             lattice of the input, map_d = identity;
+//   backward: S = dy, A = w^T (m contiguous), P = OH*OW, map_s = identity,
+//             map_d = the stride lattice of dx (the other elements of dx are zero
+//             and are cleared by a fill kernel first).
+// For stride 1 both maps are the identity and a channel plane is one contiguous row
+// of the GEMM, so operands and results move as 16-byte vectors.
+//
+// A workgroup owns 64 result channels x BN = 32*PT positions (positions run across
+// image boundaries; PT = 2 by default) and has 8 waves with two roles, as the other MFMA
+// kernels here:
+//   waves 0-3 (loaders) fetch chunk c+2 (32 contraction channels of the source tile
+//     and of the weight tile) into registers while chunk c+1 waits in a second
+//     register set, and store it into the LDS buffer the MFMA waves are not reading;
+//   waves 4-7 (MFMA), arranged 2 (positions) x 2 (channels), own 16*PT positions x 32
+//     channels each and issue the chunk's MFMAs from 8-byte LDS fragment reads.
+// One barrier per chunk; two LDS buffers.
+//
+// LDS layouts (one buffer): source xs[16 pairs][XPS] with float2 {channel 2j, 2j+1} per
+// position, so one 8-byte read feeds two MFMAs (the k index of v_mfma_f32_16x16x4_f32
+// is the lane group; the first MFMA takes the even channels of a pair-step, the
+// second the odd ones).  Weights: forward as[64 m][APW] (k contiguous, the memory
+// order), backward as[16 pairs][APS] with float2 per result channel.  Pitches are
+// chosen so that the 32 lanes of one read pass touch distinct banks.
+//
+// The matrix-core operands are swapped against the usual convention: the source
+// tile is the A operand (rows = positions), the weights the B operand, so that a
+// lane's four accumulator values are four consecutive positions of one channel and
+// leave as one 16-byte store.
+#include "conv2d_mfma.h"
+
+namespace flhip {
+namespace {
+
+constexpr int KC = 32;                 // contraction channels per chunk
+constexpr int NPAIR = KC / 2;
+constexpr int BM = MFMA_BM;            // result channels per workgroup
+constexpr int APW = KC + 4;            // forward weight pitch: 16 channels x 2 lane groups hit 64 banks
+constexpr int APS = 2 * BM + 32;       // backward weight pair stride (== 32 mod 64)
+constexpr int LTHREADS = 256;
+constexpr int OOB = (int)0x80000000;
+
+struct PwParams {
+  int Kc, Mo;            // contraction / result channels
+  int SP, DP;            // elements per source / result channel plane
+  int P, Ptot;           // GEMM positions per image, over all images
+  int OW;                // positions per row of the strided lattice
+  int rowstep, colstep;  // lattice: element (q / OW) * rowstep + (q % OW) * colstep
+  int src_map, dst_map;  // 1 = that side goes through the lattice
+  int vec_w;             // weight tile by 16-byte loads
+  int nchunks, mtiles, ptiles;
+  unsigned src_bytes, wgt_bytes, dst_bytes;
+};
+
+__device__ __forceinline__ int lattice(const PwParams& p, int q) {
+  const int r = q / p.OW;
+  return r * p.rowstep + (q - r * p.OW) * p.colstep;
+}
+
+template <typename P>
+__device__ __forceinline__ int lattice_w(const P& p, int q) {
+  const int r = q / p.OW;
+  return r * p.rowstep + (q - r * p.OW) * p.colstep;
+}
+
+template <typename T>
+__device__ __forceinline__ void buf_st1(__amdgpu_buffer_rsrc_t r, int byte_off, float v, T*);
+template <>
+__device__ __forceinline__ void buf_st1<float>(__amdgpu_buffer_rsrc_t r, int byte_off, float v, float*) {
+  __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, byte_off, 0, 0);
+}
+template <>
+__device__ __forceinline__ void buf_st1<bf16_t>(__amdgpu_buffer_rsrc_t r, int byte_off, float v, bf16_t*) {
+  __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16(v), r, byte_off, 0, 0);
+}
+__device__ __forceinline__ void buf_st4v(__amdgpu_buffer_rsrc_t r, int byte_off, floatx4 v, float*) {
+  const uintx4_t t = {__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]),
+                      __float_as_uint(v[3])};
+  __builtin_amdgcn_raw_buffer_store_b128(t, r, byte_off, 0, 0);
+}
+__device__ __forceinline__ void buf_st4v(__amdgpu_buffer_rsrc_t r, int byte_off, floatx4 v, bf16_t*) {
+  const uintx2_t t = {(uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16),
+                      (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16)};
+  __builtin_amdgcn_raw_buffer_store_b64(t, r, byte_off, 0, 0);
+}
+
+template <typename T, bool BWD, int PT, bool VEC>
+__global__ void __launch_bounds__(MFMA_THREADS)
+pointwise_conv_kernel(PwParams p, const T* __restrict__ src, const T* __restrict__ wgt,
+                      const float* __restrict__ bias, T* __restrict__ dst) {
+  constexpr int BN = 32 * PT;               // positions per workgroup
+  constexpr int XPS = 2 * BN + 32;          // source pair stride in words (== 32 mod 64)
+  constexpr int QN = BN / 4;                // position quads per tile
+  constexpr int JSTEP = LTHREADS / QN;      // pairs covered by one sweep of the loader threads
+  constexpr int NJ = NPAIR / JSTEP;         // sweeps per chunk
+  constexpr int ASZ = BWD ? NPAIR * APS : BM * APW;
+  constexpr int BUF = NPAIR * XPS + ASZ;
+  constexpr int esz = (int)sizeof(T);
+  static_assert(NJ >= 1 && NJ * JSTEP == NPAIR, "tile shape");
+  extern __shared__ float lds[];            // [2][BUF]: source tile, then weight tile
+
+  // XCD-aware tile order: consecutive workgroups go to different XCDs, so the tiles
+  // that share a source tile (all channel tiles of one position tile) are put on
+  // one XCD, back to back
+  const int id = blockIdx.x, xcd = id & 7, seq = id >> 3;
+  const int mtile = __builtin_amdgcn_readfirstlane(seq % p.mtiles);
+  const int ptile = __builtin_amdgcn_readfirstlane((seq / p.mtiles) * 8 + xcd);
+  if (ptile >= p.ptiles) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int tileP0 = ptile * BN;
+  const int n = p.nchunks;
+
+  if (wave < 4) {
+    // ================================ loaders ====================================
+    const __amdgpu_buffer_rsrc_t srsrc = make_rsrc(src, p.src_bytes);
+    const __amdgpu_buffer_rsrc_t wrsrc = make_rsrc(wgt, p.wgt_bytes);
+    const int pq = tid % QN, j0 = tid / QN;
+    const int SPb = p.SP * esz;
+    // byte offset of channel 0 at this thread's four positions; OOB past the end
+    int sb[VEC ? 1 : 4];
+    {
+      const int Pg = tileP0 + 4 * pq;
+      if (VEC) {
+        const int ni = Pg / p.P, q = Pg - ni * p.P;
+        sb[0] = Pg < p.Ptot ? (ni * p.Kc * p.SP + q) * esz : OOB;
+      } else {
+#pragma unroll
+        for (int e = 0; e < (VEC ? 1 : 4); ++e) {
+          const int Pe = Pg + e;
+          const int ni = Pe / p.P, q = Pe - ni * p.P;
+          sb[e] = Pe < p.Ptot ? (ni * p.Kc * p.SP + (p.src_map ? lattice(p, q) : q)) * esz : OOB;
+        }
+      }
+    }
+    // weight tile shares: forward (m, 4 consecutive k), backward (pair, 4 consecutive m)
+    const int wm = BWD ? (tid & 15) * 4 : tid >> 3;       // backward: first of 4 channels
+    const int wk = BWD ? (tid >> 4) * 2 : (tid & 7) * 4;  // first contraction index inside the chunk
+    const int m0 = mtile * BM;
+
+    auto load = [&](int c, float4 (&sr)[NJ][2], float4 (&wr)[2]) {
+      const int k0 = c * KC;
+#pragma unroll
+      for (int i = 0; i < NJ; ++i) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int k = k0 + 2 * (j0 + i * JSTEP) + h;
+          const bool kok = k < p.Kc;
+          if (VEC) {
+            sr[i][h] = buf_ld4(srsrc, (kok && sb[0] != OOB) ? sb[0] + k * SPb : OOB, src);
+          } else {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              v[e] = buf_ld(srsrc, (kok && sb[VEC ? 0 : e] != OOB) ? sb[VEC ? 0 : e] + k * SPb : OOB, src);
+            sr[i][h] = make_float4(v[0], v[1], v[2], v[3]);
+          }
+        }
+      }
+      if (!BWD) {
+        // rows m = wm and wm + 32, columns k0 + wk .. +3 of w[m][k]
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int m = m0 + wm + 32 * i, k = k0 + wk;
+          const int off = (m * p.Kc + k) * esz;
+          if (p.vec_w) {
+            wr[i] = buf_ld4(wrsrc, (m < p.Mo && k < p.Kc) ? off : OOB, wgt);
+          } else {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              v[e] = buf_ld(wrsrc, (m < p.Mo && k + e < p.Kc) ? off + e * esz : OOB, wgt);
+            wr[i] = make_float4(v[0], v[1], v[2], v[3]);
+          }
+        }
+      } else {
+        // rows k = k0 + wk and +1, columns m0 + wm .. +3 of w[k][m]
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int k = k0 + wk + h, m = m0 + wm;
+          const int off = (k * p.Mo + m) * esz;
+          if (p.vec_w) {
+            wr[h] = buf_ld4(wrsrc, (k < p.Kc && m < p.Mo) ? off : OOB, wgt);
+          } else {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              v[e] = buf_ld(wrsrc, (k < p.Kc && m + e < p.Mo) ? off + e * esz : OOB, wgt);
+            wr[h] = make_float4(v[0], v[1], v[2], v[3]);
+          }
+        }
+      }
+    };
+    auto store = [&](int buf, const float4 (&sr)[NJ][2], const float4 (&wr)[2]) {
+      float* xs = lds + buf * BUF;
+      float* as = xs + NPAIR * XPS;
+#pragma unroll
+      for (int i = 0; i < NJ; ++i) {
+        float4* d = reinterpret_cast<float4*>(xs + (j0 + i * JSTEP) * XPS + 8 * pq);
+        d[0] = make_float4(sr[i][0].x, sr[i][1].x, sr[i][0].y, sr[i][1].y);
+        d[1] = make_float4(sr[i][0].z, sr[i][1].z, sr[i][0].w, sr[i][1].w);
+      }
+      if (!BWD) {
+        *reinterpret_cast<float4*>(as + wm * APW + wk) = wr[0];
+        *reinterpret_cast<float4*>(as + (wm + 32) * APW + wk) = wr[1];
+      } else {
+        float4* d = reinterpret_cast<float4*>(as + (wk >> 1) * APS + 2 * wm);
+        d[0] = make_float4(wr[0].x, wr[1].x, wr[0].y, wr[1].y);
+        d[1] = make_float4(wr[0].z, wr[1].z, wr[0].w, wr[1].w);
+      }
+    };
+
+    float4 srA[NJ][2], wrA[2], srB[NJ][2], wrB[2];
+    load(0, srA, wrA);
+    store(0, srA, wrA);
+    load(1, srB, wrB);
+    __syncthreads();
+    for (int c = 0; c < n; c += 2) {
+      load(c + 2, srA, wrA);
+      store(1, srB, wrB);                      // chunk c+1
+      __syncthreads();
+      if (c + 1 >= n) break;
+      load(c + 3, srB, wrB);
+      store(0, srA, wrA);                      // chunk c+2
+      __syncthreads();
+    }
+    return;
+  }
+
+  // ================================ MFMA waves ===================================
+  const int cw = wave - 4;
+  const int wp = cw & 1, wc = cw >> 1;
+  const int fr = lane & 15, fg = lane >> 4;
+  floatx4 acc[PT][2];
+#pragma unroll
+  for (int i = 0; i < PT; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  __syncthreads();                             // chunk 0 is in buffer 0
+  for (int c = 0; c < n; ++c) {
+    const float* xs = lds + (c & 1) * BUF + fg * XPS + (wp * PT * 16 + fr) * 2;
+    const float* as = lds + (c & 1) * BUF + NPAIR * XPS +
+                      (BWD ? fg * APS + (wc * 32 + fr) * 2 : (wc * 32 + fr) * APW + 2 * fg);
+#pragma unroll
+    for (int s = 0; s < KC / 8; ++s) {
+      float2 a[PT], b[2];
+#pragma unroll
+      for (int i = 0; i < PT; ++i)
+        a[i] = *reinterpret_cast<const float2*>(xs + 4 * s * XPS + i * 32);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        b[j] = *reinterpret_cast<const float2*>(as + (BWD ? 4 * s * APS + j * 32 : j * 16 * APW + 8 * s));
+#pragma unroll
+      for (int i = 0; i < PT; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].x, b[j].x, acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].y, b[j].y, acc[i][j], 0, 0, 0);
+        }
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: a lane holds positions Pg .. Pg+3 of channel ch per accumulator ----
+  const __amdgpu_buffer_rsrc_t drsrc = make_rsrc(dst, p.dst_bytes);
+#pragma unroll
+  for (int i = 0; i < PT; ++i) {
+    const int Pg = tileP0 + (wp * PT + i) * 16 + 4 * fg;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int ch = mtile * BM + wc * 32 + j * 16 + fr;
+      floatx4 v = acc[i][j];
+      if (bias && ch < p.Mo) {
+        const float bv = bias[ch];
+        v[0] += bv; v[1] += bv; v[2] += bv; v[3] += bv;
+      }
+      if (VEC) {
+        const int ni = Pg / p.P, q = Pg - ni * p.P;
+        const bool ok = Pg < p.Ptot && ch < p.Mo;
+        buf_st4v(drsrc, ok ? ((ni * p.Mo + ch) * p.DP + q) * esz : OOB, v, dst);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int Pe = Pg + e;
+          const int ni = Pe / p.P, q = Pe - ni * p.P;
+          const bool ok = Pe < p.Ptot && ch < p.Mo;
+          const int off = ((ni * p.Mo + ch) * p.DP + (p.dst_map ? lattice(p, q) : q)) * esz;
+          buf_st1<T>(drsrc, ok ? off : OOB, v[e], dst);
+        }
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) zero_kernel(T* __restrict__ p, size_t n16, size_t n) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  uint4* q = reinterpret_cast<uint4*>(p);
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride)
+    q[i] = make_uint4(0, 0, 0, 0);
+  constexpr size_t per = 16 / sizeof(T);
+  for (size_t i = n16 * per + (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) p[i] = (T)0;
+}
+
+template <typename T, bool BWD, int PT, bool VEC>
+int launch_tile(const PwParams& p0, const void* src, const void* wgt, const float* bias, void* dst,
+                hipStream_t s) {
+  PwParams p = p0;
+  constexpr int BN = 32 * PT;
+  p.ptiles = (p.Ptot + BN - 1) / BN;
+  const size_t shmem = (size_t)2 * (NPAIR * (2 * BN + 32) + (BWD ? NPAIR * APS : BM * APW)) * sizeof(float);
+  auto kernel = pointwise_conv_kernel<T, BWD, PT, VEC>;
+  if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
+  const unsigned grid = (unsigned)(((p.ptiles + 7) / 8) * 8 * p.mtiles);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(MFMA_THREADS), shmem, s, p, static_cast<const T*>(src),
+                     static_cast<const T*>(wgt), bias, static_cast<T*>(dst));
+  return check_launch("conv2d 1x1 (mfma)");
+}
+
+template <typename T, bool BWD>
+int launch_pw(const PwParams& p, bool vec, const void* src, const void* wgt, const float* bias,
+              void* dst, hipStream_t s) {
+  // 64 x 64 tiles: four workgroups share a CU (39 KB of LDS each), so the load
+  // latency at the start of one tile and the stores at its end overlap the MFMA phase
+  // of the others; measured faster than 64 x 128 and 64 x 256 on every ResNet-50 1x1
+  // layer (FLHIP_PW_PT=4|8 selects those, a measurement aid)
+  int pt = 2;
+  if (const char* e = getenv("FLHIP_PW_PT")) {
+    const int v = atoi(e);
+    if (v == 2 || v == 4 || v == 8) pt = v;
+  }
+  if (vec) {
+    if (pt == 8) return launch_tile<T, BWD, 8, true>(p, src, wgt, bias, dst, s);
+    if (pt == 4) return launch_tile<T, BWD, 4, true>(p, src, wgt, bias, dst, s);
+    return launch_tile<T, BWD, 2, true>(p, src, wgt, bias, dst, s);
+  }
+  if (pt == 8) return launch_tile<T, BWD, 8, false>(p, src, wgt, bias, dst, s);
+  if (pt == 4) return launch_tile<T, BWD, 4, false>(p, src, wgt, bias, dst, s);
+  return launch_tile<T, BWD, 2, false>(p, src, wgt, bias, dst, s);
+}
+
+bool pw_applies(const ConvGeom& g) {
+  return g.KH == 1 && g.KW == 1 && g.py == 0 && g.px == 0 && g.groups == 1;
+}
+
+
+// ---- filter gradient of a 1x1 convolution ---------------------------------------------
+//   dw[m][c] = sum over (n, q) of dy[n][m][q] * x[n][c][map(q)]   (+ db[m] = sum of dy)
+// is a GEMM whose contraction runs over positions, which are contiguous in memory in
+// both operands, so the tiles go to LDS in memory order [row][position] (pitch 36: the
+// 32 lanes of one 8-byte read pass hit distinct banks) and a lane's float2 holds two
+// consecutive positions = the k index of two MFMAs.  A workgroup owns 64 (m) x 64 (c)
+// of dw and one slice of the positions; it writes its tile (and, for the first column
+// tile, the bias sums collected by the loader threads) to the workspace, and the
+// fixed-order reduction kernel shared with the other filter-gradient kernels adds the
+// slices.  Same wave roles and barrier scheme as above; four workgroups per CU.
+constexpr int PC = 32;                 // positions per chunk
+constexpr int WPITCH = PC + 4;
+
+struct PwWgradParams {
+  int Mo, C;             // channels of dy / of x
+  int P, Ptot, SP;       // positions per image (dy), over all images; elements per x plane
+  int OW, rowstep, colstep, x_map;
+  int pps, nsplit;       // positions per slice (multiple of PC), slices
+  int ctiles, mtiles;
+  int E;                 // Mo * C
+  int want_db;
+  unsigned x_bytes, dy_bytes;
+};
+
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(MFMA_THREADS)
+pointwise_wgrad_kernel(PwWgradParams p, const T* __restrict__ x, const T* __restrict__ dy,
+                       float* __restrict__ out) {
+  constexpr int TILE = BM * WPITCH;
+  constexpr int esz = (int)sizeof(T);
+  __shared__ float lds[2][2][TILE];          // [buffer][dy tile, x tile]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int split = blockIdx.x;
+  const int ctile = __builtin_amdgcn_readfirstlane(blockIdx.y % p.ctiles);
+  const int mtile = __builtin_amdgcn_readfirstlane(blockIdx.y / p.ctiles);
+  const int pos0 = split * p.pps;
+  const int pos1 = min(pos0 + p.pps, p.Ptot);
+  const int n = (pos1 - pos0 + PC - 1) / PC;
+  float* part = out + (size_t)split * (p.nsplit > 1 ? (size_t)p.E + p.Mo : 0);
+
+  if (wave < 4) {
+    // ================================ loaders ====================================
+    const __amdgpu_buffer_rsrc_t xrsrc = make_rsrc(x, p.x_bytes);
+    const __amdgpu_buffer_rsrc_t yrsrc = make_rsrc(dy, p.dy_bytes);
+    const int row = tid >> 3, kq = tid & 7;             // rows row and row + 32, positions 4kq..+3
+    // image and in-plane index of this thread's positions, advanced chunk by chunk
+    int ni[VEC ? 1 : 4], qi[VEC ? 1 : 4];
+#pragma unroll
+    for (int e = 0; e < (VEC ? 1 : 4); ++e) {
+      const int Pe = pos0 + 4 * kq + e;
+      ni[e] = Pe / p.P;
+      qi[e] = Pe - ni[e] * p.P;
+    }
+    const bool do_db = p.want_db && ctile == 0;
+    float dbs[2] = {0.f, 0.f};
+    const int mrow = mtile * BM + row, crow = ctile * BM + row;
+
+    auto load = [&](int c, float4 (&yr)[2], float4 (&xr)[2]) {
+      const int Pg = pos0 + c * PC + 4 * kq;
+      int yo[VEC ? 1 : 4], xo[VEC ? 1 : 4];    // element offsets of channel 0, -1 = past the slice
+#pragma unroll
+      for (int e = 0; e < (VEC ? 1 : 4); ++e) {
+        const bool ok = Pg + e < pos1;
+        yo[e] = ok ? ni[e] * p.Mo * p.P + qi[e] : -1;
+        xo[e] = ok ? ni[e] * p.C * p.SP + (p.x_map ? lattice_w(p, qi[e]) : qi[e]) : -1;
+        qi[e] += PC;
+        while (qi[e] >= p.P) {
+          qi[e] -= p.P;
+          ++ni[e];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int m = mrow + 32 * i, ch = crow + 32 * i;
+        if (VEC) {
+          yr[i] = buf_ld4(yrsrc, (yo[0] >= 0 && m < p.Mo) ? (yo[0] + m * p.P) * esz : OOB, dy);
+          xr[i] = buf_ld4(xrsrc, (xo[0] >= 0 && ch < p.C) ? (xo[0] + ch * p.SP) * esz : OOB, x);
+        } else {
+          float a[4], b[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            a[e] = buf_ld(yrsrc, (yo[VEC ? 0 : e] >= 0 && m < p.Mo) ? (yo[VEC ? 0 : e] + m * p.P) * esz : OOB, dy);
+            b[e] = buf_ld(xrsrc, (xo[VEC ? 0 : e] >= 0 && ch < p.C) ? (xo[VEC ? 0 : e] + ch * p.SP) * esz : OOB, x);
+          }
+          yr[i] = make_float4(a[0], a[1], a[2], a[3]);
+          xr[i] = make_float4(b[0], b[1], b[2], b[3]);
+        }
+      }
+    };
+    auto store = [&](int buf, const float4 (&yr)[2], const float4 (&xr)[2]) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        *reinterpret_cast<float4*>(&lds[buf][0][(row + 32 * i) * WPITCH + 4 * kq]) = yr[i];
+        *reinterpret_cast<float4*>(&lds[buf][1][(row + 32 * i) * WPITCH + 4 * kq]) = xr[i];
+        if (do_db) dbs[i] += (yr[i].x + yr[i].y) + (yr[i].z + yr[i].w);
+      }
+    };
+
+    float4 yA[2], xA[2], yB[2], xB[2];
+    load(0, yA, xA);
+    store(0, yA, xA);
+    load(1, yB, xB);
+    __syncthreads();
+    for (int c = 0; c < n; c += 2) {
+      load(c + 2, yA, xA);
+      store(1, yB, xB);                        // chunk c+1 (zeros past the slice)
+      __syncthreads();
+      if (c + 1 >= n) break;
+      load(c + 3, yB, xB);
+      store(0, yA, xA);                        // chunk c+2
+      __syncthreads();
+    }
+    if (do_db) {
+      // the 8 threads that share a row are neighbours in the wave
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        float v = dbs[i];
+        v += __shfl_xor(v, 1, 64);
+        v += __shfl_xor(v, 2, 64);
+        v += __shfl_xor(v, 4, 64);
+        const int m = mrow + 32 * i;
+        if (kq == 0 && m < p.Mo) part[p.E + m] = v;
+      }
+    }
+    return;
+  }
+
+  // ================================ MFMA waves ===================================
+  const int cw = wave - 4;
+  const int wm = cw & 1, wn = cw >> 1;
+  const int fr = lane & 15, fg = lane >> 4;
+  floatx4 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  __syncthreads();
+  for (int c = 0; c < n; ++c) {
+    const float* ys = &lds[c & 1][0][(wm * 32 + fr) * WPITCH + 2 * fg];
+    const float* xs = &lds[c & 1][1][(wn * 32 + fr) * WPITCH + 2 * fg];
+#pragma unroll
+    for (int s = 0; s < PC / 8; ++s) {
+      float2 a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        a[i] = *reinterpret_cast<const float2*>(ys + i * 16 * WPITCH + 8 * s);
+        b[i] = *reinterpret_cast<const float2*>(xs + i * 16 * WPITCH + 8 * s);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].x, b[j].x, acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].y, b[j].y, acc[i][j], 0, 0, 0);
+        }
+    }
+    __syncthreads();
+  }
+  // lane: rows m0 + 4*fg + r, column c0 + fr of each accumulator
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int ch = ctile * BM + wn * 32 + j * 16 + fr;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = mtile * BM + wm * 32 + i * 16 + 4 * fg + r;
+        if (m < p.Mo && ch < p.C) part[(size_t)m * p.C + ch] = acc[i][j][r];
+      }
+    }
+}
+
+bool pw_wgrad_plan(const ConvGeom& g, PwWgradParams* p) {
+  if (!pw_applies(g)) return false;
+  p->Mo = g.K; p->C = g.C;
+  p->P = g.OH * g.OW; p->Ptot = g.N * p->P; p->SP = g.H * g.W;
+  p->OW = g.OW; p->rowstep = g.sy * g.W; p->colstep = g.sx;
+  p->x_map = (g.sy != 1 || g.sx != 1) ? 1 : 0;
+  p->ctiles = (g.C + BM - 1) / BM;
+  p->mtiles = (g.K + BM - 1) / BM;
+  p->E = g.K * g.C;
+  const long long base = (long long)p->ctiles * p->mtiles;
+  if (base > 65535) return false;
+  long long ns = 4ll * mfma_num_cus() / base;
+  const long long max_ns = (p->Ptot + 255) / 256;
+  if (ns > max_ns) ns = max_ns;
+  if (ns < 1) ns = 1;
+  long long pps = (p->Ptot + ns - 1) / ns;
+  pps = (pps + PC - 1) / PC * PC;
+  p->pps = (int)pps;
+  p->nsplit = (int)((p->Ptot + pps - 1) / pps);
+  return true;
+}
+
+}  // namespace
+
+int mfma_pointwise_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w,
+                            const float* bias, void* y, hipStream_t s) {
+  if (!pw_applies(g)) return -1;
+  const long long esz = dtype == FLHIP_F32 ? 4 : 2;
+  const long long sb = (long long)g.N * g.C * g.H * g.W * esz, db = (long long)g.N * g.K * g.OH * g.OW * esz;
+  const long long wb = (long long)g.K * g.C * esz;
+  if (sb >= (1ll << 31) || db >= (1ll << 31) || wb >= (1ll << 31)) return -1;
+  PwParams p{};
+  p.Kc = g.C; p.Mo = g.K; p.SP = g.H * g.W; p.DP = g.OH * g.OW;
+  p.P = g.OH * g.OW; p.Ptot = g.N * p.P; p.OW = g.OW;
+  p.rowstep = g.sy * g.W; p.colstep = g.sx;
+  p.src_map = (g.sy != 1 || g.sx != 1) ? 1 : 0;
+  p.dst_map = 0;
+  p.vec_w = (g.C % 4 == 0) ? 1 : 0;
+  p.nchunks = (g.C + KC - 1) / KC;
+  p.mtiles = (g.K + BM - 1) / BM;
+  p.src_bytes = (unsigned)sb; p.wgt_bytes = (unsigned)wb; p.dst_bytes = (unsigned)db;
+  const bool vec = !p.src_map && p.P % 4 == 0;
+  return dtype == FLHIP_F32 ? launch_pw<float, false>(p, vec, x, w, bias, y, s)
+                            : launch_pw<bf16_t, false>(p, vec, x, w, bias, y, s);
+}
+
+int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
+                                 hipStream_t s) {
+  if (!pw_applies(g)) return -1;
+  const long long esz = dtype == FLHIP_F32 ? 4 : 2;
+  const long long sb = (long long)g.N * g.K * g.OH * g.OW * esz, db = (long long)g.N * g.C * g.H * g.W * esz;
+  const long long wb = (long long)g.K * g.C * esz;
+  if (sb >= (1ll << 31) || db >= (1ll << 31) || wb >= (1ll << 31)) return -1;
+  PwParams p{};
+  p.Kc = g.K; p.Mo = g.C; p.SP = g.OH * g.OW; p.DP = g.H * g.W;
+  p.P = g.OH * g.OW; p.Ptot = g.N * p.P; p.OW = g.OW;
+  p.rowstep = g.sy * g.W; p.colstep = g.sx;
+  p.src_map = 0;
+  // dx covers more than the lattice when a stride skips elements or the last rows /
+  // columns are never reached; those elements are zero
+  const bool full = g.sy == 1 && g.sx == 1 && g.OH == g.H && g.OW == g.W;
+  p.dst_map = full ? 0 : 1;
+  p.vec_w = (g.C % 4 == 0) ? 1 : 0;
+  p.nchunks = (g.K + KC - 1) / KC;
+  p.mtiles = (g.C + BM - 1) / BM;
+  p.src_bytes = (unsigned)sb; p.wgt_bytes = (unsigned)wb; p.dst_bytes = (unsigned)db;
+  if (!full) {
+    const size_t nel = (size_t)g.N * g.C * g.H * g.W;
+    const size_t n16 = (size_t)db / 16;
+    size_t blocks = (n16 + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    if (blocks < 1) blocks = 1;
+    if (dtype == FLHIP_F32)
+      hipLaunchKernelGGL((zero_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, s, static_cast<float*>(dx), n16, nel);
+    else
+      hipLaunchKernelGGL((zero_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, static_cast<bf16_t*>(dx), n16, nel);
+  }
+  const bool vec = full && p.P % 4 == 0;
+  return dtype == FLHIP_F32 ? launch_pw<float, true>(p, vec, dy, w, nullptr, dx, s)
+                            : launch_pw<bf16_t, true>(p, vec, dy, w, nullptr, dx, s);
+}
+
+size_t mfma_pointwise_wgrad_ws(const ConvGeom& g) {
+  PwWgradParams p{};
+  if (!pw_wgrad_plan(g, &p)) return 0;
+  return p.nsplit > 1 ? (size_t)p.nsplit * ((size_t)p.E + p.Mo) * sizeof(float) : 0;
+}
+
+int mfma_pointwise_wgrad(const ConvGeom& g, int dtype, const void* x, const void* dy, float* dw,
+                         float* db, void* ws, size_t ws_bytes, hipStream_t s) {
+  if (!dw) return -1;   // bias gradient alone: the plain reduction kernel
+  PwWgradParams p{};
+  if (!pw_wgrad_plan(g, &p)) return -1;
+  const long long esz = dtype == FLHIP_F32 ? 4 : 2;
+  const long long xb = (long long)g.N * g.C * g.H * g.W * esz, yb = (long long)g.N * g.K * g.OH * g.OW * esz;
+  if (xb >= (1ll << 31) || yb >= (1ll << 31)) return -1;
+  p.x_bytes = (unsigned)xb;
+  p.dy_bytes = (unsigned)yb;
+  p.want_db = db != nullptr;
+  if (p.nsplit > 1 && (!ws || ws_bytes < (size_t)p.nsplit * ((size_t)p.E + p.Mo) * sizeof(float)))
+    return fail(FLHIP_INVALID_ARGUMENT, "conv2d_bwd_filter: workspace too small");
+  // a single slice writes dw in place; its bias sums need a home of their own
+  if (p.nsplit == 1 && db) return -1;
+  float* out = p.nsplit > 1 ? static_cast<float*>(ws) : dw;
+  const dim3 grid((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles));
+  const bool vec = !p.x_map && p.P % 4 == 0;
+  if (dtype == FLHIP_F32) {
+    if (vec)
+      hipLaunchKernelGGL((pointwise_wgrad_kernel<float, true>), grid, dim3(MFMA_THREADS), 0, s, p,
+                         static_cast<const float*>(x), static_cast<const float*>(dy), out);
+    else
+      hipLaunchKernelGGL((pointwise_wgrad_kernel<float, false>), grid, dim3(MFMA_THREADS), 0, s, p,
+                         static_cast<const float*>(x), static_cast<const float*>(dy), out);
+  } else {
+    if (vec)
+      hipLaunchKernelGGL((pointwise_wgrad_kernel<bf16_t, true>), grid, dim3(MFMA_THREADS), 0, s, p,
+                         static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), out);
+    else
+      hipLaunchKernelGGL((pointwise_wgrad_kernel<bf16_t, false>), grid, dim3(MFMA_THREADS), 0, s, p,
+                         static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), out);
+  }
+  if (const int rc = check_launch("conv2d_bwd_filter 1x1 (mfma)")) return rc;
+  if (p.nsplit > 1) {
+    wgrad_reduce_launch(static_cast<const float*>(ws), p.nsplit, p.E, p.Mo, p.want_db, dw, db, s);
+    return check_launch("conv2d_bwd_filter 1x1 (reduce)");
+  }
+  return FLHIP_OK;
+}
+
+}  // namespace flhip

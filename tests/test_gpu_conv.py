@@ -40,6 +40,15 @@ MORE = [
     ((2, 40, 6, 16), (72, 40, 3, 3), (1, 1), (1, 1), (1, 1), 1),        # channel tails on both sides (bf16 matrix-core path)
     ((1, 96, 5, 8), (32, 48, 2, 3), (1, 1), (1, 1), (1, 1), 2),         # groups, 2x3 window (bf16 generic tap loop)
     ((1, 20, 6, 16), (24, 20, 3, 3), (1, 1), (1, 1), (1, 1), 1),        # bf16 matrix-core path, weights not 16-byte friendly
+    # 1x1 as GEMM: positions across image boundaries, channel tails, odd planes (element-wise
+    # path), strides (lattice on one side, zero fill of dx), several chunks of 32 channels
+    ((3, 64, 12, 12), (128, 64, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((2, 256, 8, 8), (64, 256, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((5, 70, 7, 7), (50, 70, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((2, 33, 6, 10), (65, 33, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((3, 96, 14, 14), (160, 96, 1, 1), (2, 2), (0, 0), (1, 1), 1),
+    ((2, 40, 9, 11), (24, 40, 1, 1), (2, 3), (0, 0), (1, 1), 1),
+    ((40, 32, 28, 28), (64, 32, 1, 1), (1, 1), (0, 0), (1, 1), 1),      # enough positions for the 64 x 256 tile
 ]
 ALL = LIB_CASES + MORE
 
