@@ -38,9 +38,15 @@ int mfma_pointwise_conv_fwd(const ConvGeom& g, int dtype, const void* x, const v
                             const float* bias, void* y, hipStream_t s);
 int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w,
                                  void* dx, hipStream_t s);
+// windows with several taps on the same tile machinery, any stride / padding / dilation
+int mfma_tapped_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w,
+                         const float* bias, void* y, hipStream_t s);
+int mfma_tapped_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w,
+                              void* dx, hipStream_t s);
 size_t mfma_pointwise_wgrad_ws(const ConvGeom& g);
+// windows = false: only 1x1 without padding; true: any window, one tap per workgroup
 int mfma_pointwise_wgrad(const ConvGeom& g, int dtype, const void* x, const void* dy, float* dw,
-                         float* db, void* ws, size_t ws_bytes, hipStream_t s);
+                         float* db, void* ws, size_t ws_bytes, bool windows, hipStream_t s);
 
 // Adds the slices of a split filter gradient in a fixed order (conv2d_mfma_wgrad.hip):
 // slice s holds E floats of dw followed by K floats of db at part + s * (E + K).

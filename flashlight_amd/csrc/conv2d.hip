@@ -177,7 +177,9 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
     if (d->dtype == FLHIP_BF16 && !algo_is("gather") && !algo_is("convert"))
       r = mfma_slab16_conv_fwd(g, x, w, bias, y, s);
     if (r < 0 && !algo_is("gather")) r = mfma_pointwise_conv_fwd(g, d->dtype, x, w, bias, y, s);
+    if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r < 0 && !algo_is("gather")) r = mfma_slab_conv_fwd(g, d->dtype, x, w, bias, y, s);
+    if (r < 0 && !algo_is("gather")) r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r < 0) r = mfma_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r >= 0) return r;
   }
@@ -208,7 +210,9 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
     if (d->dtype == FLHIP_BF16 && !algo_is("gather") && !algo_is("convert"))
       r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s);
     if (r < 0 && !algo_is("gather")) r = mfma_pointwise_conv_bwd_data(g, d->dtype, dy, w, dx, s);
+    if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0 && !algo_is("gather")) r = mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s);
+    if (r < 0 && !algo_is("gather")) r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0) r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r >= 0) return r;
   }
@@ -241,8 +245,10 @@ extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, 
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !algo_is("gather") && !algo_is("convert"))
       r = mfma_wgrad16(g, x, dy, dw, db, ws, ws_bytes, s);
-    if (r < 0 && !algo_is("gather")) r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
+    if (r < 0 && !algo_is("gather"))
+      r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, algo_is("tapped"), s);
     if (r < 0 && !algo_is("gather")) r = mfma_slab_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
+    if (r < 0 && !algo_is("gather")) r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, true, s);
     if (r < 0) r = mfma_conv_bwd_filter(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
     if (r >= 0) return r;
   }

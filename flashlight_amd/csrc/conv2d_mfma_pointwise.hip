@@ -62,12 +62,6 @@ __device__ __forceinline__ int lattice(const PwParams& p, int q) {
   return r * p.rowstep + (q - r * p.OW) * p.colstep;
 }
 
-template <typename P>
-__device__ __forceinline__ int lattice_w(const P& p, int q) {
-  const int r = q / p.OW;
-  return r * p.rowstep + (q - r * p.OW) * p.colstep;
-}
-
 template <typename T>
 __device__ __forceinline__ void buf_st1(__amdgpu_buffer_rsrc_t r, int byte_off, float v, T*);
 template <>
@@ -345,6 +339,320 @@ int launch_pw(const PwParams& p, bool vec, const void* src, const void* wgt, con
   return launch_tile<T, BWD, 2, false>(p, src, wgt, bias, dst, s);
 }
 
+// ---- windows with several taps, any stride, padding and dilation ------------------------
+// The same GEMM with the contraction running over (channel chunk, tap): for a tap the
+// source position of a result position is shifted by the tap's (dh, dw) and is
+// outside the image for some positions (padding), which the loaders turn into
+// out-of-range offsets (zero).  Positions are enumerated per "class":
+//   forward : one class, the whole result grid, every tap;
+//   backward: one class per residue ((ih + py) mod sy, (iw + px) mod sx) of the dx
+//             grid.  Only the taps with kh*dil_y = that residue (mod sy) reach a class,
+//             and for those (ih + py - kh*dil_y) / sy is exact, so a class is a stride-1
+//             problem over dy whose results land on a lattice of dx.  Every element of dx
+//             belongs to exactly one class (a class without taps stores zeros), and no
+//             multiplication is spent on taps that cannot contribute.
+// Tiles are 64 channels x 64 positions of one class; loads and stores are element-wise.
+constexpr int MAX_CLASSES = 16;
+constexpr int MAX_TAPS = 128;          // over all classes
+
+struct TapClass {
+  int tile0;             // first position tile of the class
+  int Hc, Wc;            // class grid
+  int h0, w0;            // result coordinates of class grid (0, 0)
+  int bh, bw;            // source coordinates of class grid (0, 0) at shift (0, 0)
+  int tap0, ntaps;
+};
+struct Tap {
+  short dh, dw;          // source shift
+  int tmem;              // tap index in the weights (kh * KW + kw)
+};
+struct TapParams {
+  int N, Kc, Mo;
+  int SH, SW, DH, DW;    // source / result planes
+  int KHW;
+  int ssh, ssw;          // source step per class grid step
+  int rsh, rsw;          // result step per class grid step
+  int kchunks, mtiles, ptiles, nclasses;
+  unsigned src_bytes, wgt_bytes, dst_bytes;
+  TapClass cls[MAX_CLASSES];
+  Tap taps[MAX_TAPS];
+};
+
+template <typename T, bool BWD>
+__global__ void __launch_bounds__(MFMA_THREADS)
+tapped_conv_kernel(TapParams p, const T* __restrict__ src, const T* __restrict__ wgt,
+                   const float* __restrict__ bias, T* __restrict__ dst) {
+  constexpr int PT = 2, BN = 32 * PT;
+  constexpr int XPS = 2 * BN + 32;
+  constexpr int QN = BN / 4;
+  constexpr int JSTEP = LTHREADS / QN;
+  constexpr int ASZ = BWD ? NPAIR * APS : BM * APW;
+  constexpr int BUF = NPAIR * XPS + ASZ;
+  constexpr int esz = (int)sizeof(T);
+  static_assert(JSTEP == NPAIR, "one sweep of the loader threads covers a chunk");
+  __shared__ float lds[2 * BUF];
+
+  const int id = blockIdx.x, xcd = id & 7, seq = id >> 3;
+  const int mtile = __builtin_amdgcn_readfirstlane(seq % p.mtiles);
+  const int ptile = __builtin_amdgcn_readfirstlane((seq / p.mtiles) * 8 + xcd);
+  if (ptile >= p.ptiles) return;
+  int cl = 0;
+  while (cl + 1 < p.nclasses && ptile >= p.cls[cl + 1].tile0) ++cl;
+  cl = __builtin_amdgcn_readfirstlane(cl);
+  const int Hc = p.cls[cl].Hc, Wc = p.cls[cl].Wc, ntaps = p.cls[cl].ntaps, tap0 = p.cls[cl].tap0;
+  const int Pc = Hc * Wc, Pctot = p.N * Pc;
+  const int tileP0 = (ptile - p.cls[cl].tile0) * BN;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = p.kchunks * ntaps;
+
+  if (wave < 4) {
+    // ================================ loaders ====================================
+    const __amdgpu_buffer_rsrc_t srsrc = make_rsrc(src, p.src_bytes);
+    const __amdgpu_buffer_rsrc_t wrsrc = make_rsrc(wgt, p.wgt_bytes);
+    const int pq = tid % QN, j0 = tid / QN;
+    const int SPb = p.SH * p.SW * esz;
+    // per position: byte offset of (image, channel 0, row 0, column 0) and the source
+    // coordinates at shift (0, 0); a position past the class gets a row that fails
+    // every bounds test
+    int nb[4], sh0[4], sw0[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int Pe = tileP0 + 4 * pq + e;
+      const int ni = Pe / Pc, r = Pe - ni * Pc;
+      const int hc = r / Wc, wc = r - hc * Wc;
+      nb[e] = ni * p.Kc * SPb;
+      sh0[e] = Pe < Pctot ? hc * p.ssh + p.cls[cl].bh : -(1 << 24);
+      sw0[e] = wc * p.ssw + p.cls[cl].bw;
+    }
+    const int wm = BWD ? (tid & 15) * 4 : tid >> 3;
+    const int wk = BWD ? (tid >> 4) * 2 : (tid & 7) * 4;
+    const int m0 = mtile * BM;
+    int kc = 0, ti = 0;                        // chunk = (channel chunk kc, tap ti), taps inner
+
+    auto load = [&](float4 (&sr)[2], float4 (&wr)[2]) {
+      const Tap tp = p.taps[min(tap0 + ti, MAX_TAPS - 1)];
+      const int k0 = kc * KC;
+      int so[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int ih = sh0[e] + tp.dh, iw = sw0[e] + tp.dw;
+        const bool ok = (unsigned)ih < (unsigned)p.SH && (unsigned)iw < (unsigned)p.SW;
+        so[e] = ok ? nb[e] + (ih * p.SW + iw) * esz : OOB;
+      }
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int k = k0 + 2 * j0 + h;
+        const bool kok = k < p.Kc && ntaps > 0;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = buf_ld(srsrc, (kok && so[e] != OOB) ? so[e] + k * SPb : OOB, src);
+        sr[h] = make_float4(v[0], v[1], v[2], v[3]);
+      }
+      const int tstep = p.KHW * esz;
+      if (!BWD) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const int m = m0 + wm + 32 * i, k = k0 + wk;
+          const int off = ((m * p.Kc + k) * p.KHW + tp.tmem) * esz;
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            v[e] = buf_ld(wrsrc, (m < p.Mo && k + e < p.Kc && ntaps > 0) ? off + e * tstep : OOB, wgt);
+          wr[i] = make_float4(v[0], v[1], v[2], v[3]);
+        }
+      } else {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int k = k0 + wk + h, m = m0 + wm;
+          const int off = ((k * p.Mo + m) * p.KHW + tp.tmem) * esz;
+          float v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            v[e] = buf_ld(wrsrc, (k < p.Kc && m + e < p.Mo && ntaps > 0) ? off + e * tstep : OOB, wgt);
+          wr[h] = make_float4(v[0], v[1], v[2], v[3]);
+        }
+      }
+      if (++ti >= ntaps) {
+        ti = 0;
+        ++kc;                                   // chunks past the end read channels >= Kc: zeros
+      }
+    };
+    auto store = [&](int buf, const float4 (&sr)[2], const float4 (&wr)[2]) {
+      float* xs = lds + buf * BUF;
+      float* as = xs + NPAIR * XPS;
+      float4* d = reinterpret_cast<float4*>(xs + j0 * XPS + 8 * pq);
+      d[0] = make_float4(sr[0].x, sr[1].x, sr[0].y, sr[1].y);
+      d[1] = make_float4(sr[0].z, sr[1].z, sr[0].w, sr[1].w);
+      if (!BWD) {
+        *reinterpret_cast<float4*>(as + wm * APW + wk) = wr[0];
+        *reinterpret_cast<float4*>(as + (wm + 32) * APW + wk) = wr[1];
+      } else {
+        float4* a = reinterpret_cast<float4*>(as + (wk >> 1) * APS + 2 * wm);
+        a[0] = make_float4(wr[0].x, wr[1].x, wr[0].y, wr[1].y);
+        a[1] = make_float4(wr[0].z, wr[1].z, wr[0].w, wr[1].w);
+      }
+    };
+
+    float4 srA[2], wrA[2], srB[2], wrB[2];
+    load(srA, wrA);
+    store(0, srA, wrA);
+    load(srB, wrB);
+    __syncthreads();
+    for (int c = 0; c < n; c += 2) {
+      load(srA, wrA);
+      store(1, srB, wrB);
+      __syncthreads();
+      if (c + 1 >= n) break;
+      load(srB, wrB);
+      store(0, srA, wrA);
+      __syncthreads();
+    }
+    return;
+  }
+
+  // ================================ MFMA waves ===================================
+  const int cw = wave - 4;
+  const int wp = cw & 1, wc = cw >> 1;
+  const int fr = lane & 15, fg = lane >> 4;
+  floatx4 acc[PT][2];
+#pragma unroll
+  for (int i = 0; i < PT; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  __syncthreads();
+  for (int c = 0; c < n; ++c) {
+    const float* xs = lds + (c & 1) * BUF + fg * XPS + (wp * PT * 16 + fr) * 2;
+    const float* as = lds + (c & 1) * BUF + NPAIR * XPS +
+                      (BWD ? fg * APS + (wc * 32 + fr) * 2 : (wc * 32 + fr) * APW + 2 * fg);
+#pragma unroll
+    for (int s = 0; s < KC / 8; ++s) {
+      float2 a[PT], b[2];
+#pragma unroll
+      for (int i = 0; i < PT; ++i)
+        a[i] = *reinterpret_cast<const float2*>(xs + 4 * s * XPS + i * 32);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        b[j] = *reinterpret_cast<const float2*>(as + (BWD ? 4 * s * APS + j * 32 : j * 16 * APW + 8 * s));
+#pragma unroll
+      for (int i = 0; i < PT; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].x, b[j].x, acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].y, b[j].y, acc[i][j], 0, 0, 0);
+        }
+    }
+    __syncthreads();
+  }
+
+  const __amdgpu_buffer_rsrc_t drsrc = make_rsrc(dst, p.dst_bytes);
+  const int h0 = p.cls[cl].h0, w0 = p.cls[cl].w0;
+#pragma unroll
+  for (int i = 0; i < PT; ++i) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int Pe = tileP0 + (wp * PT + i) * 16 + 4 * fg + e;
+      const int ni = Pe / Pc, r = Pe - ni * Pc;
+      const int hc = r / Wc, wcl = r - hc * Wc;
+      const int pix = (h0 + hc * p.rsh) * p.DW + w0 + wcl * p.rsw;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int ch = mtile * BM + wc * 32 + j * 16 + fr;
+        const bool ok = Pe < Pctot && ch < p.Mo;
+        float v = acc[i][j][e];
+        if (bias && ch < p.Mo) v += bias[ch];
+        buf_st1<T>(drsrc, ok ? ((ni * p.Mo + ch) * p.DH * p.DW + pix) * esz : OOB, v, dst);
+      }
+    }
+  }
+}
+
+template <bool BWD>
+bool tapped_plan(const ConvGeom& g, TapParams* p) {
+  if (g.groups != 1 || g.KH * g.KW > MAX_TAPS) return false;
+  // a chunk is 32 contraction channels of one tap: with few channels most of it is
+  // padding, and the kernel that flattens (channel, tap) into one contraction does better
+  const int kc = BWD ? g.K : g.C;
+  if ((kc + KC - 1) / KC * KC * 2 > 3 * kc) return false;
+  p->N = g.N;
+  p->KHW = g.KH * g.KW;
+  p->nclasses = 0;
+  int ntaps = 0, tiles = 0;
+  auto add_class = [&](TapClass c) {
+    c.tile0 = tiles;
+    const long long pos = (long long)g.N * c.Hc * c.Wc;
+    tiles += (int)((pos + 63) / 64);
+    p->cls[p->nclasses++] = c;
+  };
+  if (!BWD) {
+    p->Kc = g.C; p->Mo = g.K; p->SH = g.H; p->SW = g.W; p->DH = g.OH; p->DW = g.OW;
+    p->ssh = g.sy; p->ssw = g.sx; p->rsh = 1; p->rsw = 1;
+    TapClass c{};
+    c.Hc = g.OH; c.Wc = g.OW; c.h0 = 0; c.w0 = 0; c.bh = -g.py; c.bw = -g.px;
+    c.tap0 = 0; c.ntaps = p->KHW;
+    for (int kh = 0; kh < g.KH; ++kh)
+      for (int kw = 0; kw < g.KW; ++kw)
+        p->taps[ntaps++] = Tap{(short)(kh * g.dly), (short)(kw * g.dlx), kh * g.KW + kw};
+    add_class(c);
+  } else {
+    p->Kc = g.K; p->Mo = g.C; p->SH = g.OH; p->SW = g.OW; p->DH = g.H; p->DW = g.W;
+    p->ssh = 1; p->ssw = 1; p->rsh = g.sy; p->rsw = g.sx;
+    if (g.sy * g.sx > MAX_CLASSES) return false;
+    for (int a = 0; a < g.sy; ++a)
+      for (int b = 0; b < g.sx; ++b) {
+        TapClass c{};
+        c.h0 = ((a - g.py) % g.sy + g.sy) % g.sy;
+        c.w0 = ((b - g.px) % g.sx + g.sx) % g.sx;
+        c.Hc = c.h0 < g.H ? (g.H - 1 - c.h0) / g.sy + 1 : 0;
+        c.Wc = c.w0 < g.W ? (g.W - 1 - c.w0) / g.sx + 1 : 0;
+        if (c.Hc == 0 || c.Wc == 0) continue;
+        c.bh = (c.h0 + g.py - a) / g.sy;
+        c.bw = (c.w0 + g.px - b) / g.sx;
+        c.tap0 = ntaps;
+        for (int kh = 0; kh < g.KH; ++kh)
+          for (int kw = 0; kw < g.KW; ++kw) {
+            if ((kh * g.dly) % g.sy != a || (kw * g.dlx) % g.sx != b) continue;
+            if (ntaps >= MAX_TAPS) return false;
+            p->taps[ntaps++] = Tap{(short)(-(kh * g.dly - a) / g.sy), (short)(-(kw * g.dlx - b) / g.sx),
+                                   kh * g.KW + kw};
+          }
+        c.ntaps = ntaps - c.tap0;
+        add_class(c);
+      }
+  }
+  if (p->nclasses == 0) return false;
+  p->ptiles = tiles;
+  p->kchunks = (p->Kc + KC - 1) / KC;
+  p->mtiles = (p->Mo + BM - 1) / BM;
+  if ((g.KH - 1) * g.dly >= (1 << 14) || (g.KW - 1) * g.dlx >= (1 << 14)) return false;
+  return true;
+}
+
+template <bool BWD>
+int launch_tapped(const ConvGeom& g, int dtype, const void* src, const void* wgt, const float* bias,
+                  void* dst, hipStream_t s) {
+  TapParams p{};
+  if (!tapped_plan<BWD>(g, &p)) return -1;
+  const long long esz = dtype == FLHIP_F32 ? 4 : 2;
+  const long long xb = (long long)g.N * g.C * g.H * g.W * esz, yb = (long long)g.N * g.K * g.OH * g.OW * esz;
+  const long long wb = (long long)g.K * g.C * g.KH * g.KW * esz;
+  if (xb >= (1ll << 31) || yb >= (1ll << 31) || wb >= (1ll << 31)) return -1;
+  p.src_bytes = (unsigned)(BWD ? yb : xb);
+  p.dst_bytes = (unsigned)(BWD ? xb : yb);
+  p.wgt_bytes = (unsigned)wb;
+  const unsigned grid = (unsigned)(((p.ptiles + 7) / 8) * 8 * p.mtiles);
+  if (dtype == FLHIP_F32)
+    hipLaunchKernelGGL((tapped_conv_kernel<float, BWD>), dim3(grid), dim3(MFMA_THREADS), 0, s, p,
+                       static_cast<const float*>(src), static_cast<const float*>(wgt), bias,
+                       static_cast<float*>(dst));
+  else
+    hipLaunchKernelGGL((tapped_conv_kernel<bf16_t, BWD>), dim3(grid), dim3(MFMA_THREADS), 0, s, p,
+                       static_cast<const bf16_t*>(src), static_cast<const bf16_t*>(wgt), bias,
+                       static_cast<bf16_t*>(dst));
+  return check_launch("conv2d (tapped mfma)");
+}
+
 bool pw_applies(const ConvGeom& g) {
   return g.KH == 1 && g.KW == 1 && g.py == 0 && g.px == 0 && g.groups == 1;
 }
@@ -366,7 +674,8 @@ constexpr int WPITCH = PC + 4;
 struct PwWgradParams {
   int Mo, C;             // channels of dy / of x
   int P, Ptot, SP;       // positions per image (dy), over all images; elements per x plane
-  int OW, rowstep, colstep, x_map;
+  int OW, x_map;         // x_map: x goes through the window geometry below
+  int H, W, KW, KHW, sy, sx, py, px, dly, dlx;
   int pps, nsplit;       // positions per slice (multiple of PC), slices
   int ctiles, mtiles;
   int E;                 // Mo * C
@@ -386,6 +695,7 @@ pointwise_wgrad_kernel(PwWgradParams p, const T* __restrict__ x, const T* __rest
   const int split = blockIdx.x;
   const int ctile = __builtin_amdgcn_readfirstlane(blockIdx.y % p.ctiles);
   const int mtile = __builtin_amdgcn_readfirstlane(blockIdx.y / p.ctiles);
+  const int tap = blockIdx.z;                            // one window tap per workgroup
   const int pos0 = split * p.pps;
   const int pos1 = min(pos0 + p.pps, p.Ptot);
   const int n = (pos1 - pos0 + PC - 1) / PC;
@@ -404,7 +714,8 @@ pointwise_wgrad_kernel(PwWgradParams p, const T* __restrict__ x, const T* __rest
       ni[e] = Pe / p.P;
       qi[e] = Pe - ni[e] * p.P;
     }
-    const bool do_db = p.want_db && ctile == 0;
+    const bool do_db = p.want_db && ctile == 0 && tap == 0;
+    const int tdh = (tap / p.KW) * p.dly - p.py, tdw = (tap % p.KW) * p.dlx - p.px;
     float dbs[2] = {0.f, 0.f};
     const int mrow = mtile * BM + row, crow = ctile * BM + row;
 
@@ -415,7 +726,15 @@ pointwise_wgrad_kernel(PwWgradParams p, const T* __restrict__ x, const T* __rest
       for (int e = 0; e < (VEC ? 1 : 4); ++e) {
         const bool ok = Pg + e < pos1;
         yo[e] = ok ? ni[e] * p.Mo * p.P + qi[e] : -1;
-        xo[e] = ok ? ni[e] * p.C * p.SP + (p.x_map ? lattice_w(p, qi[e]) : qi[e]) : -1;
+        int xq = qi[e];
+        bool okx = ok;
+        if (!VEC && p.x_map) {
+          const int oh = qi[e] / p.OW, ow = qi[e] - oh * p.OW;
+          const int ih = oh * p.sy + tdh, iw = ow * p.sx + tdw;
+          okx = ok && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
+          xq = ih * p.W + iw;
+        }
+        xo[e] = okx ? ni[e] * p.C * p.SP + xq : -1;
         qi[e] += PC;
         while (qi[e] >= p.P) {
           qi[e] -= p.P;
@@ -519,22 +838,27 @@ pointwise_wgrad_kernel(PwWgradParams p, const T* __restrict__ x, const T* __rest
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int m = mtile * BM + wm * 32 + i * 16 + 4 * fg + r;
-        if (m < p.Mo && ch < p.C) part[(size_t)m * p.C + ch] = acc[i][j][r];
+        if (m < p.Mo && ch < p.C) part[((size_t)m * p.C + ch) * p.KHW + tap] = acc[i][j][r];
       }
     }
 }
 
 bool pw_wgrad_plan(const ConvGeom& g, PwWgradParams* p) {
-  if (!pw_applies(g)) return false;
+  if (g.groups != 1) return false;
+  // 64-channel column tiles: with few input channels the kernel that flattens
+  // (channel, tap) into the columns wastes less
+  if (!pw_applies(g) && (g.C + BM - 1) / BM * BM * 2 > 3 * g.C) return false;
   p->Mo = g.K; p->C = g.C;
   p->P = g.OH * g.OW; p->Ptot = g.N * p->P; p->SP = g.H * g.W;
-  p->OW = g.OW; p->rowstep = g.sy * g.W; p->colstep = g.sx;
-  p->x_map = (g.sy != 1 || g.sx != 1) ? 1 : 0;
+  p->OW = g.OW;
+  p->H = g.H; p->W = g.W; p->KW = g.KW; p->KHW = g.KH * g.KW;
+  p->sy = g.sy; p->sx = g.sx; p->py = g.py; p->px = g.px; p->dly = g.dly; p->dlx = g.dlx;
+  p->x_map = (g.sy != 1 || g.sx != 1 || !pw_applies(g)) ? 1 : 0;
   p->ctiles = (g.C + BM - 1) / BM;
   p->mtiles = (g.K + BM - 1) / BM;
-  p->E = g.K * g.C;
-  const long long base = (long long)p->ctiles * p->mtiles;
-  if (base > 65535) return false;
+  p->E = g.K * g.C * p->KHW;
+  const long long base = (long long)p->ctiles * p->mtiles * p->KHW;
+  if ((long long)p->ctiles * p->mtiles > 65535 || p->KHW > 65535) return false;
   long long ns = 4ll * mfma_num_cus() / base;
   const long long max_ns = (p->Ptot + 255) / 256;
   if (ns > max_ns) ns = max_ns;
@@ -613,8 +937,9 @@ size_t mfma_pointwise_wgrad_ws(const ConvGeom& g) {
 }
 
 int mfma_pointwise_wgrad(const ConvGeom& g, int dtype, const void* x, const void* dy, float* dw,
-                         float* db, void* ws, size_t ws_bytes, hipStream_t s) {
+                         float* db, void* ws, size_t ws_bytes, bool windows, hipStream_t s) {
   if (!dw) return -1;   // bias gradient alone: the plain reduction kernel
+  if (!windows && !pw_applies(g)) return -1;
   PwWgradParams p{};
   if (!pw_wgrad_plan(g, &p)) return -1;
   const long long esz = dtype == FLHIP_F32 ? 4 : 2;
@@ -628,7 +953,7 @@ int mfma_pointwise_wgrad(const ConvGeom& g, int dtype, const void* x, const void
   // a single slice writes dw in place; its bias sums need a home of their own
   if (p.nsplit == 1 && db) return -1;
   float* out = p.nsplit > 1 ? static_cast<float*>(ws) : dw;
-  const dim3 grid((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles));
+  const dim3 grid((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles), (unsigned)p.KHW);
   const bool vec = !p.x_map && p.P % 4 == 0;
   if (dtype == FLHIP_F32) {
     if (vec)
@@ -651,6 +976,16 @@ int mfma_pointwise_wgrad(const ConvGeom& g, int dtype, const void* x, const void
     return check_launch("conv2d_bwd_filter 1x1 (reduce)");
   }
   return FLHIP_OK;
+}
+
+int mfma_tapped_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w, const float* bias,
+                         void* y, hipStream_t s) {
+  return launch_tapped<false>(g, dtype, x, w, bias, y, s);
+}
+
+int mfma_tapped_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
+                              hipStream_t s) {
+  return launch_tapped<true>(g, dtype, dy, w, nullptr, dx, s);
 }
 
 }  // namespace flhip
