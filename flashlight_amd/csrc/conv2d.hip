@@ -129,6 +129,14 @@ static bool algo_is(const char* name) {
 }
 static bool force_direct() { return algo_is("direct"); }
 
+// Stride-1 windows over long rows (the 21x1 speech layers: rows of 1500): the gather
+// kernel's one-position-per-thread loads are whole contiguous runs there and it
+// measures faster than the tapped GEMM, except for backward-data into few channels.
+static bool long_rows(const ConvGeom& g, bool bwd) {
+  if (algo_is("tapped")) return false;
+  return g.sy == 1 && g.sx == 1 && g.OW >= 64 && (!bwd || g.C >= 128);
+}
+
 static int make_geom(const flhip_conv_desc* d, ConvGeom* g) {
   int32_t OH, OW;
   const int rc = flhip_conv2d_out_dims(d, &OH, &OW);
@@ -179,7 +187,8 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
     if (r < 0 && !algo_is("gather")) r = mfma_pointwise_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r < 0 && !algo_is("gather")) r = mfma_slab_conv_fwd(g, d->dtype, x, w, bias, y, s);
-    if (r < 0 && !algo_is("gather")) r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s);
+    if (r < 0 && !algo_is("gather") && !long_rows(g, false))
+      r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r < 0) r = mfma_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r >= 0) return r;
   }
@@ -212,7 +221,8 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
     if (r < 0 && !algo_is("gather")) r = mfma_pointwise_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0 && !algo_is("gather")) r = mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s);
-    if (r < 0 && !algo_is("gather")) r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s);
+    if (r < 0 && !algo_is("gather") && !long_rows(g, true))
+      r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0) r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r >= 0) return r;
   }

@@ -354,6 +354,7 @@ int launch_pw(const PwParams& p, bool vec, const void* src, const void* wgt, con
 // Tiles are 64 channels x 64 positions of one class; loads and stores are element-wise.
 constexpr int MAX_CLASSES = 16;
 constexpr int MAX_TAPS = 128;          // over all classes
+constexpr int DEPTH = 2;               // chunks in flight per loader thread (even); 4 measured no faster
 
 struct TapClass {
   int tile0;             // first position tile of the class
@@ -384,12 +385,10 @@ tapped_conv_kernel(TapParams p, const T* __restrict__ src, const T* __restrict__
                    const float* __restrict__ bias, T* __restrict__ dst) {
   constexpr int PT = 2, BN = 32 * PT;
   constexpr int XPS = 2 * BN + 32;
-  constexpr int QN = BN / 4;
-  constexpr int JSTEP = LTHREADS / QN;
   constexpr int ASZ = BWD ? NPAIR * APS : BM * APW;
   constexpr int BUF = NPAIR * XPS + ASZ;
   constexpr int esz = (int)sizeof(T);
-  static_assert(JSTEP == NPAIR, "one sweep of the loader threads covers a chunk");
+  static_assert(BN == 64 && NPAIR == 16, "a loader wave covers 64 positions x 4 channel pairs");
   __shared__ float lds[2 * BUF];
 
   const int id = blockIdx.x, xcd = id & 7, seq = id >> 3;
@@ -408,69 +407,54 @@ tapped_conv_kernel(TapParams p, const T* __restrict__ src, const T* __restrict__
 
   if (wave < 4) {
     // ================================ loaders ====================================
+    // A thread owns one position of the tile (lane = position, so a wave's load of one
+    // channel is one contiguous run wherever the source step is 1) and the four channel
+    // pairs 4*wave .. 4*wave+3 of a chunk.
     const __amdgpu_buffer_rsrc_t srsrc = make_rsrc(src, p.src_bytes);
     const __amdgpu_buffer_rsrc_t wrsrc = make_rsrc(wgt, p.wgt_bytes);
-    const int pq = tid % QN, j0 = tid / QN;
     const int SPb = p.SH * p.SW * esz;
-    // per position: byte offset of (image, channel 0, row 0, column 0) and the source
-    // coordinates at shift (0, 0); a position past the class gets a row that fails
-    // every bounds test
-    int nb[4], sh0[4], sw0[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int Pe = tileP0 + 4 * pq + e;
+    int nb, sh0, sw0;
+    {
+      const int Pe = tileP0 + lane;
       const int ni = Pe / Pc, r = Pe - ni * Pc;
-      const int hc = r / Wc, wc = r - hc * Wc;
-      nb[e] = ni * p.Kc * SPb;
-      sh0[e] = Pe < Pctot ? hc * p.ssh + p.cls[cl].bh : -(1 << 24);
-      sw0[e] = wc * p.ssw + p.cls[cl].bw;
+      const int hc = r / Wc, wcl = r - hc * Wc;
+      nb = ni * p.Kc * SPb;
+      // a position past the class gets a row that fails every bounds test
+      sh0 = Pe < Pctot ? hc * p.ssh + p.cls[cl].bh : -(1 << 24);
+      sw0 = wcl * p.ssw + p.cls[cl].bw;
     }
-    const int wm = BWD ? (tid & 15) * 4 : tid >> 3;
-    const int wk = BWD ? (tid >> 4) * 2 : (tid & 7) * 4;
+    // weight tile: lanes run along the dimension whose stride is one tap group (KHW
+    // elements); forward (k = tid % 32, m = tid / 32 + 8i), backward (m = tid % 64,
+    // k = tid / 64 + 4i)
+    const int wl = BWD ? tid & 63 : tid & 31;
+    const int wo = BWD ? tid >> 6 : tid >> 5;
     const int m0 = mtile * BM;
     int kc = 0, ti = 0;                        // chunk = (channel chunk kc, tap ti), taps inner
 
-    auto load = [&](float4 (&sr)[2], float4 (&wr)[2]) {
+    auto load = [&](float (&sr)[8], float (&wr)[8]) {
       const Tap tp = p.taps[min(tap0 + ti, MAX_TAPS - 1)];
       const int k0 = kc * KC;
-      int so[4];
+      const int ih = sh0 + tp.dh, iw = sw0 + tp.dw;
+      const bool ok = (unsigned)ih < (unsigned)p.SH && (unsigned)iw < (unsigned)p.SW && ntaps > 0;
+      const int so = nb + (ih * p.SW + iw) * esz + (k0 + 8 * wave) * SPb;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int ih = sh0[e] + tp.dh, iw = sw0[e] + tp.dw;
-        const bool ok = (unsigned)ih < (unsigned)p.SH && (unsigned)iw < (unsigned)p.SW;
-        so[e] = ok ? nb[e] + (ih * p.SW + iw) * esz : OOB;
-      }
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int k = k0 + 2 * j0 + h;
-        const bool kok = k < p.Kc && ntaps > 0;
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = buf_ld(srsrc, (kok && so[e] != OOB) ? so[e] + k * SPb : OOB, src);
-        sr[h] = make_float4(v[0], v[1], v[2], v[3]);
-      }
-      const int tstep = p.KHW * esz;
+      for (int h = 0; h < 8; ++h)
+        sr[h] = buf_ld(srsrc, (ok && k0 + 8 * wave + h < p.Kc) ? so + h * SPb : OOB, src);
       if (!BWD) {
+        const int k = k0 + wl;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          const int m = m0 + wm + 32 * i, k = k0 + wk;
-          const int off = ((m * p.Kc + k) * p.KHW + tp.tmem) * esz;
-          float v[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            v[e] = buf_ld(wrsrc, (m < p.Mo && k + e < p.Kc && ntaps > 0) ? off + e * tstep : OOB, wgt);
-          wr[i] = make_float4(v[0], v[1], v[2], v[3]);
+        for (int i = 0; i < 8; ++i) {
+          const int m = m0 + wo + 8 * i;
+          wr[i] = buf_ld(wrsrc, (m < p.Mo && k < p.Kc && ntaps > 0) ? ((m * p.Kc + k) * p.KHW + tp.tmem) * esz : OOB,
+                         wgt);
         }
       } else {
+        const int m = m0 + wl;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const int k = k0 + wk + h, m = m0 + wm;
-          const int off = ((k * p.Mo + m) * p.KHW + tp.tmem) * esz;
-          float v[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            v[e] = buf_ld(wrsrc, (k < p.Kc && m + e < p.Mo && ntaps > 0) ? off + e * tstep : OOB, wgt);
-          wr[h] = make_float4(v[0], v[1], v[2], v[3]);
+        for (int i = 0; i < 8; ++i) {
+          const int k = k0 + wo + 4 * i;
+          wr[i] = buf_ld(wrsrc, (m < p.Mo && k < p.Kc && ntaps > 0) ? ((k * p.Mo + m) * p.KHW + tp.tmem) * esz : OOB,
+                         wgt);
         }
       }
       if (++ti >= ntaps) {
@@ -478,35 +462,39 @@ tapped_conv_kernel(TapParams p, const T* __restrict__ src, const T* __restrict__
         ++kc;                                   // chunks past the end read channels >= Kc: zeros
       }
     };
-    auto store = [&](int buf, const float4 (&sr)[2], const float4 (&wr)[2]) {
+    auto store = [&](int buf, const float (&sr)[8], const float (&wr)[8]) {
       float* xs = lds + buf * BUF;
       float* as = xs + NPAIR * XPS;
-      float4* d = reinterpret_cast<float4*>(xs + j0 * XPS + 8 * pq);
-      d[0] = make_float4(sr[0].x, sr[1].x, sr[0].y, sr[1].y);
-      d[1] = make_float4(sr[0].z, sr[1].z, sr[0].w, sr[1].w);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        *reinterpret_cast<float2*>(xs + (4 * wave + j) * XPS + 2 * lane) = make_float2(sr[2 * j], sr[2 * j + 1]);
       if (!BWD) {
-        *reinterpret_cast<float4*>(as + wm * APW + wk) = wr[0];
-        *reinterpret_cast<float4*>(as + (wm + 32) * APW + wk) = wr[1];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) as[(wo + 8 * i) * APW + wl] = wr[i];
       } else {
-        float4* a = reinterpret_cast<float4*>(as + (wk >> 1) * APS + 2 * wm);
-        a[0] = make_float4(wr[0].x, wr[1].x, wr[0].y, wr[1].y);
-        a[1] = make_float4(wr[0].z, wr[1].z, wr[0].w, wr[1].w);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int k = wo + 4 * i;
+          as[(k >> 1) * APS + 2 * wl + (k & 1)] = wr[i];
+        }
       }
     };
 
-    float4 srA[2], wrA[2], srB[2], wrB[2];
-    load(srA, wrA);
-    store(0, srA, wrA);
-    load(srB, wrB);
+    // DEPTH register sets: the loads of chunk c+DEPTH are issued while chunk c+1 is
+    // stored, so a load has DEPTH-1 chunk periods to come back
+    float sr[DEPTH][8], wr[DEPTH][8];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) load(sr[d], wr[d]);
+    store(0, sr[0], wr[0]);
     __syncthreads();
-    for (int c = 0; c < n; c += 2) {
-      load(srA, wrA);
-      store(1, srB, wrB);
-      __syncthreads();
-      if (c + 1 >= n) break;
-      load(srB, wrB);
-      store(0, srA, wrA);
-      __syncthreads();
+    for (int c = 0; c < n; c += DEPTH) {
+#pragma unroll
+      for (int u = 0; u < DEPTH; ++u) {
+        if (c + u >= n) break;
+        load(sr[u], wr[u]);                                          // chunk c+u+DEPTH
+        store((u + 1) & 1, sr[(u + 1) % DEPTH], wr[(u + 1) % DEPTH]);  // chunk c+u+1
+        __syncthreads();
+      }
     }
     return;
   }
