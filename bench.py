@@ -14,6 +14,7 @@ events on the stream the kernels are launched on (torch's current stream, whose
 handle is passed through the C ABI).
 """
 import argparse
+import ctypes as C
 import json
 import os
 import sys
@@ -37,6 +38,9 @@ def parse():
     ap.add_argument("--dtype", choices=["f32", "bf16"], default="f32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--only", default="", help="comma list of ops to time (debugging/profiling)")
+    ap.add_argument("--layers", choices=["resnet50", "speech"], default="",
+                    help="instead of the bench line: time every conv layer of configs[4] (ResNet-50, batch 32) "
+                         "or configs[3] (21x1 speech layers) in all three passes and print a table")
     return ap.parse_args()
 
 
@@ -55,6 +59,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     tdt = torch.float32 if a.dtype == "f32" else torch.bfloat16
+    if a.layers:
+        return layer_sweep(a, fa, torch, tdt)
     gen = torch.Generator(device=dev).manual_seed(0)
 
     def randn(*shape, scale=1.0, shift=0.0):
@@ -263,6 +269,80 @@ def main():
     out["cpu_onednn"] = cpu_onednn
     out["cpu_onednn_bandwidth_ops"] = cpu_bw
     print(json.dumps(out))
+    return 0
+
+
+# (count in the network, N, C, H, W, K, KH, KW, sy, sx, py, px); ResNet-50 v1.5 as built by
+# flashlight/pkg/vision/models/Resnet.cpp:210-230 (stride on the 3x3), batch 32
+RESNET50_LAYERS = [(1, 32, 3, 224, 224, 64, 7, 7, 2, 2, 3, 3)] + [
+    (cnt, 32, c, h, h, k, ks, ks, s, s, ks // 2, ks // 2) for (cnt, h, c, k, ks, s) in [
+        (1, 56, 64, 64, 1, 1), (4, 56, 64, 256, 1, 1), (2, 56, 256, 64, 1, 1), (3, 56, 64, 64, 3, 1),
+        (1, 56, 256, 128, 1, 1), (1, 56, 128, 128, 3, 2), (1, 56, 256, 512, 1, 2), (4, 28, 128, 512, 1, 1),
+        (3, 28, 512, 128, 1, 1), (3, 28, 128, 128, 3, 1), (1, 28, 512, 256, 1, 1), (1, 28, 256, 256, 3, 2),
+        (1, 28, 512, 1024, 1, 2), (6, 14, 256, 1024, 1, 1), (5, 14, 1024, 256, 1, 1), (5, 14, 256, 256, 3, 1),
+        (1, 14, 1024, 512, 1, 1), (1, 14, 512, 512, 3, 2), (1, 14, 1024, 2048, 1, 2), (3, 7, 512, 2048, 1, 1),
+        (2, 7, 2048, 512, 1, 1), (2, 7, 512, 512, 3, 1)]]
+# configs[3]: [1500, 1, 80, 16] through three 21x1 SAME convolutions, the last with stride 2
+SPEECH_LAYERS = [(1, 16, 80, 1, 1500, 250, 1, 21, 1, 1, 0, 10), (1, 16, 250, 1, 1500, 250, 1, 21, 1, 1, 0, 10),
+                 (1, 16, 250, 1, 1500, 250, 1, 21, 1, 2, 0, 10)]
+
+
+def layer_sweep(a, fa, torch, tdt):
+    """Per-layer times of the three conv passes through the C ABI (HIP events around
+    a.steps launches after a.warmup); the first layer of a network has no backward-data
+    in training (its input needs no gradient), so it is left out of the totals."""
+    capi, L = fa.capi, fa.capi.lib()
+    tag = capi.F32 if tdt == torch.float32 else capi.BF16
+    S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: C.c_void_p(t.data_ptr())
+
+    def timed(fn):
+        for _ in range(max(a.warmup, 1)):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(a.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / a.steps * 1e3
+
+    def chk(rc):
+        if rc != 0:
+            raise RuntimeError(L.flhip_last_error())
+
+    layers = RESNET50_LAYERS if a.layers == "resnet50" else SPEECH_LAYERS
+    tot, flops = [0.0, 0.0, 0.0], 0.0
+    print("| n | input NxCxHxW | K | window | stride | GFLOP | fwd us (TFLOP/s) | bwd-data us | bwd-filter us |")
+    print("|---|---|---|---|---|---|---|---|---|")
+    for i, (cnt, N, Ci, H, W, K, kh, kw, sy, sx, py, px) in enumerate(layers):
+        x = torch.randn(N, Ci, H, W, device="cuda").to(tdt)
+        w = (torch.randn(K, Ci, kh, kw, device="cuda") / (Ci * kh * kw) ** 0.5).to(tdt)
+        cd = capi.ConvDesc(N, Ci, H, W, K, kh, kw, sy, sx, py, px, 1, 1, 1, tag)
+        oh, ow = C.c_int32(), C.c_int32()
+        chk(L.flhip_conv2d_out_dims(C.byref(cd), C.byref(oh), C.byref(ow)))
+        y = torch.empty(N, K, oh.value, ow.value, device="cuda", dtype=tdt)
+        dy, dx = torch.randn_like(y), torch.empty_like(x)
+        dw = torch.empty(K, Ci, kh, kw, device="cuda")
+        nws = max(L.flhip_conv2d_workspace_bytes(C.byref(cd), p) for p in (capi.CONV_FWD, capi.CONV_BWD_DATA,
+                                                                           capi.CONV_BWD_FILTER))
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device="cuda")
+        gf = 2.0 * N * K * oh.value * ow.value * Ci * kh * kw / 1e9
+        t = [timed(lambda: chk(L.flhip_conv2d_fwd(C.byref(cd), P(x), P(w), None, P(y), P(ws), nws, S))),
+             timed(lambda: chk(L.flhip_conv2d_bwd_data(C.byref(cd), P(dy), P(w), P(dx), P(ws), nws, S))),
+             timed(lambda: chk(L.flhip_conv2d_bwd_filter(C.byref(cd), P(x), P(dy), P(dw), None, P(ws), nws, S)))]
+        first = i == 0
+        for j in range(3):
+            if not (first and j == 1):
+                tot[j] += cnt * t[j]
+                flops += cnt * gf
+        print("| %d | %dx%dx%dx%d | %d | %dx%d | %d,%d | %.2f | %.1f (%.1f) | %.1f (%.1f) | %.1f (%.1f) |" % (
+            cnt, N, Ci, H, W, K, kh, kw, sy, sx, gf, t[0], gf / t[0] * 1e3, t[1], gf / t[1] * 1e3, t[2],
+            gf / t[2] * 1e3), flush=True)
+    print("totals over the network (counts applied, first layer without bwd-data): fwd %.2f ms, bwd-data %.2f ms, "
+          "bwd-filter %.2f ms, sum %.2f ms for %.1f GFLOP = %.1f TFLOP/s (%s)" % (
+              tot[0] / 1e3, tot[1] / 1e3, tot[2] / 1e3, sum(tot) / 1e3, flops, flops / sum(tot) * 1e3, a.dtype))
     return 0
 
 
