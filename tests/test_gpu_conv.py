@@ -139,3 +139,97 @@ def test_invalid_arguments_raise():
         fa.conv2d(x, torch.zeros((4, 4, 9, 9), device="cuda"), None)   # kernel > input
     with pytest.raises(RuntimeError):
         fa.conv2d(x.double(), torch.zeros((4, 4, 3, 3), device="cuda").double(), None)
+
+
+# ---- full sizes of the BASELINE configurations ------------------------------------------
+# The CPU checker needs minutes at these sizes, so the device results are checked through
+# what does not depend on size: (1) randomly sampled result elements against their defining
+# sums written with torch indexing in float64 (shares no code with the kernels or the C
+# checker), (2) the adjoint identities <conv(x, w), dy> = <x, bwdData(dy, w)> = <w, bwdFilter(x, dy)>
+# over the whole tensors, (3) a one-tap identity filter reproduces the shifted input bit for bit.
+FULL = [
+    # x NCHW, w KCHW, stride, pad: configs[1] (the bench shape), then layers of configs[4] / configs[3]
+    ((32, 64, 56, 56), (64, 64, 3, 3), (1, 1), (1, 1)),
+    ((32, 64, 56, 56), (256, 64, 1, 1), (1, 1), (0, 0)),
+    ((32, 256, 56, 56), (512, 256, 1, 1), (2, 2), (0, 0)),
+    ((32, 128, 56, 56), (128, 128, 3, 3), (2, 2), (1, 1)),
+    ((32, 256, 14, 14), (256, 256, 3, 3), (1, 1), (1, 1)),
+    ((32, 512, 7, 7), (512, 512, 3, 3), (1, 1), (1, 1)),
+    ((32, 2048, 7, 7), (512, 2048, 1, 1), (1, 1), (0, 0)),
+    ((32, 3, 224, 224), (64, 3, 7, 7), (2, 2), (3, 3)),
+    ((16, 250, 1, 1500), (250, 250, 1, 21), (1, 2), (0, 10)),
+]
+
+
+def _sampled_refs(x, w, b, dy, st, pd, rng, nsamp=48):
+    """float64 definitions of randomly chosen elements of y, dx, dw (and all of db)."""
+    import torch.nn.functional as F
+    N, Cc, H, W = x.shape
+    K, _, KH, KW = w.shape
+    OH, OW = dy.shape[2], dy.shape[3]
+    x64, w64, dy64 = x.double(), w.double(), dy.double()
+    xp = F.pad(x64, (pd[1], pd[1], pd[0], pd[0]))
+    out = {"y": [], "dx": [], "dw": []}
+    for _ in range(nsamp):
+        n, k, oh, ow = (int(rng.integers(v)) for v in (N, K, OH, OW))
+        win = xp[n, :, oh * st[0]:oh * st[0] + KH, ow * st[1]:ow * st[1] + KW]
+        out["y"].append(((n, k, oh, ow), float((win * w64[k]).sum() + b[k].double())))
+        n, c, ih, iw = (int(rng.integers(v)) for v in (N, Cc, H, W))
+        acc = 0.0
+        for kh in range(KH):
+            for kw_ in range(KW):
+                th, tw = ih + pd[0] - kh, iw + pd[1] - kw_
+                if th % st[0] or tw % st[1]:
+                    continue
+                o_h, o_w = th // st[0], tw // st[1]
+                if 0 <= o_h < OH and 0 <= o_w < OW:
+                    acc += float((dy64[n, :, o_h, o_w] * w64[:, c, kh, kw_]).sum())
+        out["dx"].append(((n, c, ih, iw), acc))
+        k, c, kh, kw_ = (int(rng.integers(v)) for v in (K, Cc, KH, KW))
+        xs_ = xp[:, c, kh:kh + (OH - 1) * st[0] + 1:st[0], kw_:kw_ + (OW - 1) * st[1] + 1:st[1]]
+        out["dw"].append(((k, c, kh, kw_), float((xs_ * dy64[:, k]).sum())))
+    return out, dy64.sum(dim=(0, 2, 3))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", FULL)
+def test_full_size_properties(shape, dtype):
+    xs, ws, st, pd = shape
+    if dtype == torch.bfloat16 and shape is not FULL[0] and shape is not FULL[3]:
+        pytest.skip("bf16 at full size: the bench shape and one strided layer")
+    rng = np.random.default_rng(41)
+    gen = torch.Generator(device="cuda").manual_seed(41)
+    x = torch.randn(xs, device="cuda", generator=gen).to(dtype)
+    w = (torch.randn(ws, device="cuda", generator=gen) / (ws[1] * ws[2] * ws[3]) ** 0.5).to(dtype)
+    b = torch.rand(ws[0], device="cuda", generator=gen) * 2 - 1
+    kw = dict(sx=st[1], sy=st[0], px=pd[1], py=pd[0])
+    y = fa.conv2d(x, w, b, **kw)
+    dy = torch.randn(y.shape, device="cuda", generator=gen).to(dtype)
+    dx = fa.conv2d_backward_data(dy, xs, w, **kw)
+    dw, db = fa.conv2d_backward_filter_bias(dy, x, ws, True, **kw)
+    refs, db_ref = _sampled_refs(x, w, b, dy, st, pd, rng)
+    lo = dtype == torch.bfloat16
+    for name, got, tol in (("y", y, 4e-3 if lo else 1e-4), ("dx", dx, 4e-3 if lo else 1e-4), ("dw", dw, 1e-4)):
+        g = np.array([float(got[idx]) for idx, _ in refs[name]])
+        r = np.array([v for _, v in refs[name]])
+        assert rel_l2(g, r) <= tol, (name, rel_l2(g, r))
+    assert rel_l2(host(db), db_ref.cpu().numpy()) <= 1e-4
+    # adjoint identities over the whole tensors (float64 inner products on the device)
+    y_nb = fa.conv2d(x, w, None, **kw)
+    a = float((y_nb.double() * dy.double()).sum())
+    bdx = float((x.double() * dx.double()).sum())
+    cdw = float((w.double() * dw.double()).sum())
+    scale = float(y_nb.double().norm() * dy.double().norm())
+    tol = (3e-3 if lo else 2e-5) * scale
+    assert abs(a - cdw) <= tol and abs(a - bdx) <= tol, (a, bdx, cdw, scale)
+    # a filter with a single 1 copies the (shifted, strided) input exactly
+    kh, kw_ = ws[2] // 2, ws[3] - 1
+    wi = torch.zeros(ws, device="cuda")
+    nd = min(ws[0], ws[1])
+    wi[torch.arange(nd), torch.arange(nd), kh, kw_] = 1.0
+    yi = fa.conv2d(x, wi.to(dtype), None, **kw)
+    xp = torch.nn.functional.pad(x, (pd[1], pd[1], pd[0], pd[0]))
+    OH, OW = y.shape[2], y.shape[3]
+    want = xp[:, :nd, kh:kh + (OH - 1) * st[0] + 1:st[0], kw_:kw_ + (OW - 1) * st[1] + 1:st[1]]
+    assert torch.equal(yi[:, :nd], want)
+    assert not yi[:, nd:].any()
