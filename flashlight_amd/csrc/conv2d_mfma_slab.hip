@@ -592,7 +592,7 @@ bool plan(SlabParams* p, size_t* shmem, bool bwd, bool aligned) {
     p->stage_ok = p->DW % 4 == 0 && (size_t)32 * sp * sizeof(float) <= *shmem - BM * sizeof(float);
   }
   // a tile with few positions would leave the matrix cores idle: not worth it
-  return best_r * p->DW >= 64;
+  return best_r * p->DW >= 48;
 }
 
 template <typename T, bool BWD>

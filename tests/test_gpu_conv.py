@@ -40,6 +40,8 @@ MORE = [
     ((2, 40, 6, 16), (72, 40, 3, 3), (1, 1), (1, 1), (1, 1), 1),        # channel tails on both sides (bf16 matrix-core path)
     ((1, 96, 5, 8), (32, 48, 2, 3), (1, 1), (1, 1), (1, 1), 2),         # groups, 2x3 window (bf16 generic tap loop)
     ((1, 20, 6, 16), (24, 20, 3, 3), (1, 1), (1, 1), (1, 1), 1),        # bf16 matrix-core path, weights not 16-byte friendly
+    ((3, 32, 7, 7), (64, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),         # whole 7x7 planes per tile; rows of 7 and 14 in the
+    ((2, 64, 14, 14), (96, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),       # row-slab filter gradient (k-steps past the row end)
     # 1x1 as GEMM: positions across image boundaries, channel tails, odd planes (element-wise
     # path), strides (lattice on one side, zero fill of dx), several chunks of 32 channels
     ((3, 64, 12, 12), (128, 64, 1, 1), (1, 1), (0, 0), (1, 1), 1),
