@@ -693,93 +693,126 @@ pointwise_wgrad_kernel(PwWgradParams p, const T* __restrict__ x, const T* __rest
     // ================================ loaders ====================================
     const __amdgpu_buffer_rsrc_t xrsrc = make_rsrc(x, p.x_bytes);
     const __amdgpu_buffer_rsrc_t yrsrc = make_rsrc(dy, p.dy_bytes);
-    const int row = tid >> 3, kq = tid & 7;             // rows row and row + 32, positions 4kq..+3
-    // image and in-plane index of this thread's positions, advanced chunk by chunk
-    int ni[VEC ? 1 : 4], qi[VEC ? 1 : 4];
-#pragma unroll
-    for (int e = 0; e < (VEC ? 1 : 4); ++e) {
-      const int Pe = pos0 + 4 * kq + e;
-      ni[e] = Pe / p.P;
-      qi[e] = Pe - ni[e] * p.P;
-    }
     const bool do_db = p.want_db && ctile == 0 && tap == 0;
-    const int tdh = (tap / p.KW) * p.dly - p.py, tdw = (tap % p.KW) * p.dlx - p.px;
-    float dbs[2] = {0.f, 0.f};
-    const int mrow = mtile * BM + row, crow = ctile * BM + row;
-
-    auto load = [&](int c, float4 (&yr)[2], float4 (&xr)[2]) {
-      const int Pg = pos0 + c * PC + 4 * kq;
-      int yo[VEC ? 1 : 4], xo[VEC ? 1 : 4];    // element offsets of channel 0, -1 = past the slice
+    if (VEC) {
+      // ---- 16-byte loads: a thread owns rows `row` and `row + 32`, positions 4kq .. 4kq+3 ----
+      const int row = tid >> 3, kq = tid & 7;
+      int ni = (pos0 + 4 * kq) / p.P, qi = (pos0 + 4 * kq) - ni * p.P;
+      float dbs[2] = {0.f, 0.f};
+      const int mrow = mtile * BM + row, crow = ctile * BM + row;
+      auto load = [&](int c, float4 (&yr)[2], float4 (&xr)[2]) {
+        const bool ok = pos0 + c * PC + 4 * kq < pos1;
+        const int yo = ni * p.Mo * p.P + qi, xo = ni * p.C * p.SP + qi;
+        qi += PC;
+        while (qi >= p.P) {
+          qi -= p.P;
+          ++ni;
+        }
 #pragma unroll
-      for (int e = 0; e < (VEC ? 1 : 4); ++e) {
-        const bool ok = Pg + e < pos1;
-        yo[e] = ok ? ni[e] * p.Mo * p.P + qi[e] : -1;
-        int xq = qi[e];
+        for (int i = 0; i < 2; ++i) {
+          const int m = mrow + 32 * i, ch = crow + 32 * i;
+          yr[i] = buf_ld4(yrsrc, (ok && m < p.Mo) ? (yo + m * p.P) * esz : OOB, dy);
+          xr[i] = buf_ld4(xrsrc, (ok && ch < p.C) ? (xo + ch * p.SP) * esz : OOB, x);
+        }
+      };
+      auto store = [&](int buf, const float4 (&yr)[2], const float4 (&xr)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          *reinterpret_cast<float4*>(&lds[buf][0][(row + 32 * i) * WPITCH + 4 * kq]) = yr[i];
+          *reinterpret_cast<float4*>(&lds[buf][1][(row + 32 * i) * WPITCH + 4 * kq]) = xr[i];
+          if (do_db) dbs[i] += (yr[i].x + yr[i].y) + (yr[i].z + yr[i].w);
+        }
+      };
+      float4 yA[2], xA[2], yB[2], xB[2];
+      load(0, yA, xA);
+      store(0, yA, xA);
+      load(1, yB, xB);
+      __syncthreads();
+      for (int c = 0; c < n; c += 2) {
+        load(c + 2, yA, xA);
+        store(1, yB, xB);                        // chunk c+1 (zeros past the slice)
+        __syncthreads();
+        if (c + 1 >= n) break;
+        load(c + 3, yB, xB);
+        store(0, yA, xA);                        // chunk c+2
+        __syncthreads();
+      }
+      if (do_db) {
+        // the 8 threads that share a row are neighbours in the wave
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          float v = dbs[i];
+          v += __shfl_xor(v, 1, 64);
+          v += __shfl_xor(v, 2, 64);
+          v += __shfl_xor(v, 4, 64);
+          const int m = mrow + 32 * i;
+          if (kq == 0 && m < p.Mo) part[p.E + m] = v;
+        }
+      }
+    } else {
+      // ---- element-wise loads: a lane owns one position of the chunk (so a wave's load
+      // of a row is a contiguous run wherever the geometry allows) and rows r0 + 8i ----
+      const int pl = tid & 31, r0 = tid >> 5;
+      int ni = (pos0 + pl) / p.P, qi = (pos0 + pl) - ni * p.P;
+      const int tdh = (tap / p.KW) * p.dly - p.py, tdw = (tap % p.KW) * p.dlx - p.px;
+      float dbs[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      const int mrow = mtile * BM + r0, crow = ctile * BM + r0;
+      auto load = [&](int c, float (&yr)[8], float (&xr)[8]) {
+        const bool ok = pos0 + c * PC + pl < pos1;
+        const int yo = ni * p.Mo * p.P + qi;
+        int xq = qi;
         bool okx = ok;
-        if (!VEC && p.x_map) {
-          const int oh = qi[e] / p.OW, ow = qi[e] - oh * p.OW;
+        if (p.x_map) {
+          const int oh = qi / p.OW, ow = qi - oh * p.OW;
           const int ih = oh * p.sy + tdh, iw = ow * p.sx + tdw;
           okx = ok && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
           xq = ih * p.W + iw;
         }
-        xo[e] = okx ? ni[e] * p.C * p.SP + xq : -1;
-        qi[e] += PC;
-        while (qi[e] >= p.P) {
-          qi[e] -= p.P;
-          ++ni[e];
+        const int xo = ni * p.C * p.SP + xq;
+        qi += PC;
+        while (qi >= p.P) {
+          qi -= p.P;
+          ++ni;
         }
-      }
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int m = mrow + 32 * i, ch = crow + 32 * i;
-        if (VEC) {
-          yr[i] = buf_ld4(yrsrc, (yo[0] >= 0 && m < p.Mo) ? (yo[0] + m * p.P) * esz : OOB, dy);
-          xr[i] = buf_ld4(xrsrc, (xo[0] >= 0 && ch < p.C) ? (xo[0] + ch * p.SP) * esz : OOB, x);
-        } else {
-          float a[4], b[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            a[e] = buf_ld(yrsrc, (yo[VEC ? 0 : e] >= 0 && m < p.Mo) ? (yo[VEC ? 0 : e] + m * p.P) * esz : OOB, dy);
-            b[e] = buf_ld(xrsrc, (xo[VEC ? 0 : e] >= 0 && ch < p.C) ? (xo[VEC ? 0 : e] + ch * p.SP) * esz : OOB, x);
-          }
-          yr[i] = make_float4(a[0], a[1], a[2], a[3]);
-          xr[i] = make_float4(b[0], b[1], b[2], b[3]);
+        for (int i = 0; i < 8; ++i) {
+          const int m = mrow + 8 * i, ch = crow + 8 * i;
+          yr[i] = buf_ld(yrsrc, (ok && m < p.Mo) ? (yo + m * p.P) * esz : OOB, dy);
+          xr[i] = buf_ld(xrsrc, (okx && ch < p.C) ? (xo + ch * p.SP) * esz : OOB, x);
         }
-      }
-    };
-    auto store = [&](int buf, const float4 (&yr)[2], const float4 (&xr)[2]) {
+      };
+      auto store = [&](int buf, const float (&yr)[8], const float (&xr)[8]) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        *reinterpret_cast<float4*>(&lds[buf][0][(row + 32 * i) * WPITCH + 4 * kq]) = yr[i];
-        *reinterpret_cast<float4*>(&lds[buf][1][(row + 32 * i) * WPITCH + 4 * kq]) = xr[i];
-        if (do_db) dbs[i] += (yr[i].x + yr[i].y) + (yr[i].z + yr[i].w);
+        for (int i = 0; i < 8; ++i) {
+          lds[buf][0][(r0 + 8 * i) * WPITCH + pl] = yr[i];
+          lds[buf][1][(r0 + 8 * i) * WPITCH + pl] = xr[i];
+          if (do_db) dbs[i] += yr[i];
+        }
+      };
+      float yA[8], xA[8], yB[8], xB[8];
+      load(0, yA, xA);
+      store(0, yA, xA);
+      load(1, yB, xB);
+      __syncthreads();
+      for (int c = 0; c < n; c += 2) {
+        load(c + 2, yA, xA);
+        store(1, yB, xB);
+        __syncthreads();
+        if (c + 1 >= n) break;
+        load(c + 3, yB, xB);
+        store(0, yA, xA);
+        __syncthreads();
       }
-    };
-
-    float4 yA[2], xA[2], yB[2], xB[2];
-    load(0, yA, xA);
-    store(0, yA, xA);
-    load(1, yB, xB);
-    __syncthreads();
-    for (int c = 0; c < n; c += 2) {
-      load(c + 2, yA, xA);
-      store(1, yB, xB);                        // chunk c+1 (zeros past the slice)
-      __syncthreads();
-      if (c + 1 >= n) break;
-      load(c + 3, yB, xB);
-      store(0, yA, xA);                        // chunk c+2
-      __syncthreads();
-    }
-    if (do_db) {
-      // the 8 threads that share a row are neighbours in the wave
+      if (do_db) {
+        // the 32 lanes that share a row are one half of a wave
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        float v = dbs[i];
-        v += __shfl_xor(v, 1, 64);
-        v += __shfl_xor(v, 2, 64);
-        v += __shfl_xor(v, 4, 64);
-        const int m = mrow + 32 * i;
-        if (kq == 0 && m < p.Mo) part[p.E + m] = v;
+        for (int i = 0; i < 8; ++i) {
+          float v = dbs[i];
+#pragma unroll
+          for (int o = 1; o < 32; o <<= 1) v += __shfl_xor(v, o, 64);
+          const int m = mrow + 8 * i;
+          if (pl == 0 && m < p.Mo) part[p.E + m] = v;
+        }
       }
     }
     return;
