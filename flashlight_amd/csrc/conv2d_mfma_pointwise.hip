@@ -116,21 +116,15 @@ pointwise_conv_kernel(PwParams p, const T* __restrict__ src, const T* __restrict
     const __amdgpu_buffer_rsrc_t wrsrc = make_rsrc(wgt, p.wgt_bytes);
     const int pq = tid % QN, j0 = tid / QN;
     const int SPb = p.SP * esz;
-    // byte offset of channel 0 at this thread's four positions; OOB past the end
-    int sb[VEC ? 1 : 4];
+    // 16-byte path: byte offset of channel 0 at this thread's four positions; element-wise
+    // path: a lane owns one position of the tile (a wave's load of one channel is then a
+    // contiguous run wherever the map allows) and the wave the channel pairs 4*wave .. +3
+    static_assert(VEC || PT == 2, "the element-wise loaders assume 64 positions per tile");
+    int sb;
     {
-      const int Pg = tileP0 + 4 * pq;
-      if (VEC) {
-        const int ni = Pg / p.P, q = Pg - ni * p.P;
-        sb[0] = Pg < p.Ptot ? (ni * p.Kc * p.SP + q) * esz : OOB;
-      } else {
-#pragma unroll
-        for (int e = 0; e < (VEC ? 1 : 4); ++e) {
-          const int Pe = Pg + e;
-          const int ni = Pe / p.P, q = Pe - ni * p.P;
-          sb[e] = Pe < p.Ptot ? (ni * p.Kc * p.SP + (p.src_map ? lattice(p, q) : q)) * esz : OOB;
-        }
-      }
+      const int Pg = VEC ? tileP0 + 4 * pq : tileP0 + lane;
+      const int ni = Pg / p.P, q = Pg - ni * p.P;
+      sb = Pg < p.Ptot ? (ni * p.Kc * p.SP + ((!VEC && p.src_map) ? lattice(p, q) : q)) * esz : OOB;
     }
     // weight tile shares: forward (m, 4 consecutive k), backward (pair, 4 consecutive m)
     const int wm = BWD ? (tid & 15) * 4 : tid >> 3;       // backward: first of 4 channels
@@ -139,21 +133,26 @@ pointwise_conv_kernel(PwParams p, const T* __restrict__ src, const T* __restrict
 
     auto load = [&](int c, float4 (&sr)[NJ][2], float4 (&wr)[2]) {
       const int k0 = c * KC;
+      if (VEC) {
 #pragma unroll
-      for (int i = 0; i < NJ; ++i) {
+        for (int i = 0; i < NJ; ++i) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int k = k0 + 2 * (j0 + i * JSTEP) + h;
+            sr[i][h] = buf_ld4(srsrc, (k < p.Kc && sb != OOB) ? sb + k * SPb : OOB, src);
+          }
+        }
+      } else {
+        // sr[0][h] = channels k0 + 8*wave + 4h .. +3 at this lane's position
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-          const int k = k0 + 2 * (j0 + i * JSTEP) + h;
-          const bool kok = k < p.Kc;
-          if (VEC) {
-            sr[i][h] = buf_ld4(srsrc, (kok && sb[0] != OOB) ? sb[0] + k * SPb : OOB, src);
-          } else {
-            float v[4];
+          float v[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              v[e] = buf_ld(srsrc, (kok && sb[VEC ? 0 : e] != OOB) ? sb[VEC ? 0 : e] + k * SPb : OOB, src);
-            sr[i][h] = make_float4(v[0], v[1], v[2], v[3]);
+          for (int e = 0; e < 4; ++e) {
+            const int k = k0 + 8 * wave + 4 * h + e;
+            v[e] = buf_ld(srsrc, (k < p.Kc && sb != OOB) ? sb + k * SPb : OOB, src);
           }
+          sr[0][h] = make_float4(v[0], v[1], v[2], v[3]);
         }
       }
       if (!BWD) {
@@ -193,11 +192,19 @@ pointwise_conv_kernel(PwParams p, const T* __restrict__ src, const T* __restrict
     auto store = [&](int buf, const float4 (&sr)[NJ][2], const float4 (&wr)[2]) {
       float* xs = lds + buf * BUF;
       float* as = xs + NPAIR * XPS;
+      if (VEC) {
 #pragma unroll
-      for (int i = 0; i < NJ; ++i) {
-        float4* d = reinterpret_cast<float4*>(xs + (j0 + i * JSTEP) * XPS + 8 * pq);
-        d[0] = make_float4(sr[i][0].x, sr[i][1].x, sr[i][0].y, sr[i][1].y);
-        d[1] = make_float4(sr[i][0].z, sr[i][1].z, sr[i][0].w, sr[i][1].w);
+        for (int i = 0; i < NJ; ++i) {
+          float4* d = reinterpret_cast<float4*>(xs + (j0 + i * JSTEP) * XPS + 8 * pq);
+          d[0] = make_float4(sr[i][0].x, sr[i][1].x, sr[i][0].y, sr[i][1].y);
+          d[1] = make_float4(sr[i][0].z, sr[i][1].z, sr[i][0].w, sr[i][1].w);
+        }
+      } else {
+        float* d = xs + 4 * wave * XPS + 2 * lane;
+        *reinterpret_cast<float2*>(d) = make_float2(sr[0][0].x, sr[0][0].y);
+        *reinterpret_cast<float2*>(d + XPS) = make_float2(sr[0][0].z, sr[0][0].w);
+        *reinterpret_cast<float2*>(d + 2 * XPS) = make_float2(sr[0][1].x, sr[0][1].y);
+        *reinterpret_cast<float2*>(d + 3 * XPS) = make_float2(sr[0][1].z, sr[0][1].w);
       }
       if (!BWD) {
         *reinterpret_cast<float4*>(as + wm * APW + wk) = wr[0];
@@ -334,8 +341,6 @@ int launch_pw(const PwParams& p, bool vec, const void* src, const void* wgt, con
     if (pt == 4) return launch_tile<T, BWD, 4, true>(p, src, wgt, bias, dst, s);
     return launch_tile<T, BWD, 2, true>(p, src, wgt, bias, dst, s);
   }
-  if (pt == 8) return launch_tile<T, BWD, 8, false>(p, src, wgt, bias, dst, s);
-  if (pt == 4) return launch_tile<T, BWD, 4, false>(p, src, wgt, bias, dst, s);
   return launch_tile<T, BWD, 2, false>(p, src, wgt, bias, dst, s);
 }
 
