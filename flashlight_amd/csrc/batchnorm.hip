@@ -471,6 +471,106 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
   });
 }
 
+// ---- resident kernels for rows that are not 16-byte friendly (inner % 4 != 0) -----------
+// Same idea with one element per slot: a workgroup owns a feature, a thread holds K
+// elements of x (and, backward, of dy) in registers, lanes walk consecutive elements so
+// a wave's load is a contiguous run.  Forward moves 2T bytes, backward exactly 3T.
+__device__ __forceinline__ void buf_st(__amdgpu_buffer_rsrc_t r, int byte_off, float v, float*) {
+  __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, byte_off, 0, 0);
+}
+__device__ __forceinline__ void buf_st(__amdgpu_buffer_rsrc_t r, int byte_off, float v, bf16_t*) {
+  __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16(v), r, byte_off, 0, 0);
+}
+
+// byte offsets of this thread's elements e = tid + THREADS*k of feature blockIdx.x;
+// out-of-range slots get an offset past the descriptor (loads give 0, stores are dropped)
+template <int THREADS, int K, int ESZ>
+__device__ __forceinline__ void res1_offsets(const BnGeom& g, int (&off)[K]) {
+  constexpr int OOB = (int)0x80000000;
+  const int inner = (int)g.inner, c = blockIdx.x;
+  int q = threadIdx.x;
+  int o = q / inner, i = q - o * inner;
+  const int so = THREADS / inner, si = THREADS - so * inner;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    off[k] = q < (int)g.units ? ((o * (int)g.C + c) * inner + i) * ESZ : OOB;
+    q += THREADS;
+    o += so;
+    i += si;
+    if (i >= inner) {
+      i -= inner;
+      ++o;
+    }
+  }
+}
+
+template <typename T, int THREADS, int K>
+__global__ void __launch_bounds__(THREADS)
+bn_train_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restrict__ y,
+                   BnTrainArgs a) {
+  __shared__ float red[THREADS / 64];
+  __shared__ float sh[2];
+  constexpr int OOB = (int)0x80000000;
+  const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
+  const long long c = blockIdx.x;
+  const float shift = ld(x, (size_t)(c * g.inner));
+  int off[K];
+  res1_offsets<THREADS, K, (int)sizeof(T)>(g, off);
+  float xv[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) xv[k] = buf_ld(xr_, off[k], x);
+  float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    const float t = off[k] != OOB ? xv[k] - shift : 0.f;
+    s1 += t;
+    s2 += t * t;
+  }
+  s1 = block_sum(s1, red);
+  s2 = block_sum(s2, red);
+  finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh);
+  __syncthreads();
+  const float mean = sh[0];
+  const float scale = (a.gamma ? a.gamma[c] : 1.f) * sh[1];
+  const float bt = a.beta ? a.beta[c] : 0.f;
+#pragma unroll
+  for (int k = 0; k < K; ++k) buf_st(yr_, off[k], (xv[k] - mean) * scale + bt, y);
+}
+
+template <typename T, int THREADS, int K>
+__global__ void __launch_bounds__(THREADS)
+bn_bwd_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, const T* __restrict__ dy,
+                 T* __restrict__ dx, BnBwdArgs a) {
+  __shared__ float red[THREADS / 64];
+  __shared__ float sh[4];
+  const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes),
+                               dxr_ = make_rsrc(dx, bytes);
+  const long long c = blockIdx.x;
+  const float mean = a.save_mean[c];
+  int off[K];
+  res1_offsets<THREADS, K, (int)sizeof(T)>(g, off);
+  float xv[K], dv[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    xv[k] = buf_ld(xr_, off[k], x);
+    dv[k] = buf_ld(dyr_, off[k], dy);
+  }
+  float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+  for (int k = 0; k < K; ++k) {
+    // out-of-range slots loaded zeros for dy, so they add nothing
+    s1 += dv[k];
+    s2 += dv[k] * (xv[k] - mean);
+  }
+  s1 = block_sum(s1, red);
+  s2 = block_sum(s2, red);
+  finish_bwd(g, a, c, (double)s1, (double)s2, true, sh);
+  __syncthreads();
+  const float kdy = sh[1], kx = sh[2], k0 = sh[3];
+#pragma unroll
+  for (int k = 0; k < K; ++k) buf_st(dxr_, off[k], kdy * dv[k] + (kx * (xv[k] - mean) + k0), dx);
+}
+
 // ---- column mode (inner == 1) ----------------------------------------------
 // block = 64 features x 4 row lanes; grid = (ceil(C/64), S); slice s owns rows
 // [s*ups, (s+1)*ups).
@@ -650,7 +750,18 @@ static ResPlan resident_plan(const BnGeom& g, int vec, int min_c) {
     return 0;
   }();
   ResPlan r{0, 0, 0};
-  if (mode == 1 || vec != 4) return r;
+  if (mode == 1 || vec == 0) return r;
+  if (vec == 1) {
+    // element-wise variant: up to 32 elements per thread
+    if (g.units > 32 * 1024 || g.inner > 0x7fffffff) return r;
+    if (g.outer * g.C * g.inner * 4 >= (1ll << 31)) return r;
+    if (mode != 2 && g.C < min_c) return r;
+    r.threads = g.units <= 8 * 256 ? 256 : 1024;
+    const int need = (int)((g.units + r.threads - 1) / r.threads);
+    r.k = need <= 8 ? 8 : need <= 16 ? 16 : 32;
+    r.need = need;
+    return r;
+  }
   if (g.units > (long long)RES_KMAX * 1024) return r;
   if (g.outer * g.C * g.inner * 4 >= (1ll << 31)) return r;   // 32-bit buffer offsets
   if (mode != 2 && g.C < min_c) return r;
@@ -702,6 +813,19 @@ static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws
   T* yp = static_cast<T*>(y);
   {
     const ResPlan r = resident_plan(g, vec, RES_MIN_C_FWD);
+    if (vec == 1 && r.threads) {
+      const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
+      const dim3 grid((unsigned)g.C);
+      if (r.threads == 256)
+        hipLaunchKernelGGL((bn_train_resident1<T, 256, 8>), grid, dim3(256), 0, s, g, bytes, xp, yp, a);
+      else if (r.k == 8)
+        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 8>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a);
+      else if (r.k == 16)
+        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 16>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a);
+      else
+        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 32>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a);
+      return check_launch("bn_fwd_train (resident, element-wise)");
+    }
     if (r.threads == 256) return launch_train_resident<T, 256, 8>(g, xp, yp, a, s);
     if (r.threads == 1024) {
       if (r.k == 8) return launch_train_resident<T, 1024, 8>(g, xp, yp, a, s);
@@ -735,6 +859,19 @@ static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void
   T* dxp = static_cast<T*>(dx);
   {
     const ResPlan r = resident_plan(g, vec, RES_MIN_C_BWD);
+    if (vec == 1 && r.threads) {
+      const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
+      const dim3 grid((unsigned)g.C);
+      if (r.threads == 256)
+        hipLaunchKernelGGL((bn_bwd_resident1<T, 256, 8>), grid, dim3(256), 0, s, g, bytes, xp, dyp, dxp, a);
+      else if (r.k == 8)
+        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 8>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a);
+      else if (r.k == 16)
+        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 16>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a);
+      else
+        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 32>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a);
+      return check_launch("bn_bwd (resident, element-wise)");
+    }
     if (r.threads == 256) return launch_bwd_resident<T, 256, 8>(g, r.need, xp, dyp, dxp, a, s);
     if (r.threads == 1024) {
       if (r.k == 8) return launch_bwd_resident<T, 1024, 8>(g, r.need, xp, dyp, dxp, a, s);

@@ -27,6 +27,12 @@ CASES = [
     ((28, 28, 128, 20), [2]),       # one workgroup of 1024 threads per feature, 8 vectors per thread
     ((56, 56, 128, 11), [2]),       # ... 16 vectors per thread
     ((56, 56, 128, 22), [2]),       # ... 25 vectors per thread, part of dy re-read
+    # rows that are not 16-byte friendly: element-wise resident kernels
+    ((4, 130, 7, 7), [2]),          # 256 threads, mostly idle slots
+    ((32, 128, 7, 7), [2]),         # the 7x7 planes of the last ResNet stage
+    ((12, 128, 1, 750), [2]),       # speech rows after the stride-2 layer, 16 elements per thread
+    ((5, 128, 53, 101), [2]),       # 32 elements per thread
+    ((3, 64, 9, 9), [2]),           # forward resident, backward split (fewer than 128 features)
 ]
 
 
