@@ -40,7 +40,7 @@ def _compile(src):
 
 HOST = os.path.join(HERE, "host")
 HOST_LIB = os.path.join(LIBDIR, "libflhip_host.so")
-HOST_SOURCES = ["HipTensor.cpp", "HipAutogradExtension.cpp", "Functions.cpp", "Modules.cpp"]
+HOST_SOURCES = ["HipTensor.cpp", "HipAutogradExtension.cpp", "Functions.cpp", "Modules.cpp", "Resnet.cpp"]
 HOST_TEST_SRC = os.path.join(ROOT, "tests", "cpp", "test_host_extension.cpp")
 HOST_TEST_BIN = os.path.join(ROOT, "tests", "cpp", "bin", "test_host_extension")
 
@@ -64,6 +64,12 @@ def build_host(verbose=True):
                      "-L" + LIBDIR, "-lflhip_host", "-lflhip", "-L" + oracle, "-lflref",
                      "-Wl,-rpath,$ORIGIN/../../../flashlight_amd/lib",
                      "-Wl,-rpath,$ORIGIN/../../../oracle"] + hiplibs
+        subprocess.check_call(cmd)
+        # the ResNet-50 step program needs no CPU checker
+        rsrc = os.path.join(os.path.dirname(HOST_TEST_SRC), "test_resnet_step.cpp")
+        rbin = os.path.join(os.path.dirname(HOST_TEST_BIN), "test_resnet_step")
+        cmd = cxx + ["-o", rbin, rsrc, "-L" + LIBDIR, "-lflhip_host", "-lflhip",
+                     "-Wl,-rpath,$ORIGIN/../../../flashlight_amd/lib"] + hiplibs
         subprocess.check_call(cmd)
     if verbose:
         print("built", HOST_LIB)

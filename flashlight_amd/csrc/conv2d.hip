@@ -128,6 +128,12 @@ static bool algo_is(const char* name) {
   return e && strcmp(e, name) == 0;
 }
 static bool force_direct() { return algo_is("direct"); }
+// FLHIP_CONV_SKIP = comma list of kernel families to leave out of the dispatch
+// (bf16, gemm1x1, slab, tapped): a measurement / debugging aid like FLHIP_CONV_ALGO
+static bool skip(const char* name) {
+  const char* e = getenv("FLHIP_CONV_SKIP");
+  return algo_is("gather") || (e && strstr(e, name) != nullptr);
+}
 
 // Stride-1 windows over long rows (the 21x1 speech layers: rows of 1500): the gather
 // kernel's one-position-per-thread loads are whole contiguous runs there and it
@@ -182,12 +188,12 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
   hipStream_t s = as_stream(stream);
   if (!force_direct()) {
     int r = -1;
-    if (d->dtype == FLHIP_BF16 && !algo_is("gather") && !algo_is("convert"))
+    if (d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
       r = mfma_slab16_conv_fwd(g, x, w, bias, y, s);
-    if (r < 0 && !algo_is("gather")) r = mfma_pointwise_conv_fwd(g, d->dtype, x, w, bias, y, s);
+    if (r < 0 && !skip("gemm1x1")) r = mfma_pointwise_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s);
-    if (r < 0 && !algo_is("gather")) r = mfma_slab_conv_fwd(g, d->dtype, x, w, bias, y, s);
-    if (r < 0 && !algo_is("gather") && !long_rows(g, false))
+    if (r < 0 && !skip("slab")) r = mfma_slab_conv_fwd(g, d->dtype, x, w, bias, y, s);
+    if (r < 0 && !skip("tapped") && !long_rows(g, false))
       r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r < 0) r = mfma_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r >= 0) return r;
@@ -216,12 +222,12 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
   hipStream_t s = as_stream(stream);
   if (!force_direct()) {
     int r = -1;
-    if (d->dtype == FLHIP_BF16 && !algo_is("gather") && !algo_is("convert"))
+    if (d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
       r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s);
-    if (r < 0 && !algo_is("gather")) r = mfma_pointwise_conv_bwd_data(g, d->dtype, dy, w, dx, s);
+    if (r < 0 && !skip("gemm1x1")) r = mfma_pointwise_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s);
-    if (r < 0 && !algo_is("gather")) r = mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s);
-    if (r < 0 && !algo_is("gather") && !long_rows(g, true))
+    if (r < 0 && !skip("slab")) r = mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s);
+    if (r < 0 && !skip("tapped") && !long_rows(g, true))
       r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0) r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r >= 0) return r;
@@ -253,12 +259,12 @@ extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, 
     const size_t need = flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER);
     FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter: workspace too small");
     int r = -1;
-    if (d->dtype == FLHIP_BF16 && !algo_is("gather") && !algo_is("convert"))
+    if (d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
       r = mfma_wgrad16(g, x, dy, dw, db, ws, ws_bytes, s);
-    if (r < 0 && !algo_is("gather"))
+    if (r < 0 && !skip("gemm1x1"))
       r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, algo_is("tapped"), s);
-    if (r < 0 && !algo_is("gather")) r = mfma_slab_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
-    if (r < 0 && !algo_is("gather")) r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, true, s);
+    if (r < 0 && !skip("slab")) r = mfma_slab_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
+    if (r < 0 && !skip("tapped")) r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, true, s);
     if (r < 0) r = mfma_conv_bwd_filter(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
     if (r >= 0) return r;
   }

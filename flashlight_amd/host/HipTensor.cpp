@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 
 #include <cstring>
+#include <map>
+#include <mutex>
 
 #include "flhip.h"
 
@@ -15,6 +17,71 @@ void hipCheck(hipError_t e, const char* what) {
 }
 void* g_stream = nullptr;
 
+// Freed buffers are kept and handed out again by size class instead of going back to the
+// driver: hipFree waits for the device, and a training step frees hundreds of
+// intermediate tensors.  Reuse needs no event because every kernel of this backend is
+// enqueued on the one backend stream, in program order.  Flashlight has a caching memory
+// manager in the same place (flashlight/fl/memory/managers/CachingMemoryManager.cpp).
+class DevicePool {
+ public:
+  static DevicePool& get() {
+    static DevicePool* pool = new DevicePool;   // never destroyed: the HIP runtime may be gone by then
+    return *pool;
+  }
+  static size_t sizeClass(size_t n) {
+    const size_t q = n < (1u << 20) ? 512 : (1u << 20);
+    return (n + q - 1) / q * q;
+  }
+  void* take(size_t n, size_t* granted) {
+    const size_t cls = sizeClass(n);
+    *granted = cls;
+    {
+      std::lock_guard<std::mutex> lock(mu_);
+      auto it = free_.find(cls);
+      if (it != free_.end() && !it->second.empty()) {
+        void* p = it->second.back();
+        it->second.pop_back();
+        cached_ -= cls;
+        return p;
+      }
+    }
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, cls);
+    if (e != hipSuccess) {
+      // out of memory with buffers parked here: give them back and try once more
+      (void)hipGetLastError();
+      release();
+      e = hipMalloc(&p, cls);
+    }
+    hipCheck(e, "hipMalloc");
+    return p;
+  }
+  void give(void* p, size_t cls) {
+    std::lock_guard<std::mutex> lock(mu_);
+    free_[cls].push_back(p);
+    cached_ += cls;
+  }
+  void release() {
+    std::map<size_t, std::vector<void*>> all;
+    {
+      std::lock_guard<std::mutex> lock(mu_);
+      all.swap(free_);
+      cached_ = 0;
+    }
+    for (auto& kv : all)
+      for (void* p : kv.second) (void)hipFree(p);
+  }
+  size_t cachedBytes() {
+    std::lock_guard<std::mutex> lock(mu_);
+    return cached_;
+  }
+
+ private:
+  std::mutex mu_;
+  std::map<size_t, std::vector<void*>> free_;
+  size_t cached_ = 0;
+};
+
 int tag(dtype t) {
   if (t == dtype::f32) return FLHIP_F32;
   if (t == dtype::bf16) return FLHIP_BF16;
@@ -23,11 +90,18 @@ int tag(dtype t) {
 }  // namespace
 
 void* hipBackendStream() { return g_stream; }
-void setHipBackendStream(void* stream) { g_stream = stream; }
+void setHipBackendStream(void* stream) {
+  // cached buffers are reused in program order of one stream: drain the old one first
+  if (stream != g_stream) sync();
+  g_stream = stream;
+}
 void sync() { hipCheck(hipStreamSynchronize((hipStream_t)g_stream), "sync"); }
 
+void emptyDeviceCache() { DevicePool::get().release(); }
+size_t deviceCacheBytes() { return DevicePool::get().cachedBytes(); }
+
 Tensor::Buffer::~Buffer() {
-  if (ptr) (void)hipFree(ptr);
+  if (ptr) DevicePool::get().give(ptr, bytes);
 }
 
 Tensor::Tensor(const Shape& shape, dtype type) : shape_(shape), type_(type) {
@@ -35,8 +109,7 @@ Tensor::Tensor(const Shape& shape, dtype type) : shape_(shape), type_(type) {
   if (shape.elements() < 0) throw std::invalid_argument("Tensor: negative dimension");
   if (n == 0) return;
   buf_ = std::make_shared<Buffer>();
-  hipCheck(hipMalloc(&buf_->ptr, n), "hipMalloc");
-  buf_->bytes = n;
+  buf_->ptr = DevicePool::get().take(n, &buf_->bytes);   // bytes = the size class granted
 }
 
 Tensor Tensor::fromHost(const Shape& shape, dtype type, const void* data) {

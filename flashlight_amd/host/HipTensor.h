@@ -72,6 +72,10 @@ class DevicePtr {
 
 // The stream every kernel of this backend is enqueued on (hipStream_t as void*;
 // nullptr = the null stream), and fl::sync() for it.
+// Device buffers of destroyed tensors are cached for reuse; these return them to the
+// driver / report how many bytes are parked.
+void emptyDeviceCache();
+size_t deviceCacheBytes();
 void* hipBackendStream();
 void setHipBackendStream(void* stream);
 void sync();

@@ -19,6 +19,19 @@ def test_host_extension_program():
     assert "all host extension checks passed" in r.stdout
 
 
+@pytest.mark.gpu
+def test_resnet50_step_program():
+    """ResNet-50 forward + backward from the host modules at batch 2: shapes, gradients for
+    all 161 parameter tensors, matrix-core kernels against the direct kernels end to end."""
+    exe = os.path.join(ROOT, "tests", "cpp", "bin", "test_resnet_step")
+    assert os.path.exists(exe), "build it with `python -m flashlight_amd.build`"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=110)
+    print(r.stdout)
+    print(r.stderr)
+    assert r.returncode == 0, r.stdout[-3000:]
+    assert "ResNet-50 step checks passed" in r.stdout
+
+
 def test_host_library_is_built_and_links_the_c_abi():
     lib = os.path.join(ROOT, "flashlight_amd", "lib", "libflhip_host.so")
     assert os.path.exists(lib)
