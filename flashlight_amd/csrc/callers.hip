@@ -7,6 +7,7 @@
 // Matrices are column-major like Flashlight tensors: element (r, c) of an R x C
 // matrix is at r + c*R.
 #include "common.h"
+#include "conv2d.h"
 
 namespace flhip {
 namespace {
@@ -309,6 +310,13 @@ extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, in
   FLHIP_REQUIRE(A && B && C, "matmul: null argument");
   FLHIP_REQUIRE(M > 0 && N > 0 && K > 0, "matmul: sizes must be positive");
   FLHIP_REQUIRE(dtype_ok(dtype), "matmul: unknown dtype");
+  // the matrix-core kernels of the 1x1 convolutions take the three products fl::linear
+  // needs; the tiled vector-ALU kernel below covers the rest
+  if (!(trans_a && trans_b) && !getenv("FLHIP_MATMUL_VALU")) {
+    const int rc = mfma_gemm(dtype, trans_a ? 1 : trans_b ? 2 : 0, A, B, C, M, N, K, bias_rows,
+                             as_stream(stream));
+    if (rc >= 0) return rc;
+  }
   const dim3 grid((unsigned)((M + GT - 1) / GT), (unsigned)((N + GT - 1) / GT));
   FLHIP_REQUIRE(grid.y <= 65535, "matmul: too many columns");
   if (dtype == FLHIP_F32)

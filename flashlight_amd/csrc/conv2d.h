@@ -37,7 +37,11 @@ int mfma_slab_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const 
 int mfma_pointwise_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w,
                             const float* bias, void* y, hipStream_t s);
 int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w,
-                                 void* dx, hipStream_t s);
+                                 void* dx, hipStream_t s, const float* bias = nullptr);
+// column-major C = op(A) op(B) on the 1x1 kernels (mode 0: A B, 1: A^T B, 2: A B^T);
+// -1 when it does not apply
+int mfma_gemm(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,
+              const float* bias_rows, hipStream_t s);
 // windows with several taps on the same tile machinery, any stride / padding / dilation
 int mfma_tapped_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w,
                          const float* bias, void* y, hipStream_t s);

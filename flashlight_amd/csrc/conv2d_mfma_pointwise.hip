@@ -921,7 +921,7 @@ int mfma_pointwise_conv_fwd(const ConvGeom& g, int dtype, const void* x, const v
 }
 
 int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
-                                 hipStream_t s) {
+                                 hipStream_t s, const float* bias) {
   if (!pw_applies(g)) return -1;
   const long long esz = dtype == FLHIP_F32 ? 4 : 2;
   const long long sb = (long long)g.N * g.K * g.OH * g.OW * esz, db = (long long)g.N * g.C * g.H * g.W * esz;
@@ -952,8 +952,8 @@ int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, c
       hipLaunchKernelGGL((zero_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, static_cast<bf16_t*>(dx), n16, nel);
   }
   const bool vec = full && p.P % 4 == 0;
-  return dtype == FLHIP_F32 ? launch_pw<float, true>(p, vec, dy, w, nullptr, dx, s)
-                            : launch_pw<bf16_t, true>(p, vec, dy, w, nullptr, dx, s);
+  return dtype == FLHIP_F32 ? launch_pw<float, true>(p, vec, dy, w, bias, dx, s)
+                            : launch_pw<bf16_t, true>(p, vec, dy, w, bias, dx, s);
 }
 
 size_t mfma_pointwise_wgrad_ws(const ConvGeom& g) {
@@ -1012,6 +1012,36 @@ int mfma_tapped_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void
 int mfma_tapped_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
                               hipStream_t s) {
   return launch_tapped<true>(g, dtype, dy, w, nullptr, dx, s);
+}
+
+// Column-major matrix products on the same kernels: a matrix with its columns as
+// "images" of one position each is a 1x1-convolution operand.
+//   mode 0, C = A B    : A (M x K) is stored [k][m] = backward-data weights, B [n][k], C [n][m]
+//   mode 1, C = A^T B  : A stored (K x M) = [m][k] = forward weights
+//   mode 2, C = A B^T  : B stored (N x K) = [k][n]; C[n][m] = sum_k B[k][n] A[k][m] is the filter
+//                        gradient with the rows of B as dy and of A as x (fp32 only: that kernel
+//                        writes fp32; single slice only: there is no workspace here)
+// bias_rows (fp32[M] or null) is added to every column in modes 0 and 1.  Returns -1 when
+// the product does not fit these kernels.
+int mfma_gemm(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,
+              const float* bias_rows, hipStream_t s) {
+  ConvGeom g{};
+  g.H = g.W = g.OH = g.OW = g.KH = g.KW = 1;
+  g.sy = g.sx = g.dly = g.dlx = g.groups = 1;
+  if (mode == 0) {
+    g.N = N; g.C = M; g.K = K; g.Cg = M; g.Kg = K;
+    return mfma_pointwise_conv_bwd_data(g, dtype, B, A, C, s, bias_rows);
+  }
+  if (mode == 1) {
+    g.N = N; g.C = K; g.K = M; g.Cg = K; g.Kg = M;
+    return mfma_pointwise_conv_fwd(g, dtype, B, A, bias_rows, C, s);
+  }
+  if (mode == 2 && dtype == FLHIP_F32 && !bias_rows) {
+    g.N = K; g.C = M; g.K = N; g.Cg = M; g.Kg = N;
+    if (mfma_pointwise_wgrad_ws(g) != 0) return -1;
+    return mfma_pointwise_wgrad(g, dtype, A, B, static_cast<float*>(C), nullptr, nullptr, 0, false, s);
+  }
+  return -1;
 }
 
 }  // namespace flhip
