@@ -49,7 +49,7 @@ def build_host(verbose=True):
     """The C++ host layer (HipTensor, HipAutogradExtension, caller closures) and its
     test program; both link libflhip.so, the test also links the CPU checker."""
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
-    cxx = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-Wall", "-D__HIP_PLATFORM_AMD__",
+    cxx = [os.environ.get("CXX", "g++"), "-O2", "-g", "-rdynamic", "-std=c++17", "-Wall", "-D__HIP_PLATFORM_AMD__",
            "-I" + os.path.join(rocm, "include"), "-I" + os.path.join(ROOT, "include"), "-I" + HOST]
     hiplibs = ["-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(rocm, "lib")]
     cmd = cxx + ["-fPIC", "-shared", "-o", HOST_LIB]

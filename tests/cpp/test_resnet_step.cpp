@@ -5,6 +5,9 @@
 // With arguments `<batch> <steps>`: times the step (forward, loss, backward).
 #include <chrono>
 #include <cmath>
+#include <csignal>
+#include <execinfo.h>
+#include <unistd.h>
 #include <cstdio>
 #include <cstdlib>
 #include <random>
@@ -43,7 +46,20 @@ static Variable step(Sequential& model, const Variable& in, const Variable& targ
   return loss;
 }
 
+// a crash of the host code should say where: unbuffered output and a backtrace
+static void onCrash(int sig) {
+  void* frames[64];
+  const int n = backtrace(frames, 64);
+  const char msg[] = "host test: fatal signal, backtrace:\n";
+  (void)!write(2, msg, sizeof(msg) - 1);
+  backtrace_symbols_fd(frames, n, 2);
+  _exit(128 + sig);
+}
+
 int main(int argc, char** argv) {
+  std::setvbuf(stdout, nullptr, _IONBF, 0);
+  std::signal(SIGSEGV, onCrash);
+  std::signal(SIGBUS, onCrash);
   try {
     const int B = argc > 1 ? std::atoi(argv[1]) : 2;
     const int steps = argc > 2 ? std::atoi(argv[2]) : 0;
@@ -66,7 +82,8 @@ int main(int argc, char** argv) {
       const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / steps;
       std::printf("forward + loss + backward: %.2f ms per step (batch %d, %.1f images/s), loss %.4f, "
                   "device cache %.1f MB\n", ms, B, B / ms * 1e3, last, deviceCacheBytes() / 1e6);
-      return 0;
+      std::fflush(stdout);
+      _exit(0);
     }
 
     int fail = 0;
@@ -107,7 +124,8 @@ int main(int argc, char** argv) {
       if (!(e <= tol)) { std::printf("FAILED: gradient %zu\n", i); ++fail; }
     }
     std::printf(fail ? "%d check(s) FAILED\n" : "ResNet-50 step checks passed\n", fail);
-    return fail ? 1 : 0;
+    std::fflush(stdout);
+    _exit(fail ? 1 : 0);   // no static destructors: see test_host_extension.cpp
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
     return 2;
