@@ -8,7 +8,8 @@
 //   flashlight/fl/test/nn/ModuleTest.cpp:338-353 (batching invariance),
 // one training step of the README MNIST convnet (README.md:45-84) through the tape, and
 // the nn modules over those functions (flashlight/fl/test/nn/ModuleTest.cpp:670-719 for
-// LayerNorm; Sequential, BatchNorm statistics, a ResNet bottleneck with its residual add).
+// LayerNorm; Sequential, BatchNorm statistics, a ResNet bottleneck with its residual add,
+// the 21x1 convolution / batch norm / ReLU stack of the speech configuration).
 #include <algorithm>
 #include <cmath>
 #include <csignal>
@@ -634,6 +635,80 @@ static void testBottleneck() {
   CHECK(throws<std::invalid_argument>([&] { t3 + c1(in); }));   // shapes differ
 }
 
+// configs[3]: three (Conv 21x1 SAME -> BatchNorm over axis 2 -> ReLU) layers on [T, 1, 80, B],
+// channels 80 -> 250 -> 250 -> 250, strides 1, 1, 2 along time, from modules; forward and
+// backward against the CPU checker (T shortened so the checker stays fast).
+static void testSpeechStack() {
+  std::printf("speech stack (21x1 convolutions, batch norm, ReLU)\n");
+  const int T = 180, B = 3, chans[4] = {80, 250, 250, 250}, strides[3] = {1, 1, 2};
+  setSeed(17);
+  std::vector<Conv2D> convs;
+  std::vector<BatchNorm> bns;
+  for (int l = 0; l < 3; ++l) {
+    convs.emplace_back(chans[l], chans[l + 1], 21, 1, strides[l], 1, PaddingMode::SAME, PaddingMode::SAME);
+    bns.emplace_back(2, chans[l + 1]);
+  }
+  auto x = randn((size_t)B * 80 * T, 71);
+  Variable in(Tensor::fromVector({T, 1, 80, B}, x), true);
+  Variable h = in;
+  for (int l = 0; l < 3; ++l) h = relu(bns[l](convs[l](h)));
+  const int Tout = T / 2;
+  CHECK(h.shape() == Shape({Tout, 1, 250, B}));
+  auto dy = randn((size_t)B * 250 * Tout, 72);
+  h.backward(Variable(Tensor::fromVector(h.shape(), dy), false));
+
+  // ---- CPU checker: keep every layer's tensors for the way back ----------------------
+  struct Layer {
+    flref_conv d;
+    std::vector<float> in, a, n, r, w, b, g, z, mean, var;
+    int64_t hw;
+  };
+  std::vector<Layer> L(3);
+  std::vector<float> cur = x;
+  int t = T;
+  for (int l = 0; l < 3; ++l) {
+    Layer& y = L[l];
+    const int pad = derivePadding(t, 21, strides[l], -1, 1);
+    y.d = flref_conv{B, chans[l], 1, t, chans[l + 1], 1, 21, 1, strides[l], 0, pad, 1, 1, 1};
+    int32_t oh, ow;
+    flref_conv_out(&y.d, &oh, &ow);
+    y.hw = (int64_t)oh * ow;
+    const size_t no = (size_t)B * chans[l + 1] * y.hw;
+    y.in = cur;
+    y.w = hostOf(convs[l].param(0)); y.b = hostOf(convs[l].param(1));
+    y.g = hostOf(bns[l].param(0)); y.z = hostOf(bns[l].param(1));
+    y.a.resize(no); y.n.resize(no); y.r.resize(no); y.mean.resize(chans[l + 1]); y.var.resize(chans[l + 1]);
+    flref_conv2d_fwd(&y.d, y.in.data(), y.w.data(), y.b.data(), y.a.data());
+    flref_bn_fwd_train(B, chans[l + 1], y.hw, y.a.data(), y.g.data(), y.z.data(), 1e-5, y.n.data(), y.mean.data(), y.var.data());
+    flref_relu_fwd((int64_t)no, y.n.data(), y.r.data());
+    cur = y.r;
+    t = ow;
+  }
+  CHECK(t == Tout && relL2(hostOf(h), cur) <= 1e-4);
+  std::vector<float> grad = dy;
+  for (int l = 2; l >= 0; --l) {
+    Layer& y = L[l];
+    const size_t no = y.a.size();
+    std::vector<float> gn(no), ga(no), dg(chans[l + 1]), dbn(chans[l + 1]), dw(y.w.size()), dbias(chans[l + 1]), gin(y.in.size());
+    flref_relu_bwd((int64_t)no, grad.data(), y.n.data(), gn.data());
+    flref_bn_bwd(B, chans[l + 1], y.hw, y.a.data(), gn.data(), y.g.data(), y.mean.data(), y.var.data(), 1e-5, ga.data(),
+                 dg.data(), dbn.data());
+    flref_conv2d_bwd_filter(&y.d, y.in.data(), ga.data(), dw.data(), dbias.data());
+    flref_conv2d_bwd_data(&y.d, ga.data(), y.w.data(), gin.data());
+    CHECK(relL2(hostOf(convs[l].param(0).grad()), dw) <= 3e-4);
+    CHECK(relL2(hostOf(bns[l].param(0).grad()), dg) <= 3e-4 && relL2(hostOf(bns[l].param(1).grad()), dbn) <= 3e-4);
+    // the bias gradient of a convolution followed by batch norm is zero up to rounding:
+    // compare it on the scale of the filter gradient
+    double num = 0, den = 0;
+    const auto gb = hostOf(convs[l].param(1).grad());
+    for (size_t i = 0; i < gb.size(); ++i) num += ((double)gb[i] - dbias[i]) * ((double)gb[i] - dbias[i]);
+    for (float v : dw) den += (double)v * v;
+    CHECK(std::sqrt(num) <= 1e-4 * std::sqrt(den));
+    grad = gin;
+  }
+  CHECK(relL2(hostOf(in.grad()), grad) <= 3e-4);
+}
+
 // a crash of the host code should say where: unbuffered output and a backtrace
 static void onCrash(int sig) {
   void* frames[64];
@@ -666,6 +741,7 @@ int main() {
     testBatchNormModule();
     testLayerNormModule();
     testBottleneck();
+    testSpeechStack();
     fl::sync();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
