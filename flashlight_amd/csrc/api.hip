@@ -27,12 +27,9 @@ __global__ void __launch_bounds__(256) convert_kernel(const S* __restrict__ src,
     st(dst, i, ld(src, i));
 }
 
-template <typename T>
-__global__ void __launch_bounds__(256) add_kernel(const T* a, const T* b, T* out, size_t n) {
-  const size_t stride = (size_t)gridDim.x * 256;
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
-    st(out, i, ld(a, i) + ld(b, i));
-}
+struct OpAdd {
+  __device__ float operator()(float a, float b) const { return a + b; }
+};
 
 }  // namespace flhip
 
@@ -115,13 +112,9 @@ extern "C" int flhip_add(const void* a, const void* b, void* out, size_t n, int 
   FLHIP_REQUIRE(dtype_ok(dtype), "add: unknown dtype");
   if (n == 0) return FLHIP_OK;
   FLHIP_REQUIRE(a && b && out, "add: null pointer");
-  size_t blocks = (n + 255) / 256;
-  if (blocks > 16384) blocks = 16384;
   if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((add_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
-                       (const float*)a, (const float*)b, (float*)out, n);
+    launch_elementwise((const float*)a, (const float*)b, (float*)out, n, OpAdd{}, as_stream(stream));
   else
-    hipLaunchKernelGGL((add_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0,
-                       as_stream(stream), (const bf16_t*)a, (const bf16_t*)b, (bf16_t*)out, n);
+    launch_elementwise((const bf16_t*)a, (const bf16_t*)b, (bf16_t*)out, n, OpAdd{}, as_stream(stream));
   return check_launch("add");
 }

@@ -13,24 +13,12 @@ namespace flhip {
 namespace {
 
 // ---- ReLU = max(x, 0) and its mask backward (Functions.cpp:329-338, 1787-1789) ----
-template <typename T>
-__global__ void __launch_bounds__(256) relu_fwd_kernel(const T* __restrict__ x, T* __restrict__ y,
-                                                       size_t n) {
-  const size_t stride = (size_t)gridDim.x * 256;
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
-    const float v = ld(x, i);
-    st(y, i, v > 0.f ? v : 0.f);       // fl::maximum(x, 0): NaN compares false -> 0
-  }
-}
-
-template <typename T>
-__global__ void __launch_bounds__(256) relu_bwd_kernel(const T* __restrict__ dy,
-                                                       const T* __restrict__ x,
-                                                       T* __restrict__ dx, size_t n) {
-  const size_t stride = (size_t)gridDim.x * 256;
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
-    st(dx, i, ld(x, i) > 0.f ? ld(dy, i) : 0.f);
-}
+struct OpRelu {      // fl::maximum(x, 0): NaN compares false -> 0
+  __device__ float operator()(float x, float) const { return x > 0.f ? x : 0.f; }
+};
+struct OpReluBwd {   // (dy, x) -> dy where x > 0
+  __device__ float operator()(float dy, float x) const { return x > 0.f ? dy : 0.f; }
+};
 
 // ---- C = op(A) op(B) (+ bias per row), 64 x 64 tiles, 256 threads, 4 x 4 per thread ----
 constexpr int GT = 64, GK = 16;
@@ -282,11 +270,9 @@ extern "C" int flhip_relu_fwd(const void* x, void* y, size_t n, int dtype, void*
   FLHIP_REQUIRE(dtype_ok(dtype), "relu: unknown dtype");
   if (n == 0) return FLHIP_OK;
   if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((relu_fwd_kernel<float>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream),
-                       (const float*)x, (float*)y, n);
+    launch_elementwise((const float*)x, (const float*)nullptr, (float*)y, n, OpRelu{}, as_stream(stream));
   else
-    hipLaunchKernelGGL((relu_fwd_kernel<bf16_t>), dim3(blocks_for(n)), dim3(256), 0,
-                       as_stream(stream), (const bf16_t*)x, (bf16_t*)y, n);
+    launch_elementwise((const bf16_t*)x, (const bf16_t*)nullptr, (bf16_t*)y, n, OpRelu{}, as_stream(stream));
   return check_launch("relu");
 }
 
@@ -296,11 +282,9 @@ extern "C" int flhip_relu_bwd(const void* dy, const void* x, void* dx, size_t n,
   FLHIP_REQUIRE(dtype_ok(dtype), "relu_bwd: unknown dtype");
   if (n == 0) return FLHIP_OK;
   if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((relu_bwd_kernel<float>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream),
-                       (const float*)dy, (const float*)x, (float*)dx, n);
+    launch_elementwise((const float*)dy, (const float*)x, (float*)dx, n, OpReluBwd{}, as_stream(stream));
   else
-    hipLaunchKernelGGL((relu_bwd_kernel<bf16_t>), dim3(blocks_for(n)), dim3(256), 0,
-                       as_stream(stream), (const bf16_t*)dy, (const bf16_t*)x, (bf16_t*)dx, n);
+    launch_elementwise((const bf16_t*)dy, (const bf16_t*)x, (bf16_t*)dx, n, OpReluBwd{}, as_stream(stream));
   return check_launch("relu_bwd");
 }
 

@@ -161,6 +161,46 @@ __device__ __forceinline__ float block_sum(float v, float* smem) {
   return r;
 }
 
+// ---- elementwise kernels ------------------------------------------------------------
+// out[i] = op(a[i], b[i]) (b may be null for a unary op), four elements per thread through
+// 16-byte (float) / 8-byte (bf16) accesses; launch_elementwise handles tails and pointers
+// that are not aligned for that with the element-wise kernel.  out may alias a or b.
+template <typename T, typename Op>
+__global__ void __launch_bounds__(256) ew_vec_kernel(const T* a, const T* b,
+                                                     T* out, size_t nvec, Op op) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += stride) {
+    const float4 va = ld4(a, 4 * i);
+    const float4 vb = b ? ld4(b, 4 * i) : va;
+    st4(out, 4 * i, make_float4(op(va.x, vb.x), op(va.y, vb.y), op(va.z, vb.z), op(va.w, vb.w)));
+  }
+}
+template <typename T, typename Op>
+__global__ void __launch_bounds__(256) ew_kernel(const T* a, const T* b,
+                                                 T* out, size_t n, Op op) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    const float va = ld(a, i);
+    st(out, i, op(va, b ? ld(b, i) : va));
+  }
+}
+template <typename T, typename Op>
+inline void launch_elementwise(const T* a, const T* b, T* out, size_t n, Op op, hipStream_t s) {
+  auto blocks = [](size_t work) {
+    size_t k = (work + 255) / 256;
+    return (unsigned)(k > 65536 ? 65536 : k < 1 ? 1 : k);
+  };
+  const uintptr_t al = 4 * sizeof(T);
+  const bool aligned = reinterpret_cast<uintptr_t>(a) % al == 0 && reinterpret_cast<uintptr_t>(out) % al == 0 &&
+                       (!b || reinterpret_cast<uintptr_t>(b) % al == 0);
+  const size_t nvec = aligned ? n / 4 : 0;
+  if (nvec) hipLaunchKernelGGL((ew_vec_kernel<T, Op>), dim3(blocks(nvec)), dim3(256), 0, s, a, b, out, nvec, op);
+  const size_t done = nvec * 4;
+  if (done < n)
+    hipLaunchKernelGGL((ew_kernel<T, Op>), dim3(blocks(n - done)), dim3(256), 0, s, a + done, b ? b + done : b,
+                       out + done, n - done, op);
+}
+
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
 inline bool dtype_ok(int32_t dt) { return dt == FLHIP_F32 || dt == FLHIP_BF16; }
