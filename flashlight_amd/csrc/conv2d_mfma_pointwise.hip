@@ -83,6 +83,34 @@ __device__ __forceinline__ void buf_st4v(__amdgpu_buffer_rsrc_t r, int byte_off,
   __builtin_amdgcn_raw_buffer_store_b64(t, r, byte_off, 0, 0);
 }
 
+// The MFMA waves' share of one chunk (32 contraction channels = 4 pair-steps): wave
+// (wp, wc) multiplies positions wp*16*PT .. by channels wc*32 .. out of the LDS buffer
+// `buf` (source tile, then weight tile) into its PT x 2 accumulator tiles.
+template <bool BWD, int PT>
+__device__ __forceinline__ void mfma_chunk(const float* buf, int wp, int wc, int fr, int fg,
+                                           floatx4 (&acc)[PT][2]) {
+  constexpr int XPS = 2 * 32 * PT + 32;
+  const float* xs = buf + fg * XPS + (wp * PT * 16 + fr) * 2;
+  const float* as = buf + NPAIR * XPS + (BWD ? fg * APS + (wc * 32 + fr) * 2 : (wc * 32 + fr) * APW + 2 * fg);
+#pragma unroll
+  for (int s = 0; s < KC / 8; ++s) {
+    float2 a[PT], b[2];
+#pragma unroll
+    for (int i = 0; i < PT; ++i) a[i] = *reinterpret_cast<const float2*>(xs + 4 * s * XPS + i * 32);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      b[j] = *reinterpret_cast<const float2*>(as + (BWD ? 4 * s * APS + j * 32 : j * 16 * APW + 8 * s));
+#pragma unroll
+    for (int i = 0; i < PT; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        // .x / .y: the even / odd channel of the lane group's pair = two k-steps
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].x, b[j].x, acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].y, b[j].y, acc[i][j], 0, 0, 0);
+      }
+  }
+}
+
 template <typename T, bool BWD, int PT, bool VEC>
 __global__ void __launch_bounds__(MFMA_THREADS)
 pointwise_conv_kernel(PwParams p, const T* __restrict__ src, const T* __restrict__ wgt,
@@ -245,26 +273,7 @@ pointwise_conv_kernel(PwParams p, const T* __restrict__ src, const T* __restrict
 
   __syncthreads();                             // chunk 0 is in buffer 0
   for (int c = 0; c < n; ++c) {
-    const float* xs = lds + (c & 1) * BUF + fg * XPS + (wp * PT * 16 + fr) * 2;
-    const float* as = lds + (c & 1) * BUF + NPAIR * XPS +
-                      (BWD ? fg * APS + (wc * 32 + fr) * 2 : (wc * 32 + fr) * APW + 2 * fg);
-#pragma unroll
-    for (int s = 0; s < KC / 8; ++s) {
-      float2 a[PT], b[2];
-#pragma unroll
-      for (int i = 0; i < PT; ++i)
-        a[i] = *reinterpret_cast<const float2*>(xs + 4 * s * XPS + i * 32);
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-        b[j] = *reinterpret_cast<const float2*>(as + (BWD ? 4 * s * APS + j * 32 : j * 16 * APW + 8 * s));
-#pragma unroll
-      for (int i = 0; i < PT; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].x, b[j].x, acc[i][j], 0, 0, 0);
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].y, b[j].y, acc[i][j], 0, 0, 0);
-        }
-    }
+    mfma_chunk<BWD, PT>(lds + (c & 1) * BUF, wp, wc, fr, fg, acc);
     __syncthreads();
   }
 
@@ -514,28 +523,9 @@ tapped_conv_kernel(TapParams p, const T* __restrict__ src, const T* __restrict__
 #pragma unroll
     for (int j = 0; j < 2; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  __syncthreads();
+  __syncthreads();                             // chunk 0 is in buffer 0
   for (int c = 0; c < n; ++c) {
-    const float* xs = lds + (c & 1) * BUF + fg * XPS + (wp * PT * 16 + fr) * 2;
-    const float* as = lds + (c & 1) * BUF + NPAIR * XPS +
-                      (BWD ? fg * APS + (wc * 32 + fr) * 2 : (wc * 32 + fr) * APW + 2 * fg);
-#pragma unroll
-    for (int s = 0; s < KC / 8; ++s) {
-      float2 a[PT], b[2];
-#pragma unroll
-      for (int i = 0; i < PT; ++i)
-        a[i] = *reinterpret_cast<const float2*>(xs + 4 * s * XPS + i * 32);
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-        b[j] = *reinterpret_cast<const float2*>(as + (BWD ? 4 * s * APS + j * 32 : j * 16 * APW + 8 * s));
-#pragma unroll
-      for (int i = 0; i < PT; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].x, b[j].x, acc[i][j], 0, 0, 0);
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].y, b[j].y, acc[i][j], 0, 0, 0);
-        }
-    }
+    mfma_chunk<BWD, PT>(lds + (c & 1) * BUF, wp, wc, fr, fg, acc);
     __syncthreads();
   }
 
