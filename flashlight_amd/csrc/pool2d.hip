@@ -361,6 +361,94 @@ pool_w3s2_bwd(PoolGeom g, const T* __restrict__ dy, const uint8_t* __restrict__ 
   }
 }
 
+// ---------------------------------------------------------------------------
+// Fast path: 2x2 window, stride 2, no padding, H % 2 == 0, W % 4 == 0 (the pooling of
+// the README convnet and of VGG-style networks).  Windows do not overlap: a thread owns
+// four input columns x two rows = two windows, reads / writes them as 16-byte vectors,
+// and every input element belongs to exactly one window, so the backward pass is a
+// plain streaming write.  Candidate order (kh, kw) and the strict comparison keep the
+// first-maximum rule and the summation order of the generic kernels.
+// ---------------------------------------------------------------------------
+template <typename T, int MODE>
+__global__ void __launch_bounds__(256)
+pool_w2s2_fwd(PoolGeom g, const T* __restrict__ x, T* __restrict__ y, uint8_t* __restrict__ argmax,
+              size_t items) {
+  const size_t it = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (it >= items) return;
+  const int TQ = g.W >> 2;
+  const int tq = (int)(it % TQ);
+  const size_t t = it / TQ;
+  const int oh = (int)(t % g.OH);
+  const size_t plane = t / g.OH;
+  const size_t xo = (plane * g.H + 2 * oh) * (size_t)g.W + 4 * tq;
+  const float4 r0 = ld4(x, xo), r1 = ld4(x, xo + g.W);
+  const float c[2][4] = {{r0.x, r0.y, r1.x, r1.y}, {r0.z, r0.w, r1.z, r1.w}};
+  float out[2];
+  int idx[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    if (MODE == FLHIP_POOL_MAX) {
+      float best = -FLT_MAX;
+      int bi = 0;
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        if (c[j][k] > best) {
+          best = c[j][k];
+          bi = k;
+        }
+      out[j] = best;
+      idx[j] = bi;
+    } else {
+      out[j] = (((c[j][0] + c[j][1]) + c[j][2]) + c[j][3]) / 4.f;
+      idx[j] = 0;
+    }
+  }
+  const size_t yo = (plane * g.OH + oh) * (size_t)g.OW + 2 * tq;
+  st2(y, yo, out[0], out[1]);
+  if (MODE == FLHIP_POOL_MAX && argmax)
+    *reinterpret_cast<uint16_t*>(argmax + yo) = (uint16_t)(idx[0] | (idx[1] << 8));
+}
+
+template <typename T, int MODE>
+__global__ void __launch_bounds__(256)
+pool_w2s2_bwd(PoolGeom g, const T* __restrict__ dy, const uint8_t* __restrict__ argmax,
+              T* __restrict__ dx, size_t items) {
+  const size_t it = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (it >= items) return;
+  const int TQ = g.W >> 2;
+  const int tq = (int)(it % TQ);
+  const size_t t = it / TQ;
+  const int oh = (int)(t % g.OH);
+  const size_t plane = t / g.OH;
+  const size_t yo = (plane * g.OH + oh) * (size_t)g.OW + 2 * tq;
+  const float2 d = ld2(dy, yo);
+  float v[2][4];
+  if (MODE == FLHIP_POOL_MAX) {
+    const uint16_t am = *reinterpret_cast<const uint16_t*>(argmax + yo);
+    const int i0 = am & 0xff, i1 = am >> 8;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      v[0][k] = i0 == k ? d.x : 0.f;
+      v[1][k] = i1 == k ? d.y : 0.f;
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      v[0][k] = d.x / 4.f;
+      v[1][k] = d.y / 4.f;
+    }
+  }
+  const size_t xo = (plane * g.H + 2 * oh) * (size_t)g.W + 4 * tq;
+  st4(dx, xo, make_float4(v[0][0], v[0][1], v[1][0], v[1][1]));
+  st4(dx, xo + g.W, make_float4(v[0][2], v[0][3], v[1][2], v[1][3]));
+}
+
+static bool w2s2_applies(const PoolGeom& g, const void* a, const void* b, const void* am) {
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b);
+  return g.wy == 2 && g.wx == 2 && g.sy == 2 && g.sx == 2 && g.py == 0 && g.px == 0 &&
+         g.W % 4 == 0 && g.H % 2 == 0 && bits % 16 == 0 && reinterpret_cast<uintptr_t>(am) % 2 == 0;
+}
+
 static bool w3s2_applies(const PoolGeom& g, const void* a, const void* b, const void* am) {
   const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b);
   return g.wy == 3 && g.wx == 3 && g.sy == 2 && g.sx == 2 && g.py == 1 && g.px == 1 &&
@@ -374,6 +462,15 @@ static int launch_fwd(const PoolGeom& g, int mode, const void* x, void* y,
   const dim3 grid((unsigned)((total + 255) / 256)), block(256);
   const T* xp = static_cast<const T*>(x);
   T* yp = static_cast<T*>(y);
+  if (w2s2_applies(g, x, y, argmax)) {
+    const size_t items = (size_t)g.N * g.C * g.OH * (g.W / 4);
+    const dim3 fgrid((unsigned)((items + 255) / 256));
+    if (mode == FLHIP_POOL_MAX)
+      hipLaunchKernelGGL((pool_w2s2_fwd<T, FLHIP_POOL_MAX>), fgrid, block, 0, s, g, xp, yp, argmax, items);
+    else   // no padding: both average modes divide by 4
+      hipLaunchKernelGGL((pool_w2s2_fwd<T, FLHIP_POOL_AVG_INCLUDE_PADDING>), fgrid, block, 0, s, g, xp, yp, argmax, items);
+    return check_launch("pool2d_fwd");
+  }
   if (w3s2_applies(g, x, y, argmax)) {
     const int TQ = g.W / 4, nstrips = (g.OH + POOL_OHB - 1) / POOL_OHB;
     const size_t items = (size_t)g.N * g.C * nstrips * TQ;
@@ -410,6 +507,15 @@ static int launch_bwd(const PoolGeom& g, int mode, const void* dy,
   const dim3 grid((unsigned)((total + 255) / 256)), block(256);
   const T* dyp = static_cast<const T*>(dy);
   T* dxp = static_cast<T*>(dx);
+  if (w2s2_applies(g, dy, dx, argmax)) {
+    const size_t items = (size_t)g.N * g.C * g.OH * (g.W / 4);
+    const dim3 fgrid((unsigned)((items + 255) / 256));
+    if (mode == FLHIP_POOL_MAX)
+      hipLaunchKernelGGL((pool_w2s2_bwd<T, FLHIP_POOL_MAX>), fgrid, block, 0, s, g, dyp, argmax, dxp, items);
+    else
+      hipLaunchKernelGGL((pool_w2s2_bwd<T, FLHIP_POOL_AVG_INCLUDE_PADDING>), fgrid, block, 0, s, g, dyp, argmax, dxp, items);
+    return check_launch("pool2d_bwd");
+  }
   if (w3s2_applies(g, dy, dx, argmax)) {
     const int TQ = g.W / 4, nstrips = (g.OH + POOL_OHB - 1) / POOL_OHB;
     const size_t items = (size_t)g.N * g.C * nstrips * TQ;

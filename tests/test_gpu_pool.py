@@ -24,6 +24,10 @@ MORE = [
     ((2, 3, 37, 24), (3, 3), (2, 2), (1, 1)),     # fast path, odd height, short last strip
     ((5, 3, 2, 4), (3, 3), (2, 2), (1, 1)),       # fast path, tiny planes
     ((1, 2, 18, 8), (3, 3), (2, 2), (1, 1)),
+    ((3, 5, 56, 56), (2, 2), (2, 2), (0, 0)),     # 2x2 stride 2: non-overlapping fast path
+    ((2, 3, 6, 260), (2, 2), (2, 2), (0, 0)),     # ... rows wider than a wave
+    ((2, 3, 7, 8), (2, 2), (2, 2), (0, 0)),       # odd height: generic kernels
+    ((2, 3, 8, 6), (2, 2), (2, 2), (0, 0)),       # W % 4 != 0: generic kernels
 ]
 ALL = GEOMS + MORE
 
