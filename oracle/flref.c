@@ -513,3 +513,250 @@ void flref_cce_bwd(int classes, int cols, const float* grad, const int32_t* targ
       dx[(size_t)c * classes + k] = (t != ignore && k == t) ? (float)(-g) : 0.f;
   }
 }
+
+
+/* ---- rnn / rnnBackward ------------------------------------------------------------- */
+static int rnn_gates(int mode) { return mode == 2 ? 4 : mode == 3 ? 3 : 1; }
+
+int64_t flref_rnn_param_count(const flref_rnn* d) {
+  const int64_t G = rnn_gates(d->mode), H = d->hidden, D = d->bidirectional ? 2 : 1;
+  int64_t n = 0;
+  for (int l = 0; l < d->layers; ++l) {
+    const int64_t in = l == 0 ? d->input_size : D * H;
+    n += D * (G * H * (in + H) + 2 * G * H);
+  }
+  return n;
+}
+
+/* offsets of pseudo-layer pl inside the flat weight vector */
+static void rnn_offsets(const flref_rnn* d, int pl, int64_t* W, int64_t* R, int64_t* bW, int64_t* bR) {
+  const int64_t G = rnn_gates(d->mode), H = d->hidden, D = d->bidirectional ? 2 : 1;
+  int64_t off = 0, mats = 0;
+  for (int p = 0; p < d->layers * D; ++p) {
+    const int64_t in = p / D == 0 ? d->input_size : D * H;
+    if (p == pl) {
+      *W = off;
+      *R = off + G * H * in;
+    }
+    off += G * H * (in + H);
+  }
+  mats = off;
+  *bW = mats + (int64_t)pl * 2 * G * H;
+  *bR = *bW + G * H;
+}
+
+static double sigm(double v) { return 1.0 / (1.0 + exp(-v)); }
+
+/* Everything one pseudo-layer keeps for the way back, in step order s (time t = s for
+ * the forward direction, T-1-s for the backward one). */
+typedef struct rnn_tape {
+  double* hprev; /* [T+1][B][H]: state before step s; entry T = final state */
+  double* cprev; /* LSTM, same shape */
+  double* gate;  /* [T][G][B][H] activations */
+  double* rn;    /* GRU: R_n h + b_Rn, [T][B][H] */
+} rnn_tape;
+
+static void rnn_layer_fwd(const flref_rnn* d, int pl, const double* in, int64_t inl, const float* w,
+                          const float* hx, const float* cx, double* out, rnn_tape* tp) {
+  const int G = rnn_gates(d->mode), H = d->hidden, D = d->bidirectional ? 2 : 1, T = d->T, B = d->B;
+  const int dir = pl % D;
+  int64_t oW = 0, oR = 0, obW = 0, obR = 0;
+  rnn_offsets(d, pl, &oW, &oR, &obW, &obR);
+  const size_t BH = (size_t)B * H;
+  for (size_t i = 0; i < BH; ++i) {
+    tp->hprev[i] = hx ? hx[(size_t)pl * BH + i] : 0.0;
+    if (tp->cprev) tp->cprev[i] = cx ? cx[(size_t)pl * BH + i] : 0.0;
+  }
+  double* a = (double*)malloc(sizeof(double) * G * H);
+  double* r = (double*)malloc(sizeof(double) * G * H);
+  for (int s = 0; s < T; ++s) {
+    const int t = dir ? T - 1 - s : s;
+    const double* hp = tp->hprev + (size_t)s * BH;
+    double* hn = tp->hprev + (size_t)(s + 1) * BH;
+    for (int b = 0; b < B; ++b) {
+      const double* xin = in + ((size_t)t * B + b) * inl;
+      for (int q = 0; q < G * H; ++q) {
+        double sa = w[obW + q], sr = w[obR + q];
+        for (int64_t i = 0; i < inl; ++i) sa += (double)w[oW + (int64_t)q * inl + i] * xin[i];
+        for (int j = 0; j < H; ++j) sr += (double)w[oR + (int64_t)q * H + j] * hp[(size_t)b * H + j];
+        a[q] = sa;
+        r[q] = sr;
+      }
+      for (int h = 0; h < H; ++h) {
+        double* gt = tp->gate + (size_t)s * G * BH + (size_t)b * H + h; /* + g*BH */
+        double hv;
+        if (d->mode == 0 || d->mode == 1) {
+          const double pre = a[h] + r[h];
+          hv = d->mode == 0 ? (pre > 0 ? pre : 0.0) : tanh(pre);
+          gt[0] = hv;
+        } else if (d->mode == 2) {
+          const double ig = sigm(a[h] + r[h]), fg = sigm(a[H + h] + r[H + h]);
+          const double gg = tanh(a[2 * H + h] + r[2 * H + h]), og = sigm(a[3 * H + h] + r[3 * H + h]);
+          const double c = fg * tp->cprev[(size_t)s * BH + (size_t)b * H + h] + ig * gg;
+          tp->cprev[(size_t)(s + 1) * BH + (size_t)b * H + h] = c;
+          hv = og * tanh(c);
+          gt[0] = ig; gt[BH] = fg; gt[2 * BH] = gg; gt[3 * BH] = og;
+        } else {
+          const double rg = sigm(a[h] + r[h]), zg = sigm(a[H + h] + r[H + h]);
+          const double rn = r[2 * H + h];
+          const double ng = tanh(a[2 * H + h] + rg * rn);
+          tp->rn[(size_t)s * BH + (size_t)b * H + h] = rn;
+          hv = (1.0 - zg) * ng + zg * hp[(size_t)b * H + h];
+          gt[0] = rg; gt[BH] = zg; gt[2 * BH] = ng;
+        }
+        hn[(size_t)b * H + h] = hv;
+        out[((size_t)t * B + b) * D * H + (size_t)dir * H + h] = hv;
+      }
+    }
+  }
+  free(a);
+  free(r);
+}
+
+static rnn_tape rnn_tape_new(const flref_rnn* d) {
+  const size_t BH = (size_t)d->B * d->hidden, T = d->T, G = rnn_gates(d->mode);
+  rnn_tape tp;
+  tp.hprev = (double*)calloc((T + 1) * BH, sizeof(double));
+  tp.cprev = d->mode == 2 ? (double*)calloc((T + 1) * BH, sizeof(double)) : NULL;
+  tp.gate = (double*)calloc(T * G * BH, sizeof(double));
+  tp.rn = d->mode == 3 ? (double*)calloc(T * BH, sizeof(double)) : NULL;
+  return tp;
+}
+static void rnn_tape_free(rnn_tape* tp) {
+  free(tp->hprev); free(tp->cprev); free(tp->gate); free(tp->rn);
+}
+
+/* runs the whole stack; acts[l] = input of layer l (acts[layers] = y), tapes per pseudo-layer */
+static void rnn_stack_fwd(const flref_rnn* d, const float* x, const float* hx, const float* cx,
+                          const float* w, double** acts, rnn_tape* tapes) {
+  const int H = d->hidden, D = d->bidirectional ? 2 : 1, T = d->T, B = d->B;
+  const size_t n0 = (size_t)T * B * d->input_size;
+  acts[0] = (double*)malloc(sizeof(double) * n0);
+  for (size_t i = 0; i < n0; ++i) acts[0][i] = x[i];
+  for (int l = 0; l < d->layers; ++l) {
+    const int64_t inl = l == 0 ? d->input_size : D * H;
+    acts[l + 1] = (double*)calloc((size_t)T * B * D * H, sizeof(double));
+    for (int dir = 0; dir < D; ++dir) {
+      tapes[l * D + dir] = rnn_tape_new(d);
+      rnn_layer_fwd(d, l * D + dir, acts[l], inl, w, hx, cx, acts[l + 1], &tapes[l * D + dir]);
+    }
+  }
+}
+
+void flref_rnn_fwd(const flref_rnn* d, const float* x, const float* hx, const float* cx,
+                   const float* w, float* y, float* hy, float* cy) {
+  const int H = d->hidden, D = d->bidirectional ? 2 : 1, T = d->T, B = d->B, PL = d->layers * D;
+  double** acts = (double**)calloc(d->layers + 1, sizeof(double*));
+  rnn_tape* tapes = (rnn_tape*)calloc(PL, sizeof(rnn_tape));
+  rnn_stack_fwd(d, x, hx, cx, w, acts, tapes);
+  const size_t ny = (size_t)T * B * D * H, BH = (size_t)B * H;
+  for (size_t i = 0; i < ny; ++i) y[i] = (float)acts[d->layers][i];
+  for (int pl = 0; pl < PL; ++pl)
+    for (size_t i = 0; i < BH; ++i) {
+      hy[(size_t)pl * BH + i] = (float)tapes[pl].hprev[(size_t)T * BH + i];
+      if (cy && d->mode == 2) cy[(size_t)pl * BH + i] = (float)tapes[pl].cprev[(size_t)T * BH + i];
+    }
+  for (int l = 0; l <= d->layers; ++l) free(acts[l]);
+  for (int pl = 0; pl < PL; ++pl) rnn_tape_free(&tapes[pl]);
+  free(acts);
+  free(tapes);
+}
+
+void flref_rnn_bwd(const flref_rnn* d, const float* x, const float* hx, const float* cx,
+                   const float* w, const float* dy, const float* dhy, const float* dcy,
+                   float* dx, float* dhx, float* dcx, float* dw) {
+  const int G = rnn_gates(d->mode), H = d->hidden, D = d->bidirectional ? 2 : 1, T = d->T, B = d->B;
+  const int PL = d->layers * D;
+  const size_t BH = (size_t)B * H;
+  double** acts = (double**)calloc(d->layers + 1, sizeof(double*));
+  rnn_tape* tapes = (rnn_tape*)calloc(PL, sizeof(rnn_tape));
+  rnn_stack_fwd(d, x, hx, cx, w, acts, tapes);
+  const int64_t nw = flref_rnn_param_count(d);
+  double* gw = (double*)calloc((size_t)nw, sizeof(double));
+  const size_t ny = (size_t)T * B * D * H;
+  double* gout = (double*)calloc(ny, sizeof(double));          /* gradient of the layer output */
+  if (dy) for (size_t i = 0; i < ny; ++i) gout[i] = dy[i];
+  double* ga = (double*)malloc(sizeof(double) * G * H);        /* input-side pre-activation grads */
+  double* gr = (double*)malloc(sizeof(double) * G * H);        /* recurrent-side */
+  for (int l = d->layers - 1; l >= 0; --l) {
+    const int64_t inl = l == 0 ? d->input_size : D * H;
+    double* gin = (double*)calloc((size_t)T * B * inl, sizeof(double));
+    for (int dir = 0; dir < D; ++dir) {
+      const int pl = l * D + dir;
+      const rnn_tape* tp = &tapes[pl];
+      int64_t oW = 0, oR = 0, obW = 0, obR = 0;
+      rnn_offsets(d, pl, &oW, &oR, &obW, &obR);
+      double* gh = (double*)calloc(BH, sizeof(double));        /* dL/dh flowing back in time */
+      double* gc = (double*)calloc(BH, sizeof(double));
+      for (size_t i = 0; i < BH; ++i) {
+        gh[i] = dhy ? dhy[(size_t)pl * BH + i] : 0.0;
+        gc[i] = (dcy && d->mode == 2) ? dcy[(size_t)pl * BH + i] : 0.0;
+      }
+      double* ghp = (double*)malloc(sizeof(double) * BH);
+      for (int s = T - 1; s >= 0; --s) {
+        const int t = dir ? T - 1 - s : s;
+        const double* hp = tp->hprev + (size_t)s * BH;
+        for (size_t i = 0; i < BH; ++i) ghp[i] = 0.0;
+        for (int b = 0; b < B; ++b) {
+          const double* xin = acts[l] + ((size_t)t * B + b) * inl;
+          for (int h = 0; h < H; ++h) {
+            const size_t e = (size_t)b * H + h;
+            const double* gt = tp->gate + (size_t)s * G * BH + e;
+            const double go = gout[((size_t)t * B + b) * D * H + (size_t)dir * H + h] + gh[e];
+            if (d->mode == 0 || d->mode == 1) {
+              const double hv = gt[0];
+              const double gp = d->mode == 0 ? (hv > 0 ? go : 0.0) : go * (1.0 - hv * hv);
+              ga[h] = gr[h] = gp;
+            } else if (d->mode == 2) {
+              const double ig = gt[0], fg = gt[BH], gg = gt[2 * BH], og = gt[3 * BH];
+              const double c = tp->cprev[(size_t)(s + 1) * BH + e], cp = tp->cprev[(size_t)s * BH + e];
+              const double tc = tanh(c);
+              const double dc = gc[e] + go * og * (1.0 - tc * tc);
+              ga[h] = gr[h] = dc * gg * ig * (1.0 - ig);
+              ga[H + h] = gr[H + h] = dc * cp * fg * (1.0 - fg);
+              ga[2 * H + h] = gr[2 * H + h] = dc * ig * (1.0 - gg * gg);
+              ga[3 * H + h] = gr[3 * H + h] = go * tc * og * (1.0 - og);
+              gc[e] = dc * fg;
+            } else {
+              const double rg = gt[0], zg = gt[BH], ng = gt[2 * BH], rn = tp->rn[(size_t)s * BH + e];
+              const double dn = go * (1.0 - zg) * (1.0 - ng * ng);
+              ga[h] = gr[h] = dn * rn * rg * (1.0 - rg);
+              ga[H + h] = gr[H + h] = go * (hp[e] - ng) * zg * (1.0 - zg);
+              ga[2 * H + h] = dn;
+              gr[2 * H + h] = dn * rg;
+              ghp[e] += go * zg;
+            }
+          }
+          for (int q = 0; q < G * H; ++q) {
+            gw[obW + q] += ga[q];
+            gw[obR + q] += gr[q];
+            for (int64_t i = 0; i < inl; ++i) {
+              gw[oW + (int64_t)q * inl + i] += ga[q] * xin[i];
+              gin[((size_t)t * B + b) * inl + i] += ga[q] * (double)w[oW + (int64_t)q * inl + i];
+            }
+            for (int j = 0; j < H; ++j) {
+              gw[oR + (int64_t)q * H + j] += gr[q] * hp[(size_t)b * H + j];
+              ghp[(size_t)b * H + j] += gr[q] * (double)w[oR + (int64_t)q * H + j];
+            }
+          }
+        }
+        for (size_t i = 0; i < BH; ++i) gh[i] = ghp[i];
+      }
+      for (size_t i = 0; i < BH; ++i) {
+        if (dhx) dhx[(size_t)pl * BH + i] = (float)gh[i];
+        if (dcx && d->mode == 2) dcx[(size_t)pl * BH + i] = (float)gc[i];
+      }
+      free(gh); free(gc); free(ghp);
+    }
+    free(gout);
+    gout = gin;
+  }
+  const size_t nx = (size_t)T * B * d->input_size;
+  for (size_t i = 0; i < nx; ++i) dx[i] = (float)gout[i];
+  for (int64_t i = 0; i < nw; ++i) dw[i] = (float)gw[i];
+  free(gout); free(ga); free(gr); free(gw);
+  for (int l = 0; l <= d->layers; ++l) free(acts[l]);
+  for (int pl = 0; pl < PL; ++pl) rnn_tape_free(&tapes[pl]);
+  free(acts);
+  free(tapes);
+}

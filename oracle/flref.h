@@ -120,6 +120,29 @@ int flref_cce_fwd(int classes, int cols, const float* logp, const int32_t* targe
 void flref_cce_bwd(int classes, int cols, const float* grad, const int32_t* target, int ignore,
                    int reduction, float count, float* dx);
 
+/* ---- AutogradExtension::rnn / rnnBackward (flashlight/fl/autograd/tensor/
+ * AutogradExtension.h:96-106,167-179) with the semantics of the cuDNN extension
+ * (backend/cudnn/RNN.cpp:62-375; the oneDNN one has no backward, onednn/RNN.cpp:558-573):
+ * x [T][B][input] (Flashlight [input, B, T]), hx / hy / cx / cy [layers*dirs][B][hidden],
+ * y [T][B][dirs*hidden] (forward direction first), all row-major.  The weights are one
+ * flat vector in cuDNN's order: per pseudo-layer (layer-major, forward direction first)
+ * the input matrices of every gate ([hidden][in], row-major) then the recurrent ones
+ * ([hidden][hidden]); after all matrices, per pseudo-layer the input biases then the
+ * recurrent biases.  Gates: LSTM i, f, g, o; GRU r, z, n with
+ * n = tanh(W_n x + b_Wn + r * (R_n h + b_Rn)), h' = (1 - z) * n + z * h.
+ * mode: 0 ReLU, 1 tanh, 2 LSTM, 3 GRU (flashlight/fl/common/Defines.h:62-67).  No dropout. */
+typedef struct flref_rnn {
+  int32_t input_size, hidden, layers, bidirectional, mode, T, B;
+} flref_rnn;
+int64_t flref_rnn_param_count(const flref_rnn* d);
+/* hx, cx may be NULL (zeros); cy may be NULL */
+void flref_rnn_fwd(const flref_rnn* d, const float* x, const float* hx, const float* cx,
+                   const float* w, float* y, float* hy, float* cy);
+/* dy, dhy, dcy may be NULL (zeros); dhx, dcx may be NULL (not wanted) */
+void flref_rnn_bwd(const flref_rnn* d, const float* x, const float* hx, const float* cx,
+                   const float* w, const float* dy, const float* dhy, const float* dcy,
+                   float* dx, float* dhx, float* dcx, float* dw);
+
 #ifdef __cplusplus
 }
 #endif

@@ -312,3 +312,51 @@ def layer_norm_bwd(dy, x, xhat, mean, var, shape_whcn, norm_axes, eps, w=None):
         g, dw, db = affine_bwd(*view, dy, xhat, w)
     dx, _, _ = bn_bwd(*bnv, x, g, np.ones(bnv[1], np.float32), mean, var, eps)
     return dx, dw, db
+
+
+# ---- rnn / rnnBackward (cuDNN semantics, flat cuDNN weight order; see flref.h) ------------
+RNN_RELU, RNN_TANH, RNN_LSTM, RNN_GRU = 0, 1, 2, 3
+
+
+class RnnDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("input_size", "hidden", "layers", "bidirectional", "mode", "T", "B")]
+
+
+def rnn_desc(input_size, hidden, layers, bidirectional, mode, T, B):
+    return RnnDesc(input_size, hidden, layers, int(bool(bidirectional)), mode, T, B)
+
+
+def rnn_param_count(d):
+    f = lib().flref_rnn_param_count
+    f.restype = C.c_int64
+    return int(f(C.byref(d)))
+
+
+def _opt(a):
+    return None if a is None else _f32(a)
+
+
+def rnn_fwd(d, x, w, hx=None, cx=None):
+    """x [T, B, input], hx / cx [layers*dirs, B, hidden] or None -> (y, hy, cy or None)"""
+    x, w, hx, cx = _f32(x), _f32(w), _opt(hx), _opt(cx)
+    D = 2 if d.bidirectional else 1
+    y = np.empty((d.T, d.B, D * d.hidden), np.float32)
+    hy = np.empty((d.layers * D, d.B, d.hidden), np.float32)
+    cy = np.empty_like(hy) if d.mode == RNN_LSTM else None
+    lib().flref_rnn_fwd(C.byref(d), _p(x), _p(hx) if hx is not None else None, _p(cx) if cx is not None else None,
+                        _p(w), _p(y), _p(hy), _p(cy) if cy is not None else None)
+    return y, hy, cy
+
+
+def rnn_bwd(d, x, w, hx=None, cx=None, dy=None, dhy=None, dcy=None):
+    """-> (dx, dhx, dcx or None, dw)"""
+    x, w, hx, cx, dy, dhy, dcy = _f32(x), _f32(w), _opt(hx), _opt(cx), _opt(dy), _opt(dhy), _opt(dcy)
+    D = 2 if d.bidirectional else 1
+    dx = np.empty_like(x)
+    dhx = np.empty((d.layers * D, d.B, d.hidden), np.float32)
+    dcx = np.empty_like(dhx) if d.mode == RNN_LSTM else None
+    dw = np.empty_like(w)
+    q = lambda a: _p(a) if a is not None else None
+    lib().flref_rnn_bwd(C.byref(d), _p(x), q(hx), q(cx), _p(w), q(dy), q(dhy), q(dcy), _p(dx), _p(dhx), q(dcx),
+                        _p(dw))
+    return dx, dhx, dcx, dw
