@@ -26,6 +26,11 @@ class BnDesc(C.Structure):
                 ("dtype", C.c_int32)]
 
 
+class RnnDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in ("input_size", "hidden_size", "num_layers", "bidirectional", "mode",
+                                         "seq_len", "batch", "dtype")]
+
+
 # every symbol include/flhip.h declares: name -> (restype, argtypes)
 _VP, _SZ, _I32P = C.c_void_p, C.c_size_t, C.POINTER(C.c_int32)
 SYMBOLS = {
@@ -60,6 +65,12 @@ SYMBOLS = {
     "flhip_cce_fwd": (C.c_int, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int, _VP]),
     "flhip_cce_bwd": (C.c_int, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int, C.c_int32, C.c_int,
                                 _VP]),
+    "flhip_rnn_param_count": (C.c_size_t, [_VP]),
+    "flhip_rnn_reserve_bytes": (C.c_size_t, [_VP]),
+    "flhip_rnn_workspace_bytes": (C.c_size_t, [_VP]),
+    "flhip_rnn_fwd": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, C.c_size_t, _VP, C.c_size_t, _VP]),
+    "flhip_rnn_bwd": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, C.c_size_t, _VP, _VP, _VP, _VP, _VP,
+                                C.c_size_t, _VP]),
     "flhip_affine_fwd": (C.c_int, [_VP, _VP, _VP, _VP, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int,
                                    _VP]),
     "flhip_affine_bwd_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int64, C.c_int64, C.c_int]),

@@ -1,0 +1,451 @@
+// rnn / rnnBackward: ReLU / tanh RNN, LSTM and GRU, stacked and bidirectional, with the
+// semantics and the flat weight order of the cuDNN calls the reference makes
+// (flashlight/fl/autograd/tensor/backend/cudnn/RNN.cpp:62-375): per pseudo-layer
+// (layer-major, forward direction first) the input matrices of every gate
+// ([hidden][in], row-major) then the recurrent ones; after all matrices, per
+// pseudo-layer the input biases then the recurrent biases.  Gates: LSTM i, f, g, o;
+// GRU r, z, n with n = tanh(W_n x + b_Wn + r * (R_n h + b_Rn)), h' = (1-z)*n + z*h.
+//
+// Structure: the input projections of all time steps of a pseudo-layer are one matrix
+// product; the recurrence is a loop over time of (recurrent product, gate kernel).
+// The products go through flhip_matmul (matrix cores where the shapes allow).  The
+// forward pass keeps, per pseudo-layer and in step order, the state before every step,
+// the gate activations and (GRU) R_n h + b_Rn in the reserve buffer; the backward pass
+// walks the steps in reverse, writes the pre-activation gradients of all steps, and
+// turns them into dx, dW, dR and the bias gradients with four products / reductions.
+// Layouts follow Flashlight: x [input, B, T] column-major = memory [T][B][input], etc.
+// fp32 only; no dropout between layers (the closure's dropProb must be 0).
+#include <algorithm>
+
+#include "common.h"
+
+extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, int32_t N, int32_t K,
+                            int trans_a, int trans_b, const float* bias_rows, int dtype, void* stream);
+extern "C" int flhip_sum_columns(const void* x, float* out, int32_t rows, int32_t cols, int dtype,
+                                 void* stream);
+
+namespace flhip {
+namespace {
+
+enum { RNN_RELU = 0, RNN_TANH = 1, RNN_LSTM = 2, RNN_GRU = 3 };
+
+struct RnnGeom {
+  int I, H, L, D, mode, T, B, G;
+  size_t BH, GH;
+  size_t nparams;
+};
+
+inline int gates_of(int mode) { return mode == RNN_LSTM ? 4 : mode == RNN_GRU ? 3 : 1; }
+
+int make_geom(const flhip_rnn_desc* d, RnnGeom* g) {
+  FLHIP_REQUIRE(d, "rnn: null descriptor");
+  FLHIP_REQUIRE(d->input_size > 0 && d->hidden_size > 0 && d->num_layers > 0 && d->seq_len > 0 &&
+                    d->batch > 0,
+                "rnn: sizes must be positive");
+  FLHIP_REQUIRE(d->mode >= RNN_RELU && d->mode <= RNN_GRU, "rnn: unknown mode");
+  FLHIP_REQUIRE(d->dtype == FLHIP_F32, "rnn: f32 only");
+  g->I = d->input_size; g->H = d->hidden_size; g->L = d->num_layers; g->D = d->bidirectional ? 2 : 1;
+  g->mode = d->mode; g->T = d->seq_len; g->B = d->batch; g->G = gates_of(d->mode);
+  g->BH = (size_t)g->B * g->H;
+  g->GH = (size_t)g->G * g->H;
+  size_t n = 0;
+  for (int l = 0; l < g->L; ++l) {
+    const size_t in = l == 0 ? g->I : (size_t)g->D * g->H;
+    n += g->D * (g->GH * (in + g->H) + 2 * g->GH);
+  }
+  g->nparams = n;
+  FLHIP_REQUIRE((size_t)g->T * g->B * std::max<size_t>(g->GH, (size_t)g->D * g->H) < (1u << 30) &&
+                    n < (1u << 30),
+                "rnn: problem too large for 32-bit indices");
+  return FLHIP_OK;
+}
+
+struct Offsets {
+  size_t W, R, bW, bR;
+};
+Offsets offsets(const RnnGeom& g, int pl) {
+  Offsets o{};
+  size_t off = 0;
+  for (int p = 0; p < g.L * g.D; ++p) {
+    const size_t in = p / g.D == 0 ? g.I : (size_t)g.D * g.H;
+    if (p == pl) {
+      o.W = off;
+      o.R = off + g.GH * in;
+    }
+    off += g.GH * (in + g.H);
+  }
+  o.bW = off + (size_t)pl * 2 * g.GH;
+  o.bR = o.bW + g.GH;
+  return o;
+}
+
+// reserve buffer, in floats: per pseudo-layer {HP [(T+1)*BH], CP [(T+1)*BH] (LSTM),
+// GT [T*B*GH], RN [T*BH] (GRU)}, then the outputs of layers 0 .. L-2 ([T*B*D*H] each)
+struct Reserve {
+  size_t per_pl, hp, cp, gt, rn, acts, total;
+};
+Reserve reserve_layout(const RnnGeom& g) {
+  Reserve r{};
+  size_t o = 0;
+  r.hp = o; o += (size_t)(g.T + 1) * g.BH;
+  r.cp = o; if (g.mode == RNN_LSTM) o += (size_t)(g.T + 1) * g.BH;
+  r.gt = o; o += (size_t)g.T * g.B * g.GH;
+  r.rn = o; if (g.mode == RNN_GRU) o += (size_t)g.T * g.BH;
+  r.per_pl = o;
+  r.acts = r.per_pl * g.L * g.D;
+  r.total = r.acts + (size_t)(g.L - 1) * g.T * g.B * g.D * g.H;
+  return r;
+}
+
+// workspace, in floats (one call): forward {XP [T*B*GH], RP [B*GH], bias [GH]};
+// backward {dGW [T*B*GH], dGR [T*B*GH], gout [T*B*D*H], gin [T*B*inmax], tmp [T*B*inmax],
+// dh_dir [2*BH], dh_rec [BH], dc [BH]}
+size_t workspace_floats(const RnnGeom& g) {
+  const size_t TB = (size_t)g.T * g.B, inmax = std::max<size_t>(g.I, (size_t)g.D * g.H);
+  const size_t fwd = TB * g.GH + g.B * g.GH + g.GH;
+  const size_t bwd = 2 * TB * g.GH + TB * g.D * g.H + 2 * TB * inmax + 4 * g.BH;
+  return std::max(fwd, bwd) + 64;
+}
+
+__device__ __forceinline__ float sigm(float v) { return 1.f / (1.f + expf(-v)); }
+
+// bsum[q] = bW[q] + bR[q], except the GRU n gate, whose recurrent bias stays inside
+// r * (R_n h + b_Rn)
+__global__ void __launch_bounds__(256) rnn_bias_kernel(const float* __restrict__ bW, const float* __restrict__ bR,
+                                                       float* __restrict__ bsum, int GH, int H, int mode) {
+  const int q = blockIdx.x * 256 + threadIdx.x;
+  if (q >= GH) return;
+  bsum[q] = (mode == RNN_GRU && q >= 2 * H) ? bW[q] : bW[q] + bR[q];
+}
+
+__global__ void __launch_bounds__(256) rnn_init_kernel(const float* __restrict__ src, float* __restrict__ dst, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) dst[i] = src ? src[i] : 0.f;
+}
+
+__global__ void __launch_bounds__(256) rnn_add2_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                       float* __restrict__ out, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) out[i] = (a ? a[i] : 0.f) + (b ? b[i] : 0.f);
+}
+
+struct CellFwd {
+  const float* xp;    // [B][GH] input projection (+ biases) of this time step
+  const float* rp;    // [B][GH] recurrent projection
+  const float* bRn;   // GRU: recurrent bias of the n gate [H]
+  const float* hp;    // [B][H] state before the step
+  const float* cp;    // LSTM
+  float* hn;          // [B][H] state after the step
+  float* cn;
+  float* gt;          // [B][GH] gate activations kept for the backward pass
+  float* rn;          // GRU: R_n h + b_Rn
+  float* out;         // layer output at this time step, this direction's slice; row pitch ldo
+  float* hy;          // final state of the pseudo-layer (written at the last step) or null
+  float* cy;
+  int ldo;
+};
+
+template <int MODE>
+__global__ void __launch_bounds__(256) rnn_cell_fwd(CellFwd a, int B, int H) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= B * H) return;
+  const int b = e / H, h = e - b * H;
+  constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1;
+  const size_t q = (size_t)b * G * H + h;
+  float hv;
+  if (MODE == RNN_RELU || MODE == RNN_TANH) {
+    const float pre = a.xp[q] + a.rp[q];
+    hv = MODE == RNN_RELU ? (pre > 0.f ? pre : 0.f) : tanhf(pre);
+    a.gt[q] = hv;
+  } else if (MODE == RNN_LSTM) {
+    const float ig = sigm(a.xp[q] + a.rp[q]), fg = sigm(a.xp[q + H] + a.rp[q + H]);
+    const float gg = tanhf(a.xp[q + 2 * H] + a.rp[q + 2 * H]), og = sigm(a.xp[q + 3 * H] + a.rp[q + 3 * H]);
+    const float c = fg * a.cp[e] + ig * gg;
+    a.cn[e] = c;
+    if (a.cy) a.cy[e] = c;
+    hv = og * tanhf(c);
+    a.gt[q] = ig; a.gt[q + H] = fg; a.gt[q + 2 * H] = gg; a.gt[q + 3 * H] = og;
+  } else {
+    const float rg = sigm(a.xp[q] + a.rp[q]), zg = sigm(a.xp[q + H] + a.rp[q + H]);
+    const float rn = a.rp[q + 2 * H] + a.bRn[h];
+    const float ng = tanhf(a.xp[q + 2 * H] + rg * rn);
+    a.rn[e] = rn;
+    hv = (1.f - zg) * ng + zg * a.hp[e];
+    a.gt[q] = rg; a.gt[q + H] = zg; a.gt[q + 2 * H] = ng;
+  }
+  a.hn[e] = hv;
+  a.out[(size_t)b * a.ldo + h] = hv;
+  if (a.hy) a.hy[e] = hv;
+}
+
+struct CellBwd {
+  const float* gout;  // gradient of the layer output at this time step, this direction's slice; pitch ldo (may be null)
+  const float* dh_a;  // gradient reaching h through the recurrence: direct part ...
+  const float* dh_b;  // ... and the part through the recurrent matrices (either may be null)
+  float* dc;          // LSTM: in = gradient of c after the step, out = of c before it
+  const float* gt;    // gate activations of the step
+  const float* cp;    // LSTM: c before the step
+  const float* cn;    //       c after the step
+  const float* hp;    // state before the step
+  const float* rn;    // GRU
+  float* dgw;         // [B][GH] pre-activation gradients seen by the input side
+  float* dgr;         // [B][GH] ... by the recurrent side
+  float* dh_dir;      // [B][H] direct gradient towards the previous state (GRU: go * z, else 0)
+  int ldo;
+};
+
+template <int MODE>
+__global__ void __launch_bounds__(256) rnn_cell_bwd(CellBwd a, int B, int H) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= B * H) return;
+  const int b = e / H, h = e - b * H;
+  constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1;
+  const size_t q = (size_t)b * G * H + h;
+  float go = a.gout ? a.gout[(size_t)b * a.ldo + h] : 0.f;
+  if (a.dh_a) go += a.dh_a[e];
+  if (a.dh_b) go += a.dh_b[e];
+  float direct = 0.f;
+  if (MODE == RNN_RELU || MODE == RNN_TANH) {
+    const float hv = a.gt[q];
+    const float gp = MODE == RNN_RELU ? (hv > 0.f ? go : 0.f) : go * (1.f - hv * hv);
+    a.dgw[q] = gp;
+    a.dgr[q] = gp;
+  } else if (MODE == RNN_LSTM) {
+    const float ig = a.gt[q], fg = a.gt[q + H], gg = a.gt[q + 2 * H], og = a.gt[q + 3 * H];
+    const float tc = tanhf(a.cn[e]);
+    const float dc = a.dc[e] + go * og * (1.f - tc * tc);
+    const float v0 = dc * gg * ig * (1.f - ig), v1 = dc * a.cp[e] * fg * (1.f - fg);
+    const float v2 = dc * ig * (1.f - gg * gg), v3 = go * tc * og * (1.f - og);
+    a.dgw[q] = v0; a.dgw[q + H] = v1; a.dgw[q + 2 * H] = v2; a.dgw[q + 3 * H] = v3;
+    a.dgr[q] = v0; a.dgr[q + H] = v1; a.dgr[q + 2 * H] = v2; a.dgr[q + 3 * H] = v3;
+    a.dc[e] = dc * fg;
+  } else {
+    const float rg = a.gt[q], zg = a.gt[q + H], ng = a.gt[q + 2 * H], rn = a.rn[e];
+    const float dn = go * (1.f - zg) * (1.f - ng * ng);
+    const float v0 = dn * rn * rg * (1.f - rg), v1 = go * (a.hp[e] - ng) * zg * (1.f - zg);
+    a.dgw[q] = v0; a.dgw[q + H] = v1; a.dgw[q + 2 * H] = dn;
+    a.dgr[q] = v0; a.dgr[q + H] = v1; a.dgr[q + 2 * H] = dn * rg;
+    direct = go * zg;
+  }
+  a.dh_dir[e] = direct;
+}
+
+inline unsigned nblocks(size_t n) { return (unsigned)((n + 255) / 256); }
+
+int mm(const float* A, const float* B, float* C, size_t M, size_t N, size_t K, int ta, int tb,
+       const float* bias, hipStream_t s) {
+  return flhip_matmul(A, B, C, (int32_t)M, (int32_t)N, (int32_t)K, ta, tb, bias, FLHIP_F32, s);
+}
+
+template <int MODE>
+int forward_pl(const RnnGeom& g, int pl, const float* in, size_t inl, const float* w, const float* hx,
+               const float* cx, float* out, float* hy, float* cy, float* res, float* ws, hipStream_t s) {
+  const Reserve r = reserve_layout(g);
+  const Offsets o = offsets(g, pl);
+  const int dir = pl % g.D;
+  const size_t TB = (size_t)g.T * g.B;
+  float* HP = res + (size_t)pl * r.per_pl + r.hp;
+  float* CP = res + (size_t)pl * r.per_pl + r.cp;
+  float* GT = res + (size_t)pl * r.per_pl + r.gt;
+  float* RN = res + (size_t)pl * r.per_pl + r.rn;
+  float* XP = ws;
+  float* RP = XP + TB * g.GH;
+  float* bsum = RP + (size_t)g.B * g.GH;
+  hipLaunchKernelGGL(rnn_bias_kernel, dim3(nblocks(g.GH)), dim3(256), 0, s, w + o.bW, w + o.bR, bsum,
+                     (int)g.GH, g.H, g.mode);
+  // XP [GH x TB] = W [GH x in] (row-major = a column-major in x GH matrix, transposed) * IN [in x TB]
+  if (const int rc = mm(w + o.W, in, XP, g.GH, TB, inl, 1, 0, bsum, s)) return rc;
+  hipLaunchKernelGGL(rnn_init_kernel, dim3(nblocks(g.BH)), dim3(256), 0, s, hx ? hx + (size_t)pl * g.BH : nullptr,
+                     HP, g.BH);
+  if (MODE == RNN_LSTM)
+    hipLaunchKernelGGL(rnn_init_kernel, dim3(nblocks(g.BH)), dim3(256), 0, s,
+                       cx ? cx + (size_t)pl * g.BH : nullptr, CP, g.BH);
+  for (int st = 0; st < g.T; ++st) {
+    const int t = dir ? g.T - 1 - st : st;
+    if (const int rc = mm(w + o.R, HP + (size_t)st * g.BH, RP, g.GH, g.B, g.H, 1, 0, nullptr, s)) return rc;
+    CellFwd a{};
+    a.xp = XP + (size_t)t * g.B * g.GH;
+    a.rp = RP;
+    a.bRn = w + o.bR + 2 * g.H;
+    a.hp = HP + (size_t)st * g.BH;
+    a.cp = CP + (size_t)st * g.BH;
+    a.hn = HP + (size_t)(st + 1) * g.BH;
+    a.cn = CP + (size_t)(st + 1) * g.BH;
+    a.gt = GT + (size_t)st * g.B * g.GH;
+    a.rn = RN + (size_t)st * g.BH;
+    a.ldo = g.D * g.H;
+    a.out = out + (size_t)t * g.B * a.ldo + (size_t)dir * g.H;
+    const bool last = st == g.T - 1;
+    a.hy = last ? hy + (size_t)pl * g.BH : nullptr;
+    a.cy = (last && cy && MODE == RNN_LSTM) ? cy + (size_t)pl * g.BH : nullptr;
+    hipLaunchKernelGGL((rnn_cell_fwd<MODE>), dim3(nblocks(g.BH)), dim3(256), 0, s, a, g.B, g.H);
+  }
+  return check_launch("rnn_fwd");
+}
+
+template <int MODE>
+int backward_pl(const RnnGeom& g, int pl, const float* in, size_t inl, const float* w, const float* gout,
+                const float* dhy, const float* dcy, float* gin, bool first_dir, float* dhx, float* dcx,
+                float* dw, const float* res, float* ws, hipStream_t s) {
+  const Reserve r = reserve_layout(g);
+  const Offsets o = offsets(g, pl);
+  const int dir = pl % g.D;
+  const size_t TB = (size_t)g.T * g.B, inmax = std::max<size_t>(g.I, (size_t)g.D * g.H);
+  const float* HP = res + (size_t)pl * r.per_pl + r.hp;
+  const float* CP = res + (size_t)pl * r.per_pl + r.cp;
+  const float* GT = res + (size_t)pl * r.per_pl + r.gt;
+  const float* RN = res + (size_t)pl * r.per_pl + r.rn;
+  float* dGW = ws;
+  float* dGR = dGW + TB * g.GH;
+  float* tmp = dGR + TB * g.GH + TB * g.D * g.H + TB * inmax;   // behind gout and gin
+  float* dh_dir = tmp + TB * inmax;                               // two buffers, alternating
+  float* dh_rec = dh_dir + 2 * g.BH;
+  float* dc = dh_rec + g.BH;
+  if (MODE == RNN_LSTM)
+    hipLaunchKernelGGL(rnn_init_kernel, dim3(nblocks(g.BH)), dim3(256), 0, s,
+                       dcy ? dcy + (size_t)pl * g.BH : nullptr, dc, g.BH);
+  const float* dha = dhy ? dhy + (size_t)pl * g.BH : nullptr;   // direct part for the first step walked
+  const float* dhb = nullptr;
+  for (int st = g.T - 1; st >= 0; --st) {
+    const int t = dir ? g.T - 1 - st : st;
+    CellBwd a{};
+    a.ldo = g.D * g.H;
+    a.gout = gout ? gout + (size_t)t * g.B * a.ldo + (size_t)dir * g.H : nullptr;
+    a.dh_a = dha;
+    a.dh_b = dhb;
+    a.dc = dc;
+    a.gt = GT + (size_t)st * g.B * g.GH;
+    a.cp = CP + (size_t)st * g.BH;
+    a.cn = CP + (size_t)(st + 1) * g.BH;
+    a.hp = HP + (size_t)st * g.BH;
+    a.rn = RN + (size_t)st * g.BH;
+    a.dgw = dGW + (size_t)t * g.B * g.GH;
+    a.dgr = dGR + (size_t)st * g.B * g.GH;
+    a.dh_dir = dh_dir + (size_t)(st & 1) * g.BH;
+    hipLaunchKernelGGL((rnn_cell_bwd<MODE>), dim3(nblocks(g.BH)), dim3(256), 0, s, a, g.B, g.H);
+    // gradient through the recurrent matrices: dh_rec [H x B] = R^T [H x GH] * dGR[st] [GH x B]
+    if (const int rc = mm(w + o.R, a.dgr, dh_rec, g.H, g.B, g.GH, 0, 0, nullptr, s)) return rc;
+    dha = a.dh_dir;
+    dhb = dh_rec;
+  }
+  if (dhx) hipLaunchKernelGGL(rnn_add2_kernel, dim3(nblocks(g.BH)), dim3(256), 0, s, dha, dhb, dhx + (size_t)pl * g.BH, g.BH);
+  if (dcx && MODE == RNN_LSTM)
+    hipLaunchKernelGGL(rnn_init_kernel, dim3(nblocks(g.BH)), dim3(256), 0, s, dc, dcx + (size_t)pl * g.BH, g.BH);
+  // gradient of the layer input: gin [in x TB] (+)= W^T [in x GH] * dGW [GH x TB]
+  float* gdst = first_dir ? gin : tmp;
+  if (const int rc = mm(w + o.W, dGW, gdst, inl, TB, g.GH, 0, 0, nullptr, s)) return rc;
+  if (!first_dir)
+    hipLaunchKernelGGL(rnn_add2_kernel, dim3(nblocks(TB * inl)), dim3(256), 0, s, gin, tmp, gin, TB * inl);
+  // dW [GH][in] row-major = column-major in x GH = IN [in x TB] * dGW^T; dR likewise with the
+  // states before each step; the bias gradients are the row sums
+  if (const int rc = mm(in, dGW, dw + o.W, inl, g.GH, TB, 0, 1, nullptr, s)) return rc;
+  if (const int rc = mm(HP, dGR, dw + o.R, g.H, g.GH, TB, 0, 1, nullptr, s)) return rc;
+  if (const int rc = flhip_sum_columns(dGW, dw + o.bW, (int32_t)g.GH, (int32_t)TB, FLHIP_F32, s)) return rc;
+  if (const int rc = flhip_sum_columns(dGR, dw + o.bR, (int32_t)g.GH, (int32_t)TB, FLHIP_F32, s)) return rc;
+  return check_launch("rnn_bwd");
+}
+
+}  // namespace
+}  // namespace flhip
+
+using namespace flhip;
+
+extern "C" size_t flhip_rnn_param_count(const flhip_rnn_desc* d) {
+  RnnGeom g;
+  return make_geom(d, &g) == FLHIP_OK ? g.nparams : 0;
+}
+extern "C" size_t flhip_rnn_reserve_bytes(const flhip_rnn_desc* d) {
+  RnnGeom g;
+  return make_geom(d, &g) == FLHIP_OK ? reserve_layout(g).total * sizeof(float) : 0;
+}
+extern "C" size_t flhip_rnn_workspace_bytes(const flhip_rnn_desc* d) {
+  RnnGeom g;
+  return make_geom(d, &g) == FLHIP_OK ? workspace_floats(g) * sizeof(float) : 0;
+}
+
+extern "C" int flhip_rnn_fwd(const flhip_rnn_desc* d, const void* x, const void* hx, const void* cx,
+                             const void* w, void* y, void* hy, void* cy, void* reserve,
+                             size_t reserve_bytes, void* ws, size_t ws_bytes, void* stream) {
+  RnnGeom g;
+  const int rc0 = make_geom(d, &g);
+  if (rc0 != FLHIP_OK) return rc0;
+  FLHIP_REQUIRE(x && w && y && hy, "rnn_fwd: null argument");
+  FLHIP_REQUIRE(reserve && reserve_bytes >= flhip_rnn_reserve_bytes(d), "rnn_fwd: reserve buffer too small");
+  FLHIP_REQUIRE(ws && ws_bytes >= flhip_rnn_workspace_bytes(d), "rnn_fwd: workspace too small");
+  hipStream_t s = as_stream(stream);
+  const Reserve r = reserve_layout(g);
+  float* res = static_cast<float*>(reserve);
+  const float* wf = static_cast<const float*>(w);
+  const size_t act = (size_t)g.T * g.B * g.D * g.H;
+  for (int l = 0; l < g.L; ++l) {
+    const float* in = l == 0 ? static_cast<const float*>(x) : res + r.acts + (size_t)(l - 1) * act;
+    float* out = l == g.L - 1 ? static_cast<float*>(y) : res + r.acts + (size_t)l * act;
+    const size_t inl = l == 0 ? g.I : (size_t)g.D * g.H;
+    for (int dir = 0; dir < g.D; ++dir) {
+      const int pl = l * g.D + dir;
+      int rc;
+      auto args = [&](auto fn) {
+        return fn(g, pl, in, inl, wf, static_cast<const float*>(hx), static_cast<const float*>(cx), out,
+                  static_cast<float*>(hy), static_cast<float*>(cy), res, static_cast<float*>(ws), s);
+      };
+      switch (g.mode) {
+        case RNN_RELU: rc = args(forward_pl<RNN_RELU>); break;
+        case RNN_TANH: rc = args(forward_pl<RNN_TANH>); break;
+        case RNN_LSTM: rc = args(forward_pl<RNN_LSTM>); break;
+        default: rc = args(forward_pl<RNN_GRU>);
+      }
+      if (rc != FLHIP_OK) return rc;
+    }
+  }
+  return FLHIP_OK;
+}
+
+extern "C" int flhip_rnn_bwd(const flhip_rnn_desc* d, const void* x, const void* w, const void* dy,
+                             const void* dhy, const void* dcy, const void* reserve,
+                             size_t reserve_bytes, void* dx, void* dhx, void* dcx, void* dw, void* ws,
+                             size_t ws_bytes, void* stream) {
+  RnnGeom g;
+  const int rc0 = make_geom(d, &g);
+  if (rc0 != FLHIP_OK) return rc0;
+  FLHIP_REQUIRE(x && w && dx && dw, "rnn_bwd: null argument");
+  FLHIP_REQUIRE(reserve && reserve_bytes >= flhip_rnn_reserve_bytes(d),
+                "rnn_bwd: needs the reserve buffer of the forward pass");
+  FLHIP_REQUIRE(ws && ws_bytes >= flhip_rnn_workspace_bytes(d), "rnn_bwd: workspace too small");
+  hipStream_t s = as_stream(stream);
+  const Reserve r = reserve_layout(g);
+  const float* res = static_cast<const float*>(reserve);
+  const float* wf = static_cast<const float*>(w);
+  float* wsf = static_cast<float*>(ws);
+  const size_t TB = (size_t)g.T * g.B, act = TB * g.D * g.H, inmax = std::max<size_t>(g.I, (size_t)g.D * g.H);
+  float* goutbuf = wsf + 2 * TB * g.GH;
+  float* ginbuf = goutbuf + act;
+  const float* gout = static_cast<const float*>(dy);   // gradient of the top layer's output (may be null)
+  for (int l = g.L - 1; l >= 0; --l) {
+    const float* in = l == 0 ? static_cast<const float*>(x) : res + r.acts + (size_t)(l - 1) * act;
+    const size_t inl = l == 0 ? g.I : (size_t)g.D * g.H;
+    float* gin = l == 0 ? static_cast<float*>(dx) : ginbuf;
+    for (int dir = 0; dir < g.D; ++dir) {
+      const int pl = l * g.D + dir;
+      int rc;
+      auto args = [&](auto fn) {
+        return fn(g, pl, in, inl, wf, gout, static_cast<const float*>(dhy), static_cast<const float*>(dcy), gin,
+                  dir == 0, static_cast<float*>(dhx), static_cast<float*>(dcx), static_cast<float*>(dw), res,
+                  wsf, s);
+      };
+      switch (g.mode) {
+        case RNN_RELU: rc = args(backward_pl<RNN_RELU>); break;
+        case RNN_TANH: rc = args(backward_pl<RNN_TANH>); break;
+        case RNN_LSTM: rc = args(backward_pl<RNN_LSTM>); break;
+        default: rc = args(backward_pl<RNN_GRU>);
+      }
+      if (rc != FLHIP_OK) return rc;
+    }
+    if (l > 0) {
+      // the gradient of this layer's input is the gradient of the output of the layer below
+      if (const int rc = flhip_copy_bytes(ginbuf, goutbuf, TB * inl * sizeof(float), stream)) return rc;
+      gout = goutbuf;
+    }
+  }
+  (void)inmax;
+  return FLHIP_OK;
+}

@@ -471,3 +471,75 @@ def layer_norm_backward(grad_output, ctx, weight=None):
         g, dw, db = affine_backward(g, ctx["xhat"], weight, ctx["view"])
     dx, _, _ = batchnorm_backward(g, ctx["x4"], None, ctx["sm"], ctx["si"], ctx["comp"])
     return dx.reshape(grad_output.shape), dw, db
+
+
+# ---- rnn / rnnBackward -----------------------------------------------------------------
+RNN_RELU, RNN_TANH, RNN_LSTM, RNN_GRU = 0, 1, 2, 3
+
+
+def _rnn_desc(x, hidden_size, num_layers, mode, bidirectional):
+    if x.dim() != 3 or x.dtype != torch.float32:
+        raise ValueError("rnn: input must be fp32 [seq, batch, input] (Flashlight [input, batch, seq])")
+    T, B, I = x.shape
+    return capi.RnnDesc(I, hidden_size, num_layers, int(bool(bidirectional)), int(mode), T, B, capi.F32)
+
+
+def rnn_param_count(input_size, hidden_size, num_layers, mode, bidirectional):
+    d = capi.RnnDesc(input_size, hidden_size, num_layers, int(bool(bidirectional)), int(mode), 1, 1, capi.F32)
+    return capi.lib().flhip_rnn_param_count(C.byref(d))
+
+
+def rnn(input, hidden_state, cell_state, weights, hidden_size, num_layers, mode, bidirectional,
+        dropout=0.0):
+    """AutogradExtension::rnn -> (output, hiddenOut, cellOut or None, reserve).  Tensors are
+    torch views of the Flashlight ones (shape reversed): input [seq, batch, input], states
+    [layers*dirs, batch, hidden], output [seq, batch, dirs*hidden]; weights flat in cuDNN's
+    order.  reserve goes to rnn_backward (the payload of the reference's closure)."""
+    if dropout != 0.0:
+        raise ValueError("rnn: dropout between layers is not supported by this backend")
+    x, w = _dev(input, "input"), _dev(weights, "weights")
+    d = _rnn_desc(x, hidden_size, num_layers, mode, bidirectional)
+    L = capi.lib()
+    if w.numel() != L.flhip_rnn_param_count(C.byref(d)):
+        raise ValueError("invalid # of parameters or wrong input shape for RNN")
+    D = 2 if bidirectional else 1
+    sshape = (num_layers * D, d.batch, hidden_size)
+    for t, name in ((hidden_state, "hidden"), (cell_state, "cell")):
+        if t is not None and t.numel() and tuple(t.shape) != sshape:
+            raise ValueError("invalid %s state dims for RNN" % name)
+    if cell_state is not None and cell_state.numel() and mode != RNN_LSTM:
+        raise ValueError("invalid cell state dims for RNN")
+    hx = _dev(hidden_state, "hiddenState") if hidden_state is not None and hidden_state.numel() else None
+    cx = _dev(cell_state, "cellState") if cell_state is not None and cell_state.numel() else None
+    y = torch.empty((d.seq_len, d.batch, D * hidden_size), dtype=torch.float32, device=x.device)
+    hy = torch.empty(sshape, dtype=torch.float32, device=x.device)
+    cy = torch.empty(sshape, dtype=torch.float32, device=x.device) if mode == RNN_LSTM else None
+    nres, nws = L.flhip_rnn_reserve_bytes(C.byref(d)), L.flhip_rnn_workspace_bytes(C.byref(d))
+    reserve, ws = _ws(nres, x.device), _ws(nws, x.device)
+    capi.check(L.flhip_rnn_fwd(C.byref(d), _ptr(x), _ptr(hx), _ptr(cx), _ptr(w), _ptr(y), _ptr(hy), _ptr(cy),
+                               _ptr(reserve), nres, _ptr(ws), nws, _stream()))
+    return y, hy, cy, reserve
+
+
+def rnn_backward(input, weights, reserve, hidden_size, num_layers, mode, bidirectional,
+                 grad_output=None, grad_hidden=None, grad_cell=None):
+    """AutogradExtension::rnnBackward -> (gradInput, gradHidden, gradCell or None, gradWeights);
+    missing output gradients count as zero (Functions.cpp:1677-1699)."""
+    x, w = _dev(input, "input"), _dev(weights, "weights")
+    d = _rnn_desc(x, hidden_size, num_layers, mode, bidirectional)
+    L = capi.lib()
+    D = 2 if bidirectional else 1
+    sshape = (num_layers * D, d.batch, hidden_size)
+    dx = torch.empty_like(x)
+    dhx = torch.empty(sshape, dtype=torch.float32, device=x.device)
+    dcx = torch.empty(sshape, dtype=torch.float32, device=x.device) if mode == RNN_LSTM else None
+    dw = torch.empty_like(w)
+    nres, nws = L.flhip_rnn_reserve_bytes(C.byref(d)), L.flhip_rnn_workspace_bytes(C.byref(d))
+    if reserve is None or reserve.numel() < nres:
+        raise ValueError("rnnBackward: needs the reserve buffer of the forward pass")
+    ws = _ws(nws, x.device)
+    opt = lambda t, n: _ptr(_dev(t, n)) if t is not None and t.numel() else None
+    capi.check(L.flhip_rnn_bwd(C.byref(d), _ptr(x), _ptr(w), opt(grad_output, "gradOutput"),
+                               opt(grad_hidden, "gradHidden"), opt(grad_cell, "gradCell"), _ptr(reserve), nres,
+                               _ptr(dx), _ptr(dhx), _ptr(dcx), _ptr(dw), _ptr(ws), nws, _stream()))
+    return dx, dhx, dcx, dw

@@ -269,6 +269,35 @@ int flhip_cce_bwd(const float* grad, const int32_t* target, const float* stats, 
  * counters are calibrated against when measuring the kernels above. */
 int flhip_copy_bytes(const void* src, void* dst, size_t bytes, void* stream);
 
+/* ---- rnn / rnnBackward (flashlight/fl/autograd/tensor/AutogradExtension.h:96-106,
+ * 167-179) with the semantics and the flat weight order of the cuDNN calls behind
+ * CudnnAutogradExtension::rnn (backend/cudnn/RNN.cpp:62-375): per pseudo-layer
+ * (layer-major, forward direction first) the input matrices of every gate
+ * ([hidden][in], row-major) then the recurrent ones; after all matrices, per
+ * pseudo-layer the input biases then the recurrent biases.  Gates: LSTM i, f, g, o;
+ * GRU r, z, n.  mode: 0 ReLU, 1 tanh, 2 LSTM, 3 GRU (fl::RnnMode).  x is Flashlight
+ * [input, batch, seq] (memory [seq][batch][input]), hx / cx / hy / cy
+ * [hidden, batch, layers*dirs], y [hidden*dirs, batch, seq].  fp32 only; no dropout. */
+typedef struct flhip_rnn_desc {
+  int32_t input_size, hidden_size, num_layers, bidirectional, mode, seq_len, batch, dtype;
+} flhip_rnn_desc;
+/* number of weight elements (cudnnGetRNNParamsSize / element size); 0 for a bad descriptor */
+size_t flhip_rnn_param_count(const flhip_rnn_desc* d);
+/* the reserve buffer carries the forward pass's states and gate activations to the
+ * backward pass (cuDNN's reserve space, RNN.cpp:154-160); the workspace is scratch */
+size_t flhip_rnn_reserve_bytes(const flhip_rnn_desc* d);
+size_t flhip_rnn_workspace_bytes(const flhip_rnn_desc* d);
+/* hx, cx may be NULL (zero initial state); cy may be NULL */
+int flhip_rnn_fwd(const flhip_rnn_desc* d, const void* x, const void* hx, const void* cx,
+                  const void* w, void* y, void* hy, void* cy, void* reserve,
+                  size_t reserve_bytes, void* workspace, size_t workspace_bytes, void* stream);
+/* dy, dhy, dcy may be NULL (zero gradient, the closure's empty tensors,
+ * Functions.cpp:1677-1699); dhx, dcx may be NULL; dw has flhip_rnn_param_count elements */
+int flhip_rnn_bwd(const flhip_rnn_desc* d, const void* x, const void* w, const void* dy,
+                  const void* dhy, const void* dcy, const void* reserve, size_t reserve_bytes,
+                  void* dx, void* dhx, void* dcx, void* dw, void* workspace,
+                  size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
