@@ -14,7 +14,11 @@
 namespace fl {
 
 namespace detail {
-struct RNNGradData;
+// gradients of the three rnn outputs, filled by the closures of the outputs that were
+// differentiated (flashlight/fl/autograd/tensor/AutogradOps.h:356-360)
+struct RNNGradData {
+  Tensor dy, dhy, dcy;
+};
 // Opaque forward -> backward state (AutogradExtension.h:26-42).  The caller
 // creates the payload only when some input needs a gradient
 // (flashlight/fl/autograd/Functions.h:84-89); the forward op fills `data`.

@@ -1,6 +1,7 @@
 #include "Functions.h"
 
 #include <algorithm>
+#include <tuple>
 #include <unordered_set>
 
 #include "flhip.h"
@@ -205,6 +206,45 @@ Variable batchnorm(const Variable& input, const Variable& weight, const Variable
     if (!bs.isEmpty()) bs.addGrad(Variable(std::get<2>(g).reshaped(bs.shape()).astype(bs.type()), false));
   };
   return Variable(output, {input, weight, bias}, gradFunc);
+}
+
+std::tuple<Variable, Variable, Variable> rnn(const Variable& input, const Variable& hiddenState,
+                                             const Variable& cellState, const Variable& weights,
+                                             int hiddenSize, int numLayers, RnnMode mode,
+                                             bool bidirectional, float dropProb) {
+  auto payload = createPayload({&input, &hiddenState, &cellState, &weights});
+  Tensor output, hiddenOut, cellOut;
+  std::tie(output, hiddenOut, cellOut) =
+      ext(input).rnn(input.tensor(), hiddenState.tensor(), cellState.tensor(), weights.tensor(), hiddenSize,
+                     numLayers, mode, bidirectional, dropProb, payload);
+  auto gradData = std::make_shared<detail::RNNGradData>();
+  auto gradFunc = [output, numLayers, hiddenSize, mode, bidirectional, dropProb, gradData, payload](
+                      std::vector<Variable>& inputs, const Variable&) {
+    auto& in = inputs[0];
+    auto& hs = inputs[1];
+    auto& cs = inputs[2];
+    auto& wt = inputs[3];
+    if (!(in.isCalcGrad() || hs.isCalcGrad() || cs.isCalcGrad() || wt.isCalcGrad())) return;
+    auto g = ext(in).rnnBackward(in.tensor(), hs.tensor(), cs.tensor(), wt.tensor(), gradData, output, numLayers,
+                                 hiddenSize, mode, bidirectional, dropProb, payload);
+    in.addGrad(Variable(std::get<0>(g).astype(in.type()), false));
+    if (!hs.isEmpty()) hs.addGrad(Variable(std::get<1>(g).astype(hs.type()), false));
+    if (!cs.isEmpty()) cs.addGrad(Variable(std::get<2>(g).astype(cs.type()), false));
+    wt.addGrad(Variable(std::get<3>(g).astype(wt.type()), false));
+  };
+  // one node that owns the backward call; the three outputs hang off it and only record
+  // their gradients (Functions.cpp:1675-1703)
+  Variable dummy(Tensor(), {input, hiddenState, cellState, weights}, gradFunc);
+  auto record = [gradData](Tensor detail::RNNGradData::*slot) {
+    return [gradData, slot](std::vector<Variable>& inputs, const Variable& gradOutput) {
+      if (!inputs[0].isGradAvailable()) inputs[0].addGrad(Variable(Tensor(), false));
+      (*gradData).*slot = gradOutput.tensor();
+    };
+  };
+  Variable yv(output, {dummy}, record(&detail::RNNGradData::dy));
+  Variable hyv(hiddenOut, {dummy}, record(&detail::RNNGradData::dhy));
+  Variable cyv(cellOut, {dummy}, record(&detail::RNNGradData::dcy));
+  return std::make_tuple(yv, hyv, cyv);
 }
 
 namespace {

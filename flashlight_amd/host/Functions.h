@@ -10,6 +10,7 @@
 
 #include <functional>
 #include <memory>
+#include <tuple>
 #include <vector>
 
 #include "AutogradExtension.h"
@@ -66,6 +67,13 @@ Variable pool2d(const Variable& input, int wx, int wy, int sx = 1, int sy = 1, i
 Variable batchnorm(const Variable& input, const Variable& weight, const Variable& bias,
                    Variable& runningMean, Variable& runningVar, const std::vector<int>& axes,
                    bool train, double momentum, double epsilon);
+
+// fl::rnn (Functions.cpp:1606-1706): input [input, batch, seq], states [hidden, batch,
+// layers*dirs] (empty = zeros), weights flat in cuDNN's order -> (output, hidden, cell)
+std::tuple<Variable, Variable, Variable> rnn(const Variable& input, const Variable& hiddenState,
+                                             const Variable& cellState, const Variable& weights,
+                                             int hiddenSize, int numLayers, RnnMode mode,
+                                             bool bidirectional, float dropProb);
 
 // flashlight/fl/common/Defines.h:83-87
 enum class ReduceMode { NONE = 0, MEAN = 1, SUM = 2 };

@@ -348,17 +348,100 @@ std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::batchnormBackward(
   return std::make_tuple(gradInput, gradWeight, gradBias);   // always all three (:278)
 }
 
-// ---- rnn: not part of this backend ------------------------------------------------
-std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::rnn(
-    const Tensor&, const Tensor&, const Tensor&, const Tensor&, const int, const int, const RnnMode,
-    const bool, const float, std::shared_ptr<detail::AutogradPayload>) {
-  throw std::runtime_error("HipAutogradExtension::rnn is not implemented");
+// ---- rnn (flashlight/fl/autograd/tensor/backend/cudnn/RNN.cpp:62-375) -------------------
+namespace {
+struct HipRnnPayload : detail::AutogradPayloadData {
+  Tensor reserve;   // states and gate activations of the forward pass
+};
+
+flhip_rnn_desc rnnDesc(const Tensor& input, int hiddenSize, int numLayers, RnnMode mode, bool bidirectional) {
+  if (input.type() != dtype::f32) throw std::runtime_error("HipAutogradExtension::rnn: f32 only");
+  flhip_rnn_desc d{};
+  d.input_size = (int32_t)input.dim(0);
+  d.batch = input.ndim() < 2 ? 1 : (int32_t)input.dim(1);
+  d.seq_len = input.ndim() < 3 ? 1 : (int32_t)input.dim(2);
+  d.hidden_size = hiddenSize;
+  d.num_layers = numLayers;
+  d.bidirectional = bidirectional ? 1 : 0;
+  d.mode = (int32_t)mode;
+  d.dtype = FLHIP_F32;
+  return d;
 }
+}  // namespace
+
+std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::rnn(
+    const Tensor& input, const Tensor& hiddenState, const Tensor& cellState, const Tensor& weights,
+    const int hiddenSize, const int numLayers, const RnnMode mode, const bool bidirectional,
+    const float dropProb, std::shared_ptr<detail::AutogradPayload> autogradPayload) {
+  if (input.isEmpty()) throw std::runtime_error("HipAutogradExtension::rnn: empty input");
+  for (const Tensor* t : {&hiddenState, &cellState, &weights})
+    if (!t->isEmpty() && t->type() != input.type())
+      throw std::invalid_argument("rnn doesn't support binary operations with Tensors of different types");
+  if (dropProb != 0.f)
+    throw std::runtime_error("HipAutogradExtension::rnn: dropout between layers is not supported");
+  const flhip_rnn_desc d = rnnDesc(input, hiddenSize, numLayers, mode, bidirectional);
+  const Dim totalLayers = numLayers * (bidirectional ? 2 : 1), outSize = hiddenSize * (bidirectional ? 2 : 1);
+  // RNN.cpp:97-113
+  if (!hiddenState.isEmpty()) {
+    const Dim hb = hiddenState.ndim() < 2 ? 1 : hiddenState.dim(1), hl = hiddenState.ndim() < 3 ? 1 : hiddenState.dim(2);
+    if (!(hiddenState.dim(0) == hiddenSize && hb == d.batch && hl == totalLayers))
+      throw std::invalid_argument("invalid hidden state dims for RNN");
+  }
+  if (!cellState.isEmpty() &&
+      !(mode == RnnMode::LSTM && cellState.ndim() == 3 && cellState.dim(0) == hiddenSize &&
+        cellState.dim(1) == d.batch && cellState.dim(2) == totalLayers))
+    throw std::invalid_argument("invalid cell state dims for RNN");
+  if ((size_t)weights.elements() != flhip_rnn_param_count(&d) || flhip_rnn_param_count(&d) == 0)
+    throw std::invalid_argument("invalid # of parameters or wrong input shape for RNN");   // :123-133
+
+  Tensor y({outSize, d.batch, d.seq_len}, input.type());
+  Tensor hy({(Dim)hiddenSize, d.batch, totalLayers}, input.type());
+  Tensor cy = mode == RnnMode::LSTM ? Tensor(hy.shape(), input.type()) : Tensor();
+  const size_t resBytes = flhip_rnn_reserve_bytes(&d), wsBytes = flhip_rnn_workspace_bytes(&d);
+  Tensor reserve({(Dim)resBytes}, dtype::u8);
+  Tensor ws = workspace(wsBytes);
+  DevicePtr xp(input), hp(hiddenState), cp(cellState), wp(weights), yp(y), hyp(hy), cyp(cy), rp(reserve), wsp(ws);
+  check(flhip_rnn_fwd(&d, xp.get(), hp.get(), cp.get(), wp.get(), yp.get(), hyp.get(), cyp.get(), rp.get(),
+                      resBytes, wsp.get(), wsBytes, hipBackendStream()));
+  if (autogradPayload) {
+    auto payload = std::make_shared<HipRnnPayload>();
+    payload->reserve = reserve;
+    autogradPayload->data = payload;
+  }
+  return std::make_tuple(y, hy, cy);
+}
+
 std::tuple<Tensor, Tensor, Tensor, Tensor> HipAutogradExtension::rnnBackward(
-    const Tensor&, const Tensor&, const Tensor&, const Tensor&,
-    const std::shared_ptr<detail::RNNGradData>, const Tensor&, const int, const int, const RnnMode,
-    const bool, const float, std::shared_ptr<detail::AutogradPayload>) {
-  throw std::runtime_error("HipAutogradExtension::rnnBackward is not implemented");
+    const Tensor& input, const Tensor& hiddenState, const Tensor& cellState, const Tensor& weights,
+    const std::shared_ptr<detail::RNNGradData> gradData, const Tensor& output, const int numLayers,
+    const int hiddenSize, const RnnMode mode, const bool bidirectional, const float,
+    std::shared_ptr<detail::AutogradPayload> autogradPayload) {
+  if (!autogradPayload || !autogradPayload->data)   // RNN.cpp:246-249
+    throw std::invalid_argument("HipAutogradExtension::rnnBackward given null or empty autograd payload");
+  auto payload = std::dynamic_pointer_cast<HipRnnPayload>(autogradPayload->data);
+  if (!payload) throw std::invalid_argument("rnnBackward: payload of another operation");
+  if (!gradData) throw std::invalid_argument("rnnBackward: no gradient data");
+  const flhip_rnn_desc d = rnnDesc(input, hiddenSize, numLayers, mode, bidirectional);
+  const Dim totalLayers = numLayers * (bidirectional ? 2 : 1);
+  // output gradients nobody produced are zero (RNN.cpp:262-275)
+  for (const Tensor* t : {&gradData->dy, &gradData->dhy, &gradData->dcy})
+    if (!t->isEmpty() && t->type() != dtype::f32) throw std::runtime_error("rnnBackward: f32 only");
+  if (!gradData->dy.isEmpty() && gradData->dy.elements() != output.elements())
+    throw std::invalid_argument("rnnBackward: gradient of the output has the wrong size");
+  Tensor dx(input.shape(), input.type());
+  Tensor dhx({(Dim)hiddenSize, d.batch, totalLayers}, input.type());
+  Tensor dcx = mode == RnnMode::LSTM ? Tensor(dhx.shape(), input.type()) : Tensor();
+  Tensor dw(weights.shape(), weights.type());
+  const size_t resBytes = flhip_rnn_reserve_bytes(&d), wsBytes = flhip_rnn_workspace_bytes(&d);
+  Tensor ws = workspace(wsBytes);
+  DevicePtr xp(input), wp(weights), dyp(gradData->dy), dhyp(gradData->dhy), dcyp(gradData->dcy),
+      rp(payload->reserve), dxp(dx), dhxp(dhx), dcxp(dcx), dwp(dw), wsp(ws);
+  check(flhip_rnn_bwd(&d, xp.get(), wp.get(), dyp.get(), dhyp.get(), mode == RnnMode::LSTM ? dcyp.get() : nullptr,
+                      rp.get(), resBytes, dxp.get(), dhxp.get(), dcxp.get(), dwp.get(), wsp.get(), wsBytes,
+                      hipBackendStream()));
+  (void)hiddenState;
+  (void)cellState;
+  return std::make_tuple(dx, dhx, dcx, dw);
 }
 
 }  // namespace fl

@@ -1,5 +1,7 @@
 #include "Modules.h"
 
+#include "flhip.h"
+
 #include <algorithm>
 #include <cmath>
 #include <random>
@@ -307,6 +309,59 @@ std::string LayerNorm::prettyString() const {
   ss << "LayerNorm ( axis : { ";
   for (int a : axis_) ss << a << " ";
   ss << "} , size : " << axisSize_ << ")";
+  return ss.str();
+}
+
+// ---- RNN -------------------------------------------------------------------------------
+int64_t detail::getNumRnnParams(int inputSize, int hiddenSize, int numLayers, RnnMode mode, bool bidirectional) {
+  flhip_rnn_desc d{};
+  d.input_size = inputSize; d.hidden_size = hiddenSize; d.num_layers = numLayers;
+  d.bidirectional = bidirectional ? 1 : 0; d.mode = (int32_t)mode; d.seq_len = 1; d.batch = 1; d.dtype = FLHIP_F32;
+  const size_t n = flhip_rnn_param_count(&d);
+  if (n == 0) throw std::invalid_argument("RNN: invalid sizes");
+  return (int64_t)n;
+}
+
+RNN::RNN(int inputSize, int hiddenSize, int numLayers, RnnMode mode, bool bidirectional, float dropProb)
+    : inputSize_(inputSize), hiddenSize_(hiddenSize), numLayers_(numLayers), mode_(mode),
+      bidirectional_(bidirectional), dropProb_(dropProb) {
+  const int64_t n = detail::getNumRnnParams(inputSize_, hiddenSize_, numLayers_, mode_, bidirectional_);
+  const double stdv = std::sqrt(1.0 / (double)hiddenSize_);
+  params_ = {uniform(Shape({(Dim)n}), -stdv, stdv, dtype::f32, true)};
+}
+
+std::vector<Variable> RNN::forward(const std::vector<Variable>& inputs) {
+  if (inputs.empty() || inputs.size() > 3) throw std::invalid_argument("Invalid inputs size");
+  const Variable& input = inputs[0];
+  const Variable hiddenState = inputs.size() >= 2 ? inputs[1] : Variable();
+  const Variable cellState = inputs.size() == 3 ? inputs[2] : Variable();
+  const float dropProb = train_ ? dropProb_ : 0.f;
+  auto res = rnn(input, hiddenState, cellState, params_[0].astype(input.type()), hiddenSize_, numLayers_, mode_,
+                 bidirectional_, dropProb);
+  std::vector<Variable> output(1, std::get<0>(res));
+  if (inputs.size() >= 2) output.push_back(std::get<1>(res));
+  if (inputs.size() == 3) output.push_back(std::get<2>(res));
+  return output;
+}
+
+std::tuple<Variable, Variable> RNN::forward(const Variable& input, const Variable& hiddenState) {
+  auto r = forward(std::vector<Variable>{input, hiddenState});
+  return std::make_tuple(r[0], r[1]);
+}
+
+std::tuple<Variable, Variable, Variable> RNN::forward(const Variable& input, const Variable& hiddenState,
+                                                      const Variable& cellState) {
+  auto r = forward(std::vector<Variable>{input, hiddenState, cellState});
+  return std::make_tuple(r[0], r[1], r[2]);
+}
+
+std::string RNN::prettyString() const {
+  std::ostringstream ss;
+  ss << (mode_ == RnnMode::RELU ? "RNN (relu)" : mode_ == RnnMode::TANH ? "RNN (tanh)" : mode_ == RnnMode::LSTM ? "LSTM" : "GRU");
+  ss << " (" << inputSize_ << "->" << (bidirectional_ ? 2 * hiddenSize_ : hiddenSize_) << ")";
+  if (numLayers_ > 1) ss << " (" << numLayers_ << "-layer)";
+  if (bidirectional_) ss << " (bidirectional)";
+  if (dropProb_ > 0) ss << " (dropout=" << dropProb_ << ")";
   return ss.str();
 }
 

@@ -209,6 +209,31 @@ class Linear : public UnaryModule {
   bool bias_;
 };
 
+// flashlight/fl/nn/modules/RNN.cpp:19-170: one flat weight vector in cuDNN's order,
+// uniform(+-sqrt(1/hidden)); forward takes {input[, hidden[, cell]]} and returns as many
+// outputs as it got inputs
+namespace detail {
+int64_t getNumRnnParams(int inputSize, int hiddenSize, int numLayers, RnnMode mode, bool bidirectional);
+}
+class RNN : public Module {
+ public:
+  RNN(int inputSize, int hiddenSize, int numLayers, RnnMode mode, bool bidirectional = false,
+      float dropProb = 0.0);
+  std::vector<Variable> forward(const std::vector<Variable>& inputs) override;
+  Variable forward(const Variable& input) { return forward(std::vector<Variable>{input}).front(); }
+  Variable operator()(const Variable& input) { return forward(input); }
+  std::tuple<Variable, Variable> forward(const Variable& input, const Variable& hiddenState);
+  std::tuple<Variable, Variable, Variable> forward(const Variable& input, const Variable& hiddenState,
+                                                   const Variable& cellState);
+  std::string prettyString() const override;
+
+ private:
+  int inputSize_, hiddenSize_, numLayers_;
+  RnnMode mode_;
+  bool bidirectional_;
+  float dropProb_;
+};
+
 class ReLU : public UnaryModule {          // Activations.cpp:58-70
  public:
   using UnaryModule::forward;

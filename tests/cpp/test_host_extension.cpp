@@ -87,7 +87,7 @@ static void testRegistration() {
     return std::unique_ptr<AutogradExtension>(new HipAutogradExtension());
   }));
   CHECK(throws<std::invalid_argument>([] { getAutogradExtension(TensorBackendType::Stub); }));
-  CHECK(throws<std::runtime_error>([&] {
+  CHECK(throws<std::runtime_error>([&] {   // an empty input
     Tensor t;
     e.rnn(t, t, t, t, 1, 1, RnnMode::LSTM, false, 0.f, nullptr);
   }));
@@ -709,6 +709,78 @@ static void testSpeechStack() {
   CHECK(relL2(hostOf(in.grad()), grad) <= 3e-4);
 }
 
+// rnn / rnnBackward through the closure and the RNN module (flashlight/fl/test/autograd/
+// AutogradRnnTest.cpp:24-90 uses 2 layers, hidden 2, input 2, bidirectional; here against
+// the CPU checker instead of finite differences)
+static void testRnn() {
+  std::printf("rnn\n");
+  const RnnMode modes[4] = {RnnMode::RELU, RnnMode::TANH, RnnMode::LSTM, RnnMode::GRU};
+  const int64_t expected[4] = {56, 56, 224, 168};   // AutogradRnnTest.cpp:37-49
+  for (int mi = 0; mi < 4; ++mi) {
+    const RnnMode mode = modes[mi];
+    const int I = 2, H = 2, L = 2, B = 2, T = 3, D = 2;
+    CHECK(detail::getNumRnnParams(I, H, L, mode, true) == expected[mi]);
+    flref_rnn d{I, H, L, 1, (int32_t)mode, T, B};
+    const int64_t n = flref_rnn_param_count(&d);
+    CHECK(n == expected[mi]);
+    auto w = randn((size_t)n, 80 + mi, 0.5f), x = randn((size_t)T * B * I, 90 + mi);
+    auto hx = randn((size_t)L * D * B * H, 91 + mi), cx = randn(hx.size(), 92 + mi);
+    auto dy = randn((size_t)T * B * D * H, 93 + mi), dhy = randn(hx.size(), 94 + mi);
+    const bool lstm = mode == RnnMode::LSTM;
+    std::vector<float> y(dy.size()), hy(hx.size()), cy(hx.size());
+    flref_rnn_fwd(&d, x.data(), hx.data(), lstm ? cx.data() : nullptr, w.data(), y.data(), hy.data(), lstm ? cy.data() : nullptr);
+    std::vector<float> dx(x.size()), dhx(hx.size()), dcx(hx.size()), dw(w.size());
+    flref_rnn_bwd(&d, x.data(), hx.data(), lstm ? cx.data() : nullptr, w.data(), dy.data(), nullptr, nullptr, dx.data(),
+                  dhx.data(), lstm ? dcx.data() : nullptr, dw.data());
+
+    Variable in(Tensor::fromVector({I, B, T}, x), true), wt(Tensor::fromVector({(Dim)n}, w), true);
+    Variable h0(Tensor::fromVector({H, B, L * D}, hx), true);
+    Variable c0 = lstm ? Variable(Tensor::fromVector({H, B, L * D}, cx), true) : Variable();
+    Variable yv, hyv, cyv;
+    std::tie(yv, hyv, cyv) = rnn(in, h0, c0, wt, H, L, mode, true, 0.f);
+    CHECK(yv.shape() == Shape({D * H, B, T}) && hyv.shape() == Shape({H, B, L * D}));
+    CHECK(relL2(hostOf(yv), y) <= 1e-4 && relL2(hostOf(hyv), hy) <= 1e-4);
+    if (lstm) CHECK(relL2(hostOf(cyv), cy) <= 1e-4); else CHECK(cyv.isEmpty());
+    yv.backward(Variable(Tensor::fromVector(yv.shape(), dy), false));
+    CHECK(relL2(hostOf(in.grad()), dx) <= 2e-4 && relL2(hostOf(wt.grad()), dw) <= 2e-4);
+    CHECK(relL2(hostOf(h0.grad()), dhx) <= 2e-4);
+    if (lstm) CHECK(relL2(hostOf(c0.grad()), dcx) <= 2e-4);
+
+    // only the final hidden state differentiated, no initial states
+    flref_rnn_bwd(&d, x.data(), nullptr, nullptr, w.data(), nullptr, dhy.data(), nullptr, dx.data(), dhx.data(),
+                  lstm ? dcx.data() : nullptr, dw.data());
+    Variable in2(Tensor::fromVector({I, B, T}, x), true), wt2(Tensor::fromVector({(Dim)n}, w), true);
+    std::tie(yv, hyv, cyv) = rnn(in2, Variable(), Variable(), wt2, H, L, mode, true, 0.f);
+    hyv.backward(Variable(Tensor::fromVector(hyv.shape(), dhy), false));
+    CHECK(relL2(hostOf(in2.grad()), dx) <= 2e-4 && relL2(hostOf(wt2.grad()), dw) <= 2e-4);
+
+    // errors of the reference (cudnn/RNN.cpp:97-133)
+    Variable badw(Tensor::fromVector({(Dim)n - 1}, std::vector<float>((size_t)n - 1, 0.f)), false);
+    CHECK(throws<std::invalid_argument>([&] { rnn(in2, Variable(), Variable(), badw, H, L, mode, true, 0.f); }));
+    Variable badh(Tensor::fromVector({H + 1, B, L * D}, std::vector<float>((size_t)(H + 1) * B * L * D, 0.f)), false);
+    CHECK(throws<std::invalid_argument>([&] { rnn(in2, badh, Variable(), wt2, H, L, mode, true, 0.f); }));
+    if (!lstm) CHECK(throws<std::invalid_argument>([&] { rnn(in2, Variable(), h0, wt2, H, L, mode, true, 0.f); }));
+  }
+  // the module: parameter vector, one to three inputs -> as many outputs
+  setSeed(23);
+  RNN lstm(5, 4, 2, RnnMode::LSTM, true);
+  CHECK(lstm.params().size() == 1 && lstm.param(0).elements() == detail::getNumRnnParams(5, 4, 2, RnnMode::LSTM, true));
+  for (float f : hostOf(lstm.param(0))) CHECK(std::fabs(f) <= 0.5f);
+  CHECK(lstm.prettyString() == "LSTM (5->8) (2-layer) (bidirectional)");
+  Variable xin(Tensor::fromVector({5, 3, 6}, randn(90, 99)), true);
+  Variable out = lstm(xin);
+  CHECK(out.shape() == Shape({8, 3, 6}));
+  auto r3 = lstm.forward(std::vector<Variable>{xin, Variable(), Variable()});
+  CHECK(r3.size() == 3 && r3[1].shape() == Shape({4, 3, 4}) && r3[2].shape() == Shape({4, 3, 4}));
+  out.backward(Variable(Tensor::full(out.shape(), 1., dtype::f32), false));
+  CHECK(lstm.param(0).isGradAvailable() && xin.isGradAvailable());
+  CHECK(throws<std::invalid_argument>([&] { lstm.forward(std::vector<Variable>{}); }));
+  RNN drop(5, 4, 2, RnnMode::GRU, false, 0.3f);
+  CHECK(throws<std::runtime_error>([&] { drop(xin); }));   // dropout between layers is not provided
+  drop.eval();
+  CHECK(drop(xin).shape() == Shape({4, 3, 6}));            // eval: no dropout (RNN.cpp:74)
+}
+
 // a crash of the host code should say where: unbuffered output and a backtrace
 static void onCrash(int sig) {
   void* frames[64];
@@ -742,6 +814,7 @@ int main() {
     testLayerNormModule();
     testBottleneck();
     testSpeechStack();
+    testRnn();
     fl::sync();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
