@@ -35,13 +35,14 @@ int mfma_slab_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const 
 // 1x1 convolutions without padding as GEMMs (conv2d_mfma_pointwise.hip); same return
 // convention.
 int mfma_pointwise_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w,
-                            const float* bias, void* y, hipStream_t s);
+                            const float* bias, void* y, hipStream_t s, int ksplit = 1);
 int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w,
-                                 void* dx, hipStream_t s, const float* bias = nullptr);
+                                 void* dx, hipStream_t s, const float* bias = nullptr, int ksplit = 1);
 // column-major C = op(A) op(B) on the 1x1 kernels (mode 0: A B, 1: A^T B, 2: A B^T);
 // -1 when it does not apply
 int mfma_gemm(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,
-              const float* bias_rows, hipStream_t s);
+              const float* bias_rows, hipStream_t s, int ksplit = 1);
+int mfma_gemm_slices(int K, int ksplit);
 // windows with several taps on the same tile machinery, any stride / padding / dilation
 int mfma_tapped_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w,
                          const float* bias, void* y, hipStream_t s);
@@ -50,7 +51,8 @@ int mfma_tapped_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, cons
 size_t mfma_pointwise_wgrad_ws(const ConvGeom& g);
 // windows = false: only 1x1 without padding; true: any window, one tap per workgroup
 int mfma_pointwise_wgrad(const ConvGeom& g, int dtype, const void* x, const void* dy, float* dw,
-                         float* db, void* ws, size_t ws_bytes, bool windows, hipStream_t s);
+                         float* db, void* ws, size_t ws_bytes, bool windows, hipStream_t s,
+                         int max_slices = 0);
 
 // Adds the slices of a split filter gradient in a fixed order (conv2d_mfma_wgrad.hip):
 // slice s holds E floats of dw followed by K floats of db at part + s * (E + K).

@@ -54,6 +54,8 @@ struct PwParams {
   int src_map, dst_map;  // 1 = that side goes through the lattice
   int vec_w;             // weight tile by 16-byte loads
   int nchunks, mtiles, ptiles;
+  int cps;               // chunks per contraction slice (blockIdx.y); == nchunks without split-K
+  unsigned dst_slice;    // elements between the partial results of consecutive slices
   unsigned src_bytes, wgt_bytes, dst_bytes;
 };
 
@@ -136,7 +138,9 @@ pointwise_conv_kernel(PwParams p, const T* __restrict__ src, const T* __restrict
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int tileP0 = ptile * BN;
-  const int n = p.nchunks;
+  // split-K: slice blockIdx.y takes chunks [c0, c0 + n) and writes its own partial result
+  const int c0 = blockIdx.y * p.cps;
+  const int n = min(p.nchunks - c0, p.cps);
 
   if (wave < 4) {
     // ================================ loaders ====================================
@@ -160,7 +164,7 @@ pointwise_conv_kernel(PwParams p, const T* __restrict__ src, const T* __restrict
     const int m0 = mtile * BM;
 
     auto load = [&](int c, float4 (&sr)[NJ][2], float4 (&wr)[2]) {
-      const int k0 = c * KC;
+      const int k0 = (c0 + c) * KC;
       if (VEC) {
 #pragma unroll
         for (int i = 0; i < NJ; ++i) {
@@ -278,7 +282,7 @@ pointwise_conv_kernel(PwParams p, const T* __restrict__ src, const T* __restrict
   }
 
   // ---- epilogue: a lane holds positions Pg .. Pg+3 of channel ch per accumulator ----
-  const __amdgpu_buffer_rsrc_t drsrc = make_rsrc(dst, p.dst_bytes);
+  const __amdgpu_buffer_rsrc_t drsrc = make_rsrc(dst + (size_t)blockIdx.y * p.dst_slice, p.dst_bytes);
 #pragma unroll
   for (int i = 0; i < PT; ++i) {
     const int Pg = tileP0 + (wp * PT + i) * 16 + 4 * fg;
@@ -286,7 +290,7 @@ pointwise_conv_kernel(PwParams p, const T* __restrict__ src, const T* __restrict
     for (int j = 0; j < 2; ++j) {
       const int ch = mtile * BM + wc * 32 + j * 16 + fr;
       floatx4 v = acc[i][j];
-      if (bias && ch < p.Mo) {
+      if (bias && ch < p.Mo && blockIdx.y == 0) {
         const float bv = bias[ch];
         v[0] += bv; v[1] += bv; v[2] += bv; v[3] += bv;
       }
@@ -328,7 +332,9 @@ int launch_tile(const PwParams& p0, const void* src, const void* wgt, const floa
   auto kernel = pointwise_conv_kernel<T, BWD, PT, VEC>;
   if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
   const unsigned grid = (unsigned)(((p.ptiles + 7) / 8) * 8 * p.mtiles);
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(MFMA_THREADS), shmem, s, p, static_cast<const T*>(src),
+  if (p.cps <= 0 || p.cps > p.nchunks) p.cps = p.nchunks;
+  const unsigned slices = (unsigned)((p.nchunks + p.cps - 1) / p.cps);
+  hipLaunchKernelGGL(kernel, dim3(grid, slices), dim3(MFMA_THREADS), shmem, s, p, static_cast<const T*>(src),
                      static_cast<const T*>(wgt), bias, static_cast<T*>(dst));
   return check_launch("conv2d 1x1 (mfma)");
 }
@@ -859,7 +865,7 @@ pointwise_wgrad_kernel(PwWgradParams p, const T* __restrict__ x, const T* __rest
     }
 }
 
-bool pw_wgrad_plan(const ConvGeom& g, PwWgradParams* p) {
+bool pw_wgrad_plan(const ConvGeom& g, PwWgradParams* p, int max_slices = 0) {
   if (g.groups != 1) return false;
   // 64-channel column tiles: with few input channels the kernel that flattens
   // (channel, tap) into the columns wastes less
@@ -878,6 +884,7 @@ bool pw_wgrad_plan(const ConvGeom& g, PwWgradParams* p) {
   long long ns = 4ll * mfma_num_cus() / base;
   const long long max_ns = (p->Ptot + 255) / 256;
   if (ns > max_ns) ns = max_ns;
+  if (max_slices > 0 && ns > max_slices) ns = max_slices;
   if (ns < 1) ns = 1;
   long long pps = (p->Ptot + ns - 1) / ns;
   pps = (pps + PC - 1) / PC * PC;
@@ -889,7 +896,7 @@ bool pw_wgrad_plan(const ConvGeom& g, PwWgradParams* p) {
 }  // namespace
 
 int mfma_pointwise_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w,
-                            const float* bias, void* y, hipStream_t s) {
+                            const float* bias, void* y, hipStream_t s, int ksplit) {
   if (!pw_applies(g)) return -1;
   const long long esz = dtype == FLHIP_F32 ? 4 : 2;
   const long long sb = (long long)g.N * g.C * g.H * g.W * esz, db = (long long)g.N * g.K * g.OH * g.OW * esz;
@@ -906,12 +913,18 @@ int mfma_pointwise_conv_fwd(const ConvGeom& g, int dtype, const void* x, const v
   p.mtiles = (g.K + BM - 1) / BM;
   p.src_bytes = (unsigned)sb; p.wgt_bytes = (unsigned)wb; p.dst_bytes = (unsigned)db;
   const bool vec = !p.src_map && p.P % 4 == 0;
+  if (ksplit > 1) {
+    if (dtype != FLHIP_F32 || db * ksplit >= (1ll << 31)) return -1;
+    p.cps = (p.nchunks + ksplit - 1) / ksplit;
+    p.dst_slice = (unsigned)(db / esz);
+    p.dst_bytes = (unsigned)db;
+  }
   return dtype == FLHIP_F32 ? launch_pw<float, false>(p, vec, x, w, bias, y, s)
                             : launch_pw<bf16_t, false>(p, vec, x, w, bias, y, s);
 }
 
 int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
-                                 hipStream_t s, const float* bias) {
+                                 hipStream_t s, const float* bias, int ksplit) {
   if (!pw_applies(g)) return -1;
   const long long esz = dtype == FLHIP_F32 ? 4 : 2;
   const long long sb = (long long)g.N * g.K * g.OH * g.OW * esz, db = (long long)g.N * g.C * g.H * g.W * esz;
@@ -942,6 +955,11 @@ int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, c
       hipLaunchKernelGGL((zero_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, static_cast<bf16_t*>(dx), n16, nel);
   }
   const bool vec = full && p.P % 4 == 0;
+  if (ksplit > 1) {
+    if (dtype != FLHIP_F32 || !full || db * ksplit >= (1ll << 31)) return -1;
+    p.cps = (p.nchunks + ksplit - 1) / ksplit;
+    p.dst_slice = (unsigned)(db / esz);
+  }
   return dtype == FLHIP_F32 ? launch_pw<float, true>(p, vec, dy, w, bias, dx, s)
                             : launch_pw<bf16_t, true>(p, vec, dy, w, bias, dx, s);
 }
@@ -953,11 +971,11 @@ size_t mfma_pointwise_wgrad_ws(const ConvGeom& g) {
 }
 
 int mfma_pointwise_wgrad(const ConvGeom& g, int dtype, const void* x, const void* dy, float* dw,
-                         float* db, void* ws, size_t ws_bytes, bool windows, hipStream_t s) {
+                         float* db, void* ws, size_t ws_bytes, bool windows, hipStream_t s, int max_slices) {
   if (!dw) return -1;   // bias gradient alone: the plain reduction kernel
   if (!windows && !pw_applies(g)) return -1;
   PwWgradParams p{};
-  if (!pw_wgrad_plan(g, &p)) return -1;
+  if (!pw_wgrad_plan(g, &p, max_slices)) return -1;
   const long long esz = dtype == FLHIP_F32 ? 4 : 2;
   const long long xb = (long long)g.N * g.C * g.H * g.W * esz, yb = (long long)g.N * g.K * g.OH * g.OW * esz;
   if (xb >= (1ll << 31) || yb >= (1ll << 31)) return -1;
@@ -1011,27 +1029,42 @@ int mfma_tapped_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, cons
 //   mode 2, C = A B^T  : B stored (N x K) = [k][n]; C[n][m] = sum_k B[k][n] A[k][m] is the filter
 //                        gradient with the rows of B as dy and of A as x (fp32 only: that kernel
 //                        writes fp32; single slice only: there is no workspace here)
-// bias_rows (fp32[M] or null) is added to every column in modes 0 and 1.  Returns -1 when
-// the product does not fit these kernels.
+// bias_rows (fp32[M] or null) is added to every column in modes 0 and 1.  ksplit > 1 (modes
+// 0 and 1, fp32): the contraction is cut into that many slices at most, slice s writes its
+// partial product at C + s*M*N and the caller adds them (the number of slices written is
+// ceil(chunks / ceil(chunks / ksplit)) with chunks = ceil(K / 32): see mfma_gemm_slices).
+// Returns -1 when the product does not fit these kernels.
 int mfma_gemm(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,
-              const float* bias_rows, hipStream_t s) {
+              const float* bias_rows, hipStream_t s, int ksplit) {
   ConvGeom g{};
   g.H = g.W = g.OH = g.OW = g.KH = g.KW = 1;
   g.sy = g.sx = g.dly = g.dlx = g.groups = 1;
   if (mode == 0) {
     g.N = N; g.C = M; g.K = K; g.Cg = M; g.Kg = K;
-    return mfma_pointwise_conv_bwd_data(g, dtype, B, A, C, s, bias_rows);
+    return mfma_pointwise_conv_bwd_data(g, dtype, B, A, C, s, bias_rows, ksplit);
   }
   if (mode == 1) {
     g.N = N; g.C = K; g.K = M; g.Cg = K; g.Kg = M;
-    return mfma_pointwise_conv_fwd(g, dtype, B, A, bias_rows, C, s);
+    return mfma_pointwise_conv_fwd(g, dtype, B, A, bias_rows, C, s, ksplit);
   }
-  if (mode == 2 && dtype == FLHIP_F32 && !bias_rows) {
+  if (mode == 2 && dtype == FLHIP_F32 && !bias_rows && ksplit <= 1) {
     g.N = K; g.C = M; g.K = N; g.Cg = M; g.Kg = N;
-    if (mfma_pointwise_wgrad_ws(g) != 0) return -1;
-    return mfma_pointwise_wgrad(g, dtype, A, B, static_cast<float*>(C), nullptr, nullptr, 0, false, s);
+    // no workspace here, so one slice of the contraction per tile: fine when there are
+    // enough 64 x 64 tiles to occupy the machine or the contraction is short
+    const long long tiles = (long long)((M + BM - 1) / BM) * ((N + BM - 1) / BM);
+    if (tiles < 64 && mfma_pointwise_wgrad_ws(g) != 0) return -1;
+    return mfma_pointwise_wgrad(g, dtype, A, B, static_cast<float*>(C), nullptr, nullptr, 0, false, s, 1);
   }
   return -1;
+}
+
+// number of partial products mfma_gemm writes for a contraction of length K cut into at
+// most ksplit slices
+int mfma_gemm_slices(int K, int ksplit) {
+  const int chunks = (K + KC - 1) / KC;
+  if (ksplit <= 1) return 1;
+  const int cps = (chunks + ksplit - 1) / ksplit;
+  return (chunks + cps - 1) / cps;
 }
 
 }  // namespace flhip

@@ -18,6 +18,7 @@
 #include <algorithm>
 
 #include "common.h"
+#include "conv2d.h"
 
 extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, int32_t N, int32_t K,
                             int trans_a, int trans_b, const float* bias_rows, int dtype, void* stream);
@@ -99,11 +100,27 @@ Reserve reserve_layout(const RnnGeom& g) {
 
 // workspace, in floats (one call): forward {XP [T*B*GH], RP [B*GH], bias [GH]};
 // backward {dGW [T*B*GH], dGR [T*B*GH], gout [T*B*D*H], gin [T*B*inmax], tmp [T*B*inmax],
-// dh_dir [2*BH], dh_rec [BH], dc [BH]}
+// dh_dir [2*BH], dc [BH], dh_rec [slices*BH]}
+// The recurrent products of one time step are small (batch columns): their contraction is
+// cut into slices so that enough workgroups run, and the gate kernels add the partial
+// products.  Slices for a product with M rows, N columns, contraction K:
+int step_slices(size_t M, size_t N, size_t K, int* ksplit) {
+  const long long tiles = (long long)((M + 63) / 64) * ((N + 63) / 64), chunks = (long long)(K + 31) / 32;
+  // from 32 tiles on, one step is bound by its two launches, not by the product
+  long long k = tiles >= 32 ? 1 : 256 / tiles;
+  if (k > chunks / 4) k = chunks / 4;   // at least four chunks of 32 per slice
+  if (k > 32) k = 32;
+  if (k < 1) k = 1;
+  *ksplit = (int)k;
+  return mfma_gemm_slices((int)K, (int)k);
+}
+
 size_t workspace_floats(const RnnGeom& g) {
   const size_t TB = (size_t)g.T * g.B, inmax = std::max<size_t>(g.I, (size_t)g.D * g.H);
-  const size_t fwd = TB * g.GH + g.B * g.GH + g.GH;
-  const size_t bwd = 2 * TB * g.GH + TB * g.D * g.H + 2 * TB * inmax + 4 * g.BH;
+  int k;
+  const size_t sf = step_slices(g.GH, g.B, g.H, &k), sb = step_slices(g.H, g.B, g.GH, &k);
+  const size_t fwd = TB * g.GH + sf * g.B * g.GH + g.GH;
+  const size_t bwd = 2 * TB * g.GH + TB * g.D * g.H + 2 * TB * inmax + (3 + sb) * g.BH;
   return std::max(fwd, bwd) + 64;
 }
 
@@ -123,15 +140,21 @@ __global__ void __launch_bounds__(256) rnn_init_kernel(const float* __restrict__
   if (i < n) dst[i] = src ? src[i] : 0.f;
 }
 
-__global__ void __launch_bounds__(256) rnn_add2_kernel(const float* __restrict__ a, const float* __restrict__ b,
-                                                       float* __restrict__ out, size_t n) {
+// out = a + sum of nb slices of b (either may be null); out may be a
+__global__ void __launch_bounds__(256) rnn_add2_kernel(const float* a, const float* __restrict__ b, int nb,
+                                                       float* out, size_t n) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n) out[i] = (a ? a[i] : 0.f) + (b ? b[i] : 0.f);
+  if (i >= n) return;
+  float v = a ? a[i] : 0.f;
+  if (b)
+    for (int k = 0; k < nb; ++k) v += b[(size_t)k * n + i];
+  out[i] = v;
 }
 
 struct CellFwd {
   const float* xp;    // [B][GH] input projection (+ biases) of this time step
-  const float* rp;    // [B][GH] recurrent projection
+  const float* rp;    // [nrp][B][GH] recurrent projection, in nrp partial products
+  int nrp;
   const float* bRn;   // GRU: recurrent bias of the n gate [H]
   const float* hp;    // [B][H] state before the step
   const float* cp;    // LSTM
@@ -152,22 +175,30 @@ __global__ void __launch_bounds__(256) rnn_cell_fwd(CellFwd a, int B, int H) {
   const int b = e / H, h = e - b * H;
   constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1;
   const size_t q = (size_t)b * G * H + h;
+  float rp[G];
+#pragma unroll
+  for (int gq = 0; gq < G; ++gq) rp[gq] = 0.f;
+  for (int k = 0; k < a.nrp; ++k) {
+    const float* r = a.rp + (size_t)k * B * G * H + q;
+#pragma unroll
+    for (int gq = 0; gq < G; ++gq) rp[gq] += r[gq * H];
+  }
   float hv;
   if (MODE == RNN_RELU || MODE == RNN_TANH) {
-    const float pre = a.xp[q] + a.rp[q];
+    const float pre = a.xp[q] + rp[0];
     hv = MODE == RNN_RELU ? (pre > 0.f ? pre : 0.f) : tanhf(pre);
     a.gt[q] = hv;
   } else if (MODE == RNN_LSTM) {
-    const float ig = sigm(a.xp[q] + a.rp[q]), fg = sigm(a.xp[q + H] + a.rp[q + H]);
-    const float gg = tanhf(a.xp[q + 2 * H] + a.rp[q + 2 * H]), og = sigm(a.xp[q + 3 * H] + a.rp[q + 3 * H]);
+    const float ig = sigm(a.xp[q] + rp[0]), fg = sigm(a.xp[q + H] + rp[1]);
+    const float gg = tanhf(a.xp[q + 2 * H] + rp[G > 2 ? 2 : 0]), og = sigm(a.xp[q + 3 * H] + rp[G > 3 ? 3 : 0]);
     const float c = fg * a.cp[e] + ig * gg;
     a.cn[e] = c;
     if (a.cy) a.cy[e] = c;
     hv = og * tanhf(c);
     a.gt[q] = ig; a.gt[q + H] = fg; a.gt[q + 2 * H] = gg; a.gt[q + 3 * H] = og;
   } else {
-    const float rg = sigm(a.xp[q] + a.rp[q]), zg = sigm(a.xp[q + H] + a.rp[q + H]);
-    const float rn = a.rp[q + 2 * H] + a.bRn[h];
+    const float rg = sigm(a.xp[q] + rp[0]), zg = sigm(a.xp[q + H] + rp[G > 1 ? 1 : 0]);
+    const float rn = rp[G > 2 ? 2 : 0] + a.bRn[h];
     const float ng = tanhf(a.xp[q + 2 * H] + rg * rn);
     a.rn[e] = rn;
     hv = (1.f - zg) * ng + zg * a.hp[e];
@@ -181,7 +212,8 @@ __global__ void __launch_bounds__(256) rnn_cell_fwd(CellFwd a, int B, int H) {
 struct CellBwd {
   const float* gout;  // gradient of the layer output at this time step, this direction's slice; pitch ldo (may be null)
   const float* dh_a;  // gradient reaching h through the recurrence: direct part ...
-  const float* dh_b;  // ... and the part through the recurrent matrices (either may be null)
+  const float* dh_b;  // ... and the part through the recurrent matrices, in ndhb partial products
+  int ndhb;           //     (either pointer may be null)
   float* dc;          // LSTM: in = gradient of c after the step, out = of c before it
   const float* gt;    // gate activations of the step
   const float* cp;    // LSTM: c before the step
@@ -203,7 +235,8 @@ __global__ void __launch_bounds__(256) rnn_cell_bwd(CellBwd a, int B, int H) {
   const size_t q = (size_t)b * G * H + h;
   float go = a.gout ? a.gout[(size_t)b * a.ldo + h] : 0.f;
   if (a.dh_a) go += a.dh_a[e];
-  if (a.dh_b) go += a.dh_b[e];
+  if (a.dh_b)
+    for (int k = 0; k < a.ndhb; ++k) go += a.dh_b[(size_t)k * B * H + e];
   float direct = 0.f;
   if (MODE == RNN_RELU || MODE == RNN_TANH) {
     const float hv = a.gt[q];
@@ -237,6 +270,19 @@ int mm(const float* A, const float* B, float* C, size_t M, size_t N, size_t K, i
   return flhip_matmul(A, B, C, (int32_t)M, (int32_t)N, (int32_t)K, ta, tb, bias, FLHIP_F32, s);
 }
 
+// C = op(A) B in `*slices` partial products at C + k*M*N (see step_slices)
+int mm_sliced(const float* A, const float* B, float* C, size_t M, size_t N, size_t K, int ta, int* slices,
+              hipStream_t s) {
+  int ksplit;
+  const int ns = step_slices(M, N, K, &ksplit);
+  if (ns > 1 && mfma_gemm(FLHIP_F32, ta ? 1 : 0, A, B, C, (int)M, (int)N, (int)K, nullptr, s, ksplit) >= 0) {
+    *slices = ns;
+    return check_launch("rnn (recurrent product)");
+  }
+  *slices = 1;
+  return mm(A, B, C, M, N, K, ta, 0, nullptr, s);
+}
+
 template <int MODE>
 int forward_pl(const RnnGeom& g, int pl, const float* in, size_t inl, const float* w, const float* hx,
                const float* cx, float* out, float* hy, float* cy, float* res, float* ws, hipStream_t s) {
@@ -250,7 +296,8 @@ int forward_pl(const RnnGeom& g, int pl, const float* in, size_t inl, const floa
   float* RN = res + (size_t)pl * r.per_pl + r.rn;
   float* XP = ws;
   float* RP = XP + TB * g.GH;
-  float* bsum = RP + (size_t)g.B * g.GH;
+  int kdummy;
+  float* bsum = RP + (size_t)step_slices(g.GH, g.B, g.H, &kdummy) * g.B * g.GH;
   hipLaunchKernelGGL(rnn_bias_kernel, dim3(nblocks(g.GH)), dim3(256), 0, s, w + o.bW, w + o.bR, bsum,
                      (int)g.GH, g.H, g.mode);
   // XP [GH x TB] = W [GH x in] (row-major = a column-major in x GH matrix, transposed) * IN [in x TB]
@@ -262,10 +309,12 @@ int forward_pl(const RnnGeom& g, int pl, const float* in, size_t inl, const floa
                        cx ? cx + (size_t)pl * g.BH : nullptr, CP, g.BH);
   for (int st = 0; st < g.T; ++st) {
     const int t = dir ? g.T - 1 - st : st;
-    if (const int rc = mm(w + o.R, HP + (size_t)st * g.BH, RP, g.GH, g.B, g.H, 1, 0, nullptr, s)) return rc;
+    int nrp = 1;
+    if (const int rc = mm_sliced(w + o.R, HP + (size_t)st * g.BH, RP, g.GH, g.B, g.H, 1, &nrp, s)) return rc;
     CellFwd a{};
     a.xp = XP + (size_t)t * g.B * g.GH;
     a.rp = RP;
+    a.nrp = nrp;
     a.bRn = w + o.bR + 2 * g.H;
     a.hp = HP + (size_t)st * g.BH;
     a.cp = CP + (size_t)st * g.BH;
@@ -299,13 +348,14 @@ int backward_pl(const RnnGeom& g, int pl, const float* in, size_t inl, const flo
   float* dGR = dGW + TB * g.GH;
   float* tmp = dGR + TB * g.GH + TB * g.D * g.H + TB * inmax;   // behind gout and gin
   float* dh_dir = tmp + TB * inmax;                               // two buffers, alternating
-  float* dh_rec = dh_dir + 2 * g.BH;
-  float* dc = dh_rec + g.BH;
+  float* dc = dh_dir + 2 * g.BH;
+  float* dh_rec = dc + g.BH;                                      // as many slices as step_slices says
   if (MODE == RNN_LSTM)
     hipLaunchKernelGGL(rnn_init_kernel, dim3(nblocks(g.BH)), dim3(256), 0, s,
                        dcy ? dcy + (size_t)pl * g.BH : nullptr, dc, g.BH);
   const float* dha = dhy ? dhy + (size_t)pl * g.BH : nullptr;   // direct part for the first step walked
   const float* dhb = nullptr;
+  int ndhb = 1;
   for (int st = g.T - 1; st >= 0; --st) {
     const int t = dir ? g.T - 1 - st : st;
     CellBwd a{};
@@ -313,6 +363,7 @@ int backward_pl(const RnnGeom& g, int pl, const float* in, size_t inl, const flo
     a.gout = gout ? gout + (size_t)t * g.B * a.ldo + (size_t)dir * g.H : nullptr;
     a.dh_a = dha;
     a.dh_b = dhb;
+    a.ndhb = ndhb;
     a.dc = dc;
     a.gt = GT + (size_t)st * g.B * g.GH;
     a.cp = CP + (size_t)st * g.BH;
@@ -324,18 +375,20 @@ int backward_pl(const RnnGeom& g, int pl, const float* in, size_t inl, const flo
     a.dh_dir = dh_dir + (size_t)(st & 1) * g.BH;
     hipLaunchKernelGGL((rnn_cell_bwd<MODE>), dim3(nblocks(g.BH)), dim3(256), 0, s, a, g.B, g.H);
     // gradient through the recurrent matrices: dh_rec [H x B] = R^T [H x GH] * dGR[st] [GH x B]
-    if (const int rc = mm(w + o.R, a.dgr, dh_rec, g.H, g.B, g.GH, 0, 0, nullptr, s)) return rc;
+    if (const int rc = mm_sliced(w + o.R, a.dgr, dh_rec, g.H, g.B, g.GH, 0, &ndhb, s)) return rc;
     dha = a.dh_dir;
     dhb = dh_rec;
   }
-  if (dhx) hipLaunchKernelGGL(rnn_add2_kernel, dim3(nblocks(g.BH)), dim3(256), 0, s, dha, dhb, dhx + (size_t)pl * g.BH, g.BH);
+  if (dhx)
+    hipLaunchKernelGGL(rnn_add2_kernel, dim3(nblocks(g.BH)), dim3(256), 0, s, dha, dhb, ndhb, dhx + (size_t)pl * g.BH,
+                       g.BH);
   if (dcx && MODE == RNN_LSTM)
     hipLaunchKernelGGL(rnn_init_kernel, dim3(nblocks(g.BH)), dim3(256), 0, s, dc, dcx + (size_t)pl * g.BH, g.BH);
   // gradient of the layer input: gin [in x TB] (+)= W^T [in x GH] * dGW [GH x TB]
   float* gdst = first_dir ? gin : tmp;
   if (const int rc = mm(w + o.W, dGW, gdst, inl, TB, g.GH, 0, 0, nullptr, s)) return rc;
   if (!first_dir)
-    hipLaunchKernelGGL(rnn_add2_kernel, dim3(nblocks(TB * inl)), dim3(256), 0, s, gin, tmp, gin, TB * inl);
+    hipLaunchKernelGGL(rnn_add2_kernel, dim3(nblocks(TB * inl)), dim3(256), 0, s, gin, tmp, 1, gin, TB * inl);
   // dW [GH][in] row-major = column-major in x GH = IN [in x TB] * dGW^T; dR likewise with the
   // states before each step; the bias gradients are the row sums
   if (const int rc = mm(in, dGW, dw + o.W, inl, g.GH, TB, 0, 1, nullptr, s)) return rc;
