@@ -67,18 +67,131 @@ matmul_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ 
 }
 
 // ---- out[r] = sum over columns of x[r, c]  (sumAs(gradOutput, bias), Functions.cpp:1287) ----
+// 16 rows (one 64-byte run per column) and 64 column groups per workgroup, so that a
+// few thousand rows by many columns still fill the machine; fixed summation order
+template <typename T>
+__global__ void __launch_bounds__(1024)
+sum_cols_kernel(const T* __restrict__ x, float* __restrict__ out, int R, int Cn) {
+  __shared__ float red[64][17];
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const int r = blockIdx.x * 16 + tx;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  if (r < R) {
+    int c = ty;
+    for (; c + 192 < Cn; c += 256) {
+      s0 += ld(x, (size_t)r + (size_t)c * R);
+      s1 += ld(x, (size_t)r + (size_t)(c + 64) * R);
+      s2 += ld(x, (size_t)r + (size_t)(c + 128) * R);
+      s3 += ld(x, (size_t)r + (size_t)(c + 192) * R);
+    }
+    for (; c < Cn; c += 64) s0 += ld(x, (size_t)r + (size_t)c * R);
+  }
+  red[ty][tx] = (s0 + s1) + (s2 + s3);
+  __syncthreads();
+  if (ty == 0 && r < R) {
+    float s = 0.f;
+#pragma unroll 8
+    for (int k = 0; k < 64; ++k) s += red[k][tx];
+    out[r] = s;
+  }
+}
+
+// ---- C [M x N] = A [M x K] * B^T with B [N x K], column-major: both operands are
+// contiguous along the dimension that survives, which is how the 16x16x4 matrix-core
+// instruction wants its operands (a lane per row / column, lane groups along the
+// contraction).  64 x 64 tile per workgroup, four waves of 2 x 2 instruction tiles,
+// contraction in chunks of 32 double-buffered through LDS as quads {k..k+3} per row so
+// that one 16-byte LDS read feeds four instructions.  blockIdx.y cuts the contraction
+// into slices, each writing its own partial product (f32) at C + slice * M * N.
 template <typename T>
 __global__ void __launch_bounds__(256)
-sum_cols_kernel(const T* __restrict__ x, float* __restrict__ out, int R, int Cn) {
-  __shared__ float red[4][64];
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-  const int r = blockIdx.x * 64 + tx;
-  float s = 0.f;
-  if (r < R)
-    for (int c = ty; c < Cn; c += 4) s += ld(x, (size_t)r + (size_t)c * R);
-  red[ty][tx] = s;
+gemm_nt_kernel(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int M, int N, int K,
+               int mtiles, int cps) {
+  __shared__ __align__(16) float As[2][8][64][4];
+  __shared__ __align__(16) float Bs[2][8][64][4];
+  const int tid = threadIdx.x, lm = tid & 63, lq = tid >> 6;
+  const int wave = tid >> 6, lane = tid & 63, fr = lane & 15, fg = lane >> 4;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = (blockIdx.x % mtiles) * 64, n0 = (blockIdx.x / mtiles) * 64;
+  const int nchunks = (K + 31) / 32;
+  const int cbeg = blockIdx.y * cps, cend = min(nchunks, cbeg + cps);
+  const bool am = m0 + lm < M, bn = n0 + lm < N;
+  const T* ap = A + m0 + lm;
+  const T* bp = B + n0 + lm;
+  float sa[2][4], sb[2][4];
+  auto gload = [&](int c) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int k = c * 32 + 4 * (lq + 4 * h) + j;
+        sa[h][j] = (am && k < K) ? ld(ap, (size_t)k * M) : 0.f;
+        sb[h][j] = (bn && k < K) ? ld(bp, (size_t)k * N) : 0.f;
+      }
+  };
+  auto sstore = [&](int buf) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      *reinterpret_cast<float4*>(As[buf][lq + 4 * h][lm]) = make_float4(sa[h][0], sa[h][1], sa[h][2], sa[h][3]);
+      *reinterpret_cast<float4*>(Bs[buf][lq + 4 * h][lm]) = make_float4(sb[h][0], sb[h][1], sb[h][2], sb[h][3]);
+    }
+  };
+  floatx4_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+  if (cbeg < cend) {
+    gload(cbeg);
+    sstore(0);
+  }
   __syncthreads();
-  if (ty == 0 && r < R) out[r] = (red[0][tx] + red[1][tx]) + (red[2][tx] + red[3][tx]);
+  for (int c = cbeg; c < cend; ++c) {
+    const int buf = (c - cbeg) & 1;
+    if (c + 1 < cend) gload(c + 1);
+#pragma unroll
+    for (int g16 = 0; g16 < 2; ++g16) {
+      const int q = g16 * 4 + fg;
+      float4 a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        a[i] = *reinterpret_cast<const float4*>(As[buf][q][(2 * wm + i) * 16 + fr]);
+        b[i] = *reinterpret_cast<const float4*>(Bs[buf][q][(2 * wn + i) * 16 + fr]);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].x, b[j].x, acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].y, b[j].y, acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].z, b[j].z, acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i].w, b[j].w, acc[i][j], 0, 0, 0);
+        }
+    }
+    if (c + 1 < cend) sstore(buf ^ 1);
+    __syncthreads();
+  }
+  T* cp = C + (size_t)blockIdx.y * M * N;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int m = m0 + (2 * wm + i) * 16 + 4 * fg, n = n0 + (2 * wn + j) * 16 + fr;
+      if (n >= N) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (m + r < M) st(cp, (size_t)(m + r) + (size_t)n * M, acc[i][j][r]);
+    }
+}
+
+template <typename T>
+int gemm_nt_launch(const T* A, const T* B, T* C, int M, int N, int K, int slices, hipStream_t s) {
+  const int mtiles = (M + 63) / 64, ntiles = (N + 63) / 64, nchunks = (K + 31) / 32;
+  if ((long long)mtiles * ntiles > 0x7fffffffll) return -1;
+  const int cps = (nchunks + slices - 1) / slices;
+  hipLaunchKernelGGL((gemm_nt_kernel<T>), dim3((unsigned)(mtiles * ntiles), (unsigned)slices), dim3(256), 0, s, A,
+                     B, C, M, N, K, mtiles, cps);
+  return check_launch("matmul (A * B^T)");
 }
 
 // ---- logSoftmax over dimension 0 of a C x X matrix (Functions.cpp:1044-1070) ----
@@ -261,6 +374,19 @@ AffinePlan affine_plan(long long outer, long long mid, long long inner, int scal
 }
 
 }  // namespace
+
+// C = A * B^T on the matrix cores (see gemm_nt_kernel); with slices > 1 (f32 only) C
+// receives that many partial products, M * N floats apart, in slice order.  The number
+// of slices actually written is ceil(chunks / ceil(chunks / slices)), chunks = ceil(K / 32).
+int gemm_nt(int dtype, const void* A, const void* B, void* C, int M, int N, int K, int slices, hipStream_t s) {
+  if (slices < 1 || (slices > 1 && dtype != FLHIP_F32)) return -1;
+  return dtype == FLHIP_F32
+             ? gemm_nt_launch(static_cast<const float*>(A), static_cast<const float*>(B), static_cast<float*>(C), M,
+                              N, K, slices, s)
+             : gemm_nt_launch(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(B),
+                              static_cast<bf16_t*>(C), M, N, K, slices, s);
+}
+
 }  // namespace flhip
 
 using namespace flhip;
@@ -296,6 +422,10 @@ extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, in
   FLHIP_REQUIRE(dtype_ok(dtype), "matmul: unknown dtype");
   // the matrix-core kernels of the 1x1 convolutions take the three products fl::linear
   // needs; the tiled vector-ALU kernel below covers the rest
+  if (!trans_a && trans_b && !getenv("FLHIP_MATMUL_VALU")) {
+    const int rc = gemm_nt(dtype, A, B, C, M, N, K, 1, as_stream(stream));
+    if (rc >= 0) return rc;
+  }
   if (!(trans_a && trans_b) && !getenv("FLHIP_MATMUL_VALU")) {
     const int rc = mfma_gemm(dtype, trans_a ? 1 : trans_b ? 2 : 0, A, B, C, M, N, K, bias_rows,
                              as_stream(stream));
@@ -318,12 +448,12 @@ extern "C" int flhip_sum_columns(const void* x, float* out, int32_t rows, int32_
   FLHIP_REQUIRE(x && out, "sum_columns: null argument");
   FLHIP_REQUIRE(rows > 0 && cols > 0, "sum_columns: sizes must be positive");
   FLHIP_REQUIRE(dtype_ok(dtype), "sum_columns: unknown dtype");
-  const dim3 grid((unsigned)((rows + 63) / 64));
+  const dim3 grid((unsigned)((rows + 15) / 16));
   if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((sum_cols_kernel<float>), grid, dim3(256), 0, as_stream(stream),
+    hipLaunchKernelGGL((sum_cols_kernel<float>), grid, dim3(1024), 0, as_stream(stream),
                        (const float*)x, out, rows, cols);
   else
-    hipLaunchKernelGGL((sum_cols_kernel<bf16_t>), grid, dim3(256), 0, as_stream(stream),
+    hipLaunchKernelGGL((sum_cols_kernel<bf16_t>), grid, dim3(1024), 0, as_stream(stream),
                        (const bf16_t*)x, out, rows, cols);
   return check_launch("sum_columns");
 }

@@ -43,6 +43,9 @@ int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, c
 int mfma_gemm(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,
               const float* bias_rows, hipStream_t s, int ksplit = 1);
 int mfma_gemm_slices(int K, int ksplit);
+// column-major C = A * B^T on a kernel of its own (both operands contiguous along the
+// surviving dimension); slices > 1 (f32): partial products M * N floats apart
+int gemm_nt(int dtype, const void* A, const void* B, void* C, int M, int N, int K, int slices, hipStream_t s);
 // windows with several taps on the same tile machinery, any stride / padding / dilation
 int mfma_tapped_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w,
                          const float* bias, void* y, hipStream_t s);

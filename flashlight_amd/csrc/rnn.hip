@@ -115,13 +115,73 @@ int step_slices(size_t M, size_t N, size_t K, int* ksplit) {
   return mfma_gemm_slices((int)K, (int)k);
 }
 
-size_t workspace_floats(const RnnGeom& g) {
+// The fused path (one launch per time step for both directions) keeps the projections
+// and gradients of both directions at once: forward {XP [D][T*B*GH], bias [D][GH]};
+// backward = the layout above, then for the second direction {dGW, dGR, dh_dir [2*BH], dc [BH]}.
+// slices of the contraction for the weight-gradient products (A * B^T over all time steps
+// and batch columns): enough 64 x 64 tiles times slices to fill the machine several
+// times over, at least eight chunks of 32 per slice
+int wgrad_slices(size_t M, size_t N, size_t K) {
+  const long long tiles = (long long)((M + 63) / 64) * ((N + 63) / 64), chunks = (long long)(K + 31) / 32;
+  long long ns = 1024 / tiles;
+  if (ns > chunks / 8) ns = chunks / 8;
+  if (ns > 16) ns = 16;
+  if (ns < 1) ns = 1;
+  const long long cps = (chunks + ns - 1) / ns;
+  return (int)((chunks + cps - 1) / cps);
+}
+
+int mm(const float* A, const float* B, float* C, size_t M, size_t N, size_t K, int ta, int tb,
+       const float* bias, hipStream_t s) {
+  return flhip_matmul(A, B, C, (int32_t)M, (int32_t)N, (int32_t)K, ta, tb, bias, FLHIP_F32, s);
+}
+
+// C = op(A) B in `*slices` partial products at C + k*M*N (see step_slices)
+int mm_sliced(const float* A, const float* B, float* C, size_t M, size_t N, size_t K, int ta, int* slices,
+              hipStream_t s) {
+  int ksplit;
+  const int ns = step_slices(M, N, K, &ksplit);
+  if (ns > 1 && mfma_gemm(FLHIP_F32, ta ? 1 : 0, A, B, C, (int)M, (int)N, (int)K, nullptr, s, ksplit) >= 0) {
+    *slices = ns;
+    return check_launch("rnn (recurrent product)");
+  }
+  *slices = 1;
+  return mm(A, B, C, M, N, K, ta, 0, nullptr, s);
+}
+
+
+// ... and at the end the partial products of the sliced weight-gradient products
+size_t wgrad_scratch(const RnnGeom& g) {
+  const size_t TB = (size_t)g.T * g.B, inmax = std::max<size_t>(g.I, (size_t)g.D * g.H);
+  size_t n = 0;
+  for (size_t M : {(size_t)g.I, inmax, (size_t)g.H}) {
+    const int ns = wgrad_slices(M, g.GH, TB);
+    if (ns > 1) n = std::max(n, (size_t)ns * M * g.GH);
+  }
+  return n;
+}
+
+size_t wgrad_scratch_offset(const RnnGeom& g) {
   const size_t TB = (size_t)g.T * g.B, inmax = std::max<size_t>(g.I, (size_t)g.D * g.H);
   int k;
-  const size_t sf = step_slices(g.GH, g.B, g.H, &k), sb = step_slices(g.H, g.B, g.GH, &k);
-  const size_t fwd = TB * g.GH + sf * g.B * g.GH + g.GH;
-  const size_t bwd = 2 * TB * g.GH + TB * g.D * g.H + 2 * TB * inmax + (3 + sb) * g.BH;
+  const size_t sb = step_slices(g.H, g.B, g.GH, &k);
+  return 2 * TB * g.GH + TB * g.D * g.H + 2 * TB * inmax + (3 + sb) * g.BH +
+         (size_t)(g.D - 1) * (2 * TB * g.GH + 3 * g.BH);
+}
+
+size_t workspace_floats(const RnnGeom& g) {
+  const size_t TB = (size_t)g.T * g.B;
+  int k;
+  const size_t sf = step_slices(g.GH, g.B, g.H, &k);
+  const size_t fwd = std::max(TB * g.GH + sf * g.B * g.GH + g.GH, (size_t)g.D * (TB * g.GH + g.GH));
+  const size_t bwd = wgrad_scratch_offset(g) + wgrad_scratch(g);
   return std::max(fwd, bwd) + 64;
+}
+
+// the fused step kernels tile the hidden state by 16 and hold at most 64 batch columns
+bool fused_applies(const RnnGeom& g) {
+  static const bool off = getenv("FLHIP_RNN_UNFUSED") != nullptr;
+  return !off && g.H % 16 == 0 && g.B <= 64;
 }
 
 __device__ __forceinline__ float sigm(float v) { return 1.f / (1.f + expf(-v)); }
@@ -153,8 +213,9 @@ __global__ void __launch_bounds__(256) rnn_add2_kernel(const float* a, const flo
 
 struct CellFwd {
   const float* xp;    // [B][GH] input projection (+ biases) of this time step
-  const float* rp;    // [nrp][B][GH] recurrent projection, in nrp partial products
+  const float* rp;    // [nrp][B][GH] recurrent projection, in nrp partial products (two-kernel path)
   int nrp;
+  const float* R;     // [GH][H] recurrent matrices (fused path)
   const float* bRn;   // GRU: recurrent bias of the n gate [H]
   const float* hp;    // [B][H] state before the step
   const float* cp;    // LSTM
@@ -168,28 +229,18 @@ struct CellFwd {
   int ldo;
 };
 
+// gate math of one (batch b, hidden h) element; rp = its recurrent projections, one per gate
 template <int MODE>
-__global__ void __launch_bounds__(256) rnn_cell_fwd(CellFwd a, int B, int H) {
-  const int e = blockIdx.x * 256 + threadIdx.x;
-  if (e >= B * H) return;
-  const int b = e / H, h = e - b * H;
+__device__ __forceinline__ void cell_fwd_apply(const CellFwd& a, int b, int h, int H, const float* rp) {
   constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1;
-  const size_t q = (size_t)b * G * H + h;
-  float rp[G];
-#pragma unroll
-  for (int gq = 0; gq < G; ++gq) rp[gq] = 0.f;
-  for (int k = 0; k < a.nrp; ++k) {
-    const float* r = a.rp + (size_t)k * B * G * H + q;
-#pragma unroll
-    for (int gq = 0; gq < G; ++gq) rp[gq] += r[gq * H];
-  }
+  const size_t e = (size_t)b * H + h, q = (size_t)b * G * H + h;
   float hv;
   if (MODE == RNN_RELU || MODE == RNN_TANH) {
     const float pre = a.xp[q] + rp[0];
     hv = MODE == RNN_RELU ? (pre > 0.f ? pre : 0.f) : tanhf(pre);
     a.gt[q] = hv;
   } else if (MODE == RNN_LSTM) {
-    const float ig = sigm(a.xp[q] + rp[0]), fg = sigm(a.xp[q + H] + rp[1]);
+    const float ig = sigm(a.xp[q] + rp[0]), fg = sigm(a.xp[q + H] + rp[G > 1 ? 1 : 0]);
     const float gg = tanhf(a.xp[q + 2 * H] + rp[G > 2 ? 2 : 0]), og = sigm(a.xp[q + 3 * H] + rp[G > 3 ? 3 : 0]);
     const float c = fg * a.cp[e] + ig * gg;
     a.cn[e] = c;
@@ -209,11 +260,114 @@ __global__ void __launch_bounds__(256) rnn_cell_fwd(CellFwd a, int B, int H) {
   if (a.hy) a.hy[e] = hv;
 }
 
+template <int MODE>
+__global__ void __launch_bounds__(256) rnn_cell_fwd(CellFwd a, int B, int H) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= B * H) return;
+  const int b = e / H, h = e - b * H;
+  constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1;
+  const size_t q = (size_t)b * G * H + h;
+  float rp[G];
+#pragma unroll
+  for (int gq = 0; gq < G; ++gq) rp[gq] = 0.f;
+  for (int k = 0; k < a.nrp; ++k) {
+    const float* r = a.rp + (size_t)k * B * G * H + q;
+#pragma unroll
+    for (int gq = 0; gq < G; ++gq) rp[gq] += r[gq * H];
+  }
+  cell_fwd_apply<MODE>(a, b, h, H, rp);
+}
+
+// One time step of up to two directions in one launch: recurrent product and gate math.
+// A workgroup owns four hidden units (blockIdx.x) of one direction (blockIdx.y): its
+// 16-row matrix-core tile is {gate g, unit hh} = row 4*g + hh of the recurrent
+// matrices, its columns are the batch (NBT tiles of 16, batch <= 64), and the four
+// waves split the contraction over the hidden state in interleaved chunks of 16.  A
+// lane's 16-byte load supplies the operands of four 16x16x4 products (the k index of a
+// lane group is permuted the same way on both operands).  The partial tiles meet in
+// LDS, then one thread per (batch, unit) applies the gates.  Needs H % 16 == 0.
+struct StepFwd {
+  CellFwd d[2];
+  int B, H;
+};
+
+template <int MODE, int NBT>
+__global__ void __launch_bounds__(256) rnn_step_fwd(StepFwd p) {
+  constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1, NB = NBT * 16;
+  __shared__ float red[4][16][NB + 1];
+  const CellFwd& a = p.d[blockIdx.y];
+  const int H = p.H, B = p.B, h0 = blockIdx.x * 4;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, fr = lane & 15, fg = lane >> 4;
+  const int gate = fr >> 2;
+  const bool av = gate < G;
+  const float* ap = a.R + ((size_t)(av ? gate : 0) * H + h0 + (fr & 3)) * H + 4 * fg;
+  const float* bp[NBT];
+  bool bv[NBT];
+#pragma unroll
+  for (int nt = 0; nt < NBT; ++nt) {
+    const int b = nt * 16 + fr;
+    bv[nt] = b < B;
+    bp[nt] = a.hp + (size_t)(bv[nt] ? b : 0) * H + 4 * fg;
+  }
+  floatx4_t acc[NBT];
+#pragma unroll
+  for (int nt = 0; nt < NBT; ++nt) acc[nt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+  // U chunks are in flight per wave at a time: the loop is bound by the latency of
+  // its loads, not by the products
+  constexpr int U = NBT == 4 ? 4 : 8;
+  const int chunks = H >> 4;
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int c0 = wave; c0 < chunks; c0 += 4 * U) {
+    float4 ra[U], rb[U][NBT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      // every load is issued (from a clamped, valid address) before any is used
+      const int c = min(c0 + 4 * u, chunks - 1);
+      ra[u] = *reinterpret_cast<const float4*>(ap + c * 16);
+#pragma unroll
+      for (int nt = 0; nt < NBT; ++nt) rb[u][nt] = *reinterpret_cast<const float4*>(bp[nt] + c * 16);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const bool in = c0 + 4 * u < chunks;
+      if (!(in && av)) ra[u] = zero4;
+#pragma unroll
+      for (int nt = 0; nt < NBT; ++nt)
+        if (!(in && bv[nt])) rb[u][nt] = zero4;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float av4[4] = {ra[u].x, ra[u].y, ra[u].z, ra[u].w};
+#pragma unroll
+      for (int nt = 0; nt < NBT; ++nt) {
+        const float bv4[4] = {rb[u][nt].x, rb[u][nt].y, rb[u][nt].z, rb[u][nt].w};
+#pragma unroll
+        for (int m = 0; m < 4; ++m) acc[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(av4[m], bv4[m], acc[nt], 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int nt = 0; nt < NBT; ++nt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][4 * fg + r][nt * 16 + fr] = acc[nt][r];
+  __syncthreads();
+  if (tid < 4 * B) {
+    const int b = tid >> 2, hh = tid & 3;
+    float rp[G];
+#pragma unroll
+    for (int gq = 0; gq < G; ++gq)
+      rp[gq] = (red[0][gq * 4 + hh][b] + red[1][gq * 4 + hh][b]) + (red[2][gq * 4 + hh][b] + red[3][gq * 4 + hh][b]);
+    cell_fwd_apply<MODE>(a, b, h0 + hh, H, rp);
+  }
+}
+
 struct CellBwd {
   const float* gout;  // gradient of the layer output at this time step, this direction's slice; pitch ldo (may be null)
   const float* dh_a;  // gradient reaching h through the recurrence: direct part ...
   const float* dh_b;  // ... and the part through the recurrent matrices, in ndhb partial products
   int ndhb;           //     (either pointer may be null)
+  const float* R;         // fused path: recurrent matrices [GH][H] and the recurrent-side
+  const float* dgr_next;  // pre-activation gradients [B][GH] of the step walked before (or null)
   float* dc;          // LSTM: in = gradient of c after the step, out = of c before it
   const float* gt;    // gate activations of the step
   const float* cp;    // LSTM: c before the step
@@ -226,17 +380,15 @@ struct CellBwd {
   int ldo;
 };
 
+// gradient math of one (batch b, hidden h) element; rec = gradient arriving through the
+// recurrent matrices
 template <int MODE>
-__global__ void __launch_bounds__(256) rnn_cell_bwd(CellBwd a, int B, int H) {
-  const int e = blockIdx.x * 256 + threadIdx.x;
-  if (e >= B * H) return;
-  const int b = e / H, h = e - b * H;
+__device__ __forceinline__ void cell_bwd_apply(const CellBwd& a, int b, int h, int H, float rec) {
   constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1;
-  const size_t q = (size_t)b * G * H + h;
+  const size_t e = (size_t)b * H + h, q = (size_t)b * G * H + h;
   float go = a.gout ? a.gout[(size_t)b * a.ldo + h] : 0.f;
   if (a.dh_a) go += a.dh_a[e];
-  if (a.dh_b)
-    for (int k = 0; k < a.ndhb; ++k) go += a.dh_b[(size_t)k * B * H + e];
+  go += rec;
   float direct = 0.f;
   if (MODE == RNN_RELU || MODE == RNN_TANH) {
     const float hv = a.gt[q];
@@ -263,24 +415,110 @@ __global__ void __launch_bounds__(256) rnn_cell_bwd(CellBwd a, int B, int H) {
   a.dh_dir[e] = direct;
 }
 
-inline unsigned nblocks(size_t n) { return (unsigned)((n + 255) / 256); }
-
-int mm(const float* A, const float* B, float* C, size_t M, size_t N, size_t K, int ta, int tb,
-       const float* bias, hipStream_t s) {
-  return flhip_matmul(A, B, C, (int32_t)M, (int32_t)N, (int32_t)K, ta, tb, bias, FLHIP_F32, s);
+template <int MODE>
+__global__ void __launch_bounds__(256) rnn_cell_bwd(CellBwd a, int B, int H) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= B * H) return;
+  const int b = e / H, h = e - b * H;
+  float rec = 0.f;
+  if (a.dh_b)
+    for (int k = 0; k < a.ndhb; ++k) rec += a.dh_b[(size_t)k * B * H + e];
+  cell_bwd_apply<MODE>(a, b, h, H, rec);
 }
 
-// C = op(A) B in `*slices` partial products at C + k*M*N (see step_slices)
-int mm_sliced(const float* A, const float* B, float* C, size_t M, size_t N, size_t K, int ta, int* slices,
-              hipStream_t s) {
-  int ksplit;
-  const int ns = step_slices(M, N, K, &ksplit);
-  if (ns > 1 && mfma_gemm(FLHIP_F32, ta ? 1 : 0, A, B, C, (int)M, (int)N, (int)K, nullptr, s, ksplit) >= 0) {
-    *slices = ns;
-    return check_launch("rnn (recurrent product)");
+// One backward time step of up to two directions in one launch.  A workgroup owns 16
+// hidden units of one direction: rows of its matrix-core tile are the units (columns
+// of the recurrent matrices, 64 contiguous bytes per contraction index), columns the
+// batch, and its eight waves split the contraction over the gate rows (G*H) in
+// interleaved chunks of 16; the partial tiles meet in LDS and the threads then apply
+// the gate gradients of the step, which become the next launch's operand.  H % 16 == 0.
+struct StepBwd {
+  CellBwd d[2];
+  int B, H;
+};
+
+template <int MODE, int NBT>
+__global__ void __launch_bounds__(512) rnn_step_bwd(StepBwd p) {
+  constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1, NB = NBT * 16;
+  __shared__ float red[8][16][NB + 1];
+  const CellBwd& a = p.d[blockIdx.y];
+  const int H = p.H, B = p.B, h0 = blockIdx.x * 16, GH = G * H;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, fr = lane & 15, fg = lane >> 4;
+  const bool have = a.dgr_next != nullptr;
+  if (have) {
+    const float* ap = a.R + (size_t)(4 * fg) * H + h0 + fr;
+    const float* bp[NBT];
+    bool bv[NBT];
+#pragma unroll
+    for (int nt = 0; nt < NBT; ++nt) {
+      const int b = nt * 16 + fr;
+      bv[nt] = b < B;
+      bp[nt] = a.dgr_next + (size_t)(bv[nt] ? b : 0) * GH + 4 * fg;
+    }
+    floatx4_t acc[NBT];
+#pragma unroll
+    for (int nt = 0; nt < NBT; ++nt) acc[nt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+    constexpr int U = NBT == 4 ? 4 : 8;   // chunks in flight per wave
+    const int chunks = GH >> 4;
+    const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int c0 = wave; c0 < chunks; c0 += 8 * U) {
+      float ra[U][4];
+      float4 rb[U][NBT];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int c = min(c0 + 8 * u, chunks - 1);
+#pragma unroll
+        for (int m = 0; m < 4; ++m) ra[u][m] = ap[((size_t)c * 16 + m) * H];
+#pragma unroll
+        for (int nt = 0; nt < NBT; ++nt) rb[u][nt] = *reinterpret_cast<const float4*>(bp[nt] + c * 16);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const bool in = c0 + 8 * u < chunks;
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+          if (!in) ra[u][m] = 0.f;
+#pragma unroll
+        for (int nt = 0; nt < NBT; ++nt)
+          if (!(in && bv[nt])) rb[u][nt] = zero4;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int nt = 0; nt < NBT; ++nt) {
+          const float bv4[4] = {rb[u][nt].x, rb[u][nt].y, rb[u][nt].z, rb[u][nt].w};
+#pragma unroll
+          for (int m = 0; m < 4; ++m)
+            acc[nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[u][m], bv4[m], acc[nt], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int nt = 0; nt < NBT; ++nt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave][4 * fg + r][nt * 16 + fr] = acc[nt][r];
   }
-  *slices = 1;
-  return mm(A, B, C, M, N, K, ta, 0, nullptr, s);
+  __syncthreads();
+  for (int e = tid; e < 16 * B; e += 512) {
+    const int b = e >> 4, hh = e & 15;
+    float rec = 0.f;
+    if (have) {
+#pragma unroll
+      for (int wv = 0; wv < 8; ++wv) rec += red[wv][hh][b];
+    }
+    cell_bwd_apply<MODE>(a, b, h0 + hh, H, rec);
+  }
+}
+
+inline unsigned nblocks(size_t n) { return (unsigned)((n + 255) / 256); }
+
+// dst [M x N] = A [M x K] * B^T, through `scratch` when the contraction is cut into slices
+int mm_nt(const float* A, const float* B, float* dst, size_t M, size_t N, size_t K, float* scratch, hipStream_t s) {
+  const int ns = wgrad_slices(M, N, K);
+  if (ns <= 1) return gemm_nt(FLHIP_F32, A, B, dst, (int)M, (int)N, (int)K, 1, s);
+  if (const int rc = gemm_nt(FLHIP_F32, A, B, scratch, (int)M, (int)N, (int)K, ns, s)) return rc;
+  hipLaunchKernelGGL(rnn_add2_kernel, dim3(nblocks(M * N)), dim3(256), 0, s, (const float*)nullptr, scratch, ns, dst,
+                     M * N);
+  return FLHIP_OK;
 }
 
 template <int MODE>
@@ -328,6 +566,63 @@ int forward_pl(const RnnGeom& g, int pl, const float* in, size_t inl, const floa
     a.hy = last ? hy + (size_t)pl * g.BH : nullptr;
     a.cy = (last && cy && MODE == RNN_LSTM) ? cy + (size_t)pl * g.BH : nullptr;
     hipLaunchKernelGGL((rnn_cell_fwd<MODE>), dim3(nblocks(g.BH)), dim3(256), 0, s, a, g.B, g.H);
+  }
+  return check_launch("rnn_fwd");
+}
+
+template <int MODE, int NBT>
+void launch_step_fwd(const StepFwd& p, int D, hipStream_t s) {
+  hipLaunchKernelGGL((rnn_step_fwd<MODE, NBT>), dim3(p.H / 4, D), dim3(256), 0, s, p);
+}
+
+// one layer, all directions: per direction the input projection of all steps, then one
+// launch per time step for both directions
+template <int MODE>
+int forward_layer_fused(const RnnGeom& g, int l, const float* in, size_t inl, const float* w, const float* hx,
+                        const float* cx, float* out, float* hy, float* cy, float* res, float* ws, hipStream_t s) {
+  const Reserve r = reserve_layout(g);
+  const size_t TB = (size_t)g.T * g.B;
+  for (int dir = 0; dir < g.D; ++dir) {
+    const int pl = l * g.D + dir;
+    const Offsets o = offsets(g, pl);
+    float* XP = ws + (size_t)dir * TB * g.GH;
+    float* bsum = ws + (size_t)g.D * TB * g.GH + (size_t)dir * g.GH;
+    hipLaunchKernelGGL(rnn_bias_kernel, dim3(nblocks(g.GH)), dim3(256), 0, s, w + o.bW, w + o.bR, bsum,
+                       (int)g.GH, g.H, g.mode);
+    if (const int rc = mm(w + o.W, in, XP, g.GH, TB, inl, 1, 0, bsum, s)) return rc;
+    hipLaunchKernelGGL(rnn_init_kernel, dim3(nblocks(g.BH)), dim3(256), 0, s,
+                       hx ? hx + (size_t)pl * g.BH : nullptr, res + (size_t)pl * r.per_pl + r.hp, g.BH);
+    if (MODE == RNN_LSTM)
+      hipLaunchKernelGGL(rnn_init_kernel, dim3(nblocks(g.BH)), dim3(256), 0, s,
+                         cx ? cx + (size_t)pl * g.BH : nullptr, res + (size_t)pl * r.per_pl + r.cp, g.BH);
+  }
+  for (int st = 0; st < g.T; ++st) {
+    StepFwd p{};
+    p.B = g.B;
+    p.H = g.H;
+    for (int dir = 0; dir < g.D; ++dir) {
+      const int pl = l * g.D + dir, t = dir ? g.T - 1 - st : st;
+      const Offsets o = offsets(g, pl);
+      float* base = res + (size_t)pl * r.per_pl;
+      CellFwd& a = p.d[dir];
+      a.xp = ws + (size_t)dir * TB * g.GH + (size_t)t * g.B * g.GH;
+      a.R = w + o.R;
+      a.bRn = w + o.bR + 2 * g.H;
+      a.hp = base + r.hp + (size_t)st * g.BH;
+      a.cp = base + r.cp + (size_t)st * g.BH;
+      a.hn = base + r.hp + (size_t)(st + 1) * g.BH;
+      a.cn = base + r.cp + (size_t)(st + 1) * g.BH;
+      a.gt = base + r.gt + (size_t)st * g.B * g.GH;
+      a.rn = base + r.rn + (size_t)st * g.BH;
+      a.ldo = g.D * g.H;
+      a.out = out + (size_t)t * g.B * a.ldo + (size_t)dir * g.H;
+      const bool last = st == g.T - 1;
+      a.hy = last ? hy + (size_t)pl * g.BH : nullptr;
+      a.cy = (last && cy && MODE == RNN_LSTM) ? cy + (size_t)pl * g.BH : nullptr;
+    }
+    if (g.B <= 16) launch_step_fwd<MODE, 1>(p, g.D, s);
+    else if (g.B <= 32) launch_step_fwd<MODE, 2>(p, g.D, s);
+    else launch_step_fwd<MODE, 4>(p, g.D, s);
   }
   return check_launch("rnn_fwd");
 }
@@ -391,10 +686,89 @@ int backward_pl(const RnnGeom& g, int pl, const float* in, size_t inl, const flo
     hipLaunchKernelGGL(rnn_add2_kernel, dim3(nblocks(TB * inl)), dim3(256), 0, s, gin, tmp, 1, gin, TB * inl);
   // dW [GH][in] row-major = column-major in x GH = IN [in x TB] * dGW^T; dR likewise with the
   // states before each step; the bias gradients are the row sums
-  if (const int rc = mm(in, dGW, dw + o.W, inl, g.GH, TB, 0, 1, nullptr, s)) return rc;
-  if (const int rc = mm(HP, dGR, dw + o.R, g.H, g.GH, TB, 0, 1, nullptr, s)) return rc;
+  float* scratch = ws + wgrad_scratch_offset(g);
+  if (const int rc = mm_nt(in, dGW, dw + o.W, inl, g.GH, TB, scratch, s)) return rc;
+  if (const int rc = mm_nt(HP, dGR, dw + o.R, g.H, g.GH, TB, scratch, s)) return rc;
   if (const int rc = flhip_sum_columns(dGW, dw + o.bW, (int32_t)g.GH, (int32_t)TB, FLHIP_F32, s)) return rc;
   if (const int rc = flhip_sum_columns(dGR, dw + o.bR, (int32_t)g.GH, (int32_t)TB, FLHIP_F32, s)) return rc;
+  return check_launch("rnn_bwd");
+}
+
+template <int MODE, int NBT>
+void launch_step_bwd(const StepBwd& p, int D, hipStream_t s) {
+  hipLaunchKernelGGL((rnn_step_bwd<MODE, NBT>), dim3(p.H / 16, D), dim3(512), 0, s, p);
+}
+
+template <int MODE>
+int backward_layer_fused(const RnnGeom& g, int l, const float* in, size_t inl, const float* w, const float* gout,
+                         const float* dhy, const float* dcy, float* gin, float* dhx, float* dcx, float* dw,
+                         const float* res, float* ws, hipStream_t s) {
+  const Reserve r = reserve_layout(g);
+  const size_t TB = (size_t)g.T * g.B, inmax = std::max<size_t>(g.I, (size_t)g.D * g.H);
+  int kdummy;
+  const size_t sb = step_slices(g.H, g.B, g.GH, &kdummy);
+  float* tmp = ws + 2 * TB * g.GH + TB * g.D * g.H + TB * inmax;
+  float* dh_rec = tmp + TB * inmax + 3 * g.BH;
+  float* second = dh_rec + sb * g.BH;
+  float *dGW[2], *dGR[2], *dh_dir[2], *dc[2];
+  dGW[0] = ws; dGR[0] = ws + TB * g.GH; dh_dir[0] = tmp + TB * inmax; dc[0] = dh_dir[0] + 2 * g.BH;
+  dGW[1] = second; dGR[1] = second + TB * g.GH; dh_dir[1] = second + 2 * TB * g.GH; dc[1] = dh_dir[1] + 2 * g.BH;
+  if (MODE == RNN_LSTM)
+    for (int dir = 0; dir < g.D; ++dir)
+      hipLaunchKernelGGL(rnn_init_kernel, dim3(nblocks(g.BH)), dim3(256), 0, s,
+                         dcy ? dcy + (size_t)(l * g.D + dir) * g.BH : nullptr, dc[dir], g.BH);
+  for (int st = g.T - 1; st >= 0; --st) {
+    StepBwd p{};
+    p.B = g.B;
+    p.H = g.H;
+    for (int dir = 0; dir < g.D; ++dir) {
+      const int pl = l * g.D + dir, t = dir ? g.T - 1 - st : st;
+      const Offsets o = offsets(g, pl);
+      const float* base = res + (size_t)pl * r.per_pl;
+      CellBwd& a = p.d[dir];
+      a.ldo = g.D * g.H;
+      a.gout = gout ? gout + (size_t)t * g.B * a.ldo + (size_t)dir * g.H : nullptr;
+      const bool first = st == g.T - 1;
+      a.dh_a = first ? (dhy ? dhy + (size_t)pl * g.BH : nullptr) : dh_dir[dir] + (size_t)((st + 1) & 1) * g.BH;
+      a.R = w + o.R;
+      a.dgr_next = first ? nullptr : dGR[dir] + (size_t)(st + 1) * g.B * g.GH;
+      a.dc = dc[dir];
+      a.gt = base + r.gt + (size_t)st * g.B * g.GH;
+      a.cp = base + r.cp + (size_t)st * g.BH;
+      a.cn = base + r.cp + (size_t)(st + 1) * g.BH;
+      a.hp = base + r.hp + (size_t)st * g.BH;
+      a.rn = base + r.rn + (size_t)st * g.BH;
+      a.dgw = dGW[dir] + (size_t)t * g.B * g.GH;
+      a.dgr = dGR[dir] + (size_t)st * g.B * g.GH;
+      a.dh_dir = dh_dir[dir] + (size_t)(st & 1) * g.BH;
+    }
+    if (g.B <= 16) launch_step_bwd<MODE, 1>(p, g.D, s);
+    else if (g.B <= 32) launch_step_bwd<MODE, 2>(p, g.D, s);
+    else launch_step_bwd<MODE, 4>(p, g.D, s);
+  }
+  for (int dir = 0; dir < g.D; ++dir) {
+    const int pl = l * g.D + dir;
+    const Offsets o = offsets(g, pl);
+    const float* HP = res + (size_t)pl * r.per_pl + r.hp;
+    if (dhx) {
+      int ndhb = 1;
+      if (const int rc = mm_sliced(w + o.R, dGR[dir], dh_rec, g.H, g.B, g.GH, 0, &ndhb, s)) return rc;
+      hipLaunchKernelGGL(rnn_add2_kernel, dim3(nblocks(g.BH)), dim3(256), 0, s, dh_dir[dir], dh_rec, ndhb,
+                         dhx + (size_t)pl * g.BH, g.BH);
+    }
+    if (dcx && MODE == RNN_LSTM)
+      hipLaunchKernelGGL(rnn_init_kernel, dim3(nblocks(g.BH)), dim3(256), 0, s, dc[dir], dcx + (size_t)pl * g.BH,
+                         g.BH);
+    float* gdst = dir == 0 ? gin : tmp;
+    if (const int rc = mm(w + o.W, dGW[dir], gdst, inl, TB, g.GH, 0, 0, nullptr, s)) return rc;
+    if (dir)
+      hipLaunchKernelGGL(rnn_add2_kernel, dim3(nblocks(TB * inl)), dim3(256), 0, s, gin, tmp, 1, gin, TB * inl);
+    float* scratch = ws + wgrad_scratch_offset(g);
+    if (const int rc = mm_nt(in, dGW[dir], dw + o.W, inl, g.GH, TB, scratch, s)) return rc;
+    if (const int rc = mm_nt(HP, dGR[dir], dw + o.R, g.H, g.GH, TB, scratch, s)) return rc;
+    if (const int rc = flhip_sum_columns(dGW[dir], dw + o.bW, (int32_t)g.GH, (int32_t)TB, FLHIP_F32, s)) return rc;
+    if (const int rc = flhip_sum_columns(dGR[dir], dw + o.bR, (int32_t)g.GH, (int32_t)TB, FLHIP_F32, s)) return rc;
+  }
   return check_launch("rnn_bwd");
 }
 
@@ -434,6 +808,21 @@ extern "C" int flhip_rnn_fwd(const flhip_rnn_desc* d, const void* x, const void*
     const float* in = l == 0 ? static_cast<const float*>(x) : res + r.acts + (size_t)(l - 1) * act;
     float* out = l == g.L - 1 ? static_cast<float*>(y) : res + r.acts + (size_t)l * act;
     const size_t inl = l == 0 ? g.I : (size_t)g.D * g.H;
+    if (fused_applies(g)) {
+      int rc;
+      auto args = [&](auto fn) {
+        return fn(g, l, in, inl, wf, static_cast<const float*>(hx), static_cast<const float*>(cx), out,
+                  static_cast<float*>(hy), static_cast<float*>(cy), res, static_cast<float*>(ws), s);
+      };
+      switch (g.mode) {
+        case RNN_RELU: rc = args(forward_layer_fused<RNN_RELU>); break;
+        case RNN_TANH: rc = args(forward_layer_fused<RNN_TANH>); break;
+        case RNN_LSTM: rc = args(forward_layer_fused<RNN_LSTM>); break;
+        default: rc = args(forward_layer_fused<RNN_GRU>);
+      }
+      if (rc != FLHIP_OK) return rc;
+      continue;
+    }
     for (int dir = 0; dir < g.D; ++dir) {
       const int pl = l * g.D + dir;
       int rc;
@@ -477,21 +866,36 @@ extern "C" int flhip_rnn_bwd(const flhip_rnn_desc* d, const void* x, const void*
     const float* in = l == 0 ? static_cast<const float*>(x) : res + r.acts + (size_t)(l - 1) * act;
     const size_t inl = l == 0 ? g.I : (size_t)g.D * g.H;
     float* gin = l == 0 ? static_cast<float*>(dx) : ginbuf;
-    for (int dir = 0; dir < g.D; ++dir) {
-      const int pl = l * g.D + dir;
+    if (fused_applies(g)) {
       int rc;
       auto args = [&](auto fn) {
-        return fn(g, pl, in, inl, wf, gout, static_cast<const float*>(dhy), static_cast<const float*>(dcy), gin,
-                  dir == 0, static_cast<float*>(dhx), static_cast<float*>(dcx), static_cast<float*>(dw), res,
-                  wsf, s);
+        return fn(g, l, in, inl, wf, gout, static_cast<const float*>(dhy), static_cast<const float*>(dcy), gin,
+                  static_cast<float*>(dhx), static_cast<float*>(dcx), static_cast<float*>(dw), res, wsf, s);
       };
       switch (g.mode) {
-        case RNN_RELU: rc = args(backward_pl<RNN_RELU>); break;
-        case RNN_TANH: rc = args(backward_pl<RNN_TANH>); break;
-        case RNN_LSTM: rc = args(backward_pl<RNN_LSTM>); break;
-        default: rc = args(backward_pl<RNN_GRU>);
+        case RNN_RELU: rc = args(backward_layer_fused<RNN_RELU>); break;
+        case RNN_TANH: rc = args(backward_layer_fused<RNN_TANH>); break;
+        case RNN_LSTM: rc = args(backward_layer_fused<RNN_LSTM>); break;
+        default: rc = args(backward_layer_fused<RNN_GRU>);
       }
       if (rc != FLHIP_OK) return rc;
+    } else {
+      for (int dir = 0; dir < g.D; ++dir) {
+        const int pl = l * g.D + dir;
+        int rc;
+        auto args = [&](auto fn) {
+          return fn(g, pl, in, inl, wf, gout, static_cast<const float*>(dhy), static_cast<const float*>(dcy),
+                    gin, dir == 0, static_cast<float*>(dhx), static_cast<float*>(dcx), static_cast<float*>(dw),
+                    res, wsf, s);
+        };
+        switch (g.mode) {
+          case RNN_RELU: rc = args(backward_pl<RNN_RELU>); break;
+          case RNN_TANH: rc = args(backward_pl<RNN_TANH>); break;
+          case RNN_LSTM: rc = args(backward_pl<RNN_LSTM>); break;
+          default: rc = args(backward_pl<RNN_GRU>);
+        }
+        if (rc != FLHIP_OK) return rc;
+      }
     }
     if (l > 0) {
       // the gradient of this layer's input is the gradient of the output of the layer below

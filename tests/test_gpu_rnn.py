@@ -22,6 +22,14 @@ MODES = [flref.RNN_RELU, flref.RNN_TANH, flref.RNN_LSTM, flref.RNN_GRU]
     (6, 4, 2, False, 1, 4, False),         # one step
     (40, 64, 2, True, 20, 8, True),        # sizes that reach the matrix-core products
     (80, 96, 1, False, 33, 5, False),
+    # hidden sizes that are multiples of 16 with at most 64 batch columns take the fused
+    # step kernels: one, two and four batch tiles, fewer contraction chunks than waves,
+    # a single batch column; 65 columns and the sizes above take the two-kernel steps
+    (24, 16, 1, True, 4, 17, True),
+    (10, 48, 2, True, 5, 33, True),
+    (12, 128, 1, False, 7, 64, False),
+    (9, 160, 2, True, 6, 1, True),
+    (12, 32, 1, True, 4, 65, True),
 ])
 def test_rnn_forward_backward(mode, I, H, L, bidir, T, B, states):
     rng = np.random.default_rng(1000 * mode + I + H + L + T)
