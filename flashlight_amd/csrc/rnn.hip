@@ -229,30 +229,51 @@ struct CellFwd {
   int ldo;
 };
 
-// gate math of one (batch b, hidden h) element; rp = its recurrent projections, one per gate
+// gate math of one (batch b, hidden h) element, in two halves so that a kernel can issue
+// the loads before it computes the recurrent projections rp (one per gate)
 template <int MODE>
-__device__ __forceinline__ void cell_fwd_apply(const CellFwd& a, int b, int h, int H, const float* rp) {
+struct CellFwdIn {
+  float xp[MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1];
+  float prev;   // LSTM: c before the step; GRU: h before the step
+  float bRn;
+};
+
+template <int MODE>
+__device__ __forceinline__ CellFwdIn<MODE> cell_fwd_load(const CellFwd& a, int b, int h, int H) {
+  constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1;
+  const size_t e = (size_t)b * H + h, q = (size_t)b * G * H + h;
+  CellFwdIn<MODE> in;
+#pragma unroll
+  for (int gq = 0; gq < G; ++gq) in.xp[gq] = a.xp[q + (size_t)gq * H];
+  in.prev = MODE == RNN_LSTM ? a.cp[e] : MODE == RNN_GRU ? a.hp[e] : 0.f;
+  in.bRn = MODE == RNN_GRU ? a.bRn[h] : 0.f;
+  return in;
+}
+
+template <int MODE>
+__device__ __forceinline__ void cell_fwd_finish(const CellFwd& a, int b, int h, int H, const CellFwdIn<MODE>& in,
+                                                const float* rp) {
   constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1;
   const size_t e = (size_t)b * H + h, q = (size_t)b * G * H + h;
   float hv;
   if (MODE == RNN_RELU || MODE == RNN_TANH) {
-    const float pre = a.xp[q] + rp[0];
+    const float pre = in.xp[0] + rp[0];
     hv = MODE == RNN_RELU ? (pre > 0.f ? pre : 0.f) : tanhf(pre);
     a.gt[q] = hv;
   } else if (MODE == RNN_LSTM) {
-    const float ig = sigm(a.xp[q] + rp[0]), fg = sigm(a.xp[q + H] + rp[G > 1 ? 1 : 0]);
-    const float gg = tanhf(a.xp[q + 2 * H] + rp[G > 2 ? 2 : 0]), og = sigm(a.xp[q + 3 * H] + rp[G > 3 ? 3 : 0]);
-    const float c = fg * a.cp[e] + ig * gg;
+    const float ig = sigm(in.xp[0] + rp[0]), fg = sigm(in.xp[G > 1 ? 1 : 0] + rp[G > 1 ? 1 : 0]);
+    const float gg = tanhf(in.xp[G > 2 ? 2 : 0] + rp[G > 2 ? 2 : 0]), og = sigm(in.xp[G > 3 ? 3 : 0] + rp[G > 3 ? 3 : 0]);
+    const float c = fg * in.prev + ig * gg;
     a.cn[e] = c;
     if (a.cy) a.cy[e] = c;
     hv = og * tanhf(c);
     a.gt[q] = ig; a.gt[q + H] = fg; a.gt[q + 2 * H] = gg; a.gt[q + 3 * H] = og;
   } else {
-    const float rg = sigm(a.xp[q] + rp[0]), zg = sigm(a.xp[q + H] + rp[G > 1 ? 1 : 0]);
-    const float rn = rp[G > 2 ? 2 : 0] + a.bRn[h];
-    const float ng = tanhf(a.xp[q + 2 * H] + rg * rn);
+    const float rg = sigm(in.xp[0] + rp[0]), zg = sigm(in.xp[G > 1 ? 1 : 0] + rp[G > 1 ? 1 : 0]);
+    const float rn = rp[G > 2 ? 2 : 0] + in.bRn;
+    const float ng = tanhf(in.xp[G > 2 ? 2 : 0] + rg * rn);
     a.rn[e] = rn;
-    hv = (1.f - zg) * ng + zg * a.hp[e];
+    hv = (1.f - zg) * ng + zg * in.prev;
     a.gt[q] = rg; a.gt[q + H] = zg; a.gt[q + 2 * H] = ng;
   }
   a.hn[e] = hv;
@@ -267,6 +288,7 @@ __global__ void __launch_bounds__(256) rnn_cell_fwd(CellFwd a, int B, int H) {
   const int b = e / H, h = e - b * H;
   constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1;
   const size_t q = (size_t)b * G * H + h;
+  const CellFwdIn<MODE> in = cell_fwd_load<MODE>(a, b, h, H);
   float rp[G];
 #pragma unroll
   for (int gq = 0; gq < G; ++gq) rp[gq] = 0.f;
@@ -275,7 +297,7 @@ __global__ void __launch_bounds__(256) rnn_cell_fwd(CellFwd a, int B, int H) {
 #pragma unroll
     for (int gq = 0; gq < G; ++gq) rp[gq] += r[gq * H];
   }
-  cell_fwd_apply<MODE>(a, b, h, H, rp);
+  cell_fwd_finish<MODE>(a, b, h, H, in, rp);
 }
 
 // One time step of up to two directions in one launch: recurrent product and gate math.
@@ -285,19 +307,26 @@ __global__ void __launch_bounds__(256) rnn_cell_fwd(CellFwd a, int B, int H) {
 // waves split the contraction over the hidden state in interleaved chunks of 16.  A
 // lane's 16-byte load supplies the operands of four 16x16x4 products (the k index of a
 // lane group is permuted the same way on both operands).  The partial tiles meet in
-// LDS, then one thread per (batch, unit) applies the gates.  Needs H % 16 == 0.
+// LDS, then one thread per (batch, unit) applies the gates; those threads issue the
+// loads of their gate inputs before the product, so that the two latencies overlap.
+// Needs H % 16 == 0.
 struct StepFwd {
   CellFwd d[2];
   int B, H;
 };
+constexpr int STEP_FWD_WAVES = 4;
 
 template <int MODE, int NBT>
-__global__ void __launch_bounds__(256) rnn_step_fwd(StepFwd p) {
-  constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1, NB = NBT * 16;
-  __shared__ float red[4][16][NB + 1];
+__global__ void __launch_bounds__(64 * STEP_FWD_WAVES) rnn_step_fwd(StepFwd p) {
+  constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1, NB = NBT * 16, W = STEP_FWD_WAVES;
+  __shared__ float red[W][16][NB + 1];
   const CellFwd& a = p.d[blockIdx.y];
   const int H = p.H, B = p.B, h0 = blockIdx.x * 4;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, fr = lane & 15, fg = lane >> 4;
+  const bool cell = tid < 4 * B;
+  const int cb = tid >> 2, ch = h0 + (tid & 3);
+  CellFwdIn<MODE> cin{};
+  if (cell) cin = cell_fwd_load<MODE>(a, cb, ch, H);
   const int gate = fr >> 2;
   const bool av = gate < G;
   const float* ap = a.R + ((size_t)(av ? gate : 0) * H + h0 + (fr & 3)) * H + 4 * fg;
@@ -317,19 +346,19 @@ __global__ void __launch_bounds__(256) rnn_step_fwd(StepFwd p) {
   constexpr int U = NBT == 4 ? 4 : 8;
   const int chunks = H >> 4;
   const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int c0 = wave; c0 < chunks; c0 += 4 * U) {
+  for (int c0 = wave; c0 < chunks; c0 += W * U) {
     float4 ra[U], rb[U][NBT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // every load is issued (from a clamped, valid address) before any is used
-      const int c = min(c0 + 4 * u, chunks - 1);
+      const int c = min(c0 + W * u, chunks - 1);
       ra[u] = *reinterpret_cast<const float4*>(ap + c * 16);
 #pragma unroll
       for (int nt = 0; nt < NBT; ++nt) rb[u][nt] = *reinterpret_cast<const float4*>(bp[nt] + c * 16);
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const bool in = c0 + 4 * u < chunks;
+      const bool in = c0 + W * u < chunks;
       if (!(in && av)) ra[u] = zero4;
 #pragma unroll
       for (int nt = 0; nt < NBT; ++nt)
@@ -351,13 +380,17 @@ __global__ void __launch_bounds__(256) rnn_step_fwd(StepFwd p) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[wave][4 * fg + r][nt * 16 + fr] = acc[nt][r];
   __syncthreads();
-  if (tid < 4 * B) {
-    const int b = tid >> 2, hh = tid & 3;
+  if (cell) {
+    const int hh = tid & 3;
     float rp[G];
 #pragma unroll
-    for (int gq = 0; gq < G; ++gq)
-      rp[gq] = (red[0][gq * 4 + hh][b] + red[1][gq * 4 + hh][b]) + (red[2][gq * 4 + hh][b] + red[3][gq * 4 + hh][b]);
-    cell_fwd_apply<MODE>(a, b, h0 + hh, H, rp);
+    for (int gq = 0; gq < G; ++gq) {
+      float v = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < W; ++wv) v += red[wv][gq * 4 + hh][cb];
+      rp[gq] = v;
+    }
+    cell_fwd_finish<MODE>(a, cb, ch, H, cin, rp);
   }
 }
 
@@ -380,34 +413,59 @@ struct CellBwd {
   int ldo;
 };
 
-// gradient math of one (batch b, hidden h) element; rec = gradient arriving through the
-// recurrent matrices
+// gradient math of one (batch b, hidden h) element in two halves (loads, then math and
+// stores); rec = gradient arriving through the recurrent matrices
 template <int MODE>
-__device__ __forceinline__ void cell_bwd_apply(const CellBwd& a, int b, int h, int H, float rec) {
+struct CellBwdIn {
+  float go;     // gradient of the output + direct recurrent part
+  float gt[MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1];
+  float cn, cp, dc;   // LSTM
+  float hp, rn;       // GRU
+};
+
+template <int MODE>
+__device__ __forceinline__ CellBwdIn<MODE> cell_bwd_load(const CellBwd& a, int b, int h, int H) {
   constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1;
   const size_t e = (size_t)b * H + h, q = (size_t)b * G * H + h;
-  float go = a.gout ? a.gout[(size_t)b * a.ldo + h] : 0.f;
-  if (a.dh_a) go += a.dh_a[e];
-  go += rec;
+  CellBwdIn<MODE> in{};
+  in.go = a.gout ? a.gout[(size_t)b * a.ldo + h] : 0.f;
+  if (a.dh_a) in.go += a.dh_a[e];
+#pragma unroll
+  for (int gq = 0; gq < G; ++gq) in.gt[gq] = a.gt[q + (size_t)gq * H];
+  if (MODE == RNN_LSTM) {
+    in.cn = a.cn[e]; in.cp = a.cp[e]; in.dc = a.dc[e];
+  }
+  if (MODE == RNN_GRU) {
+    in.hp = a.hp[e]; in.rn = a.rn[e];
+  }
+  return in;
+}
+
+template <int MODE>
+__device__ __forceinline__ void cell_bwd_finish(const CellBwd& a, int b, int h, int H, const CellBwdIn<MODE>& in,
+                                                float rec) {
+  constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1;
+  const size_t e = (size_t)b * H + h, q = (size_t)b * G * H + h;
+  const float go = in.go + rec;
   float direct = 0.f;
   if (MODE == RNN_RELU || MODE == RNN_TANH) {
-    const float hv = a.gt[q];
+    const float hv = in.gt[0];
     const float gp = MODE == RNN_RELU ? (hv > 0.f ? go : 0.f) : go * (1.f - hv * hv);
     a.dgw[q] = gp;
     a.dgr[q] = gp;
   } else if (MODE == RNN_LSTM) {
-    const float ig = a.gt[q], fg = a.gt[q + H], gg = a.gt[q + 2 * H], og = a.gt[q + 3 * H];
-    const float tc = tanhf(a.cn[e]);
-    const float dc = a.dc[e] + go * og * (1.f - tc * tc);
-    const float v0 = dc * gg * ig * (1.f - ig), v1 = dc * a.cp[e] * fg * (1.f - fg);
+    const float ig = in.gt[0], fg = in.gt[G > 1 ? 1 : 0], gg = in.gt[G > 2 ? 2 : 0], og = in.gt[G > 3 ? 3 : 0];
+    const float tc = tanhf(in.cn);
+    const float dc = in.dc + go * og * (1.f - tc * tc);
+    const float v0 = dc * gg * ig * (1.f - ig), v1 = dc * in.cp * fg * (1.f - fg);
     const float v2 = dc * ig * (1.f - gg * gg), v3 = go * tc * og * (1.f - og);
     a.dgw[q] = v0; a.dgw[q + H] = v1; a.dgw[q + 2 * H] = v2; a.dgw[q + 3 * H] = v3;
     a.dgr[q] = v0; a.dgr[q + H] = v1; a.dgr[q + 2 * H] = v2; a.dgr[q + 3 * H] = v3;
     a.dc[e] = dc * fg;
   } else {
-    const float rg = a.gt[q], zg = a.gt[q + H], ng = a.gt[q + 2 * H], rn = a.rn[e];
+    const float rg = in.gt[0], zg = in.gt[G > 1 ? 1 : 0], ng = in.gt[G > 2 ? 2 : 0], rn = in.rn;
     const float dn = go * (1.f - zg) * (1.f - ng * ng);
-    const float v0 = dn * rn * rg * (1.f - rg), v1 = go * (a.hp[e] - ng) * zg * (1.f - zg);
+    const float v0 = dn * rn * rg * (1.f - rg), v1 = go * (in.hp - ng) * zg * (1.f - zg);
     a.dgw[q] = v0; a.dgw[q + H] = v1; a.dgw[q + 2 * H] = dn;
     a.dgr[q] = v0; a.dgr[q + H] = v1; a.dgr[q + 2 * H] = dn * rg;
     direct = go * zg;
@@ -420,72 +478,82 @@ __global__ void __launch_bounds__(256) rnn_cell_bwd(CellBwd a, int B, int H) {
   const int e = blockIdx.x * 256 + threadIdx.x;
   if (e >= B * H) return;
   const int b = e / H, h = e - b * H;
+  const CellBwdIn<MODE> in = cell_bwd_load<MODE>(a, b, h, H);
   float rec = 0.f;
   if (a.dh_b)
     for (int k = 0; k < a.ndhb; ++k) rec += a.dh_b[(size_t)k * B * H + e];
-  cell_bwd_apply<MODE>(a, b, h, H, rec);
+  cell_bwd_finish<MODE>(a, b, h, H, in, rec);
 }
 
 // One backward time step of up to two directions in one launch.  A workgroup owns 16
 // hidden units of one direction: rows of its matrix-core tile are the units (columns
 // of the recurrent matrices, 64 contiguous bytes per contraction index), columns the
-// batch, and its eight waves split the contraction over the gate rows (G*H) in
-// interleaved chunks of 16; the partial tiles meet in LDS and the threads then apply
-// the gate gradients of the step, which become the next launch's operand.  H % 16 == 0.
+// batch.  Its sixteen waves split the contraction over the gate rows (G*H) in
+// interleaved chunks of 16 (with four batch tiles: eight groups of two waves, each wave
+// two of the tiles); the partial tiles meet in LDS and one thread per (unit, batch)
+// applies the gate gradients of the step, which become the next launch's operand.
+// Those threads issue their loads before the product.  H % 16 == 0.
 struct StepBwd {
   CellBwd d[2];
   int B, H;
 };
 
 template <int MODE, int NBT>
-__global__ void __launch_bounds__(512) rnn_step_bwd(StepBwd p) {
+__global__ void __launch_bounds__(1024) rnn_step_bwd(StepBwd p) {
   constexpr int G = MODE == RNN_LSTM ? 4 : MODE == RNN_GRU ? 3 : 1, NB = NBT * 16;
-  __shared__ float red[8][16][NB + 1];
+  constexpr int NW = NBT == 4 ? 2 : NBT;      // batch tiles per wave
+  constexpr int KG = 16 / (NBT / NW);         // wave groups along the contraction
+  __shared__ float red[KG][16][NB + 1];
   const CellBwd& a = p.d[blockIdx.y];
   const int H = p.H, B = p.B, h0 = blockIdx.x * 16, GH = G * H;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, fr = lane & 15, fg = lane >> 4;
+  const bool cell = tid < 16 * B;
+  const int cb = tid >> 4, ch = h0 + (tid & 15);
+  CellBwdIn<MODE> cin{};
+  if (cell) cin = cell_bwd_load<MODE>(a, cb, ch, H);
   const bool have = a.dgr_next != nullptr;
   if (have) {
+    const int kg = wave % KG, nt0 = (wave / KG) * NW;
     const float* ap = a.R + (size_t)(4 * fg) * H + h0 + fr;
-    const float* bp[NBT];
-    bool bv[NBT];
+    const float* bp[NW];
+    bool bv[NW];
 #pragma unroll
-    for (int nt = 0; nt < NBT; ++nt) {
-      const int b = nt * 16 + fr;
+    for (int nt = 0; nt < NW; ++nt) {
+      const int b = (nt0 + nt) * 16 + fr;
       bv[nt] = b < B;
       bp[nt] = a.dgr_next + (size_t)(bv[nt] ? b : 0) * GH + 4 * fg;
     }
-    floatx4_t acc[NBT];
+    floatx4_t acc[NW];
 #pragma unroll
-    for (int nt = 0; nt < NBT; ++nt) acc[nt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-    constexpr int U = NBT == 4 ? 4 : 8;   // chunks in flight per wave
+    for (int nt = 0; nt < NW; ++nt) acc[nt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+    constexpr int U = NW == 2 ? 4 : 8;   // chunks in flight per wave (registers: 128 per thread)
     const int chunks = GH >> 4;
     const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int c0 = wave; c0 < chunks; c0 += 8 * U) {
+    for (int c0 = kg; c0 < chunks; c0 += KG * U) {
       float ra[U][4];
-      float4 rb[U][NBT];
+      float4 rb[U][NW];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int c = min(c0 + 8 * u, chunks - 1);
+        const int c = min(c0 + KG * u, chunks - 1);
 #pragma unroll
         for (int m = 0; m < 4; ++m) ra[u][m] = ap[((size_t)c * 16 + m) * H];
 #pragma unroll
-        for (int nt = 0; nt < NBT; ++nt) rb[u][nt] = *reinterpret_cast<const float4*>(bp[nt] + c * 16);
+        for (int nt = 0; nt < NW; ++nt) rb[u][nt] = *reinterpret_cast<const float4*>(bp[nt] + c * 16);
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const bool in = c0 + 8 * u < chunks;
+        const bool in = c0 + KG * u < chunks;
 #pragma unroll
         for (int m = 0; m < 4; ++m)
           if (!in) ra[u][m] = 0.f;
 #pragma unroll
-        for (int nt = 0; nt < NBT; ++nt)
+        for (int nt = 0; nt < NW; ++nt)
           if (!(in && bv[nt])) rb[u][nt] = zero4;
       }
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
-        for (int nt = 0; nt < NBT; ++nt) {
+        for (int nt = 0; nt < NW; ++nt) {
           const float bv4[4] = {rb[u][nt].x, rb[u][nt].y, rb[u][nt].z, rb[u][nt].w};
 #pragma unroll
           for (int m = 0; m < 4; ++m)
@@ -493,19 +561,18 @@ __global__ void __launch_bounds__(512) rnn_step_bwd(StepBwd p) {
         }
     }
 #pragma unroll
-    for (int nt = 0; nt < NBT; ++nt)
+    for (int nt = 0; nt < NW; ++nt)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) red[wave][4 * fg + r][nt * 16 + fr] = acc[nt][r];
+      for (int r = 0; r < 4; ++r) red[kg][4 * fg + r][(nt0 + nt) * 16 + fr] = acc[nt][r];
   }
   __syncthreads();
-  for (int e = tid; e < 16 * B; e += 512) {
-    const int b = e >> 4, hh = e & 15;
+  if (cell) {
     float rec = 0.f;
     if (have) {
 #pragma unroll
-      for (int wv = 0; wv < 8; ++wv) rec += red[wv][hh][b];
+      for (int k = 0; k < KG; ++k) rec += red[k][tid & 15][cb];
     }
-    cell_bwd_apply<MODE>(a, b, h0 + hh, H, rec);
+    cell_bwd_finish<MODE>(a, cb, ch, H, cin, rec);
   }
 }
 
@@ -572,7 +639,7 @@ int forward_pl(const RnnGeom& g, int pl, const float* in, size_t inl, const floa
 
 template <int MODE, int NBT>
 void launch_step_fwd(const StepFwd& p, int D, hipStream_t s) {
-  hipLaunchKernelGGL((rnn_step_fwd<MODE, NBT>), dim3(p.H / 4, D), dim3(256), 0, s, p);
+  hipLaunchKernelGGL((rnn_step_fwd<MODE, NBT>), dim3(p.H / 4, D), dim3(64 * STEP_FWD_WAVES), 0, s, p);
 }
 
 // one layer, all directions: per direction the input projection of all steps, then one
@@ -696,7 +763,7 @@ int backward_pl(const RnnGeom& g, int pl, const float* in, size_t inl, const flo
 
 template <int MODE, int NBT>
 void launch_step_bwd(const StepBwd& p, int D, hipStream_t s) {
-  hipLaunchKernelGGL((rnn_step_bwd<MODE, NBT>), dim3(p.H / 16, D), dim3(512), 0, s, p);
+  hipLaunchKernelGGL((rnn_step_bwd<MODE, NBT>), dim3(p.H / 16, D), dim3(1024), 0, s, p);
 }
 
 template <int MODE>

@@ -34,7 +34,8 @@ def test_relu(dtype):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("fin,fout,batch", [(3136, 1024, 16), (1024, 10, 64), (37, 21, 9), (5, 130, 1), (200, 1, 70)])
+@pytest.mark.parametrize("fin,fout,batch", [(3136, 1024, 16), (1024, 10, 64), (37, 21, 9), (5, 130, 1), (200, 1, 70),
+                                             (96, 80, 300), (130, 67, 1000)])
 def test_linear(fin, fout, batch, dtype):
     rng = np.random.default_rng(fin + fout + batch)
     x = _round(rng.standard_normal((batch, fin)).astype(np.float32), dtype)
