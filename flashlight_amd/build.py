@@ -40,7 +40,8 @@ def _compile(src):
 
 HOST = os.path.join(HERE, "host")
 HOST_LIB = os.path.join(LIBDIR, "libflhip_host.so")
-HOST_SOURCES = ["HipTensor.cpp", "HipAutogradExtension.cpp", "Functions.cpp", "Modules.cpp", "Resnet.cpp"]
+HOST_SOURCES = ["HipTensor.cpp", "HipAutogradExtension.cpp", "Functions.cpp", "Modules.cpp", "Resnet.cpp",
+                "SequentialBuilder.cpp"]
 HOST_TEST_SRC = os.path.join(ROOT, "tests", "cpp", "test_host_extension.cpp")
 HOST_TEST_BIN = os.path.join(ROOT, "tests", "cpp", "bin", "test_host_extension")
 

@@ -323,13 +323,21 @@ Variable relu(const Variable& input) {
 }
 
 Variable moddims(const Variable& input, const Shape& dims) {
-  // one -1 is inferred from the element count (Functions.cpp:797-815)
+  // a 0 keeps the input's dimension, one -1 is inferred from the element count
+  // (Functions.cpp:969-1008)
   std::vector<Dim> d = dims.get();
+  for (size_t i = 0; i < d.size(); ++i)
+    if (d[i] == 0) {
+      if ((int)i >= input.tensor().ndim())
+        throw std::invalid_argument("moddims: tried to infer dimension " + std::to_string(i) +
+                                    " which exceeds the number of dimensions of the input.");
+      d[i] = input.tensor().dim((int)i);
+    }
   Dim known = 1;
   int infer = -1;
   for (size_t i = 0; i < d.size(); ++i) {
     if (d[i] == -1) {
-      if (infer >= 0) throw std::invalid_argument("moddims: only one dimension may be -1");
+      if (infer >= 0) throw std::invalid_argument("moddims: too many dimensions infer");
       infer = (int)i;
     } else {
       known *= d[i];

@@ -1,0 +1,147 @@
+#include "SequentialBuilder.h"
+
+#include <fstream>
+#include <sstream>
+#include <stdexcept>
+
+namespace fl {
+namespace pkg {
+namespace runtime {
+namespace {
+
+std::string trim(const std::string& s) {
+  const char* ws = " \t\r\n";
+  const size_t a = s.find_first_not_of(ws);
+  if (a == std::string::npos) return "";
+  return s.substr(a, s.find_last_not_of(ws) - a + 1);
+}
+
+void replaceAll(std::string& s, const std::string& from, const std::string& to) {
+  for (size_t pos = 0; (pos = s.find(from, pos)) != std::string::npos; pos += to.size()) s.replace(pos, from.size(), to);
+}
+
+std::vector<std::string> splitOnWhitespace(const std::string& s) {
+  std::istringstream in(s);
+  std::vector<std::string> out;
+  for (std::string tok; in >> tok;) out.push_back(tok);
+  return out;
+}
+
+[[noreturn]] void failParse(const std::string& line) { throw std::invalid_argument("Failed parsing - " + line); }
+
+int toInt(const std::string& s, const std::string& line) {
+  try {
+    size_t used = 0;
+    const int v = std::stoi(s, &used);
+    if (used != s.size()) failParse(line);
+    return v;
+  } catch (const std::invalid_argument&) {
+    failParse(line);
+  } catch (const std::out_of_range&) {
+    failParse(line);
+  }
+}
+
+// one module from one line (SequentialBuilder.cpp:98-640)
+ModulePtr parseLine(const std::string& line) {
+  const std::vector<std::string> p = splitOnWhitespace(line);
+  if (p.empty()) failParse(line);
+  const size_t n = p.size();
+  auto inRange = [&](size_t a, size_t c) { return a <= n && n <= c; };
+  auto I = [&](size_t i) { return toInt(p[i], line); };
+  const std::string& op = p[0];
+
+  if (op == "V") {
+    if (n < 2) failParse(line);
+    std::vector<Dim> dims;
+    for (size_t i = 1; i < n; ++i) dims.push_back(I(i));
+    return std::make_shared<View>(Shape(dims));
+  }
+  if (op == "C" || op == "C1") {
+    if (!inRange(5, 7)) failParse(line);
+    const int px = n >= 6 ? I(5) : 0, dx = n >= 7 ? I(6) : 1;
+    return std::make_shared<Conv2D>(I(1), I(2), I(3), 1, I(4), 1, px, 0, dx, 1);
+  }
+  if (op == "C2") {
+    if (!inRange(7, 11)) failParse(line);
+    const int px = n >= 8 ? I(7) : 0, py = n >= 9 ? I(8) : 0, dx = n >= 10 ? I(9) : 1, dy = n >= 11 ? I(10) : 1;
+    return std::make_shared<Conv2D>(I(1), I(2), I(3), I(4), I(5), I(6), px, py, dx, dy);
+  }
+  if (op == "L") {
+    if (!inRange(3, 4)) failParse(line);
+    const bool bias = !(n == 4 && p[3] == "0");
+    return std::make_shared<Linear>(I(1), I(2), bias);
+  }
+  if (op == "BN") {
+    if (!inRange(3, 5)) failParse(line);
+    std::vector<int> axes;
+    for (size_t i = 2; i < n; ++i) axes.push_back(I(i));
+    return std::make_shared<BatchNorm>(axes, I(1));
+  }
+  if (op == "LN") {
+    if (!inRange(2, 4)) failParse(line);
+    std::vector<int> axes;
+    for (size_t i = 1; i < n; ++i) axes.push_back(I(i));
+    // the reference rejects the pre-2020 spelling "LN 3" (SequentialBuilder.cpp:340-349)
+    if (axes == std::vector<int>{3}) failParse(line);
+    return std::make_shared<LayerNorm>(axes);
+  }
+  if (op == "M" || op == "A") {
+    if (n < 5) failParse(line);
+    const int px = n > 5 ? I(5) : 0, py = n > 6 ? I(6) : 0;
+    return std::make_shared<Pool2D>(I(1), I(2), I(3), I(4), px, py,
+                                    op == "A" ? PoolingMode::AVG_INCLUDE_PADDING : PoolingMode::MAX);
+  }
+  if (op == "R") {
+    if (n != 1) failParse(line);
+    return std::make_shared<ReLU>();
+  }
+  if (op == "LSM") {
+    if (n != 2) failParse(line);
+    return std::make_shared<LogSoftmax>(I(1));
+  }
+  if (op == "RNN" || op == "GRU" || op == "LSTM") {
+    if (n < 3) failParse(line);
+    const RnnMode mode = op == "RNN" ? RnnMode::RELU : op == "GRU" ? RnnMode::GRU : RnnMode::LSTM;
+    const int layers = n > 3 ? I(3) : 1;
+    const bool bidirectional = n > 4 ? I(4) > 0 : false;
+    const float dropout = n > 5 ? std::stof(p[5]) : 0.0f;
+    return std::make_shared<RNN>(I(1), I(2), layers, mode, bidirectional, dropout);
+  }
+  static const char* const absent[] = {"RO", "PD", "TR", "CFR", "POSEMB", "SINPOSEMB", "TDS", "AC", "E", "ADAPTIVEE",
+                                       "WN", "DO", "ELU", "R6", "PR", "LG", "HT", "T", "GLU", "SH", "RES", "SKIP",
+                                       "SKIPL", "SAUG", "PC"};
+  for (const char* a : absent)
+    if (op == a)
+      throw std::invalid_argument("buildSequentialModule: module '" + op +
+                                  "' is not provided by this backend - " + line);
+  failParse(line);
+}
+
+}  // namespace
+
+std::shared_ptr<fl::Sequential> buildSequentialModule(const std::vector<std::string>& lines, int64_t nFeatures,
+                                                      int64_t nClasses) {
+  auto net = std::make_shared<fl::Sequential>();
+  for (const std::string& raw : lines) {
+    std::string l = trim(raw);
+    replaceAll(l, "NFEAT", std::to_string(nFeatures));
+    replaceAll(l, "NLABEL", std::to_string(nClasses));
+    if (l.empty() || l[0] == '#') continue;   // blank lines and comments
+    net->add(parseLine(l));
+  }
+  return net;
+}
+
+std::shared_ptr<fl::Sequential> buildSequentialModule(const std::string& archfile, int64_t nFeatures,
+                                                      int64_t nClasses) {
+  std::ifstream in(archfile);
+  if (!in) throw std::runtime_error("fl::pkg::runtime::buildSequentialModule given invalid arch filepath");
+  std::vector<std::string> lines;
+  for (std::string s; std::getline(in, s);) lines.push_back(s);
+  return buildSequentialModule(lines, nFeatures, nClasses);
+}
+
+}  // namespace runtime
+}  // namespace pkg
+}  // namespace fl

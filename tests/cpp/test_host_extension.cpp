@@ -24,6 +24,7 @@
 
 #include "Functions.h"
 #include "Modules.h"
+#include "SequentialBuilder.h"
 #include "HipAutogradExtension.h"
 #include "flref.h"
 
@@ -709,6 +710,95 @@ static void testSpeechStack() {
   CHECK(relL2(hostOf(in.grad()), grad) <= 3e-4);
 }
 
+// Architecture lines (flashlight/pkg/runtime/common/SequentialBuilder.cpp:28-67, 98-640): a
+// network built from text must be the network built by hand from the same modules - same
+// parameters from the same seed, bit-identical outputs and gradients.
+static void testArchBuilder() {
+  std::printf("architecture lines\n");
+  using fl::pkg::runtime::buildSequentialModule;
+  const std::vector<std::string> arch = {
+      "# speech-style stack, then a recurrent layer and a classifier",
+      "",
+      "  V -1 1 NFEAT 0  ",
+      "C NFEAT 48 21 1 -1",
+      "BN 48 2",
+      "R",
+      "C2 48 64 5 1 2 1 -1 0 1 1",
+      "LN 0 1 2",
+      "R",
+      "M 2 1 2 1",
+      "V 0 64 -1",
+      "V 64 -1 1",      // [T, C, B] memory is not [C, T, B]: only the shapes matter to this test
+      "GRU 64 32 1 1",
+      "V 64 -1",
+      "L 64 NLABEL 0",
+      "LSM 0",
+  };
+  const int T = 40, F = 12, B = 3, NL = 7;
+  setSeed(91);
+  auto net = buildSequentialModule(arch, F, NL);
+  CHECK(net->modules().size() == 14);
+  setSeed(91);
+  Sequential ref;
+  ref.add(View(Shape({-1, 1, F, 0})));
+  ref.add(Conv2D(F, 48, 21, 1, 1, 1, -1, 0, 1, 1));
+  ref.add(BatchNorm(std::vector<int>{2}, 48));
+  ref.add(ReLU());
+  ref.add(Conv2D(48, 64, 5, 1, 2, 1, -1, 0, 1, 1));
+  ref.add(LayerNorm(std::vector<int>{0, 1, 2}));
+  ref.add(ReLU());
+  ref.add(Pool2D(2, 1, 2, 1, 0, 0, PoolingMode::MAX));
+  ref.add(View(Shape({0, 64, -1})));
+  ref.add(View(Shape({64, -1, 1})));
+  ref.add(RNN(64, 32, 1, RnnMode::GRU, true, 0.0f));
+  ref.add(View(Shape({64, -1})));
+  ref.add(Linear(64, NL, false));
+  ref.add(LogSoftmax(0));
+  CHECK(net->params().size() == ref.params().size());
+  for (size_t i = 0; i < ref.params().size() && i < net->params().size(); ++i)
+    CHECK(net->param((int)i).shape() == ref.param((int)i).shape() &&
+          hostOf(net->param((int)i)) == hostOf(ref.param((int)i)));
+  auto x = randn((size_t)T * F * B, 92);
+  Variable in1(Tensor::fromVector({T, F, 1, B}, x), true), in2(Tensor::fromVector({T, F, 1, B}, x), true);
+  Variable y1 = net->forward(in1), y2 = ref.forward(in2);
+  CHECK(y1.shape() == y2.shape() && y1.shape().dim(0) == NL);
+  CHECK(hostOf(y1) == hostOf(y2));
+  auto dy = randn((size_t)y1.tensor().elements(), 93);
+  y1.backward(Variable(Tensor::fromVector(y1.shape(), dy), false));
+  y2.backward(Variable(Tensor::fromVector(y2.shape(), dy), false));
+  CHECK(hostOf(in1.grad()) == hostOf(in2.grad()));
+  for (size_t i = 0; i < ref.params().size() && i < net->params().size(); ++i)
+    CHECK(hostOf(net->param((int)i).grad()) == hostOf(ref.param((int)i).grad()));
+
+  // optional arguments and their defaults
+  auto one = [](const std::string& l) { return buildSequentialModule(std::vector<std::string>{l}, 1, 1)->module(0); };
+  CHECK(one("C 3 4 5 2")->prettyString() == Conv2D(3, 4, 5, 1, 2, 1, 0, 0, 1, 1).prettyString());
+  CHECK(one("C1 3 4 5 2 1 2")->prettyString() == Conv2D(3, 4, 5, 1, 2, 1, 1, 0, 2, 1).prettyString());
+  CHECK(one("C2 3 4 5 6 1 2")->prettyString() == Conv2D(3, 4, 5, 6, 1, 2, 0, 0, 1, 1).prettyString());
+  CHECK(one("A 3 3 2 2 1 1")->prettyString() == Pool2D(3, 3, 2, 2, 1, 1, PoolingMode::AVG_INCLUDE_PADDING).prettyString());
+  CHECK(one("L 5 6")->params().size() == 2 && one("L 5 6 0")->params().size() == 1 && one("L 5 6 1")->params().size() == 2);
+  CHECK(one("LSTM 4 5 2 1")->prettyString() == RNN(4, 5, 2, RnnMode::LSTM, true, 0.0f).prettyString());
+  CHECK(one("RNN 4 5")->prettyString() == RNN(4, 5, 1, RnnMode::RELU, false, 0.0f).prettyString());
+  CHECK(one("BN 8 0 1")->prettyString() == BatchNorm(std::vector<int>{0, 1}, 8).prettyString());
+  // malformed lines, lines for modules that do not exist here, a missing file
+  for (const char* bad : {"C 3 4 5", "C2 3 4 5 6 1", "L 5", "BN 8", "LN", "LN 3", "M 2 2 2", "R 1", "LSM", "GRU 4",
+                          "C 3 x 5 1", "XYZ 1 2", "RO 1 0 2 3", "DO 0.2", "TDS 10 21 80", "RES 2 1 3", "PC f16"})
+    CHECK(throws<std::invalid_argument>([&] { one(bad); }));
+  CHECK(throws<std::runtime_error>([] { buildSequentialModule(std::string("/nonexistent/arch.txt"), 1, 1); }));
+  // from a file
+  const std::string path = "/tmp/flhip_arch_test_" + std::to_string((long)getpid()) + ".arch";
+  if (FILE* f = std::fopen(path.c_str(), "w")) {
+    for (const std::string& l : arch) std::fprintf(f, "%s\n", l.c_str());
+    std::fclose(f);
+    setSeed(91);
+    auto net2 = buildSequentialModule(path, F, NL);
+    CHECK(net2->modules().size() == 14 && hostOf(net2->param(0)) == hostOf(ref.param(0)));
+    std::remove(path.c_str());
+  } else {
+    CHECK(false);
+  }
+}
+
 // rnn / rnnBackward through the closure and the RNN module (flashlight/fl/test/autograd/
 // AutogradRnnTest.cpp:24-90 uses 2 layers, hidden 2, input 2, bidirectional; here against
 // the CPU checker instead of finite differences)
@@ -815,6 +905,7 @@ int main() {
     testBottleneck();
     testSpeechStack();
     testRnn();
+    testArchBuilder();
     fl::sync();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
