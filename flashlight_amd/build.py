@@ -72,6 +72,12 @@ def build_host(verbose=True):
         cmd = cxx + ["-o", rbin, rsrc, "-L" + LIBDIR, "-lflhip_host", "-lflhip",
                      "-Wl,-rpath,$ORIGIN/../../../flashlight_amd/lib"] + hiplibs
         subprocess.check_call(cmd)
+        # neither do the finite-difference Jacobian tests
+        jsrc = os.path.join(os.path.dirname(HOST_TEST_SRC), "test_jacobian.cpp")
+        jbin = os.path.join(os.path.dirname(HOST_TEST_BIN), "test_jacobian")
+        cmd = cxx + ["-o", jbin, jsrc, "-L" + LIBDIR, "-lflhip_host", "-lflhip",
+                     "-Wl,-rpath,$ORIGIN/../../../flashlight_amd/lib"] + hiplibs
+        subprocess.check_call(cmd)
     if verbose:
         print("built", HOST_LIB)
     return HOST_LIB

@@ -1,5 +1,5 @@
-"""Runs the C++ test program of the host layer (HipTensor, registration,
-HipAutogradExtension, caller closures) on the GPU."""
+"""Runs the C++ test programs of the host layer (HipTensor, registration,
+HipAutogradExtension, caller closures, modules, Jacobians) on the GPU."""
 import os
 import subprocess
 
@@ -30,6 +30,21 @@ def test_resnet50_step_program():
     print(r.stderr)
     assert r.returncode == 0, r.stdout[-3000:]
     assert "ResNet-50 step checks passed" in r.stdout
+
+
+@pytest.mark.gpu
+def test_jacobian_program():
+    """The reference's finite-difference Jacobian tests of conv2d, pool2d, batchnorm (one and
+    several feature axes, the LayerNorm axes) and rnn, with its shapes and tolerances
+    (AutogradConv2DTest.cpp:21-74,137-213, AutogradTest.cpp:333-337,
+    AutogradNormalizationTest.cpp:228-256,294-324,365-383, AutogradRnnTest.cpp:24-160)."""
+    exe = os.path.join(ROOT, "tests", "cpp", "bin", "test_jacobian")
+    assert os.path.exists(exe), "build it with `python -m flashlight_amd.build`"
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=110)
+    print(r.stdout)
+    print(r.stderr)
+    assert r.returncode == 0, r.stdout[-3000:]
+    assert "all Jacobian checks passed" in r.stdout
 
 
 def test_host_library_is_built_and_links_the_c_abi():
