@@ -166,6 +166,51 @@ static void testBatchingInvariance() {
   }
 }
 
+// ModuleTest.cpp:177-194 (ConvPadding: SAME padding with strides and dilation),
+// :382-396 (ConvolutionWithGroupFwd) and :398-413 (PoolingFwd): a batch equals its
+// samples run one by one, with the reference's module arguments, sizes and tolerances
+static void testModuleShapesAndBatching() {
+  std::printf("module shapes and batching\n");
+  setSeed(5);
+  {
+    // written as in the reference: its `true, 1` land on the dilation arguments (1, 1)
+    Conv2D conv1(30, 100, 3, 5, 2, 1, PaddingMode::SAME, 0, true, 1);
+    Conv2D conv2(30, 100, 3, 5, 2, 1, PaddingMode::SAME, PaddingMode::SAME, true, 1);
+    Conv2D conv3(30, 100, 10, 10, 1, 1, PaddingMode::SAME, PaddingMode::SAME, 4, 4);
+    Variable input(Tensor::fromVector({32, 32, 30, 2}, randn((size_t)32 * 32 * 30 * 2, 41)), false);
+    CHECK(conv1(input).shape() == Shape({16, 28, 100, 2}));
+    CHECK(conv2(input).shape() == Shape({16, 32, 100, 2}));
+    CHECK(conv3(input).shape() == Shape({32, 32, 100, 2}));
+  }
+  const int W = 120, H = 100, C = 30, N = 10;
+  auto x = randn((size_t)N * C * H * W, 42);
+  for (auto& v : x) v = 0.5f + 0.25f * v;
+  auto batched = [&](Module& m, double tol, bool sameShape) {
+    Variable in(Tensor::fromVector({W, H, C, N}, x), false);
+    Variable out = m.forward({in}).front();
+    if (sameShape) CHECK(out.shape() == in.shape());
+    const std::vector<float> full = out.tensor().toHostVector();
+    const size_t per = full.size() / N, pin = (size_t)C * H * W;
+    for (int n = 0; n < N; ++n) {
+      std::vector<float> xi(x.begin() + n * pin, x.begin() + (n + 1) * pin);
+      const std::vector<float> one =
+          m.forward({Variable(Tensor::fromVector({W, H, C, 1}, xi), false)}).front().tensor().toHostVector();
+      double worst = one.size() == per ? 0 : 1e30;
+      for (size_t i = 0; i < per && i < one.size(); ++i)
+        worst = std::max(worst, (double)std::fabs(one[i] - full[n * per + i]));
+      CHECK(worst <= tol);
+    }
+  };
+  // as written in the reference, whose `true, 2` are dilation (1, 2), not bias and groups;
+  // the grouped module follows
+  Conv2D conv(30, 50, 9, 7, 2, 3, 3, 2, true, 2);
+  batched(conv, 1e-5, false);
+  Conv2D grouped(30, 50, 9, 7, 2, 3, 3, 2, 1, 1, true, 2);
+  batched(grouped, 1e-5, false);
+  Pool2D pool(9, 7, 1, 1, PaddingMode::SAME, PaddingMode::SAME);
+  batched(pool, 1e-7, true);
+}
+
 static void testPool() {
   std::printf("pool2d\n");
   const int W = 12, H = 10, C = 3, N = 2;
@@ -906,6 +951,7 @@ int main() {
     testSpeechStack();
     testRnn();
     testArchBuilder();
+    testModuleShapesAndBatching();
     fl::sync();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
