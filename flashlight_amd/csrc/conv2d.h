@@ -38,6 +38,11 @@ int mfma_pointwise_conv_fwd(const ConvGeom& g, int dtype, const void* x, const v
                             const float* bias, void* y, hipStream_t s, int ksplit = 1);
 int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w,
                                  void* dx, hipStream_t s, const float* bias = nullptr, int ksplit = 1);
+// bf16 storage on the bf16 matrix cores: 1x1 stride-1 windows over planes that are a
+// multiple of 4 positions, channel counts multiples of 8; -1 otherwise
+int mfma_pointwise16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
+                              hipStream_t s);
+int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s);
 // column-major C = op(A) op(B) on the 1x1 kernels (mode 0: A B, 1: A^T B, 2: A B^T);
 // -1 when it does not apply
 int mfma_gemm(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,

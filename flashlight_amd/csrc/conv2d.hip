@@ -189,6 +189,8 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
   if (!force_direct()) {
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
+      r = mfma_pointwise16_conv_fwd(g, x, w, bias, y, s);
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
       r = mfma_slab16_conv_fwd(g, x, w, bias, y, s);
     if (r < 0 && !skip("gemm1x1")) r = mfma_pointwise_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s);
@@ -223,6 +225,8 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
   if (!force_direct()) {
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
+      r = mfma_pointwise16_conv_bwd_data(g, dy, w, dx, s);
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
       r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s);
     if (r < 0 && !skip("gemm1x1")) r = mfma_pointwise_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s);

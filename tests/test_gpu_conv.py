@@ -51,6 +51,11 @@ MORE = [
     ((3, 96, 14, 14), (160, 96, 1, 1), (2, 2), (0, 0), (1, 1), 1),
     ((2, 40, 9, 11), (24, 40, 1, 1), (2, 3), (0, 0), (1, 1), 1),
     ((40, 32, 28, 28), (64, 32, 1, 1), (1, 1), (0, 0), (1, 1), 1),      # enough positions for the 64 x 256 tile
+    # bf16 matrix-core 1x1 kernels (planes of 4k positions, channels multiples of 8): channel
+    # tails on both sides and fewer positions than one tile; an image boundary inside a tile
+    ((3, 40, 6, 6), (72, 40, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((2, 72, 10, 14), (24, 72, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((5, 136, 14, 14), (200, 136, 1, 1), (1, 1), (0, 0), (1, 1), 1),
 ]
 ALL = LIB_CASES + MORE
 
