@@ -43,6 +43,9 @@ int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, c
 int mfma_pointwise16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
                               hipStream_t s);
 int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s);
+size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g);
+int mfma_pointwise16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
+                           size_t ws_bytes, hipStream_t s);
 // column-major C = op(A) op(B) on the 1x1 kernels (mode 0: A B, 1: A^T B, 2: A B^T);
 // -1 when it does not apply
 int mfma_gemm(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,

@@ -169,8 +169,10 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
     const size_t b = mfma_slab_wgrad_ws(g, d->dtype);
     const size_t c = d->dtype == FLHIP_BF16 ? mfma_wgrad16_ws(g) : 0;
     const size_t e = mfma_pointwise_wgrad_ws(g);
+    const size_t f = d->dtype == FLHIP_BF16 ? mfma_pointwise16_wgrad_ws(g) : 0;
     if (b > a) a = b;
     if (e > a) a = e;
+    if (f > a) a = f;
     return c > a ? c : a;
   }
   return 0;
@@ -264,6 +266,8 @@ extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, 
     FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter: workspace too small");
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
+      r = mfma_pointwise16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
       r = mfma_wgrad16(g, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0 && !skip("gemm1x1"))
       r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, algo_is("tapped"), s);

@@ -233,6 +233,156 @@ int launch_pw16(const ConvGeom& g, const void* src, const void* w, const float* 
   return check_launch(BWD ? "conv2d_bwd_data 1x1 (bf16 mfma)" : "conv2d_fwd 1x1 (bf16 mfma)");
 }
 
+// ---- filter gradient -------------------------------------------------------------------
+constexpr int PG_KC = 64;          // positions per chunk (two instructions deep)
+constexpr int PG_P = PG_KC + 8;    // LDS pitch (elements): 16-byte reads, rows 144 bytes apart
+
+struct Pw16WgradParams {
+  int C, Mo, P, Ptot;
+  int ctiles, mtiles;
+  int nchunks, cps, nsplit;   // chunks of 64 positions over the batch, per slice, slices
+  int E, want_db;
+};
+
+// grid (slice, channel-tile pair).  A workgroup owns dw[64 m][64 c] and one slice of the
+// positions of the whole batch; thread t loads 16 positions (four 8-byte runs, each inside
+// one image) of row t / 4 of both operands per chunk.  out: slice-major partial results
+// [nsplit][E + Mo] (dw tile values, then the bias sums), or dw / db themselves when there
+// is one slice.
+__global__ void __launch_bounds__(256)
+pw16_wgrad_kernel(Pw16WgradParams p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy,
+                  float* __restrict__ out, float* __restrict__ db_direct) {
+  __shared__ __align__(16) uint16_t Ds[2][64 * PG_P];
+  __shared__ __align__(16) uint16_t Xs[2][64 * PG_P];
+  const int slice = blockIdx.x, mtile = blockIdx.y / p.ctiles, ctile = blockIdx.y - mtile * p.ctiles;
+  const int m0 = mtile * 64, c0 = ctile * 64;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, fr = lane & 15, fg = lane >> 4;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int cbeg = slice * p.cps, cend = min(p.nchunks, cbeg + p.cps);
+
+  const int row = tid >> 2, piece = (tid & 3) * 16;
+  const bool mv = m0 + row < p.Mo, cv = c0 + row < p.C;
+  // position run g of this thread in chunk c: Q = c*64 + piece + 4*g; q[g] = its offset in
+  // the image, od/ox[g] = element offsets of (image, row 0) + q in dy / x
+  int q[4];
+  long long od[4], ox[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const long long Q = (long long)cbeg * PG_KC + piece + 4 * g;
+    const int n = (int)(Q / p.P);
+    q[g] = (int)(Q - (long long)n * p.P);
+    od[g] = (long long)n * p.Mo * p.P + q[g];
+    ox[g] = (long long)n * p.C * p.P + q[g];
+  }
+  const long long drow = (long long)(m0 + row) * p.P, xrow = (long long)(c0 + row) * p.P;
+  const long long dlim = (long long)(p.Ptot / p.P) * p.Mo * p.P;   // == N * Mo * P
+  uintx2_t sd[4], sx[4];
+  float bsum = 0.f;
+  const bool do_bias = p.want_db && ctile == 0;
+  auto gload = [&]() {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const bool in = od[g] < dlim;     // past the last image: nothing left
+      sd[g] = (in && mv) ? *reinterpret_cast<const uintx2_t*>(dy + od[g] + drow) : uintx2_t{0u, 0u};
+      sx[g] = (in && cv) ? *reinterpret_cast<const uintx2_t*>(x + ox[g] + xrow) : uintx2_t{0u, 0u};
+      // next chunk: 64 positions on, possibly into the following images
+      q[g] += PG_KC; od[g] += PG_KC; ox[g] += PG_KC;
+      while (q[g] >= p.P) {
+        q[g] -= p.P;
+        od[g] += (long long)(p.Mo - 1) * p.P;
+        ox[g] += (long long)(p.C - 1) * p.P;
+      }
+    }
+  };
+  auto sstore = [&](int buf) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      *reinterpret_cast<uintx2_t*>(&Ds[buf][row * PG_P + piece + 4 * g]) = sd[g];
+      *reinterpret_cast<uintx2_t*>(&Xs[buf][row * PG_P + piece + 4 * g]) = sx[g];
+      if (do_bias) {
+        bsum += bf16_to_f32((bf16_t)(sd[g].x & 0xffffu)) + bf16_to_f32((bf16_t)(sd[g].x >> 16));
+        bsum += bf16_to_f32((bf16_t)(sd[g].y & 0xffffu)) + bf16_to_f32((bf16_t)(sd[g].y >> 16));
+      }
+    }
+  };
+
+  floatx4 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  if (cbeg < cend) {
+    gload();
+    sstore(0);
+  }
+  __syncthreads();
+  for (int c = cbeg; c < cend; ++c) {
+    const int buf = (c - cbeg) & 1;
+    if (c + 1 < cend) gload();
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      bf16x8 a[2], b[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        a[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>(&Ds[buf][((2 * wm + i) * 16 + fr) * PG_P + ks * 32 + 8 * fg]));
+        b[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>(&Xs[buf][((2 * wn + i) * 16 + fr) * PG_P + ks * 32 + 8 * fg]));
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (c + 1 < cend) sstore(buf ^ 1);
+    __syncthreads();
+  }
+
+  float* o = out + (size_t)slice * (p.nsplit > 1 ? (size_t)p.E + p.Mo : 0);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int c = c0 + (2 * wn + j) * 16 + fr;
+      if (c >= p.C) continue;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = m0 + (2 * wm + i) * 16 + 4 * fg + r;
+        if (m < p.Mo) o[(size_t)m * p.C + c] = acc[i][j][r];
+      }
+    }
+  if (do_bias) {
+    bsum += __shfl_xor(bsum, 1, 64);
+    bsum += __shfl_xor(bsum, 2, 64);
+    if ((tid & 3) == 0 && mv) {
+      if (p.nsplit > 1) o[p.E + m0 + row] = bsum;
+      else db_direct[m0 + row] = bsum;
+    }
+  }
+}
+
+bool pw16_wgrad_plan(const ConvGeom& g, Pw16WgradParams* p) {
+  if (!pw16_applies(g)) return false;
+  p->C = g.C; p->Mo = g.K; p->P = g.H * g.W;
+  const long long ptot = (long long)g.N * p->P;
+  if (ptot * std::max(g.C, g.K) >= (1ll << 31)) return false;
+  p->Ptot = (int)ptot;
+  p->ctiles = (g.C + 63) / 64;
+  p->mtiles = (g.K + 63) / 64;
+  p->nchunks = (int)((ptot + PG_KC - 1) / PG_KC);
+  p->E = g.K * g.C;
+  const long long tiles = (long long)p->ctiles * p->mtiles;
+  if (tiles > 65535) return false;
+  // every slice costs a write and a read of the whole gradient: fewer slices for large ones
+  // (measured on the ResNet-50 layers)
+  const int mult = p->E >= 100000 ? 2 : 4;
+  long long ns = (long long)mult * mfma_num_cus() / tiles;
+  if (ns > p->nchunks / 4) ns = p->nchunks / 4;    // at least four chunks per slice
+  if (ns < 1) ns = 1;
+  p->cps = (int)((p->nchunks + ns - 1) / ns);
+  p->nsplit = (p->nchunks + p->cps - 1) / p->cps;
+  return true;
+}
+
 }  // namespace
 
 int mfma_pointwise16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
@@ -244,6 +394,27 @@ int mfma_pointwise16_conv_fwd(const ConvGeom& g, const void* x, const void* w, c
 int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s) {
   if (!pw16_applies(g)) return -1;
   return launch_pw16<true>(g, dy, w, nullptr, dx, s);
+}
+
+size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g) {
+  Pw16WgradParams p{};
+  if (!pw16_wgrad_plan(g, &p)) return 0;
+  return p.nsplit > 1 ? (size_t)p.nsplit * ((size_t)p.E + p.Mo) * sizeof(float) : 0;
+}
+
+int mfma_pointwise16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
+                           size_t ws_bytes, hipStream_t s) {
+  if (!dw) return -1;
+  Pw16WgradParams p{};
+  if (!pw16_wgrad_plan(g, &p)) return -1;
+  p.want_db = db != nullptr;
+  const size_t need = p.nsplit > 1 ? (size_t)p.nsplit * ((size_t)p.E + p.Mo) * sizeof(float) : 0;
+  if (need && (!ws || ws_bytes < need)) return fail(FLHIP_INVALID_ARGUMENT, "conv2d_bwd_filter: workspace too small");
+  float* out = p.nsplit > 1 ? static_cast<float*>(ws) : dw;
+  hipLaunchKernelGGL(pw16_wgrad_kernel, dim3((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles)), dim3(256), 0, s, p,
+                     static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), out, db);
+  if (p.nsplit > 1) wgrad_reduce_launch(static_cast<const float*>(ws), p.nsplit, p.E, p.Mo, p.want_db, dw, db, s);
+  return check_launch("conv2d_bwd_filter 1x1 (bf16 mfma)");
 }
 
 }  // namespace flhip
