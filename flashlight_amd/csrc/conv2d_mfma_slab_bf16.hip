@@ -127,16 +127,19 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
     const int img_base = (img * p.SC + grp * p.SCg) * p.SH * p.SW;
     // slab unit u: bits 0-1 channel group, bits 2-3 low bits of the slab row, then the
     // group of 8 image columns, then the high bits of the row (see the bank note above)
-    const int qrow = p.SW >> 3, rs_hi = (p.RS + 3) >> 2;
+    const int qrow = (p.SW + 7) >> 3, rs_hi = (p.RS + 3) >> 2;
     const int n_units = CG * 4 * qrow * rs_hi;
     int xg[NXU_MAX], xl[NXU_MAX];                // global byte offset of channel 0 of the group, LDS cell
     int xc[NXU_MAX];                             // first channel of the unit within the chunk
+    int xn[NXU_MAX];                             // columns of the unit inside the row (the last unit of a
+                                                 // row of 8k+2..6 columns reads into the next row: zeroed)
 #pragma unroll
     for (int i = 0; i < NXU_MAX; ++i) {
       const int u = tid + GTHREADS * i;
       xg[i] = OOB;
       xl[i] = p.x_cells - 8;
       xc[i] = 0;
+      xn[i] = 8;
       if (u < n_units) {
         const int cg = u & 3, rl = (u >> 2) & 3;
         const int t = u >> 4;
@@ -144,6 +147,7 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
         const int rs = rh * 4 + rl;
         const int sr = r0 + p.min_sh + rs;
         xc[i] = cg * 8;
+        xn[i] = min(8, p.SW - 8 * q);
         if (rs < p.RS) {
           xl[i] = cg * p.XPL + rs * p.WSP + p.XOFF + 8 * q;
           if ((unsigned)sr < (unsigned)p.SH) xg[i] = (img_base + (cg * 8 * p.SH + sr) * p.SW + 8 * q) * 2;
@@ -157,7 +161,7 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
     // 8x8 transpose of 16-bit values: in[k] = 8 consecutive positions of channel k;
     // cell t = the 8 channels of position t.  Column 2t+s of channels 2k, 2k+1 is the
     // low (s = 0) or high (s = 1) half of dword t of the two rows.
-    auto transpose_store = [&](const uint4 (&in)[8], uint4* dst) {
+    auto transpose_store = [&](const uint4 (&in)[8], uint4* dst, int valid = 8) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         unsigned lo[4], hi[4];
@@ -168,8 +172,8 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
           lo[k] = __builtin_amdgcn_perm(o, e, 0x05040100u);
           hi[k] = __builtin_amdgcn_perm(o, e, 0x07060302u);
         }
-        dst[2 * t] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-        dst[2 * t + 1] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        dst[2 * t] = 2 * t < valid ? make_uint4(lo[0], lo[1], lo[2], lo[3]) : make_uint4(0u, 0u, 0u, 0u);
+        dst[2 * t + 1] = 2 * t + 1 < valid ? make_uint4(hi[0], hi[1], hi[2], hi[3]) : make_uint4(0u, 0u, 0u, 0u);
       }
     };
     auto ld16 = [&](__amdgpu_buffer_rsrc_t r, int off) {
@@ -190,7 +194,7 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
     auto store_x = [&](int buf) {
       uint4* xs = Xs + buf * p.x_cells;
 #pragma unroll
-      for (int i = 0; i < NXU_MAX; ++i) transpose_store(xv[i], xs + xl[i]);
+      for (int i = 0; i < NXU_MAX; ++i) transpose_store(xv[i], xs + xl[i], xn[i]);
     };
     // runs the chunk pipeline with the given weight loader / storer
     auto pipeline = [&](auto&& load_w, auto&& store_w) {
@@ -499,7 +503,8 @@ void layout(Slab16Params* p, int R) {
   p->RS = R + (p->KH - 1) * p->dly;
   p->XOFF = std::max(0, -p->min_sw);
   const int max_sc = p->min_sw + p->DW - 1 + (p->KW - 1) * p->dlx;   // last source column read
-  p->WSP = round_to_residue(p->XOFF + std::max(max_sc + 1, p->SW), 4, 16);
+  // a row is stored in units of 8 columns: room for the last, possibly partial one
+  p->WSP = round_to_residue(p->XOFF + std::max(max_sc + 1, (p->SW + 7) / 8 * 8), 4, 16);
   p->XPL = round_to_residue(p->RS * p->WSP, 1, 16);
   p->x_cells = CG * p->XPL + 8;
   // plane pitch = 2 (mod 16): the cell stores of the backward-data transpose spread
@@ -510,7 +515,9 @@ void layout(Slab16Params* p, int R) {
 
 bool plan(Slab16Params* p, size_t* shmem) {
   if (p->KHW > KHW_MAX) return false;
-  if (p->SW % 8 != 0) return false;              // rows are read 16 bytes at a time
+  // rows are read 16 bytes at a time from 4-byte aligned addresses (the last unit of a row
+  // may run into the next row or past the tensor: masked / out of range)
+  if (p->SW % 2 != 0) return false;
   const int max_pos = 2 * NT_MAX * 16;
   if (p->DW > max_pos) return false;
   const int cus = mfma_num_cus();
@@ -520,7 +527,7 @@ bool plan(Slab16Params* p, size_t* shmem) {
     layout(p, R);
     const size_t bytes = (size_t)2 * (p->x_cells + p->a_cells) * 16;
     if (bytes > 156 * 1024) break;
-    if (CG * 4 * (p->SW / 8) * ((p->RS + 3) / 4) > GTHREADS * NXU_MAX) break;
+    if (CG * 4 * ((p->SW + 7) / 8) * ((p->RS + 3) / 4) > GTHREADS * NXU_MAX) break;
     const long long tiles = (long long)p->N * ((p->DH + R - 1) / R) * p->mtiles * p->groups;
     const long long rounds = (tiles + cus - 1) / cus;
     const int nb = (R * p->DW + 15) / 16;

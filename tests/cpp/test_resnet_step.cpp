@@ -10,6 +10,7 @@
 #include <unistd.h>
 #include <cstdio>
 #include <cstdlib>
+#include <string>
 #include <random>
 #include <vector>
 
@@ -73,6 +74,10 @@ int main(int argc, char** argv) {
     Variable target(Tensor::fromHost(Shape({B}), dtype::s32, labels.data()), false);
 
     if (steps > 0) {
+      // "bf16" as third argument: bf16 activations, parameters cast per call by the modules
+      // (fp32 master copies, fp32 batch-norm parameters and statistics)
+      const bool half = argc > 3 && std::string(argv[3]) == "bf16";
+      if (half) in = Variable(in.tensor().astype(dtype::bf16), false);
       for (int i = 0; i < 3; ++i) step(*model, in, target);
       fl::sync();
       const auto t0 = std::chrono::steady_clock::now();
@@ -80,8 +85,8 @@ int main(int argc, char** argv) {
       for (int i = 0; i < steps; ++i) last = step(*model, in, target).tensor().toHostVector()[0];
       fl::sync();
       const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / steps;
-      std::printf("forward + loss + backward: %.2f ms per step (batch %d, %.1f images/s), loss %.4f, "
-                  "device cache %.1f MB\n", ms, B, B / ms * 1e3, last, deviceCacheBytes() / 1e6);
+      std::printf("forward + loss + backward (%s): %.2f ms per step (batch %d, %.1f images/s), loss %.4f, "
+                  "device cache %.1f MB\n", half ? "bf16" : "f32", ms, B, B / ms * 1e3, last, deviceCacheBytes() / 1e6);
       std::fflush(stdout);
       // timing mode leaves through exit() so that a profiler's exit handlers run
       std::exit(0);
