@@ -238,7 +238,7 @@ wgrad_kernel(WgradParams p, const T* __restrict__ x, const T* __restrict__ dy,
     default: run(std::integral_constant<int, 8>{}); break;
   }
 
-  if (do_db && tid < m_lim) {
+  if (do_db && tid < min(m_lim, BM)) {
     const int ch = grp * p.Kg + mtile * BM + tid;
     if (p.nsplit > 1)
       o[p.E + ch] = dbacc;

@@ -199,7 +199,7 @@ wgrad_slab_kernel(WSlabParams p, const T* __restrict__ x, const T* __restrict__ 
         }
       }
       __syncthreads();                      // tile parked, partials written
-      if (do_db && tid < m_lim) {
+      if (do_db && tid < min(m_lim, BM)) {
         float s = 0.f;
         for (int q = 0; q < qy; ++q) s += dbpart[tid * qy + q];
         write_db(s);
@@ -292,7 +292,7 @@ wgrad_slab_kernel(WSlabParams p, const T* __restrict__ x, const T* __restrict__ 
       sum_db(r + 1);
       __syncthreads();
     }
-    if (sum_rows && tid < m_lim) write_db(dbacc);
+    if (sum_rows && tid < min(m_lim, BM)) write_db(dbacc);
     __syncthreads();                        // tile parked
     if (p.stage_ok) store_tile();
     return;

@@ -60,6 +60,7 @@ struct W16Params {
   int total_rows;
   int E;               // K*Cg*9
   int want_db;
+  int tail;            // dwords (column pairs) of a row's last 8-column unit that lie inside the row
   unsigned x_bytes, dy_bytes;
 };
 
@@ -161,11 +162,20 @@ wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restri
       for (int i = 0; i < NDI; ++i)
         r.yv[i] = __builtin_amdgcn_raw_buffer_load_b128(yrsrc, live ? yg[i] + yb : OOB, 0, 0);
     };
+    // the last unit of a row of 8k+2..6 columns has read into the next row: zero that part
+    auto in_row = [&](uintx4_t v) {
+      if (last_q) {
+        v.y = p.tail > 1 ? v.y : 0u;
+        v.z = p.tail > 2 ? v.z : 0u;
+        v.w = p.tail > 3 ? v.w : 0u;
+      }
+      return v;
+    };
     auto store_row = [&](int buf, const RowRegs& r) {
       uint4* b = lds16 + buf * p.buf_cells;
 #pragma unroll
       for (int i = 0; i < NXI; ++i) {
-        const uintx4_t v = r.xv[i];
+        const uintx4_t v = in_row(r.xv[i]);
         // element left of the eight (high half of the left lane's last dword) and
         // right of them (low half of the right lane's first dword); zero at row ends
         unsigned left = __shfl_up(v.w, 1, 64), right = __shfl_down(v.x, 1, 64);
@@ -183,7 +193,7 @@ wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restri
       }
 #pragma unroll
       for (int i = 0; i < NDI; ++i) {
-        const uintx4_t v = r.yv[i];
+        const uintx4_t v = in_row(r.yv[i]);
         if (yl[i] >= 0) b[yl[i]] = make_uint4(v.x, v.y, v.z, v.w);
         float s = 0.f;
 #pragma unroll
@@ -226,7 +236,7 @@ wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restri
       }
     }
     __syncthreads();                        // tile parked, partials written
-    if (do_db && tid < m_lim) {
+    if (do_db && tid < min(m_lim, BM)) {
       float s = 0.f;
       for (int k = 0; k < p.Q; ++k) s += dbpart[tid * p.Q + k];
       const int ch = grp * p.Kg + mtile * BM + tid;
@@ -319,11 +329,13 @@ wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restri
 
 bool plan(const ConvGeom& g, W16Params* p) {
   if (g.KH != 3 || g.KW != 3 || g.sy != 1 || g.sx != 1 || g.px != 1 || g.dlx != 1) return false;
-  if (g.Cg % CB != 0 || g.OW % 8 != 0 || g.W != g.OW || g.OW > 64) return false;
+  // rows are read in units of 8 columns from 4-byte aligned addresses
+  if (g.Cg % CB != 0 || g.OW % 2 != 0 || g.W != g.OW || g.OW > 64) return false;
   p->N = g.N; p->C = g.C; p->H = g.H; p->W = g.W; p->K = g.K; p->OH = g.OH; p->OW = g.OW;
   p->py = g.py; p->dly = g.dly;
   p->groups = g.groups; p->Cg = g.Cg; p->Kg = g.Kg;
-  p->Q = g.OW / 8;
+  p->Q = (g.OW + 7) / 8;
+  p->tail = (g.OW - 8 * (p->Q - 1)) / 2;
   p->RPW = 64 / p->Q;
   if (CB * 3 > NXI * 4 * p->RPW || BM > NDI * 4 * p->RPW) return false;
   const int owp = (g.OW + 31) & ~31;

@@ -56,6 +56,9 @@ MORE = [
     ((3, 40, 6, 6), (72, 40, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     ((2, 72, 10, 14), (24, 72, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     ((5, 136, 14, 14), (200, 136, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    # bias gradient with more than one tile of 64 filters (each tile writes only its own sums)
+    ((2, 32, 8, 16), (136, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((2, 64, 20, 20), (160, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
 ]
 ALL = LIB_CASES + MORE
 
