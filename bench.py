@@ -41,6 +41,8 @@ def parse():
     ap.add_argument("--layers", choices=["resnet50", "speech"], default="",
                     help="instead of the bench line: time every conv layer of configs[4] (ResNet-50, batch 32) "
                          "or configs[3] (21x1 speech layers) in all three passes and print a table")
+    ap.add_argument("--rnn", action="store_true",
+                    help="instead of the bench line: time rnn / rnnBackward (LSTM, GRU) at a few sizes")
     return ap.parse_args()
 
 
@@ -61,6 +63,8 @@ def main():
     tdt = torch.float32 if a.dtype == "f32" else torch.bfloat16
     if a.layers:
         return layer_sweep(a, fa, torch, tdt)
+    if a.rnn:
+        return rnn_sweep(a, fa, torch)
     gen = torch.Generator(device=dev).manual_seed(0)
 
     def randn(*shape, scale=1.0, shift=0.0):
@@ -285,6 +289,38 @@ RESNET50_LAYERS = [(1, 32, 3, 224, 224, 64, 7, 7, 2, 2, 3, 3)] + [
 # configs[3]: [1500, 1, 80, 16] through three 21x1 SAME convolutions, the last with stride 2
 SPEECH_LAYERS = [(1, 16, 80, 1, 1500, 250, 1, 21, 1, 1, 0, 10), (1, 16, 250, 1, 1500, 250, 1, 21, 1, 1, 0, 10),
                  (1, 16, 250, 1, 1500, 250, 1, 21, 1, 2, 0, 10)]
+
+
+def rnn_sweep(a, fa, torch):
+    """Wall-clock times of rnn / rnnBackward through the C ABI (a.steps calls after a.warmup);
+    TFLOP/s counts the matrix products only (input and recurrent projections; twice that
+    in the backward pass)."""
+    ops = fa.ops
+    def timed(fn):
+        for _ in range(max(a.warmup, 1)):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(a.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / a.steps * 1e3
+    for mode, name, gates in ((ops.RNN_LSTM, "LSTM", 4), (ops.RNN_GRU, "GRU", 3)):
+        for (I, H, L, bidir, T, B) in ((512, 512, 2, True, 200, 32), (1024, 1024, 1, False, 100, 64),
+                                       (256, 256, 2, False, 50, 16)):
+            n = ops.rnn_param_count(I, H, L, mode, bidir)
+            x = torch.randn(T, B, I, device="cuda")
+            w = torch.randn(n, device="cuda") / H ** 0.5
+            y, hy, cy, res = ops.rnn(x, None, None, w, H, L, mode, bidir)
+            dy = torch.randn_like(y)
+            tf = timed(lambda: ops.rnn(x, None, None, w, H, L, mode, bidir))
+            tb = timed(lambda: ops.rnn_backward(x, w, res, H, L, mode, bidir, dy))
+            D = 2 if bidir else 1
+            fl = sum(D * 2.0 * gates * H * ((I if l == 0 else D * H) + H) * T * B for l in range(L))
+            print("%-4s input %d hidden %d layers %d dirs %d T %d batch %d: fwd %.2f ms (%.1f TFLOP/s)  "
+                  "bwd %.2f ms (%.1f TFLOP/s)" % (name, I, H, L, D, T, B, tf, fl / tf / 1e9, tb, 2 * fl / tb / 1e9),
+                  flush=True)
+    return 0
 
 
 def layer_sweep(a, fa, torch, tdt):
