@@ -56,9 +56,11 @@ int mfma_gemm_slices(int K, int ksplit);
 int gemm_nt(int dtype, const void* A, const void* B, void* C, int M, int N, int K, int slices, hipStream_t s);
 // windows with several taps on the same tile machinery, any stride / padding / dilation
 int mfma_tapped_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w,
-                         const float* bias, void* y, hipStream_t s);
+                         const float* bias, void* y, hipStream_t s, void* ws = nullptr, size_t ws_bytes = 0);
 int mfma_tapped_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w,
-                              void* dx, hipStream_t s);
+                              void* dx, hipStream_t s, void* ws = nullptr, size_t ws_bytes = 0);
+// with that many bytes of workspace the weights are reordered so that a tap's tile is contiguous
+size_t mfma_tapped_ws(const ConvGeom& g, int dtype, bool bwd);
 size_t mfma_pointwise_wgrad_ws(const ConvGeom& g);
 // windows = false: only 1x1 without padding; true: any window, one tap per workgroup
 int mfma_pointwise_wgrad(const ConvGeom& g, int dtype, const void* x, const void* dy, float* dw,

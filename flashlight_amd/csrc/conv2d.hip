@@ -138,8 +138,12 @@ static bool skip(const char* name) {
 // Stride-1 windows over long rows (the 21x1 speech layers: rows of 1500): the gather
 // kernel's one-position-per-thread loads are whole contiguous runs there and it
 // measures faster than the tapped GEMM, except for backward-data into few channels.
-static bool long_rows(const ConvGeom& g, bool bwd) {
+// With its weights reordered (workspace present) the tapped GEMM wins from 128 contraction
+// channels on.
+static bool long_rows(const ConvGeom& g, int dtype, bool bwd, size_t ws_bytes) {
   if (algo_is("tapped")) return false;
+  const size_t need = mfma_tapped_ws(g, dtype, bwd);
+  if (need && ws_bytes >= need && (bwd ? g.K : g.C) >= 128) return false;
   return g.sy == 1 && g.sx == 1 && g.OW >= 64 && (!bwd || g.C >= 128);
 }
 
@@ -175,14 +179,16 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
     if (f > a) a = f;
     return c > a ? c : a;
   }
+  // forward / backward-data: the kernels for windows with several taps read reordered
+  // weights when the caller brings room for them (they run without it, slower)
+  if (pass == FLHIP_CONV_FWD) return mfma_tapped_ws(g, d->dtype, false);
+  if (pass == FLHIP_CONV_BWD_DATA) return mfma_tapped_ws(g, d->dtype, true);
   return 0;
 }
 
 extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const void* w,
                                 const float* bias, void* y, void* ws, size_t ws_bytes,
                                 void* stream) {
-  (void)ws;
-  (void)ws_bytes;
   FLHIP_REQUIRE(d && x && w && y, "conv2d_fwd: null argument");
   ConvGeom g;
   const int rc = make_geom(d, &g);
@@ -195,10 +201,10 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
       r = mfma_slab16_conv_fwd(g, x, w, bias, y, s);
     if (r < 0 && !skip("gemm1x1")) r = mfma_pointwise_conv_fwd(g, d->dtype, x, w, bias, y, s);
-    if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s);
+    if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s, ws, ws_bytes);
     if (r < 0 && !skip("slab")) r = mfma_slab_conv_fwd(g, d->dtype, x, w, bias, y, s);
-    if (r < 0 && !skip("tapped") && !long_rows(g, false))
-      r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s);
+    if (r < 0 && !skip("tapped") && !long_rows(g, d->dtype, false, ws ? ws_bytes : 0))
+      r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s, ws, ws_bytes);
     if (r < 0) r = mfma_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r >= 0) return r;
   }
@@ -217,8 +223,6 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
 
 extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, const void* w,
                                      void* dx, void* ws, size_t ws_bytes, void* stream) {
-  (void)ws;
-  (void)ws_bytes;
   FLHIP_REQUIRE(d && dy && w && dx, "conv2d_bwd_data: null argument");
   ConvGeom g;
   const int rc = make_geom(d, &g);
@@ -231,10 +235,10 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
       r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s);
     if (r < 0 && !skip("gemm1x1")) r = mfma_pointwise_conv_bwd_data(g, d->dtype, dy, w, dx, s);
-    if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s);
+    if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
     if (r < 0 && !skip("slab")) r = mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s);
-    if (r < 0 && !skip("tapped") && !long_rows(g, true))
-      r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s);
+    if (r < 0 && !skip("tapped") && !long_rows(g, d->dtype, true, ws ? ws_bytes : 0))
+      r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
     if (r < 0) r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r >= 0) return r;
   }

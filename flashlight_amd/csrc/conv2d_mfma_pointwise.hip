@@ -394,6 +394,7 @@ struct TapParams {
   int ssh, ssw;          // source step per class grid step
   int rsh, rsw;          // result step per class grid step
   int kchunks, mtiles, ptiles, nclasses;
+  int wre;               // weights were reordered to [tap][row][column] (see reorder_taps_kernel)
   unsigned src_bytes, wgt_bytes, dst_bytes;
   TapClass cls[MAX_CLASSES];
   Tap taps[MAX_TAPS];
@@ -465,16 +466,16 @@ tapped_conv_kernel(TapParams p, const T* __restrict__ src, const T* __restrict__
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           const int m = m0 + wo + 8 * i;
-          wr[i] = buf_ld(wrsrc, (m < p.Mo && k < p.Kc && ntaps > 0) ? ((m * p.Kc + k) * p.KHW + tp.tmem) * esz : OOB,
-                         wgt);
+          const int wo_ = p.wre ? (tp.tmem * p.Mo + m) * p.Kc + k : (m * p.Kc + k) * p.KHW + tp.tmem;
+          wr[i] = buf_ld(wrsrc, (m < p.Mo && k < p.Kc && ntaps > 0) ? wo_ * esz : OOB, wgt);
         }
       } else {
         const int m = m0 + wl;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           const int k = k0 + wo + 4 * i;
-          wr[i] = buf_ld(wrsrc, (m < p.Mo && k < p.Kc && ntaps > 0) ? ((k * p.Mo + m) * p.KHW + tp.tmem) * esz : OOB,
-                         wgt);
+          const int wo_ = p.wre ? (tp.tmem * p.Kc + k) * p.Mo + m : (k * p.Mo + m) * p.KHW + tp.tmem;
+          wr[i] = buf_ld(wrsrc, (m < p.Mo && k < p.Kc && ntaps > 0) ? wo_ * esz : OOB, wgt);
         }
       }
       if (++ti >= ntaps) {
@@ -618,9 +619,22 @@ bool tapped_plan(const ConvGeom& g, TapParams* p) {
   return true;
 }
 
+// The weights of one tap are KHW elements apart in memory ([filter][channel][tap]): a
+// wave's load of a weight tile touches one 4-byte element per 4*KHW bytes.  With a
+// workspace the weights are first copied to [tap][filter][channel] (a transpose of a
+// (filter*channel) x KHW matrix, a few microseconds), where the same loads are contiguous.
+template <typename T>
+__global__ void __launch_bounds__(256) reorder_taps_kernel(const T* __restrict__ in, T* __restrict__ out, int rows,
+                                                           int khw) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (long long)rows * khw) return;
+  const int t = (int)(i / rows), r = (int)(i - (long long)t * rows);
+  out[i] = in[(long long)r * khw + t];
+}
+
 template <bool BWD>
 int launch_tapped(const ConvGeom& g, int dtype, const void* src, const void* wgt, const float* bias,
-                  void* dst, hipStream_t s) {
+                  void* dst, hipStream_t s, void* ws, size_t ws_bytes) {
   TapParams p{};
   if (!tapped_plan<BWD>(g, &p)) return -1;
   const long long esz = dtype == FLHIP_F32 ? 4 : 2;
@@ -630,6 +644,19 @@ int launch_tapped(const ConvGeom& g, int dtype, const void* src, const void* wgt
   p.src_bytes = (unsigned)(BWD ? yb : xb);
   p.dst_bytes = (unsigned)(BWD ? xb : yb);
   p.wgt_bytes = (unsigned)wb;
+  static const bool no_reorder = getenv("FLHIP_TAPPED_NO_REORDER") != nullptr;
+  if (ws && ws_bytes >= (size_t)wb && p.KHW > 1 && !no_reorder) {
+    const int rows = g.K * g.C;
+    const long long total = (long long)rows * p.KHW;
+    if (dtype == FLHIP_F32)
+      hipLaunchKernelGGL((reorder_taps_kernel<float>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+                         static_cast<const float*>(wgt), static_cast<float*>(ws), rows, p.KHW);
+    else
+      hipLaunchKernelGGL((reorder_taps_kernel<bf16_t>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+                         static_cast<const bf16_t*>(wgt), static_cast<bf16_t*>(ws), rows, p.KHW);
+    wgt = ws;
+    p.wre = 1;
+  }
   const unsigned grid = (unsigned)(((p.ptiles + 7) / 8) * 8 * p.mtiles);
   if (dtype == FLHIP_F32)
     hipLaunchKernelGGL((tapped_conv_kernel<float, BWD>), dim3(grid), dim3(MFMA_THREADS), 0, s, p,
@@ -1013,13 +1040,20 @@ int mfma_pointwise_wgrad(const ConvGeom& g, int dtype, const void* x, const void
 }
 
 int mfma_tapped_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w, const float* bias,
-                         void* y, hipStream_t s) {
-  return launch_tapped<false>(g, dtype, x, w, bias, y, s);
+                         void* y, hipStream_t s, void* ws, size_t ws_bytes) {
+  return launch_tapped<false>(g, dtype, x, w, bias, y, s, ws, ws_bytes);
 }
 
 int mfma_tapped_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
-                              hipStream_t s) {
-  return launch_tapped<true>(g, dtype, dy, w, nullptr, dx, s);
+                              hipStream_t s, void* ws, size_t ws_bytes) {
+  return launch_tapped<true>(g, dtype, dy, w, nullptr, dx, s, ws, ws_bytes);
+}
+
+// bytes of workspace with which the tapped kernels read reordered weights (0: not their shape)
+size_t mfma_tapped_ws(const ConvGeom& g, int dtype, bool bwd) {
+  TapParams p{};
+  if (g.KH * g.KW <= 1 || !(bwd ? tapped_plan<true>(g, &p) : tapped_plan<false>(g, &p))) return 0;
+  return (size_t)g.K * g.C * g.KH * g.KW * (dtype == FLHIP_F32 ? 4 : 2);
 }
 
 // Column-major matrix products on the same kernels: a matrix with its columns as

@@ -112,7 +112,9 @@ const char* flhip_arch(void);
 int flhip_conv2d_out_dims(const flhip_conv_desc* d, int32_t* OH, int32_t* OW);
 int flhip_pool2d_out_dims(const flhip_pool_desc* d, int32_t* OH, int32_t* OW);
 
-/* Scratch a convolution pass needs (0 is possible). */
+/* Scratch a convolution pass uses (0 is possible).  The filter gradient needs it (partial
+ * results of the sliced contraction); forward and backward-data run without it too, but
+ * with it the kernels for strided / long windows read weights reordered per tap. */
 size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pass);
 
 /* AutogradExtension::conv2d (AutogradExtension.h:58-69; oneDNN peer

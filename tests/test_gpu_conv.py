@@ -138,6 +138,35 @@ def test_batching_invariance_on_device():
         assert np.allclose(y1[0], y[n], atol=1e-5, rtol=0)
 
 
+@pytest.mark.parametrize("shape", [((2, 128, 9, 40), (136, 128, 1, 21), (1, 2), (0, 10)),
+                                   ((2, 128, 15, 15), (160, 128, 3, 3), (2, 2), (1, 1))])
+def test_forward_and_backward_data_without_workspace(shape):
+    """Forward and backward-data take a workspace only to reorder the weights of strided /
+    long windows; without it they must give the same results (same products, same order)."""
+    import ctypes as C
+    from flashlight_amd import capi
+    xs, ws_, st, pd = shape
+    rng = np.random.default_rng(77)
+    x = dev(rng.standard_normal(xs).astype(np.float32))
+    w = dev((rng.standard_normal(ws_) / 30).astype(np.float32))
+    kw = dict(sx=st[1], sy=st[0], px=pd[1], py=pd[0], dx=1, dy=1, groups=1)
+    y = fa.conv2d(x, w, None, **kw)
+    dy = dev(rng.standard_normal(tuple(y.shape)).astype(np.float32))
+    dx = fa.conv2d_backward_data(dy, xs, w, **kw)
+    L = capi.lib()
+    cd = capi.ConvDesc(xs[0], xs[1], xs[2], xs[3], ws_[0], ws_[2], ws_[3], st[0], st[1], pd[0], pd[1], 1, 1, 1,
+                       capi.F32)
+    assert L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_FWD) == w.numel() * 4
+    assert L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_BWD_DATA) == w.numel() * 4
+    S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: C.c_void_p(t.data_ptr())
+    y0, dx0 = torch.empty_like(y), torch.empty_like(dx)
+    assert L.flhip_conv2d_fwd(C.byref(cd), P(x), P(w), None, P(y0), None, 0, S) == 0
+    assert L.flhip_conv2d_bwd_data(C.byref(cd), P(dy), P(w), P(dx0), None, 0, S) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(y0, y) and torch.equal(dx0, dx)
+
+
 def test_invalid_arguments_raise():
     x = torch.zeros((1, 4, 8, 8), device="cuda")
     w = torch.zeros((4, 3, 3, 3), device="cuda")
