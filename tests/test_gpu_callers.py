@@ -53,6 +53,28 @@ def test_linear(fin, fout, batch, dtype):
     assert rel_l2(host(db), flref.sum_columns(fout, batch, dy)) <= 1e-5
 
 
+@pytest.mark.parametrize("M,N,K", [(5, 7, 3), (64, 64, 16), (70, 33, 129), (1, 9, 200), (130, 67, 300)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_matmul_all_forms_through_the_c_abi(M, N, K, ta, tb, with_bias):
+    """flhip_matmul: C = op(A) op(B) (+ bias per row) in all four transposition forms, whichever
+    kernel takes them (1x1-convolution GEMMs, the A * B^T kernel, the tiled vector-ALU kernel)."""
+    import ctypes as C
+    from flashlight_amd import capi
+    rng = np.random.default_rng(M * 1000 + N * 10 + K)
+    A = rng.standard_normal((M, K) if ta else (K, M)).astype(np.float32)   # storage as in the oracle's test
+    B = rng.standard_normal((K, N) if tb else (N, K)).astype(np.float32)
+    bias = rng.standard_normal(M).astype(np.float32) if with_bias else None
+    want = flref.matmul(M, N, K, A, B, ta, tb, bias)
+    Ad, Bd, Cd = dev(A), dev(B), torch.empty(N, M, device="cuda")
+    bd = dev(bias) if with_bias else None
+    P = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None
+    S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = capi.lib().flhip_matmul(P(Ad), P(Bd), P(Cd), M, N, K, int(ta), int(tb), P(bd), capi.F32, S)
+    assert rc == 0
+    assert rel_l2(host(Cd), want) <= 1e-5
+
+
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("classes,cols", [(10, 64), (1000, 7), (1, 5), (65, 3)])
 def test_logsoftmax(classes, cols, dtype):
