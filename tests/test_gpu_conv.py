@@ -167,6 +167,41 @@ def test_forward_and_backward_data_without_workspace(shape):
     assert torch.equal(y0, y) and torch.equal(dx0, dx)
 
 
+def _random_cases(n, seed):
+    """Seeded random geometries biased towards the conditions the kernel families key on:
+    1x1 and 3x3 windows, even / odd rows, planes of 4k positions, channel counts around the
+    multiples of 8 / 32 / 64, strides, more than 64 filters."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < n:
+        k = int(rng.choice([1, 1, 3, 3, 3, 5]))
+        kh, kwd = (k, k) if rng.random() < 0.8 else (1, int(rng.choice([3, 7, 21])))
+        s_ = int(rng.choice([1, 1, 1, 2]))
+        g = int(rng.choice([1, 1, 1, 2]))
+        cin = int(rng.choice([8, 16, 24, 32, 40, 64, 72, 96, 130])) * g
+        cout = int(rng.choice([8, 24, 32, 64, 72, 96, 136, 200])) * g
+        H, W = int(rng.integers(4, 17)), int(rng.choice([6, 7, 8, 10, 12, 14, 16, 18, 20, 28]))
+        if kh == 1 and kwd > 1:
+            H = int(rng.integers(1, 4)); W = int(rng.integers(30, 90))
+        ph = kh // 2 if rng.random() < 0.8 else 0
+        pw = kwd // 2 if rng.random() < 0.8 else 0
+        N = int(rng.integers(1, 5))
+        if H + 2 * ph < kh or W + 2 * pw < kwd:
+            continue
+        if N * cin * H * W * cout // g * kh * kwd > 6e8:     # keep the CPU oracle quick
+            continue
+        out.append(((N, cin, H, W), (cout, cin // g, kh, kwd), (s_, s_), (ph, pw), (1, 1), g))
+    return out
+
+
+@pytest.mark.parametrize("case", _random_cases(40, 20251125))
+def test_random_geometries(case):
+    for dtype, tol, tight_w in ((torch.float32, F32_TOL, 1e-4), (torch.bfloat16, BF16_TOL, 1e-4)):
+        for name, (got, ref) in _run(case, 3, dtype).items():
+            lim = tol if dtype == torch.float32 else (tight_w if name in ("dw", "db") else 4e-3)
+            assert rel_l2(got, ref) <= lim, (case, dtype, name, rel_l2(got, ref))
+
+
 def test_invalid_arguments_raise():
     x = torch.zeros((1, 4, 8, 8), device="cuda")
     w = torch.zeros((4, 3, 3, 3), device="cuda")
