@@ -966,7 +966,8 @@ extern "C" int flhip_rnn_bwd(const flhip_rnn_desc* d, const void* x, const void*
     }
     if (l > 0) {
       // the gradient of this layer's input is the gradient of the output of the layer below
-      if (const int rc = flhip_copy_bytes(ginbuf, goutbuf, TB * inl * sizeof(float), stream)) return rc;
+      hipLaunchKernelGGL(rnn_add2_kernel, dim3(nblocks(TB * inl)), dim3(256), 0, s, ginbuf, (const float*)nullptr, 0,
+                         goutbuf, TB * inl);
       gout = goutbuf;
     }
   }

@@ -30,6 +30,8 @@ MODES = [flref.RNN_RELU, flref.RNN_TANH, flref.RNN_LSTM, flref.RNN_GRU]
     (12, 128, 1, False, 7, 64, False),
     (9, 160, 2, True, 6, 1, True),
     (12, 32, 1, True, 4, 65, True),
+    (5, 7, 2, False, 3, 1, True),          # stacked, layer activations of 21 floats (no 16-byte multiple)
+    (3, 5, 3, True, 3, 1, False),
 ])
 def test_rnn_forward_backward(mode, I, H, L, bidir, T, B, states):
     rng = np.random.default_rng(1000 * mode + I + H + L + T)
