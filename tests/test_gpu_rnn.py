@@ -64,6 +64,24 @@ def test_rnn_forward_backward(mode, I, H, L, bidir, T, B, states):
         assert rel_l2(host(dcx), rdcx) <= 2e-4
 
 
+def _random_configs(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(n):
+        out.append((int(rng.integers(0, 4)), int(rng.integers(1, 70)),
+                    int(rng.choice([16, 32, 48, 64, 80, 96, 128, 20, 7])), int(rng.integers(1, 4)),
+                    bool(rng.integers(0, 2)), int(rng.integers(1, 9)),
+                    int(rng.choice([1, 2, 5, 16, 17, 31, 32, 33, 48, 64, 65, 70])), bool(rng.integers(0, 2))))
+    return out
+
+
+@pytest.mark.parametrize("mode,I,H,L,bidir,T,B,states", _random_configs(30, 11))
+def test_random_configurations(mode, I, H, L, bidir, T, B, states):
+    """Seeded random sizes around the conditions of the fused step kernels (hidden sizes that
+    are / are not multiples of 16, batches around the 16-column tiles and the limit of 64)."""
+    test_rnn_forward_backward(mode, I, H, L, bidir, T, B, states)
+
+
 @pytest.mark.parametrize("mode", [flref.RNN_LSTM, flref.RNN_GRU])
 def test_missing_output_gradients_are_zero(mode):
     # only y was differentiated: the closure hands empty dhy / dcy (Functions.cpp:1677-1699)
