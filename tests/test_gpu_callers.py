@@ -24,11 +24,12 @@ def _round(a, dtype):
 
 
 @pytest.mark.parametrize("dtype", DT)
-def test_relu(dtype):
+@pytest.mark.parametrize("n", [5000, 4, 5, 7, 4099, 1 << 20])
+def test_relu(dtype, n):
     rng = np.random.default_rng(60)
-    x = _round(rng.standard_normal(5000).astype(np.float32), dtype)
+    x = _round(rng.standard_normal(n).astype(np.float32), dtype)
     x[:4] = [0.0, -0.0, np.inf, -np.inf]
-    dy = _round(rng.standard_normal(5000).astype(np.float32), dtype)
+    dy = _round(rng.standard_normal(n).astype(np.float32), dtype)
     assert np.array_equal(host(ops.relu(dev(x, dtype))), flref.relu_fwd(x))
     assert np.array_equal(host(ops.relu_backward(dev(dy, dtype), dev(x, dtype))), flref.relu_bwd(dy, x))
 
