@@ -960,7 +960,7 @@ int main() {
   std::printf(g_fail ? "%d check(s) FAILED\n" : "all host extension checks passed\n", g_fail);
   // leave without running static destructors: the order in which the HIP runtime, the
   // OpenMP runtime of the CPU checker and this program's own statics go down at exit is
-  // not under this program's control, and a crash there would lose the verdict above
+  // not under this program's control, and a crash there would lose the result printed above
   std::fflush(stdout);
   _exit(g_fail ? 1 : 0);
 }
