@@ -22,6 +22,12 @@
  *   batchnorm train / infer / backward: the closed forms of the reference's
  *     tests (AutogradNormalizationTest.cpp:37-226), invariants sum(dx) == 0 and
  *     sum(dx*xhat) == 0, finite differences, library routines.
+ *   caller closures (relu, matmul / linear, sum over columns, logSoftmax,
+ *     categoricalCrossEntropy, the LayerNorm affine part): float64 numpy
+ *     definitions and torch.nn.functional with its autograd.
+ *   rnn / rnnBackward: torch.nn.RNN / LSTM / GRU in float64 (same gate formulas and
+ *     weight order as cuDNN), forward and autograd, stacked and bidirectional, and
+ *     the parameter counts of the reference's test (AutogradRnnTest.cpp:37-49).
  * Not pinned by anything the reference holds ("parity unpinned" there, fixed
  * here by the definition above and checked against oneDNN through PyTorch):
  * the max-pool tie order and the running-statistics update for momentum != 0.
