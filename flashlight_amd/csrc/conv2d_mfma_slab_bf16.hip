@@ -515,9 +515,12 @@ void layout(Slab16Params* p, int R) {
 
 bool plan(Slab16Params* p, size_t* shmem) {
   if (p->KHW > KHW_MAX) return false;
-  // rows are read 16 bytes at a time from 4-byte aligned addresses (the last unit of a row
-  // may run into the next row or past the tensor: masked / out of range)
-  if (p->SW % 2 != 0) return false;
+  // rows are read 16 bytes at a time from addresses that are only 2- or 4-byte aligned when
+  // the row length is not a multiple of 8 (buffer loads take any alignment in the unaligned
+  // access mode the compute queues run in); the last unit of a row may run into the next
+  // row or past the tensor: masked / out of range.  1x1 windows over odd rows are left to
+  // the GEMM kernels.
+  if (p->SW % 2 != 0 && p->KHW == 1) return false;
   const int max_pos = 2 * NT_MAX * 16;
   if (p->DW > max_pos) return false;
   const int cus = mfma_num_cus();
@@ -548,11 +551,50 @@ bool plan(Slab16Params* p, size_t* shmem) {
     const int npos = best_r * p->DW, sp = ((npos + 3) & ~3) + 4;
     p->stage_ok = p->DW % 4 == 0 && (size_t)32 * sp * sizeof(float) <= *shmem - BM * sizeof(float);
   }
-  return best_r * p->DW >= 64;
+  // (a whole 7x7 plane, 49 positions, is worth it for a window with several taps)
+  return best_r * p->DW >= (p->KHW > 1 ? 48 : 64);
+}
+
+// Rows of odd length: a 16-byte read may start 2 bytes off a dword boundary, and the one
+// whose window straddles the end of the source tensor loses the tensor's last element to
+// the range check (which works on whole dwords; widening the range would read past the
+// caller's buffer).  The main kernel therefore sees that one element as zero, and this
+// kernel, launched behind it on the same stream, adds the element's term to the few
+// results of the last image that contain it: one thread per result of the box rows
+// [r0, r0+nr) x columns [c0, c0+nc) x the channels of the last group (those results are
+// rounded to bf16 twice).
+template <bool BWD>
+__global__ void __launch_bounds__(256)
+slab16_tail_fix(ConvGeom g, const bf16_t* __restrict__ src, const bf16_t* __restrict__ w,
+                bf16_t* __restrict__ dst, int r0, int nr, int c0, int nc) {
+  const int nch = BWD ? g.Cg : g.Kg;
+  const int idx = blockIdx.x * 256 + threadIdx.x;
+  if (idx >= nch * nr * nc) return;
+  const int col = c0 + idx % nc, row = r0 + (idx / nc) % nr, chl = idx / (nc * nr);
+  const int n = g.N - 1, grp = g.groups - 1, khw = g.KH * g.KW;
+  // the tap through which this result sees the last source element
+  const int th = BWD ? row + g.py - (g.OH - 1) : g.H - 1 - row + g.py;
+  const int tw = BWD ? col + g.px - (g.OW - 1) : g.W - 1 - col + g.px;
+  if (th < 0 || tw < 0 || th % g.dly != 0 || tw % g.dlx != 0) return;
+  const int kh = th / g.dly, kw = tw / g.dlx;
+  if (kh >= g.KH || kw >= g.KW) return;
+  const size_t nsrc = BWD ? (size_t)g.N * g.K * g.OH * g.OW : (size_t)g.N * g.C * g.H * g.W;
+  const float last = ld(src, nsrc - 1);
+  size_t o;
+  float wv;
+  if (!BWD) {
+    const int k = grp * g.Kg + chl;
+    wv = ld(w, ((size_t)k * g.Cg + (g.Cg - 1)) * khw + kh * g.KW + kw);
+    o = (((size_t)n * g.K + k) * g.OH + row) * g.OW + col;
+  } else {
+    wv = ld(w, ((size_t)(g.K - 1) * g.Cg + chl) * khw + kh * g.KW + kw);
+    o = (((size_t)n * g.C + grp * g.Cg + chl) * g.H + row) * g.W + col;
+  }
+  st(dst, o, ld(dst, o) + last * wv);
 }
 
 template <bool BWD>
-int launch(Slab16Params& p, const void* src, const void* wgt, const float* bias, void* dst,
+int launch(const ConvGeom& g, Slab16Params& p, const void* src, const void* wgt, const float* bias, void* dst,
            hipStream_t s) {
   const long long sbytes = (long long)p.N * p.SC * p.SH * p.SW * 2;
   const long long wbytes = (long long)p.groups * p.w_group_stride * 2;
@@ -574,6 +616,23 @@ int launch(Slab16Params& p, const void* src, const void* wgt, const float* bias,
   const dim3 grid((unsigned)(p.N * p.tiles_per_image), (unsigned)(p.mtiles * p.groups));
   hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const bf16_t*>(src),
                      static_cast<const bf16_t*>(wgt), bias, static_cast<bf16_t*>(dst));
+  if (p.SW & 1) {
+    // results of the last image whose window reaches the last source element (stride 1)
+    int r0, r1, c0, c1;
+    if (!BWD) {
+      r0 = std::max(0, g.H - 1 + g.py - (g.KH - 1) * g.dly); r1 = std::min(g.OH - 1, g.H - 1 + g.py);
+      c0 = std::max(0, g.W - 1 + g.px - (g.KW - 1) * g.dlx); c1 = std::min(g.OW - 1, g.W - 1 + g.px);
+    } else {
+      r0 = std::max(0, g.OH - 1 - g.py); r1 = std::min(g.H - 1, g.OH - 1 - g.py + (g.KH - 1) * g.dly);
+      c0 = std::max(0, g.OW - 1 - g.px); c1 = std::min(g.W - 1, g.OW - 1 - g.px + (g.KW - 1) * g.dlx);
+    }
+    if (r1 >= r0 && c1 >= c0) {
+      const int nr = r1 - r0 + 1, nc = c1 - c0 + 1, total = (BWD ? g.Cg : g.Kg) * nr * nc;
+      hipLaunchKernelGGL((slab16_tail_fix<BWD>), dim3((total + 255) / 256), dim3(256), 0, s, g,
+                         static_cast<const bf16_t*>(src), static_cast<const bf16_t*>(wgt),
+                         static_cast<bf16_t*>(dst), r0, nr, c0, nc);
+    }
+  }
   return check_launch("conv2d (bf16 mfma slab)");
 }
 
@@ -604,7 +663,7 @@ int mfma_slab16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const 
   if (g.sy != 1 || g.sx != 1) return -1;
   Slab16Params p{};
   fill_fwd(g, &p);
-  return launch<false>(p, x, w, bias, y, s);
+  return launch<false>(g, p, x, w, bias, y, s);
 }
 
 int mfma_slab16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx,
@@ -612,7 +671,7 @@ int mfma_slab16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, 
   if (g.sy != 1 || g.sx != 1) return -1;
   Slab16Params p{};
   fill_bwd(g, &p);
-  return launch<true>(p, dy, w, nullptr, dx, s);
+  return launch<true>(g, p, dy, w, nullptr, dx, s);
 }
 
 }  // namespace flhip
