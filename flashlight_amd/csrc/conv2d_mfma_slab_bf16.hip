@@ -56,6 +56,7 @@ struct Slab16Params {
   int sh0, sw0;          // window shift of tap (0,0): fwd -py,-px ; bwd +py,+px
   int shs, sws;          // shift step per kh / kw: fwd +dly,+dlx ; bwd -dly,-dlx
   int min_sh, min_sw;    // smallest shifts (slab origin relative to the result origin)
+  int psh, psw;          // source step per result row / column (forward: the stride; backward-data: 1)
   int groups, SCg, DCg;
   int a_mstride, a_cstride, w_group_stride;
   int R, RS;             // result rows per tile, slab rows
@@ -145,7 +146,7 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
         const int t = u >> 4;
         const int q = t % qrow, rh = t / qrow;
         const int rs = rh * 4 + rl;
-        const int sr = r0 + p.min_sh + rs;
+        const int sr = r0 * p.psh + p.min_sh + rs;
         xc[i] = cg * 8;
         xn[i] = min(8, p.SW - 8 * q);
         if (rs < p.RS) {
@@ -356,7 +357,7 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
       if (pos >= npos) pos = 0;                  // padding lanes compute a discarded column
       int w;
       const int r = fast_div(pos, p.DW, inv_dw, &w);
-      bp[j] = (lds_cell)Xs + (fk * p.XPL + r * p.WSP + w + p.XOFF + first);
+      bp[j] = (lds_cell)Xs + (fk * p.XPL + r * p.psh * p.WSP + w * p.psw + p.XOFF + first);
     }
     lds_cell ap = (lds_cell)As + (fk * p.APL + (wm * 32 + fr) * p.KHW);
 
@@ -500,9 +501,9 @@ inline int round_to_residue(int v, int r, int m) { return v + ((r - v) % m + m) 
 
 void layout(Slab16Params* p, int R) {
   p->R = R;
-  p->RS = R + (p->KH - 1) * p->dly;
+  p->RS = (R - 1) * p->psh + (p->KH - 1) * p->dly + 1;
   p->XOFF = std::max(0, -p->min_sw);
-  const int max_sc = p->min_sw + p->DW - 1 + (p->KW - 1) * p->dlx;   // last source column read
+  const int max_sc = p->min_sw + (p->DW - 1) * p->psw + (p->KW - 1) * p->dlx;   // last source column read
   // a row is stored in units of 8 columns: room for the last, possibly partial one
   p->WSP = round_to_residue(p->XOFF + std::max(max_sc + 1, (p->SW + 7) / 8 * 8), 4, 16);
   p->XPL = round_to_residue(p->RS * p->WSP, 1, 16);
@@ -573,8 +574,8 @@ slab16_tail_fix(ConvGeom g, const bf16_t* __restrict__ src, const bf16_t* __rest
   const int col = c0 + idx % nc, row = r0 + (idx / nc) % nr, chl = idx / (nc * nr);
   const int n = g.N - 1, grp = g.groups - 1, khw = g.KH * g.KW;
   // the tap through which this result sees the last source element
-  const int th = BWD ? row + g.py - (g.OH - 1) : g.H - 1 - row + g.py;
-  const int tw = BWD ? col + g.px - (g.OW - 1) : g.W - 1 - col + g.px;
+  const int th = BWD ? row + g.py - (g.OH - 1) : g.H - 1 - row * g.sy + g.py;
+  const int tw = BWD ? col + g.px - (g.OW - 1) : g.W - 1 - col * g.sx + g.px;
   if (th < 0 || tw < 0 || th % g.dly != 0 || tw % g.dlx != 0) return;
   const int kh = th / g.dly, kw = tw / g.dlx;
   if (kh >= g.KH || kw >= g.KW) return;
@@ -617,11 +618,11 @@ int launch(const ConvGeom& g, Slab16Params& p, const void* src, const void* wgt,
   hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const bf16_t*>(src),
                      static_cast<const bf16_t*>(wgt), bias, static_cast<bf16_t*>(dst));
   if (p.SW & 1) {
-    // results of the last image whose window reaches the last source element (stride 1)
+    // results of the last image whose window reaches the last source element
     int r0, r1, c0, c1;
     if (!BWD) {
-      r0 = std::max(0, g.H - 1 + g.py - (g.KH - 1) * g.dly); r1 = std::min(g.OH - 1, g.H - 1 + g.py);
-      c0 = std::max(0, g.W - 1 + g.px - (g.KW - 1) * g.dlx); c1 = std::min(g.OW - 1, g.W - 1 + g.px);
+      r0 = (std::max(0, g.H - 1 + g.py - (g.KH - 1) * g.dly) + g.sy - 1) / g.sy; r1 = std::min(g.OH - 1, (g.H - 1 + g.py) / g.sy);
+      c0 = (std::max(0, g.W - 1 + g.px - (g.KW - 1) * g.dlx) + g.sx - 1) / g.sx; c1 = std::min(g.OW - 1, (g.W - 1 + g.px) / g.sx);
     } else {
       r0 = std::max(0, g.OH - 1 - g.py); r1 = std::min(g.H - 1, g.OH - 1 - g.py + (g.KH - 1) * g.dly);
       c0 = std::max(0, g.OW - 1 - g.px); c1 = std::min(g.W - 1, g.OW - 1 - g.px + (g.KW - 1) * g.dlx);
@@ -641,6 +642,7 @@ void fill_fwd(const ConvGeom& g, Slab16Params* p) {
   p->KH = g.KH; p->KW = g.KW; p->KHW = g.KH * g.KW; p->dly = g.dly; p->dlx = g.dlx;
   p->sh0 = -g.py; p->sw0 = -g.px; p->shs = g.dly; p->sws = g.dlx;
   p->min_sh = -g.py; p->min_sw = -g.px;
+  p->psh = g.sy; p->psw = g.sx;
   p->groups = g.groups; p->SCg = g.Cg; p->DCg = g.Kg;
   p->a_mstride = g.Cg * p->KHW; p->a_cstride = p->KHW; p->w_group_stride = g.Kg * g.Cg * p->KHW;
   p->mtiles = (g.Kg + BM - 1) / BM;
@@ -651,6 +653,7 @@ void fill_bwd(const ConvGeom& g, Slab16Params* p) {
   p->KH = g.KH; p->KW = g.KW; p->KHW = g.KH * g.KW; p->dly = g.dly; p->dlx = g.dlx;
   p->sh0 = g.py; p->sw0 = g.px; p->shs = -g.dly; p->sws = -g.dlx;
   p->min_sh = g.py - (g.KH - 1) * g.dly; p->min_sw = g.px - (g.KW - 1) * g.dlx;
+  p->psh = 1; p->psw = 1;
   p->groups = g.groups; p->SCg = g.Kg; p->DCg = g.Cg;
   p->a_mstride = p->KHW; p->a_cstride = g.Cg * p->KHW; p->w_group_stride = g.Kg * g.Cg * p->KHW;
   p->mtiles = (g.Cg + BM - 1) / BM;
@@ -660,7 +663,8 @@ void fill_bwd(const ConvGeom& g, Slab16Params* p) {
 
 int mfma_slab16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
                          hipStream_t s) {
-  if (g.sy != 1 || g.sx != 1) return -1;
+  // strides: results step through the slab; 1x1 windows with a stride are left to the GEMM kernels
+  if ((g.sy != 1 || g.sx != 1) && g.KH * g.KW == 1) return -1;
   Slab16Params p{};
   fill_fwd(g, &p);
   return launch<false>(g, p, x, w, bias, y, s);
