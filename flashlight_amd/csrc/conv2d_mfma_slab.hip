@@ -57,6 +57,7 @@ struct SlabParams {
   int sh0, sw0;          // window shift of tap (0,0): fwd -py,-px ; bwd +py,+px
   int shs, sws;          // shift step per kh / kw: fwd +dly,+dlx ; bwd -dly,-dlx
   int min_sh, min_sw;    // smallest shifts (slab origin relative to the result origin)
+  int psh, psw;          // source step per result row / column (forward: the stride; backward-data: 1)
   int groups, SCg, DCg;
   int a_mstride, a_cstride, w_group_stride;
   int R, RS;             // result rows per tile, slab rows
@@ -152,7 +153,7 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
           int rem, q;
           const int cp = fast_div(u, per_pair, inv_pp, &rem);
           const int rs = fast_div(rem, qrow, inv_q, &q);
-          const int sr = r0 + p.min_sh + rs;
+          const int sr = r0 * p.psh + p.min_sh + rs;
           xl[i] = cp * XPW + (rs * p.WSP + p.XOFF + 4 * q) * 2;
           if ((unsigned)sr < (unsigned)p.SH)
             xg[i] = (img_base + (2 * cp * p.SH + sr) * p.SW + 4 * q) * esz;
@@ -247,7 +248,7 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
           int q, sc;
           const int c = fast_div(e, per_chan, inv_pc, &q);
           const int rs = fast_div(q, p.SW, inv_sw, &sc);
-          const int sr = r0 + p.min_sh + rs;
+          const int sr = r0 * p.psh + p.min_sh + rs;
           xl[i] = (c >> 1) * XPW + (rs * p.WSP + p.XOFF + sc) * 2 + (c & 1);
           if ((unsigned)sr < (unsigned)p.SH) xg[i] = (img_base + (c * p.SH + sr) * p.SW + sc) * esz;
           if (c < tail) xlive |= 1u << i;
@@ -361,7 +362,7 @@ slab_conv_kernel(SlabParams p, const T* __restrict__ src, const T* __restrict__ 
       int w;
       const int r = fast_div(pos, p.DW, inv_dw, &w);
       bp[j] = (lds_f2)(reinterpret_cast<const float2*>(Xs)) +
-              (fk * p.XPH + r * p.WSP + w + p.XOFF + first);
+              (fk * p.XPH + r * p.psh * p.WSP + w * p.psw + p.XOFF + first);
     }
     // weights of this lane: rows wm*32 + fr (+16), channels 2*fk and 2*fk+1
     lds_f1 a1 = (lds_f1)As + ((wm * 32 + fr) * p.APW + 2 * fk * p.KHW);       // forward
@@ -530,9 +531,9 @@ inline int round_to_residue(int v, int r, int m) { return v + ((r - v) % m + m) 
 // LDS layout of a tile of R result rows.
 void layout(SlabParams* p, int R, bool bwd) {
   p->R = R;
-  p->RS = R + (p->KH - 1) * p->dly;
+  p->RS = (R - 1) * p->psh + (p->KH - 1) * p->dly + 1;
   p->XOFF = (std::max(0, -p->min_sw) + 3) & ~3;
-  const int max_sc = p->min_sw + p->DW - 1 + (p->KW - 1) * p->dlx;   // last source column read
+  const int max_sc = p->min_sw + (p->DW - 1) * p->psw + (p->KW - 1) * p->dlx;   // last source column read
   p->WSP = (p->XOFF + std::max(max_sc + 1, p->SW) + 3) & ~3;
   // pair-plane pitch = 16 (mod 32) positions: the four k-indices of a fragment read
   // start 32 banks apart
@@ -621,12 +622,14 @@ int launch(SlabParams& p, const void* src, const void* wgt, const float* bias, v
 
 int mfma_slab_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w,
                        const float* bias, void* y, hipStream_t s) {
-  if (g.sy != 1 || g.sx != 1) return -1;
+  // strides: results step through the slab; 1x1 windows with a stride are left to the GEMM kernels
+  if ((g.sy != 1 || g.sx != 1) && g.KH * g.KW == 1) return -1;
   SlabParams p{};
   p.N = g.N; p.SC = g.C; p.SH = g.H; p.SW = g.W; p.DC = g.K; p.DH = g.OH; p.DW = g.OW;
   p.KH = g.KH; p.KW = g.KW; p.KHW = g.KH * g.KW; p.dly = g.dly; p.dlx = g.dlx;
   p.sh0 = -g.py; p.sw0 = -g.px; p.shs = g.dly; p.sws = g.dlx;
   p.min_sh = -g.py; p.min_sw = -g.px;
+  p.psh = g.sy; p.psw = g.sx;
   p.groups = g.groups; p.SCg = g.Cg; p.DCg = g.Kg;
   p.a_mstride = g.Cg * p.KHW; p.a_cstride = p.KHW; p.w_group_stride = g.Kg * g.Cg * p.KHW;
   p.mtiles = (g.Kg + BM - 1) / BM;
@@ -642,6 +645,7 @@ int mfma_slab_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const 
   p.KH = g.KH; p.KW = g.KW; p.KHW = g.KH * g.KW; p.dly = g.dly; p.dlx = g.dlx;
   p.sh0 = g.py; p.sw0 = g.px; p.shs = -g.dly; p.sws = -g.dlx;
   p.min_sh = g.py - (g.KH - 1) * g.dly; p.min_sw = g.px - (g.KW - 1) * g.dlx;
+  p.psh = 1; p.psw = 1;
   p.groups = g.groups; p.SCg = g.Kg; p.DCg = g.Cg;
   p.a_mstride = p.KHW; p.a_cstride = g.Cg * p.KHW; p.w_group_stride = g.Kg * g.Cg * p.KHW;
   p.mtiles = (g.Cg + BM - 1) / BM;
