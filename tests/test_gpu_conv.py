@@ -56,6 +56,12 @@ MORE = [
     ((3, 40, 6, 6), (72, 40, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     ((2, 72, 10, 14), (24, 72, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     ((5, 136, 14, 14), (200, 136, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    # strided forward through the slab kernels (results step through the slab): with dilation,
+    # different strides per axis, groups, odd rows (bf16: the tensor's last element is patched in)
+    ((2, 32, 13, 17), (40, 32, 3, 3), (2, 2), (2, 2), (2, 2), 1),
+    ((3, 64, 16, 16), (64, 64, 3, 3), (2, 1), (1, 1), (1, 2), 1),
+    ((2, 64, 15, 21), (96, 32, 3, 3), (3, 2), (1, 1), (1, 1), 2),
+    ((4, 64, 11, 11), (64, 64, 3, 3), (2, 2), (1, 1), (1, 1), 1),
     # bias gradient with more than one tile of 64 filters (each tile writes only its own sums)
     ((2, 32, 8, 16), (136, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),
     ((2, 64, 20, 20), (160, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
