@@ -13,8 +13,11 @@
 // contracts over m and gathers like the source.  Positions are the rows of the
 // instruction tile, so a lane ends up with four consecutive positions of one result
 // channel: one 8-byte store.  Positions are flattened over the batch (a plane of 14x14
-// would waste a quarter of a 128-wide tile per image); planes must be a multiple of 4
-// positions so that a 4-position run stays inside one image and is 8-byte aligned.
+// would waste a quarter of a 128-wide tile per image).  When a plane is not a multiple
+// of 4 positions (7x7) a 4-position run starts at any even byte and may begin in one
+// image and end in the next: the ODD variants load such a run as the last four positions
+// of the first image and the first four of the second and shift the two together, and
+// store it element by element.
 //
 //   filter gradient  dw[m][c] = sum_{n,q} dy[m][q] x[c][q]   (+ db[m] = sum dy)
 // contracts over positions, contiguous in both operands: both tiles are read from LDS
@@ -56,10 +59,30 @@ __device__ __forceinline__ bf16x8 gather8(const uint16_t* tile, int pitch, int r
   return as_bf16x8(a, b, c, d);
 }
 
+// 8 bytes at any 2-byte boundary
+__device__ __forceinline__ uintx2_t load8_any(const bf16_t* p) {
+  uintx2_t v;
+  __builtin_memcpy(&v, p, 8);
+  return v;
+}
+__device__ __forceinline__ void store8_any(bf16_t* p, uintx2_t v) { __builtin_memcpy(p, &v, 8); }
+// a: the last four positions of an image's row, b: the first four of the next image's;
+// result: the last rem (1..3) of a followed by the first 4 - rem of b
+__device__ __forceinline__ uintx2_t merge_runs(uintx2_t a, uintx2_t b, int rem) {
+  const uint64_t A = ((uint64_t)a.y << 32) | a.x, B = ((uint64_t)b.y << 32) | b.x;
+  const uint64_t v = (A >> (16 * (4 - rem))) | (B << (16 * rem));
+  return uintx2_t{(uint32_t)v, (uint32_t)(v >> 32)};
+}
+
 // BWD = false: forward (weights [Mo][Kc]); true: backward-data (weights [Kc][Mo]).
 // MT = 16-channel result tiles per workgroup (4: 64 result channels; 8 was measured and
 // is slower on every ResNet-50 layer, as is loading two chunks ahead instead of one).
-template <bool BWD, int MT>
+// ODD: planes that are not a multiple of 4 positions (at least 4).
+// PF = chunks whose global loads are in flight while one is multiplied: 1 when the grid
+// fills the chip several times over (other workgroups hide the latency), 4 for small grids
+// with long contractions (7x7 planes: about 100 workgroups of up to 64 chunks each, one
+// wave per SIMD), where a chunk otherwise costs one trip to memory.
+template <bool BWD, int MT, bool ODD, int PF>
 __global__ void __launch_bounds__(256)
 pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __restrict__ wgt,
                  const float* __restrict__ bias, bf16_t* __restrict__ dst) {
@@ -84,9 +107,18 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
   const int q = q0 + lq;
   const bool qv = q < p.Ptot;
   const int img = qv ? q / p.P : 0, pos = qv ? q - img * p.P : 0;
-  const bf16_t* sp = src + (size_t)img * p.Kc * p.P + pos;
+  // ODD: a run with fewer than 4 positions left in its image continues in the next one
+  const int rem = p.P - pos;
+  const bool cross = ODD && qv && rem < 4, nextv = cross && q + rem < p.Ptot;
+  const bf16_t* sp = src + (size_t)img * p.Kc * p.P + (cross ? p.P - 4 : pos);
+  const bf16_t* sp2 = nextv ? src + (size_t)(img + 1) * p.Kc * p.P : sp;
+  // LATE: every load issues, from an address inside its tensor, and what lies outside the
+  // tile is zeroed when the registers go to LDS (nothing between a load and the next one
+  // depends on loaded data)
+  constexpr bool LATE = ODD || PF > 1;
   struct Stage {
     uintx2_t x[4];
+    uintx2_t xb[ODD ? 4 : 1];   // ODD: the same rows of the next image
     uintx4_t w[WQ];
   };
   // weights: forward rows m = tid / 4 (+ 64), 8 contraction elements (tid % 4) * 8;
@@ -97,19 +129,27 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int k = k0 + lr + 8 * i;
-      st.x[i] = (qv && k < p.Kc) ? *reinterpret_cast<const uintx2_t*>(sp + (size_t)k * p.P) : uintx2_t{0u, 0u};
+      // LATE: row clamped into the tensor (no branch, no select on the way to the load)
+      const uint32_t off = (uint32_t)min(k, p.Kc - 1) * (uint32_t)p.P;
+      if (ODD) {
+        st.x[i] = load8_any(sp + off);
+        st.xb[i] = load8_any(sp2 + off);
+      } else if (LATE) {
+        st.x[i] = *reinterpret_cast<const uintx2_t*>(sp + off);
+      } else {
+        st.x[i] = (qv && k < p.Kc) ? *reinterpret_cast<const uintx2_t*>(sp + (size_t)k * p.P) : uintx2_t{0u, 0u};
+      }
     }
 #pragma unroll
     for (int h = 0; h < WQ; ++h) {
-      if (BWD) {
-        const int k = k0 + wr, m = m0 + wc + 64 * h;
-        st.w[h] = (k < p.Kc && m < p.Mo) ? *reinterpret_cast<const uintx4_t*>(wgt + (size_t)k * p.Mo + m)
-                                         : uintx4_t{0u, 0u, 0u, 0u};
-      } else {
-        const int m = m0 + wr + 64 * h, k = k0 + wc;
-        st.w[h] = (m < p.Mo && k < p.Kc) ? *reinterpret_cast<const uintx4_t*>(wgt + (size_t)m * p.Kc + k)
-                                         : uintx4_t{0u, 0u, 0u, 0u};
-      }
+      const int k = BWD ? k0 + wr : k0 + wc, m = BWD ? m0 + wc + 64 * h : m0 + wr + 64 * h;
+      const bool in = k < p.Kc && m < p.Mo;
+      const size_t off = BWD ? (size_t)k * p.Mo + m : (size_t)m * p.Kc + k;
+      // LATE: the 8-element piece clamped into the matrix (both dimensions are multiples of 8)
+      const uint32_t offc = BWD ? (uint32_t)min(k, p.Kc - 1) * (uint32_t)p.Mo + (uint32_t)min(m, p.Mo - 8)
+                                : (uint32_t)min(m, p.Mo - 1) * (uint32_t)p.Kc + (uint32_t)min(k, p.Kc - 8);
+      if (LATE) st.w[h] = *reinterpret_cast<const uintx4_t*>(wgt + offc);
+      else st.w[h] = in ? *reinterpret_cast<const uintx4_t*>(wgt + off) : uintx4_t{0u, 0u, 0u, 0u};
     }
   };
   // Weights live in LDS as [result channel m][contraction k], 8-element contraction groups
@@ -117,26 +157,38 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
   // holds eight result channels of one k per piece and scatters them (the swizzle spreads
   // those 16-bit stores over the banks).
   auto wslot = [](int m, int g) { return m * PB_WP + 8 * (g ^ ((m >> 3) & 3)); };
-  auto sstore = [&](int buf, const Stage& st) {
+  auto sstore = [&](int c, const Stage& st) {
+    const int buf = c & 1;
     uint16_t* X = Xs0 + buf * XSZ;
     uint16_t* Wt = Ws0 + buf * WSZ;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
+      uintx2_t v = st.x[i];
+      if (ODD) {   // no branch: every lane shifts, lanes whose run crosses keep the result
+        const uintx2_t mr = merge_runs(v, nextv ? st.xb[i] : uintx2_t{0u, 0u}, cross ? rem : 1);
+        v = cross ? mr : v;
+      }
+      if (LATE && !(qv && c * PB_KC + lr + 8 * i < p.Kc)) v = uintx2_t{0u, 0u};
       uint32_t* d = reinterpret_cast<uint32_t*>(&X[(lr + 8 * i) * PB_XP + lq]);
-      d[0] = st.x[i].x;
-      d[1] = st.x[i].y;
+      d[0] = v.x;
+      d[1] = v.y;
     }
 #pragma unroll
     for (int h = 0; h < WQ; ++h) {
+      uintx4_t wv = st.w[h];
+      if (LATE) {
+        const int k = BWD ? c * PB_KC + wr : c * PB_KC + wc, m = BWD ? m0 + wc + 64 * h : m0 + wr + 64 * h;
+        if (!(k < p.Kc && m < p.Mo)) wv = uintx4_t{0u, 0u, 0u, 0u};
+      }
       if (BWD) {
-        const uint32_t v[4] = {st.w[h].x, st.w[h].y, st.w[h].z, st.w[h].w};
+        const uint32_t v[4] = {wv.x, wv.y, wv.z, wv.w};
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int m = wc + 64 * h + e;
           Wt[wslot(m, wr >> 3) + (wr & 7)] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
         }
       } else {
-        *reinterpret_cast<uintx4_t*>(&Wt[wslot(wr + 64 * h, wc >> 3)]) = st.w[h];
+        *reinterpret_cast<uintx4_t*>(&Wt[wslot(wr + 64 * h, wc >> 3)]) = wv;
       }
     }
   };
@@ -162,15 +214,51 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
   };
 
   const int n = p.nchunks;
-  Stage st;
-  gload(0, st);
-  sstore(0, st);
-  __syncthreads();
-  for (int c = 0; c < n; ++c) {
-    if (c + 1 < n) gload(c + 1, st);
-    compute(c & 1);
-    if (c + 1 < n) sstore((c + 1) & 1, st);
+  if (PF == 1) {
+    Stage st;
+    gload(0, st);
+    sstore(0, st);
     __syncthreads();
+    for (int c = 0; c < n; ++c) {
+      if (c + 1 < n) gload(c + 1, st);
+      compute(c & 1);
+      if (c + 1 < n) sstore(c + 1, st);
+      __syncthreads();
+    }
+  } else {
+    // st[c % PF] holds chunk c from its load until it is copied to LDS one iteration
+    // before its product; then the register set takes chunk c + PF
+    Stage st[PF];
+#pragma unroll
+    for (int j = 0; j < PF; ++j)
+      if (j < n) gload(j, st[j]);
+    sstore(0, st[0]);
+    __syncthreads();
+    // while every chunk of a round has a successor PF on: no conditions, so the waits for
+    // a register set's loads can be counted exactly; then the last one or two rounds
+    int c0 = 0;
+    for (; c0 + 2 * PF <= n; c0 += PF) {
+#pragma unroll
+      for (int j = 0; j < PF; ++j) {
+        const int c = c0 + j;
+        gload(c + PF, st[j]);
+        compute(c & 1);
+        sstore(c + 1, st[(j + 1) % PF]);
+        __syncthreads();
+      }
+    }
+    for (; c0 < n; c0 += PF) {
+#pragma unroll
+      for (int j = 0; j < PF; ++j) {
+        const int c = c0 + j;
+        if (c < n) {
+          if (c + PF < n) gload(c + PF, st[j]);
+          compute(c & 1);
+          if (c + 1 < n) sstore(c + 1, st[(j + 1) % PF]);
+          __syncthreads();
+        }
+      }
+    }
   }
 
   // ---- results: a lane holds positions wave*32 + i*16 + 4*fg .. +3 of channel j*16 + fr.
@@ -189,7 +277,26 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
       *reinterpret_cast<uintx2_t*>(&Ys[ml * YP + wave * 32 + i * 16 + 4 * fg]) = o;
     }
   __syncthreads();
-  if ((p.P & 7) == 0) {
+  if (ODD) {
+    const int pc = (tid & 31) * 4, qo = q0 + pc;
+    if (qo < p.Ptot) {
+      const int im = qo / p.P, po = qo - im * p.P, left = p.P - po;
+      bf16_t* dp = dst + (size_t)im * p.Mo * p.P + po;
+      bf16_t* dp2 = dst + (size_t)(im + 1) * p.Mo * p.P - left;   // element e >= left: position e - left of the next image
+      for (int ml = tid >> 5; ml < BM && m0 + ml < p.Mo; ml += 8) {
+        const uintx2_t v = *reinterpret_cast<const uintx2_t*>(&Ys[ml * YP + pc]);
+        const size_t row = (size_t)(m0 + ml) * p.P;
+        if (left >= 4) {
+          store8_any(dp + row, v);
+        } else {
+          const uint32_t e4[4] = {v.x & 0xffffu, v.x >> 16, v.y & 0xffffu, v.y >> 16};
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (qo + e < p.Ptot) (e < left ? dp : dp2)[row + e] = (bf16_t)e4[e];
+        }
+      }
+    }
+  } else if ((p.P & 7) == 0) {
     const int pc = (tid & 15) * 8, qo = q0 + pc;
     if (qo < p.Ptot) {
       const int im = qo / p.P, po = qo - im * p.P;
@@ -210,7 +317,7 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
 
 bool pw16_applies(const ConvGeom& g) {
   return g.KH == 1 && g.KW == 1 && g.py == 0 && g.px == 0 && g.groups == 1 && g.sy == 1 && g.sx == 1 &&
-         g.OH == g.H && g.OW == g.W && (g.H * g.W) % 4 == 0 && g.C % 8 == 0 && g.K % 8 == 0;
+         g.OH == g.H && g.OW == g.W && g.H * g.W >= 4 && g.C % 8 == 0 && g.K % 8 == 0;
 }
 
 template <bool BWD>
@@ -227,9 +334,23 @@ int launch_pw16(const ConvGeom& g, const void* src, const void* w, const float* 
   p.mtiles = (p.Mo + 63) / 64;
   const long long grid = (long long)((p.ptiles + 7) / 8) * 8 * p.mtiles;
   if (grid > 0x7fffffffll) return -1;
-  hipLaunchKernelGGL((pw16_conv_kernel<BWD, 4>), dim3((unsigned)grid), dim3(256), 0, s, p,
-                     static_cast<const bf16_t*>(src), static_cast<const bf16_t*>(w), bias,
-                     static_cast<bf16_t*>(dst));
+  // deep prefetch for grids of at most one workgroup per CU with at least 8 chunks (measured
+  // on the ResNet-50 layers: 20 to 30 % faster there, slower on every larger grid);
+  // FLHIP_PW16_PF = 1 / 4 forces one or the other
+  bool deep = grid <= (long long)mfma_num_cus() && p.nchunks >= 8;
+  if (const char* e = getenv("FLHIP_PW16_PF")) deep = atoi(e) > 1;
+  const bool odd = p.P % 4 != 0;
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), 0, s, p, static_cast<const bf16_t*>(src),
+                       static_cast<const bf16_t*>(w), bias, static_cast<bf16_t*>(dst));
+  };
+  if (odd) {
+    if (deep) go(pw16_conv_kernel<BWD, 4, true, 4>);
+    else go(pw16_conv_kernel<BWD, 4, true, 1>);
+  } else {
+    if (deep) go(pw16_conv_kernel<BWD, 4, false, 4>);
+    else go(pw16_conv_kernel<BWD, 4, false, 1>);
+  }
   return check_launch(BWD ? "conv2d_bwd_data 1x1 (bf16 mfma)" : "conv2d_fwd 1x1 (bf16 mfma)");
 }
 
@@ -246,9 +367,11 @@ struct Pw16WgradParams {
 
 // grid (slice, channel-tile pair).  A workgroup owns dw[64 m][64 c] and one slice of the
 // positions of the whole batch; thread t loads 16 positions (four 8-byte runs, each inside
-// one image) of row t / 4 of both operands per chunk.  out: slice-major partial results
+// one image; ODD: planes not a multiple of 4 positions, where a run may end in the next
+// image) of row t / 4 of both operands per chunk.  out: slice-major partial results
 // [nsplit][E + Mo] (dw tile values, then the bias sums), or dw / db themselves when there
 // is one slice.
+template <bool ODD>
 __global__ void __launch_bounds__(256)
 pw16_wgrad_kernel(Pw16WgradParams p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy,
                   float* __restrict__ out, float* __restrict__ db_direct) {
@@ -283,8 +406,26 @@ pw16_wgrad_kernel(Pw16WgradParams p, const bf16_t* __restrict__ x, const bf16_t*
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       const bool in = od[g] < dlim;     // past the last image: nothing left
-      sd[g] = (in && mv) ? *reinterpret_cast<const uintx2_t*>(dy + od[g] + drow) : uintx2_t{0u, 0u};
-      sx[g] = (in && cv) ? *reinterpret_cast<const uintx2_t*>(x + ox[g] + xrow) : uintx2_t{0u, 0u};
+      if (ODD) {
+        // a run with fewer than 4 positions left in its image continues in the next one
+        // (if there is one); all loads issue, from addresses inside the tensors
+        const int rem = p.P - q[g];
+        const bool cross = rem < 4;
+        const int back = cross ? 4 - rem : 0;
+        const long long nd = od[g] - q[g] + (long long)p.Mo * p.P, nx = ox[g] - q[g] + (long long)p.C * p.P;
+        const bool nin = cross && nd < dlim;
+        uintx2_t a = load8_any(dy + ((in && mv) ? od[g] - back + drow : 0));
+        uintx2_t b = load8_any(dy + ((nin && mv) ? nd + drow : 0));
+        if (cross) a = merge_runs(a, nin ? b : uintx2_t{0u, 0u}, rem);
+        sd[g] = (in && mv) ? a : uintx2_t{0u, 0u};
+        a = load8_any(x + ((in && cv) ? ox[g] - back + xrow : 0));
+        b = load8_any(x + ((nin && cv) ? nx + xrow : 0));
+        if (cross) a = merge_runs(a, nin ? b : uintx2_t{0u, 0u}, rem);
+        sx[g] = (in && cv) ? a : uintx2_t{0u, 0u};
+      } else {
+        sd[g] = (in && mv) ? *reinterpret_cast<const uintx2_t*>(dy + od[g] + drow) : uintx2_t{0u, 0u};
+        sx[g] = (in && cv) ? *reinterpret_cast<const uintx2_t*>(x + ox[g] + xrow) : uintx2_t{0u, 0u};
+      }
       // next chunk: 64 positions on, possibly into the following images
       q[g] += PG_KC; od[g] += PG_KC; ox[g] += PG_KC;
       while (q[g] >= p.P) {
@@ -411,8 +552,13 @@ int mfma_pointwise16_wgrad(const ConvGeom& g, const void* x, const void* dy, flo
   const size_t need = p.nsplit > 1 ? (size_t)p.nsplit * ((size_t)p.E + p.Mo) * sizeof(float) : 0;
   if (need && (!ws || ws_bytes < need)) return fail(FLHIP_INVALID_ARGUMENT, "conv2d_bwd_filter: workspace too small");
   float* out = p.nsplit > 1 ? static_cast<float*>(ws) : dw;
-  hipLaunchKernelGGL(pw16_wgrad_kernel, dim3((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles)), dim3(256), 0, s, p,
-                     static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), out, db);
+  const dim3 grid((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles));
+  if (p.P % 4 == 0)
+    hipLaunchKernelGGL(pw16_wgrad_kernel<false>, grid, dim3(256), 0, s, p, static_cast<const bf16_t*>(x),
+                       static_cast<const bf16_t*>(dy), out, db);
+  else
+    hipLaunchKernelGGL(pw16_wgrad_kernel<true>, grid, dim3(256), 0, s, p, static_cast<const bf16_t*>(x),
+                       static_cast<const bf16_t*>(dy), out, db);
   if (p.nsplit > 1) wgrad_reduce_launch(static_cast<const float*>(ws), p.nsplit, p.E, p.Mo, p.want_db, dw, db, s);
   return check_launch("conv2d_bwd_filter 1x1 (bf16 mfma)");
 }

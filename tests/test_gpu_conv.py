@@ -56,6 +56,18 @@ MORE = [
     ((3, 40, 6, 6), (72, 40, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     ((2, 72, 10, 14), (24, 72, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     ((5, 136, 14, 14), (200, 136, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    # the same kernels over planes that are not a multiple of 4 positions: 4-position runs that
+    # start in one image and end in the next (or nowhere: the last image), planes of 5 and 6
+    ((5, 72, 7, 7), (40, 72, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((6, 136, 7, 7), (200, 136, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((1, 32, 7, 7), (64, 32, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((3, 64, 5, 9), (24, 64, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((7, 16, 1, 5), (16, 16, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((9, 24, 2, 3), (8, 24, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    # long contractions on small grids (several chunks in flight): 9 and 11 chunks of 32
+    ((3, 264, 7, 7), (72, 264, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((2, 40, 5, 5), (328, 40, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((2, 296, 6, 6), (344, 296, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     # strided forward through the slab kernels (results step through the slab): with dilation,
     # different strides per axis, groups, odd rows (bf16: the tensor's last element is patched in)
     ((2, 32, 13, 17), (40, 32, 3, 3), (2, 2), (2, 2), (2, 2), 1),
