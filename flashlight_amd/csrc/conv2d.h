@@ -38,11 +38,15 @@ int mfma_pointwise_conv_fwd(const ConvGeom& g, int dtype, const void* x, const v
                             const float* bias, void* y, hipStream_t s, int ksplit = 1);
 int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w,
                                  void* dx, hipStream_t s, const float* bias = nullptr, int ksplit = 1);
-// bf16 storage on the bf16 matrix cores: 1x1 stride-1 windows over planes that are a
-// multiple of 4 positions, channel counts multiples of 8; -1 otherwise
+// bf16 storage on the bf16 matrix cores: 1x1 windows without padding over planes of at
+// least 4 positions, channel counts multiples of 8; -1 otherwise.  Strided windows need
+// mfma_pointwise16_lattice_ws() bytes of workspace (the input's lattice points / the compact
+// gradient) and return -1 without it.
 int mfma_pointwise16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
-                              hipStream_t s);
-int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s);
+                              hipStream_t s, void* ws = nullptr, size_t ws_bytes = 0);
+int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s,
+                                   void* ws = nullptr, size_t ws_bytes = 0);
+size_t mfma_pointwise16_lattice_ws(const ConvGeom& g);
 size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g);
 int mfma_pointwise16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
                            size_t ws_bytes, hipStream_t s);

@@ -181,8 +181,12 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
   }
   // forward / backward-data: the kernels for windows with several taps read reordered
   // weights when the caller brings room for them (they run without it, slower)
-  if (pass == FLHIP_CONV_FWD) return mfma_tapped_ws(g, d->dtype, false);
-  if (pass == FLHIP_CONV_BWD_DATA) return mfma_tapped_ws(g, d->dtype, true);
+  // (bf16: strided 1x1 windows gather the input's lattice points / spread a compact gradient)
+  if (pass == FLHIP_CONV_FWD || pass == FLHIP_CONV_BWD_DATA) {
+    const size_t a = mfma_tapped_ws(g, d->dtype, pass == FLHIP_CONV_BWD_DATA);
+    const size_t b = d->dtype == FLHIP_BF16 ? mfma_pointwise16_lattice_ws(g) : 0;
+    return a > b ? a : b;
+  }
   return 0;
 }
 
@@ -197,7 +201,7 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
   if (!force_direct()) {
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
-      r = mfma_pointwise16_conv_fwd(g, x, w, bias, y, s);
+      r = mfma_pointwise16_conv_fwd(g, x, w, bias, y, s, ws, ws_bytes);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
       r = mfma_slab16_conv_fwd(g, x, w, bias, y, s);
     if (r < 0 && !skip("gemm1x1")) r = mfma_pointwise_conv_fwd(g, d->dtype, x, w, bias, y, s);
@@ -231,7 +235,7 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
   if (!force_direct()) {
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
-      r = mfma_pointwise16_conv_bwd_data(g, dy, w, dx, s);
+      r = mfma_pointwise16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
       r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s);
     if (r < 0 && !skip("gemm1x1")) r = mfma_pointwise_conv_bwd_data(g, d->dtype, dy, w, dx, s);

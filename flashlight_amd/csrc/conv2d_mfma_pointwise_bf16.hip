@@ -524,30 +524,135 @@ bool pw16_wgrad_plan(const ConvGeom& g, Pw16WgradParams* p) {
   return true;
 }
 
+// ---- strided 1x1 windows ---------------------------------------------------------------
+// A 1x1 window with strides reads the input on a lattice.  With room for the lattice
+// points as a tensor of their own ([N][C][OH][OW]) the three passes become the stride-1
+// passes above plus one copy: gather the lattice (forward, filter gradient) or spread the
+// compact gradient over a zeroed dx (backward-data).
+__global__ void __launch_bounds__(256)
+lattice_gather_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ xc, int H, int W, int OH, int OW,
+                      int sy, int sx, uint32_t total) {
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  if (i >= total) return;
+  const uint32_t ow = i % OW, t = i / OW, oh = t % OH, plane = t / OH;
+  xc[i] = x[((size_t)plane * H + (size_t)oh * sy) * W + (size_t)ow * sx];
+}
+
+// thread = VEC consecutive elements of a row of dx (W a multiple of VEC)
+template <int VEC>
+__global__ void __launch_bounds__(256)
+lattice_scatter_kernel(const bf16_t* __restrict__ dxc, bf16_t* __restrict__ dx, int H, int W, int OH, int OW,
+                       int sy, int sx, uint32_t total) {
+  const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+  if (i >= total) return;
+  const uint32_t per_row = W / VEC, w0 = (i % per_row) * VEC, t = i / per_row, h = t % H, plane = t / H;
+  const bool rowv = h % sy == 0;
+  const bf16_t* src = dxc + ((size_t)plane * OH + h / sy) * OW;
+  uint16_t v[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    const uint32_t w = w0 + e;
+    v[e] = (rowv && w % sx == 0) ? src[w / sx] : (uint16_t)0;
+  }
+  bf16_t* d = dx + ((size_t)plane * H + h) * W + w0;
+  if constexpr (VEC == 8) {
+    *reinterpret_cast<uintx4_t*>(d) = uintx4_t{v[0] | ((uint32_t)v[1] << 16), v[2] | ((uint32_t)v[3] << 16),
+                                               v[4] | ((uint32_t)v[5] << 16), v[6] | ((uint32_t)v[7] << 16)};
+  } else if constexpr (VEC == 4) {
+    *reinterpret_cast<uintx2_t*>(d) = uintx2_t{v[0] | ((uint32_t)v[1] << 16), v[2] | ((uint32_t)v[3] << 16)};
+  } else if constexpr (VEC == 2) {
+    *reinterpret_cast<uint32_t*>(d) = v[0] | ((uint32_t)v[1] << 16);
+  } else {
+    d[0] = v[0];
+  }
+}
+
+// the stride-1 problem over the lattice points, if the kernels above take it
+bool pw16_strided_plan(const ConvGeom& g, ConvGeom* c) {
+  if (!(g.KH == 1 && g.KW == 1 && g.py == 0 && g.px == 0 && g.groups == 1 && (g.sy > 1 || g.sx > 1))) return false;
+  *c = g;
+  c->H = g.OH; c->W = g.OW; c->sy = 1; c->sx = 1;
+  return pw16_applies(*c);
+}
+size_t lattice_bytes(const ConvGeom& c) {   // the gathered input / compact dx, rounded for what follows it
+  return (((size_t)c.N * c.C * c.H * c.W * sizeof(bf16_t)) + 255) & ~(size_t)255;
+}
+void lattice_gather(const ConvGeom& g, const void* x, void* xc, hipStream_t s) {
+  const uint32_t total = (uint32_t)((size_t)g.N * g.C * g.OH * g.OW);
+  hipLaunchKernelGGL(lattice_gather_kernel, dim3((total + 255) / 256), dim3(256), 0, s, static_cast<const bf16_t*>(x),
+                     static_cast<bf16_t*>(xc), g.H, g.W, g.OH, g.OW, g.sy, g.sx, total);
+}
+void lattice_scatter(const ConvGeom& g, const void* dxc, void* dx, hipStream_t s) {
+  const int vec = ((uintptr_t)dx & 15) ? 1 : g.W % 8 == 0 ? 8 : g.W % 4 == 0 ? 4 : g.W % 2 == 0 ? 2 : 1;
+  const uint32_t total = (uint32_t)((size_t)g.N * g.C * g.H * g.W / vec);
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3((total + 255) / 256), dim3(256), 0, s, static_cast<const bf16_t*>(dxc),
+                       static_cast<bf16_t*>(dx), g.H, g.W, g.OH, g.OW, g.sy, g.sx, total);
+  };
+  if (vec == 8) go(lattice_scatter_kernel<8>);
+  else if (vec == 4) go(lattice_scatter_kernel<4>);
+  else if (vec == 2) go(lattice_scatter_kernel<2>);
+  else go(lattice_scatter_kernel<1>);
+}
+
 }  // namespace
 
+size_t mfma_pointwise16_lattice_ws(const ConvGeom& g) {
+  ConvGeom c;
+  return pw16_strided_plan(g, &c) ? lattice_bytes(c) : 0;
+}
+
 int mfma_pointwise16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
-                              hipStream_t s) {
+                              hipStream_t s, void* ws, size_t ws_bytes) {
+  ConvGeom c;
+  if (pw16_strided_plan(g, &c)) {
+    if (!ws || ws_bytes < lattice_bytes(c)) return -1;
+    lattice_gather(g, x, ws, s);
+    return launch_pw16<false>(c, ws, w, bias, y, s);
+  }
   if (!pw16_applies(g)) return -1;
   return launch_pw16<false>(g, x, w, bias, y, s);
 }
 
-int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s) {
+int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s,
+                                   void* ws, size_t ws_bytes) {
+  ConvGeom c;
+  if (pw16_strided_plan(g, &c)) {
+    if (!ws || ws_bytes < lattice_bytes(c)) return -1;
+    const int rc = launch_pw16<true>(c, dy, w, nullptr, ws, s);
+    if (rc != FLHIP_OK) return rc;
+    lattice_scatter(g, ws, dx, s);
+    return check_launch("conv2d_bwd_data strided 1x1 (bf16 mfma)");
+  }
   if (!pw16_applies(g)) return -1;
   return launch_pw16<true>(g, dy, w, nullptr, dx, s);
 }
 
-size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g) {
+size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g0) {
+  ConvGeom g = g0;
+  size_t lattice = 0;
+  if (pw16_strided_plan(g0, &g)) lattice = lattice_bytes(g);
   Pw16WgradParams p{};
   if (!pw16_wgrad_plan(g, &p)) return 0;
-  return p.nsplit > 1 ? (size_t)p.nsplit * ((size_t)p.E + p.Mo) * sizeof(float) : 0;
+  return lattice + (p.nsplit > 1 ? (size_t)p.nsplit * ((size_t)p.E + p.Mo) * sizeof(float) : 0);
 }
 
-int mfma_pointwise16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
+int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, float* dw, float* db, void* ws,
                            size_t ws_bytes, hipStream_t s) {
   if (!dw) return -1;
+  ConvGeom g = g0;
+  const bool strided = pw16_strided_plan(g0, &g);
   Pw16WgradParams p{};
   if (!pw16_wgrad_plan(g, &p)) return -1;
+  if (strided) {
+    // the lattice points of x first, the slices of the gradient behind them
+    const size_t lb = lattice_bytes(g);
+    if (!ws || ws_bytes < lb) return fail(FLHIP_INVALID_ARGUMENT, "conv2d_bwd_filter: workspace too small");
+    lattice_gather(g0, x, ws, s);
+    x = ws;
+    ws = static_cast<char*>(ws) + lb;
+    ws_bytes -= lb;
+  }
   p.want_db = db != nullptr;
   const size_t need = p.nsplit > 1 ? (size_t)p.nsplit * ((size_t)p.E + p.Mo) * sizeof(float) : 0;
   if (need && (!ws || ws_bytes < need)) return fail(FLHIP_INVALID_ARGUMENT, "conv2d_bwd_filter: workspace too small");

@@ -64,6 +64,11 @@ MORE = [
     ((3, 64, 5, 9), (24, 64, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     ((7, 16, 1, 5), (16, 16, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     ((9, 24, 2, 3), (8, 24, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    # strided 1x1 in bf16: the input's lattice points are gathered into the workspace, the compact
+    # input gradient is spread over dx in 16- / 8- / 4- / 2-byte pieces
+    ((2, 64, 16, 24), (72, 64, 1, 1), (2, 2), (0, 0), (1, 1), 1),
+    ((2, 64, 10, 12), (40, 64, 1, 1), (3, 2), (0, 0), (1, 1), 1),
+    ((3, 32, 9, 10), (16, 32, 1, 1), (2, 3), (0, 0), (1, 1), 1),
     # long contractions on small grids (several chunks in flight): 9 and 11 chunks of 32
     ((3, 264, 7, 7), (72, 264, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     ((2, 40, 5, 5), (328, 40, 1, 1), (1, 1), (0, 0), (1, 1), 1),
