@@ -366,9 +366,9 @@ struct Pw16WgradParams {
 };
 
 // grid (slice, channel-tile pair).  A workgroup owns dw[64 m][64 c] and one slice of the
-// positions of the whole batch; thread t loads 16 positions (four 8-byte runs, each inside
+// positions of the whole batch; per chunk thread t loads one 8-byte run of 4 positions (inside
 // one image; ODD: planes not a multiple of 4 positions, where a run may end in the next
-// image) of row t / 4 of both operands per chunk.  out: slice-major partial results
+// image) of rows t / 16 + 16 g, g = 0..3, of both operands.  out: slice-major partial results
 // [nsplit][E + Mo] (dw tile values, then the bias sums), or dw / db themselves when there
 // is one slice.
 template <bool ODD>
@@ -383,66 +383,73 @@ pw16_wgrad_kernel(Pw16WgradParams p, const bf16_t* __restrict__ x, const bf16_t*
   const int wm = wave >> 1, wn = wave & 1;
   const int cbeg = slice * p.cps, cend = min(p.nchunks, cbeg + p.cps);
 
-  const int row = tid >> 2, piece = (tid & 3) * 16;
-  const bool mv = m0 + row < p.Mo, cv = c0 + row < p.C;
-  // position run g of this thread in chunk c: Q = c*64 + piece + 4*g; q[g] = its offset in
-  // the image, od/ox[g] = element offsets of (image, row 0) + q in dy / x
-  int q[4];
-  long long od[4], ox[4];
+  // loader roles: 16 lanes cover the 64 positions of a chunk row (128 contiguous bytes), so a
+  // wave's load touches 4 rows (with 4 lanes per row it touched 16 for the same bytes, and the
+  // kernel ran at the rate of those requests); a thread loads rows lrow + 16 g, g = 0..3
+  const int lrow = tid >> 4, lpos = (tid & 15) * 4;
+  bool mv[4], cv[4];
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    const long long Q = (long long)cbeg * PG_KC + piece + 4 * g;
-    const int n = (int)(Q / p.P);
-    q[g] = (int)(Q - (long long)n * p.P);
-    od[g] = (long long)n * p.Mo * p.P + q[g];
-    ox[g] = (long long)n * p.C * p.P + q[g];
+    mv[g] = m0 + lrow + 16 * g < p.Mo;
+    cv[g] = c0 + lrow + 16 * g < p.C;
   }
-  const long long drow = (long long)(m0 + row) * p.P, xrow = (long long)(c0 + row) * p.P;
+  // the thread's run of chunk c: positions Q = c*64 + lpos .. + 3 of the batch; q = Q's offset
+  // in its image, od / ox = element offsets of (image, row 0) + q in dy / x
+  int q;
+  long long od, ox;
+  {
+    const long long Q = (long long)cbeg * PG_KC + lpos;
+    const int n = (int)(Q / p.P);
+    q = (int)(Q - (long long)n * p.P);
+    od = (long long)n * p.Mo * p.P + q;
+    ox = (long long)n * p.C * p.P + q;
+  }
+  const long long drow = (long long)(m0 + lrow) * p.P, xrow = (long long)(c0 + lrow) * p.P, rstep = 16ll * p.P;
   const long long dlim = (long long)(p.Ptot / p.P) * p.Mo * p.P;   // == N * Mo * P
   uintx2_t sd[4], sx[4];
-  float bsum = 0.f;
+  float bsum[4] = {0.f, 0.f, 0.f, 0.f};
   const bool do_bias = p.want_db && ctile == 0;
   auto gload = [&]() {
+    const bool in = od < dlim;     // past the last image: nothing left
+    // ODD: a run with fewer than 4 positions left in its image continues in the next one
+    // (if there is one); all loads issue, from addresses inside the tensors
+    const int rem = p.P - q;
+    const bool cross = ODD && rem < 4;
+    const int back = cross ? 4 - rem : 0;
+    const long long nd = od - q + (long long)p.Mo * p.P, nx = ox - q + (long long)p.C * p.P;
+    const bool nin = cross && nd < dlim;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      const bool in = od[g] < dlim;     // past the last image: nothing left
       if (ODD) {
-        // a run with fewer than 4 positions left in its image continues in the next one
-        // (if there is one); all loads issue, from addresses inside the tensors
-        const int rem = p.P - q[g];
-        const bool cross = rem < 4;
-        const int back = cross ? 4 - rem : 0;
-        const long long nd = od[g] - q[g] + (long long)p.Mo * p.P, nx = ox[g] - q[g] + (long long)p.C * p.P;
-        const bool nin = cross && nd < dlim;
-        uintx2_t a = load8_any(dy + ((in && mv) ? od[g] - back + drow : 0));
-        uintx2_t b = load8_any(dy + ((nin && mv) ? nd + drow : 0));
+        uintx2_t a = load8_any(dy + ((in && mv[g]) ? od - back + drow + g * rstep : 0));
+        uintx2_t b = load8_any(dy + ((nin && mv[g]) ? nd + drow + g * rstep : 0));
         if (cross) a = merge_runs(a, nin ? b : uintx2_t{0u, 0u}, rem);
-        sd[g] = (in && mv) ? a : uintx2_t{0u, 0u};
-        a = load8_any(x + ((in && cv) ? ox[g] - back + xrow : 0));
-        b = load8_any(x + ((nin && cv) ? nx + xrow : 0));
+        sd[g] = (in && mv[g]) ? a : uintx2_t{0u, 0u};
+        a = load8_any(x + ((in && cv[g]) ? ox - back + xrow + g * rstep : 0));
+        b = load8_any(x + ((nin && cv[g]) ? nx + xrow + g * rstep : 0));
         if (cross) a = merge_runs(a, nin ? b : uintx2_t{0u, 0u}, rem);
-        sx[g] = (in && cv) ? a : uintx2_t{0u, 0u};
+        sx[g] = (in && cv[g]) ? a : uintx2_t{0u, 0u};
       } else {
-        sd[g] = (in && mv) ? *reinterpret_cast<const uintx2_t*>(dy + od[g] + drow) : uintx2_t{0u, 0u};
-        sx[g] = (in && cv) ? *reinterpret_cast<const uintx2_t*>(x + ox[g] + xrow) : uintx2_t{0u, 0u};
+        sd[g] = (in && mv[g]) ? *reinterpret_cast<const uintx2_t*>(dy + od + drow + g * rstep) : uintx2_t{0u, 0u};
+        sx[g] = (in && cv[g]) ? *reinterpret_cast<const uintx2_t*>(x + ox + xrow + g * rstep) : uintx2_t{0u, 0u};
       }
-      // next chunk: 64 positions on, possibly into the following images
-      q[g] += PG_KC; od[g] += PG_KC; ox[g] += PG_KC;
-      while (q[g] >= p.P) {
-        q[g] -= p.P;
-        od[g] += (long long)(p.Mo - 1) * p.P;
-        ox[g] += (long long)(p.C - 1) * p.P;
-      }
+    }
+    // next chunk: 64 positions on, possibly into the following images
+    q += PG_KC; od += PG_KC; ox += PG_KC;
+    while (q >= p.P) {
+      q -= p.P;
+      od += (long long)(p.Mo - 1) * p.P;
+      ox += (long long)(p.C - 1) * p.P;
     }
   };
   auto sstore = [&](int buf) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      *reinterpret_cast<uintx2_t*>(&Ds[buf][row * PG_P + piece + 4 * g]) = sd[g];
-      *reinterpret_cast<uintx2_t*>(&Xs[buf][row * PG_P + piece + 4 * g]) = sx[g];
+      *reinterpret_cast<uintx2_t*>(&Ds[buf][(lrow + 16 * g) * PG_P + lpos]) = sd[g];
+      *reinterpret_cast<uintx2_t*>(&Xs[buf][(lrow + 16 * g) * PG_P + lpos]) = sx[g];
       if (do_bias) {
-        bsum += bf16_to_f32((bf16_t)(sd[g].x & 0xffffu)) + bf16_to_f32((bf16_t)(sd[g].x >> 16));
-        bsum += bf16_to_f32((bf16_t)(sd[g].y & 0xffffu)) + bf16_to_f32((bf16_t)(sd[g].y >> 16));
+        bsum[g] += bf16_to_f32((bf16_t)(sd[g].x & 0xffffu)) + bf16_to_f32((bf16_t)(sd[g].x >> 16));
+        bsum[g] += bf16_to_f32((bf16_t)(sd[g].y & 0xffffu)) + bf16_to_f32((bf16_t)(sd[g].y >> 16));
       }
     }
   };
@@ -492,11 +499,17 @@ pw16_wgrad_kernel(Pw16WgradParams p, const bf16_t* __restrict__ x, const bf16_t*
       }
     }
   if (do_bias) {
-    bsum += __shfl_xor(bsum, 1, 64);
-    bsum += __shfl_xor(bsum, 2, 64);
-    if ((tid & 3) == 0 && mv) {
-      if (p.nsplit > 1) o[p.E + m0 + row] = bsum;
-      else db_direct[m0 + row] = bsum;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      float b = bsum[g];
+      b += __shfl_xor(b, 1, 64);
+      b += __shfl_xor(b, 2, 64);
+      b += __shfl_xor(b, 4, 64);
+      b += __shfl_xor(b, 8, 64);
+      if ((tid & 15) == 0 && mv[g]) {
+        if (p.nsplit > 1) o[p.E + m0 + lrow + 16 * g] = b;
+        else db_direct[m0 + lrow + 16 * g] = b;
+      }
     }
   }
 }
