@@ -41,12 +41,13 @@ int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, c
 // bf16 storage on the bf16 matrix cores: 1x1 windows without padding over planes of at
 // least 4 positions, channel counts multiples of 8; -1 otherwise.  Strided windows need
 // mfma_pointwise16_lattice_ws() bytes of workspace (the input's lattice points / the compact
-// gradient) and return -1 without it.
+// gradient) and return -1 without it; so do the backward passes of strided windows with 2 to 9
+// taps, which gather the taps next to the channels (bwd = true in the query).
 int mfma_pointwise16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
                               hipStream_t s, void* ws = nullptr, size_t ws_bytes = 0);
 int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s,
                                    void* ws = nullptr, size_t ws_bytes = 0);
-size_t mfma_pointwise16_lattice_ws(const ConvGeom& g);
+size_t mfma_pointwise16_lattice_ws(const ConvGeom& g, bool bwd);
 size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g);
 int mfma_pointwise16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
                            size_t ws_bytes, hipStream_t s);

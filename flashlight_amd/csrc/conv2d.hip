@@ -184,7 +184,7 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
   // (bf16: strided 1x1 windows gather the input's lattice points / spread a compact gradient)
   if (pass == FLHIP_CONV_FWD || pass == FLHIP_CONV_BWD_DATA) {
     const size_t a = mfma_tapped_ws(g, d->dtype, pass == FLHIP_CONV_BWD_DATA);
-    const size_t b = d->dtype == FLHIP_BF16 ? mfma_pointwise16_lattice_ws(g) : 0;
+    const size_t b = d->dtype == FLHIP_BF16 ? mfma_pointwise16_lattice_ws(g, pass == FLHIP_CONV_BWD_DATA) : 0;
     return a > b ? a : b;
   }
   return 0;

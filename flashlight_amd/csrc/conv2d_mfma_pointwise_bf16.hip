@@ -608,11 +608,126 @@ void lattice_scatter(const ConvGeom& g, const void* dxc, void* dx, hipStream_t s
   else go(lattice_scatter_kernel<1>);
 }
 
+
+// ---- strided windows with several taps (backward passes) ---------------------------------
+// The same idea one step further: with the window's taps gathered next to the channels,
+//   xc[n][c * T + tap][oh][ow] = x[n][c][oh sy + kh dly - py][ow sx + kw dlx - px]  (0 outside),
+// a strided 3x3 convolution is a 1x1 stride-1 one over C * T channels whose weight matrix is
+// the OIHW filter as it lies in memory.  The filter gradient gathers xc and runs the 1x1
+// filter-gradient kernel; backward-data runs the 1x1 kernel into the workspace (one bf16
+// plane per channel and tap) and sums the taps that reach each element of dx in fp32.
+// A workgroup handles the T planes of one (image, channel): contiguous in xc.
+// PAIR: a thread makes two neighbouring columns (rows of even length) and stores 4 bytes
+template <bool PAIR>
+__global__ void __launch_bounds__(256)
+taps_gather_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ xc, ConvGeom g) {
+  constexpr int V = PAIR ? 2 : 1;
+  const int P = g.OH * g.OW, T = g.KH * g.KW, PV = P / V, OWV = g.OW / V;
+  const bf16_t* xp = x + (size_t)blockIdx.x * g.H * g.W;
+  bf16_t* op = xc + (size_t)blockIdx.x * T * P;
+  for (int tap = 0; tap < T; ++tap) {
+    const int kh = tap / g.KW, kw = tap - kh * g.KW;
+    const int dh = kh * g.dly - g.py, dw = kw * g.dlx - g.px;
+    for (int qv = threadIdx.x; qv < PV; qv += blockDim.x) {
+      const int oh = qv / OWV, ow = (qv - oh * OWV) * V;
+      const int ih = oh * g.sy + dh;
+      const bool rv = (unsigned)ih < (unsigned)g.H;
+      uint32_t v[V];
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const int iw = (ow + e) * g.sx + dw;
+        v[e] = (rv && (unsigned)iw < (unsigned)g.W) ? xp[ih * g.W + iw] : (bf16_t)0;
+      }
+      if constexpr (PAIR) *reinterpret_cast<uint32_t*>(op + tap * P + 2 * qv) = v[0] | (v[1] << 16);
+      else op[tap * P + qv] = (bf16_t)v[0];
+    }
+  }
+}
+
+// S2: strides 2, no dilation (the index arithmetic then needs no division by a stride);
+// PAIR as above, over the columns of dx
+template <bool S2, bool PAIR>
+__global__ void __launch_bounds__(256)
+taps_spread_kernel(const bf16_t* __restrict__ dxc, bf16_t* __restrict__ dx, ConvGeom g) {
+  constexpr int V = PAIR ? 2 : 1;
+  const int P = g.OH * g.OW, T = g.KH * g.KW, WV = g.W / V;
+  const bf16_t* cp = dxc + (size_t)blockIdx.x * T * P;
+  bf16_t* dp = dx + (size_t)blockIdx.x * g.H * g.W;
+  for (int ev = threadIdx.x; ev < g.H * WV; ev += blockDim.x) {
+    const int h = ev / WV, w0 = (ev - h * WV) * V;
+    float acc[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const int w = w0 + e;
+      acc[e] = 0.f;
+      if (S2) {
+        // taps kh with h + py - kh even: kh = (h + py) & 1, + 2, ...
+        for (int kh = (h + g.py) & 1; kh < g.KH; kh += 2) {
+          const int oh = (h + g.py - kh) >> 1;
+          if (h + g.py - kh < 0 || oh >= g.OH) continue;
+          for (int kw = (w + g.px) & 1; kw < g.KW; kw += 2) {
+            const int ow = (w + g.px - kw) >> 1;
+            if (w + g.px - kw < 0 || ow >= g.OW) continue;
+            acc[e] += bf16_to_f32(cp[(kh * g.KW + kw) * P + oh * g.OW + ow]);
+          }
+        }
+      } else {
+        for (int kh = 0; kh < g.KH; ++kh) {
+          const int a = h + g.py - kh * g.dly;
+          if (a < 0 || a % g.sy != 0 || a / g.sy >= g.OH) continue;
+          for (int kw = 0; kw < g.KW; ++kw) {
+            const int b = w + g.px - kw * g.dlx;
+            if (b < 0 || b % g.sx != 0 || b / g.sx >= g.OW) continue;
+            acc[e] += bf16_to_f32(cp[(kh * g.KW + kw) * P + (a / g.sy) * g.OW + b / g.sx]);
+          }
+        }
+      }
+    }
+    if constexpr (PAIR)
+      *reinterpret_cast<uint32_t*>(dp + 2 * ev) = (uint32_t)f32_to_bf16(acc[0]) | ((uint32_t)f32_to_bf16(acc[1]) << 16);
+    else
+      dp[ev] = f32_to_bf16(acc[0]);
+  }
+}
+
+// threads per workgroup for a plane of `items` work items
+inline unsigned plane_threads(int items) { return items >= 256 ? 256u : (unsigned)((items + 63) / 64 * 64); }
+
+void taps_gather(const ConvGeom& g, const void* x, void* xc, hipStream_t s) {
+  const bool pair = g.OW % 2 == 0 && ((uintptr_t)xc & 3) == 0;
+  const dim3 grid((unsigned)(g.N * g.C)), block(plane_threads(g.OH * g.OW / (pair ? 2 : 1)));
+  if (pair) hipLaunchKernelGGL(taps_gather_kernel<true>, grid, block, 0, s, static_cast<const bf16_t*>(x), static_cast<bf16_t*>(xc), g);
+  else hipLaunchKernelGGL(taps_gather_kernel<false>, grid, block, 0, s, static_cast<const bf16_t*>(x), static_cast<bf16_t*>(xc), g);
+}
+void taps_spread(const ConvGeom& g, const void* dxc, void* dx, hipStream_t s) {
+  const bool pair = g.W % 2 == 0 && ((uintptr_t)dx & 3) == 0;
+  const bool s2 = g.sy == 2 && g.sx == 2 && g.dly == 1 && g.dlx == 1;
+  const dim3 grid((unsigned)(g.N * g.C)), block(plane_threads(g.H * g.W / (pair ? 2 : 1)));
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, block, 0, s, static_cast<const bf16_t*>(dxc), static_cast<bf16_t*>(dx), g);
+  };
+  if (s2) { if (pair) go(taps_spread_kernel<true, true>); else go(taps_spread_kernel<true, false>); }
+  else { if (pair) go(taps_spread_kernel<false, true>); else go(taps_spread_kernel<false, false>); }
+}
+
+bool pw16_taps_plan(const ConvGeom& g, ConvGeom* c) {
+  const int T = g.KH * g.KW;
+  if (!(g.groups == 1 && T > 1 && T <= 9 && (g.sy > 1 || g.sx > 1))) return false;
+  if ((long long)g.N * g.C * T * g.OH * g.OW >= (1ll << 31)) return false;
+  *c = g;
+  c->C = g.C * T; c->Cg = c->C;
+  c->H = g.OH; c->W = g.OW;
+  c->KH = 1; c->KW = 1; c->sy = 1; c->sx = 1; c->py = 0; c->px = 0; c->dly = 1; c->dlx = 1;
+  return pw16_applies(*c);
+}
+
 }  // namespace
 
-size_t mfma_pointwise16_lattice_ws(const ConvGeom& g) {
+size_t mfma_pointwise16_lattice_ws(const ConvGeom& g, bool bwd) {
   ConvGeom c;
-  return pw16_strided_plan(g, &c) ? lattice_bytes(c) : 0;
+  if (pw16_strided_plan(g, &c)) return lattice_bytes(c);
+  if (bwd && !getenv("FLHIP_PW16_NO_TAPS") && pw16_taps_plan(g, &c)) return lattice_bytes(c);
+  return 0;
 }
 
 int mfma_pointwise16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
@@ -637,6 +752,13 @@ int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void
     lattice_scatter(g, ws, dx, s);
     return check_launch("conv2d_bwd_data strided 1x1 (bf16 mfma)");
   }
+  if (!getenv("FLHIP_PW16_NO_TAPS") && pw16_taps_plan(g, &c)) {
+    if (!ws || ws_bytes < lattice_bytes(c)) return -1;
+    const int rc = launch_pw16<true>(c, dy, w, nullptr, ws, s);
+    if (rc != FLHIP_OK) return rc;
+    taps_spread(g, ws, dx, s);
+    return check_launch("conv2d_bwd_data strided window (bf16 mfma)");
+  }
   if (!pw16_applies(g)) return -1;
   return launch_pw16<true>(g, dy, w, nullptr, dx, s);
 }
@@ -644,7 +766,8 @@ int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void
 size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g0) {
   ConvGeom g = g0;
   size_t lattice = 0;
-  if (pw16_strided_plan(g0, &g)) lattice = lattice_bytes(g);
+  if (pw16_strided_plan(g0, &g) || (!getenv("FLHIP_PW16_NO_TAPS") && pw16_taps_plan(g0, &g))) lattice = lattice_bytes(g);
+  else g = g0;
   Pw16WgradParams p{};
   if (!pw16_wgrad_plan(g, &p)) return 0;
   return lattice + (p.nsplit > 1 ? (size_t)p.nsplit * ((size_t)p.E + p.Mo) * sizeof(float) : 0);
@@ -655,13 +778,16 @@ int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, fl
   if (!dw) return -1;
   ConvGeom g = g0;
   const bool strided = pw16_strided_plan(g0, &g);
+  const bool taps = !strided && !getenv("FLHIP_PW16_NO_TAPS") && pw16_taps_plan(g0, &g);
+  if (!strided && !taps) g = g0;
   Pw16WgradParams p{};
   if (!pw16_wgrad_plan(g, &p)) return -1;
-  if (strided) {
-    // the lattice points of x first, the slices of the gradient behind them
+  if (strided || taps) {
+    // the gathered input first, the slices of the gradient behind it
     const size_t lb = lattice_bytes(g);
     if (!ws || ws_bytes < lb) return fail(FLHIP_INVALID_ARGUMENT, "conv2d_bwd_filter: workspace too small");
-    lattice_gather(g0, x, ws, s);
+    if (strided) lattice_gather(g0, x, ws, s);
+    else taps_gather(g0, x, ws, s);
     x = ws;
     ws = static_cast<char*>(ws) + lb;
     ws_bytes -= lb;
