@@ -115,8 +115,8 @@ int flhip_pool2d_out_dims(const flhip_pool_desc* d, int32_t* OH, int32_t* OW);
 /* Scratch a convolution pass uses (0 is possible).  The filter gradient needs it (partial
  * results of the sliced contraction); forward and backward-data run without it too, but
  * with it the kernels for strided / long windows read weights reordered per tap, and
- * strided 1x1 windows in bf16 storage run on the bf16 matrix cores over a gathered copy
- * of the input's lattice points. */
+ * strided windows in bf16 storage run on the bf16 matrix cores over a gathered copy of
+ * the input's lattice points (1x1, all passes) or of its taps (up to 9, backward passes). */
 size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pass);
 
 /* AutogradExtension::conv2d (AutogradExtension.h:58-69; oneDNN peer

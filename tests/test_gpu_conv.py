@@ -69,6 +69,12 @@ MORE = [
     ((2, 64, 16, 24), (72, 64, 1, 1), (2, 2), (0, 0), (1, 1), 1),
     ((2, 64, 10, 12), (40, 64, 1, 1), (3, 2), (0, 0), (1, 1), 1),
     ((3, 32, 9, 10), (16, 32, 1, 1), (2, 3), (0, 0), (1, 1), 1),
+    # strided windows in bf16, backward passes through gathered taps: 2x2 / 3x3 / 1x3 windows, stride 2
+    # (pairs of columns) and other strides, dilation, odd planes, padding larger than the window reach
+    ((2, 32, 12, 16), (24, 32, 3, 3), (2, 2), (1, 1), (1, 1), 1),
+    ((3, 16, 9, 9), (16, 16, 2, 2), (2, 2), (0, 0), (1, 1), 1),
+    ((2, 24, 10, 15), (16, 24, 1, 3), (1, 3), (0, 2), (1, 2), 1),
+    ((2, 16, 14, 14), (32, 16, 3, 3), (2, 2), (2, 2), (1, 1), 1),
     # long contractions on small grids (several chunks in flight): 9 and 11 chunks of 32
     ((3, 264, 7, 7), (72, 264, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     ((2, 40, 5, 5), (328, 40, 1, 1), (1, 1), (0, 0), (1, 1), 1),
