@@ -196,6 +196,36 @@ def test_forward_and_backward_data_without_workspace(shape):
     assert torch.equal(y0, y) and torch.equal(dx0, dx)
 
 
+@pytest.mark.parametrize("shape", [((3, 64, 14, 14), (96, 64, 1, 1), (2, 2), (0, 0)),
+                                   ((2, 32, 12, 16), (40, 32, 3, 3), (2, 2), (1, 1))])
+def test_bf16_strided_windows_without_workspace(shape):
+    """bf16 storage: strided 1x1 windows (all passes) and the backward-data pass of strided 3x3
+    windows reach the bf16 matrix cores through a gathered copy in the workspace; without it the
+    same calls take the converting kernels.  Both agree to bf16 rounding."""
+    import ctypes as C
+    from flashlight_amd import capi
+    xs, ws_, st, pd = shape
+    rng = np.random.default_rng(78)
+    x = dev(bf16_round(rng.standard_normal(xs).astype(np.float32))).to(torch.bfloat16)
+    w = dev(bf16_round((rng.standard_normal(ws_) / 20).astype(np.float32))).to(torch.bfloat16)
+    kw = dict(sx=st[1], sy=st[0], px=pd[1], py=pd[0], dx=1, dy=1, groups=1)
+    y = fa.conv2d(x, w, None, **kw)
+    dy = dev(bf16_round(rng.standard_normal(tuple(y.shape)).astype(np.float32))).to(torch.bfloat16)
+    dx = fa.conv2d_backward_data(dy, xs, w, **kw)
+    L = capi.lib()
+    cd = capi.ConvDesc(xs[0], xs[1], xs[2], xs[3], ws_[0], ws_[2], ws_[3], st[0], st[1], pd[0], pd[1], 1, 1, 1,
+                       capi.BF16)
+    lattice = xs[0] * xs[1] * ws_[2] * ws_[3] * y.shape[2] * y.shape[3] * 2
+    assert L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_BWD_DATA) >= lattice
+    S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: C.c_void_p(t.data_ptr())
+    y0, dx0 = torch.empty_like(y), torch.empty_like(dx)
+    assert L.flhip_conv2d_fwd(C.byref(cd), P(x), P(w), None, P(y0), None, 0, S) == 0
+    assert L.flhip_conv2d_bwd_data(C.byref(cd), P(dy), P(w), P(dx0), None, 0, S) == 0
+    torch.cuda.synchronize()
+    assert rel_l2(host(y0), host(y)) <= 1e-2 and rel_l2(host(dx0), host(dx)) <= 1e-2
+
+
 def _random_cases(n, seed):
     """Seeded random geometries biased towards the conditions the kernel families key on:
     1x1 and 3x3 windows, even / odd rows, planes of 4k positions, channel counts around the
