@@ -609,7 +609,7 @@ void lattice_scatter(const ConvGeom& g, const void* dxc, void* dx, hipStream_t s
 }
 
 
-// ---- strided windows with several taps (backward passes) ---------------------------------
+// ---- strided windows with several taps (backward passes), odd rows (filter gradient) ------
 // The same idea one step further: with the window's taps gathered next to the channels,
 //   xc[n][c * T + tap][oh][ow] = x[n][c][oh sy + kh dly - py][ow sx + kw dlx - px]  (0 outside),
 // a strided 3x3 convolution is a 1x1 stride-1 one over C * T channels whose weight matrix is
@@ -710,9 +710,13 @@ void taps_spread(const ConvGeom& g, const void* dxc, void* dx, hipStream_t s) {
   else { if (pair) go(taps_spread_kernel<false, true>); else go(taps_spread_kernel<false, false>); }
 }
 
-bool pw16_taps_plan(const ConvGeom& g, ConvGeom* c) {
+bool pw16_taps_plan(const ConvGeom& g, ConvGeom* c, bool wgrad = false) {
   const int T = g.KH * g.KW;
-  if (!(g.groups == 1 && T > 1 && T <= 9 && (g.sy > 1 || g.sx > 1))) return false;
+  // stride 1: only the filter gradient over rows of odd length, which the row kernel for bf16
+  // storage does not take (7x7 planes: 84 us through the taps, 138 us converting; over even rows
+  // the row kernel is as fast or faster)
+  const bool s1ok = wgrad && g.OW % 2 != 0;
+  if (!(g.groups == 1 && T > 1 && T <= 9 && (g.sy > 1 || g.sx > 1 || s1ok))) return false;
   if ((long long)g.N * g.C * T * g.OH * g.OW >= (1ll << 31)) return false;
   *c = g;
   c->C = g.C * T; c->Cg = c->C;
@@ -766,7 +770,7 @@ int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void
 size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g0) {
   ConvGeom g = g0;
   size_t lattice = 0;
-  if (pw16_strided_plan(g0, &g) || (!getenv("FLHIP_PW16_NO_TAPS") && pw16_taps_plan(g0, &g))) lattice = lattice_bytes(g);
+  if (pw16_strided_plan(g0, &g) || (!getenv("FLHIP_PW16_NO_TAPS") && pw16_taps_plan(g0, &g, true))) lattice = lattice_bytes(g);
   else g = g0;
   Pw16WgradParams p{};
   if (!pw16_wgrad_plan(g, &p)) return 0;
@@ -778,7 +782,7 @@ int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, fl
   if (!dw) return -1;
   ConvGeom g = g0;
   const bool strided = pw16_strided_plan(g0, &g);
-  const bool taps = !strided && !getenv("FLHIP_PW16_NO_TAPS") && pw16_taps_plan(g0, &g);
+  const bool taps = !strided && !getenv("FLHIP_PW16_NO_TAPS") && pw16_taps_plan(g0, &g, true);
   if (!strided && !taps) g = g0;
   Pw16WgradParams p{};
   if (!pw16_wgrad_plan(g, &p)) return -1;

@@ -75,6 +75,9 @@ MORE = [
     ((3, 16, 9, 9), (16, 16, 2, 2), (2, 2), (0, 0), (1, 1), 1),
     ((2, 24, 10, 15), (16, 24, 1, 3), (1, 3), (0, 2), (1, 2), 1),
     ((2, 16, 14, 14), (32, 16, 3, 3), (2, 2), (2, 2), (1, 1), 1),
+    # stride-1 windows over rows of odd length: bf16 filter gradient through gathered taps
+    ((4, 64, 7, 7), (72, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((2, 16, 6, 13), (24, 16, 2, 3), (1, 1), (1, 0), (1, 2), 1),
     # long contractions on small grids (several chunks in flight): 9 and 11 chunks of 32
     ((3, 264, 7, 7), (72, 264, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     ((2, 40, 5, 5), (328, 40, 1, 1), (1, 1), (0, 0), (1, 1), 1),
