@@ -590,7 +590,11 @@ bool pw16_strided_plan(const ConvGeom& g, ConvGeom* c) {
 size_t lattice_bytes(const ConvGeom& c) {   // the gathered input / compact dx, rounded for what follows it
   return (((size_t)c.N * c.C * c.H * c.W * sizeof(bf16_t)) + 255) & ~(size_t)255;
 }
+bool taps_gather(const ConvGeom& g, const void* x, void* xc, hipStream_t s);
 void lattice_gather(const ConvGeom& g, const void* x, void* xc, hipStream_t s) {
+  // the gather kernel of the windows with several taps (T = 1 here) is the faster copy
+  // (11 / 7 us against 15 / 9 us on the 56x56 / 28x28 downsample layers of ResNet-50)
+  if (taps_gather(g, x, xc, s)) return;
   const uint32_t total = (uint32_t)((size_t)g.N * g.C * g.OH * g.OW);
   hipLaunchKernelGGL(lattice_gather_kernel, dim3((total + 255) / 256), dim3(256), 0, s, static_cast<const bf16_t*>(x),
                      static_cast<bf16_t*>(xc), g.H, g.W, g.OH, g.OW, g.sy, g.sx, total);
@@ -618,18 +622,23 @@ void lattice_scatter(const ConvGeom& g, const void* dxc, void* dx, hipStream_t s
 // plane per channel and tap) and sums the taps that reach each element of dx in fp32.
 // A workgroup handles the T planes of one (image, channel): contiguous in xc.
 // PAIR: a thread makes two neighbouring columns (rows of even length) and stores 4 bytes
+// Both kernels below: a workgroup per (image, channel) with threads laid out (columns, rows) over
+// the plane - the first dimension is the next power of two that covers a row - so that no index
+// needs a division (with a flat index the divisions, not memory, set the pace of these copies).
 template <bool PAIR>
 __global__ void __launch_bounds__(256)
 taps_gather_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ xc, ConvGeom g) {
   constexpr int V = PAIR ? 2 : 1;
-  const int P = g.OH * g.OW, T = g.KH * g.KW, PV = P / V, OWV = g.OW / V;
-  const bf16_t* xp = x + (size_t)blockIdx.x * g.H * g.W;
-  bf16_t* op = xc + (size_t)blockIdx.x * T * P;
+  const int P = g.OH * g.OW, T = g.KH * g.KW;
+  const int tx = threadIdx.x, ow = tx * V;
+  const unsigned plane = blockIdx.x * blockDim.z + threadIdx.z;   // small planes: several per workgroup
+  if (ow >= g.OW || plane >= (unsigned)(g.N * g.C)) return;
+  const bf16_t* xp = x + (size_t)plane * g.H * g.W;
+  bf16_t* op = xc + (size_t)plane * T * P;
   for (int tap = 0; tap < T; ++tap) {
     const int kh = tap / g.KW, kw = tap - kh * g.KW;
     const int dh = kh * g.dly - g.py, dw = kw * g.dlx - g.px;
-    for (int qv = threadIdx.x; qv < PV; qv += blockDim.x) {
-      const int oh = qv / OWV, ow = (qv - oh * OWV) * V;
+    for (int oh = threadIdx.y; oh < g.OH; oh += blockDim.y) {
       const int ih = oh * g.sy + dh;
       const bool rv = (unsigned)ih < (unsigned)g.H;
       uint32_t v[V];
@@ -638,39 +647,50 @@ taps_gather_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ xc, ConvGe
         const int iw = (ow + e) * g.sx + dw;
         v[e] = (rv && (unsigned)iw < (unsigned)g.W) ? xp[ih * g.W + iw] : (bf16_t)0;
       }
-      if constexpr (PAIR) *reinterpret_cast<uint32_t*>(op + tap * P + 2 * qv) = v[0] | (v[1] << 16);
-      else op[tap * P + qv] = (bf16_t)v[0];
+      bf16_t* o = op + tap * P + oh * g.OW + ow;
+      if constexpr (PAIR) *reinterpret_cast<uint32_t*>(o) = v[0] | (v[1] << 16);
+      else *o = (bf16_t)v[0];
     }
   }
 }
 
-// S2: strides 2, no dilation (the index arithmetic then needs no division by a stride);
-// PAIR as above, over the columns of dx
+// S2: strides 2, no dilation (parity picks the taps that reach an element, no division by a
+// stride); PAIR as above, over the columns of dx
 template <bool S2, bool PAIR>
 __global__ void __launch_bounds__(256)
 taps_spread_kernel(const bf16_t* __restrict__ dxc, bf16_t* __restrict__ dx, ConvGeom g) {
   constexpr int V = PAIR ? 2 : 1;
-  const int P = g.OH * g.OW, T = g.KH * g.KW, WV = g.W / V;
-  const bf16_t* cp = dxc + (size_t)blockIdx.x * T * P;
-  bf16_t* dp = dx + (size_t)blockIdx.x * g.H * g.W;
-  for (int ev = threadIdx.x; ev < g.H * WV; ev += blockDim.x) {
-    const int h = ev / WV, w0 = (ev - h * WV) * V;
+  const int P = g.OH * g.OW, T = g.KH * g.KW;
+  const int w0 = threadIdx.x * V;
+  const unsigned plane = blockIdx.x * blockDim.z + threadIdx.z;
+  if (w0 >= g.W || plane >= (unsigned)(g.N * g.C)) return;
+  const bf16_t* cp = dxc + (size_t)plane * T * P;
+  bf16_t* dp = dx + (size_t)plane * g.H * g.W;
+  for (int h = threadIdx.y; h < g.H; h += blockDim.y) {
     float acc[V];
 #pragma unroll
     for (int e = 0; e < V; ++e) {
       const int w = w0 + e;
       acc[e] = 0.f;
       if (S2) {
-        // taps kh with h + py - kh even: kh = (h + py) & 1, + 2, ...
-        for (int kh = (h + g.py) & 1; kh < g.KH; kh += 2) {
-          const int oh = (h + g.py - kh) >> 1;
-          if (h + g.py - kh < 0 || oh >= g.OH) continue;
-          for (int kw = (w + g.px) & 1; kw < g.KW; kw += 2) {
-            const int ow = (w + g.px - kw) >> 1;
-            if (w + g.px - kw < 0 || ow >= g.OW) continue;
-            acc[e] += bf16_to_f32(cp[(kh * g.KW + kw) * P + oh * g.OW + ow]);
+        // the taps with h + py - kh and w + px - kw even: kh = ((h + py) & 1) + 2a, kw likewise
+        // (windows of at most 4 x 4); the four loads are issued together
+        const int kh0 = (h + g.py) & 1, kw0 = (w + g.px) & 1;
+        uint32_t ld[2][2];
+        bool ok[2][2];
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+          for (int b = 0; b < 2; ++b) {
+            const int kh = kh0 + 2 * a, kw = kw0 + 2 * b;
+            const int dh = h + g.py - kh, dw = w + g.px - kw;
+            ok[a][b] = kh < g.KH && kw < g.KW && dh >= 0 && dw >= 0 && (dh >> 1) < g.OH && (dw >> 1) < g.OW;
+            ld[a][b] = cp[ok[a][b] ? (kh * g.KW + kw) * P + (dh >> 1) * g.OW + (dw >> 1) : 0];
           }
-        }
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+          for (int b = 0; b < 2; ++b) acc[e] += ok[a][b] ? bf16_to_f32((bf16_t)ld[a][b]) : 0.f;
       } else {
         for (int kh = 0; kh < g.KH; ++kh) {
           const int a = h + g.py - kh * g.dly;
@@ -683,31 +703,45 @@ taps_spread_kernel(const bf16_t* __restrict__ dxc, bf16_t* __restrict__ dx, Conv
         }
       }
     }
-    if constexpr (PAIR)
-      *reinterpret_cast<uint32_t*>(dp + 2 * ev) = (uint32_t)f32_to_bf16(acc[0]) | ((uint32_t)f32_to_bf16(acc[1]) << 16);
-    else
-      dp[ev] = f32_to_bf16(acc[0]);
+    bf16_t* o = dp + h * g.W + w0;
+    if constexpr (PAIR) *reinterpret_cast<uint32_t*>(o) = (uint32_t)f32_to_bf16(acc[0]) | ((uint32_t)f32_to_bf16(acc[1]) << 16);
+    else *o = f32_to_bf16(acc[0]);
   }
 }
 
-// threads per workgroup for a plane of `items` work items
-inline unsigned plane_threads(int items) { return items >= 256 ? 256u : (unsigned)((items + 63) / 64 * 64); }
+// (columns, rows, planes) threads for planes of cols x rows work items: 256 in all, the first
+// dimension the next power of two >= cols; rows wider than 256 items do not get here
+inline bool plane_block(int cols, int rows, dim3* b) {
+  unsigned bx = 1;
+  while ((int)bx < cols) bx <<= 1;
+  if (bx > 256) return false;
+  unsigned by = 256 / bx;
+  while (by > 1 && (int)(by / 2) >= rows) by >>= 1;
+  *b = dim3(bx, by, 256 / (bx * by));   // planes smaller than 256 items share a workgroup
+  return true;
+}
 
-void taps_gather(const ConvGeom& g, const void* x, void* xc, hipStream_t s) {
+bool taps_gather(const ConvGeom& g, const void* x, void* xc, hipStream_t s) {
   const bool pair = g.OW % 2 == 0 && ((uintptr_t)xc & 3) == 0;
-  const dim3 grid((unsigned)(g.N * g.C)), block(plane_threads(g.OH * g.OW / (pair ? 2 : 1)));
+  dim3 block;
+  if (!plane_block(g.OW / (pair ? 2 : 1), g.OH, &block)) return false;
+  const dim3 grid((unsigned)((g.N * g.C + block.z - 1) / block.z));
   if (pair) hipLaunchKernelGGL(taps_gather_kernel<true>, grid, block, 0, s, static_cast<const bf16_t*>(x), static_cast<bf16_t*>(xc), g);
   else hipLaunchKernelGGL(taps_gather_kernel<false>, grid, block, 0, s, static_cast<const bf16_t*>(x), static_cast<bf16_t*>(xc), g);
+  return true;
 }
-void taps_spread(const ConvGeom& g, const void* dxc, void* dx, hipStream_t s) {
+bool taps_spread(const ConvGeom& g, const void* dxc, void* dx, hipStream_t s) {
   const bool pair = g.W % 2 == 0 && ((uintptr_t)dx & 3) == 0;
-  const bool s2 = g.sy == 2 && g.sx == 2 && g.dly == 1 && g.dlx == 1;
-  const dim3 grid((unsigned)(g.N * g.C)), block(plane_threads(g.H * g.W / (pair ? 2 : 1)));
+  const bool s2 = g.sy == 2 && g.sx == 2 && g.dly == 1 && g.dlx == 1 && g.KH <= 4 && g.KW <= 4;
+  dim3 block;
+  if (!plane_block(g.W / (pair ? 2 : 1), g.H, &block)) return false;
+  const dim3 grid((unsigned)((g.N * g.C + block.z - 1) / block.z));
   auto go = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, block, 0, s, static_cast<const bf16_t*>(dxc), static_cast<bf16_t*>(dx), g);
   };
   if (s2) { if (pair) go(taps_spread_kernel<true, true>); else go(taps_spread_kernel<true, false>); }
   else { if (pair) go(taps_spread_kernel<false, true>); else go(taps_spread_kernel<false, false>); }
+  return true;
 }
 
 bool pw16_taps_plan(const ConvGeom& g, ConvGeom* c, bool wgrad = false) {
@@ -718,6 +752,7 @@ bool pw16_taps_plan(const ConvGeom& g, ConvGeom* c, bool wgrad = false) {
   const bool s1ok = wgrad && g.OW % 2 != 0;
   if (!(g.groups == 1 && T > 1 && T <= 9 && (g.sy > 1 || g.sx > 1 || s1ok))) return false;
   if ((long long)g.N * g.C * T * g.OH * g.OW >= (1ll << 31)) return false;
+  if (g.W > 256 || g.OW > 256) return false;   // a row of the plane per row of threads
   *c = g;
   c->C = g.C * T; c->Cg = c->C;
   c->H = g.OH; c->W = g.OW;
@@ -760,7 +795,7 @@ int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void
     if (!ws || ws_bytes < lattice_bytes(c)) return -1;
     const int rc = launch_pw16<true>(c, dy, w, nullptr, ws, s);
     if (rc != FLHIP_OK) return rc;
-    taps_spread(g, ws, dx, s);
+    if (!taps_spread(g, ws, dx, s)) return fail(FLHIP_RUNTIME_ERROR, "conv2d_bwd_data: plane too wide for the spread kernel");
     return check_launch("conv2d_bwd_data strided window (bf16 mfma)");
   }
   if (!pw16_applies(g)) return -1;
@@ -791,7 +826,7 @@ int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, fl
     const size_t lb = lattice_bytes(g);
     if (!ws || ws_bytes < lb) return fail(FLHIP_INVALID_ARGUMENT, "conv2d_bwd_filter: workspace too small");
     if (strided) lattice_gather(g0, x, ws, s);
-    else taps_gather(g0, x, ws, s);
+    else if (!taps_gather(g0, x, ws, s)) return fail(FLHIP_RUNTIME_ERROR, "conv2d_bwd_filter: plane too wide for the gather kernel");
     x = ws;
     ws = static_cast<char*>(ws) + lb;
     ws_bytes -= lb;
