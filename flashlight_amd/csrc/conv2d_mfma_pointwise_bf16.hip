@@ -528,7 +528,7 @@ bool pw16_wgrad_plan(const ConvGeom& g, Pw16WgradParams* p) {
   if (tiles > 65535) return false;
   // every slice costs a write and a read of the whole gradient: fewer slices for large ones
   // (measured on the ResNet-50 layers)
-  const int mult = p->E >= 100000 ? 2 : 4;
+  const int mult = p->E >= 100000 ? 3 : 4;
   long long ns = (long long)mult * mfma_num_cus() / tiles;
   if (ns > p->nchunks / 4) ns = p->nchunks / 4;    // at least four chunks per slice
   if (ns < 1) ns = 1;
