@@ -78,6 +78,10 @@ MORE = [
     # stride-1 windows over rows of odd length: bf16 filter gradient through gathered taps
     ((4, 64, 7, 7), (72, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
     ((2, 16, 6, 13), (24, 16, 2, 3), (1, 1), (1, 0), (1, 2), 1),
+    # rows wider than the copy kernels' thread layout (256 items): the flat lattice copy for 1x1,
+    # the converting kernels for windows with several taps
+    ((1, 16, 2, 700), (16, 16, 1, 1), (1, 2), (0, 0), (1, 1), 1),
+    ((1, 8, 4, 600), (8, 8, 3, 3), (2, 2), (1, 1), (1, 1), 1),
     # long contractions on small grids (several chunks in flight): 9 and 11 chunks of 32
     ((3, 264, 7, 7), (72, 264, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     ((2, 40, 5, 5), (328, 40, 1, 1), (1, 1), (0, 0), (1, 1), 1),
