@@ -51,6 +51,11 @@ size_t mfma_pointwise16_lattice_ws(const ConvGeom& g, bool bwd);
 size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g);
 int mfma_pointwise16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
                            size_t ws_bytes, hipStream_t s);
+// fp32, stride 1, few tiles and a long contraction: the contraction in slices through
+// mfma_pointwise_split_ws() bytes of workspace; -1 when it does not apply or the room is missing
+size_t mfma_pointwise_split_ws(const ConvGeom& g, int dtype, bool bwd);
+int mfma_pointwise_conv_split(const ConvGeom& g, int dtype, bool bwd, const void* src, const void* w,
+                              const float* bias, void* dst, void* ws, size_t ws_bytes, hipStream_t s);
 // column-major C = op(A) op(B) on the 1x1 kernels (mode 0: A B, 1: A^T B, 2: A B^T);
 // -1 when it does not apply
 int mfma_gemm(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,

@@ -184,7 +184,8 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
   // (bf16: strided 1x1 windows gather the input's lattice points / spread a compact gradient)
   if (pass == FLHIP_CONV_FWD || pass == FLHIP_CONV_BWD_DATA) {
     const size_t a = mfma_tapped_ws(g, d->dtype, pass == FLHIP_CONV_BWD_DATA);
-    const size_t b = d->dtype == FLHIP_BF16 ? mfma_pointwise16_lattice_ws(g, pass == FLHIP_CONV_BWD_DATA) : 0;
+    const size_t b = d->dtype == FLHIP_BF16 ? mfma_pointwise16_lattice_ws(g, pass == FLHIP_CONV_BWD_DATA)
+                                            : pass == FLHIP_CONV_BWD_DATA ? mfma_pointwise_split_ws(g, d->dtype, true) : 0;
     return a > b ? a : b;
   }
   return 0;
@@ -238,6 +239,7 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
       r = mfma_pointwise16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
       r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s);
+    if (r < 0 && !skip("gemm1x1")) r = mfma_pointwise_conv_split(g, d->dtype, true, dy, w, nullptr, dx, ws, ws_bytes, s);
     if (r < 0 && !skip("gemm1x1")) r = mfma_pointwise_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
     if (r < 0 && !skip("slab")) r = mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s);

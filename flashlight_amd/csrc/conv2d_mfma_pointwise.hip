@@ -991,6 +991,48 @@ int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, c
                             : launch_pw<bf16_t, true>(p, vec, dy, w, bias, dx, s);
 }
 
+// ---- split contraction for 1x1 stride-1 fp32 layers with few tiles ----------------------
+// 7x7 planes with 2048 channels to contract: 200 tiles of 64 chunks each on 256 CUs.  With
+// workspace for the partial results the contraction is cut into slices (blockIdx.y of the
+// kernel above; the bias goes with slice 0) that the fixed-order reduction kernel adds.
+// The dispatch uses it for backward-data only (512 -> 2048 channels over 7x7: 91 -> 68 us);
+// forward over the same shapes measured no faster with it (54 -> 56 us).
+// Returns the request to pass as ksplit (1: no split); *slices = partial results written.
+static int pw_split_request(const ConvGeom& g, bool bwd, int* slices) {
+  *slices = 1;
+  if (!pw_applies(g) || g.sy != 1 || g.sx != 1 || g.OH != g.H || g.OW != g.W) return 1;
+  const int Kc = bwd ? g.K : g.C, Mo = bwd ? g.C : g.K;
+  const long long tiles = (((long long)g.N * g.H * g.W + 63) / 64) * ((Mo + BM - 1) / BM);
+  const int chunks = (Kc + KC - 1) / KC;
+  if (chunks < 32 || tiles > mfma_num_cus()) return 1;
+  long long ks = 2ll * mfma_num_cus() / tiles;
+  if (ks > 8) ks = 8;
+  if (ks > chunks / 8) ks = chunks / 8;      // at least 8 chunks per slice
+  if (ks < 2) return 1;
+  *slices = mfma_gemm_slices(Kc, (int)ks);
+  return (int)ks;
+}
+
+size_t mfma_pointwise_split_ws(const ConvGeom& g, int dtype, bool bwd) {
+  int slices;
+  if (dtype != FLHIP_F32 || pw_split_request(g, bwd, &slices) <= 1) return 0;
+  return (size_t)slices * g.N * (bwd ? g.C : g.K) * g.H * g.W * sizeof(float);
+}
+
+int mfma_pointwise_conv_split(const ConvGeom& g, int dtype, bool bwd, const void* src, const void* w,
+                              const float* bias, void* dst, void* ws, size_t ws_bytes, hipStream_t s) {
+  int slices;
+  if (dtype != FLHIP_F32) return -1;
+  const int ks = pw_split_request(g, bwd, &slices);
+  const size_t E = (size_t)g.N * (bwd ? g.C : g.K) * g.H * g.W;
+  if (ks <= 1 || slices <= 1 || !ws || ws_bytes < slices * E * sizeof(float) || E >= (1ull << 31)) return -1;
+  const int rc = bwd ? mfma_pointwise_conv_bwd_data(g, dtype, src, w, ws, s, nullptr, ks)
+                     : mfma_pointwise_conv_fwd(g, dtype, src, w, bias, ws, s, ks);
+  if (rc != FLHIP_OK) return rc;
+  wgrad_reduce_launch(static_cast<const float*>(ws), slices, (int)E, 0, 0, static_cast<float*>(dst), nullptr, s);
+  return check_launch("conv2d 1x1 (split contraction)");
+}
+
 size_t mfma_pointwise_wgrad_ws(const ConvGeom& g) {
   PwWgradParams p{};
   if (!pw_wgrad_plan(g, &p)) return 0;

@@ -82,6 +82,10 @@ MORE = [
     # the converting kernels for windows with several taps
     ((1, 16, 2, 700), (16, 16, 1, 1), (1, 2), (0, 0), (1, 1), 1),
     ((1, 8, 4, 600), (8, 8, 3, 3), (2, 2), (1, 1), (1, 1), 1),
+    # fp32 1x1 backward-data with few tiles and 33 chunks to contract: slices through the workspace,
+    # added in a fixed order (plane of 4k positions, odd plane)
+    ((2, 40, 6, 6), (1056, 40, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((2, 72, 7, 7), (1032, 72, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     # long contractions on small grids (several chunks in flight): 9 and 11 chunks of 32
     ((3, 264, 7, 7), (72, 264, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     ((2, 40, 5, 5), (328, 40, 1, 1), (1, 1), (0, 0), (1, 1), 1),
