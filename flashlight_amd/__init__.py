@@ -13,6 +13,7 @@ from .ops import (  # noqa: F401
     conv2d,
     conv2d_backward_data,
     conv2d_backward_filter_bias,
+    conv2d_backward_filter_bias_static,
     derive_padding,
     pool2d,
     pool2d_backward,

@@ -8,6 +8,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libflhip.so")
 OK, INVALID_ARGUMENT, RUNTIME_ERROR = 0, 1, 2
 F32, BF16 = 0, 1
 CONV_FWD, CONV_BWD_DATA, CONV_BWD_FILTER = 0, 1, 2
+STATIC_SCRATCH_BYTES = 40 << 20      # FLHIP_STATIC_SCRATCH_BYTES
 
 
 class ConvDesc(C.Structure):
@@ -43,6 +44,7 @@ SYMBOLS = {
     "flhip_conv2d_fwd": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
     "flhip_conv2d_bwd_data": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _SZ, _VP]),
     "flhip_conv2d_bwd_filter": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
+    "flhip_conv2d_bwd_filter_static": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _VP]),
     "flhip_pool2d_fwd": (C.c_int, [C.POINTER(PoolDesc), _VP, _VP, _VP, _VP]),
     "flhip_pool2d_bwd": (C.c_int, [C.POINTER(PoolDesc), _VP, _VP, _VP, _VP]),
     "flhip_bn_workspace_bytes": (_SZ, [C.POINTER(BnDesc)]),

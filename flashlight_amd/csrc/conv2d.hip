@@ -5,7 +5,14 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "conv2d.h"
+
+// Scratch of flhip_conv2d_bwd_filter_static: lives in the code object, one copy per
+// device the library is loaded on, never freed.  The name is only a host-side handle;
+// the per-device address comes from hipGetSymbolAddress (static_scratch()).
+static __device__ __align__(256) unsigned char scratch[FLHIP_STATIC_SCRATCH_BYTES];
 
 namespace flhip {
 
@@ -160,6 +167,27 @@ static int make_geom(const flhip_conv_desc* d, ConvGeom* g) {
   return FLHIP_OK;
 }
 
+// Device address of `scratch` on the current device, looked up once per device.
+static int static_scratch(void** out) {
+  enum { MAX_DEVICES = 64 };
+  static std::mutex mu;
+  static void* addr[MAX_DEVICES] = {};
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(FLHIP_RUNTIME_ERROR, std::string("hipGetDevice: ") + hipGetErrorString(e));
+  if (dev < 0 || dev >= MAX_DEVICES) return fail(FLHIP_RUNTIME_ERROR, "static scratch: device index out of range");
+  std::lock_guard<std::mutex> lock(mu);
+  if (!addr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return fail(FLHIP_RUNTIME_ERROR, std::string("hipGetSymbolAddress(scratch): ") + hipGetErrorString(e));
+    addr[dev] = p;
+  }
+  *out = addr[dev];
+  return FLHIP_OK;
+}
+
 }  // namespace flhip
 
 using namespace flhip;
@@ -304,4 +332,25 @@ extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, 
                          static_cast<const bf16_t*>(dy), db);
   }
   return check_launch("conv2d_bwd_filter");
+}
+
+extern "C" int flhip_conv2d_bwd_filter_static(const flhip_conv_desc* d, const void* x, const void* dy,
+                                              float* dw, float* db, void* stream) {
+  FLHIP_REQUIRE(d, "conv2d_bwd_filter_static: null argument");
+  ConvGeom g;
+  const int rc = make_geom(d, &g);
+  if (rc != FLHIP_OK) return rc;
+  const size_t need = flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER);
+  if (need > (size_t)FLHIP_STATIC_SCRATCH_BYTES)
+    return fail(FLHIP_INVALID_ARGUMENT,
+                "conv2d_bwd_filter_static: this geometry needs " + std::to_string(need) +
+                    " bytes of scratch, the static buffer holds " +
+                    std::to_string((size_t)FLHIP_STATIC_SCRATCH_BYTES) +
+                    "; use flhip_conv2d_bwd_filter with a caller workspace");
+  void* ptr = nullptr;
+  const int rs = static_scratch(&ptr);
+  if (rs != FLHIP_OK) return rs;
+  // same plan as the workspace entry point given exactly `need` bytes: every partial
+  // the reduction reads is written by this call first, so nothing has to be cleared
+  return flhip_conv2d_bwd_filter(d, x, dy, dw, db, ptr, need, stream);
 }

@@ -141,6 +141,25 @@ def conv2d_backward_filter_bias(grad_output, input, weights_shape, want_bias, sx
     return dw, db
 
 
+def conv2d_backward_filter_bias_static(grad_output, input, dw, db, sx=1, sy=1, px=0, py=0, dx=1,
+                                       dy=1, groups=1):
+    """flhip_conv2d_bwd_filter_static: the filter / bias gradient written into the
+    caller's fp32 tensors `dw` (weight shape) and `db` (or None), with the partial
+    results in the library's static buffer.  Neither this wrapper nor the library
+    allocates device memory."""
+    g, x = _dev(grad_output, "gradOutput"), _dev(input, "input")
+    if dw.dtype != torch.float32 or (db is not None and db.dtype != torch.float32):
+        raise ValueError("conv2dBackwardFilterBias: gradients are fp32")
+    d = _conv_desc(x.shape, tuple(dw.shape), sx, sy, px, py, dx, dy, groups, _dtype_tag(x))
+    oh, ow = C.c_int32(), C.c_int32()
+    capi.check(capi.lib().flhip_conv2d_out_dims(C.byref(d), C.byref(oh), C.byref(ow)))
+    if tuple(g.shape) != (d.N, d.K, oh.value, ow.value):
+        raise ValueError("conv2dBackwardFilterBias: gradOutput shape does not match the geometry")
+    capi.check(capi.lib().flhip_conv2d_bwd_filter_static(C.byref(d), _ptr(x), _ptr(g), _ptr(dw),
+                                                         _ptr(db), _stream()))
+    return dw, db
+
+
 def _pool_desc(x_shape4, wx, wy, sx, sy, px, py, mode, tag):
     N, Cc, H, W = x_shape4
     return capi.PoolDesc(N, Cc, H, W, wy, wx, sy, sx, py, px, int(mode), tag)

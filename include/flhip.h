@@ -140,6 +140,21 @@ int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x,
                             const void* dy, float* dw, float* db, void* ws,
                             size_t ws_bytes, void* stream);
 
+/* The same filter / bias gradient for callers that cannot allocate device memory (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It
+ * has no counterpart in the reference.  The partial results of the sliced contraction
+ * go to a buffer of FLHIP_STATIC_SCRATCH_BYTES that is part of the library's code
+ * object (each GPU the library runs on holds one copy until the process ends); no
+ * hipMalloc / hipFree or other allocating call is made.  Geometries whose
+ * flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER) exceeds that size are refused
+ * with FLHIP_INVALID_ARGUMENT.  Results are bit-identical to flhip_conv2d_bwd_filter.
+ * The device of `stream` must be the current device.  All calls on one GPU share the
+ * buffer: calls that overlap in time on one GPU (different streams, or threads) race. */
+#define FLHIP_STATIC_SCRATCH_BYTES (40u << 20)
+int flhip_conv2d_bwd_filter_static(const flhip_conv_desc* d, const void* x,
+                                   const void* dy, float* dw, float* db,
+                                   void* stream);
+
 /* AutogradExtension::pool2d (AutogradExtension.h:71-80; oneDNN peer
  * onednn/Pool2D.cpp:78-176).  For FLHIP_POOL_MAX with argmax != NULL the kernel
  * also writes one byte per output: the window-relative index kh*wx + kw of the
