@@ -129,6 +129,37 @@ def test_errors():
         fa.batchnorm(x, torch.zeros(5, device="cuda"), None, None, None, [2], True, 0.0, 1e-5)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_full_size_oracle(dtype):
+    """configs[2] at its stated size (56x56x256, batch 32, values N(0.5, 2), gamma N(1, 0.1),
+    eps 1e-5, momentum 0.1): y, saved statistics, running statistics, dx, dgamma, dbeta
+    against the CPU checker, whole tensors."""
+    rng = np.random.default_rng(57)
+    N, Cc, HW = 32, 256, 56 * 56
+    x = (rng.standard_normal((N, Cc, 56, 56), dtype=np.float32) * np.float32(2 ** 0.5) + np.float32(0.5))
+    dy = rng.standard_normal((N, Cc, 56, 56), dtype=np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(Cc)).astype(np.float32)
+    beta = np.zeros(Cc, np.float32)
+    lo = dtype == torch.bfloat16
+    if lo:
+        x, dy = bf16_round(x), bf16_round(dy)
+    y_ref, mean, var = flref.bn_fwd_train(N, Cc, HW, x, gamma, beta, 1e-5)
+    dx_ref, dg_ref, db_ref = flref.bn_bwd(N, Cc, HW, x, dy, gamma, mean, var, 1e-5)
+    rm, rv = torch.zeros(Cc, device="cuda"), torch.ones(Cc, device="cuda")
+    xd, dyd = dev(x, dtype), dev(dy, dtype)
+    y, sm, si = fa.batchnorm(xd, dev(gamma), dev(beta), rm, rv, [2], True, 0.1, 1e-5)
+    dx, dg, db = fa.batchnorm_backward(dyd, xd, dev(gamma), sm, si, [2])
+    tol = 4e-3 if lo else 1e-4
+    assert rel_l2(host(y), y_ref) <= tol
+    assert rel_l2(host(dx), dx_ref) <= tol
+    assert rel_l2(host(dg), dg_ref) <= 1e-4 and rel_l2(host(db), db_ref) <= 1e-4
+    assert rel_l2(host(sm), mean) <= 1e-5
+    assert rel_l2(host(si), 1 / np.sqrt(var.astype(np.float64) + 1e-5)) <= 1e-5
+    M = N * HW
+    assert rel_l2(host(rm), 0.1 * mean) <= 1e-5
+    assert rel_l2(host(rv), 0.9 + 0.1 * var.astype(np.float64) * M / (M - 1)) <= 1e-5
+
+
 def test_full_size_invariants():
     # cfg-3 shape: per-feature sums of dx and of dx*xhat vanish; y has zero mean
     # and unit variance per feature.

@@ -194,14 +194,14 @@ def test_layer_norm_needs_contiguous_complement():
 
 
 
-def test_mnist_convnet_training_step():
+@pytest.mark.parametrize("B", [16, 64])
+def test_mnist_convnet_training_step(B):
     """configs[0]: View, Conv2D 1->32 5x5 SAME, ReLU, Pool2D max 2x2 s2, Conv2D 32->64 5x5
     SAME, ReLU, Pool2D, View, Linear 3136->1024, ReLU, Linear 1024->10, LogSoftmax, then
     categoricalCrossEntropy (reference README); dropout left out (it is a random mask, not
     part of the path).  Forward and the gradient closures in tape order, device against
     oracle, every parameter gradient compared."""
-    rng = np.random.default_rng(80)
-    B = 16
+    rng = np.random.default_rng(80)       # batch 64 is the size configs[0] states
     x = rng.standard_normal((B, 1, 28, 28)).astype(np.float32)
     labels = rng.integers(0, 10, B).astype(np.int32)
     P = _mnist_params(rng)

@@ -286,11 +286,12 @@ def test_invalid_arguments_raise():
 
 
 # ---- full sizes of the BASELINE configurations ------------------------------------------
-# The CPU checker needs minutes at these sizes, so the device results are checked through
-# what does not depend on size: (1) randomly sampled result elements against their defining
-# sums written with torch indexing in float64 (shares no code with the kernels or the C
-# checker), (2) the adjoint identities <conv(x, w), dy> = <x, bwdData(dy, w)> = <w, bwdFilter(x, dy)>
-# over the whole tensors, (3) a one-tap identity filter reproduces the shifted input bit for bit.
+# Two kinds of checks at these sizes.  test_full_size_oracle compares whole results with the CPU
+# checker (a pass takes it 0.2 - 3 s).  test_full_size_properties checks what does not depend on
+# the checker at all: (1) randomly sampled result elements against their defining sums written
+# with torch indexing in float64 (shares no code with the kernels or the C checker), (2) the
+# adjoint identities <conv(x, w), dy> = <x, bwdData(dy, w)> = <w, bwdFilter(x, dy)> over the whole
+# tensors, (3) a one-tap identity filter reproduces the shifted input bit for bit.
 FULL = [
     # x NCHW, w KCHW, stride, pad: configs[1] (the bench shape), then layers of configs[4] / configs[3]
     ((32, 64, 56, 56), (64, 64, 3, 3), (1, 1), (1, 1)),
@@ -302,7 +303,22 @@ FULL = [
     ((32, 2048, 7, 7), (512, 2048, 1, 1), (1, 1), (0, 0)),
     ((32, 3, 224, 224), (64, 3, 7, 7), (2, 2), (3, 3)),
     ((16, 250, 1, 1500), (250, 250, 1, 21), (1, 2), (0, 10)),
+    # the other two layers of configs[3]
+    ((16, 80, 1, 1500), (250, 80, 1, 21), (1, 1), (0, 10)),
+    ((16, 250, 1, 1500), (250, 250, 1, 21), (1, 1), (0, 10)),
 ]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", FULL)
+def test_full_size_oracle(shape, dtype):
+    """y, dx, dw, db of every full-size layer against the CPU checker, whole tensors."""
+    xs, ws, st, pd = shape
+    lo = dtype == torch.bfloat16
+    for name, (got, ref) in _run((xs, ws, st, pd, (1, 1), 1), 43, dtype).items():
+        tol = (1e-4 if name in ("dw", "db") else 4e-3) if lo else F32_TOL
+        assert got.shape == ref.shape, name
+        assert rel_l2(got, ref) <= tol, (name, rel_l2(got, ref))
 
 
 def _sampled_refs(x, w, b, dy, st, pd, rng, nsamp=48):
@@ -339,8 +355,6 @@ def _sampled_refs(x, w, b, dy, st, pd, rng, nsamp=48):
 @pytest.mark.parametrize("shape", FULL)
 def test_full_size_properties(shape, dtype):
     xs, ws, st, pd = shape
-    if dtype == torch.bfloat16 and shape is not FULL[0] and shape is not FULL[3]:
-        pytest.skip("bf16 at full size: the bench shape and one strided layer")
     rng = np.random.default_rng(41)
     gen = torch.Generator(device="cuda").manual_seed(41)
     x = torch.randn(xs, device="cuda", generator=gen).to(dtype)

@@ -92,10 +92,34 @@ def test_backward_without_payload_raises():
         fa.pool2d_backward(dy, (1, 1, 8, 8), None, 2, 2, 2, 2, 0, 0, mode=0)
 
 
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_full_size_oracle(mode):
+    """configs[2] at its stated size (112x112x64, batch 32, values on a 1/8 grid so that ties
+    occur in most windows): values, argmax bytes and the routed gradient bit for bit against
+    the CPU checker."""
+    rng = np.random.default_rng(46)
+    x = (np.round(rng.standard_normal((32, 64, 112, 112), dtype=np.float32) * 8) / 8).astype(np.float32)
+    dy = rng.standard_normal((32, 64, 56, 56), dtype=np.float32)
+    d = flref.pool_desc(x.shape, (3, 3), (2, 2), (1, 1), mode)
+    y_ref, am_ref = flref.pool2d_fwd(d, x)
+    dx_ref = flref.pool2d_bwd(d, dy, am_ref)
+    y, am = fa.pool2d(dev(x), 3, 3, 2, 2, 1, 1, mode=mode)
+    dx = fa.pool2d_backward(dev(dy), x.shape, am, 3, 3, 2, 2, 1, 1, mode=mode)
+    assert np.array_equal(host(y), y_ref)
+    if mode == 0:
+        am_h = am.cpu().numpy()
+        assert np.array_equal(am_h, am_ref)
+        # the grid does produce ties: count windows whose maximum occurs more than once
+        xp = np.pad(x[:2], ((0, 0), (0, 0), (1, 1), (1, 1)), constant_values=-np.inf)
+        hits = sum((xp[:, :, kh:kh + 111:2, kw:kw + 111:2] == y_ref[:2]).astype(np.int32)
+                   for kh in range(3) for kw in range(3))
+        assert (hits >= 2).mean() > 0.05
+    assert np.array_equal(host(dx), dx_ref)
+
+
 def test_full_size_properties():
-    # cfg-3 size: gradient mass is conserved and idempotence of max over its
-    # own output positions; sizes the CPU checker would take too long on are
-    # covered by these size-independent properties.
+    # cfg-3 size, independent of the checker: gradient mass is conserved and
+    # max-pooling routes every output to a position that holds its value.
     g = torch.Generator(device="cuda").manual_seed(45)
     x = torch.round(torch.randn((32, 64, 112, 112), device="cuda", generator=g) * 8) / 8
     dy = torch.randn((32, 64, 56, 56), device="cuda", generator=g)
