@@ -42,45 +42,53 @@ HOST = os.path.join(HERE, "host")
 HOST_LIB = os.path.join(LIBDIR, "libflhip_host.so")
 HOST_SOURCES = ["HipTensor.cpp", "HipAutogradExtension.cpp", "Functions.cpp", "Modules.cpp", "Resnet.cpp",
                 "SequentialBuilder.cpp"]
-HOST_TEST_SRC = os.path.join(ROOT, "tests", "cpp", "test_host_extension.cpp")
-HOST_TEST_BIN = os.path.join(ROOT, "tests", "cpp", "bin", "test_host_extension")
+TESTS_DIR = os.path.join(ROOT, "tests", "cpp")
+TESTS_BIN = os.path.join(TESTS_DIR, "bin")
+# test program -> links the CPU checker?
+TEST_PROGRAMS = {"test_host_extension": True, "test_resnet_step": True, "test_jacobian": False}
 
 
-def build_host(verbose=True):
-    """The C++ host layer (HipTensor, HipAutogradExtension, caller closures) and its
-    test program; both link libflhip.so, the test also links the CPU checker."""
+def _host_cxx():
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
     cxx = [os.environ.get("CXX", "g++"), "-O2", "-g", "-rdynamic", "-std=c++17", "-Wall", "-D__HIP_PLATFORM_AMD__",
            "-I" + os.path.join(rocm, "include"), "-I" + os.path.join(ROOT, "include"), "-I" + HOST]
     hiplibs = ["-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(rocm, "lib")]
+    return cxx, hiplibs
+
+
+def build_host(verbose=True):
+    """The C++ host layer (HipTensor, HipAutogradExtension, caller closures, modules):
+    libflhip_host.so, linked against libflhip.so.  Needs nothing outside the package."""
+    cxx, hiplibs = _host_cxx()
     cmd = cxx + ["-fPIC", "-shared", "-o", HOST_LIB]
     cmd += [os.path.join(HOST, f) for f in HOST_SOURCES]
     cmd += ["-L" + LIBDIR, "-lflhip", "-Wl,-rpath,$ORIGIN"] + hiplibs
     subprocess.check_call(cmd)
-    if os.path.exists(HOST_TEST_SRC):
-        os.makedirs(os.path.dirname(HOST_TEST_BIN), exist_ok=True)
-        oracle = os.path.join(ROOT, "oracle")
-        subprocess.check_call(["make", "-C", oracle, "libflref.so"], stdout=subprocess.DEVNULL)
-        cmd = cxx + ["-I" + oracle, "-o", HOST_TEST_BIN, HOST_TEST_SRC,
-                     "-L" + LIBDIR, "-lflhip_host", "-lflhip", "-L" + oracle, "-lflref",
-                     "-Wl,-rpath,$ORIGIN/../../../flashlight_amd/lib",
-                     "-Wl,-rpath,$ORIGIN/../../../oracle"] + hiplibs
-        subprocess.check_call(cmd)
-        # the ResNet-50 step program needs no CPU checker
-        rsrc = os.path.join(os.path.dirname(HOST_TEST_SRC), "test_resnet_step.cpp")
-        rbin = os.path.join(os.path.dirname(HOST_TEST_BIN), "test_resnet_step")
-        cmd = cxx + ["-o", rbin, rsrc, "-L" + LIBDIR, "-lflhip_host", "-lflhip",
-                     "-Wl,-rpath,$ORIGIN/../../../flashlight_amd/lib"] + hiplibs
-        subprocess.check_call(cmd)
-        # neither do the finite-difference Jacobian tests
-        jsrc = os.path.join(os.path.dirname(HOST_TEST_SRC), "test_jacobian.cpp")
-        jbin = os.path.join(os.path.dirname(HOST_TEST_BIN), "test_jacobian")
-        cmd = cxx + ["-o", jbin, jsrc, "-L" + LIBDIR, "-lflhip_host", "-lflhip",
-                     "-Wl,-rpath,$ORIGIN/../../../flashlight_amd/lib"] + hiplibs
-        subprocess.check_call(cmd)
     if verbose:
         print("built", HOST_LIB)
     return HOST_LIB
+
+
+def build_tests(verbose=True):
+    """The C++ test programs under tests/cpp (not part of the product): they link the two
+    libraries above and, where they compare with it, the CPU checker oracle/libflref.so."""
+    cxx, hiplibs = _host_cxx()
+    os.makedirs(TESTS_BIN, exist_ok=True)
+    oracle = os.path.join(ROOT, "oracle")
+    subprocess.check_call(["make", "-C", oracle, "libflref.so"], stdout=subprocess.DEVNULL)
+
+    def one(item):
+        name, with_checker = item
+        cmd = cxx + ["-o", os.path.join(TESTS_BIN, name), os.path.join(TESTS_DIR, name + ".cpp"),
+                     "-L" + LIBDIR, "-lflhip_host", "-lflhip", "-Wl,-rpath,$ORIGIN/../../../flashlight_amd/lib"]
+        if with_checker:
+            cmd += ["-I" + oracle, "-L" + oracle, "-lflref", "-Wl,-rpath,$ORIGIN/../../../oracle"]
+        subprocess.check_call(cmd + hiplibs)
+        return name
+    with ThreadPoolExecutor(max_workers=3) as ex:
+        names = list(ex.map(one, TEST_PROGRAMS.items()))
+    if verbose:
+        print("built", ", ".join(names))
 
 
 def build(verbose=True):
@@ -98,3 +106,5 @@ def build(verbose=True):
 
 if __name__ == "__main__":
     build()
+    if os.path.isdir(TESTS_DIR):
+        build_tests()

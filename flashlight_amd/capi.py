@@ -38,6 +38,7 @@ SYMBOLS = {
     "flhip_last_error": (C.c_char_p, []),
     "flhip_version": (C.c_int, []),
     "flhip_arch": (C.c_char_p, []),
+    "flhip_set_option": (C.c_int, [C.c_char_p, C.c_char_p]),
     "flhip_conv2d_out_dims": (C.c_int, [C.POINTER(ConvDesc), _I32P, _I32P]),
     "flhip_pool2d_out_dims": (C.c_int, [C.POINTER(PoolDesc), _I32P, _I32P]),
     "flhip_conv2d_workspace_bytes": (_SZ, [C.POINTER(ConvDesc), C.c_int]),
@@ -56,6 +57,7 @@ SYMBOLS = {
                                 _SZ, _VP]),
     "flhip_copy_bytes": (C.c_int, [_VP, _VP, _SZ, _VP]),
     "flhip_convert": (C.c_int, [_VP, C.c_int, _VP, C.c_int, _SZ, _VP]),
+    "flhip_fill": (C.c_int, [_VP, C.c_double, _SZ, C.c_int, _VP]),
     "flhip_add": (C.c_int, [_VP, _VP, _VP, _SZ, C.c_int, _VP]),
     "flhip_relu_fwd": (C.c_int, [_VP, _VP, _SZ, C.c_int, _VP]),
     "flhip_relu_bwd": (C.c_int, [_VP, _VP, _VP, _SZ, C.c_int, _VP]),
@@ -108,3 +110,8 @@ def check(rc):
     if rc == INVALID_ARGUMENT:
         raise ValueError(msg)      # std::invalid_argument
     raise RuntimeError(msg)        # std::runtime_error
+
+
+def set_option(name, value=None):
+    """flhip_set_option: a measurement / debugging switch (value None = default)."""
+    check(lib().flhip_set_option(name.encode(), None if value is None else str(value).encode()))

@@ -1,7 +1,84 @@
 // Error state, version and the calibration copy kernel of the C ABI.
+#include <stdlib.h>
+#include <string.h>
+
+#include <mutex>
+
 #include "common.h"
 
 namespace flhip {
+
+// ---- process-wide switches ----
+static Options g_options;
+static std::once_flag g_options_once;
+
+// One switch from its text; value == nullptr restores the default.  false: unknown name or value.
+static bool apply_option(Options& o, const char* name, const char* v) {
+  const Options def;
+  auto flag = [&](bool* f) {
+    *f = v != nullptr && strcmp(v, "0") != 0;
+    return true;
+  };
+  if (!strcmp(name, "CONV_ALGO")) {
+    if (!v || !*v) o.conv_algo = def.conv_algo;
+    else if (!strcmp(v, "direct")) o.conv_algo = Options::ALGO_DIRECT;
+    else if (!strcmp(v, "gather")) o.conv_algo = Options::ALGO_GATHER;
+    else if (!strcmp(v, "tapped")) o.conv_algo = Options::ALGO_TAPPED;
+    else if (!strcmp(v, "convert")) o.conv_algo = Options::ALGO_CONVERT;
+    else if (!strcmp(v, "auto")) o.conv_algo = Options::ALGO_AUTO;
+    else return false;
+    return true;
+  }
+  if (!strcmp(name, "CONV_SKIP")) {
+    unsigned m = 0;
+    if (v) {
+      if (strstr(v, "bf16")) m |= Options::SKIP_BF16;
+      if (strstr(v, "gemm1x1")) m |= Options::SKIP_GEMM1X1;
+      if (strstr(v, "slab")) m |= Options::SKIP_SLAB;
+      if (strstr(v, "tapped")) m |= Options::SKIP_TAPPED;
+    }
+    o.conv_skip = m;
+    return true;
+  }
+  if (!strcmp(name, "PW_PT")) {
+    const int n = v ? atoi(v) : def.pw_pt;
+    if (n != 2 && n != 4 && n != 8) return false;
+    o.pw_pt = n;
+    return true;
+  }
+  if (!strcmp(name, "PW16_PF")) {
+    const int n = v ? atoi(v) : 0;
+    if (n != 0 && n != 1 && n != 4) return false;
+    o.pw16_pf = n;
+    return true;
+  }
+  if (!strcmp(name, "BN_ALGO")) {
+    if (!v || !*v || !strcmp(v, "auto")) o.bn_algo = 0;
+    else if (!strcmp(v, "split")) o.bn_algo = 1;
+    else if (!strcmp(v, "resident")) o.bn_algo = 2;
+    else return false;
+    return true;
+  }
+  if (!strcmp(name, "PW16_NO_TAPS")) return flag(&o.pw16_no_taps);
+  if (!strcmp(name, "TAPPED_NO_REORDER")) return flag(&o.tapped_no_reorder);
+  if (!strcmp(name, "MATMUL_VALU")) return flag(&o.matmul_valu);
+  if (!strcmp(name, "RNN_UNFUSED")) return flag(&o.rnn_unfused);
+  return false;
+}
+
+static void options_from_environment() {
+  static const char* const names[] = {"CONV_ALGO", "CONV_SKIP", "PW_PT", "PW16_PF", "BN_ALGO", "PW16_NO_TAPS",
+                                      "TAPPED_NO_REORDER", "MATMUL_VALU", "RNN_UNFUSED"};
+  for (const char* n : names) {
+    const std::string var = std::string("FLHIP_") + n;
+    if (const char* v = getenv(var.c_str())) apply_option(g_options, n, v);   // unknown values keep the default
+  }
+}
+
+const Options& options() {
+  std::call_once(g_options_once, options_from_environment);
+  return g_options;
+}
 
 static thread_local std::string g_last_error;
 
@@ -27,6 +104,12 @@ __global__ void __launch_bounds__(256) convert_kernel(const S* __restrict__ src,
     st(dst, i, ld(src, i));
 }
 
+template <typename D>
+__global__ void __launch_bounds__(256) fill_kernel(D* __restrict__ dst, float value, size_t n) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) st(dst, i, value);
+}
+
 struct OpAdd {
   __device__ float operator()(float a, float b) const { return a + b; }
 };
@@ -38,6 +121,16 @@ using namespace flhip;
 extern "C" const char* flhip_last_error(void) { return g_last_error.c_str(); }
 extern "C" int flhip_version(void) { return 100; }
 extern "C" const char* flhip_arch(void) { return "gfx950"; }
+
+extern "C" int flhip_set_option(const char* name, const char* value) {
+  FLHIP_REQUIRE(name, "set_option: null name");
+  options();   // the environment is read first, so a later first use cannot undo this call
+  if (!strncmp(name, "FLHIP_", 6)) name += 6;
+  if (!apply_option(g_options, name, value))
+    return fail(FLHIP_INVALID_ARGUMENT, std::string("set_option: unknown switch or value: ") + name + "=" +
+                                            (value ? value : "(null)"));
+  return FLHIP_OK;
+}
 
 extern "C" int flhip_conv2d_out_dims(const flhip_conv_desc* d, int32_t* OH, int32_t* OW) {
   FLHIP_REQUIRE(d && OH && OW, "conv2d_out_dims: null argument");
@@ -105,6 +198,21 @@ extern "C" int flhip_convert(const void* src, int src_dtype, void* dst, int dst_
   else
     hipLaunchKernelGGL((convert_kernel<bf16_t, bf16_t>), grid, block, 0, s, (const bf16_t*)src, (bf16_t*)dst, n);
   return check_launch("convert");
+}
+
+extern "C" int flhip_fill(void* dst, double value, size_t n, int dtype, void* stream) {
+  FLHIP_REQUIRE(dtype_ok(dtype), "fill: unknown dtype");
+  if (n == 0) return FLHIP_OK;
+  FLHIP_REQUIRE(dst, "fill: null pointer");
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  if (dtype == FLHIP_F32)
+    hipLaunchKernelGGL((fill_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), (float*)dst,
+                       (float)value, n);
+  else
+    hipLaunchKernelGGL((fill_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), (bf16_t*)dst,
+                       (float)value, n);
+  return check_launch("fill");
 }
 
 extern "C" int flhip_add(const void* a, const void* b, void* out, size_t n, int dtype,

@@ -743,12 +743,7 @@ struct ResPlan {
   int threads, k, need;
 };
 static ResPlan resident_plan(const BnGeom& g, int vec, int min_c) {
-  static const int mode = [] {
-    const char* e = getenv("FLHIP_BN_ALGO");
-    if (e && !strcmp(e, "split")) return 1;
-    if (e && !strcmp(e, "resident")) return 2;
-    return 0;
-  }();
+  const int mode = options().bn_algo;
   ResPlan r{0, 0, 0};
   if (mode == 1 || vec == 0) return r;
   if (vec == 1) {

@@ -422,11 +422,11 @@ extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, in
   FLHIP_REQUIRE(dtype_ok(dtype), "matmul: unknown dtype");
   // the matrix-core kernels of the 1x1 convolutions take the three products fl::linear
   // needs; the tiled vector-ALU kernel below covers the rest
-  if (!trans_a && trans_b && !bias_rows && !getenv("FLHIP_MATMUL_VALU")) {
+  if (!trans_a && trans_b && !bias_rows && !options().matmul_valu) {
     const int rc = gemm_nt(dtype, A, B, C, M, N, K, 1, as_stream(stream));
     if (rc >= 0) return rc;
   }
-  if (!(trans_a && trans_b) && !getenv("FLHIP_MATMUL_VALU")) {
+  if (!(trans_a && trans_b) && !options().matmul_valu) {
     const int rc = mfma_gemm(dtype, trans_a ? 1 : trans_b ? 2 : 0, A, B, C, M, N, K, bias_rows,
                              as_stream(stream));
     if (rc >= 0) return rc;

@@ -201,6 +201,25 @@ inline void launch_elementwise(const T* a, const T* b, T* out, size_t n, Op op, 
                        out + done, n - done, op);
 }
 
+// ---- process-wide switches ---------------------------------------------------------
+// Measurement / debugging aids.  They are read from the environment (FLHIP_<NAME>) once,
+// when the library first needs them, and can be changed afterwards only through
+// flhip_set_option(); no entry point calls getenv on its per-call path.
+struct Options {
+  enum { ALGO_AUTO = 0, ALGO_DIRECT, ALGO_GATHER, ALGO_TAPPED, ALGO_CONVERT };
+  enum { SKIP_BF16 = 1, SKIP_GEMM1X1 = 2, SKIP_SLAB = 4, SKIP_TAPPED = 8 };
+  int conv_algo = ALGO_AUTO;      // CONV_ALGO = direct | gather | tapped | convert
+  unsigned conv_skip = 0;         // CONV_SKIP = comma list of bf16, gemm1x1, slab, tapped
+  int pw_pt = 2;                  // PW_PT = 2 | 4 | 8: position-tile width of the fp32 1x1 kernels / 32
+  int pw16_pf = 0;                // PW16_PF = 1 | 4: chunks in flight in the bf16 1x1 kernels (0: by grid size)
+  bool pw16_no_taps = false;      // PW16_NO_TAPS: bf16 windows with several taps stay off the gathered-taps path
+  bool tapped_no_reorder = false; // TAPPED_NO_REORDER: tapped kernels read the original weight layout
+  bool matmul_valu = false;       // MATMUL_VALU: flhip_matmul stays off the matrix cores
+  bool rnn_unfused = false;       // RNN_UNFUSED: two-kernel rnn steps
+  int bn_algo = 0;                // BN_ALGO = split (1) | resident (2)
+};
+const Options& options();
+
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
 inline bool dtype_ok(int32_t dt) { return dt == FLHIP_F32 || dt == FLHIP_BF16; }

@@ -1,10 +1,7 @@
 // conv2d / conv2dBackwardData / conv2dBackwardFilterBias entry points, and the
 // direct (one thread per result) kernels that cover every geometry.  The MFMA
 // implicit-GEMM kernels in conv2d_mfma.hip are used whenever they accept the
-// shape; FLHIP_CONV_ALGO=direct in the environment forces the kernels here.
-#include <stdlib.h>
-#include <string.h>
-
+// shape; the switch CONV_ALGO=direct forces the kernels here.
 #include <mutex>
 
 #include "conv2d.h"
@@ -127,20 +124,17 @@ conv_bwd_bias_kernel(ConvGeom g, const T* __restrict__ dy, float* __restrict__ d
   if (threadIdx.x == 0) db[k] = acc;
 }
 
-// FLHIP_CONV_ALGO: "direct" = one-thread-per-result kernels, "gather" = skip the
-// LDS-slab kernels, "convert" = skip the bf16 matrix-core kernels (bf16 storage is
-// then converted on load and multiplied in fp32); anything else = fastest applicable.
-static bool algo_is(const char* name) {
-  const char* e = getenv("FLHIP_CONV_ALGO");
-  return e && strcmp(e, name) == 0;
+// Switch CONV_ALGO: direct = one-thread-per-result kernels, gather = skip the LDS-slab
+// kernels, convert = skip the bf16 matrix-core kernels (bf16 storage is then converted on
+// load and multiplied in fp32), tapped = prefer the tapped GEMM; otherwise the fastest
+// applicable.  CONV_SKIP leaves kernel families out of the dispatch.
+static bool algo_is(int a) { return options().conv_algo == a; }
+static bool force_direct() { return algo_is(Options::ALGO_DIRECT); }
+static bool skip(unsigned family) {
+  return algo_is(Options::ALGO_GATHER) || (options().conv_skip & family) != 0;
 }
-static bool force_direct() { return algo_is("direct"); }
-// FLHIP_CONV_SKIP = comma list of kernel families to leave out of the dispatch
-// (bf16, gemm1x1, slab, tapped): a measurement / debugging aid like FLHIP_CONV_ALGO
-static bool skip(const char* name) {
-  const char* e = getenv("FLHIP_CONV_SKIP");
-  return algo_is("gather") || (e && strstr(e, name) != nullptr);
-}
+static const unsigned SK_BF16 = Options::SKIP_BF16, SK_GEMM = Options::SKIP_GEMM1X1, SK_SLAB = Options::SKIP_SLAB,
+                      SK_TAPPED = Options::SKIP_TAPPED;
 
 // Stride-1 windows over long rows (the 21x1 speech layers: rows of 1500): the gather
 // kernel's one-position-per-thread loads are whole contiguous runs there and it
@@ -148,7 +142,7 @@ static bool skip(const char* name) {
 // With its weights reordered (workspace present) the tapped GEMM wins from 128 contraction
 // channels on.
 static bool long_rows(const ConvGeom& g, int dtype, bool bwd, size_t ws_bytes) {
-  if (algo_is("tapped")) return false;
+  if (algo_is(Options::ALGO_TAPPED)) return false;
   const size_t need = mfma_tapped_ws(g, dtype, bwd);
   if (need && ws_bytes >= need && (bwd ? g.K : g.C) >= 128) return false;
   return g.sy == 1 && g.sx == 1 && g.OW >= 64 && (!bwd || g.C >= 128);
@@ -229,14 +223,14 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
   hipStream_t s = as_stream(stream);
   if (!force_direct()) {
     int r = -1;
-    if (d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
+    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pointwise16_conv_fwd(g, x, w, bias, y, s, ws, ws_bytes);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_slab16_conv_fwd(g, x, w, bias, y, s);
-    if (r < 0 && !skip("gemm1x1")) r = mfma_pointwise_conv_fwd(g, d->dtype, x, w, bias, y, s);
-    if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s, ws, ws_bytes);
-    if (r < 0 && !skip("slab")) r = mfma_slab_conv_fwd(g, d->dtype, x, w, bias, y, s);
-    if (r < 0 && !skip("tapped") && !long_rows(g, d->dtype, false, ws ? ws_bytes : 0))
+    if (r < 0 && !skip(SK_GEMM)) r = mfma_pointwise_conv_fwd(g, d->dtype, x, w, bias, y, s);
+    if (r < 0 && algo_is(Options::ALGO_TAPPED)) r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s, ws, ws_bytes);
+    if (r < 0 && !skip(SK_SLAB)) r = mfma_slab_conv_fwd(g, d->dtype, x, w, bias, y, s);
+    if (r < 0 && !skip(SK_TAPPED) && !long_rows(g, d->dtype, false, ws ? ws_bytes : 0))
       r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s, ws, ws_bytes);
     if (r < 0) r = mfma_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r >= 0) return r;
@@ -263,15 +257,15 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
   hipStream_t s = as_stream(stream);
   if (!force_direct()) {
     int r = -1;
-    if (d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
+    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pointwise16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s);
-    if (r < 0 && !skip("gemm1x1")) r = mfma_pointwise_conv_split(g, d->dtype, true, dy, w, nullptr, dx, ws, ws_bytes, s);
-    if (r < 0 && !skip("gemm1x1")) r = mfma_pointwise_conv_bwd_data(g, d->dtype, dy, w, dx, s);
-    if (r < 0 && algo_is("tapped")) r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
-    if (r < 0 && !skip("slab")) r = mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s);
-    if (r < 0 && !skip("tapped") && !long_rows(g, d->dtype, true, ws ? ws_bytes : 0))
+    if (r < 0 && !skip(SK_GEMM)) r = mfma_pointwise_conv_split(g, d->dtype, true, dy, w, nullptr, dx, ws, ws_bytes, s);
+    if (r < 0 && !skip(SK_GEMM)) r = mfma_pointwise_conv_bwd_data(g, d->dtype, dy, w, dx, s);
+    if (r < 0 && algo_is(Options::ALGO_TAPPED)) r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
+    if (r < 0 && !skip(SK_SLAB)) r = mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s);
+    if (r < 0 && !skip(SK_TAPPED) && !long_rows(g, d->dtype, true, ws ? ws_bytes : 0))
       r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
     if (r < 0) r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r >= 0) return r;
@@ -303,14 +297,14 @@ extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, 
     const size_t need = flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER);
     FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter: workspace too small");
     int r = -1;
-    if (d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
+    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pointwise16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip("bf16") && !algo_is("convert"))
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_wgrad16(g, x, dy, dw, db, ws, ws_bytes, s);
-    if (r < 0 && !skip("gemm1x1"))
-      r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, algo_is("tapped"), s);
-    if (r < 0 && !skip("slab")) r = mfma_slab_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
-    if (r < 0 && !skip("tapped")) r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, true, s);
+    if (r < 0 && !skip(SK_GEMM))
+      r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, algo_is(Options::ALGO_TAPPED), s);
+    if (r < 0 && !skip(SK_SLAB)) r = mfma_slab_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
+    if (r < 0 && !skip(SK_TAPPED)) r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, true, s);
     if (r < 0) r = mfma_conv_bwd_filter(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
     if (r >= 0) return r;
   }

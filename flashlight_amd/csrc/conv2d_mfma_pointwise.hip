@@ -345,12 +345,8 @@ int launch_pw(const PwParams& p, bool vec, const void* src, const void* wgt, con
   // 64 x 64 tiles: four workgroups share a CU (39 KB of LDS each), so the load
   // latency at the start of one tile and the stores at its end overlap the MFMA phase
   // of the others; measured faster than 64 x 128 and 64 x 256 on every ResNet-50 1x1
-  // layer (FLHIP_PW_PT=4|8 selects those, a measurement aid)
-  int pt = 2;
-  if (const char* e = getenv("FLHIP_PW_PT")) {
-    const int v = atoi(e);
-    if (v == 2 || v == 4 || v == 8) pt = v;
-  }
+  // layer (the switch PW_PT=4|8 selects those, a measurement aid)
+  const int pt = options().pw_pt;
   if (vec) {
     if (pt == 8) return launch_tile<T, BWD, 8, true>(p, src, wgt, bias, dst, s);
     if (pt == 4) return launch_tile<T, BWD, 4, true>(p, src, wgt, bias, dst, s);
@@ -644,7 +640,7 @@ int launch_tapped(const ConvGeom& g, int dtype, const void* src, const void* wgt
   p.src_bytes = (unsigned)(BWD ? yb : xb);
   p.dst_bytes = (unsigned)(BWD ? xb : yb);
   p.wgt_bytes = (unsigned)wb;
-  static const bool no_reorder = getenv("FLHIP_TAPPED_NO_REORDER") != nullptr;
+  const bool no_reorder = options().tapped_no_reorder;
   if (ws && ws_bytes >= (size_t)wb && p.KHW > 1 && !no_reorder) {
     const int rows = g.K * g.C;
     const long long total = (long long)rows * p.KHW;

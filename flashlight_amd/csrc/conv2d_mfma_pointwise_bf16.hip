@@ -338,7 +338,7 @@ int launch_pw16(const ConvGeom& g, const void* src, const void* w, const float* 
   // on the ResNet-50 layers: 20 to 30 % faster there, slower on every larger grid);
   // FLHIP_PW16_PF = 1 / 4 forces one or the other
   bool deep = grid <= (long long)mfma_num_cus() && p.nchunks >= 8;
-  if (const char* e = getenv("FLHIP_PW16_PF")) deep = atoi(e) > 1;
+  if (options().pw16_pf) deep = options().pw16_pf > 1;
   const bool odd = p.P % 4 != 0;
   auto go = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), 0, s, p, static_cast<const bf16_t*>(src),
@@ -765,7 +765,7 @@ bool pw16_taps_plan(const ConvGeom& g, ConvGeom* c, bool wgrad = false) {
 size_t mfma_pointwise16_lattice_ws(const ConvGeom& g, bool bwd) {
   ConvGeom c;
   if (pw16_strided_plan(g, &c)) return lattice_bytes(c);
-  if (bwd && !getenv("FLHIP_PW16_NO_TAPS") && pw16_taps_plan(g, &c)) return lattice_bytes(c);
+  if (bwd && !options().pw16_no_taps && pw16_taps_plan(g, &c)) return lattice_bytes(c);
   return 0;
 }
 
@@ -791,7 +791,7 @@ int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void
     lattice_scatter(g, ws, dx, s);
     return check_launch("conv2d_bwd_data strided 1x1 (bf16 mfma)");
   }
-  if (!getenv("FLHIP_PW16_NO_TAPS") && pw16_taps_plan(g, &c)) {
+  if (!options().pw16_no_taps && pw16_taps_plan(g, &c)) {
     if (!ws || ws_bytes < lattice_bytes(c)) return -1;
     const int rc = launch_pw16<true>(c, dy, w, nullptr, ws, s);
     if (rc != FLHIP_OK) return rc;
@@ -805,7 +805,7 @@ int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void
 size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g0) {
   ConvGeom g = g0;
   size_t lattice = 0;
-  if (pw16_strided_plan(g0, &g) || (!getenv("FLHIP_PW16_NO_TAPS") && pw16_taps_plan(g0, &g, true))) lattice = lattice_bytes(g);
+  if (pw16_strided_plan(g0, &g) || (!options().pw16_no_taps && pw16_taps_plan(g0, &g, true))) lattice = lattice_bytes(g);
   else g = g0;
   Pw16WgradParams p{};
   if (!pw16_wgrad_plan(g, &p)) return 0;
@@ -817,7 +817,7 @@ int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, fl
   if (!dw) return -1;
   ConvGeom g = g0;
   const bool strided = pw16_strided_plan(g0, &g);
-  const bool taps = !strided && !getenv("FLHIP_PW16_NO_TAPS") && pw16_taps_plan(g0, &g, true);
+  const bool taps = !strided && !options().pw16_no_taps && pw16_taps_plan(g0, &g, true);
   if (!strided && !taps) g = g0;
   Pw16WgradParams p{};
   if (!pw16_wgrad_plan(g, &p)) return -1;

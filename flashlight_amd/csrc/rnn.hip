@@ -180,8 +180,7 @@ size_t workspace_floats(const RnnGeom& g) {
 
 // the fused step kernels tile the hidden state by 16 and hold at most 64 batch columns
 bool fused_applies(const RnnGeom& g) {
-  static const bool off = getenv("FLHIP_RNN_UNFUSED") != nullptr;
-  return !off && g.H % 16 == 0 && g.B <= 64;
+  return !options().rnn_unfused && g.H % 16 == 0 && g.B <= 64;
 }
 
 __device__ __forceinline__ float sigm(float v) { return 1.f / (1.f + expf(-v)); }

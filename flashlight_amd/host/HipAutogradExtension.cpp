@@ -17,8 +17,10 @@ struct Registry {
   std::map<TensorBackendType, std::unique_ptr<AutogradExtension>> instances;
 };
 Registry& registry() {
-  static Registry r;
-  return r;
+  // never destroyed: extension instances own device tensors (their workspace), and a
+  // process may unload the HIP runtime before its own static destructors run
+  static Registry* r = new Registry;
+  return *r;
 }
 }  // namespace
 

@@ -124,9 +124,11 @@ Tensor Tensor::fromHost(const Shape& shape, dtype type, const void* data) {
 }
 
 Tensor Tensor::full(const Shape& shape, double value, dtype type) {
-  if (type != dtype::f32) throw std::runtime_error("Tensor::full: f32 only");
-  std::vector<float> v((size_t)shape.elements(), (float)value);
-  return fromHost(shape, type, v.data());
+  // a fill kernel on the backend stream: no host buffer, no synchronisation
+  Tensor t(shape, type);
+  if (flhip_fill(t.device(), value, (size_t)t.elements(), tag(type), g_stream) != FLHIP_OK)
+    throw std::runtime_error(flhip_last_error());
+  return t;
 }
 
 void Tensor::toHost(void* dst) const {

@@ -107,6 +107,19 @@ const char* flhip_last_error(void);
 int flhip_version(void);
 const char* flhip_arch(void);
 
+/* Measurement / debugging switches.  Each is read once from the environment variable
+ * FLHIP_<name> when the library first needs it; afterwards only this call changes it
+ * (value NULL restores the default; the FLHIP_ prefix on `name` is optional).  Not to be
+ * called while another thread is inside the library.  Results stay within the stated
+ * tolerances under every setting; the switches only choose between kernels.
+ *   CONV_ALGO = direct | gather | tapped | convert | auto    CONV_SKIP = bf16,gemm1x1,slab,tapped
+ *   PW_PT = 2 | 4 | 8    PW16_PF = 0 | 1 | 4    BN_ALGO = split | resident | auto
+ *   PW16_NO_TAPS, TAPPED_NO_REORDER, MATMUL_VALU, RNN_UNFUSED = 1 | 0
+ * Unknown names or values return FLHIP_INVALID_ARGUMENT.  The nearest thing in the
+ * reference is the kernel-choice options object of its cuDNN extension
+ * (createBenchmarkOptions, flashlight/fl/autograd/tensor/backend/cudnn/CudnnAutogradExtension.h:25). */
+int flhip_set_option(const char* name, const char* value);
+
 /* Output extents of the geometries above; return FLHIP_INVALID_ARGUMENT when the
  * geometry is not valid (non-positive sizes, window larger than padded input…). */
 int flhip_conv2d_out_dims(const flhip_conv_desc* d, int32_t* OH, int32_t* OW);
@@ -209,6 +222,11 @@ int flhip_bn_bwd(const flhip_bn_desc* d, const void* x, const void* dy,
  * and FL_ADJUST_INPUT_TYPE, flashlight/fl/autograd/Functions.h:57-82). */
 int flhip_convert(const void* src, int src_dtype, void* dst, int dst_dtype,
                   size_t n, void* stream);
+
+/* dst[i] = value for n elements of `dtype`: fl::full as the extension uses it for
+ * default running statistics (onednn/BatchNorm.cpp:116-122), enqueued like every other
+ * kernel (no host buffer, no synchronisation; safe under graph capture). */
+int flhip_fill(void* dst, double value, size_t n, int dtype, void* stream);
 
 /* out = a + b over n elements of `dtype` (out may alias a or b): the gradient
  * accumulation of Variable::addGrad (flashlight/fl/autograd/Variable.cpp:185-218). */

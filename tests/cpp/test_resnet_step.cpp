@@ -8,6 +8,8 @@
 #include <csignal>
 #include <execinfo.h>
 #include <unistd.h>
+
+#include "flhip.h"
 #include <cstdio>
 #include <cstdlib>
 #include <string>
@@ -94,7 +96,7 @@ int main(int argc, char** argv) {
 
     int fail = 0;
     auto run = [&](const char* algo) {
-      if (algo) setenv("FLHIP_CONV_ALGO", algo, 1); else unsetenv("FLHIP_CONV_ALGO");
+      if (flhip_set_option("CONV_ALGO", algo) != FLHIP_OK) throw std::runtime_error(flhip_last_error());
       StepResult r;
       r.loss = step(*model, in, target).tensor().toHostVector()[0];
       for (size_t i : {size_t(0), size_t(1), params.size() / 2, params.size() - 2, params.size() - 1})
@@ -111,7 +113,7 @@ int main(int argc, char** argv) {
     const StepResult a2 = run(nullptr);          // the kernels are deterministic: bit-identical
     const StepResult b = run("direct");
     const StepResult g = run("gather");          // matrix cores again, another summation order
-    unsetenv("FLHIP_CONV_ALGO");
+    flhip_set_option("CONV_ALGO", nullptr);
     std::printf("loss %.6f (default) %.6f (direct kernels) %.6f (gather kernels)\n", a.loss, b.loss, g.loss);
     if (!std::isfinite(a.loss) || std::fabs(a.loss - b.loss) > 1e-4f * std::fabs(b.loss)) { std::printf("FAILED: loss\n"); ++fail; }
     // The step is a chain of 53 convolutions, each followed by a batch norm, and of ReLU
@@ -131,7 +133,7 @@ int main(int argc, char** argv) {
     }
     std::printf(fail ? "%d check(s) FAILED\n" : "ResNet-50 step checks passed\n", fail);
     std::fflush(stdout);
-    _exit(fail ? 1 : 0);   // no static destructors: see test_host_extension.cpp
+    return fail ? 1 : 0;
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
     return 2;
