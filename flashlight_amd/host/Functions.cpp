@@ -1,4 +1,5 @@
 #include "Functions.h"
+#include "OpObserver.h"
 
 #include <algorithm>
 #include <tuple>
@@ -42,6 +43,7 @@ void Variable::addGrad(const Variable& childGrad) {
     grad_->grad.reset(new Variable(childGrad.tensor(), false));
     return;
   }
+  detail::OpScope scope("addGrad");
   Tensor sum(shape(), type());
   const int tag = type() == dtype::f32 ? FLHIP_F32 : FLHIP_BF16;
   if (type() != dtype::f32 && type() != dtype::bf16)
@@ -49,6 +51,7 @@ void Variable::addGrad(const Variable& childGrad) {
   if (flhip_add(grad_->grad->tensor().device(), childGrad.tensor().device(), sum.device(),
                 (size_t)sum.elements(), tag, hipBackendStream()) != FLHIP_OK)
     throw std::runtime_error(flhip_last_error());
+  if (scope.on()) scope.done({grad_->grad->tensor(), childGrad.tensor()}, {sum});
   grad_->grad.reset(new Variable(sum, false));
 }
 
@@ -263,10 +266,12 @@ Variable add(const Variable& lhs, const Variable& rhs) {
   dtypesMatch("add", {&lhs, &rhs});
   if (lhs.shape() != rhs.shape())
     throw std::invalid_argument("add: shapes must match (no broadcasting on this backend)");
+  detail::OpScope scope("add");
   const int tag = tagOf(lhs.type(), "add");
   Tensor out(lhs.shape(), lhs.type());
   check(flhip_add(lhs.tensor().device(), rhs.tensor().device(), out.device(), (size_t)out.elements(), tag,
                   hipBackendStream()));
+  if (scope.on()) scope.done({lhs.tensor(), rhs.tensor()}, {out});
   auto gradFunc = [](std::vector<Variable>& inputs, const Variable& gradOutput) {
     inputs[0].addGrad(Variable(gradOutput.tensor(), false));
     inputs[1].addGrad(Variable(gradOutput.tensor(), false));
@@ -307,16 +312,20 @@ Variable detail::affine(const Variable& input, const Variable& weight, const Var
 }
 
 Variable relu(const Variable& input) {
+  detail::OpScope scope("relu");
   Tensor out(input.shape(), input.type());
   check(flhip_relu_fwd(input.tensor().device(), out.device(), (size_t)out.elements(),
                        tagOf(input.type(), "relu"), hipBackendStream()));
+  if (scope.on()) scope.done({input.tensor()}, {out});
   auto gradFunc = [](std::vector<Variable>& inputs, const Variable& gradOutput) {
     // mask = (input > 0) (Functions.cpp:333-335)
     auto& in = inputs[0];
     if (!in.isCalcGrad()) return;
+    detail::OpScope scope("reluBackward");
     Tensor g(in.shape(), gradOutput.type());
     check(flhip_relu_bwd(gradOutput.tensor().device(), in.tensor().device(), g.device(),
                          (size_t)g.elements(), tagOf(g.type(), "relu"), hipBackendStream()));
+    if (scope.on()) scope.done({gradOutput.tensor(), in.tensor()}, {g});
     in.addGrad(Variable(g, false));
   };
   return Variable(out, {input}, gradFunc);
@@ -373,34 +382,43 @@ Variable linear(const Variable& input, const Variable& weight, const Variable& b
     throw std::invalid_argument("linear: bias must have one element per output feature");
   // the tiled bias is added in fp32 inside the product (Functions.cpp:1267-1272)
   const Tensor b32 = hasBias ? bias.tensor().astype(dtype::f32) : Tensor();
+  detail::OpScope scope("linear");
   Tensor output(Shape(oshape), input.type());
   check(flhip_matmul(weight.tensor().device(), input.tensor().device(), output.device(), (int32_t)out,
                      (int32_t)frames, (int32_t)in, 0, 0, static_cast<const float*>(b32.device()), tag,
                      hipBackendStream()));
+  if (scope.on()) scope.done({input.tensor(), weight.tensor(), b32}, {output}, {out, in, frames});
   auto gradFunc = [hasBias, tag, out, in, frames](std::vector<Variable>& inputs,
                                                   const Variable& gradOutput) {
     // Functions.cpp:1276-1303
+    detail::OpScope scope("linearBackward");
     auto& x = inputs[0];
     auto& wt = inputs[1];
     const void* g = gradOutput.tensor().device();
+    Tensor dxT, dwT, dbT;
     if (hasBias && inputs[2].isCalcGrad()) {
       Tensor db(inputs[2].shape(), dtype::f32);
       check(flhip_sum_columns(g, static_cast<float*>(db.device()), (int32_t)out, (int32_t)frames, tag,
                               hipBackendStream()));
-      inputs[2].addGrad(Variable(db.astype(inputs[2].type()), false));
+      dbT = db;
     }
     if (x.isCalcGrad()) {
       Tensor dx(x.shape(), x.type());
       check(flhip_matmul(wt.tensor().device(), g, dx.device(), (int32_t)in, (int32_t)frames,
                          (int32_t)out, 1, 0, nullptr, tag, hipBackendStream()));
-      x.addGrad(Variable(dx, false));
+      dxT = dx;
     }
     if (wt.isCalcGrad()) {
       Tensor dw(wt.shape(), wt.type());
       check(flhip_matmul(g, x.tensor().device(), dw.device(), (int32_t)out, (int32_t)in,
                          (int32_t)frames, 0, 1, nullptr, tag, hipBackendStream()));
-      wt.addGrad(Variable(dw, false));
+      dwT = dw;
     }
+    // event: inputs {gradOutput, input, weight}, outputs {dx, dw, db (each may be empty)}, ints {out, in, frames}
+    if (scope.on()) scope.done({gradOutput.tensor(), x.tensor(), wt.tensor()}, {dxT, dwT, dbT}, {out, in, frames});
+    if (!dbT.isEmpty()) inputs[2].addGrad(Variable(dbT.astype(inputs[2].type()), false));
+    if (!dxT.isEmpty()) x.addGrad(Variable(dxT, false));
+    if (!dwT.isEmpty()) wt.addGrad(Variable(dwT, false));
   };
   if (hasBias) return Variable(output, {input, weight, bias}, gradFunc);
   return Variable(output, {input, weight}, gradFunc);
@@ -410,15 +428,19 @@ Variable logSoftmax(const Variable& input, int dim) {
   if (dim != 0) throw std::invalid_argument("logSoftmax: only dimension 0 is supported by this backend");
   const int tag = tagOf(input.type(), "logSoftmax");
   const Dim classes = input.tensor().dim(0), cols = input.tensor().elements() / classes;
+  detail::OpScope scope("logSoftmax");
   Tensor result(input.shape(), input.type());
   check(flhip_logsoftmax_fwd(input.tensor().device(), result.device(), (int32_t)classes, (int32_t)cols,
                              tag, hipBackendStream()));
+  if (scope.on()) scope.done({input.tensor()}, {result}, {classes, cols});
   auto gradFunc = [result, tag, classes, cols](std::vector<Variable>& inputs,
                                                const Variable& gradOutput) {
     // gradOutput - exp(result) * sum(gradOutput) (Functions.cpp:1061-1066)
+    detail::OpScope scope("logSoftmaxBackward");
     Tensor g(result.shape(), result.type());
     check(flhip_logsoftmax_bwd(gradOutput.tensor().device(), result.device(), g.device(),
                                (int32_t)classes, (int32_t)cols, tag, hipBackendStream()));
+    if (scope.on()) scope.done({gradOutput.tensor(), result}, {g}, {classes, cols});
     inputs[0].addGrad(Variable(g.astype(inputs[0].type()), false));
   };
   return Variable(result, {input}, gradFunc);
@@ -437,6 +459,7 @@ Variable categoricalCrossEntropy(const Variable& input, const Variable& targets,
     throw std::invalid_argument("categoricalCrossEntropy: targets must be s32 on this backend");
   const int tag = tagOf(input.type(), "categoricalCrossEntropy");
   const Dim C = input.tensor().dim(0), X = targets.tensor().elements();
+  detail::OpScope scope("categoricalCrossEntropy");
   Tensor stats(Shape({4}), dtype::f32);
   Tensor per = reduction == ReduceMode::NONE ? Tensor(targets.shape(), dtype::f32) : Tensor();
   check(flhip_cce_fwd(input.tensor().device(), static_cast<const int32_t*>(targets.tensor().device()),
@@ -454,18 +477,21 @@ Variable categoricalCrossEntropy(const Variable& input, const Variable& targets,
     const float v = reduction == ReduceMode::MEAN ? st[3] : st[0];
     result = Tensor::fromHost(Shape({1}), dtype::f32, &v);
   }
+  if (scope.on()) scope.done({input.tensor(), targets.tensor()}, {result, stats}, {C, X, (int)reduction, ignoreIndex});
   const Shape inShape = input.shape();
   const dtype inType = input.type();
   const Tensor tg = targets.tensor();
   auto gradFunc = [stats, tg, inShape, inType, tag, C, X, reduction, ignoreIndex](
                       std::vector<Variable>& inputs, const Variable& gradOutput) {
     // tile(grad / denominator) * mask (Functions.cpp:1131-1150)
+    detail::OpScope scope("categoricalCrossEntropyBackward");
     Tensor g(inShape, inType);
     const Tensor go = gradOutput.tensor().astype(dtype::f32);
     check(flhip_cce_bwd(static_cast<const float*>(go.device()),
                         static_cast<const int32_t*>(tg.device()),
                         static_cast<const float*>(stats.device()), g.device(), (int32_t)C, (int32_t)X,
                         (int)reduction, ignoreIndex, tag, hipBackendStream()));
+    if (scope.on()) scope.done({go, tg, stats}, {g}, {C, X, (int)reduction, ignoreIndex});
     inputs[0].addGrad(Variable(g, false));
   };
   return Variable(result, {input, targets}, gradFunc);

@@ -1,4 +1,5 @@
 #include "HipAutogradExtension.h"
+#include "OpObserver.h"
 
 #include <algorithm>
 #include <map>
@@ -134,6 +135,7 @@ Tensor HipAutogradExtension::conv2d(const Tensor& input, const Tensor& weights, 
                                     std::shared_ptr<detail::AutogradPayload>) {
   if (input.type() != weights.type())
     throw std::invalid_argument("conv2d: input and weights must have the same type");
+  detail::OpScope scope("conv2d");
   const int tag = dtypeTag(input.type(), "conv2d");
   flhip_conv_desc d = convDesc(input.shape(), weights, sx, sy, px, py, dx, dy, groups, tag, "conv2d");
   int32_t OH = 0, OW = 0;
@@ -148,6 +150,8 @@ Tensor HipAutogradExtension::conv2d(const Tensor& input, const Tensor& weights, 
   DevicePtr xp(input), wp(weights), bp(b), yp(output), wsp(ws);
   check(flhip_conv2d_fwd(&d, xp.get(), wp.get(), static_cast<const float*>(bp.get()), yp.get(),
                          wsp.get(), wsBytes, hipBackendStream()));
+  // event: inputs {input, weights, bias}, outputs {output}, ints {sx, sy, px, py, dx, dy, groups}
+  if (scope.on()) scope.done({input, weights, b}, {output}, {sx, sy, px, py, dx, dy, groups});
   return output;
 }
 
@@ -159,6 +163,7 @@ Tensor HipAutogradExtension::conv2dBackwardData(const Tensor& gradOutput, const 
                                                 std::shared_ptr<detail::AutogradPayload>) {
   if (gradOutput.type() != weight.type())
     throw std::invalid_argument("conv2dBackwardData: gradOutput and weights must have the same type");
+  detail::OpScope scope("conv2dBackwardData");
   const int tag = dtypeTag(gradOutput.type(), "conv2dBackwardData");
   flhip_conv_desc d =
       convDesc(input.shape(), weight, sx, sy, px, py, dx, dy, groups, tag, "conv2dBackwardData");
@@ -172,6 +177,8 @@ Tensor HipAutogradExtension::conv2dBackwardData(const Tensor& gradOutput, const 
   DevicePtr gp(gradOutput), wp(weight), op(gradInput), wsp(ws);
   check(flhip_conv2d_bwd_data(&d, gp.get(), wp.get(), op.get(), wsp.get(), wsBytes,
                               hipBackendStream()));
+  // event: inputs {gradOutput, weights}, outputs {gradInput}, ints as conv2d
+  if (scope.on()) scope.done({gradOutput, weight}, {gradInput}, {sx, sy, px, py, dx, dy, groups});
   return gradInput;
 }
 
@@ -182,6 +189,7 @@ std::pair<Tensor, Tensor> HipAutogradExtension::conv2dBackwardFilterBias(
     std::shared_ptr<detail::AutogradPayload>) {
   if (gradOutput.type() != input.type())
     throw std::invalid_argument("conv2dBackwardFilterBias: gradOutput and input must have the same type");
+  detail::OpScope scope("conv2dBackwardFilterBias");
   const int tag = dtypeTag(input.type(), "conv2dBackwardFilterBias");
   flhip_conv_desc d = convDesc(input.shape(), weights, sx, sy, px, py, dx, dy, groups, tag,
                                "conv2dBackwardFilterBias");
@@ -202,6 +210,8 @@ std::pair<Tensor, Tensor> HipAutogradExtension::conv2dBackwardFilterBias(
   check(flhip_conv2d_bwd_filter(&d, xp.get(), gp.get(), static_cast<float*>(dwp.get()),
                                 static_cast<float*>(dbp.get()), wsp.get(), wsBytes,
                                 hipBackendStream()));
+  // event: inputs {gradOutput, input}, outputs {gradWeights, gradBias (may be empty)}, ints as conv2d
+  if (scope.on()) scope.done({gradOutput, input}, {gradWeights, gradBias}, {sx, sy, px, py, dx, dy, groups});
   return {gradWeights, gradBias};
 }
 
@@ -228,6 +238,7 @@ Tensor HipAutogradExtension::pool2d(const Tensor& input, const int wx, const int
                                     std::shared_ptr<detail::AutogradPayload> autogradPayload) {
   if (input.ndim() < 1 || input.ndim() > 4)
     throw std::invalid_argument("pool2d: input must have 1 to 4 dimensions");
+  detail::OpScope scope("pool2d");
   const bool train = autogradPayload != nullptr;    // onednn/Pool2D.cpp:88
   flhip_pool_desc d = poolDesc(input.shape(), wx, wy, sx, sy, px, py, mode, dtypeTag(input.type(), "pool2d"));
   int32_t OH = 0, OW = 0;
@@ -238,6 +249,8 @@ Tensor HipAutogradExtension::pool2d(const Tensor& input, const int wx, const int
   if (train) autogradPayload->data = payload;
   DevicePtr xp(input), yp(output), ap(payload->argmax);
   check(flhip_pool2d_fwd(&d, xp.get(), yp.get(), static_cast<uint8_t*>(ap.get()), hipBackendStream()));
+  // event: inputs {input}, outputs {output, argmax (may be empty)}, ints {wx, wy, sx, sy, px, py, mode}
+  if (scope.on()) scope.done({input}, {output, payload->argmax}, {wx, wy, sx, sy, px, py, (int)mode});
   return output;
 }
 
@@ -246,6 +259,7 @@ Tensor HipAutogradExtension::pool2dBackward(const Tensor& gradOutput, const Tens
                                             const int sx, const int sy, const int px, const int py,
                                             const PoolingMode mode,
                                             std::shared_ptr<detail::AutogradPayload> autogradPayload) {
+  detail::OpScope scope("pool2dBackward");
   if (!autogradPayload || !autogradPayload->data)   // onednn/Pool2D.cpp:190-193
     throw std::invalid_argument("HipAutogradExtension::pool2dBackward given null or empty payload");
   auto payload = std::dynamic_pointer_cast<HipPool2DPayload>(autogradPayload->data);
@@ -263,6 +277,8 @@ Tensor HipAutogradExtension::pool2dBackward(const Tensor& gradOutput, const Tens
   DevicePtr gp(gradOutput), ap(payload->argmax), op(gradInput);
   check(flhip_pool2d_bwd(&d, gp.get(), static_cast<const uint8_t*>(ap.get()), op.get(),
                          hipBackendStream()));
+  // event: inputs {gradOutput, argmax}, outputs {gradInput}, ints as pool2d
+  if (scope.on()) scope.done({gradOutput, payload->argmax}, {gradInput}, {wx, wy, sx, sy, px, py, (int)mode});
   return gradInput;
 }
 
@@ -273,6 +289,7 @@ Tensor HipAutogradExtension::batchnorm(Tensor& saveMean, Tensor& saveVar, const 
                                        const std::vector<int>& axes, const bool train,
                                        const double momentum, const double epsilon,
                                        std::shared_ptr<detail::AutogradPayload> autogradPayload) {
+  detail::OpScope scope("batchnorm");
   const int tag = dtypeTag(input.type(), "batchnorm");
   flhip_bn_desc d = bnDesc(input, axes, tag);
   const Dim nfeat = (Dim)d.C;
@@ -294,6 +311,8 @@ Tensor HipAutogradExtension::batchnorm(Tensor& saveMean, Tensor& saveVar, const 
                              static_cast<const float*>(rmp.get()),
                              static_cast<const float*>(rvp.get()), epsilon, yp.get(),
                              hipBackendStream()));
+    if (scope.on())
+      scope.done({input, gamma, beta, runningMean, runningVar}, {output}, {d.outer, d.C, d.inner, 0}, {momentum, epsilon});
     return output;
   }
   // like the cuDNN extension (cudnn/BatchNorm.cpp:138-162): saveMean holds the batch
@@ -314,6 +333,11 @@ Tensor HipAutogradExtension::batchnorm(Tensor& saveMean, Tensor& saveVar, const 
     payload->saveInvStd = saveVar;
     autogradPayload->data = payload;
   }
+  // event: inputs {input, gamma, beta, runningMean, runningVar (both after the update)}, outputs {output, saveMean,
+  // saveInvStd}, ints {outer, features, inner, train}, reals {momentum, epsilon}
+  if (scope.on())
+    scope.done({input, gamma, beta, runningMean, runningVar}, {output, saveMean, saveVar}, {d.outer, d.C, d.inner, 1},
+               {momentum, epsilon});
   return output;
 }
 
@@ -321,6 +345,7 @@ std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::batchnormBackward(
     const Tensor& gradOutput, const Tensor& saveMean, const Tensor& saveVar, const Tensor& input,
     const Tensor& weight, const std::vector<int>& axes, const bool train, const float,
     std::shared_ptr<detail::AutogradPayload> autogradPayload) {
+  detail::OpScope scope("batchnormBackward");
   if (!train)   // cudnn/BatchNorm.cpp:196-199
     throw std::logic_error("HipAutogradExtension::batchnormBackward: only train mode has a backward pass");
   Tensor mean = saveMean, invstd = saveVar;
@@ -347,6 +372,10 @@ std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::batchnormBackward(
                      static_cast<const float*>(mp.get()), static_cast<const float*>(ip.get()),
                      dxp.get(), static_cast<float*>(dgp.get()), static_cast<float*>(dbp.get()),
                      wsp.get(), wsBytes, hipBackendStream()));
+  // event: inputs {gradOutput, input, gamma, saveMean, saveInvStd}, outputs {gradInput, gradWeight, gradBias},
+  // ints {outer, features, inner}
+  if (scope.on())
+    scope.done({gradOutput, input, gamma, mean, invstd}, {gradInput, gradWeight, gradBias}, {d.outer, d.C, d.inner});
   return std::make_tuple(gradInput, gradWeight, gradBias);   // always all three (:278)
 }
 
@@ -375,6 +404,7 @@ std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::rnn(
     const Tensor& input, const Tensor& hiddenState, const Tensor& cellState, const Tensor& weights,
     const int hiddenSize, const int numLayers, const RnnMode mode, const bool bidirectional,
     const float dropProb, std::shared_ptr<detail::AutogradPayload> autogradPayload) {
+  detail::OpScope scope("rnn");
   if (input.isEmpty()) throw std::runtime_error("HipAutogradExtension::rnn: empty input");
   for (const Tensor* t : {&hiddenState, &cellState, &weights})
     if (!t->isEmpty() && t->type() != input.type())
@@ -410,6 +440,7 @@ std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::rnn(
     payload->reserve = reserve;
     autogradPayload->data = payload;
   }
+  if (scope.on()) scope.done({input, hiddenState, cellState, weights}, {y, hy, cy}, {hiddenSize, numLayers, (int)mode, bidirectional});
   return std::make_tuple(y, hy, cy);
 }
 
@@ -418,6 +449,7 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> HipAutogradExtension::rnnBackward(
     const std::shared_ptr<detail::RNNGradData> gradData, const Tensor& output, const int numLayers,
     const int hiddenSize, const RnnMode mode, const bool bidirectional, const float,
     std::shared_ptr<detail::AutogradPayload> autogradPayload) {
+  detail::OpScope scope("rnnBackward");
   if (!autogradPayload || !autogradPayload->data)   // RNN.cpp:246-249
     throw std::invalid_argument("HipAutogradExtension::rnnBackward given null or empty autograd payload");
   auto payload = std::dynamic_pointer_cast<HipRnnPayload>(autogradPayload->data);
@@ -443,6 +475,7 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> HipAutogradExtension::rnnBackward(
                       hipBackendStream()));
   (void)hiddenState;
   (void)cellState;
+  if (scope.on()) scope.done({input, weights, gradData->dy, gradData->dhy, gradData->dcy}, {dx, dhx, dcx, dw}, {hiddenSize, numLayers, (int)mode, bidirectional});
   return std::make_tuple(dx, dhx, dcx, dw);
 }
 

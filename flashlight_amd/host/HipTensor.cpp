@@ -1,4 +1,5 @@
 #include "HipTensor.h"
+#include "OpObserver.h"
 
 #include <hip/hip_runtime.h>
 
@@ -89,6 +90,86 @@ int tag(dtype t) {
 }
 }  // namespace
 
+namespace detail {
+namespace {
+OpObserver* g_observer = nullptr;
+}
+OpObserver* opObserver() { return g_observer; }
+void setOpObserver(OpObserver* observer) { g_observer = observer; }
+}  // namespace detail
+
+// ---- StepProfiler -------------------------------------------------------------------
+struct StepProfiler::Impl {
+  struct Span {
+    std::string op;
+    hipEvent_t start, stop;
+  };
+  std::vector<Span> spans;
+  std::vector<hipEvent_t> spare;
+  int depth = 0;
+  hipEvent_t event() {
+    if (!spare.empty()) {
+      hipEvent_t e = spare.back();
+      spare.pop_back();
+      return e;
+    }
+    hipEvent_t e;
+    hipCheck(hipEventCreate(&e), "hipEventCreate");
+    return e;
+  }
+};
+
+StepProfiler::StepProfiler() : impl_(new Impl) {}
+StepProfiler::~StepProfiler() {
+  if (detail::opObserver() == this) detail::setOpObserver(nullptr);
+  for (auto& s : impl_->spans) {
+    (void)hipEventDestroy(s.start);
+    (void)hipEventDestroy(s.stop);
+  }
+  for (hipEvent_t e : impl_->spare) (void)hipEventDestroy(e);
+  delete impl_;
+}
+
+void StepProfiler::begin(const char* op) {
+  if (impl_->depth++ > 0) return;
+  Impl::Span s{op, impl_->event(), impl_->event()};
+  hipCheck(hipEventRecord(s.start, (hipStream_t)g_stream), "hipEventRecord");
+  impl_->spans.push_back(s);
+}
+
+void StepProfiler::end(const detail::OpEvent&) {
+  if (--impl_->depth > 0) return;
+  hipCheck(hipEventRecord(impl_->spans.back().stop, (hipStream_t)g_stream), "hipEventRecord");
+}
+
+std::map<std::string, StepProfiler::Entry> StepProfiler::collect() {
+  sync();
+  impl_->depth = 0;
+  std::map<std::string, Entry> out;
+  double busy = 0;
+  for (auto& s : impl_->spans) {
+    float ms = 0;
+    hipCheck(hipEventElapsedTime(&ms, s.start, s.stop), "hipEventElapsedTime");
+    out[s.op].ms += ms;
+    out[s.op].calls += 1;
+    busy += ms;
+  }
+  if (!impl_->spans.empty()) {
+    float span = 0;
+    hipCheck(hipEventElapsedTime(&span, impl_->spans.front().start, impl_->spans.back().stop), "hipEventElapsedTime");
+    out["(span)"].ms = span;
+    out["(span)"].calls = 1;
+    out["(gaps)"].ms = span - busy;
+    out["(gaps)"].calls = 1;
+  }
+  for (auto& s : impl_->spans) {
+    impl_->spare.push_back(s.start);
+    impl_->spare.push_back(s.stop);
+  }
+  impl_->spans.clear();
+  return out;
+}
+
 void* hipBackendStream() { return g_stream; }
 void setHipBackendStream(void* stream) {
   // cached buffers are reused in program order of one stream: drain the old one first
@@ -157,9 +238,11 @@ Tensor Tensor::astype(dtype t) const {
     r.type_ = isEmpty() ? t : type_;
     return r;
   }
+  detail::OpScope scope("astype");
   Tensor out(shape_, t);
   const int rc = flhip_convert(device(), tag(type_), out.device(), tag(t), (size_t)elements(), g_stream);
   if (rc != FLHIP_OK) throw std::runtime_error(flhip_last_error());
+  if (scope.on()) scope.done({*this}, {out});
   return out;
 }
 

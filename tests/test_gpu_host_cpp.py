@@ -21,8 +21,11 @@ def test_host_extension_program():
 
 @pytest.mark.gpu
 def test_resnet50_step_program():
-    """ResNet-50 forward + backward from the host modules at batch 2: shapes, gradients for
-    all 161 parameter tensors, matrix-core kernels against the direct kernels end to end."""
+    """configs[4] at batch 2, fp32 and bf16 storage: every operation of a real ResNet-50 step
+    (conv / batch norm / pooling forward and backward, ReLU, residual adds, casts, the
+    classifier and the loss) replayed on the CPU checker with the operation's own device
+    inputs, at the stated tolerances; shapes, gradients for all 161 parameter tensors,
+    run-to-run bit identity."""
     exe = os.path.join(ROOT, "tests", "cpp", "bin", "test_resnet_step")
     assert os.path.exists(exe), "build it with `python -m flashlight_amd.build`"
     r = subprocess.run([exe], capture_output=True, text=True, timeout=110)
