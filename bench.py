@@ -6,8 +6,13 @@ stage-2 3x3 shape (input 56x56x64, batch 32, 64 filters, stride 1, pad 1); the
 headline value is the pair's TFLOP/s over exactly --steps steps.  The
 bandwidth-bound half of the metric (batchnormBackward at 56x56x256x32,
 pool2dBackward max/avg 3x3 s2 p1 at 112x112x64x32) is timed the same way in
-its own loops and reported in `ops`, with buffer sets rotated so that no call
-finds its operands in the 256 MB memory-side cache.
+its own loops and reported in `ops`, with whole buffer sets (inputs AND outputs)
+rotated over more than 512 MB so that no call finds its operands in the 256 MB
+memory-side cache.  Every figure is the median of 5 timed repeats of --steps calls.
+
+`--step resnet50|speech` instead runs whole training steps through the C++ host
+layer (flashlight_amd/lib/flhip_step_bench) and prints their time with a breakdown
+per operation class.
 
 All inputs are resident in HBM before any timed region starts.  Timing uses HIP
 events on the stream the kernels are launched on (torch's current stream, whose
@@ -33,7 +38,7 @@ MEASURED_TRAFFIC = {"conv2d_bwd_data_f32": 61.8e6}
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--steps", type=int, default=0, help="timed steps (default 100; 20 for --step)")
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--dtype", choices=["f32", "bf16"], default="f32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
@@ -41,6 +46,11 @@ def parse():
     ap.add_argument("--layers", choices=["resnet50", "speech"], default="",
                     help="instead of the bench line: time every conv layer of configs[4] (ResNet-50, batch 32) "
                          "or configs[3] (21x1 speech layers) in all three passes and print a table")
+    ap.add_argument("--step", choices=["resnet50", "speech"], default="",
+                    help="instead of the bench line: a whole training step of configs[4] (ResNet-50, 224x224x3) or "
+                         "configs[3] (speech stack) through the host modules, with a per-operation-class breakdown")
+    ap.add_argument("--batch", type=int, default=0, help="batch size for --step (default 64 / 16)")
+    ap.add_argument("--repeats", type=int, default=5, help="timed repeats of --steps calls; the median is reported")
     ap.add_argument("--rnn", action="store_true",
                     help="instead of the bench line: time rnn / rnnBackward (LSTM, GRU) at a few sizes")
     return ap.parse_args()
@@ -48,10 +58,14 @@ def parse():
 
 def main():
     a = parse()
+    if a.steps <= 0:
+        a.steps = 20 if a.step else 100
     if a.gpus != 1:
         sys.stderr.write("bench.py: this build runs on one GPU; --gpus %d is not supported "
                          "(no collectives or sharding are part of it)\n" % a.gpus)
         return 2
+    if a.step:
+        return step_bench(a)
     import torch
     if not torch.cuda.is_available():
         sys.stderr.write("bench.py: no GPU visible\n")
@@ -70,20 +84,26 @@ def main():
     def randn(*shape, scale=1.0, shift=0.0):
         return torch.randn(shape, device=dev, generator=gen) * scale + shift
 
-    def timed(fn, steps, warmup):
-        """Average seconds per call over exactly `steps` calls."""
+    def timed(fn, steps, warmup, spread=None):
+        """Seconds per call: `repeats` brackets of exactly `steps` calls each (HIP events on
+        the launch stream), the median bracket reported; `spread` receives min and max."""
         for i in range(warmup):
             fn(i)
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        e0.record()
-        for i in range(steps):
-            fn(i)
-        e1.record()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        return e0.elapsed_time(e1) * 1e-3 / steps, wall / steps
+        runs = []
+        for _ in range(max(a.repeats, 1)):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0 = time.perf_counter()
+            e0.record()
+            for i in range(steps):
+                fn(i)
+            e1.record()
+            torch.cuda.synchronize()
+            runs.append((e0.elapsed_time(e1) * 1e-3 / steps, (time.perf_counter() - t0) / steps))
+        runs.sort()
+        if spread is not None:
+            spread["us_min"], spread["us_max"] = runs[0][0] * 1e6, runs[-1][0] * 1e6
+        return runs[len(runs) // 2]
 
     only = set(x for x in a.only.split(",") if x)
     want = lambda name: not only or name in only
@@ -141,11 +161,12 @@ def main():
                          ("conv2d_bwd_filter_bias", f_bwd_filter)):
             if not want(name):
                 continue
-            s, _ = timed(fn, a.steps, a.warmup)
+            sp = {}
+            s, _ = timed(fn, a.steps, a.warmup, sp)
             ach = CONV_FLOP / s / 1e12
             ops.append({"op": name, "workload": "32x64x56x56, 64 filters 3x3 s1 p1", "dtype": dname,
                         "us": s * 1e6, "bound": "mfma", "achieved": ach, "peak": peak_mfma,
-                        "unit": "TFLOP/s", "frac": ach / peak_mfma})
+                        "unit": "TFLOP/s", "frac": ach / peak_mfma, **sp})
         return res
 
     pair_s, pair_wall = conv_block(a.dtype, True)
@@ -156,11 +177,12 @@ def main():
         conv_block(other, False)
 
     # ---- bandwidth ops at cfg 3 (fp32) ----------------------------------------
-    def bw_op(name, workload, nbytes, fn, nsets):
+    def bw_op(name, workload, nbytes, fn, nsets, footprint):
         if not want(name):
             return
         checked(fn)
-        s, _ = timed(fn, a.steps, a.warmup)
+        sp = {}
+        s, _ = timed(fn, a.steps, a.warmup, sp)
         ach = nbytes / s / 1e9
         # the same call on one buffer set every time: operands may sit in the 256 MB
         # memory-side cache (reported beside the cold figure, never as `achieved`)
@@ -168,14 +190,14 @@ def main():
         ops.append({"op": name, "workload": workload, "dtype": "f32", "us": s * 1e6,
                     "bound": "hbm", "achieved": ach, "peak": PEAK["hbm_GBps"], "unit": "GB/s",
                     "frac": ach / PEAK["hbm_GBps"], "algorithmic_bytes": nbytes,
-                    "buffer_sets_rotated": nsets, "us_cache_warm": warm * 1e6,
-                    "GBps_cache_warm": nbytes / warm / 1e9})
+                    "buffer_sets_rotated": nsets, "rotation_footprint_MB": footprint / 1e6,
+                    "us_cache_warm": warm * 1e6, "GBps_cache_warm": nbytes / warm / 1e9, **sp})
 
     if want("batchnorm_bwd") or want("batchnorm_fwd_train"):
-        nsets = 2
+        nsets = 3            # x, dy and the output of every set: 3 x 308 MB
         bx = [randn(32, 256, 56, 56, scale=2 ** 0.5, shift=0.5) for _ in range(nsets)]
         bdy = [randn(32, 256, 56, 56) for _ in range(nsets)]
-        bout = torch.empty_like(bx[0])
+        bout = [torch.empty_like(bx[0]) for _ in range(nsets)]
         gamma = randn(256, scale=0.1, shift=1.0)
         beta = torch.zeros(256, device=dev)
         rm, rv = torch.zeros(256, device=dev), torch.ones(256, device=dev)
@@ -186,44 +208,48 @@ def main():
         bws = torch.empty(max(bnws, 16), dtype=torch.uint8, device=dev)
         sm = [torch.empty(256, device=dev) for _ in range(nsets)]
         si = [torch.empty(256, device=dev) for _ in range(nsets)]
-        bdp, boutp, bwsp = C.byref(bd), P(bout), P(bws)
-        bxp, bdyp = [P(t) for t in bx], [P(t) for t in bdy]
+        bdp, bwsp = C.byref(bd), P(bws)
+        bxp, bdyp, boutp = [P(t) for t in bx], [P(t) for t in bdy], [P(t) for t in bout]
         smp, sip = [P(t) for t in sm], [P(t) for t in si]
         gp, btp, rmp, rvp, dgp, dbtp = P(gamma), P(beta), P(rm), P(rv), P(dg), P(dbt)
-        f_bn_fwd = lambda i: L.flhip_bn_fwd_train(bdp, bxp[i % nsets], gp, btp, boutp,
+        f_bn_fwd = lambda i: L.flhip_bn_fwd_train(bdp, bxp[i % nsets], gp, btp, boutp[i % nsets],
                                                   smp[i % nsets], sip[i % nsets], rmp, rvp,
                                                   0.1, 1e-5, bwsp, bnws, S)
         for i in range(nsets):
             capi.check(f_bn_fwd(i))
-        bw_op("batchnorm_fwd_train", "56x56x256x32, axes {2}", 2 * T, f_bn_fwd, nsets)
+        bw_op("batchnorm_fwd_train", "56x56x256x32, axes {2}", 2 * T, f_bn_fwd, nsets, nsets * 2 * T)
         bw_op("batchnorm_bwd", "56x56x256x32, axes {2}", 3 * T,
               lambda i: L.flhip_bn_bwd(bdp, bxp[i % nsets], bdyp[i % nsets], gp, smp[i % nsets],
-                                       sip[i % nsets], boutp, dgp, dbtp, bwsp, bnws, S), nsets)
+                                       sip[i % nsets], boutp[i % nsets], dgp, dbtp, bwsp, bnws, S),
+              nsets, nsets * 3 * T)
         del bx, bdy, bout
 
     if any(want(n) for n in ("pool2d_max_fwd", "pool2d_max_bwd", "pool2d_avg_fwd", "pool2d_avg_bwd")):
-        nsets = 3
+        nsets = 5            # x (or dx), y (or dy) and the argmax bytes of every set: 5 x 135 MB
         px_ = [torch.round(randn(32, 64, 112, 112) * 8) / 8 for _ in range(nsets)]
         pdy = [randn(32, 64, 56, 56) for _ in range(nsets)]
         pam = [torch.empty((32, 64, 56, 56), dtype=torch.uint8, device=dev) for _ in range(nsets)]
-        pyo = torch.empty((32, 64, 56, 56), device=dev)
-        pdx = torch.empty((32, 64, 112, 112), device=dev)
+        pyo = [torch.empty((32, 64, 56, 56), device=dev) for _ in range(nsets)]
+        pdx = [torch.empty((32, 64, 112, 112), device=dev) for _ in range(nsets)]
         pdm = capi.PoolDesc(32, 64, 112, 112, 3, 3, 2, 2, 1, 1, 0, capi.F32)
         pda = capi.PoolDesc(32, 64, 112, 112, 3, 3, 2, 2, 1, 1, 2, capi.F32)
-        pdmp, pdap, pyop, pdxp = C.byref(pdm), C.byref(pda), P(pyo), P(pdx)
+        pdmp, pdap = C.byref(pdm), C.byref(pda)
+        pyop, pdxp = [P(t) for t in pyo], [P(t) for t in pdx]
         pxp, pdyp, pamp = [P(t) for t in px_], [P(t) for t in pdy], [P(t) for t in pam]
-        f_max_fwd = lambda i: L.flhip_pool2d_fwd(pdmp, pxp[i % nsets], pyop, pamp[i % nsets], S)
+        f_max_fwd = lambda i: L.flhip_pool2d_fwd(pdmp, pxp[i % nsets], pyop[i % nsets], pamp[i % nsets], S)
         for i in range(nsets):
             capi.check(f_max_fwd(i))
         nx, ny = px_[0].numel() * 4, pdy[0].numel() * 4
         wl = "112x112x64x32, 3x3 s2 p1"
-        bw_op("pool2d_max_fwd", wl, nx + ny + ny // 4, f_max_fwd, nsets)
+        bw_op("pool2d_max_fwd", wl, nx + ny + ny // 4, f_max_fwd, nsets, nsets * (nx + ny + ny // 4))
         bw_op("pool2d_max_bwd", wl, nx + ny + ny // 4,
-              lambda i: L.flhip_pool2d_bwd(pdmp, pdyp[i % nsets], pamp[i % nsets], pdxp, S), nsets)
+              lambda i: L.flhip_pool2d_bwd(pdmp, pdyp[i % nsets], pamp[i % nsets], pdxp[i % nsets], S),
+              nsets, nsets * (nx + ny + ny // 4))
         bw_op("pool2d_avg_fwd", wl, nx + ny,
-              lambda i: L.flhip_pool2d_fwd(pdap, pxp[i % nsets], pyop, None, S), nsets)
+              lambda i: L.flhip_pool2d_fwd(pdap, pxp[i % nsets], pyop[i % nsets], None, S), nsets, nsets * (nx + ny))
         bw_op("pool2d_avg_bwd", wl, nx + ny,
-              lambda i: L.flhip_pool2d_bwd(pdap, pdyp[i % nsets], None, pdxp, S), nsets)
+              lambda i: L.flhip_pool2d_bwd(pdap, pdyp[i % nsets], None, pdxp[i % nsets], S), nsets,
+              nsets * (nx + ny))
         del px_, pdy, pam, pyo, pdx
 
     if "copy" in only:
@@ -232,7 +258,7 @@ def main():
         cb = torch.empty_like(ca)
         cap, cbp = P(ca), P(cb)
         bw_op("copy", "flhip_copy_bytes 256 MiB", 2 * (256 << 20),
-              lambda i: L.flhip_copy_bytes(cap, cbp, 256 << 20, S), 1)
+              lambda i: L.flhip_copy_bytes(cap, cbp, 256 << 20, S), 1, 2 * (256 << 20))
 
     torch.cuda.synchronize()
     by = {}
@@ -241,9 +267,9 @@ def main():
         by.setdefault(o["op"] + "_" + o["dtype"] if other_conv else o["op"], o)
 
     # ---- CPU baselines (rank 0, bounded sample) --------------------------------
-    cpu_baseline = cpu_onednn = cpu_bw = None
+    cpu_port = cpu_onednn = cpu_bw = None
     if not a.no_cpu and not only:
-        cpu_baseline, cpu_onednn = cpu_legs()
+        cpu_port, cpu_onednn = cpu_legs()
         cpu_bw = cpu_bandwidth_legs()
 
     out = {
@@ -251,7 +277,7 @@ def main():
         "value": (2 * CONV_FLOP / pair_s / 1e12) if pair_s else None,
         "unit": "TFLOP/s",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": pair_s * 1e3 if pair_s else None,
+        "ms_per_step": pair_s * 1e3 if pair_s else None, "repeats": a.repeats,
         "wall_ms_per_step": pair_wall * 1e3 if pair_wall else None,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": a.dtype, "data": "synthetic",
@@ -268,9 +294,20 @@ def main():
             "bound": "mfma", "achieved": o["achieved"], "peak": o["peak"], "unit": "TFLOP/s",
             "frac": o["frac"], "avg_launch_us": o["us"],
             "traffic": MEASURED_TRAFFIC.get("conv2d_bwd_data_" + a.dtype)}
+    if "conv2d_bwd_filter_bias" in by:
+        o = by["conv2d_bwd_filter_bias"]
+        out["roofline_bwd_filter"] = {
+            "kernel": "wgrad_slab_kernel<float> + wgrad_reduce_kernel (conv2dBackwardFilterBias, two launches per call)"
+                      if a.dtype == "f32" else "wgrad16_kernel + wgrad_reduce_kernel",
+            "bound": "mfma", "achieved": o["achieved"], "peak": o["peak"], "unit": "TFLOP/s",
+            "frac": o["frac"], "avg_call_us": o["us"],
+            "traffic": MEASURED_TRAFFIC.get("conv2d_bwd_filter_" + a.dtype)}
     out["ops"] = ops
-    out["cpu_baseline"] = cpu_baseline
-    out["cpu_onednn"] = cpu_onednn
+    # the reference's CPU path: the oneDNN primitives its extension requests (through PyTorch-CPU,
+    # whose embedded oneDNN executes them); the C restatement used as the parity checker is listed
+    # beside it
+    out["cpu_baseline"] = cpu_onednn
+    out["cpu_port"] = cpu_port
     out["cpu_onednn_bandwidth_ops"] = cpu_bw
     print(json.dumps(out))
     return 0
@@ -430,9 +467,11 @@ def cpu_legs():
         if el > 8.0:
             break
     onednn = {"value": 2 * CONV_FLOP * reps / el / 1e12, "unit": "TFLOP/s", "cores": threads,
-              "kind": "oneDNN %s via PyTorch-CPU aten::convolution_backward (the primitives the "
-                      "reference's oneDNN extension requests), full batch 32" % _onednn_version(),
-              "sample": "%d repetitions, %.1f s" % (reps, el)}
+              "kind": "reference",
+              "detail": "oneDNN %s through PyTorch-CPU aten::convolution_backward: the backward-data and "
+                        "backward-weights(+bias) primitives the reference's oneDNN extension requests "
+                        "(its own C++ cannot be built offline)" % _onednn_version(),
+              "sample": "%d repetitions of the pair on the full batch of 32, %.1f s" % (reps, el)}
     return port, onednn
 
 
@@ -471,6 +510,12 @@ def cpu_bandwidth_legs():
     leg("batchnorm_fwd_train", 2 * T,
         lambda: torch.ops.aten.native_batch_norm(x, gamma, beta, None, None, True, 0.0, 1e-5))
 
+    y_, sm_, sv_ = torch.ops.aten.native_batch_norm(x, gamma, beta, None, None, True, 0.0, 1e-5)
+    leg("batchnorm_bwd", 3 * T,
+        lambda: torch.ops.aten.native_batch_norm_backward(dy, x, gamma, None, None, sm_, sv_, True, 1e-5,
+                                                          [True, True, True]))
+    del y_
+
     def bn_fwd_bwd():
         xr = x.to_dense().requires_grad_(True)
         y = F.batch_norm(xr.to_mkldnn(), None, None, gamma, beta, True, 0.0, 1e-5)
@@ -483,6 +528,10 @@ def cpu_bandwidth_legs():
     leg("pool2d_max_fwd", nx + ny + ny // 4, lambda: torch.max_pool2d(px, 3, 2, 1))
     leg("pool2d_avg_fwd", nx + ny, lambda: F.avg_pool2d(px, 3, 2, 1, count_include_pad=False))
     pdy = torch.randn(32, 64, 56, 56, generator=g).to_mkldnn()
+    leg("pool2d_avg_bwd", nx + ny,
+        lambda: torch.ops.aten.avg_pool2d_backward(pdy, px, [3, 3], [2, 2], [1, 1], False, False, None))
+    # max pooling's backward primitive needs the forward primitive's workspace, which PyTorch only keeps
+    # inside autograd: its time alone is the difference of the two legs "fwd+bwd" and "fwd" below
 
     def pool_fwd_bwd(avg):
         xr = px.to_dense().requires_grad_(True)
@@ -494,6 +543,30 @@ def cpu_bandwidth_legs():
     leg("pool2d_avg_fwd+bwd (autograd, includes layout conversions)", 2 * (nx + ny),
         lambda: pool_fwd_bwd(True))
     return out
+
+
+def step_bench(a):
+    """Whole training steps through the C++ host layer: runs flashlight_amd/lib/flhip_step_bench
+    (built by flashlight_amd.build) and prints its JSON line."""
+    import subprocess
+    exe = os.path.join(ROOT, "flashlight_amd", "lib", "flhip_step_bench")
+    if not os.path.exists(exe):
+        sys.stderr.write("bench.py: %s is missing; build it with `python -m flashlight_amd.build`\n" % exe)
+        return 1
+    batch = a.batch or (64 if a.step == "resnet50" else 16)
+    r = subprocess.run([exe, a.step, str(batch), str(a.steps), str(min(a.warmup, 5)), a.dtype],
+                       capture_output=True, text=True)
+    sys.stderr.write(r.stderr)
+    if r.returncode != 0:
+        return r.returncode
+    rec = json.loads(r.stdout.strip().splitlines()[-1])
+    bd = rec["breakdown_ms"]
+    conv = sum(v for k, v in bd.items() if k.startswith("conv_"))
+    busy = sum(v for k, v in bd.items() if k not in ("span", "host_gaps"))
+    rec["conv_share_of_device_time"] = conv / busy if busy else None
+    rec["non_conv_share_of_device_time"] = 1 - conv / busy if busy else None
+    print(json.dumps(rec))
+    return 0
 
 
 def _onednn_version():

@@ -40,6 +40,7 @@ def _compile(src):
 
 HOST = os.path.join(HERE, "host")
 HOST_LIB = os.path.join(LIBDIR, "libflhip_host.so")
+STEP_BENCH = os.path.join(LIBDIR, "flhip_step_bench")
 HOST_SOURCES = ["HipTensor.cpp", "HipAutogradExtension.cpp", "Functions.cpp", "Modules.cpp", "Resnet.cpp",
                 "SequentialBuilder.cpp"]
 TESTS_DIR = os.path.join(ROOT, "tests", "cpp")
@@ -64,8 +65,12 @@ def build_host(verbose=True):
     cmd += [os.path.join(HOST, f) for f in HOST_SOURCES]
     cmd += ["-L" + LIBDIR, "-lflhip", "-Wl,-rpath,$ORIGIN"] + hiplibs
     subprocess.check_call(cmd)
+    # the whole-step benchmark program bench.py runs for its step workloads
+    cmd = cxx + ["-o", STEP_BENCH, os.path.join(HOST, "step_bench.cpp"), "-L" + LIBDIR, "-lflhip_host", "-lflhip",
+                 "-Wl,-rpath,$ORIGIN"] + hiplibs
+    subprocess.check_call(cmd)
     if verbose:
-        print("built", HOST_LIB)
+        print("built", HOST_LIB, "and", STEP_BENCH)
     return HOST_LIB
 
 

@@ -1,0 +1,147 @@
+// Whole training steps through the host layer, timed: the ResNet-50 step of configs[4]
+// (224x224x3, forward + logSoftmax / categoricalCrossEntropy + backward) and the speech
+// stack of configs[3] (three 21x1 convolutions, each with batch norm and ReLU, forward +
+// backward).  Prints one JSON object: wall time per step and, from a second, instrumented
+// run, the device time per operation class (HIP events around every operation of the
+// host layer) with the idle gaps between operations.
+//
+// usage: flhip_step_bench resnet50|speech [batch] [steps] [warmup] [f32|bf16]
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <map>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "OpObserver.h"
+#include "Resnet.h"
+
+using namespace fl;
+
+namespace {
+std::vector<float> randn(size_t n, unsigned seed) {
+  std::mt19937 gen(seed);
+  std::normal_distribution<float> d(0.f, 1.f);
+  std::vector<float> v(n);
+  for (auto& x : v) x = d(gen);
+  return v;
+}
+
+// operation name -> class of the breakdown
+const char* classOf(const std::string& op) {
+  static const std::map<std::string, const char*> m = {
+      {"conv2d", "conv_fwd"}, {"conv2dBackwardData", "conv_bwd_data"}, {"conv2dBackwardFilterBias", "conv_bwd_filter"},
+      {"batchnorm", "bn_fwd"}, {"batchnormBackward", "bn_bwd"}, {"batchnormRelu", "bn_fwd"}, {"batchnormReluBackward", "bn_bwd"},
+      {"pool2d", "pool_fwd"}, {"pool2dBackward", "pool_bwd"},
+      {"relu", "relu_add"}, {"reluBackward", "relu_add"}, {"add", "relu_add"}, {"addGrad", "relu_add"},
+      {"astype", "casts"}, {"linear", "linear"}, {"linearBackward", "linear"},
+      {"logSoftmax", "loss"}, {"logSoftmaxBackward", "loss"}, {"categoricalCrossEntropy", "loss"},
+      {"categoricalCrossEntropyBackward", "loss"}, {"(gaps)", "host_gaps"}, {"(span)", "span"}};
+  auto it = m.find(op);
+  return it == m.end() ? "other" : it->second;
+}
+}  // namespace
+
+int main(int argc, char** argv) {
+  try {
+    const std::string model = argc > 1 ? argv[1] : "resnet50";
+    const int B = argc > 2 ? std::atoi(argv[2]) : (model == "speech" ? 16 : 64);
+    const int steps = argc > 3 ? std::atoi(argv[3]) : 10;
+    const int warmup = argc > 4 ? std::atoi(argv[4]) : 3;
+    const bool half = argc > 5 && std::string(argv[5]) == "bf16";
+    setSeed(3);
+
+    std::function<float()> step;
+    std::shared_ptr<Sequential> net;
+    std::vector<Conv2D> convs;
+    std::vector<BatchNorm> bns;
+    Variable in, target, gradOut;
+    double flop = 0;   // convolution FLOP of one step (forward + both backward passes)
+    if (model == "resnet50") {
+      net = pkg::vision::resnet50();
+      Tensor x = Tensor::fromVector({224, 224, 3, B}, randn((size_t)B * 3 * 224 * 224, 1));
+      in = Variable(half ? x.astype(dtype::bf16) : x, false);
+      std::vector<int32_t> labels(B);
+      std::mt19937 gen(5);
+      for (int i = 0; i < B; ++i) labels[i] = (int32_t)(gen() % 1000);
+      target = Variable(Tensor::fromHost(Shape({B}), dtype::s32, labels.data()), false);
+      step = [&]() {
+        net->zeroGrad();
+        Variable out = logSoftmax(net->forward(in), 0);
+        Variable loss = categoricalCrossEntropy(out, target);
+        loss.backward(Variable(Tensor::fromVector({1}, {1.f}), false));
+        return loss.tensor().toHostVector()[0];
+      };
+    } else if (model == "speech") {
+      const int T = 1500, chans[4] = {80, 250, 250, 250}, strides[3] = {1, 1, 2};
+      for (int l = 0; l < 3; ++l) {
+        convs.emplace_back(chans[l], chans[l + 1], 21, 1, strides[l], 1, PaddingMode::SAME, PaddingMode::SAME);
+        bns.emplace_back(2, chans[l + 1]);
+        flop += 3.0 * 2.0 * B * chans[l + 1] * (double)(T / strides[l]) * chans[l] * 21;
+      }
+      Tensor x = Tensor::fromVector({T, 1, 80, B}, randn((size_t)B * 80 * T, 71));
+      in = Variable(half ? x.astype(dtype::bf16) : x, true);
+      Tensor g = Tensor::fromVector({T / 2, 1, 250, B}, randn((size_t)B * 250 * (T / 2), 72));
+      gradOut = Variable(half ? g.astype(dtype::bf16) : g, false);
+      step = [&]() {
+        for (auto& c : convs) c.zeroGrad();
+        for (auto& b : bns) b.zeroGrad();
+        in.zeroGrad();
+        Variable h = in;
+        for (int l = 0; l < 3; ++l) h = relu(bns[l](convs[l](h)));
+        h.backward(gradOut);
+        fl::sync();
+        return 0.f;
+      };
+    } else {
+      std::fprintf(stderr, "unknown model %s\n", model.c_str());
+      return 2;
+    }
+
+    float loss = 0;
+    for (int i = 0; i < warmup; ++i) loss = step();
+    fl::sync();
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < steps; ++i) loss = step();
+    fl::sync();
+    const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / steps;
+
+    // instrumented run: device time per operation
+    StepProfiler prof;
+    detail::setOpObserver(&prof);
+    const int psteps = steps < 5 ? steps : 5;
+    for (int i = 0; i < psteps; ++i) step();
+    detail::setOpObserver(nullptr);
+    const auto table = prof.collect();
+    std::map<std::string, StepProfiler::Entry> classes;
+    for (const auto& kv : table) {
+      auto& c = classes[classOf(kv.first)];
+      c.ms += kv.second.ms / psteps;
+      c.calls += kv.second.calls / psteps;
+    }
+
+    std::printf("{\"model\": \"%s\", \"batch\": %d, \"dtype\": \"%s\", \"steps\": %d, \"warmup\": %d, \"ms_per_step\": %.4f, "
+                "\"samples_per_s\": %.1f, \"loss\": %.5f, \"conv_gflop_per_step\": %.2f, \"device_cache_mb\": %.1f, "
+                "\"breakdown_ms\": {",
+                model.c_str(), B, half ? "bf16" : "f32", steps, warmup, ms, B / ms * 1e3, loss, flop / 1e9,
+                deviceCacheBytes() / 1e6);
+    bool first = true;
+    for (const auto& kv : classes) {
+      std::printf("%s\"%s\": %.4f", first ? "" : ", ", kv.first.c_str(), kv.second.ms);
+      first = false;
+    }
+    std::printf("}, \"calls\": {");
+    first = true;
+    for (const auto& kv : classes) {
+      std::printf("%s\"%s\": %ld", first ? "" : ", ", kv.first.c_str(), kv.second.calls);
+      first = false;
+    }
+    std::printf("}}\n");
+    std::fflush(stdout);
+    return 0;
+  } catch (const std::exception& e) {
+    std::fprintf(stderr, "step bench failed: %s\n", e.what());
+    return 2;
+  }
+}
