@@ -75,6 +75,7 @@ SYMBOLS = {
     "flhip_rnn_fwd": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, C.c_size_t, _VP, C.c_size_t, _VP]),
     "flhip_rnn_bwd": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, C.c_size_t, _VP, _VP, _VP, _VP, _VP,
                                 C.c_size_t, _VP]),
+    "flhip_reorder": (C.c_int, [_VP, _VP, C.POINTER(C.c_int64), C.POINTER(C.c_int32), C.c_int, _VP]),
     "flhip_affine_fwd": (C.c_int, [_VP, _VP, _VP, _VP, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_int,
                                    _VP]),
     "flhip_affine_bwd_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int64, C.c_int64, C.c_int]),

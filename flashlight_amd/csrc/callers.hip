@@ -305,6 +305,25 @@ affine_fwd_kernel(const T* __restrict__ x, const T* __restrict__ w, const T* __r
   }
 }
 
+// dst[i0, i1, i2, i3] = src[...] with dst dimension k taken from src dimension perm[k]
+// (column-major, dimension 0 fastest); one thread per dst element, writes coalesced
+struct ReorderGeom {
+  long long d[4];    // dst extents
+  long long ss[4];   // src stride of the dimension that dst dimension k walks
+};
+template <typename T>
+__global__ void __launch_bounds__(256)
+reorder_kernel(const T* __restrict__ src, T* __restrict__ dst, size_t n, ReorderGeom g) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += stride) {
+    size_t t = e;
+    const size_t i0 = t % (size_t)g.d[0]; t /= (size_t)g.d[0];
+    const size_t i1 = t % (size_t)g.d[1]; t /= (size_t)g.d[1];
+    const size_t i2 = t % (size_t)g.d[2]; t /= (size_t)g.d[2];
+    dst[e] = src[i0 * g.ss[0] + i1 * g.ss[1] + i2 * g.ss[2] + t * g.ss[3]];
+  }
+}
+
 // Backward: dx = w * dy, and per parameter element the partial sums of dy * x and dy
 // over slice blockIdx.y of its elements: part[(m * S + s) * 2 + {0, 1}].
 template <typename T>
@@ -520,6 +539,35 @@ extern "C" int flhip_cce_bwd(const float* grad, const int32_t* target, const flo
                        as_stream(stream), grad, target, stats, (bf16_t*)dx, classes, cols, reduction,
                        ignore_index);
   return check_launch("cce_bwd");
+}
+
+extern "C" int flhip_reorder(const void* src, void* dst, const int64_t* dims, const int32_t* perm,
+                             int dtype, void* stream) {
+  FLHIP_REQUIRE(src && dst && dims && perm, "reorder: null argument");
+  FLHIP_REQUIRE(dtype_ok(dtype), "reorder: unknown dtype");
+  long long sstride[4], st = 1;
+  unsigned seen = 0;
+  for (int k = 0; k < 4; ++k) {
+    FLHIP_REQUIRE(dims[k] > 0, "reorder: sizes must be positive");
+    FLHIP_REQUIRE(perm[k] >= 0 && perm[k] < 4, "reorder: permutation entry out of range");
+    seen |= 1u << perm[k];
+    sstride[k] = st;
+    st *= dims[k];
+  }
+  FLHIP_REQUIRE(seen == 0xf, "reorder: not a permutation of the four dimensions");
+  ReorderGeom g;
+  for (int k = 0; k < 4; ++k) {
+    g.d[k] = dims[perm[k]];
+    g.ss[k] = sstride[perm[k]];
+  }
+  const size_t n = (size_t)st;
+  if (dtype == FLHIP_F32)
+    hipLaunchKernelGGL((reorder_kernel<float>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream),
+                       (const float*)src, (float*)dst, n, g);
+  else
+    hipLaunchKernelGGL((reorder_kernel<bf16_t>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream),
+                       (const bf16_t*)src, (bf16_t*)dst, n, g);
+  return check_launch("reorder");
 }
 
 extern "C" int flhip_affine_fwd(const void* x, const void* w, const void* b, void* y, int64_t outer,

@@ -363,6 +363,41 @@ Variable moddims(const Variable& input, const Shape& dims) {
   return Variable(input.tensor().reshaped(target), {input}, gradFunc);
 }
 
+namespace {
+Tensor reorderTensor(const Tensor& in, const std::vector<int>& perm) {
+  detail::OpScope scope("reorder");
+  int64_t dims[4] = {1, 1, 1, 1};
+  int32_t pm[4] = {0, 1, 2, 3};
+  for (int i = 0; i < in.ndim(); ++i) dims[i] = in.dim(i);
+  for (size_t i = 0; i < perm.size(); ++i) pm[i] = perm[i];
+  std::vector<Dim> oshape(in.ndim());
+  for (int i = 0; i < in.ndim(); ++i) oshape[i] = in.dim(perm[i]);
+  Tensor out(Shape(oshape), in.type());
+  check(flhip_reorder(in.device(), out.device(), dims, pm, tagOf(in.type(), "reorder"), hipBackendStream()));
+  if (scope.on()) scope.done({in}, {out}, {pm[0], pm[1], pm[2], pm[3]});
+  return out;
+}
+}  // namespace
+
+Variable reorder(const Variable& input, const Shape& dims) {
+  const int nd = input.ndim();
+  if (dims.ndim() != nd || nd > 4)
+    throw std::invalid_argument("reorder: expects one entry per dimension of the input (at most 4)");
+  std::vector<int> perm(nd), inverse(nd);
+  std::vector<bool> seen(nd, false);
+  for (int i = 0; i < nd; ++i) {
+    const Dim d = dims.dim(i);
+    if (d < 0 || d >= nd || seen[(size_t)d]) throw std::invalid_argument("reorder: not a permutation of the dimensions");
+    seen[(size_t)d] = true;
+    perm[i] = (int)d;
+    inverse[(size_t)d] = i;
+  }
+  auto gradFunc = [inverse](std::vector<Variable>& inputs, const Variable& gradOutput) {
+    inputs[0].addGrad(Variable(reorderTensor(gradOutput.tensor(), inverse), false));
+  };
+  return Variable(reorderTensor(input.tensor(), perm), {input}, gradFunc);
+}
+
 Variable linear(const Variable& input, const Variable& weight) {
   return linear(input, weight, Variable());
 }

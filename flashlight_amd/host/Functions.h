@@ -93,6 +93,9 @@ Variable affine(const Variable& input, const Variable& weight, const Variable& b
 Variable relu(const Variable& input);
 // fl::moddims / View: same data, new shape; one dimension may be -1 (Functions.cpp:790-829)
 Variable moddims(const Variable& input, const Shape& dims);
+// fl::reorder (Functions.cpp:1010-1042): dimension k of the result is dimension dims[k] of the
+// input; the gradient is reordered back with the inverse permutation
+Variable reorder(const Variable& input, const Shape& dims);
 // fl::linear (Functions.cpp:1255-1309): weight [out, in], input [in, ...], bias [out] or empty
 Variable linear(const Variable& input, const Variable& weight, const Variable& bias);
 Variable linear(const Variable& input, const Variable& weight);

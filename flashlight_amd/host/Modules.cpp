@@ -277,30 +277,53 @@ Variable LayerNorm::forward(const Variable& in) {
   }
   const int maxAxis = *std::max_element(axisComplement_.begin(), axisComplement_.end());
   const int minAxis = *std::min_element(axisComplement_.begin(), axisComplement_.end());
-  if ((int)axisComplement_.size() != maxAxis - minAxis + 1)
-    throw std::invalid_argument("LayerNorm: a non-contiguous axis complement needs a reorder, which "
-                                "this backend does not provide");
+  bool axesContinuous = (int)axisComplement_.size() == maxAxis - minAxis + 1;
+  // per-element parameters over normalised axes that are not contiguous take the reorder too: the
+  // broadcast kernel wants them side by side, and the two reorders cancel
+  if (affine_ && axisSize_ != kLnVariableAxisSize && axis_.back() - axis_.front() + 1 != (int)axis_.size())
+    axesContinuous = false;
+  // a complement that is not contiguous: reorder so that the normalised axes lead and the
+  // complement follows, batch-normalise over the trailing axes, reorder back (:63-86, 98-108)
+  Variable inputToBn = input;
+  std::vector<int> inNormAxes = axisComplement_, normAxes = axis_;
+  std::vector<Dim> reorderDims, restoreDims((size_t)input.ndim());
+  if (!axesContinuous) {
+    for (int d : axis_) reorderDims.push_back(d);
+    inNormAxes.clear();
+    for (int d : axisComplement_) {
+      inNormAxes.push_back((int)reorderDims.size());
+      reorderDims.push_back(d);
+    }
+    for (size_t i = 0; i < reorderDims.size(); ++i) restoreDims[(size_t)reorderDims[i]] = (Dim)i;
+    inputToBn = reorder(input, Shape(reorderDims));
+    for (size_t i = 0; i < axis_.size(); ++i) normAxes[i] = (int)i;
+  }
   Variable dummyInMean, dummyInVar;
   const Variable none(Tensor(), false);
-  Variable output = batchnorm(input, none, none, dummyInMean, dummyInVar, axisComplement_, true, 0.0,
+  Variable output = batchnorm(inputToBn, none, none, dummyInMean, dummyInVar, inNormAxes, true, 0.0,
                               epsilon_);
+  // The scale and shift broadcast one parameter element per position along the normalised
+  // axes (:110-128).  After a reorder they are applied before reordering back: the
+  // normalised axes lead there, in the parameters' own order, so the broadcast is the
+  // contiguous [outer][mid][inner] one; the result is the same as tiling over the restored
+  // tensor.
   if (affine_) {
     const Variable weight = params_[0].astype(output.type());
     const Variable bias = params_[1].astype(output.type());
     if (axisSize_ == kLnVariableAxisSize) {
       output = detail::affine(output, weight, bias, 1, 1, output.elements(), true);
     } else {
-      // the parameters take the input's shape with the complement axes set to 1
-      if (axis_.empty() || axis_.back() - axis_.front() + 1 != (int)axis_.size())
+      if (normAxes.empty() || normAxes.back() - normAxes.front() + 1 != (int)normAxes.size())
         throw std::invalid_argument("LayerNorm: per-element parameters need contiguous normalised axes");
       Dim inner = 1, mid = 1, outer = 1;
-      for (int d = 0; d < input.ndim(); ++d)
-        (d < axis_.front() ? inner : d <= axis_.back() ? mid : outer) *= input.dim(d);
+      for (int d = 0; d < output.ndim(); ++d)
+        (d < normAxes.front() ? inner : d <= normAxes.back() ? mid : outer) *= output.dim(d);
       if (mid != axisSize_)
         throw std::invalid_argument("[LayerNorm] Input size along the norm axis doesn't with axisSize.");
       output = detail::affine(output, weight, bias, outer, mid, inner, false);
     }
   }
+  if (!axesContinuous) output = reorder(output, Shape(restoreDims));
   return moddims(output, in.shape());
 }
 

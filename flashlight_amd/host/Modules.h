@@ -175,8 +175,8 @@ class BatchNorm : public UnaryModule {
 };
 
 // flashlight/fl/nn/modules/LayerNorm.cpp:20-160: normalises over `axis` by calling
-// batchnorm over the complement axes; the complement must be contiguous here (the
-// other case needs a reorder, which this backend does not provide)
+// batchnorm over the complement axes; a complement that is not contiguous goes through
+// fl::reorder as in the reference
 constexpr int kLnVariableAxisSize = -1;
 class LayerNorm : public UnaryModule {
  public:

@@ -452,6 +452,23 @@ def affine_backward(grad_output, input, weight, view):
     return dx, dw, db
 
 
+def reorder(input, perm_whcn):
+    """fl::reorder on the Flashlight view of `input` (torch shape reversed, padded to four
+    dimensions): Flashlight dimension k of the result is dimension perm_whcn[k] of the
+    input.  -> a new contiguous tensor (torch shape = reversed result shape)."""
+    x = _dev(input, "input")
+    whcn = list(x.shape)[::-1]
+    whcn += [1] * (4 - len(whcn))
+    perm = [int(v) for v in perm_whcn]
+    if sorted(perm) != [0, 1, 2, 3]:
+        raise ValueError("reorder: not a permutation of the four dimensions")
+    out = torch.empty([whcn[k] for k in perm][::-1], dtype=x.dtype, device=x.device)
+    dims = (C.c_int64 * 4)(*whcn)
+    pm = (C.c_int32 * 4)(*perm)
+    capi.check(capi.lib().flhip_reorder(_ptr(x), _ptr(out), dims, pm, _dtype_tag(x), _stream()))
+    return out
+
+
 def _layer_norm_axes(shape, norm_axes):
     whcn = list(shape)[::-1]
     if len(whcn) > 4:
@@ -459,36 +476,61 @@ def _layer_norm_axes(shape, norm_axes):
     whcn += [1] * (4 - len(whcn))
     norm = sorted(int(a) for a in norm_axes)
     comp = [d for d in range(4) if d not in norm]
-    if not comp or comp != list(range(comp[0], comp[-1] + 1)):
-        raise ValueError("LayerNorm: a non-contiguous axis complement needs a reorder, "
-                         "which this backend does not provide")
-    return whcn, norm, comp
+    if not comp:
+        raise ValueError("LayerNorm: no axis left to batch over")
+    contiguous = comp == list(range(comp[0], comp[-1] + 1))
+    return whcn, norm, comp, contiguous
 
 
 def layer_norm(input, norm_axes, epsilon=1e-5, weight=None, bias=None):
     """fl::LayerNorm::forward (nn/modules/LayerNorm.cpp:42-131): batchnorm in train mode
     over the complement of the normalised axes with no parameters and no running
-    statistics, then the broadcast scale and shift.  -> (output, ctx for the backward)."""
+    statistics, then the broadcast scale and shift.  When the complement axes are not
+    contiguous the tensor is reordered first (normalised axes, then the complement) and
+    the result reordered back, as the reference does; the scale and shift are then
+    applied in the reordered layout, where the normalised axes are the leading ones.
+    -> (output, ctx for the backward)."""
     x = _dev(input, "input")
-    whcn, norm, comp = _layer_norm_axes(x.shape, norm_axes)
+    whcn, norm, comp, contiguous = _layer_norm_axes(x.shape, norm_axes)
+    if weight is not None and weight.numel() > 1 and norm != list(range(norm[0], norm[-1] + 1)):
+        contiguous = False       # the broadcast of per-element parameters needs leading normalised axes too
     x4 = x.reshape(whcn[::-1])
-    xhat, sm, si = batchnorm(x4, None, None, None, None, comp, True, 0.0, epsilon)
-    ctx = {"x4": x4, "xhat": xhat, "sm": sm, "si": si, "comp": comp, "view": None}
+    ctx = {"view": None, "perm": None, "shape": tuple(x.shape)}
+    if contiguous:
+        bn_axes, w4 = comp, whcn
+    else:
+        ctx["perm"] = norm + comp
+        x4 = reorder(x4, ctx["perm"])
+        w4 = [whcn[k] for k in ctx["perm"]]
+        bn_axes = list(range(len(norm), 4))
+        norm = list(range(len(norm)))
+    xhat, sm, si = batchnorm(x4, None, None, None, None, bn_axes, True, 0.0, epsilon)
+    ctx.update({"x4": x4, "xhat": xhat, "sm": sm, "si": si, "comp": bn_axes})
     out = xhat
     if weight is not None:
-        ctx["view"] = _affine_view(whcn, norm, weight.numel())
+        ctx["view"] = _affine_view(w4, norm, weight.numel())
         out = affine(xhat, weight, bias, ctx["view"])
+    if ctx["perm"] is not None:
+        inv = [ctx["perm"].index(k) for k in range(4)]
+        out = reorder(out, inv)
     return out.reshape(x.shape), ctx
 
 
 def layer_norm_backward(grad_output, ctx, weight=None):
     """-> (gradInput, gradWeight, gradBias) of `layer_norm` (the last two None without
     parameters)."""
-    g = _dev(grad_output, "gradOutput").reshape(ctx["x4"].shape)
+    g = _dev(grad_output, "gradOutput")
+    if ctx["perm"] is not None:
+        whcn = list(g.shape)[::-1]
+        whcn += [1] * (4 - len(whcn))
+        g = reorder(g.reshape(whcn[::-1]), ctx["perm"])
+    g = g.reshape(ctx["x4"].shape)
     dw = db = None
     if ctx["view"] is not None:
         g, dw, db = affine_backward(g, ctx["xhat"], weight, ctx["view"])
     dx, _, _ = batchnorm_backward(g, ctx["x4"], None, ctx["sm"], ctx["si"], ctx["comp"])
+    if ctx["perm"] is not None:
+        dx = reorder(dx, [ctx["perm"].index(k) for k in range(4)])
     return dx.reshape(grad_output.shape), dw, db
 
 

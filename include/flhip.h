@@ -258,6 +258,14 @@ int flhip_matmul(const void* A, const void* B, void* C, int32_t M, int32_t N,
 int flhip_sum_columns(const void* x, float* out, int32_t rows, int32_t cols, int dtype,
                       void* stream);
 
+/* fl::reorder (flashlight/fl/autograd/Functions.cpp:1010-1042) of a tensor with the four
+ * column-major extents dims[0..3] (dims[0] fastest; pad with 1): dimension k of dst is
+ * dimension perm[k] of src.  LayerNorm uses it when the axes it batches over are not
+ * contiguous (flashlight/fl/nn/modules/LayerNorm.cpp:63-86, 98-108).  src and dst must not
+ * overlap. */
+int flhip_reorder(const void* src, void* dst, const int64_t* dims, const int32_t* perm,
+                  int dtype, void* stream);
+
 /* The affine part of fl::LayerNorm (flashlight/fl/nn/modules/LayerNorm.cpp:110-128),
  * tileAs(weight, input) * output + tileAs(bias, input), on a tensor viewed as
  * [outer][mid][inner] (inner fastest): y = w[m] * x + b[m] with one parameter element

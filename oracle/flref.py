@@ -275,7 +275,8 @@ def cce_bwd(shape, grad, target, count, reduction=1, ignore=-1):
 # ---- fl::LayerNorm::forward (flashlight/fl/nn/modules/LayerNorm.cpp:42-131) restated on
 # the functions above: the shape is padded to 4 dimensions, batchnorm runs in train mode
 # over the complement of the normalised axes with no parameters, then the broadcast
-# scale and shift.  Only a contiguous complement is restated (the other case reorders).
+# scale and shift.  A non-contiguous complement goes through the reference's reorder
+# (numpy transposes here), LayerNorm.cpp:63-86 and 98-108.
 def layer_norm_plan(shape_whcn, norm_axes, nparam):
     whcn = list(shape_whcn) + [1] * (4 - len(shape_whcn))
     norm = sorted(norm_axes)
@@ -294,23 +295,89 @@ def layer_norm_plan(shape_whcn, norm_axes, nparam):
     return bn_view(whcn, comp), view
 
 
+def _ln_reorder(shape_whcn, norm_axes, nparam=0):
+    """The reorder of LayerNorm.cpp:63-86 for a non-contiguous complement, or None: Flashlight
+    dims = normalised axes (ascending) then the complement; batchnorm then runs over the
+    last len(comp) dims.  Returned as numpy axes of the row-major array (reversed order).
+    Per-element parameters over normalised axes that are not contiguous take this general
+    path too (the transposes cancel; the broadcast is then plain numpy)."""
+    whcn = list(shape_whcn) + [1] * (4 - len(shape_whcn))
+    norm = sorted(norm_axes)
+    comp = [d for d in range(4) if d not in norm]
+    norm_ok = nparam <= 1 or norm == list(range(norm[0], norm[-1] + 1))
+    if comp == list(range(comp[0], comp[-1] + 1)) and norm_ok:
+        return None
+    order = norm + comp                                   # Flashlight dim i of the result = dim order[i]
+    np_axes = [3 - d for d in order][::-1]                # numpy (row-major) axes of the result
+    new_whcn = [whcn[d] for d in order]
+    return whcn, norm, comp, np_axes, new_whcn
+
+
+def _ln_bshape(whcn, norm):
+    """numpy broadcast shape of per-element parameters: the tensor's shape with the complement
+    axes set to 1 (LayerNorm.cpp:113-124)."""
+    return [whcn[d] if d in norm else 1 for d in range(4)][::-1]
+
+
 def layer_norm_fwd(x, shape_whcn, norm_axes, eps, w=None, b=None):
     """-> (y, xhat, mean, var); x is the flat/any-shape array of the tensor's memory."""
-    bnv, view = layer_norm_plan(shape_whcn, norm_axes, 0 if w is None else np.size(w))
+    ro = _ln_reorder(shape_whcn, norm_axes, 0 if w is None else np.size(w))
+    if ro is None:
+        bnv, view = layer_norm_plan(shape_whcn, norm_axes, 0 if w is None else np.size(w))
+        ones, zeros = np.ones(bnv[1], np.float32), np.zeros(bnv[1], np.float32)
+        xhat, mean, var = bn_fwd_train(*bnv, x, ones, zeros, eps)
+        y = xhat if w is None else affine_fwd(*view, xhat, w, b)
+        return y, xhat, mean, var
+    whcn, norm, comp, np_axes, new_whcn = ro
+    x4 = np.asarray(x, np.float32).reshape(whcn[::-1])
+    xr = np.ascontiguousarray(x4.transpose(np_axes))                       # reorder(input, reorderDims)
+    bnv = bn_view(new_whcn, list(range(len(norm), 4)))
     ones, zeros = np.ones(bnv[1], np.float32), np.zeros(bnv[1], np.float32)
-    xhat, mean, var = bn_fwd_train(*bnv, x, ones, zeros, eps)
-    y = xhat if w is None else affine_fwd(*view, xhat, w, b)
+    xh_r, mean, var = bn_fwd_train(*bnv, xr, ones, zeros, eps)
+    xhat = np.ascontiguousarray(xh_r.reshape(xr.shape).transpose(np.argsort(np_axes)))   # restore
+    y = xhat
+    if w is not None:
+        if np.size(w) == 1:
+            y = (np.float32(w.reshape(-1)[0]) * xhat + np.float32(b.reshape(-1)[0])).astype(np.float32)
+        else:
+            bs = _ln_bshape(whcn, norm)
+            y = (np.asarray(w, np.float32).reshape(bs) * xhat + np.asarray(b, np.float32).reshape(bs)).astype(np.float32)
     return y, xhat, mean, var
 
 
 def layer_norm_bwd(dy, x, xhat, mean, var, shape_whcn, norm_axes, eps, w=None):
     """-> (dx, dw, db)"""
-    bnv, view = layer_norm_plan(shape_whcn, norm_axes, 0 if w is None else np.size(w))
+    ro = _ln_reorder(shape_whcn, norm_axes, 0 if w is None else np.size(w))
+    if ro is None:
+        bnv, view = layer_norm_plan(shape_whcn, norm_axes, 0 if w is None else np.size(w))
+        dw = db = None
+        g = dy
+        if w is not None:
+            g, dw, db = affine_bwd(*view, dy, xhat, w)
+        dx, _, _ = bn_bwd(*bnv, x, g, np.ones(bnv[1], np.float32), mean, var, eps)
+        return dx, dw, db
+    whcn, norm, comp, np_axes, new_whcn = ro
+    shape = whcn[::-1]
+    dy4 = np.asarray(dy, np.float32).reshape(shape)
+    xh4 = np.asarray(xhat, np.float32).reshape(shape)
     dw = db = None
-    g = dy
+    g = dy4
     if w is not None:
-        g, dw, db = affine_bwd(*view, dy, xhat, w)
-    dx, _, _ = bn_bwd(*bnv, x, g, np.ones(bnv[1], np.float32), mean, var, eps)
+        d64, h64 = dy4.astype(np.float64), xh4.astype(np.float64)
+        if np.size(w) == 1:
+            dw = np.array([(d64 * h64).sum()], np.float32)
+            db = np.array([d64.sum()], np.float32)
+            g = (np.float32(np.asarray(w).reshape(-1)[0]) * dy4).astype(np.float32)
+        else:
+            red = tuple(3 - d for d in comp)
+            dw = (d64 * h64).sum(axis=red).reshape(-1).astype(np.float32)
+            db = d64.sum(axis=red).reshape(-1).astype(np.float32)
+            g = (np.asarray(w, np.float32).reshape(_ln_bshape(whcn, norm)) * dy4).astype(np.float32)
+    xr = np.ascontiguousarray(np.asarray(x, np.float32).reshape(shape).transpose(np_axes))
+    gr = np.ascontiguousarray(g.transpose(np_axes))
+    bnv = bn_view(new_whcn, list(range(len(norm), 4)))
+    dx_r, _, _ = bn_bwd(*bnv, xr, gr, np.ones(bnv[1], np.float32), mean, var, eps)
+    dx = np.ascontiguousarray(dx_r.reshape(xr.shape).transpose(np.argsort(np_axes)))
     return dx, dw, db
 
 

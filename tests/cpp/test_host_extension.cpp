@@ -592,9 +592,62 @@ static void testLayerNormModule() {
   Variable input3(Tensor::fromVector({4, 4, 3}, randn(48, 52)), true);
   LayerNorm module4(std::vector<int>{0}, eps, false);
   CHECK(module4.forward(input3).shape() == input3.shape());
-  // a complement that is not contiguous needs a reorder
-  LayerNorm module5(std::vector<int>{0, 2}, eps, false);
-  CHECK(throws<std::invalid_argument>([&] { module5.forward(input); }));
+  // a complement that is not contiguous goes through fl::reorder (LayerNorm.cpp:63-86): normalise
+  // over dimensions {0, 2} of [4, 4, 3, F], i.e. per (h, n) over (w, c); direct definition
+  {
+    LayerNorm module5(std::vector<int>{0, 2}, eps, false);
+    std::vector<float> want5(x.size());
+    for (int n = 0; n < F; ++n)
+      for (int h = 0; h < 4; ++h) {
+        auto at = [&](int w_, int c) { return ((size_t)(n * 3 + c) * 4 + h) * 4 + w_; };
+        double m = 0, v = 0;
+        for (int c = 0; c < 3; ++c) for (int w_ = 0; w_ < 4; ++w_) m += x[at(w_, c)];
+        m /= 12;
+        for (int c = 0; c < 3; ++c) for (int w_ = 0; w_ < 4; ++w_) v += (x[at(w_, c)] - m) * (x[at(w_, c)] - m);
+        v /= 12;
+        for (int c = 0; c < 3; ++c) for (int w_ = 0; w_ < 4; ++w_) want5[at(w_, c)] = (float)((x[at(w_, c)] - m) / std::sqrt(v + eps));
+      }
+    Variable out5 = module5.forward(input);
+    CHECK(out5.shape() == input.shape() && relL2(hostOf(out5), want5) <= 1e-4);
+  }
+  // normalise dimension 1 of [W, H, C, N] with one scale / shift element per h (complement {0, 2, 3}):
+  // equals the contiguous case on the tensor transposed by hand to [H, W, C, N], outputs and gradients
+  {
+    const int W_ = 6, H_ = 5, C_ = 3, N_ = 4;
+    auto xa = randn((size_t)W_ * H_ * C_ * N_, 57, 1.5f, 0.2f), dya = randn(xa.size(), 58);
+    auto wa = randn(H_, 59, 0.3f, 1.f), ba = randn(H_, 60);
+    std::vector<float> xb(xa.size()), dyb(xa.size());
+    auto ia = [&](int w_, int h, int r) { return ((size_t)r * H_ + h) * W_ + w_; };   // r = (n, c) flattened
+    auto ib = [&](int w_, int h, int r) { return ((size_t)r * W_ + w_) * H_ + h; };
+    for (int r = 0; r < C_ * N_; ++r)
+      for (int h = 0; h < H_; ++h)
+        for (int w_ = 0; w_ < W_; ++w_) { xb[ib(w_, h, r)] = xa[ia(w_, h, r)]; dyb[ib(w_, h, r)] = dya[ia(w_, h, r)]; }
+    LayerNorm lnA(1, eps, true, H_), lnB(0, eps, true, H_);
+    for (LayerNorm* m : {&lnA, &lnB}) {
+      m->setParams(Variable(Tensor::fromVector({H_}, wa), true), 0);
+      m->setParams(Variable(Tensor::fromVector({H_}, ba), true), 1);
+    }
+    Variable va(Tensor::fromVector({W_, H_, C_, N_}, xa), true), vb(Tensor::fromVector({H_, W_, C_, N_}, xb), true);
+    Variable oa = lnA.forward(va), ob = lnB.forward(vb);
+    oa.backward(Variable(Tensor::fromVector({W_, H_, C_, N_}, dya), false));
+    ob.backward(Variable(Tensor::fromVector({H_, W_, C_, N_}, dyb), false));
+    auto unperm = [&](const std::vector<float>& b_) {
+      std::vector<float> a_(b_.size());
+      for (int r = 0; r < C_ * N_; ++r)
+        for (int h = 0; h < H_; ++h)
+          for (int w_ = 0; w_ < W_; ++w_) a_[ia(w_, h, r)] = b_[ib(w_, h, r)];
+      return a_;
+    };
+    CHECK(oa.shape() == Shape({W_, H_, C_, N_}));
+    CHECK(relL2(hostOf(oa), unperm(hostOf(ob))) <= 1e-6);
+    CHECK(relL2(hostOf(va.grad()), unperm(hostOf(vb.grad()))) <= 1e-6);
+    CHECK(relL2(hostOf(lnA.param(0).grad()), hostOf(lnB.param(0).grad())) <= 1e-6);
+    CHECK(relL2(hostOf(lnA.param(1).grad()), hostOf(lnB.param(1).grad())) <= 1e-6);
+    // fl::reorder itself: the inverse permutation restores the tensor bit for bit
+    Variable rr = reorder(reorder(va, Shape({2, 0, 3, 1})), Shape({1, 3, 0, 2}));
+    CHECK(hostOf(rr) == xa);
+    CHECK(throws<std::invalid_argument>([&] { reorder(va, Shape({0, 0, 1, 2})); }));
+  }
   CHECK(throws<std::invalid_argument>([&] { LayerNorm(std::vector<int>{3}, eps, true, F + 1).forward(input); }));
 
   // [C, T, B], normalise C with per-element scale and shift; forward and backward against

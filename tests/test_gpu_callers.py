@@ -155,6 +155,13 @@ def test_affine(outer, mid, inner, scalar, dtype):
     ((512, 50, 8), (0,), None),
     ((20, 4, 3, 16), (3,), "per"),
     ((56, 56, 64, 4), (0, 1, 2), "per"),
+    # non-contiguous complement: through the device reorder (LayerNorm.cpp:63-86)
+    ((6, 5, 4, 3), (1,), "per"),
+    ((6, 5, 4, 3), (1, 2), None),
+    ((6, 5, 4, 3), (0, 2), "scalar"),
+    ((4, 7, 3, 2), (1, 3), "per"),
+    ((32, 50, 16), (1,), "per"),
+    ((40, 30, 8, 6), (0, 3), "per"),
 ])
 def test_layer_norm(whcn, norm, params, dtype):
     # fl::LayerNorm::forward (nn/modules/LayerNorm.cpp:42-131) = the extension's batchnorm
@@ -185,12 +192,28 @@ def test_layer_norm(whcn, norm, params, dtype):
         assert rel_l2(host(dw), rdw) <= tol and rel_l2(host(db), rdb) <= tol
 
 
-def test_layer_norm_needs_contiguous_complement():
-    x = dev(np.zeros((2, 3, 4, 5), np.float32))
-    with pytest.raises(ValueError):
-        ops.layer_norm(x, (0, 2))
+def test_layer_norm_argument_errors():
     with pytest.raises(ValueError):
         ops.layer_norm(dev(np.zeros((2, 2, 2, 2, 2), np.float32)), (0,))
+    with pytest.raises(ValueError):
+        ops.layer_norm(dev(np.zeros((2, 3, 4, 5), np.float32)), (0, 1, 2, 3))   # nothing left to batch over
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("whcn,perm", [((6, 5, 4, 3), (1, 0, 2, 3)), ((6, 5, 4, 3), (3, 2, 1, 0)),
+                                       ((7, 1, 9, 2), (2, 3, 0, 1)), ((64, 33, 1, 1), (1, 0, 2, 3)),
+                                       ((5, 4, 3), (0, 2, 1, 3))])
+def test_reorder_is_a_transpose(whcn, perm, dtype):
+    # fl::reorder: result dimension k = input dimension perm[k]; bit-exact copy
+    rng = np.random.default_rng(sum(whcn))
+    w4 = list(whcn) + [1] * (4 - len(whcn))
+    x = _round(rng.standard_normal(tuple(w4[::-1])).astype(np.float32), dtype)
+    y = ops.reorder(dev(x, dtype).reshape(tuple(whcn[::-1])), perm)
+    want = x.transpose([3 - p for p in perm][::-1])
+    assert tuple(y.shape) == want.shape
+    assert np.array_equal(host(y), want)
+    with pytest.raises(ValueError):
+        ops.reorder(dev(x, dtype), (0, 0, 1, 2))
 
 
 

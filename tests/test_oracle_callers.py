@@ -132,6 +132,13 @@ def test_affine_against_numpy_broadcast(outer, mid, inner, scalar):
     ((16, 7, 3), (0,), None),
     ((5, 4, 3, 2), (3,), "per"),
     ((8, 3), (0, 1), "scalar"),
+    # non-contiguous complement: the reorder branch (LayerNorm.cpp:63-86)
+    ((6, 5, 4, 3), (1,), "per"),
+    ((6, 5, 4, 3), (1, 2), None),
+    ((6, 5, 4, 3), (0, 2), "scalar"),
+    ((4, 7, 3, 2), (1, 3), "per"),
+    ((5, 4, 6), (1,), "per"),
+    ((6, 5, 4, 3), (0, 3), "per"),         # contiguous complement, parameters over axes that are not
 ])
 def test_layer_norm_restated_on_batchnorm_is_layer_norm(whcn, norm, params):
     # LayerNorm.cpp:42-131 against torch.nn.functional.layer_norm (float64) and its autograd
