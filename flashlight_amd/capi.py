@@ -55,6 +55,10 @@ SYMBOLS = {
                                       _VP, _VP]),
     "flhip_bn_bwd": (C.c_int, [C.POINTER(BnDesc), _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
                                 _SZ, _VP]),
+    "flhip_bn_act_fwd_train": (C.c_int, [C.POINTER(BnDesc), _VP, _VP, _VP, _VP, C.c_int, _VP, _VP, _VP, _VP, _VP,
+                                          C.c_double, C.c_double, _VP, _SZ, _VP]),
+    "flhip_bn_act_bwd": (C.c_int, [C.POINTER(BnDesc), _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
+                                    _SZ, _VP]),
     "flhip_copy_bytes": (C.c_int, [_VP, _VP, _SZ, _VP]),
     "flhip_convert": (C.c_int, [_VP, C.c_int, _VP, C.c_int, _SZ, _VP]),
     "flhip_fill": (C.c_int, [_VP, C.c_double, _SZ, C.c_int, _VP]),

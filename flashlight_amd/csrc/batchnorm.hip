@@ -182,10 +182,26 @@ __device__ __forceinline__ void finish_stats(const BnGeom& g, const BnTrainArgs&
   }
 }
 
-template <typename T, int VEC>
+// Fused epilogue of the forward kernels (FUSE instantiations): y = relu(bn(x) + residual),
+// residual optional, ReLU optional.
+template <typename T>
+struct BnFuseFwd {
+  const T* res;   // may be null
+  int relu;
+};
+// Fused prologue of the backward kernels: the incoming gradient passes the ReLU mask of the
+// forward result y first (dz = dy where y > 0), and dz itself can be written out for the
+// residual branch.
+template <typename T>
+struct BnFuseBwd {
+  const T* y;     // forward result (after the ReLU)
+  T* dres;        // may be null
+};
+
+template <typename T, int VEC, bool FUSE = false>
 __global__ void __launch_bounds__(256)
 bn_train_apply_seg(BnGeom g, const T* __restrict__ x, T* __restrict__ y,
-                   const float* __restrict__ ws, BnTrainArgs a) {
+                   const float* __restrict__ ws, BnTrainArgs a, BnFuseFwd<T> fu = BnFuseFwd<T>{nullptr, 0}) {
   __shared__ float sh[2];
   if (threadIdx.x < 64) {
     double p0, p1;
@@ -199,39 +215,53 @@ bn_train_apply_seg(BnGeom g, const T* __restrict__ x, T* __restrict__ y,
   const float scale = gm * sh[1];
   const float bt = a.beta ? a.beta[blockIdx.x] : 0.f;
   bn_seg_visit<VEC, true>(g, [&](const size_t (&off)[BN_UN], int n) {
-    Vec<T, VEC> v[BN_UN];
+    Vec<T, VEC> v[BN_UN], r[BN_UN];
 #pragma unroll
     for (int k = 0; k < BN_UN; ++k) v[k].load(x, off[k]);
+    if (FUSE && fu.res) {
+#pragma unroll
+      for (int k = 0; k < BN_UN; ++k) r[k].load(fu.res, off[k]);
+    }
 #pragma unroll
     for (int k = 0; k < BN_UN; ++k) {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) v[k].v[e] = (v[k].v[e] - mean) * scale + bt;
+      for (int e = 0; e < VEC; ++e) {
+        float t = (v[k].v[e] - mean) * scale + bt;
+        if (FUSE) {
+          if (fu.res) t += r[k].v[e];
+          if (fu.relu) t = t > 0.f ? t : 0.f;
+        }
+        v[k].v[e] = t;
+      }
       if (k < n) v[k].store(y, off[k]);
     }
   });
 }
 
 // ---- backward, segment mode ------------------------------------------------
-template <typename T, int VEC>
+template <typename T, int VEC, bool FUSE = false>
 __global__ void __launch_bounds__(256)
 bn_bwd_stats_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
-                 const float* __restrict__ save_mean, float* __restrict__ ws) {
+                 const float* __restrict__ save_mean, float* __restrict__ ws,
+                 BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr}) {
   __shared__ float red[8];
   float s1 = 0.f, s2 = 0.f;
   const long long c = blockIdx.x;
   const float mean = save_mean[c];
   bn_seg_visit<VEC, false>(g, [&](const size_t (&off)[BN_UN], int n) {
-    Vec<T, VEC> a[BN_UN], b[BN_UN];
+    Vec<T, VEC> a[BN_UN], b[BN_UN], m[BN_UN];
 #pragma unroll
     for (int k = 0; k < BN_UN; ++k) {
       a[k].load(x, off[k]);
       b[k].load(dy, off[k]);
+      if (FUSE) m[k].load(fu.y, off[k]);
     }
 #pragma unroll
     for (int k = 0; k < BN_UN; ++k) {
       float p1 = 0.f, p2 = 0.f;
 #pragma unroll
       for (int e = 0; e < VEC; ++e) {
+        if (FUSE) b[k].v[e] = m[k].v[e] > 0.f ? b[k].v[e] : 0.f;
         p1 += b[k].v[e];
         p2 += b[k].v[e] * (a[k].v[e] - mean);
       }
@@ -275,10 +305,11 @@ __device__ __forceinline__ void finish_bwd(const BnGeom& g, const BnBwdArgs& a, 
   }
 }
 
-template <typename T, int VEC>
+template <typename T, int VEC, bool FUSE = false>
 __global__ void __launch_bounds__(256)
 bn_bwd_apply_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
-                 T* __restrict__ dx, const float* __restrict__ ws, BnBwdArgs a) {
+                 T* __restrict__ dx, const float* __restrict__ ws, BnBwdArgs a,
+                 BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr}) {
   __shared__ float sh[4];
   if (threadIdx.x < 64) {
     double p0, p1;
@@ -288,17 +319,24 @@ bn_bwd_apply_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
   __syncthreads();
   const float mean = sh[0], kdy = sh[1], kx = sh[2], k0 = sh[3];
   bn_seg_visit<VEC, true>(g, [&](const size_t (&off)[BN_UN], int n) {
-    Vec<T, VEC> v[BN_UN], w[BN_UN];
+    Vec<T, VEC> v[BN_UN], w[BN_UN], m[BN_UN];
 #pragma unroll
     for (int k = 0; k < BN_UN; ++k) {
       v[k].load(x, off[k]);
       w[k].load(dy, off[k]);
+      if (FUSE) m[k].load(fu.y, off[k]);
     }
 #pragma unroll
     for (int k = 0; k < BN_UN; ++k) {
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) v[k].v[e] = kdy * w[k].v[e] + (kx * (v[k].v[e] - mean) + k0);
-      if (k < n) v[k].store(dx, off[k]);
+      for (int e = 0; e < VEC; ++e) {
+        if (FUSE) w[k].v[e] = m[k].v[e] > 0.f ? w[k].v[e] : 0.f;
+        v[k].v[e] = kdy * w[k].v[e] + (kx * (v[k].v[e] - mean) + k0);
+      }
+      if (k < n) {
+        v[k].store(dx, off[k]);
+        if (FUSE && fu.dres) w[k].store(fu.dres, off[k]);
+      }
     }
   });
 }
@@ -319,10 +357,11 @@ constexpr int RES_MIN_C_BWD = 128;
 // offset is relative to the tensor base and goes through a buffer descriptor; slots
 // past the feature get an offset past the descriptor's range, so their loads return
 // zero and their stores are dropped without a branch.
-template <int RES_THREADS, int K, int ESZ, int FENCE, bool REV = false, typename F>
+template <int RES_THREADS, int K, int ESZ, int FENCE, bool REV = false, int VEC = 4, typename F>
 __device__ __forceinline__ void res_visit(const BnGeom& g, F&& f) {
   constexpr int OOB = (int)0x80000000;
-  const int innerV = (int)(g.inner >> 2);
+  const int innerV = (int)(g.inner / VEC);
+  const int units = (int)(g.units * 4 / VEC);      // g.units counts 4-element vectors
   const int c = blockIdx.x;
   // REV walks k = K-1 .. 0: what the previous walk loaded last is asked for first,
   // while the caches still hold it
@@ -330,8 +369,8 @@ __device__ __forceinline__ void res_visit(const BnGeom& g, F&& f) {
   int o = q / innerV, i = q - o * innerV;
   const int so = RES_THREADS / innerV, si = RES_THREADS - so * innerV;
   const int row = (int)(g.C * g.inner) * ESZ;                 // bytes between outer slices
-  int off = ((o * (int)g.C + c) * (int)g.inner + i * 4) * ESZ;
-  const int step = so * row + si * 4 * ESZ;
+  int off = ((o * (int)g.C + c) * (int)g.inner + i * VEC) * ESZ;
+  const int step = so * row + si * VEC * ESZ;
   const int wrap = row - (int)g.inner * ESZ;
   // Each walk recomputes its offsets (two or three adds per vector): keeping the K
   // offsets of the first walk alive for the next one would cost K registers.
@@ -339,7 +378,7 @@ __device__ __forceinline__ void res_visit(const BnGeom& g, F&& f) {
 #pragma unroll
   for (int kk = 0; kk < K; ++kk) {
     const int k = REV ? K - 1 - kk : kk;
-    const bool in = q < (int)g.units;
+    const bool in = q < units;
     f(k, in ? off : OOB, in);
     // FENCE > 0: finish each group of FENCE vectors before starting the next, or the
     // scheduler overlaps the temporaries of all K vectors and runs out of registers
@@ -390,10 +429,10 @@ __device__ __forceinline__ void buf_st4(__amdgpu_buffer_rsrc_t r, int byte_off, 
   __builtin_amdgcn_raw_buffer_store_b64(t, r, byte_off, 0, 2);
 }
 
-template <typename T, int RES_THREADS, int K>
+template <typename T, int RES_THREADS, int K, bool FUSE = false>
 __global__ void __launch_bounds__(RES_THREADS)
 bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restrict__ y,
-                  BnTrainArgs a) {
+                  BnTrainArgs a, BnFuseFwd<T> fu = BnFuseFwd<T>{nullptr, 0}) {
   __shared__ float red[RES_THREADS / 64];
   __shared__ float sh[2];
   constexpr int ESZ = (int)sizeof(T);
@@ -421,6 +460,17 @@ bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restri
   const float mean = sh[0];
   const float scale = (a.gamma ? a.gamma[c] : 1.f) * sh[1];
   const float bt = a.beta ? a.beta[c] : 0.f;
+  if (FUSE) {
+    const __amdgpu_buffer_rsrc_t rr_ = make_rsrc(fu.res ? fu.res : x, fu.res ? bytes : 0u);   // no residual: loads give 0
+    const float lo = fu.relu ? 0.f : -__builtin_huge_valf();
+    res_visit<RES_THREADS, K, ESZ, 4>(g, [&](int k, int off, bool) {
+      const float4 r = buf_ld4_stream(rr_, off, x);
+      const float4 v = make_float4(fmaxf((xr[k].x - mean) * scale + bt + r.x, lo), fmaxf((xr[k].y - mean) * scale + bt + r.y, lo),
+                                   fmaxf((xr[k].z - mean) * scale + bt + r.z, lo), fmaxf((xr[k].w - mean) * scale + bt + r.w, lo));
+      buf_st4(yr_, off, v, y);
+    });
+    return;
+  }
   res_visit<RES_THREADS, K, ESZ, 1>(g, [&](int k, int off, bool) {
     const float4 v = make_float4((xr[k].x - mean) * scale + bt, (xr[k].y - mean) * scale + bt,
                                  (xr[k].z - mean) * scale + bt, (xr[k].w - mean) * scale + bt);
@@ -428,10 +478,14 @@ bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restri
   });
 }
 
-template <typename T, int RES_THREADS, int K>
+__device__ __forceinline__ float4 relu_mask(float4 d, float4 y) {
+  return make_float4(y.x > 0.f ? d.x : 0.f, y.y > 0.f ? d.y : 0.f, y.z > 0.f ? d.z : 0.f, y.w > 0.f ? d.w : 0.f);
+}
+
+template <typename T, int RES_THREADS, int K, bool FUSE = false>
 __global__ void __launch_bounds__(RES_THREADS)
 bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, const T* __restrict__ dy,
-                T* __restrict__ dx, BnBwdArgs a) {
+                T* __restrict__ dx, BnBwdArgs a, BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr}) {
   extern __shared__ float4 dyl[];           // [klim][threads], klim <= min(K, RES_KL)
   __shared__ float red[RES_THREADS / 64];
   __shared__ float sh[4];
@@ -445,7 +499,8 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
   res_visit<RES_THREADS, K, ESZ, 0>(g, [&](int k, int off, bool in) { xr[k] = buf_ld4_stream(xr_, off, x); });
   res_visit<RES_THREADS, K, ESZ, 4>(g, [&](int k, int off, bool in) {
     // dy vectors that stay in LDS are read once; the others come back in the second walk
-    const float4 d = k < klim ? buf_ld4_stream(dyr_, off, dy) : buf_ld4(dyr_, off, dy);
+    float4 d = k < klim ? buf_ld4_stream(dyr_, off, dy) : buf_ld4(dyr_, off, dy);
+    if (FUSE) d = relu_mask(d, k < klim ? buf_ld4_stream(make_rsrc(fu.y, bytes), off, dy) : buf_ld4(make_rsrc(fu.y, bytes), off, dy));
     if (k < klim) dyl[k * RES_THREADS + threadIdx.x] = d;
     const float p1 = (d.x + d.y) + (d.z + d.w);
     const float p2 = (d.x * (xr[k].x - mean) + d.y * (xr[k].y - mean)) +
@@ -462,12 +517,160 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
   __syncthreads();
   const float kdy = sh[1], kx = sh[2], k0 = sh[3];
   res_visit<RES_THREADS, K, ESZ, 4, true>(g, [&](int k, int off, bool) {
-    const float4 d = k < klim ? dyl[k * RES_THREADS + threadIdx.x] : buf_ld4(dyr_, off, dy);
+    float4 d = k < klim ? dyl[k * RES_THREADS + threadIdx.x] : buf_ld4(dyr_, off, dy);
+    // the part of dy that did not fit in LDS passes the mask again (y re-read with it)
+    if (FUSE && k >= klim) d = relu_mask(d, buf_ld4(make_rsrc(fu.y, bytes), off, dy));
     const float4 v = make_float4(kdy * d.x + (kx * (xr[k].x - mean) + k0),
                                  kdy * d.y + (kx * (xr[k].y - mean) + k0),
                                  kdy * d.z + (kx * (xr[k].z - mean) + k0),
                                  kdy * d.w + (kx * (xr[k].w - mean) + k0));
     buf_st4(dxr_, off, v, dx);
+    if (FUSE && fu.dres) buf_st4(make_rsrc(fu.dres, bytes), off, d, dx);
+  });
+}
+
+// ---- resident kernels for bf16 storage, eight elements (16 bytes) per slot ----------------
+// The same two kernels with the x values kept packed: a register holds two bf16 values, so a
+// feature of up to 8 * 25 * 1024 elements stays on chip (56x56 planes at batch 64, which the
+// 4-wide kernels above hand to the two-pass path), and every load and store moves 16 bytes
+// per lane.  Values are unpacked (a shift / a mask) each time they are used.
+__device__ __forceinline__ uint4 buf_ld8(__amdgpu_buffer_rsrc_t r, int byte_off, bool stream) {
+  const uintx4_t v = stream ? __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 2)
+                            : __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void buf_st8(__amdgpu_buffer_rsrc_t r, int byte_off, uint4 v) {
+  const uintx4_t t = {v.x, v.y, v.z, v.w};
+  __builtin_amdgcn_raw_buffer_store_b128(t, r, byte_off, 0, 2);
+}
+__device__ __forceinline__ float bf_lo(uint32_t u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+__device__ __forceinline__ uint32_t bf_pack(float lo, float hi) {
+  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+// keeps the halves of d whose counterpart in y is a positive bf16 value
+__device__ __forceinline__ uint32_t relu_mask2(uint32_t d, uint32_t y) {
+  const uint32_t lo = (int)(y << 16) > 0 ? 0x0000ffffu : 0u;
+  const uint32_t hi = (int)(y & 0xffff0000u) > 0 ? 0xffff0000u : 0u;
+  return d & (lo | hi);
+}
+// Makes the packed values opaque to the optimiser: without it the unpacked floats of one
+// walk over the resident vectors are kept alive for the next walk (8 registers per vector)
+// instead of being recomputed from the 4 packed ones.
+__device__ __forceinline__ void opaque(uint4& v) { asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
+__device__ __forceinline__ uint4 relu_mask8(uint4 d, uint4 y) {
+  return make_uint4(relu_mask2(d.x, y.x), relu_mask2(d.y, y.y), relu_mask2(d.z, y.z), relu_mask2(d.w, y.w));
+}
+
+template <int RES_THREADS, int K, bool FUSE = false>
+__global__ void __launch_bounds__(RES_THREADS)
+bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_t* __restrict__ y,
+                   BnTrainArgs a, BnFuseFwd<bf16_t> fu = BnFuseFwd<bf16_t>{nullptr, 0}) {
+  __shared__ float red[RES_THREADS / 64];
+  __shared__ float sh[2];
+  const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
+  const long long c = blockIdx.x;
+  const float shift = ld(x, (size_t)(c * g.inner));
+  uint4 xr[K];
+  float s1 = 0.f, s2 = 0.f;
+  res_visit<RES_THREADS, K, 2, 0, false, 8>(g, [&](int k, int off, bool) { xr[k] = buf_ld8(xr_, off, true); });
+  res_visit<RES_THREADS, K, 2, 1, false, 8>(g, [&](int k, int, bool in) {
+    opaque(xr[k]);
+    const uint32_t w[4] = {xr[k].x, xr[k].y, xr[k].z, xr[k].w};
+    float p1 = 0.f, p2 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float t0 = bf_lo(w[j]) - shift, t1 = bf_hi(w[j]) - shift;
+      p1 += t0 + t1;
+      p2 += t0 * t0 + t1 * t1;
+    }
+    s1 += in ? p1 : 0.f;
+    s2 += in ? p2 : 0.f;
+    asm volatile("" : "+v"(s1), "+v"(s2));
+  });
+  s1 = block_sum(s1, red);
+  s2 = block_sum(s2, red);
+  finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh);
+  __syncthreads();
+  const float mean = sh[0];
+  const float scale = (a.gamma ? a.gamma[c] : 1.f) * sh[1];
+  const float bt = a.beta ? a.beta[c] : 0.f;
+  const __amdgpu_buffer_rsrc_t rr_ = make_rsrc((FUSE && fu.res) ? fu.res : x, (FUSE && fu.res) ? bytes : 0u);
+  const float lo = (FUSE && fu.relu) ? 0.f : -__builtin_huge_valf();
+  res_visit<RES_THREADS, K, 2, 1, false, 8>(g, [&](int k, int off, bool) {
+    // one 32-bit word (two values) at a time, results written over the packed input: the
+    // vector is not needed again
+    uint4 v = xr[k];
+    opaque(v);
+    if (FUSE) {
+      const uint4 rv = buf_ld8(rr_, off, true);      // no residual: the empty range reads zeros
+      v.x = bf_pack(fmaxf((bf_lo(v.x) - mean) * scale + bt + bf_lo(rv.x), lo), fmaxf((bf_hi(v.x) - mean) * scale + bt + bf_hi(rv.x), lo));
+      __builtin_amdgcn_sched_barrier(0);   // one word at a time: the packing temporaries of all four do not fit
+      v.y = bf_pack(fmaxf((bf_lo(v.y) - mean) * scale + bt + bf_lo(rv.y), lo), fmaxf((bf_hi(v.y) - mean) * scale + bt + bf_hi(rv.y), lo));
+      __builtin_amdgcn_sched_barrier(0);   // one word at a time: the packing temporaries of all four do not fit
+      v.z = bf_pack(fmaxf((bf_lo(v.z) - mean) * scale + bt + bf_lo(rv.z), lo), fmaxf((bf_hi(v.z) - mean) * scale + bt + bf_hi(rv.z), lo));
+      __builtin_amdgcn_sched_barrier(0);   // one word at a time: the packing temporaries of all four do not fit
+      v.w = bf_pack(fmaxf((bf_lo(v.w) - mean) * scale + bt + bf_lo(rv.w), lo), fmaxf((bf_hi(v.w) - mean) * scale + bt + bf_hi(rv.w), lo));
+    } else {
+      v.x = bf_pack((bf_lo(v.x) - mean) * scale + bt, (bf_hi(v.x) - mean) * scale + bt);
+      v.y = bf_pack((bf_lo(v.y) - mean) * scale + bt, (bf_hi(v.y) - mean) * scale + bt);
+      v.z = bf_pack((bf_lo(v.z) - mean) * scale + bt, (bf_hi(v.z) - mean) * scale + bt);
+      v.w = bf_pack((bf_lo(v.w) - mean) * scale + bt, (bf_hi(v.w) - mean) * scale + bt);
+    }
+    buf_st8(yr_, off, v);
+  });
+}
+
+template <int RES_THREADS, int K, bool FUSE = false>
+__global__ void __launch_bounds__(RES_THREADS)
+bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy,
+                 bf16_t* __restrict__ dx, BnBwdArgs a, BnFuseBwd<bf16_t> fu = BnFuseBwd<bf16_t>{nullptr, nullptr}) {
+  extern __shared__ uint4 dyl8[];           // [klim][threads] packed gradients (after the mask)
+  __shared__ float red[RES_THREADS / 64];
+  __shared__ float sh[4];
+  const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes),
+                               dxr_ = make_rsrc(dx, bytes);
+  const __amdgpu_buffer_rsrc_t yr_ = make_rsrc(FUSE ? fu.y : x, FUSE ? bytes : 0u);
+  const __amdgpu_buffer_rsrc_t drr_ = make_rsrc((FUSE && fu.dres) ? fu.dres : dx, (FUSE && fu.dres) ? bytes : 0u);
+  const long long c = blockIdx.x;
+  const float mean = a.save_mean[c];
+  uint4 xr[K];
+  float s1 = 0.f, s2 = 0.f;
+  res_visit<RES_THREADS, K, 2, 0, false, 8>(g, [&](int k, int off, bool) { xr[k] = buf_ld8(xr_, off, true); });
+  res_visit<RES_THREADS, K, 2, 4, false, 8>(g, [&](int k, int off, bool in) {
+    uint4 d = buf_ld8(dyr_, off, k < klim);
+    if (FUSE) d = relu_mask8(d, buf_ld8(yr_, off, k < klim));
+    if (k < klim) dyl8[k * RES_THREADS + threadIdx.x] = d;
+    opaque(xr[k]);
+    const uint32_t dw[4] = {d.x, d.y, d.z, d.w}, xw[4] = {xr[k].x, xr[k].y, xr[k].z, xr[k].w};
+    float p1 = 0.f, p2 = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float d0 = bf_lo(dw[j]), d1 = bf_hi(dw[j]);
+      p1 += d0 + d1;
+      p2 += d0 * (bf_lo(xw[j]) - mean) + d1 * (bf_hi(xw[j]) - mean);
+    }
+    s1 += in ? p1 : 0.f;
+    s2 += in ? p2 : 0.f;
+    asm volatile("" : "+v"(s1), "+v"(s2));
+  });
+  s1 = block_sum(s1, red);
+  s2 = block_sum(s2, red);
+  finish_bwd(g, a, c, (double)s1, (double)s2, true, sh);
+  __syncthreads();
+  const float kdy = sh[1], kx = sh[2], k0 = sh[3];
+  res_visit<RES_THREADS, K, 2, 4, true, 8>(g, [&](int k, int off, bool) {
+    uint4 d = k < klim ? dyl8[k * RES_THREADS + threadIdx.x] : buf_ld8(dyr_, off, false);
+    if (FUSE && k >= klim) d = relu_mask8(d, buf_ld8(yr_, off, false));
+    opaque(xr[k]);
+    const uint32_t dw[4] = {d.x, d.y, d.z, d.w}, xw[4] = {xr[k].x, xr[k].y, xr[k].z, xr[k].w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      o[j] = bf_pack(kdy * bf_lo(dw[j]) + (kx * (bf_lo(xw[j]) - mean) + k0),
+                     kdy * bf_hi(dw[j]) + (kx * (bf_hi(xw[j]) - mean) + k0));
+    buf_st8(dxr_, off, make_uint4(o[0], o[1], o[2], o[3]));
+    if (FUSE) buf_st8(drr_, off, d);               // no residual branch: the empty range drops the store
   });
 }
 
@@ -504,10 +707,10 @@ __device__ __forceinline__ void res1_offsets(const BnGeom& g, int (&off)[K]) {
   }
 }
 
-template <typename T, int THREADS, int K>
+template <typename T, int THREADS, int K, bool FUSE = false>
 __global__ void __launch_bounds__(THREADS)
 bn_train_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restrict__ y,
-                   BnTrainArgs a) {
+                   BnTrainArgs a, BnFuseFwd<T> fu = BnFuseFwd<T>{nullptr, 0}) {
   __shared__ float red[THREADS / 64];
   __shared__ float sh[2];
   constexpr int OOB = (int)0x80000000;
@@ -533,14 +736,24 @@ bn_train_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restr
   const float mean = sh[0];
   const float scale = (a.gamma ? a.gamma[c] : 1.f) * sh[1];
   const float bt = a.beta ? a.beta[c] : 0.f;
+  if (FUSE) {
+    const __amdgpu_buffer_rsrc_t rr_ = make_rsrc(fu.res ? fu.res : x, fu.res ? bytes : 0u);   // no residual: loads give 0
+    const float lo = fu.relu ? 0.f : -__builtin_huge_valf();
+    float rv[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) rv[k] = buf_ld(rr_, off[k], x);
+#pragma unroll
+    for (int k = 0; k < K; ++k) buf_st(yr_, off[k], fmaxf((xv[k] - mean) * scale + bt + rv[k], lo), y);
+    return;
+  }
 #pragma unroll
   for (int k = 0; k < K; ++k) buf_st(yr_, off[k], (xv[k] - mean) * scale + bt, y);
 }
 
-template <typename T, int THREADS, int K>
+template <typename T, int THREADS, int K, bool FUSE = false>
 __global__ void __launch_bounds__(THREADS)
 bn_bwd_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, const T* __restrict__ dy,
-                 T* __restrict__ dx, BnBwdArgs a) {
+                 T* __restrict__ dx, BnBwdArgs a, BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr}) {
   __shared__ float red[THREADS / 64];
   __shared__ float sh[4];
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes),
@@ -554,6 +767,11 @@ bn_bwd_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, const T* __r
   for (int k = 0; k < K; ++k) {
     xv[k] = buf_ld(xr_, off[k], x);
     dv[k] = buf_ld(dyr_, off[k], dy);
+  }
+  if (FUSE) {
+    const __amdgpu_buffer_rsrc_t yr_ = make_rsrc(fu.y, bytes);
+#pragma unroll
+    for (int k = 0; k < K; ++k) dv[k] = buf_ld(yr_, off[k], dy) > 0.f ? dv[k] : 0.f;
   }
   float s1 = 0.f, s2 = 0.f;
 #pragma unroll
@@ -569,6 +787,11 @@ bn_bwd_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, const T* __r
   const float kdy = sh[1], kx = sh[2], k0 = sh[3];
 #pragma unroll
   for (int k = 0; k < K; ++k) buf_st(dxr_, off[k], kdy * dv[k] + (kx * (xv[k] - mean) + k0), dx);
+  if (FUSE && fu.dres) {
+    const __amdgpu_buffer_rsrc_t rr_ = make_rsrc(fu.dres, bytes);
+#pragma unroll
+    for (int k = 0; k < K; ++k) buf_st(rr_, off[k], dv[k], dx);
+  }
 }
 
 // ---- column mode (inner == 1) ----------------------------------------------
@@ -772,21 +995,86 @@ static ResPlan resident_plan(const BnGeom& g, int vec, int min_c) {
   return r;
 }
 
-template <typename T, int THREADS, int K>
+// bf16 storage, rows of a multiple of 8 elements: shape of the 8-wide resident kernels
+// (threads = 0: they do not apply)
+static ResPlan resident8_plan(const BnGeom& g, int vec, int dtype, int min_c) {
+  ResPlan r{0, 0, 0};
+  const int mode = options().bn_algo;
+  if (mode == 1 || vec != 4 || dtype != FLHIP_BF16 || g.inner % 8 != 0) return r;
+  const long long units8 = g.units / 2;
+  if (units8 > (long long)RES_KMAX * 1024) return r;
+  if (g.outer * g.C * g.inner * 2 >= (1ll << 31)) return r;   // 32-bit buffer offsets
+  if (mode != 2 && g.C < min_c) return r;
+  if (units8 <= 8 * 256) {
+    r.threads = 256;
+    r.k = 8;
+  } else {
+    r.threads = 1024;
+    const int need = (int)((units8 + 1023) / 1024);
+    r.k = need <= 8 ? 8 : need <= 16 ? 16 : RES_KMAX;
+  }
+  r.need = (int)((units8 + r.threads - 1) / r.threads);
+  return r;
+}
+
+template <int THREADS, int K, bool FUSE>
+static int launch_train_resident8(const BnGeom& g, const bf16_t* x, bf16_t* y, const BnTrainArgs& a,
+                                  const BnFuseFwd<bf16_t>& fu, hipStream_t s) {
+  const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * 2);
+  hipLaunchKernelGGL((bn_train_resident8<THREADS, K, FUSE>), dim3((unsigned)g.C), dim3(THREADS), 0, s, g, bytes, x, y,
+                     a, fu);
+  return check_launch("bn_fwd_train (resident, 8-wide)");
+}
+
+template <int THREADS, int K, bool FUSE>
+static int launch_bwd_resident8(const BnGeom& g, int need, const bf16_t* x, const bf16_t* dy, bf16_t* dx,
+                                const BnBwdArgs& a, const BnFuseBwd<bf16_t>& fu, hipStream_t s) {
+  constexpr int KL = K < RES_KL ? K : RES_KL;
+  constexpr size_t max_shmem = (size_t)KL * THREADS * sizeof(uint4);
+  auto kernel = bn_bwd_resident8<THREADS, K, FUSE>;
+  static const hipError_t attr = hipFuncSetAttribute(
+      reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)max_shmem);
+  if (attr != hipSuccess)
+    return fail(FLHIP_RUNTIME_ERROR, std::string("bn_bwd: LDS limit: ") + hipGetErrorString(attr));
+  const int klim = need < KL ? need : KL;
+  const size_t shmem = (size_t)klim * THREADS * sizeof(uint4);
+  const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * 2);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)g.C), dim3(THREADS), shmem, s, g, bytes, klim, x, dy, dx, a, fu);
+  return check_launch("bn_bwd (resident, 8-wide)");
+}
+
+template <bool FUSE>
+static int run_train8(const BnGeom& g, const ResPlan& r, const bf16_t* x, bf16_t* y, const BnTrainArgs& a,
+                      const BnFuseFwd<bf16_t>& fu, hipStream_t s) {
+  if (r.threads == 256) return launch_train_resident8<256, 8, FUSE>(g, x, y, a, fu, s);
+  if (r.k == 8) return launch_train_resident8<1024, 8, FUSE>(g, x, y, a, fu, s);
+  if (r.k == 16) return launch_train_resident8<1024, 16, FUSE>(g, x, y, a, fu, s);
+  return launch_train_resident8<1024, RES_KMAX, FUSE>(g, x, y, a, fu, s);
+}
+template <bool FUSE>
+static int run_bwd8(const BnGeom& g, const ResPlan& r, const bf16_t* x, const bf16_t* dy, bf16_t* dx,
+                    const BnBwdArgs& a, const BnFuseBwd<bf16_t>& fu, hipStream_t s) {
+  if (r.threads == 256) return launch_bwd_resident8<256, 8, FUSE>(g, r.need, x, dy, dx, a, fu, s);
+  if (r.k == 8) return launch_bwd_resident8<1024, 8, FUSE>(g, r.need, x, dy, dx, a, fu, s);
+  if (r.k == 16) return launch_bwd_resident8<1024, 16, FUSE>(g, r.need, x, dy, dx, a, fu, s);
+  return launch_bwd_resident8<1024, RES_KMAX, FUSE>(g, r.need, x, dy, dx, a, fu, s);
+}
+
+template <typename T, int THREADS, int K, bool FUSE>
 static int launch_train_resident(const BnGeom& g, const T* x, T* y, const BnTrainArgs& a,
-                                 hipStream_t s) {
+                                 const BnFuseFwd<T>& fu, hipStream_t s) {
   const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
-  hipLaunchKernelGGL((bn_train_resident<T, THREADS, K>), dim3((unsigned)g.C), dim3(THREADS), 0, s,
-                     g, bytes, x, y, a);
+  hipLaunchKernelGGL((bn_train_resident<T, THREADS, K, FUSE>), dim3((unsigned)g.C), dim3(THREADS), 0, s,
+                     g, bytes, x, y, a, fu);
   return check_launch("bn_fwd_train (resident)");
 }
 
-template <typename T, int THREADS, int K>
+template <typename T, int THREADS, int K, bool FUSE>
 static int launch_bwd_resident(const BnGeom& g, int need, const T* x, const T* dy, T* dx,
-                               const BnBwdArgs& a, hipStream_t s) {
+                               const BnBwdArgs& a, const BnFuseBwd<T>& fu, hipStream_t s) {
   constexpr int KL = K < RES_KL ? K : RES_KL;
   constexpr size_t max_shmem = (size_t)KL * THREADS * sizeof(float4);
-  auto kernel = bn_bwd_resident<T, THREADS, K>;
+  auto kernel = bn_bwd_resident<T, THREADS, K, FUSE>;
   static const hipError_t attr = hipFuncSetAttribute(
       reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
       (int)max_shmem);
@@ -797,38 +1085,46 @@ static int launch_bwd_resident(const BnGeom& g, int need, const T* x, const T* d
   const size_t shmem = (size_t)klim * THREADS * sizeof(float4);
   const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
   hipLaunchKernelGGL(kernel, dim3((unsigned)g.C), dim3(THREADS), shmem, s, g, bytes, klim, x, dy,
-                     dx, a);
+                     dx, a, fu);
   return check_launch("bn_bwd (resident)");
 }
 
-template <typename T>
+// FUSE: with the epilogue y = relu(bn(x) + residual) (segment modes only)
+template <typename T, bool FUSE>
 static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws,
-                     const BnTrainArgs& a, hipStream_t s) {
+                     const BnTrainArgs& a, const BnFuseFwd<T>& fu, hipStream_t s) {
   const T* xp = static_cast<const T*>(x);
   T* yp = static_cast<T*>(y);
+  if (sizeof(T) == 2) {
+    const ResPlan r8 = resident8_plan(g, vec, FLHIP_BF16, RES_MIN_C_FWD);
+    if (r8.threads)
+      return run_train8<FUSE>(g, r8, reinterpret_cast<const bf16_t*>(xp), reinterpret_cast<bf16_t*>(yp), a,
+                              reinterpret_cast<const BnFuseFwd<bf16_t>&>(fu), s);
+  }
   {
     const ResPlan r = resident_plan(g, vec, RES_MIN_C_FWD);
     if (vec == 1 && r.threads) {
       const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
       const dim3 grid((unsigned)g.C);
       if (r.threads == 256)
-        hipLaunchKernelGGL((bn_train_resident1<T, 256, 8>), grid, dim3(256), 0, s, g, bytes, xp, yp, a);
+        hipLaunchKernelGGL((bn_train_resident1<T, 256, 8, FUSE>), grid, dim3(256), 0, s, g, bytes, xp, yp, a, fu);
       else if (r.k == 8)
-        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 8>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a);
+        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 8, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a, fu);
       else if (r.k == 16)
-        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 16>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a);
+        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 16, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a, fu);
       else
-        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 32>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a);
+        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 32, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a, fu);
       return check_launch("bn_fwd_train (resident, element-wise)");
     }
-    if (r.threads == 256) return launch_train_resident<T, 256, 8>(g, xp, yp, a, s);
+    if (r.threads == 256) return launch_train_resident<T, 256, 8, FUSE>(g, xp, yp, a, fu, s);
     if (r.threads == 1024) {
-      if (r.k == 8) return launch_train_resident<T, 1024, 8>(g, xp, yp, a, s);
-      if (r.k == 16) return launch_train_resident<T, 1024, 16>(g, xp, yp, a, s);
-      return launch_train_resident<T, 1024, RES_KMAX>(g, xp, yp, a, s);
+      if (r.k == 8) return launch_train_resident<T, 1024, 8, FUSE>(g, xp, yp, a, fu, s);
+      if (r.k == 16) return launch_train_resident<T, 1024, 16, FUSE>(g, xp, yp, a, fu, s);
+      return launch_train_resident<T, 1024, RES_KMAX, FUSE>(g, xp, yp, a, fu, s);
     }
   }
   if (vec == 0) {
+    if (FUSE) return fail(FLHIP_INVALID_ARGUMENT, "bn_act: per-activation mode (inner == 1) has no fused kernels");
     const dim3 grid((unsigned)((g.C + 63) / 64), g.S);
     hipLaunchKernelGGL((bn_stats_col<T, false>), grid, dim3(256), 0, s, g, xp, (const T*)nullptr,
                        (const float*)nullptr, ws);
@@ -837,55 +1133,63 @@ static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws
     const dim3 grid((unsigned)g.C, g.S);
     if (vec == 4) {
       hipLaunchKernelGGL((bn_stats_seg<T, 4>), grid, dim3(256), 0, s, g, xp, ws);
-      hipLaunchKernelGGL((bn_train_apply_seg<T, 4>), grid, dim3(256), 0, s, g, xp, yp, ws, a);
+      hipLaunchKernelGGL((bn_train_apply_seg<T, 4, FUSE>), grid, dim3(256), 0, s, g, xp, yp, ws, a, fu);
     } else {
       hipLaunchKernelGGL((bn_stats_seg<T, 1>), grid, dim3(256), 0, s, g, xp, ws);
-      hipLaunchKernelGGL((bn_train_apply_seg<T, 1>), grid, dim3(256), 0, s, g, xp, yp, ws, a);
+      hipLaunchKernelGGL((bn_train_apply_seg<T, 1, FUSE>), grid, dim3(256), 0, s, g, xp, yp, ws, a, fu);
     }
   }
   return check_launch("bn_fwd_train");
 }
 
-template <typename T>
+// FUSE: the gradient first passes the ReLU mask of the forward result
+template <typename T, bool FUSE>
 static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void* dx, float* ws,
-                   const BnBwdArgs& a, hipStream_t s) {
+                   const BnBwdArgs& a, const BnFuseBwd<T>& fu, hipStream_t s) {
   const T* xp = static_cast<const T*>(x);
   const T* dyp = static_cast<const T*>(dy);
   T* dxp = static_cast<T*>(dx);
+  if (sizeof(T) == 2) {
+    const ResPlan r8 = resident8_plan(g, vec, FLHIP_BF16, RES_MIN_C_BWD);
+    if (r8.threads)
+      return run_bwd8<FUSE>(g, r8, reinterpret_cast<const bf16_t*>(xp), reinterpret_cast<const bf16_t*>(dyp),
+                            reinterpret_cast<bf16_t*>(dxp), a, reinterpret_cast<const BnFuseBwd<bf16_t>&>(fu), s);
+  }
   {
     const ResPlan r = resident_plan(g, vec, RES_MIN_C_BWD);
     if (vec == 1 && r.threads) {
       const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
       const dim3 grid((unsigned)g.C);
       if (r.threads == 256)
-        hipLaunchKernelGGL((bn_bwd_resident1<T, 256, 8>), grid, dim3(256), 0, s, g, bytes, xp, dyp, dxp, a);
+        hipLaunchKernelGGL((bn_bwd_resident1<T, 256, 8, FUSE>), grid, dim3(256), 0, s, g, bytes, xp, dyp, dxp, a, fu);
       else if (r.k == 8)
-        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 8>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a);
+        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 8, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a, fu);
       else if (r.k == 16)
-        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 16>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a);
+        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 16, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a, fu);
       else
-        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 32>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a);
+        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 32, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a, fu);
       return check_launch("bn_bwd (resident, element-wise)");
     }
-    if (r.threads == 256) return launch_bwd_resident<T, 256, 8>(g, r.need, xp, dyp, dxp, a, s);
+    if (r.threads == 256) return launch_bwd_resident<T, 256, 8, FUSE>(g, r.need, xp, dyp, dxp, a, fu, s);
     if (r.threads == 1024) {
-      if (r.k == 8) return launch_bwd_resident<T, 1024, 8>(g, r.need, xp, dyp, dxp, a, s);
-      if (r.k == 16) return launch_bwd_resident<T, 1024, 16>(g, r.need, xp, dyp, dxp, a, s);
-      return launch_bwd_resident<T, 1024, RES_KMAX>(g, r.need, xp, dyp, dxp, a, s);
+      if (r.k == 8) return launch_bwd_resident<T, 1024, 8, FUSE>(g, r.need, xp, dyp, dxp, a, fu, s);
+      if (r.k == 16) return launch_bwd_resident<T, 1024, 16, FUSE>(g, r.need, xp, dyp, dxp, a, fu, s);
+      return launch_bwd_resident<T, 1024, RES_KMAX, FUSE>(g, r.need, xp, dyp, dxp, a, fu, s);
     }
   }
   if (vec == 0) {
+    if (FUSE) return fail(FLHIP_INVALID_ARGUMENT, "bn_act: per-activation mode (inner == 1) has no fused kernels");
     const dim3 grid((unsigned)((g.C + 63) / 64), g.S);
     hipLaunchKernelGGL((bn_stats_col<T, true>), grid, dim3(256), 0, s, g, xp, dyp, a.save_mean, ws);
     hipLaunchKernelGGL((bn_bwd_apply_col<T>), grid, dim3(256), 0, s, g, xp, dyp, dxp, ws, a);
   } else {
     const dim3 grid((unsigned)g.C, g.S);
     if (vec == 4) {
-      hipLaunchKernelGGL((bn_bwd_stats_seg<T, 4>), grid, dim3(256), 0, s, g, xp, dyp, a.save_mean, ws);
-      hipLaunchKernelGGL((bn_bwd_apply_seg<T, 4>), grid, dim3(256), 0, s, g, xp, dyp, dxp, ws, a);
+      hipLaunchKernelGGL((bn_bwd_stats_seg<T, 4, FUSE>), grid, dim3(256), 0, s, g, xp, dyp, a.save_mean, ws, fu);
+      hipLaunchKernelGGL((bn_bwd_apply_seg<T, 4, FUSE>), grid, dim3(256), 0, s, g, xp, dyp, dxp, ws, a, fu);
     } else {
-      hipLaunchKernelGGL((bn_bwd_stats_seg<T, 1>), grid, dim3(256), 0, s, g, xp, dyp, a.save_mean, ws);
-      hipLaunchKernelGGL((bn_bwd_apply_seg<T, 1>), grid, dim3(256), 0, s, g, xp, dyp, dxp, ws, a);
+      hipLaunchKernelGGL((bn_bwd_stats_seg<T, 1, FUSE>), grid, dim3(256), 0, s, g, xp, dyp, a.save_mean, ws, fu);
+      hipLaunchKernelGGL((bn_bwd_apply_seg<T, 1, FUSE>), grid, dim3(256), 0, s, g, xp, dyp, dxp, ws, a, fu);
     }
   }
   return check_launch("bn_bwd");
@@ -919,8 +1223,31 @@ extern "C" int flhip_bn_fwd_train(const flhip_bn_desc* d, const void* x, const f
   FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_fwd_train: workspace too small");
   const BnTrainArgs a{gamma, beta, save_mean, save_invstd, run_mean, run_var, momentum, eps};
   return d->dtype == FLHIP_F32
-             ? run_train<float>(g, vec, x, y, static_cast<float*>(ws), a, as_stream(stream))
-             : run_train<bf16_t>(g, vec, x, y, static_cast<float*>(ws), a, as_stream(stream));
+             ? run_train<float, false>(g, vec, x, y, static_cast<float*>(ws), a, BnFuseFwd<float>{nullptr, 0}, as_stream(stream))
+             : run_train<bf16_t, false>(g, vec, x, y, static_cast<float*>(ws), a, BnFuseFwd<bf16_t>{nullptr, 0}, as_stream(stream));
+}
+
+extern "C" int flhip_bn_act_fwd_train(const flhip_bn_desc* d, const void* x, const float* gamma,
+                                      const float* beta, const void* residual, int relu, void* y,
+                                      float* save_mean, float* save_invstd, float* run_mean,
+                                      float* run_var, double momentum, double eps, void* ws,
+                                      size_t ws_bytes, void* stream) {
+  BnGeom g;
+  int vec;
+  const int rc = make_geom(d, &g, &vec);
+  if (rc != FLHIP_OK) return rc;
+  FLHIP_REQUIRE(x && y, "bn_act_fwd_train: null tensor");
+  FLHIP_REQUIRE((run_mean == nullptr) == (run_var == nullptr),
+                "bn_act_fwd_train: running mean and variance must be given together");
+  FLHIP_REQUIRE(momentum >= 0.0 && momentum <= 1.0, "bn_act_fwd_train: momentum must lie in [0, 1]");
+  FLHIP_REQUIRE(eps >= 0.0, "bn_act_fwd_train: epsilon must be non-negative");
+  FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_act_fwd_train: workspace too small");
+  const BnTrainArgs a{gamma, beta, save_mean, save_invstd, run_mean, run_var, momentum, eps};
+  return d->dtype == FLHIP_F32
+             ? run_train<float, true>(g, vec, x, y, static_cast<float*>(ws), a,
+                                      BnFuseFwd<float>{static_cast<const float*>(residual), relu}, as_stream(stream))
+             : run_train<bf16_t, true>(g, vec, x, y, static_cast<float*>(ws), a,
+                                       BnFuseFwd<bf16_t>{static_cast<const bf16_t*>(residual), relu}, as_stream(stream));
 }
 
 extern "C" int flhip_bn_fwd_infer(const flhip_bn_desc* d, const void* x, const float* gamma,
@@ -960,6 +1287,27 @@ extern "C" int flhip_bn_bwd(const flhip_bn_desc* d, const void* x, const void* d
   FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_bwd: workspace too small");
   const BnBwdArgs a{gamma, save_mean, save_invstd, dgamma, dbeta};
   return d->dtype == FLHIP_F32
-             ? run_bwd<float>(g, vec, x, dy, dx, static_cast<float*>(ws), a, as_stream(stream))
-             : run_bwd<bf16_t>(g, vec, x, dy, dx, static_cast<float*>(ws), a, as_stream(stream));
+             ? run_bwd<float, false>(g, vec, x, dy, dx, static_cast<float*>(ws), a, BnFuseBwd<float>{nullptr, nullptr}, as_stream(stream))
+             : run_bwd<bf16_t, false>(g, vec, x, dy, dx, static_cast<float*>(ws), a, BnFuseBwd<bf16_t>{nullptr, nullptr}, as_stream(stream));
+}
+
+extern "C" int flhip_bn_act_bwd(const flhip_bn_desc* d, const void* x, const void* dy, const void* y,
+                                const float* gamma, const float* save_mean, const float* save_invstd,
+                                void* dx, void* dresidual, float* dgamma, float* dbeta, void* ws,
+                                size_t ws_bytes, void* stream) {
+  BnGeom g;
+  int vec;
+  const int rc = make_geom(d, &g, &vec);
+  if (rc != FLHIP_OK) return rc;
+  FLHIP_REQUIRE(x && dy && dx && y, "bn_act_bwd: null tensor");
+  FLHIP_REQUIRE(save_mean && save_invstd, "bn_act_bwd: needs the saved statistics of the forward pass");
+  FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_act_bwd: workspace too small");
+  const BnBwdArgs a{gamma, save_mean, save_invstd, dgamma, dbeta};
+  return d->dtype == FLHIP_F32
+             ? run_bwd<float, true>(g, vec, x, dy, dx, static_cast<float*>(ws), a,
+                                    BnFuseBwd<float>{static_cast<const float*>(y), static_cast<float*>(dresidual)},
+                                    as_stream(stream))
+             : run_bwd<bf16_t, true>(g, vec, x, dy, dx, static_cast<float*>(ws), a,
+                                     BnFuseBwd<bf16_t>{static_cast<const bf16_t*>(y), static_cast<bf16_t*>(dresidual)},
+                                     as_stream(stream));
 }

@@ -34,12 +34,11 @@ typedef uint16_t bf16_t;  // raw bits
 __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
   return __uint_as_float(((uint32_t)v) << 16);
 }
-// round to nearest even; NaN stays NaN
+// round to nearest even; NaN stays NaN.  gfx950 converts in hardware (v_cvt_pk_bf16_f32, two
+// values per instruction when neighbours are converted together); the host pass of the
+// compiler only parses this.
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+  return __builtin_bit_cast(unsigned short, static_cast<__bf16>(f));
 }
 
 __device__ __forceinline__ float ld(const float* p, size_t i) { return p[i]; }

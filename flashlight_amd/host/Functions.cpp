@@ -1,4 +1,5 @@
 #include "Functions.h"
+#include "HipAutogradExtension.h"
 #include "OpObserver.h"
 
 #include <algorithm>
@@ -70,7 +71,18 @@ Variable Variable::astype(dtype newType) const {
   auto gradFunc = [oldType](std::vector<Variable>& inputs, const Variable& gradOutput) {
     inputs[0].addGrad(Variable(gradOutput.tensor().astype(oldType), false));
   };
-  return Variable(tensor().astype(newType), {*this}, gradFunc);
+  Variable out(tensor().astype(newType), {*this}, gradFunc);
+  out.grad_->isCast = out.grad_->calcGrad;
+  return out;
+}
+
+void Variable::addGradWide(const Tensor& grad) {
+  if (!grad_->calcGrad) return;
+  if (grad_->isCast && !grad_->inputs.empty() && grad.type() != type() && grad_->inputs[0].type() == grad.type()) {
+    grad_->inputs[0].addGrad(Variable(grad, false));
+    return;
+  }
+  addGrad(Variable(grad.astype(type()), false));
 }
 
 std::vector<Variable> Variable::build() const {
@@ -157,8 +169,8 @@ Variable conv2d(const Variable& input, const Variable& weights, const Variable& 
       const Tensor bs = biasGrad ? inputs[2].tensor() : Tensor();
       auto grads = e.conv2dBackwardFilterBias(gradOutput.tensor(), in.tensor(), wt.tensor(), bs, sx,
                                               sy, px, py, dx, dy, groups, nullptr, nullptr, payload);
-      if (wt.isCalcGrad()) wt.addGrad(Variable(grads.first.astype(wt.type()), false));
-      if (biasGrad) inputs[2].addGrad(Variable(grads.second.astype(inputs[2].type()), false));
+      if (wt.isCalcGrad()) wt.addGradWide(grads.first);
+      if (biasGrad) inputs[2].addGradWide(grads.second);
     }
   };
   if (hasBias) return Variable(output, {input, weights, bias}, gradFunc);
@@ -208,6 +220,45 @@ Variable batchnorm(const Variable& input, const Variable& weight, const Variable
     if (!wt.isEmpty()) wt.addGrad(Variable(std::get<1>(g).reshaped(wt.shape()).astype(wt.type()), false));
     if (!bs.isEmpty()) bs.addGrad(Variable(std::get<2>(g).reshaped(bs.shape()).astype(bs.type()), false));
   };
+  return Variable(output, {input, weight, bias}, gradFunc);
+}
+
+Variable detail::batchnormRelu(const Variable& input, const Variable& weight, const Variable& bias,
+                               Variable& runningMean, Variable& runningVar, const std::vector<int>& axes,
+                               double momentum, double epsilon, const Variable& residual) {
+  auto* hip = dynamic_cast<HipAutogradExtension*>(&ext(input));
+  const bool perActivation = !axes.empty() && *std::min_element(axes.begin(), axes.end()) == 0;
+  if (!hip || perActivation) {
+    Variable y = batchnorm(input, weight, bias, runningMean, runningVar, axes, true, momentum, epsilon);
+    return relu(residual.isEmpty() ? y : y + residual);
+  }
+  for (const Variable* v : {&weight, &bias})
+    if (!v->isEmpty() && v->type() != input.type() && v->type() != dtype::f32)
+      throw std::invalid_argument("batchnormRelu: parameters must have the input's type or f32");
+  const bool hasResidual = !residual.isEmpty();
+  if (hasResidual) dtypesMatch("batchnormRelu", {&input, &residual});
+  auto payload = createPayload({&input, &weight, &bias, &residual});
+  auto saveMean = std::make_shared<Tensor>();
+  auto saveVar = std::make_shared<Tensor>();
+  Tensor output = hip->batchnormRelu(*saveMean, *saveVar, input.tensor(), weight.tensor(), bias.tensor(),
+                                     runningMean.tensor(), runningVar.tensor(), axes, momentum, epsilon,
+                                     residual.tensor(), payload);
+  auto gradFunc = [saveMean, saveVar, axes, output, hasResidual, payload](std::vector<Variable>& inputs,
+                                                                          const Variable& gradOutput) {
+    auto& in = inputs[0];
+    auto& wt = inputs[1];
+    auto& bs = inputs[2];
+    const bool resGrad = hasResidual && inputs[3].isCalcGrad();
+    if (!in.isCalcGrad() && !wt.isCalcGrad() && !bs.isCalcGrad() && !resGrad) return;
+    auto* h = dynamic_cast<HipAutogradExtension*>(&ext(in));
+    auto g = h->batchnormReluBackward(gradOutput.tensor(), output, *saveMean, *saveVar, in.tensor(), wt.tensor(),
+                                      axes, resGrad, payload);
+    in.addGrad(Variable(std::get<0>(g).astype(in.type()), false));
+    if (!wt.isEmpty()) wt.addGrad(Variable(std::get<1>(g).reshaped(wt.shape()).astype(wt.type()), false));
+    if (!bs.isEmpty()) bs.addGrad(Variable(std::get<2>(g).reshaped(bs.shape()).astype(bs.type()), false));
+    if (resGrad) inputs[3].addGrad(Variable(std::get<3>(g), false));
+  };
+  if (hasResidual) return Variable(output, {input, weight, bias, residual}, gradFunc);
   return Variable(output, {input, weight, bias}, gradFunc);
 }
 

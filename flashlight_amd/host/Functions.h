@@ -40,12 +40,21 @@ class Variable {
   bool isGradAvailable() const { return grad_->grad != nullptr; }
   Variable& grad() const;
   void addGrad(const Variable& childGrad);
+  // Adds a gradient that an operation produced in a wider type than this Variable (the fp32
+  // filter / bias gradients of a convolution over bf16 storage).  When this Variable is a cast
+  // of one that has the gradient's type (astype of an fp32 master parameter), the gradient
+  // goes to that one as it is: the reference's path, astype to this type here and back in the
+  // cast's own gradient function (Functions.cpp:1391-1410, Variable.cpp:100-108), rounds it to
+  // the narrow type for nothing and costs two conversion kernels per parameter.  Otherwise
+  // the same as addGrad(astype).
+  void addGradWide(const Tensor& grad);
   void zeroGrad() { grad_->grad.reset(); }
   void backward(const Variable& grad, bool retainGraph = false);
 
  private:
   struct SharedGrad {
     bool calcGrad = false;
+    bool isCast = false;   // result of astype(): inputs[0] is the source
     std::vector<Variable> inputs;
     std::unique_ptr<Variable> grad;
     GradFunc gradFunc;
@@ -82,6 +91,14 @@ enum class ReduceMode { NONE = 0, MEAN = 1, SUM = 2 };
 Variable add(const Variable& lhs, const Variable& rhs);
 inline Variable operator+(const Variable& lhs, const Variable& rhs) { return add(lhs, rhs); }
 namespace detail {
+// relu(batchnorm(input, ...) + residual) in train mode, residual optional (an empty Variable):
+// the tail of a ResNet block (flashlight/pkg/vision/models/Resnet.cpp:95-140).  On the HIP
+// extension with feature axes that do not start at dimension 0 this is one fused pass forward
+// and one backward; otherwise the three reference functions are composed.  Same gradients
+// either way.
+Variable batchnormRelu(const Variable& input, const Variable& weight, const Variable& bias,
+                       Variable& runningMean, Variable& runningVar, const std::vector<int>& axes,
+                       double momentum, double epsilon, const Variable& residual);
 // tileAs(weight, input) * input + tileAs(bias, input) on the [outer][mid][inner] view of
 // the input, one parameter element per mid index or a single one (scalar): the affine
 // part of LayerNorm (flashlight/fl/nn/modules/LayerNorm.cpp:110-128)

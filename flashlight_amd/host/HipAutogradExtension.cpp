@@ -379,6 +379,92 @@ std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::batchnormBackward(
   return std::make_tuple(gradInput, gradWeight, gradBias);   // always all three (:278)
 }
 
+// ---- batch norm fused with the residual add and the ReLU ----------------------------------------
+Tensor HipAutogradExtension::batchnormRelu(Tensor& saveMean, Tensor& saveVar, const Tensor& input,
+                                           const Tensor& weight, const Tensor& bias, Tensor& runningMean,
+                                           Tensor& runningVar, const std::vector<int>& axes,
+                                           const double momentum, const double epsilon, const Tensor& residual,
+                                           std::shared_ptr<detail::AutogradPayload> autogradPayload) {
+  detail::OpScope scope("batchnormRelu");
+  const int tag = dtypeTag(input.type(), "batchnormRelu");
+  flhip_bn_desc d = bnDesc(input, axes, tag);
+  const Dim nfeat = (Dim)d.C;
+  for (const Tensor* t : {&weight, &bias, static_cast<const Tensor*>(&runningMean),
+                          static_cast<const Tensor*>(&runningVar)})
+    if (!t->isEmpty() && t->elements() != nfeat)
+      throw std::invalid_argument("batchnormRelu: parameters must have one element per feature");
+  if (!residual.isEmpty() && (residual.type() != input.type() || residual.shape() != input.shape()))
+    throw std::invalid_argument("batchnormRelu: the residual must match the input");
+  if (runningVar.isEmpty()) runningVar = Tensor::full({nfeat}, 1., dtype::f32);
+  if (runningMean.isEmpty()) runningMean = Tensor::full({nfeat}, 0., dtype::f32);
+  if (runningMean.type() != dtype::f32 || runningVar.type() != dtype::f32)
+    throw std::invalid_argument("batchnormRelu: running statistics must be f32");
+  const Tensor gamma = asF32(weight), beta = asF32(bias);
+  Tensor output(input.shape(), input.type());
+  saveMean = Tensor({nfeat}, dtype::f32);
+  saveVar = Tensor({nfeat}, dtype::f32);
+  const size_t wsBytes = flhip_bn_workspace_bytes(&d);
+  Tensor ws = workspace(wsBytes);
+  DevicePtr xp(input), gp(gamma), bp(beta), rp(residual), yp(output), rmp(runningMean), rvp(runningVar),
+      smp(saveMean), sip(saveVar), wsp(ws);
+  check(flhip_bn_act_fwd_train(&d, xp.get(), static_cast<const float*>(gp.get()),
+                               static_cast<const float*>(bp.get()), rp.get(), 1, yp.get(),
+                               static_cast<float*>(smp.get()), static_cast<float*>(sip.get()),
+                               static_cast<float*>(rmp.get()), static_cast<float*>(rvp.get()), momentum, epsilon,
+                               wsp.get(), wsBytes, hipBackendStream()));
+  if (autogradPayload) {
+    auto payload = std::make_shared<HipBatchNormPayload>();
+    payload->saveMean = saveMean;
+    payload->saveInvStd = saveVar;
+    autogradPayload->data = payload;
+  }
+  // event: inputs {input, gamma, beta, runningMean, runningVar, residual (may be empty)}, outputs {output, saveMean,
+  // saveInvStd}, ints {outer, features, inner, train = 1}, reals {momentum, epsilon}
+  if (scope.on())
+    scope.done({input, gamma, beta, runningMean, runningVar, residual}, {output, saveMean, saveVar},
+               {d.outer, d.C, d.inner, 1}, {momentum, epsilon});
+  return output;
+}
+
+std::tuple<Tensor, Tensor, Tensor, Tensor> HipAutogradExtension::batchnormReluBackward(
+    const Tensor& gradOutput, const Tensor& output, const Tensor& saveMean, const Tensor& saveVar,
+    const Tensor& input, const Tensor& weight, const std::vector<int>& axes, const bool wantResidualGrad,
+    std::shared_ptr<detail::AutogradPayload> autogradPayload) {
+  detail::OpScope scope("batchnormReluBackward");
+  Tensor mean = saveMean, invstd = saveVar;
+  if (autogradPayload && autogradPayload->data) {
+    auto payload = std::dynamic_pointer_cast<HipBatchNormPayload>(autogradPayload->data);
+    if (!payload) throw std::invalid_argument("batchnormReluBackward: payload of another operation");
+    mean = payload->saveMean;
+    invstd = payload->saveInvStd;
+  }
+  if (mean.isEmpty() || invstd.isEmpty())
+    throw std::invalid_argument("HipAutogradExtension::batchnormReluBackward given null or empty payload");
+  if (gradOutput.type() != input.type() || gradOutput.shape() != input.shape() ||
+      output.type() != input.type() || output.shape() != input.shape())
+    throw std::invalid_argument("batchnormReluBackward: gradOutput and output must match the input");
+  flhip_bn_desc d = bnDesc(input, axes, dtypeTag(input.type(), "batchnormReluBackward"));
+  const Dim nfeat = (Dim)d.C;
+  const Tensor gamma = asF32(weight);
+  Tensor gradInput(input.shape(), input.type());
+  Tensor gradResidual = wantResidualGrad ? Tensor(input.shape(), input.type()) : Tensor();
+  Tensor gradWeight({nfeat}, dtype::f32), gradBias({nfeat}, dtype::f32);
+  const size_t wsBytes = flhip_bn_workspace_bytes(&d);
+  Tensor ws = workspace(wsBytes);
+  DevicePtr xp(input), dyp(gradOutput), yp(output), gp(gamma), mp(mean), ip(invstd), dxp(gradInput),
+      drp(gradResidual), dgp(gradWeight), dbp(gradBias), wsp(ws);
+  check(flhip_bn_act_bwd(&d, xp.get(), dyp.get(), yp.get(), static_cast<const float*>(gp.get()),
+                         static_cast<const float*>(mp.get()), static_cast<const float*>(ip.get()), dxp.get(),
+                         drp.get(), static_cast<float*>(dgp.get()), static_cast<float*>(dbp.get()), wsp.get(),
+                         wsBytes, hipBackendStream()));
+  // event: inputs {gradOutput, input, gamma, saveMean, saveInvStd, output}, outputs {gradInput, gradWeight,
+  // gradBias, gradResidual (may be empty)}, ints {outer, features, inner}
+  if (scope.on())
+    scope.done({gradOutput, input, gamma, mean, invstd, output}, {gradInput, gradWeight, gradBias, gradResidual},
+               {d.outer, d.C, d.inner});
+  return std::make_tuple(gradInput, gradWeight, gradBias, gradResidual);
+}
+
 // ---- rnn (flashlight/fl/autograd/tensor/backend/cudnn/RNN.cpp:62-375) -------------------
 namespace {
 struct HipRnnPayload : detail::AutogradPayloadData {

@@ -52,6 +52,21 @@ class HipAutogradExtension : public AutogradExtension {
       const std::shared_ptr<detail::RNNGradData>, const Tensor&, const int, const int,
       const RnnMode, const bool, const float, std::shared_ptr<detail::AutogradPayload>) override;
 
+  // Not part of fl::AutogradExtension: batch norm (train mode, feature axes not starting at
+  // dimension 0) fused with the residual add and the ReLU that follow it in a ResNet block,
+  // output = relu(batchnorm(input) + residual) (residual may be empty), and its backward,
+  // which returns (gradInput, gradWeight, gradBias, gradResidual); gradResidual is only
+  // produced when wantResidualGrad.  fl::detail::batchnormRelu reaches them when the tensor's
+  // extension is this class and composes the three reference operators otherwise.
+  Tensor batchnormRelu(Tensor& saveMean, Tensor& saveVar, const Tensor& input, const Tensor& weight,
+                       const Tensor& bias, Tensor& runningMean, Tensor& runningVar,
+                       const std::vector<int>& axes, const double momentum, const double epsilon,
+                       const Tensor& residual, std::shared_ptr<detail::AutogradPayload> payload);
+  std::tuple<Tensor, Tensor, Tensor, Tensor> batchnormReluBackward(
+      const Tensor& gradOutput, const Tensor& output, const Tensor& saveMean, const Tensor& saveVar,
+      const Tensor& input, const Tensor& weight, const std::vector<int>& axes, const bool wantResidualGrad,
+      std::shared_ptr<detail::AutogradPayload> payload);
+
  private:
   Tensor workspace(size_t bytes);   // grown on demand, reused across calls
   Tensor ws_;

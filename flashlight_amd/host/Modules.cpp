@@ -235,6 +235,22 @@ Variable BatchNorm::forward(const Variable& input) {
                    runningMean_, runningVar_, featAxis_, train_ || !trackStats_, avgFactor, epsilon_);
 }
 
+Variable BatchNorm::forwardRelu(const Variable& input, const Variable& residual) {
+  if (!(train_ || !trackStats_)) {
+    // inference with running statistics: no fused kernel, the composition is exact
+    Variable y = forward(input);
+    return relu(residual.isEmpty() ? y : y + residual);
+  }
+  double avgFactor = 0.0;
+  if (train_ && trackStats_) {
+    ++numBatchesTracked_;
+    avgFactor = momentum_ < 0 ? 1.0 / numBatchesTracked_ : momentum_;
+  }
+  const Variable none(Tensor(), false);
+  return detail::batchnormRelu(input, params_.empty() ? none : params_[0], params_.empty() ? none : params_[1],
+                               runningMean_, runningVar_, featAxis_, avgFactor, epsilon_, residual);
+}
+
 std::string BatchNorm::prettyString() const {
   std::ostringstream ss;
   ss << "BatchNorm ( axis : { ";

@@ -160,6 +160,9 @@ class BatchNorm : public UnaryModule {
             bool affine = true, bool trackStats = true);
   using UnaryModule::forward;
   Variable forward(const Variable& input) override;
+  // relu(forward(input) + residual), residual optional (an empty Variable): the same
+  // bookkeeping as forward(); one fused pass on the HIP extension in train mode
+  Variable forwardRelu(const Variable& input, const Variable& residual = Variable());
   std::string prettyString() const override;
   Variable runningMean() const { return runningMean_; }
   Variable runningVar() const { return runningVar_; }

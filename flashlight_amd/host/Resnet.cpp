@@ -19,17 +19,45 @@ std::shared_ptr<Sequential> projection(int inC, int outC, int stride) {
   return s;
 }
 
-// main path through modules [0, last), plus the shortcut, then the final ReLU
+bool g_fuse = true;
+
+BatchNorm* asBatchNorm(const std::shared_ptr<Module>& m) { return dynamic_cast<BatchNorm*>(m.get()); }
+
+// main path through modules [0, last) in groups of (convolution, BatchNorm, ReLU), plus the
+// shortcut, then the final ReLU (Resnet.cpp:95-140)
 std::vector<Variable> residual(const Container& c, int mainModules, const std::vector<Variable>& inputs) {
   std::vector<Variable> out = inputs;
-  for (int i = 0; i + 1 < mainModules; ++i) out = c.module(i)->forward(out);
   const std::vector<Variable> shortcut =
       (int)c.modules().size() > mainModules ? c.module(mainModules)->forward(inputs) : inputs;
-  return c.module(mainModules - 1)->forward({out[0] + shortcut[0]});
+  if (!g_fuse) {
+    for (int i = 0; i + 1 < mainModules; ++i) out = c.module(i)->forward(out);
+    return c.module(mainModules - 1)->forward({out[0] + shortcut[0]});
+  }
+  for (int i = 0; i < mainModules; i += 3) {
+    out = c.module(i)->forward(out);
+    BatchNorm* bn = asBatchNorm(c.module(i + 1));
+    const bool last = i + 3 >= mainModules;
+    if (bn) {
+      out = {bn->forwardRelu(out[0], last ? shortcut[0] : Variable())};
+    } else {
+      out = c.module(i + 1)->forward(out);
+      out = c.module(i + 2)->forward(last ? std::vector<Variable>{out[0] + shortcut[0]} : out);
+    }
+  }
+  return out;
 }
 }  // namespace
 
-ConvBnAct::ConvBnAct(int inC, int outC, int kw, int kh, int sx, int sy, bool bn, bool act) {
+void setFusedBatchNormRelu(bool on) { g_fuse = on; }
+bool fusedBatchNormRelu() { return g_fuse; }
+
+std::vector<Variable> ConvBnAct::forward(const std::vector<Variable>& inputs) {
+  if (!(g_fuse && bn_ && act_)) return Sequential::forward(inputs);
+  std::vector<Variable> out = module(0)->forward(inputs);
+  return {asBatchNorm(module(1))->forwardRelu(out[0])};
+}
+
+ConvBnAct::ConvBnAct(int inC, int outC, int kw, int kh, int sx, int sy, bool bn, bool act) : bn_(bn), act_(act) {
   add(std::make_shared<Conv2D>(inC, outC, kw, kh, sx, sy, kSame, kSame, 1, 1, /* bias */ !bn));
   if (bn) add(std::make_shared<BatchNorm>(2, outC));
   if (act) add(std::make_shared<ReLU>());

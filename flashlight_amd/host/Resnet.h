@@ -12,9 +12,19 @@ namespace fl {
 namespace pkg {
 namespace vision {
 
+// BatchNorm -> ReLU and BatchNorm -> "+ shortcut" -> ReLU run as one fused operation in these
+// blocks (BatchNorm::forwardRelu) unless switched off; same results to rounding, same gradients.
+void setFusedBatchNormRelu(bool on);
+bool fusedBatchNormRelu();
+
 class ConvBnAct : public Sequential {
  public:
   ConvBnAct(int inC, int outC, int kw, int kh, int sx = 1, int sy = 1, bool bn = true, bool act = true);
+  using Sequential::forward;
+  std::vector<Variable> forward(const std::vector<Variable>& inputs) override;
+
+ private:
+  bool bn_, act_;
 };
 
 // two 3x3 convolutions + shortcut (ResNet-18/34)

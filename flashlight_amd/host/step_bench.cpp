@@ -5,7 +5,8 @@
 // run, the device time per operation class (HIP events around every operation of the
 // host layer) with the idle gaps between operations.
 //
-// usage: flhip_step_bench resnet50|speech [batch] [steps] [warmup] [f32|bf16]
+// usage: flhip_step_bench resnet50|speech [batch] [steps] [warmup] [f32|bf16] [unfused]
+// ("unfused": BatchNorm, residual add and ReLU as three operations, the reference's composition)
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -50,6 +51,8 @@ int main(int argc, char** argv) {
     const int steps = argc > 3 ? std::atoi(argv[3]) : 10;
     const int warmup = argc > 4 ? std::atoi(argv[4]) : 3;
     const bool half = argc > 5 && std::string(argv[5]) == "bf16";
+    const bool unfused = argc > 6 && std::string(argv[6]) == "unfused";
+    pkg::vision::setFusedBatchNormRelu(!unfused);
     setSeed(3);
 
     std::function<float()> step;
@@ -89,7 +92,7 @@ int main(int argc, char** argv) {
         for (auto& b : bns) b.zeroGrad();
         in.zeroGrad();
         Variable h = in;
-        for (int l = 0; l < 3; ++l) h = relu(bns[l](convs[l](h)));
+        for (int l = 0; l < 3; ++l) h = unfused ? relu(bns[l](convs[l](h))) : bns[l].forwardRelu(convs[l](h));
         h.backward(gradOut);
         fl::sync();
         return 0.f;
@@ -121,10 +124,10 @@ int main(int argc, char** argv) {
       c.calls += kv.second.calls / psteps;
     }
 
-    std::printf("{\"model\": \"%s\", \"batch\": %d, \"dtype\": \"%s\", \"steps\": %d, \"warmup\": %d, \"ms_per_step\": %.4f, "
+    std::printf("{\"model\": \"%s\", \"batch\": %d, \"dtype\": \"%s\", \"fused_bn_relu\": %s, \"steps\": %d, \"warmup\": %d, \"ms_per_step\": %.4f, "
                 "\"samples_per_s\": %.1f, \"loss\": %.5f, \"conv_gflop_per_step\": %.2f, \"device_cache_mb\": %.1f, "
                 "\"breakdown_ms\": {",
-                model.c_str(), B, half ? "bf16" : "f32", steps, warmup, ms, B / ms * 1e3, loss, flop / 1e9,
+                model.c_str(), B, half ? "bf16" : "f32", unfused ? "false" : "true", steps, warmup, ms, B / ms * 1e3, loss, flop / 1e9,
                 deviceCacheBytes() / 1e6);
     bool first = true;
     for (const auto& kv : classes) {

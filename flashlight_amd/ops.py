@@ -282,6 +282,51 @@ def batchnorm_backward(grad_output, input, weight, save_mean, save_invstd, axes)
     return dx, dg, db
 
 
+def batchnorm_relu(input, weight, bias, running_mean, running_var, axes, momentum, epsilon,
+                   residual=None, relu=True):
+    """flhip_bn_act_fwd_train: relu(batchnorm(input) + residual) in train mode, one pass over
+    the tensor -> (output, saveMean, saveInvStd).  residual is optional."""
+    x = _dev(input, "input")
+    outer, Cc, inner = bn_view(x.shape, axes)
+    d = capi.BnDesc(outer, Cc, inner, _dtype_tag(x))
+    g, b = _f32vec(weight, Cc, "weight"), _f32vec(bias, Cc, "bias")
+    r = _dev(residual, "residual")
+    if r is not None and (r.shape != x.shape or r.dtype != x.dtype):
+        raise ValueError("batchnormRelu: the residual must match the input")
+    y = torch.empty_like(x)
+    sm = torch.empty((Cc,), dtype=torch.float32, device=x.device)
+    si = torch.empty((Cc,), dtype=torch.float32, device=x.device)
+    nws = capi.lib().flhip_bn_workspace_bytes(C.byref(d))
+    ws = _ws(nws, x.device)
+    capi.check(capi.lib().flhip_bn_act_fwd_train(
+        C.byref(d), _ptr(x), _ptr(g), _ptr(b), _ptr(r), int(bool(relu)), _ptr(y), _ptr(sm), _ptr(si),
+        _ptr(_dev(running_mean, "runningMean")), _ptr(_dev(running_var, "runningVar")),
+        float(momentum), float(epsilon), _ptr(ws), nws, _stream()))
+    return y, sm, si
+
+
+def batchnorm_relu_backward(grad_output, input, output, weight, save_mean, save_invstd, axes,
+                            want_residual_grad=False):
+    """flhip_bn_act_bwd -> (gradInput, gradWeight, gradBias, gradResidual or None): the
+    gradient passes the ReLU mask of `output` (the forward result), then batchnormBackward."""
+    g, x, y = _dev(grad_output, "gradOutput"), _dev(input, "input"), _dev(output, "output")
+    if g.dtype != x.dtype or g.shape != x.shape or y.dtype != x.dtype or y.shape != x.shape:
+        raise ValueError("batchnormReluBackward: gradOutput and output must match the input")
+    outer, Cc, inner = bn_view(x.shape, axes)
+    d = capi.BnDesc(outer, Cc, inner, _dtype_tag(x))
+    w = _f32vec(weight, Cc, "weight")
+    dx = torch.empty_like(x)
+    dr = torch.empty_like(x) if want_residual_grad else None
+    dg = torch.empty((Cc,), dtype=torch.float32, device=x.device)
+    db = torch.empty((Cc,), dtype=torch.float32, device=x.device)
+    nws = capi.lib().flhip_bn_workspace_bytes(C.byref(d))
+    ws = _ws(nws, x.device)
+    capi.check(capi.lib().flhip_bn_act_bwd(C.byref(d), _ptr(x), _ptr(g), _ptr(y), _ptr(w), _ptr(save_mean),
+                                           _ptr(save_invstd), _ptr(dx), _ptr(dr), _ptr(dg), _ptr(db),
+                                           _ptr(ws), nws, _stream()))
+    return dx, dg, db, dr
+
+
 # ---- operations of the caller closures (flashlight/fl/autograd/Functions.cpp) -------
 # Shapes follow the rule of the rest of this module: a torch tensor's shape is the
 # Flashlight shape reversed (same memory).  A Flashlight [features, batch] matrix is a

@@ -216,6 +216,27 @@ int flhip_bn_bwd(const flhip_bn_desc* d, const void* x, const void* dy,
                  const float* save_invstd, void* dx, float* dgamma,
                  float* dbeta, void* ws, size_t ws_bytes, void* stream);
 
+/* Batch norm fused with what follows it in a ResNet block (ConvBnAct and the block tails of
+ * flashlight/pkg/vision/models/Resnet.cpp:27-46, 95-140: BatchNorm -> ReLU, and BatchNorm ->
+ * "+ shortcut" -> ReLU): y = relu(bn(x) + residual) in the one pass that writes y, instead of
+ * three trips through memory.  residual may be NULL; relu == 0 leaves the ReLU out.  Every
+ * other argument as flhip_bn_fwd_train.  Segment mode only (inner > 1): per-activation
+ * views return FLHIP_INVALID_ARGUMENT.  The reference has no fused counterpart; it composes
+ * AutogradExtension::batchnorm, operator+ and fl::relu (Functions.cpp:111-121, 329-338). */
+int flhip_bn_act_fwd_train(const flhip_bn_desc* d, const void* x, const float* gamma,
+                           const float* beta, const void* residual, int relu, void* y,
+                           float* save_mean, float* save_invstd, float* run_mean,
+                           float* run_var, double momentum, double eps, void* ws,
+                           size_t ws_bytes, void* stream);
+
+/* Its backward: dz = dy where y > 0, else 0 (y = the forward result, the ReLU's mask); then
+ * the batch-norm backward of flhip_bn_bwd on dz.  dresidual (may be NULL) receives dz, the
+ * gradient of the residual input.  For a forward call with relu == 0 use flhip_bn_bwd. */
+int flhip_bn_act_bwd(const flhip_bn_desc* d, const void* x, const void* dy, const void* y,
+                     const float* gamma, const float* save_mean, const float* save_invstd,
+                     void* dx, void* dresidual, float* dgamma, float* dbeta, void* ws,
+                     size_t ws_bytes, void* stream);
+
 /* Storage conversion between FLHIP_F32 and FLHIP_BF16 (round to nearest even) of n
  * elements; same dtype = copy.  Serves the casts the caller closures make around
  * the extension (Tensor::astype in flashlight/fl/autograd/Functions.cpp:1558-1561

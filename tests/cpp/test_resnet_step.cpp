@@ -332,13 +332,17 @@ int main(int argc, char** argv) {
   try {
     const int B = argc > 1 ? std::atoi(argv[1]) : 2;
     int fail = 0;
-    float lossOf[2] = {0, 0};
-    for (int pass = 0; pass < 2; ++pass) {
-      const bool half = pass == 1;
+    float lossOf[3] = {0, 0, 0};
+    // fp32 and bf16 with BatchNorm -> (+ shortcut) -> ReLU fused (the default), then bf16 with the
+    // three reference operators composed
+    for (int pass = 0; pass < 3; ++pass) {
+      const bool half = pass >= 1;
+      pkg::vision::setFusedBatchNormRelu(pass < 2);
       setSeed(3);
       auto model = pkg::vision::resnet50();
       const auto params = model->params();
-      std::printf("ResNet-50, %s, batch %d: %zu parameter tensors\n", half ? "bf16 storage" : "fp32", B, params.size());
+      std::printf("ResNet-50, %s, %s, batch %d: %zu parameter tensors\n", half ? "bf16 storage" : "fp32",
+                  pass < 2 ? "fused batch norm + ReLU" : "composed operators", B, params.size());
       Tensor x = Tensor::fromVector({224, 224, 3, B}, randn((size_t)B * 3 * 224 * 224, 1));
       Variable in(half ? x.astype(dtype::bf16) : x, false);
       std::vector<int32_t> labels(B);
@@ -370,7 +374,8 @@ int main(int argc, char** argv) {
         ops += kv.second.calls;
       }
       std::printf("  %ld results checked against the CPU checker\n", ops);
-      for (const char* need : {"conv2d", "conv2dBackwardData", "conv2dBackwardFilterBias dw", "pool2d values", "pool2dBackward"}) {
+      for (const char* need : {"conv2d", "conv2dBackwardData", "conv2dBackwardFilterBias dw", "pool2d values", "pool2dBackward",
+                               pass < 2 ? "batchnormRelu y" : "batchnorm y", pass < 2 ? "batchnormReluBackward dx" : "relu"}) {
         bool seen = false;
         for (const auto& kv : checker.stats) seen = seen || kv.first.rfind(need, 0) == 0;
         if (!seen) { std::printf("FAILED: no %s in the step\n", need); ++fail; }
@@ -389,10 +394,12 @@ int main(int argc, char** argv) {
       lossOf[pass] = a.loss;
     }
     // same weights, same input up to bf16 rounding: the losses agree to the bf16 bound
-    if (std::fabs(lossOf[0] - lossOf[1]) > 2e-2f * std::fabs(lossOf[0])) {
-      std::printf("FAILED: bf16 loss %.6f against fp32 loss %.6f\n", lossOf[1], lossOf[0]);
-      ++fail;
-    }
+    for (int pass = 1; pass < 3; ++pass)
+      if (std::fabs(lossOf[0] - lossOf[pass]) > 2e-2f * std::fabs(lossOf[0])) {
+        std::printf("FAILED: bf16 loss %.6f against fp32 loss %.6f\n", lossOf[pass], lossOf[0]);
+        ++fail;
+      }
+    pkg::vision::setFusedBatchNormRelu(true);
     std::printf(fail ? "%d check(s) FAILED\n" : "ResNet-50 step checks passed\n", fail);
     std::fflush(stdout);
     return fail ? 1 : 0;

@@ -33,6 +33,12 @@ CASES = [
     ((12, 128, 1, 750), [2]),       # speech rows after the stride-2 layer, 16 elements per thread
     ((5, 128, 53, 101), [2]),       # 32 elements per thread
     ((3, 64, 9, 9), [2]),           # forward resident, backward split (fewer than 128 features)
+    # bf16 storage: the 8-wide resident kernels (rows of a multiple of 8 elements) with 256 threads, and with
+    # 8 / 16 / 25 vectors per thread; fp32 takes the two-pass kernels for the largest
+    ((4, 128, 16, 16), [2]),
+    ((20, 128, 56, 56), [2]),
+    ((40, 128, 56, 56), [2]),
+    ((48, 128, 56, 56), [2]),
 ]
 
 
@@ -177,3 +183,65 @@ def test_full_size_invariants():
     assert s < 1e-1, s     # 1e5 elements per feature of magnitude ~1
     xh = (x.double() - sm.double().view(1, -1, 1, 1)) * si.double().view(1, -1, 1, 1)
     assert (dx.double() * xh).sum(dim=(0, 2, 3)).abs().max().item() < 1.0
+
+
+# ---- batch norm fused with ReLU and the residual add ---------------------------------------
+# against the checker's composition batchnorm -> (+ residual) -> relu and relu' -> batchnormBackward,
+# over every kernel family (resident 4-wide with 8 / 16 / 25 vectors, element-wise resident, split)
+FUSED = [
+    ((4, 16, 14, 14), [2]),         # small: resident, 256 threads
+    ((28, 28, 128, 20)[::-1], [2]),
+    ((56, 56, 128, 11)[::-1], [2]),  # 16 vectors per thread
+    ((56, 56, 128, 22)[::-1], [2]),  # 25 vectors per thread, part of dy (and of the mask) re-read
+    ((32, 128, 7, 7), [2]),         # element-wise resident
+    ((3, 64, 9, 9), [2]),           # forward resident, backward split
+    ((2, 5, 3, 7), [1, 2]),         # split, element-wise
+    ((6, 8, 60, 60), [2]),          # split, 4-wide
+    ((48, 128, 56, 56), [2]),       # bf16: 8-wide resident with 25 vectors per thread, part of dy and y re-read
+    ((40, 128, 56, 56), [2]),       # bf16: 16 vectors
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("with_residual", [False, True])
+@pytest.mark.parametrize("shape,axes", FUSED)
+def test_fused_bn_relu(shape, axes, with_residual, dtype):
+    from flashlight_amd import ops
+    rng = np.random.default_rng(len(shape) + shape[1] + int(with_residual))
+    lo = dtype == torch.bfloat16
+    rnd = bf16_round if lo else (lambda a: a)
+    x = rnd((rng.standard_normal(shape) * 1.5 + 0.3).astype(np.float32))
+    res = rnd(rng.standard_normal(shape).astype(np.float32)) if with_residual else None
+    dy = rnd(rng.standard_normal(shape).astype(np.float32))
+    outer, Cc, inner = ops.bn_view(shape, axes)
+    gamma = (1 + 0.2 * rng.standard_normal(Cc)).astype(np.float32)
+    beta = (0.3 * rng.standard_normal(Cc)).astype(np.float32)
+    yb, mean, var = flref.bn_fwd_train(outer, Cc, inner, x, gamma, beta, 1e-5)
+    pre = yb + (res if with_residual else 0)
+    y_ref = flref.relu_fwd(pre)
+    y, sm, si = ops.batchnorm_relu(dev(x, dtype), dev(gamma), dev(beta), None, None, axes, 0.1, 1e-5,
+                                   None if res is None else dev(res, dtype))
+    tol = 4e-3 if lo else 1e-4
+    assert rel_l2(host(y), y_ref) <= tol
+    assert rel_l2(host(sm), mean) <= 1e-5
+    # backward on the device's own forward result (its mask), like the tape does
+    yh = host(y)
+    dz_ref = flref.relu_bwd(dy, yh)
+    dx_ref, dg_ref, db_ref = flref.bn_bwd(outer, Cc, inner, x, dz_ref, gamma, mean, var, 1e-5)
+    dx, dg, db, dr = ops.batchnorm_relu_backward(dev(dy, dtype), dev(x, dtype), y, dev(gamma), sm, si, axes,
+                                                 want_residual_grad=with_residual)
+    assert rel_l2(host(dx), dx_ref) <= tol
+    assert rel_l2(host(dg), dg_ref) <= 1e-4 and rel_l2(host(db), db_ref) <= 1e-4
+    if with_residual:
+        assert np.array_equal(host(dr), dz_ref.reshape(shape))
+    # relu == 0: batch norm plus residual only
+    y2, _, _ = ops.batchnorm_relu(dev(x, dtype), dev(gamma), dev(beta), None, None, axes, 0.1, 1e-5,
+                                  None if res is None else dev(res, dtype), relu=False)
+    assert rel_l2(host(y2), pre) <= tol
+
+
+def test_fused_bn_relu_refuses_per_activation_mode():
+    from flashlight_amd import ops
+    x = torch.zeros((4, 3, 5, 5), device="cuda")
+    with pytest.raises(ValueError):
+        ops.batchnorm_relu(x, None, None, None, None, [0, 1, 2], 0.1, 1e-5)
