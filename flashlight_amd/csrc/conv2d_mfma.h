@@ -7,6 +7,7 @@
 namespace flhip {
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int MFMA_THREADS = 512;   // 8 waves: 2 per SIMD
 constexpr int MFMA_BM = 64;         // result rows (channels) per workgroup

@@ -1,5 +1,5 @@
 // Stride-1 convolution (forward and backward-data) for small windows in bf16
-// storage on the bf16 matrix cores (v_mfma_f32_16x16x32_bf16, fp32 accumulate).
+// storage on the bf16 matrix cores (v_mfma_f32_32x32x16_bf16, fp32 accumulate).
 //
 // Same tiling as the fp32 slab kernel: a workgroup owns R whole result rows of one
 // image x 64 result channels; per chunk of 32 source channels the source rows
@@ -329,19 +329,35 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
   }
 
   // =============================== MFMA waves ====================================
+  // v_mfma_f32_32x32x16_bf16: a wave owns 32 result channels (lane l: channel l % 32,
+  // contraction group l / 32) and NT blocks of 32 positions.  A chunk of 32 source channels
+  // is two k-steps: lane half h reads the 16-byte cells of channel groups h and h + 2.
+  // From one wave per SIMD the 32x32 shape issues at 2.4 PFLOP/s (measured), 16x16x32 at
+  // 0.85.  Positions left over after the last whole block of 32, when there are at most 16,
+  // run as one 16x16x32 block (S16) on the second wave of the pair.
   const int cw = wave - 4;
   const int wm = cw & 1, wn = cw >> 1;
-  const int base = p.NB >> 1, rem = p.NB & 1;
-  const int nt = base + (wn < rem ? 1 : 0);
-  const int nb0 = wn * base + min(wn, rem);
-  const int fr = lane & 15, fk = lane >> 4;
-  auto run = [&](auto ntc) {
+  const int npos_full = p.R * p.DW;
+  const int rem32 = npos_full & 31;
+  const int nb32 = (npos_full >> 5) + (rem32 > 16 ? 1 : 0);
+  const bool small = rem32 > 0 && rem32 <= 16;
+  const int base = nb32 >> 1, odd = nb32 & 1;
+  const int nt = base + (wn < odd ? 1 : 0);
+  const int nb0 = wn * base + min(wn, odd);
+  const bool has16 = small && wn == 1;
+  const int fr = lane & 31, fh = lane >> 5;        // 32x32 fragments
+  const int fr16 = lane & 15, fk16 = lane >> 4;    // 16x16 fragments of the small block
+  auto run = [&](auto ntc, auto s16c) {
     constexpr int NT = decltype(ntc)::value;
-    floatx4 acc[2][NT];
+    constexpr int NTA = NT > 0 ? NT : 1;
+    constexpr bool S16 = decltype(s16c)::value;
+    floatx16 acc[NTA];
+    floatx4 acc16[2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
-      for (int j = 0; j < NT; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+      for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+    acc16[0] = acc16[1] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     const int row_step = p.shs * p.WSP, col_step = p.sws;            // window row / column
     const int origin = (p.sh0 - p.min_sh) * p.WSP + p.sw0;           // tap (0,0)
@@ -350,51 +366,89 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
     const bool static33 = p.KH == 3 && p.KW == 3 && p.dlx == 1;
     const int first = origin + (static33 ? (BWD ? 2 : 0) * col_step : 0);
     const float inv_dw = 1.0f / (float)p.DW;
-    lds_cell bp[NT];
+    const int xg2 = 2 * p.XPL, ag2 = 2 * p.APL;    // from channel group h to group h + 2
+    lds_cell bp[NTA];
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
-      int pos = (nb0 + j) * 16 + fr;
+      int pos = (nb0 + j) * 32 + fr;
       if (pos >= npos) pos = 0;                  // padding lanes compute a discarded column
       int w;
       const int r = fast_div(pos, p.DW, inv_dw, &w);
-      bp[j] = (lds_cell)Xs + (fk * p.XPL + r * p.psh * p.WSP + w * p.psw + p.XOFF + first);
+      bp[j] = (lds_cell)Xs + (fh * p.XPL + r * p.psh * p.WSP + w * p.psw + p.XOFF + first);
     }
-    lds_cell ap = (lds_cell)As + (fk * p.APL + (wm * 32 + fr) * p.KHW);
+    lds_cell ap = (lds_cell)As + (fh * p.APL + (wm * 32 + fr) * p.KHW);
+    lds_cell bq = (lds_cell)Xs, aq = (lds_cell)As + (fk16 * p.APL + (wm * 32 + fr16) * p.KHW);
+    if (S16) {
+      int pos = nb32 * 32 + fr16;
+      if (pos >= npos) pos = 0;
+      int w;
+      const int r = fast_div(pos, p.DW, inv_dw, &w);
+      bq += fk16 * p.XPL + r * p.psh * p.WSP + w * p.psw + p.XOFF + first;
+    }
 
     auto frag = [](uint4 v) { return __builtin_bit_cast(bf16x8, v); };
-    auto mma2 = [&](int j, uint4 a0, uint4 a1, uint4 b) {
-      acc[0][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(a0), frag(b), acc[0][j], 0, 0, 0);
-      acc[1][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(a1), frag(b), acc[1][j], 0, 0, 0);
+    auto mma32 = [&](int j, uint4 a, uint4 b) {
+      acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(a), frag(b), acc[j], 0, 0, 0);
+    };
+    auto mma16 = [&](uint4 a0, uint4 a1, uint4 b) {
+      acc16[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(a0), frag(b), acc16[0], 0, 0, 0);
+      acc16[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(a1), frag(b), acc16[1], 0, 0, 0);
     };
 
     __syncthreads();                             // chunk 0 is in buffer 0
     for (int c = 0; c < n; ++c) {
       if (static33) {
         constexpr int T0 = BWD ? 2 : 0, TD = BWD ? -1 : 1;   // kw of the first tap, kw step
-        uint4 b[NT], a0, a1;
-        a0 = ap[T0];
-        a1 = ap[16 * 9 + T0];
+        uint4 b[NTA][2], a0, a1, sa0, sa1, sb;
+        if (NT > 0) {
+          a0 = ap[T0];
+          a1 = ap[ag2 + T0];
+        }
 #pragma unroll
-        for (int j = 0; j < NT; ++j) b[j] = bp[j][0];
-        // tap t: MFMAs on (a0, a1, b); behind each pair the fragment of tap t+1 is read
-        // into the b register just used
+        for (int j = 0; j < NT; ++j) {
+          b[j][0] = bp[j][0];
+          b[j][1] = bp[j][xg2];
+        }
+        if (S16) {
+          sa0 = aq[T0];
+          sa1 = aq[16 * 9 + T0];
+          sb = bq[0];
+        }
+        // tap t: first k-step of every block, then the second; behind each second step the
+        // fragments of tap t+1 are read into the registers just used
 #define FLHIP_TAP16(NEXT_TAP, NEXT_OFF)                                  \
   {                                                                      \
     __builtin_amdgcn_sched_barrier(0);                                   \
-    const uint4 n0 = ap[NEXT_TAP], n1 = ap[16 * 9 + (NEXT_TAP)];         \
+    uint4 n0, n1, m0, m1;                                                \
+    if (NT > 0) {                                                        \
+      n0 = ap[NEXT_TAP];                                                 \
+      n1 = ap[ag2 + (NEXT_TAP)];                                         \
+    }                                                                    \
+    _Pragma("unroll") for (int j = 0; j < NT; ++j) mma32(j, a0, b[j][0]); \
     _Pragma("unroll") for (int j = 0; j < NT; ++j) {                     \
-      mma2(j, a0, a1, b[j]);                                             \
-      b[j] = bp[j][NEXT_OFF];                                            \
+      mma32(j, a1, b[j][1]);                                             \
+      b[j][0] = bp[j][NEXT_OFF];                                         \
+      b[j][1] = bp[j][xg2 + (NEXT_OFF)];                                 \
+    }                                                                    \
+    if (S16) {                                                           \
+      m0 = aq[NEXT_TAP];                                                 \
+      m1 = aq[16 * 9 + (NEXT_TAP)];                                      \
+      mma16(sa0, sa1, sb);                                               \
+      sb = bq[NEXT_OFF];                                                 \
+      sa0 = m0;                                                          \
+      sa1 = m1;                                                          \
     }                                                                    \
     a0 = n0;                                                             \
     a1 = n1;                                                             \
-    _Pragma("unroll") for (int q = 0; q < NT + 2; ++q) {                 \
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);                 \
+    _Pragma("unroll") for (int q = 0; q < 2 * NT + 2 + (S16 ? 3 : 0); ++q) { \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                 \
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                 \
     }                                                                    \
     __builtin_amdgcn_sched_barrier(0);                                   \
   }
-#define FLHIP_NEXT_ROW16 _Pragma("unroll") for (int j = 0; j < NT; ++j) bp[j] += row_step;
+#define FLHIP_NEXT_ROW16                                                 \
+  _Pragma("unroll") for (int j = 0; j < NT; ++j) bp[j] += row_step;      \
+  bq += row_step;
         FLHIP_TAP16(T0 + TD, 1)
         FLHIP_TAP16(T0 + 2 * TD, 2)
         FLHIP_NEXT_ROW16
@@ -408,19 +462,29 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
 #undef FLHIP_NEXT_ROW16
 #undef FLHIP_TAP16
 #pragma unroll
-        for (int j = 0; j < NT; ++j) mma2(j, a0, a1, b[j]);
+        for (int j = 0; j < NT; ++j) mma32(j, a0, b[j][0]);
+#pragma unroll
+        for (int j = 0; j < NT; ++j) mma32(j, a1, b[j][1]);
+        if (S16) mma16(sa0, sa1, sb);
       } else {
         int tap = 0;
         for (int kh = 0; kh < p.KH; ++kh) {
           for (int kw = 0; kw < p.KW; ++kw, ++tap) {
-            const uint4 a0 = ap[tap], a1 = ap[16 * p.KHW + tap];
+            if (NT > 0) {
+              const uint4 a0 = ap[tap], a1 = ap[ag2 + tap];
 #pragma unroll
-            for (int j = 0; j < NT; ++j) mma2(j, a0, a1, bp[j][0]);
+              for (int j = 0; j < NT; ++j) mma32(j, a0, bp[j][0]);
+#pragma unroll
+              for (int j = 0; j < NT; ++j) mma32(j, a1, bp[j][xg2]);
+            }
+            if (S16) mma16(aq[tap], aq[16 * p.KHW + tap], bq[0]);
 #pragma unroll
             for (int j = 0; j < NT; ++j) bp[j] += col_step;
+            bq += col_step;
           }
 #pragma unroll
           for (int j = 0; j < NT; ++j) bp[j] += row_step - p.KW * col_step;
+          bq += row_step - p.KW * col_step;
         }
       }
       // back to the first tap, in the other buffer
@@ -429,23 +493,34 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
         const int xd = sign * p.x_cells - (p.KH - 1) * row_step - (static33 ? 0 : row_step);
 #pragma unroll
         for (int j = 0; j < NT; ++j) bp[j] += xd;
+        bq += xd;
         ap += sign * p.a_cells;
+        aq += sign * p.a_cells;
       }
       __syncthreads();
     }
 
     // ---- epilogue ----------------------------------------------------------------
+    // accumulator element r of a 32x32 block: channel (r / 4) * 8 + fh * 4 + r % 4, position fr;
+    // of a 16x16 block i: channel i * 16 + fk16 * 4 + r, position fr16
     if (staged) {
       for (int h = 0; h < 2; ++h) {
         if (wm == h) {
 #pragma unroll
           for (int j = 0; j < NT; ++j) {
-            const int pos = (nb0 + j) * 16 + fr;
+            const int pos = (nb0 + j) * 32 + fr;
+            if (pos < npos) {
+#pragma unroll
+              for (int r = 0; r < 16; ++r) lds[((r >> 2) * 8 + fh * 4 + (r & 3)) * SP + pos] = acc[j][r];
+            }
+          }
+          if (S16) {
+            const int pos = nb32 * 32 + fr16;
             if (pos < npos) {
 #pragma unroll
               for (int i = 0; i < 2; ++i)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) lds[(i * 16 + fk * 4 + r) * SP + pos] = acc[i][j][r];
+                for (int r = 0; r < 4; ++r) lds[(i * 16 + fk16 * 4 + r) * SP + pos] = acc16[i][r];
             }
           }
         }
@@ -455,45 +530,39 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
       }
       return;
     }
-    float bv[2][4];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) bv[i][r] = bias_lds[wm * 32 + i * 16 + fk * 4 + r];
     const size_t out_base = (size_t)img * p.DC * p.DH * p.DW + (size_t)r0 * p.DW;
-#pragma unroll
-    for (int j = 0; j < NT; ++j) {
-      const int pos = (nb0 + j) * 16 + fr;
-      if (pos < npos) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int m = wm * 32 + i * 16 + fk * 4 + r;
-            if (m < m_lim) {
-              const int ch = grp * p.DCg + mtile * BM + m;
-              st(dst, out_base + (size_t)ch * p.DH * p.DW + pos, acc[i][j][r] + bv[i][r]);
-            }
-          }
+    auto put = [&](int m, int pos, float v) {
+      if (m < m_lim && pos < npos) {
+        const int ch = grp * p.DCg + mtile * BM + m;
+        st(dst, out_base + (size_t)ch * p.DH * p.DW + pos, v + bias_lds[m]);
       }
+    };
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) put(wm * 32 + (r >> 2) * 8 + fh * 4 + (r & 3), (nb0 + j) * 32 + fr, acc[j][r]);
+    if (S16) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) put(wm * 32 + i * 16 + fk16 * 4 + r, nb32 * 32 + fr16, acc16[i][r]);
     }
   };
 
+  using std::integral_constant;
+#define FLHIP_RUN(N)                                                                        \
+  case N:                                                                                   \
+    if (has16) run(integral_constant<int, N>{}, integral_constant<bool, true>{});           \
+    else run(integral_constant<int, N>{}, integral_constant<bool, false>{});                \
+    break;
   switch (nt) {
-    case 0: case 1: run(std::integral_constant<int, 1>{}); break;
-    case 2: run(std::integral_constant<int, 2>{}); break;
-    case 3: run(std::integral_constant<int, 3>{}); break;
-    case 4: run(std::integral_constant<int, 4>{}); break;
-    case 5: run(std::integral_constant<int, 5>{}); break;
-    case 6: run(std::integral_constant<int, 6>{}); break;
-    case 7: run(std::integral_constant<int, 7>{}); break;
-    case 8: run(std::integral_constant<int, 8>{}); break;
-    case 9: run(std::integral_constant<int, 9>{}); break;
-    case 10: run(std::integral_constant<int, 10>{}); break;
-    case 11: run(std::integral_constant<int, 11>{}); break;
-    case 12: run(std::integral_constant<int, 12>{}); break;
-    default: run(std::integral_constant<int, 13>{}); break;
+    FLHIP_RUN(0) FLHIP_RUN(1) FLHIP_RUN(2) FLHIP_RUN(3) FLHIP_RUN(4) FLHIP_RUN(5) FLHIP_RUN(6)
+    default:
+      if (has16) run(integral_constant<int, 7>{}, integral_constant<bool, true>{});
+      else run(integral_constant<int, 7>{}, integral_constant<bool, false>{});
+      break;
   }
+#undef FLHIP_RUN
 }
 
 // smallest value >= v that is congruent to r modulo m
