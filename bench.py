@@ -32,7 +32,8 @@ PEAK = {"hbm_GBps": 8000.0, "f32_TFLOPs": 157.3, "bf16_TFLOPs": 2500.0}
 CONV_FLOP = 2 * 32 * 64 * 56 * 56 * 64 * 9          # one pass, 7.398752256e9
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by
 # the same counters on the library's copy kernel (see profiles/); None = not measured.
-MEASURED_TRAFFIC = {"conv2d_bwd_data_f32": 61.8e6}
+MEASURED_TRAFFIC = {"conv2d_bwd_data_f32": 61.7e6, "conv2d_bwd_filter_f32": 93.7e6,
+                    "conv2d_bwd_data_bf16": 32.5e6, "conv2d_bwd_filter_bf16": 67.0e6}
 
 
 def parse():
