@@ -45,6 +45,27 @@ Variable kaimingUniform(const Shape& shape, int fanIn, dtype type, bool calcGrad
   return uniform(shape, -limit, limit, type, calcGrad);
 }
 
+Variable normal(const Shape& shape, double stdv, double mean, dtype type, bool calcGrad) {
+  // stdv * randn + mean (Init.cpp:28-30)
+  std::normal_distribution<double> d(0.0, 1.0);
+  std::vector<float> v((size_t)shape.elements());
+  for (auto& x : v) x = (float)(stdv * d(generator()) + mean);
+  return Variable(fromFloats(shape, type, v), calcGrad);
+}
+
+Variable kaimingNormal(const Shape& shape, int fanIn, dtype type, bool calcGrad) {
+  return normal(shape, std::sqrt(1.0 / (double)fanIn), 0.0, type, calcGrad);   // Init.cpp:42-48
+}
+
+Variable glorotUniform(const Shape& shape, int fanIn, int fanOut, dtype type, bool calcGrad) {
+  const double limit = std::sqrt(3.0) * std::sqrt(2.0 / (double)(fanIn + fanOut));   // Init.cpp:50-58
+  return uniform(shape, -limit, limit, type, calcGrad);
+}
+
+Variable glorotNormal(const Shape& shape, int fanIn, int fanOut, dtype type, bool calcGrad) {
+  return normal(shape, std::sqrt(2.0 / (double)(fanIn + fanOut)), 0.0, type, calcGrad);   // Init.cpp:60-68
+}
+
 // ---- Module ----------------------------------------------------------------------------
 Variable Module::param(int position) const {
   if (!(position >= 0 && position < (int)params_.size()))

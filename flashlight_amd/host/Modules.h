@@ -22,6 +22,12 @@ Variable constant(double val, const Shape& shape, dtype type = dtype::f32, bool 
 Variable uniform(const Shape& shape, double min = 0, double max = 1, dtype type = dtype::f32,
                  bool calcGrad = true);
 Variable kaimingUniform(const Shape& shape, int fanIn, dtype type = dtype::f32, bool calcGrad = true);
+// flashlight/fl/nn/Init.cpp:19-31, 42-48, 50-68: stdv * randn + mean; kaimingNormal has stdv = sqrt(1 / fanIn);
+// the Glorot pair uses stdv = sqrt(2 / (fanIn + fanOut)) (uniform: limit sqrt(3) * stdv)
+Variable normal(const Shape& shape, double stdv = 1, double mean = 0, dtype type = dtype::f32, bool calcGrad = true);
+Variable kaimingNormal(const Shape& shape, int fanIn, dtype type = dtype::f32, bool calcGrad = true);
+Variable glorotUniform(const Shape& shape, int fanIn, int fanOut, dtype type = dtype::f32, bool calcGrad = true);
+Variable glorotNormal(const Shape& shape, int fanIn, int fanOut, dtype type = dtype::f32, bool calcGrad = true);
 
 // ---- Module (flashlight/fl/nn/modules/Module.cpp:17-112) --------------------------------
 class Module {

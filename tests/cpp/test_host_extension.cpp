@@ -169,6 +169,32 @@ static void testBatchingInvariance() {
 // ModuleTest.cpp:177-194 (ConvPadding: SAME padding with strides and dilation),
 // :382-396 (ConvolutionWithGroupFwd) and :398-413 (PoolingFwd): a batch equals its
 // samples run one by one, with the reference's module arguments, sizes and tolerances
+// Init.cpp:33-68: moments of the initialisers (the reference's InitTest checks shapes and types only)
+static void testInit() {
+  std::printf("initialisers\n");
+  setSeed(11);
+  const int fanIn = 576, n = 64 * 576;
+  auto moments = [&](const Variable& v, double* mean, double* var, double* lo, double* hi) {
+    const auto h = v.tensor().toHostVector();
+    double s = 0, q = 0;
+    *lo = 1e30; *hi = -1e30;
+    for (float x : h) { s += x; q += (double)x * x; *lo = std::min<double>(*lo, x); *hi = std::max<double>(*hi, x); }
+    *mean = s / h.size();
+    *var = q / h.size() - *mean * *mean;
+  };
+  double m, v, lo, hi;
+  moments(kaimingNormal(Shape({3, 3, 64, 64}), fanIn), &m, &v, &lo, &hi);
+  CHECK(std::fabs(m) < 3e-4 && std::fabs(v * fanIn - 1.0) < 0.03);
+  moments(kaimingUniform(Shape({3, 3, 64, 64}), fanIn), &m, &v, &lo, &hi);
+  const double lim = std::sqrt(3.0 / fanIn);
+  CHECK(std::fabs(m) < 3e-4 && std::fabs(v * fanIn - 1.0) < 0.03 && lo >= -lim && hi <= lim);
+  moments(glorotNormal(Shape({n}), 100, 300), &m, &v, &lo, &hi);
+  CHECK(std::fabs(v * 200 - 1.0) < 0.03);
+  moments(glorotUniform(Shape({n}), 100, 300), &m, &v, &lo, &hi);
+  CHECK(std::fabs(v * 200 - 1.0) < 0.03 && hi <= std::sqrt(3.0 / 200));
+  CHECK(kaimingNormal(Shape({4, 4}), 16, dtype::bf16).type() == dtype::bf16);
+}
+
 static void testModuleShapesAndBatching() {
   std::printf("module shapes and batching\n");
   setSeed(5);
@@ -1005,6 +1031,7 @@ int main() {
     testRnn();
     testArchBuilder();
     testModuleShapesAndBatching();
+    testInit();
     fl::sync();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());
