@@ -6,11 +6,12 @@
 //   backward-data  dx[c][q] = sum_m w[m][c] dy[m][q]
 // contract over the ROW index of the source, but an MFMA lane wants eight consecutive
 // contraction indices of one position.  The source tile goes to LDS as it is in memory
-// ([32 channels][128 positions]) and a lane gathers its eight channels with eight 16-bit
-// LDS reads (a pitch of 130 elements puts the four lane groups of a read in disjoint
-// banks); eight matrix instructions per wave and chunk pay for 16 + 4 such reads.
+// ([32 channels][128 positions]) and a lane fetches its eight channels with two
+// transposing reads (ds_read_b64_tr_b16: 16 lanes pass the addresses of four channel rows
+// x four 8-byte pieces and each receives four channels of one position); a pitch of 288
+// bytes keeps the four rows of a read in disjoint banks.
 // Weights: forward [m][c] is contraction-contiguous (16-byte LDS reads), backward-data
-// contracts over m and gathers like the source.  Positions are the rows of the
+// contracts over m: its tile is copied as it is and read like the source.  Positions are the rows of the
 // instruction tile, so a lane ends up with four consecutive positions of one result
 // channel: one 8-byte store.  Positions are flattened over the batch (a plane of 14x14
 // would waste a quarter of a 128-wide tile per image).  When a plane is not a multiple
@@ -35,8 +36,9 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int PB_BP = 128;    // positions per workgroup
 constexpr int PB_KC = 32;     // contraction per chunk = K of one instruction
-constexpr int PB_XP = PB_BP + 2;   // source tile pitch (elements)
-constexpr int PB_WP = PB_KC + 8;   // weight tile pitch ([result channel][contraction])
+constexpr int PB_XP = PB_BP + 16;  // source tile pitch (elements): 288 bytes, four rows' 32-byte pieces in disjoint banks
+constexpr int PB_WP = PB_KC + 8;   // weight tile pitch, forward ([result channel][contraction])
+constexpr int PB_WPB = 64 + 8;     // weight tile pitch, backward-data ([contraction][64 result channels])
 
 struct Pw16Params {
   int Kc, Mo;        // contraction channels, result channels
@@ -49,14 +51,21 @@ __device__ __forceinline__ bf16x8 as_bf16x8(uint32_t a, uint32_t b, uint32_t c, 
   return __builtin_bit_cast(bf16x8, v);
 }
 
-// eight elements of one column, rows r0 .. r0+7, of a 16-bit LDS tile
-__device__ __forceinline__ bf16x8 gather8(const uint16_t* tile, int pitch, int r0, int col) {
-  const uint16_t* t = tile + r0 * pitch + col;
-  const uint32_t a = (uint32_t)t[0] | ((uint32_t)t[pitch] << 16);
-  const uint32_t b = (uint32_t)t[2 * pitch] | ((uint32_t)t[3 * pitch] << 16);
-  const uint32_t c = (uint32_t)t[4 * pitch] | ((uint32_t)t[5 * pitch] << 16);
-  const uint32_t d = (uint32_t)t[6 * pitch] | ((uint32_t)t[7 * pitch] << 16);
-  return as_bf16x8(a, b, c, d);
+// Eight elements of one column of a 16-bit LDS tile stored [row][column]: rows r0 .. r0+7
+// of column c0 + s for lane s of each group of 16 lanes, by two transposing reads
+// (ds_read_b64_tr_b16).  In such a read lane s of a group passes the address of four
+// consecutive elements ("row slot" s) and receives element s % 4 of the row slots
+// s / 4, s / 4 + 4, s / 4 + 8, s / 4 + 12.  With row slot s pointing at columns
+// c0 + 4 * (s % 4) .. + 3 of tile row r0 + s / 4, lane s receives rows r0 .. r0 + 3 of
+// column c0 + s.  c0 and the pitch are multiples of 4 elements (8-byte addresses).
+typedef short shortx4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ bf16x8 gather8_tr(const uint16_t* tile, int pitch, int r0, int c0, int s) {
+  typedef __attribute__((address_space(3))) shortx4_t* lds_ptr;
+  const uint16_t* t = tile + (r0 + (s >> 2)) * pitch + c0 + 4 * (s & 3);
+  const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)t);
+  const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(t + 4 * pitch));
+  const uintx2_t l = __builtin_bit_cast(uintx2_t, lo), h = __builtin_bit_cast(uintx2_t, hi);
+  return as_bf16x8(l.x, l.y, h.x, h.y);
 }
 
 // 8 bytes at any 2-byte boundary
@@ -87,6 +96,8 @@ __global__ void __launch_bounds__(256)
 pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __restrict__ wgt,
                  const float* __restrict__ bias, bf16_t* __restrict__ dst) {
   constexpr int BM = MT * 16, WQ = BM / 64;      // result channels; 16-byte weight pieces per thread
+  static_assert(!BWD || BM == 64, "the backward-data weight tile is [contraction][64 result channels]");
+  static_assert(PB_KC * PB_WPB <= 64 * PB_WP, "both weight layouts share one buffer size");
   constexpr int XSZ = PB_KC * PB_XP;             // elements per source buffer
   constexpr int WSZ = BM * PB_WP;                // per weight buffer, [m][k] in both directions
   constexpr int YP = PB_BP + 8;                  // result staging pitch
@@ -152,10 +163,9 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
       else st.w[h] = in ? *reinterpret_cast<const uintx4_t*>(wgt + off) : uintx4_t{0u, 0u, 0u, 0u};
     }
   };
-  // Weights live in LDS as [result channel m][contraction k], 8-element contraction groups
-  // g stored at group slot g ^ ((m >> 3) & 3).  Forward copies 16-byte pieces; backward-data
-  // holds eight result channels of one k per piece and scatters them (the swizzle spreads
-  // those 16-bit stores over the banks).
+  // Forward weights live in LDS as [result channel m][contraction k], 8-element contraction
+  // groups g stored at group slot g ^ ((m >> 3) & 3); backward-data weights as in memory,
+  // [contraction k][result channel m], read by transposing reads like the source.
   auto wslot = [](int m, int g) { return m * PB_WP + 8 * (g ^ ((m >> 3) & 3)); };
   auto sstore = [&](int c, const Stage& st) {
     const int buf = c & 1;
@@ -181,12 +191,7 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
         if (!(k < p.Kc && m < p.Mo)) wv = uintx4_t{0u, 0u, 0u, 0u};
       }
       if (BWD) {
-        const uint32_t v[4] = {wv.x, wv.y, wv.z, wv.w};
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int m = wc + 64 * h + e;
-          Wt[wslot(m, wr >> 3) + (wr & 7)] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
-        }
+        *reinterpret_cast<uintx4_t*>(&Wt[wr * PB_WPB + wc]) = wv;
       } else {
         *reinterpret_cast<uintx4_t*>(&Wt[wslot(wr + 64 * h, wc >> 3)]) = wv;
       }
@@ -204,10 +209,11 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
     const uint16_t* Wt = Ws0 + buf * WSZ;
     bf16x8 a[2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) a[i] = gather8(X, PB_XP, 8 * fg, wave * 32 + i * 16 + fr);
+    for (int i = 0; i < 2; ++i) a[i] = gather8_tr(X, PB_XP, 8 * fg, wave * 32 + i * 16, fr);
 #pragma unroll
     for (int j = 0; j < MT; ++j) {
-      const bf16x8 b = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>(&Wt[wslot(j * 16 + fr, fg)]));
+      const bf16x8 b = BWD ? gather8_tr(Wt, PB_WPB, 8 * fg, j * 16, fr)
+                           : __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>(&Wt[wslot(j * 16 + fr, fg)]));
 #pragma unroll
       for (int i = 0; i < 2; ++i) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b, acc[i][j], 0, 0, 0);
     }
