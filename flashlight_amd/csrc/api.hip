@@ -36,6 +36,7 @@ static bool apply_option(Options& o, const char* name, const char* v) {
       if (strstr(v, "gemm1x1")) m |= Options::SKIP_GEMM1X1;
       if (strstr(v, "slab")) m |= Options::SKIP_SLAB;
       if (strstr(v, "tapped")) m |= Options::SKIP_TAPPED;
+      if (strstr(v, "strip")) m |= Options::SKIP_STRIP;
     }
     o.conv_skip = m;
     return true;

@@ -41,6 +41,14 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
   return __builtin_bit_cast(unsigned short, static_cast<__bf16>(f));
 }
 
+// two values in one instruction: a in the low half of the result, b in the high half
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  typedef float pack_f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 pack_bf16x2 __attribute__((ext_vector_type(2)));
+  const pack_f32x2 f = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, pack_bf16x2));
+}
+
 __device__ __forceinline__ float ld(const float* p, size_t i) { return p[i]; }
 __device__ __forceinline__ float ld(const bf16_t* p, size_t i) {
   return bf16_to_f32(p[i]);
@@ -66,8 +74,8 @@ __device__ __forceinline__ void st4(float* p, size_t i, float4 v) {
 }
 __device__ __forceinline__ void st4(bf16_t* p, size_t i, float4 v) {
   uint2 r;
-  r.x = (uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16);
-  r.y = (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16);
+  r.x = pack_bf16(v.x, v.y);
+  r.y = pack_bf16(v.z, v.w);
   *reinterpret_cast<uint2*>(p + i) = r;
 }
 
@@ -80,8 +88,7 @@ __device__ __forceinline__ void st4_stream(float* p, size_t i, float4 v) {
   __builtin_nontemporal_store(t, reinterpret_cast<floatx4_t*>(p + i));
 }
 __device__ __forceinline__ void st4_stream(bf16_t* p, size_t i, float4 v) {
-  const uintx2_t t = {(uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16),
-                      (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16)};
+  const uintx2_t t = {pack_bf16(v.x, v.y), pack_bf16(v.z, v.w)};
   __builtin_nontemporal_store(t, reinterpret_cast<uintx2_t*>(p + i));
 }
 
@@ -206,9 +213,9 @@ inline void launch_elementwise(const T* a, const T* b, T* out, size_t n, Op op, 
 // flhip_set_option(); no entry point calls getenv on its per-call path.
 struct Options {
   enum { ALGO_AUTO = 0, ALGO_DIRECT, ALGO_GATHER, ALGO_TAPPED, ALGO_CONVERT };
-  enum { SKIP_BF16 = 1, SKIP_GEMM1X1 = 2, SKIP_SLAB = 4, SKIP_TAPPED = 8 };
+  enum { SKIP_BF16 = 1, SKIP_GEMM1X1 = 2, SKIP_SLAB = 4, SKIP_TAPPED = 8, SKIP_STRIP = 16 };
   int conv_algo = ALGO_AUTO;      // CONV_ALGO = direct | gather | tapped | convert
-  unsigned conv_skip = 0;         // CONV_SKIP = comma list of bf16, gemm1x1, slab, tapped
+  unsigned conv_skip = 0;         // CONV_SKIP = comma list of bf16, gemm1x1, slab, tapped, strip
   int pw_pt = 2;                  // PW_PT = 2 | 4 | 8: position-tile width of the fp32 1x1 kernels / 32
   int pw16_pf = 0;                // PW16_PF = 1 | 4: chunks in flight in the bf16 1x1 kernels (0: by grid size)
   bool pw16_no_taps = false;      // PW16_NO_TAPS: bf16 windows with several taps stay off the gathered-taps path

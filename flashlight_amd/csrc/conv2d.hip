@@ -225,6 +225,8 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pointwise16_conv_fwd(g, x, w, bias, y, s, ws, ws_bytes);
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_STRIP) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_strip16_conv_fwd(g, x, w, bias, y, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_slab16_conv_fwd(g, x, w, bias, y, s);
     if (r < 0 && !skip(SK_GEMM)) r = mfma_pointwise_conv_fwd(g, d->dtype, x, w, bias, y, s);
@@ -259,6 +261,8 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pointwise16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes);
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_STRIP) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_strip16_conv_bwd_data(g, dy, w, dx, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s);
     if (r < 0 && !skip(SK_GEMM)) r = mfma_pointwise_conv_split(g, d->dtype, true, dy, w, nullptr, dx, ws, ws_bytes, s);

@@ -99,6 +99,11 @@ MORE = [
     # bias gradient with more than one tile of 64 filters (each tile writes only its own sums)
     ((2, 32, 8, 16), (136, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),
     ((2, 64, 20, 20), (160, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    # bf16 strip kernel (3x3, 64 source channels per group, rows of 40 .. 64 columns, strips of 7 rows):
+    # two strips, first / last strip at the image border; groups with two 64-channel tiles; full-width rows
+    ((2, 64, 14, 56), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((1, 128, 7, 40), (256, 64, 3, 3), (1, 1), (1, 1), (1, 1), 2),
+    ((1, 64, 21, 64), (128, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
 ]
 ALL = LIB_CASES + MORE
 
