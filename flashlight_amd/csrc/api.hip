@@ -37,6 +37,7 @@ static bool apply_option(Options& o, const char* name, const char* v) {
       if (strstr(v, "slab")) m |= Options::SKIP_SLAB;
       if (strstr(v, "tapped")) m |= Options::SKIP_TAPPED;
       if (strstr(v, "strip")) m |= Options::SKIP_STRIP;
+      if (strstr(v, "first")) m |= Options::SKIP_FIRST;
     }
     o.conv_skip = m;
     return true;

@@ -84,6 +84,13 @@ void wgrad_reduce_launch(const float* part, int nsplit, int E, int K, int want_d
 
 // bf16-storage variants on the bf16 matrix cores (conv2d_mfma_slab_bf16.hip,
 // conv2d_mfma_wgrad_slab_bf16.hip); same return convention.
+// bf16 forward of a first layer: few input channels, window rows of at most 8 columns, even column stride
+// (conv2d_mfma_first_bf16.hip)
+int mfma_first16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
+                          hipStream_t s);
+size_t mfma_first16_wgrad_ws(const ConvGeom& g);
+int mfma_first16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
+                       size_t ws_bytes, hipStream_t s);
 // bf16 3x3 stride-1 pad-1 over 64 source channels, whole contraction per workgroup (conv2d_mfma_strip_bf16.hip)
 int mfma_strip16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
                           hipStream_t s);

@@ -196,6 +196,8 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
     const size_t c = d->dtype == FLHIP_BF16 ? mfma_wgrad16_ws(g) : 0;
     const size_t e = mfma_pointwise_wgrad_ws(g);
     const size_t f = d->dtype == FLHIP_BF16 ? mfma_pointwise16_wgrad_ws(g) : 0;
+    const size_t h = d->dtype == FLHIP_BF16 ? mfma_first16_wgrad_ws(g) : 0;
+    if (h > a) a = h;
     if (b > a) a = b;
     if (e > a) a = e;
     if (f > a) a = f;
@@ -225,6 +227,8 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pointwise16_conv_fwd(g, x, w, bias, y, s, ws, ws_bytes);
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_FIRST) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_first16_conv_fwd(g, x, w, bias, y, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_STRIP) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_strip16_conv_fwd(g, x, w, bias, y, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
@@ -303,6 +307,8 @@ extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, 
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pointwise16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_FIRST) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_first16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_wgrad16(g, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0 && !skip(SK_GEMM))

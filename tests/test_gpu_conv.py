@@ -104,6 +104,13 @@ MORE = [
     ((2, 64, 14, 56), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
     ((1, 128, 7, 40), (256, 64, 3, 3), (1, 1), (1, 1), (1, 1), 2),
     ((1, 64, 21, 64), (128, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    # bf16 first-layer kernel (few channels, window rows within 8 columns, even column stride): the stem's
+    # window with odd / even padding, a last run of positions that is not full, one channel, a 5x6 window
+    # with different strides per axis, more than 64 filters
+    ((2, 3, 32, 32), (64, 3, 7, 7), (2, 2), (3, 3), (1, 1), 1),
+    ((3, 3, 24, 40), (32, 3, 7, 7), (2, 2), (3, 3), (1, 1), 1),
+    ((2, 1, 32, 32), (32, 1, 5, 5), (2, 2), (2, 2), (1, 1), 1),
+    ((2, 4, 12, 30), (96, 4, 5, 6), (1, 2), (2, 3), (1, 1), 1),
 ]
 ALL = LIB_CASES + MORE
 
