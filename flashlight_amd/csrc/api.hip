@@ -38,6 +38,7 @@ static bool apply_option(Options& o, const char* name, const char* v) {
       if (strstr(v, "tapped")) m |= Options::SKIP_TAPPED;
       if (strstr(v, "strip")) m |= Options::SKIP_STRIP;
       if (strstr(v, "first")) m |= Options::SKIP_FIRST;
+      if (strstr(v, "wgrad128")) m |= Options::SKIP_WGRAD128;
     }
     o.conv_skip = m;
     return true;

@@ -543,6 +543,199 @@ bool pw16_wgrad_plan(const ConvGeom& g, Pw16WgradParams* p) {
   return true;
 }
 
+// ---- filter gradient, 128 x 128 tiles -------------------------------------------------------
+// For layers with at least 128 channels on both sides.  dw[m][c] = sum over (image, position) of
+// dy[m][q] x[c][q]: both operands are contiguous along the contraction, so a fragment (one row,
+// 8 consecutive positions) is 16 bytes of memory and 16 bytes of LDS - no transposes anywhere.
+// A workgroup (4 waves, each 64 x 64 results on v_mfma_f32_32x32x16_bf16) owns dw[128 m][128 c]
+// and a slice of the chunks; a chunk = up to 64 positions of ONE image (planes of 49 positions are
+// one chunk of four steps, the last with one position; 196 = 3 chunks + one of one step), so a
+// row piece never leaves its image.  Thread t loads the 16-byte piece t % 8 of rows t / 8 + 32 g
+// (g = 0..3) of both tiles: 8 lanes cover a row's 128 bytes.  A piece that reaches past the end
+// of its row is masked in registers (it reads the first bytes of the next row; the very last
+// row of a tensor instead reads the 16 bytes that END at the row's end and shifts them down).
+constexpr int PG2_T = 128;         // tile side
+constexpr int PG2_P = 64 + 8;      // LDS pitch (elements)
+
+struct Pw16Wgrad2Params {
+  int C, Mo, P, N;
+  int ctiles, mtiles;
+  int cpi;                    // chunks per image
+  int nchunks, cps, nsplit;   // chunks over the batch, per slice, slices
+  int E, want_db;
+  unsigned x_bytes, dy_bytes;
+};
+
+__global__ void __launch_bounds__(256, 2)
+pw16_wgrad2_kernel(Pw16Wgrad2Params p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy,
+                   float* __restrict__ out, float* __restrict__ db_direct) {
+  extern __shared__ __align__(16) uint16_t lds_pg2[];     // [2 buffers][dy rows 0..127, x rows 128..255][PG2_P]
+  constexpr int OOB = (int)0x80000000;
+  const int slice = blockIdx.x, mtile = blockIdx.y / p.ctiles, ctile = blockIdx.y - mtile * p.ctiles;
+  const int m0 = mtile * PG2_T, c0 = ctile * PG2_T;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, fr = lane & 31, fh = lane >> 5;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int cbeg = slice * p.cps, cend = min(p.nchunks, cbeg + p.cps);
+  const __amdgpu_buffer_rsrc_t drsrc = make_rsrc(dy, p.dy_bytes), xrsrc = make_rsrc(x, p.x_bytes);
+
+  const int piece = tid & 7, lrow = tid >> 3;
+  int drow[4], xrow[4];        // element offset of the row inside an image, or -1
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int m = m0 + lrow + 32 * g, c = c0 + lrow + 32 * g;
+    drow[g] = m < p.Mo ? m * p.P : -1;
+    xrow[g] = c < p.C ? c * p.P : -1;
+  }
+  const float inv_cpi = 1.0f / (float)p.cpi;
+  uintx4_t sd[4], sx[4];
+  float bsum[4] = {0.f, 0.f, 0.f, 0.f};
+  const bool do_bias = p.want_db && ctile == 0;
+
+  // one operand's four pieces of chunk ch; v = positions of the piece inside the row (<= 0: none)
+  auto load4 = [&](__amdgpu_buffer_rsrc_t rsrc, const int (&row)[4], int img_elems, unsigned total_bytes, int n, int q,
+                   int v, uintx4_t (&dst)[4]) {
+    // elements of the piece inside the row -> dword masks
+    unsigned mk[4];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) mk[d] = (v > 2 * d ? 0x0000ffffu : 0u) | (v > 2 * d + 1 ? 0xffff0000u : 0u);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int off = (n * img_elems + row[g] + q) * 2;
+      const bool live = row[g] >= 0 && v > 0;
+      // the last row of the tensor: a piece that would pass its end
+      const bool last = live && v < 8 && (unsigned)(off + 16) > total_bytes;
+      uintx4_t t = __builtin_amdgcn_raw_buffer_load_b128(rsrc, live && !last ? off : OOB, 0, 0);
+      if (__builtin_amdgcn_ballot_w64(last) != 0) {
+        if (last) {
+          const uintx4_t u = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off - 2 * (8 - v), 0, 0);
+          const unsigned long long lo = ((unsigned long long)u.y << 32) | u.x, hi = ((unsigned long long)u.w << 32) | u.z;
+          const int sh = 16 * (8 - v);
+          const unsigned long long rl = sh >= 64 ? hi >> (sh - 64) : (lo >> sh) | (hi << (64 - sh));
+          const unsigned long long rh = sh >= 64 ? 0ull : hi >> sh;
+          t = uintx4_t{(unsigned)rl, (unsigned)(rl >> 32), (unsigned)rh, (unsigned)(rh >> 32)};
+        }
+      }
+      dst[g] = uintx4_t{t.x & mk[0], t.y & mk[1], t.z & mk[2], t.w & mk[3]};
+    }
+  };
+  auto gload = [&](int ch) {
+    int k;
+    const int n = fast_div(ch, p.cpi, inv_cpi, &k);
+    const int q = k * 64 + 8 * piece;
+    const int v = p.P - q;
+    load4(drsrc, drow, p.Mo * p.P, p.dy_bytes, n, q, v, sd);
+    load4(xrsrc, xrow, p.C * p.P, p.x_bytes, n, q, v, sx);
+  };
+  auto sstore = [&](int buf) {
+    uint16_t* b = lds_pg2 + buf * (2 * PG2_T * PG2_P);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      *reinterpret_cast<uintx4_t*>(b + (lrow + 32 * g) * PG2_P + 8 * piece) = sd[g];
+      *reinterpret_cast<uintx4_t*>(b + (PG2_T + lrow + 32 * g) * PG2_P + 8 * piece) = sx[g];
+      if (do_bias) {
+        const unsigned w4[4] = {sd[g].x, sd[g].y, sd[g].z, sd[g].w};
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          bsum[g] += bf16_to_f32((bf16_t)(w4[d] & 0xffffu)) + bf16_to_f32((bf16_t)(w4[d] >> 16));
+      }
+    }
+  };
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  if (cbeg < cend) {
+    gload(cbeg);
+    sstore(0);
+  }
+  __syncthreads();
+  for (int ch = cbeg; ch < cend; ++ch) {
+    const int buf = (ch - cbeg) & 1;
+    if (ch + 1 < cend) gload(ch + 1);
+    // steps of 16 positions that hold any: the chunk's positions are P - 64 k
+    int k;
+    fast_div(ch, p.cpi, inv_cpi, &k);
+    const int nks = min(4, (p.P - 64 * k + 15) >> 4);
+    const uint16_t* b = lds_pg2 + buf * (2 * PG2_T * PG2_P);
+    const uint16_t* ap = b + (wm * 64 + fr) * PG2_P + 8 * fh;
+    const uint16_t* bp = b + (PG2_T + wn * 64 + fr) * PG2_P + 8 * fh;
+    for (int ks = 0; ks < nks; ++ks) {
+      bf16x8 af[2], bf[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        af[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>(ap + i * 32 * PG2_P + 16 * ks));
+        bf[i] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>(bp + i * 32 * PG2_P + 16 * ks));
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    }
+    if (ch + 1 < cend) sstore(buf ^ 1);
+    __syncthreads();
+  }
+
+  // element r of acc[i][j]: row m0 + wm*64 + i*32 + (r/4)*8 + fh*4 + r%4, column c0 + wn*64 + j*32 + fr
+  float* o = out + (size_t)slice * (p.nsplit > 1 ? (size_t)p.E + p.Mo : 0);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int c = c0 + wn * 64 + j * 32 + fr;
+      if (c >= p.C) continue;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * 64 + i * 32 + (r >> 2) * 8 + fh * 4 + (r & 3);
+        if (m < p.Mo) o[(size_t)m * p.C + c] = acc[i][j][r];
+      }
+    }
+  if (do_bias) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      float bsm = bsum[g];
+      bsm += __shfl_xor(bsm, 1, 64);
+      bsm += __shfl_xor(bsm, 2, 64);
+      bsm += __shfl_xor(bsm, 4, 64);
+      const int m = m0 + lrow + 32 * g;
+      if (piece == 0 && m < p.Mo) {
+        if (p.nsplit > 1) o[p.E + m] = bsm;
+        else db_direct[m] = bsm;
+      }
+    }
+  }
+}
+
+bool pw16_wgrad2_plan(const ConvGeom& g, Pw16Wgrad2Params* p) {
+  if (!pw16_applies(g) || g.C < PG2_T || g.K < PG2_T || g.H * g.W < 8) return false;
+  p->C = g.C; p->Mo = g.K; p->P = g.H * g.W; p->N = g.N;
+  const long long xb = (long long)g.N * g.C * p->P * 2, db = (long long)g.N * g.K * p->P * 2;
+  if (xb >= (1ll << 31) || db >= (1ll << 31)) return false;
+  p->x_bytes = (unsigned)xb;
+  p->dy_bytes = (unsigned)db;
+  p->ctiles = (g.C + PG2_T - 1) / PG2_T;
+  p->mtiles = (g.K + PG2_T - 1) / PG2_T;
+  p->cpi = (p->P + 63) / 64;
+  p->nchunks = g.N * p->cpi;
+  p->E = g.K * g.C;
+  const long long tiles = (long long)p->ctiles * p->mtiles;
+  if (tiles > 65535) return false;
+  // every slice writes and re-reads the whole gradient
+#ifndef PG2_MULT
+#define PG2_MULT 2
+#endif
+  long long ns = (long long)PG2_MULT * mfma_num_cus() / tiles;
+  if (ns > p->nchunks / 4) ns = p->nchunks / 4;    // at least four chunks per slice
+  if (ns < 1) ns = 1;
+  p->cps = (int)((p->nchunks + ns - 1) / ns);
+  p->nsplit = (p->nchunks + p->cps - 1) / p->cps;
+  return true;
+}
+
 // ---- strided 1x1 windows ---------------------------------------------------------------
 // A 1x1 window with strides reads the input on a lattice.  With room for the lattice
 // points as a tensor of their own ([N][C][OH][OW]) the three passes become the stride-1
@@ -815,7 +1008,11 @@ size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g0) {
   else g = g0;
   Pw16WgradParams p{};
   if (!pw16_wgrad_plan(g, &p)) return 0;
-  return lattice + (p.nsplit > 1 ? (size_t)p.nsplit * ((size_t)p.E + p.Mo) * sizeof(float) : 0);
+  size_t need = p.nsplit > 1 ? (size_t)p.nsplit * ((size_t)p.E + p.Mo) * sizeof(float) : 0;
+  Pw16Wgrad2Params p2{};
+  if (pw16_wgrad2_plan(g, &p2) && p2.nsplit > 1)
+    need = std::max(need, (size_t)p2.nsplit * ((size_t)p2.E + p2.Mo) * sizeof(float));
+  return lattice + need;
 }
 
 int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, float* dw, float* db, void* ws,
@@ -836,6 +1033,20 @@ int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, fl
     x = ws;
     ws = static_cast<char*>(ws) + lb;
     ws_bytes -= lb;
+  }
+  Pw16Wgrad2Params p2{};
+  if (!(options().conv_skip & Options::SKIP_WGRAD128) && pw16_wgrad2_plan(g, &p2) && reinterpret_cast<uintptr_t>(x) % 4 == 0 &&
+      reinterpret_cast<uintptr_t>(dy) % 4 == 0) {
+    p2.want_db = db != nullptr;
+    const size_t need2 = p2.nsplit > 1 ? (size_t)p2.nsplit * ((size_t)p2.E + p2.Mo) * sizeof(float) : 0;
+    const size_t shmem = (size_t)2 * 2 * PG2_T * PG2_P * sizeof(uint16_t);
+    if ((!need2 || (ws && ws_bytes >= need2)) && mfma_allow_lds(reinterpret_cast<const void*>(pw16_wgrad2_kernel), shmem)) {
+      float* out2 = p2.nsplit > 1 ? static_cast<float*>(ws) : dw;
+      hipLaunchKernelGGL(pw16_wgrad2_kernel, dim3((unsigned)p2.nsplit, (unsigned)(p2.ctiles * p2.mtiles)), dim3(256), shmem, s,
+                         p2, static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), out2, db);
+      if (p2.nsplit > 1) wgrad_reduce_launch(static_cast<const float*>(ws), p2.nsplit, p2.E, p2.Mo, p2.want_db, dw, db, s);
+      return check_launch("conv2d_bwd_filter 1x1 (bf16 mfma, 128 x 128 tiles)");
+    }
   }
   p.want_db = db != nullptr;
   const size_t need = p.nsplit > 1 ? (size_t)p.nsplit * ((size_t)p.E + p.Mo) * sizeof(float) : 0;

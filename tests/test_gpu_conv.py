@@ -104,6 +104,11 @@ MORE = [
     ((2, 64, 14, 56), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
     ((1, 128, 7, 40), (256, 64, 3, 3), (1, 1), (1, 1), (1, 1), 2),
     ((1, 64, 21, 64), (128, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    # bf16 1x1 filter gradient on 128 x 128 tiles (at least 128 channels on both sides): planes of 49 and 25
+    # positions (row pieces masked / the tensor's last row shifted), channel tails, a plane of 3 chunks + 4
+    ((3, 136, 7, 7), (160, 136, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((2, 128, 5, 5), (128, 128, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((2, 128, 14, 14), (256, 128, 1, 1), (1, 1), (0, 0), (1, 1), 1),
     # bf16 first-layer kernel (few channels, window rows within 8 columns, even column stride): the stem's
     # window with odd / even padding, a last run of positions that is not full, one channel, a 5x6 window
     # with different strides per axis, more than 64 filters
