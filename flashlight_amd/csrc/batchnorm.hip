@@ -965,6 +965,9 @@ static int make_geom(const flhip_bn_desc* d, BnGeom* g, int* vec) {
 struct ResPlan {
   int threads, k, need;
 };
+#ifndef BN_SMALL_K
+#define BN_SMALL_K 16
+#endif
 static ResPlan resident_plan(const BnGeom& g, int vec, int min_c) {
   const int mode = options().bn_algo;
   ResPlan r{0, 0, 0};
@@ -974,7 +977,9 @@ static ResPlan resident_plan(const BnGeom& g, int vec, int min_c) {
     if (g.units > 32 * 1024 || g.inner > 0x7fffffff) return r;
     if (g.outer * g.C * g.inner * 4 >= (1ll << 31)) return r;
     if (mode != 2 && g.C < min_c) return r;
-    r.threads = g.units <= 8 * 256 ? 256 : 1024;
+    // short rows: workgroups of 4 waves (more of them per CU, cheaper barriers, more loads in
+    // flight per thread) as long as a thread holds at most 16 elements
+    r.threads = g.units <= BN_SMALL_K * 256 ? 256 : 1024;
     const int need = (int)((g.units + r.threads - 1) / r.threads);
     r.k = need <= 8 ? 8 : need <= 16 ? 16 : 32;
     r.need = need;
@@ -983,9 +988,9 @@ static ResPlan resident_plan(const BnGeom& g, int vec, int min_c) {
   if (g.units > (long long)RES_KMAX * 1024) return r;
   if (g.outer * g.C * g.inner * 4 >= (1ll << 31)) return r;   // 32-bit buffer offsets
   if (mode != 2 && g.C < min_c) return r;
-  if (g.units <= 8 * 256) {
+  if (g.units <= BN_SMALL_K * 256) {
     r.threads = 256;
-    r.k = 8;
+    r.k = g.units <= 8 * 256 ? 8 : 16;
   } else {
     r.threads = 1024;
     const int need = (int)((g.units + 1023) / 1024);
@@ -1005,9 +1010,9 @@ static ResPlan resident8_plan(const BnGeom& g, int vec, int dtype, int min_c) {
   if (units8 > (long long)RES_KMAX * 1024) return r;
   if (g.outer * g.C * g.inner * 2 >= (1ll << 31)) return r;   // 32-bit buffer offsets
   if (mode != 2 && g.C < min_c) return r;
-  if (units8 <= 8 * 256) {
+  if (units8 <= BN_SMALL_K * 256) {
     r.threads = 256;
-    r.k = 8;
+    r.k = units8 <= 8 * 256 ? 8 : 16;
   } else {
     r.threads = 1024;
     const int need = (int)((units8 + 1023) / 1024);
@@ -1046,7 +1051,8 @@ static int launch_bwd_resident8(const BnGeom& g, int need, const bf16_t* x, cons
 template <bool FUSE>
 static int run_train8(const BnGeom& g, const ResPlan& r, const bf16_t* x, bf16_t* y, const BnTrainArgs& a,
                       const BnFuseFwd<bf16_t>& fu, hipStream_t s) {
-  if (r.threads == 256) return launch_train_resident8<256, 8, FUSE>(g, x, y, a, fu, s);
+  if (r.threads == 256 && r.k == 8) return launch_train_resident8<256, 8, FUSE>(g, x, y, a, fu, s);
+  if (r.threads == 256) return launch_train_resident8<256, 16, FUSE>(g, x, y, a, fu, s);
   if (r.k == 8) return launch_train_resident8<1024, 8, FUSE>(g, x, y, a, fu, s);
   if (r.k == 16) return launch_train_resident8<1024, 16, FUSE>(g, x, y, a, fu, s);
   return launch_train_resident8<1024, RES_KMAX, FUSE>(g, x, y, a, fu, s);
@@ -1054,7 +1060,8 @@ static int run_train8(const BnGeom& g, const ResPlan& r, const bf16_t* x, bf16_t
 template <bool FUSE>
 static int run_bwd8(const BnGeom& g, const ResPlan& r, const bf16_t* x, const bf16_t* dy, bf16_t* dx,
                     const BnBwdArgs& a, const BnFuseBwd<bf16_t>& fu, hipStream_t s) {
-  if (r.threads == 256) return launch_bwd_resident8<256, 8, FUSE>(g, r.need, x, dy, dx, a, fu, s);
+  if (r.threads == 256 && r.k == 8) return launch_bwd_resident8<256, 8, FUSE>(g, r.need, x, dy, dx, a, fu, s);
+  if (r.threads == 256) return launch_bwd_resident8<256, 16, FUSE>(g, r.need, x, dy, dx, a, fu, s);
   if (r.k == 8) return launch_bwd_resident8<1024, 8, FUSE>(g, r.need, x, dy, dx, a, fu, s);
   if (r.k == 16) return launch_bwd_resident8<1024, 16, FUSE>(g, r.need, x, dy, dx, a, fu, s);
   return launch_bwd_resident8<1024, RES_KMAX, FUSE>(g, r.need, x, dy, dx, a, fu, s);
@@ -1106,8 +1113,10 @@ static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws
     if (vec == 1 && r.threads) {
       const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
       const dim3 grid((unsigned)g.C);
-      if (r.threads == 256)
+      if (r.threads == 256 && r.k == 8)
         hipLaunchKernelGGL((bn_train_resident1<T, 256, 8, FUSE>), grid, dim3(256), 0, s, g, bytes, xp, yp, a, fu);
+      else if (r.threads == 256)
+        hipLaunchKernelGGL((bn_train_resident1<T, 256, 16, FUSE>), grid, dim3(256), 0, s, g, bytes, xp, yp, a, fu);
       else if (r.k == 8)
         hipLaunchKernelGGL((bn_train_resident1<T, 1024, 8, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a, fu);
       else if (r.k == 16)
@@ -1116,7 +1125,8 @@ static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws
         hipLaunchKernelGGL((bn_train_resident1<T, 1024, 32, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a, fu);
       return check_launch("bn_fwd_train (resident, element-wise)");
     }
-    if (r.threads == 256) return launch_train_resident<T, 256, 8, FUSE>(g, xp, yp, a, fu, s);
+    if (r.threads == 256 && r.k == 8) return launch_train_resident<T, 256, 8, FUSE>(g, xp, yp, a, fu, s);
+    if (r.threads == 256) return launch_train_resident<T, 256, 16, FUSE>(g, xp, yp, a, fu, s);
     if (r.threads == 1024) {
       if (r.k == 8) return launch_train_resident<T, 1024, 8, FUSE>(g, xp, yp, a, fu, s);
       if (r.k == 16) return launch_train_resident<T, 1024, 16, FUSE>(g, xp, yp, a, fu, s);
@@ -1160,8 +1170,10 @@ static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void
     if (vec == 1 && r.threads) {
       const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
       const dim3 grid((unsigned)g.C);
-      if (r.threads == 256)
+      if (r.threads == 256 && r.k == 8)
         hipLaunchKernelGGL((bn_bwd_resident1<T, 256, 8, FUSE>), grid, dim3(256), 0, s, g, bytes, xp, dyp, dxp, a, fu);
+      else if (r.threads == 256)
+        hipLaunchKernelGGL((bn_bwd_resident1<T, 256, 16, FUSE>), grid, dim3(256), 0, s, g, bytes, xp, dyp, dxp, a, fu);
       else if (r.k == 8)
         hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 8, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a, fu);
       else if (r.k == 16)
@@ -1170,7 +1182,8 @@ static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void
         hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 32, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a, fu);
       return check_launch("bn_bwd (resident, element-wise)");
     }
-    if (r.threads == 256) return launch_bwd_resident<T, 256, 8, FUSE>(g, r.need, xp, dyp, dxp, a, fu, s);
+    if (r.threads == 256 && r.k == 8) return launch_bwd_resident<T, 256, 8, FUSE>(g, r.need, xp, dyp, dxp, a, fu, s);
+    if (r.threads == 256) return launch_bwd_resident<T, 256, 16, FUSE>(g, r.need, xp, dyp, dxp, a, fu, s);
     if (r.threads == 1024) {
       if (r.k == 8) return launch_bwd_resident<T, 1024, 8, FUSE>(g, r.need, xp, dyp, dxp, a, fu, s);
       if (r.k == 16) return launch_bwd_resident<T, 1024, 16, FUSE>(g, r.need, xp, dyp, dxp, a, fu, s);

@@ -165,6 +165,27 @@ def test_conv_bf16(case):
         assert rel_l2(got, ref) <= tight, (name, rel_l2(got, ref))
 
 
+# Shapes that the newer bf16 kernel families take, run again with the family switched off: the kernels
+# they replaced (still the path of neighbouring shapes) stay checked against the CPU checker on the same data.
+FAMILY_CASES = [
+    ("strip", ((2, 64, 14, 56), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1)),
+    ("first", ((2, 3, 32, 32), (64, 3, 7, 7), (2, 2), (3, 3), (1, 1), 1)),
+    ("wgrad128", ((3, 136, 7, 7), (160, 136, 1, 1), (1, 1), (0, 0), (1, 1), 1)),
+]
+
+
+@pytest.mark.parametrize("family,case", FAMILY_CASES)
+def test_conv_bf16_with_family_switched_off(family, case):
+    from flashlight_amd import capi
+    capi.set_option("CONV_SKIP", family)
+    try:
+        for name, (got, ref) in _run(case, 33, torch.bfloat16).items():
+            tight = 1e-4 if name in ("dw", "db") else 4e-3
+            assert rel_l2(got, ref) <= tight, (family, name, rel_l2(got, ref))
+    finally:
+        capi.set_option("CONV_SKIP", None)
+
+
 def test_bias_gradient_alone_and_empty_bias():
     # the caller passes an empty bias when its gradient is not needed
     # (flashlight/fl/autograd/Functions.cpp:1391-1395)
