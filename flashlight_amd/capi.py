@@ -29,7 +29,8 @@ class BnDesc(C.Structure):
 
 class RnnDesc(C.Structure):
     _fields_ = [(n, C.c_int32) for n in ("input_size", "hidden_size", "num_layers", "bidirectional", "mode",
-                                         "seq_len", "batch", "dtype")]
+                                         "seq_len", "batch", "dtype")] + [
+        ("dropout", C.c_float), ("seed_lo", C.c_uint32), ("seed_hi", C.c_uint32)]
 
 
 # every symbol include/flhip.h declares: name -> (restype, argtypes)

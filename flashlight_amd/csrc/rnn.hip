@@ -34,6 +34,8 @@ struct RnnGeom {
   int I, H, L, D, mode, T, B, G;
   size_t BH, GH;
   size_t nparams;
+  float dropout;
+  uint32_t seed_lo, seed_hi;
 };
 
 inline int gates_of(int mode) { return mode == RNN_LSTM ? 4 : mode == RNN_GRU ? 3 : 1; }
@@ -45,6 +47,8 @@ int make_geom(const flhip_rnn_desc* d, RnnGeom* g) {
                 "rnn: sizes must be positive");
   FLHIP_REQUIRE(d->mode >= RNN_RELU && d->mode <= RNN_GRU, "rnn: unknown mode");
   FLHIP_REQUIRE(d->dtype == FLHIP_F32, "rnn: f32 only");
+  FLHIP_REQUIRE(d->dropout >= 0.f && d->dropout < 1.f, "rnn: dropout must be in [0, 1)");
+  g->dropout = d->dropout; g->seed_lo = d->seed_lo; g->seed_hi = d->seed_hi;
   g->I = d->input_size; g->H = d->hidden_size; g->L = d->num_layers; g->D = d->bidirectional ? 2 : 1;
   g->mode = d->mode; g->T = d->seq_len; g->B = d->batch; g->G = gates_of(d->mode);
   g->BH = (size_t)g->B * g->H;
@@ -192,6 +196,21 @@ __global__ void __launch_bounds__(256) rnn_bias_kernel(const float* __restrict__
   const int q = blockIdx.x * 256 + threadIdx.x;
   if (q >= GH) return;
   bsum[q] = (mode == RNN_GRU && q >= 2 * H) ? bW[q] : bW[q] + bR[q];
+}
+
+// Dropout between layers: x[i] *= keep(i) / (1 - p) over the output sequence of `layer`, with the
+// counter-based mask of (seed, layer, i): two rounds of a 32-bit finaliser, the top 24 bits as
+// a uniform number in [0, 1).  The backward pass applies the same mask to the gradient.
+__global__ void __launch_bounds__(256) rnn_dropout_kernel(float* __restrict__ x, size_t n, uint32_t seed_lo,
+                                                          uint32_t seed_hi, uint32_t layer, float p, float scale) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  uint32_t h = (uint32_t)i * 0x9E3779B1u ^ seed_lo;
+  h ^= h >> 16; h *= 0x85EBCA6Bu; h ^= h >> 13; h *= 0xC2B2AE35u; h ^= h >> 16;
+  h += seed_hi + layer * 0x632BE5ABu;
+  h ^= h >> 16; h *= 0x85EBCA6Bu; h ^= h >> 13; h *= 0xC2B2AE35u; h ^= h >> 16;
+  const bool keep = (float)(h >> 8) * (1.0f / 16777216.0f) >= p;
+  x[i] = keep ? x[i] * scale : 0.f;
 }
 
 __global__ void __launch_bounds__(256) rnn_init_kernel(const float* __restrict__ src, float* __restrict__ dst, size_t n) {
@@ -887,25 +906,30 @@ extern "C" int flhip_rnn_fwd(const flhip_rnn_desc* d, const void* x, const void*
         default: rc = args(forward_layer_fused<RNN_GRU>);
       }
       if (rc != FLHIP_OK) return rc;
-      continue;
-    }
-    for (int dir = 0; dir < g.D; ++dir) {
-      const int pl = l * g.D + dir;
-      int rc;
-      auto args = [&](auto fn) {
-        return fn(g, pl, in, inl, wf, static_cast<const float*>(hx), static_cast<const float*>(cx), out,
-                  static_cast<float*>(hy), static_cast<float*>(cy), res, static_cast<float*>(ws), s);
-      };
-      switch (g.mode) {
-        case RNN_RELU: rc = args(forward_pl<RNN_RELU>); break;
-        case RNN_TANH: rc = args(forward_pl<RNN_TANH>); break;
-        case RNN_LSTM: rc = args(forward_pl<RNN_LSTM>); break;
-        default: rc = args(forward_pl<RNN_GRU>);
+    } else {
+      for (int dir = 0; dir < g.D; ++dir) {
+        const int pl = l * g.D + dir;
+        int rc;
+        auto args = [&](auto fn) {
+          return fn(g, pl, in, inl, wf, static_cast<const float*>(hx), static_cast<const float*>(cx), out,
+                    static_cast<float*>(hy), static_cast<float*>(cy), res, static_cast<float*>(ws), s);
+        };
+        switch (g.mode) {
+          case RNN_RELU: rc = args(forward_pl<RNN_RELU>); break;
+          case RNN_TANH: rc = args(forward_pl<RNN_TANH>); break;
+          case RNN_LSTM: rc = args(forward_pl<RNN_LSTM>); break;
+          default: rc = args(forward_pl<RNN_GRU>);
+        }
+        if (rc != FLHIP_OK) return rc;
       }
-      if (rc != FLHIP_OK) return rc;
     }
+    // what the next layer reads (and the backward pass reads again as that layer's input); the
+    // layer's own recurrence and hy / cy used the states kept beside it in the reserve buffer
+    if (g.dropout > 0.f && l + 1 < g.L)
+      hipLaunchKernelGGL(rnn_dropout_kernel, dim3(nblocks(act)), dim3(256), 0, s, out, act, g.seed_lo, g.seed_hi,
+                         (uint32_t)l, g.dropout, 1.0f / (1.0f - g.dropout));
   }
-  return FLHIP_OK;
+  return check_launch("rnn_fwd");
 }
 
 extern "C" int flhip_rnn_bwd(const flhip_rnn_desc* d, const void* x, const void* w, const void* dy,
@@ -968,6 +992,9 @@ extern "C" int flhip_rnn_bwd(const flhip_rnn_desc* d, const void* x, const void*
       hipLaunchKernelGGL(rnn_add2_kernel, dim3(nblocks(TB * inl)), dim3(256), 0, s, ginbuf, (const float*)nullptr, 0,
                          goutbuf, TB * inl);
       gout = goutbuf;
+      if (g.dropout > 0.f)
+        hipLaunchKernelGGL(rnn_dropout_kernel, dim3(nblocks(act)), dim3(256), 0, s, goutbuf, act, g.seed_lo, g.seed_hi,
+                           (uint32_t)(l - 1), g.dropout, 1.0f / (1.0f - g.dropout));
     }
   }
   (void)inmax;

@@ -469,9 +469,11 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> HipAutogradExtension::batchnormReluBa
 namespace {
 struct HipRnnPayload : detail::AutogradPayloadData {
   Tensor reserve;   // states and gate activations of the forward pass
+  unsigned long long seed = 0;   // of the dropout mask between layers
 };
 
-flhip_rnn_desc rnnDesc(const Tensor& input, int hiddenSize, int numLayers, RnnMode mode, bool bidirectional) {
+flhip_rnn_desc rnnDesc(const Tensor& input, int hiddenSize, int numLayers, RnnMode mode, bool bidirectional,
+                       float dropProb, unsigned long long seed) {
   if (input.type() != dtype::f32) throw std::runtime_error("HipAutogradExtension::rnn: f32 only");
   flhip_rnn_desc d{};
   d.input_size = (int32_t)input.dim(0);
@@ -482,9 +484,15 @@ flhip_rnn_desc rnnDesc(const Tensor& input, int hiddenSize, int numLayers, RnnMo
   d.bidirectional = bidirectional ? 1 : 0;
   d.mode = (int32_t)mode;
   d.dtype = FLHIP_F32;
+  if (!(dropProb >= 0.f && dropProb < 1.f)) throw std::invalid_argument("rnn: dropout must be in [0, 1)");
+  d.dropout = numLayers > 1 ? dropProb : 0.f;   // between layers only (RNN.cpp:83-90)
+  d.seed_lo = (uint32_t)seed;
+  d.seed_hi = (uint32_t)(seed >> 32);
   return d;
 }
 }  // namespace
+
+unsigned long long nextSeed();   // Modules.cpp: the process-wide generator
 
 std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::rnn(
     const Tensor& input, const Tensor& hiddenState, const Tensor& cellState, const Tensor& weights,
@@ -495,9 +503,8 @@ std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::rnn(
   for (const Tensor* t : {&hiddenState, &cellState, &weights})
     if (!t->isEmpty() && t->type() != input.type())
       throw std::invalid_argument("rnn doesn't support binary operations with Tensors of different types");
-  if (dropProb != 0.f)
-    throw std::runtime_error("HipAutogradExtension::rnn: dropout between layers is not supported");
-  const flhip_rnn_desc d = rnnDesc(input, hiddenSize, numLayers, mode, bidirectional);
+  const unsigned long long seed = dropProb > 0.f ? nextSeed() : 0ull;
+  const flhip_rnn_desc d = rnnDesc(input, hiddenSize, numLayers, mode, bidirectional, dropProb, seed);
   const Dim totalLayers = numLayers * (bidirectional ? 2 : 1), outSize = hiddenSize * (bidirectional ? 2 : 1);
   // RNN.cpp:97-113
   if (!hiddenState.isEmpty()) {
@@ -524,6 +531,7 @@ std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::rnn(
   if (autogradPayload) {
     auto payload = std::make_shared<HipRnnPayload>();
     payload->reserve = reserve;
+    payload->seed = seed;
     autogradPayload->data = payload;
   }
   if (scope.on()) scope.done({input, hiddenState, cellState, weights}, {y, hy, cy}, {hiddenSize, numLayers, (int)mode, bidirectional});
@@ -533,7 +541,7 @@ std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::rnn(
 std::tuple<Tensor, Tensor, Tensor, Tensor> HipAutogradExtension::rnnBackward(
     const Tensor& input, const Tensor& hiddenState, const Tensor& cellState, const Tensor& weights,
     const std::shared_ptr<detail::RNNGradData> gradData, const Tensor& output, const int numLayers,
-    const int hiddenSize, const RnnMode mode, const bool bidirectional, const float,
+    const int hiddenSize, const RnnMode mode, const bool bidirectional, const float dropProb,
     std::shared_ptr<detail::AutogradPayload> autogradPayload) {
   detail::OpScope scope("rnnBackward");
   if (!autogradPayload || !autogradPayload->data)   // RNN.cpp:246-249
@@ -541,7 +549,7 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> HipAutogradExtension::rnnBackward(
   auto payload = std::dynamic_pointer_cast<HipRnnPayload>(autogradPayload->data);
   if (!payload) throw std::invalid_argument("rnnBackward: payload of another operation");
   if (!gradData) throw std::invalid_argument("rnnBackward: no gradient data");
-  const flhip_rnn_desc d = rnnDesc(input, hiddenSize, numLayers, mode, bidirectional);
+  const flhip_rnn_desc d = rnnDesc(input, hiddenSize, numLayers, mode, bidirectional, dropProb, payload->seed);
   const Dim totalLayers = numLayers * (bidirectional ? 2 : 1);
   // output gradients nobody produced are zero (RNN.cpp:262-275)
   for (const Tensor* t : {&gradData->dy, &gradData->dhy, &gradData->dcy})

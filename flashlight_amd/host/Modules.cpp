@@ -24,6 +24,7 @@ Tensor fromFloats(const Shape& shape, dtype type, const std::vector<float>& v) {
 }  // namespace
 
 void setSeed(unsigned long long seed) { generator().seed(seed); }
+unsigned long long nextSeed() { return generator()(); }
 
 Variable constant(double val, const Shape& shape, dtype type, bool calcGrad) {
   return Variable(fromFloats(shape, type, std::vector<float>((size_t)shape.elements(), (float)val)),

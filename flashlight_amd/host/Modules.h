@@ -18,6 +18,8 @@ namespace fl {
 // ---- initialisation (flashlight/fl/nn/Init.cpp:21-48, 142-200) --------------------------
 // Values are drawn on the host from one process-wide generator and copied to the device.
 void setSeed(unsigned long long seed);
+// 64 fresh bits of that generator: the seed of a device-side mask (dropout between rnn layers)
+unsigned long long nextSeed();
 Variable constant(double val, const Shape& shape, dtype type = dtype::f32, bool calcGrad = true);
 Variable uniform(const Shape& shape, double min = 0, double max = 1, dtype type = dtype::f32,
                  bool calcGrad = true);

@@ -583,11 +583,15 @@ def layer_norm_backward(grad_output, ctx, weight=None):
 RNN_RELU, RNN_TANH, RNN_LSTM, RNN_GRU = 0, 1, 2, 3
 
 
-def _rnn_desc(x, hidden_size, num_layers, mode, bidirectional):
+def _rnn_desc(x, hidden_size, num_layers, mode, bidirectional, dropout=0.0, seed=0):
     if x.dim() != 3 or x.dtype != torch.float32:
         raise ValueError("rnn: input must be fp32 [seq, batch, input] (Flashlight [input, batch, seq])")
+    if not 0.0 <= dropout < 1.0:
+        raise ValueError("rnn: dropout must be in [0, 1)")
     T, B, I = x.shape
-    return capi.RnnDesc(I, hidden_size, num_layers, int(bool(bidirectional)), int(mode), T, B, capi.F32)
+    # dropout acts between layers only (backend/cudnn/RNN.cpp:83-90)
+    return capi.RnnDesc(I, hidden_size, num_layers, int(bool(bidirectional)), int(mode), T, B, capi.F32,
+                        float(dropout) if num_layers > 1 else 0.0, seed & 0xffffffff, (seed >> 32) & 0xffffffff)
 
 
 def rnn_param_count(input_size, hidden_size, num_layers, mode, bidirectional):
@@ -596,15 +600,14 @@ def rnn_param_count(input_size, hidden_size, num_layers, mode, bidirectional):
 
 
 def rnn(input, hidden_state, cell_state, weights, hidden_size, num_layers, mode, bidirectional,
-        dropout=0.0):
+        dropout=0.0, seed=0):
     """AutogradExtension::rnn -> (output, hiddenOut, cellOut or None, reserve).  Tensors are
     torch views of the Flashlight ones (shape reversed): input [seq, batch, input], states
     [layers*dirs, batch, hidden], output [seq, batch, dirs*hidden]; weights flat in cuDNN's
-    order.  reserve goes to rnn_backward (the payload of the reference's closure)."""
-    if dropout != 0.0:
-        raise ValueError("rnn: dropout between layers is not supported by this backend")
+    order.  reserve goes to rnn_backward (the payload of the reference's closure), together
+    with the same dropout and seed (the mask between layers is a function of the seed)."""
     x, w = _dev(input, "input"), _dev(weights, "weights")
-    d = _rnn_desc(x, hidden_size, num_layers, mode, bidirectional)
+    d = _rnn_desc(x, hidden_size, num_layers, mode, bidirectional, dropout, seed)
     L = capi.lib()
     if w.numel() != L.flhip_rnn_param_count(C.byref(d)):
         raise ValueError("invalid # of parameters or wrong input shape for RNN")
@@ -628,11 +631,11 @@ def rnn(input, hidden_state, cell_state, weights, hidden_size, num_layers, mode,
 
 
 def rnn_backward(input, weights, reserve, hidden_size, num_layers, mode, bidirectional,
-                 grad_output=None, grad_hidden=None, grad_cell=None):
+                 grad_output=None, grad_hidden=None, grad_cell=None, dropout=0.0, seed=0):
     """AutogradExtension::rnnBackward -> (gradInput, gradHidden, gradCell or None, gradWeights);
     missing output gradients count as zero (Functions.cpp:1677-1699)."""
     x, w = _dev(input, "input"), _dev(weights, "weights")
-    d = _rnn_desc(x, hidden_size, num_layers, mode, bidirectional)
+    d = _rnn_desc(x, hidden_size, num_layers, mode, bidirectional, dropout, seed)
     L = capi.lib()
     D = 2 if bidirectional else 1
     sshape = (num_layers * D, d.batch, hidden_size)

@@ -343,9 +343,16 @@ int flhip_copy_bytes(const void* src, void* dst, size_t bytes, void* stream);
  * pseudo-layer the input biases then the recurrent biases.  Gates: LSTM i, f, g, o;
  * GRU r, z, n.  mode: 0 ReLU, 1 tanh, 2 LSTM, 3 GRU (fl::RnnMode).  x is Flashlight
  * [input, batch, seq] (memory [seq][batch][input]), hx / cx / hy / cy
- * [hidden, batch, layers*dirs], y [hidden*dirs, batch, seq].  fp32 only; no dropout. */
+ * [hidden, batch, layers*dirs], y [hidden*dirs, batch, seq].  fp32 only.
+ * dropout (RNN.cpp:83-90, training): the output sequence of every layer but the last is
+ * multiplied by keep / (1 - dropout) before the next layer reads it; the states hy / cy are
+ * not touched.  keep is a counter-based mask of (seed, layer, element index) - cuDNN draws
+ * from a generator of its own, so WHICH elements fall is particular to this library; the
+ * backward call must be given the descriptor of its forward call (same dropout and seed). */
 typedef struct flhip_rnn_desc {
   int32_t input_size, hidden_size, num_layers, bidirectional, mode, seq_len, batch, dtype;
+  float dropout;              /* 0 <= dropout < 1; 0 = none */
+  uint32_t seed_lo, seed_hi;  /* of the dropout mask */
 } flhip_rnn_desc;
 /* number of weight elements (cudnnGetRNNParamsSize / element size); 0 for a bad descriptor */
 size_t flhip_rnn_param_count(const flhip_rnn_desc* d);

@@ -627,6 +627,16 @@ static void rnn_tape_free(rnn_tape* tp) {
 }
 
 /* runs the whole stack; acts[l] = input of layer l (acts[layers] = y), tapes per pseudo-layer */
+/* counter-based mask: two rounds of a 32-bit finaliser over (index, layer, seed); the top 24
+ * bits as a uniform number in [0, 1) */
+int flref_dropout_keep(uint32_t seed_lo, uint32_t seed_hi, uint32_t layer, uint32_t index, float dropout) {
+  uint32_t h = index * 0x9E3779B1u ^ seed_lo;
+  h ^= h >> 16; h *= 0x85EBCA6Bu; h ^= h >> 13; h *= 0xC2B2AE35u; h ^= h >> 16;
+  h += seed_hi + layer * 0x632BE5ABu;
+  h ^= h >> 16; h *= 0x85EBCA6Bu; h ^= h >> 13; h *= 0xC2B2AE35u; h ^= h >> 16;
+  return (float)(h >> 8) * (1.0f / 16777216.0f) >= dropout;
+}
+
 static void rnn_stack_fwd(const flref_rnn* d, const float* x, const float* hx, const float* cx,
                           const float* w, double** acts, rnn_tape* tapes) {
   const int H = d->hidden, D = d->bidirectional ? 2 : 1, T = d->T, B = d->B;
@@ -639,6 +649,13 @@ static void rnn_stack_fwd(const flref_rnn* d, const float* x, const float* hx, c
     for (int dir = 0; dir < D; ++dir) {
       tapes[l * D + dir] = rnn_tape_new(d);
       rnn_layer_fwd(d, l * D + dir, acts[l], inl, w, hx, cx, acts[l + 1], &tapes[l * D + dir]);
+    }
+    /* dropout on what the next layer reads (the layer's own recurrence used the states in its tape) */
+    if (d->dropout > 0.f && l + 1 < d->layers) {
+      const size_t n = (size_t)T * B * D * H;
+      const double scale = 1.0 / (1.0 - (double)d->dropout);
+      for (size_t i = 0; i < n; ++i)
+        acts[l + 1][i] = flref_dropout_keep(d->seed_lo, d->seed_hi, (uint32_t)l, (uint32_t)i, d->dropout) ? acts[l + 1][i] * scale : 0.0;
     }
   }
 }
@@ -750,6 +767,13 @@ void flref_rnn_bwd(const flref_rnn* d, const float* x, const float* hx, const fl
     }
     free(gout);
     gout = gin;
+    /* gin is the gradient of what this layer read: the dropped output of the layer below */
+    if (d->dropout > 0.f && l > 0) {
+      const size_t n = (size_t)T * B * D * H;
+      const double scale = 1.0 / (1.0 - (double)d->dropout);
+      for (size_t i = 0; i < n; ++i)
+        gout[i] = flref_dropout_keep(d->seed_lo, d->seed_hi, (uint32_t)(l - 1), (uint32_t)i, d->dropout) ? gout[i] * scale : 0.0;
+    }
   }
   const size_t nx = (size_t)T * B * d->input_size;
   for (size_t i = 0; i < nx; ++i) dx[i] = (float)gout[i];

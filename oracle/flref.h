@@ -136,10 +136,20 @@ void flref_cce_bwd(int classes, int cols, const float* grad, const int32_t* targ
  * ([hidden][hidden]); after all matrices, per pseudo-layer the input biases then the
  * recurrent biases.  Gates: LSTM i, f, g, o; GRU r, z, n with
  * n = tanh(W_n x + b_Wn + r * (R_n h + b_Rn)), h' = (1 - z) * n + z * h.
- * mode: 0 ReLU, 1 tanh, 2 LSTM, 3 GRU (flashlight/fl/common/Defines.h:62-67).  No dropout. */
+ * mode: 0 ReLU, 1 tanh, 2 LSTM, 3 GRU (flashlight/fl/common/Defines.h:62-67).
+ * dropout > 0 (training, flashlight/fl/autograd/tensor/backend/cudnn/RNN.cpp:83-90): the
+ * output sequence of every layer but the last is multiplied, element by element, by
+ * keep / (1 - dropout) before the next layer reads it; keep = flref_dropout_keep().  cuDNN
+ * draws its mask from a generator of its own: which elements are dropped is a property
+ * of this restatement (parity unpinned against the reference), where the mask is applied
+ * and how it scales follows cuDNN's documented behaviour and is checked against torch. */
 typedef struct flref_rnn {
   int32_t input_size, hidden, layers, bidirectional, mode, T, B;
+  float dropout;
+  uint32_t seed_lo, seed_hi;
 } flref_rnn;
+/* 1 if element `index` of the output of layer `layer` is kept */
+int flref_dropout_keep(uint32_t seed_lo, uint32_t seed_hi, uint32_t layer, uint32_t index, float dropout);
 int64_t flref_rnn_param_count(const flref_rnn* d);
 /* hx, cx may be NULL (zeros); cy may be NULL */
 void flref_rnn_fwd(const flref_rnn* d, const float* x, const float* hx, const float* cx,

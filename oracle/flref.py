@@ -386,11 +386,21 @@ RNN_RELU, RNN_TANH, RNN_LSTM, RNN_GRU = 0, 1, 2, 3
 
 
 class RnnDesc(C.Structure):
-    _fields_ = [(n, C.c_int32) for n in ("input_size", "hidden", "layers", "bidirectional", "mode", "T", "B")]
+    _fields_ = [(n, C.c_int32) for n in ("input_size", "hidden", "layers", "bidirectional", "mode", "T", "B")] + [
+        ("dropout", C.c_float), ("seed_lo", C.c_uint32), ("seed_hi", C.c_uint32)]
 
 
-def rnn_desc(input_size, hidden, layers, bidirectional, mode, T, B):
-    return RnnDesc(input_size, hidden, layers, int(bool(bidirectional)), mode, T, B)
+def rnn_desc(input_size, hidden, layers, bidirectional, mode, T, B, dropout=0.0, seed=0):
+    return RnnDesc(input_size, hidden, layers, int(bool(bidirectional)), mode, T, B, float(dropout),
+                   seed & 0xffffffff, (seed >> 32) & 0xffffffff)
+
+
+def dropout_keep(seed, layer, n, dropout):
+    """the keep mask of the first n elements of the output of `layer` (bool array)"""
+    f = lib().flref_dropout_keep
+    f.restype = C.c_int
+    f.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_float]
+    return np.array([f(seed & 0xffffffff, (seed >> 32) & 0xffffffff, layer, i, dropout) for i in range(n)], bool)
 
 
 def rnn_param_count(d):

@@ -55,6 +55,11 @@ static double relL2(const std::vector<float>& a, const std::vector<float>& b) {
   }
   return den > 0 ? std::sqrt(num / den) : std::sqrt(num);
 }
+static double maxAbsDiff(const std::vector<float>& a, const std::vector<float>& b) {
+  double m = a.size() == b.size() ? 0 : 1e30;
+  for (size_t i = 0; i < a.size() && i < b.size(); ++i) m = std::max(m, std::fabs((double)a[i] - b[i]));
+  return m;
+}
 static float bf16round(float f) {
   uint32_t u;
   std::memcpy(&u, &f, 4);
@@ -989,10 +994,40 @@ static void testRnn() {
   out.backward(Variable(Tensor::full(out.shape(), 1., dtype::f32), false));
   CHECK(lstm.param(0).isGradAvailable() && xin.isGradAvailable());
   CHECK(throws<std::invalid_argument>([&] { lstm.forward(std::vector<Variable>{}); }));
+  // dropout between layers (cudnn/RNN.cpp:83-90): training draws a fresh mask per call, the
+  // backward pass reuses the mask of its forward pass, eval switches it off (RNN.cpp:74)
   RNN drop(5, 4, 2, RnnMode::GRU, false, 0.3f);
-  CHECK(throws<std::runtime_error>([&] { drop(xin); }));   // dropout between layers is not provided
+  setSeed(31);
+  Variable xd(Tensor::fromVector({5, 3, 6}, randn(90, 98)), true);
+  Variable d1 = drop(xd), d2 = drop(xd);
+  CHECK(d1.shape() == Shape({4, 3, 6}));
+  CHECK(maxAbsDiff(hostOf(d1), hostOf(d2)) > 1e-4);         // two masks
+  setSeed(31);
+  CHECK(maxAbsDiff(hostOf(drop(xd)), hostOf(d1)) == 0.0);   // the same seed, the same mask
+  {
+    // against the CPU checker with the mask of this call: the seed is the generator's next draw
+    setSeed(77);
+    const unsigned long long seed = nextSeed();
+    setSeed(77);
+    Variable yd = drop(xd);
+    flref_rnn d{5, 4, 2, 0, (int32_t)RnnMode::GRU, 6, 3, 0.3f, (uint32_t)seed, (uint32_t)(seed >> 32)};
+    const std::vector<float> wv = hostOf(drop.param(0)), xv = hostOf(xd);
+    std::vector<float> y(4 * 3 * 6), hy(4 * 3 * 2), dxr(xv.size()), dhx(hy.size()), dwr(wv.size());
+    flref_rnn_fwd(&d, xv.data(), nullptr, nullptr, wv.data(), y.data(), hy.data(), nullptr);
+    CHECK(relL2(hostOf(yd), y) < 1e-5);
+    const std::vector<float> dy = randn(y.size(), 97);
+    flref_rnn_bwd(&d, xv.data(), nullptr, nullptr, wv.data(), dy.data(), nullptr, nullptr, dxr.data(), dhx.data(), nullptr,
+                  dwr.data());
+    xd.zeroGrad();
+    drop.zeroGrad();
+    yd.backward(Variable(Tensor::fromVector(yd.shape(), dy), false));
+    CHECK(relL2(hostOf(xd.grad()), dxr) < 1e-4);
+    CHECK(relL2(hostOf(drop.param(0).grad()), dwr) < 1e-4);
+  }
   drop.eval();
-  CHECK(drop(xin).shape() == Shape({4, 3, 6}));            // eval: no dropout (RNN.cpp:74)
+  Variable e1 = drop(xd), e2 = drop(xd);
+  CHECK(e1.shape() == Shape({4, 3, 6}) && maxAbsDiff(hostOf(e1), hostOf(e2)) == 0.0);   // eval: no dropout
+  CHECK(throws<std::invalid_argument>([&] { RNN bad(5, 4, 2, RnnMode::GRU, false, 1.0f); bad(xd); }));
 }
 
 // a crash of the host code should say where: unbuffered output and a backtrace

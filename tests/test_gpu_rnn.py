@@ -112,7 +112,60 @@ def test_rnn_errors():
     with pytest.raises(ValueError):
         ops.rnn(x, None, dev(np.zeros((1, 2, 5), np.float32)), w, 5, 1, ops.RNN_TANH, False)   # cell state without LSTM
     with pytest.raises(ValueError):
-        ops.rnn(x, None, None, w, 5, 1, ops.RNN_TANH, False, dropout=0.5)
+        ops.rnn(x, None, None, w, 5, 1, ops.RNN_TANH, False, dropout=1.5)   # not a probability
     y, hy, cy, reserve = ops.rnn(x, None, None, w, 5, 1, ops.RNN_TANH, False)
     with pytest.raises(ValueError):
         ops.rnn_backward(x, w, None, 5, 1, ops.RNN_TANH, False, y)           # no payload
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("I,H,L,bidir,T,B,p", [
+    (4, 3, 3, True, 5, 2, 0.5),            # the two-kernel steps
+    (10, 48, 2, True, 5, 33, 0.3),         # the fused step kernels
+    (40, 64, 3, False, 12, 8, 0.2),
+    (5, 7, 2, False, 3, 1, 0.7),
+])
+def test_rnn_dropout_between_layers(mode, I, H, L, bidir, T, B, p):
+    """Dropout on the output sequence of every layer but the last (backend/cudnn/RNN.cpp:83-90):
+    same mask (a function of the seed) and scale as the CPU checker, forward and backward;
+    another seed gives another result, one layer ignores the setting."""
+    rng = np.random.default_rng(2000 * mode + I + H + L + T)
+    D = 2 if bidir else 1
+    seed = 0xC0FFEE1234567
+    d = flref.rnn_desc(I, H, L, bidir, mode, T, B, dropout=p, seed=seed)
+    w = (rng.standard_normal(flref.rnn_param_count(d)) / np.sqrt(H)).astype(np.float32)
+    x = rng.standard_normal((T, B, I)).astype(np.float32)
+    hx = rng.standard_normal((L * D, B, H)).astype(np.float32)
+    cx = rng.standard_normal((L * D, B, H)).astype(np.float32) if mode == flref.RNN_LSTM else None
+    dy = rng.standard_normal((T, B, D * H)).astype(np.float32)
+    dhy = rng.standard_normal((L * D, B, H)).astype(np.float32)
+    dcy = rng.standard_normal((L * D, B, H)).astype(np.float32) if mode == flref.RNN_LSTM else None
+    ry, rhy, rcy = flref.rnn_fwd(d, x, w, hx, cx)
+    rdx, rdhx, rdcx, rdw = flref.rnn_bwd(d, x, w, hx, cx, dy, dhy, dcy)
+
+    o = lambda a: None if a is None else dev(a)
+    y, hy, cy, reserve = ops.rnn(dev(x), o(hx), o(cx), dev(w), H, L, mode, bidir, dropout=p, seed=seed)
+    assert rel_l2(host(y), ry) <= 1e-4 and rel_l2(host(hy), rhy) <= 1e-4
+    if mode == flref.RNN_LSTM:
+        assert rel_l2(host(cy), rcy) <= 1e-4
+    dx, dhx, dcx, dw = ops.rnn_backward(dev(x), dev(w), reserve, H, L, mode, bidir, dev(dy), dev(dhy), o(dcy),
+                                        dropout=p, seed=seed)
+    assert rel_l2(host(dx), rdx) <= 2e-4
+    assert rel_l2(host(dhx), rdhx) <= 2e-4
+    assert rel_l2(host(dw), rdw) <= 2e-4
+    if mode == flref.RNN_LSTM:
+        assert rel_l2(host(dcx), rdcx) <= 2e-4
+    y2 = ops.rnn(dev(x), o(hx), o(cx), dev(w), H, L, mode, bidir, dropout=p, seed=seed + 1)[0]
+    assert rel_l2(host(y2), ry) > 1e-3
+    y3 = ops.rnn(dev(x), o(hx), o(cx), dev(w), H, L, mode, bidir, dropout=p, seed=seed)[0]
+    assert torch.equal(y3, y)
+
+
+def test_rnn_dropout_needs_more_than_one_layer_and_a_valid_probability():
+    x = dev(np.zeros((3, 2, 4), np.float32))
+    w = dev(np.zeros(ops.rnn_param_count(4, 5, 1, flref.RNN_GRU, False), np.float32))
+    a = ops.rnn(x, None, None, w, 5, 1, flref.RNN_GRU, False)[0]
+    b = ops.rnn(x, None, None, w, 5, 1, flref.RNN_GRU, False, dropout=0.9, seed=3)[0]
+    assert torch.equal(a, b)
+    with pytest.raises(ValueError):
+        ops.rnn(x, None, None, w, 5, 1, flref.RNN_GRU, False, dropout=1.0)
