@@ -103,13 +103,15 @@ strip16_conv_kernel(Strip16Params p, const bf16_t* __restrict__ src, const bf16_
       out[2 * t + 1] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
     }
   };
-  // Source unit = (channel group, slab row, 8 columns), numbered columns first, then channel
-  // groups, then rows: a load instruction reads whole rows of 8 channels (runs of 16 x columns
-  // bytes) and its 16-byte stores spread evenly over the 16 bank groups (plane pitch = 1,
-  // 8 columns = 8 mod 16 cells).  The matrix waves take the first 256 units (slab rows 0 .. 4)
-  // and store them before the first barrier; the other waves request the later rows only when
-  // their weights have arrived (memory serves the early rows first) and store them while the
-  // matrix waves fetch their weight fragments.  Weights are requested first: they are needed first.
+  // Source unit = (channel group, 8 columns of a slab row).  The strip's rows of one channel are
+  // contiguous in memory (R + 2 rows x DW / 8 pieces of 16 bytes), so pieces are numbered t along
+  // that run and a lane takes (t % 2, channel group, t / 2): a load instruction reads pairs of
+  // adjacent pieces, 128 contiguous bytes per channel group and wave, and the 16-byte stores of 8
+  // consecutive lanes (2 pieces x 4 channel groups: +8 and +1 cells) fall in 8 different bank
+  // groups.  The matrix waves take the first 256 units (slab rows 0 .. 4) and store them before
+  // the first barrier; the other waves request the later rows only when their weights have
+  // arrived (memory serves the early rows first) and store them while the matrix waves fetch
+  // their weight fragments.  Weights are requested first: they are needed first.
   uint4 xv[8];
   int xl = ST_CG * XPL;
   {
@@ -119,9 +121,10 @@ strip16_conv_kernel(Strip16Params p, const bf16_t* __restrict__ src, const bf16_
     const int chan_bytes = DH * DW * 2;
     const int unit = tid < 256 ? tid + 256 : tid - 256;
     int xg = OOB;
-    if (unit < ST_CG * qrow * RS) {
-      const int t = (unit * p.qmagic) >> 16, q = unit - t * qrow;   // t = row * 8 + channel group
-      const int cg = t & 7, rs = t >> 3;
+    const int xt = 2 * (unit >> 4) + (unit & 1);
+    if (xt < qrow * RS) {
+      const int cg = (unit >> 1) & 7;
+      const int rs = (xt * p.qmagic) >> 16, q = xt - rs * qrow;
       const int sr = r0 - 1 + rs;
       xl = cg * XPL + rs * WSP + ST_XOFF + 8 * q;
       if ((unsigned)sr < (unsigned)DH)
@@ -172,15 +175,15 @@ strip16_conv_kernel(Strip16Params p, const bf16_t* __restrict__ src, const bf16_
       if (wave < 4) load_x();
     } else {
       // backward-data: memory is [contraction channel][(result channel, tap)]; unit =
-      // (channel group, 8 consecutive (result channel, tap) values), transposed like the slab;
-      // 8 consecutive units (one 128-byte line per channel) x 8 channel groups per wave
+      // (channel group, 8 consecutive (result channel, tap) values), transposed like the slab and
+      // numbered like the slab's units (pairs of adjacent pieces x channel groups)
       constexpr int EG = ST_BM * 9 / 8;     // 72 units per channel group
       const int cstride_bytes = p.a_cstride * 2;
       int wg[2], wl[2];
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         const int u = tid + ST_THREADS * i;
-        const int cg = (u >> 3) & 7, eg = (u >> 6) * 8 + (u & 7);
+        const int cg = (u >> 1) & 7, eg = 2 * (u >> 4) + (u & 1);
         wg[i] = OOB;
         wl[i] = ST_CG * APL;
         if (eg < EG) {

@@ -1024,6 +1024,30 @@ static void testRnn() {
     CHECK(relL2(hostOf(xd.grad()), dxr) < 1e-4);
     CHECK(relL2(hostOf(drop.param(0).grad()), dwr) < 1e-4);
   }
+  {
+    // 16-bit storage: the same call on bf16 tensors equals the fp32 call on the rounded values,
+    // rounded once more on the way out
+    const int I = 6, H = 8, L = 2, T = 5, B = 3;
+    const int64_t n = detail::getNumRnnParams(I, H, L, RnnMode::LSTM, true);
+    std::vector<float> wv = randn((size_t)n, 61, 0.3f), xv = randn((size_t)I * B * T, 62);
+    for (auto& f : wv) f = bf16round(f);
+    for (auto& f : xv) f = bf16round(f);
+    Variable x32(Tensor::fromVector({I, B, T}, xv), true), w32(Tensor::fromVector({(Dim)n}, wv), true);
+    Variable x16(x32.tensor().astype(dtype::bf16), true), w16(w32.tensor().astype(dtype::bf16), true);
+    Variable y32, h32, c32, y16, h16, c16;
+    std::tie(y32, h32, c32) = rnn(x32, Variable(), Variable(), w32, H, L, RnnMode::LSTM, true, 0.f);
+    std::tie(y16, h16, c16) = rnn(x16, Variable(), Variable(), w16, H, L, RnnMode::LSTM, true, 0.f);
+    CHECK(y16.type() == dtype::bf16 && h16.type() == dtype::bf16 && c16.type() == dtype::bf16);
+    CHECK(relL2(hostOf(Variable(y16.tensor().astype(dtype::f32), false)), hostOf(y32)) < 4e-3);
+    const std::vector<float> gy = randn((size_t)y32.elements(), 63);
+    std::vector<float> gyr = gy;
+    for (auto& f : gyr) f = bf16round(f);
+    y32.backward(Variable(Tensor::fromVector(y32.shape(), gyr), false));
+    y16.backward(Variable(Tensor::fromVector(y16.shape(), gyr).astype(dtype::bf16), false));
+    CHECK(x16.grad().type() == dtype::bf16 && w16.grad().type() == dtype::bf16);
+    CHECK(relL2(hostOf(Variable(x16.grad().tensor().astype(dtype::f32), false)), hostOf(x32.grad())) < 4e-3);
+    CHECK(relL2(hostOf(Variable(w16.grad().tensor().astype(dtype::f32), false)), hostOf(w32.grad())) < 4e-3);
+  }
   drop.eval();
   Variable e1 = drop(xd), e2 = drop(xd);
   CHECK(e1.shape() == Shape({4, 3, 6}) && maxAbsDiff(hostOf(e1), hostOf(e2)) == 0.0);   // eval: no dropout
