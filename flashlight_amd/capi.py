@@ -45,6 +45,7 @@ SYMBOLS = {
     "flhip_conv2d_workspace_bytes": (_SZ, [C.POINTER(ConvDesc), C.c_int]),
     "flhip_conv2d_fwd": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
     "flhip_conv2d_bwd_data": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _SZ, _VP]),
+    "flhip_conv2d_bwd_data_add": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
     "flhip_conv2d_bwd_filter": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
     "flhip_conv2d_bwd_filter_static": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _VP]),
     "flhip_pool2d_fwd": (C.c_int, [C.POINTER(PoolDesc), _VP, _VP, _VP, _VP]),

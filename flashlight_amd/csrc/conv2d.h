@@ -45,6 +45,8 @@ int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, c
 // taps, which gather the taps next to the channels (bwd = true in the query).
 int mfma_pointwise16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
                               hipStream_t s, void* ws = nullptr, size_t ws_bytes = 0);
+int mfma_pointwise16_conv_bwd_data_add(const ConvGeom& g, const void* dy, const void* w, const void* addend, void* dx,
+                                       hipStream_t s);
 int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s,
                                    void* ws = nullptr, size_t ws_bytes = 0);
 size_t mfma_pointwise16_lattice_ws(const ConvGeom& g, bool bwd);

@@ -291,6 +291,24 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
   return check_launch("conv2d_bwd_data");
 }
 
+extern "C" int flhip_conv2d_bwd_data_add(const flhip_conv_desc* d, const void* dy, const void* w,
+                                         const void* addend, void* dx, void* ws, size_t ws_bytes, void* stream) {
+  FLHIP_REQUIRE(d && dy && w && dx && addend, "conv2d_bwd_data_add: null argument");
+  ConvGeom g;
+  const int rc = make_geom(d, &g);
+  if (rc != FLHIP_OK) return rc;
+  hipStream_t s = as_stream(stream);
+  if (!force_direct() && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT)) {
+    const int r = mfma_pointwise16_conv_bwd_data_add(g, dy, w, addend, dx, s);
+    if (r >= 0) return r;
+  }
+  // every other kernel: the plain pass, then the element-wise sum (dx may not alias addend here)
+  FLHIP_REQUIRE(dx != addend, "conv2d_bwd_data_add: dx aliases addend");
+  const int r = flhip_conv2d_bwd_data(d, dy, w, dx, ws, ws_bytes, stream);
+  if (r != FLHIP_OK) return r;
+  return flhip_add(dx, addend, dx, (size_t)g.N * g.C * g.H * g.W, d->dtype, stream);
+}
+
 extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, const void* dy,
                                        float* dw, float* db, void* ws, size_t ws_bytes,
                                        void* stream) {

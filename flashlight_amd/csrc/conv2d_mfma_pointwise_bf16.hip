@@ -83,7 +83,16 @@ __device__ __forceinline__ uintx2_t merge_runs(uintx2_t a, uintx2_t b, int rem) 
   return uintx2_t{(uint32_t)v, (uint32_t)(v >> 32)};
 }
 
+// a + b on two bf16 values per dword, each sum rounded to bf16 (what an element-wise add of the
+// two tensors would give)
+__device__ __forceinline__ uint32_t add_bf16x2(uint32_t a, uint32_t b) {
+  return pack_bf16(__uint_as_float(a << 16) + __uint_as_float(b << 16),
+                   __uint_as_float(a & 0xffff0000u) + __uint_as_float(b & 0xffff0000u));
+}
+
 // BWD = false: forward (weights [Mo][Kc]); true: backward-data (weights [Kc][Mo]).
+// addend (or null): a tensor of the result's shape that is added to the rounded result (the
+// gradient a variable already holds, when this pass delivers its second one).
 // MT = 16-channel result tiles per workgroup (4: 64 result channels; 8 was measured and
 // is slower on every ResNet-50 layer, as is loading two chunks ahead instead of one).
 // ODD: planes that are not a multiple of 4 positions (at least 4).
@@ -94,7 +103,7 @@ __device__ __forceinline__ uintx2_t merge_runs(uintx2_t a, uintx2_t b, int rem) 
 template <bool BWD, int MT, bool ODD, int PF>
 __global__ void __launch_bounds__(256)
 pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __restrict__ wgt,
-                 const float* __restrict__ bias, bf16_t* __restrict__ dst) {
+                 const float* __restrict__ bias, bf16_t* __restrict__ dst, const bf16_t* __restrict__ addend) {
   constexpr int BM = MT * 16, WQ = BM / 64;      // result channels; 16-byte weight pieces per thread
   static_assert(!BWD || BM == 64, "the backward-data weight tile is [contraction][64 result channels]");
   static_assert(PB_KC * PB_WPB <= 64 * PB_WP, "both weight layouts share one buffer size");
@@ -290,15 +299,22 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
       bf16_t* dp = dst + (size_t)im * p.Mo * p.P + po;
       bf16_t* dp2 = dst + (size_t)(im + 1) * p.Mo * p.P - left;   // element e >= left: position e - left of the next image
       for (int ml = tid >> 5; ml < BM && m0 + ml < p.Mo; ml += 8) {
-        const uintx2_t v = *reinterpret_cast<const uintx2_t*>(&Ys[ml * YP + pc]);
+        uintx2_t v = *reinterpret_cast<const uintx2_t*>(&Ys[ml * YP + pc]);
         const size_t row = (size_t)(m0 + ml) * p.P;
         if (left >= 4) {
+          if (addend) {
+            const uintx2_t a = load8_any(addend + (dp - dst) + row);
+            v = uintx2_t{add_bf16x2(v.x, a.x), add_bf16x2(v.y, a.y)};
+          }
           store8_any(dp + row, v);
         } else {
           const uint32_t e4[4] = {v.x & 0xffffu, v.x >> 16, v.y & 0xffffu, v.y >> 16};
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            if (qo + e < p.Ptot) (e < left ? dp : dp2)[row + e] = (bf16_t)e4[e];
+            if (qo + e < p.Ptot) {
+              bf16_t* o = (e < left ? dp : dp2) + row + e;
+              *o = addend ? f32_to_bf16(bf16_to_f32((bf16_t)e4[e]) + bf16_to_f32(addend[o - dst])) : (bf16_t)e4[e];
+            }
         }
       }
     }
@@ -307,16 +323,28 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
     if (qo < p.Ptot) {
       const int im = qo / p.P, po = qo - im * p.P;
       bf16_t* dp = dst + (size_t)im * p.Mo * p.P + po;
-      for (int ml = tid >> 4; ml < BM && m0 + ml < p.Mo; ml += 16)
-        *reinterpret_cast<uintx4_t*>(dp + (size_t)(m0 + ml) * p.P) = *reinterpret_cast<const uintx4_t*>(&Ys[ml * YP + pc]);
+      for (int ml = tid >> 4; ml < BM && m0 + ml < p.Mo; ml += 16) {
+        uintx4_t v = *reinterpret_cast<const uintx4_t*>(&Ys[ml * YP + pc]);
+        if (addend) {
+          const uintx4_t a = *reinterpret_cast<const uintx4_t*>(addend + (dp - dst) + (size_t)(m0 + ml) * p.P);
+          v = uintx4_t{add_bf16x2(v.x, a.x), add_bf16x2(v.y, a.y), add_bf16x2(v.z, a.z), add_bf16x2(v.w, a.w)};
+        }
+        *reinterpret_cast<uintx4_t*>(dp + (size_t)(m0 + ml) * p.P) = v;
+      }
     }
   } else {
     const int pc = (tid & 31) * 4, qo = q0 + pc;
     if (qo < p.Ptot) {
       const int im = qo / p.P, po = qo - im * p.P;
       bf16_t* dp = dst + (size_t)im * p.Mo * p.P + po;
-      for (int ml = tid >> 5; ml < BM && m0 + ml < p.Mo; ml += 8)
-        *reinterpret_cast<uintx2_t*>(dp + (size_t)(m0 + ml) * p.P) = *reinterpret_cast<const uintx2_t*>(&Ys[ml * YP + pc]);
+      for (int ml = tid >> 5; ml < BM && m0 + ml < p.Mo; ml += 8) {
+        uintx2_t v = *reinterpret_cast<const uintx2_t*>(&Ys[ml * YP + pc]);
+        if (addend) {
+          const uintx2_t a = *reinterpret_cast<const uintx2_t*>(addend + (dp - dst) + (size_t)(m0 + ml) * p.P);
+          v = uintx2_t{add_bf16x2(v.x, a.x), add_bf16x2(v.y, a.y)};
+        }
+        *reinterpret_cast<uintx2_t*>(dp + (size_t)(m0 + ml) * p.P) = v;
+      }
     }
   }
 }
@@ -327,7 +355,8 @@ bool pw16_applies(const ConvGeom& g) {
 }
 
 template <bool BWD>
-int launch_pw16(const ConvGeom& g, const void* src, const void* w, const float* bias, void* dst, hipStream_t s) {
+int launch_pw16(const ConvGeom& g, const void* src, const void* w, const float* bias, void* dst, hipStream_t s,
+                const void* addend = nullptr) {
   Pw16Params p{};
   p.Kc = BWD ? g.K : g.C;
   p.Mo = BWD ? g.C : g.K;
@@ -348,7 +377,7 @@ int launch_pw16(const ConvGeom& g, const void* src, const void* w, const float* 
   const bool odd = p.P % 4 != 0;
   auto go = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), 0, s, p, static_cast<const bf16_t*>(src),
-                       static_cast<const bf16_t*>(w), bias, static_cast<bf16_t*>(dst));
+                       static_cast<const bf16_t*>(w), bias, static_cast<bf16_t*>(dst), static_cast<const bf16_t*>(addend));
   };
   if (odd) {
     if (deep) go(pw16_conv_kernel<BWD, 4, true, 4>);
@@ -999,6 +1028,16 @@ int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void
   }
   if (!pw16_applies(g)) return -1;
   return launch_pw16<true>(g, dy, w, nullptr, dx, s);
+}
+
+// dx = addend + backward-data, in the kernel's own result pass; -1 when this geometry's
+// backward-data pass is not the plain 1x1 kernel
+int mfma_pointwise16_conv_bwd_data_add(const ConvGeom& g, const void* dy, const void* w, const void* addend, void* dx,
+                                       hipStream_t s) {
+  ConvGeom c;
+  if (pw16_strided_plan(g, &c) || (!options().pw16_no_taps && pw16_taps_plan(g, &c)) || !pw16_applies(g)) return -1;
+  if (reinterpret_cast<uintptr_t>(addend) % 16 != 0) return -1;
+  return launch_pw16<true>(g, dy, w, nullptr, dx, s, addend);
 }
 
 size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g0) {

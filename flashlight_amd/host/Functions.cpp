@@ -159,9 +159,17 @@ Variable conv2d(const Variable& input, const Variable& weights, const Variable& 
     auto& wt = inputs[1];
     AutogradExtension& e = ext(in);
     if (in.isCalcGrad()) {
-      Tensor g = e.conv2dBackwardData(gradOutput.tensor(), in.tensor(), wt.tensor(), sx, sy, px, py,
-                                      dx, dy, groups, nullptr, payload);
-      in.addGrad(Variable(g, false));
+      auto* hip = detail::fusedGradAdd() ? dynamic_cast<HipAutogradExtension*>(&e) : nullptr;
+      if (hip && in.isGradAvailable() && in.grad().type() == gradOutput.type() && in.grad().shape() == in.shape()) {
+        // the second gradient of this variable (the first came down the shortcut): summed where
+        // the pass writes its result
+        in.replaceGrad(hip->conv2dBackwardDataAdd(gradOutput.tensor(), in.tensor(), wt.tensor(), in.grad().tensor(),
+                                                  sx, sy, px, py, dx, dy, groups));
+      } else {
+        Tensor g = e.conv2dBackwardData(gradOutput.tensor(), in.tensor(), wt.tensor(), sx, sy, px, py,
+                                        dx, dy, groups, nullptr, payload);
+        in.addGrad(Variable(g, false));
+      }
     }
     const bool biasGrad = hasBias && inputs.size() > 2 && inputs[2].isCalcGrad();
     if (wt.isCalcGrad() || biasGrad) {
@@ -222,6 +230,12 @@ Variable batchnorm(const Variable& input, const Variable& weight, const Variable
   };
   return Variable(output, {input, weight, bias}, gradFunc);
 }
+
+namespace {
+bool g_fusedGradAdd = true;
+}
+void detail::setFusedGradAdd(bool on) { g_fusedGradAdd = on; }
+bool detail::fusedGradAdd() { return g_fusedGradAdd; }
 
 Variable detail::batchnormRelu(const Variable& input, const Variable& weight, const Variable& bias,
                                Variable& runningMean, Variable& runningVar, const std::vector<int>& axes,

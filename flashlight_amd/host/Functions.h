@@ -49,6 +49,9 @@ class Variable {
   // the same as addGrad(astype).
   void addGradWide(const Tensor& grad);
   void zeroGrad() { grad_->grad.reset(); }
+  // the gradient accumulated so far is replaced by `sum` (an operation that added its own
+  // contribution to it in the pass that produced it)
+  void replaceGrad(const Tensor& sum) { grad_->grad.reset(new Variable(sum, false)); }
   void backward(const Variable& grad, bool retainGraph = false);
 
  private:
@@ -91,6 +94,11 @@ enum class ReduceMode { NONE = 0, MEAN = 1, SUM = 2 };
 Variable add(const Variable& lhs, const Variable& rhs);
 inline Variable operator+(const Variable& lhs, const Variable& rhs) { return add(lhs, rhs); }
 namespace detail {
+// Whether the backward-data pass of fl::conv2d adds the gradient its input already holds in the
+// pass that writes its result (HipAutogradExtension::conv2dBackwardDataAdd) instead of leaving
+// the sum to Variable::addGrad.  The values are the same bit for bit.  Default: on.
+void setFusedGradAdd(bool on);
+bool fusedGradAdd();
 // relu(batchnorm(input, ...) + residual) in train mode, residual optional (an empty Variable):
 // the tail of a ResNet block (flashlight/pkg/vision/models/Resnet.cpp:95-140).  On the HIP
 // extension with feature axes that do not start at dimension 0 this is one fused pass forward

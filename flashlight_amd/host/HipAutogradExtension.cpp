@@ -182,6 +182,33 @@ Tensor HipAutogradExtension::conv2dBackwardData(const Tensor& gradOutput, const 
   return gradInput;
 }
 
+Tensor HipAutogradExtension::conv2dBackwardDataAdd(const Tensor& gradOutput, const Tensor& input,
+                                                   const Tensor& weight, const Tensor& addend, const int sx,
+                                                   const int sy, const int px, const int py, const int dx,
+                                                   const int dy, const int groups) {
+  if (gradOutput.type() != weight.type() || addend.type() != gradOutput.type())
+    throw std::invalid_argument("conv2dBackwardDataAdd: gradOutput, weights and addend must have the same type");
+  if (addend.shape() != input.shape())
+    throw std::invalid_argument("conv2dBackwardDataAdd: addend must have the input's shape");
+  detail::OpScope scope("conv2dBackwardDataAdd");
+  const int tag = dtypeTag(gradOutput.type(), "conv2dBackwardDataAdd");
+  flhip_conv_desc d =
+      convDesc(input.shape(), weight, sx, sy, px, py, dx, dy, groups, tag, "conv2dBackwardDataAdd");
+  int32_t OH = 0, OW = 0;
+  check(flhip_conv2d_out_dims(&d, &OH, &OW));
+  if (gradOutput.shape() != Shape({OW, OH, d.K, d.N}))
+    throw std::invalid_argument("conv2dBackwardDataAdd: gradOutput shape does not match the geometry");
+  Tensor gradInput(input.shape(), gradOutput.type());
+  const size_t wsBytes = flhip_conv2d_workspace_bytes(&d, FLHIP_CONV_BWD_DATA);
+  Tensor ws = workspace(wsBytes);
+  DevicePtr gp(gradOutput), wp(weight), ap(addend), op(gradInput), wsp(ws);
+  check(flhip_conv2d_bwd_data_add(&d, gp.get(), wp.get(), ap.get(), op.get(), wsp.get(), wsBytes,
+                                  hipBackendStream()));
+  // event: inputs {gradOutput, weights, addend}, outputs {gradInput}, ints as conv2d
+  if (scope.on()) scope.done({gradOutput, weight, addend}, {gradInput}, {sx, sy, px, py, dx, dy, groups});
+  return gradInput;
+}
+
 std::pair<Tensor, Tensor> HipAutogradExtension::conv2dBackwardFilterBias(
     const Tensor& gradOutput, const Tensor& input, const Tensor& weights, const Tensor& bias,
     const int sx, const int sy, const int px, const int py, const int dx, const int dy,

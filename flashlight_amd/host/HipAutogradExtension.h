@@ -62,6 +62,11 @@ class HipAutogradExtension : public AutogradExtension {
                        const Tensor& bias, Tensor& runningMean, Tensor& runningVar,
                        const std::vector<int>& axes, const double momentum, const double epsilon,
                        const Tensor& residual, std::shared_ptr<detail::AutogradPayload> payload);
+  // addend + conv2dBackwardData(...): the closure's backward-data pass and the addGrad behind it
+  // in one pass over the result (flhip_conv2d_bwd_data_add)
+  Tensor conv2dBackwardDataAdd(const Tensor& gradOutput, const Tensor& input, const Tensor& weights,
+                               const Tensor& addend, const int sx, const int sy, const int px, const int py,
+                               const int dx, const int dy, const int groups);
   std::tuple<Tensor, Tensor, Tensor, Tensor> batchnormReluBackward(
       const Tensor& gradOutput, const Tensor& output, const Tensor& saveMean, const Tensor& saveVar,
       const Tensor& input, const Tensor& weight, const std::vector<int>& axes, const bool wantResidualGrad,

@@ -32,7 +32,8 @@ std::vector<float> randn(size_t n, unsigned seed) {
 // operation name -> class of the breakdown
 const char* classOf(const std::string& op) {
   static const std::map<std::string, const char*> m = {
-      {"conv2d", "conv_fwd"}, {"conv2dBackwardData", "conv_bwd_data"}, {"conv2dBackwardFilterBias", "conv_bwd_filter"},
+      {"conv2d", "conv_fwd"}, {"conv2dBackwardData", "conv_bwd_data"}, {"conv2dBackwardDataAdd", "conv_bwd_data"},
+      {"conv2dBackwardFilterBias", "conv_bwd_filter"},
       {"batchnorm", "bn_fwd"}, {"batchnormBackward", "bn_bwd"}, {"batchnormRelu", "bn_fwd"}, {"batchnormReluBackward", "bn_bwd"},
       {"pool2d", "pool_fwd"}, {"pool2dBackward", "pool_bwd"},
       {"relu", "relu_add"}, {"reluBackward", "relu_add"}, {"add", "relu_add"}, {"addGrad", "relu_add"},
@@ -53,6 +54,7 @@ int main(int argc, char** argv) {
     const bool half = argc > 5 && std::string(argv[5]) == "bf16";
     const bool unfused = argc > 6 && std::string(argv[6]) == "unfused";
     pkg::vision::setFusedBatchNormRelu(!unfused);
+    detail::setFusedGradAdd(!unfused);
     setSeed(3);
 
     std::function<float()> step;

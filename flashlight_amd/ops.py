@@ -103,9 +103,10 @@ def conv2d(input, weights, bias, sx=1, sy=1, px=0, py=0, dx=1, dy=1, groups=1):
 
 
 def conv2d_backward_data(grad_output, input_shape, weights, sx=1, sy=1, px=0, py=0, dx=1, dy=1,
-                         groups=1):
+                         groups=1, addend=None):
     """AutogradExtension::conv2dBackwardData; only the input's shape is needed
-    (onednn/Conv2D.cpp:285)."""
+    (onednn/Conv2D.cpp:285).  addend: a gradient the input already holds; the result is then
+    addend + the pass's result (Variable::addGrad), in one pass where the kernel allows it."""
     g, w = _dev(grad_output, "gradOutput"), _dev(weights, "weights")
     tag = _dtype_tag(g)
     d = _conv_desc(tuple(input_shape), w.shape, sx, sy, px, py, dx, dy, groups, tag)
@@ -116,6 +117,13 @@ def conv2d_backward_data(grad_output, input_shape, weights, sx=1, sy=1, px=0, py
     out = torch.empty(tuple(input_shape), dtype=g.dtype, device=g.device)
     nws = capi.lib().flhip_conv2d_workspace_bytes(C.byref(d), capi.CONV_BWD_DATA)
     ws = _ws(nws, g.device)
+    if addend is not None:
+        a = _dev(addend, "addend")
+        if tuple(a.shape) != tuple(input_shape) or a.dtype != g.dtype:
+            raise ValueError("conv2dBackwardData: addend must have the input's shape and the gradient's type")
+        capi.check(capi.lib().flhip_conv2d_bwd_data_add(C.byref(d), _ptr(g), _ptr(w), _ptr(a), _ptr(out),
+                                                        _ptr(ws), nws, _stream()))
+        return out
     capi.check(capi.lib().flhip_conv2d_bwd_data(C.byref(d), _ptr(g), _ptr(w), _ptr(out),
                                                 _ptr(ws), nws, _stream()))
     return out

@@ -145,6 +145,17 @@ int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy,
                           const void* w, void* dx, void* ws, size_t ws_bytes,
                           void* stream);
 
+/* dx = addend + conv2dBackwardData(dy, w): the backward-data pass of the conv2d closure
+ * (flashlight/fl/autograd/Functions.cpp:1362-1389) followed by Variable::addGrad
+ * (Variable.cpp:185-218) when the input already holds a gradient (the shortcut's, at the head
+ * of a residual block), in one pass over dx where the kernel allows it (bf16 1x1 stride 1;
+ * everything else runs the two operations).  Both terms are rounded to the storage type
+ * before the sum, so the result equals the two separate calls bit for bit.  addend has dx's
+ * shape and type; dx must not alias it. */
+int flhip_conv2d_bwd_data_add(const flhip_conv_desc* d, const void* dy, const void* w,
+                              const void* addend, void* dx, void* ws, size_t ws_bytes,
+                              void* stream);
+
 /* AutogradExtension::conv2dBackwardFilterBias (AutogradExtension.h:124-138;
  * oneDNN peer onednn/Conv2D.cpp:377-507): dw (fp32, weight shape) and, when db
  * is not NULL, db[k] = sum of dy over n, oh, ow (fp32).  dw may be NULL to get

@@ -149,6 +149,14 @@ class OracleChecker : public detail::OpObserver {
       std::vector<float> dx((size_t)out[0].elements());
       flref_conv2d_bwd_data(&d, dy.data(), w.data(), dx.data());
       cmp(op, out[0], dx);
+    } else if (op == "conv2dBackwardDataAdd") {
+      // the pass's result and the gradient the input already held, each in the storage type, summed
+      const flref_conv d = convGeom(out[0].shape(), in[1].shape(), e.ints);
+      const auto dy = host(in[0]), w = host(in[1]), add = host(in[2]);
+      std::vector<float> dx((size_t)out[0].elements());
+      flref_conv2d_bwd_data(&d, dy.data(), w.data(), dx.data());
+      for (size_t i = 0; i < dx.size(); ++i) dx[i] += add[i];
+      cmp(op, out[0], dx);
     } else if (op == "conv2dBackwardFilterBias") {
       const flref_conv d = convGeom(in[1].shape(), out[0].shape(), e.ints);
       const auto dy = host(in[0]), x = host(in[1]);
@@ -338,6 +346,7 @@ int main(int argc, char** argv) {
     for (int pass = 0; pass < 3; ++pass) {
       const bool half = pass >= 1;
       pkg::vision::setFusedBatchNormRelu(pass < 2);
+      detail::setFusedGradAdd(pass < 2);
       setSeed(3);
       auto model = pkg::vision::resnet50();
       const auto params = model->params();
@@ -375,7 +384,8 @@ int main(int argc, char** argv) {
       }
       std::printf("  %ld results checked against the CPU checker\n", ops);
       for (const char* need : {"conv2d", "conv2dBackwardData", "conv2dBackwardFilterBias dw", "pool2d values", "pool2dBackward",
-                               pass < 2 ? "batchnormRelu y" : "batchnorm y", pass < 2 ? "batchnormReluBackward dx" : "relu"}) {
+                               pass < 2 ? "batchnormRelu y" : "batchnorm y", pass < 2 ? "batchnormReluBackward dx" : "relu",
+                               pass < 2 ? "conv2dBackwardDataAdd" : "addGrad"}) {
         bool seen = false;
         for (const auto& kv : checker.stats) seen = seen || kv.first.rfind(need, 0) == 0;
         if (!seen) { std::printf("FAILED: no %s in the step\n", need); ++fail; }
@@ -400,6 +410,7 @@ int main(int argc, char** argv) {
         ++fail;
       }
     pkg::vision::setFusedBatchNormRelu(true);
+    detail::setFusedGradAdd(true);
     std::printf(fail ? "%d check(s) FAILED\n" : "ResNet-50 step checks passed\n", fail);
     std::fflush(stdout);
     return fail ? 1 : 0;

@@ -186,6 +186,30 @@ def test_conv_bf16_with_family_switched_off(family, case):
         capi.set_option("CONV_SKIP", None)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [
+    ((3, 72, 14, 16), (40, 72, 1, 1), (1, 1), (0, 0)),     # bf16: the 1x1 kernel's own result pass, 16-byte pieces
+    ((2, 64, 6, 6), (136, 64, 1, 1), (1, 1), (0, 0)),      # planes of 36 positions: 8-byte pieces
+    ((5, 64, 7, 7), (64, 64, 1, 1), (1, 1), (0, 0)),       # planes of 49: runs that cross into the next image
+    ((2, 32, 9, 9), (48, 32, 3, 3), (1, 1), (1, 1)),       # every other kernel: the pass, then the sum
+    ((2, 64, 14, 14), (64, 64, 1, 1), (2, 2), (0, 0)),     # strided 1x1: through the workspace, then the sum
+])
+def test_backward_data_add_equals_the_two_operations(shape, dtype):
+    """flhip_conv2d_bwd_data_add = conv2dBackwardData followed by Variable::addGrad, bit for bit."""
+    xs, ws_, st, pd = shape
+    rng = np.random.default_rng(41)
+    w = dev((rng.standard_normal(ws_) / np.sqrt(ws_[1] * ws_[2] * ws_[3])).astype(np.float32), dtype)
+    oh = (xs[2] + 2 * pd[0] - ws_[2]) // st[0] + 1
+    ow = (xs[3] + 2 * pd[1] - ws_[3]) // st[1] + 1
+    dy = dev(rng.standard_normal((xs[0], ws_[0], oh, ow)).astype(np.float32), dtype)
+    held = dev(rng.standard_normal(xs).astype(np.float32), dtype)
+    kw = dict(sx=st[1], sy=st[0], px=pd[1], py=pd[0])
+    plain = fa.conv2d_backward_data(dy, xs, w, **kw)
+    fused = fa.conv2d_backward_data(dy, xs, w, addend=held, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(fused, plain + held)
+
+
 def test_bias_gradient_alone_and_empty_bias():
     # the caller passes an empty bias when its gradient is not needed
     # (flashlight/fl/autograd/Functions.cpp:1391-1395)
