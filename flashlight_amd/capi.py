@@ -63,6 +63,7 @@ SYMBOLS = {
                                     _SZ, _VP]),
     "flhip_copy_bytes": (C.c_int, [_VP, _VP, _SZ, _VP]),
     "flhip_convert": (C.c_int, [_VP, C.c_int, _VP, C.c_int, _SZ, _VP]),
+    "flhip_convert_many": (C.c_int, [C.POINTER(_VP), C.POINTER(_VP), C.POINTER(_SZ), C.c_int, C.c_int, C.c_int, _VP]),
     "flhip_fill": (C.c_int, [_VP, C.c_double, _SZ, C.c_int, _VP]),
     "flhip_add": (C.c_int, [_VP, _VP, _VP, _SZ, C.c_int, _VP]),
     "flhip_relu_fwd": (C.c_int, [_VP, _VP, _SZ, C.c_int, _VP]),

@@ -107,6 +107,35 @@ __global__ void __launch_bounds__(256) convert_kernel(const S* __restrict__ src,
     st(dst, i, ld(src, i));
 }
 
+// Several conversions in one launch: up to CM_MAX (source, destination, length) triples travel in
+// the kernel arguments; workgroup b works on the triple whose range of 2048-element pieces
+// contains b.
+constexpr int CM_MAX = 64;
+struct ConvertMany {
+  const void* src[CM_MAX];
+  void* dst[CM_MAX];
+  unsigned first[CM_MAX + 1];   // first piece of entry i; first[count] = pieces in all
+  unsigned long long n[CM_MAX];
+  int count;
+};
+template <typename S, typename D>
+__global__ void __launch_bounds__(256) convert_many_kernel(ConvertMany a) {
+  int lo = 0, hi = a.count;          // the entry with first[e] <= blockIdx.x < first[e + 1]
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (a.first[mid] <= blockIdx.x) lo = mid; else hi = mid;
+  }
+  const S* src = static_cast<const S*>(a.src[lo]);
+  D* dst = static_cast<D*>(a.dst[lo]);
+  const size_t base = (size_t)(blockIdx.x - a.first[lo]) * 2048;
+  const size_t n = a.n[lo];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const size_t i = base + (size_t)k * 256 + threadIdx.x;
+    if (i < n) st(dst, i, ld(src, i));
+  }
+}
+
 template <typename D>
 __global__ void __launch_bounds__(256) fill_kernel(D* __restrict__ dst, float value, size_t n) {
   const size_t stride = (size_t)gridDim.x * 256;
@@ -201,6 +230,40 @@ extern "C" int flhip_convert(const void* src, int src_dtype, void* dst, int dst_
   else
     hipLaunchKernelGGL((convert_kernel<bf16_t, bf16_t>), grid, block, 0, s, (const bf16_t*)src, (bf16_t*)dst, n);
   return check_launch("convert");
+}
+
+extern "C" int flhip_convert_many(const void* const* src, void* const* dst, const size_t* n, int count,
+                                  int src_dtype, int dst_dtype, void* stream) {
+  FLHIP_REQUIRE(dtype_ok(src_dtype) && dtype_ok(dst_dtype), "convert_many: unknown dtype");
+  FLHIP_REQUIRE(count >= 0 && (count == 0 || (src && dst && n)), "convert_many: null argument");
+  hipStream_t s = as_stream(stream);
+  for (int i0 = 0; i0 < count; i0 += CM_MAX) {
+    ConvertMany a{};
+    unsigned pieces = 0;
+    for (int i = i0; i < count && i < i0 + CM_MAX; ++i) {
+      if (n[i] == 0) continue;
+      FLHIP_REQUIRE(src[i] && dst[i], "convert_many: null pointer");
+      FLHIP_REQUIRE(n[i] < (1ull << 40), "convert_many: tensor too large");
+      a.src[a.count] = src[i];
+      a.dst[a.count] = dst[i];
+      a.n[a.count] = n[i];
+      a.first[a.count] = pieces;
+      pieces += (unsigned)((n[i] + 2047) / 2048);
+      ++a.count;
+    }
+    if (a.count == 0) continue;
+    a.first[a.count] = pieces;
+    const dim3 grid(pieces), block(256);
+    if (src_dtype == FLHIP_F32 && dst_dtype == FLHIP_F32)
+      hipLaunchKernelGGL((convert_many_kernel<float, float>), grid, block, 0, s, a);
+    else if (src_dtype == FLHIP_F32)
+      hipLaunchKernelGGL((convert_many_kernel<float, bf16_t>), grid, block, 0, s, a);
+    else if (dst_dtype == FLHIP_F32)
+      hipLaunchKernelGGL((convert_many_kernel<bf16_t, float>), grid, block, 0, s, a);
+    else
+      hipLaunchKernelGGL((convert_many_kernel<bf16_t, bf16_t>), grid, block, 0, s, a);
+  }
+  return check_launch("convert_many");
 }
 
 extern "C" int flhip_fill(void* dst, double value, size_t n, int dtype, void* stream) {

@@ -340,6 +340,30 @@ def batchnorm_relu_backward(grad_output, input, output, weight, save_mean, save_
 # Flashlight shape reversed (same memory).  A Flashlight [features, batch] matrix is a
 # torch [batch, features] tensor.
 
+def astype(input, dtype):
+    """Tensor::astype between fp32 and bf16 (round to nearest even)."""
+    x = _dev(input, "input")
+    out = torch.empty_like(x, dtype=dtype)
+    capi.check(capi.lib().flhip_convert(_ptr(x), _dtype_tag(x), _ptr(out), _dtype_tag(out), x.numel(), _stream()))
+    return out
+
+
+def astype_many(inputs, dtype):
+    """The same conversion of a list of tensors of one type, in one launch per 64 of them."""
+    xs = [_dev(t, "input") for t in inputs]
+    if not xs:
+        return []
+    if any(x.dtype != xs[0].dtype for x in xs):
+        raise ValueError("astype_many: the tensors must share a type")
+    outs = [torch.empty_like(x, dtype=dtype) for x in xs]
+    n = len(xs)
+    src = (C.c_void_p * n)(*[x.data_ptr() for x in xs])
+    dst = (C.c_void_p * n)(*[o.data_ptr() for o in outs])
+    cnt = (C.c_size_t * n)(*[x.numel() for x in xs])
+    capi.check(capi.lib().flhip_convert_many(src, dst, cnt, n, _dtype_tag(xs[0]), _dtype_tag(outs[0]), _stream()))
+    return outs
+
+
 def relu(input):
     """fl::relu (Functions.cpp:1787-1789)."""
     x = _dev(input, "input")

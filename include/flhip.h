@@ -254,6 +254,13 @@ int flhip_bn_act_bwd(const flhip_bn_desc* d, const void* x, const void* dy, cons
  * and FL_ADJUST_INPUT_TYPE, flashlight/fl/autograd/Functions.h:57-82). */
 int flhip_convert(const void* src, int src_dtype, void* dst, int dst_dtype,
                   size_t n, void* stream);
+/* The same conversion of `count` tensors (src[i] -> dst[i], n[i] elements; host arrays of device
+ * pointers) in one launch per 64 of them: the per-step casts of a network's fp32 master weights
+ * to the storage type of its activations (the astype calls of Conv2D / Linear::forward,
+ * flashlight/fl/nn/modules/Conv2D.cpp:157-176, Linear.cpp:60-72) are dozens of tensors of a few
+ * kilobytes to megabytes, each a launch of its own otherwise. */
+int flhip_convert_many(const void* const* src, void* const* dst, const size_t* n, int count,
+                       int src_dtype, int dst_dtype, void* stream);
 
 /* dst[i] = value for n elements of `dtype`: fl::full as the extension uses it for
  * default running statistics (onednn/BatchNorm.cpp:116-122), enqueued like every other

@@ -283,3 +283,19 @@ def test_mnist_convnet_training_step(B):
     got = dict(w1=dw1, b1=db1, w2=dw2, b2=db2, w3=dw3, b3=db3, w4=dw4, b4=db4)
     for k in sorted(R):
         assert rel_l2(host(got[k]), R[k]) <= 1e-4, (k, rel_l2(host(got[k]), R[k]))
+
+
+def test_astype_many_equals_astype():
+    """flhip_convert_many: every tensor converted as flhip_convert would, whatever its length
+    (empty, shorter than a piece of 2048 elements, several pieces), more tensors than fit in one launch."""
+    rng = np.random.default_rng(77)
+    sizes = [0, 1, 7, 2047, 2048, 2049, 5000, 64 * 64 * 9, 100003] + [int(v) for v in rng.integers(1, 9000, 70)]
+    xs = [dev(rng.standard_normal(n).astype(np.float32)) for n in sizes]
+    many = ops.astype_many(xs, torch.bfloat16)
+    for x, m in zip(xs, many):
+        assert m.dtype == torch.bfloat16 and torch.equal(m, ops.astype(x, torch.bfloat16))
+        assert torch.equal(m, x.to(torch.bfloat16))           # round to nearest even
+    back = ops.astype_many(many, torch.float32)
+    for m, b in zip(many, back):
+        assert torch.equal(b, m.float())
+    assert ops.astype_many([], torch.bfloat16) == []
