@@ -4,6 +4,7 @@
 
 #include <algorithm>
 #include <tuple>
+#include <unordered_map>
 #include <unordered_set>
 
 #include "flhip.h"
@@ -65,15 +66,55 @@ void Variable::setCalcGrad(bool calcGrad) {
   }
 }
 
-Variable Variable::astype(dtype newType) const {
-  if (newType == type()) return *this;
+namespace {
+struct ParamCasts {
+  dtype to;
+  std::unordered_map<const void*, Variable> nodes;
+};
+ParamCasts* g_paramCasts = nullptr;
+}  // namespace
+
+detail::ParamCastScope::ParamCastScope(const std::vector<Variable>& params, dtype to) {
+  if (g_paramCasts) return;   // an outer scope made the casts
+  std::vector<Variable> todo;
+  std::vector<Tensor> src;
+  std::unordered_set<const void*> seen;
+  for (const auto& p : params)
+    if (!p.isEmpty() && p.type() != to && seen.insert(p.id()).second) {
+      todo.push_back(p);
+      src.push_back(p.tensor());
+    }
+  if (todo.empty()) return;
+  const std::vector<Tensor> converted = Tensor::astypeMany(src, to);
+  auto* casts = new ParamCasts{to, {}};
+  for (size_t i = 0; i < todo.size(); ++i) casts->nodes.emplace(todo[i].id(), todo[i].castNode(converted[i]));
+  g_paramCasts = casts;
+  owner_ = true;
+}
+
+detail::ParamCastScope::~ParamCastScope() {
+  if (!owner_) return;
+  delete g_paramCasts;
+  g_paramCasts = nullptr;
+}
+
+Variable Variable::castNode(const Tensor& converted) const {
   const dtype oldType = type();
   auto gradFunc = [oldType](std::vector<Variable>& inputs, const Variable& gradOutput) {
     inputs[0].addGrad(Variable(gradOutput.tensor().astype(oldType), false));
   };
-  Variable out(tensor().astype(newType), {*this}, gradFunc);
+  Variable out(converted, {*this}, gradFunc);
   out.grad_->isCast = out.grad_->calcGrad;
   return out;
+}
+
+Variable Variable::astype(dtype newType) const {
+  if (newType == type()) return *this;
+  if (g_paramCasts && g_paramCasts->to == newType) {
+    const auto it = g_paramCasts->nodes.find(id());
+    if (it != g_paramCasts->nodes.end()) return it->second;
+  }
+  return castNode(tensor().astype(newType));
 }
 
 void Variable::addGradWide(const Tensor& grad) {

@@ -37,6 +37,11 @@ class Variable {
   void setCalcGrad(bool calcGrad);
   // differentiable cast (Variable.cpp:100-108); f32 <-> bf16 here
   Variable astype(dtype type) const;
+  // the cast node of this variable around a conversion that was made elsewhere (one of many in
+  // one launch): same graph node as astype() builds
+  Variable castNode(const Tensor& converted) const;
+  // identity of the variable's shared state (copies of a Variable share it)
+  const void* id() const { return grad_.get(); }
   bool isGradAvailable() const { return grad_->grad != nullptr; }
   Variable& grad() const;
   void addGrad(const Variable& childGrad);
@@ -94,6 +99,20 @@ enum class ReduceMode { NONE = 0, MEAN = 1, SUM = 2 };
 Variable add(const Variable& lhs, const Variable& rhs);
 inline Variable operator+(const Variable& lhs, const Variable& rhs) { return add(lhs, rhs); }
 namespace detail {
+// While a ParamCastScope is alive, Variable::astype(to) of the variables it was given returns the
+// cast node the scope made for it: all of them converted in one launch (Tensor::astypeMany)
+// instead of one launch per module and step.  Nested scopes do nothing; the outermost one owns
+// the nodes and drops them when it ends (the graph keeps the ones it uses).
+class ParamCastScope {
+ public:
+  ParamCastScope(const std::vector<Variable>& params, dtype to);
+  ~ParamCastScope();
+  ParamCastScope(const ParamCastScope&) = delete;
+  ParamCastScope& operator=(const ParamCastScope&) = delete;
+
+ private:
+  bool owner_ = false;
+};
 // Whether the backward-data pass of fl::conv2d adds the gradient its input already holds in the
 // pass that writes its result (HipAutogradExtension::conv2dBackwardDataAdd) instead of leaving
 // the sum to Variable::addGrad.  The values are the same bit for bit.  Default: on.

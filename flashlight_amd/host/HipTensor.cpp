@@ -246,6 +246,35 @@ Tensor Tensor::astype(dtype t) const {
   return out;
 }
 
+std::vector<Tensor> Tensor::astypeMany(const std::vector<Tensor>& in, dtype t) {
+  std::vector<Tensor> out(in.size());
+  std::vector<const void*> src;
+  std::vector<void*> dst;
+  std::vector<size_t> n;
+  std::vector<Tensor> evIn, evOut;
+  int from = -1;
+  for (size_t i = 0; i < in.size(); ++i) {
+    if (in[i].isEmpty() || in[i].type() == t) {
+      out[i] = in[i].astype(t);
+      continue;
+    }
+    if (from >= 0 && tag(in[i].type()) != from) throw std::invalid_argument("astypeMany: the tensors must share a type");
+    from = tag(in[i].type());
+    out[i] = Tensor(in[i].shape(), t);
+    src.push_back(in[i].device());
+    dst.push_back(out[i].device());
+    n.push_back((size_t)in[i].elements());
+    evIn.push_back(in[i]);
+    evOut.push_back(out[i]);
+  }
+  if (src.empty()) return out;
+  detail::OpScope scope("astype");
+  const int rc = flhip_convert_many(src.data(), dst.data(), n.data(), (int)src.size(), from, tag(t), g_stream);
+  if (rc != FLHIP_OK) throw std::runtime_error(flhip_last_error());
+  if (scope.on()) scope.done(evIn, evOut);   // pairs: inputs[i] -> outputs[i]
+  return out;
+}
+
 Tensor Tensor::reshaped(const Shape& s) const {
   if (s.elements() != shape_.elements()) throw std::invalid_argument("reshape: element count differs");
   Tensor r = *this;

@@ -39,6 +39,9 @@ class Tensor {
 
   // Tensor::astype for f32 <-> bf16; other conversions are not part of this path.
   Tensor astype(dtype t) const;
+  // the same conversion of several tensors of one type in one launch per 64 of them
+  // (flhip_convert_many); tensors that already have type t come back as they are
+  static std::vector<Tensor> astypeMany(const std::vector<Tensor>& in, dtype t);
   // same buffer, different shape (fl::reshape / moddims)
   Tensor reshaped(const Shape& s) const;
   // a + b elementwise (Variable::addGrad, flashlight/fl/autograd/Variable.cpp:185-218)

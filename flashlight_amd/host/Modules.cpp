@@ -1,5 +1,7 @@
 #include "Modules.h"
 
+#include <memory>
+
 #include "flhip.h"
 
 #include <algorithm>
@@ -121,13 +123,29 @@ void Container::setParams(const Variable& var, int position) {
     if (c.position == position) modules_[c.module]->setParams(var, c.index);
 }
 
+std::vector<Variable> Container::castParams() const {
+  std::vector<Variable> all;
+  for (const auto& m : modules_) {
+    const auto p = m->castParams();
+    all.insert(all.end(), p.begin(), p.end());
+  }
+  return all;
+}
+
 std::vector<Variable> Sequential::forward(const std::vector<Variable>& inputs) {
+  // activations in another type than the fp32 parameters: every module's casts in one launch
+  std::unique_ptr<detail::ParamCastScope> casts;
+  if (!inputs.empty() && !inputs[0].isEmpty() && inputs[0].type() != dtype::f32)
+    casts.reset(new detail::ParamCastScope(castParams(), inputs[0].type()));
   auto output = inputs;
   for (auto& m : modules_) output = m->forward(output);
   return output;
 }
 
 Variable Sequential::forward(const Variable& input) {
+  std::unique_ptr<detail::ParamCastScope> casts;
+  if (!input.isEmpty() && input.type() != dtype::f32)
+    casts.reset(new detail::ParamCastScope(castParams(), input.type()));
   std::vector<Variable> output = {input};
   for (auto& m : modules_) output = m->forward(output);
   if (output.size() != 1) throw std::invalid_argument("Module output size is not 1");

@@ -46,6 +46,9 @@ class Module {
   virtual std::vector<Variable> forward(const std::vector<Variable>& inputs) = 0;
   std::vector<Variable> operator()(const std::vector<Variable>& inputs) { return forward(inputs); }
   virtual std::string prettyString() const = 0;
+  // the parameters this module converts to its input's type in forward() (astype); containers
+  // convert them for all their modules at once (detail::ParamCastScope)
+  virtual std::vector<Variable> castParams() const { return {}; }
 
  protected:
   Module() = default;
@@ -97,6 +100,7 @@ class Container : public Module {
   void train() override;
   void eval() override;
   void setParams(const Variable& var, int position) override;
+  std::vector<Variable> castParams() const override;
 
  protected:
   struct ChildParam {
@@ -136,6 +140,7 @@ class Conv2D : public UnaryModule {
   using UnaryModule::forward;
   Variable forward(const Variable& input) override;
   std::string prettyString() const override;
+  std::vector<Variable> castParams() const override { return params_; }
 
  private:
   int nIn_, nOut_, xFilter_, yFilter_, xStride_, yStride_, xPad_, yPad_, xDilation_, yDilation_;
@@ -214,6 +219,7 @@ class Linear : public UnaryModule {
   using UnaryModule::forward;
   Variable forward(const Variable& input) override;
   std::string prettyString() const override;
+  std::vector<Variable> castParams() const override { return params_; }
 
  private:
   int nIn_, nOut_;
@@ -237,6 +243,7 @@ class RNN : public Module {
   std::tuple<Variable, Variable, Variable> forward(const Variable& input, const Variable& hiddenState,
                                                    const Variable& cellState);
   std::string prettyString() const override;
+  std::vector<Variable> castParams() const override { return params_; }
 
  private:
   int inputSize_, hiddenSize_, numLayers_;

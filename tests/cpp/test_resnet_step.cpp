@@ -252,8 +252,11 @@ class OracleChecker : public detail::OpObserver {
       // one fp32 addition, rounded once to the storage type: exact in both
       same(op, host(out[0]), out[0].type() == dtype::bf16 ? toBf16(c) : c);
     } else if (op == "astype") {
-      const auto a = host(in[0]);
-      same(op, host(out[0]), out[0].type() == dtype::bf16 ? toBf16(a) : a);
+      // one conversion or several in one launch: inputs[i] -> outputs[i]
+      for (size_t i = 0; i < in.size() && i < out.size(); ++i) {
+        const auto a = host(in[i]);
+        same(op, host(out[i]), out[i].type() == dtype::bf16 ? toBf16(a) : a);
+      }
     } else if (op == "linear") {
       const int M = (int)e.ints[0], K = (int)e.ints[1], N = (int)e.ints[2];
       const auto x = host(in[0]), w = host(in[1]), b = host(in[2]);
