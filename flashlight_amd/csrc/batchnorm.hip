@@ -353,6 +353,16 @@ constexpr int RES_KL = 9;             // dy vectors per thread parked in LDS (9 
 constexpr int RES_MIN_C_FWD = 64;     // fewer features leave too many CUs idle
 constexpr int RES_MIN_C_BWD = 128;
 
+// Feature of this workgroup in the resident kernels (one workgroup per feature).  Workgroups go to
+// the 8 XCDs in turn; numbering features so that XCD x gets the contiguous range
+// [x * C / 8, (x + 1) * C / 8) keeps the cache lines that neighbouring features share - rows of 98
+// or 392 bytes on 7x7 / 14x14 planes start and end inside a line - in ONE XCD's L2 instead of
+// fetching them into two.
+__device__ __forceinline__ int res_feature(const BnGeom& g) {
+  const int b = blockIdx.x, C = (int)g.C;
+  return (C & 7) ? b : (b & 7) * (C >> 3) + (b >> 3);
+}
+
 // Walks this thread's vectors q = tid + 1024*k: f(k, byte offset, in range).  The
 // offset is relative to the tensor base and goes through a buffer descriptor; slots
 // past the feature get an offset past the descriptor's range, so their loads return
@@ -362,7 +372,7 @@ __device__ __forceinline__ void res_visit(const BnGeom& g, F&& f) {
   constexpr int OOB = (int)0x80000000;
   const int innerV = (int)(g.inner / VEC);
   const int units = (int)(g.units * 4 / VEC);      // g.units counts 4-element vectors
-  const int c = blockIdx.x;
+  const int c = res_feature(g);
   // REV walks k = K-1 .. 0: what the previous walk loaded last is asked for first,
   // while the caches still hold it
   int q = threadIdx.x + (REV ? (K - 1) * RES_THREADS : 0);
@@ -437,7 +447,7 @@ bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restri
   __shared__ float sh[2];
   constexpr int ESZ = (int)sizeof(T);
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
-  const long long c = blockIdx.x;
+  const long long c = res_feature(g);
   const float shift = ld(x, (size_t)(c * g.inner));
   float4 xr[K];
   float s1 = 0.f, s2 = 0.f;
@@ -492,7 +502,7 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
   constexpr int ESZ = (int)sizeof(T);
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes),
                                dxr_ = make_rsrc(dx, bytes);
-  const long long c = blockIdx.x;
+  const long long c = res_feature(g);
   const float mean = a.save_mean[c];
   float4 xr[K];
   float s1 = 0.f, s2 = 0.f;
@@ -569,7 +579,7 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
   __shared__ float red[RES_THREADS / 64];
   __shared__ float sh[2];
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
-  const long long c = blockIdx.x;
+  const long long c = res_feature(g);
   const float shift = ld(x, (size_t)(c * g.inner));
   uint4 xr[K];
   float s1 = 0.f, s2 = 0.f;
@@ -632,7 +642,7 @@ bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ 
                                dxr_ = make_rsrc(dx, bytes);
   const __amdgpu_buffer_rsrc_t yr_ = make_rsrc(FUSE ? fu.y : x, FUSE ? bytes : 0u);
   const __amdgpu_buffer_rsrc_t drr_ = make_rsrc((FUSE && fu.dres) ? fu.dres : dx, (FUSE && fu.dres) ? bytes : 0u);
-  const long long c = blockIdx.x;
+  const long long c = res_feature(g);
   const float mean = a.save_mean[c];
   uint4 xr[K];
   float s1 = 0.f, s2 = 0.f;
@@ -690,7 +700,7 @@ __device__ __forceinline__ void buf_st(__amdgpu_buffer_rsrc_t r, int byte_off, f
 template <int THREADS, int K, int ESZ>
 __device__ __forceinline__ void res1_offsets(const BnGeom& g, int (&off)[K]) {
   constexpr int OOB = (int)0x80000000;
-  const int inner = (int)g.inner, c = blockIdx.x;
+  const int inner = (int)g.inner, c = res_feature(g);
   int q = threadIdx.x;
   int o = q / inner, i = q - o * inner;
   const int so = THREADS / inner, si = THREADS - so * inner;
@@ -715,7 +725,7 @@ bn_train_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restr
   __shared__ float sh[2];
   constexpr int OOB = (int)0x80000000;
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
-  const long long c = blockIdx.x;
+  const long long c = res_feature(g);
   const float shift = ld(x, (size_t)(c * g.inner));
   int off[K];
   res1_offsets<THREADS, K, (int)sizeof(T)>(g, off);
@@ -758,7 +768,7 @@ bn_bwd_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, const T* __r
   __shared__ float sh[4];
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes),
                                dxr_ = make_rsrc(dx, bytes);
-  const long long c = blockIdx.x;
+  const long long c = res_feature(g);
   const float mean = a.save_mean[c];
   int off[K];
   res1_offsets<THREADS, K, (int)sizeof(T)>(g, off);
