@@ -50,7 +50,7 @@ def parse():
     ap.add_argument("--step", choices=["resnet50", "speech"], default="",
                     help="instead of the bench line: a whole training step of configs[4] (ResNet-50, 224x224x3) or "
                          "configs[3] (speech stack) through the host modules, with a per-operation-class breakdown")
-    ap.add_argument("--batch", type=int, default=0, help="batch size for --step (default 64 / 16)")
+    ap.add_argument("--batch", type=int, default=0, help="batch size for --step (default 64 / 16) and --layers (default 32 / 16)")
     ap.add_argument("--repeats", type=int, default=5, help="timed repeats of --steps calls; the median is reported")
     ap.add_argument("--rnn", action="store_true",
                     help="instead of the bench line: time rnn / rnnBackward (LSTM, GRU) at a few sizes")
@@ -391,6 +391,7 @@ def layer_sweep(a, fa, torch, tdt):
     print("| n | input NxCxHxW | K | window | stride | GFLOP | fwd us (TFLOP/s) | bwd-data us | bwd-filter us |")
     print("|---|---|---|---|---|---|---|---|---|")
     for i, (cnt, N, Ci, H, W, K, kh, kw, sy, sx, py, px) in enumerate(layers):
+        N = a.batch or N
         x = torch.randn(N, Ci, H, W, device="cuda").to(tdt)
         w = (torch.randn(K, Ci, kh, kw, device="cuda") / (Ci * kh * kw) ** 0.5).to(tdt)
         cd = capi.ConvDesc(N, Ci, H, W, K, kh, kw, sy, sx, py, px, 1, 1, 1, tag)

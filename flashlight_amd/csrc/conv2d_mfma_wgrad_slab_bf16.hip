@@ -34,9 +34,9 @@ constexpr int CB = 32;           // input channels per workgroup
 constexpr int NCOL = CB * 9;     // columns of the tile
 constexpr int THREADS = 512;
 constexpr int NTW = 9;           // 16-column blocks per MFMA wave
-constexpr int NXI = 3;           // x units (one (c,kh) row piece of 8 columns) per loader thread and row
-constexpr int NDI = 2;           // dy units per loader thread and row
-constexpr int NSET = 4;          // rows in flight in loader registers
+constexpr int NXI_MAX = 3;       // x units (one (c,kh) row piece of 8 columns) per loader thread and step
+constexpr int NDI_MAX = 2;       // dy units per loader thread and step
+constexpr int NSET = 8;          // steps in flight in loader registers (memory latency / time per step)
 constexpr int SPW = NCOL + 4;    // pitch of the parked result tile (words)
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -50,21 +50,26 @@ struct W16Params {
   int N, C, H, W, K, OH, OW;
   int py, dly;
   int groups, Cg, Kg;
-  int Q;               // 8-column groups per row
+  int G;               // output rows per step: rows of at most 16 (8) columns go two (four) at a
+                       // time, side by side in the 32 positions of a k-step
+  int Qr;              // 8-column groups per output row
+  int Q;               // 8-column groups per step (G * Qr)
+  int OHG;             // steps per image (OH / G)
   int RPW;             // rows per loader wave pass (64 / Q)
-  int nks;             // k-steps of 32 positions per row
+  int nks;             // k-steps of 32 positions per step
   int PB;              // LDS row pitch in bytes
   int buf_cells;       // 16-byte cells per LDS buffer (xs then ds)
   int nhalves, mtiles;
-  int nsplit, rps;     // K-splits, (image,row) pairs per split
-  int total_rows;
+  int nsplit, rps;     // K-splits, steps per split
+  int total_rows;      // steps in all (N * OH / G)
   int E;               // K*Cg*9
   int want_db;
   int tail;            // dwords (column pairs) of a row's last 8-column unit that lie inside the row
   unsigned x_bytes, dy_bytes;
 };
 
-__global__ void __launch_bounds__(THREADS, 2)
+template <int NXI, int NDI>
+__global__ void __launch_bounds__(THREADS, 1)
 wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy,
                float* __restrict__ out, float* __restrict__ db_out) {
   extern __shared__ uint4 lds16[];
@@ -111,9 +116,11 @@ wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restri
     const bool do_db = p.want_db && half == 0;
     // A wave pass covers RPW rows of Q units; lane = row_in_pass * Q + q, so the
     // columns next to a unit's eight are in the adjacent lanes.
+    // (q = the unit's cell in the step: output row q / Qr of the step, columns 8 * (q % Qr)...)
     const int rl = lane / p.Q, q = lane - rl * p.Q;
+    const int rsub = q / p.Qr, qq = q - rsub * p.Qr;
     const bool lane_ok = rl < p.RPW;
-    const bool first_q = q == 0, last_q = q == p.Q - 1;
+    const bool first_q = qq == 0, last_q = qq == p.Qr - 1;
     // x rows: index xr = c*3 + kh (96 per tile); dy rows: m (64 per tile)
     int xg[NXI], xl[NXI], xkh[NXI];
 #pragma unroll
@@ -126,7 +133,7 @@ wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restri
         const int c = xr / 3, kh = xr - c * 3;
         xkh[i] = kh;
         xl[i] = xr * 3 * pcells + q;           // cell of the kw = 0 copy; kw copies are pcells apart
-        xg[i] = ((grp * p.Cg + half * CB + c) * HW + 8 * q) * 2;
+        xg[i] = ((grp * p.Cg + half * CB + c) * HW + rsub * p.W + 8 * qq) * 2;
       }
     }
     int yg[NDI], yl[NDI];
@@ -137,7 +144,7 @@ wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restri
       yl[i] = -1;
       if (lane_ok && m < BM) {
         yl[i] = ds_cell0 + m * pcells + q;
-        if (m < m_lim) yg[i] = ((grp * p.Kg + mtile * BM + m) * OHW + 8 * q) * 2;
+        if (m < m_lim) yg[i] = ((grp * p.Kg + mtile * BM + m) * OHW + rsub * p.OW + 8 * qq) * 2;
       }
     }
     float dbp[NDI];
@@ -149,15 +156,15 @@ wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restri
     };
     auto load_row = [&](int row, RowRegs& r) {
       const bool live = row < row_end;
-      const int img = row / p.OH, oh = row - img * p.OH;
+      const int img = row / p.OHG, oh = (row - img * p.OHG) * p.G + rsub;
 #pragma unroll
       for (int i = 0; i < NXI; ++i) {
         const int ih = oh - p.py + xkh[i] * p.dly;
         const bool ok = live && (unsigned)ih < (unsigned)p.H;
         r.xv[i] = __builtin_amdgcn_raw_buffer_load_b128(
-            xrsrc, ok ? xg[i] + (img * p.C * HW + ih * p.W) * 2 : OOB, 0, 0);
+            xrsrc, ok ? xg[i] + (img * p.C * HW + (ih - rsub) * p.W) * 2 : OOB, 0, 0);
       }
-      const int yb = (img * p.K * OHW + oh * p.OW) * 2;
+      const int yb = (img * p.K * OHW + (oh - rsub) * p.OW) * 2;
 #pragma unroll
       for (int i = 0; i < NDI; ++i)
         r.yv[i] = __builtin_amdgcn_raw_buffer_load_b128(yrsrc, live ? yg[i] + yb : OOB, 0, 0);
@@ -195,34 +202,36 @@ wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restri
       for (int i = 0; i < NDI; ++i) {
         const uintx4_t v = in_row(r.yv[i]);
         if (yl[i] >= 0) b[yl[i]] = make_uint4(v.x, v.y, v.z, v.w);
-        float s = 0.f;
+        if (do_db) {
+          float s = 0.f;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          const unsigned d = k == 0 ? v.x : k == 1 ? v.y : k == 2 ? v.z : v.w;
-          s += __uint_as_float(d << 16) + __uint_as_float(d & 0xffff0000u);
+          for (int k = 0; k < 4; ++k) {
+            const unsigned d = k == 0 ? v.x : k == 1 ? v.y : k == 2 ? v.z : v.w;
+            s += __uint_as_float(d << 16) + __uint_as_float(d & 0xffff0000u);
+          }
+          dbp[i] += s;
         }
-        dbp[i] += s;
       }
     };
 
-    // rows r..r+1 in LDS before the first barrier, r+2..r+5 in registers
+    // steps r..r+1 in LDS before the first barrier, r+2..r+1+NSET in registers
     RowRegs set[NSET];
 #pragma unroll
     for (int u = 0; u < NSET; ++u) load_row(row_begin + u, set[u]);
     if (nrows > 0) store_row(0, set[0]);
-    load_row(row_begin + 4, set[0]);
+    load_row(row_begin + NSET, set[0]);
     if (nrows > 1) store_row(1, set[1]);
-    load_row(row_begin + 5, set[1]);
+    load_row(row_begin + NSET + 1, set[1]);
     __syncthreads();
-    // iteration r: the MFMA waves work on row r; row r+2 (register set (r+2)%4) goes
-    // to buffer (r+2)%3 and the set is refilled with row r+6
+    // iteration r: the MFMA waves work on step r; step r+2 (register set (r+2)%NSET) goes
+    // to buffer (r+2)%3 and the set is refilled with step r+2+NSET
     for (int r4 = 0; r4 < nrows; r4 += NSET) {
 #pragma unroll
       for (int u = 0; u < NSET; ++u) {
         const int r = r4 + u;
         if (r < nrows) {
           if (r + 2 < nrows) store_row((r + 2) % 3, set[(u + 2) % NSET]);
-          load_row(row_begin + r + 6, set[(u + 2) % NSET]);
+          load_row(row_begin + r + 2 + NSET, set[(u + 2) % NSET]);
           __syncthreads();
         }
       }
@@ -368,11 +377,15 @@ bool plan(const ConvGeom& g, W16Params* p) {
   p->N = g.N; p->C = g.C; p->H = g.H; p->W = g.W; p->K = g.K; p->OH = g.OH; p->OW = g.OW;
   p->py = g.py; p->dly = g.dly;
   p->groups = g.groups; p->Cg = g.Cg; p->Kg = g.Kg;
-  p->Q = (g.OW + 7) / 8;
-  p->tail = (g.OW - 8 * (p->Q - 1)) / 2;
+  p->Qr = (g.OW + 7) / 8;
+  p->tail = (g.OW - 8 * (p->Qr - 1)) / 2;
+  // short rows share a k-step of 32 positions (the images' row count permitting)
+  p->G = (p->Qr == 1 && g.OH % 4 == 0) ? 4 : (p->Qr <= 2 && g.OH % 2 == 0) ? 2 : 1;
+  p->Q = p->G * p->Qr;
+  p->OHG = g.OH / p->G;
   p->RPW = 64 / p->Q;
-  if (CB * 3 > NXI * 4 * p->RPW || BM > NDI * 4 * p->RPW) return false;
-  const int owp = (g.OW + 31) & ~31;
+  if (CB * 3 > NXI_MAX * 4 * p->RPW || BM > NDI_MAX * 4 * p->RPW) return false;
+  const int owp = (8 * p->Q + 31) & ~31;
   p->nks = owp / 32;
   p->PB = owp * 2 + 16;
   p->buf_cells = (NCOL + BM) * (p->PB / 16) + 1;   // + one cell: the read-ahead past the last row
@@ -380,7 +393,7 @@ bool plan(const ConvGeom& g, W16Params* p) {
   if ((size_t)(BM * SPW + BM * p->Q) * sizeof(float) > (size_t)3 * p->buf_cells * 16) return false;
   p->nhalves = g.Cg / CB;
   p->mtiles = (g.Kg + BM - 1) / BM;
-  p->total_rows = g.N * g.OH;
+  p->total_rows = g.N * p->OHG;
   p->E = g.K * g.Cg * 9;
   const long long base_wgs = (long long)p->nhalves * p->mtiles * g.groups;
   if (p->nhalves * p->mtiles > 65535 || g.groups > 65535) return false;
@@ -422,7 +435,9 @@ int mfma_wgrad16(const ConvGeom& g, const void* x, const void* dy, float* dw, fl
   float* out = p.nsplit > 1 ? static_cast<float*>(ws) : dw;
   if (reinterpret_cast<uintptr_t>(out) % 16 != 0) return -1;
   const size_t shmem = (size_t)3 * p.buf_cells * 16;
-  auto kernel = wgrad16_kernel;
+  // loader units per thread and step the shape needs (fewer = fewer loader instructions)
+  const bool small = CB * 3 <= 2 * 4 * p.RPW && BM <= 4 * p.RPW;
+  auto kernel = small ? wgrad16_kernel<2, 1> : wgrad16_kernel<NXI_MAX, NDI_MAX>;
   if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
   const dim3 grid(p.nsplit, p.nhalves * p.mtiles, g.groups);
   hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const bf16_t*>(x),
