@@ -94,6 +94,12 @@ size_t mfma_first16_wgrad_ws(const ConvGeom& g);
 int mfma_first16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
                        size_t ws_bytes, hipStream_t s);
 // bf16 3x3 stride-1 pad-1 over 64 source channels, whole contraction per workgroup (conv2d_mfma_strip_bf16.hip)
+// bf16 1x1 stride-1 convolutions with operand tiles copied to LDS by the loads themselves
+// (conv2d_mfma_pointwise_dma_bf16.hip); -1 when the shape is not theirs.  addend (or null): added
+// to the rounded input gradient.
+int mfma_pwd16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y, hipStream_t s);
+int mfma_pwd16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, const void* addend, void* dx,
+                             hipStream_t s);
 int mfma_strip16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
                           hipStream_t s);
 int mfma_strip16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s);

@@ -225,7 +225,9 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
   hipStream_t s = as_stream(stream);
   if (!force_direct()) {
     int r = -1;
-    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
+    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_pwd16_conv_fwd(g, x, w, bias, y, s);
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pointwise16_conv_fwd(g, x, w, bias, y, s, ws, ws_bytes);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_FIRST) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_first16_conv_fwd(g, x, w, bias, y, s);
@@ -263,7 +265,9 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
   hipStream_t s = as_stream(stream);
   if (!force_direct()) {
     int r = -1;
-    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
+    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_pwd16_conv_bwd_data(g, dy, w, nullptr, dx, s);
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pointwise16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_STRIP) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_strip16_conv_bwd_data(g, dy, w, dx, s);
@@ -299,7 +303,8 @@ extern "C" int flhip_conv2d_bwd_data_add(const flhip_conv_desc* d, const void* d
   if (rc != FLHIP_OK) return rc;
   hipStream_t s = as_stream(stream);
   if (!force_direct() && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT)) {
-    const int r = mfma_pointwise16_conv_bwd_data_add(g, dy, w, addend, dx, s);
+    int r = skip(Options::SKIP_PWDMA) ? -1 : mfma_pwd16_conv_bwd_data(g, dy, w, addend, dx, s);
+    if (r < 0) r = mfma_pointwise16_conv_bwd_data_add(g, dy, w, addend, dx, s);
     if (r >= 0) return r;
   }
   // every other kernel: the plain pass, then the element-wise sum (dx may not alias addend here)

@@ -1,0 +1,340 @@
+// 1x1 stride-1 convolutions in bf16 storage, forward and backward-data, on
+// v_mfma_f32_32x32x16_bf16 with operand tiles that the memory pipeline itself copies into
+// LDS (buffer loads with the LDS modifier, 16 bytes per lane): no wave spends vector
+// instructions on loading, all four waves multiply, and up to seven stages of 32 contraction
+// channels are in flight per workgroup.  Made for the layers whose planes are small
+// (14x14, 7x7): few workgroups, long contractions, where a stage must not cost a trip to
+// memory and a pass over a loader's registers.
+//
+//   forward        y[m][q]  = sum_c w[m][c]  x[c][q]  (+ bias[m])
+//   backward-data  dx[c][q] = sum_m w[m][c] dy[m][q]
+//
+// Positions: a plane of P positions is cut into cells of 8 (16 bytes); the last cell of a
+// plane ENDS at the plane's last position (it starts at P - 8 and repeats positions of the
+// cell before it when P is not a multiple of 8), so no cell reaches into the next row of
+// the tensor and every cell is loaded and stored whole.  Cells are numbered over the batch
+// (image * cells-per-plane + cell); a workgroup owns 16 of them (128 position slots) x 128
+// result channels.  Repeated positions are computed twice from the same operands in the same
+// order and stored twice with the same value.
+//
+// LDS ring of 4 or 8 stages.  The loads into LDS are written as inline assembly: for the builtin
+// the compiler inserts its own waits in front of the transposing reads, and those wait for
+// every load in flight, which would leave nothing in flight.  The kernel counts its loads
+// itself (s_waitcnt vmcnt(n) before the barrier that publishes a stage).
+//   source   [32 channels][128 slots], pitch 288 bytes: as in memory, fetched by lanes as
+//            8 channels of one position with transposing reads (ds_read_b64_tr_b16)
+//   weights  forward [128 result channels][32 contraction], pitch 80 bytes, 16-byte reads;
+//            backward-data [32 contraction][128 result channels] like the source
+// A load instruction fills 64 consecutive 16-byte cells of LDS, one per lane; the lanes that
+// fall on the unused cells of a pitch, on result channels past the last or on cells past the
+// batch pass an offset beyond the tensor (the range check of the buffer descriptor then
+// returns zeros without a fetch); those rows only reach results that are not stored.
+// Positions are the rows of the instruction tile: a lane holds 4 consecutive positions of a
+// result channel; results go through LDS and leave as whole cells.
+#include <algorithm>
+
+#include "conv2d_mfma.h"
+
+namespace flhip {
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short shortx4_t __attribute__((ext_vector_type(4)));
+typedef int intx4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* lds_void_t;
+typedef __attribute__((address_space(3))) shortx4_t* lds_tr_t;
+
+constexpr int PD_KC = 32;                          // contraction channels per stage
+constexpr int PD_BM = 128;                         // result channels per workgroup
+constexpr int PD_CELLS = 16;                       // position cells per workgroup
+constexpr int PD_XC = PD_CELLS + 2;                // cells per row of a [32][128] tile
+constexpr int PD_XP = PD_XC * 8;                   // the same in elements
+constexpr int PD_WC = 5;                           // cells per row of the forward weight tile (4 + 1)
+constexpr int PD_WP = PD_WC * 8;
+constexpr int PD_XCELLS = PD_KC * PD_XC;           // 576 = 9 load instructions
+constexpr int PD_WCELLS = PD_BM * PD_WC;           // 640 = 10 load instructions (backward-data uses 576)
+constexpr int PD_STAGE = PD_XCELLS + PD_WCELLS;    // cells per stage
+// Stages in the ring, NS: 4 (76 KiB, two workgroups per CU: one multiplies while the other starts
+// or stores) for grids that fill the chip more than once, 8 (152 KiB) for grids of at most one
+// workgroup per CU, where only the depth of the ring hides the way to memory.  Loads run
+// NS - 2 stages ahead of the stage being read.
+constexpr int PD_YP = 8 * PD_CELLS + 8;            // result staging pitch (elements)
+
+struct PwdParams {
+  int Kc, Mo;           // contraction channels, result channels
+  int P, Pc;            // positions and cells per plane
+  int ncells;           // cells over the batch
+  int nstages, mtiles, ctiles;
+  unsigned src_bytes, w_bytes, dst_bytes;
+};
+
+// rows r0 .. r0+7 of column c0 + s of a 16-bit tile stored [row][column] (see the 1x1 kernels
+// with register staging for the lane map of the transposing read)
+__device__ __forceinline__ bf16x8 pd_gather8(const uint16_t* tile, int pitch, int r0, int c0, int s) {
+  const uint16_t* t = tile + (r0 + (s >> 2)) * pitch + c0 + 4 * (s & 3);
+  const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)t);
+  const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(t + 4 * pitch));
+  const uintx2_t l = __builtin_bit_cast(uintx2_t, lo), h = __builtin_bit_cast(uintx2_t, hi);
+  const uintx4_t v = {l.x, l.y, h.x, h.y};
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+__device__ __forceinline__ uint32_t pd_add_bf16x2(uint32_t a, uint32_t b) {
+  return pack_bf16(__uint_as_float(a << 16) + __uint_as_float(b << 16),
+                   __uint_as_float(a & 0xffff0000u) + __uint_as_float(b & 0xffff0000u));
+}
+
+#define PD_WAIT_VM(N) asm volatile("s_waitcnt vmcnt(" #N ")" ::: "memory")
+// at most 4 * STAGES of this wave's loads outstanding (every wave issues at least 4 per stage)
+template <int STAGES>
+__device__ __forceinline__ void pd_wait_stages() {
+  static_assert(STAGES == 0 || STAGES == 1 || STAGES == 2 || STAGES == 5 || STAGES == 6, "counts in use");
+  if (STAGES == 0) PD_WAIT_VM(0);
+  if (STAGES == 1) PD_WAIT_VM(4);
+  if (STAGES == 2) PD_WAIT_VM(8);
+  if (STAGES == 5) PD_WAIT_VM(20);
+  if (STAGES == 6) PD_WAIT_VM(24);
+}
+
+// raw buffer descriptor (the words of make_rsrc) as four scalars for the inline assembly below
+__device__ __forceinline__ intx4_t pd_rsrc(const void* ptr, unsigned bytes) {
+  const uint64_t a = reinterpret_cast<uint64_t>(ptr);
+  return intx4_t{__builtin_amdgcn_readfirstlane((int)(uint32_t)a),
+                 __builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xffffu)),
+                 __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
+}
+// 64 lanes x 16 bytes from rsrc + voff (per lane) + soff to the 1 KiB of LDS at lds_addr (workgroup
+// address, the same for all lanes): lane l lands at lds_addr + 16 l.  m0 is not declared as clobbered (the
+// compiler reserves it and warns); nothing else in these kernels uses it: no LDS-load builtin, no
+// relative register moves, no messages.
+__device__ __forceinline__ void pd_load_lds(intx4_t rsrc, unsigned lds_addr, int voff, int soff) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
+
+template <bool BWD, int PD_NS>
+__global__ void __launch_bounds__(256, PD_NS == 4 ? 2 : 1)
+pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __restrict__ wgt,
+                  const float* __restrict__ bias, bf16_t* __restrict__ dst, const bf16_t* __restrict__ addend) {
+  constexpr int PD_D = PD_NS - 2;
+  __shared__ __align__(16) uint4 ring[PD_NS * PD_STAGE];
+  uint16_t* const ys = reinterpret_cast<uint16_t*>(ring);      // result staging, once the ring is done with
+  static_assert(PD_BM * PD_YP * 2 <= PD_NS * PD_STAGE * 16, "the staged results fit in the ring");
+  constexpr int NXI = PD_XCELLS / 64, NWI = (BWD ? PD_XCELLS : PD_WCELLS) / 64, NI = NXI + NWI;
+  static_assert(PD_XCELLS % 64 == 0 && PD_WCELLS % 64 == 0, "whole load instructions");
+  static_assert(NI <= 20 && NI > 16, "five load instructions per wave at most, four at least");
+  static_assert(PD_NS % 2 == 0, "ring and register sets repeat with the unrolled loop");
+
+  // consecutive workgroups go to different XCDs: the channel tiles that share a source tile
+  // run back to back on one XCD
+  const int id = blockIdx.x, xcd = id & 7, seq = id >> 3;
+  const int mtile = seq % p.mtiles, ctile = (seq / p.mtiles) * 8 + xcd;
+  if (ctile >= p.ctiles) return;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int m0 = mtile * PD_BM, cell0 = ctile * PD_CELLS;
+  const intx4_t xrs = pd_rsrc(src, p.src_bytes), wrs = pd_rsrc(wgt, p.w_bytes);
+
+  // ---- load roles: instruction ii = wave + 4 n of a stage; lane -> LDS cell ii * 64 + lane.
+  // Per instruction, the same for all lanes: descriptor, LDS offset, bytes to advance per stage.
+  int voff[5];
+  intx4_t lrs[5];
+  int loff[5], lstep[5];
+#pragma unroll
+  for (int n = 0; n < 5; ++n) {
+    const int ii = wave + 4 * n;
+    const bool isx = ii < NXI;
+    lrs[n] = isx ? xrs : wrs;
+    loff[n] = (isx ? ii * 64 : PD_XCELLS + (ii - NXI) * 64) * 16;
+    lstep[n] = isx ? PD_KC * 2 * p.P : BWD ? PD_KC * 2 * p.Mo : PD_KC * 2;
+    voff[n] = (int)0x80000000;      // past every tensor: such a lane fetches nothing and its cell gets zeros
+    if (ii < NXI) {
+      const int L = ii * 64 + lane, row = L / PD_XC, c = L - row * PD_XC;
+      const int cell = cell0 + c;
+      if (c < PD_CELLS && cell < p.ncells) {
+        const int img = cell / p.Pc, j = cell - img * p.Pc;
+        voff[n] = ((img * p.Kc + row) * p.P + min(8 * j, p.P - 8)) * 2;
+      }
+    } else if (ii < NI) {
+      const int L = (ii - NXI) * 64 + lane;
+      if (BWD) {
+        const int row = L / PD_XC, c = L - row * PD_XC, mo = m0 + 8 * c;
+        if (c < PD_CELLS && mo < p.Mo) voff[n] = (row * p.Mo + mo) * 2;
+      } else {
+        const int m = L / PD_WC, c = L - m * PD_WC;
+        if (c < 4 && m0 + m < p.Mo) voff[n] = ((m0 + m) * p.Kc + 8 * c) * 2;
+      }
+    }
+  }
+  const bool fifth = wave + 16 < NI;
+  auto issue = [&](int t, uint4* ring) {
+    const unsigned base = (unsigned)reinterpret_cast<uintptr_t>((lds_void_t)ring);
+#pragma unroll
+    for (int n = 0; n < 4; ++n) pd_load_lds(lrs[n], base + loff[n], voff[n], t * lstep[n]);
+    if (fifth) pd_load_lds(lrs[4], base + loff[4], voff[4], t * lstep[4]);
+  };
+
+  // ---- fragments: wave = (position half wp, channel half wm), 2 x 2 blocks of 32 x 32
+  const int wp = wave & 1, wm = wave >> 1;
+  const int fh = lane >> 5, fq = (lane >> 4) & 1, fs = lane & 15, fr = lane & 31;
+  bf16x8 fa[2][2][2], fb[2][2][2];      // [register set][k-step of 16][block]
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+#define PD_READ(RING, SET)                                                                              \
+  {                                                                                                     \
+    const uint16_t* X_ = reinterpret_cast<const uint16_t*>(RING);                                       \
+    const uint16_t* W_ = reinterpret_cast<const uint16_t*>(RING + PD_XCELLS);                           \
+    _Pragma("unroll") for (int ks = 0; ks < 2; ++ks) {                                                  \
+      _Pragma("unroll") for (int i = 0; i < 2; ++i)                                                     \
+        fa[SET][ks][i] = pd_gather8(X_, PD_XP, ks * 16 + 8 * fh, wp * 64 + i * 32 + 16 * fq, fs);       \
+      _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                     \
+        fb[SET][ks][j] = BWD ? pd_gather8(W_, PD_XP, ks * 16 + 8 * fh, wm * 64 + j * 32 + 16 * fq, fs)  \
+                             : __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>(           \
+                                   &W_[(wm * 64 + j * 32 + fr) * PD_WP + ks * 16 + 8 * fh]));           \
+    }                                                                                                   \
+  }
+#define PD_MULT(SET)                                                                                    \
+  _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                      \
+    _Pragma("unroll") for (int i = 0; i < 2; ++i)                                                       \
+      _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                     \
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][ks][i], fb[SET][ks][j], acc[i][j], 0, 0, 0);
+
+  const int n = p.nstages;
+  // stages 0 .. D in flight, stage 0 in registers
+#pragma unroll
+  for (int st = 0; st <= PD_D; ++st)
+    if (st < n) issue(st, ring + st * PD_STAGE);
+  if (PD_D < n) pd_wait_stages<PD_D>();     // stages 1 .. D may be outstanding
+  else pd_wait_stages<0>();
+  __syncthreads();
+  PD_READ(ring, 0)
+
+  // iteration t: the stage t + 1 has landed for every wave (wait for this wave's loads, then the
+  // barrier); the loads of stage t + 1 + D go to the slot whose fragments were multiplied in
+  // iteration t - 1; the fragments of stage t + 1 are read while those of stage t are multiplied
+#define PD_ITER(U)                                                                                  \
+  if (U < PD_NS) {                                                                                  \
+    const int t = t0 + U;                                                                           \
+    if (t < n) {                                                                                    \
+      if (t + 1 < n) {                                                                              \
+        if (t + PD_D < n) pd_wait_stages<PD_D - 1>();                                               \
+        else pd_wait_stages<0>();                                                                   \
+        __syncthreads();                                                                            \
+        if (t + 1 + PD_D < n) issue(t + 1 + PD_D, ring + ((U + 1 + PD_D) % PD_NS) * PD_STAGE);      \
+        PD_READ((ring + ((U + 1) % PD_NS) * PD_STAGE), (U + 1) % 2)                                 \
+      }                                                                                             \
+      PD_MULT(U % 2)                                                                                \
+    }                                                                                               \
+  }
+  for (int t0 = 0; t0 < n; t0 += PD_NS) {
+    PD_ITER(0) PD_ITER(1) PD_ITER(2) PD_ITER(3) PD_ITER(4) PD_ITER(5) PD_ITER(6) PD_ITER(7)
+  }
+#undef PD_ITER
+#undef PD_MULT
+#undef PD_READ
+
+  __syncthreads();      // every wave has read its last fragments: the ring becomes the staging tile
+  // ---- results: element r of block (i, j): slot wp*64 + i*32 + (r/4)*8 + fh*4 + r%4 of channel
+  // wm*64 + j*32 + fr.  [channel][slot] in LDS, then whole cells to memory.
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int ml = wm * 64 + j * 32 + fr;
+    const float bv = (!BWD && bias && m0 + ml < p.Mo) ? bias[m0 + ml] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const uintx2_t o = {pack_bf16(acc[i][j][4 * g] + bv, acc[i][j][4 * g + 1] + bv),
+                            pack_bf16(acc[i][j][4 * g + 2] + bv, acc[i][j][4 * g + 3] + bv)};
+        *reinterpret_cast<uintx2_t*>(&ys[ml * PD_YP + wp * 64 + i * 32 + g * 8 + fh * 4]) = o;
+      }
+  }
+  __syncthreads();
+  {
+    const int c = tid & 15, cell = cell0 + c;
+    if (cell < p.ncells) {
+      const int img = cell / p.Pc, j = cell - img * p.Pc;
+      const int base = (img * p.Mo + m0) * p.P + min(8 * j, p.P - 8);
+      const __amdgpu_buffer_rsrc_t drs = make_rsrc(dst, p.dst_bytes);
+      const __amdgpu_buffer_rsrc_t ars = make_rsrc(addend ? addend : dst, p.dst_bytes);
+      for (int ml = tid >> 4; ml < PD_BM && m0 + ml < p.Mo; ml += 16) {
+        uintx4_t v = *reinterpret_cast<const uintx4_t*>(&ys[ml * PD_YP + 8 * c]);
+        const int off = (base + ml * p.P) * 2;
+        if (addend) {
+          const uintx4_t a = __builtin_amdgcn_raw_buffer_load_b128(ars, off, 0, 0);
+          v = uintx4_t{pd_add_bf16x2(v.x, a.x), pd_add_bf16x2(v.y, a.y), pd_add_bf16x2(v.z, a.z),
+                       pd_add_bf16x2(v.w, a.w)};
+        }
+        __builtin_amdgcn_raw_buffer_store_b128(v, drs, off, 0, 0);
+      }
+    }
+  }
+}
+
+bool pwd16_applies(const ConvGeom& g, bool bwd) {
+  if (!(g.KH == 1 && g.KW == 1 && g.py == 0 && g.px == 0 && g.groups == 1 && g.sy == 1 && g.sx == 1 &&
+        g.OH == g.H && g.OW == g.W && g.C % 8 == 0 && g.K % 8 == 0))
+    return false;
+  const int kc = bwd ? g.K : g.C, mo = bwd ? g.C : g.K;
+  if (kc % PD_KC != 0 || g.H * g.W < 8) return false;
+  // measured on the ResNet-50 layers at batch 32 and 64: ahead of the kernels with register staging
+  // on planes up to 28x28 (by 10 to 45 %), behind them on 56x56 planes (those layers run at the
+  // speed of memory there, several workgroups per CU); a tile of 128 result channels wants more than 64.
+  // FLHIP_PW16_PF set (1 or 4) lifts the rule (tests, measurements).
+  return options().pw16_pf != 0 || (g.H * g.W <= 1024 && mo > 64);
+}
+
+template <bool BWD>
+int launch_pwd16(const ConvGeom& g, const void* src, const void* w, const float* bias, void* dst, const void* addend,
+                 hipStream_t s) {
+  if (!pwd16_applies(g, BWD)) return -1;
+  PwdParams p{};
+  p.Kc = BWD ? g.K : g.C;
+  p.Mo = BWD ? g.C : g.K;
+  p.P = g.H * g.W;
+  p.Pc = (p.P + 7) / 8;
+  const long long sb = (long long)g.N * p.Kc * p.P * 2, db = (long long)g.N * p.Mo * p.P * 2;
+  const long long wb = (long long)p.Kc * p.Mo * 2;
+  // 32-bit byte offsets, with room for the rows of a last tile that lie past the tensor
+  if (std::max(sb, db) + (long long)(PD_BM + PD_KC) * p.P * 2 >= (1ll << 31) || wb + PD_BM * p.Kc * 2ll >= (1ll << 31))
+    return -1;
+  p.src_bytes = (unsigned)sb;
+  p.dst_bytes = (unsigned)db;
+  p.w_bytes = (unsigned)wb;
+  p.ncells = g.N * p.Pc;
+  p.nstages = p.Kc / PD_KC;
+  p.mtiles = (p.Mo + PD_BM - 1) / PD_BM;
+  p.ctiles = (p.ncells + PD_CELLS - 1) / PD_CELLS;
+  const long long grid = (long long)((p.ctiles + 7) / 8) * 8 * p.mtiles;
+  if (grid > 0x7fffffffll) return -1;
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), 0, s, p, static_cast<const bf16_t*>(src),
+                       static_cast<const bf16_t*>(w), bias, static_cast<bf16_t*>(dst),
+                       static_cast<const bf16_t*>(addend));
+  };
+  // the deep ring for grids of at most one workgroup per CU (FLHIP_PW16_PF = 1 / 4 forces the shallow / deep one)
+  bool deep = (long long)p.ctiles * p.mtiles <= (long long)mfma_num_cus();
+  if (options().pw16_pf) deep = options().pw16_pf > 1;
+  if (deep) go(pwd16_conv_kernel<BWD, 8>);
+  else go(pwd16_conv_kernel<BWD, 4>);
+  return check_launch(BWD ? "conv2d_bwd_data 1x1 (bf16 mfma, direct-to-LDS)" : "conv2d_fwd 1x1 (bf16 mfma, direct-to-LDS)");
+}
+
+}  // namespace
+
+int mfma_pwd16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y, hipStream_t s) {
+  return launch_pwd16<false>(g, x, w, bias, y, nullptr, s);
+}
+
+int mfma_pwd16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, const void* addend, void* dx,
+                             hipStream_t s) {
+  return launch_pwd16<true>(g, dy, w, nullptr, dx, addend, s);
+}
+
+}  // namespace flhip

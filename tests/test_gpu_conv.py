@@ -99,6 +99,13 @@ MORE = [
     # bias gradient with more than one tile of 64 filters (each tile writes only its own sums)
     ((2, 32, 8, 16), (136, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),
     ((2, 64, 20, 20), (160, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    # bf16 3x3 filter gradient over short rows: four rows of 8 / two rows of 14 or 6 columns share a
+    # step of 32 positions (images of 8, 14 and 6 rows; a filter tail; several images per split), and
+    # an odd row count that keeps one row per step
+    ((3, 32, 8, 8), (64, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((3, 64, 14, 14), (72, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((2, 32, 6, 6), (32, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((2, 32, 7, 12), (40, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),
     # bf16 strip kernel (3x3, 64 source channels per group, rows of 40 .. 64 columns, strips of 7 rows):
     # two strips, first / last strip at the image border; groups with two 64-channel tiles; full-width rows
     ((2, 64, 14, 56), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
@@ -171,6 +178,7 @@ FAMILY_CASES = [
     ("strip", ((2, 64, 14, 56), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1)),
     ("first", ((2, 3, 32, 32), (64, 3, 7, 7), (2, 2), (3, 3), (1, 1), 1)),
     ("wgrad128", ((3, 136, 7, 7), (160, 136, 1, 1), (1, 1), (0, 0), (1, 1), 1)),
+    ("pwdma", ((3, 256, 14, 14), (136, 256, 1, 1), (1, 1), (0, 0), (1, 1), 1)),
 ]
 
 
@@ -186,8 +194,40 @@ def test_conv_bf16_with_family_switched_off(family, case):
         capi.set_option("CONV_SKIP", None)
 
 
+# bf16 1x1 kernels whose tiles are copied to LDS by the loads themselves: the dispatch picks them for small
+# planes and more than 64 result channels; PW16_PF = 1 / 4 lifts that rule and fixes the ring depth (4 / 8
+# stages), so both depths run on planes that are / are not a multiple of 8 positions (the last cell of a
+# plane then repeats positions), the smallest plane (8), tails in the result channels, fewer stages than the
+# ring holds (1, 3) and more (5, 9, 20), several tiles of positions, and with both weight layouts (forward,
+# backward-data).
+DIRECT_LDS_CASES = [
+    ((3, 96, 14, 14), (136, 96, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((5, 160, 7, 7), (200, 160, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((2, 32, 2, 4), (24, 32, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((4, 288, 5, 9), (64, 288, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((2, 640, 6, 7), (40, 640, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((19, 64, 7, 7), (128, 64, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+    ((1, 128, 28, 28), (256, 128, 1, 1), (1, 1), (0, 0), (1, 1), 1),
+]
+
+
+@pytest.mark.parametrize("depth", [1, 4])
+@pytest.mark.parametrize("case", DIRECT_LDS_CASES)
+def test_conv_bf16_1x1_loaded_straight_to_lds(case, depth):
+    from flashlight_amd import capi
+    capi.set_option("PW16_PF", depth)
+    try:
+        for name, (got, ref) in _run(case, 35, torch.bfloat16).items():
+            tight = 1e-4 if name in ("dw", "db") else 4e-3
+            assert rel_l2(got, ref) <= tight, (depth, name, rel_l2(got, ref))
+    finally:
+        capi.set_option("PW16_PF", None)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("shape", [
+    ((3, 256, 14, 14), (136, 256, 1, 1), (1, 1), (0, 0)),  # bf16: tiles loaded straight to LDS, whole cells (196 positions)
+    ((5, 128, 7, 7), (160, 128, 1, 1), (1, 1), (0, 0)),    # the same with planes of 49 (a plane's last cell repeats positions)
     ((3, 72, 14, 16), (40, 72, 1, 1), (1, 1), (0, 0)),     # bf16: the 1x1 kernel's own result pass, 16-byte pieces
     ((2, 64, 6, 6), (136, 64, 1, 1), (1, 1), (0, 0)),      # planes of 36 positions: 8-byte pieces
     ((5, 64, 7, 7), (64, 64, 1, 1), (1, 1), (0, 0)),       # planes of 49: runs that cross into the next image
