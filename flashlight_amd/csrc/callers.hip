@@ -194,6 +194,104 @@ int gemm_nt_launch(const T* A, const T* B, T* C, int M, int N, int K, int slices
   return check_launch("matmul (A * B^T)");
 }
 
+// ---- products with few columns (N <= 128: fl::linear on a batch of feature vectors) ----
+// The matrix-core kernels tile columns per image and have one position per column here; these two
+// kernels spread a thin product over the whole chip on the vector ALUs instead (a 1000 x 2048 x 64
+// product is 0.26 GFLOP).
+//
+// C (M x N) = A (M x K, column-major) * B (K x N) + bias.  A workgroup owns 64 rows x SK_NT columns;
+// its 16 waves split the contraction.  B's block is staged in LDS as fp32 [k][SK_NT] and read by
+// all lanes at once (same address: a broadcast); lane = row, so A is read in whole rows of 64.
+constexpr int SK_NT = 8, SK_KC = 2048;
+template <typename T>
+__global__ void __launch_bounds__(1024)
+matmul_nn_skinny(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int M, int N, int K,
+                 const float* __restrict__ bias) {
+  __shared__ __align__(16) float sm[SK_KC * SK_NT];      // 64 KiB: B's block, then the waves' partial sums
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int m = blockIdx.x * 64 + lane, n0 = blockIdx.y * SK_NT;
+  const bool mv = m < M;
+  float acc[SK_NT];
+#pragma unroll
+  for (int j = 0; j < SK_NT; ++j) acc[j] = 0.f;
+  for (int kc = 0; kc < K; kc += SK_KC) {
+    const int kn = min(SK_KC, K - kc);
+    if (kc) __syncthreads();
+    for (int e = tid; e < kn * SK_NT; e += 1024) {
+      const int j = e / kn, k = e - j * kn;               // consecutive threads walk k, contiguous in B
+      sm[k * SK_NT + j] = (n0 + j < N) ? ld(B, (size_t)(n0 + j) * K + kc + k) : 0.f;
+    }
+    __syncthreads();
+    const int per = (kn + 15) / 16, k0 = wave * per, k1 = min(kn, k0 + per);
+#pragma unroll 4
+    for (int k = k0; k < k1; ++k) {
+      const float a = mv ? ld(A, (size_t)(kc + k) * M + m) : 0.f;
+      const float4 b0 = *reinterpret_cast<const float4*>(&sm[k * SK_NT]);
+      const float4 b1 = *reinterpret_cast<const float4*>(&sm[k * SK_NT + 4]);
+      acc[0] += a * b0.x; acc[1] += a * b0.y; acc[2] += a * b0.z; acc[3] += a * b0.w;
+      acc[4] += a * b1.x; acc[5] += a * b1.y; acc[6] += a * b1.z; acc[7] += a * b1.w;
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < SK_NT; ++j) sm[(wave * SK_NT + j) * 64 + lane] = acc[j];
+  __syncthreads();
+  if (tid < SK_NT * 64) {
+    const int j = tid >> 6;
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) s += sm[(w * SK_NT + j) * 64 + lane];
+    if (mv && n0 + j < N) st(C, (size_t)(n0 + j) * M + m, s + (bias ? bias[m] : 0.f));
+  }
+}
+
+// C (M x N) = A^T * B with A stored K x M: both operands are contiguous along the contraction.  A wave
+// owns 8 x 8 results; its lanes stride over k and the 64 sums are reduced across the wave at the end.
+template <typename T>
+__global__ void __launch_bounds__(256)
+matmul_tn_skinny(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C, int M, int N, int K,
+                 int mtiles, int tiles) {
+  const int lane = threadIdx.x & 63;
+  const int w = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (w >= tiles) return;
+  const int m0 = (w % mtiles) * 8, n0 = (w / mtiles) * 8;
+  float acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = 0.f;
+  // rows / columns past the matrix read the last valid one; their sums are not stored
+  size_t ao[8], bo[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    ao[i] = (size_t)min(m0 + i, M - 1) * K;
+    bo[i] = (size_t)min(n0 + i, N - 1) * K;
+  }
+  for (int k = lane; k < K; k += 64) {
+    float a[8], b[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      a[i] = ld(A, ao[i] + k);
+      b[i] = ld(B, bo[i] + k);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[i][j] += a[i] * b[j];
+  }
+  float mine = 0.f;      // lane l keeps the sum of result (l % 8, l / 8)
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float s = wave_sum(acc[i][j]);
+      if (lane == j * 8 + i) mine = s;
+    }
+  const int mi = m0 + (lane & 7), nj = n0 + (lane >> 3);
+  if (mi < M && nj < N) st(C, (size_t)nj * M + mi, mine);
+}
+
 // ---- logSoftmax over dimension 0 of a C x X matrix (Functions.cpp:1044-1070) ----
 // one wave per column
 template <typename T>
@@ -439,6 +537,31 @@ extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, in
   FLHIP_REQUIRE(A && B && C, "matmul: null argument");
   FLHIP_REQUIRE(M > 0 && N > 0 && K > 0, "matmul: sizes must be positive");
   FLHIP_REQUIRE(dtype_ok(dtype), "matmul: unknown dtype");
+  // thin products (a batch of feature vectors through fl::linear): the kernels made for them
+  if (N <= 128 && !trans_b && !options().matmul_valu) {
+    hipStream_t s = as_stream(stream);
+    if (!trans_a) {
+      const dim3 grid((unsigned)((M + 63) / 64), (unsigned)((N + SK_NT - 1) / SK_NT));
+      if (dtype == FLHIP_F32)
+        hipLaunchKernelGGL((matmul_nn_skinny<float>), grid, dim3(1024), 0, s, (const float*)A, (const float*)B,
+                           (float*)C, M, N, K, bias_rows);
+      else
+        hipLaunchKernelGGL((matmul_nn_skinny<bf16_t>), grid, dim3(1024), 0, s, (const bf16_t*)A, (const bf16_t*)B,
+                           (bf16_t*)C, M, N, K, bias_rows);
+      return check_launch("matmul (thin, A * B)");
+    }
+    if (!bias_rows) {
+      const int mtiles = (M + 7) / 8, tiles = mtiles * ((N + 7) / 8);
+      const dim3 grid((unsigned)((tiles + 3) / 4));
+      if (dtype == FLHIP_F32)
+        hipLaunchKernelGGL((matmul_tn_skinny<float>), grid, dim3(256), 0, s, (const float*)A, (const float*)B,
+                           (float*)C, M, N, K, mtiles, tiles);
+      else
+        hipLaunchKernelGGL((matmul_tn_skinny<bf16_t>), grid, dim3(256), 0, s, (const bf16_t*)A, (const bf16_t*)B,
+                           (bf16_t*)C, M, N, K, mtiles, tiles);
+      return check_launch("matmul (thin, A^T * B)");
+    }
+  }
   // the matrix-core kernels of the 1x1 convolutions take the three products fl::linear
   // needs; the tiled vector-ALU kernel below covers the rest
   if (!trans_a && trans_b && !bias_rows && !options().matmul_valu) {

@@ -997,13 +997,24 @@ size_t mfma_pointwise16_lattice_ws(const ConvGeom& g, bool bwd) {
   return 0;
 }
 
+// the compact 1x1 problem of a strided layer: on the kernels that load straight to LDS where those
+// are ahead, else on the ones above
+template <bool BWD>
+int launch_compact(const ConvGeom& c, const void* src, const void* w, const float* bias, void* dst, hipStream_t s) {
+  if (!(options().conv_skip & Options::SKIP_PWDMA)) {
+    const int r = BWD ? mfma_pwd16_conv_bwd_data(c, src, w, nullptr, dst, s) : mfma_pwd16_conv_fwd(c, src, w, bias, dst, s);
+    if (r >= 0) return r;
+  }
+  return launch_pw16<BWD>(c, src, w, bias, dst, s);
+}
+
 int mfma_pointwise16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
                               hipStream_t s, void* ws, size_t ws_bytes) {
   ConvGeom c;
   if (pw16_strided_plan(g, &c)) {
     if (!ws || ws_bytes < lattice_bytes(c)) return -1;
     lattice_gather(g, x, ws, s);
-    return launch_pw16<false>(c, ws, w, bias, y, s);
+    return launch_compact<false>(c, ws, w, bias, y, s);
   }
   if (!pw16_applies(g)) return -1;
   return launch_pw16<false>(g, x, w, bias, y, s);
@@ -1014,14 +1025,14 @@ int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void
   ConvGeom c;
   if (pw16_strided_plan(g, &c)) {
     if (!ws || ws_bytes < lattice_bytes(c)) return -1;
-    const int rc = launch_pw16<true>(c, dy, w, nullptr, ws, s);
+    const int rc = launch_compact<true>(c, dy, w, nullptr, ws, s);
     if (rc != FLHIP_OK) return rc;
     lattice_scatter(g, ws, dx, s);
     return check_launch("conv2d_bwd_data strided 1x1 (bf16 mfma)");
   }
   if (!options().pw16_no_taps && pw16_taps_plan(g, &c)) {
     if (!ws || ws_bytes < lattice_bytes(c)) return -1;
-    const int rc = launch_pw16<true>(c, dy, w, nullptr, ws, s);
+    const int rc = launch_compact<true>(c, dy, w, nullptr, ws, s);
     if (rc != FLHIP_OK) return rc;
     if (!taps_spread(g, ws, dx, s)) return fail(FLHIP_RUNTIME_ERROR, "conv2d_bwd_data: plane too wide for the spread kernel");
     return check_launch("conv2d_bwd_data strided window (bf16 mfma)");
