@@ -1020,6 +1020,9 @@ static ResPlan resident8_plan(const BnGeom& g, int vec, int dtype, int min_c) {
   if (units8 > (long long)RES_KMAX * 1024) return r;
   if (g.outer * g.C * g.inner * 2 >= (1ll << 31)) return r;   // 32-bit buffer offsets
   if (mode != 2 && g.C < min_c) return r;
+  // fewer than 128 features of more than 16 vectors per thread (64 features of 56x56 planes at batch
+  // 64): the 64 workgroups of a quarter-full chip lose to the two-pass kernels (28.7 against 21.6 us)
+  if (mode != 2 && g.C < 128 && units8 > 16 * 1024) return r;
   if (units8 <= BN_SMALL_K * 256) {
     r.threads = 256;
     r.k = units8 <= 8 * 256 ? 8 : 16;
