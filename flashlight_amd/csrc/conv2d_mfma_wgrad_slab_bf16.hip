@@ -14,11 +14,16 @@
 // fragment read fall on distinct banks).  The three shifted copies are made in
 // registers from one aligned 16-byte load per 8 columns: the neighbouring columns
 // come from the adjacent lanes, v_alignbit_b32 shifts by one element.
-// 8 waves, two roles: waves 0-3 keep four rows in flight in registers (a row of
-// MFMA work is far shorter than memory latency) and write row r+2 while waves 4-7
-// (2 along m x 2 along the columns, 32 x 144 each) work on row r out of three LDS
-// buffers; fragments of the next k-step - or of the next row, which is complete one
-// barrier earlier - are read into the registers just used.  One barrier per row.
+// A step is one output row, or - rows of at most 16 (8) columns, images of an even (multiple of
+// four) number of rows - two (four) consecutive rows of an image side by side in the 32 positions
+// of a k-step: a step costs about 0.6 us whatever it holds (barrier, loader instructions), so a
+// 14x14 layer runs twice as fast two rows to a step.
+// 8 waves, two roles: waves 0-3 keep four steps in flight in registers (a step of
+// MFMA work is far shorter than memory latency) and write step r+2 while waves 4-7
+// (2 along m x 2 along the columns, 32 x 144 each) work on step r out of three LDS
+// buffers; fragments of the next k-step - or of the next step, which is complete one
+// barrier earlier - are read into the registers just used.  One barrier per step.  The loader
+// loops are compiled for the units per thread a shape needs (2 + 1 for rows up to 32 columns).
 // Partial tiles go to the workspace and are added in a fixed order by
 // wgrad_reduce_kernel; the bias gradient is summed from the dy values as they pass
 // through the loader registers.
@@ -36,7 +41,7 @@ constexpr int THREADS = 512;
 constexpr int NTW = 9;           // 16-column blocks per MFMA wave
 constexpr int NXI_MAX = 3;       // x units (one (c,kh) row piece of 8 columns) per loader thread and step
 constexpr int NDI_MAX = 2;       // dy units per loader thread and step
-constexpr int NSET = 8;          // steps in flight in loader registers (memory latency / time per step)
+constexpr int NSET = 4;          // steps in flight in loader registers
 constexpr int SPW = NCOL + 4;    // pitch of the parked result tile (words)
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -69,7 +74,7 @@ struct W16Params {
 };
 
 template <int NXI, int NDI>
-__global__ void __launch_bounds__(THREADS, 1)
+__global__ void __launch_bounds__(THREADS, 2)
 wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy,
                float* __restrict__ out, float* __restrict__ db_out) {
   extern __shared__ uint4 lds16[];
