@@ -52,7 +52,7 @@ static bool apply_option(Options& o, const char* name, const char* v) {
   }
   if (!strcmp(name, "PW16_PF")) {
     const int n = v ? atoi(v) : 0;
-    if (n != 0 && n != 1 && n != 4) return false;
+    if (n != 0 && n != 1 && n != 2 && n != 4 && n != 8) return false;
     o.pw16_pf = n;
     return true;
   }

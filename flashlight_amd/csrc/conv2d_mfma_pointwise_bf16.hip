@@ -373,7 +373,7 @@ int launch_pw16(const ConvGeom& g, const void* src, const void* w, const float* 
   // on the ResNet-50 layers: 20 to 30 % faster there, slower on every larger grid);
   // FLHIP_PW16_PF = 1 / 4 forces one or the other
   bool deep = grid <= (long long)mfma_num_cus() && p.nchunks >= 8;
-  if (options().pw16_pf) deep = options().pw16_pf > 1;
+  if (options().pw16_pf) deep = options().pw16_pf >= 4;
   const bool odd = p.P % 4 != 0;
   auto go = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), 0, s, p, static_cast<const bf16_t*>(src),

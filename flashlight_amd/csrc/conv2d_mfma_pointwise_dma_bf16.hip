@@ -45,15 +45,17 @@ typedef __attribute__((address_space(3))) void* lds_void_t;
 typedef __attribute__((address_space(3))) shortx4_t* lds_tr_t;
 
 constexpr int PD_KC = 32;                          // contraction channels per stage
-constexpr int PD_BM = 128;                         // result channels per workgroup
+constexpr int PD_BM = 128;                         // result channels per workgroup (64 for grids that would leave CUs idle)
 constexpr int PD_CELLS = 16;                       // position cells per workgroup
 constexpr int PD_XC = PD_CELLS + 2;                // cells per row of a [32][128] tile
 constexpr int PD_XP = PD_XC * 8;                   // the same in elements
 constexpr int PD_WC = 5;                           // cells per row of the forward weight tile (4 + 1)
 constexpr int PD_WP = PD_WC * 8;
 constexpr int PD_XCELLS = PD_KC * PD_XC;           // 576 = 9 load instructions
-constexpr int PD_WCELLS = PD_BM * PD_WC;           // 640 = 10 load instructions (backward-data uses 576)
-constexpr int PD_STAGE = PD_XCELLS + PD_WCELLS;    // cells per stage
+// weight tile of BM result channels: forward [BM][32] (10 / 5 load instructions), backward-data [32][BM] with two
+// unused cells per row (9 / 5 load instructions)
+constexpr int pd_wcells(bool bwd, int bm) { return bwd ? PD_KC * (bm / 8 + 2) : bm * PD_WC; }
+constexpr int pd_stage(int bm) { return PD_XCELLS + bm * PD_WC; }   // cells per stage (the forward tile is the larger one)
 // Stages in the ring, NS: 4 (76 KiB, two workgroups per CU: one multiplies while the other starts
 // or stores) for grids that fill the chip more than once, 8 (152 KiB) for grids of at most one
 // workgroup per CU, where only the depth of the ring hides the way to memory.  Loads run
@@ -85,15 +87,19 @@ __device__ __forceinline__ uint32_t pd_add_bf16x2(uint32_t a, uint32_t b) {
 }
 
 #define PD_WAIT_VM(N) asm volatile("s_waitcnt vmcnt(" #N ")" ::: "memory")
-// at most 4 * STAGES of this wave's loads outstanding (every wave issues at least 4 per stage)
-template <int STAGES>
-__device__ __forceinline__ void pd_wait_stages() {
-  static_assert(STAGES == 0 || STAGES == 1 || STAGES == 2 || STAGES == 5 || STAGES == 6, "counts in use");
-  if (STAGES == 0) PD_WAIT_VM(0);
-  if (STAGES == 1) PD_WAIT_VM(4);
-  if (STAGES == 2) PD_WAIT_VM(8);
-  if (STAGES == 5) PD_WAIT_VM(20);
-  if (STAGES == 6) PD_WAIT_VM(24);
+// at most N of this wave's loads outstanding
+template <int N>
+__device__ __forceinline__ void pd_wait_loads() {
+  static_assert(N == 0 || N == 3 || N == 4 || N == 6 || N == 8 || N == 15 || N == 18 || N == 20 || N == 24, "counts in use");
+  if (N == 0) PD_WAIT_VM(0);
+  if (N == 3) PD_WAIT_VM(3);
+  if (N == 4) PD_WAIT_VM(4);
+  if (N == 6) PD_WAIT_VM(6);
+  if (N == 8) PD_WAIT_VM(8);
+  if (N == 15) PD_WAIT_VM(15);
+  if (N == 18) PD_WAIT_VM(18);
+  if (N == 20) PD_WAIT_VM(20);
+  if (N == 24) PD_WAIT_VM(24);
 }
 
 // raw buffer descriptor (the words of make_rsrc) as four scalars for the inline assembly below
@@ -112,17 +118,21 @@ __device__ __forceinline__ void pd_load_lds(intx4_t rsrc, unsigned lds_addr, int
                :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 
-template <bool BWD, int PD_NS>
+template <bool BWD, int PD_NS, int BM>
 __global__ void __launch_bounds__(256, PD_NS == 4 ? 2 : 1)
 pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __restrict__ wgt,
                   const float* __restrict__ bias, bf16_t* __restrict__ dst, const bf16_t* __restrict__ addend) {
+  static_assert(BM == 128 || BM == 64, "tile heights in use");
   constexpr int PD_D = PD_NS - 2;
+  constexpr int PD_STAGE = pd_stage(BM);
+  constexpr int WXC = BM / 8 + 2, WXP = WXC * 8;               // backward-data weight tile: cells / elements per row
   __shared__ __align__(16) uint4 ring[PD_NS * PD_STAGE];
   uint16_t* const ys = reinterpret_cast<uint16_t*>(ring);      // result staging, once the ring is done with
-  static_assert(PD_BM * PD_YP * 2 <= PD_NS * PD_STAGE * 16, "the staged results fit in the ring");
-  constexpr int NXI = PD_XCELLS / 64, NWI = (BWD ? PD_XCELLS : PD_WCELLS) / 64, NI = NXI + NWI;
-  static_assert(PD_XCELLS % 64 == 0 && PD_WCELLS % 64 == 0, "whole load instructions");
-  static_assert(NI <= 20 && NI > 16, "five load instructions per wave at most, four at least");
+  static_assert(BM * PD_YP * 2 <= PD_NS * PD_STAGE * 16, "the staged results fit in the ring");
+  constexpr int NXI = PD_XCELLS / 64, NWI = pd_wcells(BWD, BM) / 64, NI = NXI + NWI;
+  static_assert(PD_XCELLS % 64 == 0 && pd_wcells(BWD, BM) % 64 == 0, "whole load instructions");
+  static_assert(NI <= 20 && NI >= 12, "five load instructions per wave at most, three at least");
+  constexpr int MINL = NI / 4;                                  // loads every wave issues per stage at least
   static_assert(PD_NS % 2 == 0, "ring and register sets repeat with the unrolled loop");
 
   // consecutive workgroups go to different XCDs: the channel tiles that share a source tile
@@ -132,7 +142,7 @@ pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __r
   if (ctile >= p.ctiles) return;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int m0 = mtile * PD_BM, cell0 = ctile * PD_CELLS;
+  const int m0 = mtile * BM, cell0 = ctile * PD_CELLS;
   const intx4_t xrs = pd_rsrc(src, p.src_bytes), wrs = pd_rsrc(wgt, p.w_bytes);
 
   // ---- load roles: instruction ii = wave + 4 n of a stage; lane -> LDS cell ii * 64 + lane.
@@ -158,29 +168,32 @@ pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __r
     } else if (ii < NI) {
       const int L = (ii - NXI) * 64 + lane;
       if (BWD) {
-        const int row = L / PD_XC, c = L - row * PD_XC, mo = m0 + 8 * c;
-        if (c < PD_CELLS && mo < p.Mo) voff[n] = (row * p.Mo + mo) * 2;
+        const int row = L / WXC, c = L - row * WXC, mo = m0 + 8 * c;
+        if (c < BM / 8 && mo < p.Mo) voff[n] = (row * p.Mo + mo) * 2;
       } else {
         const int m = L / PD_WC, c = L - m * PD_WC;
         if (c < 4 && m0 + m < p.Mo) voff[n] = ((m0 + m) * p.Kc + 8 * c) * 2;
       }
     }
   }
-  const bool fifth = wave + 16 < NI;
+  const bool fourth = wave + 12 < NI, fifth = wave + 16 < NI;
   auto issue = [&](int t, uint4* ring) {
     const unsigned base = (unsigned)reinterpret_cast<uintptr_t>((lds_void_t)ring);
 #pragma unroll
-    for (int n = 0; n < 4; ++n) pd_load_lds(lrs[n], base + loff[n], voff[n], t * lstep[n]);
+    for (int n = 0; n < 3; ++n) pd_load_lds(lrs[n], base + loff[n], voff[n], t * lstep[n]);
+    if (fourth) pd_load_lds(lrs[3], base + loff[3], voff[3], t * lstep[3]);
     if (fifth) pd_load_lds(lrs[4], base + loff[4], voff[4], t * lstep[4]);
   };
 
-  // ---- fragments: wave = (position half wp, channel half wm), 2 x 2 blocks of 32 x 32
-  const int wp = wave & 1, wm = wave >> 1;
+  // ---- fragments: 128 result channels: wave = (position half, channel half), 2 x 2 blocks of 32 x 32;
+  // 64 result channels: wave = position quarter, 1 x 2 blocks
+  constexpr int NA = BM == 128 ? 2 : 1;
+  const int pos0 = BM == 128 ? (wave & 1) * 64 : wave * 32, mw0 = BM == 128 ? (wave >> 1) * 64 : 0;
   const int fh = lane >> 5, fq = (lane >> 4) & 1, fs = lane & 15, fr = lane & 31;
-  bf16x8 fa[2][2][2], fb[2][2][2];      // [register set][k-step of 16][block]
-  floatx16 acc[2][2];
+  bf16x8 fa[2][2][NA], fb[2][2][2];      // [register set][k-step of 16][block]
+  floatx16 acc[NA][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < NA; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -191,17 +204,17 @@ pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __r
     const uint16_t* X_ = reinterpret_cast<const uint16_t*>(RING);                                       \
     const uint16_t* W_ = reinterpret_cast<const uint16_t*>(RING + PD_XCELLS);                           \
     _Pragma("unroll") for (int ks = 0; ks < 2; ++ks) {                                                  \
-      _Pragma("unroll") for (int i = 0; i < 2; ++i)                                                     \
-        fa[SET][ks][i] = pd_gather8(X_, PD_XP, ks * 16 + 8 * fh, wp * 64 + i * 32 + 16 * fq, fs);       \
+      _Pragma("unroll") for (int i = 0; i < NA; ++i)                                                    \
+        fa[SET][ks][i] = pd_gather8(X_, PD_XP, ks * 16 + 8 * fh, pos0 + i * 32 + 16 * fq, fs);          \
       _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                     \
-        fb[SET][ks][j] = BWD ? pd_gather8(W_, PD_XP, ks * 16 + 8 * fh, wm * 64 + j * 32 + 16 * fq, fs)  \
+        fb[SET][ks][j] = BWD ? pd_gather8(W_, WXP, ks * 16 + 8 * fh, mw0 + j * 32 + 16 * fq, fs)        \
                              : __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>(           \
-                                   &W_[(wm * 64 + j * 32 + fr) * PD_WP + ks * 16 + 8 * fh]));           \
+                                   &W_[(mw0 + j * 32 + fr) * PD_WP + ks * 16 + 8 * fh]));               \
     }                                                                                                   \
   }
 #define PD_MULT(SET)                                                                                    \
   _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                      \
-    _Pragma("unroll") for (int i = 0; i < 2; ++i)                                                       \
+    _Pragma("unroll") for (int i = 0; i < NA; ++i)                                                      \
       _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                     \
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][ks][i], fb[SET][ks][j], acc[i][j], 0, 0, 0);
 
@@ -210,8 +223,8 @@ pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __r
 #pragma unroll
   for (int st = 0; st <= PD_D; ++st)
     if (st < n) issue(st, ring + st * PD_STAGE);
-  if (PD_D < n) pd_wait_stages<PD_D>();     // stages 1 .. D may be outstanding
-  else pd_wait_stages<0>();
+  if (PD_D < n) pd_wait_loads<MINL * PD_D>();     // stages 1 .. D may be outstanding
+  else pd_wait_loads<0>();
   __syncthreads();
   PD_READ(ring, 0)
 
@@ -223,8 +236,8 @@ pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __r
     const int t = t0 + U;                                                                           \
     if (t < n) {                                                                                    \
       if (t + 1 < n) {                                                                              \
-        if (t + PD_D < n) pd_wait_stages<PD_D - 1>();                                               \
-        else pd_wait_stages<0>();                                                                   \
+        if (t + PD_D < n) pd_wait_loads<MINL * (PD_D - 1)>();                                       \
+        else pd_wait_loads<0>();                                                                    \
         __syncthreads();                                                                            \
         if (t + 1 + PD_D < n) issue(t + 1 + PD_D, ring + ((U + 1 + PD_D) % PD_NS) * PD_STAGE);      \
         PD_READ((ring + ((U + 1) % PD_NS) * PD_STAGE), (U + 1) % 2)                                 \
@@ -240,19 +253,19 @@ pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __r
 #undef PD_READ
 
   __syncthreads();      // every wave has read its last fragments: the ring becomes the staging tile
-  // ---- results: element r of block (i, j): slot wp*64 + i*32 + (r/4)*8 + fh*4 + r%4 of channel
-  // wm*64 + j*32 + fr.  [channel][slot] in LDS, then whole cells to memory.
+  // ---- results: element r of block (i, j): slot pos0 + i*32 + (r/4)*8 + fh*4 + r%4 of channel
+  // mw0 + j*32 + fr.  [channel][slot] in LDS, then whole cells to memory.
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    const int ml = wm * 64 + j * 32 + fr;
+    const int ml = mw0 + j * 32 + fr;
     const float bv = (!BWD && bias && m0 + ml < p.Mo) ? bias[m0 + ml] : 0.f;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < NA; ++i)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const uintx2_t o = {pack_bf16(acc[i][j][4 * g] + bv, acc[i][j][4 * g + 1] + bv),
                             pack_bf16(acc[i][j][4 * g + 2] + bv, acc[i][j][4 * g + 3] + bv)};
-        *reinterpret_cast<uintx2_t*>(&ys[ml * PD_YP + wp * 64 + i * 32 + g * 8 + fh * 4]) = o;
+        *reinterpret_cast<uintx2_t*>(&ys[ml * PD_YP + pos0 + i * 32 + g * 8 + fh * 4]) = o;
       }
   }
   __syncthreads();
@@ -263,7 +276,7 @@ pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __r
       const int base = (img * p.Mo + m0) * p.P + min(8 * j, p.P - 8);
       const __amdgpu_buffer_rsrc_t drs = make_rsrc(dst, p.dst_bytes);
       const __amdgpu_buffer_rsrc_t ars = make_rsrc(addend ? addend : dst, p.dst_bytes);
-      for (int ml = tid >> 4; ml < PD_BM && m0 + ml < p.Mo; ml += 16) {
+      for (int ml = tid >> 4; ml < BM && m0 + ml < p.Mo; ml += 16) {
         uintx4_t v = *reinterpret_cast<const uintx4_t*>(&ys[ml * PD_YP + 8 * c]);
         const int off = (base + ml * p.P) * 2;
         if (addend) {
@@ -286,7 +299,7 @@ bool pwd16_applies(const ConvGeom& g, bool bwd) {
   // measured on the ResNet-50 layers at batch 32 and 64: ahead of the kernels with register staging
   // on planes up to 28x28 (by 10 to 45 %), behind them on 56x56 planes (those layers run at the
   // speed of memory there, several workgroups per CU); a tile of 128 result channels wants more than 64.
-  // FLHIP_PW16_PF set (1 or 4) lifts the rule (tests, measurements).
+  // FLHIP_PW16_PF set lifts the rule (tests, measurements).
   return options().pw16_pf != 0 || (g.H * g.W <= 1024 && mo > 64);
 }
 
@@ -309,8 +322,15 @@ int launch_pwd16(const ConvGeom& g, const void* src, const void* w, const float*
   p.w_bytes = (unsigned)wb;
   p.ncells = g.N * p.Pc;
   p.nstages = p.Kc / PD_KC;
-  p.mtiles = (p.Mo + PD_BM - 1) / PD_BM;
   p.ctiles = (p.ncells + PD_CELLS - 1) / PD_CELLS;
+  // tiles of 64 result channels when tiles of 128 would leave half of the CUs without a workgroup (7x7 planes
+  // with 512 result channels at batch 64: 112 workgroups of 64 stages); the deep ring for grids of at most one
+  // workgroup per CU.  FLHIP_PW16_PF = 1 / 4 forces the shallow / deep ring with tiles of 128, 2 / 8 with tiles of 64.
+  const int cus = mfma_num_cus(), pf = options().pw16_pf;
+  bool small = (long long)p.ctiles * ((p.Mo + PD_BM - 1) / PD_BM) <= cus / 2;
+  if (pf) small = pf == 2 || pf == 8;
+  const int bm = small ? 64 : PD_BM;
+  p.mtiles = (p.Mo + bm - 1) / bm;
   const long long grid = (long long)((p.ctiles + 7) / 8) * 8 * p.mtiles;
   if (grid > 0x7fffffffll) return -1;
   auto go = [&](auto kernel) {
@@ -318,11 +338,15 @@ int launch_pwd16(const ConvGeom& g, const void* src, const void* w, const float*
                        static_cast<const bf16_t*>(w), bias, static_cast<bf16_t*>(dst),
                        static_cast<const bf16_t*>(addend));
   };
-  // the deep ring for grids of at most one workgroup per CU (FLHIP_PW16_PF = 1 / 4 forces the shallow / deep one)
-  bool deep = (long long)p.ctiles * p.mtiles <= (long long)mfma_num_cus();
-  if (options().pw16_pf) deep = options().pw16_pf > 1;
-  if (deep) go(pwd16_conv_kernel<BWD, 8>);
-  else go(pwd16_conv_kernel<BWD, 4>);
+  bool deep = (long long)p.ctiles * p.mtiles <= (long long)cus;
+  if (pf) deep = pf >= 4;
+  if (small) {
+    if (deep) go(pwd16_conv_kernel<BWD, 8, 64>);
+    else go(pwd16_conv_kernel<BWD, 4, 64>);
+  } else {
+    if (deep) go(pwd16_conv_kernel<BWD, 8, 128>);
+    else go(pwd16_conv_kernel<BWD, 4, 128>);
+  }
   return check_launch(BWD ? "conv2d_bwd_data 1x1 (bf16 mfma, direct-to-LDS)" : "conv2d_fwd 1x1 (bf16 mfma, direct-to-LDS)");
 }
 

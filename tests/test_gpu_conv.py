@@ -196,7 +196,7 @@ def test_conv_bf16_with_family_switched_off(family, case):
 
 # bf16 1x1 kernels whose tiles are copied to LDS by the loads themselves: the dispatch picks them for small
 # planes and more than 64 result channels; PW16_PF = 1 / 4 lifts that rule and fixes the ring depth (4 / 8
-# stages), so both depths run on planes that are / are not a multiple of 8 positions (the last cell of a
+# stages; 2 / 8: the same with tiles of 64 result channels), so all four kernels run on planes that are / are not a multiple of 8 positions (the last cell of a
 # plane then repeats positions), the smallest plane (8), tails in the result channels, fewer stages than the
 # ring holds (1, 3) and more (5, 9, 20), several tiles of positions, and with both weight layouts (forward,
 # backward-data).
@@ -211,7 +211,7 @@ DIRECT_LDS_CASES = [
 ]
 
 
-@pytest.mark.parametrize("depth", [1, 4])
+@pytest.mark.parametrize("depth", [1, 4, 2, 8])
 @pytest.mark.parametrize("case", DIRECT_LDS_CASES)
 def test_conv_bf16_1x1_loaded_straight_to_lds(case, depth):
     from flashlight_amd import capi
