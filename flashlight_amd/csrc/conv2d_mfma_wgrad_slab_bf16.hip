@@ -384,8 +384,9 @@ bool plan(const ConvGeom& g, W16Params* p) {
   p->groups = g.groups; p->Cg = g.Cg; p->Kg = g.Kg;
   p->Qr = (g.OW + 7) / 8;
   p->tail = (g.OW - 8 * (p->Qr - 1)) / 2;
-  // short rows share a k-step of 32 positions (the images' row count permitting)
-  p->G = (p->Qr == 1 && g.OH % 4 == 0) ? 4 : (p->Qr <= 2 && g.OH % 2 == 0) ? 2 : 1;
+  // short rows share a step (the images' row count permitting): four rows of 8 columns or two of at most 16
+  // side by side in the 32 positions of a k-step, two rows of at most 32 columns as two k-steps
+  p->G = (p->Qr == 1 && g.OH % 4 == 0) ? 4 : (p->Qr <= 4 && g.OH % 2 == 0) ? 2 : 1;
   p->Q = p->G * p->Qr;
   p->OHG = g.OH / p->G;
   p->RPW = 64 / p->Q;
