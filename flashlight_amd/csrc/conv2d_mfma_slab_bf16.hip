@@ -60,6 +60,9 @@ struct Slab16Params {
   int groups, SCg, DCg;
   int a_mstride, a_cstride, w_group_stride;
   int R, RS;             // result rows per tile, slab rows
+  int VS;                // images per tile (1: a tile is R rows of one image).  VS > 1 (3x3, stride 1, pad 1, planes
+                         // that fit a tile whole): VS images stacked with one shared zero row between them; R counts
+                         // the rows of the stack, of which every (DH + 1)-th is not a result
   int WSP, XOFF;         // slab row pitch (positions), slab column of image column 0
   int XPL, APL;          // plane pitches in cells: slab, weights
   int tiles_per_image, mtiles;
@@ -86,7 +89,7 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
   const int grp = __builtin_amdgcn_readfirstlane(blockIdx.y / p.mtiles);
   const int mtile = __builtin_amdgcn_readfirstlane(blockIdx.y % p.mtiles);
   const int m_lim = p.DCg - mtile * BM;
-  const int rows = min(p.R, p.DH - r0);          // result rows of this tile
+  const int rows = p.VS > 1 ? p.R : min(p.R, p.DH - r0);          // result rows of this tile
   const int n = p.nchunks;
   const int npos = rows * p.DW;
 
@@ -125,7 +128,7 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
     const __amdgpu_buffer_rsrc_t wrsrc = make_rsrc(wgt, p.wt_bytes);
     constexpr int OOB = (int)0x80000000;
     const int chan_bytes = p.SH * p.SW * 2;
-    const int img_base = (img * p.SC + grp * p.SCg) * p.SH * p.SW;
+    const int img_base = (img * p.VS * p.SC + grp * p.SCg) * p.SH * p.SW;
     // slab unit u: bits 0-1 channel group, bits 2-3 low bits of the slab row, then the
     // group of 8 image columns, then the high bits of the row (see the bank note above)
     const int qrow = (p.SW + 7) >> 3, rs_hi = (p.RS + 3) >> 2;
@@ -146,12 +149,19 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
         const int t = u >> 4;
         const int q = t % qrow, rh = t / qrow;
         const int rs = rh * 4 + rl;
-        const int sr = r0 * p.psh + p.min_sh + rs;
+        int sr = r0 * p.psh + p.min_sh + rs;
+        int stacked = 0;                         // image of the stack this slab row belongs to
+        if (p.VS > 1 && sr >= 0) {
+          stacked = sr / (p.SH + 1);
+          sr -= stacked * (p.SH + 1);            // sr == SH: the zero row between two images
+          if (img * p.VS + stacked >= p.N) sr = -1;
+        }
         xc[i] = cg * 8;
         xn[i] = min(8, p.SW - 8 * q);
         if (rs < p.RS) {
           xl[i] = cg * p.XPL + rs * p.WSP + p.XOFF + 8 * q;
-          if ((unsigned)sr < (unsigned)p.SH) xg[i] = (img_base + (cg * 8 * p.SH + sr) * p.SW + 8 * q) * 2;
+          if ((unsigned)sr < (unsigned)p.SH)
+            xg[i] = (img_base + stacked * p.SC * p.SH * p.SW + (cg * 8 * p.SH + sr) * p.SW + 8 * q) * 2;
         }
       }
     }
@@ -530,11 +540,20 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
       }
       return;
     }
-    const size_t out_base = (size_t)img * p.DC * p.DH * p.DW + (size_t)r0 * p.DW;
+    const size_t out_base = (size_t)img * p.VS * p.DC * p.DH * p.DW + (size_t)r0 * p.DW;
     auto put = [&](int m, int pos, float v) {
       if (m < m_lim && pos < npos) {
         const int ch = grp * p.DCg + mtile * BM + m;
-        st(dst, out_base + (size_t)ch * p.DH * p.DW + pos, v + bias_lds[m]);
+        if (p.VS > 1) {
+          // row of the stack -> (image, row); the row between two images is not a result
+          int w;
+          const int rr = fast_div(pos, p.DW, inv_dw, &w);
+          const int si = rr / (p.DH + 1), row = rr - si * (p.DH + 1);
+          if (row < p.DH && img * p.VS + si < p.N)
+            st(dst, out_base + ((size_t)si * p.DC + ch) * p.DH * p.DW + row * p.DW + w, v + bias_lds[m]);
+        } else {
+          st(dst, out_base + (size_t)ch * p.DH * p.DW + pos, v + bias_lds[m]);
+        }
       }
     };
 #pragma unroll
@@ -611,15 +630,36 @@ bool plan(Slab16Params* p, size_t* shmem) {
     }
   }
   if (best_r == 0) return false;
+  p->VS = 1;
+  // Planes that fit a tile whole and still make more than one round of workgroups (7x7 at batch 64): a chunk
+  // of such a tile costs one trip to memory whatever it holds, so tiles of several images, stacked with one
+  // shared zero row between them, take the rounds out (3x3, stride 1, pad 1: the row above an image and the
+  // row below the one before it are the same zero row).
+  if (best_r == p->DH && p->KH == 3 && p->psh == 1 && p->psw == 1 && p->dly == 1 && p->min_sh == -1 && p->SH == p->DH) {
+    const long long tiles1 = (long long)p->N * p->mtiles * p->groups;
+    int vs = 1;
+    const int forced = options().conv_stack;      // measurement / test switch: this many images per tile where it fits
+    while (2 * vs <= p->N && (forced ? 2 * vs <= forced : tiles1 / (2 * vs) >= cus) &&
+           (2 * vs * (p->DH + 1) - 1) * p->DW <= max_pos) {
+      layout(p, 2 * vs * (p->DH + 1) - 1);
+      if ((size_t)2 * (p->x_cells + p->a_cells) * 16 > 156 * 1024) break;
+      if (CG * 4 * ((p->SW + 7) / 8) * ((p->RS + 3) / 4) > GTHREADS * NXU_MAX) break;
+      vs *= 2;
+    }
+    if (vs > 1) {
+      p->VS = vs;
+      best_r = vs * (p->DH + 1) - 1;
+    }
+  }
   layout(p, best_r);
   if ((CG * BM * p->KHW + GTHREADS - 1) / GTHREADS > NAU_MAX) return false;
-  p->tiles_per_image = (p->DH + best_r - 1) / best_r;
+  p->tiles_per_image = p->VS > 1 ? 1 : (p->DH + best_r - 1) / best_r;
   p->NB = (best_r * p->DW + 15) / 16;
   p->nchunks = (p->SCg + CKB - 1) / CKB;
   *shmem = (size_t)2 * (p->x_cells + p->a_cells) * 16 + BM * sizeof(float);
   {
     const int npos = best_r * p->DW, sp = ((npos + 3) & ~3) + 4;
-    p->stage_ok = p->DW % 4 == 0 && (size_t)32 * sp * sizeof(float) <= *shmem - BM * sizeof(float);
+    p->stage_ok = p->VS == 1 && p->DW % 4 == 0 && (size_t)32 * sp * sizeof(float) <= *shmem - BM * sizeof(float);
   }
   // (a whole 7x7 plane, 49 positions, is worth it for a window with several taps)
   return best_r * p->DW >= (p->KHW > 1 ? 48 : 64);
@@ -683,7 +723,7 @@ int launch(const ConvGeom& g, Slab16Params& p, const void* src, const void* wgt,
   }
   auto kernel = slab16_conv_kernel<BWD>;
   if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
-  const dim3 grid((unsigned)(p.N * p.tiles_per_image), (unsigned)(p.mtiles * p.groups));
+  const dim3 grid((unsigned)(p.VS > 1 ? (p.N + p.VS - 1) / p.VS : p.N * p.tiles_per_image), (unsigned)(p.mtiles * p.groups));
   hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const bf16_t*>(src),
                      static_cast<const bf16_t*>(wgt), bias, static_cast<bf16_t*>(dst));
   if (p.SW & 1) {

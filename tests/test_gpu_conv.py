@@ -224,6 +224,26 @@ def test_conv_bf16_1x1_loaded_straight_to_lds(case, depth):
         capi.set_option("PW16_PF", None)
 
 
+# bf16 3x3 kernel with several images per tile (planes that fit a tile whole, stacked with one shared zero
+# row between them; the dispatch does this when single images would make more than one round of workgroups):
+# 2 and 4 images of 7x7 / 5x6 / 8x8 planes per tile, an image count that leaves the last tile short, a filter tail.
+@pytest.mark.parametrize("stack", [2, 4])
+@pytest.mark.parametrize("case", [
+    ((5, 64, 7, 7), (72, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((7, 32, 5, 6), (64, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((4, 96, 8, 8), (32, 96, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+])
+def test_conv_bf16_3x3_stacked_images(case, stack):
+    from flashlight_amd import capi
+    capi.set_option("CONV_STACK", stack)
+    try:
+        for name, (got, ref) in _run(case, 37, torch.bfloat16).items():
+            tight = 1e-4 if name in ("dw", "db") else 4e-3
+            assert rel_l2(got, ref) <= tight, (stack, name, rel_l2(got, ref))
+    finally:
+        capi.set_option("CONV_STACK", None)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("shape", [
     ((3, 256, 14, 14), (136, 256, 1, 1), (1, 1), (0, 0)),  # bf16: tiles loaded straight to LDS, whole cells (196 positions)
