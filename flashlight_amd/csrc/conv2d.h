@@ -100,6 +100,9 @@ int mfma_first16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* 
 int mfma_pwd16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y, hipStream_t s);
 int mfma_pwd16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, const void* addend, void* dx,
                              hipStream_t s);
+// their filter gradient (no bias gradient; at least 128 channels on both sides); partial tiles in ws
+size_t mfma_pwd16_wgrad_ws(const ConvGeom& g);
+int mfma_pwd16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, void* ws, size_t ws_bytes, hipStream_t s);
 int mfma_strip16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
                           hipStream_t s);
 int mfma_strip16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s);

@@ -1062,6 +1062,7 @@ size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g0) {
   Pw16Wgrad2Params p2{};
   if (pw16_wgrad2_plan(g, &p2) && p2.nsplit > 1)
     need = std::max(need, (size_t)p2.nsplit * ((size_t)p2.E + p2.Mo) * sizeof(float));
+  need = std::max(need, mfma_pwd16_wgrad_ws(g));
   return lattice + need;
 }
 
@@ -1083,6 +1084,10 @@ int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, fl
     x = ws;
     ws = static_cast<char*>(ws) + lb;
     ws_bytes -= lb;
+  }
+  if (!db && !(options().conv_skip & Options::SKIP_PWDMA)) {
+    const int r = mfma_pwd16_wgrad(g, x, dy, dw, ws, ws_bytes, s);
+    if (r >= 0) return r;
   }
   Pw16Wgrad2Params p2{};
   if (!(options().conv_skip & Options::SKIP_WGRAD128) && pw16_wgrad2_plan(g, &p2) && reinterpret_cast<uintptr_t>(x) % 4 == 0 &&

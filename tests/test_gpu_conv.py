@@ -224,6 +224,38 @@ def test_conv_bf16_1x1_loaded_straight_to_lds(case, depth):
         capi.set_option("PW16_PF", None)
 
 
+# bf16 1x1 filter gradient without a bias gradient, at least 128 channels on both sides: the kernel whose
+# tiles the loads copy straight to LDS.  Planes of 8k positions; planes whose last cell repeats positions
+# (196, 49, 25, 9: the repeated part of the dy cell is zeroed in LDS); one stage, a slice that ends inside an
+# image, channel tails on both sides, more images than one slice holds.
+@pytest.mark.parametrize("xs,K", [
+    ((3, 128, 14, 14), 128), ((5, 136, 7, 7), 160), ((2, 128, 8, 8), 256), ((9, 256, 5, 5), 128),
+    ((4, 128, 3, 3), 136), ((1, 128, 2, 4), 128), ((40, 128, 7, 7), 128), ((2, 384, 28, 28), 128),
+])
+def test_bf16_1x1_filter_gradient_alone(xs, K):
+    rng = np.random.default_rng(xs[0] * 131 + K)
+    ws = (K, xs[1], 1, 1)
+    x = bf16_round(rng.standard_normal(xs).astype(np.float32))
+    dy = bf16_round(rng.standard_normal((xs[0], K, xs[2], xs[3])).astype(np.float32))
+    d = flref.conv_desc(xs, ws, (1, 1), (0, 0), (1, 1), 1)
+    dw_ref, _ = flref.conv2d_bwd_filter(d, x, dy)
+    from flashlight_amd import capi
+    capi.set_option("PW16_PF", 1)            # also on the planes the dispatch leaves to the older kernel
+    try:
+        dw, db = fa.conv2d_backward_filter_bias(dev(dy, torch.bfloat16), dev(x, torch.bfloat16), ws, False)
+    finally:
+        capi.set_option("PW16_PF", None)
+    assert db is None
+    assert rel_l2(host(dw), dw_ref) <= 1e-4, rel_l2(host(dw), dw_ref)
+    # the same through the kernels with register staging
+    capi.set_option("CONV_SKIP", "pwdma")
+    try:
+        dw2, _ = fa.conv2d_backward_filter_bias(dev(dy, torch.bfloat16), dev(x, torch.bfloat16), ws, False)
+    finally:
+        capi.set_option("CONV_SKIP", None)
+    assert rel_l2(host(dw2), dw_ref) <= 1e-4
+
+
 # bf16 3x3 kernel with several images per tile (planes that fit a tile whole, stacked with one shared zero
 # row between them; the dispatch does this when single images would make more than one round of workgroups):
 # 2 and 4 images of 7x7 / 5x6 / 8x8 planes per tile, an image count that leaves the last tile short, a filter tail.
