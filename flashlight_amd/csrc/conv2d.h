@@ -102,6 +102,8 @@ int mfma_pwd16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, c
                              hipStream_t s);
 // their filter gradient (no bias gradient; at least 128 channels on both sides); partial tiles in ws
 size_t mfma_pwd16_wgrad_ws(const ConvGeom& g);
+// workgroups the bf16 slab kernel's forward pass would launch (0: not its shape)
+long long mfma_slab16_conv_fwd_workgroups(const ConvGeom& g);
 int mfma_pwd16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, void* ws, size_t ws_bytes, hipStream_t s);
 int mfma_strip16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
                           hipStream_t s);

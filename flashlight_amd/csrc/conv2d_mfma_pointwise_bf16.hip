@@ -988,12 +988,26 @@ bool pw16_taps_plan(const ConvGeom& g, ConvGeom* c, bool wgrad = false) {
   return pw16_applies(*c);
 }
 
+// Forward through gathered taps (the gather writes 9/4 of the input for a 3x3 stride-2 window, the product
+// then runs as a 1x1 layer over C * T channels): where the product goes to the kernels that load straight to LDS
+// this beats the slab kernel's strided forward pass (whose loader moves 2.5 times the bytes per product there)
+// when that pass would need two rounds of workgroups or more: the stride-2 3x3 layers of ResNet-50 at batch 64
+// take 110 / 65 / 102 us on the slab kernel and 73 / 58 / 77 us this way; at batch 32 (one round, two for the
+// first) 37 / 33 / 55 against 42 / 45 / 67.
+bool pw16_taps_forward(const ConvGeom& g, const ConvGeom& c) {
+  if (!((g.sy > 1 || g.sx > 1) && !(options().conv_skip & Options::SKIP_PWDMA) && c.H * c.W <= 1024 && c.K > 64 &&
+        c.C % 32 == 0))
+    return false;
+  const long long slab = mfma_slab16_conv_fwd_workgroups(g);
+  return slab == 0 || slab >= 2 * (long long)mfma_num_cus();
+}
+
 }  // namespace
 
 size_t mfma_pointwise16_lattice_ws(const ConvGeom& g, bool bwd) {
   ConvGeom c;
   if (pw16_strided_plan(g, &c)) return lattice_bytes(c);
-  if (bwd && !options().pw16_no_taps && pw16_taps_plan(g, &c)) return lattice_bytes(c);
+  if (!options().pw16_no_taps && pw16_taps_plan(g, &c) && (bwd || pw16_taps_forward(g, c))) return lattice_bytes(c);
   return 0;
 }
 
@@ -1016,6 +1030,9 @@ int mfma_pointwise16_conv_fwd(const ConvGeom& g, const void* x, const void* w, c
     lattice_gather(g, x, ws, s);
     return launch_compact<false>(c, ws, w, bias, y, s);
   }
+  if (!options().pw16_no_taps && pw16_taps_plan(g, &c) && pw16_taps_forward(g, c) && ws && ws_bytes >= lattice_bytes(c) &&
+      taps_gather(g, x, ws, s))
+    return launch_compact<false>(c, ws, w, bias, y, s);
   if (!pw16_applies(g)) return -1;
   return launch_pw16<false>(g, x, w, bias, y, s);
 }

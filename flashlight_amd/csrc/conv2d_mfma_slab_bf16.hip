@@ -770,6 +770,16 @@ void fill_bwd(const ConvGeom& g, Slab16Params* p) {
 
 }  // namespace
 
+// workgroups the forward pass below would launch (0: the shape is not this kernel's)
+long long mfma_slab16_conv_fwd_workgroups(const ConvGeom& g) {
+  if ((g.sy != 1 || g.sx != 1) && g.KH * g.KW == 1) return 0;
+  Slab16Params p{};
+  fill_fwd(g, &p);
+  size_t shmem = 0;
+  if (!plan(&p, &shmem)) return 0;
+  return (long long)(p.VS > 1 ? (p.N + p.VS - 1) / p.VS : p.N * p.tiles_per_image) * p.mtiles * p.groups;
+}
+
 int mfma_slab16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
                          hipStream_t s) {
   // strides: results step through the slab; 1x1 windows with a stride are left to the GEMM kernels
