@@ -61,6 +61,11 @@ SYMBOLS = {
                                           C.c_double, C.c_double, _VP, _SZ, _VP]),
     "flhip_bn_act_bwd": (C.c_int, [C.POINTER(BnDesc), _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
                                     _SZ, _VP]),
+    "flhip_bn_act_mask_bytes": (_SZ, [C.POINTER(BnDesc)]),
+    "flhip_bn_act_fwd_train_mask": (C.c_int, [C.POINTER(BnDesc), _VP, _VP, _VP, _VP, C.c_int, _VP, _VP, _VP, _VP, _VP,
+                                               _VP, C.c_double, C.c_double, _VP, _SZ, _VP]),
+    "flhip_bn_act_bwd_mask": (C.c_int, [C.POINTER(BnDesc), _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP, _VP,
+                                         _SZ, _VP]),
     "flhip_copy_bytes": (C.c_int, [_VP, _VP, _SZ, _VP]),
     "flhip_convert": (C.c_int, [_VP, C.c_int, _VP, C.c_int, _SZ, _VP]),
     "flhip_convert_many": (C.c_int, [C.POINTER(_VP), C.POINTER(_VP), C.POINTER(_SZ), C.c_int, C.c_int, C.c_int, _VP]),

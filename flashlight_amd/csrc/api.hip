@@ -63,6 +63,12 @@ static bool apply_option(Options& o, const char* name, const char* v) {
     else return false;
     return true;
   }
+  if (!strcmp(name, "CONV_ROWS")) {
+    const int n = v ? atoi(v) : 0;
+    if (n < 0 || n > 64) return false;
+    o.conv_rows = n;
+    return true;
+  }
   if (!strcmp(name, "CONV_STACK")) {
     const int n = v ? atoi(v) : 0;
     if (n != 0 && n != 1 && n != 2 && n != 4 && n != 8) return false;
@@ -77,7 +83,7 @@ static bool apply_option(Options& o, const char* name, const char* v) {
 }
 
 static void options_from_environment() {
-  static const char* const names[] = {"CONV_ALGO", "CONV_SKIP", "PW_PT", "PW16_PF", "CONV_STACK", "BN_ALGO", "PW16_NO_TAPS",
+  static const char* const names[] = {"CONV_ALGO", "CONV_SKIP", "PW_PT", "PW16_PF", "CONV_ROWS", "CONV_STACK", "BN_ALGO", "PW16_NO_TAPS",
                                       "TAPPED_NO_REORDER", "MATMUL_VALU", "RNN_UNFUSED"};
   for (const char* n : names) {
     const std::string var = std::string("FLHIP_") + n;

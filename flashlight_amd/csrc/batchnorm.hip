@@ -188,6 +188,7 @@ template <typename T>
 struct BnFuseFwd {
   const T* res;   // may be null
   int relu;
+  uint8_t* mask;  // may be null: one byte per 4 consecutive elements, bit e = (y[4 i + e] > 0)
 };
 // Fused prologue of the backward kernels: the incoming gradient passes the ReLU mask of the
 // forward result y first (dz = dy where y > 0), and dz itself can be written out for the
@@ -196,12 +197,30 @@ template <typename T>
 struct BnFuseBwd {
   const T* y;     // forward result (after the ReLU)
   T* dres;        // may be null
+  const uint8_t* mask;   // may be null; when given it stands for y > 0 and y is not read (an eighth of
+                         // the bytes of a bf16 y, a sixteenth of an fp32 one)
 };
 
-template <typename T, int VEC, bool FUSE = false>
+// value as it reads back from storage of type T
+__device__ __forceinline__ float rounded(float v, const float*) { return v; }
+__device__ __forceinline__ float rounded(float v, const bf16_t*) { return bf16_to_f32(f32_to_bf16(v)); }
+// the ReLU mask of the vector at element offset `off` as values that compare like y: from the mask bytes
+// when the caller has them (4-element vectors only), else from y itself
+template <int VEC, bool MASK, typename T>
+__device__ __forceinline__ void seg_mask_load(Vec<T, VEC>& m, const BnFuseBwd<T>& fu, size_t off) {
+  if (VEC == 4 && MASK) {
+    const unsigned bits = fu.mask[off >> 2];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) m.v[e] = (bits >> e) & 1u ? 1.f : 0.f;
+  } else {
+    m.load(fu.y, off);
+  }
+}
+
+template <typename T, int VEC, int FUSE = 0>
 __global__ void __launch_bounds__(256)
 bn_train_apply_seg(BnGeom g, const T* __restrict__ x, T* __restrict__ y,
-                   const float* __restrict__ ws, BnTrainArgs a, BnFuseFwd<T> fu = BnFuseFwd<T>{nullptr, 0}) {
+                   const float* __restrict__ ws, BnTrainArgs a, BnFuseFwd<T> fu = BnFuseFwd<T>{nullptr, 0, nullptr}) {
   __shared__ float sh[2];
   if (threadIdx.x < 64) {
     double p0, p1;
@@ -233,28 +252,37 @@ bn_train_apply_seg(BnGeom g, const T* __restrict__ x, T* __restrict__ y,
         }
         v[k].v[e] = t;
       }
-      if (k < n) v[k].store(y, off[k]);
+      if (k < n) {
+        v[k].store(y, off[k]);
+        if (FUSE == 2 && VEC == 4) {
+          unsigned bits = 0;
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) bits |= (rounded(v[k].v[e], y) > 0.f ? 1u : 0u) << e;
+          fu.mask[off[k] >> 2] = (uint8_t)bits;
+        }
+      }
     }
   });
 }
 
 // ---- backward, segment mode ------------------------------------------------
-template <typename T, int VEC, bool FUSE = false>
+template <typename T, int VEC, int FUSE = 0>
 __global__ void __launch_bounds__(256)
 bn_bwd_stats_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
                  const float* __restrict__ save_mean, float* __restrict__ ws,
-                 BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr}) {
+                 BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr, nullptr}) {
   __shared__ float red[8];
   float s1 = 0.f, s2 = 0.f;
   const long long c = blockIdx.x;
   const float mean = save_mean[c];
+  constexpr bool MASK = FUSE == 2 && VEC == 4;   // the ReLU mask comes as bytes, not from y
   bn_seg_visit<VEC, false>(g, [&](const size_t (&off)[BN_UN], int n) {
     Vec<T, VEC> a[BN_UN], b[BN_UN], m[BN_UN];
 #pragma unroll
     for (int k = 0; k < BN_UN; ++k) {
       a[k].load(x, off[k]);
       b[k].load(dy, off[k]);
-      if (FUSE) m[k].load(fu.y, off[k]);
+      if (FUSE) seg_mask_load<VEC, MASK>(m[k], fu, off[k]);
     }
 #pragma unroll
     for (int k = 0; k < BN_UN; ++k) {
@@ -305,11 +333,11 @@ __device__ __forceinline__ void finish_bwd(const BnGeom& g, const BnBwdArgs& a, 
   }
 }
 
-template <typename T, int VEC, bool FUSE = false>
+template <typename T, int VEC, int FUSE = 0>
 __global__ void __launch_bounds__(256)
 bn_bwd_apply_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
                  T* __restrict__ dx, const float* __restrict__ ws, BnBwdArgs a,
-                 BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr}) {
+                 BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr, nullptr}) {
   __shared__ float sh[4];
   if (threadIdx.x < 64) {
     double p0, p1;
@@ -318,13 +346,14 @@ bn_bwd_apply_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
   }
   __syncthreads();
   const float mean = sh[0], kdy = sh[1], kx = sh[2], k0 = sh[3];
+  constexpr bool MASK = FUSE == 2 && VEC == 4;   // the ReLU mask comes as bytes, not from y
   bn_seg_visit<VEC, true>(g, [&](const size_t (&off)[BN_UN], int n) {
     Vec<T, VEC> v[BN_UN], w[BN_UN], m[BN_UN];
 #pragma unroll
     for (int k = 0; k < BN_UN; ++k) {
       v[k].load(x, off[k]);
       w[k].load(dy, off[k]);
-      if (FUSE) m[k].load(fu.y, off[k]);
+      if (FUSE) seg_mask_load<VEC, MASK>(m[k], fu, off[k]);
     }
 #pragma unroll
     for (int k = 0; k < BN_UN; ++k) {
@@ -362,6 +391,14 @@ __device__ __forceinline__ int res_feature(const BnGeom& g) {
   const int b = blockIdx.x, C = (int)g.C;
   return (C & 7) ? b : (b & 7) * (C >> 3) + (b >> 3);
 }
+
+// The mask bytes of the fused kernels (one byte per 4 consecutive elements) through a buffer descriptor: the byte
+// of the vector at byte offset `off` of a tensor of `esz`-byte elements is off / (4 esz); the out-of-range offset
+// of the walks below (0x80000000) lands past the mask as well.  No mask: an empty range (stores dropped).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t mask_rsrc(const uint8_t* mask, const void* any, unsigned bytes, int esz) {
+  return make_rsrc(mask ? (const void*)mask : any, mask ? bytes >> (esz == 2 ? 3 : 4) : 0u);
+}
+__device__ __forceinline__ int mask_off(int off, int esz) { return (int)((unsigned)off >> (esz == 2 ? 3 : 4)); }
 
 // Walks this thread's vectors q = tid + 1024*k: f(k, byte offset, in range).  The
 // offset is relative to the tensor base and goes through a buffer descriptor; slots
@@ -439,10 +476,10 @@ __device__ __forceinline__ void buf_st4(__amdgpu_buffer_rsrc_t r, int byte_off, 
   __builtin_amdgcn_raw_buffer_store_b64(t, r, byte_off, 0, 2);
 }
 
-template <typename T, int RES_THREADS, int K, bool FUSE = false>
+template <typename T, int RES_THREADS, int K, int FUSE = 0>
 __global__ void __launch_bounds__(RES_THREADS)
 bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restrict__ y,
-                  BnTrainArgs a, BnFuseFwd<T> fu = BnFuseFwd<T>{nullptr, 0}) {
+                  BnTrainArgs a, BnFuseFwd<T> fu = BnFuseFwd<T>{nullptr, 0, nullptr}) {
   __shared__ float red[RES_THREADS / 64];
   __shared__ float sh[2];
   constexpr int ESZ = (int)sizeof(T);
@@ -472,12 +509,18 @@ bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restri
   const float bt = a.beta ? a.beta[c] : 0.f;
   if (FUSE) {
     const __amdgpu_buffer_rsrc_t rr_ = make_rsrc(fu.res ? fu.res : x, fu.res ? bytes : 0u);   // no residual: loads give 0
+    const __amdgpu_buffer_rsrc_t mr_ = mask_rsrc(FUSE == 2 ? fu.mask : nullptr, x, bytes, ESZ);   // one byte per vector
     const float lo = fu.relu ? 0.f : -__builtin_huge_valf();
     res_visit<RES_THREADS, K, ESZ, 4>(g, [&](int k, int off, bool) {
       const float4 r = buf_ld4_stream(rr_, off, x);
       const float4 v = make_float4(fmaxf((xr[k].x - mean) * scale + bt + r.x, lo), fmaxf((xr[k].y - mean) * scale + bt + r.y, lo),
                                    fmaxf((xr[k].z - mean) * scale + bt + r.z, lo), fmaxf((xr[k].w - mean) * scale + bt + r.w, lo));
       buf_st4(yr_, off, v, y);
+      if (FUSE == 2) {
+        const unsigned bits = (rounded(v.x, y) > 0.f ? 1u : 0u) | (rounded(v.y, y) > 0.f ? 2u : 0u) |
+                              (rounded(v.z, y) > 0.f ? 4u : 0u) | (rounded(v.w, y) > 0.f ? 8u : 0u);
+        __builtin_amdgcn_raw_buffer_store_b8((uint8_t)bits, mr_, mask_off(off, ESZ), 0, 0);
+      }
     });
     return;
   }
@@ -491,11 +534,14 @@ bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restri
 __device__ __forceinline__ float4 relu_mask(float4 d, float4 y) {
   return make_float4(y.x > 0.f ? d.x : 0.f, y.y > 0.f ? d.y : 0.f, y.z > 0.f ? d.z : 0.f, y.w > 0.f ? d.w : 0.f);
 }
+__device__ __forceinline__ float4 relu_bits(float4 d, unsigned bits) {
+  return make_float4(bits & 1u ? d.x : 0.f, bits & 2u ? d.y : 0.f, bits & 4u ? d.z : 0.f, bits & 8u ? d.w : 0.f);
+}
 
-template <typename T, int RES_THREADS, int K, bool FUSE = false>
+template <typename T, int RES_THREADS, int K, int FUSE = 0>
 __global__ void __launch_bounds__(RES_THREADS)
 bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, const T* __restrict__ dy,
-                T* __restrict__ dx, BnBwdArgs a, BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr}) {
+                T* __restrict__ dx, BnBwdArgs a, BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr, nullptr}) {
   extern __shared__ float4 dyl[];           // [klim][threads], klim <= min(K, RES_KL)
   __shared__ float red[RES_THREADS / 64];
   __shared__ float sh[4];
@@ -507,10 +553,14 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
   float4 xr[K];
   float s1 = 0.f, s2 = 0.f;
   res_visit<RES_THREADS, K, ESZ, 0>(g, [&](int k, int off, bool in) { xr[k] = buf_ld4_stream(xr_, off, x); });
+  constexpr bool MASK = FUSE == 2;   // the ReLU mask comes as bytes, not from y
   res_visit<RES_THREADS, K, ESZ, 4>(g, [&](int k, int off, bool in) {
     // dy vectors that stay in LDS are read once; the others come back in the second walk
     float4 d = k < klim ? buf_ld4_stream(dyr_, off, dy) : buf_ld4(dyr_, off, dy);
-    if (FUSE) d = relu_mask(d, k < klim ? buf_ld4_stream(make_rsrc(fu.y, bytes), off, dy) : buf_ld4(make_rsrc(fu.y, bytes), off, dy));
+    if (FUSE) {
+      if (MASK) d = relu_bits(d, __builtin_amdgcn_raw_buffer_load_b8(mask_rsrc(fu.mask, x, bytes, ESZ), mask_off(off, ESZ), 0, 0));
+      else d = relu_mask(d, k < klim ? buf_ld4_stream(make_rsrc(fu.y, bytes), off, dy) : buf_ld4(make_rsrc(fu.y, bytes), off, dy));
+    }
     if (k < klim) dyl[k * RES_THREADS + threadIdx.x] = d;
     const float p1 = (d.x + d.y) + (d.z + d.w);
     const float p2 = (d.x * (xr[k].x - mean) + d.y * (xr[k].y - mean)) +
@@ -529,7 +579,10 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
   res_visit<RES_THREADS, K, ESZ, 4, true>(g, [&](int k, int off, bool) {
     float4 d = k < klim ? dyl[k * RES_THREADS + threadIdx.x] : buf_ld4(dyr_, off, dy);
     // the part of dy that did not fit in LDS passes the mask again (y re-read with it)
-    if (FUSE && k >= klim) d = relu_mask(d, buf_ld4(make_rsrc(fu.y, bytes), off, dy));
+    if (FUSE && k >= klim) {
+      if (MASK) d = relu_bits(d, __builtin_amdgcn_raw_buffer_load_b8(mask_rsrc(fu.mask, x, bytes, ESZ), mask_off(off, ESZ), 0, 0));
+      else d = relu_mask(d, buf_ld4(make_rsrc(fu.y, bytes), off, dy));
+    }
     const float4 v = make_float4(kdy * d.x + (kx * (xr[k].x - mean) + k0),
                                  kdy * d.y + (kx * (xr[k].y - mean) + k0),
                                  kdy * d.z + (kx * (xr[k].z - mean) + k0),
@@ -571,11 +624,25 @@ __device__ __forceinline__ void opaque(uint4& v) { asm volatile("" : "+v"(v.x), 
 __device__ __forceinline__ uint4 relu_mask8(uint4 d, uint4 y) {
   return make_uint4(relu_mask2(d.x, y.x), relu_mask2(d.y, y.y), relu_mask2(d.z, y.z), relu_mask2(d.w, y.w));
 }
+// the same from the two mask bytes of the vector: bit e of byte j stands for element 4 j + e
+__device__ __forceinline__ uint32_t relu_bits2(uint32_t d, unsigned lo, unsigned hi) {
+  return (lo ? d & 0x0000ffffu : 0u) | (hi ? d & 0xffff0000u : 0u);
+}
+__device__ __forceinline__ uint4 relu_bits8(uint4 d, unsigned b) {
+  return make_uint4(relu_bits2(d.x, b & 1u, b & 2u), relu_bits2(d.y, b & 4u, b & 8u), relu_bits2(d.z, b & 0x100u, b & 0x200u),
+                    relu_bits2(d.w, b & 0x400u, b & 0x800u));
+}
 
-template <int RES_THREADS, int K, bool FUSE = false>
+// A value every lane holds alike, moved to a scalar register (the vector registers of the
+// resident kernels are all taken by the held elements).
+__device__ __forceinline__ float uniform(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+}
+
+template <int RES_THREADS, int K, int FUSE = 0>
 __global__ void __launch_bounds__(RES_THREADS)
 bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_t* __restrict__ y,
-                   BnTrainArgs a, BnFuseFwd<bf16_t> fu = BnFuseFwd<bf16_t>{nullptr, 0}) {
+                   BnTrainArgs a, BnFuseFwd<bf16_t> fu = BnFuseFwd<bf16_t>{nullptr, 0, nullptr}) {
   __shared__ float red[RES_THREADS / 64];
   __shared__ float sh[2];
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
@@ -602,10 +669,11 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
   s2 = block_sum(s2, red);
   finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh);
   __syncthreads();
-  const float mean = sh[0];
-  const float scale = (a.gamma ? a.gamma[c] : 1.f) * sh[1];
-  const float bt = a.beta ? a.beta[c] : 0.f;
+  const float mean = uniform(sh[0]);
+  const float scale = uniform((a.gamma ? a.gamma[c] : 1.f) * sh[1]);
+  const float bt = uniform(a.beta ? a.beta[c] : 0.f);
   const __amdgpu_buffer_rsrc_t rr_ = make_rsrc((FUSE && fu.res) ? fu.res : x, (FUSE && fu.res) ? bytes : 0u);
+  const __amdgpu_buffer_rsrc_t mr_ = mask_rsrc(FUSE == 2 ? fu.mask : nullptr, x, bytes, 2);
   const float lo = (FUSE && fu.relu) ? 0.f : -__builtin_huge_valf();
   res_visit<RES_THREADS, K, 2, 1, false, 8>(g, [&](int k, int off, bool) {
     // one 32-bit word (two values) at a time, results written over the packed input: the
@@ -614,13 +682,23 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
     opaque(v);
     if (FUSE) {
       const uint4 rv = buf_ld8(rr_, off, true);      // no residual: the empty range reads zeros
+      // (relu leaves no NaN, so the sign tests on the packed words equal y > 0)
+      auto pos = [](uint32_t w, unsigned blo, unsigned bhi) {
+        return ((int)(w << 16) > 0 ? blo : 0u) | ((int)(w & 0xffff0000u) > 0 ? bhi : 0u);
+      };
       v.x = bf_pack(fmaxf((bf_lo(v.x) - mean) * scale + bt + bf_lo(rv.x), lo), fmaxf((bf_hi(v.x) - mean) * scale + bt + bf_hi(rv.x), lo));
+      unsigned bits = pos(v.x, 1u, 2u);
       __builtin_amdgcn_sched_barrier(0);   // one word at a time: the packing temporaries of all four do not fit
       v.y = bf_pack(fmaxf((bf_lo(v.y) - mean) * scale + bt + bf_lo(rv.y), lo), fmaxf((bf_hi(v.y) - mean) * scale + bt + bf_hi(rv.y), lo));
-      __builtin_amdgcn_sched_barrier(0);   // one word at a time: the packing temporaries of all four do not fit
+      bits |= pos(v.y, 4u, 8u);
+      __builtin_amdgcn_sched_barrier(0);
       v.z = bf_pack(fmaxf((bf_lo(v.z) - mean) * scale + bt + bf_lo(rv.z), lo), fmaxf((bf_hi(v.z) - mean) * scale + bt + bf_hi(rv.z), lo));
-      __builtin_amdgcn_sched_barrier(0);   // one word at a time: the packing temporaries of all four do not fit
+      bits |= pos(v.z, 0x100u, 0x200u);
+      __builtin_amdgcn_sched_barrier(0);
       v.w = bf_pack(fmaxf((bf_lo(v.w) - mean) * scale + bt + bf_lo(rv.w), lo), fmaxf((bf_hi(v.w) - mean) * scale + bt + bf_hi(rv.w), lo));
+      bits |= pos(v.w, 0x400u, 0x800u);
+      // two mask bytes per vector (8 elements)
+      if (FUSE == 2) __builtin_amdgcn_raw_buffer_store_b16((uint16_t)bits, mr_, mask_off(off, 2), 0, 0);
     } else {
       v.x = bf_pack((bf_lo(v.x) - mean) * scale + bt, (bf_hi(v.x) - mean) * scale + bt);
       v.y = bf_pack((bf_lo(v.y) - mean) * scale + bt, (bf_hi(v.y) - mean) * scale + bt);
@@ -631,25 +709,30 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
   });
 }
 
-template <int RES_THREADS, int K, bool FUSE = false>
+template <int RES_THREADS, int K, int FUSE = 0>
 __global__ void __launch_bounds__(RES_THREADS)
 bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy,
-                 bf16_t* __restrict__ dx, BnBwdArgs a, BnFuseBwd<bf16_t> fu = BnFuseBwd<bf16_t>{nullptr, nullptr}) {
+                 bf16_t* __restrict__ dx, BnBwdArgs a, BnFuseBwd<bf16_t> fu = BnFuseBwd<bf16_t>{nullptr, nullptr, nullptr}) {
   extern __shared__ uint4 dyl8[];           // [klim][threads] packed gradients (after the mask)
   __shared__ float red[RES_THREADS / 64];
   __shared__ float sh[4];
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes),
                                dxr_ = make_rsrc(dx, bytes);
-  const __amdgpu_buffer_rsrc_t yr_ = make_rsrc(FUSE ? fu.y : x, FUSE ? bytes : 0u);
+  const __amdgpu_buffer_rsrc_t yr_ = make_rsrc((FUSE && fu.y) ? fu.y : x, (FUSE && fu.y) ? bytes : 0u);
+  const __amdgpu_buffer_rsrc_t mr_ = mask_rsrc(FUSE == 2 ? fu.mask : nullptr, x, bytes, 2);
   const __amdgpu_buffer_rsrc_t drr_ = make_rsrc((FUSE && fu.dres) ? fu.dres : dx, (FUSE && fu.dres) ? bytes : 0u);
   const long long c = res_feature(g);
   const float mean = a.save_mean[c];
   uint4 xr[K];
   float s1 = 0.f, s2 = 0.f;
   res_visit<RES_THREADS, K, 2, 0, false, 8>(g, [&](int k, int off, bool) { xr[k] = buf_ld8(xr_, off, true); });
+  constexpr bool MASK = FUSE == 2;   // the ReLU mask comes as bytes, not from y
   res_visit<RES_THREADS, K, 2, 4, false, 8>(g, [&](int k, int off, bool in) {
     uint4 d = buf_ld8(dyr_, off, k < klim);
-    if (FUSE) d = relu_mask8(d, buf_ld8(yr_, off, k < klim));
+    if (FUSE) {
+      if (MASK) d = relu_bits8(d, __builtin_amdgcn_raw_buffer_load_b16(mr_, mask_off(off, 2), 0, 0));
+      else d = relu_mask8(d, buf_ld8(yr_, off, k < klim));
+    }
     if (k < klim) dyl8[k * RES_THREADS + threadIdx.x] = d;
     opaque(xr[k]);
     const uint32_t dw[4] = {d.x, d.y, d.z, d.w}, xw[4] = {xr[k].x, xr[k].y, xr[k].z, xr[k].w};
@@ -671,7 +754,10 @@ bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ 
   const float kdy = sh[1], kx = sh[2], k0 = sh[3];
   res_visit<RES_THREADS, K, 2, 4, true, 8>(g, [&](int k, int off, bool) {
     uint4 d = k < klim ? dyl8[k * RES_THREADS + threadIdx.x] : buf_ld8(dyr_, off, false);
-    if (FUSE && k >= klim) d = relu_mask8(d, buf_ld8(yr_, off, false));
+    if (FUSE && k >= klim) {
+      if (MASK) d = relu_bits8(d, __builtin_amdgcn_raw_buffer_load_b16(mr_, mask_off(off, 2), 0, 0));
+      else d = relu_mask8(d, buf_ld8(yr_, off, false));
+    }
     opaque(xr[k]);
     const uint32_t dw[4] = {d.x, d.y, d.z, d.w}, xw[4] = {xr[k].x, xr[k].y, xr[k].z, xr[k].w};
     uint32_t o[4];
@@ -717,10 +803,10 @@ __device__ __forceinline__ void res1_offsets(const BnGeom& g, int (&off)[K]) {
   }
 }
 
-template <typename T, int THREADS, int K, bool FUSE = false>
+template <typename T, int THREADS, int K, int FUSE = 0>
 __global__ void __launch_bounds__(THREADS)
 bn_train_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restrict__ y,
-                   BnTrainArgs a, BnFuseFwd<T> fu = BnFuseFwd<T>{nullptr, 0}) {
+                   BnTrainArgs a, BnFuseFwd<T> fu = BnFuseFwd<T>{nullptr, 0, nullptr}) {
   __shared__ float red[THREADS / 64];
   __shared__ float sh[2];
   constexpr int OOB = (int)0x80000000;
@@ -760,10 +846,10 @@ bn_train_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restr
   for (int k = 0; k < K; ++k) buf_st(yr_, off[k], (xv[k] - mean) * scale + bt, y);
 }
 
-template <typename T, int THREADS, int K, bool FUSE = false>
+template <typename T, int THREADS, int K, int FUSE = 0>
 __global__ void __launch_bounds__(THREADS)
 bn_bwd_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, const T* __restrict__ dy,
-                 T* __restrict__ dx, BnBwdArgs a, BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr}) {
+                 T* __restrict__ dx, BnBwdArgs a, BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr, nullptr}) {
   __shared__ float red[THREADS / 64];
   __shared__ float sh[4];
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes),
@@ -1035,7 +1121,7 @@ static ResPlan resident8_plan(const BnGeom& g, int vec, int dtype, int min_c) {
   return r;
 }
 
-template <int THREADS, int K, bool FUSE>
+template <int THREADS, int K, int FUSE>
 static int launch_train_resident8(const BnGeom& g, const bf16_t* x, bf16_t* y, const BnTrainArgs& a,
                                   const BnFuseFwd<bf16_t>& fu, hipStream_t s) {
   const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * 2);
@@ -1044,7 +1130,7 @@ static int launch_train_resident8(const BnGeom& g, const bf16_t* x, bf16_t* y, c
   return check_launch("bn_fwd_train (resident, 8-wide)");
 }
 
-template <int THREADS, int K, bool FUSE>
+template <int THREADS, int K, int FUSE>
 static int launch_bwd_resident8(const BnGeom& g, int need, const bf16_t* x, const bf16_t* dy, bf16_t* dx,
                                 const BnBwdArgs& a, const BnFuseBwd<bf16_t>& fu, hipStream_t s) {
   constexpr int KL = K < RES_KL ? K : RES_KL;
@@ -1061,7 +1147,7 @@ static int launch_bwd_resident8(const BnGeom& g, int need, const bf16_t* x, cons
   return check_launch("bn_bwd (resident, 8-wide)");
 }
 
-template <bool FUSE>
+template <int FUSE>
 static int run_train8(const BnGeom& g, const ResPlan& r, const bf16_t* x, bf16_t* y, const BnTrainArgs& a,
                       const BnFuseFwd<bf16_t>& fu, hipStream_t s) {
   if (r.threads == 256 && r.k == 8) return launch_train_resident8<256, 8, FUSE>(g, x, y, a, fu, s);
@@ -1070,7 +1156,7 @@ static int run_train8(const BnGeom& g, const ResPlan& r, const bf16_t* x, bf16_t
   if (r.k == 16) return launch_train_resident8<1024, 16, FUSE>(g, x, y, a, fu, s);
   return launch_train_resident8<1024, RES_KMAX, FUSE>(g, x, y, a, fu, s);
 }
-template <bool FUSE>
+template <int FUSE>
 static int run_bwd8(const BnGeom& g, const ResPlan& r, const bf16_t* x, const bf16_t* dy, bf16_t* dx,
                     const BnBwdArgs& a, const BnFuseBwd<bf16_t>& fu, hipStream_t s) {
   if (r.threads == 256 && r.k == 8) return launch_bwd_resident8<256, 8, FUSE>(g, r.need, x, dy, dx, a, fu, s);
@@ -1080,7 +1166,7 @@ static int run_bwd8(const BnGeom& g, const ResPlan& r, const bf16_t* x, const bf
   return launch_bwd_resident8<1024, RES_KMAX, FUSE>(g, r.need, x, dy, dx, a, fu, s);
 }
 
-template <typename T, int THREADS, int K, bool FUSE>
+template <typename T, int THREADS, int K, int FUSE>
 static int launch_train_resident(const BnGeom& g, const T* x, T* y, const BnTrainArgs& a,
                                  const BnFuseFwd<T>& fu, hipStream_t s) {
   const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
@@ -1089,7 +1175,7 @@ static int launch_train_resident(const BnGeom& g, const T* x, T* y, const BnTrai
   return check_launch("bn_fwd_train (resident)");
 }
 
-template <typename T, int THREADS, int K, bool FUSE>
+template <typename T, int THREADS, int K, int FUSE>
 static int launch_bwd_resident(const BnGeom& g, int need, const T* x, const T* dy, T* dx,
                                const BnBwdArgs& a, const BnFuseBwd<T>& fu, hipStream_t s) {
   constexpr int KL = K < RES_KL ? K : RES_KL;
@@ -1109,12 +1195,14 @@ static int launch_bwd_resident(const BnGeom& g, int need, const T* x, const T* d
   return check_launch("bn_bwd (resident)");
 }
 
-// FUSE: with the epilogue y = relu(bn(x) + residual) (segment modes only)
-template <typename T, bool FUSE>
+// FUSE: with the epilogue y = relu(bn(x) + residual) (segment modes only); 2: the ReLU's mask is also
+// written as bytes
+template <typename T, int FUSE>
 static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws,
                      const BnTrainArgs& a, const BnFuseFwd<T>& fu, hipStream_t s) {
   const T* xp = static_cast<const T*>(x);
   T* yp = static_cast<T*>(y);
+  constexpr int F1 = FUSE == 2 ? 1 : FUSE;   // element-wise kernels: no mask-byte form (never asked for: vec == 4 only)
   if (sizeof(T) == 2) {
     const ResPlan r8 = resident8_plan(g, vec, FLHIP_BF16, RES_MIN_C_FWD);
     if (r8.threads)
@@ -1127,15 +1215,15 @@ static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws
       const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
       const dim3 grid((unsigned)g.C);
       if (r.threads == 256 && r.k == 8)
-        hipLaunchKernelGGL((bn_train_resident1<T, 256, 8, FUSE>), grid, dim3(256), 0, s, g, bytes, xp, yp, a, fu);
+        hipLaunchKernelGGL((bn_train_resident1<T, 256, 8, F1>), grid, dim3(256), 0, s, g, bytes, xp, yp, a, fu);
       else if (r.threads == 256)
-        hipLaunchKernelGGL((bn_train_resident1<T, 256, 16, FUSE>), grid, dim3(256), 0, s, g, bytes, xp, yp, a, fu);
+        hipLaunchKernelGGL((bn_train_resident1<T, 256, 16, F1>), grid, dim3(256), 0, s, g, bytes, xp, yp, a, fu);
       else if (r.k == 8)
-        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 8, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a, fu);
+        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 8, F1>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a, fu);
       else if (r.k == 16)
-        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 16, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a, fu);
+        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 16, F1>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a, fu);
       else
-        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 32, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a, fu);
+        hipLaunchKernelGGL((bn_train_resident1<T, 1024, 32, F1>), grid, dim3(1024), 0, s, g, bytes, xp, yp, a, fu);
       return check_launch("bn_fwd_train (resident, element-wise)");
     }
     if (r.threads == 256 && r.k == 8) return launch_train_resident<T, 256, 8, FUSE>(g, xp, yp, a, fu, s);
@@ -1159,19 +1247,20 @@ static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws
       hipLaunchKernelGGL((bn_train_apply_seg<T, 4, FUSE>), grid, dim3(256), 0, s, g, xp, yp, ws, a, fu);
     } else {
       hipLaunchKernelGGL((bn_stats_seg<T, 1>), grid, dim3(256), 0, s, g, xp, ws);
-      hipLaunchKernelGGL((bn_train_apply_seg<T, 1, FUSE>), grid, dim3(256), 0, s, g, xp, yp, ws, a, fu);
+      hipLaunchKernelGGL((bn_train_apply_seg<T, 1, F1>), grid, dim3(256), 0, s, g, xp, yp, ws, a, fu);
     }
   }
   return check_launch("bn_fwd_train");
 }
 
-// FUSE: the gradient first passes the ReLU mask of the forward result
-template <typename T, bool FUSE>
+// FUSE: the gradient first passes the ReLU mask of the forward result, read from y (1) or from the mask bytes (2)
+template <typename T, int FUSE>
 static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void* dx, float* ws,
                    const BnBwdArgs& a, const BnFuseBwd<T>& fu, hipStream_t s) {
   const T* xp = static_cast<const T*>(x);
   const T* dyp = static_cast<const T*>(dy);
   T* dxp = static_cast<T*>(dx);
+  constexpr int F1 = FUSE == 2 ? 1 : FUSE;   // element-wise kernels: no mask-byte form (never asked for: vec == 4 only)
   if (sizeof(T) == 2) {
     const ResPlan r8 = resident8_plan(g, vec, FLHIP_BF16, RES_MIN_C_BWD);
     if (r8.threads)
@@ -1184,15 +1273,15 @@ static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void
       const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
       const dim3 grid((unsigned)g.C);
       if (r.threads == 256 && r.k == 8)
-        hipLaunchKernelGGL((bn_bwd_resident1<T, 256, 8, FUSE>), grid, dim3(256), 0, s, g, bytes, xp, dyp, dxp, a, fu);
+        hipLaunchKernelGGL((bn_bwd_resident1<T, 256, 8, F1>), grid, dim3(256), 0, s, g, bytes, xp, dyp, dxp, a, fu);
       else if (r.threads == 256)
-        hipLaunchKernelGGL((bn_bwd_resident1<T, 256, 16, FUSE>), grid, dim3(256), 0, s, g, bytes, xp, dyp, dxp, a, fu);
+        hipLaunchKernelGGL((bn_bwd_resident1<T, 256, 16, F1>), grid, dim3(256), 0, s, g, bytes, xp, dyp, dxp, a, fu);
       else if (r.k == 8)
-        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 8, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a, fu);
+        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 8, F1>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a, fu);
       else if (r.k == 16)
-        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 16, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a, fu);
+        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 16, F1>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a, fu);
       else
-        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 32, FUSE>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a, fu);
+        hipLaunchKernelGGL((bn_bwd_resident1<T, 1024, 32, F1>), grid, dim3(1024), 0, s, g, bytes, xp, dyp, dxp, a, fu);
       return check_launch("bn_bwd (resident, element-wise)");
     }
     if (r.threads == 256 && r.k == 8) return launch_bwd_resident<T, 256, 8, FUSE>(g, r.need, xp, dyp, dxp, a, fu, s);
@@ -1214,8 +1303,8 @@ static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void
       hipLaunchKernelGGL((bn_bwd_stats_seg<T, 4, FUSE>), grid, dim3(256), 0, s, g, xp, dyp, a.save_mean, ws, fu);
       hipLaunchKernelGGL((bn_bwd_apply_seg<T, 4, FUSE>), grid, dim3(256), 0, s, g, xp, dyp, dxp, ws, a, fu);
     } else {
-      hipLaunchKernelGGL((bn_bwd_stats_seg<T, 1, FUSE>), grid, dim3(256), 0, s, g, xp, dyp, a.save_mean, ws, fu);
-      hipLaunchKernelGGL((bn_bwd_apply_seg<T, 1, FUSE>), grid, dim3(256), 0, s, g, xp, dyp, dxp, ws, a, fu);
+      hipLaunchKernelGGL((bn_bwd_stats_seg<T, 1, F1>), grid, dim3(256), 0, s, g, xp, dyp, a.save_mean, ws, fu);
+      hipLaunchKernelGGL((bn_bwd_apply_seg<T, 1, F1>), grid, dim3(256), 0, s, g, xp, dyp, dxp, ws, a, fu);
     }
   }
   return check_launch("bn_bwd");
@@ -1249,8 +1338,38 @@ extern "C" int flhip_bn_fwd_train(const flhip_bn_desc* d, const void* x, const f
   FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_fwd_train: workspace too small");
   const BnTrainArgs a{gamma, beta, save_mean, save_invstd, run_mean, run_var, momentum, eps};
   return d->dtype == FLHIP_F32
-             ? run_train<float, false>(g, vec, x, y, static_cast<float*>(ws), a, BnFuseFwd<float>{nullptr, 0}, as_stream(stream))
-             : run_train<bf16_t, false>(g, vec, x, y, static_cast<float*>(ws), a, BnFuseFwd<bf16_t>{nullptr, 0}, as_stream(stream));
+             ? run_train<float, 0>(g, vec, x, y, static_cast<float*>(ws), a, BnFuseFwd<float>{nullptr, 0, nullptr}, as_stream(stream))
+             : run_train<bf16_t, 0>(g, vec, x, y, static_cast<float*>(ws), a, BnFuseFwd<bf16_t>{nullptr, 0, nullptr}, as_stream(stream));
+}
+
+static int bn_act_fwd_train_impl(const flhip_bn_desc* d, const void* x, const float* gamma,
+                                 const float* beta, const void* residual, int relu, void* y,
+                                 void* mask, bool want_mask, float* save_mean, float* save_invstd,
+                                 float* run_mean, float* run_var, double momentum, double eps,
+                                 void* ws, size_t ws_bytes, void* stream) {
+  BnGeom g;
+  int vec;
+  const int rc = make_geom(d, &g, &vec);
+  if (rc != FLHIP_OK) return rc;
+  FLHIP_REQUIRE(x && y, "bn_act_fwd_train: null tensor");
+  FLHIP_REQUIRE(!want_mask || (mask && vec == 4),
+                "bn_act_fwd_train_mask: needs a mask buffer and rows of a multiple of 4 elements "
+                "(flhip_bn_act_mask_bytes tells)");
+  FLHIP_REQUIRE((run_mean == nullptr) == (run_var == nullptr),
+                "bn_act_fwd_train: running mean and variance must be given together");
+  FLHIP_REQUIRE(momentum >= 0.0 && momentum <= 1.0, "bn_act_fwd_train: momentum must lie in [0, 1]");
+  FLHIP_REQUIRE(eps >= 0.0, "bn_act_fwd_train: epsilon must be non-negative");
+  FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_act_fwd_train: workspace too small");
+  const BnTrainArgs a{gamma, beta, save_mean, save_invstd, run_mean, run_var, momentum, eps};
+  uint8_t* mk = want_mask ? static_cast<uint8_t*>(mask) : nullptr;
+  const BnFuseFwd<float> f32{static_cast<const float*>(residual), relu, mk};
+  const BnFuseFwd<bf16_t> f16{static_cast<const bf16_t*>(residual), relu, mk};
+  float* wsf = static_cast<float*>(ws);
+  if (d->dtype == FLHIP_F32)
+    return mk ? run_train<float, 2>(g, vec, x, y, wsf, a, f32, as_stream(stream))
+              : run_train<float, 1>(g, vec, x, y, wsf, a, f32, as_stream(stream));
+  return mk ? run_train<bf16_t, 2>(g, vec, x, y, wsf, a, f16, as_stream(stream))
+            : run_train<bf16_t, 1>(g, vec, x, y, wsf, a, f16, as_stream(stream));
 }
 
 extern "C" int flhip_bn_act_fwd_train(const flhip_bn_desc* d, const void* x, const float* gamma,
@@ -1258,22 +1377,22 @@ extern "C" int flhip_bn_act_fwd_train(const flhip_bn_desc* d, const void* x, con
                                       float* save_mean, float* save_invstd, float* run_mean,
                                       float* run_var, double momentum, double eps, void* ws,
                                       size_t ws_bytes, void* stream) {
-  BnGeom g;
-  int vec;
-  const int rc = make_geom(d, &g, &vec);
-  if (rc != FLHIP_OK) return rc;
-  FLHIP_REQUIRE(x && y, "bn_act_fwd_train: null tensor");
-  FLHIP_REQUIRE((run_mean == nullptr) == (run_var == nullptr),
-                "bn_act_fwd_train: running mean and variance must be given together");
-  FLHIP_REQUIRE(momentum >= 0.0 && momentum <= 1.0, "bn_act_fwd_train: momentum must lie in [0, 1]");
-  FLHIP_REQUIRE(eps >= 0.0, "bn_act_fwd_train: epsilon must be non-negative");
-  FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_act_fwd_train: workspace too small");
-  const BnTrainArgs a{gamma, beta, save_mean, save_invstd, run_mean, run_var, momentum, eps};
-  return d->dtype == FLHIP_F32
-             ? run_train<float, true>(g, vec, x, y, static_cast<float*>(ws), a,
-                                      BnFuseFwd<float>{static_cast<const float*>(residual), relu}, as_stream(stream))
-             : run_train<bf16_t, true>(g, vec, x, y, static_cast<float*>(ws), a,
-                                       BnFuseFwd<bf16_t>{static_cast<const bf16_t*>(residual), relu}, as_stream(stream));
+  return bn_act_fwd_train_impl(d, x, gamma, beta, residual, relu, y, nullptr, false, save_mean, save_invstd,
+                               run_mean, run_var, momentum, eps, ws, ws_bytes, stream);
+}
+
+extern "C" size_t flhip_bn_act_mask_bytes(const flhip_bn_desc* d) {
+  if (!d || d->outer <= 0 || d->C <= 0 || d->inner <= 1 || d->inner % 4 != 0) return 0;
+  return (size_t)d->outer * (size_t)d->C * (size_t)d->inner / 4;
+}
+
+extern "C" int flhip_bn_act_fwd_train_mask(const flhip_bn_desc* d, const void* x, const float* gamma,
+                                           const float* beta, const void* residual, int relu, void* y,
+                                           void* mask, float* save_mean, float* save_invstd,
+                                           float* run_mean, float* run_var, double momentum, double eps,
+                                           void* ws, size_t ws_bytes, void* stream) {
+  return bn_act_fwd_train_impl(d, x, gamma, beta, residual, relu, y, mask, true, save_mean, save_invstd,
+                               run_mean, run_var, momentum, eps, ws, ws_bytes, stream);
 }
 
 extern "C" int flhip_bn_fwd_infer(const flhip_bn_desc* d, const void* x, const float* gamma,
@@ -1313,27 +1432,49 @@ extern "C" int flhip_bn_bwd(const flhip_bn_desc* d, const void* x, const void* d
   FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_bwd: workspace too small");
   const BnBwdArgs a{gamma, save_mean, save_invstd, dgamma, dbeta};
   return d->dtype == FLHIP_F32
-             ? run_bwd<float, false>(g, vec, x, dy, dx, static_cast<float*>(ws), a, BnFuseBwd<float>{nullptr, nullptr}, as_stream(stream))
-             : run_bwd<bf16_t, false>(g, vec, x, dy, dx, static_cast<float*>(ws), a, BnFuseBwd<bf16_t>{nullptr, nullptr}, as_stream(stream));
+             ? run_bwd<float, 0>(g, vec, x, dy, dx, static_cast<float*>(ws), a, BnFuseBwd<float>{nullptr, nullptr, nullptr}, as_stream(stream))
+             : run_bwd<bf16_t, 0>(g, vec, x, dy, dx, static_cast<float*>(ws), a, BnFuseBwd<bf16_t>{nullptr, nullptr, nullptr}, as_stream(stream));
+}
+
+static int bn_act_bwd_impl(const flhip_bn_desc* d, const void* x, const void* dy, const void* y,
+                           const void* mask, const float* gamma, const float* save_mean,
+                           const float* save_invstd, void* dx, void* dresidual, float* dgamma,
+                           float* dbeta, void* ws, size_t ws_bytes, void* stream) {
+  BnGeom g;
+  int vec;
+  const int rc = make_geom(d, &g, &vec);
+  if (rc != FLHIP_OK) return rc;
+  FLHIP_REQUIRE(x && dy && dx && (y || mask), "bn_act_bwd: null tensor");
+  FLHIP_REQUIRE(!mask || vec == 4, "bn_act_bwd_mask: rows must hold a multiple of 4 elements");
+  FLHIP_REQUIRE(save_mean && save_invstd, "bn_act_bwd: needs the saved statistics of the forward pass");
+  FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_act_bwd: workspace too small");
+  const BnBwdArgs a{gamma, save_mean, save_invstd, dgamma, dbeta};
+  const uint8_t* mk = static_cast<const uint8_t*>(mask);
+  const BnFuseBwd<float> f32{static_cast<const float*>(y), static_cast<float*>(dresidual), mk};
+  const BnFuseBwd<bf16_t> f16{static_cast<const bf16_t*>(y), static_cast<bf16_t*>(dresidual), mk};
+  float* wsf = static_cast<float*>(ws);
+  // FUSE = 1: the mask is read from y, 2: from the mask bytes
+  if (d->dtype == FLHIP_F32)
+    return mk ? run_bwd<float, 2>(g, vec, x, dy, dx, wsf, a, f32, as_stream(stream))
+              : run_bwd<float, 1>(g, vec, x, dy, dx, wsf, a, f32, as_stream(stream));
+  return mk ? run_bwd<bf16_t, 2>(g, vec, x, dy, dx, wsf, a, f16, as_stream(stream))
+            : run_bwd<bf16_t, 1>(g, vec, x, dy, dx, wsf, a, f16, as_stream(stream));
 }
 
 extern "C" int flhip_bn_act_bwd(const flhip_bn_desc* d, const void* x, const void* dy, const void* y,
                                 const float* gamma, const float* save_mean, const float* save_invstd,
                                 void* dx, void* dresidual, float* dgamma, float* dbeta, void* ws,
                                 size_t ws_bytes, void* stream) {
-  BnGeom g;
-  int vec;
-  const int rc = make_geom(d, &g, &vec);
-  if (rc != FLHIP_OK) return rc;
-  FLHIP_REQUIRE(x && dy && dx && y, "bn_act_bwd: null tensor");
-  FLHIP_REQUIRE(save_mean && save_invstd, "bn_act_bwd: needs the saved statistics of the forward pass");
-  FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_act_bwd: workspace too small");
-  const BnBwdArgs a{gamma, save_mean, save_invstd, dgamma, dbeta};
-  return d->dtype == FLHIP_F32
-             ? run_bwd<float, true>(g, vec, x, dy, dx, static_cast<float*>(ws), a,
-                                    BnFuseBwd<float>{static_cast<const float*>(y), static_cast<float*>(dresidual)},
-                                    as_stream(stream))
-             : run_bwd<bf16_t, true>(g, vec, x, dy, dx, static_cast<float*>(ws), a,
-                                     BnFuseBwd<bf16_t>{static_cast<const bf16_t*>(y), static_cast<bf16_t*>(dresidual)},
-                                     as_stream(stream));
+  FLHIP_REQUIRE(y, "bn_act_bwd: null tensor");
+  return bn_act_bwd_impl(d, x, dy, y, nullptr, gamma, save_mean, save_invstd, dx, dresidual, dgamma, dbeta, ws,
+                         ws_bytes, stream);
+}
+
+extern "C" int flhip_bn_act_bwd_mask(const flhip_bn_desc* d, const void* x, const void* dy, const void* mask,
+                                     const float* gamma, const float* save_mean, const float* save_invstd,
+                                     void* dx, void* dresidual, float* dgamma, float* dbeta, void* ws,
+                                     size_t ws_bytes, void* stream) {
+  FLHIP_REQUIRE(mask, "bn_act_bwd_mask: null mask");
+  return bn_act_bwd_impl(d, x, dy, nullptr, mask, gamma, save_mean, save_invstd, dx, dresidual, dgamma, dbeta, ws,
+                         ws_bytes, stream);
 }

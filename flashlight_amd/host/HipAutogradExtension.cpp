@@ -75,6 +75,7 @@ struct HipPool2DPayload : detail::AutogradPayloadData {
 };
 struct HipBatchNormPayload : detail::AutogradPayloadData {
   Tensor saveMean, saveInvStd;   // fp32 per feature
+  Tensor reluMask;               // batchnormRelu: one byte per 4 elements of the result, bit e = (y[4i+e] > 0)
 };
 
 flhip_conv_desc convDesc(const Shape& in, const Tensor& weights, int sx, int sy, int px, int py,
@@ -432,17 +433,29 @@ Tensor HipAutogradExtension::batchnormRelu(Tensor& saveMean, Tensor& saveVar, co
   saveVar = Tensor({nfeat}, dtype::f32);
   const size_t wsBytes = flhip_bn_workspace_bytes(&d);
   Tensor ws = workspace(wsBytes);
+  // with a tape to feed, the ReLU's mask goes along as bits: the backward pass then reads a quarter
+  // of a byte per element instead of the whole result
+  const size_t maskBytes = autogradPayload ? flhip_bn_act_mask_bytes(&d) : 0;
+  Tensor mask = maskBytes ? Tensor({(Dim)maskBytes}, dtype::u8) : Tensor();
   DevicePtr xp(input), gp(gamma), bp(beta), rp(residual), yp(output), rmp(runningMean), rvp(runningVar),
-      smp(saveMean), sip(saveVar), wsp(ws);
-  check(flhip_bn_act_fwd_train(&d, xp.get(), static_cast<const float*>(gp.get()),
-                               static_cast<const float*>(bp.get()), rp.get(), 1, yp.get(),
-                               static_cast<float*>(smp.get()), static_cast<float*>(sip.get()),
-                               static_cast<float*>(rmp.get()), static_cast<float*>(rvp.get()), momentum, epsilon,
-                               wsp.get(), wsBytes, hipBackendStream()));
+      smp(saveMean), sip(saveVar), wsp(ws), mkp(mask);
+  if (maskBytes)
+    check(flhip_bn_act_fwd_train_mask(&d, xp.get(), static_cast<const float*>(gp.get()),
+                                      static_cast<const float*>(bp.get()), rp.get(), 1, yp.get(), mkp.get(),
+                                      static_cast<float*>(smp.get()), static_cast<float*>(sip.get()),
+                                      static_cast<float*>(rmp.get()), static_cast<float*>(rvp.get()), momentum,
+                                      epsilon, wsp.get(), wsBytes, hipBackendStream()));
+  else
+    check(flhip_bn_act_fwd_train(&d, xp.get(), static_cast<const float*>(gp.get()),
+                                 static_cast<const float*>(bp.get()), rp.get(), 1, yp.get(),
+                                 static_cast<float*>(smp.get()), static_cast<float*>(sip.get()),
+                                 static_cast<float*>(rmp.get()), static_cast<float*>(rvp.get()), momentum, epsilon,
+                                 wsp.get(), wsBytes, hipBackendStream()));
   if (autogradPayload) {
     auto payload = std::make_shared<HipBatchNormPayload>();
     payload->saveMean = saveMean;
     payload->saveInvStd = saveVar;
+    payload->reluMask = mask;
     autogradPayload->data = payload;
   }
   // event: inputs {input, gamma, beta, runningMean, runningVar, residual (may be empty)}, outputs {output, saveMean,
@@ -458,12 +471,13 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> HipAutogradExtension::batchnormReluBa
     const Tensor& input, const Tensor& weight, const std::vector<int>& axes, const bool wantResidualGrad,
     std::shared_ptr<detail::AutogradPayload> autogradPayload) {
   detail::OpScope scope("batchnormReluBackward");
-  Tensor mean = saveMean, invstd = saveVar;
+  Tensor mean = saveMean, invstd = saveVar, mask;
   if (autogradPayload && autogradPayload->data) {
     auto payload = std::dynamic_pointer_cast<HipBatchNormPayload>(autogradPayload->data);
     if (!payload) throw std::invalid_argument("batchnormReluBackward: payload of another operation");
     mean = payload->saveMean;
     invstd = payload->saveInvStd;
+    mask = payload->reluMask;
   }
   if (mean.isEmpty() || invstd.isEmpty())
     throw std::invalid_argument("HipAutogradExtension::batchnormReluBackward given null or empty payload");
@@ -479,11 +493,20 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> HipAutogradExtension::batchnormReluBa
   const size_t wsBytes = flhip_bn_workspace_bytes(&d);
   Tensor ws = workspace(wsBytes);
   DevicePtr xp(input), dyp(gradOutput), yp(output), gp(gamma), mp(mean), ip(invstd), dxp(gradInput),
-      drp(gradResidual), dgp(gradWeight), dbp(gradBias), wsp(ws);
-  check(flhip_bn_act_bwd(&d, xp.get(), dyp.get(), yp.get(), static_cast<const float*>(gp.get()),
-                         static_cast<const float*>(mp.get()), static_cast<const float*>(ip.get()), dxp.get(),
-                         drp.get(), static_cast<float*>(dgp.get()), static_cast<float*>(dbp.get()), wsp.get(),
-                         wsBytes, hipBackendStream()));
+      drp(gradResidual), dgp(gradWeight), dbp(gradBias), wsp(ws), mkp(mask);
+  if (!mask.isEmpty()) {
+    if ((size_t)mask.elements() != flhip_bn_act_mask_bytes(&d))
+      throw std::invalid_argument("batchnormReluBackward: payload of another call");
+    check(flhip_bn_act_bwd_mask(&d, xp.get(), dyp.get(), mkp.get(), static_cast<const float*>(gp.get()),
+                                static_cast<const float*>(mp.get()), static_cast<const float*>(ip.get()), dxp.get(),
+                                drp.get(), static_cast<float*>(dgp.get()), static_cast<float*>(dbp.get()), wsp.get(),
+                                wsBytes, hipBackendStream()));
+  } else {
+    check(flhip_bn_act_bwd(&d, xp.get(), dyp.get(), yp.get(), static_cast<const float*>(gp.get()),
+                           static_cast<const float*>(mp.get()), static_cast<const float*>(ip.get()), dxp.get(),
+                           drp.get(), static_cast<float*>(dgp.get()), static_cast<float*>(dbp.get()), wsp.get(),
+                           wsBytes, hipBackendStream()));
+  }
   // event: inputs {gradOutput, input, gamma, saveMean, saveInvStd, output}, outputs {gradInput, gradWeight,
   // gradBias, gradResidual (may be empty)}, ints {outer, features, inner}
   if (scope.on())

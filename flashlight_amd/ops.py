@@ -291,9 +291,11 @@ def batchnorm_backward(grad_output, input, weight, save_mean, save_invstd, axes)
 
 
 def batchnorm_relu(input, weight, bias, running_mean, running_var, axes, momentum, epsilon,
-                   residual=None, relu=True):
+                   residual=None, relu=True, want_mask=False):
     """flhip_bn_act_fwd_train: relu(batchnorm(input) + residual) in train mode, one pass over
-    the tensor -> (output, saveMean, saveInvStd).  residual is optional."""
+    the tensor -> (output, saveMean, saveInvStd).  residual is optional.  want_mask: through
+    flhip_bn_act_fwd_train_mask, with a fourth result, the ReLU's mask as bytes (one per 4
+    elements) for batchnorm_relu_backward; rows must hold a multiple of 4 elements."""
     x = _dev(input, "input")
     outer, Cc, inner = bn_view(x.shape, axes)
     d = capi.BnDesc(outer, Cc, inner, _dtype_tag(x))
@@ -306,20 +308,33 @@ def batchnorm_relu(input, weight, bias, running_mean, running_var, axes, momentu
     si = torch.empty((Cc,), dtype=torch.float32, device=x.device)
     nws = capi.lib().flhip_bn_workspace_bytes(C.byref(d))
     ws = _ws(nws, x.device)
+    rm, rv = _dev(running_mean, "runningMean"), _dev(running_var, "runningVar")
+    if want_mask:
+        nmask = capi.lib().flhip_bn_act_mask_bytes(C.byref(d))
+        if nmask == 0:
+            raise ValueError("batchnormRelu: the mask form needs rows of a multiple of 4 elements")
+        mask = torch.empty((nmask,), dtype=torch.uint8, device=x.device)
+        capi.check(capi.lib().flhip_bn_act_fwd_train_mask(
+            C.byref(d), _ptr(x), _ptr(g), _ptr(b), _ptr(r), int(bool(relu)), _ptr(y), _ptr(mask), _ptr(sm),
+            _ptr(si), _ptr(rm), _ptr(rv), float(momentum), float(epsilon), _ptr(ws), nws, _stream()))
+        return y, sm, si, mask
     capi.check(capi.lib().flhip_bn_act_fwd_train(
         C.byref(d), _ptr(x), _ptr(g), _ptr(b), _ptr(r), int(bool(relu)), _ptr(y), _ptr(sm), _ptr(si),
-        _ptr(_dev(running_mean, "runningMean")), _ptr(_dev(running_var, "runningVar")),
-        float(momentum), float(epsilon), _ptr(ws), nws, _stream()))
+        _ptr(rm), _ptr(rv), float(momentum), float(epsilon), _ptr(ws), nws, _stream()))
     return y, sm, si
 
 
 def batchnorm_relu_backward(grad_output, input, output, weight, save_mean, save_invstd, axes,
-                            want_residual_grad=False):
+                            want_residual_grad=False, mask=None):
     """flhip_bn_act_bwd -> (gradInput, gradWeight, gradBias, gradResidual or None): the
-    gradient passes the ReLU mask of `output` (the forward result), then batchnormBackward."""
+    gradient passes the ReLU mask of `output` (the forward result), then batchnormBackward.
+    With `mask` (the fourth result of batchnorm_relu(want_mask=True)) the call goes through
+    flhip_bn_act_bwd_mask and `output` is not read (it may be None)."""
     g, x, y = _dev(grad_output, "gradOutput"), _dev(input, "input"), _dev(output, "output")
-    if g.dtype != x.dtype or g.shape != x.shape or y.dtype != x.dtype or y.shape != x.shape:
-        raise ValueError("batchnormReluBackward: gradOutput and output must match the input")
+    if g.dtype != x.dtype or g.shape != x.shape:
+        raise ValueError("batchnormReluBackward: gradOutput must match the input")
+    if mask is None and (y is None or y.dtype != x.dtype or y.shape != x.shape):
+        raise ValueError("batchnormReluBackward: output must match the input")
     outer, Cc, inner = bn_view(x.shape, axes)
     d = capi.BnDesc(outer, Cc, inner, _dtype_tag(x))
     w = _f32vec(weight, Cc, "weight")
@@ -329,6 +344,14 @@ def batchnorm_relu_backward(grad_output, input, output, weight, save_mean, save_
     db = torch.empty((Cc,), dtype=torch.float32, device=x.device)
     nws = capi.lib().flhip_bn_workspace_bytes(C.byref(d))
     ws = _ws(nws, x.device)
+    if mask is not None:
+        m = _dev(mask, "mask")
+        if m.dtype != torch.uint8 or m.numel() != capi.lib().flhip_bn_act_mask_bytes(C.byref(d)) or m.numel() == 0:
+            raise ValueError("batchnormReluBackward: the mask must be the byte tensor of the forward call")
+        capi.check(capi.lib().flhip_bn_act_bwd_mask(C.byref(d), _ptr(x), _ptr(g), _ptr(m), _ptr(w), _ptr(save_mean),
+                                                    _ptr(save_invstd), _ptr(dx), _ptr(dr), _ptr(dg), _ptr(db),
+                                                    _ptr(ws), nws, _stream()))
+        return dx, dg, db, dr
     capi.check(capi.lib().flhip_bn_act_bwd(C.byref(d), _ptr(x), _ptr(g), _ptr(y), _ptr(w), _ptr(save_mean),
                                            _ptr(save_invstd), _ptr(dx), _ptr(dr), _ptr(dg), _ptr(db),
                                            _ptr(ws), nws, _stream()))

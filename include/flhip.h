@@ -113,7 +113,7 @@ const char* flhip_arch(void);
  * called while another thread is inside the library.  Results stay within the stated
  * tolerances under every setting; the switches only choose between kernels.
  *   CONV_ALGO = direct | gather | tapped | convert | auto    CONV_SKIP = bf16,gemm1x1,slab,tapped,strip,first,wgrad128,pwdma
- *   PW_PT = 2 | 4 | 8    PW16_PF = 0 | 1 | 2 | 4 | 8    CONV_STACK = 0 | 1 | 2 | 4 | 8    BN_ALGO = split | resident | auto
+ *   PW_PT = 2 | 4 | 8    PW16_PF = 0 | 1 | 2 | 4 | 8    CONV_ROWS = 0 .. 64    CONV_STACK = 0 | 1 | 2 | 4 | 8    BN_ALGO = split | resident | auto
  *   PW16_NO_TAPS, TAPPED_NO_REORDER, MATMUL_VALU, RNN_UNFUSED = 1 | 0
  * Unknown names or values return FLHIP_INVALID_ARGUMENT.  The nearest thing in the
  * reference is the kernel-choice options object of its cuDNN extension
@@ -247,6 +247,24 @@ int flhip_bn_act_bwd(const flhip_bn_desc* d, const void* x, const void* dy, cons
                      const float* gamma, const float* save_mean, const float* save_invstd,
                      void* dx, void* dresidual, float* dgamma, float* dbeta, void* ws,
                      size_t ws_bytes, void* stream);
+
+/* The same pair with the ReLU's mask kept as bits instead of read back from y: the forward
+ * call also writes one byte per 4 consecutive elements (bit e of byte i set where
+ * y[4*i + e] > 0), the backward call reads those bytes in place of y: a quarter of a byte
+ * per element instead of the 2 or 4 bytes of the forward result.  Rows must hold a
+ * multiple of 4 elements (inner % 4 == 0): flhip_bn_act_mask_bytes gives the size of the
+ * mask buffer, 0 where this form does not apply.  The gradients equal flhip_bn_act_bwd's bit
+ * for bit.  Like the pair above, no counterpart in the reference. */
+size_t flhip_bn_act_mask_bytes(const flhip_bn_desc* d);
+int flhip_bn_act_fwd_train_mask(const flhip_bn_desc* d, const void* x, const float* gamma,
+                                const float* beta, const void* residual, int relu, void* y,
+                                void* mask, float* save_mean, float* save_invstd,
+                                float* run_mean, float* run_var, double momentum, double eps,
+                                void* ws, size_t ws_bytes, void* stream);
+int flhip_bn_act_bwd_mask(const flhip_bn_desc* d, const void* x, const void* dy, const void* mask,
+                          const float* gamma, const float* save_mean, const float* save_invstd,
+                          void* dx, void* dresidual, float* dgamma, float* dbeta, void* ws,
+                          size_t ws_bytes, void* stream);
 
 /* Storage conversion between FLHIP_F32 and FLHIP_BF16 (round to nearest even) of n
  * elements; same dtype = copy.  Serves the casts the caller closures make around

@@ -234,6 +234,22 @@ def test_fused_bn_relu(shape, axes, with_residual, dtype):
     assert rel_l2(host(dg), dg_ref) <= 1e-4 and rel_l2(host(db), db_ref) <= 1e-4
     if with_residual:
         assert np.array_equal(host(dr), dz_ref.reshape(shape))
+    # the same pair with the ReLU's mask kept as one byte per 4 elements: same forward result, the
+    # bytes hold y > 0 bit by bit, and the backward pass that reads them gives the same bits as
+    # the one that reads y
+    args = (dev(x, dtype), dev(gamma), dev(beta), None, None, axes, 0.1, 1e-5, None if res is None else dev(res, dtype))
+    if inner % 4 == 0:
+        ym, _, _, mask = ops.batchnorm_relu(*args, want_mask=True)
+        assert torch.equal(ym, y)
+        bits = (yh.reshape(-1, 4) > 0).astype(np.uint8)
+        assert np.array_equal(mask.cpu().numpy(), bits[:, 0] | bits[:, 1] << 1 | bits[:, 2] << 2 | bits[:, 3] << 3)
+        got = ops.batchnorm_relu_backward(dev(dy, dtype), dev(x, dtype), None, dev(gamma), sm, si, axes,
+                                          want_residual_grad=with_residual, mask=mask)
+        for a, b in zip(got, (dx, dg, db, dr)):
+            assert (a is None and b is None) or torch.equal(a, b)
+    else:
+        with pytest.raises(ValueError):
+            ops.batchnorm_relu(*args, want_mask=True)
     # relu == 0: batch norm plus residual only
     y2, _, _ = ops.batchnorm_relu(dev(x, dtype), dev(gamma), dev(beta), None, None, axes, 0.1, 1e-5,
                                   None if res is None else dev(res, dtype), relu=False)
