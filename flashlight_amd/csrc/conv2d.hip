@@ -193,7 +193,9 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
     // the larger of the two filter-gradient plans, so either kernel can run
     size_t a = mfma_conv_bwd_filter_ws(g, d->dtype);
     const size_t b = mfma_slab_wgrad_ws(g, d->dtype);
-    const size_t c = d->dtype == FLHIP_BF16 ? mfma_wgrad16_ws(g) : 0;
+    size_t c = d->dtype == FLHIP_BF16 ? mfma_wgrad16_ws(g) : 0;
+    const size_t c2 = d->dtype == FLHIP_BF16 ? mfma_wgrad_dma16_ws(g) : 0;
+    if (c2 > c) c = c2;
     const size_t e = mfma_pointwise_wgrad_ws(g);
     const size_t f = d->dtype == FLHIP_BF16 ? mfma_pointwise16_wgrad_ws(g) : 0;
     const size_t h = d->dtype == FLHIP_BF16 ? mfma_first16_wgrad_ws(g) : 0;
@@ -332,6 +334,8 @@ extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, 
       r = mfma_pointwise16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_FIRST) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_first16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_wgrad_dma16(g, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_wgrad16(g, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0 && !skip(SK_GEMM))

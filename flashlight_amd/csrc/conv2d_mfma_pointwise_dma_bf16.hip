@@ -34,14 +34,13 @@
 #include <algorithm>
 
 #include "conv2d_mfma.h"
+#include "lds_direct.h"
 
 namespace flhip {
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short shortx4_t __attribute__((ext_vector_type(4)));
-typedef int intx4_t __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) void* lds_void_t;
 typedef __attribute__((address_space(3))) shortx4_t* lds_tr_t;
 
 constexpr int PD_KC = 32;                          // contraction channels per stage
@@ -86,7 +85,6 @@ __device__ __forceinline__ uint32_t pd_add_bf16x2(uint32_t a, uint32_t b) {
                    __uint_as_float(a & 0xffff0000u) + __uint_as_float(b & 0xffff0000u));
 }
 
-#define PD_WAIT_VM(N) asm volatile("s_waitcnt vmcnt(" #N ")" ::: "memory")
 // at most N of this wave's loads outstanding
 template <int N>
 __device__ __forceinline__ void pd_wait_loads() {
@@ -100,22 +98,6 @@ __device__ __forceinline__ void pd_wait_loads() {
   if (N == 18) PD_WAIT_VM(18);
   if (N == 20) PD_WAIT_VM(20);
   if (N == 24) PD_WAIT_VM(24);
-}
-
-// raw buffer descriptor (the words of make_rsrc) as four scalars for the inline assembly below
-__device__ __forceinline__ intx4_t pd_rsrc(const void* ptr, unsigned bytes) {
-  const uint64_t a = reinterpret_cast<uint64_t>(ptr);
-  return intx4_t{__builtin_amdgcn_readfirstlane((int)(uint32_t)a),
-                 __builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xffffu)),
-                 __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
-}
-// 64 lanes x 16 bytes from rsrc + voff (per lane) + soff to the 1 KiB of LDS at lds_addr (workgroup
-// address, the same for all lanes): lane l lands at lds_addr + 16 l.  m0 is not declared as clobbered (the
-// compiler reserves it and warns); nothing else in these kernels uses it: no LDS-load builtin, no
-// relative register moves, no messages.
-__device__ __forceinline__ void pd_load_lds(intx4_t rsrc, unsigned lds_addr, int voff, int soff) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-               :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 }
 
 template <bool BWD, int PD_NS, int BM>

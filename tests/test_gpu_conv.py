@@ -256,6 +256,42 @@ def test_bf16_1x1_filter_gradient_alone(xs, K):
     assert rel_l2(host(dw2), dw_ref) <= 1e-4
 
 
+# bf16 3x3 filter gradient with at least 64 channels on both sides: the kernel whose operand rows the loads
+# copy straight to LDS.  Rows of 8k positions and rows whose last cell repeats positions (28, 14, 12, 20, 9:
+# zeroed in the input rows); two or four 16-position steps per row; ranges of rows that start and end inside an
+# image and that span several images; several tiles; with and without the bias gradient (dy times ones, the
+# repeated positions counted once).
+@pytest.mark.parametrize("with_bias", [False, True])
+@pytest.mark.parametrize("xs,K", [
+    ((2, 64, 56, 56), 64), ((3, 64, 28, 28), 128), ((5, 128, 14, 14), 64), ((7, 64, 5, 12), 64),
+    ((2, 128, 9, 20), 128), ((1, 64, 3, 8), 64), ((9, 64, 4, 9), 64), ((2, 64, 6, 40), 64), ((1, 64, 1, 64), 64),
+    ((70, 64, 7, 16), 64),
+])
+def test_bf16_3x3_filter_gradient_rows_to_lds(xs, K, with_bias):
+    rng = np.random.default_rng(xs[0] * 17 + xs[3] + K)
+    ws = (K, xs[1], 3, 3)
+    x = bf16_round(rng.standard_normal(xs).astype(np.float32))
+    dy = bf16_round(rng.standard_normal((xs[0], K, xs[2], xs[3])).astype(np.float32))
+    d = flref.conv_desc(xs, ws, (1, 1), (1, 1), (1, 1), 1)
+    dw_ref, db_ref = flref.conv2d_bwd_filter(d, x, dy)
+    from flashlight_amd import capi
+    capi.set_option("PW16_PF", 1)            # also on the short rows the dispatch leaves to the older kernel
+    try:
+        dw, db = fa.conv2d_backward_filter_bias(dev(dy, torch.bfloat16), dev(x, torch.bfloat16), ws, with_bias, px=1, py=1)
+    finally:
+        capi.set_option("PW16_PF", None)
+    assert rel_l2(host(dw), dw_ref) <= 1e-4, rel_l2(host(dw), dw_ref)
+    if with_bias:
+        assert rel_l2(host(db), db_ref) <= 1e-4, rel_l2(host(db), db_ref)
+    # the same through the kernel with register staging
+    capi.set_option("CONV_SKIP", "pwdma")
+    try:
+        dw2, _ = fa.conv2d_backward_filter_bias(dev(dy, torch.bfloat16), dev(x, torch.bfloat16), ws, False, px=1, py=1)
+    finally:
+        capi.set_option("CONV_SKIP", None)
+    assert rel_l2(host(dw2), dw_ref) <= 1e-4
+
+
 # bf16 3x3 kernel with several images per tile (planes that fit a tile whole, stacked with one shared zero
 # row between them; the dispatch does this when single images would make more than one round of workgroups):
 # 2 and 4 images of 7x7 / 5x6 / 8x8 planes per tile, an image count that leaves the last tile short, a filter tail.
