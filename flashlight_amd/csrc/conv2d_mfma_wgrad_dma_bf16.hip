@@ -373,15 +373,17 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
   WD_STAMP(8)
 }
 
-// part[split][tap][K][C] (+ [K] bias sums) -> dw[K][C][tap], db[K]; the splits are added in a fixed order
-constexpr int WD_RTY = 16;
-__global__ void __launch_bounds__(64 * WD_RTY)
+// part[split][tap][K][C] (+ [K] bias sums) -> dw[K][C][tap], db[K]; the splits are added in a fixed order.
+// A workgroup of 16 x 16 threads owns 64 consecutive elements (16 threads x 4), its 16 rows of threads share the
+// splits: small workgroups, so that a gradient of 36864 elements still spreads over every CU.
+constexpr int WD_RTX = 16, WD_RTY = 16;
+__global__ void __launch_bounds__(WD_RTX * WD_RTY)
 wgrad_taps_reduce_kernel(const float* __restrict__ part, int nsplit, int K, int C, int want_db,
                          float* __restrict__ dw, float* __restrict__ db) {
-  __shared__ float4 red[WD_RTY][64];
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  __shared__ float4 red[WD_RTY][WD_RTX];
+  const int tx = threadIdx.x % WD_RTX, ty = threadIdx.x / WD_RTX;
   const int E = K * C * 9;
-  const int e = (blockIdx.x * 64 + tx) * 4;
+  const int e = (blockIdx.x * WD_RTX + tx) * 4;
   const int total = E + (want_db ? K : 0);
   const size_t stride = (size_t)E + K;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -484,7 +486,7 @@ int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw
   else WD_LAUNCH(4)
 #undef WD_LAUNCH
   const int total = p.E + (p.want_db ? p.K : 0);
-  hipLaunchKernelGGL(wgrad_taps_reduce_kernel, dim3((total + 255) / 256), dim3(64 * WD_RTY), 0, s, part, p.nsplit, p.K,
+  hipLaunchKernelGGL(wgrad_taps_reduce_kernel, dim3((total + 4 * WD_RTX - 1) / (4 * WD_RTX)), dim3(WD_RTX * WD_RTY), 0, s, part, p.nsplit, p.K,
                      p.C, p.want_db, dw, db);
   return check_launch("conv2d_bwd_filter 3x3 (bf16 mfma, direct-to-LDS)");
 }
