@@ -15,8 +15,9 @@
 //   sum_ow dy[ow] x[ow + kw - 1] = sum_iw D_kw[iw] x[iw],   D_kw[iw] = dy[iw - kw + 1]
 // (zero outside the row).  D_1 is the dy row as loaded; D_0 and D_2 are made from it by an
 // LDS -> LDS pass (a 16-byte cell and one element of its neighbour, shifted by v_alignbit), two
-// stages ahead of the multiplications.  Nine accumulator tiles (kh, kw) of 32 x 32 per wave,
-// waves 2 (result channels) x 2 (input channels); a row is 2 or 4 steps of 16 positions.
+// stages ahead of the multiplications.  Nine accumulator tiles (kh, kw) of 32 x 32 per wave;
+// the tile is 2 (result channels) x 2 (input channels) such blocks, two waves per block; a row is
+// 2 or 4 steps of 16 positions.
 //
 // Rows of W positions are cut into cells of 8 (16 bytes); when W is not a multiple of 8 the
 // last cell ENDS at the row's last position and repeats positions of the cell before it; the
@@ -97,33 +98,43 @@ namespace {
 #define WD_STAMP(i) {}
 #endif
 
+// NK16: steps of 16 positions per row (2 or 4).  Eight waves: two per 32 x 32 block of the tile (and per SIMD), which
+// take alternate steps of a row and add their accumulators through LDS at the end: while one of them shifts,
+// computes addresses or waits for LDS, the other one's matrix instructions run (one wave per block: 1.3 us per row
+// of 56 positions instead of 1.15).
+constexpr int NW = 8;
 template <int NK16>
-__global__ void __launch_bounds__(256, 1)
+__global__ void __launch_bounds__(64 * NW, 1)
 wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy, float* __restrict__ out) {
+  static_assert(NK16 == 2 || NK16 == 4, "shapes in use");
   extern __shared__ __align__(16) char wd_lds[];
   char* const dring = wd_lds;                                   // [WD_NSD] dy rows
   char* const xring = wd_lds + WD_NSD * WD_SLOT;                // [WD_NSX] input rows
   char* const shift = wd_lds + (WD_NSD + WD_NSX) * WD_SLOT;     // [WD_NSH buffers][D_0, D_2]
   constexpr int OOB = (int)0x80000000;
+  constexpr int THREADS = 64 * NW;
   constexpr int NCU = 2 * NK16;                                 // cells of a row that the multiplications read
+  constexpr int NLB = 8 / NW;                                   // 8-row blocks of a slot that a wave loads
+  constexpr int NSW = NK16 * 4 / NW;                            // steps of a row per wave
   const int split = blockIdx.x, mtile = blockIdx.y / p.ctiles, ctile = blockIdx.y - mtile * p.ctiles;
   const int m0 = mtile * WD_T, c0 = ctile * WD_T;
   const int tid = threadIdx.x, lane = tid & 63, fr = lane & 31, fh = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave >> 1, wn = wave & 1;
+  const int blk = wave & 3, half = wave >> 2;                   // block of the tile; which steps of a row
+  const int wm = blk >> 1, wn = blk & 1;
   const int row_begin = split * p.rps, nrows = min(row_begin + p.rps, p.total_rows) - row_begin;
   const intx4_t drs = pd_rsrc(dy, p.dy_bytes), xrs = pd_rsrc(x, p.x_bytes);
   const int P = p.H * p.W;
 
-  // ---- loads: instruction i (0, 1) of a wave fills rows 8 (4 i + wave) .. + 7 of a slot; lane -> row + lane / 8, LDS
+  // ---- loads: instruction i of a wave fills rows 8 (NW i + wave) .. + 7 of a slot; lane -> row + lane / 8, LDS
   // cell lane % 8, i.e. the row's cell (lane % 8) ^ (lane / 8)
   const int lrow = lane >> 3, lcell = (lane & 7) ^ lrow;
   const bool cell_ok = lcell < p.ncell;
   const int lpos = lcell == p.ncell - 1 ? p.W - 8 : 8 * lcell;  // first position of the lane's cell
-  int xoff[2], doff[2];
+  int xoff[NLB], doff[NLB];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int r = 8 * (4 * i + wave) + lrow;
+  for (int i = 0; i < NLB; ++i) {
+    const int r = 8 * (NW * i + wave) + lrow;
     xoff[i] = cell_ok ? ((c0 + r) * P + lpos) * 2 : OOB;
     doff[i] = cell_ok ? ((m0 + r) * P + lpos) * 2 : OOB;
   }
@@ -145,10 +156,10 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
     const bool x_in = ih >= 0 && ih < p.H;
     const int xs = (img * p.C * p.H + ih) * p.W * 2, ds = (img * p.K * p.H + oh) * p.W * 2;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      pd_load_lds(xrs, lds0 + (WD_NSD + islot_x) * WD_SLOT + (4 * i + wave) * 1024,
+    for (int i = 0; i < NLB; ++i) {
+      pd_load_lds(xrs, lds0 + (WD_NSD + islot_x) * WD_SLOT + (NW * i + wave) * 1024,
                   (x_in && xoff[i] != OOB) ? xoff[i] + xs : OOB, 0);
-      pd_load_lds(drs, lds0 + islot_d * WD_SLOT + (4 * i + wave) * 1024, (rows && doff[i] != OOB) ? doff[i] + ds : OOB, 0);
+      pd_load_lds(drs, lds0 + islot_d * WD_SLOT + (NW * i + wave) * 1024, (rows && doff[i] != OOB) ? doff[i] + ds : OOB, 0);
     }
     islot_d = islot_d + 1 == WD_NSD ? 0 : islot_d + 1;
     islot_x = islot_x + 1 == WD_NSX ? 0 : islot_x + 1;
@@ -158,8 +169,8 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
   auto fix_tail = [&](int xs) {
     if (p.dup != 0 && lcell == p.ncell - 1) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        char* q = xring + xs * WD_SLOT + (4 * i + wave) * 1024 + lane * 16;
+      for (int i = 0; i < NLB; ++i) {
+        char* q = xring + xs * WD_SLOT + (NW * i + wave) * 1024 + lane * 16;
         int d = p.dup, at = 0;
         if (d >= 4) {
           *reinterpret_cast<uintx2_t*>(q) = uintx2_t{0u, 0u};
@@ -177,16 +188,16 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
   };
 
   // ---- the two shifted copies of a dy row: a thread makes cells (row, cell) = (idx / NCU, idx % NCU),
-  // idx = tid + 256 i.  D_0 = positions + 1 (the element after the cell comes from the next cell, zero past the
+  // idx = tid + THREADS i.  D_0 = positions + 1 (the element after the cell comes from the next cell, zero past the
   // row), D_2 = positions - 1 (the element before it from the cell before, zero before the row).  The reads of
   // a stage are issued in one go and the results written later, so the multiplications in between hide them.
-  constexpr int NSH = (WD_T * NCU + 255) / 256;
+  constexpr int NSH = (WD_T * NCU + THREADS - 1) / THREADS;
   int sh_cell[NSH], sh_nx[NSH], sh_pv[NSH];      // byte offsets in a slot: the cell, the element after it, the one before
   unsigned sh_skip[NSH];                          // elements at the head of the cell that repeat positions (bias sums)
   bool sh_on[NSH], sh_has_nx[NSH], sh_has_pv[NSH];
 #pragma unroll
   for (int i = 0; i < NSH; ++i) {
-    const int idx = tid + 256 * i;
+    const int idx = tid + THREADS * i;
     const int r = (idx / NCU) & (WD_T - 1), c = idx % NCU, sw = r & 7;
     const bool in = c < p.ncell;
     const int pos = c == p.ncell - 1 ? p.W - 8 : 8 * c;
@@ -243,11 +254,14 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
     }
   };
 
-  // ---- fragments: lane -> row fr of a 32-row block, k-octet fh of a 16-position step
-  static_assert(NK16 == 2 || NK16 == 4, "an even number of steps: a stage starts on fragment set 0");
-  int foff[NK16];                       // byte offset of the lane's cell of step s in its row
+  // ---- fragments: lane -> row fr of a 32-row block, k-octet fh of a 16-position step; the wave's step j of a row
+  // is step half + 2 j
+  int foff[NSW];                        // byte offset of the lane's cell of step j in its row
 #pragma unroll
-  for (int s = 0; s < NK16; ++s) foff[s] = ((2 * s + fh) ^ (fr & 7)) * 16;
+  for (int j = 0; j < NSW; ++j) {
+    const int sstep = half + 2 * j;
+    foff[j] = ((2 * sstep + fh) ^ (fr & 7)) * 16;
+  }
   const int arow = (wm * 32 + fr) * 128, brow = (wn * 32 + fr) * 128;
   floatx16 acc[3][3];
 #pragma unroll
@@ -261,12 +275,13 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
   if (nrows > 0) {
     // Stage t multiplies while: the loads of stage t + 1 + D are issued, the shifted copies of stage t + 2 are made
     // (its loads are waited for before the barrier of iteration t), and the fragments of stage t + 1's first step
-    // are fetched behind the last products of stage t.  Every wave issues 4 loads per stage.
-    static_assert(WD_D == 3, "the load counts below: 4 loads per stage and wave");
+    // are fetched behind the last products of stage t.  Every wave issues 2 NLB loads per stage.
+    static_assert(WD_D == 3, "the load counts below");
 #pragma unroll
     for (int st = 0; st <= WD_D; ++st)
       if (st < nstages) issue();
-    if (WD_D + 1 <= nstages) PD_WAIT_VM(8);          // stages 2 .. D may be outstanding: 0 and 1 have landed
+    static_assert(NLB == 1, "two loads per stage and wave");
+    if (WD_D + 1 <= nstages) PD_WAIT_VM(4);           // stages 2 .. D may be outstanding: 0 and 1 have landed
     else PD_WAIT_VM(0);
     fix_tail(0);
     fix_tail(1);
@@ -279,14 +294,14 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
       if (nstages > 1) m1_ = gc.next(p.H, &img, &ih);
     }
     bf16x8 fa[2][3], fb[2][3];
-#define WD_FRAGS(SET, S, D0, D1, B0, B1, B2)                                                           \
+#define WD_FRAGS(SET, J, D0, D1, B0, B1, B2)                                                           \
   {                                                                                                    \
-    fa[SET][0] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((D0) + foff[S]));       \
-    fa[SET][1] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((D1) + foff[S]));       \
-    fa[SET][2] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((D0) + WD_SLOT + foff[S])); \
-    fb[SET][0] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((B0) + foff[S]));       \
-    fb[SET][1] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((B1) + foff[S]));       \
-    fb[SET][2] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((B2) + foff[S]));       \
+    fa[SET][0] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((D0) + foff[J]));       \
+    fa[SET][1] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((D1) + foff[J]));       \
+    fa[SET][2] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((D0) + WD_SLOT + foff[J])); \
+    fb[SET][0] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((B0) + foff[J]));       \
+    fb[SET][1] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((B1) + foff[J]));       \
+    fb[SET][2] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((B2) + foff[J]));       \
   }
 #define WD_MULT(SET)                                                                                   \
   _Pragma("unroll") for (int kh = 0; kh < 3; ++kh)                                                     \
@@ -297,7 +312,7 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
       const int nd2 = nd + 1 == WD_NSD ? 0 : nd + 1, nx2 = nx + 1 == WD_NSX ? 0 : nx + 1, nb2 = nb + 1 == WD_NSH ? 0 : nb + 1;
       m2_ = false;
       if (t + 2 < nstages) {
-        if (t + 1 + WD_D <= nstages) PD_WAIT_VM(4);      // stages t + 3 .. t + D may be outstanding
+        if (t + 1 + WD_D <= nstages) PD_WAIT_VM(2);     // stages t + 3 .. t + D may be outstanding
         else PD_WAIT_VM(0);
         fix_tail(nx2);
         int img, ih;
@@ -316,21 +331,30 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
       const char* e1 = dring + nd * WD_SLOT + arow;
       const char* e0 = shift + nb * 2 * WD_SLOT + arow;
       const char* c2 = xring + nx * WD_SLOT + brow;
-      if (m0_) {
-        // (set 0 holds step 0: fetched at the end of the iteration before)
-        WD_FRAGS(1, 1, d0, d1, b0, b1, b2)
-        WD_MULT(0)
-      }
-      if (m2_) shift_writes(nb2);
-      if (m0_) {
-#pragma unroll
-        for (int s = 1; s < NK16; ++s) {
-          if (s + 1 < NK16) WD_FRAGS((s + 1) & 1, (s + 1 < NK16 ? s + 1 : 0), d0, d1, b0, b1, b2)
-          else if (m1_) WD_FRAGS(0, 0, e0, e1, b1, b2, c2)
-          WD_MULT(s & 1)
+      if (NSW == 1) {
+        // one step per row and wave: no second register set to fetch ahead into; the other wave of the SIMD covers the wait
+        if (m0_) {
+          WD_FRAGS(0, 0, d0, d1, b0, b1, b2)
+          WD_MULT(0)
         }
-      } else if (m1_) {
-        WD_FRAGS(0, 0, e0, e1, b1, b2, c2)
+        if (m2_) shift_writes(nb2);
+      } else {
+        if (m0_) {
+          // (set 0 holds the first step: fetched at the end of the iteration before)
+          WD_FRAGS(1, 1, d0, d1, b0, b1, b2)
+          WD_MULT(0)
+        }
+        if (m2_) shift_writes(nb2);
+        if (m0_) {
+#pragma unroll
+          for (int j = 1; j < NSW; ++j) {
+            if (j + 1 < NSW) WD_FRAGS((j + 1) & 1, (j + 1 < NSW ? j + 1 : 0), d0, d1, b0, b1, b2)
+            else if (m1_) WD_FRAGS(0, 0, e0, e1, b1, b2, c2)
+            WD_MULT(j & 1)
+          }
+        } else if (m1_) {
+          WD_FRAGS(0, 0, e0, e1, b1, b2, c2)
+        }
       }
       sd = nd;
       sx = nx;
@@ -347,22 +371,62 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
   float* o = out + (size_t)split * ((size_t)p.E + p.K);
   const size_t KC = (size_t)p.K * p.C;
   const int c = c0 + wn * 32 + fr;
+  {
+    // The two waves of a block add their accumulators through LDS: taps 0..4 end up in the first wave, taps 5..8 in
+    // the second (the other wave's values parked as [block][tap][4 registers][lane] cells of 16 bytes: 80 KB from the
+    // second waves, then 64 KB from the first), then each stores its share.
+    static_assert(WD_LDS >= 4 * 9 * 4 * 64 * 16, "the parked accumulators fit");
+    uintx4_t* park = reinterpret_cast<uintx4_t*>(wd_lds);
+    auto parked = [&](int tap, int q) {
+      return tap < 5 ? ((blk * 5 + tap) * 4 + q) * 64 + lane : 4 * 5 * 4 * 64 + ((blk * 4 + tap - 5) * 4 + q) * 64 + lane;
+    };
+    __syncthreads();
 #pragma unroll
-  for (int kh = 0; kh < 3; ++kh)
+    for (int kh = 0; kh < 3; ++kh)
 #pragma unroll
-    for (int kw = 0; kw < 3; ++kw)
+      for (int kw = 0; kw < 3; ++kw) {
+        const int tap = kh * 3 + kw;
+        const bool mine = (tap < 5) == (half == 0);          // this wave keeps the tap
+        if (!mine) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm * 32 + (r >> 2) * 8 + fh * 4 + (r & 3);
-        o[(kh * 3 + kw) * KC + (size_t)m * p.C + c] = acc[kh][kw][r];
+          for (int q = 0; q < 4; ++q)
+            park[parked(tap, q)] =
+                uintx4_t{__float_as_uint(acc[kh][kw][4 * q]), __float_as_uint(acc[kh][kw][4 * q + 1]),
+                         __float_as_uint(acc[kh][kw][4 * q + 2]), __float_as_uint(acc[kh][kw][4 * q + 3])};
+        }
       }
+    __syncthreads();
+#pragma unroll
+    for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+      for (int kw = 0; kw < 3; ++kw) {
+        const int tap = kh * 3 + kw;
+        const bool mine = (tap < 5) == (half == 0);
+        if (mine) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const uintx4_t v = park[parked(tap, q)];
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const int r = 4 * q + k;
+              const int m = m0 + wm * 32 + (r >> 2) * 8 + fh * 4 + (r & 3);
+              // the first wave's value first: the same order of the two terms in both shares
+              const float lo = half == 0 ? acc[kh][kw][r] : __uint_as_float(w[k]);
+              const float hi = half == 0 ? __uint_as_float(w[k]) : acc[kh][kw][r];
+              o[tap * KC + (size_t)m * p.C + c] = lo + hi;
+            }
+          }
+        }
+      }
+  }
   if (do_db) {
     // a row's sums sit in the threads idx = row * NCU .. + NCU - 1: through LDS, added in a fixed order
     float* sums = reinterpret_cast<float*>(wd_lds);
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < NSH; ++i)
-      if (sh_on[i]) sums[tid + 256 * i] = dbsum[i];
+      if (sh_on[i]) sums[tid + THREADS * i] = dbsum[i];
     __syncthreads();
     if (tid < WD_T) {
       float t = 0.f;
@@ -480,7 +544,7 @@ int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw
 #define WD_LAUNCH(NK)                                                                                      \
   {                                                                                                        \
     if (!mfma_allow_lds(reinterpret_cast<const void*>(wgrad_dma_kernel<NK>), WD_LDS)) return -1;           \
-    hipLaunchKernelGGL(wgrad_dma_kernel<NK>, grid, dim3(256), WD_LDS, s, p, xp, dyp, part);                \
+    hipLaunchKernelGGL(wgrad_dma_kernel<NK>, grid, dim3(64 * NW), WD_LDS, s, p, xp, dyp, part);            \
   }
   if (nk16 <= 2) WD_LAUNCH(2)
   else WD_LAUNCH(4)
