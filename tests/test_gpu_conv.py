@@ -224,13 +224,15 @@ def test_conv_bf16_1x1_loaded_straight_to_lds(case, depth):
         capi.set_option("PW16_PF", None)
 
 
-# bf16 1x1 filter gradient without a bias gradient, at least 128 channels on both sides: the kernel whose
+# bf16 1x1 filter gradient without a bias gradient, at least 64 channels on both sides: the kernel whose
 # tiles the loads copy straight to LDS.  Planes of 8k positions; planes whose last cell repeats positions
 # (196, 49, 25, 9: the repeated part of the dy cell is zeroed in LDS); one stage, a slice that ends inside an
 # image, channel tails on both sides, more images than one slice holds.
 @pytest.mark.parametrize("xs,K", [
     ((3, 128, 14, 14), 128), ((5, 136, 7, 7), 160), ((2, 128, 8, 8), 256), ((9, 256, 5, 5), 128),
     ((4, 128, 3, 3), 136), ((1, 128, 2, 4), 128), ((40, 128, 7, 7), 128), ((2, 384, 28, 28), 128),
+    # a side of 64 to 127 channels: half-filled tiles
+    ((2, 64, 56, 56), 256), ((3, 256, 14, 14), 64), ((2, 64, 8, 8), 64), ((5, 72, 7, 7), 136), ((2, 200, 6, 6), 96),
 ])
 def test_bf16_1x1_filter_gradient_alone(xs, K):
     rng = np.random.default_rng(xs[0] * 131 + K)
