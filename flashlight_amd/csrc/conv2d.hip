@@ -330,12 +330,14 @@ extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, 
     const size_t need = flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER);
     FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter: workspace too small");
     int r = -1;
-    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
+    // (3x3 stride 1 with rows copied straight to LDS first: it also takes the 7x7 planes that would otherwise go
+    // through gathered taps below)
+    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_wgrad_dma16(g, x, dy, dw, db, ws, ws_bytes, s);
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pointwise16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_FIRST) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_first16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_wgrad_dma16(g, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_wgrad16(g, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0 && !skip(SK_GEMM))

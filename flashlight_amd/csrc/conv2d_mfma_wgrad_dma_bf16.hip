@@ -60,6 +60,8 @@ struct WdParams {
   int N, C, K, H, W;
   int ncell;              // cells per row
   int dup;                // positions the last cell repeats
+  int keep;               // positions of a cell that belong to the row (8; W in whole-image stages over rows of W < 8)
+  int img;                // a stage is a whole image
   int ctiles, mtiles;
   int total_rows, rps, nsplit;
   int E;                  // K * C * 9
@@ -102,11 +104,18 @@ namespace {
 // take alternate steps of a row and add their accumulators through LDS at the end: while one of them shifts,
 // computes addresses or waits for LDS, the other one's matrix instructions run (one wave per block: 1.3 us per row
 // of 56 positions instead of 1.15).
+//
+// IMG: planes of at most 7 rows of at most 8 positions (7x7): a stage is a whole image, row j in cell j of the 64
+// position slots, cell 7 (and every row past the image) zero.  The three input rows of output row j are cells
+// (j + kh - 1) mod 8 of the same slot - row -1 and row H both land on a zero cell - so there is no ring of rows and
+// no stage that only loads.  A cell of a row of W < 8 positions ends with positions of the next row: they are zeroed in
+// the input cells and masked out of the shifted dy copies.  The one cell of each tensor that would reach past its
+// end is loaded as zeros and filled in by its lane with plain loads.
 constexpr int NW = 8;
-template <int NK16>
+template <int NK16, bool IMG>
 __global__ void __launch_bounds__(64 * NW, 1)
 wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy, float* __restrict__ out) {
-  static_assert(NK16 == 2 || NK16 == 4, "shapes in use");
+  static_assert((NK16 == 2 || NK16 == 4) && (!IMG || NK16 == 4), "shapes in use");
   extern __shared__ __align__(16) char wd_lds[];
   char* const dring = wd_lds;                                   // [WD_NSD] dy rows
   char* const xring = wd_lds + WD_NSD * WD_SLOT;                // [WD_NSX] input rows
@@ -129,8 +138,9 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
   // ---- loads: instruction i of a wave fills rows 8 (NW i + wave) .. + 7 of a slot; lane -> row + lane / 8, LDS
   // cell lane % 8, i.e. the row's cell (lane % 8) ^ (lane / 8)
   const int lrow = lane >> 3, lcell = (lane & 7) ^ lrow;
-  const bool cell_ok = lcell < p.ncell;
-  const int lpos = lcell == p.ncell - 1 ? p.W - 8 : 8 * lcell;  // first position of the lane's cell
+  // (IMG: cell = row of the image)
+  const bool cell_ok = IMG ? lcell < p.H : lcell < p.ncell;
+  const int lpos = IMG ? lcell * p.W : (lcell == p.ncell - 1 ? p.W - 8 : 8 * lcell);  // first position of the lane's cell
   int xoff[NLB], doff[NLB];
 #pragma unroll
   for (int i = 0; i < NLB; ++i) {
@@ -144,15 +154,23 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
   gi.start(row_begin, p.H, nrows);
   gc.start(row_begin, p.H, nrows);
   int nstages = 0;
-  {
+  if (IMG) {
+    nstages = nrows;                    // a "row" of the range is an image
+  } else {
     const int n_first = row_begin / p.H, n_last = (row_begin + nrows - 1) / p.H;
     nstages = nrows + 2 * (n_last - n_first + 1);
   }
-  int islot_d = 0, islot_x = 0;
+  int islot_d = 0, islot_x = 0, issued = 0;
   auto issue = [&]() {
-    int img, ih;
-    const int oh = gi.oh;
-    const bool rows = gi.next(p.H, &img, &ih);
+    int img, ih = 0, oh = 0;
+    bool rows = true;
+    if (IMG) {
+      img = row_begin + issued;
+    } else {
+      oh = gi.oh;
+      rows = gi.next(p.H, &img, &ih);
+    }
+    ++issued;
     const bool x_in = ih >= 0 && ih < p.H;
     const int xs = (img * p.C * p.H + ih) * p.W * 2, ds = (img * p.K * p.H + oh) * p.W * 2;
 #pragma unroll
@@ -164,9 +182,27 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
     islot_d = islot_d + 1 == WD_NSD ? 0 : islot_d + 1;
     islot_x = islot_x + 1 == WD_NSX ? 0 : islot_x + 1;
   };
-  // zeros over the repeated positions (the first p.dup of the row's last cell) of the input cells this lane loaded
-  // into slot xs (its loads have landed)
-  auto fix_tail = [&](int xs) {
+  // After this lane's loads of a stage have landed: zeros over the repeated positions (the first p.dup of the row's
+  // last cell) of the input cells it loaded into slot xs.  IMG (stage = image `img`, dy slot ds): zeros over the
+  // positions past the row in its input cells, and the cell at the very end of either tensor, which was loaded as
+  // zeros (the last two bytes of its 16 lie past the tensor), is filled in with plain loads.
+  auto fix_tail = [&](int xs, int ds, int img) {
+    if (IMG) {
+      if (p.keep < 8 && cell_ok) {
+#pragma unroll
+        for (int i = 0; i < NLB; ++i) {
+          uint16_t* q = reinterpret_cast<uint16_t*>(xring + xs * WD_SLOT + (NW * i + wave) * 1024 + lane * 16);
+          uint16_t* qd = reinterpret_cast<uint16_t*>(dring + ds * WD_SLOT + (NW * i + wave) * 1024 + lane * 16);
+          const int ox = xoff[i] + img * p.C * P * 2, od = doff[i] + img * p.K * P * 2;
+          if ((unsigned)ox + 16u > p.x_bytes)
+            for (int e = 0; e < p.keep; ++e) q[e] = x[(ox >> 1) + e];
+          if ((unsigned)od + 16u > p.dy_bytes)
+            for (int e = 0; e < p.keep; ++e) qd[e] = dy[(od >> 1) + e];
+          for (int e = p.keep; e < 8; ++e) q[e] = 0;
+        }
+      }
+      return;
+    }
     if (p.dup != 0 && lcell == p.ncell - 1) {
 #pragma unroll
       for (int i = 0; i < NLB; ++i) {
@@ -193,23 +229,29 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
   // a stage are issued in one go and the results written later, so the multiplications in between hide them.
   constexpr int NSH = (WD_T * NCU + THREADS - 1) / THREADS;
   int sh_cell[NSH], sh_nx[NSH], sh_pv[NSH];      // byte offsets in a slot: the cell, the element after it, the one before
-  unsigned sh_skip[NSH];                          // elements at the head of the cell that repeat positions (bias sums)
+  unsigned sh_skip[NSH], sh_keep[NSH];            // elements [skip, keep) of the cell count: the head may repeat positions,
+                                                  // the tail may belong to the next row (IMG)
+  uint32_t sh_mask[NSH][4];                       // the same tail as a mask over the cell's four words
   bool sh_on[NSH], sh_has_nx[NSH], sh_has_pv[NSH];
 #pragma unroll
   for (int i = 0; i < NSH; ++i) {
     const int idx = tid + THREADS * i;
     const int r = (idx / NCU) & (WD_T - 1), c = idx % NCU, sw = r & 7;
-    const bool in = c < p.ncell;
+    const bool in = IMG ? c < p.H : c < p.ncell;
     const int pos = c == p.ncell - 1 ? p.W - 8 : 8 * c;
     const int cn = min(c + 1, 7), start = cn == p.ncell - 1 ? p.W - 8 : 8 * cn;
     const int cp = max(c - 1, 0);                 // starts at 8 cp (only the last cell of a row is moved)
     sh_on[i] = idx < WD_T * NCU;
     sh_cell[i] = r * 128 + ((c ^ sw) << 4);
-    sh_has_nx[i] = in && pos + 8 < p.W;
-    sh_has_pv[i] = in && pos > 0;
+    sh_has_nx[i] = !IMG && in && pos + 8 < p.W;
+    sh_has_pv[i] = !IMG && in && pos > 0;
     sh_nx[i] = r * 128 + ((cn ^ sw) << 4) + (sh_has_nx[i] ? 2 * (pos + 8 - start) : 0);
     sh_pv[i] = r * 128 + ((cp ^ sw) << 4) + (sh_has_pv[i] ? 2 * (pos - 1 - 8 * cp) : 0);
-    sh_skip[i] = !in ? 8u : (c == p.ncell - 1 ? (unsigned)p.dup : 0u);
+    sh_skip[i] = !in ? 8u : (!IMG && c == p.ncell - 1 ? (unsigned)p.dup : 0u);
+    sh_keep[i] = IMG ? (unsigned)p.keep : 8u;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      sh_mask[i][k] = (2u * k < sh_keep[i] ? 0xffffu : 0u) | (2u * k + 1 < sh_keep[i] ? 0xffff0000u : 0u);
   }
   uintx4_t sh_v[NSH];
   uint32_t sh_a[NSH], sh_b[NSH];
@@ -231,7 +273,8 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
 #pragma unroll
     for (int i = 0; i < NSH; ++i) {
       // cells past the row hold zeros (the loads wrote them), so do their copies
-      const uintx4_t v = sh_v[i];
+      const uintx4_t v = uintx4_t{sh_v[i].x & sh_mask[i][0], sh_v[i].y & sh_mask[i][1], sh_v[i].z & sh_mask[i][2],
+                                  sh_v[i].w & sh_mask[i][3]};
       const uint32_t nx = sh_has_nx[i] ? sh_a[i] : 0u, pv = sh_has_pv[i] ? sh_b[i] : 0u;
       if (sh_on[i]) {
         char* o = dst + sh_cell[i];
@@ -246,7 +289,7 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
         float t = 0.f;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-          t += 2u * k >= sh_skip[i] ? __uint_as_float(w[k] << 16) : 0.f;
+          t += 2u * k >= sh_skip[i] ? __uint_as_float(w[k] << 16) : 0.f;          // (the tail is masked already)
           t += 2u * k + 1 >= sh_skip[i] ? __uint_as_float(w[k] & 0xffff0000u) : 0.f;
         }
         dbsum[i] += sh_on[i] ? t : 0.f;
@@ -262,6 +305,15 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
     const int sstep = half + 2 * j;
     foff[j] = ((2 * sstep + fh) ^ (fr & 7)) * 16;
   }
+  // input rows: the same cell of three slots (rows of a ring), or - IMG - the cells (row + kh - 1) mod 8 of one slot
+  int boff[NSW][3];
+#pragma unroll
+  for (int j = 0; j < NSW; ++j)
+#pragma unroll
+    for (int kh = 0; kh < 3; ++kh) {
+      const int cell = 2 * (half + 2 * j) + fh;
+      boff[j][kh] = IMG ? ((((cell + kh - 1) & 7) ^ (fr & 7)) * 16) : foff[j];
+    }
   const int arow = (wm * 32 + fr) * 128, brow = (wn * 32 + fr) * 128;
   floatx16 acc[3][3];
 #pragma unroll
@@ -283,30 +335,47 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
     static_assert(NLB == 1, "two loads per stage and wave");
     if (WD_D + 1 <= nstages) PD_WAIT_VM(4);           // stages 2 .. D may be outstanding: 0 and 1 have landed
     else PD_WAIT_VM(0);
-    fix_tail(0);
-    fix_tail(1);
-    // (stages 0 and 1 only load: no shifted copies to make, no fragments to fetch)
+    fix_tail(0, 0, row_begin);
+    if (nstages > 1) fix_tail(1, 1, row_begin + 1);
     int sd = 0, sx = 0, sb = 0;          // slots of stage t: dy ring, input ring, shifted copies
     bool m0_ = false, m1_ = false, m2_ = false;   // whether stages t, t + 1, t + 2 multiply
-    {
+    if (IMG) {
+      m0_ = true;
+      m1_ = nstages > 1;
+    } else {
+      // (stages 0 and 1 only load: no shifted copies to make, no fragments to fetch)
       int img, ih;
       m0_ = gc.next(p.H, &img, &ih);
       if (nstages > 1) m1_ = gc.next(p.H, &img, &ih);
     }
+    WD_STAMP(1)
     bf16x8 fa[2][3], fb[2][3];
 #define WD_FRAGS(SET, J, D0, D1, B0, B1, B2)                                                           \
   {                                                                                                    \
     fa[SET][0] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((D0) + foff[J]));       \
     fa[SET][1] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((D1) + foff[J]));       \
     fa[SET][2] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((D0) + WD_SLOT + foff[J])); \
-    fb[SET][0] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((B0) + foff[J]));       \
-    fb[SET][1] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((B1) + foff[J]));       \
-    fb[SET][2] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((B2) + foff[J]));       \
+    fb[SET][0] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((B0) + boff[J][0]));    \
+    fb[SET][1] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((B1) + boff[J][1]));    \
+    fb[SET][2] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>((B2) + boff[J][2]));    \
   }
 #define WD_MULT(SET)                                                                                   \
   _Pragma("unroll") for (int kh = 0; kh < 3; ++kh)                                                     \
     _Pragma("unroll") for (int kw = 0; kw < 3; ++kw)                                                   \
       acc[kh][kw] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][kw], fb[SET][kh], acc[kh][kw], 0, 0, 0);
+    if (IMG) {
+      // the first two stages multiply too: their shifted copies, and the first fragments of stage 0
+      __syncthreads();
+      shift_reads(0);
+      shift_writes(0);
+      if (nstages > 1) {
+        shift_reads(1);
+        shift_writes(1);
+      }
+      __syncthreads();
+      const char* xs0 = xring + brow;
+      WD_FRAGS(0, 0, shift + arow, dring + arow, xs0, xs0, xs0)
+    }
     for (int t = 0; t < nstages; ++t) {
       const int nd = sd + 1 == WD_NSD ? 0 : sd + 1, nx = sx + 1 == WD_NSX ? 0 : sx + 1, nb = sb + 1 == WD_NSH ? 0 : sb + 1;
       const int nd2 = nd + 1 == WD_NSD ? 0 : nd + 1, nx2 = nx + 1 == WD_NSX ? 0 : nx + 1, nb2 = nb + 1 == WD_NSH ? 0 : nb + 1;
@@ -314,23 +383,31 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
       if (t + 2 < nstages) {
         if (t + 1 + WD_D <= nstages) PD_WAIT_VM(2);     // stages t + 3 .. t + D may be outstanding
         else PD_WAIT_VM(0);
-        fix_tail(nx2);
-        int img, ih;
-        m2_ = gc.next(p.H, &img, &ih);
+        fix_tail(nx2, nd2, row_begin + t + 2);
+        if (IMG) {
+          m2_ = true;
+        } else {
+          int img, ih;
+          m2_ = gc.next(p.H, &img, &ih);
+        }
       }
+      if (t == 4) WD_STAMP(2)
       __syncthreads();
+      if (t == 4) WD_STAMP(3)
       if (t + 1 + WD_D < nstages) issue();
       if (m2_) shift_reads(nd2);
       // operands of stage t and of stage t + 1 (for its first fragments)
       const char* d1 = dring + sd * WD_SLOT + arow;
       const char* d0 = shift + sb * 2 * WD_SLOT + arow;
       const int x1 = sx == 0 ? WD_NSX - 1 : sx - 1, x0 = x1 == 0 ? WD_NSX - 1 : x1 - 1;
-      const char* b0 = xring + x0 * WD_SLOT + brow;
-      const char* b1 = xring + x1 * WD_SLOT + brow;
       const char* b2 = xring + sx * WD_SLOT + brow;
+      const char* b0 = IMG ? b2 : xring + x0 * WD_SLOT + brow;
+      const char* b1 = IMG ? b2 : xring + x1 * WD_SLOT + brow;
       const char* e1 = dring + nd * WD_SLOT + arow;
       const char* e0 = shift + nb * 2 * WD_SLOT + arow;
       const char* c2 = xring + nx * WD_SLOT + brow;
+      const char* c0_ = IMG ? c2 : b1;      // input rows of stage t + 1
+      const char* c1_ = IMG ? c2 : b2;
       if (NSW == 1) {
         // one step per row and wave: no second register set to fetch ahead into; the other wave of the SIMD covers the wait
         if (m0_) {
@@ -349,13 +426,15 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
 #pragma unroll
           for (int j = 1; j < NSW; ++j) {
             if (j + 1 < NSW) WD_FRAGS((j + 1) & 1, (j + 1 < NSW ? j + 1 : 0), d0, d1, b0, b1, b2)
-            else if (m1_) WD_FRAGS(0, 0, e0, e1, b1, b2, c2)
+            else if (m1_) WD_FRAGS(0, 0, e0, e1, c0_, c1_, c2)
             WD_MULT(j & 1)
           }
         } else if (m1_) {
-          WD_FRAGS(0, 0, e0, e1, b1, b2, c2)
+          WD_FRAGS(0, 0, e0, e1, c0_, c1_, c2)
         }
       }
+      if (t == 4) WD_STAMP(5)
+      if (t == 8) WD_STAMP(6)
       sd = nd;
       sx = nx;
       sb = nb;
@@ -489,21 +568,67 @@ wgrad_taps_reduce_kernel(const float* __restrict__ part, int nsplit, int K, int 
   }
 }
 
+// The same reduction for few splits of a large gradient (512 x 512 filters over 7x7 planes: 4 splits of 9.4 MB): a
+// thread owns four input channels of a result channel, adds its nine taps over the splits in order and writes the
+// 36 values as they lie in dw (the kernel above would write them as 4-byte pieces 36 bytes apart).
+__global__ void __launch_bounds__(64)
+wgrad_taps_gather_reduce_kernel(const float* __restrict__ part, int nsplit, int K, int C, int want_db,
+                                float* __restrict__ dw, float* __restrict__ db) {
+  const int KC = K * C, E = KC * 9;
+  const size_t stride = (size_t)E + K;
+  const int item = blockIdx.x * 64 + threadIdx.x;       // (result channel, group of four input channels)
+  if (item * 4 < KC) {
+    float4 acc[9];
+#pragma unroll
+    for (int tap = 0; tap < 9; ++tap) acc[tap] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int sp = 0; sp < nsplit; ++sp) {
+      float4 v[9];
+#pragma unroll
+      for (int tap = 0; tap < 9; ++tap)
+        v[tap] = *reinterpret_cast<const float4*>(part + (size_t)sp * stride + (size_t)tap * KC + (size_t)item * 4);
+#pragma unroll
+      for (int tap = 0; tap < 9; ++tap) {
+        acc[tap].x += v[tap].x; acc[tap].y += v[tap].y; acc[tap].z += v[tap].z; acc[tap].w += v[tap].w;
+      }
+    }
+    // dw[(m * C + c) * 9 + tap], c = 4 consecutive channels: 36 consecutive values
+    float o[36];
+#pragma unroll
+    for (int tap = 0; tap < 9; ++tap) {
+      o[tap] = acc[tap].x;
+      o[9 + tap] = acc[tap].y;
+      o[18 + tap] = acc[tap].z;
+      o[27 + tap] = acc[tap].w;
+    }
+    float4* dst = reinterpret_cast<float4*>(dw + (size_t)item * 36);
+#pragma unroll
+    for (int q = 0; q < 9; ++q) dst[q] = make_float4(o[4 * q], o[4 * q + 1], o[4 * q + 2], o[4 * q + 3]);
+  }
+  if (want_db && item < K) {
+    float t = 0.f;
+    for (int sp = 0; sp < nsplit; ++sp) t += part[(size_t)sp * stride + E + item];
+    db[item] = t;
+  }
+}
+
 bool wd_plan(const ConvGeom& g, WdParams* p) {
   if (!(g.KH == 3 && g.KW == 3 && g.sy == 1 && g.sx == 1 && g.py == 1 && g.px == 1 && g.dly == 1 && g.dlx == 1 &&
         g.groups == 1 && g.OH == g.H && g.OW == g.W))
     return false;
-  if (g.C % WD_T != 0 || g.K % WD_T != 0 || g.W < 8 || g.W > 64) return false;
+  const bool img = g.H <= 7 && g.W <= 8 && g.W >= 2;       // whole images per stage
+  if (g.C % WD_T != 0 || g.K % WD_T != 0 || (!img && g.W < 8) || g.W > 64) return false;
   const long long xb = (long long)g.N * g.C * g.H * g.W * 2, db = (long long)g.N * g.K * g.H * g.W * 2;
   if (xb >= (1ll << 31) || db >= (1ll << 31)) return false;
   p->N = g.N; p->C = g.C; p->K = g.K; p->H = g.H; p->W = g.W;
-  p->ncell = (g.W + 7) / 8;
-  p->dup = 8 * p->ncell - g.W;
+  p->ncell = img ? 1 : (g.W + 7) / 8;
+  p->dup = img ? 0 : 8 * p->ncell - g.W;
+  p->keep = img ? g.W : 8;
+  p->img = img;
   p->x_bytes = (unsigned)xb;
   p->dy_bytes = (unsigned)db;
   p->ctiles = g.C / WD_T;
   p->mtiles = g.K / WD_T;
-  p->total_rows = g.N * g.H;
+  p->total_rows = img ? g.N : g.N * g.H;        // stages: images, or rows
   p->E = g.K * g.C * 9;
   const long long tiles = (long long)p->ctiles * p->mtiles;
   if (tiles > 65535) return false;
@@ -532,7 +657,8 @@ int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw
   if (!dw || !wd_plan(g, &p)) return -1;
   if (!ws || ws_bytes < wd_ws_bytes(p)) return -1;
   p.want_db = db != nullptr;
-  const int nk16 = (p.ncell + 1) / 2;
+  const bool img = p.img != 0;
+  const int nk16 = img ? 4 : (p.ncell + 1) / 2;
   // measured on the ResNet-50 layers at batch 64 against the kernel with register staging: ahead on rows of 56
   // positions (35 against 42 us), behind on rows of 28 and 14 (a stage of one short row is mostly its fixed costs).
   // FLHIP_PW16_PF set lifts the rule (tests).
@@ -541,15 +667,21 @@ int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw
   float* part = static_cast<float*>(ws);
   const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* dyp = static_cast<const bf16_t*>(dy);
-#define WD_LAUNCH(NK)                                                                                      \
-  {                                                                                                        \
-    if (!mfma_allow_lds(reinterpret_cast<const void*>(wgrad_dma_kernel<NK>), WD_LDS)) return -1;           \
-    hipLaunchKernelGGL(wgrad_dma_kernel<NK>, grid, dim3(64 * NW), WD_LDS, s, p, xp, dyp, part);            \
+#define WD_LAUNCH(NK, IM)                                                                                      \
+  {                                                                                                            \
+    if (!mfma_allow_lds(reinterpret_cast<const void*>(wgrad_dma_kernel<NK, IM>), WD_LDS)) return -1;           \
+    hipLaunchKernelGGL((wgrad_dma_kernel<NK, IM>), grid, dim3(64 * NW), WD_LDS, s, p, xp, dyp, part);          \
   }
-  if (nk16 <= 2) WD_LAUNCH(2)
-  else WD_LAUNCH(4)
+  if (img) WD_LAUNCH(4, true)
+  else if (nk16 <= 2) WD_LAUNCH(2, false)
+  else WD_LAUNCH(4, false)
 #undef WD_LAUNCH
   const int total = p.E + (p.want_db ? p.K : 0);
+  if (p.nsplit <= 16 && p.K * p.C >= 128 * 128 && reinterpret_cast<uintptr_t>(dw) % 16 == 0) {
+    hipLaunchKernelGGL(wgrad_taps_gather_reduce_kernel, dim3((p.K * p.C / 4 + 63) / 64), dim3(64), 0, s, part, p.nsplit,
+                       p.K, p.C, p.want_db, dw, db);
+    return check_launch("conv2d_bwd_filter 3x3 (bf16 mfma, direct-to-LDS)");
+  }
   hipLaunchKernelGGL(wgrad_taps_reduce_kernel, dim3((total + 4 * WD_RTX - 1) / (4 * WD_RTX)), dim3(WD_RTX * WD_RTY), 0, s, part, p.nsplit, p.K,
                      p.C, p.want_db, dw, db);
   return check_launch("conv2d_bwd_filter 3x3 (bf16 mfma, direct-to-LDS)");

@@ -268,6 +268,12 @@ def test_bf16_1x1_filter_gradient_alone(xs, K):
     ((2, 64, 56, 56), 64), ((3, 64, 28, 28), 128), ((5, 128, 14, 14), 64), ((7, 64, 5, 12), 64),
     ((2, 128, 9, 20), 128), ((1, 64, 3, 8), 64), ((9, 64, 4, 9), 64), ((2, 64, 6, 40), 64), ((1, 64, 1, 64), 64),
     ((70, 64, 7, 16), 64),
+    # planes of at most 7 rows of at most 8 positions: a stage is a whole image (positions of the next row at the end
+    # of a cell zeroed / masked, the last cell of either tensor filled in by hand)
+    ((5, 64, 7, 7), 64), ((3, 128, 5, 6), 64), ((9, 64, 4, 8), 128), ((2, 64, 7, 3), 64), ((40, 64, 7, 7), 64),
+    ((1, 64, 1, 2), 64), ((6, 64, 2, 5), 192),
+    # few splits of a larger gradient: the reduce kernel that writes the gradient in memory order
+    ((3, 128, 5, 6), 128), ((2, 128, 7, 7), 192), ((2, 128, 9, 40), 128),
 ])
 def test_bf16_3x3_filter_gradient_rows_to_lds(xs, K, with_bias):
     rng = np.random.default_rng(xs[0] * 17 + xs[3] + K)
