@@ -62,6 +62,7 @@ struct WdParams {
   int dup;                // positions the last cell repeats
   int keep;               // positions of a cell that belong to the row (8; W in whole-image stages over rows of W < 8)
   int img;                // a stage is a whole image
+  int G;                  // output rows per stage (0: whole image)
   int ctiles, mtiles;
   int total_rows, rps, nsplit;
   int E;                  // K * C * 9
@@ -111,11 +112,20 @@ namespace {
 // no stage that only loads.  A cell of a row of W < 8 positions ends with positions of the next row: they are zeroed in
 // the input cells and masked out of the shifted dy copies.  The one cell of each tensor that would reach past its
 // end is loaded as zeros and filled in by its lane with plain loads.
+//
+// G = 2, 4 (rows of at most 32 / 16 positions): a stage is a group of G output rows, row j of the group in cells
+// j * 8 / G ... of the 64 position slots.  Its input slot holds the rows G g - 1 ... G g + G - 2; the two rows below
+// them are the first two of the NEXT stage's slot, which the loads have brought in already (they run ahead), so
+// the first group of an image needs no stage before it (row -1 is loaded as zeros); after the last group of an
+// image or of the workgroup's range one stage only loads (the rows below the last group).
 constexpr int NW = 8;
-template <int NK16, bool IMG>
+template <int NK16, int G>
 __global__ void __launch_bounds__(64 * NW, 1)
 wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy, float* __restrict__ out) {
-  static_assert((NK16 == 2 || NK16 == 4) && (!IMG || NK16 == 4), "shapes in use");
+  constexpr bool IMG = G == 0;          // a stage is a whole image
+  constexpr bool GRP = G >= 2;          // a stage is a group of G rows
+  constexpr int CPR = GRP ? 8 / G : 8;  // cells of a row in a slot
+  static_assert((NK16 == 2 || NK16 == 4) && (G == 1 || NK16 == 4) && (G == 0 || G == 1 || G == 2 || G == 4), "shapes in use");
   extern __shared__ __align__(16) char wd_lds[];
   char* const dring = wd_lds;                                   // [WD_NSD] dy rows
   char* const xring = wd_lds + WD_NSD * WD_SLOT;                // [WD_NSX] input rows
@@ -138,9 +148,11 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
   // ---- loads: instruction i of a wave fills rows 8 (NW i + wave) .. + 7 of a slot; lane -> row + lane / 8, LDS
   // cell lane % 8, i.e. the row's cell (lane % 8) ^ (lane / 8)
   const int lrow = lane >> 3, lcell = (lane & 7) ^ lrow;
-  // (IMG: cell = row of the image)
-  const bool cell_ok = IMG ? lcell < p.H : lcell < p.ncell;
-  const int lpos = IMG ? lcell * p.W : (lcell == p.ncell - 1 ? p.W - 8 : 8 * lcell);  // first position of the lane's cell
+  // (IMG: cell = row of the image; GRP: cell = (row of the group, cell of the row))
+  const int lj = GRP ? lcell / CPR : 0, lcq = GRP ? lcell % CPR : lcell;
+  const bool cell_ok = IMG ? lcell < p.H : lcq < p.ncell;
+  // first position of the lane's cell (GRP: in its row)
+  const int lpos = IMG ? lcell * p.W : (lcq == p.ncell - 1 ? p.W - 8 : 8 * lcq);
   int xoff[NLB], doff[NLB];
 #pragma unroll
   for (int i = 0; i < NLB; ++i) {
@@ -154,7 +166,27 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
   gi.start(row_begin, p.H, nrows);
   gc.start(row_begin, p.H, nrows);
   int nstages = 0;
-  if (IMG) {
+  const int GH = GRP ? (p.H + G - 1) / G : 1;          // groups per image; a "row" of the range is a group
+  // GRP: the groups of the range in order, one loading stage after the last group of an image and of the range
+  struct { int n, g, left; bool post; } qi{row_begin / GH, row_begin % GH, nrows, false}, qc = qi;
+  auto grp_next = [&](auto& q, int* img, int* grp) -> bool {
+    *img = q.n;
+    *grp = q.g;
+    if (q.post) {                       // the rows below the group before
+      q.post = false;
+      if (q.g == GH) { q.g = 0; ++q.n; }
+      return false;
+    }
+    --q.left;
+    ++q.g;
+    if (q.g == GH || q.left == 0) q.post = true;
+    return true;
+  };
+  if (GRP) {
+    const int n_first = row_begin / GH, n_last = (row_begin + nrows - 1) / GH;
+    // one loading stage per image the range ends in or passes the end of (the range's own end included)
+    nstages = nrows + (n_last - n_first + 1);
+  } else if (IMG) {
     nstages = nrows;                    // a "row" of the range is an image
   } else {
     const int n_first = row_begin / p.H, n_last = (row_begin + nrows - 1) / p.H;
@@ -164,20 +196,25 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
   auto issue = [&]() {
     int img, ih = 0, oh = 0;
     bool rows = true;
-    if (IMG) {
+    if (GRP) {
+      int grp;
+      rows = grp_next(qi, &img, &grp);
+      ih = G * grp - 1 + lj;            // the lane's input row, and its output row
+      oh = G * grp + lj;
+    } else if (IMG) {
       img = row_begin + issued;
     } else {
       oh = gi.oh;
       rows = gi.next(p.H, &img, &ih);
     }
     ++issued;
-    const bool x_in = ih >= 0 && ih < p.H;
+    const bool x_in = ih >= 0 && ih < p.H, d_in = rows && oh < p.H;
     const int xs = (img * p.C * p.H + ih) * p.W * 2, ds = (img * p.K * p.H + oh) * p.W * 2;
 #pragma unroll
     for (int i = 0; i < NLB; ++i) {
       pd_load_lds(xrs, lds0 + (WD_NSD + islot_x) * WD_SLOT + (NW * i + wave) * 1024,
                   (x_in && xoff[i] != OOB) ? xoff[i] + xs : OOB, 0);
-      pd_load_lds(drs, lds0 + islot_d * WD_SLOT + (NW * i + wave) * 1024, (rows && doff[i] != OOB) ? doff[i] + ds : OOB, 0);
+      pd_load_lds(drs, lds0 + islot_d * WD_SLOT + (NW * i + wave) * 1024, (d_in && doff[i] != OOB) ? doff[i] + ds : OOB, 0);
     }
     islot_d = islot_d + 1 == WD_NSD ? 0 : islot_d + 1;
     islot_x = islot_x + 1 == WD_NSX ? 0 : islot_x + 1;
@@ -203,7 +240,7 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
       }
       return;
     }
-    if (p.dup != 0 && lcell == p.ncell - 1) {
+    if (p.dup != 0 && lcq == p.ncell - 1) {
 #pragma unroll
       for (int i = 0; i < NLB; ++i) {
         char* q = xring + xs * WD_SLOT + (NW * i + wave) * 1024 + lane * 16;
@@ -237,17 +274,18 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
   for (int i = 0; i < NSH; ++i) {
     const int idx = tid + THREADS * i;
     const int r = (idx / NCU) & (WD_T - 1), c = idx % NCU, sw = r & 7;
-    const bool in = IMG ? c < p.H : c < p.ncell;
-    const int pos = c == p.ncell - 1 ? p.W - 8 : 8 * c;
-    const int cn = min(c + 1, 7), start = cn == p.ncell - 1 ? p.W - 8 : 8 * cn;
-    const int cp = max(c - 1, 0);                 // starts at 8 cp (only the last cell of a row is moved)
+    const int cq = GRP ? c % CPR : c;            // the cell inside its row; the neighbours are cells of the same row
+    const bool in = IMG ? c < p.H : cq < p.ncell;
+    const int pos = cq == p.ncell - 1 ? p.W - 8 : 8 * cq;
+    const int cn = min(c + 1, 7), start = cq + 1 == p.ncell - 1 ? p.W - 8 : 8 * (cq + 1);
+    const int cp = max(c - 1, 0);                 // starts at 8 (cq - 1) (only the last cell of a row is moved)
     sh_on[i] = idx < WD_T * NCU;
     sh_cell[i] = r * 128 + ((c ^ sw) << 4);
     sh_has_nx[i] = !IMG && in && pos + 8 < p.W;
     sh_has_pv[i] = !IMG && in && pos > 0;
     sh_nx[i] = r * 128 + ((cn ^ sw) << 4) + (sh_has_nx[i] ? 2 * (pos + 8 - start) : 0);
-    sh_pv[i] = r * 128 + ((cp ^ sw) << 4) + (sh_has_pv[i] ? 2 * (pos - 1 - 8 * cp) : 0);
-    sh_skip[i] = !in ? 8u : (!IMG && c == p.ncell - 1 ? (unsigned)p.dup : 0u);
+    sh_pv[i] = r * 128 + ((cp ^ sw) << 4) + (sh_has_pv[i] ? 2 * (pos - 1 - 8 * (cq - 1)) : 0);
+    sh_skip[i] = !in ? 8u : (!IMG && cq == p.ncell - 1 ? (unsigned)p.dup : 0u);
     sh_keep[i] = IMG ? (unsigned)p.keep : 8u;
 #pragma unroll
     for (int k = 0; k < 4; ++k)
@@ -305,14 +343,23 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
     const int sstep = half + 2 * j;
     foff[j] = ((2 * sstep + fh) ^ (fr & 7)) * 16;
   }
-  // input rows: the same cell of three slots (rows of a ring), or - IMG - the cells (row + kh - 1) mod 8 of one slot
+  // input rows: the same cell of three slots (rows of a ring); IMG: the cells (row + kh - 1) mod 8 of one slot;
+  // GRP: row j + kh of this stage's slot, or row j + kh - G of the next stage's (bnext)
   int boff[NSW][3];
+  bool bnext[NSW][3];
 #pragma unroll
   for (int j = 0; j < NSW; ++j)
 #pragma unroll
     for (int kh = 0; kh < 3; ++kh) {
       const int cell = 2 * (half + 2 * j) + fh;
-      boff[j][kh] = IMG ? ((((cell + kh - 1) & 7) ^ (fr & 7)) * 16) : foff[j];
+      bnext[j][kh] = false;
+      if (GRP) {
+        const int rho = cell / CPR + kh;          // the same for both halves of the wave: a row has at least 2 cells
+        bnext[j][kh] = __builtin_amdgcn_readfirstlane(rho >= G ? 1 : 0) != 0;
+        boff[j][kh] = ((((rho % G) * CPR + cell % CPR)) ^ (fr & 7)) * 16;
+      } else {
+        boff[j][kh] = IMG ? ((((cell + kh - 1) & 7) ^ (fr & 7)) * 16) : foff[j];
+      }
     }
   const int arow = (wm * 32 + fr) * 128, brow = (wn * 32 + fr) * 128;
   floatx16 acc[3][3];
@@ -339,7 +386,11 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
     if (nstages > 1) fix_tail(1, 1, row_begin + 1);
     int sd = 0, sx = 0, sb = 0;          // slots of stage t: dy ring, input ring, shifted copies
     bool m0_ = false, m1_ = false, m2_ = false;   // whether stages t, t + 1, t + 2 multiply
-    if (IMG) {
+    if (GRP) {
+      int img, grp;
+      m0_ = grp_next(qc, &img, &grp);
+      m1_ = grp_next(qc, &img, &grp);
+    } else if (IMG) {
       m0_ = true;
       m1_ = nstages > 1;
     } else {
@@ -363,7 +414,7 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
   _Pragma("unroll") for (int kh = 0; kh < 3; ++kh)                                                     \
     _Pragma("unroll") for (int kw = 0; kw < 3; ++kw)                                                   \
       acc[kh][kw] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][kw], fb[SET][kh], acc[kh][kw], 0, 0, 0);
-    if (IMG) {
+    if (IMG || GRP) {
       // the first two stages multiply too: their shifted copies, and the first fragments of stage 0
       __syncthreads();
       shift_reads(0);
@@ -374,7 +425,8 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
       }
       __syncthreads();
       const char* xs0 = xring + brow;
-      WD_FRAGS(0, 0, shift + arow, dring + arow, xs0, xs0, xs0)
+      const char* xs1 = xring + WD_SLOT + brow;
+      WD_FRAGS(0, 0, shift + arow, dring + arow, (bnext[0][0] ? xs1 : xs0), (bnext[0][1] ? xs1 : xs0), (bnext[0][2] ? xs1 : xs0))
     }
     for (int t = 0; t < nstages; ++t) {
       const int nd = sd + 1 == WD_NSD ? 0 : sd + 1, nx = sx + 1 == WD_NSX ? 0 : sx + 1, nb = sb + 1 == WD_NSH ? 0 : sb + 1;
@@ -384,7 +436,10 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
         if (t + 1 + WD_D <= nstages) PD_WAIT_VM(2);     // stages t + 3 .. t + D may be outstanding
         else PD_WAIT_VM(0);
         fix_tail(nx2, nd2, row_begin + t + 2);
-        if (IMG) {
+        if (GRP) {
+          int img, grp;
+          m2_ = grp_next(qc, &img, &grp);
+        } else if (IMG) {
           m2_ = true;
         } else {
           int img, ih;
@@ -400,37 +455,41 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
       const char* d1 = dring + sd * WD_SLOT + arow;
       const char* d0 = shift + sb * 2 * WD_SLOT + arow;
       const int x1 = sx == 0 ? WD_NSX - 1 : sx - 1, x0 = x1 == 0 ? WD_NSX - 1 : x1 - 1;
-      const char* b2 = xring + sx * WD_SLOT + brow;
-      const char* b0 = IMG ? b2 : xring + x0 * WD_SLOT + brow;
-      const char* b1 = IMG ? b2 : xring + x1 * WD_SLOT + brow;
+      const char* bc = xring + sx * WD_SLOT + brow;       // this stage's input slot, the next stage's, the one after
+      const char* bn = xring + nx * WD_SLOT + brow;
+      const char* bn2 = xring + nx2 * WD_SLOT + brow;
+      const char* br1 = xring + x1 * WD_SLOT + brow;      // the rows of the two stages before (ring of single rows)
+      const char* br0 = xring + x0 * WD_SLOT + brow;
       const char* e1 = dring + nd * WD_SLOT + arow;
       const char* e0 = shift + nb * 2 * WD_SLOT + arow;
-      const char* c2 = xring + nx * WD_SLOT + brow;
-      const char* c0_ = IMG ? c2 : b1;      // input rows of stage t + 1
-      const char* c1_ = IMG ? c2 : b2;
+      // input rows of tap row kh for the wave's step J of stage t (T = 0) or t + 1 (T = 1)
+#define WD_B(T, J, KH)                                                                                     \
+  (GRP ? (bnext[J][KH] ? ((T) ? bn2 : bn) : ((T) ? bn : bc))                                               \
+       : IMG ? ((T) ? bn : bc)                                                                             \
+             : ((KH) == 2 ? ((T) ? bn : bc) : (KH) == 1 ? ((T) ? bc : br1) : ((T) ? br1 : br0)))
       if (NSW == 1) {
         // one step per row and wave: no second register set to fetch ahead into; the other wave of the SIMD covers the wait
         if (m0_) {
-          WD_FRAGS(0, 0, d0, d1, b0, b1, b2)
+          WD_FRAGS(0, 0, d0, d1, WD_B(0, 0, 0), WD_B(0, 0, 1), WD_B(0, 0, 2))
           WD_MULT(0)
         }
         if (m2_) shift_writes(nb2);
       } else {
         if (m0_) {
           // (set 0 holds the first step: fetched at the end of the iteration before)
-          WD_FRAGS(1, 1, d0, d1, b0, b1, b2)
+          WD_FRAGS(1, 1, d0, d1, WD_B(0, 1, 0), WD_B(0, 1, 1), WD_B(0, 1, 2))
           WD_MULT(0)
         }
         if (m2_) shift_writes(nb2);
         if (m0_) {
 #pragma unroll
           for (int j = 1; j < NSW; ++j) {
-            if (j + 1 < NSW) WD_FRAGS((j + 1) & 1, (j + 1 < NSW ? j + 1 : 0), d0, d1, b0, b1, b2)
-            else if (m1_) WD_FRAGS(0, 0, e0, e1, c0_, c1_, c2)
+            if (j + 1 < NSW) WD_FRAGS((j + 1) & 1, (j + 1 < NSW ? j + 1 : 0), d0, d1, WD_B(0, (j + 1 < NSW ? j + 1 : 0), 0), WD_B(0, (j + 1 < NSW ? j + 1 : 0), 1), WD_B(0, (j + 1 < NSW ? j + 1 : 0), 2))
+            else if (m1_) WD_FRAGS(0, 0, e0, e1, WD_B(1, 0, 0), WD_B(1, 0, 1), WD_B(1, 0, 2))
             WD_MULT(j & 1)
           }
         } else if (m1_) {
-          WD_FRAGS(0, 0, e0, e1, c0_, c1_, c2)
+          WD_FRAGS(0, 0, e0, e1, WD_B(1, 0, 0), WD_B(1, 0, 1), WD_B(1, 0, 2))
         }
       }
       if (t == 4) WD_STAMP(5)
@@ -441,6 +500,7 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
       m0_ = m1_;
       m1_ = m2_;
     }
+#undef WD_B
 #undef WD_MULT
 #undef WD_FRAGS
   }
@@ -624,11 +684,12 @@ bool wd_plan(const ConvGeom& g, WdParams* p) {
   p->dup = img ? 0 : 8 * p->ncell - g.W;
   p->keep = img ? g.W : 8;
   p->img = img;
+  p->G = img ? 0 : g.W <= 16 ? 4 : g.W <= 32 ? 2 : 1;
   p->x_bytes = (unsigned)xb;
   p->dy_bytes = (unsigned)db;
   p->ctiles = g.C / WD_T;
   p->mtiles = g.K / WD_T;
-  p->total_rows = img ? g.N : g.N * g.H;        // stages: images, or rows
+  p->total_rows = img ? g.N : g.N * ((g.H + (p->G - 1)) / (p->G > 1 ? p->G : 1));        // stages: images, rows or groups of rows
   p->E = g.K * g.C * 9;
   const long long tiles = (long long)p->ctiles * p->mtiles;
   if (tiles > 65535) return false;
@@ -657,27 +718,27 @@ int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw
   if (!dw || !wd_plan(g, &p)) return -1;
   if (!ws || ws_bytes < wd_ws_bytes(p)) return -1;
   p.want_db = db != nullptr;
-  const bool img = p.img != 0;
-  const int nk16 = img ? 4 : (p.ncell + 1) / 2;
-  // measured on the ResNet-50 layers at batch 64 against the kernel with register staging: ahead on rows of 56
-  // positions (35 against 42 us), behind on rows of 28 and 14 (a stage of one short row is mostly its fixed costs).
-  // FLHIP_PW16_PF set lifts the rule (tests).
-  if (!options().pw16_pf && nk16 < 3) return -1;
+  // measured on the ResNet-50 layers at batch 64 against the kernel with register staging: 56x56 planes 36 against
+  // 42 us, 28x28 (two rows per stage) 36 against 40, 14x14 (four rows) 43 against 52, 7x7 (whole images) 47 against 94
+  // through gathered taps
   const dim3 grid((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles));
   float* part = static_cast<float*>(ws);
   const bf16_t* xp = static_cast<const bf16_t*>(x);
   const bf16_t* dyp = static_cast<const bf16_t*>(dy);
-#define WD_LAUNCH(NK, IM)                                                                                      \
+#define WD_LAUNCH(NK, GR)                                                                                      \
   {                                                                                                            \
-    if (!mfma_allow_lds(reinterpret_cast<const void*>(wgrad_dma_kernel<NK, IM>), WD_LDS)) return -1;           \
-    hipLaunchKernelGGL((wgrad_dma_kernel<NK, IM>), grid, dim3(64 * NW), WD_LDS, s, p, xp, dyp, part);          \
+    if (!mfma_allow_lds(reinterpret_cast<const void*>(wgrad_dma_kernel<NK, GR>), WD_LDS)) return -1;           \
+    hipLaunchKernelGGL((wgrad_dma_kernel<NK, GR>), grid, dim3(64 * NW), WD_LDS, s, p, xp, dyp, part);          \
   }
-  if (img) WD_LAUNCH(4, true)
-  else if (nk16 <= 2) WD_LAUNCH(2, false)
-  else WD_LAUNCH(4, false)
+  if (p.G == 0) WD_LAUNCH(4, 0)
+  else if (p.G == 1) WD_LAUNCH(4, 1)
+  else if (p.G == 2) WD_LAUNCH(4, 2)
+  else WD_LAUNCH(4, 4)
 #undef WD_LAUNCH
   const int total = p.E + (p.want_db ? p.K : 0);
-  if (p.nsplit <= 16 && p.K * p.C >= 128 * 128 && reinterpret_cast<uintptr_t>(dw) % 16 == 0) {
+  // (a thread of it walks all splits and taps: it needs a gradient large enough for a few waves per CU;
+  // 256 x 256 filters in 16 splits: 40 us against 7 us of the kernel below)
+  if (p.nsplit <= 8 && p.K * p.C >= 256 * 512 && reinterpret_cast<uintptr_t>(dw) % 16 == 0) {
     hipLaunchKernelGGL(wgrad_taps_gather_reduce_kernel, dim3((p.K * p.C / 4 + 63) / 64), dim3(64), 0, s, part, p.nsplit,
                        p.K, p.C, p.want_db, dw, db);
     return check_launch("conv2d_bwd_filter 3x3 (bf16 mfma, direct-to-LDS)");

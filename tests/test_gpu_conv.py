@@ -273,7 +273,7 @@ def test_bf16_1x1_filter_gradient_alone(xs, K):
     ((5, 64, 7, 7), 64), ((3, 128, 5, 6), 64), ((9, 64, 4, 8), 128), ((2, 64, 7, 3), 64), ((40, 64, 7, 7), 64),
     ((1, 64, 1, 2), 64), ((6, 64, 2, 5), 192),
     # few splits of a larger gradient: the reduce kernel that writes the gradient in memory order
-    ((3, 128, 5, 6), 128), ((2, 128, 7, 7), 192), ((2, 128, 9, 40), 128),
+    ((3, 256, 5, 6), 512), ((2, 512, 7, 7), 256),
 ])
 def test_bf16_3x3_filter_gradient_rows_to_lds(xs, K, with_bias):
     rng = np.random.default_rng(xs[0] * 17 + xs[3] + K)
