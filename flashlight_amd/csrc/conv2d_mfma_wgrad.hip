@@ -297,6 +297,36 @@ wgrad_reduce_kernel(const float* __restrict__ part, int nsplit, int E, int K, in
   }
 }
 
+// Few partial streams (at most 8) of a large gradient: a thread owns four elements and adds the splits in order, all
+// its loads in flight at once (the kernel above spreads the splits over 16 rows of threads: with 8 splits half of a
+// workgroup idles and every thread has one load in flight - 512 x 2048 filters in 8 splits: 16.9 us).
+__global__ void __launch_bounds__(256)
+wgrad_reduce_few_kernel(const float* __restrict__ part, int nsplit, int E, int K, int want_db,
+                        float* __restrict__ dw, float* __restrict__ db) {
+  const int e = (blockIdx.x * 256 + threadIdx.x) * 4;
+  const int total = E + (want_db ? K : 0);
+  const size_t stride = (size_t)E + K;
+  if (e >= total) return;
+  float4 v[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u)
+    v[u] = u < nsplit ? *reinterpret_cast<const float4*>(part + (size_t)u * stride + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 r = v[0];
+#pragma unroll
+  for (int u = 1; u < 8; ++u) {
+    r.x += v[u].x; r.y += v[u].y; r.z += v[u].z; r.w += v[u].w;
+  }
+  const float rv[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int ek = e + k;
+    if (ek < E)
+      dw[ek] = rv[k];
+    else if (ek < total)
+      db[ek - E] = rv[k];
+  }
+}
+
 // element-wise variant for sizes that are not multiples of four
 __global__ void __launch_bounds__(256)
 wgrad_reduce_kernel1(const float* __restrict__ part, int nsplit, int E, int K, int want_db,
@@ -376,7 +406,9 @@ bool wgrad_split(WgradParams* p, const ConvGeom& g) {
 void wgrad_reduce_launch(const float* part, int nsplit, int E, int K, int want_db, float* dw,
                          float* db, hipStream_t s) {
   const int total = E + (want_db ? K : 0);
-  if ((E + K) % 4 == 0 && reinterpret_cast<uintptr_t>(part) % 16 == 0)
+  if ((E + K) % 4 == 0 && reinterpret_cast<uintptr_t>(part) % 16 == 0 && nsplit <= 8 && total >= (1 << 18))
+    hipLaunchKernelGGL(wgrad_reduce_few_kernel, dim3((total + 1023) / 1024), dim3(256), 0, s, part, nsplit, E, K, want_db, dw, db);
+  else if ((E + K) % 4 == 0 && reinterpret_cast<uintptr_t>(part) % 16 == 0)
     hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((total + 255) / 256), dim3(64 * RED_TY), 0, s, part,
                        nsplit, E, K, want_db, dw, db);
   else

@@ -641,15 +641,22 @@ wgrad_taps_gather_reduce_kernel(const float* __restrict__ part, int nsplit, int 
     float4 acc[9];
 #pragma unroll
     for (int tap = 0; tap < 9; ++tap) acc[tap] = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int sp = 0; sp < nsplit; ++sp) {
-      float4 v[9];
+    // two splits' loads in flight at a time (18 of 16 bytes per thread)
+    for (int sp = 0; sp < nsplit; sp += 2) {
+      float4 v[2][9];
 #pragma unroll
-      for (int tap = 0; tap < 9; ++tap)
-        v[tap] = *reinterpret_cast<const float4*>(part + (size_t)sp * stride + (size_t)tap * KC + (size_t)item * 4);
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int tap = 0; tap < 9; ++tap) {
-        acc[tap].x += v[tap].x; acc[tap].y += v[tap].y; acc[tap].z += v[tap].z; acc[tap].w += v[tap].w;
-      }
+        for (int tap = 0; tap < 9; ++tap)
+          v[u][tap] = sp + u < nsplit
+                          ? *reinterpret_cast<const float4*>(part + (size_t)(sp + u) * stride + (size_t)tap * KC + (size_t)item * 4)
+                          : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int tap = 0; tap < 9; ++tap) {
+          acc[tap].x += v[u][tap].x; acc[tap].y += v[u][tap].y; acc[tap].z += v[u][tap].z; acc[tap].w += v[u][tap].w;
+        }
     }
     // dw[(m * C + c) * 9 + tap], c = 4 consecutive channels: 36 consecutive values
     float o[36];
