@@ -297,8 +297,8 @@ wgrad_reduce_kernel(const float* __restrict__ part, int nsplit, int E, int K, in
   }
 }
 
-// Few partial streams (at most 8) of a large gradient: a thread owns four elements and adds the splits in order, all
-// its loads in flight at once (the kernel above spreads the splits over 16 rows of threads: with 8 splits half of a
+// Few partial streams (at most 16) of a large gradient: a thread owns four elements and adds the splits in order, eight
+// loads in flight at a time (the kernel above spreads the splits over 16 rows of threads: with 8 splits half of a
 // workgroup idles and every thread has one load in flight - 512 x 2048 filters in 8 splits: 16.9 us).
 __global__ void __launch_bounds__(256)
 wgrad_reduce_few_kernel(const float* __restrict__ part, int nsplit, int E, int K, int want_db,
@@ -307,14 +307,17 @@ wgrad_reduce_few_kernel(const float* __restrict__ part, int nsplit, int E, int K
   const int total = E + (want_db ? K : 0);
   const size_t stride = (size_t)E + K;
   if (e >= total) return;
-  float4 v[8];
+  float4 r = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int s0 = 0; s0 < nsplit; s0 += 8) {
+    float4 v[8];
 #pragma unroll
-  for (int u = 0; u < 8; ++u)
-    v[u] = u < nsplit ? *reinterpret_cast<const float4*>(part + (size_t)u * stride + e) : make_float4(0.f, 0.f, 0.f, 0.f);
-  float4 r = v[0];
+    for (int u = 0; u < 8; ++u)
+      v[u] = s0 + u < nsplit ? *reinterpret_cast<const float4*>(part + (size_t)(s0 + u) * stride + e)
+                             : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-  for (int u = 1; u < 8; ++u) {
-    r.x += v[u].x; r.y += v[u].y; r.z += v[u].z; r.w += v[u].w;
+    for (int u = 0; u < 8; ++u) {
+      r.x += v[u].x; r.y += v[u].y; r.z += v[u].z; r.w += v[u].w;
+    }
   }
   const float rv[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
@@ -406,7 +409,7 @@ bool wgrad_split(WgradParams* p, const ConvGeom& g) {
 void wgrad_reduce_launch(const float* part, int nsplit, int E, int K, int want_db, float* dw,
                          float* db, hipStream_t s) {
   const int total = E + (want_db ? K : 0);
-  if ((E + K) % 4 == 0 && reinterpret_cast<uintptr_t>(part) % 16 == 0 && nsplit <= 8 && total >= (1 << 18))
+  if ((E + K) % 4 == 0 && reinterpret_cast<uintptr_t>(part) % 16 == 0 && nsplit <= 16 && total >= (1 << 18))
     hipLaunchKernelGGL(wgrad_reduce_few_kernel, dim3((total + 1023) / 1024), dim3(256), 0, s, part, nsplit, E, K, want_db, dw, db);
   else if ((E + K) % 4 == 0 && reinterpret_cast<uintptr_t>(part) % 16 == 0)
     hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((total + 255) / 256), dim3(64 * RED_TY), 0, s, part,
