@@ -723,7 +723,7 @@ int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw
                      hipStream_t s) {
   WdParams p{};
   if (!dw || !wd_plan(g, &p)) return -1;
-  if (!ws || ws_bytes < wd_ws_bytes(p)) return -1;
+  if (!ws || ws_bytes < wd_ws_bytes(p) || reinterpret_cast<uintptr_t>(ws) % 16 != 0) return -1;   // (the reduce kernels read 16 bytes at a time)
   p.want_db = db != nullptr;
   // measured on the ResNet-50 layers at batch 64 against the kernel with register staging: 56x56 planes 36 against
   // 42 us, 28x28 (two rows per stage) 36 against 40, 14x14 (four rows) 43 against 52, 7x7 (whole images) 47 against 94
