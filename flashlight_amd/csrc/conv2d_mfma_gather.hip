@@ -30,6 +30,9 @@
 // v_mfma_f32_16x16x4_f32 operand layout (lane l of 64):
 //   A operand: A[i = l%16][k = l/16]     B operand: B[k = l/16][j = l%16]
 //   result   : D[i = 4*(l/16) + r][j = l%16], r = 0..3
+#include <map>
+#include <mutex>
+#include <utility>
 #include "conv2d_mfma.h"
 
 namespace flhip {
@@ -50,8 +53,17 @@ int mfma_num_cus() {
 bool mfma_allow_lds(const void* func, size_t bytes) {
   if (bytes <= 64 * 1024) return true;
   if (bytes > 160 * 1024) return false;
-  return hipFuncSetAttribute(func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) ==
-         hipSuccess;
+  // the limit is kept per (kernel, device): raised once, not on every launch
+  static std::mutex mu;
+  static std::map<std::pair<const void*, int>, size_t> raised;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  std::lock_guard<std::mutex> lock(mu);
+  size_t& have = raised[std::make_pair(func, dev)];
+  if (bytes <= have) return true;
+  if (hipFuncSetAttribute(func, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) return false;
+  have = bytes;
+  return true;
 }
 
 namespace {
