@@ -1,23 +1,24 @@
 // Filter (and bias) gradient of 3x3 stride-1 pad-1 convolutions in bf16 storage on
 // v_mfma_f32_32x32x16_bf16, with the operand rows copied into LDS by the memory pipeline
 // itself (buffer loads with the LDS modifier): no wave spends vector instructions on loading,
-// all four waves multiply.
+// all eight waves multiply.
 //
 //   dw[m][c][kh][kw] = sum over images n and positions (oh, ow) of
 //                      dy[n][m][oh][ow] * x[n][c][oh + kh - 1][ow + kw - 1]
 //
 // The contraction runs over positions, which are contiguous in memory in both operands.  A
-// stage is one output row (n, oh): the dy row of 64 result channels and ONE new input row
-// (n, oh + 1) of 64 input channels; the input rows oh - 1 and oh are still in LDS from the two
-// stages before (a ring of rows), so every row of both tensors is fetched once per tile.  The
-// vertical taps kh are those three input rows; the horizontal taps kw are taken on the dy
-// side, where they cost a third of the rows: with iw = ow + kw - 1,
+// stage is 64 position slots: one output row of 33 to 64 positions (described here; groups of
+// shorter rows and whole small images: at the kernel), i.e. the dy row of 64 result channels
+// and ONE new input row (n, oh + 1) of 64 input channels; the input rows oh - 1 and oh are
+// still in LDS from the two stages before (a ring of rows), so every row of both tensors is
+// fetched once per tile.  The vertical taps kh are those three input rows; the horizontal taps
+// kw are taken on the dy side, where they cost a third of the rows: with iw = ow + kw - 1,
 //   sum_ow dy[ow] x[ow + kw - 1] = sum_iw D_kw[iw] x[iw],   D_kw[iw] = dy[iw - kw + 1]
 // (zero outside the row).  D_1 is the dy row as loaded; D_0 and D_2 are made from it by an
 // LDS -> LDS pass (a 16-byte cell and one element of its neighbour, shifted by v_alignbit), two
-// stages ahead of the multiplications.  Nine accumulator tiles (kh, kw) of 32 x 32 per wave;
-// the tile is 2 (result channels) x 2 (input channels) such blocks, two waves per block; a row is
-// 2 or 4 steps of 16 positions.
+// stages ahead of the multiplications.  The tile is 2 (result channels) x 2 (input channels)
+// blocks of 32 x 32 with nine accumulator tiles (kh, kw) each; two waves per block take
+// alternate 16-position steps of a stage and add their accumulators through LDS at the end.
 //
 // Rows of W positions are cut into cells of 8 (16 bytes); when W is not a multiple of 8 the
 // last cell ENDS at the row's last position and repeats positions of the cell before it; the
@@ -28,12 +29,12 @@
 // the 32 rows of a fragment read spread over the banks (a lane fetches the cell that belongs
 // where it writes).
 //
-// A workgroup owns a 64 x 64 tile of (result, input) channels over a range of (image, row)
-// pairs; at the start of the range and of every image two stages only load (rows oh - 1 and oh).
-// One barrier per stage; while stage t multiplies, the loads of stage t + 1 + WD_D are issued,
-// the shifted copies of stage t + 2 are made and the first fragments of stage t + 1 are
-// fetched.  Partial tiles go to the workspace as [tap][result channel][input channel] (so a
-// lane's 16 values of a tap leave as coalesced rows) and are added in a fixed order by
+// A workgroup owns a 64 x 64 tile of (result, input) channels over a range of stages; with one
+// row per stage two stages only load at the start of the range and of every image (rows oh - 1
+// and oh).  One barrier per stage; while stage t multiplies, the loads of stage t + 1 + WD_D
+// are issued, the shifted copies of stage t + 2 are made and the first fragments of stage
+// t + 1 are fetched.  Partial tiles go to the workspace as [tap][result channel][input channel]
+// (so a lane's 16 values of a tap leave as coalesced rows) and are added in a fixed order by
 // wgrad_taps_reduce_kernel, which writes [result channel][input channel][tap].  The bias
 // gradient is summed from the dy cells as they pass through the registers of the shifting
 // pass (the positions a last cell repeats left out), in the workgroups of the first tile
