@@ -60,6 +60,8 @@ static bool apply_option(Options& o, const char* name, const char* v) {
     if (!v || !*v || !strcmp(v, "auto")) o.bn_algo = 0;
     else if (!strcmp(v, "split")) o.bn_algo = 1;
     else if (!strcmp(v, "resident")) o.bn_algo = 2;
+    else if (!strcmp(v, "pair")) o.bn_algo = 3;
+    else if (!strcmp(v, "pairalone")) o.bn_algo = 4;
     else return false;
     return true;
   }

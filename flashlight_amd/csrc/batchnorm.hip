@@ -10,6 +10,8 @@
 // inner == 1 ("column" kernels, per-activation mode): features are contiguous, a
 // wave covers 64 features and rows are strided by C.
 #include <stdlib.h>
+#include <atomic>
+#include <chrono>
 #include <string.h>
 
 #include "common.h"
@@ -404,15 +406,16 @@ __device__ __forceinline__ int mask_off(int off, int esz) { return (int)((unsign
 // offset is relative to the tensor base and goes through a buffer descriptor; slots
 // past the feature get an offset past the descriptor's range, so their loads return
 // zero and their stores are dropped without a branch.
+// (q0, feature: a workgroup that owns the vectors from q0 on of a feature other than res_feature's)
 template <int RES_THREADS, int K, int ESZ, int FENCE, bool REV = false, int VEC = 4, typename F>
-__device__ __forceinline__ void res_visit(const BnGeom& g, F&& f) {
+__device__ __forceinline__ void res_visit(const BnGeom& g, F&& f, int q0 = 0, int feature = -1) {
   constexpr int OOB = (int)0x80000000;
   const int innerV = (int)(g.inner / VEC);
   const int units = (int)(g.units * 4 / VEC);      // g.units counts 4-element vectors
-  const int c = res_feature(g);
+  const int c = feature >= 0 ? feature : res_feature(g);
   // REV walks k = K-1 .. 0: what the previous walk loaded last is asked for first,
   // while the caches still hold it
-  int q = threadIdx.x + (REV ? (K - 1) * RES_THREADS : 0);
+  int q = threadIdx.x + q0 + (REV ? (K - 1) * RES_THREADS : 0);
   int o = q / innerV, i = q - o * innerV;
   const int so = RES_THREADS / innerV, si = RES_THREADS - so * innerV;
   const int row = (int)(g.C * g.inner) * ESZ;                 // bytes between outer slices
@@ -590,6 +593,101 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
     buf_st4(dxr_, off, v, dx);
     if (FUSE && fu.dres) buf_st4(make_rsrc(fu.dres, bytes), off, d, dx);
   });
+}
+
+// ---- backward, a feature shared by two workgroups (fp32, features of 10 to 26 vectors per thread) ---------
+// The kernel above parks 9 of a thread's dy vectors in LDS and reads the others twice.  Here two workgroups own a
+// feature, half of its vectors each: a thread keeps its K2 vectors of x in registers and ALL its K2 vectors of dy
+// on chip (K2 - KR in LDS, KR in registers), so every tensor crosses the memory interface once (3T).  The two
+// need each other's sums.  Each publishes its own as two 64-bit words (value, launch number) with relaxed atomic
+// stores - a word is valid by itself, so no fence is needed - and polls the other's for a BOUNDED time; a workgroup
+// whose partner does not answer in time (it may not be running yet, and nothing guarantees that it ever runs
+// alongside) sums the partner's half itself from memory, with the same instructions in the same order, so the
+// result does not depend on who computed what.  No wait in this kernel is unbounded.
+// Workgroups b and b ^ 8 are partners: consecutive workgroups go to the 8 XCDs in turn, so partners share an L2.
+__device__ __forceinline__ void bn_pair_partial(const float4& d, const float4& xv, float mean, float* p1, float* p2) {
+  *p1 = (d.x + d.y) + (d.z + d.w);
+  *p2 = __fmaf_rn(d.w, xv.w - mean, __fmaf_rn(d.z, xv.z - mean, __fmaf_rn(d.y, xv.y - mean, d.x * (xv.x - mean))));
+}
+
+template <int K2, int KR>
+__global__ void __launch_bounds__(1024)
+bn_bwd_pair(BnGeom g, unsigned bytes, const float* __restrict__ x, const float* __restrict__ dy,
+            float* __restrict__ dx, BnBwdArgs a, unsigned long long* xch, unsigned epoch, unsigned spin_ticks) {
+  constexpr int T = 1024, KL = K2 - KR;
+  extern __shared__ float4 dyl[];           // [KL][T]
+  __shared__ float red[T / 64];
+  __shared__ float sh[4];
+  __shared__ float theirs[3];               // the partner's sums, and whether they arrived
+  const int tid = threadIdx.x;
+  const int b = blockIdx.x, r16 = b & 15, half = r16 >> 3, fs = (b >> 4) * 8 + (r16 & 7);
+  const int C = (int)g.C;
+  const int c = (fs & 7) * (C >> 3) + (fs >> 3);      // neighbouring features on one XCD, as res_feature
+  const int q0 = half * K2 * T, q0_theirs = (half ^ 1) * K2 * T;
+  const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes), dxr_ = make_rsrc(dx, bytes);
+  const float mean = a.save_mean[c];
+  float4 xr[K2], dr[KR > 0 ? KR : 1];
+  float s1 = 0.f, s2 = 0.f;
+  res_visit<T, K2, 4, 0>(g, [&](int k, int off, bool) { xr[k] = buf_ld4_stream(xr_, off, x); }, q0, c);
+  res_visit<T, K2, 4, 4>(g, [&](int k, int off, bool in) {
+    const float4 d = buf_ld4_stream(dyr_, off, dy);
+    if (k < KL) dyl[k * T + tid] = d;
+    else dr[k - KL < 0 ? 0 : k - KL] = d;
+    float p1, p2;
+    bn_pair_partial(d, xr[k], mean, &p1, &p2);
+    s1 += in ? p1 : 0.f;
+    s2 += in ? p2 : 0.f;
+    asm volatile("" : "+v"(s1), "+v"(s2));
+  }, q0, c);
+  s1 = block_sum(s1, red);
+  s2 = block_sum(s2, red);
+  unsigned long long* mine = xch + ((size_t)c * 2 + half) * 2;
+  unsigned long long* other = xch + ((size_t)c * 2 + (half ^ 1)) * 2;
+  if (tid == 0) {
+    __hip_atomic_store(mine + 0, ((unsigned long long)__float_as_uint(s1) << 32) | epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(mine + 1, ((unsigned long long)__float_as_uint(s2) << 32) | epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    bool got = false;
+    unsigned long long w0 = 0, w1 = 0;
+    if (spin_ticks != 0) {
+      const unsigned long long t0 = wall_clock64();
+      do {
+        w0 = __hip_atomic_load(other + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        w1 = __hip_atomic_load(other + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        got = (unsigned)w0 == epoch && (unsigned)w1 == epoch;
+        if (!got) __builtin_amdgcn_s_sleep(4);
+      } while (!got && wall_clock64() - t0 < spin_ticks);
+    }
+    theirs[0] = __uint_as_float((unsigned)(w0 >> 32));
+    theirs[1] = __uint_as_float((unsigned)(w1 >> 32));
+    theirs[2] = got ? 1.f : 0.f;
+  }
+  __syncthreads();
+  float o1 = theirs[0], o2 = theirs[1];
+  if (theirs[2] == 0.f) {
+    // the partner did not answer: its half, summed here the way it sums it
+    float t1 = 0.f, t2 = 0.f;
+    res_visit<T, K2, 4, 4>(g, [&](int, int off, bool in) {
+      const float4 xv = buf_ld4(xr_, off, x), d = buf_ld4(dyr_, off, dy);
+      float p1, p2;
+      bn_pair_partial(d, xv, mean, &p1, &p2);
+      t1 += in ? p1 : 0.f;
+      t2 += in ? p2 : 0.f;
+      asm volatile("" : "+v"(t1), "+v"(t2));
+    }, q0_theirs, c);
+    o1 = block_sum(t1, red);
+    o2 = block_sum(t2, red);
+  }
+  // the first half's sums first, in both workgroups
+  const float S1 = half == 0 ? s1 + o1 : o1 + s1, S2 = half == 0 ? s2 + o2 : o2 + s2;
+  finish_bwd(g, a, c, (double)S1, (double)S2, half == 0, sh);
+  __syncthreads();
+  const float kdy = sh[1], kx = sh[2], k0 = sh[3];
+  res_visit<T, K2, 4, 4, true>(g, [&](int k, int off, bool) {
+    const float4 d = k < KL ? dyl[k * T + tid] : dr[k - KL < 0 ? 0 : k - KL];
+    const float4 v = make_float4(kdy * d.x + (kx * (xr[k].x - mean) + k0), kdy * d.y + (kx * (xr[k].y - mean) + k0),
+                                 kdy * d.z + (kx * (xr[k].z - mean) + k0), kdy * d.w + (kx * (xr[k].w - mean) + k0));
+    buf_st4(dxr_, off, v, dx);
+  }, q0, c);
 }
 
 // ---- resident kernels for bf16 storage, eight elements (16 bytes) per slot ----------------
@@ -1253,6 +1351,46 @@ static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws
   return check_launch("bn_fwd_train");
 }
 
+// The kernel that shares a feature between two workgroups: fp32, rows of a multiple of 4 elements, features of 10
+// to 26 vectors per thread (fewer are parked in LDS whole by the one-workgroup kernel), a multiple of 8 features.
+// Selected with BN_ALGO=pair; =pairalone makes every workgroup sum its partner's half itself (the path taken when
+// the partner does not answer; tests).
+// Returns -1 when it does not apply.
+static int try_bwd_pair(const BnGeom& g, int vec, const float* x, const float* dy, float* dx, float* ws,
+                        const BnBwdArgs& a, hipStream_t s) {
+  const int mode = options().bn_algo;
+  // Only on request: measured at 56x56x256x32 it is slower than the one-workgroup kernel (57.3 against 52.8 us; it
+  // moves 3T instead of 3.45T, but 512 workgroups of 1024 threads are two rounds at one per CU, each with its own
+  // start-up, exchange and tail, and 3T in 57 us is the rate of the plain two-reads-one-write streaming kernel).
+  if ((mode != 3 && mode != 4) || vec != 4) return -1;
+  if (g.C % 8 != 0) return -1;
+  if (g.units <= (long long)RES_KL * 1024 || g.units > 26ll * 1024) return -1;
+  if (g.outer * g.C * g.inner * 4 >= (1ll << 31) || reinterpret_cast<uintptr_t>(ws) % 8 != 0) return -1;
+  // launch number: tells this launch's words in the exchange area from whatever the memory held before
+  static std::atomic<unsigned> launches{
+      (unsigned)std::chrono::steady_clock::now().time_since_epoch().count() * 2654435761u};
+  unsigned epoch = ++launches;
+  if (epoch == 0) epoch = ++launches;
+  const unsigned spin = mode == 4 ? 0u : 50000u;     // ticks of the 100 MHz wall clock: 0.5 ms
+  const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * 4);
+  const int need = (int)((g.units + 1023) / 1024);
+  auto* xch = reinterpret_cast<unsigned long long*>(ws);
+  const dim3 grid((unsigned)(2 * g.C));
+#define BN_PAIR_LAUNCH(K2, KR)                                                                                    \
+  {                                                                                                               \
+    auto kernel = bn_bwd_pair<K2, KR>;                                                                            \
+    constexpr size_t shmem = (size_t)(K2 - KR) * 1024 * sizeof(float4);                                           \
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                     \
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);   \
+    if (attr != hipSuccess) return -1;                                                                            \
+    hipLaunchKernelGGL(kernel, grid, dim3(1024), shmem, s, g, bytes, x, dy, dx, a, xch, epoch, spin);             \
+  }
+  if (need <= 16) BN_PAIR_LAUNCH(8, 0)
+  else BN_PAIR_LAUNCH(13, 4)
+#undef BN_PAIR_LAUNCH
+  return check_launch("bn_bwd (a feature on two workgroups)");
+}
+
 // FUSE: the gradient first passes the ReLU mask of the forward result, read from y (1) or from the mask bytes (2)
 template <typename T, int FUSE>
 static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void* dx, float* ws,
@@ -1266,6 +1404,11 @@ static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void
     if (r8.threads)
       return run_bwd8<FUSE>(g, r8, reinterpret_cast<const bf16_t*>(xp), reinterpret_cast<const bf16_t*>(dyp),
                             reinterpret_cast<bf16_t*>(dxp), a, reinterpret_cast<const BnFuseBwd<bf16_t>&>(fu), s);
+  }
+  if (sizeof(T) == 4 && FUSE == 0) {
+    const int rc = try_bwd_pair(g, vec, reinterpret_cast<const float*>(xp), reinterpret_cast<const float*>(dyp),
+                                reinterpret_cast<float*>(dxp), ws, a, s);
+    if (rc >= 0) return rc;
   }
   {
     const ResPlan r = resident_plan(g, vec, RES_MIN_C_BWD);
@@ -1318,7 +1461,9 @@ extern "C" size_t flhip_bn_workspace_bytes(const flhip_bn_desc* d) {
   BnGeom g;
   int vec;
   if (make_geom(d, &g, &vec) != FLHIP_OK) return 0;
-  return (size_t)g.C * g.S * 2 * sizeof(float);
+  // the partial sums of the two-pass kernels; 32 bytes per feature for the kernel that shares a feature between two workgroups
+  const size_t two_pass = (size_t)g.C * g.S * 2 * sizeof(float), pair = (size_t)g.C * 32;
+  return two_pass > pair ? two_pass : pair;
 }
 
 extern "C" int flhip_bn_fwd_train(const flhip_bn_desc* d, const void* x, const float* gamma,
