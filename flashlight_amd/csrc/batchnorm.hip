@@ -18,6 +18,16 @@
 
 namespace flhip {
 
+int mfma_num_cus();   // compute units of the current device (defined with the convolution kernels)
+
+// Time stamps of the phases of a workgroup, for builds with -DBN_STAMPS only (timing studies).
+#ifdef BN_STAMPS
+__device__ unsigned long long bn_stamps[256 * 8];
+#define BN_STAMP(i) { if (threadIdx.x == 0 && blockIdx.x < 256) bn_stamps[blockIdx.x * 8 + (i)] = wall_clock64(); }
+#else
+#define BN_STAMP(i) {}
+#endif
+
 struct BnGeom {
   long long outer, C, inner;
   int S;            // slices per feature
@@ -43,6 +53,18 @@ __device__ __forceinline__ void fold_partials(const float* __restrict__ ws, long
   }
   *a = wave_sum_f64(p0);
   *b = wave_sum_f64(p1);
+}
+
+// the two sums of a kernel together where its registers allow (the kernels that hold 25 vectors per thread
+// have none to spare for the second sum's lanes in flight)
+template <bool TOGETHER>
+__device__ __forceinline__ void block_sums(float& a, float& b, float* red) {
+  if (TOGETHER) {
+    block_sum2(a, b, red);
+  } else {
+    a = block_sum(a, red);
+    b = block_sum(b, red);
+  }
 }
 
 template <typename T, int VEC>
@@ -135,8 +157,7 @@ bn_stats_seg(BnGeom g, const T* __restrict__ x, float* __restrict__ ws) {
       }
     }
   });
-  s1 = block_sum(s1, red);
-  s2 = block_sum(s2, red);
+  block_sum2(s1, s2, red);
   if (threadIdx.x == 0) {
     ws[(c * g.S + blockIdx.y) * 2 + 0] = s1;
     ws[(c * g.S + blockIdx.y) * 2 + 1] = s2;
@@ -155,9 +176,25 @@ struct BnTrainArgs {
 
 // Mean / inverse std of feature c from the folded shifted sums; lane 0 of wave 0
 // of slice 0 also publishes the statistics.
+// Per-feature scalars of the forward kernels, loaded when the kernel starts: a load issued only where its value
+// is used (after the reduction, after the barrier) adds a trip to memory to the chain reduction -> statistics ->
+// output, which is most of the time of a layer with small planes.
+struct BnTrainPre {
+  float gamma, beta, run_mean, run_var;
+};
+__device__ __forceinline__ BnTrainPre bn_preload(const BnTrainArgs& a, long long c, bool publish = true) {
+  BnTrainPre p;
+  p.gamma = a.gamma ? a.gamma[c] : 1.f;
+  p.beta = a.beta ? a.beta[c] : 0.f;
+  const bool run = publish && a.run_mean && a.run_var && a.momentum != 0.0;
+  p.run_mean = run ? a.run_mean[c] : 0.f;
+  p.run_var = run ? a.run_var[c] : 0.f;
+  return p;
+}
+
 __device__ __forceinline__ void finish_stats(const BnGeom& g, const BnTrainArgs& a, long long c,
                                              float shift, double p0, double p1, bool publish,
-                                             float* sh /* [2] */) {
+                                             float* sh /* [2] */, const BnTrainPre* pre /* null: loaded here */) {
   if (threadIdx.x == 0) {
     const double M = (double)g.outer * (double)g.inner;
     const double m1 = p0 / M;
@@ -176,8 +213,9 @@ __device__ __forceinline__ void finish_stats(const BnGeom& g, const BnTrainArgs&
           a.run_var[c] = (float)var;
         } else {
           const double unb = M > 1.0 ? var * M / (M - 1.0) : var;
-          a.run_mean[c] = (float)((1.0 - a.momentum) * (double)a.run_mean[c] + a.momentum * mean);
-          a.run_var[c] = (float)((1.0 - a.momentum) * (double)a.run_var[c] + a.momentum * unb);
+          const double rm = pre ? pre->run_mean : a.run_mean[c], rv = pre ? pre->run_var : a.run_var[c];
+          a.run_mean[c] = (float)((1.0 - a.momentum) * rm + a.momentum * mean);
+          a.run_var[c] = (float)((1.0 - a.momentum) * rv + a.momentum * unb);
         }
       }
     }
@@ -224,17 +262,17 @@ __global__ void __launch_bounds__(256)
 bn_train_apply_seg(BnGeom g, const T* __restrict__ x, T* __restrict__ y,
                    const float* __restrict__ ws, BnTrainArgs a, BnFuseFwd<T> fu = BnFuseFwd<T>{nullptr, 0, nullptr}) {
   __shared__ float sh[2];
+  const BnTrainPre pre = bn_preload(a, blockIdx.x, blockIdx.y == 0);
   if (threadIdx.x < 64) {
     double p0, p1;
     fold_partials(ws, blockIdx.x, g.S, &p0, &p1);
     finish_stats(g, a, blockIdx.x, ld(x, (size_t)(blockIdx.x * g.inner)), p0, p1,
-                 blockIdx.y == 0, sh);
+                 blockIdx.y == 0, sh, &pre);
   }
   __syncthreads();
   const float mean = sh[0];
-  const float gm = a.gamma ? a.gamma[blockIdx.x] : 1.f;
-  const float scale = gm * sh[1];
-  const float bt = a.beta ? a.beta[blockIdx.x] : 0.f;
+  const float scale = pre.gamma * sh[1];
+  const float bt = pre.beta;
   bn_seg_visit<VEC, true>(g, [&](const size_t (&off)[BN_UN], int n) {
     Vec<T, VEC> v[BN_UN], r[BN_UN];
 #pragma unroll
@@ -301,8 +339,7 @@ bn_bwd_stats_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
       }
     }
   });
-  s1 = block_sum(s1, red);
-  s2 = block_sum(s2, red);
+  block_sum2(s1, s2, red);
   if (threadIdx.x == 0) {
     ws[(c * g.S + blockIdx.y) * 2 + 0] = s1;
     ws[(c * g.S + blockIdx.y) * 2 + 1] = s2;
@@ -318,13 +355,24 @@ struct BnBwdArgs {
 };
 
 // dx = k_dy*dy + k_x*(x-mean) + k_0 for feature c; publishes dgamma/dbeta.
+// (pre: the feature's scalars, loaded when the kernel starts - see BnTrainPre)
+struct BnBwdPre {
+  float mean, invstd, gamma;
+};
+__device__ __forceinline__ BnBwdPre bn_preload(const BnBwdArgs& a, long long c) {
+  BnBwdPre p;
+  p.mean = a.save_mean[c];
+  p.invstd = a.save_invstd[c];
+  p.gamma = a.gamma ? a.gamma[c] : 1.f;
+  return p;
+}
 __device__ __forceinline__ void finish_bwd(const BnGeom& g, const BnBwdArgs& a, long long c,
-                                           double p0, double p1, bool publish, float* sh /*[4]*/) {
+                                           double p0, double p1, bool publish, float* sh /*[4]*/, const BnBwdPre& pre) {
   if (threadIdx.x == 0) {
     const double M = (double)g.outer * (double)g.inner;
-    const double is = (double)a.save_invstd[c];
-    const double gm = a.gamma ? (double)a.gamma[c] : 1.0;
-    sh[0] = a.save_mean[c];
+    const double is = (double)pre.invstd;
+    const double gm = (double)pre.gamma;
+    sh[0] = pre.mean;
     sh[1] = (float)(gm * is);                    // k_dy
     sh[2] = (float)(-gm * is * is * is * p1 / M);  // k_x
     sh[3] = (float)(-gm * is * p0 / M);          // k_0
@@ -341,10 +389,11 @@ bn_bwd_apply_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
                  T* __restrict__ dx, const float* __restrict__ ws, BnBwdArgs a,
                  BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr, nullptr}) {
   __shared__ float sh[4];
+  const BnBwdPre pre = bn_preload(a, blockIdx.x);
   if (threadIdx.x < 64) {
     double p0, p1;
     fold_partials(ws, blockIdx.x, g.S, &p0, &p1);
-    finish_bwd(g, a, blockIdx.x, p0, p1, blockIdx.y == 0, sh);
+    finish_bwd(g, a, blockIdx.x, p0, p1, blockIdx.y == 0, sh, pre);
   }
   __syncthreads();
   const float mean = sh[0], kdy = sh[1], kx = sh[2], k0 = sh[3];
@@ -467,6 +516,31 @@ __device__ __forceinline__ float4 buf_ld4_stream(__amdgpu_buffer_rsrc_t r, int b
                      __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
 }
 
+// the same loads with the widening left for later: a vector that waits in registers stays at its storage size
+template <typename T>
+struct Raw4;
+template <>
+struct Raw4<float> {
+  uintx4_t v;
+};
+template <>
+struct Raw4<bf16_t> {
+  uintx2_t v;
+};
+__device__ __forceinline__ Raw4<float> buf_ld4_raw(__amdgpu_buffer_rsrc_t r, int byte_off, const float*) {
+  return Raw4<float>{__builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 2)};
+}
+__device__ __forceinline__ Raw4<bf16_t> buf_ld4_raw(__amdgpu_buffer_rsrc_t r, int byte_off, const bf16_t*) {
+  return Raw4<bf16_t>{__builtin_amdgcn_raw_buffer_load_b64(r, byte_off, 0, 2)};
+}
+__device__ __forceinline__ float4 widen(const Raw4<float>& w) {
+  return make_float4(__uint_as_float(w.v.x), __uint_as_float(w.v.y), __uint_as_float(w.v.z), __uint_as_float(w.v.w));
+}
+__device__ __forceinline__ float4 widen(const Raw4<bf16_t>& w) {
+  return make_float4(__uint_as_float(w.v.x << 16), __uint_as_float(w.v.x & 0xffff0000u),
+                     __uint_as_float(w.v.y << 16), __uint_as_float(w.v.y & 0xffff0000u));
+}
+
 // 16-byte (float) / 8-byte (bf16) buffer store of four values, streaming
 __device__ __forceinline__ void buf_st4(__amdgpu_buffer_rsrc_t r, int byte_off, float4 v, float*) {
   const uintx4_t t = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z),
@@ -479,19 +553,31 @@ __device__ __forceinline__ void buf_st4(__amdgpu_buffer_rsrc_t r, int byte_off, 
   __builtin_amdgcn_raw_buffer_store_b64(t, r, byte_off, 0, 2);
 }
 
-template <typename T, int RES_THREADS, int K, int FUSE = 0>
+template <typename T, int RES_THREADS, int K, int FUSE = 0, bool RES_EARLY = false>
 __global__ void __launch_bounds__(RES_THREADS)
 bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restrict__ y,
                   BnTrainArgs a, BnFuseFwd<T> fu = BnFuseFwd<T>{nullptr, 0, nullptr}) {
-  __shared__ float red[RES_THREADS / 64];
+  __shared__ float red[2 * (RES_THREADS / 64)];
   __shared__ float sh[2];
   constexpr int ESZ = (int)sizeof(T);
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
   const long long c = res_feature(g);
+  BN_STAMP(0)
   const float shift = ld(x, (size_t)(c * g.inner));
+  // (the kernels that hold 25 vectors per thread have no registers to keep the scalars through the statistics)
+  constexpr bool EARLY = K <= 16;
+  BnTrainPre pre = EARLY ? bn_preload(a, c) : BnTrainPre{};
   float4 xr[K];
   float s1 = 0.f, s2 = 0.f;
   res_visit<RES_THREADS, K, ESZ, 0>(g, [&](int k, int off, bool in) { xr[k] = buf_ld4_stream(xr_, off, x); });
+  // RES_EARLY (workgroups of 4 waves, at most two of them on a CU): the residual is fetched together with x.
+  // Fetched where it is used, four vectors at a time (what the large kernels can afford), every group waits for a
+  // trip to memory, and with so few waves on a CU nothing else runs meanwhile.  It costs a thread up to 32
+  // registers, which layers with more workgroups per CU rather spend on one more of those.
+  constexpr bool PRE = FUSE && RES_EARLY;
+  const __amdgpu_buffer_rsrc_t rr_ = make_rsrc((FUSE && fu.res) ? fu.res : x, (FUSE && fu.res) ? bytes : 0u);   // no residual: loads give 0
+  Raw4<T> rz[PRE ? K : 1];
+  if (PRE) res_visit<RES_THREADS, K, ESZ, 0>(g, [&](int k, int off, bool) { rz[k] = buf_ld4_raw(rr_, off, x); });
   res_visit<RES_THREADS, K, ESZ, 1>(g, [&](int k, int, bool in) {
     const float t0 = xr[k].x - shift, t1 = xr[k].y - shift, t2 = xr[k].z - shift,
                 t3 = xr[k].w - shift;
@@ -501,21 +587,23 @@ bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restri
     s2 += in ? p2 : 0.f;
     // both sums are finished per vector: otherwise the second one is sunk below the
     // first block reduction and drags every vector's temporaries along
-    asm volatile("" : "+v"(s1), "+v"(s2));
+    asm("" : "+v"(s1), "+v"(s2));
   });
-  s1 = block_sum(s1, red);
-  s2 = block_sum(s2, red);
-  finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh);
+  BN_STAMP(1)
+  block_sums<(K <= 16)>(s1, s2, red);
+  BN_STAMP(2)
+  finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh, EARLY ? &pre : nullptr);
   __syncthreads();
+  BN_STAMP(3)
+  if (!EARLY) pre = bn_preload(a, c, false);
   const float mean = sh[0];
-  const float scale = (a.gamma ? a.gamma[c] : 1.f) * sh[1];
-  const float bt = a.beta ? a.beta[c] : 0.f;
+  const float scale = pre.gamma * sh[1];
+  const float bt = pre.beta;
   if (FUSE) {
-    const __amdgpu_buffer_rsrc_t rr_ = make_rsrc(fu.res ? fu.res : x, fu.res ? bytes : 0u);   // no residual: loads give 0
     const __amdgpu_buffer_rsrc_t mr_ = mask_rsrc(FUSE == 2 ? fu.mask : nullptr, x, bytes, ESZ);   // one byte per vector
     const float lo = fu.relu ? 0.f : -__builtin_huge_valf();
     res_visit<RES_THREADS, K, ESZ, 4>(g, [&](int k, int off, bool) {
-      const float4 r = buf_ld4_stream(rr_, off, x);
+      const float4 r = PRE ? widen(rz[PRE ? k : 0]) : buf_ld4_stream(rr_, off, x);
       const float4 v = make_float4(fmaxf((xr[k].x - mean) * scale + bt + r.x, lo), fmaxf((xr[k].y - mean) * scale + bt + r.y, lo),
                                    fmaxf((xr[k].z - mean) * scale + bt + r.z, lo), fmaxf((xr[k].w - mean) * scale + bt + r.w, lo));
       buf_st4(yr_, off, v, y);
@@ -525,6 +613,11 @@ bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restri
         __builtin_amdgcn_raw_buffer_store_b8((uint8_t)bits, mr_, mask_off(off, ESZ), 0, 0);
       }
     });
+    BN_STAMP(4)
+#ifdef BN_STAMPS
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    BN_STAMP(5)
+#endif
     return;
   }
   res_visit<RES_THREADS, K, ESZ, 1>(g, [&](int k, int off, bool) {
@@ -546,25 +639,57 @@ __global__ void __launch_bounds__(RES_THREADS)
 bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, const T* __restrict__ dy,
                 T* __restrict__ dx, BnBwdArgs a, BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr, nullptr}) {
   extern __shared__ float4 dyl[];           // [klim][threads], klim <= min(K, RES_KL)
-  __shared__ float red[RES_THREADS / 64];
+  __shared__ float red[2 * (RES_THREADS / 64)];
   __shared__ float sh[4];
   constexpr int ESZ = (int)sizeof(T);
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes),
                                dxr_ = make_rsrc(dx, bytes);
   const long long c = res_feature(g);
-  const float mean = a.save_mean[c];
+  BN_STAMP(0)
+  const BnBwdPre pre = bn_preload(a, c);
+  const float mean = pre.mean;
   float4 xr[K];
   float s1 = 0.f, s2 = 0.f;
-  res_visit<RES_THREADS, K, ESZ, 0>(g, [&](int k, int off, bool in) { xr[k] = buf_ld4_stream(xr_, off, x); });
   constexpr bool MASK = FUSE == 2;   // the ReLU mask comes as bytes, not from y
-  res_visit<RES_THREADS, K, ESZ, 4>(g, [&](int k, int off, bool in) {
-    // dy vectors that stay in LDS are read once; the others come back in the second walk
-    float4 d = k < klim ? buf_ld4_stream(dyr_, off, dy) : buf_ld4(dyr_, off, dy);
-    if (FUSE) {
-      if (MASK) d = relu_bits(d, __builtin_amdgcn_raw_buffer_load_b8(mask_rsrc(fu.mask, x, bytes, ESZ), mask_off(off, ESZ), 0, 0));
-      else d = relu_mask(d, k < klim ? buf_ld4_stream(make_rsrc(fu.y, bytes), off, dy) : buf_ld4(make_rsrc(fu.y, bytes), off, dy));
+  // Small features (workgroups of 4 waves, or 8 vectors per thread) keep dy in registers as well, at its storage
+  // size, and fetch it together with x: in the walk below every vector's loads wait behind the sums of the
+  // vector before (the statement that pins the sums orders memory operations too), which the large kernels hide
+  // behind their 16 waves and a CU with 4 waves does not - 13 trips to memory one after the other, 10 of the
+  // 16 us of a 14x14 layer of 256 features.  Nothing is parked in LDS then, and nothing is read twice.
+  constexpr bool REGS = RES_THREADS == 256 || K <= 8;
+  constexpr int FB = 4;     // groups of four vectors, or the temporaries of all of them overlap and the registers run out
+  Raw4<T> dr[REGS ? K : 1], yw[REGS && FUSE == 1 ? K : 1];
+  unsigned mb[REGS && FUSE ? K : 1];
+  res_visit<RES_THREADS, K, ESZ, 0>(g, [&](int k, int off, bool) {
+    xr[k] = buf_ld4_stream(xr_, off, x);
+    if (REGS) {
+      dr[REGS ? k : 0] = buf_ld4_raw(dyr_, off, dy);
+      if (MASK) mb[REGS && FUSE ? k : 0] = __builtin_amdgcn_raw_buffer_load_b8(mask_rsrc(fu.mask, x, bytes, ESZ), mask_off(off, ESZ), 0, 0);
+      else if (FUSE) yw[REGS && FUSE == 1 ? k : 0] = buf_ld4_raw(make_rsrc(fu.y, bytes), off, dy);
     }
-    if (k < klim) dyl[k * RES_THREADS + threadIdx.x] = d;
+  });
+  // the gradient of vector k after the mask, from the registers
+  auto masked = [&](int k) {
+    const float4 d = widen(dr[REGS ? k : 0]);
+    return FUSE ? relu_bits(d, mb[REGS && FUSE ? k : 0]) : d;
+  };
+  res_visit<RES_THREADS, K, ESZ, FB>(g, [&](int k, int off, bool in) {
+    float4 d;
+    if (REGS) {
+      if (FUSE == 1) {
+        const float4 yv = widen(yw[REGS && FUSE == 1 ? k : 0]);
+        mb[REGS && FUSE ? k : 0] = (yv.x > 0.f ? 1u : 0u) | (yv.y > 0.f ? 2u : 0u) | (yv.z > 0.f ? 4u : 0u) | (yv.w > 0.f ? 8u : 0u);
+      }
+      d = masked(k);
+    } else {
+      // dy vectors that stay in LDS are read once; the others come back in the second walk
+      d = k < klim ? buf_ld4_stream(dyr_, off, dy) : buf_ld4(dyr_, off, dy);
+      if (FUSE) {
+        if (MASK) d = relu_bits(d, __builtin_amdgcn_raw_buffer_load_b8(mask_rsrc(fu.mask, x, bytes, ESZ), mask_off(off, ESZ), 0, 0));
+        else d = relu_mask(d, k < klim ? buf_ld4_stream(make_rsrc(fu.y, bytes), off, dy) : buf_ld4(make_rsrc(fu.y, bytes), off, dy));
+      }
+      if (k < klim) dyl[k * RES_THREADS + threadIdx.x] = d;
+    }
     const float p1 = (d.x + d.y) + (d.z + d.w);
     const float p2 = (d.x * (xr[k].x - mean) + d.y * (xr[k].y - mean)) +
                      (d.z * (xr[k].z - mean) + d.w * (xr[k].w - mean));
@@ -572,17 +697,19 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
     s2 += in ? p2 : 0.f;
     // both sums are finished per vector: otherwise the second one is sunk below the
     // first block reduction and drags every vector's temporaries along
-    asm volatile("" : "+v"(s1), "+v"(s2));
+    asm("" : "+v"(s1), "+v"(s2));
   });
-  s1 = block_sum(s1, red);
-  s2 = block_sum(s2, red);
-  finish_bwd(g, a, c, (double)s1, (double)s2, true, sh);
+  BN_STAMP(1)
+  block_sums<(K <= 16)>(s1, s2, red);
+  BN_STAMP(2)
+  finish_bwd(g, a, c, (double)s1, (double)s2, true, sh, pre);
   __syncthreads();
+  BN_STAMP(3)
   const float kdy = sh[1], kx = sh[2], k0 = sh[3];
-  res_visit<RES_THREADS, K, ESZ, 4, true>(g, [&](int k, int off, bool) {
-    float4 d = k < klim ? dyl[k * RES_THREADS + threadIdx.x] : buf_ld4(dyr_, off, dy);
+  res_visit<RES_THREADS, K, ESZ, FB, true>(g, [&](int k, int off, bool) {
+    float4 d = REGS ? masked(k) : k < klim ? dyl[k * RES_THREADS + threadIdx.x] : buf_ld4(dyr_, off, dy);
     // the part of dy that did not fit in LDS passes the mask again (y re-read with it)
-    if (FUSE && k >= klim) {
+    if (!REGS && FUSE && k >= klim) {
       if (MASK) d = relu_bits(d, __builtin_amdgcn_raw_buffer_load_b8(mask_rsrc(fu.mask, x, bytes, ESZ), mask_off(off, ESZ), 0, 0));
       else d = relu_mask(d, buf_ld4(make_rsrc(fu.y, bytes), off, dy));
     }
@@ -593,6 +720,11 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
     buf_st4(dxr_, off, v, dx);
     if (FUSE && fu.dres) buf_st4(make_rsrc(fu.dres, bytes), off, d, dx);
   });
+  BN_STAMP(4)
+#ifdef BN_STAMPS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  BN_STAMP(5)
+#endif
 }
 
 // ---- backward, a feature shared by two workgroups (fp32, features of 10 to 26 vectors per thread) ---------
@@ -616,7 +748,7 @@ bn_bwd_pair(BnGeom g, unsigned bytes, const float* __restrict__ x, const float* 
             float* __restrict__ dx, BnBwdArgs a, unsigned long long* xch, unsigned epoch, unsigned spin_ticks) {
   constexpr int T = 1024, KL = K2 - KR;
   extern __shared__ float4 dyl[];           // [KL][T]
-  __shared__ float red[T / 64];
+  __shared__ float red[2 * (T / 64)];
   __shared__ float sh[4];
   __shared__ float theirs[3];               // the partner's sums, and whether they arrived
   const int tid = threadIdx.x;
@@ -625,7 +757,8 @@ bn_bwd_pair(BnGeom g, unsigned bytes, const float* __restrict__ x, const float* 
   const int c = (fs & 7) * (C >> 3) + (fs >> 3);      // neighbouring features on one XCD, as res_feature
   const int q0 = half * K2 * T, q0_theirs = (half ^ 1) * K2 * T;
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes), dxr_ = make_rsrc(dx, bytes);
-  const float mean = a.save_mean[c];
+  const BnBwdPre pre = bn_preload(a, c);
+  const float mean = pre.mean;
   float4 xr[K2], dr[KR > 0 ? KR : 1];
   float s1 = 0.f, s2 = 0.f;
   res_visit<T, K2, 4, 0>(g, [&](int k, int off, bool) { xr[k] = buf_ld4_stream(xr_, off, x); }, q0, c);
@@ -637,7 +770,7 @@ bn_bwd_pair(BnGeom g, unsigned bytes, const float* __restrict__ x, const float* 
     bn_pair_partial(d, xr[k], mean, &p1, &p2);
     s1 += in ? p1 : 0.f;
     s2 += in ? p2 : 0.f;
-    asm volatile("" : "+v"(s1), "+v"(s2));
+    asm("" : "+v"(s1), "+v"(s2));
   }, q0, c);
   s1 = block_sum(s1, red);
   s2 = block_sum(s2, red);
@@ -672,14 +805,14 @@ bn_bwd_pair(BnGeom g, unsigned bytes, const float* __restrict__ x, const float* 
       bn_pair_partial(d, xv, mean, &p1, &p2);
       t1 += in ? p1 : 0.f;
       t2 += in ? p2 : 0.f;
-      asm volatile("" : "+v"(t1), "+v"(t2));
+      asm("" : "+v"(t1), "+v"(t2));
     }, q0_theirs, c);
     o1 = block_sum(t1, red);
     o2 = block_sum(t2, red);
   }
   // the first half's sums first, in both workgroups
   const float S1 = half == 0 ? s1 + o1 : o1 + s1, S2 = half == 0 ? s2 + o2 : o2 + s2;
-  finish_bwd(g, a, c, (double)S1, (double)S2, half == 0, sh);
+  finish_bwd(g, a, c, (double)S1, (double)S2, half == 0, sh, pre);
   __syncthreads();
   const float kdy = sh[1], kx = sh[2], k0 = sh[3];
   res_visit<T, K2, 4, 4, true>(g, [&](int k, int off, bool) {
@@ -718,17 +851,21 @@ __device__ __forceinline__ uint32_t relu_mask2(uint32_t d, uint32_t y) {
 // Makes the packed values opaque to the optimiser: without it the unpacked floats of one
 // walk over the resident vectors are kept alive for the next walk (8 registers per vector)
 // instead of being recomputed from the 4 packed ones.
-__device__ __forceinline__ void opaque(uint4& v) { asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
+// (not volatile: a volatile statement would also order the loads around it, one vector behind the other)
+__device__ __forceinline__ void opaque(uint4& v) { asm("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
 __device__ __forceinline__ uint4 relu_mask8(uint4 d, uint4 y) {
   return make_uint4(relu_mask2(d.x, y.x), relu_mask2(d.y, y.y), relu_mask2(d.z, y.z), relu_mask2(d.w, y.w));
 }
 // the same from the two mask bytes of the vector: bit e of byte j stands for element 4 j + e
-__device__ __forceinline__ uint32_t relu_bits2(uint32_t d, unsigned lo, unsigned hi) {
-  return (lo ? d & 0x0000ffffu : 0u) | (hi ? d & 0xffff0000u : 0u);
+// (bit `at` of b for the low half of the word, bit at + 1 for the high half; the two bits are spread to
+// all-ones / zero words with shifts, not with selects: eight selects per vector each want a lane mask in
+// scalar registers, and a few vectors' worth of those do not fit)
+__device__ __forceinline__ uint32_t relu_bits2(uint32_t d, unsigned b, int at) {
+  const uint32_t ml = (uint32_t)((int)(b << (31 - at)) >> 31), mh = (uint32_t)((int)(b << (30 - at)) >> 31);
+  return d & ((ml & 0x0000ffffu) | (mh & 0xffff0000u));
 }
 __device__ __forceinline__ uint4 relu_bits8(uint4 d, unsigned b) {
-  return make_uint4(relu_bits2(d.x, b & 1u, b & 2u), relu_bits2(d.y, b & 4u, b & 8u), relu_bits2(d.z, b & 0x100u, b & 0x200u),
-                    relu_bits2(d.w, b & 0x400u, b & 0x800u));
+  return make_uint4(relu_bits2(d.x, b, 0), relu_bits2(d.y, b, 2), relu_bits2(d.z, b, 8), relu_bits2(d.w, b, 10));
 }
 
 // A value every lane holds alike, moved to a scalar register (the vector registers of the
@@ -737,18 +874,26 @@ __device__ __forceinline__ float uniform(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
 }
 
-template <int RES_THREADS, int K, int FUSE = 0>
+template <int RES_THREADS, int K, int FUSE = 0, bool RES_EARLY = false>
 __global__ void __launch_bounds__(RES_THREADS)
 bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_t* __restrict__ y,
                    BnTrainArgs a, BnFuseFwd<bf16_t> fu = BnFuseFwd<bf16_t>{nullptr, 0, nullptr}) {
-  __shared__ float red[RES_THREADS / 64];
+  __shared__ float red[2 * (RES_THREADS / 64)];
   __shared__ float sh[2];
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
   const long long c = res_feature(g);
   const float shift = ld(x, (size_t)(c * g.inner));
+  // (the kernels that hold 25 vectors per thread have no registers to keep the scalars through the statistics)
+  constexpr bool EARLY = K <= 16;
+  BnTrainPre pre = EARLY ? bn_preload(a, c) : BnTrainPre{};
   uint4 xr[K];
   float s1 = 0.f, s2 = 0.f;
   res_visit<RES_THREADS, K, 2, 0, false, 8>(g, [&](int k, int off, bool) { xr[k] = buf_ld8(xr_, off, true); });
+  // (RES_EARLY: see bn_train_resident)
+  constexpr bool PRE = FUSE && RES_EARLY;
+  const __amdgpu_buffer_rsrc_t rr_ = make_rsrc((FUSE && fu.res) ? fu.res : x, (FUSE && fu.res) ? bytes : 0u);
+  uint4 rz[PRE ? K : 1];
+  if (PRE) res_visit<RES_THREADS, K, 2, 0, false, 8>(g, [&](int k, int off, bool) { rz[k] = buf_ld8(rr_, off, true); });
   res_visit<RES_THREADS, K, 2, 1, false, 8>(g, [&](int k, int, bool in) {
     opaque(xr[k]);
     const uint32_t w[4] = {xr[k].x, xr[k].y, xr[k].z, xr[k].w};
@@ -761,16 +906,15 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
     }
     s1 += in ? p1 : 0.f;
     s2 += in ? p2 : 0.f;
-    asm volatile("" : "+v"(s1), "+v"(s2));
+    asm("" : "+v"(s1), "+v"(s2));
   });
-  s1 = block_sum(s1, red);
-  s2 = block_sum(s2, red);
-  finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh);
+  block_sums<(K <= 16)>(s1, s2, red);
+  finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh, EARLY ? &pre : nullptr);
   __syncthreads();
+  if (!EARLY) pre = bn_preload(a, c, false);
   const float mean = uniform(sh[0]);
-  const float scale = uniform((a.gamma ? a.gamma[c] : 1.f) * sh[1]);
-  const float bt = uniform(a.beta ? a.beta[c] : 0.f);
-  const __amdgpu_buffer_rsrc_t rr_ = make_rsrc((FUSE && fu.res) ? fu.res : x, (FUSE && fu.res) ? bytes : 0u);
+  const float scale = uniform(pre.gamma * sh[1]);
+  const float bt = uniform(pre.beta);
   const __amdgpu_buffer_rsrc_t mr_ = mask_rsrc(FUSE == 2 ? fu.mask : nullptr, x, bytes, 2);
   const float lo = (FUSE && fu.relu) ? 0.f : -__builtin_huge_valf();
   res_visit<RES_THREADS, K, 2, 1, false, 8>(g, [&](int k, int off, bool) {
@@ -779,7 +923,7 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
     uint4 v = xr[k];
     opaque(v);
     if (FUSE) {
-      const uint4 rv = buf_ld8(rr_, off, true);      // no residual: the empty range reads zeros
+      const uint4 rv = PRE ? rz[PRE ? k : 0] : buf_ld8(rr_, off, true);      // no residual: the empty range reads zeros
       // (relu leaves no NaN, so the sign tests on the packed words equal y > 0)
       auto pos = [](uint32_t w, unsigned blo, unsigned bhi) {
         return ((int)(w << 16) > 0 ? blo : 0u) | ((int)(w & 0xffff0000u) > 0 ? bhi : 0u);
@@ -812,7 +956,7 @@ __global__ void __launch_bounds__(RES_THREADS)
 bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy,
                  bf16_t* __restrict__ dx, BnBwdArgs a, BnFuseBwd<bf16_t> fu = BnFuseBwd<bf16_t>{nullptr, nullptr, nullptr}) {
   extern __shared__ uint4 dyl8[];           // [klim][threads] packed gradients (after the mask)
-  __shared__ float red[RES_THREADS / 64];
+  __shared__ float red[2 * (RES_THREADS / 64)];
   __shared__ float sh[4];
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes),
                                dxr_ = make_rsrc(dx, bytes);
@@ -820,18 +964,40 @@ bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ 
   const __amdgpu_buffer_rsrc_t mr_ = mask_rsrc(FUSE == 2 ? fu.mask : nullptr, x, bytes, 2);
   const __amdgpu_buffer_rsrc_t drr_ = make_rsrc((FUSE && fu.dres) ? fu.dres : dx, (FUSE && fu.dres) ? bytes : 0u);
   const long long c = res_feature(g);
-  const float mean = a.save_mean[c];
+  const BnBwdPre pre = bn_preload(a, c);
+  const float mean = pre.mean;
   uint4 xr[K];
   float s1 = 0.f, s2 = 0.f;
-  res_visit<RES_THREADS, K, 2, 0, false, 8>(g, [&](int k, int off, bool) { xr[k] = buf_ld8(xr_, off, true); });
   constexpr bool MASK = FUSE == 2;   // the ReLU mask comes as bytes, not from y
-  res_visit<RES_THREADS, K, 2, 4, false, 8>(g, [&](int k, int off, bool in) {
-    uint4 d = buf_ld8(dyr_, off, k < klim);
-    if (FUSE) {
-      if (MASK) d = relu_bits8(d, __builtin_amdgcn_raw_buffer_load_b16(mr_, mask_off(off, 2), 0, 0));
-      else d = relu_mask8(d, buf_ld8(yr_, off, k < klim));
+  // (REGS: small features keep dy in registers and fetch it together with x - see bn_bwd_resident)
+  constexpr bool REGS = RES_THREADS == 256 || K <= 8;
+  constexpr int FB = 4;
+  uint4 dr[REGS ? K : 1], yw[REGS && FUSE == 1 ? K : 1];
+  unsigned mb[REGS && MASK ? K : 1];
+  res_visit<RES_THREADS, K, 2, 0, false, 8>(g, [&](int k, int off, bool) {
+    xr[k] = buf_ld8(xr_, off, true);
+    if (REGS) {
+      dr[REGS ? k : 0] = buf_ld8(dyr_, off, true);
+      if (MASK) mb[REGS && MASK ? k : 0] = __builtin_amdgcn_raw_buffer_load_b16(mr_, mask_off(off, 2), 0, 0);
+      else if (FUSE) yw[REGS && FUSE == 1 ? k : 0] = buf_ld8(yr_, off, true);
     }
-    if (k < klim) dyl8[k * RES_THREADS + threadIdx.x] = d;
+  });
+  res_visit<RES_THREADS, K, 2, FB, false, 8>(g, [&](int k, int off, bool in) {
+    uint4 d;
+    if (REGS) {
+      opaque(dr[REGS ? k : 0]);      // (or the widening of all vectors is hoisted to where they arrive)
+      d = dr[REGS ? k : 0];
+      if (MASK) d = relu_bits8(d, mb[REGS && MASK ? k : 0]);
+      else if (FUSE) d = relu_mask8(d, yw[REGS && FUSE == 1 ? k : 0]);
+      dr[REGS ? k : 0] = d;          // kept with the mask applied
+    } else {
+      d = buf_ld8(dyr_, off, k < klim);
+      if (FUSE) {
+        if (MASK) d = relu_bits8(d, __builtin_amdgcn_raw_buffer_load_b16(mr_, mask_off(off, 2), 0, 0));
+        else d = relu_mask8(d, buf_ld8(yr_, off, k < klim));
+      }
+      if (k < klim) dyl8[k * RES_THREADS + threadIdx.x] = d;
+    }
     opaque(xr[k]);
     const uint32_t dw[4] = {d.x, d.y, d.z, d.w}, xw[4] = {xr[k].x, xr[k].y, xr[k].z, xr[k].w};
     float p1 = 0.f, p2 = 0.f;
@@ -843,16 +1009,16 @@ bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ 
     }
     s1 += in ? p1 : 0.f;
     s2 += in ? p2 : 0.f;
-    asm volatile("" : "+v"(s1), "+v"(s2));
+    asm("" : "+v"(s1), "+v"(s2));
   });
-  s1 = block_sum(s1, red);
-  s2 = block_sum(s2, red);
-  finish_bwd(g, a, c, (double)s1, (double)s2, true, sh);
+  block_sums<(K <= 16)>(s1, s2, red);
+  finish_bwd(g, a, c, (double)s1, (double)s2, true, sh, pre);
   __syncthreads();
   const float kdy = sh[1], kx = sh[2], k0 = sh[3];
-  res_visit<RES_THREADS, K, 2, 4, true, 8>(g, [&](int k, int off, bool) {
-    uint4 d = k < klim ? dyl8[k * RES_THREADS + threadIdx.x] : buf_ld8(dyr_, off, false);
-    if (FUSE && k >= klim) {
+  res_visit<RES_THREADS, K, 2, FB, true, 8>(g, [&](int k, int off, bool) {
+    if (REGS) opaque(dr[REGS ? k : 0]);
+    uint4 d = REGS ? dr[REGS ? k : 0] : k < klim ? dyl8[k * RES_THREADS + threadIdx.x] : buf_ld8(dyr_, off, false);
+    if (!REGS && FUSE && k >= klim) {
       if (MASK) d = relu_bits8(d, __builtin_amdgcn_raw_buffer_load_b16(mr_, mask_off(off, 2), 0, 0));
       else d = relu_mask8(d, buf_ld8(yr_, off, false));
     }
@@ -905,17 +1071,27 @@ template <typename T, int THREADS, int K, int FUSE = 0>
 __global__ void __launch_bounds__(THREADS)
 bn_train_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restrict__ y,
                    BnTrainArgs a, BnFuseFwd<T> fu = BnFuseFwd<T>{nullptr, 0, nullptr}) {
-  __shared__ float red[THREADS / 64];
+  __shared__ float red[2 * (THREADS / 64)];
   __shared__ float sh[2];
   constexpr int OOB = (int)0x80000000;
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
   const long long c = res_feature(g);
   const float shift = ld(x, (size_t)(c * g.inner));
+  // (the kernels that hold 25 vectors per thread have no registers to keep the scalars through the statistics)
+  constexpr bool EARLY = K <= 16;
+  BnTrainPre pre = EARLY ? bn_preload(a, c) : BnTrainPre{};
   int off[K];
   res1_offsets<THREADS, K, (int)sizeof(T)>(g, off);
   float xv[K];
 #pragma unroll
   for (int k = 0; k < K; ++k) xv[k] = buf_ld(xr_, off[k], x);
+  // the residual comes with x: fetched after the statistics it would add a trip to memory
+  const __amdgpu_buffer_rsrc_t rr_ = make_rsrc((FUSE && fu.res) ? fu.res : x, (FUSE && fu.res) ? bytes : 0u);   // no residual: loads give 0
+  float rv[FUSE ? K : 1];
+  if (FUSE && EARLY) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) rv[k] = buf_ld(rr_, off[k], x);
+  }
   float s1 = 0.f, s2 = 0.f;
 #pragma unroll
   for (int k = 0; k < K; ++k) {
@@ -923,19 +1099,19 @@ bn_train_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restr
     s1 += t;
     s2 += t * t;
   }
-  s1 = block_sum(s1, red);
-  s2 = block_sum(s2, red);
-  finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh);
+  block_sums<(K <= 16)>(s1, s2, red);
+  finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh, EARLY ? &pre : nullptr);
   __syncthreads();
+  if (!EARLY) pre = bn_preload(a, c, false);
   const float mean = sh[0];
-  const float scale = (a.gamma ? a.gamma[c] : 1.f) * sh[1];
-  const float bt = a.beta ? a.beta[c] : 0.f;
+  const float scale = pre.gamma * sh[1];
+  const float bt = pre.beta;
   if (FUSE) {
-    const __amdgpu_buffer_rsrc_t rr_ = make_rsrc(fu.res ? fu.res : x, fu.res ? bytes : 0u);   // no residual: loads give 0
     const float lo = fu.relu ? 0.f : -__builtin_huge_valf();
-    float rv[K];
+    if (!EARLY) {
 #pragma unroll
-    for (int k = 0; k < K; ++k) rv[k] = buf_ld(rr_, off[k], x);
+      for (int k = 0; k < K; ++k) rv[k] = buf_ld(rr_, off[k], x);
+    }
 #pragma unroll
     for (int k = 0; k < K; ++k) buf_st(yr_, off[k], fmaxf((xv[k] - mean) * scale + bt + rv[k], lo), y);
     return;
@@ -948,12 +1124,13 @@ template <typename T, int THREADS, int K, int FUSE = 0>
 __global__ void __launch_bounds__(THREADS)
 bn_bwd_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, const T* __restrict__ dy,
                  T* __restrict__ dx, BnBwdArgs a, BnFuseBwd<T> fu = BnFuseBwd<T>{nullptr, nullptr, nullptr}) {
-  __shared__ float red[THREADS / 64];
+  __shared__ float red[2 * (THREADS / 64)];
   __shared__ float sh[4];
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes),
                                dxr_ = make_rsrc(dx, bytes);
   const long long c = res_feature(g);
-  const float mean = a.save_mean[c];
+  const BnBwdPre pre = bn_preload(a, c);
+  const float mean = pre.mean;
   int off[K];
   res1_offsets<THREADS, K, (int)sizeof(T)>(g, off);
   float xv[K], dv[K];
@@ -974,9 +1151,8 @@ bn_bwd_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, const T* __r
     s1 += dv[k];
     s2 += dv[k] * (xv[k] - mean);
   }
-  s1 = block_sum(s1, red);
-  s2 = block_sum(s2, red);
-  finish_bwd(g, a, c, (double)s1, (double)s2, true, sh);
+  block_sums<(K <= 16)>(s1, s2, red);
+  finish_bwd(g, a, c, (double)s1, (double)s2, true, sh, pre);
   __syncthreads();
   const float kdy = sh[1], kx = sh[2], k0 = sh[3];
 #pragma unroll
@@ -1223,8 +1399,12 @@ template <int THREADS, int K, int FUSE>
 static int launch_train_resident8(const BnGeom& g, const bf16_t* x, bf16_t* y, const BnTrainArgs& a,
                                   const BnFuseFwd<bf16_t>& fu, hipStream_t s) {
   const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * 2);
-  hipLaunchKernelGGL((bn_train_resident8<THREADS, K, FUSE>), dim3((unsigned)g.C), dim3(THREADS), 0, s, g, bytes, x, y,
-                     a, fu);
+  if (FUSE && THREADS == 256 && g.C <= 2 * mfma_num_cus())
+    hipLaunchKernelGGL((bn_train_resident8<THREADS, K, FUSE, (FUSE && THREADS == 256)>), dim3((unsigned)g.C), dim3(THREADS), 0, s, g,
+                       bytes, x, y, a, fu);
+  else
+    hipLaunchKernelGGL((bn_train_resident8<THREADS, K, FUSE>), dim3((unsigned)g.C), dim3(THREADS), 0, s, g, bytes, x, y,
+                       a, fu);
   return check_launch("bn_fwd_train (resident, 8-wide)");
 }
 
@@ -1239,7 +1419,7 @@ static int launch_bwd_resident8(const BnGeom& g, int need, const bf16_t* x, cons
   if (attr != hipSuccess)
     return fail(FLHIP_RUNTIME_ERROR, std::string("bn_bwd: LDS limit: ") + hipGetErrorString(attr));
   const int klim = need < KL ? need : KL;
-  const size_t shmem = (size_t)klim * THREADS * sizeof(uint4);
+  const size_t shmem = (THREADS == 256 || K <= 8) ? 0 : (size_t)klim * THREADS * sizeof(uint4);   // (small features: dy in registers)
   const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * 2);
   hipLaunchKernelGGL(kernel, dim3((unsigned)g.C), dim3(THREADS), shmem, s, g, bytes, klim, x, dy, dx, a, fu);
   return check_launch("bn_bwd (resident, 8-wide)");
@@ -1268,8 +1448,12 @@ template <typename T, int THREADS, int K, int FUSE>
 static int launch_train_resident(const BnGeom& g, const T* x, T* y, const BnTrainArgs& a,
                                  const BnFuseFwd<T>& fu, hipStream_t s) {
   const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
-  hipLaunchKernelGGL((bn_train_resident<T, THREADS, K, FUSE>), dim3((unsigned)g.C), dim3(THREADS), 0, s,
-                     g, bytes, x, y, a, fu);
+  if (FUSE && THREADS == 256 && g.C <= 2 * mfma_num_cus())
+    hipLaunchKernelGGL((bn_train_resident<T, THREADS, K, FUSE, (FUSE && THREADS == 256)>), dim3((unsigned)g.C), dim3(THREADS), 0,
+                       s, g, bytes, x, y, a, fu);
+  else
+    hipLaunchKernelGGL((bn_train_resident<T, THREADS, K, FUSE>), dim3((unsigned)g.C), dim3(THREADS), 0, s,
+                       g, bytes, x, y, a, fu);
   return check_launch("bn_fwd_train (resident)");
 }
 
@@ -1286,7 +1470,7 @@ static int launch_bwd_resident(const BnGeom& g, int need, const T* x, const T* d
     return fail(FLHIP_RUNTIME_ERROR, std::string("bn_bwd: LDS limit: ") + hipGetErrorString(attr));
   // dy vectors per thread parked in LDS: all of them when the feature is small
   const int klim = need < KL ? need : KL;
-  const size_t shmem = (size_t)klim * THREADS * sizeof(float4);
+  const size_t shmem = (THREADS == 256 || K <= 8) ? 0 : (size_t)klim * THREADS * sizeof(float4);   // (small features: dy in registers)
   const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * (long long)sizeof(T));
   hipLaunchKernelGGL(kernel, dim3((unsigned)g.C), dim3(THREADS), shmem, s, g, bytes, klim, x, dy,
                      dx, a, fu);
@@ -1623,3 +1807,9 @@ extern "C" int flhip_bn_act_bwd_mask(const flhip_bn_desc* d, const void* x, cons
   return bn_act_bwd_impl(d, x, dy, nullptr, mask, gamma, save_mean, save_invstd, dx, dresidual, dgamma, dbeta, ws,
                          ws_bytes, stream);
 }
+
+#ifdef BN_STAMPS
+extern "C" int flhip_dbg_bn_stamps(unsigned long long* host) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(flhip::bn_stamps), sizeof(unsigned long long) * 256 * 8);
+}
+#endif

@@ -167,6 +167,28 @@ __device__ __forceinline__ float block_sum(float v, float* smem) {
   return r;
 }
 
+// Two sums at once: the additions of two block_sum calls in the same order, with half the barriers.
+// smem holds 2 * (number of waves) floats.
+__device__ __forceinline__ void block_sum2(float& a, float& b, float* smem) {
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int nw = (blockDim.x + 63) >> 6;
+  a = wave_sum(a);
+  b = wave_sum(b);
+  __syncthreads();
+  if (lane == 0) {
+    smem[wid] = a;
+    smem[nw + wid] = b;
+  }
+  __syncthreads();
+  float ra = 0.f, rb = 0.f;
+  for (int i = 0; i < nw; ++i) {
+    ra += smem[i];
+    rb += smem[nw + i];
+  }
+  a = ra;
+  b = rb;
+}
+
 // ---- elementwise kernels ------------------------------------------------------------
 // out[i] = op(a[i], b[i]) (b may be null for a unary op), four elements per thread through
 // 16-byte (float) / 8-byte (bf16) accesses; launch_elementwise handles tails and pointers
