@@ -57,13 +57,13 @@ __device__ __forceinline__ void fold_partials(const float* __restrict__ ws, long
 
 // the two sums of a kernel together where its registers allow (the kernels that hold 25 vectors per thread
 // have none to spare for the second sum's lanes in flight)
-template <bool TOGETHER>
+template <bool TOGETHER, int NW = 0>
 __device__ __forceinline__ void block_sums(float& a, float& b, float* red) {
   if (TOGETHER) {
-    block_sum2(a, b, red);
+    block_sum2<NW>(a, b, red);
   } else {
-    a = block_sum(a, red);
-    b = block_sum(b, red);
+    a = block_sum<NW>(a, red);
+    b = block_sum<NW>(b, red);
   }
 }
 
@@ -157,7 +157,7 @@ bn_stats_seg(BnGeom g, const T* __restrict__ x, float* __restrict__ ws) {
       }
     }
   });
-  block_sum2(s1, s2, red);
+  block_sum2<4>(s1, s2, red);
   if (threadIdx.x == 0) {
     ws[(c * g.S + blockIdx.y) * 2 + 0] = s1;
     ws[(c * g.S + blockIdx.y) * 2 + 1] = s2;
@@ -339,7 +339,7 @@ bn_bwd_stats_seg(BnGeom g, const T* __restrict__ x, const T* __restrict__ dy,
       }
     }
   });
-  block_sum2(s1, s2, red);
+  block_sum2<4>(s1, s2, red);
   if (threadIdx.x == 0) {
     ws[(c * g.S + blockIdx.y) * 2 + 0] = s1;
     ws[(c * g.S + blockIdx.y) * 2 + 1] = s2;
@@ -590,7 +590,7 @@ bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restri
     asm("" : "+v"(s1), "+v"(s2));
   });
   BN_STAMP(1)
-  block_sums<(K <= 16)>(s1, s2, red);
+  block_sums<(K <= 16), (K <= 16 ? RES_THREADS / 64 : 0)>(s1, s2, red);
   BN_STAMP(2)
   finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh, EARLY ? &pre : nullptr);
   __syncthreads();
@@ -700,7 +700,7 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
     asm("" : "+v"(s1), "+v"(s2));
   });
   BN_STAMP(1)
-  block_sums<(K <= 16)>(s1, s2, red);
+  block_sums<(K <= 16), (K <= 16 ? RES_THREADS / 64 : 0)>(s1, s2, red);
   BN_STAMP(2)
   finish_bwd(g, a, c, (double)s1, (double)s2, true, sh, pre);
   __syncthreads();
@@ -882,6 +882,7 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
   __shared__ float sh[2];
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
   const long long c = res_feature(g);
+  BN_STAMP(0)
   const float shift = ld(x, (size_t)(c * g.inner));
   // (the kernels that hold 25 vectors per thread have no registers to keep the scalars through the statistics)
   constexpr bool EARLY = K <= 16;
@@ -908,9 +909,12 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
     s2 += in ? p2 : 0.f;
     asm("" : "+v"(s1), "+v"(s2));
   });
-  block_sums<(K <= 16)>(s1, s2, red);
+  BN_STAMP(1)
+  block_sums<(K <= 16), (K <= 16 ? RES_THREADS / 64 : 0)>(s1, s2, red);
+  BN_STAMP(2)
   finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh, EARLY ? &pre : nullptr);
   __syncthreads();
+  BN_STAMP(3)
   if (!EARLY) pre = bn_preload(a, c, false);
   const float mean = uniform(sh[0]);
   const float scale = uniform(pre.gamma * sh[1]);
@@ -949,6 +953,11 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
     }
     buf_st8(yr_, off, v);
   });
+  BN_STAMP(4)
+#ifdef BN_STAMPS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  BN_STAMP(5)
+#endif
 }
 
 template <int RES_THREADS, int K, int FUSE = 0>
@@ -964,6 +973,7 @@ bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ 
   const __amdgpu_buffer_rsrc_t mr_ = mask_rsrc(FUSE == 2 ? fu.mask : nullptr, x, bytes, 2);
   const __amdgpu_buffer_rsrc_t drr_ = make_rsrc((FUSE && fu.dres) ? fu.dres : dx, (FUSE && fu.dres) ? bytes : 0u);
   const long long c = res_feature(g);
+  BN_STAMP(0)
   const BnBwdPre pre = bn_preload(a, c);
   const float mean = pre.mean;
   uint4 xr[K];
@@ -1011,9 +1021,12 @@ bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ 
     s2 += in ? p2 : 0.f;
     asm("" : "+v"(s1), "+v"(s2));
   });
-  block_sums<(K <= 16)>(s1, s2, red);
+  BN_STAMP(1)
+  block_sums<(K <= 16), (K <= 16 ? RES_THREADS / 64 : 0)>(s1, s2, red);
+  BN_STAMP(2)
   finish_bwd(g, a, c, (double)s1, (double)s2, true, sh, pre);
   __syncthreads();
+  BN_STAMP(3)
   const float kdy = sh[1], kx = sh[2], k0 = sh[3];
   res_visit<RES_THREADS, K, 2, FB, true, 8>(g, [&](int k, int off, bool) {
     if (REGS) opaque(dr[REGS ? k : 0]);
@@ -1032,6 +1045,11 @@ bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ 
     buf_st8(dxr_, off, make_uint4(o[0], o[1], o[2], o[3]));
     if (FUSE) buf_st8(drr_, off, d);               // no residual branch: the empty range drops the store
   });
+  BN_STAMP(4)
+#ifdef BN_STAMPS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  BN_STAMP(5)
+#endif
 }
 
 // ---- resident kernels for rows that are not 16-byte friendly (inner % 4 != 0) -----------
@@ -1099,7 +1117,7 @@ bn_train_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restr
     s1 += t;
     s2 += t * t;
   }
-  block_sums<(K <= 16)>(s1, s2, red);
+  block_sums<(K <= 16), (K <= 16 ? THREADS / 64 : 0)>(s1, s2, red);
   finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh, EARLY ? &pre : nullptr);
   __syncthreads();
   if (!EARLY) pre = bn_preload(a, c, false);
@@ -1151,7 +1169,7 @@ bn_bwd_resident1(BnGeom g, unsigned bytes, const T* __restrict__ x, const T* __r
     s1 += dv[k];
     s2 += dv[k] * (xv[k] - mean);
   }
-  block_sums<(K <= 16)>(s1, s2, red);
+  block_sums<(K <= 16), (K <= 16 ? THREADS / 64 : 0)>(s1, s2, red);
   finish_bwd(g, a, c, (double)s1, (double)s2, true, sh, pre);
   __syncthreads();
   const float kdy = sh[1], kx = sh[2], k0 = sh[3];

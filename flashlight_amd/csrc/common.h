@@ -155,23 +155,28 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // Sum of `v` over the block; result valid in every thread.  `smem` holds at
 // least blockDim.x/64 floats and may be reused after the call returns.
+// (NW: the number of waves when the caller knows it at compile time - the loop over the waves' sums is then
+// unrolled and its LDS reads go out together; 0: taken from blockDim)
+template <int NW = 0>
 __device__ __forceinline__ float block_sum(float v, float* smem) {
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
-  const int nw = (blockDim.x + 63) >> 6;
+  const int nw = NW ? NW : (int)((blockDim.x + 63) >> 6);
   v = wave_sum(v);
   __syncthreads();
   if (lane == 0) smem[wid] = v;
   __syncthreads();
   float r = 0.f;
+#pragma unroll
   for (int i = 0; i < nw; ++i) r += smem[i];
   return r;
 }
 
 // Two sums at once: the additions of two block_sum calls in the same order, with half the barriers.
 // smem holds 2 * (number of waves) floats.
+template <int NW = 0>
 __device__ __forceinline__ void block_sum2(float& a, float& b, float* smem) {
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
-  const int nw = (blockDim.x + 63) >> 6;
+  const int nw = NW ? NW : (int)((blockDim.x + 63) >> 6);
   a = wave_sum(a);
   b = wave_sum(b);
   __syncthreads();
@@ -181,6 +186,7 @@ __device__ __forceinline__ void block_sum2(float& a, float& b, float* smem) {
   }
   __syncthreads();
   float ra = 0.f, rb = 0.f;
+#pragma unroll
   for (int i = 0; i < nw; ++i) {
     ra += smem[i];
     rb += smem[nw + i];
