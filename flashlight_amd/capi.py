@@ -48,6 +48,8 @@ SYMBOLS = {
     "flhip_conv2d_bwd_data_add": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
     "flhip_conv2d_bwd_filter": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
     "flhip_conv2d_bwd_filter_static": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _VP]),
+    "flhip_conv2d_gathered_bytes": (_SZ, [C.POINTER(ConvDesc)]),
+    "flhip_conv2d_bwd_filter_gathered": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _VP, _SZ, _VP]),
     "flhip_pool2d_fwd": (C.c_int, [C.POINTER(PoolDesc), _VP, _VP, _VP, _VP]),
     "flhip_pool2d_bwd": (C.c_int, [C.POINTER(PoolDesc), _VP, _VP, _VP, _VP]),
     "flhip_bn_workspace_bytes": (_SZ, [C.POINTER(BnDesc)]),

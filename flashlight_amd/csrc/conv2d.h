@@ -52,7 +52,9 @@ int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void
 size_t mfma_pointwise16_lattice_ws(const ConvGeom& g, bool bwd);
 size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g);
 int mfma_pointwise16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
-                           size_t ws_bytes, hipStream_t s);
+                           size_t ws_bytes, hipStream_t s, const void* gathered = nullptr);
+// bytes of gathered input that the forward pass leaves at the start of its workspace for the filter gradient (0: none)
+size_t mfma_pointwise16_gathered_bytes(const ConvGeom& g);
 // fp32, stride 1, few tiles and a long contraction: the contraction in slices through
 // mfma_pointwise_split_ws() bytes of workspace; -1 when it does not apply or the room is missing
 size_t mfma_pointwise_split_ws(const ConvGeom& g, int dtype, bool bwd);

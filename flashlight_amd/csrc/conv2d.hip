@@ -367,6 +367,34 @@ extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, 
   return check_launch("conv2d_bwd_filter");
 }
 
+// The forward pass of a strided layer in bf16 storage gathers the input points its windows touch into the start of
+// its workspace; the filter gradient needs the same copy.  A caller that keeps those bytes passes them here and
+// saves the second gather.
+static bool gathered_path(const flhip_conv_desc* d) {
+  return d->dtype == FLHIP_BF16 && !force_direct() && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT);
+}
+
+extern "C" size_t flhip_conv2d_gathered_bytes(const flhip_conv_desc* d) {
+  ConvGeom g;
+  if (!d || make_geom(d, &g) != FLHIP_OK || !gathered_path(d)) return 0;
+  return mfma_pointwise16_gathered_bytes(g);
+}
+
+extern "C" int flhip_conv2d_bwd_filter_gathered(const flhip_conv_desc* d, const void* gathered, const void* dy,
+                                                float* dw, float* db, void* ws, size_t ws_bytes, void* stream) {
+  FLHIP_REQUIRE(d && gathered && dy && dw, "conv2d_bwd_filter_gathered: null argument");
+  ConvGeom g;
+  const int rc = make_geom(d, &g);
+  if (rc != FLHIP_OK) return rc;
+  FLHIP_REQUIRE(gathered_path(d) && mfma_pointwise16_gathered_bytes(g) > 0,
+                "conv2d_bwd_filter_gathered: this geometry's forward pass leaves no gathered input");
+  const size_t need = flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER);
+  FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter_gathered: workspace too small");
+  const int r = mfma_pointwise16_wgrad(g, nullptr, dy, dw, db, ws, ws_bytes, as_stream(stream), gathered);
+  if (r < 0) return fail(FLHIP_INVALID_ARGUMENT, "conv2d_bwd_filter_gathered: no kernel takes the gathered input of this geometry");
+  return r;
+}
+
 extern "C" int flhip_conv2d_bwd_filter_static(const flhip_conv_desc* d, const void* x, const void* dy,
                                               float* dw, float* db, void* stream) {
   FLHIP_REQUIRE(d, "conv2d_bwd_filter_static: null argument");

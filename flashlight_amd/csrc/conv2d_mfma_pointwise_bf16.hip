@@ -1011,6 +1011,20 @@ size_t mfma_pointwise16_lattice_ws(const ConvGeom& g, bool bwd) {
   return 0;
 }
 
+// Bytes of the gathered input that the forward pass of this geometry leaves at the start of its workspace and
+// that the filter gradient would otherwise gather again (the same kernel, the same layout); 0 when the forward
+// pass does not gather.
+size_t mfma_pointwise16_gathered_bytes(const ConvGeom& g) {
+  ConvGeom c;
+  Pw16WgradParams p{};
+  if (pw16_strided_plan(g, &c)) return pw16_wgrad_plan(c, &p) ? lattice_bytes(c) : 0;
+  if (!options().pw16_no_taps && pw16_taps_plan(g, &c) && pw16_taps_forward(g, c)) {
+    ConvGeom cw;
+    if (pw16_taps_plan(g, &cw, true) && pw16_wgrad_plan(cw, &p) && lattice_bytes(cw) == lattice_bytes(c)) return lattice_bytes(c);
+  }
+  return 0;
+}
+
 // the compact 1x1 problem of a strided layer: on the kernels that load straight to LDS where those
 // are ahead, else on the ones above
 template <bool BWD>
@@ -1083,8 +1097,10 @@ size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g0) {
   return lattice + need;
 }
 
+// (gathered: the gathered input a forward pass left behind - mfma_pointwise16_gathered_bytes() of it -, taken in
+// place of x; -1 when this geometry has none)
 int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, float* dw, float* db, void* ws,
-                           size_t ws_bytes, hipStream_t s) {
+                           size_t ws_bytes, hipStream_t s, const void* gathered) {
   if (!dw) return -1;
   ConvGeom g = g0;
   const bool strided = pw16_strided_plan(g0, &g);
@@ -1092,7 +1108,10 @@ int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, fl
   if (!strided && !taps) g = g0;
   Pw16WgradParams p{};
   if (!pw16_wgrad_plan(g, &p)) return -1;
-  if (strided || taps) {
+  if (gathered) {
+    if (!(strided || taps) || mfma_pointwise16_gathered_bytes(g0) == 0) return -1;
+    x = gathered;
+  } else if (strided || taps) {
     // the gathered input first, the slices of the gradient behind it
     const size_t lb = lattice_bytes(g);
     if (!ws || ws_bytes < lb) return fail(FLHIP_INVALID_ARGUMENT, "conv2d_bwd_filter: workspace too small");

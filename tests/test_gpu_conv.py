@@ -435,6 +435,56 @@ def test_bf16_strided_windows_without_workspace(shape):
     assert rel_l2(host(y0), host(y)) <= 1e-2 and rel_l2(host(dx0), host(dx)) <= 1e-2
 
 
+@pytest.mark.parametrize("shape", [((4, 256, 56, 56), (512, 256, 1, 1), (2, 2), (0, 0)),      # ResNet-50 downsample shortcuts
+                                   ((4, 512, 28, 28), (1024, 512, 1, 1), (2, 2), (0, 0)),
+                                   ((3, 64, 14, 14), (96, 64, 1, 1), (2, 2), (0, 0)),
+                                   ((4, 128, 56, 56), (128, 128, 3, 3), (2, 2), (1, 1)),      # its strided 3x3 layers
+                                   ((4, 256, 28, 28), (256, 256, 3, 3), (2, 2), (1, 1)),
+                                   ((8, 512, 14, 14), (512, 512, 3, 3), (2, 2), (1, 1)),
+                                   ((2, 128, 28, 28), (128, 128, 3, 3), (1, 1), (1, 1))])     # stride 1: nothing gathered
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_bf16_filter_gradient_from_the_forward_pass_gather(shape, with_bias):
+    """The payload of the conv2d closure: the forward pass of a strided bf16 layer leaves the gathered input in
+    its workspace, and the filter gradient computed from it equals the one that gathers again, bit for bit (and
+    the oracle's within bf16 products summed in fp32).  Geometries that gather nothing say so and refuse."""
+    import ctypes as C
+    from flashlight_amd import capi
+    xs, ws_, st, pd = shape
+    rng = np.random.default_rng(91)
+    x = dev(bf16_round(rng.standard_normal(xs).astype(np.float32))).to(torch.bfloat16)
+    w = dev(bf16_round((rng.standard_normal(ws_) / 20).astype(np.float32))).to(torch.bfloat16)
+    kw = dict(sx=st[1], sy=st[0], px=pd[1], py=pd[0], dx=1, dy=1, groups=1)
+    y, gathered = fa.conv2d(x, w, None, keep_gathered=True, **kw)
+    assert torch.equal(y, fa.conv2d(x, w, None, **kw))
+    dy = dev(bf16_round(rng.standard_normal(tuple(y.shape)).astype(np.float32))).to(torch.bfloat16)
+    dw0, db0 = fa.conv2d_backward_filter_bias(dy, x, ws_, with_bias, **kw)
+    L = capi.lib()
+    cd = capi.ConvDesc(xs[0], xs[1], xs[2], xs[3], ws_[0], ws_[2], ws_[3], st[0], st[1], pd[0], pd[1], 1, 1, 1,
+                       capi.BF16)
+    if st == (1, 1):
+        assert gathered is None and L.flhip_conv2d_gathered_bytes(C.byref(cd)) == 0
+        S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        P = lambda t: C.c_void_p(t.data_ptr())
+        nws = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_BWD_FILTER)
+        wsb = torch.empty(max(nws, 16), dtype=torch.uint8, device="cuda")
+        assert L.flhip_conv2d_bwd_filter_gathered(C.byref(cd), P(x), P(dy), P(dw0), None, P(wsb), nws, S) == capi.INVALID_ARGUMENT
+        return
+    taps = ws_[2] * ws_[3]
+    compact = xs[0] * xs[1] * taps * y.shape[2] * y.shape[3] * 2      # (the library may round it up)
+    assert gathered is not None and compact <= gathered.numel() < compact + 4096
+    kept = gathered.clone()      # the closure keeps it while other layers use the workspace
+    dw1, db1 = fa.conv2d_backward_filter_bias(dy, x, ws_, with_bias, gathered=kept, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(dw1, dw0)
+    if with_bias:
+        assert torch.equal(db1, db0)
+    d = flref.conv_desc(xs, ws_, st, pd, (1, 1), 1)
+    ref_dw, ref_db = flref.conv2d_bwd_filter(d, host(x).astype(np.float32), host(dy).astype(np.float32), want_bias=with_bias)
+    assert rel_l2(host(dw1), ref_dw) <= 2e-3          # bf16 products, fp32 sums, another order
+    if with_bias:
+        assert rel_l2(host(db1), ref_db) <= 2e-3
+
+
 def _random_cases(n, seed):
     """Seeded random geometries biased towards the conditions the kernel families key on:
     1x1 and 3x3 windows, even / odd rows, planes of 4k positions, channel counts around the
