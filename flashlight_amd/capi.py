@@ -38,6 +38,7 @@ _VP, _SZ, _I32P = C.c_void_p, C.c_size_t, C.POINTER(C.c_int32)
 SYMBOLS = {
     "flhip_last_error": (C.c_char_p, []),
     "flhip_version": (C.c_int, []),
+    "flhip_convert_many_launches": (C.c_int, [C.POINTER(C.c_size_t), C.c_int, _I32P]),
     "flhip_arch": (C.c_char_p, []),
     "flhip_set_option": (C.c_int, [C.c_char_p, C.c_char_p]),
     "flhip_conv2d_out_dims": (C.c_int, [C.POINTER(ConvDesc), _I32P, _I32P]),

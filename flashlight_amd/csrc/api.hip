@@ -60,15 +60,7 @@ static bool apply_option(Options& o, const char* name, const char* v) {
     if (!v || !*v || !strcmp(v, "auto")) o.bn_algo = 0;
     else if (!strcmp(v, "split")) o.bn_algo = 1;
     else if (!strcmp(v, "resident")) o.bn_algo = 2;
-    else if (!strcmp(v, "pair")) o.bn_algo = 3;
-    else if (!strcmp(v, "pairalone")) o.bn_algo = 4;
     else return false;
-    return true;
-  }
-  if (!strcmp(name, "CONV_ROWS")) {
-    const int n = v ? atoi(v) : 0;
-    if (n < 0 || n > 64) return false;
-    o.conv_rows = n;
     return true;
   }
   if (!strcmp(name, "CONV_STACK")) {
@@ -85,7 +77,7 @@ static bool apply_option(Options& o, const char* name, const char* v) {
 }
 
 static void options_from_environment() {
-  static const char* const names[] = {"CONV_ALGO", "CONV_SKIP", "PW_PT", "PW16_PF", "CONV_ROWS", "CONV_STACK", "BN_ALGO", "PW16_NO_TAPS",
+  static const char* const names[] = {"CONV_ALGO", "CONV_SKIP", "PW_PT", "PW16_PF", "CONV_STACK", "BN_ALGO", "PW16_NO_TAPS",
                                       "TAPPED_NO_REORDER", "MATMUL_VALU", "RNN_UNFUSED"};
   for (const char* n : names) {
     const std::string var = std::string("FLHIP_") + n;
@@ -165,8 +157,11 @@ struct OpAdd {
 
 using namespace flhip;
 
+// most pieces (workgroups) of one convert_many launch: the grid limit
+static uint64_t convert_many_max_pieces() { return 0x7fffffffull; }
+
 extern "C" const char* flhip_last_error(void) { return g_last_error.c_str(); }
-extern "C" int flhip_version(void) { return 100; }
+extern "C" int flhip_version(void) { return FLHIP_VERSION; }
 extern "C" const char* flhip_arch(void) { return "gfx950"; }
 
 extern "C" int flhip_set_option(const char* name, const char* value) {
@@ -252,23 +247,14 @@ extern "C" int flhip_convert_many(const void* const* src, void* const* dst, cons
   FLHIP_REQUIRE(dtype_ok(src_dtype) && dtype_ok(dst_dtype), "convert_many: unknown dtype");
   FLHIP_REQUIRE(count >= 0 && (count == 0 || (src && dst && n)), "convert_many: null argument");
   hipStream_t s = as_stream(stream);
-  for (int i0 = 0; i0 < count; i0 += CM_MAX) {
-    ConvertMany a{};
-    unsigned pieces = 0;
-    for (int i = i0; i < count && i < i0 + CM_MAX; ++i) {
-      if (n[i] == 0) continue;
-      FLHIP_REQUIRE(src[i] && dst[i], "convert_many: null pointer");
-      FLHIP_REQUIRE(n[i] < (1ull << 40), "convert_many: tensor too large");
-      a.src[a.count] = src[i];
-      a.dst[a.count] = dst[i];
-      a.n[a.count] = n[i];
-      a.first[a.count] = pieces;
-      pieces += (unsigned)((n[i] + 2047) / 2048);
-      ++a.count;
-    }
-    if (a.count == 0) continue;
-    a.first[a.count] = pieces;
-    const dim3 grid(pieces), block(256);
+  // A launch holds up to CM_MAX tensors and at most 2^31 - 1 pieces of 2048 elements (the grid limit; one
+  // tensor is at most 2^29 pieces): a tensor that would pass either limit starts the next launch.
+  ConvertMany a{};
+  uint64_t pieces = 0;
+  auto flush = [&]() {
+    if (a.count == 0) return;
+    a.first[a.count] = (unsigned)pieces;
+    const dim3 grid((unsigned)pieces), block(256);
     if (src_dtype == FLHIP_F32 && dst_dtype == FLHIP_F32)
       hipLaunchKernelGGL((convert_many_kernel<float, float>), grid, block, 0, s, a);
     else if (src_dtype == FLHIP_F32)
@@ -277,8 +263,45 @@ extern "C" int flhip_convert_many(const void* const* src, void* const* dst, cons
       hipLaunchKernelGGL((convert_many_kernel<bf16_t, float>), grid, block, 0, s, a);
     else
       hipLaunchKernelGGL((convert_many_kernel<bf16_t, bf16_t>), grid, block, 0, s, a);
+    a = ConvertMany{};
+    pieces = 0;
+  };
+  for (int i = 0; i < count; ++i) {
+    if (n[i] == 0) continue;
+    FLHIP_REQUIRE(src[i] && dst[i], "convert_many: null pointer");
+    FLHIP_REQUIRE(n[i] < (1ull << 40), "convert_many: tensor too large");
+    const uint64_t mine = (n[i] + 2047) / 2048;
+    if (a.count == CM_MAX || pieces + mine > convert_many_max_pieces()) flush();
+    a.src[a.count] = src[i];
+    a.dst[a.count] = dst[i];
+    a.n[a.count] = n[i];
+    a.first[a.count] = (unsigned)pieces;
+    pieces += mine;
+    ++a.count;
   }
+  flush();
   return check_launch("convert_many");
+}
+
+extern "C" int flhip_convert_many_launches(const size_t* n, int count, int* launch_of) {
+  if (count < 0 || (count > 0 && !n)) return -1;
+  int launches = 0, held = 0;
+  uint64_t pieces = 0;
+  for (int i = 0; i < count; ++i) {
+    if (launch_of) launch_of[i] = -1;
+    if (n[i] == 0) continue;
+    if (n[i] >= (1ull << 40)) return -1;
+    const uint64_t mine = (n[i] + 2047) / 2048;
+    if (held == CM_MAX || pieces + mine > convert_many_max_pieces()) {
+      launches += held > 0;
+      held = 0;
+      pieces = 0;
+    }
+    if (launch_of) launch_of[i] = launches;
+    pieces += mine;
+    ++held;
+  }
+  return launches + (held > 0);
 }
 
 extern "C" int flhip_fill(void* dst, double value, size_t n, int dtype, void* stream) {

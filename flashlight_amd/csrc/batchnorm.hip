@@ -10,8 +10,6 @@
 // inner == 1 ("column" kernels, per-activation mode): features are contiguous, a
 // wave covers 64 features and rows are strided by C.
 #include <stdlib.h>
-#include <atomic>
-#include <chrono>
 #include <string.h>
 
 #include "common.h"
@@ -19,14 +17,6 @@
 namespace flhip {
 
 int mfma_num_cus();   // compute units of the current device (defined with the convolution kernels)
-
-// Time stamps of the phases of a workgroup, for builds with -DBN_STAMPS only (timing studies).
-#ifdef BN_STAMPS
-__device__ unsigned long long bn_stamps[256 * 8];
-#define BN_STAMP(i) { if (threadIdx.x == 0 && blockIdx.x < 256) bn_stamps[blockIdx.x * 8 + (i)] = wall_clock64(); }
-#else
-#define BN_STAMP(i) {}
-#endif
 
 struct BnGeom {
   long long outer, C, inner;
@@ -562,7 +552,6 @@ bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restri
   constexpr int ESZ = (int)sizeof(T);
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
   const long long c = res_feature(g);
-  BN_STAMP(0)
   const float shift = ld(x, (size_t)(c * g.inner));
   // (the kernels that hold 25 vectors per thread have no registers to keep the scalars through the statistics)
   constexpr bool EARLY = K <= 16;
@@ -589,12 +578,9 @@ bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restri
     // first block reduction and drags every vector's temporaries along
     asm("" : "+v"(s1), "+v"(s2));
   });
-  BN_STAMP(1)
   block_sums<(K <= 16), (K <= 16 ? RES_THREADS / 64 : 0)>(s1, s2, red);
-  BN_STAMP(2)
   finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh, EARLY ? &pre : nullptr);
   __syncthreads();
-  BN_STAMP(3)
   if (!EARLY) pre = bn_preload(a, c, false);
   const float mean = sh[0];
   const float scale = pre.gamma * sh[1];
@@ -613,11 +599,6 @@ bn_train_resident(BnGeom g, unsigned bytes, const T* __restrict__ x, T* __restri
         __builtin_amdgcn_raw_buffer_store_b8((uint8_t)bits, mr_, mask_off(off, ESZ), 0, 0);
       }
     });
-    BN_STAMP(4)
-#ifdef BN_STAMPS
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    BN_STAMP(5)
-#endif
     return;
   }
   res_visit<RES_THREADS, K, ESZ, 1>(g, [&](int k, int off, bool) {
@@ -645,7 +626,6 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes),
                                dxr_ = make_rsrc(dx, bytes);
   const long long c = res_feature(g);
-  BN_STAMP(0)
   const BnBwdPre pre = bn_preload(a, c);
   const float mean = pre.mean;
   float4 xr[K];
@@ -699,12 +679,9 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
     // first block reduction and drags every vector's temporaries along
     asm("" : "+v"(s1), "+v"(s2));
   });
-  BN_STAMP(1)
   block_sums<(K <= 16), (K <= 16 ? RES_THREADS / 64 : 0)>(s1, s2, red);
-  BN_STAMP(2)
   finish_bwd(g, a, c, (double)s1, (double)s2, true, sh, pre);
   __syncthreads();
-  BN_STAMP(3)
   const float kdy = sh[1], kx = sh[2], k0 = sh[3];
   res_visit<RES_THREADS, K, ESZ, FB, true>(g, [&](int k, int off, bool) {
     float4 d = REGS ? masked(k) : k < klim ? dyl[k * RES_THREADS + threadIdx.x] : buf_ld4(dyr_, off, dy);
@@ -720,107 +697,6 @@ bn_bwd_resident(BnGeom g, unsigned bytes, int klim, const T* __restrict__ x, con
     buf_st4(dxr_, off, v, dx);
     if (FUSE && fu.dres) buf_st4(make_rsrc(fu.dres, bytes), off, d, dx);
   });
-  BN_STAMP(4)
-#ifdef BN_STAMPS
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  BN_STAMP(5)
-#endif
-}
-
-// ---- backward, a feature shared by two workgroups (fp32, features of 10 to 26 vectors per thread) ---------
-// The kernel above parks 9 of a thread's dy vectors in LDS and reads the others twice.  Here two workgroups own a
-// feature, half of its vectors each: a thread keeps its K2 vectors of x in registers and ALL its K2 vectors of dy
-// on chip (K2 - KR in LDS, KR in registers), so every tensor crosses the memory interface once (3T).  The two
-// need each other's sums.  Each publishes its own as two 64-bit words (value, launch number) with relaxed atomic
-// stores - a word is valid by itself, so no fence is needed - and polls the other's for a BOUNDED time; a workgroup
-// whose partner does not answer in time (it may not be running yet, and nothing guarantees that it ever runs
-// alongside) sums the partner's half itself from memory, with the same instructions in the same order, so the
-// result does not depend on who computed what.  No wait in this kernel is unbounded.
-// Workgroups b and b ^ 8 are partners: consecutive workgroups go to the 8 XCDs in turn, so partners share an L2.
-__device__ __forceinline__ void bn_pair_partial(const float4& d, const float4& xv, float mean, float* p1, float* p2) {
-  *p1 = (d.x + d.y) + (d.z + d.w);
-  *p2 = __fmaf_rn(d.w, xv.w - mean, __fmaf_rn(d.z, xv.z - mean, __fmaf_rn(d.y, xv.y - mean, d.x * (xv.x - mean))));
-}
-
-template <int K2, int KR>
-__global__ void __launch_bounds__(1024)
-bn_bwd_pair(BnGeom g, unsigned bytes, const float* __restrict__ x, const float* __restrict__ dy,
-            float* __restrict__ dx, BnBwdArgs a, unsigned long long* xch, unsigned epoch, unsigned spin_ticks) {
-  constexpr int T = 1024, KL = K2 - KR;
-  extern __shared__ float4 dyl[];           // [KL][T]
-  __shared__ float red[2 * (T / 64)];
-  __shared__ float sh[4];
-  __shared__ float theirs[3];               // the partner's sums, and whether they arrived
-  const int tid = threadIdx.x;
-  const int b = blockIdx.x, r16 = b & 15, half = r16 >> 3, fs = (b >> 4) * 8 + (r16 & 7);
-  const int C = (int)g.C;
-  const int c = (fs & 7) * (C >> 3) + (fs >> 3);      // neighbouring features on one XCD, as res_feature
-  const int q0 = half * K2 * T, q0_theirs = (half ^ 1) * K2 * T;
-  const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), dyr_ = make_rsrc(dy, bytes), dxr_ = make_rsrc(dx, bytes);
-  const BnBwdPre pre = bn_preload(a, c);
-  const float mean = pre.mean;
-  float4 xr[K2], dr[KR > 0 ? KR : 1];
-  float s1 = 0.f, s2 = 0.f;
-  res_visit<T, K2, 4, 0>(g, [&](int k, int off, bool) { xr[k] = buf_ld4_stream(xr_, off, x); }, q0, c);
-  res_visit<T, K2, 4, 4>(g, [&](int k, int off, bool in) {
-    const float4 d = buf_ld4_stream(dyr_, off, dy);
-    if (k < KL) dyl[k * T + tid] = d;
-    else dr[k - KL < 0 ? 0 : k - KL] = d;
-    float p1, p2;
-    bn_pair_partial(d, xr[k], mean, &p1, &p2);
-    s1 += in ? p1 : 0.f;
-    s2 += in ? p2 : 0.f;
-    asm("" : "+v"(s1), "+v"(s2));
-  }, q0, c);
-  s1 = block_sum(s1, red);
-  s2 = block_sum(s2, red);
-  unsigned long long* mine = xch + ((size_t)c * 2 + half) * 2;
-  unsigned long long* other = xch + ((size_t)c * 2 + (half ^ 1)) * 2;
-  if (tid == 0) {
-    __hip_atomic_store(mine + 0, ((unsigned long long)__float_as_uint(s1) << 32) | epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(mine + 1, ((unsigned long long)__float_as_uint(s2) << 32) | epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    bool got = false;
-    unsigned long long w0 = 0, w1 = 0;
-    if (spin_ticks != 0) {
-      const unsigned long long t0 = wall_clock64();
-      do {
-        w0 = __hip_atomic_load(other + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        w1 = __hip_atomic_load(other + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        got = (unsigned)w0 == epoch && (unsigned)w1 == epoch;
-        if (!got) __builtin_amdgcn_s_sleep(4);
-      } while (!got && wall_clock64() - t0 < spin_ticks);
-    }
-    theirs[0] = __uint_as_float((unsigned)(w0 >> 32));
-    theirs[1] = __uint_as_float((unsigned)(w1 >> 32));
-    theirs[2] = got ? 1.f : 0.f;
-  }
-  __syncthreads();
-  float o1 = theirs[0], o2 = theirs[1];
-  if (theirs[2] == 0.f) {
-    // the partner did not answer: its half, summed here the way it sums it
-    float t1 = 0.f, t2 = 0.f;
-    res_visit<T, K2, 4, 4>(g, [&](int, int off, bool in) {
-      const float4 xv = buf_ld4(xr_, off, x), d = buf_ld4(dyr_, off, dy);
-      float p1, p2;
-      bn_pair_partial(d, xv, mean, &p1, &p2);
-      t1 += in ? p1 : 0.f;
-      t2 += in ? p2 : 0.f;
-      asm("" : "+v"(t1), "+v"(t2));
-    }, q0_theirs, c);
-    o1 = block_sum(t1, red);
-    o2 = block_sum(t2, red);
-  }
-  // the first half's sums first, in both workgroups
-  const float S1 = half == 0 ? s1 + o1 : o1 + s1, S2 = half == 0 ? s2 + o2 : o2 + s2;
-  finish_bwd(g, a, c, (double)S1, (double)S2, half == 0, sh, pre);
-  __syncthreads();
-  const float kdy = sh[1], kx = sh[2], k0 = sh[3];
-  res_visit<T, K2, 4, 4, true>(g, [&](int k, int off, bool) {
-    const float4 d = k < KL ? dyl[k * T + tid] : dr[k - KL < 0 ? 0 : k - KL];
-    const float4 v = make_float4(kdy * d.x + (kx * (xr[k].x - mean) + k0), kdy * d.y + (kx * (xr[k].y - mean) + k0),
-                                 kdy * d.z + (kx * (xr[k].z - mean) + k0), kdy * d.w + (kx * (xr[k].w - mean) + k0));
-    buf_st4(dxr_, off, v, dx);
-  }, q0, c);
 }
 
 // ---- resident kernels for bf16 storage, eight elements (16 bytes) per slot ----------------
@@ -882,7 +758,6 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
   __shared__ float sh[2];
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
   const long long c = res_feature(g);
-  BN_STAMP(0)
   const float shift = ld(x, (size_t)(c * g.inner));
   // (the kernels that hold 25 vectors per thread have no registers to keep the scalars through the statistics)
   constexpr bool EARLY = K <= 16;
@@ -909,12 +784,9 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
     s2 += in ? p2 : 0.f;
     asm("" : "+v"(s1), "+v"(s2));
   });
-  BN_STAMP(1)
   block_sums<(K <= 16), (K <= 16 ? RES_THREADS / 64 : 0)>(s1, s2, red);
-  BN_STAMP(2)
   finish_stats(g, a, c, shift, (double)s1, (double)s2, true, sh, EARLY ? &pre : nullptr);
   __syncthreads();
-  BN_STAMP(3)
   if (!EARLY) pre = bn_preload(a, c, false);
   const float mean = uniform(sh[0]);
   const float scale = uniform(pre.gamma * sh[1]);
@@ -953,11 +825,6 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
     }
     buf_st8(yr_, off, v);
   });
-  BN_STAMP(4)
-#ifdef BN_STAMPS
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  BN_STAMP(5)
-#endif
 }
 
 template <int RES_THREADS, int K, int FUSE = 0>
@@ -973,7 +840,6 @@ bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ 
   const __amdgpu_buffer_rsrc_t mr_ = mask_rsrc(FUSE == 2 ? fu.mask : nullptr, x, bytes, 2);
   const __amdgpu_buffer_rsrc_t drr_ = make_rsrc((FUSE && fu.dres) ? fu.dres : dx, (FUSE && fu.dres) ? bytes : 0u);
   const long long c = res_feature(g);
-  BN_STAMP(0)
   const BnBwdPre pre = bn_preload(a, c);
   const float mean = pre.mean;
   uint4 xr[K];
@@ -1021,12 +887,9 @@ bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ 
     s2 += in ? p2 : 0.f;
     asm("" : "+v"(s1), "+v"(s2));
   });
-  BN_STAMP(1)
   block_sums<(K <= 16), (K <= 16 ? RES_THREADS / 64 : 0)>(s1, s2, red);
-  BN_STAMP(2)
   finish_bwd(g, a, c, (double)s1, (double)s2, true, sh, pre);
   __syncthreads();
-  BN_STAMP(3)
   const float kdy = sh[1], kx = sh[2], k0 = sh[3];
   res_visit<RES_THREADS, K, 2, FB, true, 8>(g, [&](int k, int off, bool) {
     if (REGS) opaque(dr[REGS ? k : 0]);
@@ -1045,11 +908,6 @@ bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ 
     buf_st8(dxr_, off, make_uint4(o[0], o[1], o[2], o[3]));
     if (FUSE) buf_st8(drr_, off, d);               // no residual branch: the empty range drops the store
   });
-  BN_STAMP(4)
-#ifdef BN_STAMPS
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  BN_STAMP(5)
-#endif
 }
 
 // ---- resident kernels for rows that are not 16-byte friendly (inner % 4 != 0) -----------
@@ -1553,46 +1411,6 @@ static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws
   return check_launch("bn_fwd_train");
 }
 
-// The kernel that shares a feature between two workgroups: fp32, rows of a multiple of 4 elements, features of 10
-// to 26 vectors per thread (fewer are parked in LDS whole by the one-workgroup kernel), a multiple of 8 features.
-// Selected with BN_ALGO=pair; =pairalone makes every workgroup sum its partner's half itself (the path taken when
-// the partner does not answer; tests).
-// Returns -1 when it does not apply.
-static int try_bwd_pair(const BnGeom& g, int vec, const float* x, const float* dy, float* dx, float* ws,
-                        const BnBwdArgs& a, hipStream_t s) {
-  const int mode = options().bn_algo;
-  // Only on request: measured at 56x56x256x32 it is slower than the one-workgroup kernel (57.3 against 52.8 us; it
-  // moves 3T instead of 3.45T, but 512 workgroups of 1024 threads are two rounds at one per CU, each with its own
-  // start-up, exchange and tail, and 3T in 57 us is the rate of the plain two-reads-one-write streaming kernel).
-  if ((mode != 3 && mode != 4) || vec != 4) return -1;
-  if (g.C % 8 != 0) return -1;
-  if (g.units <= (long long)RES_KL * 1024 || g.units > 26ll * 1024) return -1;
-  if (g.outer * g.C * g.inner * 4 >= (1ll << 31) || reinterpret_cast<uintptr_t>(ws) % 8 != 0) return -1;
-  // launch number: tells this launch's words in the exchange area from whatever the memory held before
-  static std::atomic<unsigned> launches{
-      (unsigned)std::chrono::steady_clock::now().time_since_epoch().count() * 2654435761u};
-  unsigned epoch = ++launches;
-  if (epoch == 0) epoch = ++launches;
-  const unsigned spin = mode == 4 ? 0u : 50000u;     // ticks of the 100 MHz wall clock: 0.5 ms
-  const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * 4);
-  const int need = (int)((g.units + 1023) / 1024);
-  auto* xch = reinterpret_cast<unsigned long long*>(ws);
-  const dim3 grid((unsigned)(2 * g.C));
-#define BN_PAIR_LAUNCH(K2, KR)                                                                                    \
-  {                                                                                                               \
-    auto kernel = bn_bwd_pair<K2, KR>;                                                                            \
-    constexpr size_t shmem = (size_t)(K2 - KR) * 1024 * sizeof(float4);                                           \
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                     \
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);   \
-    if (attr != hipSuccess) return -1;                                                                            \
-    hipLaunchKernelGGL(kernel, grid, dim3(1024), shmem, s, g, bytes, x, dy, dx, a, xch, epoch, spin);             \
-  }
-  if (need <= 16) BN_PAIR_LAUNCH(8, 0)
-  else BN_PAIR_LAUNCH(13, 4)
-#undef BN_PAIR_LAUNCH
-  return check_launch("bn_bwd (a feature on two workgroups)");
-}
-
 // FUSE: the gradient first passes the ReLU mask of the forward result, read from y (1) or from the mask bytes (2)
 template <typename T, int FUSE>
 static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void* dx, float* ws,
@@ -1606,11 +1424,6 @@ static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void
     if (r8.threads)
       return run_bwd8<FUSE>(g, r8, reinterpret_cast<const bf16_t*>(xp), reinterpret_cast<const bf16_t*>(dyp),
                             reinterpret_cast<bf16_t*>(dxp), a, reinterpret_cast<const BnFuseBwd<bf16_t>&>(fu), s);
-  }
-  if (sizeof(T) == 4 && FUSE == 0) {
-    const int rc = try_bwd_pair(g, vec, reinterpret_cast<const float*>(xp), reinterpret_cast<const float*>(dyp),
-                                reinterpret_cast<float*>(dxp), ws, a, s);
-    if (rc >= 0) return rc;
   }
   {
     const ResPlan r = resident_plan(g, vec, RES_MIN_C_BWD);
@@ -1663,9 +1476,9 @@ extern "C" size_t flhip_bn_workspace_bytes(const flhip_bn_desc* d) {
   BnGeom g;
   int vec;
   if (make_geom(d, &g, &vec) != FLHIP_OK) return 0;
-  // the partial sums of the two-pass kernels; 32 bytes per feature for the kernel that shares a feature between two workgroups
-  const size_t two_pass = (size_t)g.C * g.S * 2 * sizeof(float), pair = (size_t)g.C * 32;
-  return two_pass > pair ? two_pass : pair;
+  // the partial sums of the two-pass kernels, and never less than 32 bytes per feature
+  const size_t two_pass = (size_t)g.C * g.S * 2 * sizeof(float), least = (size_t)g.C * 32;
+  return two_pass > least ? two_pass : least;
 }
 
 extern "C" int flhip_bn_fwd_train(const flhip_bn_desc* d, const void* x, const float* gamma,
@@ -1826,8 +1639,3 @@ extern "C" int flhip_bn_act_bwd_mask(const flhip_bn_desc* d, const void* x, cons
                          ws_bytes, stream);
 }
 
-#ifdef BN_STAMPS
-extern "C" int flhip_dbg_bn_stamps(unsigned long long* host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(flhip::bn_stamps), sizeof(unsigned long long) * 256 * 8);
-}
-#endif

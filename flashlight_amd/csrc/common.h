@@ -247,7 +247,6 @@ struct Options {
   int pw_pt = 2;                  // PW_PT = 2 | 4 | 8: position-tile width of the fp32 1x1 kernels / 32
   int pw16_pf = 0;                // PW16_PF = 1 / 4: one / four chunks (shallow / deep ring) in flight in the bf16 1x1 kernels, 2 / 8: the same with
                                   // tiles of 64 result channels in the direct-to-LDS kernels (0: by grid size)
-  int conv_rows = 0;              // CONV_ROWS = n: result rows per tile of the fp32 slab kernel where n fits (0: by its cost model)
   int conv_stack = 0;             // CONV_STACK = 1 | 2 | 4 | 8: images per tile of the bf16 3x3 kernel over planes that fit a tile (0: by grid size)
   bool pw16_no_taps = false;      // PW16_NO_TAPS: bf16 windows with several taps stay off the gathered-taps path
   bool tapped_no_reorder = false; // TAPPED_NO_REORDER: tapped kernels read the original weight layout

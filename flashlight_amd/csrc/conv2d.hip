@@ -304,13 +304,16 @@ extern "C" int flhip_conv2d_bwd_data_add(const flhip_conv_desc* d, const void* d
   const int rc = make_geom(d, &g);
   if (rc != FLHIP_OK) return rc;
   hipStream_t s = as_stream(stream);
+  // no kernel may see dx and addend as one buffer: the fused ones read a plane's last 16-byte cell of addend again
+  // after another workgroup may have written it (planes that are not a multiple of 8 positions), the others
+  // write dx before they read addend
+  FLHIP_REQUIRE(dx != addend, "conv2d_bwd_data_add: dx aliases addend");
   if (!force_direct() && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT)) {
     int r = skip(Options::SKIP_PWDMA) ? -1 : mfma_pwd16_conv_bwd_data(g, dy, w, addend, dx, s);
     if (r < 0) r = mfma_pointwise16_conv_bwd_data_add(g, dy, w, addend, dx, s);
     if (r >= 0) return r;
   }
-  // every other kernel: the plain pass, then the element-wise sum (dx may not alias addend here)
-  FLHIP_REQUIRE(dx != addend, "conv2d_bwd_data_add: dx aliases addend");
+  // every other kernel: the plain pass, then the element-wise sum
   const int r = flhip_conv2d_bwd_data(d, dy, w, dx, ws, ws_bytes, stream);
   if (r != FLHIP_OK) return r;
   return flhip_add(dx, addend, dx, (size_t)g.N * g.C * g.H * g.W, d->dtype, stream);

@@ -574,7 +574,6 @@ bool plan(SlabParams* p, size_t* shmem, bool bwd, bool aligned) {
     const int nb = (R * p->DW + 15) / 16;
     // time ~ rounds x (blocks of the busier MFMA wave pair) ; small fixed cost per round
     double cost = (double)rounds * ((nb + 1) / 2 + 0.5);
-    if (options().conv_rows) cost = R == options().conv_rows ? 0.0 : 1e29;     // measurement switch
     if (cost < best_cost - 1e-9) {
       best_cost = cost;
       best_r = R;

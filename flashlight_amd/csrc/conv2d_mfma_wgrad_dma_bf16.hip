@@ -93,15 +93,6 @@ struct WdStages {
   }
 };
 
-#ifdef WD_STAMPS
-}  // namespace
-__device__ unsigned long long wd_stamps[256 * 16];
-namespace {
-#define WD_STAMP(i) { if (threadIdx.x == 0 && blockIdx.y == 0 && blockIdx.x < 256) wd_stamps[blockIdx.x * 16 + (i)] = wall_clock64(); }
-#else
-#define WD_STAMP(i) {}
-#endif
-
 // NK16: steps of 16 positions per row (2 or 4).  Eight waves: two per 32 x 32 block of the tile (and per SIMD), which
 // take alternate steps of a row and add their accumulators through LDS at the end: while one of them shifts,
 // computes addresses or waits for LDS, the other one's matrix instructions run (one wave per block: 1.3 us per row
@@ -371,7 +362,6 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
 #pragma unroll
       for (int b = 0; b < 3; ++b) acc[a][b][r] = 0.f;
 
-  WD_STAMP(0)
   if (nrows > 0) {
     // Stage t multiplies while: the loads of stage t + 1 + D are issued, the shifted copies of stage t + 2 are made
     // (its loads are waited for before the barrier of iteration t), and the fragments of stage t + 1's first step
@@ -400,7 +390,6 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
       m0_ = gc.next(p.H, &img, &ih);
       if (nstages > 1) m1_ = gc.next(p.H, &img, &ih);
     }
-    WD_STAMP(1)
     bf16x8 fa[2][3], fb[2][3];
 #define WD_FRAGS(SET, J, D0, D1, B0, B1, B2)                                                           \
   {                                                                                                    \
@@ -447,9 +436,7 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
           m2_ = gc.next(p.H, &img, &ih);
         }
       }
-      if (t == 4) WD_STAMP(2)
       __syncthreads();
-      if (t == 4) WD_STAMP(3)
       if (t + 1 + WD_D < nstages) issue();
       if (m2_) shift_reads(nd2);
       // operands of stage t and of stage t + 1 (for its first fragments)
@@ -493,8 +480,6 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
           WD_FRAGS(0, 0, e0, e1, WD_B(1, 0, 0), WD_B(1, 0, 1), WD_B(1, 0, 2))
         }
       }
-      if (t == 4) WD_STAMP(5)
-      if (t == 8) WD_STAMP(6)
       sd = nd;
       sx = nx;
       sb = nb;
@@ -505,7 +490,6 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
 #undef WD_MULT
 #undef WD_FRAGS
   }
-  WD_STAMP(7)
 
   // element r of a tile: result channel m0 + wm*32 + (r/4)*8 + fh*4 + r%4, input channel c0 + wn*32 + fr
   float* o = out + (size_t)split * ((size_t)p.E + p.K);
@@ -574,7 +558,6 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
       o[p.E + m0 + tid] = t;
     }
   }
-  WD_STAMP(8)
 }
 
 // part[split][tap][K][C] (+ [K] bias sums) -> dw[K][C][tap], db[K]; the splits are added in a fixed order.
@@ -758,8 +741,3 @@ int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw
 
 }  // namespace flhip
 
-#ifdef WD_STAMPS
-extern "C" int flhip_dbg_stamps(unsigned long long* host) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(flhip::wd_stamps), sizeof(unsigned long long) * 256 * 16);
-}
-#endif

@@ -4,6 +4,7 @@
 #include <algorithm>
 #include <map>
 #include <mutex>
+#include <string>
 
 #include "flhip.h"
 
@@ -122,6 +123,12 @@ flhip_bn_desc bnDesc(const Tensor& input, const std::vector<int>& axes, int tag)
 }
 
 }  // namespace
+
+HipAutogradExtension::HipAutogradExtension() {
+  if (flhip_version() / 100 != FLHIP_VERSION / 100)
+    throw std::runtime_error("HipAutogradExtension: libflhip version " + std::to_string(flhip_version()) +
+                             " does not match the header it was compiled with (" + std::to_string(FLHIP_VERSION) + ")");
+}
 
 Tensor HipAutogradExtension::workspace(size_t bytes) {
   if (bytes == 0) return Tensor();
@@ -250,16 +257,20 @@ std::pair<Tensor, Tensor> HipAutogradExtension::conv2dBackwardFilterBias(
   std::shared_ptr<HipConv2DPayload> kept;
   if (autogradPayload && autogradPayload->data) kept = std::dynamic_pointer_cast<HipConv2DPayload>(autogradPayload->data);
   const size_t gatheredBytes = kept ? flhip_conv2d_gathered_bytes(&d) : 0;
+  // the forward pass's gathered input in place of x where the library still takes it for this geometry (a
+  // process-wide option changed between the two passes can withdraw it: then, as without a payload, from x)
+  int rc = FLHIP_INVALID_ARGUMENT;
   if (kept && gatheredBytes > 0 && kept->gathered.bytes() >= gatheredBytes) {
     DevicePtr kp(kept->gathered);
-    check(flhip_conv2d_bwd_filter_gathered(&d, kp.get(), gp.get(), static_cast<float*>(dwp.get()),
-                                           static_cast<float*>(dbp.get()), wsp.get(), wsBytes,
-                                           hipBackendStream()));
-  } else {
+    rc = flhip_conv2d_bwd_filter_gathered(&d, kp.get(), gp.get(), static_cast<float*>(dwp.get()),
+                                          static_cast<float*>(dbp.get()), wsp.get(), wsBytes,
+                                          hipBackendStream());
+    if (rc != FLHIP_OK && rc != FLHIP_INVALID_ARGUMENT) check(rc);
+  }
+  if (rc != FLHIP_OK)
     check(flhip_conv2d_bwd_filter(&d, xp.get(), gp.get(), static_cast<float*>(dwp.get()),
                                   static_cast<float*>(dbp.get()), wsp.get(), wsBytes,
                                   hipBackendStream()));
-  }
   // event: inputs {gradOutput, input}, outputs {gradWeights, gradBias (may be empty)}, ints as conv2d
   if (scope.on()) scope.done({gradOutput, input}, {gradWeights, gradBias}, {sx, sy, px, py, dx, dy, groups});
   return {gradWeights, gradBias};

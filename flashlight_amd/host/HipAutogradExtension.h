@@ -9,6 +9,8 @@ namespace fl {
 
 class HipAutogradExtension : public AutogradExtension {
  public:
+  // refuses to run on a libflhip whose descriptor layouts differ from the header this class was compiled with
+  HipAutogradExtension();
   // f32 and the private bf16 tag; the oneDNN extension supports everything but f16
   // (onednn/OneDnnAutogradExtension.cpp:12-16), the cuDNN one f16/f32/f64.
   bool isDataTypeSupported(const dtype& type) const override;

@@ -142,6 +142,13 @@ void StepProfiler::end(const detail::OpEvent&) {
   hipCheck(hipEventRecord(impl_->spans.back().stop, (hipStream_t)g_stream), "hipEventRecord");
 }
 
+// An operation that left early still closes its span (what it enqueued before leaving counts
+// towards it), so that depth returns to zero and every span has both events recorded.
+void StepProfiler::abort(const char*) {
+  if (impl_->depth <= 0 || --impl_->depth > 0) return;
+  (void)hipEventRecord(impl_->spans.back().stop, (hipStream_t)g_stream);
+}
+
 std::map<std::string, StepProfiler::Entry> StepProfiler::collect() {
   sync();
   impl_->depth = 0;

@@ -34,8 +34,11 @@ class OpObserver {
   virtual ~OpObserver() = default;
   // before the operation enqueues anything
   virtual void begin(const char* /*op*/) {}
-  // after it has enqueued everything (not called when the operation throws)
+  // after it has enqueued everything
   virtual void end(const OpEvent& /*event*/) {}
+  // in place of end() when the operation left without reporting: it threw, or it handed its
+  // work to another operation and returned.  Every begin() is followed by exactly one of the two.
+  virtual void abort(const char* /*op*/) {}
 };
 
 OpObserver* opObserver();
@@ -49,6 +52,11 @@ class OpScope {
   explicit OpScope(const char* op) : observer_(opObserver()), op_(op) {
     if (observer_) observer_->begin(op);
   }
+  ~OpScope() {
+    if (observer_ && !finished_) observer_->abort(op_);
+  }
+  OpScope(const OpScope&) = delete;
+  OpScope& operator=(const OpScope&) = delete;
   bool on() const { return observer_ != nullptr; }
   void done(std::vector<Tensor> inputs, std::vector<Tensor> outputs, std::vector<long long> ints = {},
             std::vector<double> reals = {}) {
@@ -58,12 +66,14 @@ class OpScope {
     e.outputs = std::move(outputs);
     e.ints = std::move(ints);
     e.reals = std::move(reals);
+    finished_ = true;
     observer_->end(e);
   }
 
  private:
   OpObserver* observer_;
   const char* op_;
+  bool finished_ = false;
 };
 
 }  // namespace detail
@@ -83,6 +93,7 @@ class StepProfiler : public detail::OpObserver {
   ~StepProfiler() override;
   void begin(const char* op) override;
   void end(const detail::OpEvent& event) override;
+  void abort(const char* op) override;
   // milliseconds per operation name since the last collect(), plus "(gaps)" and "(span)"
   std::map<std::string, Entry> collect();
 

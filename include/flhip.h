@@ -103,7 +103,12 @@ typedef struct flhip_bn_desc {
 
 const char* flhip_last_error(void);
 
-/* Library version, and the gfx architecture the kernels were compiled for. */
+/* Library version, and the gfx architecture the kernels were compiled for.  The version a caller was
+ * compiled against is FLHIP_VERSION; descriptor structs only ever grow at the end, and a caller must
+ * refuse to run when flhip_version() / 100 differs from FLHIP_VERSION / 100 (a layout change).
+ * 200: flhip_rnn_desc gained dropout, seed_lo, seed_hi; flhip_bn_workspace_bytes never returns less
+ * than 32 bytes per feature. */
+#define FLHIP_VERSION 201
 int flhip_version(void);
 const char* flhip_arch(void);
 
@@ -113,7 +118,7 @@ const char* flhip_arch(void);
  * called while another thread is inside the library.  Results stay within the stated
  * tolerances under every setting; the switches only choose between kernels.
  *   CONV_ALGO = direct | gather | tapped | convert | auto    CONV_SKIP = bf16,gemm1x1,slab,tapped,strip,first,wgrad128,pwdma
- *   PW_PT = 2 | 4 | 8    PW16_PF = 0 | 1 | 2 | 4 | 8    CONV_ROWS = 0 .. 64    CONV_STACK = 0 | 1 | 2 | 4 | 8    BN_ALGO = split | resident | pair | pairalone | auto
+ *   PW_PT = 2 | 4 | 8    PW16_PF = 0 | 1 | 2 | 4 | 8    CONV_STACK = 0 | 1 | 2 | 4 | 8    BN_ALGO = split | resident | auto
  *   PW16_NO_TAPS, TAPPED_NO_REORDER, MATMUL_VALU, RNN_UNFUSED = 1 | 0
  * Unknown names or values return FLHIP_INVALID_ARGUMENT.  The nearest thing in the
  * reference is the kernel-choice options object of its cuDNN extension
@@ -294,6 +299,11 @@ int flhip_convert(const void* src, int src_dtype, void* dst, int dst_dtype,
  * kilobytes to megabytes, each a launch of its own otherwise. */
 int flhip_convert_many(const void* const* src, void* const* dst, const size_t* n, int count,
                        int src_dtype, int dst_dtype, void* stream);
+/* How flhip_convert_many cuts such a list into launches (at most 64 tensors and 2^31 - 1 pieces of 2048
+ * elements each): returns the number of launches and, when launch_of is not null, the launch of
+ * every tensor (-1 for empty ones); -1 for an argument flhip_convert_many would refuse.  Host code
+ * only, no device call. */
+int flhip_convert_many_launches(const size_t* n, int count, int* launch_of);
 
 /* dst[i] = value for n elements of `dtype`: fl::full as the extension uses it for
  * default running statistics (onednn/BatchNorm.cpp:116-122), enqueued like every other

@@ -18,6 +18,7 @@
 #include <cstdio>
 #include <cstring>
 #include <functional>
+#include <map>
 #include <random>
 #include <string>
 #include <vector>
@@ -26,6 +27,7 @@
 #include "Modules.h"
 #include "SequentialBuilder.h"
 #include "HipAutogradExtension.h"
+#include "OpObserver.h"
 #include "flref.h"
 
 using namespace fl;
@@ -275,6 +277,19 @@ static void testPool() {
   CHECK(throws<std::invalid_argument>(
       [&] { e.pool2dBackward(g, t, g, 2, 2, 2, 2, 0, 0, PoolingMode::MAX, nullptr); }));
   CHECK(throws<std::invalid_argument>([&] { pool2d(small, 2, 2, 1, 1, 2, 2); }));   // pad >= window
+  // an operation that throws still pairs its begin with an abort: the profiler's depth returns to
+  // zero, later operations get spans of their own and collect() finds every event recorded
+  {
+    StepProfiler prof;
+    detail::setOpObserver(&prof);
+    CHECK(throws<std::invalid_argument>(
+        [&] { e.pool2dBackward(g, t, g, 2, 2, 2, 2, 0, 0, PoolingMode::MAX, nullptr); }));
+    Variable again = pool2d(small, 2, 2, 1, 1);
+    std::map<std::string, StepProfiler::Entry> got;
+    CHECK(!throws<std::runtime_error>([&] { got = prof.collect(); }));
+    CHECK(got["pool2dBackward"].calls == 1 && got["pool2d"].calls == 1);
+    detail::setOpObserver(nullptr);
+  }
 }
 
 static void testBatchnorm() {
@@ -767,10 +782,10 @@ static void testBottleneck() {
 
 // configs[3]: three (Conv 21x1 SAME -> BatchNorm over axis 2 -> ReLU) layers on [T, 1, 80, B],
 // channels 80 -> 250 -> 250 -> 250, strides 1, 1, 2 along time, from modules; forward and
-// backward against the CPU checker (T shortened so the checker stays fast).
-static void testSpeechStack() {
-  std::printf("speech stack (21x1 convolutions, batch norm, ReLU)\n");
-  const int T = 180, B = 3, chans[4] = {80, 250, 250, 250}, strides[3] = {1, 1, 2};
+// backward against the CPU checker, at a shortened size and at the stated one (T = 1500, B = 16).
+static void testSpeechStack(const int T, const int B) {
+  std::printf("speech stack (21x1 convolutions, batch norm, ReLU), T = %d, batch %d\n", T, B);
+  const int chans[4] = {80, 250, 250, 250}, strides[3] = {1, 1, 2};
   setSeed(17);
   std::vector<Conv2D> convs;
   std::vector<BatchNorm> bns;
@@ -1086,7 +1101,8 @@ int main() {
     testBatchNormModule();
     testLayerNormModule();
     testBottleneck();
-    testSpeechStack();
+    testSpeechStack(180, 3);
+    testSpeechStack(1500, 16);
     testRnn();
     testArchBuilder();
     testModuleShapesAndBatching();

@@ -24,8 +24,37 @@ def test_header_symbols_are_exported_and_bound():
 
 
 def test_version_and_arch():
-    assert capi.lib().flhip_version() >= 100
+    text = open(os.path.join(ROOT, "include", "flhip.h")).read()
+    declared = int(re.search(r"#define\s+FLHIP_VERSION\s+(\d+)", text).group(1))
+    assert capi.lib().flhip_version() == declared >= 200
     assert capi.lib().flhip_arch() == b"gfx950"
+
+
+def test_convert_many_launch_split():
+    """How flhip_convert_many cuts a list of tensors into launches: 64 tensors or 2^31 - 1
+    pieces of 2048 elements per launch, whichever comes first; empty tensors take no slot."""
+    lib = capi.lib()
+
+    def plan(sizes):
+        n = (C.c_size_t * len(sizes))(*sizes)
+        where = (C.c_int32 * len(sizes))()
+        launches = lib.flhip_convert_many_launches(n, len(sizes), where)
+        return launches, list(where)
+
+    assert plan([]) == (0, [])
+    assert plan([0, 0]) == (0, [-1, -1])
+    assert plan([5] * 64) == (1, [0] * 64)
+    assert plan([5] * 65) == (2, [0] * 64 + [1])
+    assert plan([5, 0] * 65)[0] == 2
+    big = (1 << 40) - 1                       # 2^29 pieces
+    launches, where = plan([big] * 9)         # three fit under 2^31 - 1, the fourth does not
+    assert launches == 3 and where == [0, 0, 0, 1, 1, 1, 2, 2, 2]
+    # exactly the grid limit fits, one more piece does not
+    limit = (1 << 31) - 1
+    rest = limit - 3 * (1 << 29)
+    assert plan([big] * 3 + [rest * 2048])[0] == 1
+    assert plan([big] * 3 + [rest * 2048 + 1])[0] == 2
+    assert plan([1 << 40])[0] == -1           # refused, like the call itself
 
 
 def test_conv_out_dims_and_errors():

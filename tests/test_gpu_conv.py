@@ -554,6 +554,17 @@ FULL = [
     # the other two layers of configs[3]
     ((16, 80, 1, 1500), (250, 80, 1, 21), (1, 1), (0, 10)),
     ((16, 250, 1, 1500), (250, 250, 1, 21), (1, 1), (0, 10)),
+    # layers of configs[4] at its stated batch 64, where the plan depends on the batch (the number of
+    # workgroups): stacked 7x7 tiles, the 14x14 3x3 layer, the three stride-2 3x3 layers (gathered taps,
+    # a workspace beyond 100 MB), the 1x1 layers of the last stage and the first 1x1 layer over 56x56 planes
+    ((64, 512, 7, 7), (512, 512, 3, 3), (1, 1), (1, 1)),
+    ((64, 256, 14, 14), (256, 256, 3, 3), (1, 1), (1, 1)),
+    ((64, 128, 56, 56), (128, 128, 3, 3), (2, 2), (1, 1)),
+    ((64, 256, 28, 28), (256, 256, 3, 3), (2, 2), (1, 1)),
+    ((64, 512, 14, 14), (512, 512, 3, 3), (2, 2), (1, 1)),
+    ((64, 2048, 7, 7), (512, 2048, 1, 1), (1, 1), (0, 0)),
+    ((64, 512, 7, 7), (2048, 512, 1, 1), (1, 1), (0, 0)),
+    ((64, 64, 56, 56), (256, 64, 1, 1), (1, 1), (0, 0)),
 ]
 
 
