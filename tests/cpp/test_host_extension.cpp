@@ -796,7 +796,11 @@ static void testSpeechStack(const int T, const int B) {
   auto x = randn((size_t)B * 80 * T, 71);
   Variable in(Tensor::fromVector({T, 1, 80, B}, x), true);
   Variable h = in;
-  for (int l = 0; l < 3; ++l) h = relu(bns[l](convs[l](h)));
+  std::vector<Variable> preRelu;       // the device's batch-norm results: the ReLU's mask on the way back
+  for (int l = 0; l < 3; ++l) {
+    preRelu.push_back(bns[l](convs[l](h)));
+    h = relu(preRelu.back());
+  }
   const int Tout = T / 2;
   CHECK(h.shape() == Shape({Tout, 1, 250, B}));
   auto dy = randn((size_t)B * 250 * Tout, 72);
@@ -835,13 +839,26 @@ static void testSpeechStack(const int T, const int B) {
     Layer& y = L[l];
     const size_t no = y.a.size();
     std::vector<float> gn(no), ga(no), dg(chans[l + 1]), dbn(chans[l + 1]), dw(y.w.size()), dbias(chans[l + 1]), gin(y.in.size());
-    flref_relu_bwd((int64_t)no, grad.data(), y.n.data(), gn.data());
+    // The ReLU's mask is the one discontinuous step: a value within rounding of zero that falls on
+    // the other side in the checker's forward pass moves a whole gradient element, and among millions
+    // of elements a dozen of those are a relative error of 1e-3.  The checker therefore takes the mask
+    // from the device's own batch-norm result, as the tape does (the results themselves agree to
+    // 1e-4 above; every other step is continuous).
+    const auto mask = hostOf(preRelu[l]);
+    size_t flips = 0;
+    for (size_t i = 0; i < no; ++i) flips += (mask[i] > 0.f) != (y.n[i] > 0.f);
+    flref_relu_bwd((int64_t)no, grad.data(), mask.data(), gn.data());
     flref_bn_bwd(B, chans[l + 1], y.hw, y.a.data(), gn.data(), y.g.data(), y.mean.data(), y.var.data(), 1e-5, ga.data(),
                  dg.data(), dbn.data());
     flref_conv2d_bwd_filter(&y.d, y.in.data(), ga.data(), dw.data(), dbias.data());
     flref_conv2d_bwd_data(&y.d, ga.data(), y.w.data(), gin.data());
-    CHECK(relL2(hostOf(convs[l].param(0).grad()), dw) <= 3e-4);
-    CHECK(relL2(hostOf(bns[l].param(0).grad()), dg) <= 3e-4 && relL2(hostOf(bns[l].param(1).grad()), dbn) <= 3e-4);
+    const double eW = relL2(hostOf(convs[l].param(0).grad()), dw), eG = relL2(hostOf(bns[l].param(0).grad()), dg),
+                 eB = relL2(hostOf(bns[l].param(1).grad()), dbn);
+    std::printf("  layer %d: %zu of %zu mask elements differ from the checker's forward pass; dw %.2e dgamma %.2e dbeta %.2e\n",
+                l, flips, no, eW, eG, eB);
+    CHECK(flips <= no / 100000 + 2);
+    CHECK(eW <= 3e-4);
+    CHECK(eG <= 3e-4 && eB <= 3e-4);
     // the bias gradient of a convolution followed by batch norm is zero up to rounding:
     // compare it on the scale of the filter gradient
     double num = 0, den = 0;
