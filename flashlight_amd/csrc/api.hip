@@ -40,6 +40,7 @@ static bool apply_option(Options& o, const char* name, const char* v) {
       if (strstr(v, "first")) m |= Options::SKIP_FIRST;
       if (strstr(v, "wgrad128")) m |= Options::SKIP_WGRAD128;
       if (strstr(v, "pwdma")) m |= Options::SKIP_PWDMA;
+      if (strstr(v, "wd32")) m |= Options::SKIP_WD32;
     }
     o.conv_skip = m;
     return true;

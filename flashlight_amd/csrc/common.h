@@ -241,7 +241,7 @@ inline void launch_elementwise(const T* a, const T* b, T* out, size_t n, Op op, 
 // flhip_set_option(); no entry point calls getenv on its per-call path.
 struct Options {
   enum { ALGO_AUTO = 0, ALGO_DIRECT, ALGO_GATHER, ALGO_TAPPED, ALGO_CONVERT };
-  enum { SKIP_BF16 = 1, SKIP_GEMM1X1 = 2, SKIP_SLAB = 4, SKIP_TAPPED = 8, SKIP_STRIP = 16, SKIP_FIRST = 32, SKIP_WGRAD128 = 64, SKIP_PWDMA = 128 };
+  enum { SKIP_BF16 = 1, SKIP_GEMM1X1 = 2, SKIP_SLAB = 4, SKIP_TAPPED = 8, SKIP_STRIP = 16, SKIP_FIRST = 32, SKIP_WGRAD128 = 64, SKIP_PWDMA = 128, SKIP_WD32 = 256 };
   int conv_algo = ALGO_AUTO;      // CONV_ALGO = direct | gather | tapped | convert
   unsigned conv_skip = 0;         // CONV_SKIP = comma list of bf16, gemm1x1, slab, tapped, strip, first, wgrad128, pwdma
   int pw_pt = 2;                  // PW_PT = 2 | 4 | 8: position-tile width of the fp32 1x1 kernels / 32

@@ -560,6 +560,486 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
   }
 }
 
+// ---- the same pass on 32 x 32 tiles -----------------------------------------------------------
+// A 64 x 64 tile per workgroup leaves few tiles (ONE for 64 -> 64 channels), so the positions are cut
+// into as many slices as there are CUs and every slice writes a whole partial gradient: 256 x 147 KB
+// written and read again by the reduce kernel, three times the bytes of the operands.  Here a
+// workgroup owns a 32 x 32 tile of (result, input) channels: four times the tiles, a quarter of the
+// slices, a quarter of the partial bytes; a slice is four times longer, so its start-up and its
+// final exchange weigh a quarter.  Each operand row is then fetched by two (K / 32, C / 32) tiles
+// instead of one: the tiles of a slice are numbered so that they run on one XCD at the same time and
+// the second fetch comes out of its L2.
+//
+// Slots are 32 rows (4 KB), a stage is one 16-byte load per lane: waves 0-3 copy the 32 dy rows,
+// waves 4-7 the 32 input rows, into two rings of W3_NS slots (stage st lives in slot st % W3_NS of
+// both).  One 32 x 32 block has 4 steps of 16 positions per stage for 8 waves, so an iteration of
+// the main loop (one barrier) covers TWO stages: wave (half, step) multiplies step `step` of stage
+// 2u + half.  Everything else a wave does in the iteration runs under its own matrix instructions:
+// the loads of the two stages W3_D ahead, the shifted dy copies of the stage four ahead (one cell
+// per thread) and the fragments of its next stage, fetched into each fragment register as soon
+// as the last product that reads it has been issued.
+// What bounds an iteration is the number of instructions a wave issues in it (a wave issues one
+// every four or five cycles, whatever their kind), so the loop is written to have few:
+//  * it is unrolled over the W3_NS / 2 positions of the rings and compiled once per half, so every LDS
+//    address is a constant plus a lane's fixed offset;
+//  * what a stage loads (image, rows) comes from a table in LDS that the workgroup fills when it starts;
+//  * every stage multiplies, also the ones that only bring input rows in (the two at the head of an
+//    image when rows are long, the one below a group of short rows) and the stage of zeros that
+//    pads an odd count: their dy rows are loaded as zeros, so their products are zeros (the input
+//    ring is cleared when the workgroup starts, so that is also true of slots no load has filled);
+//  * the bias gradient is one more matrix instruction per stage - the dy fragment times a
+//    fragment of ones with zeros at the positions a row's last cell repeats - in place of sixteen
+//    vector instructions per cell of the shifting pass.
+// At the end the eight waves' accumulators are added through LDS, three taps at a time, in a fixed order.
+constexpr int W3_T = 32;
+constexpr int W3_NS = 12;                 // slots per ring
+constexpr int W3_D = 8;                   // the loads of stages 2u + 2 + D, 2u + 3 + D are issued in iteration u
+constexpr int W3_NSH = 4;                 // shifted copies of stages 2u + 2, 2u + 3 (read in iteration u), 2u + 4, 2u + 5 (written)
+constexpr int W3_SLOT = W3_T * 128;
+constexpr int W3_MAXST = 1024;            // most stages of a workgroup: their table is 16 KB of LDS
+constexpr int W3_RING = (2 * W3_NS + 2 * W3_NSH) * W3_SLOT;
+constexpr int W3_LDS = W3_RING + W3_MAXST * 16;
+static_assert(W3_D % 2 == 0 && W3_D >= 6 && W3_NS >= W3_D + 4 && W3_NS % 4 == 0, "stages are issued in pairs; a stage's input rows stay for two more stages");
+#define W3_WAIT_VM(N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory")
+
+// What stage `st` of a workgroup's range loads: {byte offset of input row ih0 of the image in x (channel 0), ih0,
+// byte offset of dy row oh0 (channel 0), oh0 or a negative number when the stage has no dy rows (it only loads
+// input rows and does not multiply)}.  In the modes with several rows per stage a lane adds its row of the group
+// to ih0 / oh0 (and that row's bytes to the offsets); rows outside the image are loaded as zeros.
+//   G == 1: at the start of the range and of every image two stages load the input rows oh - 1 and oh, then one
+//           stage per output row oh loads dy row oh and input row oh + 1;
+//   G >= 2: a "row" of the range is a group of G output rows; a group's stage loads dy rows G g .. and input rows
+//           G g - 1 ..; after the last group of an image or of the range one stage loads the input rows below it;
+//   G == 0: a "row" of the range is an image, a stage loads it whole.
+template <int G>
+__device__ __forceinline__ int4 w3_stage(const WdParams& p, int row_begin, int nrows, int st) {
+  const int GH = G >= 2 ? (p.H + G - 1) / G : p.H;          // "rows" per image
+  int img, ih0, oh0;
+  if (G == 0) {
+    img = row_begin + st;
+    ih0 = 0;
+    oh0 = 0;
+  } else {
+    const int extra = G == 1 ? 2 : 1;                          // stages of a segment that only load
+    const int n0 = row_begin / GH, f0 = row_begin - n0 * GH;
+    const int r0 = min(GH - f0, nrows);                        // rows of the range in its first image
+    int seg, local, first, count;
+    if (st < r0 + extra) {
+      seg = 0; local = st; first = f0; count = r0;
+    } else {
+      const int s2 = st - (r0 + extra);
+      seg = 1 + s2 / (GH + extra);
+      local = s2 - (seg - 1) * (GH + extra);
+      first = 0;
+      count = min(GH, nrows - r0 - (seg - 1) * GH);
+    }
+    img = n0 + seg;
+    if (G == 1) {
+      const int oh = first + local - 2;                        // (local < 2: the two loading stages)
+      ih0 = local == 0 ? first - 1 : local == 1 ? first : oh + 1;
+      oh0 = local < 2 ? -1 : oh;
+    } else {
+      const int grp = first + min(local, count);
+      ih0 = G * grp - 1;
+      oh0 = local < count ? G * grp : -1;
+    }
+  }
+  return make_int4((img * p.C * p.H + ih0) * p.W * 2, ih0, (img * p.K * p.H + max(oh0, 0)) * p.W * 2, oh0);
+}
+
+template <int G>
+__global__ void __launch_bounds__(512, 1)
+wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy, float* __restrict__ out) {
+  constexpr bool IMG = G == 0;          // a stage is a whole image
+  constexpr bool GRP = G >= 2;          // a stage is a group of G rows
+  constexpr int CPR = GRP ? 8 / G : 8;  // cells of a row in a slot
+  static_assert(G == 0 || G == 1 || G == 2 || G == 4, "shapes in use");
+  extern __shared__ __align__(16) char wd_lds[];
+  // LDS as 32-bit addresses: a lane's fixed offset plus a constant, which the instruction carries
+  typedef __attribute__((address_space(3))) char lchar;
+  typedef __attribute__((address_space(3))) uintx4_t lu4;
+  typedef __attribute__((address_space(3))) uint16_t lu16;
+  lchar* const L = (lchar*)wd_lds;
+  constexpr int DRING = 0, XRING = W3_NS * W3_SLOT, SHIFT = 2 * W3_NS * W3_SLOT;   // byte offsets: dy rows, input rows, [buffer][D_0, D_2]
+  int4* const table = reinterpret_cast<int4*>(wd_lds + W3_RING);
+  constexpr int OOB = (int)0x80000000;
+  // workgroup -> (slice, tile): consecutive workgroup numbers go to the 8 XCDs in turn; the tiles of a slice get
+  // numbers 8 apart, so they share an L2
+  const int ntiles = p.ctiles * p.mtiles;
+  const int per = (int)gridDim.x >> 3;
+  const int lin = ((int)blockIdx.x & 7) * per + ((int)blockIdx.x >> 3);
+  if (lin >= p.nsplit * ntiles) return;
+  const int split = lin / ntiles, tile = lin - split * ntiles;
+  const int mtile = tile / p.ctiles, ctile = tile - mtile * p.ctiles;
+  const int m0 = mtile * W3_T, c0 = ctile * W3_T;
+  const int tid = threadIdx.x, lane = tid & 63, fr = lane & 31, fh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kstep = wave & 3, half = wave >> 2;                 // step of a stage; which stages
+  const bool ldx = wave >= 4;                                   // this wave copies input rows (else dy rows)
+  const int lblk = wave & 3;                                    // ... rows 8 lblk .. + 7 of the slot
+  const int row_begin = split * p.rps, nrows = min(row_begin + p.rps, p.total_rows) - row_begin;
+  const intx4_t drs = pd_rsrc(dy, p.dy_bytes), xrs = pd_rsrc(x, p.x_bytes);
+  const int P = p.H * p.W;
+  int nstages = 0;
+  if (nrows > 0) {
+    if (GRP) {
+      const int GH = (p.H + G - 1) / G;
+      nstages = nrows + ((row_begin + nrows - 1) / GH - row_begin / GH + 1);
+    } else if (IMG) {
+      nstages = nrows;
+    } else {
+      nstages = nrows + 2 * ((row_begin + nrows - 1) / p.H - row_begin / p.H + 1);
+    }
+  }
+  // (an odd count gets one stage more that loads zeros: stages go in pairs)
+  const int nst2 = (nstages + 1) & ~1;
+  for (int st = tid; st < nst2; st += 512)
+    table[st] = st < nstages ? w3_stage<G>(p, row_begin, nrows, st) : make_int4(0, -(1 << 20), 0, -1);
+  // The input ring starts as zeros: the first stages take "the rows of the stages before them" from slots that no
+  // load has filled yet, and the last stage of groups of rows takes the rows below it from the slot of a stage that
+  // does not exist.  Their dy rows are zeros, but zero times whatever LDS held is not always zero.
+  {
+    typedef __attribute__((address_space(3))) uintx4_t lu4z;
+    lu4z* z = (lu4z*)(wd_lds + W3_NS * W3_SLOT);
+#pragma unroll
+    for (int i = 0; i < W3_NS * W3_SLOT / 16 / 512; ++i) z[tid + 512 * i] = uintx4_t{0u, 0u, 0u, 0u};
+    static_assert(W3_NS * W3_SLOT % (16 * 512) == 0, "whole passes");
+  }
+
+  // ---- loads: lane -> row 8 lblk + lane / 8, LDS cell lane % 8, i.e. the row's cell (lane % 8) ^ (lane / 8)
+  const int lrow = lane >> 3, lcell = (lane & 7) ^ lrow;
+  const int lj = GRP ? lcell / CPR : 0, lcq = GRP ? lcell % CPR : lcell;
+  const bool cell_ok = IMG ? lcell < p.H : lcq < p.ncell;
+  const int lpos = IMG ? lcell * p.W : (lcq == p.ncell - 1 ? p.W - 8 : 8 * lcq);
+  // the lane's offset in the stage's row of channel 0 of its tensor (its row of a group included)
+  const int loff = cell_ok ? (((ldx ? c0 : m0) + 8 * lblk + lrow) * P + lpos + lj * p.W) * 2 : OOB;
+  const unsigned lds0 = pd_lds_addr(wd_lds) + (ldx ? XRING : DRING) + lblk * 1024;   // this wave's part of slot 0 of its ring
+  // stage table entry e into slot `slot` of the wave's ring
+  auto issue = [&](const int4 e, int slot) __attribute__((always_inline)) {
+    if (ldx) {
+      const int base = __builtin_amdgcn_readfirstlane(e.x), ih0 = __builtin_amdgcn_readfirstlane(e.y);
+      const bool in = (unsigned)(ih0 + lj) < (unsigned)p.H && loff != OOB;
+      pd_load_lds(xrs, lds0 + slot * W3_SLOT, in ? loff + base : OOB, 0);
+    } else {
+      const int base = __builtin_amdgcn_readfirstlane(e.z), oh0 = __builtin_amdgcn_readfirstlane(e.w);
+      const bool in = oh0 >= 0 && oh0 + lj < p.H && loff != OOB;
+      pd_load_lds(drs, lds0 + slot * W3_SLOT, in ? loff + base : OOB, 0);
+    }
+  };
+  // after this lane's load of a stage has landed (see the kernel above): zeros over the repeated positions of the
+  // input cell it loaded; IMG: zeros over the positions past the row in its input cell, and the cell at the very end
+  // of its tensor, which was loaded as zeros, is filled in with plain loads
+  const bool any_fix = IMG ? p.keep < 8 : (ldx && p.dup != 0);      // (the same for all lanes of a wave)
+  const int my_cell = (ldx ? XRING : DRING) + lblk * 1024 + lane * 16;
+  auto fix_tail = [&](int slot, int img) __attribute__((always_inline)) {
+    char* cellp = wd_lds + my_cell + slot * W3_SLOT;
+    if (IMG) {
+      if (cell_ok) {
+        uint16_t* q = reinterpret_cast<uint16_t*>(cellp);
+        const int o = loff + img * (ldx ? p.C : p.K) * P * 2;
+        if ((unsigned)o + 16u > (ldx ? p.x_bytes : p.dy_bytes)) {
+          const bf16_t* src = ldx ? x : dy;
+          for (int e = 0; e < p.keep; ++e) q[e] = src[(o >> 1) + e];
+        }
+        if (ldx)
+          for (int e = p.keep; e < 8; ++e) q[e] = 0;
+      }
+      return;
+    }
+    if (lcq == p.ncell - 1) {
+      int d = p.dup, at = 0;
+      if (d >= 4) {
+        *reinterpret_cast<uintx2_t*>(cellp) = uintx2_t{0u, 0u};
+        d -= 4;
+        at = 8;
+      }
+      if (d >= 2) {
+        *reinterpret_cast<uint32_t*>(cellp + at) = 0u;
+        d -= 2;
+        at += 4;
+      }
+      if (d) *reinterpret_cast<uint16_t*>(cellp + at) = 0;
+    }
+  };
+
+  // ---- the two shifted copies of a dy row: the 256 threads of a half make one cell each, (row, cell) = (idx / 8, idx % 8).
+  // D_0 = positions + 1 (the element after the cell comes from the next cell, zero past the row), D_2 = positions - 1.
+  int sh_cell, sh_nx, sh_pv;      // LDS offsets: the thread's cell in dy slot 0, the element after it, the one before
+  uint32_t sh_mask[4];      // IMG: the positions of the cell that belong to its row
+  bool sh_has_nx, sh_has_pv;
+  {
+    const int idx = tid & 255;
+    const int r = idx >> 3, c = idx & 7, sw = r & 7;
+    const int cq = GRP ? c % CPR : c;
+    const bool in = IMG ? c < p.H : cq < p.ncell;
+    const int pos = cq == p.ncell - 1 ? p.W - 8 : 8 * cq;
+    const int cn = min(c + 1, 7), start = cq + 1 == p.ncell - 1 ? p.W - 8 : 8 * (cq + 1);
+    const int cp = max(c - 1, 0);
+    sh_has_nx = !IMG && in && pos + 8 < p.W;
+    sh_has_pv = !IMG && in && pos > 0;
+    sh_cell = DRING + r * 128 + ((c ^ sw) << 4);
+    sh_nx = DRING + r * 128 + ((cn ^ sw) << 4) + (sh_has_nx ? 2 * (pos + 8 - start) : 0);
+    sh_pv = DRING + r * 128 + ((cp ^ sw) << 4) + (sh_has_pv ? 2 * (pos - 1 - 8 * (cq - 1)) : 0);
+    const unsigned keep = IMG ? (unsigned)p.keep : 8u;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) sh_mask[k] = (2u * k < keep ? 0xffffu : 0u) | (2u * k + 1 < keep ? 0xffff0000u : 0u);
+  }
+  uintx4_t sh_v;
+  uint32_t sh_a, sh_b;
+  auto shift_reads = [&](int ds_slot) __attribute__((always_inline)) {
+    sh_v = *(const lu4*)(L + sh_cell + ds_slot * W3_SLOT);
+    sh_a = *(const lu16*)(L + sh_nx + ds_slot * W3_SLOT);
+    sh_b = *(const lu16*)(L + sh_pv + ds_slot * W3_SLOT);
+  };
+  auto shift_writes = [&](int buf) __attribute__((always_inline)) {
+    lchar* o = L + sh_cell + (SHIFT - DRING) + buf * 2 * W3_SLOT;
+    uintx4_t v = sh_v;
+    if (IMG) v = uintx4_t{v.x & sh_mask[0], v.y & sh_mask[1], v.z & sh_mask[2], v.w & sh_mask[3]};
+    const uint32_t nx = sh_has_nx ? sh_a : 0u, pv = sh_has_pv ? sh_b : 0u;
+    *(lu4*)o =
+        uintx4_t{__builtin_amdgcn_alignbit(v.y, v.x, 16), __builtin_amdgcn_alignbit(v.z, v.y, 16),
+                 __builtin_amdgcn_alignbit(v.w, v.z, 16), __builtin_amdgcn_alignbit(nx, v.w, 16)};
+    *(lu4*)(o + W3_SLOT) =
+        uintx4_t{__builtin_amdgcn_alignbit(v.x, pv << 16, 16), __builtin_amdgcn_alignbit(v.y, v.x, 16),
+                 __builtin_amdgcn_alignbit(v.z, v.y, 16), __builtin_amdgcn_alignbit(v.w, v.z, 16)};
+  };
+
+  // ---- fragments: lane -> row fr of the block, k-octet fh of the wave's step
+  const int cellf = 2 * kstep + fh;                 // the lane's cell of a row of 8
+  const int fa_d = DRING + fr * 128 + ((cellf ^ (fr & 7)) * 16);      // LDS offsets: dy row of slot 0
+  const int fa_s = fa_d + (SHIFT - DRING);                             // D_0 of buffer 0 (D_2: + W3_SLOT)
+  int fb_p[3];                              // input rows of tap row kh in slot 0 ...
+  bool bnext[3];                                    // ... of the stage itself or (groups of rows) of the next stage
+#pragma unroll
+  for (int kh = 0; kh < 3; ++kh) {
+    bnext[kh] = false;
+    int cell = cellf;
+    if (GRP) {
+      const int rho = cellf / CPR + kh;
+      bnext[kh] = __builtin_amdgcn_readfirstlane(rho >= G ? 1 : 0) != 0;
+      cell = (rho % G) * CPR + cellf % CPR;
+    } else if (IMG) {
+      cell = (cellf + kh - 1) & 7;
+    }
+    fb_p[kh] = XRING + fr * 128 + ((cell ^ (fr & 7)) * 16);
+  }
+  // bias gradient: the lane's eight positions as ones, zeros where the row's last cell repeats positions, where a
+  // cell lies past the row and (IMG) where its positions belong to the next row
+  const bool do_db = p.want_db && ctile == 0;
+  bf16x8 ones;
+  {
+    const int cq = GRP ? cellf % CPR : cellf;
+    const bool in = IMG ? cellf < p.H : cq < p.ncell;
+    const int skip = !in ? 8 : (!IMG && cq == p.ncell - 1 ? p.dup : 0), keep = IMG ? p.keep : 8;
+    uint32_t w[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      w[k] = ((2 * k >= skip && 2 * k < keep) ? 0x3f80u : 0u) | ((2 * k + 1 >= skip && 2 * k + 1 < keep) ? 0x3f800000u : 0u);
+    ones = __builtin_bit_cast(bf16x8, uintx4_t{w[0], w[1], w[2], w[3]});
+  }
+  floatx16 acc[3][3], accb;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    accb[r] = 0.f;
+#pragma unroll
+    for (int a = 0; a < 3; ++a)
+#pragma unroll
+      for (int b = 0; b < 3; ++b) acc[a][b][r] = 0.f;
+  }
+
+  auto finish = [&]() __attribute__((always_inline)) {
+    // element r of a wave's tile: result channel m0 + (r/4)*8 + fh*4 + r%4, input channel c0 + fr.  The eight waves'
+    // tiles are added through LDS three taps (one kh) at a time: every wave parks its three tiles as 16-byte cells
+    // [wave][kw][r / 4][lane], then thread `cell` adds the eight copies of its cells in wave order and stores.
+    float* o = out + (size_t)split * ((size_t)p.E + p.K);
+    const size_t KC = (size_t)p.K * p.C;
+    static_assert(W3_RING >= 8 * 3 * 4 * 64 * 16, "the parked accumulators fit");
+    uintx4_t* park = reinterpret_cast<uintx4_t*>(wd_lds);
+  #pragma unroll
+    for (int kh = 0; kh < 3; ++kh) {
+      __syncthreads();
+  #pragma unroll
+      for (int kw = 0; kw < 3; ++kw)
+  #pragma unroll
+        for (int q = 0; q < 4; ++q)
+          park[((wave * 3 + kw) * 4 + q) * 64 + lane] =
+              uintx4_t{__float_as_uint(acc[kh][kw][4 * q]), __float_as_uint(acc[kh][kw][4 * q + 1]),
+                       __float_as_uint(acc[kh][kw][4 * q + 2]), __float_as_uint(acc[kh][kw][4 * q + 3])};
+      __syncthreads();
+  #pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int cell = tid + 512 * i;
+        if (cell < 768) {
+          uintx4_t v[8];
+  #pragma unroll
+          for (int w = 0; w < 8; ++w) v[w] = park[w * 768 + cell];
+          float sum[4];
+  #pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            float t = __uint_as_float(v[0][k]);
+  #pragma unroll
+            for (int w = 1; w < 8; ++w) t += __uint_as_float(v[w][k]);
+            sum[k] = t;
+          }
+          const int kw = cell >> 8, q = (cell >> 6) & 3, ln = cell & 63;
+          const int tap = kh * 3 + kw, c = c0 + (ln & 31);
+  #pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const int m = m0 + q * 8 + (ln >> 5) * 4 + k;
+            o[tap * KC + (size_t)m * p.C + c] = sum[k];
+          }
+        }
+      }
+    }
+    if (do_db) {
+      // every column of a wave's bias tile holds the same 32 sums: column 0 (lanes 0 and 32) goes through LDS as
+      // [wave][result channel], and the eight waves' sums are added in wave order
+      float* sums = reinterpret_cast<float*>(wd_lds);
+      __syncthreads();
+      if (fr == 0) {
+  #pragma unroll
+        for (int r = 0; r < 16; ++r) sums[wave * 32 + (r >> 2) * 8 + fh * 4 + (r & 3)] = accb[r];
+      }
+      __syncthreads();
+      if (tid < W3_T) {
+        float t = sums[tid];
+        for (int w = 1; w < 8; ++w) t += sums[w * 32 + tid];
+        o[p.E + m0 + tid] = t;
+      }
+    }
+  };
+
+  __syncthreads();                      // the table
+  if (nstages > 0) {
+    // every wave issues one load per stage; stages 0 .. D + 1 before the loop
+#pragma unroll
+    for (int st = 0; st < W3_D + 2; ++st)
+      if (st < nst2) issue(table[st], st);
+    if (W3_D + 2 <= nst2) W3_WAIT_VM(W3_D - 2);        // stages 4 .. D + 1 may be outstanding: 0 .. 3 have landed
+    else W3_WAIT_VM(0);
+    if (any_fix) {
+#pragma unroll
+      for (int st = 0; st < 4; ++st)
+        if (st < nstages) fix_tail(st, row_begin + st);
+    }
+    const int niter = nst2 >> 1;
+    // Compiled once per half: this wave's stages are s = 2u + HALF.
+    auto run = [&](auto half_c) __attribute__((always_inline)) {
+      constexpr int HALF = decltype(half_c)::value;
+      bf16x8 fa[3], fb[3];
+      // fragments of the stage in ring slot SL (its shifted copies in buffer SL % 4): its dy row (D_1), D_0, D_2 and its
+      // three input rows.  Ring of single rows (G == 1): the stage's own slot holds row oh + 1, the two slots before
+      // it rows oh and oh - 1.
+      auto load_fa = [&](auto sl_c) __attribute__((always_inline)) {
+        constexpr int SL = decltype(sl_c)::value;
+        fa[0] = __builtin_bit_cast(bf16x8, *(const lu4*)(L + fa_s + (SL & 3) * 2 * W3_SLOT));
+        fa[1] = __builtin_bit_cast(bf16x8, *(const lu4*)(L + fa_d + SL * W3_SLOT));
+        fa[2] = __builtin_bit_cast(bf16x8, *(const lu4*)(L + fa_s + ((SL & 3) * 2 + 1) * W3_SLOT));
+      };
+      auto load_fb = [&](auto sl_c, auto kh_c) __attribute__((always_inline)) {
+        constexpr int SL = decltype(sl_c)::value, KH = decltype(kh_c)::value;
+        constexpr int NEXT = (SL + 1) % W3_NS, PREV = (SL + W3_NS - 1) % W3_NS, PREV2 = (SL + W3_NS - 2) % W3_NS;
+        const int slot = GRP ? (bnext[KH] ? NEXT : SL) : IMG ? SL : (KH == 2 ? SL : KH == 1 ? PREV : PREV2);
+        fb[KH] = __builtin_bit_cast(bf16x8, *(const lu4*)(L + fb_p[KH] + slot * W3_SLOT));
+      };
+      using I0 = std::integral_constant<int, 0>;
+      using I1 = std::integral_constant<int, 1>;
+      using I2 = std::integral_constant<int, 2>;
+      {
+        // the shifted copies of stages 0 .. 3 (half h: stages h and 2 + h), then this wave's fragments of its first stage
+        __syncthreads();
+        shift_reads(HALF);
+        shift_writes(HALF);
+        if (2 + HALF < nst2) {
+          shift_reads(2 + HALF);
+          shift_writes(2 + HALF);
+        }
+        __syncthreads();
+        load_fa(std::integral_constant<int, HALF>{});
+        load_fb(std::integral_constant<int, HALF>{}, I0{});
+        load_fb(std::integral_constant<int, HALF>{}, I1{});
+        load_fb(std::integral_constant<int, HALF>{}, I2{});
+      }
+      // one iteration; u = PH (mod W3_NS / 2), so stage 2u + HALF + k lives in slot (2 PH + HALF + k) % W3_NS
+      auto body = [&](auto ph_c, const int u) __attribute__((always_inline)) {
+        constexpr int PH = decltype(ph_c)::value;
+        constexpr int S2 = (2 * PH + HALF + 2) % W3_NS, S4 = (2 * PH + HALF + 4) % W3_NS;      // slots of stages s + 2, s + 4
+        constexpr int F4 = (2 * PH + 4) % W3_NS, F5 = (2 * PH + 5) % W3_NS;                    // of stages 2u + 4, 2u + 5
+        constexpr int L0 = (2 * PH + 2 + W3_D) % W3_NS, L1 = (2 * PH + 3 + W3_D) % W3_NS;      // of the stages to load
+        const int sl = 2 * u + 2 + W3_D;
+        const bool more4 = 2 * u + 4 < nst2, morel = sl < nst2;
+        // the table entries of the loads, read ahead of the barrier
+        const int4 ea = table[morel ? sl : 0], eb = table[morel ? sl + 1 : 0];
+        if (more4) {
+          if (2 * u + 2 + W3_D <= nst2) W3_WAIT_VM(W3_D - 4);   // stages 2u + 6 .. 2u + 1 + D may be outstanding
+          else W3_WAIT_VM(0);
+          if (any_fix) {
+            fix_tail(F4, row_begin + 2 * u + 4);
+            if (2 * u + 5 < nstages) fix_tail(F5, row_begin + 2 * u + 5);       // (not the stage of zeros that pads an odd count)
+          }
+        }
+        __syncthreads();
+        if (morel) {
+          issue(ea, L0);
+          issue(eb, L1);
+        }
+        // (past the last stages these read and write slots that nobody reads any more)
+        shift_reads(S4);
+        // the products of stage s; each fragment register is refilled with stage s + 2's as soon as its last reader has issued
+        {
+#pragma unroll
+          for (int kw = 0; kw < 3; ++kw) acc[0][kw] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kw], fb[0], acc[0][kw], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        load_fb(std::integral_constant<int, S2>{}, I0{});
+        __builtin_amdgcn_sched_barrier(0);
+        {
+#pragma unroll
+          for (int kw = 0; kw < 3; ++kw) acc[1][kw] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kw], fb[1], acc[1][kw], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        load_fb(std::integral_constant<int, S2>{}, I1{});
+        shift_writes(S4 & 3);
+        __builtin_amdgcn_sched_barrier(0);
+        {
+#pragma unroll
+          for (int kw = 0; kw < 3; ++kw) acc[2][kw] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kw], fb[2], acc[2][kw], 0, 0, 0);
+          if (do_db) accb = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1], ones, accb, 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        load_fb(std::integral_constant<int, S2>{}, I2{});
+        load_fa(std::integral_constant<int, S2>{});
+      };
+      body(std::integral_constant<int, 0>{}, 0);
+      // (one way out of the loop: the accumulators have one live range)
+#pragma unroll 1
+      for (int u = 1; u < niter; u += 6) {
+        body(std::integral_constant<int, 1>{}, u);
+        if (u + 1 < niter) {
+          body(std::integral_constant<int, 2>{}, u + 1);
+          if (u + 2 < niter) {
+            body(std::integral_constant<int, 3>{}, u + 2);
+            if (u + 3 < niter) {
+              body(std::integral_constant<int, 4>{}, u + 3);
+              if (u + 4 < niter) {
+                body(std::integral_constant<int, 5>{}, u + 4);
+                if (u + 5 < niter) body(std::integral_constant<int, 0>{}, u + 5);
+              }
+            }
+          }
+        }
+      }
+      finish();
+    };
+    static_assert(W3_NS == 12, "the loop above is unrolled over the six positions of the rings");
+    // (each branch ends in the final exchange: the two copies of the loop never meet)
+    if (half == 0) run(std::integral_constant<int, 0>{});
+    else run(std::integral_constant<int, 1>{});
+  } else {
+    finish();
+  }
+}
+
 // part[split][tap][K][C] (+ [K] bias sums) -> dw[K][C][tap], db[K]; the splits are added in a fixed order.
 // A workgroup of 16 x 16 threads owns 64 consecutive elements (16 threads x 4), its 16 rows of threads share the
 // splits: small workgroups, so that a gradient of 36864 elements still spreads over every CU.
@@ -662,12 +1142,13 @@ wgrad_taps_gather_reduce_kernel(const float* __restrict__ part, int nsplit, int 
   }
 }
 
-bool wd_plan(const ConvGeom& g, WdParams* p) {
+// T: tile side (64: wgrad_dma_kernel, 32: wgrad_dma32_kernel)
+bool wd_plan(const ConvGeom& g, WdParams* p, int T) {
   if (!(g.KH == 3 && g.KW == 3 && g.sy == 1 && g.sx == 1 && g.py == 1 && g.px == 1 && g.dly == 1 && g.dlx == 1 &&
         g.groups == 1 && g.OH == g.H && g.OW == g.W))
     return false;
   const bool img = g.H <= 7 && g.W <= 8 && g.W >= 2;       // whole images per stage
-  if (g.C % WD_T != 0 || g.K % WD_T != 0 || (!img && g.W < 8) || g.W > 64) return false;
+  if (g.C % T != 0 || g.K % T != 0 || (!img && g.W < 8) || g.W > 64) return false;
   const long long xb = (long long)g.N * g.C * g.H * g.W * 2, db = (long long)g.N * g.K * g.H * g.W * 2;
   if (xb >= (1ll << 31) || db >= (1ll << 31)) return false;
   p->N = g.N; p->C = g.C; p->K = g.K; p->H = g.H; p->W = g.W;
@@ -678,8 +1159,8 @@ bool wd_plan(const ConvGeom& g, WdParams* p) {
   p->G = img ? 0 : g.W <= 16 ? 4 : g.W <= 32 ? 2 : 1;
   p->x_bytes = (unsigned)xb;
   p->dy_bytes = (unsigned)db;
-  p->ctiles = g.C / WD_T;
-  p->mtiles = g.K / WD_T;
+  p->ctiles = g.C / T;
+  p->mtiles = g.K / T;
   p->total_rows = img ? g.N : g.N * ((g.H + (p->G - 1)) / (p->G > 1 ? p->G : 1));        // stages: images, rows or groups of rows
   p->E = g.K * g.C * 9;
   const long long tiles = (long long)p->ctiles * p->mtiles;
@@ -689,8 +1170,17 @@ bool wd_plan(const ConvGeom& g, WdParams* p) {
   if (ns > p->total_rows / 4) ns = p->total_rows / 4;     // at least four rows per slice
   if (ns < 1) ns = 1;
   p->rps = (int)((p->total_rows + ns - 1) / ns);
+  // (the 32 x 32 kernel keeps a table of its stages in LDS: at most two stages per row and two more)
+  if (T == W3_T && p->rps > (W3_MAXST - 2) / 2) p->rps = (W3_MAXST - 2) / 2;
   p->nsplit = (p->total_rows + p->rps - 1) / p->rps;
   return true;
+}
+
+// Which tile a geometry gets.  32 x 32 tiles quarter the partial gradients that the slices write and the reduce
+// kernel reads back, and double the fetches of every operand row (from L2 when the tiles of a slice run together).
+bool wd_use32(const ConvGeom& g, WdParams* p) {
+  if (options().conv_skip & Options::SKIP_WD32) return false;
+  return wd_plan(g, p, W3_T);
 }
 
 size_t wd_ws_bytes(const WdParams& p) { return (size_t)p.nsplit * ((size_t)p.E + p.K) * sizeof(float); }
@@ -698,24 +1188,42 @@ size_t wd_ws_bytes(const WdParams& p) { return (size_t)p.nsplit * ((size_t)p.E +
 }  // namespace
 
 size_t mfma_wgrad_dma16_ws(const ConvGeom& g) {
-  WdParams p{};
-  return wd_plan(g, &p) ? wd_ws_bytes(p) : 0;
+  // the larger of the two plans, so that either kernel can run whatever the switches say at the time of the call
+  WdParams p{}, q{};
+  const size_t a = wd_plan(g, &p, WD_T) ? wd_ws_bytes(p) : 0, b = wd_plan(g, &q, W3_T) ? wd_ws_bytes(q) : 0;
+  return a > b ? a : b;
 }
 
 // -1 when the shape is not this kernel's
 int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes,
                      hipStream_t s) {
   WdParams p{};
-  if (!dw || !wd_plan(g, &p)) return -1;
+  if (!dw) return -1;
+  const bool t32 = wd_use32(g, &p);
+  if (!t32 && !wd_plan(g, &p, WD_T)) return -1;
   if (!ws || ws_bytes < wd_ws_bytes(p) || reinterpret_cast<uintptr_t>(ws) % 16 != 0) return -1;   // (the reduce kernels read 16 bytes at a time)
   p.want_db = db != nullptr;
+  float* part = static_cast<float*>(ws);
+  const bf16_t* xp = static_cast<const bf16_t*>(x);
+  const bf16_t* dyp = static_cast<const bf16_t*>(dy);
+  if (t32) {
+    const unsigned wgs = (unsigned)(p.nsplit * p.ctiles * p.mtiles);
+    const dim3 grid((wgs + 7) / 8 * 8);
+#define W3_LAUNCH(GR)                                                                                      \
+  {                                                                                                        \
+    if (!mfma_allow_lds(reinterpret_cast<const void*>(wgrad_dma32_kernel<GR>), W3_LDS)) return -1;         \
+    hipLaunchKernelGGL((wgrad_dma32_kernel<GR>), grid, dim3(512), W3_LDS, s, p, xp, dyp, part);            \
+  }
+    if (p.G == 0) W3_LAUNCH(0)
+    else if (p.G == 1) W3_LAUNCH(1)
+    else if (p.G == 2) W3_LAUNCH(2)
+    else W3_LAUNCH(4)
+#undef W3_LAUNCH
+  } else {
   // measured on the ResNet-50 layers at batch 64 against the kernel with register staging: 56x56 planes 36 against
   // 42 us, 28x28 (two rows per stage) 36 against 40, 14x14 (four rows) 43 against 52, 7x7 (whole images) 47 against 94
   // through gathered taps
   const dim3 grid((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles));
-  float* part = static_cast<float*>(ws);
-  const bf16_t* xp = static_cast<const bf16_t*>(x);
-  const bf16_t* dyp = static_cast<const bf16_t*>(dy);
 #define WD_LAUNCH(NK, GR)                                                                                      \
   {                                                                                                            \
     if (!mfma_allow_lds(reinterpret_cast<const void*>(wgrad_dma_kernel<NK, GR>), WD_LDS)) return -1;           \
@@ -726,6 +1234,7 @@ int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw
   else if (p.G == 2) WD_LAUNCH(4, 2)
   else WD_LAUNCH(4, 4)
 #undef WD_LAUNCH
+  }
   const int total = p.E + (p.want_db ? p.K : 0);
   // (a thread of it walks all splits and taps: it needs a gradient large enough for a few waves per CU;
   // 256 x 256 filters in 16 splits: 40 us against 7 us of the kernel below)

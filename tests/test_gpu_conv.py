@@ -258,8 +258,8 @@ def test_bf16_1x1_filter_gradient_alone(xs, K):
     assert rel_l2(host(dw2), dw_ref) <= 1e-4
 
 
-# bf16 3x3 filter gradient with at least 64 channels on both sides: the kernel whose operand rows the loads
-# copy straight to LDS.  Rows of 8k positions and rows whose last cell repeats positions (28, 14, 12, 20, 9:
+# bf16 3x3 filter gradient with channel counts that are multiples of 32 on both sides: the kernels whose operand rows
+# the loads copy straight to LDS (32 x 32 tiles; 64 x 64 tiles with that family switched off).  Rows of 8k positions and rows whose last cell repeats positions (28, 14, 12, 20, 9:
 # zeroed in the input rows); two or four 16-position steps per row; ranges of rows that start and end inside an
 # image and that span several images; several tiles; with and without the bias gradient (dy times ones, the
 # repeated positions counted once).
@@ -274,6 +274,10 @@ def test_bf16_1x1_filter_gradient_alone(xs, K):
     ((1, 64, 1, 2), 64), ((6, 64, 2, 5), 192),
     # few splits of a larger gradient: the reduce kernel that writes the gradient in memory order
     ((3, 256, 5, 6), 512), ((2, 512, 7, 7), 256),
+    # channel counts that only the 32 x 32 tiles take; more tiles than fit one round of workgroups on an XCD's share;
+    # more stages than the ring holds in every row shape (one row, two rows, four rows, whole images per stage)
+    ((2, 32, 10, 40), 96), ((3, 96, 14, 14), 32), ((2, 160, 6, 24), 32), ((11, 32, 7, 7), 32), ((2, 32, 40, 34), 32),
+    ((4, 32, 30, 30), 32), ((6, 32, 28, 14), 32), ((50, 32, 7, 5), 32), ((1, 576, 3, 8), 544),
 ])
 def test_bf16_3x3_filter_gradient_rows_to_lds(xs, K, with_bias):
     rng = np.random.default_rng(xs[0] * 17 + xs[3] + K)
@@ -291,13 +295,19 @@ def test_bf16_3x3_filter_gradient_rows_to_lds(xs, K, with_bias):
     assert rel_l2(host(dw), dw_ref) <= 1e-4, rel_l2(host(dw), dw_ref)
     if with_bias:
         assert rel_l2(host(db), db_ref) <= 1e-4, rel_l2(host(db), db_ref)
-    # the same through the kernel with register staging
-    capi.set_option("CONV_SKIP", "pwdma")
-    try:
-        dw2, _ = fa.conv2d_backward_filter_bias(dev(dy, torch.bfloat16), dev(x, torch.bfloat16), ws, False, px=1, py=1)
-    finally:
-        capi.set_option("CONV_SKIP", None)
-    assert rel_l2(host(dw2), dw_ref) <= 1e-4
+    # fixed order of every sum: a second run gives the same bits
+    dw1, db1 = fa.conv2d_backward_filter_bias(dev(dy, torch.bfloat16), dev(x, torch.bfloat16), ws, with_bias, px=1, py=1)
+    assert torch.equal(dw1, dw) and (not with_bias or torch.equal(db1, db))
+    # the same on 64 x 64 tiles, and through the kernel with register staging
+    for family in ("wd32", "pwdma"):
+        capi.set_option("CONV_SKIP", family)
+        try:
+            dw2, db2 = fa.conv2d_backward_filter_bias(dev(dy, torch.bfloat16), dev(x, torch.bfloat16), ws, with_bias, px=1, py=1)
+        finally:
+            capi.set_option("CONV_SKIP", None)
+        assert rel_l2(host(dw2), dw_ref) <= 1e-4, family
+        if with_bias:
+            assert rel_l2(host(db2), db_ref) <= 1e-4, family
 
 
 # bf16 3x3 kernel with several images per tile (planes that fit a tile whole, stacked with one shared zero
