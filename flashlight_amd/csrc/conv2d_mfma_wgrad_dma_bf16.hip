@@ -582,23 +582,22 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
 // every four or five cycles, whatever their kind), so the loop is written to have few:
 //  * it is unrolled over the W3_NS / 2 positions of the rings and compiled once per half, so every LDS
 //    address is a constant plus a lane's fixed offset;
-//  * what a stage loads (image, rows) comes from a table in LDS that the workgroup fills when it starts;
+//  * what a stage loads (image, rows) comes from a table of 64 stages that a wave keeps in the lanes of two
+//    registers (entry i in lane i, fetched with v_readlane) and refills every 32 iterations;
 //  * every stage multiplies, also the ones that only bring input rows in (the two at the head of an
 //    image when rows are long, the one below a group of short rows) and the stage of zeros that
-//    pads an odd count: their dy rows are loaded as zeros, so their products are zeros (the input
-//    ring is cleared when the workgroup starts, so that is also true of slots no load has filled);
+//    pads an odd count: their dy rows are loaded as zeros, so their products are zeros (slots of the
+//    input ring that no load has filled yet are cleared when the workgroup starts);
 //  * the bias gradient is one more matrix instruction per stage - the dy fragment times a
 //    fragment of ones with zeros at the positions a row's last cell repeats - in place of sixteen
 //    vector instructions per cell of the shifting pass.
 // At the end the eight waves' accumulators are added through LDS, three taps at a time, in a fixed order.
 constexpr int W3_T = 32;
-constexpr int W3_NS = 12;                 // slots per ring
-constexpr int W3_D = 8;                   // the loads of stages 2u + 2 + D, 2u + 3 + D are issued in iteration u
+constexpr int W3_NS = 16;                 // slots per ring
+constexpr int W3_D = 12;                  // the loads of stages 2u + 2 + D, 2u + 3 + D are issued in iteration u
 constexpr int W3_NSH = 4;                 // shifted copies of stages 2u + 2, 2u + 3 (read in iteration u), 2u + 4, 2u + 5 (written)
 constexpr int W3_SLOT = W3_T * 128;
-constexpr int W3_MAXST = 1024;            // most stages of a workgroup: their table is 16 KB of LDS
-constexpr int W3_RING = (2 * W3_NS + 2 * W3_NSH) * W3_SLOT;
-constexpr int W3_LDS = W3_RING + W3_MAXST * 16;
+constexpr int W3_LDS = (2 * W3_NS + 2 * W3_NSH) * W3_SLOT;     // all 160 KB of a CU
 static_assert(W3_D % 2 == 0 && W3_D >= 6 && W3_NS >= W3_D + 4 && W3_NS % 4 == 0, "stages are issued in pairs; a stage's input rows stay for two more stages");
 #define W3_WAIT_VM(N) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory")
 
@@ -661,7 +660,6 @@ wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __res
   typedef __attribute__((address_space(3))) uint16_t lu16;
   lchar* const L = (lchar*)wd_lds;
   constexpr int DRING = 0, XRING = W3_NS * W3_SLOT, SHIFT = 2 * W3_NS * W3_SLOT;   // byte offsets: dy rows, input rows, [buffer][D_0, D_2]
-  int4* const table = reinterpret_cast<int4*>(wd_lds + W3_RING);
   constexpr int OOB = (int)0x80000000;
   // workgroup -> (slice, tile): consecutive workgroup numbers go to the 8 XCDs in turn; the tiles of a slice get
   // numbers 8 apart, so they share an L2
@@ -693,19 +691,16 @@ wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __res
   }
   // (an odd count gets one stage more that loads zeros: stages go in pairs)
   const int nst2 = (nstages + 1) & ~1;
-  for (int st = tid; st < nst2; st += 512)
-    table[st] = st < nstages ? w3_stage<G>(p, row_begin, nrows, st) : make_int4(0, -(1 << 20), 0, -1);
-  // The input ring starts as zeros: the first stages take "the rows of the stages before them" from slots that no
-  // load has filled yet, and the last stage of groups of rows takes the rows below it from the slot of a stage that
-  // does not exist.  Their dy rows are zeros, but zero times whatever LDS held is not always zero.
-  {
-    typedef __attribute__((address_space(3))) uintx4_t lu4z;
-    lu4z* z = (lu4z*)(wd_lds + W3_NS * W3_SLOT);
-#pragma unroll
-    for (int i = 0; i < W3_NS * W3_SLOT / 16 / 512; ++i) z[tid + 512 * i] = uintx4_t{0u, 0u, 0u, 0u};
-    static_assert(W3_NS * W3_SLOT % (16 * 512) == 0, "whole passes");
-  }
-
+  // the wave's table of stages tbase .. tbase + 63 (lane i: stage tbase + i): offset and first row of the tensor
+  // this wave loads; stages past the last load zeros
+  int tab_base = 0, tab_row = 0;
+  auto fill_table = [&](int tbase) __attribute__((always_inline)) {
+    const int st = tbase + lane;
+    const int4 e = st < nstages ? w3_stage<G>(p, row_begin, nrows, st) : make_int4(0, -(1 << 20), 0, -1);
+    tab_base = ldx ? e.x : e.z;
+    tab_row = ldx ? e.y : e.w;
+  };
+  fill_table(0);
   // ---- loads: lane -> row 8 lblk + lane / 8, LDS cell lane % 8, i.e. the row's cell (lane % 8) ^ (lane / 8)
   const int lrow = lane >> 3, lcell = (lane & 7) ^ lrow;
   const int lj = GRP ? lcell / CPR : 0, lcq = GRP ? lcell % CPR : lcell;
@@ -714,15 +709,14 @@ wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __res
   // the lane's offset in the stage's row of channel 0 of its tensor (its row of a group included)
   const int loff = cell_ok ? (((ldx ? c0 : m0) + 8 * lblk + lrow) * P + lpos + lj * p.W) * 2 : OOB;
   const unsigned lds0 = pd_lds_addr(wd_lds) + (ldx ? XRING : DRING) + lblk * 1024;   // this wave's part of slot 0 of its ring
-  // stage table entry e into slot `slot` of the wave's ring
-  auto issue = [&](const int4 e, int slot) __attribute__((always_inline)) {
+  // stage st (in the wave's table) into slot `slot` of the wave's ring
+  auto issue = [&](int st, int slot) __attribute__((always_inline)) {
+    const int base = __builtin_amdgcn_readlane(tab_base, st & 63), row0 = __builtin_amdgcn_readlane(tab_row, st & 63);
     if (ldx) {
-      const int base = __builtin_amdgcn_readfirstlane(e.x), ih0 = __builtin_amdgcn_readfirstlane(e.y);
-      const bool in = (unsigned)(ih0 + lj) < (unsigned)p.H && loff != OOB;
+      const bool in = (unsigned)(row0 + lj) < (unsigned)p.H && loff != OOB;
       pd_load_lds(xrs, lds0 + slot * W3_SLOT, in ? loff + base : OOB, 0);
     } else {
-      const int base = __builtin_amdgcn_readfirstlane(e.z), oh0 = __builtin_amdgcn_readfirstlane(e.w);
-      const bool in = oh0 >= 0 && oh0 + lj < p.H && loff != OOB;
+      const bool in = row0 >= 0 && row0 + lj < p.H && loff != OOB;
       pd_load_lds(drs, lds0 + slot * W3_SLOT, in ? loff + base : OOB, 0);
     }
   };
@@ -853,7 +847,7 @@ wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __res
     // [wave][kw][r / 4][lane], then thread `cell` adds the eight copies of its cells in wave order and stores.
     float* o = out + (size_t)split * ((size_t)p.E + p.K);
     const size_t KC = (size_t)p.K * p.C;
-    static_assert(W3_RING >= 8 * 3 * 4 * 64 * 16, "the parked accumulators fit");
+    static_assert(W3_LDS >= 8 * 3 * 4 * 64 * 16, "the parked accumulators fit");
     uintx4_t* park = reinterpret_cast<uintx4_t*>(wd_lds);
   #pragma unroll
     for (int kh = 0; kh < 3; ++kh) {
@@ -909,12 +903,21 @@ wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __res
     }
   };
 
-  __syncthreads();                      // the table
   if (nstages > 0) {
     // every wave issues one load per stage; stages 0 .. D + 1 before the loop
 #pragma unroll
     for (int st = 0; st < W3_D + 2; ++st)
-      if (st < nst2) issue(table[st], st);
+      if (st < nst2) issue(st, st);
+    // The slots of the input ring that these loads do not fill start as zeros: the first stages take "the rows of the
+    // stages before them" from the last two slots, and the last stage of groups of rows takes the rows below it from
+    // the slot of a stage that does not exist.  Their dy rows are zeros, but zero times whatever LDS held is not
+    // always zero.  (Slots that have been loaded once hold rows of the tensor from then on.)
+    {
+      typedef __attribute__((address_space(3))) uintx4_t lu4z;
+      const int first = min(nst2, W3_D + 2);
+      lu4z* z = (lu4z*)(wd_lds + XRING + first * W3_SLOT);
+      for (int i = tid; i < (W3_NS - first) * (W3_SLOT / 16); i += 512) z[i] = uintx4_t{0u, 0u, 0u, 0u};
+    }
     if (W3_D + 2 <= nst2) W3_WAIT_VM(W3_D - 2);        // stages 4 .. D + 1 may be outstanding: 0 .. 3 have landed
     else W3_WAIT_VM(0);
     if (any_fix) {
@@ -968,8 +971,6 @@ wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __res
         constexpr int L0 = (2 * PH + 2 + W3_D) % W3_NS, L1 = (2 * PH + 3 + W3_D) % W3_NS;      // of the stages to load
         const int sl = 2 * u + 2 + W3_D;
         const bool more4 = 2 * u + 4 < nst2, morel = sl < nst2;
-        // the table entries of the loads, read ahead of the barrier
-        const int4 ea = table[morel ? sl : 0], eb = table[morel ? sl + 1 : 0];
         if (more4) {
           if (2 * u + 2 + W3_D <= nst2) W3_WAIT_VM(W3_D - 4);   // stages 2u + 6 .. 2u + 1 + D may be outstanding
           else W3_WAIT_VM(0);
@@ -980,8 +981,9 @@ wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __res
         }
         __syncthreads();
         if (morel) {
-          issue(ea, L0);
-          issue(eb, L1);
+          if ((sl & 63) == 0) fill_table(sl);      // (sl is even: a pair of stages never straddles two tables)
+          issue(sl, L0);
+          issue(sl + 1, L1);
         }
         // (past the last stages these read and write slots that nobody reads any more)
         shift_reads(S4);
@@ -1013,7 +1015,7 @@ wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __res
       body(std::integral_constant<int, 0>{}, 0);
       // (one way out of the loop: the accumulators have one live range)
 #pragma unroll 1
-      for (int u = 1; u < niter; u += 6) {
+      for (int u = 1; u < niter; u += 8) {
         body(std::integral_constant<int, 1>{}, u);
         if (u + 1 < niter) {
           body(std::integral_constant<int, 2>{}, u + 1);
@@ -1023,7 +1025,13 @@ wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __res
               body(std::integral_constant<int, 4>{}, u + 3);
               if (u + 4 < niter) {
                 body(std::integral_constant<int, 5>{}, u + 4);
-                if (u + 5 < niter) body(std::integral_constant<int, 0>{}, u + 5);
+                if (u + 5 < niter) {
+                  body(std::integral_constant<int, 6>{}, u + 5);
+                  if (u + 6 < niter) {
+                    body(std::integral_constant<int, 7>{}, u + 6);
+                    if (u + 7 < niter) body(std::integral_constant<int, 0>{}, u + 7);
+                  }
+                }
               }
             }
           }
@@ -1031,7 +1039,7 @@ wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __res
       }
       finish();
     };
-    static_assert(W3_NS == 12, "the loop above is unrolled over the six positions of the rings");
+    static_assert(W3_NS == 16, "the loop above is unrolled over the eight positions of the rings");
     // (each branch ends in the final exchange: the two copies of the loop never meet)
     if (half == 0) run(std::integral_constant<int, 0>{});
     else run(std::integral_constant<int, 1>{});
@@ -1170,17 +1178,22 @@ bool wd_plan(const ConvGeom& g, WdParams* p, int T) {
   if (ns > p->total_rows / 4) ns = p->total_rows / 4;     // at least four rows per slice
   if (ns < 1) ns = 1;
   p->rps = (int)((p->total_rows + ns - 1) / ns);
-  // (the 32 x 32 kernel keeps a table of its stages in LDS: at most two stages per row and two more)
-  if (T == W3_T && p->rps > (W3_MAXST - 2) / 2) p->rps = (W3_MAXST - 2) / 2;
   p->nsplit = (p->total_rows + p->rps - 1) / p->rps;
   return true;
 }
 
 // Which tile a geometry gets.  32 x 32 tiles quarter the partial gradients that the slices write and the reduce
 // kernel reads back, and double the fetches of every operand row (from L2 when the tiles of a slice run together).
+// Measured on the 3x3 layers of ResNet-50 (us per call with the bias gradient, 32 x 32 against 64 x 64 tiles): at batch
+// 32 every layer gains (56x56 23.2 / 27.0, 28x28 25.5 / 28.9, 14x14 31.3 / 34.9, 7x7 31.0 / 36.2: the slices of 64 x 64
+// tiles are 7 or 8 stages long there, mostly start-up); at batch 64 the first layer gains (30.3 / 34.5) and the
+// others, whose operands are then fetched 4 to 16 times, lose or draw (36.8 / 35.2, 46.0 / 43.2, 42.6 / 42.3).
 bool wd_use32(const ConvGeom& g, WdParams* p) {
   if (options().conv_skip & Options::SKIP_WD32) return false;
-  return wd_plan(g, p, W3_T);
+  if (!wd_plan(g, p, W3_T)) return false;
+  WdParams q{};
+  if (!wd_plan(g, &q, WD_T)) return true;               // channel counts that only the small tiles divide
+  return p->ctiles * p->mtiles <= 4 || q.rps < 12;
 }
 
 size_t wd_ws_bytes(const WdParams& p) { return (size_t)p.nsplit * ((size_t)p.E + p.K) * sizeof(float); }
