@@ -33,7 +33,9 @@ CONV_FLOP = 2 * 32 * 64 * 56 * 56 * 64 * 9          # one pass, 7.398752256e9
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, scaled by
 # the same counters on the library's copy kernel (see profiles/); None = not measured.
 MEASURED_TRAFFIC = {"conv2d_bwd_data_f32": 61.7e6, "conv2d_bwd_filter_f32": 93.7e6,
-                    "conv2d_bwd_data_bf16": 32.5e6, "conv2d_bwd_filter_bf16": 67.0e6}
+                    "conv2d_bwd_data_bf16": 37.0e6, "conv2d_bwd_filter_bf16": 45.3e6}
+# where those constants come from: they are typed in from that file, not read from a run of this script
+TRAFFIC_SOURCE = "profiles/bench_conv3x3_bn_pool__hbm_traffic_sq_counters.md"
 
 
 def parse():
@@ -125,17 +127,24 @@ def main():
         return fn
 
     # ---- conv pair at cfg 2 --------------------------------------------------
-    def conv_block(dname, with_pair):
-        """Times the conv ops of cfg 2 in storage type `dname`; returns the pair timing."""
+    pair_info = {}
+
+    def conv_block(dname, headline):
+        """Times the conv ops of cfg 2 in storage type `dname`.  Every figure comes twice: with whole
+        operand sets (x, dy, y, dx, dw, db) rotated over more than 512 MB per op, so that no call finds
+        its operands in the 256 MB memory-side cache (`us`), and on one set (`us_cache_warm`)."""
         tag = capi.F32 if dname == "f32" else capi.BF16
         ttype = torch.float32 if dname == "f32" else torch.bfloat16
-        x = randn(32, 64, 56, 56).to(ttype)
+        esz = 4 if dname == "f32" else 2
+        nsets = 11 * 4 // esz          # two tensors of 25.7 MB (fp32) per op and set: 565 MB per op
         w = randn(64, 64, 3, 3, scale=1.0 / 24.0).to(ttype)          # Kaiming normal, fan-in 576
         b = randn(64)
-        dy = randn(32, 64, 56, 56).to(ttype)
-        y, dx = torch.empty_like(x), torch.empty_like(x)
-        dw = torch.empty((64, 64, 3, 3), device=dev)
-        db = torch.empty(64, device=dev)
+        xs = [randn(32, 64, 56, 56).to(ttype) for _ in range(nsets)]
+        dys = [randn(32, 64, 56, 56).to(ttype) for _ in range(nsets)]
+        ys = [torch.empty_like(xs[0]) for _ in range(nsets)]
+        dxs = [torch.empty_like(xs[0]) for _ in range(nsets)]
+        dws = [torch.empty((64, 64, 3, 3), device=dev) for _ in range(nsets)]
+        dbs = [torch.empty(64, device=dev) for _ in range(nsets)]
         cd = capi.ConvDesc(32, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, tag)
         nws = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_BWD_FILTER)
         nws_f = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_FWD)
@@ -144,31 +153,43 @@ def main():
         ws_f = torch.empty(max(nws_f, 16), dtype=torch.uint8, device=dev)
         ws_d = torch.empty(max(nws_d, 16), dtype=torch.uint8, device=dev)
         peak_mfma = PEAK["f32_TFLOPs"] if dname == "f32" else PEAK["bf16_TFLOPs"]
-        cdp, xp, wp, bp, dyp, yp, dxp, dwp, dbp, wsp = (C.byref(cd), P(x), P(w), P(b), P(dy), P(y),
-                                                         P(dx), P(dw), P(db), P(ws))
-        wsfp, wsdp = P(ws_f), P(ws_d)
-        f_fwd = checked(lambda _: L.flhip_conv2d_fwd(cdp, xp, wp, bp, yp, wsfp, nws_f, S))
-        f_bwd_data = checked(lambda _: L.flhip_conv2d_bwd_data(cdp, dyp, wp, dxp, wsdp, nws_d, S))
-        f_bwd_filter = checked(lambda _: L.flhip_conv2d_bwd_filter(cdp, xp, dyp, dwp, dbp, wsp, nws, S))
+        cdp, wp, bp, wsp, wsfp, wsdp = C.byref(cd), P(w), P(b), P(ws), P(ws_f), P(ws_d)
+        xp, dyp, yp, dxp = [P(t) for t in xs], [P(t) for t in dys], [P(t) for t in ys], [P(t) for t in dxs]
+        dwp, dbp = [P(t) for t in dws], [P(t) for t in dbs]
+        f_fwd = checked(lambda i: L.flhip_conv2d_fwd(cdp, xp[i % nsets], wp, bp, yp[i % nsets], wsfp, nws_f, S))
+        f_bwd_data = checked(lambda i: L.flhip_conv2d_bwd_data(cdp, dyp[i % nsets], wp, dxp[i % nsets], wsdp, nws_d, S))
+        f_bwd_filter = checked(lambda i: L.flhip_conv2d_bwd_filter(cdp, xp[i % nsets], dyp[i % nsets], dwp[i % nsets],
+                                                                   dbp[i % nsets], wsp, nws, S))
 
         def conv_pair(i):
             f_bwd_data(i)
             f_bwd_filter(i)
 
         res = (None, None)
-        if with_pair and want("conv_pair"):
-            res = timed(conv_pair, a.steps, a.warmup)
-        for name, fn in (("conv2d_fwd", f_fwd), ("conv2d_bwd_data", f_bwd_data),
-                         ("conv2d_bwd_filter_bias", f_bwd_filter)):
+        tensor_bytes = xs[0].numel() * esz
+        if want("conv_pair"):
+            sp = {}
+            res = timed(conv_pair, a.steps, a.warmup, sp)
+            warm, _ = timed(lambda i: conv_pair(0), a.steps, a.warmup)
+            ach = 2 * CONV_FLOP / res[0] / 1e12
+            pair_info[dname] = {"us": res[0] * 1e6, "us_cache_warm": warm * 1e6, "achieved": ach, "peak": peak_mfma,
+                                "frac": ach / peak_mfma, "achieved_cache_warm": 2 * CONV_FLOP / warm / 1e12,
+                                "buffer_sets_rotated": nsets, "rotation_footprint_MB": nsets * 3 * tensor_bytes / 1e6, **sp}
+        for name, fn, ntens in (("conv2d_fwd", f_fwd, 2), ("conv2d_bwd_data", f_bwd_data, 2),
+                                ("conv2d_bwd_filter_bias", f_bwd_filter, 2)):
             if not want(name):
                 continue
             sp = {}
             s, _ = timed(fn, a.steps, a.warmup, sp)
+            warm, _ = timed(lambda i: fn(0), a.steps, a.warmup)
             ach = CONV_FLOP / s / 1e12
             ops.append({"op": name, "workload": "32x64x56x56, 64 filters 3x3 s1 p1", "dtype": dname,
                         "us": s * 1e6, "bound": "mfma", "achieved": ach, "peak": peak_mfma,
-                        "unit": "TFLOP/s", "frac": ach / peak_mfma, **sp})
-        return res
+                        "unit": "TFLOP/s", "frac": ach / peak_mfma, "buffer_sets_rotated": nsets,
+                        "rotation_footprint_MB": nsets * ntens * tensor_bytes / 1e6,
+                        "us_cache_warm": warm * 1e6, "TFLOPs_cache_warm": CONV_FLOP / warm / 1e12, **sp})
+        del xs, dys, ys, dxs
+        return res if headline else (None, None)
 
     pair_s, pair_wall = conv_block(a.dtype, True)
     # the same ops in the other storage type (bf16 storage, fp32 accumulate, when the
@@ -288,21 +309,35 @@ def main():
         "pool_max_bwd_GBps": by.get("pool2d_max_bwd", {}).get("achieved"),
         "pool_avg_bwd_GBps": by.get("pool2d_avg_bwd", {}).get("achieved"),
     }
+    if a.dtype in pair_info:
+        out["value_cache_warm"] = pair_info[a.dtype]["achieved_cache_warm"]
+        out["ms_per_step_cache_warm"] = pair_info[a.dtype]["us_cache_warm"] * 1e-3
+        out["pair"] = pair_info[a.dtype]
     if "conv2d_bwd_data" in by:
         o = by["conv2d_bwd_data"]
         out["roofline"] = {
-            "kernel": "slab_conv_kernel<float, true> (conv2dBackwardData, one launch per call)",
+            "kernel": ("slab_conv_kernel<float, true>" if a.dtype == "f32" else "strip16_conv_kernel") +
+                      " (conv2dBackwardData, one launch per call)",
             "bound": "mfma", "achieved": o["achieved"], "peak": o["peak"], "unit": "TFLOP/s",
-            "frac": o["frac"], "avg_launch_us": o["us"],
-            "traffic": MEASURED_TRAFFIC.get("conv2d_bwd_data_" + a.dtype)}
+            "frac": o["frac"], "avg_launch_us": o["us"], "avg_launch_us_cache_warm": o["us_cache_warm"],
+            "traffic": MEASURED_TRAFFIC.get("conv2d_bwd_data_" + a.dtype), "traffic_source": TRAFFIC_SOURCE}
     if "conv2d_bwd_filter_bias" in by:
         o = by["conv2d_bwd_filter_bias"]
         out["roofline_bwd_filter"] = {
             "kernel": "wgrad_slab_kernel<float> + wgrad_reduce_kernel (conv2dBackwardFilterBias, two launches per call)"
-                      if a.dtype == "f32" else "wgrad16_kernel + wgrad_reduce_kernel",
+                      if a.dtype == "f32" else "wgrad_dma32_kernel<1> + wgrad_taps_reduce_kernel",
             "bound": "mfma", "achieved": o["achieved"], "peak": o["peak"], "unit": "TFLOP/s",
-            "frac": o["frac"], "avg_call_us": o["us"],
-            "traffic": MEASURED_TRAFFIC.get("conv2d_bwd_filter_" + a.dtype)}
+            "frac": o["frac"], "avg_call_us": o["us"], "avg_call_us_cache_warm": o["us_cache_warm"],
+            "traffic": MEASURED_TRAFFIC.get("conv2d_bwd_filter_" + a.dtype), "traffic_source": TRAFFIC_SOURCE}
+    if "bf16" in pair_info:
+        # the 16-bit half of the target ("or bf16"): the same pair in bf16 storage against the bf16 matrix peak
+        pi = pair_info["bf16"]
+        out["roofline_bf16_pair"] = {
+            "kernel": "strip16_conv_kernel + wgrad_dma32_kernel<1> + wgrad_taps_reduce_kernel (three launches per step)",
+            "bound": "mfma", "achieved": pi["achieved"], "peak": pi["peak"], "unit": "TFLOP/s", "frac": pi["frac"],
+            "us_per_step": pi["us"], "us_per_step_cache_warm": pi["us_cache_warm"],
+            "traffic": (MEASURED_TRAFFIC["conv2d_bwd_data_bf16"] + MEASURED_TRAFFIC["conv2d_bwd_filter_bf16"]),
+            "traffic_source": TRAFFIC_SOURCE}
     out["ops"] = ops
     # the reference's CPU path: the oneDNN primitives its extension requests (through PyTorch-CPU,
     # whose embedded oneDNN executes them); the C restatement used as the parity checker is listed

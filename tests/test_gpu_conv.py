@@ -194,6 +194,30 @@ def test_conv_bf16_with_family_switched_off(family, case):
         capi.set_option("CONV_SKIP", None)
 
 
+# fp32 slab kernels over rows of whole 16-byte units (the 16-byte loaders) and over other rows (the element-wise
+# loaders): strides, dilation, groups, a filter tail, rows of 8 to 60 columns, a 5x1 and a 1x3 window, whole 7x7 planes.
+F32_SLAB_CASES = [
+    ((2, 64, 28, 28), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((1, 64, 20, 56), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((2, 64, 10, 16), (96, 32, 3, 3), (1, 1), (1, 1), (1, 1), 2),
+    ((1, 32, 5, 24), (64, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((3, 32, 9, 12), (40, 32, 3, 3), (1, 1), (2, 2), (2, 2), 1),
+    ((3, 64, 16, 16), (64, 64, 3, 3), (2, 1), (1, 1), (1, 2), 1),
+    ((2, 32, 12, 16), (24, 32, 3, 3), (2, 2), (1, 1), (1, 1), 1),
+    ((2, 16, 9, 20), (72, 16, 5, 1), (1, 1), (2, 0), (1, 1), 1),
+    ((2, 24, 6, 32), (32, 24, 1, 3), (1, 1), (0, 1), (1, 1), 1),
+    ((2, 8, 12, 8), (136, 8, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((3, 32, 7, 7), (64, 32, 3, 3), (1, 1), (1, 1), (1, 1), 1),
+    ((1, 16, 30, 60), (16, 16, 3, 3), (1, 1), (0, 0), (1, 1), 1),
+]
+
+
+@pytest.mark.parametrize("case", F32_SLAB_CASES)
+def test_conv_f32_slab_loaders(case):
+    for name, (got, ref) in _run(case, 36, torch.float32).items():
+        assert rel_l2(got, ref) <= F32_TOL, (name, rel_l2(got, ref))
+
+
 # bf16 1x1 kernels whose tiles are copied to LDS by the loads themselves: the dispatch picks them for small
 # planes and more than 64 result channels; PW16_PF = 1 / 4 lifts that rule and fixes the ring depth (4 / 8
 # stages; 2 / 8: the same with tiles of 64 result channels), so all four kernels run on planes that are / are not a multiple of 8 positions (the last cell of a
