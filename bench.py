@@ -49,6 +49,9 @@ def parse():
     ap.add_argument("--layers", choices=["resnet50", "speech"], default="",
                     help="instead of the bench line: time every conv layer of configs[4] (ResNet-50, batch 32) "
                          "or configs[3] (21x1 speech layers) in all three passes and print a table")
+    ap.add_argument("--plans", choices=["resnet50", "speech"], default="",
+                    help="instead of the bench line: time every kernel family (plan) of the two backward passes "
+                         "on the layers of a network and list where the fastest is not the default rule's choice")
     ap.add_argument("--step", choices=["resnet50", "speech"], default="",
                     help="instead of the bench line: a whole training step of configs[4] (ResNet-50, 224x224x3) or "
                          "configs[3] (speech stack) through the host modules, with a per-operation-class breakdown")
@@ -80,6 +83,8 @@ def main():
     tdt = torch.float32 if a.dtype == "f32" else torch.bfloat16
     if a.layers:
         return layer_sweep(a, fa, torch, tdt)
+    if a.plans:
+        return plan_sweep(a, fa, torch, tdt)
     if a.rnn:
         return rnn_sweep(a, fa, torch)
     gen = torch.Generator(device=dev).manual_seed(0)
@@ -453,6 +458,75 @@ def layer_sweep(a, fa, torch, tdt):
     print("totals over the network (counts applied, first layer without bwd-data): fwd %.2f ms, bwd-data %.2f ms, "
           "bwd-filter %.2f ms, sum %.2f ms for %.1f GFLOP = %.1f TFLOP/s (%s)" % (
               tot[0] / 1e3, tot[1] / 1e3, tot[2] / 1e3, sum(tot) / 1e3, flops, flops / sum(tot) * 1e3, a.dtype))
+    return 0
+
+
+def plan_sweep(a, fa, torch, tdt):
+    """Every plan of the two backward passes (flhip_conv2d_bwd_*_plan) on every layer of a network: the time of the
+    default rule, of the fastest plan, and which plans the library declined.  This is the measurement that
+    HipAutogradExtension::createBenchmarkOptions makes per layer at run time in benchmark mode."""
+    capi, L = fa.capi, fa.capi.lib()
+    tag = capi.F32 if tdt == torch.float32 else capi.BF16
+    S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: C.c_void_p(t.data_ptr())
+    steps = a.steps if a.steps != 100 else 20
+
+    def timed(fn):
+        for _ in range(3):
+            rc = fn()
+            if rc == capi.DECLINED:
+                return None
+            capi.check(rc)
+        torch.cuda.synchronize()
+        best = 1e30
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(steps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) / steps * 1e3)
+        return best
+
+    layers = RESNET50_LAYERS if a.plans == "resnet50" else SPEECH_LAYERS
+    nplans = L.flhip_conv2d_plan_count(capi.CONV_BWD_DATA)
+    print("| input NxCxHxW | K | window | stride | pass | default rule us | fastest plan | us | default / fastest |")
+    print("|---|---|---|---|---|---|---|---|---|")
+    gain = {"data": [0.0, 0.0], "filter": [0.0, 0.0]}
+    for i, (cnt, N, Ci, H, W, K, kh, kw, sy, sx, py, px) in enumerate(layers):
+        N = a.batch or N
+        x = torch.randn(N, Ci, H, W, device="cuda").to(tdt)
+        w = (torch.randn(K, Ci, kh, kw, device="cuda") / (Ci * kh * kw) ** 0.5).to(tdt)
+        cd = capi.ConvDesc(N, Ci, H, W, K, kh, kw, sy, sx, py, px, 1, 1, 1, tag)
+        oh, ow = C.c_int32(), C.c_int32()
+        capi.check(L.flhip_conv2d_out_dims(C.byref(cd), C.byref(oh), C.byref(ow)))
+        dy = torch.randn(N, K, oh.value, ow.value, device="cuda").to(tdt)
+        dx = torch.empty_like(x)
+        dw = torch.empty(K, Ci, kh, kw, device="cuda")
+        for pname, pas in (("data", capi.CONV_BWD_DATA), ("filter", capi.CONV_BWD_FILTER)):
+            if pname == "data" and i == 0 and a.plans == "resnet50":
+                continue                      # the first layer's input needs no gradient
+            nws = L.flhip_conv2d_workspace_bytes(C.byref(cd), pas)
+            ws = torch.empty(max(nws, 16), dtype=torch.uint8, device="cuda")
+            times = {}
+            for plan in range(-1, nplans - 1):            # (the direct kernels, the last plan, are never competitive)
+                if pas == capi.CONV_BWD_DATA:
+                    t = timed(lambda: L.flhip_conv2d_bwd_data_plan(C.byref(cd), P(dy), P(w), P(dx), P(ws), nws, plan, S))
+                else:
+                    t = timed(lambda: L.flhip_conv2d_bwd_filter_plan(C.byref(cd), P(x), P(dy), P(dw), None, P(ws), nws, plan, S))
+                if t is not None:
+                    times[plan] = t
+            best = min((p for p in times if p >= 0), key=lambda p: times[p])
+            gain[pname][0] += cnt * times[-1]
+            gain[pname][1] += cnt * times[best]
+            mark = " **" if times[best] < 0.95 * times[-1] else ""
+            print("| %dx%dx%dx%d | %d | %dx%d | %d,%d | bwd-%s | %.1f | %d: %s | %.1f | %.2f%s |" % (
+                N, Ci, H, W, K, kh, kw, sy, sx, pname, times[-1], best, L.flhip_conv2d_plan_name(pas, best).decode(),
+                times[best], times[-1] / times[best], mark), flush=True)
+    for pname in ("data", "filter"):
+        print("bwd-%s over the network (counts applied): default rule %.2f ms, fastest plan per layer %.2f ms (%s)" % (
+            pname, gain[pname][0] / 1e3, gain[pname][1] / 1e3, a.dtype))
     return 0
 
 

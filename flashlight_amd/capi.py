@@ -5,7 +5,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libflhip.so")
 
-OK, INVALID_ARGUMENT, RUNTIME_ERROR = 0, 1, 2
+OK, INVALID_ARGUMENT, RUNTIME_ERROR, DECLINED = 0, 1, 2, 3
 F32, BF16 = 0, 1
 CONV_FWD, CONV_BWD_DATA, CONV_BWD_FILTER = 0, 1, 2
 STATIC_SCRATCH_BYTES = 40 << 20      # FLHIP_STATIC_SCRATCH_BYTES
@@ -38,6 +38,10 @@ _VP, _SZ, _I32P = C.c_void_p, C.c_size_t, C.POINTER(C.c_int32)
 SYMBOLS = {
     "flhip_last_error": (C.c_char_p, []),
     "flhip_version": (C.c_int, []),
+    "flhip_conv2d_plan_count": (C.c_int, [C.c_int]),
+    "flhip_conv2d_plan_name": (C.c_char_p, [C.c_int, C.c_int]),
+    "flhip_conv2d_bwd_data_plan": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _SZ, C.c_int, _VP]),
+    "flhip_conv2d_bwd_filter_plan": (C.c_int, [C.POINTER(ConvDesc), _VP, _VP, _VP, _VP, _VP, _SZ, C.c_int, _VP]),
     "flhip_convert_many_launches": (C.c_int, [C.POINTER(C.c_size_t), C.c_int, _I32P]),
     "flhip_arch": (C.c_char_p, []),
     "flhip_set_option": (C.c_int, [C.c_char_p, C.c_char_p]),

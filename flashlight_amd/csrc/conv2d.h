@@ -116,8 +116,9 @@ int mfma_slab16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, 
                               hipStream_t s);
 // 3x3 filter gradient with operand rows copied straight to LDS (conv2d_mfma_wgrad_dma_bf16.hip)
 size_t mfma_wgrad_dma16_ws(const ConvGeom& g);
+// tile: 0 = by the measured rule, 32 / 64 = that tile side or decline
 int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes,
-                     hipStream_t s);
+                     hipStream_t s, int tile = 0);
 size_t mfma_wgrad16_ws(const ConvGeom& g);
 int mfma_wgrad16(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
                  size_t ws_bytes, hipStream_t s);

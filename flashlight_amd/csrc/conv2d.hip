@@ -258,13 +258,57 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
   return check_launch("conv2d_fwd");
 }
 
-extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, const void* w,
-                                     void* dx, void* ws, size_t ws_bytes, void* stream) {
+// The kernel families of the two backward passes, in the order of the default rule (the first that takes a geometry
+// runs it; each declines what it does not handle or, by measured rules, handles badly).  A plan number forces one
+// family: the caller times them instead of trusting the rules.
+static const char* const kBwdDataPlans[] = {"bf16 1x1, tiles loaded straight to LDS", "bf16 1x1 / gathered taps", "bf16 3x3 strip",
+                                            "bf16 slab", "1x1 GEMM, split contraction", "1x1 GEMM", "slab", "tapped GEMM",
+                                            "gather", "direct"};
+static const char* const kBwdFilterPlans[] = {"bf16 3x3 rows straight to LDS, 32 x 32 tiles", "bf16 3x3 rows straight to LDS, 64 x 64 tiles",
+                                              "bf16 1x1 / gathered taps", "bf16 first layer", "bf16 3x3 rows", "1x1 GEMM", "row slab",
+                                              "tapped GEMM", "gather", "direct"};
+constexpr int kNumPlans = 10;
+
+static int bwd_data_direct(const flhip_conv_desc* d, const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s) {
+  const size_t total = (size_t)g.N * g.C * g.H * g.W;
+  const dim3 grid((unsigned)((total + 255) / 256));
+  if (d->dtype == FLHIP_F32)
+    hipLaunchKernelGGL((conv_bwd_data_direct<float>), grid, dim3(256), 0, s, g,
+                       static_cast<const float*>(dy), static_cast<const float*>(w),
+                       static_cast<float*>(dx), total);
+  else
+    hipLaunchKernelGGL((conv_bwd_data_direct<bf16_t>), grid, dim3(256), 0, s, g,
+                       static_cast<const bf16_t*>(dy), static_cast<const bf16_t*>(w),
+                       static_cast<bf16_t*>(dx), total);
+  return check_launch("conv2d_bwd_data");
+}
+
+// plan < 0: the default rule; otherwise that family alone (FLHIP_DECLINED when it does not take the geometry)
+static int bwd_data_impl(const flhip_conv_desc* d, const void* dy, const void* w, void* dx, void* ws, size_t ws_bytes,
+                         int plan, void* stream) {
   FLHIP_REQUIRE(d && dy && w && dx, "conv2d_bwd_data: null argument");
   ConvGeom g;
   const int rc = make_geom(d, &g);
   if (rc != FLHIP_OK) return rc;
   hipStream_t s = as_stream(stream);
+  if (plan >= 0) {
+    FLHIP_REQUIRE(plan < kNumPlans, "conv2d_bwd_data: unknown plan");
+    const bool lo = d->dtype == FLHIP_BF16;
+    int r = -1;
+    switch (plan) {
+      case 0: if (lo) r = mfma_pwd16_conv_bwd_data(g, dy, w, nullptr, dx, s); break;
+      case 1: if (lo) r = mfma_pointwise16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes); break;
+      case 2: if (lo) r = mfma_strip16_conv_bwd_data(g, dy, w, dx, s); break;
+      case 3: if (lo) r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s); break;
+      case 4: r = mfma_pointwise_conv_split(g, d->dtype, true, dy, w, nullptr, dx, ws, ws_bytes, s); break;
+      case 5: r = mfma_pointwise_conv_bwd_data(g, d->dtype, dy, w, dx, s); break;
+      case 6: r = mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s); break;
+      case 7: r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes); break;
+      case 8: r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s); break;
+      default: r = bwd_data_direct(d, g, dy, w, dx, s);
+    }
+    return r < 0 ? FLHIP_DECLINED : r;
+  }
   if (!force_direct()) {
     int r = -1;
     if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
@@ -284,17 +328,26 @@ extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, c
     if (r < 0) r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r >= 0) return r;
   }
-  const size_t total = (size_t)g.N * g.C * g.H * g.W;
-  const dim3 grid((unsigned)((total + 255) / 256));
-  if (d->dtype == FLHIP_F32)
-    hipLaunchKernelGGL((conv_bwd_data_direct<float>), grid, dim3(256), 0, s, g,
-                       static_cast<const float*>(dy), static_cast<const float*>(w),
-                       static_cast<float*>(dx), total);
-  else
-    hipLaunchKernelGGL((conv_bwd_data_direct<bf16_t>), grid, dim3(256), 0, s, g,
-                       static_cast<const bf16_t*>(dy), static_cast<const bf16_t*>(w),
-                       static_cast<bf16_t*>(dx), total);
-  return check_launch("conv2d_bwd_data");
+  return bwd_data_direct(d, g, dy, w, dx, s);
+}
+
+extern "C" int flhip_conv2d_bwd_data(const flhip_conv_desc* d, const void* dy, const void* w,
+                                     void* dx, void* ws, size_t ws_bytes, void* stream) {
+  return bwd_data_impl(d, dy, w, dx, ws, ws_bytes, -1, stream);
+}
+
+extern "C" int flhip_conv2d_bwd_data_plan(const flhip_conv_desc* d, const void* dy, const void* w, void* dx, void* ws,
+                                          size_t ws_bytes, int plan, void* stream) {
+  return bwd_data_impl(d, dy, w, dx, ws, ws_bytes, plan, stream);
+}
+
+extern "C" int flhip_conv2d_plan_count(int pass) {
+  return pass == FLHIP_CONV_BWD_DATA || pass == FLHIP_CONV_BWD_FILTER ? kNumPlans : 0;
+}
+
+extern "C" const char* flhip_conv2d_plan_name(int pass, int plan) {
+  if (plan < 0 || plan >= kNumPlans) return nullptr;
+  return pass == FLHIP_CONV_BWD_DATA ? kBwdDataPlans[plan] : pass == FLHIP_CONV_BWD_FILTER ? kBwdFilterPlans[plan] : nullptr;
 }
 
 extern "C" int flhip_conv2d_bwd_data_add(const flhip_conv_desc* d, const void* dy, const void* w,
@@ -319,9 +372,30 @@ extern "C" int flhip_conv2d_bwd_data_add(const flhip_conv_desc* d, const void* d
   return flhip_add(dx, addend, dx, (size_t)g.N * g.C * g.H * g.W, d->dtype, stream);
 }
 
-extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, const void* dy,
-                                       float* dw, float* db, void* ws, size_t ws_bytes,
-                                       void* stream) {
+static int bwd_filter_direct(const flhip_conv_desc* d, const ConvGeom& g, const void* x, const void* dy, float* dw, float* db,
+                             hipStream_t s) {
+  if (dw) {
+    const dim3 grid((unsigned)(g.K * g.Cg * g.KH * g.KW));
+    if (d->dtype == FLHIP_F32)
+      hipLaunchKernelGGL((conv_bwd_filter_direct<float>), grid, dim3(256), 0, s, g,
+                         static_cast<const float*>(x), static_cast<const float*>(dy), dw);
+    else
+      hipLaunchKernelGGL((conv_bwd_filter_direct<bf16_t>), grid, dim3(256), 0, s, g,
+                         static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), dw);
+  }
+  if (db) {
+    if (d->dtype == FLHIP_F32)
+      hipLaunchKernelGGL((conv_bwd_bias_kernel<float>), dim3(g.K), dim3(256), 0, s, g,
+                         static_cast<const float*>(dy), db);
+    else
+      hipLaunchKernelGGL((conv_bwd_bias_kernel<bf16_t>), dim3(g.K), dim3(256), 0, s, g,
+                         static_cast<const bf16_t*>(dy), db);
+  }
+  return check_launch("conv2d_bwd_filter");
+}
+
+static int bwd_filter_impl(const flhip_conv_desc* d, const void* x, const void* dy, float* dw, float* db, void* ws,
+                           size_t ws_bytes, int plan, void* stream) {
   FLHIP_REQUIRE(d && dy, "conv2d_bwd_filter: null argument");
   FLHIP_REQUIRE(dw || db, "conv2d_bwd_filter: nothing to compute");
   FLHIP_REQUIRE(!dw || x, "conv2d_bwd_filter: filter gradient needs the input");
@@ -329,6 +403,26 @@ extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, 
   const int rc = make_geom(d, &g);
   if (rc != FLHIP_OK) return rc;
   hipStream_t s = as_stream(stream);
+  if (plan >= 0) {
+    FLHIP_REQUIRE(plan < kNumPlans, "conv2d_bwd_filter: unknown plan");
+    if (plan == kNumPlans - 1) return bwd_filter_direct(d, g, x, dy, dw, db, s);
+    const size_t need = flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER);
+    FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter: workspace too small");
+    const bool lo = d->dtype == FLHIP_BF16;
+    int r = -1;
+    switch (plan) {
+      case 0: if (lo) r = mfma_wgrad_dma16(g, x, dy, dw, db, ws, ws_bytes, s, 32); break;
+      case 1: if (lo) r = mfma_wgrad_dma16(g, x, dy, dw, db, ws, ws_bytes, s, 64); break;
+      case 2: if (lo) r = mfma_pointwise16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s); break;
+      case 3: if (lo) r = mfma_first16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s); break;
+      case 4: if (lo) r = mfma_wgrad16(g, x, dy, dw, db, ws, ws_bytes, s); break;
+      case 5: r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, false, s); break;
+      case 6: r = mfma_slab_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s); break;
+      case 7: r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, true, s); break;
+      default: r = mfma_conv_bwd_filter(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
+    }
+    return r < 0 ? FLHIP_DECLINED : r;
+  }
   if (!force_direct()) {
     const size_t need = flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER);
     FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter: workspace too small");
@@ -350,24 +444,18 @@ extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, 
     if (r < 0) r = mfma_conv_bwd_filter(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
     if (r >= 0) return r;
   }
-  if (dw) {
-    const dim3 grid((unsigned)(g.K * g.Cg * g.KH * g.KW));
-    if (d->dtype == FLHIP_F32)
-      hipLaunchKernelGGL((conv_bwd_filter_direct<float>), grid, dim3(256), 0, s, g,
-                         static_cast<const float*>(x), static_cast<const float*>(dy), dw);
-    else
-      hipLaunchKernelGGL((conv_bwd_filter_direct<bf16_t>), grid, dim3(256), 0, s, g,
-                         static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), dw);
-  }
-  if (db) {
-    if (d->dtype == FLHIP_F32)
-      hipLaunchKernelGGL((conv_bwd_bias_kernel<float>), dim3(g.K), dim3(256), 0, s, g,
-                         static_cast<const float*>(dy), db);
-    else
-      hipLaunchKernelGGL((conv_bwd_bias_kernel<bf16_t>), dim3(g.K), dim3(256), 0, s, g,
-                         static_cast<const bf16_t*>(dy), db);
-  }
-  return check_launch("conv2d_bwd_filter");
+  return bwd_filter_direct(d, g, x, dy, dw, db, s);
+}
+
+extern "C" int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x, const void* dy,
+                                       float* dw, float* db, void* ws, size_t ws_bytes,
+                                       void* stream) {
+  return bwd_filter_impl(d, x, dy, dw, db, ws, ws_bytes, -1, stream);
+}
+
+extern "C" int flhip_conv2d_bwd_filter_plan(const flhip_conv_desc* d, const void* x, const void* dy, float* dw, float* db,
+                                            void* ws, size_t ws_bytes, int plan, void* stream) {
+  return bwd_filter_impl(d, x, dy, dw, db, ws, ws_bytes, plan, stream);
 }
 
 // The forward pass of a strided layer in bf16 storage gathers the input points its windows touch into the start of

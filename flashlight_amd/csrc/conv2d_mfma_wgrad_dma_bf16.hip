@@ -1209,10 +1209,11 @@ size_t mfma_wgrad_dma16_ws(const ConvGeom& g) {
 
 // -1 when the shape is not this kernel's
 int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes,
-                     hipStream_t s) {
+                     hipStream_t s, int tile) {
   WdParams p{};
   if (!dw) return -1;
-  const bool t32 = wd_use32(g, &p);
+  const bool t32 = tile == 0 ? wd_use32(g, &p) : tile == W3_T && wd_plan(g, &p, W3_T);
+  if (tile == W3_T && !t32) return -1;
   if (!t32 && !wd_plan(g, &p, WD_T)) return -1;
   if (!ws || ws_bytes < wd_ws_bytes(p) || reinterpret_cast<uintptr_t>(ws) % 16 != 0) return -1;   // (the reduce kernels read 16 bytes at a time)
   p.want_db = db != nullptr;

@@ -181,24 +181,39 @@ AutogradExtension& ext(const Variable& v) { return getAutogradExtension(v.tensor
 }  // namespace
 
 Variable conv2d(const Variable& input, const Variable& weights, int sx, int sy, int px, int py,
-                int dx, int dy, int groups) {
-  return conv2d(input, weights, Variable(), sx, sy, px, py, dx, dy, groups);
+                int dx, int dy, int groups, std::shared_ptr<detail::ConvBenchmarks> benchmarks) {
+  return conv2d(input, weights, Variable(), sx, sy, px, py, dx, dy, groups, std::move(benchmarks));
 }
 
 Variable conv2d(const Variable& input, const Variable& weights, const Variable& bias, int sx,
-                int sy, int px, int py, int dx, int dy, int groups) {
+                int sy, int px, int py, int dx, int dy, int groups,
+                std::shared_ptr<detail::ConvBenchmarks> benchmarks) {
   dtypesMatch("conv2d", {&input, &weights, &bias});
   const bool hasBias = bias.tensor().elements() > 0;
   auto payload = createPayload({&input, &weights, &bias});
   Tensor output = ext(input).conv2d(input.tensor(), weights.tensor(), bias.tensor(), sx, sy, px, py,
                                     dx, dy, groups, payload);
 
-  auto gradFunc = [sx, sy, px, py, dx, dy, hasBias, groups, payload](
+  auto gradFunc = [sx, sy, px, py, dx, dy, hasBias, groups, benchmarks, payload](
                       std::vector<Variable>& inputs, const Variable& gradOutput) {
     // Functions.cpp:1362-1452
     auto& in = inputs[0];
     auto& wt = inputs[1];
     AutogradExtension& e = ext(in);
+    // The benchmarks of the two passes: made on the first backward pass in benchmark mode (:1372-1388) and handed
+    // to the extension on every pass from then on (the reference hands them over only on the pass that makes
+    // them), so that the choice they arrive at is used once the timings are complete, also with the mode off again.
+    std::shared_ptr<DynamicBenchmark> dataBench, filterBench, biasBench;
+    if (benchmarks) {
+      if (DynamicBenchmark::getBenchmarkMode()) {
+        if (!benchmarks->bwdFilterBenchmark) benchmarks->bwdFilterBenchmark = e.createBenchmarkOptions();
+        if (!benchmarks->bwdDataBenchmark) benchmarks->bwdDataBenchmark = e.createBenchmarkOptions();
+        if (!benchmarks->bwdBiasBenchmark) benchmarks->bwdBiasBenchmark = e.createBenchmarkOptions();
+      }
+      dataBench = benchmarks->bwdDataBenchmark;
+      filterBench = benchmarks->bwdFilterBenchmark;
+      biasBench = benchmarks->bwdBiasBenchmark;
+    }
     if (in.isCalcGrad()) {
       auto* hip = detail::fusedGradAdd() ? dynamic_cast<HipAutogradExtension*>(&e) : nullptr;
       if (hip && in.isGradAvailable() && in.grad().type() == gradOutput.type() && in.grad().shape() == in.shape()) {
@@ -208,7 +223,7 @@ Variable conv2d(const Variable& input, const Variable& weights, const Variable& 
                                                   sx, sy, px, py, dx, dy, groups));
       } else {
         Tensor g = e.conv2dBackwardData(gradOutput.tensor(), in.tensor(), wt.tensor(), sx, sy, px, py,
-                                        dx, dy, groups, nullptr, payload);
+                                        dx, dy, groups, dataBench, payload);
         in.addGrad(Variable(g, false));
       }
     }
@@ -217,7 +232,7 @@ Variable conv2d(const Variable& input, const Variable& weights, const Variable& 
       // an empty bias tells the extension that no bias gradient is wanted (:1391-1395)
       const Tensor bs = biasGrad ? inputs[2].tensor() : Tensor();
       auto grads = e.conv2dBackwardFilterBias(gradOutput.tensor(), in.tensor(), wt.tensor(), bs, sx,
-                                              sy, px, py, dx, dy, groups, nullptr, nullptr, payload);
+                                              sy, px, py, dx, dy, groups, filterBench, biasBench, payload);
       if (wt.isCalcGrad()) wt.addGradWide(grads.first);
       if (biasGrad) inputs[2].addGradWide(grads.second);
     }

@@ -13,6 +13,7 @@
 #include <tuple>
 #include <vector>
 
+#include "DynamicBenchmark.h"
 #include "AutogradExtension.h"
 
 namespace fl {
@@ -75,10 +76,14 @@ class Variable {
 // fl::derivePadding (flashlight/fl/nn/Utils.cpp:87-100); pad == -1 is SAME
 int derivePadding(int inSz, int filterSz, int stride, int pad, int dilation);
 
+// `benchmarks` (flashlight/fl/autograd/Functions.h: the last argument of both forms): where the backward passes keep
+// their kernel-choice benchmarks between calls; created on the first backward pass made in benchmark mode.
 Variable conv2d(const Variable& input, const Variable& weights, const Variable& bias, int sx = 1,
-                int sy = 1, int px = 0, int py = 0, int dx = 1, int dy = 1, int groups = 1);
+                int sy = 1, int px = 0, int py = 0, int dx = 1, int dy = 1, int groups = 1,
+                std::shared_ptr<detail::ConvBenchmarks> benchmarks = nullptr);
 Variable conv2d(const Variable& input, const Variable& weights, int sx = 1, int sy = 1,
-                int px = 0, int py = 0, int dx = 1, int dy = 1, int groups = 1);
+                int px = 0, int py = 0, int dx = 1, int dy = 1, int groups = 1,
+                std::shared_ptr<detail::ConvBenchmarks> benchmarks = nullptr);
 Variable pool2d(const Variable& input, int wx, int wy, int sx = 1, int sy = 1, int px = 0,
                 int py = 0, PoolingMode mode = PoolingMode::MAX);
 Variable batchnorm(const Variable& input, const Variable& weight, const Variable& bias,

@@ -1,7 +1,9 @@
 #include "HipAutogradExtension.h"
+#include "DynamicBenchmark.h"
 #include "OpObserver.h"
 
 #include <algorithm>
+#include <cstring>
 #include <map>
 #include <mutex>
 #include <string>
@@ -130,6 +132,59 @@ HipAutogradExtension::HipAutogradExtension() {
                              " does not match the header it was compiled with (" + std::to_string(FLHIP_VERSION) + ")");
 }
 
+// ---- plans of the backward passes -------------------------------------------------------------
+namespace {
+// option -1 = the default rule, 0 .. = the kernel families; remembers the geometry its timings belong to
+struct HipPlanOptions : DynamicBenchmarkOptions<int> {
+  HipPlanOptions(std::vector<int> plans, std::size_t count) : DynamicBenchmarkOptions<int>(std::move(plans), count) {}
+  // timings of another geometry (or pass) say nothing about this one: start again
+  void bind(const flhip_conv_desc& d, int pass) {
+    if (bound && pass == boundPass && std::memcmp(&d, &key, sizeof(d)) == 0) return;
+    reset();
+    key = d;
+    boundPass = pass;
+    bound = true;
+  }
+  flhip_conv_desc key{};
+  int boundPass = -1;
+  bool bound = false;
+};
+
+// Runs one backward pass under a benchmark: `run(plan)` enqueues the pass with that plan and returns the library's
+// status.  With complete timings the winner runs (benchmark mode on or off); while timings are being taken (mode on)
+// the current option runs inside audit(), and an option the library declines is struck out and the default rule
+// runs in its place, so that the call still produces its result; otherwise the default rule.
+template <typename Run>
+void runPlanned(const std::shared_ptr<DynamicBenchmark>& bench, const flhip_conv_desc& d, int pass, const Run& run,
+                void (*checkRc)(int)) {
+  if (!bench) {
+    checkRc(run(-1));
+    return;
+  }
+  auto opts = bench->getOptions<HipPlanOptions>();
+  opts->bind(d, pass);
+  if (!opts->timingsComplete() && !DynamicBenchmark::getBenchmarkMode()) {
+    checkRc(run(-1));
+    return;
+  }
+  bench->audit([&] {
+    const int rc = run(opts->currentOption());
+    if (rc == FLHIP_DECLINED) {
+      opts->penalise();
+      checkRc(run(-1));
+    } else {
+      checkRc(rc);
+    }
+  });
+}
+}  // namespace
+
+std::shared_ptr<DynamicBenchmark> HipAutogradExtension::createBenchmarkOptions() {
+  std::vector<int> plans{-1};
+  for (int i = 0; i < flhip_conv2d_plan_count(FLHIP_CONV_BWD_DATA); ++i) plans.push_back(i);
+  return std::make_shared<DynamicBenchmark>(std::make_shared<HipPlanOptions>(std::move(plans), kPlanBenchCount));
+}
+
 Tensor HipAutogradExtension::workspace(size_t bytes) {
   if (bytes == 0) return Tensor();
   if (ws_.bytes() < bytes) ws_ = Tensor({(Dim)bytes}, dtype::u8);
@@ -179,7 +234,7 @@ Tensor HipAutogradExtension::conv2dBackwardData(const Tensor& gradOutput, const 
                                                 const Tensor& weight, const int sx, const int sy,
                                                 const int px, const int py, const int dx,
                                                 const int dy, const int groups,
-                                                std::shared_ptr<DynamicBenchmark>,
+                                                std::shared_ptr<DynamicBenchmark> dataGradBenchmark,
                                                 std::shared_ptr<detail::AutogradPayload>) {
   if (gradOutput.type() != weight.type())
     throw std::invalid_argument("conv2dBackwardData: gradOutput and weights must have the same type");
@@ -195,8 +250,9 @@ Tensor HipAutogradExtension::conv2dBackwardData(const Tensor& gradOutput, const 
   const size_t wsBytes = flhip_conv2d_workspace_bytes(&d, FLHIP_CONV_BWD_DATA);
   Tensor ws = workspace(wsBytes);
   DevicePtr gp(gradOutput), wp(weight), op(gradInput), wsp(ws);
-  check(flhip_conv2d_bwd_data(&d, gp.get(), wp.get(), op.get(), wsp.get(), wsBytes,
-                              hipBackendStream()));
+  runPlanned(dataGradBenchmark, d, FLHIP_CONV_BWD_DATA, [&](int plan) {
+    return flhip_conv2d_bwd_data_plan(&d, gp.get(), wp.get(), op.get(), wsp.get(), wsBytes, plan, hipBackendStream());
+  }, &check);
   // event: inputs {gradOutput, weights}, outputs {gradInput}, ints as conv2d
   if (scope.on()) scope.done({gradOutput, weight}, {gradInput}, {sx, sy, px, py, dx, dy, groups});
   return gradInput;
@@ -232,7 +288,7 @@ Tensor HipAutogradExtension::conv2dBackwardDataAdd(const Tensor& gradOutput, con
 std::pair<Tensor, Tensor> HipAutogradExtension::conv2dBackwardFilterBias(
     const Tensor& gradOutput, const Tensor& input, const Tensor& weights, const Tensor& bias,
     const int sx, const int sy, const int px, const int py, const int dx, const int dy,
-    const int groups, std::shared_ptr<DynamicBenchmark>, std::shared_ptr<DynamicBenchmark>,
+    const int groups, std::shared_ptr<DynamicBenchmark> filterBench, std::shared_ptr<DynamicBenchmark>,
     std::shared_ptr<detail::AutogradPayload> autogradPayload) {
   if (gradOutput.type() != input.type())
     throw std::invalid_argument("conv2dBackwardFilterBias: gradOutput and input must have the same type");
@@ -267,10 +323,12 @@ std::pair<Tensor, Tensor> HipAutogradExtension::conv2dBackwardFilterBias(
                                           hipBackendStream());
     if (rc != FLHIP_OK && rc != FLHIP_INVALID_ARGUMENT) check(rc);
   }
+  // (the bias gradient comes out of the same pass: the bias benchmark of the reference's closure has nothing to choose)
   if (rc != FLHIP_OK)
-    check(flhip_conv2d_bwd_filter(&d, xp.get(), gp.get(), static_cast<float*>(dwp.get()),
-                                  static_cast<float*>(dbp.get()), wsp.get(), wsBytes,
-                                  hipBackendStream()));
+    runPlanned(filterBench, d, FLHIP_CONV_BWD_FILTER, [&](int plan) {
+      return flhip_conv2d_bwd_filter_plan(&d, xp.get(), gp.get(), static_cast<float*>(dwp.get()),
+                                          static_cast<float*>(dbp.get()), wsp.get(), wsBytes, plan, hipBackendStream());
+    }, &check);
   // event: inputs {gradOutput, input}, outputs {gradWeights, gradBias (may be empty)}, ints as conv2d
   if (scope.on()) scope.done({gradOutput, input}, {gradWeights, gradBias}, {sx, sy, px, py, dx, dy, groups});
   return {gradWeights, gradBias};

@@ -11,6 +11,13 @@ class HipAutogradExtension : public AutogradExtension {
  public:
   // refuses to run on a libflhip whose descriptor layouts differ from the header this class was compiled with
   HipAutogradExtension();
+  // One benchmark of a backward pass of one convolution: its options are "the default rule" and every kernel
+  // family of libflhip's backward passes (flhip_conv2d_plan_count), each timed kPlanBenchCount times on the first
+  // calls made in benchmark mode; the fastest then runs every later call with the same geometry (a call with
+  // another geometry starts the timings again).  The cuDNN peer offers its three kernel modes the same way
+  // (cudnn/CudnnAutogradExtension.cpp:17-25).
+  std::shared_ptr<DynamicBenchmark> createBenchmarkOptions() override;
+  static constexpr int kPlanBenchCount = 3;
   // f32 and the private bf16 tag; the oneDNN extension supports everything but f16
   // (onednn/OneDnnAutogradExtension.cpp:12-16), the cuDNN one f16/f32/f64.
   bool isDataTypeSupported(const dtype& type) const override;

@@ -1,8 +1,10 @@
 #include "HipTensor.h"
+#include "DynamicBenchmark.h"
 #include "OpObserver.h"
 
 #include <hip/hip_runtime.h>
 
+#include <chrono>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -99,6 +101,29 @@ void setOpObserver(OpObserver* observer) { g_observer = observer; }
 }  // namespace detail
 
 // ---- StepProfiler -------------------------------------------------------------------
+// ---- DynamicBenchmark --------------------------------------------------------------------
+namespace {
+bool g_benchmarkMode = false;   // flashlight/fl/common/DynamicBenchmark.cpp:13: off by default
+}
+void DynamicBenchmark::setBenchmarkMode(bool mode) { g_benchmarkMode = mode; }
+bool DynamicBenchmark::getBenchmarkMode() { return g_benchmarkMode; }
+
+// flashlight/fl/common/DynamicBenchmark.cpp:15-42: wait for the device, time the function on the host clock until
+// the device has finished what it enqueued
+void DynamicBenchmark::audit(const std::function<void()>& function, bool incrementCount) {
+  if (!g_benchmarkMode || options_->timingsComplete()) {
+    function();
+    return;
+  }
+  sync();
+  const auto t0 = std::chrono::steady_clock::now();
+  function();
+  sync();
+  const double seconds = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+  // (the function may have marked its option unusable: then there is nothing left to add to)
+  if (!options_->timingsComplete()) options_->accumulateTimeToCurrentOption(seconds, incrementCount);
+}
+
 struct StepProfiler::Impl {
   struct Span {
     std::string op;

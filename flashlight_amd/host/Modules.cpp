@@ -201,9 +201,9 @@ Variable Conv2D::forward(const Variable& input) {
   if (!(px >= 0 && py >= 0)) throw std::invalid_argument("invalid padding for Conv2D");
   if (bias_)
     return conv2d(input, params_[0].astype(input.type()), params_[1].astype(input.type()), xStride_,
-                  yStride_, px, py, xDilation_, yDilation_, groups_);
+                  yStride_, px, py, xDilation_, yDilation_, groups_, benchmarks_);
   return conv2d(input, params_[0].astype(input.type()), xStride_, yStride_, px, py, xDilation_,
-                yDilation_, groups_);
+                yDilation_, groups_, benchmarks_);
 }
 
 namespace {

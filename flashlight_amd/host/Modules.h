@@ -146,6 +146,8 @@ class Conv2D : public UnaryModule {
   int nIn_, nOut_, xFilter_, yFilter_, xStride_, yStride_, xPad_, yPad_, xDilation_, yDilation_;
   bool bias_;
   int groups_;
+  // the kernel-choice benchmarks of this layer's backward passes (flashlight/fl/nn/modules/Conv2D.h:206)
+  std::shared_ptr<detail::ConvBenchmarks> benchmarks_ = std::make_shared<detail::ConvBenchmarks>();
 };
 
 // flashlight/fl/nn/modules/Pool2D.cpp:19-52

@@ -67,6 +67,6 @@ enum class PaddingMode { SAME = -1 };
 enum class TensorBackendType { Stub, Tensor, ArrayFire, OneDnn, Jit, Hip };
 enum class TensorExtensionType { Generic, Autograd, Vision, JitOptimizer };
 
-class DynamicBenchmark;  // passed through the boundary, never used by this backend
+class DynamicBenchmark;  // DynamicBenchmark.h
 
 }  // namespace fl

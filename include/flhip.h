@@ -36,7 +36,8 @@ extern "C" {
 enum {
   FLHIP_OK = 0,
   FLHIP_INVALID_ARGUMENT = 1,
-  FLHIP_RUNTIME_ERROR = 2
+  FLHIP_RUNTIME_ERROR = 2,
+  FLHIP_DECLINED = 3     /* only from the *_plan entry points: that kernel family does not take the geometry */
 };
 
 /* Storage type of activations.  Reductions and accumulators are always fp32.
@@ -108,7 +109,7 @@ const char* flhip_last_error(void);
  * refuse to run when flhip_version() / 100 differs from FLHIP_VERSION / 100 (a layout change).
  * 200: flhip_rnn_desc gained dropout, seed_lo, seed_hi; flhip_bn_workspace_bytes never returns less
  * than 32 bytes per feature. */
-#define FLHIP_VERSION 201
+#define FLHIP_VERSION 202
 int flhip_version(void);
 const char* flhip_arch(void);
 
@@ -198,6 +199,23 @@ int flhip_conv2d_bwd_filter_gathered(const flhip_conv_desc* d, const void* gathe
 int flhip_conv2d_bwd_filter_static(const flhip_conv_desc* d, const void* x,
                                    const void* dy, float* dw, float* db,
                                    void* stream);
+
+/* Kernel choice for the two backward passes, measured instead of ruled: what the reference reaches through
+ * AutogradExtension::createBenchmarkOptions (AutogradExtension.h:53-55; the options object its caller closure makes
+ * per pass, flashlight/fl/autograd/Functions.cpp:1372-1388, and that cudnn/Conv2D.cpp:467-520, 654-707 audits).
+ * A pass has flhip_conv2d_plan_count(pass) kernel families ("plans", numbered in the order of the default rule;
+ * flhip_conv2d_plan_name gives a family's description, NULL for numbers outside the list).  The *_plan entry
+ * points are flhip_conv2d_bwd_data / flhip_conv2d_bwd_filter with one more argument: plan < 0 runs the default
+ * rule (identical to the entry points above), plan >= 0 runs that family alone, whatever the rules and
+ * switches say, or returns FLHIP_DECLINED without launching anything when the family does not take the
+ * geometry or storage type.  Workspace as for the entry points above (their size covers every plan).  Every
+ * plan meets the stated tolerances; results of different plans differ in summation order only. */
+int flhip_conv2d_plan_count(int pass);
+const char* flhip_conv2d_plan_name(int pass, int plan);
+int flhip_conv2d_bwd_data_plan(const flhip_conv_desc* d, const void* dy, const void* w, void* dx, void* ws,
+                               size_t ws_bytes, int plan, void* stream);
+int flhip_conv2d_bwd_filter_plan(const flhip_conv_desc* d, const void* x, const void* dy, float* dw, float* db,
+                                 void* ws, size_t ws_bytes, int plan, void* stream);
 
 /* AutogradExtension::pool2d (AutogradExtension.h:71-80; oneDNN peer
  * onednn/Pool2D.cpp:78-176).  For FLHIP_POOL_MAX with argmax != NULL the kernel

@@ -21,6 +21,7 @@
 #include <map>
 #include <random>
 #include <string>
+#include <unordered_set>
 #include <vector>
 
 #include "Functions.h"
@@ -28,6 +29,8 @@
 #include "SequentialBuilder.h"
 #include "HipAutogradExtension.h"
 #include "OpObserver.h"
+#include "DynamicBenchmark.h"
+#include "flhip.h"
 #include "flref.h"
 
 using namespace fl;
@@ -89,7 +92,7 @@ static void testRegistration() {
   CHECK(&e == &getAutogradExtension(TensorBackendType::Hip));       // one instance per backend
   CHECK(e.isDataTypeSupported(dtype::f32) && e.isDataTypeSupported(dtype::bf16));
   CHECK(!e.isDataTypeSupported(dtype::f16) && !e.isDataTypeSupported(dtype::f64));
-  CHECK(e.createBenchmarkOptions() == nullptr);
+  CHECK(e.createBenchmarkOptions() != nullptr && e.createBenchmarkOptions() != e.createBenchmarkOptions());   // one per pass and layer
   // a second registration for the same backend is ignored (TensorExtension.cpp:27-29)
   CHECK(!detail::registerAutogradExtension(TensorBackendType::Hip, [] {
     return std::unique_ptr<AutogradExtension>(new HipAutogradExtension());
@@ -1096,6 +1099,109 @@ static void onCrash(int sig) {
   _exit(128 + sig);
 }
 
+// Kernel choice by measurement.  The options object and audit() with the checks of the reference's own tests
+// (flashlight/fl/test/common/DynamicBenchmarkTest.cpp:30-118: options tried in order, no count without increment, the
+// fastest option wins, host time between two audits of one option does not count); then a Conv2D layer in
+// benchmark mode: every plan (the default rule and all kernel families, the declined ones struck out) is tried
+// kPlanBenchCount times per pass, the winner runs from then on and gives the same bits on every later call, the
+// gradients of every call during and after the timings match the CPU checker, another batch size starts the timings
+// again, and with the mode off nothing is timed.
+static void testDynamicBenchmark() {
+  std::printf("kernel choice by measurement (createBenchmarkOptions)\n");
+  DynamicBenchmark::setBenchmarkMode(true);
+  {
+    const size_t maxCount = 5;
+    auto options = std::make_shared<DynamicBenchmarkOptions<int>>(std::vector<int>{1, 2, 3, 4, 5}, maxCount);
+    CHECK(!options->timingsComplete() && options->currentOption() == 1);
+    for (size_t i = 0; i < maxCount * 5; ++i) options->accumulateTimeToCurrentOption(1);
+    CHECK(options->timingsComplete() && options->currentOption() == 1);
+    CHECK(throws<std::invalid_argument>([&] { options->accumulateTimeToCurrentOption(1); }));
+    options->reset();
+    CHECK(!options->timingsComplete());
+    const int before = options->currentOption();
+    options->accumulateTimeToCurrentOption(3, false);
+    options->accumulateTimeToCurrentOption(4, false);
+    CHECK(before == options->currentOption());
+    CHECK(throws<std::invalid_argument>([] { DynamicBenchmarkOptions<int>(std::vector<int>{}, 3); }));
+  }
+  {
+    const size_t maxCount = 5;
+    auto options = std::make_shared<DynamicBenchmarkOptions<int>>(std::unordered_set<int>{1, 2, 3, 4, 5}, maxCount);
+    for (size_t i = 0; i < maxCount * 5; ++i) {
+      if (options->currentOption() == 4) {
+        options->accumulateTimeToCurrentOption(1);
+      } else {
+        options->accumulateTimeToCurrentOption(10 * (i + 1), false);
+        options->accumulateTimeToCurrentOption(10 * (i + 1));
+      }
+    }
+    CHECK(options->timingsComplete() && options->currentOption() == 4);
+  }
+  {
+    // device work of three sizes: the smallest wins; host time between two audits of one option does not count
+    const std::vector<int> sizes{1 << 22, 1 << 12, 1 << 24};
+    auto options = std::make_shared<DynamicBenchmarkOptions<int>>(sizes, 4);
+    auto bench = std::make_shared<DynamicBenchmark>(options);
+    for (size_t i = 0; i < 4 * sizes.size(); ++i) {
+      const int n = bench->getOptions<DynamicBenchmarkOptions<int>>()->currentOption();
+      auto work = [&] {
+        for (int r = 0; r < 4; ++r) Tensor::full({n}, 1.0, dtype::f32);
+      };
+      bench->audit(work, false);
+      usleep(n == 1 << 12 ? 20000 : 1000);
+      bench->audit(work);
+    }
+    CHECK(options->timingsComplete() && options->currentOption() == 1 << 12);
+    // mode off: the function runs, nothing is recorded
+    options->reset();
+    DynamicBenchmark::setBenchmarkMode(false);
+    int ran = 0;
+    bench->audit([&] { ++ran; });
+    CHECK(ran == 1 && options->countOf(0) == 0 && !DynamicBenchmark::getBenchmarkMode());
+    DynamicBenchmark::setBenchmarkMode(true);
+  }
+  for (const dtype type : {dtype::f32, dtype::bf16}) {
+    const bool lo = type == dtype::bf16;
+    const int W = 14, H = 14, C = 64, K = 64;
+    setSeed(41);
+    Conv2D conv(C, K, 3, 3, 1, 1, PaddingMode::SAME, PaddingMode::SAME, 1, 1, true);
+    const auto w = hostOf(conv.param(0)), b = hostOf(conv.param(1));
+    std::vector<float> wr = w;
+    if (lo)
+      for (auto& v : wr) v = bf16round(v);
+    const int nplans = 1 + flhip_conv2d_plan_count(FLHIP_CONV_BWD_DATA);
+    const int timed = nplans * HipAutogradExtension::kPlanBenchCount;
+    std::vector<float> keptDx, keptDw;
+    for (const int N : {4, 6}) {                    // the second batch size starts the timings again
+      auto x = randn((size_t)N * C * H * W, 43 + N), dy = randn((size_t)N * K * H * W, 47 + N);
+      if (lo) {
+        for (auto& v : x) v = bf16round(v);
+        for (auto& v : dy) v = bf16round(v);
+      }
+      flref_conv d{N, C, H, W, K, 3, 3, 1, 1, 1, 1, 1, 1, 1};
+      std::vector<float> dxRef(x.size()), dwRef(w.size()), dbRef(K);
+      flref_conv2d_bwd_data(&d, dy.data(), wr.data(), dxRef.data());
+      flref_conv2d_bwd_filter(&d, x.data(), dy.data(), dwRef.data(), dbRef.data());
+      for (int it = 0; it < timed + 3; ++it) {
+        Variable in(Tensor::fromVector({W, H, C, N}, x).astype(type), true);
+        conv.zeroGrad();
+        Variable out = conv.forward(in);
+        out.backward(Variable(Tensor::fromVector(out.shape(), dy).astype(type), false));
+        const auto dx = hostOf(in.grad()), dw = hostOf(conv.param(0).grad()), db = hostOf(conv.param(1).grad());
+        CHECK(relL2(dx, dxRef) <= (lo ? 4e-3 : 1e-4));
+        CHECK(relL2(dw, dwRef) <= 1e-4 && relL2(db, dbRef) <= 1e-4);
+        if (it == timed) {
+          keptDx = dx;
+          keptDw = dw;
+        } else if (it > timed) {
+          CHECK(dx == keptDx && dw == keptDw);       // the cached choice: the same kernel, the same bits
+        }
+      }
+    }
+  }
+  DynamicBenchmark::setBenchmarkMode(false);
+}
+
 int main() {
   std::setvbuf(stdout, nullptr, _IONBF, 0);
   std::signal(SIGSEGV, onCrash);
@@ -1124,6 +1230,7 @@ int main() {
     testArchBuilder();
     testModuleShapesAndBatching();
     testInit();
+    testDynamicBenchmark();
     fl::sync();
   } catch (const std::exception& e) {
     std::printf("unexpected exception: %s\n", e.what());

@@ -115,3 +115,15 @@ def test_bn_view_and_same_padding():
     assert derive_padding(28, 5, 1, -1) == 2
     assert derive_padding(112, 3, 2, -1) == 1
     assert derive_padding(9, 3, 1, 4) == 4
+
+
+def test_plan_lists():
+    """The kernel families of the backward passes have names; the forward pass has no plans."""
+    lib = capi.lib()
+    for pas in (capi.CONV_BWD_DATA, capi.CONV_BWD_FILTER):
+        n = lib.flhip_conv2d_plan_count(pas)
+        assert n >= 2
+        names = [lib.flhip_conv2d_plan_name(pas, i) for i in range(n)]
+        assert all(names) and len(set(names)) == n
+        assert lib.flhip_conv2d_plan_name(pas, n) is None and lib.flhip_conv2d_plan_name(pas, -1) is None
+    assert lib.flhip_conv2d_plan_count(capi.CONV_FWD) == 0

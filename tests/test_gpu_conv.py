@@ -684,3 +684,84 @@ def test_full_size_properties(shape, dtype):
     want = xp[:, :nd, kh:kh + (OH - 1) * st[0] + 1:st[0], kw_:kw_ + (OW - 1) * st[1] + 1:st[1]]
     assert torch.equal(yi[:, :nd], want)
     assert not yi[:, nd:].any()
+
+
+# The backward passes with the kernel family named by the caller (flhip_conv2d_bwd_*_plan): every family either
+# declines a geometry (nothing is written) or produces the result within the stated tolerance; plan -1 is the
+# default entry point bit for bit; numbers outside the list are refused.
+PLAN_CASES = [
+    ((4, 64, 14, 14), (64, 64, 3, 3), (1, 1), (1, 1)),
+    ((2, 64, 56, 56), (64, 64, 3, 3), (1, 1), (1, 1)),
+    ((3, 128, 14, 14), (256, 128, 1, 1), (1, 1), (0, 0)),
+    ((2, 32, 15, 15), (48, 32, 3, 3), (2, 2), (1, 1)),
+    ((2, 3, 32, 32), (64, 3, 7, 7), (2, 2), (3, 3)),
+    ((2, 80, 1, 100), (250, 80, 1, 21), (1, 1), (0, 10)),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", PLAN_CASES)
+def test_backward_passes_by_plan(shape, dtype):
+    import ctypes as C
+    from flashlight_amd import capi
+    L = capi.lib()
+    xs, ws_, st, pd = shape
+    lo = dtype == torch.bfloat16
+    rng = np.random.default_rng(71)
+    x = rng.standard_normal(xs).astype(np.float32)
+    w = (rng.standard_normal(ws_) / np.sqrt(ws_[1] * ws_[2] * ws_[3])).astype(np.float32)
+    if lo:
+        x, w = bf16_round(x), bf16_round(w)
+    d = flref.conv_desc(xs, ws_, st, pd, (1, 1), 1)
+    y_shape = flref.conv2d_fwd(d, x, w, None).shape
+    dy = rng.standard_normal(y_shape).astype(np.float32)
+    if lo:
+        dy = bf16_round(dy)
+    dx_ref = flref.conv2d_bwd_data(d, dy, w)
+    dw_ref, db_ref = flref.conv2d_bwd_filter(d, x, dy)
+    xd, wd, dyd = dev(x, dtype), dev(w, dtype), dev(dy, dtype)
+    cd = capi.ConvDesc(xs[0], xs[1], xs[2], xs[3], ws_[0], ws_[2], ws_[3], st[0], st[1], pd[0], pd[1], 1, 1, 1,
+                       capi.BF16 if lo else capi.F32)
+    S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: C.c_void_p(t.data_ptr())
+    nd = L.flhip_conv2d_plan_count(capi.CONV_BWD_DATA)
+    assert nd == L.flhip_conv2d_plan_count(capi.CONV_BWD_FILTER) >= 2 and L.flhip_conv2d_plan_count(capi.CONV_FWD) == 0
+    ran = {capi.CONV_BWD_DATA: [], capi.CONV_BWD_FILTER: []}
+    for pas in (capi.CONV_BWD_DATA, capi.CONV_BWD_FILTER):
+        nws = L.flhip_conv2d_workspace_bytes(C.byref(cd), pas)
+        ws = torch.empty(max(nws, 16), dtype=torch.uint8, device="cuda")
+        results = {}
+        for plan in range(-1, nd):
+            if pas == capi.CONV_BWD_DATA:
+                out = torch.full(xs, 7.0, device="cuda", dtype=dtype)
+                rc = L.flhip_conv2d_bwd_data_plan(C.byref(cd), P(dyd), P(wd), P(out), P(ws), nws, plan, S)
+                outs = (out,)
+            else:
+                dw = torch.full(ws_, 7.0, device="cuda")
+                db = torch.full((ws_[0],), 7.0, device="cuda")
+                rc = L.flhip_conv2d_bwd_filter_plan(C.byref(cd), P(xd), P(dyd), P(dw), P(db), P(ws), nws, plan, S)
+                outs = (dw, db)
+            torch.cuda.synchronize()
+            if rc == capi.DECLINED:
+                assert plan >= 0 and all(bool((o == 7.0).all()) for o in outs), plan     # nothing was launched
+                continue
+            capi.check(rc)
+            assert L.flhip_conv2d_plan_name(pas, plan) is not None or plan < 0
+            ran[pas].append(plan)
+            results[plan] = outs
+            if pas == capi.CONV_BWD_DATA:
+                assert rel_l2(host(out), dx_ref) <= (4e-3 if lo else 1e-4), (plan, rel_l2(host(out), dx_ref))
+            else:
+                assert rel_l2(host(dw), dw_ref) <= 1e-4 and rel_l2(host(db), db_ref) <= 1e-4, plan
+        # the direct kernels take everything; the default rule is one of the plans that ran
+        assert nd - 1 in ran[pas] and len(ran[pas]) >= 3
+        assert any(all(torch.equal(a, b) for a, b in zip(results[-1], results[q])) for q in ran[pas] if q >= 0)
+    # plan -1 = the entry points without a plan
+    dx0 = fa.conv2d_backward_data(dyd, xs, wd, sx=st[1], sy=st[0], px=pd[1], py=pd[0])
+    out = torch.empty(xs, device="cuda", dtype=dtype)
+    nws = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_BWD_DATA)
+    ws = torch.empty(max(nws, 16), dtype=torch.uint8, device="cuda")
+    capi.check(L.flhip_conv2d_bwd_data_plan(C.byref(cd), P(dyd), P(wd), P(out), P(ws), nws, -1, S))
+    assert torch.equal(out, dx0)
+    assert L.flhip_conv2d_bwd_data_plan(C.byref(cd), P(dyd), P(wd), P(out), P(ws), nws, nd, S) == capi.INVALID_ARGUMENT
+    assert L.flhip_conv2d_plan_name(capi.CONV_BWD_DATA, nd) is None
