@@ -6,7 +6,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libflhip.so")
 
 OK, INVALID_ARGUMENT, RUNTIME_ERROR, DECLINED = 0, 1, 2, 3
-F32, BF16 = 0, 1
+F32, BF16, F16 = 0, 1, 2
 CONV_FWD, CONV_BWD_DATA, CONV_BWD_FILTER = 0, 1, 2
 STATIC_SCRATCH_BYTES = 40 << 20      # FLHIP_STATIC_SCRATCH_BYTES
 

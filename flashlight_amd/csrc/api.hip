@@ -232,14 +232,13 @@ extern "C" int flhip_convert(const void* src, int src_dtype, void* dst, int dst_
   if (blocks > 16384) blocks = 16384;
   const dim3 grid((unsigned)blocks), block(256);
   hipStream_t s = as_stream(stream);
-  if (src_dtype == FLHIP_F32 && dst_dtype == FLHIP_F32)
-    hipLaunchKernelGGL((convert_kernel<float, float>), grid, block, 0, s, (const float*)src, (float*)dst, n);
-  else if (src_dtype == FLHIP_F32)
-    hipLaunchKernelGGL((convert_kernel<float, bf16_t>), grid, block, 0, s, (const float*)src, (bf16_t*)dst, n);
-  else if (dst_dtype == FLHIP_F32)
-    hipLaunchKernelGGL((convert_kernel<bf16_t, float>), grid, block, 0, s, (const bf16_t*)src, (float*)dst, n);
-  else
-    hipLaunchKernelGGL((convert_kernel<bf16_t, bf16_t>), grid, block, 0, s, (const bf16_t*)src, (bf16_t*)dst, n);
+  by_dtype(src_dtype, [&](auto* sp) {
+    by_dtype(dst_dtype, [&](auto* dp) {
+      using S = FLHIP_T_OF(sp);
+      using D = FLHIP_T_OF(dp);
+      hipLaunchKernelGGL((convert_kernel<S, D>), grid, block, 0, s, static_cast<const S*>(src), static_cast<D*>(dst), n);
+    });
+  });
   return check_launch("convert");
 }
 
@@ -256,14 +255,11 @@ extern "C" int flhip_convert_many(const void* const* src, void* const* dst, cons
     if (a.count == 0) return;
     a.first[a.count] = (unsigned)pieces;
     const dim3 grid((unsigned)pieces), block(256);
-    if (src_dtype == FLHIP_F32 && dst_dtype == FLHIP_F32)
-      hipLaunchKernelGGL((convert_many_kernel<float, float>), grid, block, 0, s, a);
-    else if (src_dtype == FLHIP_F32)
-      hipLaunchKernelGGL((convert_many_kernel<float, bf16_t>), grid, block, 0, s, a);
-    else if (dst_dtype == FLHIP_F32)
-      hipLaunchKernelGGL((convert_many_kernel<bf16_t, float>), grid, block, 0, s, a);
-    else
-      hipLaunchKernelGGL((convert_many_kernel<bf16_t, bf16_t>), grid, block, 0, s, a);
+    by_dtype(src_dtype, [&](auto* sp) {
+      by_dtype(dst_dtype, [&](auto* dp) {
+        hipLaunchKernelGGL((convert_many_kernel<FLHIP_T_OF(sp), FLHIP_T_OF(dp)>), grid, block, 0, s, a);
+      });
+    });
     a = ConvertMany{};
     pieces = 0;
   };
@@ -311,12 +307,11 @@ extern "C" int flhip_fill(void* dst, double value, size_t n, int dtype, void* st
   FLHIP_REQUIRE(dst, "fill: null pointer");
   size_t blocks = (n + 255) / 256;
   if (blocks > 16384) blocks = 16384;
-  if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((fill_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), (float*)dst,
+  by_dtype(dtype, [&](auto* t) {
+    using T = FLHIP_T_OF(t);
+    hipLaunchKernelGGL((fill_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), static_cast<T*>(dst),
                        (float)value, n);
-  else
-    hipLaunchKernelGGL((fill_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), (bf16_t*)dst,
-                       (float)value, n);
+  });
   return check_launch("fill");
 }
 
@@ -325,9 +320,9 @@ extern "C" int flhip_add(const void* a, const void* b, void* out, size_t n, int 
   FLHIP_REQUIRE(dtype_ok(dtype), "add: unknown dtype");
   if (n == 0) return FLHIP_OK;
   FLHIP_REQUIRE(a && b && out, "add: null pointer");
-  if (dtype == FLHIP_F32)
-    launch_elementwise((const float*)a, (const float*)b, (float*)out, n, OpAdd{}, as_stream(stream));
-  else
-    launch_elementwise((const bf16_t*)a, (const bf16_t*)b, (bf16_t*)out, n, OpAdd{}, as_stream(stream));
+  by_dtype(dtype, [&](auto* t) {
+    using T = FLHIP_T_OF(t);
+    launch_elementwise(static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(out), n, OpAdd{}, as_stream(stream));
+  });
   return check_launch("add");
 }

@@ -234,6 +234,7 @@ struct BnFuseBwd {
 // value as it reads back from storage of type T
 __device__ __forceinline__ float rounded(float v, const float*) { return v; }
 __device__ __forceinline__ float rounded(float v, const bf16_t*) { return bf16_to_f32(f32_to_bf16(v)); }
+__device__ __forceinline__ float rounded(float v, const f16_t*) { return f16_to_f32(f32_to_f16(v)); }
 // the ReLU mask of the vector at element offset `off` as values that compare like y: from the mask bytes
 // when the caller has them (4-element vectors only), else from y itself
 template <int VEC, bool MASK, typename T>
@@ -505,6 +506,10 @@ __device__ __forceinline__ float4 buf_ld4_stream(__amdgpu_buffer_rsrc_t r, int b
   return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u),
                      __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
 }
+__device__ __forceinline__ float4 buf_ld4_stream(__amdgpu_buffer_rsrc_t r, int byte_off, const f16_t*) {
+  const uintx2_t v = __builtin_amdgcn_raw_buffer_load_b64(r, byte_off, 0, 2);
+  return make_float4(f16lo(v.x), f16hi(v.x), f16lo(v.y), f16hi(v.y));
+}
 
 // the same loads with the widening left for later: a vector that waits in registers stays at its storage size
 template <typename T>
@@ -517,11 +522,18 @@ template <>
 struct Raw4<bf16_t> {
   uintx2_t v;
 };
+template <>
+struct Raw4<f16_t> {
+  uintx2_t v;
+};
 __device__ __forceinline__ Raw4<float> buf_ld4_raw(__amdgpu_buffer_rsrc_t r, int byte_off, const float*) {
   return Raw4<float>{__builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 2)};
 }
 __device__ __forceinline__ Raw4<bf16_t> buf_ld4_raw(__amdgpu_buffer_rsrc_t r, int byte_off, const bf16_t*) {
   return Raw4<bf16_t>{__builtin_amdgcn_raw_buffer_load_b64(r, byte_off, 0, 2)};
+}
+__device__ __forceinline__ Raw4<f16_t> buf_ld4_raw(__amdgpu_buffer_rsrc_t r, int byte_off, const f16_t*) {
+  return Raw4<f16_t>{__builtin_amdgcn_raw_buffer_load_b64(r, byte_off, 0, 2)};
 }
 __device__ __forceinline__ float4 widen(const Raw4<float>& w) {
   return make_float4(__uint_as_float(w.v.x), __uint_as_float(w.v.y), __uint_as_float(w.v.z), __uint_as_float(w.v.w));
@@ -529,6 +541,9 @@ __device__ __forceinline__ float4 widen(const Raw4<float>& w) {
 __device__ __forceinline__ float4 widen(const Raw4<bf16_t>& w) {
   return make_float4(__uint_as_float(w.v.x << 16), __uint_as_float(w.v.x & 0xffff0000u),
                      __uint_as_float(w.v.y << 16), __uint_as_float(w.v.y & 0xffff0000u));
+}
+__device__ __forceinline__ float4 widen(const Raw4<f16_t>& w) {
+  return make_float4(f16lo(w.v.x), f16hi(w.v.x), f16lo(w.v.y), f16hi(w.v.y));
 }
 
 // 16-byte (float) / 8-byte (bf16) buffer store of four values, streaming
@@ -540,6 +555,10 @@ __device__ __forceinline__ void buf_st4(__amdgpu_buffer_rsrc_t r, int byte_off, 
 __device__ __forceinline__ void buf_st4(__amdgpu_buffer_rsrc_t r, int byte_off, float4 v, bf16_t*) {
   const uintx2_t t = {(uint32_t)f32_to_bf16(v.x) | ((uint32_t)f32_to_bf16(v.y) << 16),
                       (uint32_t)f32_to_bf16(v.z) | ((uint32_t)f32_to_bf16(v.w) << 16)};
+  __builtin_amdgcn_raw_buffer_store_b64(t, r, byte_off, 0, 2);
+}
+__device__ __forceinline__ void buf_st4(__amdgpu_buffer_rsrc_t r, int byte_off, float4 v, f16_t*) {
+  const uintx2_t t = {pack_f16(v.x, v.y), pack_f16(v.z, v.w)};
   __builtin_amdgcn_raw_buffer_store_b64(t, r, byte_off, 0, 2);
 }
 
@@ -919,6 +938,9 @@ __device__ __forceinline__ void buf_st(__amdgpu_buffer_rsrc_t r, int byte_off, f
 }
 __device__ __forceinline__ void buf_st(__amdgpu_buffer_rsrc_t r, int byte_off, float v, bf16_t*) {
   __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16(v), r, byte_off, 0, 0);
+}
+__device__ __forceinline__ void buf_st(__amdgpu_buffer_rsrc_t r, int byte_off, float v, f16_t*) {
+  __builtin_amdgcn_raw_buffer_store_b16(f32_to_f16(v).bits, r, byte_off, 0, 0);
 }
 
 // byte offsets of this thread's elements e = tid + THREADS*k of feature blockIdx.x;
@@ -1361,7 +1383,7 @@ static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws
   const T* xp = static_cast<const T*>(x);
   T* yp = static_cast<T*>(y);
   constexpr int F1 = FUSE == 2 ? 1 : FUSE;   // element-wise kernels: no mask-byte form (never asked for: vec == 4 only)
-  if (sizeof(T) == 2) {
+  if (std::is_same<T, bf16_t>::value) {
     const ResPlan r8 = resident8_plan(g, vec, FLHIP_BF16, RES_MIN_C_FWD);
     if (r8.threads)
       return run_train8<FUSE>(g, r8, reinterpret_cast<const bf16_t*>(xp), reinterpret_cast<bf16_t*>(yp), a,
@@ -1419,7 +1441,7 @@ static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void
   const T* dyp = static_cast<const T*>(dy);
   T* dxp = static_cast<T*>(dx);
   constexpr int F1 = FUSE == 2 ? 1 : FUSE;   // element-wise kernels: no mask-byte form (never asked for: vec == 4 only)
-  if (sizeof(T) == 2) {
+  if (std::is_same<T, bf16_t>::value) {
     const ResPlan r8 = resident8_plan(g, vec, FLHIP_BF16, RES_MIN_C_BWD);
     if (r8.threads)
       return run_bwd8<FUSE>(g, r8, reinterpret_cast<const bf16_t*>(xp), reinterpret_cast<const bf16_t*>(dyp),
@@ -1497,9 +1519,10 @@ extern "C" int flhip_bn_fwd_train(const flhip_bn_desc* d, const void* x, const f
   FLHIP_REQUIRE(eps >= 0.0, "bn_fwd_train: epsilon must be non-negative");
   FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_fwd_train: workspace too small");
   const BnTrainArgs a{gamma, beta, save_mean, save_invstd, run_mean, run_var, momentum, eps};
-  return d->dtype == FLHIP_F32
-             ? run_train<float, 0>(g, vec, x, y, static_cast<float*>(ws), a, BnFuseFwd<float>{nullptr, 0, nullptr}, as_stream(stream))
-             : run_train<bf16_t, 0>(g, vec, x, y, static_cast<float*>(ws), a, BnFuseFwd<bf16_t>{nullptr, 0, nullptr}, as_stream(stream));
+  return by_dtype(d->dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    return run_train<T, 0>(g, vec, x, y, static_cast<float*>(ws), a, BnFuseFwd<T>{nullptr, 0, nullptr}, as_stream(stream));
+  });
 }
 
 static int bn_act_fwd_train_impl(const flhip_bn_desc* d, const void* x, const float* gamma,
@@ -1522,14 +1545,13 @@ static int bn_act_fwd_train_impl(const flhip_bn_desc* d, const void* x, const fl
   FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_act_fwd_train: workspace too small");
   const BnTrainArgs a{gamma, beta, save_mean, save_invstd, run_mean, run_var, momentum, eps};
   uint8_t* mk = want_mask ? static_cast<uint8_t*>(mask) : nullptr;
-  const BnFuseFwd<float> f32{static_cast<const float*>(residual), relu, mk};
-  const BnFuseFwd<bf16_t> f16{static_cast<const bf16_t*>(residual), relu, mk};
   float* wsf = static_cast<float*>(ws);
-  if (d->dtype == FLHIP_F32)
-    return mk ? run_train<float, 2>(g, vec, x, y, wsf, a, f32, as_stream(stream))
-              : run_train<float, 1>(g, vec, x, y, wsf, a, f32, as_stream(stream));
-  return mk ? run_train<bf16_t, 2>(g, vec, x, y, wsf, a, f16, as_stream(stream))
-            : run_train<bf16_t, 1>(g, vec, x, y, wsf, a, f16, as_stream(stream));
+  return by_dtype(d->dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    const BnFuseFwd<T> fu{static_cast<const T*>(residual), relu, mk};
+    return mk ? run_train<T, 2>(g, vec, x, y, wsf, a, fu, as_stream(stream))
+              : run_train<T, 1>(g, vec, x, y, wsf, a, fu, as_stream(stream));
+  });
 }
 
 extern "C" int flhip_bn_act_fwd_train(const flhip_bn_desc* d, const void* x, const float* gamma,
@@ -1566,14 +1588,12 @@ extern "C" int flhip_bn_fwd_infer(const flhip_bn_desc* d, const void* x, const f
   const size_t total = (size_t)g.outer * g.C * g.inner;
   size_t blocks = (total + 255) / 256;
   if (blocks > 16384) blocks = 16384;
-  if (d->dtype == FLHIP_F32)
-    hipLaunchKernelGGL((bn_infer_kernel<float>), dim3((unsigned)blocks), dim3(256), 0,
-                       as_stream(stream), g, static_cast<const float*>(x), static_cast<float*>(y),
-                       gamma, beta, run_mean, run_var, (float)eps, total);
-  else
-    hipLaunchKernelGGL((bn_infer_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0,
-                       as_stream(stream), g, static_cast<const bf16_t*>(x),
-                       static_cast<bf16_t*>(y), gamma, beta, run_mean, run_var, (float)eps, total);
+  by_dtype(d->dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((bn_infer_kernel<T>), dim3((unsigned)blocks), dim3(256), 0,
+                       as_stream(stream), g, static_cast<const T*>(x),
+                       static_cast<T*>(y), gamma, beta, run_mean, run_var, (float)eps, total);
+  });
   return check_launch("bn_fwd_infer");
 }
 
@@ -1591,9 +1611,10 @@ extern "C" int flhip_bn_bwd(const flhip_bn_desc* d, const void* x, const void* d
   FLHIP_REQUIRE(save_mean && save_invstd, "bn_bwd: needs the saved statistics of the forward pass");
   FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_bwd: workspace too small");
   const BnBwdArgs a{gamma, save_mean, save_invstd, dgamma, dbeta};
-  return d->dtype == FLHIP_F32
-             ? run_bwd<float, 0>(g, vec, x, dy, dx, static_cast<float*>(ws), a, BnFuseBwd<float>{nullptr, nullptr, nullptr}, as_stream(stream))
-             : run_bwd<bf16_t, 0>(g, vec, x, dy, dx, static_cast<float*>(ws), a, BnFuseBwd<bf16_t>{nullptr, nullptr, nullptr}, as_stream(stream));
+  return by_dtype(d->dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    return run_bwd<T, 0>(g, vec, x, dy, dx, static_cast<float*>(ws), a, BnFuseBwd<T>{nullptr, nullptr, nullptr}, as_stream(stream));
+  });
 }
 
 static int bn_act_bwd_impl(const flhip_bn_desc* d, const void* x, const void* dy, const void* y,
@@ -1610,15 +1631,14 @@ static int bn_act_bwd_impl(const flhip_bn_desc* d, const void* x, const void* dy
   FLHIP_REQUIRE(ws && ws_bytes >= flhip_bn_workspace_bytes(d), "bn_act_bwd: workspace too small");
   const BnBwdArgs a{gamma, save_mean, save_invstd, dgamma, dbeta};
   const uint8_t* mk = static_cast<const uint8_t*>(mask);
-  const BnFuseBwd<float> f32{static_cast<const float*>(y), static_cast<float*>(dresidual), mk};
-  const BnFuseBwd<bf16_t> f16{static_cast<const bf16_t*>(y), static_cast<bf16_t*>(dresidual), mk};
   float* wsf = static_cast<float*>(ws);
   // FUSE = 1: the mask is read from y, 2: from the mask bytes
-  if (d->dtype == FLHIP_F32)
-    return mk ? run_bwd<float, 2>(g, vec, x, dy, dx, wsf, a, f32, as_stream(stream))
-              : run_bwd<float, 1>(g, vec, x, dy, dx, wsf, a, f32, as_stream(stream));
-  return mk ? run_bwd<bf16_t, 2>(g, vec, x, dy, dx, wsf, a, f16, as_stream(stream))
-            : run_bwd<bf16_t, 1>(g, vec, x, dy, dx, wsf, a, f16, as_stream(stream));
+  return by_dtype(d->dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    const BnFuseBwd<T> fu{static_cast<const T*>(y), static_cast<T*>(dresidual), mk};
+    return mk ? run_bwd<T, 2>(g, vec, x, dy, dx, wsf, a, fu, as_stream(stream))
+              : run_bwd<T, 1>(g, vec, x, dy, dx, wsf, a, fu, as_stream(stream));
+  });
 }
 
 extern "C" int flhip_bn_act_bwd(const flhip_bn_desc* d, const void* x, const void* dy, const void* y,

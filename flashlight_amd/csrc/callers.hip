@@ -497,11 +497,10 @@ AffinePlan affine_plan(long long outer, long long mid, long long inner, int scal
 // of slices actually written is ceil(chunks / ceil(chunks / slices)), chunks = ceil(K / 32).
 int gemm_nt(int dtype, const void* A, const void* B, void* C, int M, int N, int K, int slices, hipStream_t s) {
   if (slices < 1 || (slices > 1 && dtype != FLHIP_F32)) return -1;
-  return dtype == FLHIP_F32
-             ? gemm_nt_launch(static_cast<const float*>(A), static_cast<const float*>(B), static_cast<float*>(C), M,
-                              N, K, slices, s)
-             : gemm_nt_launch(static_cast<const bf16_t*>(A), static_cast<const bf16_t*>(B),
-                              static_cast<bf16_t*>(C), M, N, K, slices, s);
+  return by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    return gemm_nt_launch(static_cast<const T*>(A), static_cast<const T*>(B), static_cast<T*>(C), M, N, K, slices, s);
+  });
 }
 
 }  // namespace flhip
@@ -512,10 +511,10 @@ extern "C" int flhip_relu_fwd(const void* x, void* y, size_t n, int dtype, void*
   FLHIP_REQUIRE((x && y) || n == 0, "relu: null argument");
   FLHIP_REQUIRE(dtype_ok(dtype), "relu: unknown dtype");
   if (n == 0) return FLHIP_OK;
-  if (dtype == FLHIP_F32)
-    launch_elementwise((const float*)x, (const float*)nullptr, (float*)y, n, OpRelu{}, as_stream(stream));
-  else
-    launch_elementwise((const bf16_t*)x, (const bf16_t*)nullptr, (bf16_t*)y, n, OpRelu{}, as_stream(stream));
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    launch_elementwise((const T*)x, (const T*)nullptr, (T*)y, n, OpRelu{}, as_stream(stream));
+  });
   return check_launch("relu");
 }
 
@@ -524,10 +523,10 @@ extern "C" int flhip_relu_bwd(const void* dy, const void* x, void* dx, size_t n,
   FLHIP_REQUIRE((dy && x && dx) || n == 0, "relu_bwd: null argument");
   FLHIP_REQUIRE(dtype_ok(dtype), "relu_bwd: unknown dtype");
   if (n == 0) return FLHIP_OK;
-  if (dtype == FLHIP_F32)
-    launch_elementwise((const float*)dy, (const float*)x, (float*)dx, n, OpReluBwd{}, as_stream(stream));
-  else
-    launch_elementwise((const bf16_t*)dy, (const bf16_t*)x, (bf16_t*)dx, n, OpReluBwd{}, as_stream(stream));
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    launch_elementwise((const T*)dy, (const T*)x, (T*)dx, n, OpReluBwd{}, as_stream(stream));
+  });
   return check_launch("relu_bwd");
 }
 
@@ -542,23 +541,21 @@ extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, in
     hipStream_t s = as_stream(stream);
     if (!trans_a) {
       const dim3 grid((unsigned)((M + 63) / 64), (unsigned)((N + SK_NT - 1) / SK_NT));
-      if (dtype == FLHIP_F32)
-        hipLaunchKernelGGL((matmul_nn_skinny<float>), grid, dim3(1024), 0, s, (const float*)A, (const float*)B,
-                           (float*)C, M, N, K, bias_rows);
-      else
-        hipLaunchKernelGGL((matmul_nn_skinny<bf16_t>), grid, dim3(1024), 0, s, (const bf16_t*)A, (const bf16_t*)B,
-                           (bf16_t*)C, M, N, K, bias_rows);
+      by_dtype(dtype, [&](auto* t_) {
+        using T = FLHIP_T_OF(t_);
+        hipLaunchKernelGGL((matmul_nn_skinny<T>), grid, dim3(1024), 0, s, (const T*)A, (const T*)B,
+                           (T*)C, M, N, K, bias_rows);
+      });
       return check_launch("matmul (thin, A * B)");
     }
     if (!bias_rows) {
       const int mtiles = (M + 7) / 8, tiles = mtiles * ((N + 7) / 8);
       const dim3 grid((unsigned)((tiles + 3) / 4));
-      if (dtype == FLHIP_F32)
-        hipLaunchKernelGGL((matmul_tn_skinny<float>), grid, dim3(256), 0, s, (const float*)A, (const float*)B,
-                           (float*)C, M, N, K, mtiles, tiles);
-      else
-        hipLaunchKernelGGL((matmul_tn_skinny<bf16_t>), grid, dim3(256), 0, s, (const bf16_t*)A, (const bf16_t*)B,
-                           (bf16_t*)C, M, N, K, mtiles, tiles);
+      by_dtype(dtype, [&](auto* t_) {
+        using T = FLHIP_T_OF(t_);
+        hipLaunchKernelGGL((matmul_tn_skinny<T>), grid, dim3(256), 0, s, (const T*)A, (const T*)B,
+                           (T*)C, M, N, K, mtiles, tiles);
+      });
       return check_launch("matmul (thin, A^T * B)");
     }
   }
@@ -575,13 +572,12 @@ extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, in
   }
   const dim3 grid((unsigned)((M + GT - 1) / GT), (unsigned)((N + GT - 1) / GT));
   FLHIP_REQUIRE(grid.y <= 65535, "matmul: too many columns");
-  if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((matmul_kernel<float>), grid, dim3(256), 0, as_stream(stream), (const float*)A,
-                       (const float*)B, (float*)C, M, N, K, trans_a, trans_b, bias_rows);
-  else
-    hipLaunchKernelGGL((matmul_kernel<bf16_t>), grid, dim3(256), 0, as_stream(stream),
-                       (const bf16_t*)A, (const bf16_t*)B, (bf16_t*)C, M, N, K, trans_a, trans_b,
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((matmul_kernel<T>), grid, dim3(256), 0, as_stream(stream),
+                       (const T*)A, (const T*)B, (T*)C, M, N, K, trans_a, trans_b,
                        bias_rows);
+  });
   return check_launch("matmul");
 }
 
@@ -591,12 +587,11 @@ extern "C" int flhip_sum_columns(const void* x, float* out, int32_t rows, int32_
   FLHIP_REQUIRE(rows > 0 && cols > 0, "sum_columns: sizes must be positive");
   FLHIP_REQUIRE(dtype_ok(dtype), "sum_columns: unknown dtype");
   const dim3 grid((unsigned)((rows + 15) / 16));
-  if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((sum_cols_kernel<float>), grid, dim3(1024), 0, as_stream(stream),
-                       (const float*)x, out, rows, cols);
-  else
-    hipLaunchKernelGGL((sum_cols_kernel<bf16_t>), grid, dim3(1024), 0, as_stream(stream),
-                       (const bf16_t*)x, out, rows, cols);
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((sum_cols_kernel<T>), grid, dim3(1024), 0, as_stream(stream),
+                       (const T*)x, out, rows, cols);
+  });
   return check_launch("sum_columns");
 }
 
@@ -606,12 +601,11 @@ extern "C" int flhip_logsoftmax_fwd(const void* x, void* y, int32_t classes, int
   FLHIP_REQUIRE(classes > 0 && cols > 0, "logsoftmax: sizes must be positive");
   FLHIP_REQUIRE(dtype_ok(dtype), "logsoftmax: unknown dtype");
   const dim3 grid((unsigned)((cols + 3) / 4));
-  if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((logsoftmax_fwd_kernel<float>), grid, dim3(256), 0, as_stream(stream),
-                       (const float*)x, (float*)y, classes, cols);
-  else
-    hipLaunchKernelGGL((logsoftmax_fwd_kernel<bf16_t>), grid, dim3(256), 0, as_stream(stream),
-                       (const bf16_t*)x, (bf16_t*)y, classes, cols);
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((logsoftmax_fwd_kernel<T>), grid, dim3(256), 0, as_stream(stream),
+                       (const T*)x, (T*)y, classes, cols);
+  });
   return check_launch("logsoftmax");
 }
 
@@ -621,12 +615,11 @@ extern "C" int flhip_logsoftmax_bwd(const void* dy, const void* y, void* dx, int
   FLHIP_REQUIRE(classes > 0 && cols > 0, "logsoftmax_bwd: sizes must be positive");
   FLHIP_REQUIRE(dtype_ok(dtype), "logsoftmax_bwd: unknown dtype");
   const dim3 grid((unsigned)((cols + 3) / 4));
-  if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((logsoftmax_bwd_kernel<float>), grid, dim3(256), 0, as_stream(stream),
-                       (const float*)dy, (const float*)y, (float*)dx, classes, cols);
-  else
-    hipLaunchKernelGGL((logsoftmax_bwd_kernel<bf16_t>), grid, dim3(256), 0, as_stream(stream),
-                       (const bf16_t*)dy, (const bf16_t*)y, (bf16_t*)dx, classes, cols);
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((logsoftmax_bwd_kernel<T>), grid, dim3(256), 0, as_stream(stream),
+                       (const T*)dy, (const T*)y, (T*)dx, classes, cols);
+  });
   return check_launch("logsoftmax_bwd");
 }
 
@@ -636,12 +629,11 @@ extern "C" int flhip_cce_fwd(const void* logp, const int32_t* target, float* sta
   FLHIP_REQUIRE(logp && target && stats, "cce: null argument");
   FLHIP_REQUIRE(classes > 0 && cols > 0, "cce: sizes must be positive");
   FLHIP_REQUIRE(dtype_ok(dtype), "cce: unknown dtype");
-  if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((cce_fwd_kernel<float>), dim3(1), dim3(256), 0, as_stream(stream),
-                       (const float*)logp, target, stats, per_column, classes, cols, ignore_index);
-  else
-    hipLaunchKernelGGL((cce_fwd_kernel<bf16_t>), dim3(1), dim3(256), 0, as_stream(stream),
-                       (const bf16_t*)logp, target, stats, per_column, classes, cols, ignore_index);
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((cce_fwd_kernel<T>), dim3(1), dim3(256), 0, as_stream(stream),
+                       (const T*)logp, target, stats, per_column, classes, cols, ignore_index);
+  });
   return check_launch("cce");
 }
 
@@ -653,14 +645,12 @@ extern "C" int flhip_cce_bwd(const float* grad, const int32_t* target, const flo
   FLHIP_REQUIRE(reduction >= 0 && reduction <= 2, "cce_bwd: unknown reduction");
   FLHIP_REQUIRE(dtype_ok(dtype), "cce_bwd: unknown dtype");
   const size_t total = (size_t)classes * cols;
-  if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((cce_bwd_kernel<float>), dim3(blocks_for(total)), dim3(256), 0,
-                       as_stream(stream), grad, target, stats, (float*)dx, classes, cols, reduction,
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((cce_bwd_kernel<T>), dim3(blocks_for(total)), dim3(256), 0,
+                       as_stream(stream), grad, target, stats, (T*)dx, classes, cols, reduction,
                        ignore_index);
-  else
-    hipLaunchKernelGGL((cce_bwd_kernel<bf16_t>), dim3(blocks_for(total)), dim3(256), 0,
-                       as_stream(stream), grad, target, stats, (bf16_t*)dx, classes, cols, reduction,
-                       ignore_index);
+  });
   return check_launch("cce_bwd");
 }
 
@@ -684,12 +674,11 @@ extern "C" int flhip_reorder(const void* src, void* dst, const int64_t* dims, co
     g.ss[k] = sstride[perm[k]];
   }
   const size_t n = (size_t)st;
-  if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((reorder_kernel<float>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream),
-                       (const float*)src, (float*)dst, n, g);
-  else
-    hipLaunchKernelGGL((reorder_kernel<bf16_t>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream),
-                       (const bf16_t*)src, (bf16_t*)dst, n, g);
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((reorder_kernel<T>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream),
+                       (const T*)src, (T*)dst, n, g);
+  });
   return check_launch("reorder");
 }
 
@@ -700,14 +689,12 @@ extern "C" int flhip_affine_fwd(const void* x, const void* w, const void* b, voi
   FLHIP_REQUIRE(outer > 0 && mid > 0 && inner > 0, "affine: sizes must be positive");
   FLHIP_REQUIRE(dtype_ok(dtype), "affine: unknown dtype");
   const size_t n = (size_t)outer * (size_t)mid * (size_t)inner;
-  if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((affine_fwd_kernel<float>), dim3(blocks_for(n)), dim3(256), 0,
-                       as_stream(stream), (const float*)x, (const float*)w, (const float*)b,
-                       (float*)y, n, (long long)mid, (long long)inner, scalar_params ? 0 : 1);
-  else
-    hipLaunchKernelGGL((affine_fwd_kernel<bf16_t>), dim3(blocks_for(n)), dim3(256), 0,
-                       as_stream(stream), (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)b,
-                       (bf16_t*)y, n, (long long)mid, (long long)inner, scalar_params ? 0 : 1);
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((affine_fwd_kernel<T>), dim3(blocks_for(n)), dim3(256), 0,
+                       as_stream(stream), (const T*)x, (const T*)w, (const T*)b,
+                       (T*)y, n, (long long)mid, (long long)inner, scalar_params ? 0 : 1);
+  });
   return check_launch("affine");
 }
 
@@ -736,14 +723,12 @@ extern "C" int flhip_affine_bwd(const void* dy, const void* x, const void* w, vo
                   "affine_bwd: workspace too small");
   float* part = sums ? static_cast<float*>(workspace) : nullptr;
   const dim3 grid((unsigned)p.nparam, (unsigned)p.S);
-  if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((affine_bwd_kernel<float>), grid, dim3(256), 0, as_stream(stream),
-                       (const float*)dy, (const float*)x, (const float*)w, (float*)dx, part, p.per,
-                       p.chunk, p.mid, p.inner, p.S);
-  else
-    hipLaunchKernelGGL((affine_bwd_kernel<bf16_t>), grid, dim3(256), 0, as_stream(stream),
-                       (const bf16_t*)dy, (const bf16_t*)x, (const bf16_t*)w, (bf16_t*)dx, part,
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((affine_bwd_kernel<T>), grid, dim3(256), 0, as_stream(stream),
+                       (const T*)dy, (const T*)x, (const T*)w, (T*)dx, part,
                        p.per, p.chunk, p.mid, p.inner, p.S);
+  });
   if (const int rc = check_launch("affine_bwd")) return rc;
   if (sums) {
     hipLaunchKernelGGL(affine_fold_kernel, dim3((unsigned)((p.nparam + 255) / 256)), dim3(256), 0,

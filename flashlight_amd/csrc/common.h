@@ -5,6 +5,7 @@
 #include <stdint.h>
 
 #include <string>
+#include <type_traits>
 
 #include "flhip.h"
 
@@ -49,7 +50,23 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, pack_bf16x2));
 }
 
+// IEEE half storage (Flashlight's f16): a type of its own, so that the element-wise helpers below can be
+// overloaded on it.  Kernels that are templates on the storage type convert on load and store; sums are fp32.
+struct f16_t {
+  uint16_t bits;
+};
+__device__ __forceinline__ float f16_to_f32(f16_t v) { return (float)__builtin_bit_cast(_Float16, v.bits); }
+// round to nearest even (v_cvt_f16_f32)
+__device__ __forceinline__ f16_t f32_to_f16(float f) { return f16_t{__builtin_bit_cast(uint16_t, (_Float16)f)}; }
+__device__ __forceinline__ uint32_t pack_f16(float a, float b) {
+  return (uint32_t)f32_to_f16(a).bits | ((uint32_t)f32_to_f16(b).bits << 16);
+}
+__device__ __forceinline__ float f16lo(uint32_t w) { return f16_to_f32(f16_t{(uint16_t)(w & 0xffffu)}); }
+__device__ __forceinline__ float f16hi(uint32_t w) { return f16_to_f32(f16_t{(uint16_t)(w >> 16)}); }
+
 __device__ __forceinline__ float ld(const float* p, size_t i) { return p[i]; }
+__device__ __forceinline__ float ld(const f16_t* p, size_t i) { return f16_to_f32(p[i]); }
+__device__ __forceinline__ void st(f16_t* p, size_t i, float v) { p[i] = f32_to_f16(v); }
 __device__ __forceinline__ float ld(const bf16_t* p, size_t i) {
   return bf16_to_f32(p[i]);
 }
@@ -68,6 +85,16 @@ __device__ __forceinline__ float4 ld4(const bf16_t* p, size_t i) {
                      __uint_as_float(r.x & 0xffff0000u),
                      __uint_as_float(r.y << 16),
                      __uint_as_float(r.y & 0xffff0000u));
+}
+__device__ __forceinline__ float4 ld4(const f16_t* p, size_t i) {
+  uint2 r = *reinterpret_cast<const uint2*>(p + i);
+  return make_float4(f16lo(r.x), f16hi(r.x), f16lo(r.y), f16hi(r.y));
+}
+__device__ __forceinline__ void st4(f16_t* p, size_t i, float4 v) {
+  uint2 r;
+  r.x = pack_f16(v.x, v.y);
+  r.y = pack_f16(v.z, v.w);
+  *reinterpret_cast<uint2*>(p + i) = r;
 }
 __device__ __forceinline__ void st4(float* p, size_t i, float4 v) {
   *reinterpret_cast<float4*>(p + i) = v;
@@ -92,6 +119,11 @@ __device__ __forceinline__ void st4_stream(bf16_t* p, size_t i, float4 v) {
   __builtin_nontemporal_store(t, reinterpret_cast<uintx2_t*>(p + i));
 }
 
+__device__ __forceinline__ void st4_stream(f16_t* p, size_t i, float4 v) {
+  const uintx2_t t = {pack_f16(v.x, v.y), pack_f16(v.z, v.w)};
+  __builtin_nontemporal_store(t, reinterpret_cast<uintx2_t*>(p + i));
+}
+
 // ---- buffer loads ------------------------------------------------------------
 // Raw buffer descriptor over `bytes` bytes at p: loads at a byte offset at or
 // past `bytes` return zero, which is how the gathers fetch padding.
@@ -105,8 +137,16 @@ __device__ __forceinline__ float buf_ld(__amdgpu_buffer_rsrc_t r, int byte_off, 
   return bf16_to_f32((bf16_t)__builtin_amdgcn_raw_buffer_load_b16(r, byte_off, 0, 0));
 }
 
+__device__ __forceinline__ float buf_ld(__amdgpu_buffer_rsrc_t r, int byte_off, const f16_t*) {
+  return f16_to_f32(f16_t{(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(r, byte_off, 0, 0)});
+}
+
 // four consecutive elements at a byte offset (16-byte aligned for float, 8 for bf16)
 typedef unsigned uintx4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 buf_ld4(__amdgpu_buffer_rsrc_t r, int byte_off, const f16_t*) {
+  const uintx2_t v = __builtin_amdgcn_raw_buffer_load_b64(r, byte_off, 0, 0);
+  return make_float4(f16lo(v.x), f16hi(v.x), f16lo(v.y), f16hi(v.y));
+}
 __device__ __forceinline__ float4 buf_ld4(__amdgpu_buffer_rsrc_t r, int byte_off, const float*) {
   const uintx4_t v = __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, 0);
   return make_float4(__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z),
@@ -258,6 +298,17 @@ const Options& options();
 
 inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
 
-inline bool dtype_ok(int32_t dt) { return dt == FLHIP_F32 || dt == FLHIP_BF16; }
+inline bool dtype_ok(int32_t dt) { return dt == FLHIP_F32 || dt == FLHIP_BF16 || dt == FLHIP_F16; }
+inline size_t dtype_size(int32_t dt) { return dt == FLHIP_F32 ? 4 : 2; }
+
+// Calls f with a null pointer of the storage type of `dt`:
+//   by_dtype(dt, [&](auto* t) { using T = std::remove_pointer_t<decltype(t)>; return launch<T>(...); })
+template <typename F>
+inline auto by_dtype(int32_t dt, F&& f) {
+  if (dt == FLHIP_F32) return f(static_cast<float*>(nullptr));
+  if (dt == FLHIP_F16) return f(static_cast<f16_t*>(nullptr));
+  return f(static_cast<bf16_t*>(nullptr));
+}
+#define FLHIP_T_OF(t) std::remove_pointer_t<decltype(t)>
 
 }  // namespace flhip

@@ -247,14 +247,12 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
   }
   const size_t total = (size_t)g.N * g.K * g.OH * g.OW;
   const dim3 grid((unsigned)((total + 255) / 256));
-  if (d->dtype == FLHIP_F32)
-    hipLaunchKernelGGL((conv_fwd_direct<float>), grid, dim3(256), 0, s, g,
-                       static_cast<const float*>(x), static_cast<const float*>(w), bias,
-                       static_cast<float*>(y), total);
-  else
-    hipLaunchKernelGGL((conv_fwd_direct<bf16_t>), grid, dim3(256), 0, s, g,
-                       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), bias,
-                       static_cast<bf16_t*>(y), total);
+  by_dtype(d->dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((conv_fwd_direct<T>), grid, dim3(256), 0, s, g,
+                       static_cast<const T*>(x), static_cast<const T*>(w), bias,
+                       static_cast<T*>(y), total);
+  });
   return check_launch("conv2d_fwd");
 }
 
@@ -272,14 +270,12 @@ constexpr int kNumPlans = 10;
 static int bwd_data_direct(const flhip_conv_desc* d, const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s) {
   const size_t total = (size_t)g.N * g.C * g.H * g.W;
   const dim3 grid((unsigned)((total + 255) / 256));
-  if (d->dtype == FLHIP_F32)
-    hipLaunchKernelGGL((conv_bwd_data_direct<float>), grid, dim3(256), 0, s, g,
-                       static_cast<const float*>(dy), static_cast<const float*>(w),
-                       static_cast<float*>(dx), total);
-  else
-    hipLaunchKernelGGL((conv_bwd_data_direct<bf16_t>), grid, dim3(256), 0, s, g,
-                       static_cast<const bf16_t*>(dy), static_cast<const bf16_t*>(w),
-                       static_cast<bf16_t*>(dx), total);
+  by_dtype(d->dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((conv_bwd_data_direct<T>), grid, dim3(256), 0, s, g,
+                       static_cast<const T*>(dy), static_cast<const T*>(w),
+                       static_cast<T*>(dx), total);
+  });
   return check_launch("conv2d_bwd_data");
 }
 
@@ -376,20 +372,18 @@ static int bwd_filter_direct(const flhip_conv_desc* d, const ConvGeom& g, const 
                              hipStream_t s) {
   if (dw) {
     const dim3 grid((unsigned)(g.K * g.Cg * g.KH * g.KW));
-    if (d->dtype == FLHIP_F32)
-      hipLaunchKernelGGL((conv_bwd_filter_direct<float>), grid, dim3(256), 0, s, g,
-                         static_cast<const float*>(x), static_cast<const float*>(dy), dw);
-    else
-      hipLaunchKernelGGL((conv_bwd_filter_direct<bf16_t>), grid, dim3(256), 0, s, g,
-                         static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), dw);
+    by_dtype(d->dtype, [&](auto* t_) {
+      using T = FLHIP_T_OF(t_);
+      hipLaunchKernelGGL((conv_bwd_filter_direct<T>), grid, dim3(256), 0, s, g,
+                         static_cast<const T*>(x), static_cast<const T*>(dy), dw);
+    });
   }
   if (db) {
-    if (d->dtype == FLHIP_F32)
-      hipLaunchKernelGGL((conv_bwd_bias_kernel<float>), dim3(g.K), dim3(256), 0, s, g,
-                         static_cast<const float*>(dy), db);
-    else
-      hipLaunchKernelGGL((conv_bwd_bias_kernel<bf16_t>), dim3(g.K), dim3(256), 0, s, g,
-                         static_cast<const bf16_t*>(dy), db);
+    by_dtype(d->dtype, [&](auto* t_) {
+      using T = FLHIP_T_OF(t_);
+      hipLaunchKernelGGL((conv_bwd_bias_kernel<T>), dim3(g.K), dim3(256), 0, s, g,
+                         static_cast<const T*>(dy), db);
+    });
   }
   return check_launch("conv2d_bwd_filter");
 }

@@ -421,8 +421,10 @@ int mfma_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w, co
   p.mtiles = (g.Kg + BM - 1) / BM;
   p.Ptotal = g.N * g.OH * g.OW;
   p.DHW = g.OH * g.OW; p.SHW = g.H * g.W;
-  return dtype == FLHIP_F32 ? launch_gather<float, MODE_FWD>(p, x, w, bias, y, s)
-                            : launch_gather<bf16_t, MODE_FWD>(p, x, w, bias, y, s);
+  return by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    return launch_gather<T, MODE_FWD>(p, x, w, bias, y, s);
+  });
 }
 
 int mfma_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
@@ -440,11 +442,11 @@ int mfma_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void*
   p.Ptotal = g.N * g.H * g.W;
   p.DHW = g.H * g.W; p.SHW = g.OH * g.OW;
   const bool s1 = g.sy == 1 && g.sx == 1;
-  if (dtype == FLHIP_F32)
-    return s1 ? launch_gather<float, MODE_BWD_S1>(p, dy, w, nullptr, dx, s)
-              : launch_gather<float, MODE_BWD_GEN>(p, dy, w, nullptr, dx, s);
-  return s1 ? launch_gather<bf16_t, MODE_BWD_S1>(p, dy, w, nullptr, dx, s)
-            : launch_gather<bf16_t, MODE_BWD_GEN>(p, dy, w, nullptr, dx, s);
+  return by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    return s1 ? launch_gather<T, MODE_BWD_S1>(p, dy, w, nullptr, dx, s)
+              : launch_gather<T, MODE_BWD_GEN>(p, dy, w, nullptr, dx, s);
+  });
 }
 
 }  // namespace flhip

@@ -74,6 +74,14 @@ template <>
 __device__ __forceinline__ void buf_st1<bf16_t>(__amdgpu_buffer_rsrc_t r, int byte_off, float v, bf16_t*) {
   __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16(v), r, byte_off, 0, 0);
 }
+template <>
+__device__ __forceinline__ void buf_st1<f16_t>(__amdgpu_buffer_rsrc_t r, int byte_off, float v, f16_t*) {
+  __builtin_amdgcn_raw_buffer_store_b16(f32_to_f16(v).bits, r, byte_off, 0, 0);
+}
+__device__ __forceinline__ void buf_st4v(__amdgpu_buffer_rsrc_t r, int byte_off, floatx4 v, f16_t*) {
+  const uintx2_t t = {pack_f16(v[0], v[1]), pack_f16(v[2], v[3])};
+  __builtin_amdgcn_raw_buffer_store_b64(t, r, byte_off, 0, 0);
+}
 __device__ __forceinline__ void buf_st4v(__amdgpu_buffer_rsrc_t r, int byte_off, floatx4 v, float*) {
   const uintx4_t t = {__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]),
                       __float_as_uint(v[3])};
@@ -319,7 +327,7 @@ __global__ void __launch_bounds__(256) zero_kernel(T* __restrict__ p, size_t n16
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride)
     q[i] = make_uint4(0, 0, 0, 0);
   constexpr size_t per = 16 / sizeof(T);
-  for (size_t i = n16 * per + (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) p[i] = (T)0;
+  for (size_t i = n16 * per + (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) p[i] = T{};
 }
 
 template <typename T, bool BWD, int PT, bool VEC>
@@ -644,24 +652,21 @@ int launch_tapped(const ConvGeom& g, int dtype, const void* src, const void* wgt
   if (ws && ws_bytes >= (size_t)wb && p.KHW > 1 && !no_reorder) {
     const int rows = g.K * g.C;
     const long long total = (long long)rows * p.KHW;
-    if (dtype == FLHIP_F32)
-      hipLaunchKernelGGL((reorder_taps_kernel<float>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
-                         static_cast<const float*>(wgt), static_cast<float*>(ws), rows, p.KHW);
-    else
-      hipLaunchKernelGGL((reorder_taps_kernel<bf16_t>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
-                         static_cast<const bf16_t*>(wgt), static_cast<bf16_t*>(ws), rows, p.KHW);
+    by_dtype(dtype, [&](auto* t_) {
+      using T = FLHIP_T_OF(t_);
+      hipLaunchKernelGGL((reorder_taps_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+                         static_cast<const T*>(wgt), static_cast<T*>(ws), rows, p.KHW);
+    });
     wgt = ws;
     p.wre = 1;
   }
   const unsigned grid = (unsigned)(((p.ptiles + 7) / 8) * 8 * p.mtiles);
-  if (dtype == FLHIP_F32)
-    hipLaunchKernelGGL((tapped_conv_kernel<float, BWD>), dim3(grid), dim3(MFMA_THREADS), 0, s, p,
-                       static_cast<const float*>(src), static_cast<const float*>(wgt), bias,
-                       static_cast<float*>(dst));
-  else
-    hipLaunchKernelGGL((tapped_conv_kernel<bf16_t, BWD>), dim3(grid), dim3(MFMA_THREADS), 0, s, p,
-                       static_cast<const bf16_t*>(src), static_cast<const bf16_t*>(wgt), bias,
-                       static_cast<bf16_t*>(dst));
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((tapped_conv_kernel<T, BWD>), dim3(grid), dim3(MFMA_THREADS), 0, s, p,
+                       static_cast<const T*>(src), static_cast<const T*>(wgt), bias,
+                       static_cast<T*>(dst));
+  });
   return check_launch("conv2d (tapped mfma)");
 }
 
@@ -942,8 +947,10 @@ int mfma_pointwise_conv_fwd(const ConvGeom& g, int dtype, const void* x, const v
     p.dst_slice = (unsigned)(db / esz);
     p.dst_bytes = (unsigned)db;
   }
-  return dtype == FLHIP_F32 ? launch_pw<float, false>(p, vec, x, w, bias, y, s)
-                            : launch_pw<bf16_t, false>(p, vec, x, w, bias, y, s);
+  return by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    return launch_pw<T, false>(p, vec, x, w, bias, y, s);
+  });
 }
 
 int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
@@ -972,10 +979,10 @@ int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, c
     size_t blocks = (n16 + 255) / 256;
     if (blocks > 8192) blocks = 8192;
     if (blocks < 1) blocks = 1;
-    if (dtype == FLHIP_F32)
-      hipLaunchKernelGGL((zero_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, s, static_cast<float*>(dx), n16, nel);
-    else
-      hipLaunchKernelGGL((zero_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s, static_cast<bf16_t*>(dx), n16, nel);
+    by_dtype(dtype, [&](auto* t_) {
+      using T = FLHIP_T_OF(t_);
+      hipLaunchKernelGGL((zero_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, static_cast<T*>(dx), n16, nel);
+    });
   }
   const bool vec = full && p.P % 4 == 0;
   if (ksplit > 1) {
@@ -983,8 +990,10 @@ int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, c
     p.cps = (p.nchunks + ksplit - 1) / ksplit;
     p.dst_slice = (unsigned)(db / esz);
   }
-  return dtype == FLHIP_F32 ? launch_pw<float, true>(p, vec, dy, w, bias, dx, s)
-                            : launch_pw<bf16_t, true>(p, vec, dy, w, bias, dx, s);
+  return by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    return launch_pw<T, true>(p, vec, dy, w, bias, dx, s);
+  });
 }
 
 // ---- split contraction for 1x1 stride-1 fp32 layers with few tiles ----------------------
@@ -1054,21 +1063,17 @@ int mfma_pointwise_wgrad(const ConvGeom& g, int dtype, const void* x, const void
   float* out = p.nsplit > 1 ? static_cast<float*>(ws) : dw;
   const dim3 grid((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles), (unsigned)p.KHW);
   const bool vec = !p.x_map && p.P % 4 == 0;
-  if (dtype == FLHIP_F32) {
+  const int rc_ = by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
     if (vec)
-      hipLaunchKernelGGL((pointwise_wgrad_kernel<float, true>), grid, dim3(MFMA_THREADS), 0, s, p,
-                         static_cast<const float*>(x), static_cast<const float*>(dy), out);
+      hipLaunchKernelGGL((pointwise_wgrad_kernel<T, true>), grid, dim3(MFMA_THREADS), 0, s, p,
+                         static_cast<const T*>(x), static_cast<const T*>(dy), out);
     else
-      hipLaunchKernelGGL((pointwise_wgrad_kernel<float, false>), grid, dim3(MFMA_THREADS), 0, s, p,
-                         static_cast<const float*>(x), static_cast<const float*>(dy), out);
-  } else {
-    if (vec)
-      hipLaunchKernelGGL((pointwise_wgrad_kernel<bf16_t, true>), grid, dim3(MFMA_THREADS), 0, s, p,
-                         static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), out);
-    else
-      hipLaunchKernelGGL((pointwise_wgrad_kernel<bf16_t, false>), grid, dim3(MFMA_THREADS), 0, s, p,
-                         static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), out);
-  }
+      hipLaunchKernelGGL((pointwise_wgrad_kernel<T, false>), grid, dim3(MFMA_THREADS), 0, s, p,
+                         static_cast<const T*>(x), static_cast<const T*>(dy), out);
+    return 0;
+  });
+  if (rc_) return rc_;
   if (const int rc = check_launch("conv2d_bwd_filter 1x1 (mfma)")) return rc;
   if (p.nsplit > 1) {
     wgrad_reduce_launch(static_cast<const float*>(ws), p.nsplit, p.E, p.Mo, p.want_db, dw, db, s);

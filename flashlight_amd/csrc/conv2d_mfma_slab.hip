@@ -633,8 +633,10 @@ int mfma_slab_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* 
   p.groups = g.groups; p.SCg = g.Cg; p.DCg = g.Kg;
   p.a_mstride = g.Cg * p.KHW; p.a_cstride = p.KHW; p.w_group_stride = g.Kg * g.Cg * p.KHW;
   p.mtiles = (g.Kg + BM - 1) / BM;
-  return dtype == FLHIP_F32 ? launch<float, false>(p, x, w, bias, y, s)
-                            : launch<bf16_t, false>(p, x, w, bias, y, s);
+  return by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    return launch<T, false>(p, x, w, bias, y, s);
+  });
 }
 
 int mfma_slab_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx,
@@ -649,8 +651,10 @@ int mfma_slab_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const 
   p.groups = g.groups; p.SCg = g.Kg; p.DCg = g.Cg;
   p.a_mstride = p.KHW; p.a_cstride = g.Cg * p.KHW; p.w_group_stride = g.Kg * g.Cg * p.KHW;
   p.mtiles = (g.Cg + BM - 1) / BM;
-  return dtype == FLHIP_F32 ? launch<float, true>(p, dy, w, nullptr, dx, s)
-                            : launch<bf16_t, true>(p, dy, w, nullptr, dx, s);
+  return by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    return launch<T, true>(p, dy, w, nullptr, dx, s);
+  });
 }
 
 }  // namespace flhip

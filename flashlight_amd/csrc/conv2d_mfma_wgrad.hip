@@ -430,7 +430,7 @@ int mfma_conv_bwd_filter(const ConvGeom& g, int dtype, const void* x, const void
   if (!dw) return -1;   // bias gradient alone: the plain reduction kernel
   WgradParams p{};
   if (!wgrad_plan(g, &p) || !wgrad_split(&p, g)) return -1;
-  if (!(dtype == FLHIP_F32 ? wgrad_fits<float>(g, &p) : wgrad_fits<bf16_t>(g, &p))) return -1;
+  if (!by_dtype(dtype, [&](auto* t_) { return wgrad_fits<FLHIP_T_OF(t_)>(g, &p); })) return -1;
   p.want_db = db != nullptr;
   if (p.nsplit > 1 && (!ws || ws_bytes < (size_t)p.nsplit * (p.E + p.K) * sizeof(float)))
     return fail(FLHIP_INVALID_ARGUMENT, "conv2d_bwd_filter: workspace too small");
@@ -438,17 +438,15 @@ int mfma_conv_bwd_filter(const ConvGeom& g, int dtype, const void* x, const void
   const size_t shmem = (size_t)2 * (BNW * WKP + BM * WKP) * sizeof(float);
   const dim3 grid(p.nsplit, p.ntiles_n * p.mtiles, g.groups);
   float* out = p.nsplit > 1 ? static_cast<float*>(ws) : dw;
-  if (dtype == FLHIP_F32) {
-    auto kernel = wgrad_kernel<float>;
+  const int rc_ = by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    auto kernel = wgrad_kernel<T>;
     if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
-    hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const float*>(x),
-                       static_cast<const float*>(dy), out, db);
-  } else {
-    auto kernel = wgrad_kernel<bf16_t>;
-    if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
-    hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const bf16_t*>(x),
-                       static_cast<const bf16_t*>(dy), out, db);
-  }
+    hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const T*>(x),
+                       static_cast<const T*>(dy), out, db);
+    return 0;
+  });
+  if (rc_) return rc_;
   if (p.nsplit > 1)
     wgrad_reduce_launch(static_cast<const float*>(ws), p.nsplit, p.E, p.K, p.want_db, dw, db, s);
   return check_launch("conv2d_bwd_filter (mfma)");

@@ -513,17 +513,15 @@ int mfma_slab_wgrad(const ConvGeom& g, int dtype, const void* x, const void* dy,
   const dim3 grid(p.nsplit, p.nhalves * p.mtiles, g.groups);
   float* out = p.nsplit > 1 ? static_cast<float*>(ws) : dw;
   if (reinterpret_cast<uintptr_t>(out) % 16 != 0) p.stage_ok = 0;
-  if (dtype == FLHIP_F32) {
-    auto kernel = wgrad_slab_kernel<float>;
+  const int rc_ = by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    auto kernel = wgrad_slab_kernel<T>;
     if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
-    hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const float*>(x),
-                       static_cast<const float*>(dy), out, db);
-  } else {
-    auto kernel = wgrad_slab_kernel<bf16_t>;
-    if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
-    hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const bf16_t*>(x),
-                       static_cast<const bf16_t*>(dy), out, db);
-  }
+    hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const T*>(x),
+                       static_cast<const T*>(dy), out, db);
+    return 0;
+  });
+  if (rc_) return rc_;
   if (p.nsplit > 1)
     wgrad_reduce_launch(static_cast<const float*>(ws), p.nsplit, p.E, p.K, p.want_db, dw, db, s);
   return check_launch("conv2d_bwd_filter (mfma slab)");

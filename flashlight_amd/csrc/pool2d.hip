@@ -149,6 +149,13 @@ __device__ __forceinline__ void st2(float* p, size_t i, float a, float b) {
 __device__ __forceinline__ void st2(bf16_t* p, size_t i, float a, float b) {
   *reinterpret_cast<uint32_t*>(p + i) = (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
 }
+__device__ __forceinline__ void st2(f16_t* p, size_t i, float a, float b) {
+  *reinterpret_cast<uint32_t*>(p + i) = pack_f16(a, b);
+}
+__device__ __forceinline__ float2 ld2(const f16_t* p, size_t i) {
+  const uint32_t r = *reinterpret_cast<const uint32_t*>(p + i);
+  return make_float2(f16lo(r), f16hi(r));
+}
 __device__ __forceinline__ float2 ld2(const float* p, size_t i) {
   return *reinterpret_cast<const float2*>(p + i);
 }
@@ -565,8 +572,10 @@ extern "C" int flhip_pool2d_fwd(const flhip_pool_desc* d, const void* x, void* y
   if (rc != FLHIP_OK) return rc;
   if (d->mode == FLHIP_POOL_MAX && argmax)
     FLHIP_REQUIRE(d->wy * d->wx <= 256, "pool2d_fwd: argmax needs a window of at most 256 elements");
-  return d->dtype == FLHIP_F32 ? launch_fwd<float>(g, d->mode, x, y, argmax, as_stream(stream))
-                               : launch_fwd<bf16_t>(g, d->mode, x, y, argmax, as_stream(stream));
+  return by_dtype(d->dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    return launch_fwd<T>(g, d->mode, x, y, argmax, as_stream(stream));
+  });
 }
 
 extern "C" int flhip_pool2d_bwd(const flhip_pool_desc* d, const void* dy,
@@ -581,6 +590,8 @@ extern "C" int flhip_pool2d_bwd(const flhip_pool_desc* d, const void* dy,
     FLHIP_REQUIRE(argmax != nullptr, "pool2d_bwd: max pooling needs the argmax of the forward pass");
     FLHIP_REQUIRE(d->wy * d->wx <= 256, "pool2d_bwd: window of at most 256 elements");
   }
-  return d->dtype == FLHIP_F32 ? launch_bwd<float>(g, d->mode, dy, argmax, dx, as_stream(stream))
-                               : launch_bwd<bf16_t>(g, d->mode, dy, argmax, dx, as_stream(stream));
+  return by_dtype(d->dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    return launch_bwd<T>(g, d->mode, dy, argmax, dx, as_stream(stream));
+  });
 }

@@ -47,9 +47,9 @@ void Variable::addGrad(const Variable& childGrad) {
   }
   detail::OpScope scope("addGrad");
   Tensor sum(shape(), type());
-  const int tag = type() == dtype::f32 ? FLHIP_F32 : FLHIP_BF16;
-  if (type() != dtype::f32 && type() != dtype::bf16)
-    throw std::runtime_error("Variable::addGrad: f32 and bf16 only");
+  if (type() != dtype::f32 && type() != dtype::bf16 && type() != dtype::f16)
+    throw std::runtime_error("Variable::addGrad: f32, bf16 and f16 only");
+  const int tag = type() == dtype::f32 ? FLHIP_F32 : type() == dtype::bf16 ? FLHIP_BF16 : FLHIP_F16;
   if (flhip_add(grad_->grad->tensor().device(), childGrad.tensor().device(), sum.device(),
                 (size_t)sum.elements(), tag, hipBackendStream()) != FLHIP_OK)
     throw std::runtime_error(flhip_last_error());
@@ -375,7 +375,8 @@ namespace {
 int tagOf(dtype t, const char* fn) {
   if (t == dtype::f32) return FLHIP_F32;
   if (t == dtype::bf16) return FLHIP_BF16;
-  throw std::runtime_error(std::string(fn) + ": f32 and bf16 only");
+  if (t == dtype::f16) return FLHIP_F16;
+  throw std::runtime_error(std::string(fn) + ": f32, bf16 and f16 only");
 }
 void check(int rc) {
   if (rc == FLHIP_INVALID_ARGUMENT) throw std::invalid_argument(flhip_last_error());

@@ -36,7 +36,7 @@ class Variable {
   bool isCalcGrad() const { return grad_->calcGrad; }
   // flashlight/fl/autograd/Variable.cpp:155-163: switching off also drops the graph
   void setCalcGrad(bool calcGrad);
-  // differentiable cast (Variable.cpp:100-108); f32 <-> bf16 here
+  // differentiable cast (Variable.cpp:100-108); among f32, bf16 and f16 here
   Variable astype(dtype type) const;
   // the cast node of this variable around a conversion that was made elsewhere (one of many in
   // one launch): same graph node as astype() builds

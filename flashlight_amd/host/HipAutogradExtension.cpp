@@ -67,6 +67,7 @@ void check(int rc) {
 int dtypeTag(dtype t, const char* op) {
   if (t == dtype::f32) return FLHIP_F32;
   if (t == dtype::bf16) return FLHIP_BF16;
+  if (t == dtype::f16) return FLHIP_F16;
   throw std::runtime_error(std::string(op) + ": data type not supported by the HIP autograd extension");
 }
 
@@ -192,7 +193,7 @@ Tensor HipAutogradExtension::workspace(size_t bytes) {
 }
 
 bool HipAutogradExtension::isDataTypeSupported(const dtype& type) const {
-  return type == dtype::f32 || type == dtype::bf16;
+  return type == dtype::f32 || type == dtype::bf16 || type == dtype::f16;
 }
 
 // ---- conv2d -------------------------------------------------------------------
@@ -644,14 +645,15 @@ std::tuple<Tensor, Tensor, Tensor> HipAutogradExtension::rnn(
   for (const Tensor* t : {&hiddenState, &cellState, &weights})
     if (!t->isEmpty() && t->type() != input.type())
       throw std::invalid_argument("rnn doesn't support binary operations with Tensors of different types");
-  if (input.type() == dtype::bf16) {
+  if (input.type() == dtype::bf16 || input.type() == dtype::f16) {
+    const dtype lo = input.type();
     // 16-bit storage (the reference: half tensors, RNN.cpp:45): the device kernels are fp32, so the
     // tensors are widened at the boundary and the results rounded once on the way out
     auto up = [](const Tensor& t) { return t.isEmpty() ? t : t.astype(dtype::f32); };
     Tensor y, hy, cy;
     std::tie(y, hy, cy) = rnn(up(input), up(hiddenState), up(cellState), up(weights), hiddenSize, numLayers, mode,
                               bidirectional, dropProb, autogradPayload);
-    return std::make_tuple(y.astype(dtype::bf16), hy.astype(dtype::bf16), cy.isEmpty() ? cy : cy.astype(dtype::bf16));
+    return std::make_tuple(y.astype(lo), hy.astype(lo), cy.isEmpty() ? cy : cy.astype(lo));
   }
   const unsigned long long seed = dropProb > 0.f ? nextSeed() : 0ull;
   const flhip_rnn_desc d = rnnDesc(input, hiddenSize, numLayers, mode, bidirectional, dropProb, seed);
@@ -699,7 +701,8 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> HipAutogradExtension::rnnBackward(
   auto payload = std::dynamic_pointer_cast<HipRnnPayload>(autogradPayload->data);
   if (!payload) throw std::invalid_argument("rnnBackward: payload of another operation");
   if (!gradData) throw std::invalid_argument("rnnBackward: no gradient data");
-  if (input.type() == dtype::bf16) {
+  if (input.type() == dtype::bf16 || input.type() == dtype::f16) {
+    const dtype lo = input.type();
     auto up = [](const Tensor& t) { return t.isEmpty() ? t : t.astype(dtype::f32); };
     auto wide = std::make_shared<detail::RNNGradData>();
     wide->dy = up(gradData->dy);
@@ -708,8 +711,7 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> HipAutogradExtension::rnnBackward(
     Tensor dx, dhx, dcx, dw;
     std::tie(dx, dhx, dcx, dw) = rnnBackward(up(input), up(hiddenState), up(cellState), up(weights), wide, up(output),
                                             numLayers, hiddenSize, mode, bidirectional, dropProb, autogradPayload);
-    return std::make_tuple(dx.astype(dtype::bf16), dhx.astype(dtype::bf16), dcx.isEmpty() ? dcx : dcx.astype(dtype::bf16),
-                           dw.astype(dtype::bf16));
+    return std::make_tuple(dx.astype(lo), dhx.astype(lo), dcx.isEmpty() ? dcx : dcx.astype(lo), dw.astype(lo));
   }
   const flhip_rnn_desc d = rnnDesc(input, hiddenSize, numLayers, mode, bidirectional, dropProb, payload->seed);
   const Dim totalLayers = numLayers * (bidirectional ? 2 : 1);

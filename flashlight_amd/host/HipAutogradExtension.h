@@ -18,8 +18,8 @@ class HipAutogradExtension : public AutogradExtension {
   // (cudnn/CudnnAutogradExtension.cpp:17-25).
   std::shared_ptr<DynamicBenchmark> createBenchmarkOptions() override;
   static constexpr int kPlanBenchCount = 3;
-  // f32 and the private bf16 tag; the oneDNN extension supports everything but f16
-  // (onednn/OneDnnAutogradExtension.cpp:12-16), the cuDNN one f16/f32/f64.
+  // f32, f16 and the private bf16 tag (the 16-bit types are storage types: sums are fp32).  The oneDNN
+  // extension supports everything but f16 (onednn/OneDnnAutogradExtension.cpp:12-16), the cuDNN one f16/f32/f64.
   bool isDataTypeSupported(const dtype& type) const override;
 
   Tensor conv2d(const Tensor& input, const Tensor& weights, const Tensor& bias, const int sx,

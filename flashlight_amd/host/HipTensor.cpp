@@ -88,7 +88,8 @@ class DevicePool {
 int tag(dtype t) {
   if (t == dtype::f32) return FLHIP_F32;
   if (t == dtype::bf16) return FLHIP_BF16;
-  throw std::runtime_error("HIP backend: conversion supports f32 and bf16 only");
+  if (t == dtype::f16) return FLHIP_F16;
+  throw std::runtime_error("HIP backend: conversion supports f32, bf16 and f16 only");
 }
 }  // namespace
 
@@ -256,10 +257,10 @@ std::vector<float> Tensor::toHostVector() const {
   if (isEmpty()) return out;
   if (type_ == dtype::f32) {
     toHost(out.data());
-  } else if (type_ == dtype::bf16) {
+  } else if (type_ == dtype::bf16 || type_ == dtype::f16) {
     astype(dtype::f32).toHost(out.data());
   } else {
-    throw std::runtime_error("toHostVector: f32 and bf16 only");
+    throw std::runtime_error("toHostVector: f32, bf16 and f16 only");
   }
   return out;
 }

@@ -25,7 +25,7 @@ class Tensor {
   static Tensor full(const Shape& shape, double value, dtype type);
 
   void toHost(void* dst) const;             // blocking copy of the whole buffer
-  std::vector<float> toHostVector() const;  // converts f32 / bf16 to float
+  std::vector<float> toHostVector() const;  // converts f32 / bf16 / f16 to float
 
   const Shape& shape() const { return shape_; }
   dtype type() const { return type_; }
@@ -37,7 +37,7 @@ class Tensor {
   TensorBackendType backendType() const { return TensorBackendType::Hip; }
   bool isContiguous() const { return true; }
 
-  // Tensor::astype for f32 <-> bf16; other conversions are not part of this path.
+  // Tensor::astype among f32, bf16 and f16; other conversions are not part of this path.
   Tensor astype(dtype t) const;
   // the same conversion of several tensors of one type in one launch per 64 of them
   // (flhip_convert_many); tensors that already have type t come back as they are

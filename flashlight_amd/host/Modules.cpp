@@ -18,8 +18,8 @@ std::mt19937_64& generator() {
   return gen;
 }
 Tensor fromFloats(const Shape& shape, dtype type, const std::vector<float>& v) {
-  if (type != dtype::f32 && type != dtype::bf16)
-    throw std::invalid_argument("initialisation: f32 and bf16 only");
+  if (type != dtype::f32 && type != dtype::bf16 && type != dtype::f16)
+    throw std::invalid_argument("initialisation: f32, bf16 and f16 only");
   Tensor t = Tensor::fromVector(shape, v);
   return type == dtype::f32 ? t : t.astype(type);
 }

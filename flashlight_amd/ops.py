@@ -36,7 +36,12 @@ def _dtype_tag(t):
         return capi.F32
     if t.dtype == torch.bfloat16:
         return capi.BF16
+    if t.dtype == torch.float16:
+        return capi.F16
     raise RuntimeError("flashlight_amd: unsupported dtype %s" % t.dtype)
+
+
+_TAG_OF = {torch.float32: capi.F32, torch.bfloat16: capi.BF16, torch.float16: capi.F16}
 
 
 def _dev(t, name):
@@ -506,7 +511,7 @@ def categorical_cross_entropy_backward(grad_output, input_shape, dtype, targets,
     g, t = _dev(grad_output, "gradOutput").float().contiguous(), _dev(targets, "targets")
     dx = torch.empty(tuple(input_shape), dtype=dtype, device=t.device)
     classes = input_shape[-1]
-    tag = capi.F32 if dtype == torch.float32 else capi.BF16
+    tag = _TAG_OF[dtype]
     capi.check(capi.lib().flhip_cce_bwd(_ptr(g), _ptr(t), _ptr(stats), _ptr(dx), classes, t.numel(),
                                         reduction, ignore_index, tag, _stream()))
     return dx

@@ -42,10 +42,17 @@ enum {
 
 /* Storage type of activations.  Reductions and accumulators are always fp32.
  * Flashlight has no bf16 dtype (flashlight/fl/tensor/Types.h:17-30); FLHIP_BF16
- * is this library's private tag for bf16 storage with fp32 accumulate. */
+ * is this library's private tag for bf16 storage with fp32 accumulate.
+ * FLHIP_F16 is IEEE half storage, Flashlight's f16 (Types.h:17-30), which its cuDNN extension supports
+ * (cudnn/CudnnAutogradExtension.cpp:27-36) and its oneDNN extension refuses
+ * (onednn/OneDnnAutogradExtension.cpp:12-16).  Every entry point that takes FLHIP_BF16 takes FLHIP_F16 with
+ * the same meaning (16-bit tensors where bf16 ones are, fp32 ones where fp32 ones are; results rounded once,
+ * to nearest even, overflow to infinity); its tensors go through the kernels that widen their operands to
+ * fp32, not through the bf16 matrix-core families. */
 enum {
   FLHIP_F32 = 0,
-  FLHIP_BF16 = 1
+  FLHIP_BF16 = 1,
+  FLHIP_F16 = 2
 };
 
 /* fl::PoolingMode, same numeric values (flashlight/fl/common/Defines.h:53-64). */
@@ -66,7 +73,7 @@ enum {
  * [N,K,OH,OW] with OH = 1 + (H + 2*py - (1 + (KH-1)*dil_y)) / sy (integer
  * division), likewise OW (onednn/Conv2D.cpp:179-188).  Dilation uses
  * Flashlight's convention (1 = dense).  dtype = FLHIP_F32: every buffer fp32.
- * dtype = FLHIP_BF16: x, w, y, dy, dx are bf16; bias, dw, db stay fp32. */
+ * dtype = FLHIP_BF16 / FLHIP_F16: x, w, y, dy, dx are 16-bit; bias, dw, db stay fp32. */
 typedef struct flhip_conv_desc {
   int32_t N, C, H, W;
   int32_t K, KH, KW;
@@ -108,8 +115,8 @@ const char* flhip_last_error(void);
  * compiled against is FLHIP_VERSION; descriptor structs only ever grow at the end, and a caller must
  * refuse to run when flhip_version() / 100 differs from FLHIP_VERSION / 100 (a layout change).
  * 200: flhip_rnn_desc gained dropout, seed_lo, seed_hi; flhip_bn_workspace_bytes never returns less
- * than 32 bytes per feature. */
-#define FLHIP_VERSION 202
+ * than 32 bytes per feature.  202: the *_plan entry points and FLHIP_DECLINED.  203: FLHIP_F16. */
+#define FLHIP_VERSION 203
 int flhip_version(void);
 const char* flhip_arch(void);
 
@@ -304,8 +311,8 @@ int flhip_bn_act_bwd_mask(const flhip_bn_desc* d, const void* x, const void* dy,
                           void* dx, void* dresidual, float* dgamma, float* dbeta, void* ws,
                           size_t ws_bytes, void* stream);
 
-/* Storage conversion between FLHIP_F32 and FLHIP_BF16 (round to nearest even) of n
- * elements; same dtype = copy.  Serves the casts the caller closures make around
+/* Storage conversion among FLHIP_F32, FLHIP_BF16 and FLHIP_F16 (round to nearest even; between the
+ * two 16-bit types through the fp32 value) of n elements; same dtype = copy.  Serves the casts the caller closures make around
  * the extension (Tensor::astype in flashlight/fl/autograd/Functions.cpp:1558-1561
  * and FL_ADJUST_INPUT_TYPE, flashlight/fl/autograd/Functions.h:57-82). */
 int flhip_convert(const void* src, int src_dtype, void* dst, int dst_dtype,

@@ -73,6 +73,17 @@ static float bf16round(float f) {
   std::memcpy(&f, &u, 4);
   return f;
 }
+// nearest IEEE half value (ties to even), as a float
+static float f16round(float f) {
+  if (!std::isfinite(f) || f == 0.f) return f;
+  const float a = std::fabs(f);
+  if (a >= 65520.f) return std::copysign(INFINITY, f);
+  int e;
+  std::frexp(a, &e);                                   // a = m * 2^e, m in [0.5, 1)
+  const int q = e - 11 < -24 ? -24 : e - 11;           // 11 significant bits; subnormals step by 2^-24
+  return std::copysign(std::ldexp(std::nearbyint(std::ldexp(a, -q)), q), f);
+}
+static float roundTo(dtype dt, float f) { return dt == dtype::bf16 ? bf16round(f) : dt == dtype::f16 ? f16round(f) : f; }
 template <typename E>
 static bool throws(const std::function<void()>& f) {
   try {
@@ -90,8 +101,8 @@ static void testRegistration() {
   AutogradExtension& e = getAutogradExtension(TensorBackendType::Hip);
   CHECK(dynamic_cast<HipAutogradExtension*>(&e) != nullptr);
   CHECK(&e == &getAutogradExtension(TensorBackendType::Hip));       // one instance per backend
-  CHECK(e.isDataTypeSupported(dtype::f32) && e.isDataTypeSupported(dtype::bf16));
-  CHECK(!e.isDataTypeSupported(dtype::f16) && !e.isDataTypeSupported(dtype::f64));
+  CHECK(e.isDataTypeSupported(dtype::f32) && e.isDataTypeSupported(dtype::bf16) && e.isDataTypeSupported(dtype::f16));
+  CHECK(!e.isDataTypeSupported(dtype::f64) && !e.isDataTypeSupported(dtype::s32));
   CHECK(e.createBenchmarkOptions() != nullptr && e.createBenchmarkOptions() != e.createBenchmarkOptions());   // one per pass and layer
   // a second registration for the same backend is ignored (TensorExtension.cpp:27-29)
   CHECK(!detail::registerAutogradExtension(TensorBackendType::Hip, [] {
@@ -105,7 +116,7 @@ static void testRegistration() {
 }
 
 static void testConv(dtype dt, int groups, double tol) {
-  std::printf("conv2d %s groups=%d\n", dt == dtype::f32 ? "f32" : "bf16", groups);
+  std::printf("conv2d %s groups=%d\n", dt == dtype::f32 ? "f32" : dt == dtype::bf16 ? "bf16" : "f16", groups);
   // input [10,9,8,7], weights [4,3,8/groups,6], px=2, py=1
   const int W = 10, H = 9, C = 8, N = 7, KW = 4, KH = 3, K = 6, px = 2, py = 1;
   flref_conv d{N, C, H, W, K, KH, KW, 1, 1, py, px, 1, 1, groups};
@@ -113,10 +124,8 @@ static void testConv(dtype dt, int groups, double tol) {
   flref_conv_out(&d, &OH, &OW);
   auto x = randn((size_t)N * C * H * W, 1), w = randn((size_t)K * (C / groups) * KH * KW, 2, 0.2f);
   auto b = randn(K, 3), dy = randn((size_t)N * K * OH * OW, 4);
-  if (dt == dtype::bf16) {
-    for (auto* v : {&x, &w, &b, &dy})
-      for (auto& f : *v) f = bf16round(f);
-  }
+  for (auto* v : {&x, &w, &b, &dy})
+    for (auto& f : *v) f = roundTo(dt, f);
   std::vector<float> y(dy.size()), dx(x.size()), dw(w.size()), db(K);
   flref_conv2d_fwd(&d, x.data(), w.data(), b.data(), y.data());
   flref_conv2d_bwd_data(&d, dy.data(), w.data(), dx.data());
@@ -596,13 +605,15 @@ static void testBatchNormModule() {
   loose.eval();
   flref_bn_fwd_train(N, C, (int64_t)H * W, x.data(), gl.data(), bl.data(), 1e-5, y.data(), mean.data(), var.data());
   CHECK(relL2(hostOf(loose.forward(in)), y) <= 1e-4 && loose.numBatchesTracked() == 0);
-  // bf16 input keeps f32 parameters (BatchNorm.cpp:86-88)
+  // a 16-bit input keeps f32 parameters (BatchNorm.cpp:86-88: half input)
   bn.train();
-  Variable in16(in.tensor().astype(dtype::bf16), true);
-  Variable y16 = bn.forward(in16);
-  CHECK(y16.type() == dtype::bf16);
-  y16.backward(Variable(Tensor::full(y16.shape(), 1., dtype::f32).astype(dtype::bf16), false));
-  CHECK(bn.param(0).grad().type() == dtype::f32 && in16.grad().type() == dtype::bf16);
+  for (const dtype lo : {dtype::bf16, dtype::f16}) {
+    Variable in16(in.tensor().astype(lo), true);
+    Variable y16 = bn.forward(in16);
+    CHECK(y16.type() == lo);
+    y16.backward(Variable(Tensor::full(y16.shape(), 1., dtype::f32).astype(lo), false));
+    CHECK(bn.param(0).grad().type() == dtype::f32 && in16.grad().type() == lo);
+  }
 }
 
 // LayerNorm module on the reference test's shapes (ModuleTest.cpp:670-719) plus the
@@ -1214,6 +1225,8 @@ int main() {
     testConv(dtype::f32, 1, 1e-4);
     testConv(dtype::f32, 2, 1e-4);
     testConv(dtype::bf16, 1, 2e-2);
+    testConv(dtype::f16, 1, 2e-2);
+    testConv(dtype::f16, 2, 2e-2);
     testConvErrors();
     testBatchingInvariance();
     testPool();

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import flashlight_amd as fa
-from gpu_util import bf16_round, dev, host
+from gpu_util import bf16_round, dev, host, round_to
 from oracle import flref
 from refmath import rel_l2
 
@@ -54,15 +54,18 @@ def _data(shape, axes, seed, dtype):
     outer, C, inner = flref.bn_view(list(shape[::-1]), axes)
     x = (rng.standard_normal(shape) * np.sqrt(2) + 0.5).astype(np.float32)
     dy = rng.standard_normal(shape).astype(np.float32)
-    if dtype == torch.bfloat16:
-        x, dy = bf16_round(x), bf16_round(dy)
+    x, dy = round_to(x, dtype), round_to(dy, dtype)
     g = (1 + 0.1 * rng.standard_normal(C)).astype(np.float32)
     b = rng.standard_normal(C).astype(np.float32)
     return outer, C, inner, x, dy, g, b
 
 
-@pytest.mark.parametrize("shape,axes", CASES)
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+# f16 storage takes the kernels of the other two types with its own loads and stores: the shapes up to 4M elements
+TYPED_CASES = ([(s, a, dt) for s, a in CASES for dt in (torch.float32, torch.bfloat16)] +
+               [(s, a, torch.float16) for s, a in CASES if int(np.prod(s)) <= 4 << 20])
+
+
+@pytest.mark.parametrize("shape,axes,dtype", TYPED_CASES)
 def test_train_forward_backward(shape, axes, dtype):
     tol = 1e-4 if dtype == torch.float32 else 2e-2
     outer, C, inner, x, dy, g, b = _data(shape, axes, 50, dtype)
@@ -209,14 +212,14 @@ FUSED = [
 ]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("with_residual", [False, True])
 @pytest.mark.parametrize("shape,axes", FUSED)
 def test_fused_bn_relu(shape, axes, with_residual, dtype):
     from flashlight_amd import ops
     rng = np.random.default_rng(len(shape) + shape[1] + int(with_residual))
-    lo = dtype == torch.bfloat16
-    rnd = bf16_round if lo else (lambda a: a)
+    lo = dtype != torch.float32
+    rnd = lambda a: round_to(a, dtype)
     x = rnd((rng.standard_normal(shape) * 1.5 + 0.3).astype(np.float32))
     res = rnd(rng.standard_normal(shape).astype(np.float32)) if with_residual else None
     dy = rnd(rng.standard_normal(shape).astype(np.float32))

@@ -7,12 +7,12 @@ import torch
 
 import flashlight_amd as fa
 from flashlight_amd import ops
-from gpu_util import bf16_round, dev, host
+from gpu_util import dev, host, round_to
 from oracle import flref
 from refmath import rel_l2
 
 pytestmark = pytest.mark.gpu
-DT = [torch.float32, torch.bfloat16]
+DT = [torch.float32, torch.bfloat16, torch.float16]
 
 
 def _tol(dtype):
@@ -20,7 +20,7 @@ def _tol(dtype):
 
 
 def _round(a, dtype):
-    return a if dtype == torch.float32 else bf16_round(a)
+    return round_to(a, dtype)
 
 
 @pytest.mark.parametrize("dtype", DT)
@@ -299,3 +299,24 @@ def test_astype_many_equals_astype():
     for m, b in zip(many, back):
         assert torch.equal(b, m.float())
     assert ops.astype_many([], torch.bfloat16) == []
+
+
+@pytest.mark.parametrize("src,dst", [(torch.float32, torch.float16), (torch.float16, torch.float32),
+                                     (torch.bfloat16, torch.float16), (torch.float16, torch.bfloat16),
+                                     (torch.float16, torch.float16)])
+def test_astype_with_f16(src, dst):
+    """Tensor::astype to and from f16 storage: round to nearest even, overflow to infinity, subnormal results,
+    NaN kept; between the two 16-bit types through the fp32 value."""
+    rng = np.random.default_rng(78)
+    v = rng.standard_normal(10007).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 10007).astype(np.float32)
+    v[:8] = [0.0, -0.0, np.inf, -np.inf, np.nan, 65504.0, 65520.0, 5.9604645e-8]
+    x = dev(v).to(src)
+    got = ops.astype(x, dst)
+    ref = x.float().to(dst)
+    assert got.dtype == dst
+    nan = torch.isnan(ref)
+    assert torch.equal(torch.isnan(got), nan) and int(nan.sum()) == 1
+    bits = torch.int32 if dst == torch.float32 else torch.int16
+    assert torch.equal(got.view(bits)[~nan], ref.view(bits)[~nan])
+    many = ops.astype_many([x, x[:5], x[:0]], dst)
+    assert torch.equal(many[0].float().nan_to_num(7.0), got.float().nan_to_num(7.0)) and many[2].numel() == 0

@@ -7,7 +7,7 @@ import pytest
 import torch
 
 import flashlight_amd as fa
-from gpu_util import bf16_round, dev, host
+from gpu_util import bf16_round, dev, host, round_to
 from oracle import flref
 from refmath import rel_l2
 from test_oracle_conv import CASES, LIB_CASES
@@ -133,13 +133,10 @@ def _run(case, seed, dtype):
     x = rng.standard_normal(xs).astype(np.float32)
     w = (rng.standard_normal(ws) / np.sqrt(ws[1] * ws[2] * ws[3])).astype(np.float32)
     b = rng.uniform(-1, 1, ws[0]).astype(np.float32)
-    if dtype == torch.bfloat16:
-        x, w = bf16_round(x), bf16_round(w)
+    x, w = round_to(x, dtype), round_to(w, dtype)
     d = flref.conv_desc(xs, ws, st, pd, dl, g)
     y_ref = flref.conv2d_fwd(d, x, w, b)
-    dy = rng.standard_normal(y_ref.shape).astype(np.float32)
-    if dtype == torch.bfloat16:
-        dy = bf16_round(dy)
+    dy = round_to(rng.standard_normal(y_ref.shape).astype(np.float32), dtype)
     dx_ref = flref.conv2d_bwd_data(d, dy, w)
     dw_ref, db_ref = flref.conv2d_bwd_filter(d, x, dy)
     kw = dict(sx=st[1], sy=st[0], px=pd[1], py=pd[0], dx=dl[1], dy=dl[0], groups=g)
@@ -169,6 +166,15 @@ def test_conv_bf16(case):
         # hide: inputs are exact in bf16 and sums are fp32, so fp32 results (dw, db) carry
         # only summation-order error, and bf16 results one rounding (2^-9 relative).
         tight = 1e-4 if name in ("dw", "db") else 4e-3
+        assert rel_l2(got, ref) <= tight, (name, rel_l2(got, ref))
+
+
+# f16 storage goes through the kernels that widen their operands to fp32 (the bf16 matrix-core families are
+# not taken): every case once, inputs exact in f16, fp32 sums, results rounded once (2^-12 relative).
+@pytest.mark.parametrize("case", ALL)
+def test_conv_f16(case):
+    for name, (got, ref) in _run(case, 37, torch.float16).items():
+        tight = 1e-4 if name in ("dw", "db") else 1e-3
         assert rel_l2(got, ref) <= tight, (name, rel_l2(got, ref))
 
 
@@ -354,7 +360,7 @@ def test_conv_bf16_3x3_stacked_images(case, stack):
         capi.set_option("CONV_STACK", None)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("shape", [
     ((3, 256, 14, 14), (136, 256, 1, 1), (1, 1), (0, 0)),  # bf16: tiles loaded straight to LDS, whole cells (196 positions)
     ((5, 128, 7, 7), (160, 128, 1, 1), (1, 1), (0, 0)),    # the same with planes of 49 (a plane's last cell repeats positions)

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import flashlight_amd as fa
-from gpu_util import bf16_round, dev, host
+from gpu_util import dev, host, round_to
 from oracle import flref
 from test_oracle_pool import GEOMS
 
@@ -59,18 +59,20 @@ def test_pool_f32_bit_exact(geom, mode):
     assert am2 is None and np.array_equal(host(y2), y_ref)
 
 
-@pytest.mark.parametrize("geom", [ALL[0], MORE[0], MORE[1]])
-@pytest.mark.parametrize("mode", [0, 2])
-def test_pool_bf16(geom, mode):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("geom", [ALL[0], MORE[0], MORE[1], MORE[4], MORE[12], MORE[14]])
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_pool_16bit_storage(geom, mode, dtype):
     xs, win, st, pd = geom
-    x = bf16_round(_x(xs, 42))
+    x = round_to(_x(xs, 42), dtype)
     d = flref.pool_desc(xs, win, st, pd, mode)
     y_ref, am_ref = flref.pool2d_fwd(d, x)
-    dy = bf16_round(np.random.default_rng(43).standard_normal(y_ref.shape))
+    dy = round_to(np.random.default_rng(43).standard_normal(y_ref.shape), dtype)
     dx_ref = flref.pool2d_bwd(d, dy, am_ref)
     args = (win[1], win[0], st[1], st[0], pd[1], pd[0])
-    y, am = fa.pool2d(dev(x, torch.bfloat16), *args, mode=mode)
-    dx = fa.pool2d_backward(dev(dy, torch.bfloat16), xs, am, *args, mode=mode)
+    y, am = fa.pool2d(dev(x, dtype), *args, mode=mode)
+    dx = fa.pool2d_backward(dev(dy, dtype), xs, am, *args, mode=mode)
+    assert y.dtype == dtype and dx.dtype == dtype
     if mode == 0:   # selection only: exact
         assert np.array_equal(host(y), y_ref) and np.array_equal(am.cpu().numpy(), am_ref)
     else:
