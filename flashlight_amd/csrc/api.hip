@@ -41,6 +41,7 @@ static bool apply_option(Options& o, const char* name, const char* v) {
       if (strstr(v, "wgrad128")) m |= Options::SKIP_WGRAD128;
       if (strstr(v, "pwdma")) m |= Options::SKIP_PWDMA;
       if (strstr(v, "wd32")) m |= Options::SKIP_WD32;
+      if (strstr(v, "tap1d")) m |= Options::SKIP_TAP1D;
     }
     o.conv_skip = m;
     return true;
@@ -70,6 +71,12 @@ static bool apply_option(Options& o, const char* name, const char* v) {
     o.conv_stack = n;
     return true;
   }
+  if (!strcmp(name, "SLAB_WAVES")) {
+    const int n = v ? atoi(v) : 0;
+    if (n != 0 && n != 4 && n != 8) return false;
+    o.slab_waves = n;
+    return true;
+  }
   if (!strcmp(name, "PW16_NO_TAPS")) return flag(&o.pw16_no_taps);
   if (!strcmp(name, "TAPPED_NO_REORDER")) return flag(&o.tapped_no_reorder);
   if (!strcmp(name, "MATMUL_VALU")) return flag(&o.matmul_valu);
@@ -78,7 +85,7 @@ static bool apply_option(Options& o, const char* name, const char* v) {
 }
 
 static void options_from_environment() {
-  static const char* const names[] = {"CONV_ALGO", "CONV_SKIP", "PW_PT", "PW16_PF", "CONV_STACK", "BN_ALGO", "PW16_NO_TAPS",
+  static const char* const names[] = {"CONV_ALGO", "CONV_SKIP", "PW_PT", "PW16_PF", "CONV_STACK", "SLAB_WAVES", "BN_ALGO", "PW16_NO_TAPS",
                                       "TAPPED_NO_REORDER", "MATMUL_VALU", "RNN_UNFUSED"};
   for (const char* n : names) {
     const std::string var = std::string("FLHIP_") + n;

@@ -114,6 +114,14 @@ int mfma_slab16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const 
                          hipStream_t s);
 int mfma_slab16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx,
                               hipStream_t s);
+// bf16 windows of one row (KH = 1, 2 to 32 taps, column stride 1 or 2, no groups, 16 to 256 contraction channels)
+// through channels-last rows and fragment-ordered weights in mfma_tap1d16_conv_ws() bytes of workspace
+// (conv2d_mfma_tap1d_bf16.hip); -1 when the shape is not theirs or the room is missing
+size_t mfma_tap1d16_conv_ws(const ConvGeom& g, bool bwd);
+int mfma_tap1d16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y, hipStream_t s,
+                          void* ws, size_t ws_bytes);
+int mfma_tap1d16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s, void* ws,
+                               size_t ws_bytes);
 // 3x3 filter gradient with operand rows copied straight to LDS (conv2d_mfma_wgrad_dma_bf16.hip)
 size_t mfma_wgrad_dma16_ws(const ConvGeom& g);
 // tile: 0 = by the measured rule, 32 / 64 = that tile side or decline

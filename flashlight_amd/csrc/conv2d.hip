@@ -212,7 +212,8 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
     const size_t a = mfma_tapped_ws(g, d->dtype, pass == FLHIP_CONV_BWD_DATA);
     const size_t b = d->dtype == FLHIP_BF16 ? mfma_pointwise16_lattice_ws(g, pass == FLHIP_CONV_BWD_DATA)
                                             : pass == FLHIP_CONV_BWD_DATA ? mfma_pointwise_split_ws(g, d->dtype, true) : 0;
-    return a > b ? a : b;
+    const size_t c = d->dtype == FLHIP_BF16 ? mfma_tap1d16_conv_ws(g, pass == FLHIP_CONV_BWD_DATA) : 0;
+    return std::max(a, std::max(b, c));
   }
   return 0;
 }
@@ -227,7 +228,9 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
   hipStream_t s = as_stream(stream);
   if (!force_direct()) {
     int r = -1;
-    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
+    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_TAP1D) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_tap1d16_conv_fwd(g, x, w, bias, y, s, ws, ws_bytes);
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pwd16_conv_fwd(g, x, w, bias, y, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pointwise16_conv_fwd(g, x, w, bias, y, s, ws, ws_bytes);
@@ -261,7 +264,7 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
 // family: the caller times them instead of trusting the rules.
 static const char* const kBwdDataPlans[] = {"bf16 1x1, tiles loaded straight to LDS", "bf16 1x1 / gathered taps", "bf16 3x3 strip",
                                             "bf16 slab", "1x1 GEMM, split contraction", "1x1 GEMM", "slab", "tapped GEMM",
-                                            "gather", "direct"};
+                                            "gather", "direct", "bf16 one-row windows"};
 static const char* const kBwdFilterPlans[] = {"bf16 3x3 rows straight to LDS, 32 x 32 tiles", "bf16 3x3 rows straight to LDS, 64 x 64 tiles",
                                               "bf16 1x1 / gathered taps", "bf16 first layer", "bf16 3x3 rows", "1x1 GEMM", "row slab",
                                               "tapped GEMM", "gather", "direct"};
@@ -301,13 +304,16 @@ static int bwd_data_impl(const flhip_conv_desc* d, const void* dy, const void* w
       case 6: r = mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s); break;
       case 7: r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes); break;
       case 8: r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s); break;
-      default: r = bwd_data_direct(d, g, dy, w, dx, s);
+      case 9: r = bwd_data_direct(d, g, dy, w, dx, s); break;
+      default: if (lo) r = mfma_tap1d16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes);
     }
     return r < 0 ? FLHIP_DECLINED : r;
   }
   if (!force_direct()) {
     int r = -1;
-    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
+    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_TAP1D) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_tap1d16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes);
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pwd16_conv_bwd_data(g, dy, w, nullptr, dx, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pointwise16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes);

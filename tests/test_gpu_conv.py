@@ -169,6 +169,41 @@ def test_conv_bf16(case):
         assert rel_l2(got, ref) <= tight, (name, rel_l2(got, ref))
 
 
+# bf16 windows of one row (KH = 1) on the kernels that read channels-last rows and fragment-ordered weights: the speech
+# stack's 21 x 1 windows at a short length (stride 1 and 2, 80 / 250 channels: padded contractions of 96 and 256), rows
+# per image > 1, an odd length with an even window over a stride of 2, more than 128 filters without padding, every
+# padded contraction size the kernels are compiled for (32, 64, 96, 128, 256), a tile's last positions past the row.
+ONE_ROW_CASES = [
+    ((3, 80, 1, 180), (250, 80, 1, 21), (1, 1), (0, 10), (1, 1), 1),
+    ((3, 250, 1, 180), (250, 250, 1, 21), (1, 2), (0, 10), (1, 1), 1),
+    ((2, 250, 1, 90), (250, 250, 1, 21), (1, 1), (0, 10), (1, 1), 1),
+    ((2, 32, 3, 50), (40, 32, 1, 5), (1, 1), (0, 2), (1, 1), 1),
+    ((2, 48, 1, 77), (33, 48, 1, 4), (1, 2), (0, 1), (1, 1), 1),
+    ((1, 16, 2, 200), (130, 16, 1, 7), (1, 1), (0, 0), (1, 1), 1),
+    ((2, 100, 1, 97), (70, 100, 1, 9), (1, 2), (0, 4), (1, 1), 1),
+    ((2, 130, 1, 64), (20, 130, 1, 3), (1, 1), (0, 1), (1, 1), 1),
+    ((2, 64, 2, 33), (64, 64, 1, 2), (1, 2), (0, 0), (1, 1), 1),
+    ((1, 24, 1, 300), (24, 24, 1, 32), (1, 1), (0, 15), (1, 1), 1),
+]
+
+
+@pytest.mark.parametrize("case", ONE_ROW_CASES)
+def test_conv_bf16_one_row_windows(case):
+    from flashlight_amd import capi
+    res = _run(case, 38, torch.bfloat16)
+    for name, (got, ref) in res.items():
+        tight = 1e-4 if name in ("dw", "db") else 4e-3
+        assert rel_l2(got, ref) <= tight, (name, rel_l2(got, ref))
+    # the same shapes with the family switched off (the kernels it replaced) agree with it to rounding
+    capi.set_option("CONV_SKIP", "tap1d")
+    try:
+        old = _run(case, 38, torch.bfloat16)
+    finally:
+        capi.set_option("CONV_SKIP", None)
+    for name in ("y", "dx"):
+        assert rel_l2(res[name][0], old[name][0]) <= 6e-3, name
+
+
 # f16 storage goes through the kernels that widen their operands to fp32 (the bf16 matrix-core families are
 # not taken): every case once, inputs exact in f16, fp32 sums, results rounded once (2^-12 relative).
 @pytest.mark.parametrize("case", ALL)
