@@ -122,6 +122,11 @@ int mfma_tap1d16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const
                           void* ws, size_t ws_bytes);
 int mfma_tap1d16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s, void* ws,
                                size_t ws_bytes);
+// their filter gradient (6 to 21 taps, an even number of result positions per row): the channels-last rows and the
+// workgroups' tiles in mfma_tap1d16_wgrad_ws() bytes of workspace
+size_t mfma_tap1d16_wgrad_ws(const ConvGeom& g);
+int mfma_tap1d16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes,
+                       hipStream_t s);
 // 3x3 filter gradient with operand rows copied straight to LDS (conv2d_mfma_wgrad_dma_bf16.hip)
 size_t mfma_wgrad_dma16_ws(const ConvGeom& g);
 // tile: 0 = by the measured rule, 32 / 64 = that tile side or decline

@@ -199,7 +199,9 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
     const size_t e = mfma_pointwise_wgrad_ws(g);
     const size_t f = d->dtype == FLHIP_BF16 ? mfma_pointwise16_wgrad_ws(g) : 0;
     const size_t h = d->dtype == FLHIP_BF16 ? mfma_first16_wgrad_ws(g) : 0;
+    const size_t t1 = d->dtype == FLHIP_BF16 ? mfma_tap1d16_wgrad_ws(g) : 0;
     if (h > a) a = h;
+    if (t1 > a) a = t1;
     if (b > a) a = b;
     if (e > a) a = e;
     if (f > a) a = f;
@@ -267,8 +269,8 @@ static const char* const kBwdDataPlans[] = {"bf16 1x1, tiles loaded straight to 
                                             "gather", "direct", "bf16 one-row windows"};
 static const char* const kBwdFilterPlans[] = {"bf16 3x3 rows straight to LDS, 32 x 32 tiles", "bf16 3x3 rows straight to LDS, 64 x 64 tiles",
                                               "bf16 1x1 / gathered taps", "bf16 first layer", "bf16 3x3 rows", "1x1 GEMM", "row slab",
-                                              "tapped GEMM", "gather", "direct"};
-constexpr int kNumPlans = 10;
+                                              "tapped GEMM", "gather", "direct", "bf16 one-row windows"};
+constexpr int kNumPlans = 11;
 
 static int bwd_data_direct(const flhip_conv_desc* d, const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s) {
   const size_t total = (size_t)g.N * g.C * g.H * g.W;
@@ -405,7 +407,7 @@ static int bwd_filter_impl(const flhip_conv_desc* d, const void* x, const void* 
   hipStream_t s = as_stream(stream);
   if (plan >= 0) {
     FLHIP_REQUIRE(plan < kNumPlans, "conv2d_bwd_filter: unknown plan");
-    if (plan == kNumPlans - 1) return bwd_filter_direct(d, g, x, dy, dw, db, s);
+    if (plan == 9) return bwd_filter_direct(d, g, x, dy, dw, db, s);
     const size_t need = flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER);
     FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter: workspace too small");
     const bool lo = d->dtype == FLHIP_BF16;
@@ -419,7 +421,8 @@ static int bwd_filter_impl(const flhip_conv_desc* d, const void* x, const void* 
       case 5: r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, false, s); break;
       case 6: r = mfma_slab_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s); break;
       case 7: r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, true, s); break;
-      default: r = mfma_conv_bwd_filter(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
+      case 8: r = mfma_conv_bwd_filter(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s); break;
+      default: if (lo && dw) r = mfma_tap1d16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);
     }
     return r < 0 ? FLHIP_DECLINED : r;
   }
@@ -429,7 +432,9 @@ static int bwd_filter_impl(const flhip_conv_desc* d, const void* x, const void* 
     int r = -1;
     // (3x3 stride 1 with rows copied straight to LDS first: it also takes the 7x7 planes that would otherwise go
     // through gathered taps below)
-    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
+    if (d->dtype == FLHIP_BF16 && dw && !skip(SK_BF16) && !skip(Options::SKIP_TAP1D) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_tap1d16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);
+    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_wgrad_dma16(g, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pointwise16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);

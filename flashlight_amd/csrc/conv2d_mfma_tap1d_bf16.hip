@@ -392,6 +392,243 @@ int run_conv(const ConvGeom& g, bool bwd, const void* src, const void* w, const 
   }
 }
 
+
+// ---- the filter gradient -------------------------------------------------------------------
+//   dw[k][c][j] = sum over sequences and positions o of dy[k][o] x[c][o*s + j - p],  db[k] = sum dy[k][o]
+// The contraction runs over positions, 16 per matrix instruction.  dy is read as it lies in
+// memory (a lane's 8 consecutive positions of one filter are 16 contiguous bytes, fetched
+// straight into registers a few steps ahead); x comes from the channels-last rows through LDS:
+// a tap shifts whole slab rows, and transposing reads (ds_read_b64_tr_b16) hand every lane its
+// 8 positions of one channel.  A workgroup (4 waves) owns 128 filters x 32 channels x every tap
+// over a range of positions of one sequence (or several such ranges in turn); wave
+// (kh, th) owns filters 64 kh .. + 63 and TW tap slots: th = 0 the taps 0 .. TW - 2 and, in its
+// last slot, the bias gradient (dy times a tile of ones); th = 1 the taps TW - 1 .. 2 TW - 2.
+// That is 2 x TW accumulator blocks per wave, one slab fragment per two matrix instructions.
+// The slab of a range (its positions and the window's reach, 32 channels) is copied to LDS by
+// the loads themselves before the range's first step; rows are 6 cells apart for stride 1 and
+// 5 for stride 2, which keeps the four rows of a transposing read on distinct banks.
+// The workgroups' tiles go to the workspace as [range set][tile][slot][128 filters][32 channels]
+// and tap1d16_wgrad_reduce_kernel adds them in a fixed order into dw's memory order.
+typedef short shortx4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) shortx4_t* lds_tr_t;
+
+struct Tap1WParams {
+  int rows, H;          // sequences, rows per image
+  int OW, TS;           // positions of dy / of the source per sequence
+  int Cs;               // channels of the channels-last source rows
+  int K, C, KW, px;
+  int tsplit, TL;       // ranges per sequence, positions per range (a multiple of 16)
+  int units, upw;       // ranges over all sequences, ranges per workgroup
+  int ktiles, ctiles;
+  int SRW;              // slab rows
+  unsigned src_bytes, dy_bytes;
+};
+
+template <int TW, int SS>
+__global__ void __launch_bounds__(256, 1)
+tap1d16_wgrad_kernel(Tap1WParams p, const bf16_t* __restrict__ xr, const bf16_t* __restrict__ dy, float* __restrict__ part) {
+  extern __shared__ uintx4_t t1_slab[];
+  constexpr int PC = SS == 1 ? 6 : 5;           // cells per slab row (4 used)
+  constexpr int PE = PC * 8;                    // the same in elements
+  constexpr int RD = 4;                         // steps between a dy fragment's load and its use
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kh = wave & 1, th = wave >> 1;
+  const int split = blockIdx.x, tile = blockIdx.y;
+  const int kt = tile / p.ctiles, ct = tile - kt * p.ctiles;
+  const intx4_t xrs = pd_rsrc(xr, p.src_bytes);
+  const __amdgpu_buffer_rsrc_t drs = make_rsrc(dy, p.dy_bytes);
+  const unsigned slab_addr = pd_lds_addr(t1_slab);
+  const int fr = lane & 31, fg = lane >> 5, fq = (lane >> 4) & 1, fs = lane & 15;
+
+  floatx16 acc[2][TW];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int t = 0; t < TW; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][t][r] = 0.f;
+  // a tile of ones for the bias slot
+  const uintx4_t ones = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+  const bool bias_wave = th == 0;
+
+  // this lane's first transposing read of a step: row SS * (fs / 4) (+ 8 SS fg), channels 16 fq + 4 (fs % 4) .. + 3,
+  // at the wave's first tap
+  const uint16_t* const slab16 = reinterpret_cast<const uint16_t*>(t1_slab);
+  const int blane = ((8 * fg + (fs >> 2)) * SS + th * (TW - 1)) * PE + 16 * fq + 4 * (fs & 3);
+
+  const int u0 = split * p.upw, u1 = min(u0 + p.upw, p.units);
+  for (int u = u0; u < u1; ++u) {
+    const int seq = u / p.tsplit, tr = u - seq * p.tsplit;
+    const int t0 = tr * p.TL, oend = min(p.OW, t0 + p.TL);
+    if (t0 >= oend) continue;
+    const int nsteps = (oend - t0 + 15) >> 4;
+    const int tailn = (oend - t0) & 15;         // positions of a last, partial step (0: none)
+    if (u != u0) __syncthreads();                // every wave is done with the previous slab
+    // ---- slab: row R holds source position t0 * SS - px + R, channels 32 ct .. + 31
+    {
+      const int ncell = p.SRW * PC, ninstr = (ncell + 63) >> 6;
+      const float inv = 1.0f / (float)PC;
+      const int sp0 = t0 * SS - p.px;
+      for (int ii = wave; ii < ninstr; ii += 4) {
+        const int L = ii * 64 + lane;
+        int c;
+        const int R = fast_div(L, PC, inv, &c);
+        const int sp = sp0 + R;
+        int voff = T1_OOB;
+        if (R < p.SRW && c < 4 && (unsigned)sp < (unsigned)p.TS) voff = ((seq * p.TS + sp) * p.Cs + ct * 32 + 8 * c) * 2;
+        pd_load_lds(xrs, slab_addr + ii * 1024, voff, 0);
+      }
+    }
+    // ---- dy: filters kt * 128 + kh * 64 + 32 a + fr, positions t0 + 16 step + 8 fg .. + 7
+    const int n = seq / p.H, h = seq - n * p.H;
+    int aoff[2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      const int k = kt * 128 + kh * 64 + a * 32 + fr;
+      aoff[a] = k < p.K ? ((((n * p.K + k) * p.H + h) * p.OW) + t0 + 8 * fg) * 2 : T1_OOB;
+    }
+    // the partial step's mask: elements at and past oend are zero
+    uint32_t tmask[4];
+    {
+      const int cnt = tailn ? tailn - 8 * fg : 8;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) tmask[d] = cnt >= 2 * d + 2 ? 0xffffffffu : cnt == 2 * d + 1 ? 0x0000ffffu : 0u;
+    }
+    uintx4_t aq[RD][2];
+#pragma unroll
+    for (int i = 0; i < RD; ++i)
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+        aq[i][a] = __builtin_amdgcn_raw_buffer_load_b128(drs, i < nsteps ? aoff[a] : T1_OOB, i * 32, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();                              // the slab has landed for every wave
+
+#define T1W_STEP(I)                                                                                       \
+  {                                                                                                       \
+    const int st = st0 + I;                                                                               \
+    if (st < nsteps) {                                                                                    \
+      uintx4_t a0 = aq[I][0], a1 = aq[I][1];                                                              \
+      _Pragma("unroll") for (int a = 0; a < 2; ++a)                                                       \
+        aq[I][a] = __builtin_amdgcn_raw_buffer_load_b128(drs, st + RD < nsteps ? aoff[a] : T1_OOB, (st + RD) * 32, 0); \
+      if (tailn && st == nsteps - 1) {                                                                    \
+        _Pragma("unroll") for (int d = 0; d < 4; ++d) { a0[d] &= tmask[d]; a1[d] &= tmask[d]; }           \
+      }                                                                                                   \
+      const bf16x8 fa0 = __builtin_bit_cast(bf16x8, a0), fa1 = __builtin_bit_cast(bf16x8, a1);            \
+      const uint16_t* bp = slab16 + blane + st * (16 * SS * PE);                                          \
+      _Pragma("unroll") for (int t = 0; t < TW; ++t) {                                                    \
+        const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(bp + t * PE));            \
+        const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(bp + t * PE + 4 * SS * PE)); \
+        const uintx2_t l2 = __builtin_bit_cast(uintx2_t, lo), h2 = __builtin_bit_cast(uintx2_t, hi);      \
+        uintx4_t b4 = {l2.x, l2.y, h2.x, h2.y};                                                           \
+        if (t == TW - 1 && bias_wave) b4 = ones;                                                          \
+        const bf16x8 fb = __builtin_bit_cast(bf16x8, b4);                                                 \
+        acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0, fb, acc[0][t], 0, 0, 0);                 \
+        acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1, fb, acc[1][t], 0, 0, 0);                 \
+      }                                                                                                   \
+    }                                                                                                     \
+  }
+    for (int st0 = 0; st0 < nsteps; st0 += RD) {
+      T1W_STEP(0) T1W_STEP(1) T1W_STEP(2) T1W_STEP(3)
+    }
+#undef T1W_STEP
+  }
+
+  // ---- the tile: element r of block (a, t): filter 64 kh + 32 a + 8 (r / 4) + 4 fg + r % 4, channel fr
+  float* out = part + ((size_t)(split * (p.ktiles * p.ctiles) + tile) * (2 * TW) + th * TW) * 4096;
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int t = 0; t < TW; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int kl = kh * 64 + a * 32 + (r >> 2) * 8 + fg * 4 + (r & 3);
+        out[t * 4096 + kl * 32 + fr] = acc[a][t][r];
+      }
+}
+
+// dw[k][c][j] and db[k] from the tiles of nsplit range sets, added in the order of the sets.
+// Slot g of a tile: tap g for g < TW - 1, the bias gradient for g = TW - 1, tap g - 1 beyond.
+__global__ void __launch_bounds__(256)
+tap1d16_wgrad_reduce_kernel(const float* __restrict__ part, int nsplit, int tiles, int ctiles, int TW, int K, int C, int KW,
+                            float* __restrict__ dw, float* __restrict__ db) {
+  const int e = blockIdx.x * 256 + threadIdx.x;   // element of a slot: filter e / 32, channel e % 32
+  const int g = blockIdx.y, tile = blockIdx.z;
+  const int kt = tile / ctiles, ct = tile - kt * ctiles;
+  const int k = kt * 128 + (e >> 5), c = ct * 32 + (e & 31);
+  const bool is_bias = g == TW - 1;
+  const int j = g < TW - 1 ? g : g - 1;
+  if (k >= K) return;
+  if (is_bias ? (ct != 0 || (e & 31) != 0 || !db) : (c >= C || j >= KW || !dw)) return;
+  const size_t stride = (size_t)tiles * (2 * TW) * 4096;
+  const float* src = part + ((size_t)tile * (2 * TW) + g) * 4096 + e;
+  float sum = 0.f;
+  int s = 0;
+  for (; s + 4 <= nsplit; s += 4) {
+    const float v0 = src[(size_t)s * stride], v1 = src[(size_t)(s + 1) * stride], v2 = src[(size_t)(s + 2) * stride],
+                v3 = src[(size_t)(s + 3) * stride];
+    sum += v0; sum += v1; sum += v2; sum += v3;
+  }
+  for (; s < nsplit; ++s) sum += src[(size_t)s * stride];
+  if (is_bias) db[k] = sum;
+  else dw[((size_t)k * C + c) * KW + j] = sum;
+}
+
+struct Tap1WPlan {
+  Tap1WParams p;
+  int TW, SS, nsplit;
+  size_t rows_bytes, part_bytes, lds_bytes;
+};
+
+bool tap1d_wgrad_plan(const ConvGeom& g, Tap1WPlan* pl) {
+  if (g.KH != 1 || g.py != 0 || g.sy != 1 || g.dlx != 1 || g.groups != 1) return false;
+  if (g.KW < 6 || g.KW > 21 || (g.sx != 1 && g.sx != 2)) return false;
+  if (g.OH != g.H || (long long)g.N * g.H > 65535 || g.OW % 2 != 0 || g.C < 16 || g.K < 32) return false;
+  Tap1WParams& p = pl->p;
+  std::memset(&p, 0, sizeof p);
+  const int need = (g.KW + 2) / 2;              // 2 TW - 1 >= KW
+  const int TW = need <= 4 ? 4 : need <= 6 ? 6 : need <= 8 ? 8 : 11;
+  pl->TW = TW; pl->SS = g.sx;
+  p.rows = g.N * g.H; p.H = g.H; p.OW = g.OW; p.TS = g.W;
+  p.Cs = (g.C + 31) / 32 * 32;
+  p.K = g.K; p.C = g.C; p.KW = g.KW; p.px = g.px;
+  p.ktiles = (g.K + 127) / 128; p.ctiles = p.Cs / 32;
+  const int tiles = p.ktiles * p.ctiles;
+  const int PC = g.sx == 1 ? 6 : 5;
+  // ranges: enough workgroups for the chip; a range's slab must fit in LDS
+  const int want = (mfma_num_cus() + tiles - 1) / tiles;
+  int tsplit = std::max(1, (want + p.rows - 1) / p.rows);
+  for (;; ++tsplit) {
+    p.TL = ((g.OW + tsplit - 1) / tsplit + 15) / 16 * 16;
+    p.SRW = (p.TL - 1) * g.sx + 2 * TW - 1;
+    pl->lds_bytes = (size_t)(((long long)p.SRW * PC + 63) / 64) * 1024;
+    if (pl->lds_bytes <= 150 * 1024) break;
+    if (p.TL <= 16) return false;
+  }
+  p.tsplit = (g.OW + p.TL - 1) / p.TL;
+  p.units = p.rows * p.tsplit;
+  p.upw = std::max(1, p.units / std::max(1, want));
+  pl->nsplit = (p.units + p.upw - 1) / p.upw;
+  const long long rb = (long long)p.rows * p.TS * p.Cs * 2;
+  const long long yb = (long long)g.N * g.K * g.H * g.OW * 2;
+  if (rb >= (1ll << 31) || yb >= (1ll << 31)) return false;
+  p.src_bytes = (unsigned)rb; p.dy_bytes = (unsigned)yb;
+  pl->rows_bytes = ((size_t)rb + 255) & ~(size_t)255;
+  pl->part_bytes = (size_t)pl->nsplit * tiles * (2 * TW) * 4096 * sizeof(float);
+  return true;
+}
+
+template <int TW>
+int launch_wgrad(const Tap1WPlan& pl, const bf16_t* xr, const bf16_t* dy, float* part, hipStream_t s) {
+  const dim3 grid((unsigned)pl.nsplit, (unsigned)(pl.p.ktiles * pl.p.ctiles));
+  auto go = [&](auto kernel) {
+    if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), pl.lds_bytes)) return -1;
+    hipLaunchKernelGGL(kernel, grid, dim3(256), pl.lds_bytes, s, pl.p, xr, dy, part);
+    return check_launch("conv2d_bwd_filter (bf16 one-row windows)");
+  };
+  return pl.SS == 2 ? go(tap1d16_wgrad_kernel<TW, 2>) : go(tap1d16_wgrad_kernel<TW, 1>);
+}
+
 }  // namespace
 
 size_t mfma_tap1d16_conv_ws(const ConvGeom& g, bool bwd) {
@@ -407,6 +644,42 @@ int mfma_tap1d16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const
 int mfma_tap1d16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s, void* ws,
                                size_t ws_bytes) {
   return run_conv(g, true, dy, w, nullptr, dx, s, ws, ws_bytes);
+}
+
+}  // namespace flhip
+
+namespace flhip {
+
+size_t mfma_tap1d16_wgrad_ws(const ConvGeom& g) {
+  Tap1WPlan pl;
+  return tap1d_wgrad_plan(g, &pl) ? pl.rows_bytes + pl.part_bytes : 0;
+}
+
+int mfma_tap1d16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes,
+                       hipStream_t s) {
+  Tap1WPlan pl;
+  if (!tap1d_wgrad_plan(g, &pl)) return -1;
+  if (!ws || ws_bytes < pl.rows_bytes + pl.part_bytes) return -1;
+  bf16_t* xr = static_cast<bf16_t*>(ws);
+  float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + pl.rows_bytes);
+  {
+    const dim3 grid((unsigned)((g.W + 63) / 64), (unsigned)(pl.p.Cs / 32), (unsigned)pl.p.rows);
+    hipLaunchKernelGGL(tap1d16_rows_kernel, grid, dim3(256), 0, s, static_cast<const bf16_t*>(x), xr, g.C, g.H, g.W, pl.p.Cs);
+    if (const int rc = check_launch("conv2d_bwd_filter (bf16 one-row windows, rows pass)")) return rc;
+  }
+  const bf16_t* dyp = static_cast<const bf16_t*>(dy);
+  int rc;
+  switch (pl.TW) {
+    case 4: rc = launch_wgrad<4>(pl, xr, dyp, part, s); break;
+    case 6: rc = launch_wgrad<6>(pl, xr, dyp, part, s); break;
+    case 8: rc = launch_wgrad<8>(pl, xr, dyp, part, s); break;
+    default: rc = launch_wgrad<11>(pl, xr, dyp, part, s); break;
+  }
+  if (rc) return rc;
+  const int tiles = pl.p.ktiles * pl.p.ctiles;
+  hipLaunchKernelGGL(tap1d16_wgrad_reduce_kernel, dim3(16, (unsigned)(2 * pl.TW), (unsigned)tiles), dim3(256), 0, s, part, pl.nsplit,
+                     tiles, pl.p.ctiles, pl.TW, g.K, g.C, g.KW, dw, db);
+  return check_launch("conv2d_bwd_filter (bf16 one-row windows, sum)");
 }
 
 }  // namespace flhip

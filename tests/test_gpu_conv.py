@@ -184,6 +184,14 @@ ONE_ROW_CASES = [
     ((2, 130, 1, 64), (20, 130, 1, 3), (1, 1), (0, 1), (1, 1), 1),
     ((2, 64, 2, 33), (64, 64, 1, 2), (1, 2), (0, 0), (1, 1), 1),
     ((1, 24, 1, 300), (24, 24, 1, 32), (1, 1), (0, 15), (1, 1), 1),
+    # their filter gradient (6 to 21 taps, even row lengths): every tap-slot count it is compiled for (4, 6, 8, 11), a last
+    # step of 2 and of 10 positions, filters and channels that are not multiples of the tile, several ranges per row,
+    # several ranges per workgroup, two rows per image, stride 2
+    ((2, 40, 1, 98), (64, 40, 1, 6), (1, 1), (0, 2), (1, 1), 1),
+    ((3, 33, 2, 90), (150, 33, 1, 11), (1, 1), (0, 5), (1, 1), 1),
+    ((2, 64, 1, 400), (32, 64, 1, 15), (1, 2), (0, 7), (1, 1), 1),
+    ((1, 96, 1, 1000), (40, 96, 1, 16), (1, 1), (0, 8), (1, 1), 1),
+    ((40, 250, 1, 64), (250, 250, 1, 21), (1, 1), (0, 10), (1, 1), 1),
 ]
 
 
