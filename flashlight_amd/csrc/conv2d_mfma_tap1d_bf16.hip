@@ -131,7 +131,7 @@ tap1d16_weights_kernel(const bf16_t* __restrict__ w, uintx4_t* __restrict__ wf, 
 }
 
 // ---- the convolution ---------------------------------------------------------------------
-// KS k-steps per tap; DT taps per unrolled group (DT * KS >= 16 stages: the distance between a
+// KS k-steps per tap; DT taps per unrolled group (DT * KS = 12 or 16 stages: the distance between a
 // weight fragment's load and its use); SS source stride; NPH phases.
 template <int KS, int DT, int SS, int NPH>
 __global__ void __launch_bounds__(256, 1)
@@ -193,28 +193,48 @@ tap1d16_conv_kernel(Tap1Params p, const bf16_t* __restrict__ xr, const uintx4_t*
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the slab (and the first weight fragments) have landed
   __syncthreads();
 
+  // The position fragments of a stage are read two stages ahead of their use (four sets of registers in rotation;
+  // a group's stage count is a multiple of four).
   auto run = [&](floatx16 (&ac)[T1_NB], int q) __attribute__((always_inline)) {
+    constexpr int NS = DT * KS;
+    static_assert(NS % 4 == 0 && KS >= 2, "the fragment sets rotate with the unrolled group");
     const int groups = p.ntaps[q] / DT;
     const int dq = p.d0[q], last = p.nreal[q] - 1;
+    // slab offset (cells) of a tap's rows; padding taps read the rows of the last tap that exists: finite values
+    // times zero weights
+    auto toff_of = [&](int tap) {
+      const int d = dq + min(tap, last);
+      const int trow = SS == 1 ? d : (d & 1) * p.half + (d >> 1);
+      return trow * CPR;
+    };
+    uintx4_t af[4][T1_NB];
+    int tcur[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) tcur[dt] = toff_of(dt);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int b = 0; b < T1_NB; ++b) af[i][b] = ap[b][tcur[i / KS] + 2 * (i % KS)];
     for (int g = 0; g < groups; ++g) {
+      int tnext[DT];
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        // padding taps read the rows of the last tap that exists: finite values times zero weights
-        const int d = dq + min(g * DT + dt, last);
-        const int trow = SS == 1 ? d : (d & 1) * p.half + (d >> 1);
-        const int toff = trow * CPR;
+      for (int dt = 0; dt < DT; ++dt) tnext[dt] = toff_of((g + 1) * DT + dt);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          bf16x8 a[T1_NB];
+      for (int i = 0; i < NS; ++i) {
+        const int i2 = i + 2;
+        const int o2 = i2 < NS ? tcur[(i2 % NS) / KS] : tnext[(i2 % NS) / KS];
 #pragma unroll
-          for (int b = 0; b < T1_NB; ++b) a[b] = __builtin_bit_cast(bf16x8, ap[b][toff + 2 * ks]);
-          const bf16x8 w8 = __builtin_bit_cast(bf16x8, bq[dt][ks]);
-          bq[dt][ks] = __builtin_amdgcn_raw_buffer_load_b128(wrs, wlane, wpos + (dt * KS + ks) * 1024, 0);
+        for (int b = 0; b < T1_NB; ++b) af[i2 % 4][b] = ap[b][o2 + 2 * ((i2 % NS) % KS)];
+        const bf16x8 w8 = __builtin_bit_cast(bf16x8, bq[i / KS][i % KS]);
+        bq[i / KS][i % KS] = __builtin_amdgcn_raw_buffer_load_b128(wrs, wlane, wpos + i * 1024, 0);
 #pragma unroll
-          for (int b = 0; b < T1_NB; ++b) ac[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[b], w8, ac[b], 0, 0, 0);
-        }
+        for (int b = 0; b < T1_NB; ++b)
+          ac[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[i % 4][b]), w8, ac[b], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);     // (the scheduler would otherwise move every read down to its use)
       }
-      wpos += DT * KS * 1024;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) tcur[dt] = tnext[dt];
+      wpos += NS * 1024;
     }
   };
   run(acc[0], 0);
@@ -265,7 +285,14 @@ struct Tap1Plan {
   int C, H, T;           // of the source tensor, for the rows pass
 };
 
-int dt_of(int KS) { return KS >= 16 ? 1 : KS >= 8 ? 2 : KS == 6 ? 3 : KS == 4 ? 4 : KS == 2 ? 8 : 0; }
+// channels of the channels-last rows: the count padded to one the convolution kernels are compiled for
+int tap1d_cs(int C) {
+  for (int c : {32, 64, 96, 128, 256})
+    if (C <= c) return c;
+  return 0;
+}
+
+int dt_of(int KS) { return KS >= 16 ? 1 : KS >= 8 ? 2 : KS == 6 ? 2 : KS == 4 ? 4 : KS == 2 ? 8 : 0; }
 
 // bwd = false: forward; true: backward-data
 bool tap1d_plan(const ConvGeom& g, bool bwd, Tap1Plan* pl) {
@@ -274,9 +301,7 @@ bool tap1d_plan(const ConvGeom& g, bool bwd, Tap1Plan* pl) {
   if (g.OH != g.H || (long long)g.N * g.H > 65535) return false;
   const int Cc = bwd ? g.K : g.C, Mo = bwd ? g.C : g.K;
   // contraction channels padded to a count the kernel is compiled for
-  int Cs = 0;
-  for (int c : {32, 64, 96, 128, 256})
-    if (Cc <= c) { Cs = c; break; }
+  const int Cs = tap1d_cs(Cc);
   if (!Cs || Cc < 16) return false;
   const int KS = Cs / 16, DT = dt_of(KS);
   Tap1Params& p = pl->p;
@@ -386,7 +411,7 @@ int run_conv(const ConvGeom& g, bool bwd, const void* src, const void* w, const 
   switch (pl.p.KS) {
     case 2: return launch_conv<2, 8>(pl, xr, wf, bias, out, s);
     case 4: return launch_conv<4, 4>(pl, xr, wf, bias, out, s);
-    case 6: return launch_conv<6, 3>(pl, xr, wf, bias, out, s);
+    case 6: return launch_conv<6, 2>(pl, xr, wf, bias, out, s);
     case 8: return launch_conv<8, 2>(pl, xr, wf, bias, out, s);
     default: return launch_conv<16, 1>(pl, xr, wf, bias, out, s);
   }
@@ -399,15 +424,16 @@ int run_conv(const ConvGeom& g, bool bwd, const void* src, const void* w, const 
 // memory (a lane's 8 consecutive positions of one filter are 16 contiguous bytes, fetched
 // straight into registers a few steps ahead); x comes from the channels-last rows through LDS:
 // a tap shifts whole slab rows, and transposing reads (ds_read_b64_tr_b16) hand every lane its
-// 8 positions of one channel.  A workgroup (4 waves) owns 128 filters x 32 channels x every tap
-// over a range of positions of one sequence (or several such ranges in turn); wave
-// (kh, th) owns filters 64 kh .. + 63 and TW tap slots: th = 0 the taps 0 .. TW - 2 and, in its
-// last slot, the bias gradient (dy times a tile of ones); th = 1 the taps TW - 1 .. 2 TW - 2.
-// That is 2 x TW accumulator blocks per wave, one slab fragment per two matrix instructions.
+// 8 positions of one channel.  A workgroup (4 waves) owns 64 filters x 32 channels x every tap
+// over a range of positions of one sequence (or several such ranges in turn); wave w owns the
+// slots w TQ .. w TQ + TQ - 1 of both filter blocks, slot g being tap g for g < KW, the bias
+// gradient (dy times a tile of ones) for g = KW and unused beyond: 2 x TQ accumulator blocks
+// per wave (at most 192 registers, so they stay in the accumulator file), one slab fragment
+// per two matrix instructions.
 // The slab of a range (its positions and the window's reach, 32 channels) is copied to LDS by
 // the loads themselves before the range's first step; rows are 6 cells apart for stride 1 and
 // 5 for stride 2, which keeps the four rows of a transposing read on distinct banks.
-// The workgroups' tiles go to the workspace as [range set][tile][slot][128 filters][32 channels]
+// The workgroups' tiles go to the workspace as [range set][tile][slot][64 filters][32 channels]
 // and tap1d16_wgrad_reduce_kernel adds them in a fixed order into dw's memory order.
 typedef short shortx4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) shortx4_t* lds_tr_t;
@@ -424,7 +450,7 @@ struct Tap1WParams {
   unsigned src_bytes, dy_bytes;
 };
 
-template <int TW, int SS>
+template <int TQ, int SS>
 __global__ void __launch_bounds__(256, 1)
 tap1d16_wgrad_kernel(Tap1WParams p, const bf16_t* __restrict__ xr, const bf16_t* __restrict__ dy, float* __restrict__ part) {
   extern __shared__ uintx4_t t1_slab[];
@@ -433,7 +459,6 @@ tap1d16_wgrad_kernel(Tap1WParams p, const bf16_t* __restrict__ xr, const bf16_t*
   constexpr int RD = 4;                         // steps between a dy fragment's load and its use
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int kh = wave & 1, th = wave >> 1;
   const int split = blockIdx.x, tile = blockIdx.y;
   const int kt = tile / p.ctiles, ct = tile - kt * p.ctiles;
   const intx4_t xrs = pd_rsrc(xr, p.src_bytes);
@@ -441,21 +466,21 @@ tap1d16_wgrad_kernel(Tap1WParams p, const bf16_t* __restrict__ xr, const bf16_t*
   const unsigned slab_addr = pd_lds_addr(t1_slab);
   const int fr = lane & 31, fg = lane >> 5, fq = (lane >> 4) & 1, fs = lane & 15;
 
-  floatx16 acc[2][TW];
+  floatx16 acc[2][TQ];
 #pragma unroll
   for (int a = 0; a < 2; ++a)
 #pragma unroll
-    for (int t = 0; t < TW; ++t)
+    for (int t = 0; t < TQ; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][t][r] = 0.f;
   // a tile of ones for the bias slot
   const uintx4_t ones = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
-  const bool bias_wave = th == 0;
+  const int bias_slot = p.KW - wave * TQ;       // this wave's slot index of the bias gradient (outside 0 .. TQ - 1: none)
 
   // this lane's first transposing read of a step: row SS * (fs / 4) (+ 8 SS fg), channels 16 fq + 4 (fs % 4) .. + 3,
   // at the wave's first tap
   const uint16_t* const slab16 = reinterpret_cast<const uint16_t*>(t1_slab);
-  const int blane = ((8 * fg + (fs >> 2)) * SS + th * (TW - 1)) * PE + 16 * fq + 4 * (fs & 3);
+  const int blane = ((8 * fg + (fs >> 2)) * SS + wave * TQ) * PE + 16 * fq + 4 * (fs & 3);
 
   const int u0 = split * p.upw, u1 = min(u0 + p.upw, p.units);
   for (int u = u0; u < u1; ++u) {
@@ -480,12 +505,12 @@ tap1d16_wgrad_kernel(Tap1WParams p, const bf16_t* __restrict__ xr, const bf16_t*
         pd_load_lds(xrs, slab_addr + ii * 1024, voff, 0);
       }
     }
-    // ---- dy: filters kt * 128 + kh * 64 + 32 a + fr, positions t0 + 16 step + 8 fg .. + 7
+    // ---- dy: filters kt * 64 + 32 a + fr, positions t0 + 16 step + 8 fg .. + 7
     const int n = seq / p.H, h = seq - n * p.H;
     int aoff[2];
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
-      const int k = kt * 128 + kh * 64 + a * 32 + fr;
+      const int k = kt * 64 + a * 32 + fr;
       aoff[a] = k < p.K ? ((((n * p.K + k) * p.H + h) * p.OW) + t0 + 8 * fg) * 2 : T1_OOB;
     }
     // the partial step's mask: elements at and past oend are zero
@@ -504,6 +529,15 @@ tap1d16_wgrad_kernel(Tap1WParams p, const bf16_t* __restrict__ xr, const bf16_t*
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();                              // the slab has landed for every wave
 
+    // the slab fragment of slot t + 1 is read while slot t is multiplied (the first slot of a step behind the last
+    // of the step before)
+    auto bread = [&](const uint16_t* at) __attribute__((always_inline)) {
+      const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)at);
+      const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(at + 4 * SS * PE));
+      const uintx2_t l2 = __builtin_bit_cast(uintx2_t, lo), h2 = __builtin_bit_cast(uintx2_t, hi);
+      return uintx4_t{l2.x, l2.y, h2.x, h2.y};
+    };
+    uintx4_t bnext = bread(slab16 + blane);
 #define T1W_STEP(I)                                                                                       \
   {                                                                                                       \
     const int st = st0 + I;                                                                               \
@@ -516,15 +550,14 @@ tap1d16_wgrad_kernel(Tap1WParams p, const bf16_t* __restrict__ xr, const bf16_t*
       }                                                                                                   \
       const bf16x8 fa0 = __builtin_bit_cast(bf16x8, a0), fa1 = __builtin_bit_cast(bf16x8, a1);            \
       const uint16_t* bp = slab16 + blane + st * (16 * SS * PE);                                          \
-      _Pragma("unroll") for (int t = 0; t < TW; ++t) {                                                    \
-        const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(bp + t * PE));            \
-        const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(bp + t * PE + 4 * SS * PE)); \
-        const uintx2_t l2 = __builtin_bit_cast(uintx2_t, lo), h2 = __builtin_bit_cast(uintx2_t, hi);      \
-        uintx4_t b4 = {l2.x, l2.y, h2.x, h2.y};                                                           \
-        if (t == TW - 1 && bias_wave) b4 = ones;                                                          \
+      _Pragma("unroll") for (int t = 0; t < TQ; ++t) {                                                    \
+        uintx4_t b4 = bnext;                                                                              \
+        bnext = bread(t + 1 < TQ ? bp + (t + 1) * PE : bp + 16 * SS * PE);                                \
+        if (t == bias_slot) b4 = ones;                                                                    \
         const bf16x8 fb = __builtin_bit_cast(bf16x8, b4);                                                 \
         acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0, fb, acc[0][t], 0, 0, 0);                 \
         acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1, fb, acc[1][t], 0, 0, 0);                 \
+        __builtin_amdgcn_sched_barrier(0);                                                                \
       }                                                                                                   \
     }                                                                                                     \
   }
@@ -534,34 +567,35 @@ tap1d16_wgrad_kernel(Tap1WParams p, const bf16_t* __restrict__ xr, const bf16_t*
 #undef T1W_STEP
   }
 
-  // ---- the tile: element r of block (a, t): filter 64 kh + 32 a + 8 (r / 4) + 4 fg + r % 4, channel fr
-  float* out = part + ((size_t)(split * (p.ktiles * p.ctiles) + tile) * (2 * TW) + th * TW) * 4096;
+  // ---- the tile: element r of block (a, t): filter 32 a + 8 (r / 4) + 4 fg + r % 4, channel fr
+  float* out = part + ((size_t)(split * (p.ktiles * p.ctiles) + tile) * (4 * TQ) + wave * TQ) * 2048;
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+  for (int t = 0; t < TQ; ++t) {
+    if (wave * TQ + t > p.KW) continue;          // an unused slot
 #pragma unroll
-    for (int t = 0; t < TW; ++t)
+    for (int a = 0; a < 2; ++a)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int kl = kh * 64 + a * 32 + (r >> 2) * 8 + fg * 4 + (r & 3);
-        out[t * 4096 + kl * 32 + fr] = acc[a][t][r];
+        const int kl = a * 32 + (r >> 2) * 8 + fg * 4 + (r & 3);
+        out[t * 2048 + kl * 32 + fr] = acc[a][t][r];
       }
+  }
 }
 
 // dw[k][c][j] and db[k] from the tiles of nsplit range sets, added in the order of the sets.
-// Slot g of a tile: tap g for g < TW - 1, the bias gradient for g = TW - 1, tap g - 1 beyond.
+// Slot g of a tile: tap g for g < KW, the bias gradient for g = KW.
 __global__ void __launch_bounds__(256)
-tap1d16_wgrad_reduce_kernel(const float* __restrict__ part, int nsplit, int tiles, int ctiles, int TW, int K, int C, int KW,
+tap1d16_wgrad_reduce_kernel(const float* __restrict__ part, int nsplit, int tiles, int ctiles, int slots, int K, int C, int KW,
                             float* __restrict__ dw, float* __restrict__ db) {
   const int e = blockIdx.x * 256 + threadIdx.x;   // element of a slot: filter e / 32, channel e % 32
   const int g = blockIdx.y, tile = blockIdx.z;
   const int kt = tile / ctiles, ct = tile - kt * ctiles;
-  const int k = kt * 128 + (e >> 5), c = ct * 32 + (e & 31);
-  const bool is_bias = g == TW - 1;
-  const int j = g < TW - 1 ? g : g - 1;
+  const int k = kt * 64 + (e >> 5), c = ct * 32 + (e & 31);
+  const bool is_bias = g == KW;
   if (k >= K) return;
-  if (is_bias ? (ct != 0 || (e & 31) != 0 || !db) : (c >= C || j >= KW || !dw)) return;
-  const size_t stride = (size_t)tiles * (2 * TW) * 4096;
-  const float* src = part + ((size_t)tile * (2 * TW) + g) * 4096 + e;
+  if (is_bias ? (ct != 0 || (e & 31) != 0 || !db) : (c >= C || !dw)) return;
+  const size_t stride = (size_t)tiles * slots * 2048;
+  const float* src = part + ((size_t)tile * slots + g) * 2048 + e;
   float sum = 0.f;
   int s = 0;
   for (; s + 4 <= nsplit; s += 4) {
@@ -571,28 +605,28 @@ tap1d16_wgrad_reduce_kernel(const float* __restrict__ part, int nsplit, int tile
   }
   for (; s < nsplit; ++s) sum += src[(size_t)s * stride];
   if (is_bias) db[k] = sum;
-  else dw[((size_t)k * C + c) * KW + j] = sum;
+  else dw[((size_t)k * C + c) * KW + g] = sum;
 }
 
 struct Tap1WPlan {
   Tap1WParams p;
-  int TW, SS, nsplit;
+  int TQ, SS, nsplit;
   size_t rows_bytes, part_bytes, lds_bytes;
 };
 
 bool tap1d_wgrad_plan(const ConvGeom& g, Tap1WPlan* pl) {
   if (g.KH != 1 || g.py != 0 || g.sy != 1 || g.dlx != 1 || g.groups != 1) return false;
-  if (g.KW < 6 || g.KW > 21 || (g.sx != 1 && g.sx != 2)) return false;
+  if (g.KW < 6 || g.KW > 23 || (g.sx != 1 && g.sx != 2)) return false;
   if (g.OH != g.H || (long long)g.N * g.H > 65535 || g.OW % 2 != 0 || g.C < 16 || g.K < 32) return false;
   Tap1WParams& p = pl->p;
   std::memset(&p, 0, sizeof p);
-  const int need = (g.KW + 2) / 2;              // 2 TW - 1 >= KW
-  const int TW = need <= 4 ? 4 : need <= 6 ? 6 : need <= 8 ? 8 : 11;
-  pl->TW = TW; pl->SS = g.sx;
+  const int TQ = (g.KW + 1 + 3) / 4;            // KW taps and the bias gradient over four waves
+  pl->TQ = TQ; pl->SS = g.sx;
   p.rows = g.N * g.H; p.H = g.H; p.OW = g.OW; p.TS = g.W;
-  p.Cs = (g.C + 31) / 32 * 32;
+  p.Cs = tap1d_cs(g.C);
+  if (!p.Cs) return false;
   p.K = g.K; p.C = g.C; p.KW = g.KW; p.px = g.px;
-  p.ktiles = (g.K + 127) / 128; p.ctiles = p.Cs / 32;
+  p.ktiles = (g.K + 63) / 64; p.ctiles = (g.C + 31) / 32;
   const int tiles = p.ktiles * p.ctiles;
   const int PC = g.sx == 1 ? 6 : 5;
   // ranges: enough workgroups for the chip; a range's slab must fit in LDS
@@ -600,7 +634,7 @@ bool tap1d_wgrad_plan(const ConvGeom& g, Tap1WPlan* pl) {
   int tsplit = std::max(1, (want + p.rows - 1) / p.rows);
   for (;; ++tsplit) {
     p.TL = ((g.OW + tsplit - 1) / tsplit + 15) / 16 * 16;
-    p.SRW = (p.TL - 1) * g.sx + 2 * TW - 1;
+    p.SRW = (p.TL - 1) * g.sx + 4 * TQ;
     pl->lds_bytes = (size_t)(((long long)p.SRW * PC + 63) / 64) * 1024;
     if (pl->lds_bytes <= 150 * 1024) break;
     if (p.TL <= 16) return false;
@@ -614,11 +648,11 @@ bool tap1d_wgrad_plan(const ConvGeom& g, Tap1WPlan* pl) {
   if (rb >= (1ll << 31) || yb >= (1ll << 31)) return false;
   p.src_bytes = (unsigned)rb; p.dy_bytes = (unsigned)yb;
   pl->rows_bytes = ((size_t)rb + 255) & ~(size_t)255;
-  pl->part_bytes = (size_t)pl->nsplit * tiles * (2 * TW) * 4096 * sizeof(float);
+  pl->part_bytes = (size_t)pl->nsplit * tiles * (4 * TQ) * 2048 * sizeof(float);
   return true;
 }
 
-template <int TW>
+template <int TQ>
 int launch_wgrad(const Tap1WPlan& pl, const bf16_t* xr, const bf16_t* dy, float* part, hipStream_t s) {
   const dim3 grid((unsigned)pl.nsplit, (unsigned)(pl.p.ktiles * pl.p.ctiles));
   auto go = [&](auto kernel) {
@@ -626,7 +660,7 @@ int launch_wgrad(const Tap1WPlan& pl, const bf16_t* xr, const bf16_t* dy, float*
     hipLaunchKernelGGL(kernel, grid, dim3(256), pl.lds_bytes, s, pl.p, xr, dy, part);
     return check_launch("conv2d_bwd_filter (bf16 one-row windows)");
   };
-  return pl.SS == 2 ? go(tap1d16_wgrad_kernel<TW, 2>) : go(tap1d16_wgrad_kernel<TW, 1>);
+  return pl.SS == 2 ? go(tap1d16_wgrad_kernel<TQ, 2>) : go(tap1d16_wgrad_kernel<TQ, 1>);
 }
 
 }  // namespace
@@ -669,16 +703,17 @@ int mfma_tap1d16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* 
   }
   const bf16_t* dyp = static_cast<const bf16_t*>(dy);
   int rc;
-  switch (pl.TW) {
+  switch (pl.TQ) {
+    case 2: rc = launch_wgrad<2>(pl, xr, dyp, part, s); break;
+    case 3: rc = launch_wgrad<3>(pl, xr, dyp, part, s); break;
     case 4: rc = launch_wgrad<4>(pl, xr, dyp, part, s); break;
-    case 6: rc = launch_wgrad<6>(pl, xr, dyp, part, s); break;
-    case 8: rc = launch_wgrad<8>(pl, xr, dyp, part, s); break;
-    default: rc = launch_wgrad<11>(pl, xr, dyp, part, s); break;
+    case 5: rc = launch_wgrad<5>(pl, xr, dyp, part, s); break;
+    default: rc = launch_wgrad<6>(pl, xr, dyp, part, s); break;
   }
   if (rc) return rc;
   const int tiles = pl.p.ktiles * pl.p.ctiles;
-  hipLaunchKernelGGL(tap1d16_wgrad_reduce_kernel, dim3(16, (unsigned)(2 * pl.TW), (unsigned)tiles), dim3(256), 0, s, part, pl.nsplit,
-                     tiles, pl.p.ctiles, pl.TW, g.K, g.C, g.KW, dw, db);
+  hipLaunchKernelGGL(tap1d16_wgrad_reduce_kernel, dim3(8, (unsigned)(g.KW + 1), (unsigned)tiles), dim3(256), 0, s, part, pl.nsplit,
+                     tiles, pl.p.ctiles, 4 * pl.TQ, g.K, g.C, g.KW, dw, db);
   return check_launch("conv2d_bwd_filter (bf16 one-row windows, sum)");
 }
 
