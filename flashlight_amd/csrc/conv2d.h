@@ -126,7 +126,10 @@ int mfma_tap1d16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w,
 // workgroups' tiles in mfma_tap1d16_wgrad_ws() bytes of workspace
 size_t mfma_tap1d16_wgrad_ws(const ConvGeom& g);
 int mfma_tap1d16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes,
-                       hipStream_t s);
+                       hipStream_t s, const void* rows = nullptr);
+// bytes of channels-last rows that their forward pass leaves at the start of its workspace and the filter gradient
+// takes as `rows` in place of x (0: the two passes do not both apply)
+size_t mfma_tap1d16_rows_bytes(const ConvGeom& g);
 // 3x3 filter gradient with operand rows copied straight to LDS (conv2d_mfma_wgrad_dma_bf16.hip)
 size_t mfma_wgrad_dma16_ws(const ConvGeom& g);
 // tile: 0 = by the measured rule, 32 / 64 = that tile side or decline

@@ -473,6 +473,8 @@ static bool gathered_path(const flhip_conv_desc* d) {
 extern "C" size_t flhip_conv2d_gathered_bytes(const flhip_conv_desc* d) {
   ConvGeom g;
   if (!d || make_geom(d, &g) != FLHIP_OK || !gathered_path(d)) return 0;
+  // one-row windows: the forward pass's channels-last rows (that family runs first where it applies)
+  if (!skip(Options::SKIP_TAP1D) && mfma_tap1d16_conv_ws(g, false) > 0) return mfma_tap1d16_rows_bytes(g);
   return mfma_pointwise16_gathered_bytes(g);
 }
 
@@ -482,11 +484,13 @@ extern "C" int flhip_conv2d_bwd_filter_gathered(const flhip_conv_desc* d, const 
   ConvGeom g;
   const int rc = make_geom(d, &g);
   if (rc != FLHIP_OK) return rc;
-  FLHIP_REQUIRE(gathered_path(d) && mfma_pointwise16_gathered_bytes(g) > 0,
+  FLHIP_REQUIRE(flhip_conv2d_gathered_bytes(d) > 0,
                 "conv2d_bwd_filter_gathered: this geometry's forward pass leaves no gathered input");
   const size_t need = flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER);
   FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter_gathered: workspace too small");
-  const int r = mfma_pointwise16_wgrad(g, nullptr, dy, dw, db, ws, ws_bytes, as_stream(stream), gathered);
+  const bool one_row = !skip(Options::SKIP_TAP1D) && mfma_tap1d16_conv_ws(g, false) > 0;
+  const int r = one_row ? mfma_tap1d16_wgrad(g, nullptr, dy, dw, db, ws, ws_bytes, as_stream(stream), gathered)
+                        : mfma_pointwise16_wgrad(g, nullptr, dy, dw, db, ws, ws_bytes, as_stream(stream), gathered);
   if (r < 0) return fail(FLHIP_INVALID_ARGUMENT, "conv2d_bwd_filter_gathered: no kernel takes the gathered input of this geometry");
   return r;
 }

@@ -73,26 +73,52 @@ struct Tap1Params {
 };
 
 // ---- operand passes ------------------------------------------------------------------------
-// x[n][c][h][t] -> xr[n * H + h][t][Cs], channels c >= C zero.  A block transposes 32 channels x 64
-// positions through LDS.
+// x[n][c][h][t] -> xr[n * H + h][t][Cs], channels c >= C zero.  A block transposes 64 channels x 64
+// positions through LDS: pairs of positions in (rows of an even length start on 4-byte boundaries), whole 16-byte
+// cells of 8 channels out.
+template <bool PAIRS>
 __global__ void __launch_bounds__(256)
 tap1d16_rows_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ xr, int C, int H, int T, int Cs) {
-  __shared__ uint16_t tile[32][66];
-  const int t0 = blockIdx.x * 64, c0 = blockIdx.y * 32, row = blockIdx.z;
+  __shared__ uint16_t tile[64][66];
+  const int t0 = blockIdx.x * 64, c0 = blockIdx.y * 64, row = blockIdx.z;
   const int n = row / H, h = row - n * H;
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  if (PAIRS) {
+    const int tp = threadIdx.x & 31, cy = threadIdx.x >> 5;      // pair of positions, channel (+ 8 i)
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int c = c0 + ty + 4 * i, t = t0 + tx;
-    tile[ty + 4 * i][tx] = (c < C && t < T) ? x[(((size_t)n * C + c) * H + h) * T + t] : (uint16_t)0;
+    for (int i = 0; i < 8; ++i) {
+      const int c = c0 + cy + 8 * i, t = t0 + 2 * tp;
+      uint32_t v = 0u;
+      if (c < C && t < T) v = *reinterpret_cast<const uint32_t*>(x + (((size_t)n * C + c) * H + h) * T + t);   // (T is even)
+      *reinterpret_cast<uint32_t*>(&tile[cy + 8 * i][2 * tp]) = v;
+    }
+  } else {
+    const int tx = threadIdx.x & 63, cy = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int c = c0 + cy + 4 * i, t = t0 + tx;
+      tile[cy + 4 * i][tx] = (c < C && t < T) ? x[(((size_t)n * C + c) * H + h) * T + t] : (uint16_t)0;
+    }
   }
   __syncthreads();
-  const int cx = threadIdx.x & 31, tyy = threadIdx.x >> 5;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int t = t0 + tyy + 8 * i;
-    if (t < T && c0 + cx < Cs) xr[((size_t)row * T + t) * Cs + c0 + cx] = tile[cx][tyy + 8 * i];
+  for (int i = 0; i < 2; ++i) {
+    const int item = threadIdx.x + 256 * i, cell = item & 7, tl = item >> 3;
+    const int t = t0 + tl, c = c0 + 8 * cell;
+    if (t < T && c < Cs) {
+      uint32_t v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = (uint32_t)tile[8 * cell + 2 * e][tl] | ((uint32_t)tile[8 * cell + 2 * e + 1][tl] << 16);
+      *reinterpret_cast<uintx4_t*>(xr + ((size_t)row * T + t) * Cs + c) = uintx4_t{v[0], v[1], v[2], v[3]};
+    }
   }
+}
+
+static void launch_rows(const bf16_t* x, bf16_t* xr, int C, int H, int T, int Cs, int rows, hipStream_t s) {
+  const dim3 grid((unsigned)((T + 63) / 64), (unsigned)((Cs + 63) / 64), (unsigned)rows);
+  if (T % 2 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0)
+    hipLaunchKernelGGL(tap1d16_rows_kernel<true>, grid, dim3(256), 0, s, x, xr, C, H, T, Cs);
+  else
+    hipLaunchKernelGGL(tap1d16_rows_kernel<false>, grid, dim3(256), 0, s, x, xr, C, H, T, Cs);
 }
 
 struct Tap1Weights {
@@ -397,10 +423,7 @@ int run_conv(const ConvGeom& g, bool bwd, const void* src, const void* w, const 
   if (!ws || ws_bytes < pl.rows_bytes + pl.w_bytes) return -1;
   bf16_t* xr = static_cast<bf16_t*>(ws);
   uintx4_t* wf = reinterpret_cast<uintx4_t*>(static_cast<char*>(ws) + pl.rows_bytes);
-  {
-    const dim3 grid((unsigned)((pl.T + 63) / 64), (unsigned)(pl.p.Cs / 32), (unsigned)pl.p.rows);
-    hipLaunchKernelGGL(tap1d16_rows_kernel, grid, dim3(256), 0, s, static_cast<const bf16_t*>(src), xr, pl.C, pl.H, pl.T, pl.p.Cs);
-  }
+  launch_rows(static_cast<const bf16_t*>(src), xr, pl.C, pl.H, pl.T, pl.p.Cs, pl.p.rows, s);
   {
     const long long total = (long long)pl.w.mblocks * pl.w.taps_total * pl.w.KS * 64;
     hipLaunchKernelGGL(tap1d16_weights_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
@@ -689,16 +712,21 @@ size_t mfma_tap1d16_wgrad_ws(const ConvGeom& g) {
   return tap1d_wgrad_plan(g, &pl) ? pl.rows_bytes + pl.part_bytes : 0;
 }
 
+size_t mfma_tap1d16_rows_bytes(const ConvGeom& g) {
+  Tap1Plan f;
+  Tap1WPlan w;
+  return tap1d_plan(g, false, &f) && tap1d_wgrad_plan(g, &w) && f.rows_bytes == w.rows_bytes ? w.rows_bytes : 0;
+}
+
 int mfma_tap1d16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes,
-                       hipStream_t s) {
+                       hipStream_t s, const void* rows) {
   Tap1WPlan pl;
   if (!tap1d_wgrad_plan(g, &pl)) return -1;
   if (!ws || ws_bytes < pl.rows_bytes + pl.part_bytes) return -1;
-  bf16_t* xr = static_cast<bf16_t*>(ws);
+  const bf16_t* xr = static_cast<const bf16_t*>(rows ? rows : ws);
   float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + pl.rows_bytes);
-  {
-    const dim3 grid((unsigned)((g.W + 63) / 64), (unsigned)(pl.p.Cs / 32), (unsigned)pl.p.rows);
-    hipLaunchKernelGGL(tap1d16_rows_kernel, grid, dim3(256), 0, s, static_cast<const bf16_t*>(x), xr, g.C, g.H, g.W, pl.p.Cs);
+  if (!rows) {
+    launch_rows(static_cast<const bf16_t*>(x), static_cast<bf16_t*>(ws), g.C, g.H, g.W, pl.p.Cs, pl.p.rows, s);
     if (const int rc = check_launch("conv2d_bwd_filter (bf16 one-row windows, rows pass)")) return rc;
   }
   const bf16_t* dyp = static_cast<const bf16_t*>(dy);

@@ -568,6 +568,37 @@ def test_bf16_filter_gradient_from_the_forward_pass_gather(shape, with_bias):
         assert rel_l2(host(db1), ref_db) <= 2e-3
 
 
+@pytest.mark.parametrize("shape", [((3, 80, 1, 180), (250, 80, 1, 21), (1, 1), (0, 10)),
+                                   ((3, 250, 1, 180), (250, 250, 1, 21), (1, 2), (0, 10)),
+                                   ((2, 32, 3, 50), (40, 32, 1, 5), (1, 1), (0, 2))])        # 5 taps: that filter gradient declines
+def test_bf16_one_row_filter_gradient_from_the_forward_pass_rows(shape):
+    """One-row windows: the forward pass leaves its channels-last rows at the start of its workspace; the filter
+    gradient computed from them equals the one that makes the rows again, bit for bit."""
+    import ctypes as C
+    from flashlight_amd import capi
+    xs, ws_, st, pd = shape
+    rng = np.random.default_rng(92)
+    x = dev(bf16_round(rng.standard_normal(xs).astype(np.float32))).to(torch.bfloat16)
+    w = dev(bf16_round((rng.standard_normal(ws_) / 20).astype(np.float32))).to(torch.bfloat16)
+    kw = dict(sx=st[1], sy=st[0], px=pd[1], py=pd[0], dx=1, dy=1, groups=1)
+    y, rows = fa.conv2d(x, w, None, keep_gathered=True, **kw)
+    assert torch.equal(y, fa.conv2d(x, w, None, **kw))
+    if ws_[3] < 6:
+        assert rows is None
+        return
+    cs = 96 if xs[1] == 80 else 256
+    assert rows is not None and rows.numel() >= xs[0] * xs[2] * xs[3] * cs * 2
+    # the rows are the input with its channels last, padded with zeros
+    r = rows[:xs[0] * xs[2] * xs[3] * cs * 2].view(torch.bfloat16).view(xs[0], xs[2], xs[3], cs)
+    assert torch.equal(r[..., :xs[1]], x.permute(0, 2, 3, 1)) and not bool(r[..., xs[1]:].any())
+    dy = dev(bf16_round(rng.standard_normal(tuple(y.shape)).astype(np.float32))).to(torch.bfloat16)
+    dw0, db0 = fa.conv2d_backward_filter_bias(dy, x, ws_, True, **kw)
+    kept = rows.clone()
+    dw1, db1 = fa.conv2d_backward_filter_bias(dy, x, ws_, True, gathered=kept, **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(dw1, dw0) and torch.equal(db1, db0)
+
+
 def _random_cases(n, seed):
     """Seeded random geometries biased towards the conditions the kernel families key on:
     1x1 and 3x3 windows, even / odd rows, planes of 4k positions, channel counts around the
