@@ -114,22 +114,22 @@ int mfma_slab16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const 
                          hipStream_t s);
 int mfma_slab16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx,
                               hipStream_t s);
-// bf16 windows of one row (KH = 1, 2 to 32 taps, column stride 1 or 2, no groups, 16 to 256 contraction channels)
-// through channels-last rows and fragment-ordered weights in mfma_tap1d16_conv_ws() bytes of workspace
-// (conv2d_mfma_tap1d_bf16.hip); -1 when the shape is not theirs or the room is missing
-size_t mfma_tap1d16_conv_ws(const ConvGeom& g, bool bwd);
-int mfma_tap1d16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y, hipStream_t s,
-                          void* ws, size_t ws_bytes);
-int mfma_tap1d16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s, void* ws,
-                               size_t ws_bytes);
-// their filter gradient (6 to 21 taps, an even number of result positions per row): the channels-last rows and the
-// workgroups' tiles in mfma_tap1d16_wgrad_ws() bytes of workspace
-size_t mfma_tap1d16_wgrad_ws(const ConvGeom& g);
-int mfma_tap1d16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes,
-                       hipStream_t s, const void* rows = nullptr);
+// windows of one row (KH = 1, 2 to 32 taps, column stride 1 or 2, no groups, 16 to 256 contraction channels) in bf16
+// or fp32 storage through channels-last rows and fragment-ordered weights in mfma_tap1d_conv_ws() bytes of workspace
+// (conv2d_mfma_tap1d.hip); -1 when the shape is not theirs or the room is missing
+size_t mfma_tap1d_conv_ws(const ConvGeom& g, int dtype, bool bwd);
+int mfma_tap1d_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w, const float* bias, void* y, hipStream_t s,
+                        void* ws, size_t ws_bytes);
+int mfma_tap1d_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx, hipStream_t s, void* ws,
+                             size_t ws_bytes);
+// their filter gradient (6 to 23 taps; bf16: an even number of result positions per row): the channels-last rows and
+// the workgroups' tiles in mfma_tap1d_wgrad_ws() bytes of workspace
+size_t mfma_tap1d_wgrad_ws(const ConvGeom& g, int dtype);
+int mfma_tap1d_wgrad(const ConvGeom& g, int dtype, const void* x, const void* dy, float* dw, float* db, void* ws,
+                     size_t ws_bytes, hipStream_t s, const void* rows = nullptr);
 // bytes of channels-last rows that their forward pass leaves at the start of its workspace and the filter gradient
 // takes as `rows` in place of x (0: the two passes do not both apply)
-size_t mfma_tap1d16_rows_bytes(const ConvGeom& g);
+size_t mfma_tap1d_rows_bytes(const ConvGeom& g, int dtype);
 // 3x3 filter gradient with operand rows copied straight to LDS (conv2d_mfma_wgrad_dma_bf16.hip)
 size_t mfma_wgrad_dma16_ws(const ConvGeom& g);
 // tile: 0 = by the measured rule, 32 / 64 = that tile side or decline

@@ -141,6 +141,12 @@ static const unsigned SK_BF16 = Options::SKIP_BF16, SK_GEMM = Options::SKIP_GEMM
 // measures faster than the tapped GEMM, except for backward-data into few channels.
 // With its weights reordered (workspace present) the tapped GEMM wins from 128 contraction
 // channels on.
+// the one-row-window kernels take this storage type (bf16: unless the bf16 families are switched off or converted)
+static bool tap1d_on(int dtype) {
+  if (force_direct() || skip(Options::SKIP_TAP1D)) return false;
+  return dtype == FLHIP_F32 || (dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT));
+}
+
 static bool long_rows(const ConvGeom& g, int dtype, bool bwd, size_t ws_bytes) {
   if (algo_is(Options::ALGO_TAPPED)) return false;
   const size_t need = mfma_tapped_ws(g, dtype, bwd);
@@ -199,7 +205,7 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
     const size_t e = mfma_pointwise_wgrad_ws(g);
     const size_t f = d->dtype == FLHIP_BF16 ? mfma_pointwise16_wgrad_ws(g) : 0;
     const size_t h = d->dtype == FLHIP_BF16 ? mfma_first16_wgrad_ws(g) : 0;
-    const size_t t1 = d->dtype == FLHIP_BF16 ? mfma_tap1d16_wgrad_ws(g) : 0;
+    const size_t t1 = mfma_tap1d_wgrad_ws(g, d->dtype);
     if (h > a) a = h;
     if (t1 > a) a = t1;
     if (b > a) a = b;
@@ -214,7 +220,7 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
     const size_t a = mfma_tapped_ws(g, d->dtype, pass == FLHIP_CONV_BWD_DATA);
     const size_t b = d->dtype == FLHIP_BF16 ? mfma_pointwise16_lattice_ws(g, pass == FLHIP_CONV_BWD_DATA)
                                             : pass == FLHIP_CONV_BWD_DATA ? mfma_pointwise_split_ws(g, d->dtype, true) : 0;
-    const size_t c = d->dtype == FLHIP_BF16 ? mfma_tap1d16_conv_ws(g, pass == FLHIP_CONV_BWD_DATA) : 0;
+    const size_t c = mfma_tap1d_conv_ws(g, d->dtype, pass == FLHIP_CONV_BWD_DATA);
     return std::max(a, std::max(b, c));
   }
   return 0;
@@ -230,8 +236,7 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
   hipStream_t s = as_stream(stream);
   if (!force_direct()) {
     int r = -1;
-    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_TAP1D) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_tap1d16_conv_fwd(g, x, w, bias, y, s, ws, ws_bytes);
+    if (tap1d_on(d->dtype)) r = mfma_tap1d_conv_fwd(g, d->dtype, x, w, bias, y, s, ws, ws_bytes);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pwd16_conv_fwd(g, x, w, bias, y, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
@@ -266,10 +271,10 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
 // family: the caller times them instead of trusting the rules.
 static const char* const kBwdDataPlans[] = {"bf16 1x1, tiles loaded straight to LDS", "bf16 1x1 / gathered taps", "bf16 3x3 strip",
                                             "bf16 slab", "1x1 GEMM, split contraction", "1x1 GEMM", "slab", "tapped GEMM",
-                                            "gather", "direct", "bf16 one-row windows"};
+                                            "gather", "direct", "one-row windows"};
 static const char* const kBwdFilterPlans[] = {"bf16 3x3 rows straight to LDS, 32 x 32 tiles", "bf16 3x3 rows straight to LDS, 64 x 64 tiles",
                                               "bf16 1x1 / gathered taps", "bf16 first layer", "bf16 3x3 rows", "1x1 GEMM", "row slab",
-                                              "tapped GEMM", "gather", "direct", "bf16 one-row windows"};
+                                              "tapped GEMM", "gather", "direct", "one-row windows"};
 constexpr int kNumPlans = 11;
 
 static int bwd_data_direct(const flhip_conv_desc* d, const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s) {
@@ -307,14 +312,13 @@ static int bwd_data_impl(const flhip_conv_desc* d, const void* dy, const void* w
       case 7: r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes); break;
       case 8: r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s); break;
       case 9: r = bwd_data_direct(d, g, dy, w, dx, s); break;
-      default: if (lo) r = mfma_tap1d16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes);
+      default: r = mfma_tap1d_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
     }
     return r < 0 ? FLHIP_DECLINED : r;
   }
   if (!force_direct()) {
     int r = -1;
-    if (d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_TAP1D) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_tap1d16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes);
+    if (tap1d_on(d->dtype)) r = mfma_tap1d_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pwd16_conv_bwd_data(g, dy, w, nullptr, dx, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
@@ -422,7 +426,7 @@ static int bwd_filter_impl(const flhip_conv_desc* d, const void* x, const void* 
       case 6: r = mfma_slab_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s); break;
       case 7: r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, true, s); break;
       case 8: r = mfma_conv_bwd_filter(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s); break;
-      default: if (lo && dw) r = mfma_tap1d16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);
+      default: if (dw) r = mfma_tap1d_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
     }
     return r < 0 ? FLHIP_DECLINED : r;
   }
@@ -432,8 +436,7 @@ static int bwd_filter_impl(const flhip_conv_desc* d, const void* x, const void* 
     int r = -1;
     // (3x3 stride 1 with rows copied straight to LDS first: it also takes the 7x7 planes that would otherwise go
     // through gathered taps below)
-    if (d->dtype == FLHIP_BF16 && dw && !skip(SK_BF16) && !skip(Options::SKIP_TAP1D) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_tap1d16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);
+    if (dw && tap1d_on(d->dtype)) r = mfma_tap1d_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_wgrad_dma16(g, x, dy, dw, db, ws, ws_bytes, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
@@ -472,10 +475,10 @@ static bool gathered_path(const flhip_conv_desc* d) {
 
 extern "C" size_t flhip_conv2d_gathered_bytes(const flhip_conv_desc* d) {
   ConvGeom g;
-  if (!d || make_geom(d, &g) != FLHIP_OK || !gathered_path(d)) return 0;
-  // one-row windows: the forward pass's channels-last rows (that family runs first where it applies)
-  if (!skip(Options::SKIP_TAP1D) && mfma_tap1d16_conv_ws(g, false) > 0) return mfma_tap1d16_rows_bytes(g);
-  return mfma_pointwise16_gathered_bytes(g);
+  if (!d || make_geom(d, &g) != FLHIP_OK) return 0;
+  // one-row windows (bf16 and fp32): the forward pass's channels-last rows (that family runs first where it applies)
+  if (tap1d_on(d->dtype) && mfma_tap1d_conv_ws(g, d->dtype, false) > 0) return mfma_tap1d_rows_bytes(g, d->dtype);
+  return gathered_path(d) ? mfma_pointwise16_gathered_bytes(g) : 0;
 }
 
 extern "C" int flhip_conv2d_bwd_filter_gathered(const flhip_conv_desc* d, const void* gathered, const void* dy,
@@ -488,8 +491,8 @@ extern "C" int flhip_conv2d_bwd_filter_gathered(const flhip_conv_desc* d, const 
                 "conv2d_bwd_filter_gathered: this geometry's forward pass leaves no gathered input");
   const size_t need = flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER);
   FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter_gathered: workspace too small");
-  const bool one_row = !skip(Options::SKIP_TAP1D) && mfma_tap1d16_conv_ws(g, false) > 0;
-  const int r = one_row ? mfma_tap1d16_wgrad(g, nullptr, dy, dw, db, ws, ws_bytes, as_stream(stream), gathered)
+  const bool one_row = tap1d_on(d->dtype) && mfma_tap1d_conv_ws(g, d->dtype, false) > 0;
+  const int r = one_row ? mfma_tap1d_wgrad(g, d->dtype, nullptr, dy, dw, db, ws, ws_bytes, as_stream(stream), gathered)
                         : mfma_pointwise16_wgrad(g, nullptr, dy, dw, db, ws, ws_bytes, as_stream(stream), gathered);
   if (r < 0) return fail(FLHIP_INVALID_ARGUMENT, "conv2d_bwd_filter_gathered: no kernel takes the gathered input of this geometry");
   return r;

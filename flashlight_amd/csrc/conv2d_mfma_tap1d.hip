@@ -1,37 +1,41 @@
 // Convolutions with one-row windows (KH = 1, KW taps along the contiguous axis: the 21 x 1
-// windows of a wav2letter-style speech stack) in bf16 storage on v_mfma_f32_32x32x16_bf16,
-// forward and backward-data, column stride 1 or 2.
+// windows of a wav2letter-style speech stack) on the matrix cores, forward, backward-data and
+// filter gradient, column stride 1 or 2; bf16 storage on v_mfma_f32_32x32x16_bf16 and fp32 on
+// v_mfma_f32_32x32x2_f32 (the same kernels compiled for either element type).
 //
 //   forward        y[m][o]  = sum_c sum_j w[m][c][j]  x[c][o*s + j - p]   (+ bias[m])
 //   backward-data  dx[c][u] = sum_m sum_j w[m][c][j] dy[m][(u + p - j) / s]   where s divides
 //
-// A matrix instruction wants eight consecutive contraction channels of one position per
-// lane, and every tap shifts the positions by one element: with the tensors as they lie in
-// memory (channel-major rows of positions) a shifted 16-byte fragment would start on any
-// 2-byte boundary.  So two small passes first bring the operands into the order the
-// instruction reads:
+// A matrix instruction wants consecutive contraction channels of one position per lane, and
+// every tap shifts the positions by one element: with the tensors as they lie in memory
+// (channel-major rows of positions) a shifted 16-byte fragment would start on any element
+// boundary.  So two small passes first bring the operands into the order the instruction reads:
 //   rows     xr[sequence][position][Cs]: the source with its channels last, Cs = the channel
-//            count padded with zeros to a multiple of 16 (tap1d16_rows_kernel; a sequence is
-//            one (image, row) pair); a tap then shifts whole 16-byte cells;
-//   weights  wf[block of 32 result channels][tap][k-step of 16 channels][lane][8]: the
-//            fragment of every (tap, k-step) exactly as the 64 lanes hold it, in the order
-//            the kernel walks (tap1d16_weights_kernel); padded channels and taps are zero.
+//            count padded with zeros (tap1d_rows_kernel; a sequence is one (image, row) pair); a
+//            tap then shifts whole 16-byte cells (8 bf16 or 4 fp32 channels of one position);
+//   weights  wf[block of 32 result channels][tap][stage of 2 cells][lane][cell]: the fragment
+//            of every (tap, stage) exactly as the 64 lanes hold it, in the order the kernel walks
+//            (tap1d_weights_kernel); padded channels and taps are zero.
+// A stage is 16 bf16 channels (one matrix instruction per block) or 8 fp32 channels (four
+// instructions of 2 channels each: lane half h holds channels 4 h .. 4 h + 3 of the stage and
+// instruction e multiplies element e of both operands, so the four cover the stage).
 // Backward-data over a stride of 2 is two interleaved stride-1 problems (the results of even
 // and of odd index take the taps of one parity each): "phases" of one workgroup, which
 // writes both so that its stores cover whole runs of dx.
 //
-// A workgroup (4 waves) owns 96 result positions (per phase) of one sequence x 128 result
-// channels; wave w owns channels 32 w .. 32 w + 31: three (six) accumulator blocks of 32 x 32.
-//   * The source rows the tile needs (96 positions + the window's reach, every channel) are
+// A workgroup (4 waves) owns 32 NB result positions (per phase; NB = 3, or 2 where the slab of 3
+// would not fit) of one sequence x 128 result channels; wave w owns channels 32 w .. 32 w + 31:
+// NB (2 NB) accumulator blocks of 32 x 32.
+//   * The source rows the tile needs (its positions + the window's reach, every channel) are
 //     copied to LDS once, by buffer loads with the LDS modifier (no registers, no vector
-//     instructions); a row of the slab is Cs / 8 cells + 1 unused cell, which puts the eight
+//     instructions); a row of the slab is its cells + 1 unused cell, which puts the eight
 //     lanes of a 16-byte read cycle on distinct banks.  With a forward stride of 2 the slab
 //     keeps even and odd source positions apart, so a tap's 32 positions are consecutive rows.
-//   * The weights never pass through LDS: a wave's fragment of a (tap, k-step) is 1 KiB of
-//     contiguous memory, fetched straight into registers 16 stages ahead of its use.  No other
+//   * The weights never pass through LDS: a wave's fragment of a (tap, stage) is 1 KiB of
+//     contiguous memory, fetched straight into registers RW stages ahead of its use.  No other
 //     wave needs it, so the main loop has no barrier.
-//   * Per stage (16 channels of one tap) a wave reads 3 position fragments from LDS and
-//     issues 3 matrix instructions.
+//   * Per stage a wave reads NB position fragments from LDS (two stages ahead of their use) and
+//     issues NB (bf16) or 4 NB (fp32) matrix instructions.
 // Positions are the rows of the instruction tile: a lane holds 4 consecutive positions of one
 // result channel (8 with two phases), stored as one piece.
 #include <algorithm>
@@ -51,15 +55,28 @@ typedef const uintx4_t* lds_cell_t;
 #endif
 
 constexpr int T1_BM = 128;       // result channels per workgroup
-constexpr int T1_NB = 3;         // blocks of 32 positions per wave and phase
-constexpr int T1_TP = 32 * T1_NB;
 constexpr int T1_MAXTAPS = 64;   // taps over both phases, padding included
 constexpr int T1_OOB = (int)0x80000000;
+
+// element type -> channels per 16-byte cell; a stage is two cells
+template <typename T> struct Tap1Elem;
+template <> struct Tap1Elem<bf16_t> { static constexpr int CELL = 8; };
+template <> struct Tap1Elem<float> { static constexpr int CELL = 4; };
+
+// one stage of one block: acc += a (positions x stage channels) * w (stage channels x result channels)
+__device__ __forceinline__ void tap1d_mma(floatx16& acc, const uintx4_t& a, const uintx4_t& w, const bf16_t*) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, w), acc, 0, 0, 0);
+}
+__device__ __forceinline__ void tap1d_mma(floatx16& acc, const uintx4_t& a, const uintx4_t& w, const float*) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a[e]), __uint_as_float(w[e]), acc, 0, 0, 0);
+}
 
 struct Tap1Params {
   int rows, H;           // sequences (images x rows), rows per image
   int TS, TO, TOu;       // source positions, result indices per phase, result positions per sequence
-  int Cs, KS;            // padded contraction channels, Cs / 16
+  int Cs, KS;            // padded contraction channels, stages per tap
   int Mo;                // result channels
   int nph;               // phases (1; 2: results u = 2 o + q)
   int ntaps[2];          // taps per phase as stored (a multiple of the kernel's tap group)
@@ -74,21 +91,22 @@ struct Tap1Params {
 
 // ---- operand passes ------------------------------------------------------------------------
 // x[n][c][h][t] -> xr[n * H + h][t][Cs], channels c >= C zero.  A block transposes 64 channels x 64
-// positions through LDS: pairs of positions in (rows of an even length start on 4-byte boundaries), whole 16-byte
-// cells of 8 channels out.
-template <bool PAIRS>
+// positions through LDS: (bf16: pairs of positions in, where rows of an even length start on 4-byte
+// boundaries;) whole 16-byte cells out.
+template <typename T, bool PAIRS>
 __global__ void __launch_bounds__(256)
-tap1d16_rows_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ xr, int C, int H, int T, int Cs) {
-  __shared__ uint16_t tile[64][66];
+tap1d_rows_kernel(const T* __restrict__ x, T* __restrict__ xr, int C, int H, int Tn, int Cs) {
+  constexpr int CELL = Tap1Elem<T>::CELL;
+  __shared__ T tile[64][sizeof(T) == 2 ? 66 : 65];
   const int t0 = blockIdx.x * 64, c0 = blockIdx.y * 64, row = blockIdx.z;
   const int n = row / H, h = row - n * H;
-  if (PAIRS) {
+  if (PAIRS && sizeof(T) == 2) {
     const int tp = threadIdx.x & 31, cy = threadIdx.x >> 5;      // pair of positions, channel (+ 8 i)
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int c = c0 + cy + 8 * i, t = t0 + 2 * tp;
       uint32_t v = 0u;
-      if (c < C && t < T) v = *reinterpret_cast<const uint32_t*>(x + (((size_t)n * C + c) * H + h) * T + t);   // (T is even)
+      if (c < C && t < Tn) v = *reinterpret_cast<const uint32_t*>(x + (((size_t)n * C + c) * H + h) * Tn + t);   // (Tn is even)
       *reinterpret_cast<uint32_t*>(&tile[cy + 8 * i][2 * tp]) = v;
     }
   } else {
@@ -96,29 +114,31 @@ tap1d16_rows_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ xr, int C
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int c = c0 + cy + 4 * i, t = t0 + tx;
-      tile[cy + 4 * i][tx] = (c < C && t < T) ? x[(((size_t)n * C + c) * H + h) * T + t] : (uint16_t)0;
+      tile[cy + 4 * i][tx] = (c < C && t < Tn) ? x[(((size_t)n * C + c) * H + h) * Tn + t] : T{};
     }
   }
   __syncthreads();
+  constexpr int CPT = 64 / CELL;                // cells per position of the tile
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int item = threadIdx.x + 256 * i, cell = item & 7, tl = item >> 3;
-    const int t = t0 + tl, c = c0 + 8 * cell;
-    if (t < T && c < Cs) {
-      uint32_t v[4];
+  for (int i = 0; i < CPT * 64 / 256; ++i) {
+    const int item = threadIdx.x + 256 * i, cell = item % CPT, tl = item / CPT;
+    const int t = t0 + tl, c = c0 + CELL * cell;
+    if (t < Tn && c < Cs) {
+      __attribute__((aligned(16))) T v[CELL];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = (uint32_t)tile[8 * cell + 2 * e][tl] | ((uint32_t)tile[8 * cell + 2 * e + 1][tl] << 16);
-      *reinterpret_cast<uintx4_t*>(xr + ((size_t)row * T + t) * Cs + c) = uintx4_t{v[0], v[1], v[2], v[3]};
+      for (int e = 0; e < CELL; ++e) v[e] = tile[CELL * cell + e][tl];
+      *reinterpret_cast<uintx4_t*>(xr + ((size_t)row * Tn + t) * Cs + c) = *reinterpret_cast<const uintx4_t*>(v);
     }
   }
 }
 
-static void launch_rows(const bf16_t* x, bf16_t* xr, int C, int H, int T, int Cs, int rows, hipStream_t s) {
-  const dim3 grid((unsigned)((T + 63) / 64), (unsigned)((Cs + 63) / 64), (unsigned)rows);
-  if (T % 2 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0)
-    hipLaunchKernelGGL(tap1d16_rows_kernel<true>, grid, dim3(256), 0, s, x, xr, C, H, T, Cs);
+template <typename T>
+static void launch_rows(const T* x, T* xr, int C, int H, int Tn, int Cs, int rows, hipStream_t s) {
+  const dim3 grid((unsigned)((Tn + 63) / 64), (unsigned)((Cs + 63) / 64), (unsigned)rows);
+  if (sizeof(T) == 2 && Tn % 2 == 0 && reinterpret_cast<uintptr_t>(x) % 4 == 0)
+    hipLaunchKernelGGL((tap1d_rows_kernel<T, true>), grid, dim3(256), 0, s, x, xr, C, H, Tn, Cs);
   else
-    hipLaunchKernelGGL(tap1d16_rows_kernel<false>, grid, dim3(256), 0, s, x, xr, C, H, T, Cs);
+    hipLaunchKernelGGL((tap1d_rows_kernel<T, false>), grid, dim3(256), 0, s, x, xr, C, H, Tn, Cs);
 }
 
 struct Tap1Weights {
@@ -130,8 +150,10 @@ struct Tap1Weights {
   signed char tapj[T1_MAXTAPS];   // weight tap of stored tap i (-1: padding)
 };
 
+template <typename T>
 __global__ void __launch_bounds__(256)
-tap1d16_weights_kernel(const bf16_t* __restrict__ w, uintx4_t* __restrict__ wf, Tap1Weights p) {
+tap1d_weights_kernel(const T* __restrict__ w, uintx4_t* __restrict__ wf, Tap1Weights p) {
+  constexpr int CELL = Tap1Elem<T>::CELL;
   const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
   const long long total = (long long)p.mblocks * p.taps_total * p.KS * 64;
   if (idx >= total) return;
@@ -140,37 +162,38 @@ tap1d16_weights_kernel(const bf16_t* __restrict__ w, uintx4_t* __restrict__ wf, 
   const int per_block = p.taps_total * p.KS;
   const int mblk = (int)(st / per_block), s = (int)(st - (long long)mblk * per_block);
   const int tap = s / p.KS, ks = s - tap * p.KS;
-  const int m = mblk * 32 + (lane & 31), c0 = ks * 16 + (lane >> 5) * 8;
+  const int m = mblk * 32 + (lane & 31), c0 = (2 * ks + (lane >> 5)) * CELL;
   const int j = p.tapj[tap];
-  uint32_t v[4] = {0u, 0u, 0u, 0u};
-  if (j >= 0 && m < p.Mo) {
+  __attribute__((aligned(16))) T v[CELL];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int c = c0 + e;
-      if (c < p.Cc) {
-        const size_t at = p.bwd ? ((size_t)c * p.Cw + m) * p.KW + j : ((size_t)m * p.Cw + c) * p.KW + j;
-        v[e >> 1] |= (uint32_t)w[at] << (16 * (e & 1));
-      }
-    }
+  for (int e = 0; e < CELL; ++e) {
+    const int c = c0 + e;
+    v[e] = T{};
+    if (j >= 0 && m < p.Mo && c < p.Cc)
+      v[e] = w[p.bwd ? ((size_t)c * p.Cw + m) * p.KW + j : ((size_t)m * p.Cw + c) * p.KW + j];
   }
-  wf[idx] = uintx4_t{v[0], v[1], v[2], v[3]};
+  wf[idx] = *reinterpret_cast<const uintx4_t*>(v);
 }
 
 // ---- the convolution ---------------------------------------------------------------------
-// KS k-steps per tap; DT taps per unrolled group (DT * KS = 12 or 16 stages: the distance between a
-// weight fragment's load and its use); SS source stride; NPH phases.
-template <int KS, int DT, int SS, int NPH>
+// KS stages per tap; DT taps per unrolled group; RW stages between a weight fragment's load and its use (RW divides
+// DT * KS; a bf16 stage is one matrix instruction per block, an fp32 stage four longer ones); SS source stride;
+// NPH phases; NB blocks of 32 positions.
+template <typename T, int KS, int DT, int RW, int SS, int NPH, int NB>
 __global__ void __launch_bounds__(256, 1)
-tap1d16_conv_kernel(Tap1Params p, const bf16_t* __restrict__ xr, const uintx4_t* __restrict__ wf,
-                    const float* __restrict__ bias, bf16_t* __restrict__ dst) {
+tap1d_conv_kernel(Tap1Params p, const T* __restrict__ xr, const uintx4_t* __restrict__ wf,
+                  const float* __restrict__ bias, T* __restrict__ dst) {
   extern __shared__ uintx4_t t1_slab[];
+  constexpr int CELL = Tap1Elem<T>::CELL;
+  constexpr int ESZ = (int)sizeof(T);
   constexpr int CPR = 2 * KS + 1;               // cells per slab row
+  constexpr int TP = 32 * NB;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ptile = __builtin_amdgcn_readfirstlane(blockIdx.x % p.ptiles);
   const int row = __builtin_amdgcn_readfirstlane(blockIdx.x / p.ptiles);
   const int mtile = blockIdx.y;
-  const int o0 = ptile * T1_TP;
+  const int o0 = ptile * TP;
   const int s0 = o0 * SS + p.smin;              // source position of slab offset 0
 
   // ---- the slab: load instruction ii fills cells ii * 64 .. + 63, cell L = slab row L / CPR, cell L % CPR
@@ -186,44 +209,42 @@ tap1d16_conv_kernel(Tap1Params p, const bf16_t* __restrict__ xr, const uintx4_t*
       const int off = SS == 1 ? R : (R < p.half ? 2 * R : 2 * (R - p.half) + 1);
       const int sp = s0 + off;
       int voff = T1_OOB;
-      if (R < p.SR && c < 2 * KS && (unsigned)sp < (unsigned)p.TS) voff = ((row * p.TS + sp) * p.Cs + 8 * c) * 2;
+      if (R < p.SR && c < 2 * KS && (unsigned)sp < (unsigned)p.TS) voff = ((row * p.TS + sp) * p.Cs + CELL * c) * ESZ;
       pd_load_lds(xrs, base + ii * 1024, voff, 0);
     }
   }
 
-  // ---- weights: this wave's stream of fragments, DT * KS stages ahead
+  // ---- weights: this wave's stream of fragments, RW stages ahead
+  constexpr int NS = DT * KS;
+  static_assert(NS % 4 == 0 && NS % RW == 0 && KS >= 2, "fragment sets and the weight ring rotate with the unrolled group");
   const __amdgpu_buffer_rsrc_t wrs = make_rsrc(wf, p.w_bytes);
   const int mblk = mtile * (T1_BM / 32) + wave;
-  int wpos = mblk * p.taps_total * KS * 1024;   // byte offset of the next group's first stage
+  int wpos = mblk * p.taps_total * KS * 1024;   // byte offset of the stage RW ahead of the group's first
   const int wlane = lane * 16;
-  uintx4_t bq[DT][KS];
+  uintx4_t bq[RW];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) bq[dt][ks] = __builtin_amdgcn_raw_buffer_load_b128(wrs, wlane, wpos + (dt * KS + ks) * 1024, 0);
-  wpos += DT * KS * 1024;
+  for (int i = 0; i < RW; ++i) bq[i] = __builtin_amdgcn_raw_buffer_load_b128(wrs, wlane, wpos + i * 1024, 0);
+  wpos += RW * 1024;
 
-  floatx16 acc[NPH][T1_NB];
+  floatx16 acc[NPH][NB];
 #pragma unroll
   for (int q = 0; q < NPH; ++q)
 #pragma unroll
-    for (int b = 0; b < T1_NB; ++b)
+    for (int b = 0; b < NB; ++b)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[q][b][r] = 0.f;
 
   const int fr = lane & 31, fg = lane >> 5;
-  lds_cell_t ap[T1_NB];
+  lds_cell_t ap[NB];
 #pragma unroll
-  for (int b = 0; b < T1_NB; ++b) ap[b] = (lds_cell_t)t1_slab + ((b * 32 + fr) * CPR + fg);
+  for (int b = 0; b < NB; ++b) ap[b] = (lds_cell_t)t1_slab + ((b * 32 + fr) * CPR + fg);
 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the slab (and the first weight fragments) have landed
   __syncthreads();
 
   // The position fragments of a stage are read two stages ahead of their use (four sets of registers in rotation;
   // a group's stage count is a multiple of four).
-  auto run = [&](floatx16 (&ac)[T1_NB], int q) __attribute__((always_inline)) {
-    constexpr int NS = DT * KS;
-    static_assert(NS % 4 == 0 && KS >= 2, "the fragment sets rotate with the unrolled group");
+  auto run = [&](floatx16 (&ac)[NB], int q) __attribute__((always_inline)) {
     const int groups = p.ntaps[q] / DT;
     const int dq = p.d0[q], last = p.nreal[q] - 1;
     // slab offset (cells) of a tap's rows; padding taps read the rows of the last tap that exists: finite values
@@ -233,14 +254,14 @@ tap1d16_conv_kernel(Tap1Params p, const bf16_t* __restrict__ xr, const uintx4_t*
       const int trow = SS == 1 ? d : (d & 1) * p.half + (d >> 1);
       return trow * CPR;
     };
-    uintx4_t af[4][T1_NB];
+    uintx4_t af[4][NB];
     int tcur[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) tcur[dt] = toff_of(dt);
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int b = 0; b < T1_NB; ++b) af[i][b] = ap[b][tcur[i / KS] + 2 * (i % KS)];
+      for (int b = 0; b < NB; ++b) af[i][b] = ap[b][tcur[i / KS] + 2 * (i % KS)];
     for (int g = 0; g < groups; ++g) {
       int tnext[DT];
 #pragma unroll
@@ -250,12 +271,11 @@ tap1d16_conv_kernel(Tap1Params p, const bf16_t* __restrict__ xr, const uintx4_t*
         const int i2 = i + 2;
         const int o2 = i2 < NS ? tcur[(i2 % NS) / KS] : tnext[(i2 % NS) / KS];
 #pragma unroll
-        for (int b = 0; b < T1_NB; ++b) af[i2 % 4][b] = ap[b][o2 + 2 * ((i2 % NS) % KS)];
-        const bf16x8 w8 = __builtin_bit_cast(bf16x8, bq[i / KS][i % KS]);
-        bq[i / KS][i % KS] = __builtin_amdgcn_raw_buffer_load_b128(wrs, wlane, wpos + i * 1024, 0);
+        for (int b = 0; b < NB; ++b) af[i2 % 4][b] = ap[b][o2 + 2 * ((i2 % NS) % KS)];
+        const uintx4_t w8 = bq[i % RW];
+        bq[i % RW] = __builtin_amdgcn_raw_buffer_load_b128(wrs, wlane, wpos + i * 1024, 0);
 #pragma unroll
-        for (int b = 0; b < T1_NB; ++b)
-          ac[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[i % 4][b]), w8, ac[b], 0, 0, 0);
+        for (int b = 0; b < NB; ++b) tap1d_mma(ac[b], af[i % 4][b], w8, static_cast<const T*>(nullptr));
         __builtin_amdgcn_sched_barrier(0);     // (the scheduler would otherwise move every read down to its use)
       }
 #pragma unroll
@@ -273,31 +293,35 @@ tap1d16_conv_kernel(Tap1Params p, const bf16_t* __restrict__ xr, const uintx4_t*
   const int n = row / p.H, h = row - n * p.H;
   const long long rbase = (((long long)n * p.Mo + m) * p.H + h) * p.TOu;     // element offset of the result row
   const __amdgpu_buffer_rsrc_t drs = make_rsrc(dst, p.dst_bytes);
-  const bool even = (rbase & 1) == 0;
+  const bool aligned = ESZ == 4 || (rbase & 1) == 0;     // pieces start on 4-byte boundaries
 #pragma unroll
-  for (int b = 0; b < T1_NB; ++b)
+  for (int b = 0; b < NB; ++b)
 #pragma unroll
     for (int g4 = 0; g4 < 4; ++g4) {
       const int o = o0 + b * 32 + g4 * 8 + fg * 4;
-      float v[4 * NPH];
+      float v[8];
 #pragma unroll
       for (int e = 0; e < 4; ++e)
 #pragma unroll
         for (int q = 0; q < NPH; ++q) v[e * NPH + q] = acc[q][b][4 * g4 + e] + bv;
       const int u = o * NPH;
-      if (even && u + 4 * NPH <= p.TOu) {      // (u is a multiple of 4: with an even row offset the piece is 4-byte aligned)
-        if (NPH == 1) {
+      if (aligned && u + 4 * NPH <= p.TOu) {      // (u is a multiple of 4)
+        const int at = (int)((rbase + u) * ESZ);
+        if (ESZ == 4) {
+          __builtin_amdgcn_raw_buffer_store_b128(uintx4_t{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])}, drs, at, 0, 0);
+          if (NPH == 2)
+            __builtin_amdgcn_raw_buffer_store_b128(uintx4_t{__float_as_uint(v[4]), __float_as_uint(v[5]), __float_as_uint(v[6]), __float_as_uint(v[7])}, drs, at + 16, 0, 0);
+        } else if (NPH == 1) {
           const uintx2_t t = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
-          __builtin_amdgcn_raw_buffer_store_b64(t, drs, (int)((rbase + u) * 2), 0, 0);
+          __builtin_amdgcn_raw_buffer_store_b64(t, drs, at, 0, 0);
         } else {
-          const uintx4_t t = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4 * (NPH - 1)], v[4 * (NPH - 1) + 1]),
-                              pack_bf16(v[4 * (NPH - 1) + 2], v[4 * (NPH - 1) + 3])};
-          __builtin_amdgcn_raw_buffer_store_b128(t, drs, (int)((rbase + u) * 2), 0, 0);
+          const uintx4_t t = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])};
+          __builtin_amdgcn_raw_buffer_store_b128(t, drs, at, 0, 0);
         }
       } else {
 #pragma unroll
         for (int e = 0; e < 4 * NPH; ++e)
-          if (u + e < p.TOu) dst[rbase + u + e] = f32_to_bf16(v[e]);
+          if (u + e < p.TOu) st(dst, (size_t)(rbase + u + e), v[e]);
       }
     }
 }
@@ -306,7 +330,7 @@ tap1d16_conv_kernel(Tap1Params p, const bf16_t* __restrict__ xr, const uintx4_t*
 struct Tap1Plan {
   Tap1Params p;
   Tap1Weights w;
-  int SS, DT;
+  int SS, DT, NB;
   size_t rows_bytes, w_bytes, lds_bytes;
   int C, H, T;           // of the source tensor, for the rows pass
 };
@@ -318,10 +342,11 @@ int tap1d_cs(int C) {
   return 0;
 }
 
+// taps per unrolled group of the bf16 kernels (fp32: 1)
 int dt_of(int KS) { return KS >= 16 ? 1 : KS >= 8 ? 2 : KS == 6 ? 2 : KS == 4 ? 4 : KS == 2 ? 8 : 0; }
 
-// bwd = false: forward; true: backward-data
-bool tap1d_plan(const ConvGeom& g, bool bwd, Tap1Plan* pl) {
+// bwd = false: forward; true: backward-data.  esz: bytes per element (2: bf16, 4: fp32)
+bool tap1d_plan(const ConvGeom& g, bool bwd, int esz, Tap1Plan* pl) {
   if (g.KH != 1 || g.py != 0 || g.sy != 1 || g.dlx != 1 || g.groups != 1) return false;
   if (g.KW < 2 || g.KW > 32 || (g.sx != 1 && g.sx != 2)) return false;
   if (g.OH != g.H || (long long)g.N * g.H > 65535) return false;
@@ -329,7 +354,8 @@ bool tap1d_plan(const ConvGeom& g, bool bwd, Tap1Plan* pl) {
   // contraction channels padded to a count the kernel is compiled for
   const int Cs = tap1d_cs(Cc);
   if (!Cs || Cc < 16) return false;
-  const int KS = Cs / 16, DT = dt_of(KS);
+  const int cell = 16 / esz;
+  const int KS = Cs / (2 * cell), DT = esz == 2 ? dt_of(KS) : 1;
   Tap1Params& p = pl->p;
   Tap1Weights& w = pl->w;
   std::memset(&p, 0, sizeof p);
@@ -339,18 +365,18 @@ bool tap1d_plan(const ConvGeom& g, bool bwd, Tap1Plan* pl) {
   int soff[2] = {0, 0};
   if (!bwd) {
     pl->SS = g.sx; p.nph = 1;
-    p.TS = g.W; p.TO = g.OW; p.TOu = g.OW;
+    p.TS = g.W; p.TOu = g.OW;
     p.nreal[0] = g.KW; soff[0] = -g.px;
     for (int i = 0; i < g.KW; ++i) w.tapj[i] = (signed char)i;
   } else if (g.sx == 1) {
     pl->SS = 1; p.nph = 1;
-    p.TS = g.OW; p.TO = g.W; p.TOu = g.W;
+    p.TS = g.OW; p.TOu = g.W;
     p.nreal[0] = g.KW; soff[0] = g.px - (g.KW - 1);
     for (int i = 0; i < g.KW; ++i) w.tapj[i] = (signed char)(g.KW - 1 - i);
   } else {
     // u = 2 v + q takes the taps j = jq + 2 i' with jq = (q + px) & 1, from dy[v + (q + px - jq) / 2 - i']
     pl->SS = 1; p.nph = 2;
-    p.TS = g.OW; p.TO = (g.W + 1) / 2; p.TOu = g.W;
+    p.TS = g.OW; p.TOu = g.W;
     for (int q = 0; q < 2; ++q) {
       const int jq = (q + g.px) & 1;
       p.nreal[q] = (g.KW - jq + 1) / 2;
@@ -358,6 +384,7 @@ bool tap1d_plan(const ConvGeom& g, bool bwd, Tap1Plan* pl) {
       soff[q] = (q + g.px - jq) / 2 - (p.nreal[q] - 1);
     }
   }
+  p.TO = (p.TOu + p.nph - 1) / p.nph;
   int stored = 0;
   for (int q = 0; q < p.nph; ++q) {
     p.ntaps[q] = (p.nreal[q] + DT - 1) / DT * DT;
@@ -377,21 +404,27 @@ bool tap1d_plan(const ConvGeom& g, bool bwd, Tap1Plan* pl) {
     p.d0[q] = soff[q] - p.smin;
     span = std::max(span, p.d0[q] + p.nreal[q]);
   }
-  if (pl->SS == 1) {
-    p.SR = T1_TP + span - 1;
-    p.half = 0;
-  } else {
-    p.half = ((2 * (T1_TP - 1) + span - 1) >> 1) + 1;
-    p.SR = 2 * p.half;
-  }
   const int CPR = 2 * KS + 1;
-  pl->lds_bytes = (size_t)(((long long)p.SR * CPR + 63) / 64) * 1024;
-  if (pl->lds_bytes > 160 * 1024) return false;
-  p.ptiles = (p.TO + T1_TP - 1) / T1_TP;
+  // three blocks of positions per wave; two where the slab of three does not fit (fp32, 256 channels, forward stride 2)
+  pl->NB = 0;
+  for (int nb = 3; nb >= 2 && !pl->NB; --nb) {
+    const int tp = 32 * nb;
+    if (pl->SS == 1) {
+      p.SR = tp + span - 1;
+      p.half = 0;
+    } else {
+      p.half = ((2 * (tp - 1) + span - 1) >> 1) + 1;
+      p.SR = 2 * p.half;
+    }
+    pl->lds_bytes = (size_t)(((long long)p.SR * CPR + 63) / 64) * 1024;
+    if (pl->lds_bytes <= 160 * 1024 && (nb == 3 || (esz == 4 && KS == 32 && pl->SS == 2))) pl->NB = nb;
+  }
+  if (!pl->NB) return false;
+  p.ptiles = (p.TO + 32 * pl->NB - 1) / (32 * pl->NB);
   p.mtiles = (Mo + T1_BM - 1) / T1_BM;
-  const long long rb = (long long)p.rows * p.TS * Cs * 2;
+  const long long rb = (long long)p.rows * p.TS * Cs * esz;
   const long long wb = (long long)p.mtiles * (T1_BM / 32) * stored * KS * 1024;
-  const long long db = (long long)g.N * Mo * g.H * p.TOu * 2;
+  const long long db = (long long)g.N * Mo * g.H * p.TOu * esz;
   if (rb >= (1ll << 31) || wb >= (1ll << 31) || db >= (1ll << 31)) return false;
   p.src_bytes = (unsigned)rb; p.w_bytes = (unsigned)wb; p.dst_bytes = (unsigned)db;
   pl->rows_bytes = ((size_t)rb + 255) & ~(size_t)255;
@@ -403,43 +436,57 @@ bool tap1d_plan(const ConvGeom& g, bool bwd, Tap1Plan* pl) {
   return true;
 }
 
-template <int KS, int DT>
-int launch_conv(const Tap1Plan& pl, const bf16_t* xr, const uintx4_t* wf, const float* bias, bf16_t* dst, hipStream_t s) {
+template <typename T, int KS, int DT, int RW>
+int launch_conv(const Tap1Plan& pl, const T* xr, const uintx4_t* wf, const float* bias, T* dst, hipStream_t s) {
   const dim3 grid((unsigned)(pl.p.rows * pl.p.ptiles), (unsigned)pl.p.mtiles);
   auto go = [&](auto kernel) {
     if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), pl.lds_bytes)) return -1;
     hipLaunchKernelGGL(kernel, grid, dim3(256), pl.lds_bytes, s, pl.p, xr, wf, bias, dst);
-    return check_launch("conv2d (bf16 one-row windows)");
+    return check_launch("conv2d (one-row windows)");
   };
-  if (pl.p.nph == 2) return go(tap1d16_conv_kernel<KS, DT, 1, 2>);
-  if (pl.SS == 2) return go(tap1d16_conv_kernel<KS, DT, 2, 1>);
-  return go(tap1d16_conv_kernel<KS, DT, 1, 1>);
+  if (pl.NB == 2) {
+    if constexpr (sizeof(T) == 4 && KS == 32) return go(tap1d_conv_kernel<T, KS, DT, RW, 2, 1, 2>);
+    return -1;
+  }
+  if (pl.p.nph == 2) return go(tap1d_conv_kernel<T, KS, DT, RW, 1, 2, 3>);
+  if (pl.SS == 2) return go(tap1d_conv_kernel<T, KS, DT, RW, 2, 1, 3>);
+  return go(tap1d_conv_kernel<T, KS, DT, RW, 1, 1, 3>);
 }
 
+template <typename T>
 int run_conv(const ConvGeom& g, bool bwd, const void* src, const void* w, const float* bias, void* dst, hipStream_t s,
              void* ws, size_t ws_bytes) {
   Tap1Plan pl;
-  if (!tap1d_plan(g, bwd, &pl)) return -1;
+  if (!tap1d_plan(g, bwd, (int)sizeof(T), &pl)) return -1;
   if (!ws || ws_bytes < pl.rows_bytes + pl.w_bytes) return -1;
-  bf16_t* xr = static_cast<bf16_t*>(ws);
+  T* xr = static_cast<T*>(ws);
   uintx4_t* wf = reinterpret_cast<uintx4_t*>(static_cast<char*>(ws) + pl.rows_bytes);
-  launch_rows(static_cast<const bf16_t*>(src), xr, pl.C, pl.H, pl.T, pl.p.Cs, pl.p.rows, s);
+  launch_rows(static_cast<const T*>(src), xr, pl.C, pl.H, pl.T, pl.p.Cs, pl.p.rows, s);
   {
     const long long total = (long long)pl.w.mblocks * pl.w.taps_total * pl.w.KS * 64;
-    hipLaunchKernelGGL(tap1d16_weights_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
-                       static_cast<const bf16_t*>(w), wf, pl.w);
+    hipLaunchKernelGGL(tap1d_weights_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+                       static_cast<const T*>(w), wf, pl.w);
   }
-  if (const int rc = check_launch("conv2d (bf16 one-row windows, operand passes)")) return rc;
-  bf16_t* out = static_cast<bf16_t*>(dst);
-  switch (pl.p.KS) {
-    case 2: return launch_conv<2, 8>(pl, xr, wf, bias, out, s);
-    case 4: return launch_conv<4, 4>(pl, xr, wf, bias, out, s);
-    case 6: return launch_conv<6, 2>(pl, xr, wf, bias, out, s);
-    case 8: return launch_conv<8, 2>(pl, xr, wf, bias, out, s);
-    default: return launch_conv<16, 1>(pl, xr, wf, bias, out, s);
+  if (const int rc = check_launch("conv2d (one-row windows, operand passes)")) return rc;
+  T* out = static_cast<T*>(dst);
+  if constexpr (sizeof(T) == 2) {
+    switch (pl.p.KS) {
+      case 2: return launch_conv<T, 2, 8, 16>(pl, xr, wf, bias, out, s);
+      case 4: return launch_conv<T, 4, 4, 16>(pl, xr, wf, bias, out, s);
+      case 6: return launch_conv<T, 6, 2, 12>(pl, xr, wf, bias, out, s);
+      case 8: return launch_conv<T, 8, 2, 16>(pl, xr, wf, bias, out, s);
+      default: return launch_conv<T, 16, 1, 16>(pl, xr, wf, bias, out, s);
+    }
+  } else {
+    switch (pl.p.KS) {
+      case 4: return launch_conv<T, 4, 1, 4>(pl, xr, wf, bias, out, s);
+      case 8: return launch_conv<T, 8, 1, 4>(pl, xr, wf, bias, out, s);
+      case 12: return launch_conv<T, 12, 1, 4>(pl, xr, wf, bias, out, s);
+      case 16: return launch_conv<T, 16, 1, 4>(pl, xr, wf, bias, out, s);
+      default: return launch_conv<T, 32, 1, 4>(pl, xr, wf, bias, out, s);
+    }
   }
 }
-
 
 // ---- the filter gradient -------------------------------------------------------------------
 //   dw[k][c][j] = sum over sequences and positions o of dy[k][o] x[c][o*s + j - p],  db[k] = sum dy[k][o]
@@ -457,7 +504,7 @@ int run_conv(const ConvGeom& g, bool bwd, const void* src, const void* w, const 
 // the loads themselves before the range's first step; rows are 6 cells apart for stride 1 and
 // 5 for stride 2, which keeps the four rows of a transposing read on distinct banks.
 // The workgroups' tiles go to the workspace as [range set][tile][slot][64 filters][32 channels]
-// and tap1d16_wgrad_reduce_kernel adds them in a fixed order into dw's memory order.
+// and tap1d_wgrad_reduce_kernel adds them in a fixed order into dw's memory order.
 typedef short shortx4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) shortx4_t* lds_tr_t;
 
@@ -473,12 +520,17 @@ struct Tap1WParams {
   unsigned src_bytes, dy_bytes;
 };
 
-template <int TQ, int SS>
+template <typename T, int TQ, int SS>
 __global__ void __launch_bounds__(256, 1)
-tap1d16_wgrad_kernel(Tap1WParams p, const bf16_t* __restrict__ xr, const bf16_t* __restrict__ dy, float* __restrict__ part) {
+tap1d_wgrad_kernel(Tap1WParams p, const T* __restrict__ xr, const T* __restrict__ dy, float* __restrict__ part) {
   extern __shared__ uintx4_t t1_slab[];
-  constexpr int PC = SS == 1 ? 6 : 5;           // cells per slab row (4 used)
-  constexpr int PE = PC * 8;                    // the same in elements
+  constexpr int CELL = Tap1Elem<T>::CELL;
+  constexpr int ESZ = (int)sizeof(T);
+  constexpr bool LO = ESZ == 2;
+  constexpr int STEP = 2 * CELL;                // positions per step: a lane half holds CELL consecutive ones
+  constexpr int RC = 32 / CELL;                 // cells of a slab row in use (32 channels)
+  constexpr int PC = LO ? (SS == 1 ? 6 : 5) : RC + 1;   // cells per slab row
+  constexpr int PE = PC * CELL;                 // the same in elements
   constexpr int RD = 4;                         // steps between a dy fragment's load and its use
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -497,21 +549,23 @@ tap1d16_wgrad_kernel(Tap1WParams p, const bf16_t* __restrict__ xr, const bf16_t*
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][t][r] = 0.f;
   // a tile of ones for the bias slot
-  const uintx4_t ones = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+  const uint32_t one = LO ? 0x3f803f80u : 0x3f800000u;
+  const uintx4_t ones = {one, one, one, one};
   const int bias_slot = p.KW - wave * TQ;       // this wave's slot index of the bias gradient (outside 0 .. TQ - 1: none)
 
-  // this lane's first transposing read of a step: row SS * (fs / 4) (+ 8 SS fg), channels 16 fq + 4 (fs % 4) .. + 3,
-  // at the wave's first tap
-  const uint16_t* const slab16 = reinterpret_cast<const uint16_t*>(t1_slab);
-  const int blane = ((8 * fg + (fs >> 2)) * SS + wave * TQ) * PE + 16 * fq + 4 * (fs & 3);
+  // this lane's first read of a step at the wave's first tap.  bf16: transposing reads, row SS * (fs / 4) (+ 8 SS fg),
+  // channels 16 fq + 4 (fs % 4) .. + 3.  fp32: four 4-byte reads, rows SS * (4 fg + e), channel fr.
+  const T* const slabT = reinterpret_cast<const T*>(t1_slab);
+  const int blane = LO ? ((8 * fg + (fs >> 2)) * SS + wave * TQ) * PE + 16 * fq + 4 * (fs & 3)
+                       : (4 * fg * SS + wave * TQ) * PE + fr;
 
   const int u0 = split * p.upw, u1 = min(u0 + p.upw, p.units);
   for (int u = u0; u < u1; ++u) {
     const int seq = u / p.tsplit, tr = u - seq * p.tsplit;
     const int t0 = tr * p.TL, oend = min(p.OW, t0 + p.TL);
     if (t0 >= oend) continue;
-    const int nsteps = (oend - t0 + 15) >> 4;
-    const int tailn = (oend - t0) & 15;         // positions of a last, partial step (0: none)
+    const int nsteps = (oend - t0 + STEP - 1) / STEP;
+    const int tailn = (oend - t0) % STEP;       // positions of a last, partial step (0: none)
     if (u != u0) __syncthreads();                // every wave is done with the previous slab
     // ---- slab: row R holds source position t0 * SS - px + R, channels 32 ct .. + 31
     {
@@ -524,24 +578,25 @@ tap1d16_wgrad_kernel(Tap1WParams p, const bf16_t* __restrict__ xr, const bf16_t*
         const int R = fast_div(L, PC, inv, &c);
         const int sp = sp0 + R;
         int voff = T1_OOB;
-        if (R < p.SRW && c < 4 && (unsigned)sp < (unsigned)p.TS) voff = ((seq * p.TS + sp) * p.Cs + ct * 32 + 8 * c) * 2;
+        if (R < p.SRW && c < RC && (unsigned)sp < (unsigned)p.TS) voff = ((seq * p.TS + sp) * p.Cs + ct * 32 + CELL * c) * ESZ;
         pd_load_lds(xrs, slab_addr + ii * 1024, voff, 0);
       }
     }
-    // ---- dy: filters kt * 64 + 32 a + fr, positions t0 + 16 step + 8 fg .. + 7
+    // ---- dy: filters kt * 64 + 32 a + fr, positions t0 + STEP step + CELL fg .. + CELL - 1
     const int n = seq / p.H, h = seq - n * p.H;
     int aoff[2];
 #pragma unroll
     for (int a = 0; a < 2; ++a) {
       const int k = kt * 64 + a * 32 + fr;
-      aoff[a] = k < p.K ? ((((n * p.K + k) * p.H + h) * p.OW) + t0 + 8 * fg) * 2 : T1_OOB;
+      aoff[a] = k < p.K ? ((((n * p.K + k) * p.H + h) * p.OW) + t0 + CELL * fg) * ESZ : T1_OOB;
     }
     // the partial step's mask: elements at and past oend are zero
     uint32_t tmask[4];
     {
-      const int cnt = tailn ? tailn - 8 * fg : 8;
+      const int cnt = tailn ? tailn - CELL * fg : CELL;
 #pragma unroll
-      for (int d = 0; d < 4; ++d) tmask[d] = cnt >= 2 * d + 2 ? 0xffffffffu : cnt == 2 * d + 1 ? 0x0000ffffu : 0u;
+      for (int d = 0; d < 4; ++d)
+        tmask[d] = LO ? (cnt >= 2 * d + 2 ? 0xffffffffu : cnt == 2 * d + 1 ? 0x0000ffffu : 0u) : (cnt > d ? 0xffffffffu : 0u);
     }
     uintx4_t aq[RD][2];
 #pragma unroll
@@ -554,13 +609,19 @@ tap1d16_wgrad_kernel(Tap1WParams p, const bf16_t* __restrict__ xr, const bf16_t*
 
     // the slab fragment of slot t + 1 is read while slot t is multiplied (the first slot of a step behind the last
     // of the step before)
-    auto bread = [&](const uint16_t* at) __attribute__((always_inline)) {
-      const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)at);
-      const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(at + 4 * SS * PE));
-      const uintx2_t l2 = __builtin_bit_cast(uintx2_t, lo), h2 = __builtin_bit_cast(uintx2_t, hi);
-      return uintx4_t{l2.x, l2.y, h2.x, h2.y};
+    auto bread = [&](const T* at) __attribute__((always_inline)) {
+      if constexpr (LO) {
+        const shortx4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)at);
+        const shortx4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(at + 4 * SS * PE));
+        const uintx2_t l2 = __builtin_bit_cast(uintx2_t, lo), h2 = __builtin_bit_cast(uintx2_t, hi);
+        return uintx4_t{l2.x, l2.y, h2.x, h2.y};
+      } else {
+        lds_f1 f = (lds_f1)at;
+        return uintx4_t{__float_as_uint(f[0]), __float_as_uint(f[SS * PE]), __float_as_uint(f[2 * SS * PE]),
+                        __float_as_uint(f[3 * SS * PE])};
+      }
     };
-    uintx4_t bnext = bread(slab16 + blane);
+    uintx4_t bnext = bread(slabT + blane);
 #define T1W_STEP(I)                                                                                       \
   {                                                                                                       \
     const int st = st0 + I;                                                                               \
@@ -571,15 +632,13 @@ tap1d16_wgrad_kernel(Tap1WParams p, const bf16_t* __restrict__ xr, const bf16_t*
       if (tailn && st == nsteps - 1) {                                                                    \
         _Pragma("unroll") for (int d = 0; d < 4; ++d) { a0[d] &= tmask[d]; a1[d] &= tmask[d]; }           \
       }                                                                                                   \
-      const bf16x8 fa0 = __builtin_bit_cast(bf16x8, a0), fa1 = __builtin_bit_cast(bf16x8, a1);            \
-      const uint16_t* bp = slab16 + blane + st * (16 * SS * PE);                                          \
+      const T* bp = slabT + blane + st * (STEP * SS * PE);                                                \
       _Pragma("unroll") for (int t = 0; t < TQ; ++t) {                                                    \
         uintx4_t b4 = bnext;                                                                              \
-        bnext = bread(t + 1 < TQ ? bp + (t + 1) * PE : bp + 16 * SS * PE);                                \
+        bnext = bread(t + 1 < TQ ? bp + (t + 1) * PE : bp + STEP * SS * PE);                              \
         if (t == bias_slot) b4 = ones;                                                                    \
-        const bf16x8 fb = __builtin_bit_cast(bf16x8, b4);                                                 \
-        acc[0][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0, fb, acc[0][t], 0, 0, 0);                 \
-        acc[1][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1, fb, acc[1][t], 0, 0, 0);                 \
+        tap1d_mma(acc[0][t], a0, b4, static_cast<const T*>(nullptr));                                     \
+        tap1d_mma(acc[1][t], a1, b4, static_cast<const T*>(nullptr));                                     \
         __builtin_amdgcn_sched_barrier(0);                                                                \
       }                                                                                                   \
     }                                                                                                     \
@@ -608,7 +667,7 @@ tap1d16_wgrad_kernel(Tap1WParams p, const bf16_t* __restrict__ xr, const bf16_t*
 // dw[k][c][j] and db[k] from the tiles of nsplit range sets, added in the order of the sets.
 // Slot g of a tile: tap g for g < KW, the bias gradient for g = KW.
 __global__ void __launch_bounds__(256)
-tap1d16_wgrad_reduce_kernel(const float* __restrict__ part, int nsplit, int tiles, int ctiles, int slots, int K, int C, int KW,
+tap1d_wgrad_reduce_kernel(const float* __restrict__ part, int nsplit, int tiles, int ctiles, int slots, int K, int C, int KW,
                             float* __restrict__ dw, float* __restrict__ db) {
   const int e = blockIdx.x * 256 + threadIdx.x;   // element of a slot: filter e / 32, channel e % 32
   const int g = blockIdx.y, tile = blockIdx.z;
@@ -637,10 +696,11 @@ struct Tap1WPlan {
   size_t rows_bytes, part_bytes, lds_bytes;
 };
 
-bool tap1d_wgrad_plan(const ConvGeom& g, Tap1WPlan* pl) {
+bool tap1d_wgrad_plan(const ConvGeom& g, int esz, Tap1WPlan* pl) {
   if (g.KH != 1 || g.py != 0 || g.sy != 1 || g.dlx != 1 || g.groups != 1) return false;
   if (g.KW < 6 || g.KW > 23 || (g.sx != 1 && g.sx != 2)) return false;
-  if (g.OH != g.H || (long long)g.N * g.H > 65535 || g.OW % 2 != 0 || g.C < 16 || g.K < 32) return false;
+  if (g.OH != g.H || (long long)g.N * g.H > 65535 || g.C < 16 || g.K < 32) return false;
+  if (esz == 2 && g.OW % 2 != 0) return false;   // (rows of dy start on 4-byte boundaries)
   Tap1WParams& p = pl->p;
   std::memset(&p, 0, sizeof p);
   const int TQ = (g.KW + 1 + 3) / 4;            // KW taps and the bias gradient over four waves
@@ -651,7 +711,7 @@ bool tap1d_wgrad_plan(const ConvGeom& g, Tap1WPlan* pl) {
   p.K = g.K; p.C = g.C; p.KW = g.KW; p.px = g.px;
   p.ktiles = (g.K + 63) / 64; p.ctiles = (g.C + 31) / 32;
   const int tiles = p.ktiles * p.ctiles;
-  const int PC = g.sx == 1 ? 6 : 5;
+  const int PC = esz == 2 ? (g.sx == 1 ? 6 : 5) : 9;
   // ranges: enough workgroups for the chip; a range's slab must fit in LDS
   const int want = (mfma_num_cus() + tiles - 1) / tiles;
   int tsplit = std::max(1, (want + p.rows - 1) / p.rows);
@@ -666,8 +726,8 @@ bool tap1d_wgrad_plan(const ConvGeom& g, Tap1WPlan* pl) {
   p.units = p.rows * p.tsplit;
   p.upw = std::max(1, p.units / std::max(1, want));
   pl->nsplit = (p.units + p.upw - 1) / p.upw;
-  const long long rb = (long long)p.rows * p.TS * p.Cs * 2;
-  const long long yb = (long long)g.N * g.K * g.H * g.OW * 2;
+  const long long rb = (long long)p.rows * p.TS * p.Cs * esz;
+  const long long yb = (long long)g.N * g.K * g.H * g.OW * esz;
   if (rb >= (1ll << 31) || yb >= (1ll << 31)) return false;
   p.src_bytes = (unsigned)rb; p.dy_bytes = (unsigned)yb;
   pl->rows_bytes = ((size_t)rb + 255) & ~(size_t)255;
@@ -675,74 +735,85 @@ bool tap1d_wgrad_plan(const ConvGeom& g, Tap1WPlan* pl) {
   return true;
 }
 
-template <int TQ>
-int launch_wgrad(const Tap1WPlan& pl, const bf16_t* xr, const bf16_t* dy, float* part, hipStream_t s) {
+template <typename T, int TQ>
+int launch_wgrad(const Tap1WPlan& pl, const T* xr, const T* dy, float* part, hipStream_t s) {
   const dim3 grid((unsigned)pl.nsplit, (unsigned)(pl.p.ktiles * pl.p.ctiles));
   auto go = [&](auto kernel) {
     if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), pl.lds_bytes)) return -1;
     hipLaunchKernelGGL(kernel, grid, dim3(256), pl.lds_bytes, s, pl.p, xr, dy, part);
-    return check_launch("conv2d_bwd_filter (bf16 one-row windows)");
+    return check_launch("conv2d_bwd_filter (one-row windows)");
   };
-  return pl.SS == 2 ? go(tap1d16_wgrad_kernel<TQ, 2>) : go(tap1d16_wgrad_kernel<TQ, 1>);
+  return pl.SS == 2 ? go(tap1d_wgrad_kernel<T, TQ, 2>) : go(tap1d_wgrad_kernel<T, TQ, 1>);
 }
 
-}  // namespace
-
-size_t mfma_tap1d16_conv_ws(const ConvGeom& g, bool bwd) {
-  Tap1Plan pl;
-  return tap1d_plan(g, bwd, &pl) ? pl.rows_bytes + pl.w_bytes : 0;
-}
-
-int mfma_tap1d16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y, hipStream_t s,
-                          void* ws, size_t ws_bytes) {
-  return run_conv(g, false, x, w, bias, y, s, ws, ws_bytes);
-}
-
-int mfma_tap1d16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s, void* ws,
-                               size_t ws_bytes) {
-  return run_conv(g, true, dy, w, nullptr, dx, s, ws, ws_bytes);
-}
-
-}  // namespace flhip
-
-namespace flhip {
-
-size_t mfma_tap1d16_wgrad_ws(const ConvGeom& g) {
+template <typename T>
+int run_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes, hipStream_t s,
+              const void* rows) {
   Tap1WPlan pl;
-  return tap1d_wgrad_plan(g, &pl) ? pl.rows_bytes + pl.part_bytes : 0;
-}
-
-size_t mfma_tap1d16_rows_bytes(const ConvGeom& g) {
-  Tap1Plan f;
-  Tap1WPlan w;
-  return tap1d_plan(g, false, &f) && tap1d_wgrad_plan(g, &w) && f.rows_bytes == w.rows_bytes ? w.rows_bytes : 0;
-}
-
-int mfma_tap1d16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes,
-                       hipStream_t s, const void* rows) {
-  Tap1WPlan pl;
-  if (!tap1d_wgrad_plan(g, &pl)) return -1;
+  if (!tap1d_wgrad_plan(g, (int)sizeof(T), &pl)) return -1;
   if (!ws || ws_bytes < pl.rows_bytes + pl.part_bytes) return -1;
-  const bf16_t* xr = static_cast<const bf16_t*>(rows ? rows : ws);
+  const T* xr = static_cast<const T*>(rows ? rows : ws);
   float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + pl.rows_bytes);
   if (!rows) {
-    launch_rows(static_cast<const bf16_t*>(x), static_cast<bf16_t*>(ws), g.C, g.H, g.W, pl.p.Cs, pl.p.rows, s);
-    if (const int rc = check_launch("conv2d_bwd_filter (bf16 one-row windows, rows pass)")) return rc;
+    launch_rows(static_cast<const T*>(x), static_cast<T*>(ws), g.C, g.H, g.W, pl.p.Cs, pl.p.rows, s);
+    if (const int rc = check_launch("conv2d_bwd_filter (one-row windows, rows pass)")) return rc;
   }
-  const bf16_t* dyp = static_cast<const bf16_t*>(dy);
+  const T* dyp = static_cast<const T*>(dy);
   int rc;
   switch (pl.TQ) {
-    case 2: rc = launch_wgrad<2>(pl, xr, dyp, part, s); break;
-    case 3: rc = launch_wgrad<3>(pl, xr, dyp, part, s); break;
-    case 4: rc = launch_wgrad<4>(pl, xr, dyp, part, s); break;
-    case 5: rc = launch_wgrad<5>(pl, xr, dyp, part, s); break;
-    default: rc = launch_wgrad<6>(pl, xr, dyp, part, s); break;
+    case 2: rc = launch_wgrad<T, 2>(pl, xr, dyp, part, s); break;
+    case 3: rc = launch_wgrad<T, 3>(pl, xr, dyp, part, s); break;
+    case 4: rc = launch_wgrad<T, 4>(pl, xr, dyp, part, s); break;
+    case 5: rc = launch_wgrad<T, 5>(pl, xr, dyp, part, s); break;
+    default: rc = launch_wgrad<T, 6>(pl, xr, dyp, part, s); break;
   }
   if (rc) return rc;
   const int tiles = pl.p.ktiles * pl.p.ctiles;
-  hipLaunchKernelGGL(tap1d16_wgrad_reduce_kernel, dim3(8, (unsigned)(g.KW + 1), (unsigned)tiles), dim3(256), 0, s, part, pl.nsplit,
+  hipLaunchKernelGGL(tap1d_wgrad_reduce_kernel, dim3(8, (unsigned)(g.KW + 1), (unsigned)tiles), dim3(256), 0, s, part, pl.nsplit,
                      tiles, pl.p.ctiles, 4 * pl.TQ, g.K, g.C, g.KW, dw, db);
-  return check_launch("conv2d_bwd_filter (bf16 one-row windows, sum)");
+  return check_launch("conv2d_bwd_filter (one-row windows, sum)");
+}
+
+int esz_of(int dtype) { return dtype == FLHIP_F32 ? 4 : dtype == FLHIP_BF16 ? 2 : 0; }
+
+}  // namespace
+
+size_t mfma_tap1d_conv_ws(const ConvGeom& g, int dtype, bool bwd) {
+  Tap1Plan pl;
+  return esz_of(dtype) && tap1d_plan(g, bwd, esz_of(dtype), &pl) ? pl.rows_bytes + pl.w_bytes : 0;
+}
+
+int mfma_tap1d_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w, const float* bias, void* y, hipStream_t s,
+                        void* ws, size_t ws_bytes) {
+  if (dtype == FLHIP_F32) return run_conv<float>(g, false, x, w, bias, y, s, ws, ws_bytes);
+  if (dtype == FLHIP_BF16) return run_conv<bf16_t>(g, false, x, w, bias, y, s, ws, ws_bytes);
+  return -1;
+}
+
+int mfma_tap1d_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx, hipStream_t s, void* ws,
+                             size_t ws_bytes) {
+  if (dtype == FLHIP_F32) return run_conv<float>(g, true, dy, w, nullptr, dx, s, ws, ws_bytes);
+  if (dtype == FLHIP_BF16) return run_conv<bf16_t>(g, true, dy, w, nullptr, dx, s, ws, ws_bytes);
+  return -1;
+}
+
+size_t mfma_tap1d_wgrad_ws(const ConvGeom& g, int dtype) {
+  Tap1WPlan pl;
+  return esz_of(dtype) && tap1d_wgrad_plan(g, esz_of(dtype), &pl) ? pl.rows_bytes + pl.part_bytes : 0;
+}
+
+size_t mfma_tap1d_rows_bytes(const ConvGeom& g, int dtype) {
+  Tap1Plan f;
+  Tap1WPlan w;
+  const int esz = esz_of(dtype);
+  return esz && tap1d_plan(g, false, esz, &f) && tap1d_wgrad_plan(g, esz, &w) && f.rows_bytes == w.rows_bytes ? w.rows_bytes : 0;
+}
+
+int mfma_tap1d_wgrad(const ConvGeom& g, int dtype, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes,
+                     hipStream_t s, const void* rows) {
+  if (dtype == FLHIP_F32) return run_wgrad<float>(g, x, dy, dw, db, ws, ws_bytes, s, rows);
+  if (dtype == FLHIP_BF16) return run_wgrad<bf16_t>(g, x, dy, dw, db, ws, ws_bytes, s, rows);
+  return -1;
 }
 
 }  // namespace flhip

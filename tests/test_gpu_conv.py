@@ -169,7 +169,7 @@ def test_conv_bf16(case):
         assert rel_l2(got, ref) <= tight, (name, rel_l2(got, ref))
 
 
-# bf16 windows of one row (KH = 1) on the kernels that read channels-last rows and fragment-ordered weights: the speech
+# windows of one row (KH = 1), bf16 and fp32, on the kernels that read channels-last rows and fragment-ordered weights: the speech
 # stack's 21 x 1 windows at a short length (stride 1 and 2, 80 / 250 channels: padded contractions of 96 and 256), rows
 # per image > 1, an odd length with an even window over a stride of 2, more than 128 filters without padding, every
 # padded contraction size the kernels are compiled for (32, 64, 96, 128, 256), a tile's last positions past the row.
@@ -195,21 +195,23 @@ ONE_ROW_CASES = [
 ]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("case", ONE_ROW_CASES)
-def test_conv_bf16_one_row_windows(case):
+def test_conv_one_row_windows(case, dtype):
     from flashlight_amd import capi
-    res = _run(case, 38, torch.bfloat16)
+    lo = dtype == torch.bfloat16
+    res = _run(case, 38, dtype)
     for name, (got, ref) in res.items():
-        tight = 1e-4 if name in ("dw", "db") else 4e-3
+        tight = 1e-4 if (name in ("dw", "db") or not lo) else 4e-3
         assert rel_l2(got, ref) <= tight, (name, rel_l2(got, ref))
     # the same shapes with the family switched off (the kernels it replaced) agree with it to rounding
     capi.set_option("CONV_SKIP", "tap1d")
     try:
-        old = _run(case, 38, torch.bfloat16)
+        old = _run(case, 38, dtype)
     finally:
         capi.set_option("CONV_SKIP", None)
     for name in ("y", "dx"):
-        assert rel_l2(res[name][0], old[name][0]) <= 6e-3, name
+        assert rel_l2(res[name][0], old[name][0]) <= (6e-3 if lo else 1e-4), name
 
 
 # f16 storage goes through the kernels that widen their operands to fp32 (the bf16 matrix-core families are
@@ -459,7 +461,7 @@ def test_batching_invariance_on_device():
         assert np.allclose(y1[0], y[n], atol=1e-5, rtol=0)
 
 
-@pytest.mark.parametrize("shape", [((2, 128, 9, 40), (136, 128, 1, 21), (1, 2), (0, 10)),
+@pytest.mark.parametrize("shape", [((2, 128, 9, 40), (136, 128, 2, 11), (1, 2), (1, 5)),
                                    ((2, 128, 15, 15), (160, 128, 3, 3), (2, 2), (1, 1))])
 def test_forward_and_backward_data_without_workspace(shape):
     """Forward and backward-data take a workspace only to reorder the weights of strided /
@@ -486,6 +488,36 @@ def test_forward_and_backward_data_without_workspace(shape):
     assert L.flhip_conv2d_bwd_data(C.byref(cd), P(dy), P(w), P(dx0), None, 0, S) == 0
     torch.cuda.synchronize()
     assert torch.equal(y0, y) and torch.equal(dx0, dx)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_one_row_windows_without_workspace(dtype):
+    """One-row windows reach their kernels through channels-last rows and reordered weights in the workspace;
+    without it the same calls take the kernels of the other families and agree to rounding."""
+    import ctypes as C
+    from flashlight_amd import capi
+    xs, ws_, st, pd = (2, 128, 9, 40), (136, 128, 1, 21), (1, 2), (0, 10)
+    rng = np.random.default_rng(79)
+    x = dev(rng.standard_normal(xs).astype(np.float32)).to(dtype)
+    w = dev((rng.standard_normal(ws_) / 30).astype(np.float32)).to(dtype)
+    kw = dict(sx=st[1], sy=st[0], px=pd[1], py=pd[0], dx=1, dy=1, groups=1)
+    y = fa.conv2d(x, w, None, **kw)
+    dy = dev(rng.standard_normal(tuple(y.shape)).astype(np.float32)).to(dtype)
+    dx = fa.conv2d_backward_data(dy, xs, w, **kw)
+    L = capi.lib()
+    lo = dtype == torch.bfloat16
+    cd = capi.ConvDesc(xs[0], xs[1], xs[2], xs[3], ws_[0], ws_[2], ws_[3], st[0], st[1], pd[0], pd[1], 1, 1, 1,
+                       capi.BF16 if lo else capi.F32)
+    esz = 2 if lo else 4
+    assert L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_FWD) >= (x.numel() + w.numel()) * esz
+    S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: C.c_void_p(t.data_ptr())
+    y0, dx0 = torch.empty_like(y), torch.empty_like(dx)
+    assert L.flhip_conv2d_fwd(C.byref(cd), P(x), P(w), None, P(y0), None, 0, S) == 0
+    assert L.flhip_conv2d_bwd_data(C.byref(cd), P(dy), P(w), P(dx0), None, 0, S) == 0
+    torch.cuda.synchronize()
+    tol = 1e-2 if lo else 1e-5
+    assert rel_l2(host(y0), host(y)) <= tol and rel_l2(host(dx0), host(dx)) <= tol
 
 
 @pytest.mark.parametrize("shape", [((3, 64, 14, 14), (96, 64, 1, 1), (2, 2), (0, 0)),
@@ -571,15 +603,14 @@ def test_bf16_filter_gradient_from_the_forward_pass_gather(shape, with_bias):
 @pytest.mark.parametrize("shape", [((3, 80, 1, 180), (250, 80, 1, 21), (1, 1), (0, 10)),
                                    ((3, 250, 1, 180), (250, 250, 1, 21), (1, 2), (0, 10)),
                                    ((2, 32, 3, 50), (40, 32, 1, 5), (1, 1), (0, 2))])        # 5 taps: that filter gradient declines
-def test_bf16_one_row_filter_gradient_from_the_forward_pass_rows(shape):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_one_row_filter_gradient_from_the_forward_pass_rows(shape, dtype):
     """One-row windows: the forward pass leaves its channels-last rows at the start of its workspace; the filter
     gradient computed from them equals the one that makes the rows again, bit for bit."""
-    import ctypes as C
-    from flashlight_amd import capi
     xs, ws_, st, pd = shape
     rng = np.random.default_rng(92)
-    x = dev(bf16_round(rng.standard_normal(xs).astype(np.float32))).to(torch.bfloat16)
-    w = dev(bf16_round((rng.standard_normal(ws_) / 20).astype(np.float32))).to(torch.bfloat16)
+    x = dev(rng.standard_normal(xs).astype(np.float32)).to(dtype)
+    w = dev((rng.standard_normal(ws_) / 20).astype(np.float32)).to(dtype)
     kw = dict(sx=st[1], sy=st[0], px=pd[1], py=pd[0], dx=1, dy=1, groups=1)
     y, rows = fa.conv2d(x, w, None, keep_gathered=True, **kw)
     assert torch.equal(y, fa.conv2d(x, w, None, **kw))
@@ -587,11 +618,12 @@ def test_bf16_one_row_filter_gradient_from_the_forward_pass_rows(shape):
         assert rows is None
         return
     cs = 96 if xs[1] == 80 else 256
-    assert rows is not None and rows.numel() >= xs[0] * xs[2] * xs[3] * cs * 2
+    esz = 2 if dtype == torch.bfloat16 else 4
+    assert rows is not None and rows.numel() >= xs[0] * xs[2] * xs[3] * cs * esz
     # the rows are the input with its channels last, padded with zeros
-    r = rows[:xs[0] * xs[2] * xs[3] * cs * 2].view(torch.bfloat16).view(xs[0], xs[2], xs[3], cs)
+    r = rows[:xs[0] * xs[2] * xs[3] * cs * esz].view(dtype).view(xs[0], xs[2], xs[3], cs)
     assert torch.equal(r[..., :xs[1]], x.permute(0, 2, 3, 1)) and not bool(r[..., xs[1]:].any())
-    dy = dev(bf16_round(rng.standard_normal(tuple(y.shape)).astype(np.float32))).to(torch.bfloat16)
+    dy = dev(rng.standard_normal(tuple(y.shape)).astype(np.float32)).to(dtype)
     dw0, db0 = fa.conv2d_backward_filter_bias(dy, x, ws_, True, **kw)
     kept = rows.clone()
     dw1, db1 = fa.conv2d_backward_filter_bias(dy, x, ws_, True, gathered=kept, **kw)
