@@ -125,8 +125,9 @@ const char* flhip_arch(void);
  * (value NULL restores the default; the FLHIP_ prefix on `name` is optional).  Not to be
  * called while another thread is inside the library.  Results stay within the stated
  * tolerances under every setting; the switches only choose between kernels.
- *   CONV_ALGO = direct | gather | tapped | convert | auto    CONV_SKIP = bf16,gemm1x1,slab,tapped,strip,first,wgrad128,pwdma,wd32
+ *   CONV_ALGO = direct | gather | tapped | convert | auto    CONV_SKIP = bf16,gemm1x1,slab,tapped,strip,first,wgrad128,pwdma,wd32,tap1d
  *   PW_PT = 2 | 4 | 8    PW16_PF = 0 | 1 | 2 | 4 | 8    CONV_STACK = 0 | 1 | 2 | 4 | 8    BN_ALGO = split | resident | auto
+ *   SLAB_WAVES = 0 | 4 | 8
  *   PW16_NO_TAPS, TAPPED_NO_REORDER, MATMUL_VALU, RNN_UNFUSED = 1 | 0
  * Unknown names or values return FLHIP_INVALID_ARGUMENT.  The nearest thing in the
  * reference is the kernel-choice options object of its cuDNN extension
@@ -142,7 +143,10 @@ int flhip_pool2d_out_dims(const flhip_pool_desc* d, int32_t* OH, int32_t* OW);
  * results of the sliced contraction); forward and backward-data run without it too, but
  * with it the kernels for strided / long windows read weights reordered per tap, and
  * strided windows in bf16 storage run on the bf16 matrix cores over a gathered copy of
- * the input's lattice points (1x1, all passes) or of its taps (up to 9, backward passes). */
+ * the input's lattice points (1x1, all passes) or of its taps (up to 9, backward passes), and
+ * windows of one row (KH = 1, 2 to 32 taps, column stride 1 or 2: the 21 x 1 windows of a speech
+ * stack; bf16 and fp32) run on kernels that read a channels-last copy of the source and weights
+ * reordered into the order of the matrix instruction's fragments. */
 size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pass);
 
 /* AutogradExtension::conv2d (AutogradExtension.h:58-69; oneDNN peer
@@ -181,7 +185,9 @@ int flhip_conv2d_bwd_filter(const flhip_conv_desc* d, const void* x,
  * (flashlight/fl/autograd/Functions.cpp:1341-1363: `payload`, captured by gradFunc; the oneDNN peer leaves it
  * empty).  With bf16 storage the forward pass of a strided layer first gathers the input points that its
  * windows touch (a 1x1 stride-2 layer: a quarter of the input; a 3x3 stride-2 layer: one copy per tap, 9/4 of
- * it) and runs as a 1x1 stride-1 layer over that copy; the filter gradient needs the same copy.
+ * it) and runs as a 1x1 stride-1 layer over that copy; the filter gradient needs the same copy.  Likewise,
+ * in bf16 and fp32, the forward pass of a window of one row first writes the input with its channels last,
+ * and the filter gradient of such a window (6 to 23 taps) reads the same rows.
  * flhip_conv2d_gathered_bytes(d) > 0 says that flhip_conv2d_fwd leaves this copy in the first that many bytes
  * of its workspace.  A caller that keeps those bytes unchanged until the backward pass hands them to
  * flhip_conv2d_bwd_filter_gathered in place of x and saves the second gather (the six strided layers of

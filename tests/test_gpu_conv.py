@@ -627,8 +627,10 @@ def test_one_row_filter_gradient_from_the_forward_pass_rows(shape, dtype):
     dw0, db0 = fa.conv2d_backward_filter_bias(dy, x, ws_, True, **kw)
     kept = rows.clone()
     dw1, db1 = fa.conv2d_backward_filter_bias(dy, x, ws_, True, gathered=kept, **kw)
+    dw2, db2 = fa.conv2d_backward_filter_bias(dy, x, ws_, True, **kw)          # the tiles are added in a fixed order
     torch.cuda.synchronize()
     assert torch.equal(dw1, dw0) and torch.equal(db1, db0)
+    assert torch.equal(dw2, dw0) and torch.equal(db2, db0)
 
 
 def _random_cases(n, seed):
