@@ -115,7 +115,7 @@ pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __r
   static_assert(PD_XCELLS % 64 == 0 && pd_wcells(BWD, BM) % 64 == 0, "whole load instructions");
   static_assert(NI <= 20 && NI >= 12, "five load instructions per wave at most, three at least");
   constexpr int MINL = NI / 4;                                  // loads every wave issues per stage at least
-  static_assert(PD_NS % 2 == 0, "ring and register sets repeat with the unrolled loop");
+  static_assert(PD_NS == 4 || PD_NS == 8, "the ring slot is the stage number modulo a power of two");
 
   // consecutive workgroups go to different XCDs: the channel tiles that share a source tile
   // run back to back on one XCD
@@ -159,12 +159,16 @@ pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __r
     }
   }
   const bool fourth = wave + 12 < NI, fifth = wave + 16 < NI;
+  const int n = p.nstages, n2 = (n + 1) & ~1;
+  // stages are multiplied in pairs: with an odd number the stage past the contraction fetches nothing and fills its
+  // slot with zeros (both operands: it adds 0)
   auto issue = [&](int t, uint4* ring) {
     const unsigned base = (unsigned)reinterpret_cast<uintptr_t>((lds_void_t)ring);
+    const bool live = t < n;
 #pragma unroll
-    for (int n = 0; n < 3; ++n) pd_load_lds(lrs[n], base + loff[n], voff[n], t * lstep[n]);
-    if (fourth) pd_load_lds(lrs[3], base + loff[3], voff[3], t * lstep[3]);
-    if (fifth) pd_load_lds(lrs[4], base + loff[4], voff[4], t * lstep[4]);
+    for (int k = 0; k < 3; ++k) pd_load_lds(lrs[k], base + loff[k], live ? voff[k] : (int)0x80000000, t * lstep[k]);
+    if (fourth) pd_load_lds(lrs[3], base + loff[3], live ? voff[3] : (int)0x80000000, t * lstep[3]);
+    if (fifth) pd_load_lds(lrs[4], base + loff[4], live ? voff[4] : (int)0x80000000, t * lstep[4]);
   };
 
   // ---- fragments: 128 result channels: wave = (position half, channel half), 2 x 2 blocks of 32 x 32;
@@ -200,35 +204,40 @@ pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __r
       _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                     \
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][ks][i], fb[SET][ks][j], acc[i][j], 0, 0, 0);
 
-  const int n = p.nstages;
   // stages 0 .. D in flight, stage 0 in registers
 #pragma unroll
   for (int st = 0; st <= PD_D; ++st)
-    if (st < n) issue(st, ring + st * PD_STAGE);
-  if (PD_D < n) pd_wait_loads<MINL * PD_D>();     // stages 1 .. D may be outstanding
+    if (st < n2) issue(st, ring + st * PD_STAGE);
+  if (PD_D < n2) pd_wait_loads<MINL * PD_D>();      // stages 1 .. D may be outstanding
   else pd_wait_loads<0>();
   __syncthreads();
   PD_READ(ring, 0)
 
   // iteration t: the stage t + 1 has landed for every wave (wait for this wave's loads, then the
   // barrier); the loads of stage t + 1 + D go to the slot whose fragments were multiplied in
-  // iteration t - 1; the fragments of stage t + 1 are read while those of stage t are multiplied
+  // iteration t - 1; the fragments of stage t + 1 are read while those of stage t are multiplied.
+  // Only the wait and the loads depend on the stage number; the reads of one register set and the
+  // matrix instructions on the other are one block of code without branches, which the scheduler
+  // interleaves: with a branch on the stage number around them every wave waited for its reads
+  // before its first matrix instruction, and reads and products took turns.
+  constexpr int NREAD = (BWD ? 4 * NA + 8 : 4 * NA + 4), NMULT = 4 * NA;
 #define PD_ITER(U)                                                                                  \
-  if (U < PD_NS) {                                                                                  \
-    const int t = t0 + U;                                                                           \
-    if (t < n) {                                                                                    \
-      if (t + 1 < n) {                                                                              \
-        if (t + PD_D < n) pd_wait_loads<MINL * (PD_D - 1)>();                                       \
-        else pd_wait_loads<0>();                                                                    \
-        __syncthreads();                                                                            \
-        if (t + 1 + PD_D < n) issue(t + 1 + PD_D, ring + ((U + 1 + PD_D) % PD_NS) * PD_STAGE);      \
-        PD_READ((ring + ((U + 1) % PD_NS) * PD_STAGE), (U + 1) % 2)                                 \
-      }                                                                                             \
-      PD_MULT(U % 2)                                                                                \
+  {                                                                                                 \
+    if (t0 + U + PD_D < n2) pd_wait_loads<MINL * (PD_D - 1)>();                                     \
+    else pd_wait_loads<0>();                                                                        \
+    __syncthreads();                                                                                \
+    if (t0 + U + 1 + PD_D < n2) issue(t0 + U + 1 + PD_D, ring + ((s0 + U + 1 + PD_D) & (PD_NS - 1)) * PD_STAGE); \
+    PD_READ((ring + ((s0 + U + 1) & (PD_NS - 1)) * PD_STAGE), (U + 1) % 2)                          \
+    PD_MULT(U % 2)                                                                                  \
+    _Pragma("unroll") for (int q = 0; q < NMULT; ++q) {                                             \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                            \
+      __builtin_amdgcn_sched_group_barrier(0x100, (NREAD + NMULT - 1) / NMULT, 0);                  \
     }                                                                                               \
   }
-  for (int t0 = 0; t0 < n; t0 += PD_NS) {
-    PD_ITER(0) PD_ITER(1) PD_ITER(2) PD_ITER(3) PD_ITER(4) PD_ITER(5) PD_ITER(6) PD_ITER(7)
+  // two stages per trip (the register sets alternate); the ring slot is the stage number modulo the ring
+  for (int t0 = 0; t0 < n2; t0 += 2) {
+    const int s0 = t0 & (PD_NS - 1);
+    PD_ITER(0) PD_ITER(1)
   }
 #undef PD_ITER
 #undef PD_MULT
@@ -373,6 +382,7 @@ pwd16_wgrad_kernel(PwdWgradParams p, const bf16_t* __restrict__ x, const bf16_t*
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int sbeg = slice * p.sps, n = min(p.nstages, sbeg + p.sps) - sbeg;      // this slice's stages
+  const int n2 = (n + 1) & ~1;          // stages are multiplied in pairs: with an odd number one stage of zeros more
   const intx4_t drs = pd_rsrc(dy, p.dy_bytes), xrs = pd_rsrc(x, p.x_bytes);
   constexpr int OOB = (int)0x80000000;
 
@@ -392,9 +402,11 @@ pwd16_wgrad_kernel(PwdWgradParams p, const bf16_t* __restrict__ x, const bf16_t*
   const int dimg = PWG_CH / p.Pc, dj = PWG_CH - dimg * p.Pc;
   const int dy_img = p.Mo * p.P * 2, x_img = p.C * p.P * 2;
   unsigned tailq = 0;                   // bit u: the cell this lane loaded into ring slot u is the last of its plane
+  int left = n;                         // stages of this slice not yet issued: a stage past the slice fetches nothing (zeros)
   auto issue = [&](int slot) {
     const unsigned base = (unsigned)reinterpret_cast<uintptr_t>((lds_void_t)(ring + slot * PWG_STAGE));
-    const bool live = img < p.N;
+    const bool live = img < p.N && left > 0;
+    --left;
     const int col = min(8 * j, p.P - 8) * 2;
     const int od = live ? img * dy_img + col : OOB, ox = live ? img * x_img + col : OOB;
     const bool tail = live && p.dup != 0 && j == p.Pc - 1;
@@ -465,33 +477,36 @@ pwd16_wgrad_kernel(PwdWgradParams p, const bf16_t* __restrict__ x, const bf16_t*
       _Pragma("unroll") for (int jj = 0; jj < 2; ++jj)                                                       \
         acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][sk][i], fb[SET][sk][jj], acc[i][jj], 0, 0, 0);
 
-  // stages 0 .. D in flight; every wave issues 8 loads per stage
+  // stages 0 .. D in flight; every wave issues 8 loads per stage.  Only the wait and the loads depend on the
+  // stage number: the reads of one register set and the matrix instructions on the other are one block of
+  // code without branches, interleaved one matrix instruction to one read.
   if (n > 0) {
 #pragma unroll
     for (int st = 0; st <= PWG_D; ++st)
-      if (st < n) issue(st);
-    if (PWG_D < n) PD_WAIT_VM(16);
+      if (st < n2) issue(st);
+    if (PWG_D < n2) PD_WAIT_VM(16);
     else PD_WAIT_VM(0);
     fix_tail(0);
     __syncthreads();
     PWG_READ(0, 0)
 #define PWG_ITER(U)                                                                    \
   {                                                                                    \
-    const int t = t0 + U;                                                              \
-    if (t < n) {                                                                       \
-      if (t + 1 < n) {                                                                 \
-        if (t + PWG_D < n) PD_WAIT_VM(8);                                              \
-        else PD_WAIT_VM(0);                                                            \
-        fix_tail((U + 1) % PWG_NS);                                                    \
-        __syncthreads();                                                               \
-        if (t + 1 + PWG_D < n) issue((U + 1 + PWG_D) % PWG_NS);                        \
-        PWG_READ((U + 1) % PWG_NS, (U + 1) % 2)                                        \
-      }                                                                                \
-      PWG_MULT(U % 2)                                                                  \
+    if (t0 + U + PWG_D < n2) PD_WAIT_VM(8);                                            \
+    else PD_WAIT_VM(0);                                                                \
+    fix_tail((s0 + U + 1) & (PWG_NS - 1));                                             \
+    __syncthreads();                                                                   \
+    if (t0 + U + 1 + PWG_D < n2) issue((s0 + U + 1 + PWG_D) & (PWG_NS - 1));           \
+    PWG_READ((s0 + U + 1) & (PWG_NS - 1), (U + 1) % 2)                                 \
+    PWG_MULT(U % 2)                                                                    \
+    _Pragma("unroll") for (int q = 0; q < 16; ++q) {                                   \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                               \
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                               \
     }                                                                                  \
   }
-    for (int t0 = 0; t0 < n; t0 += PWG_NS) {
-      PWG_ITER(0) PWG_ITER(1) PWG_ITER(2) PWG_ITER(3)
+    // two stages per trip (the register sets alternate); the ring slot is the stage number modulo the ring
+    for (int t0 = 0; t0 < n2; t0 += 2) {
+      const int s0 = t0 & (PWG_NS - 1);
+      PWG_ITER(0) PWG_ITER(1)
     }
 #undef PWG_ITER
   }
