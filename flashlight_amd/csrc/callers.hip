@@ -224,13 +224,23 @@ matmul_nn_skinny(const T* __restrict__ A, const T* __restrict__ B, T* __restrict
     }
     __syncthreads();
     const int per = (kn + 15) / 16, k0 = wave * per, k1 = min(kn, k0 + per);
-#pragma unroll 4
-    for (int k = k0; k < k1; ++k) {
-      const float a = mv ? ld(A, (size_t)(kc + k) * M + m) : 0.f;
-      const float4 b0 = *reinterpret_cast<const float4*>(&sm[k * SK_NT]);
-      const float4 b1 = *reinterpret_cast<const float4*>(&sm[k * SK_NT + 4]);
-      acc[0] += a * b0.x; acc[1] += a * b0.y; acc[2] += a * b0.z; acc[3] += a * b0.w;
-      acc[4] += a * b1.x; acc[5] += a * b1.y; acc[6] += a * b1.z; acc[7] += a * b1.w;
+    // 16 rows of A requested before the first is used: a lane's loads are 2 or 4 bytes each, and only the
+    // number in flight hides the way to memory (steps past the wave's share repeat its last row and add 0)
+    for (int k = k0; k < k1; k += 16) {
+      float a[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const float v = ld(A, (size_t)(kc + min(k + u, k1 - 1)) * M + (mv ? m : 0));
+        a[u] = (mv && k + u < k1) ? v : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int kk = min(k + u, k1 - 1);
+        const float4 b0 = *reinterpret_cast<const float4*>(&sm[kk * SK_NT]);
+        const float4 b1 = *reinterpret_cast<const float4*>(&sm[kk * SK_NT + 4]);
+        acc[0] += a[u] * b0.x; acc[1] += a[u] * b0.y; acc[2] += a[u] * b0.z; acc[3] += a[u] * b0.w;
+        acc[4] += a[u] * b1.x; acc[5] += a[u] * b1.y; acc[6] += a[u] * b1.z; acc[7] += a[u] * b1.w;
+      }
     }
   }
   __syncthreads();
