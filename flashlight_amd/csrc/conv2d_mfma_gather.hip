@@ -357,7 +357,7 @@ gather_conv_kernel(GatherParams p, const T* __restrict__ src, const T* __restric
 }
 
 // Chooses the number of 16-position blocks per workgroup so that the tile count
-// wastes as little of the last round over the CUs as possible.
+// wastes as little of the last pass of workgroups over the CUs as possible.
 int choose_nb(long long pblocks, int mtiles_total, int slots) {
   int best = 8;
   double best_cost = 1e30;
