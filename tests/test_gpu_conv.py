@@ -668,6 +668,39 @@ def test_random_geometries(case):
             assert rel_l2(got, ref) <= lim, (case, dtype, name, rel_l2(got, ref))
 
 
+def _random_one_row_cases(n, seed):
+    """Seeded random windows of one row or one column: 2 to 23 taps, strides, dilation, paddings from none to
+    window - 1, channel counts on and off the multiples of 8 / 32 (the padded contraction sizes of the kernels for
+    such windows), lengths that leave partial tiles; also the shapes those kernels decline (few channels, dilation,
+    columns), which then run on the other families."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < n:
+        kw = int(rng.integers(2, 24))
+        s_ = int(rng.choice([1, 1, 2]))
+        dl = int(rng.choice([1, 1, 1, 2]))
+        cin = int(rng.choice([8, 16, 24, 32, 40, 64, 80, 96, 104, 128, 136, 250, 256, 13, 7]))
+        cout = int(rng.choice([8, 24, 32, 64, 72, 96, 128, 136, 200, 250, 256, 5]))
+        H, W = int(rng.choice([1, 1, 1, 2, 3])), int(rng.integers(kw + 3, 260))
+        pw = int(rng.choice([0, kw // 2, (kw - 1) * dl // 2, kw - 1, 1]))
+        N = int(rng.integers(1, 5))
+        if W + 2 * pw < (kw - 1) * dl + 1 or N * cin * H * W * cout * kw > 4e8:
+            continue
+        if rng.random() < 0.85:
+            out.append(((N, cin, H, W), (cout, cin, 1, kw), (1, s_), (0, pw), (1, dl), 1))
+        else:
+            out.append(((N, cin, W, H), (cout, cin, kw, 1), (s_, 1), (pw, 0), (dl, 1), 1))
+    return out
+
+
+@pytest.mark.parametrize("case", _random_one_row_cases(24, 20251126))
+def test_random_one_row_windows(case):
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
+        for name, (got, ref) in _run(case, 5, dtype).items():
+            lim = F32_TOL if dtype == torch.float32 or name in ("dw", "db") else 4e-3
+            assert rel_l2(got, ref) <= lim, (case, dtype, name, rel_l2(got, ref))
+
+
 def test_invalid_arguments_raise():
     x = torch.zeros((1, 4, 8, 8), device="cuda")
     w = torch.zeros((4, 3, 3, 3), device="cuda")
