@@ -589,9 +589,10 @@ int mfma_pwd16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw
   PwdWgradParams p{};
   if (!dw || !pwd16_wgrad_plan(g, &p)) return -1;
   // measured on the ResNet-50 layers at batch 64: 7 to 20 % ahead of the kernel with register staging on planes of
-  // 14x14 and more (both move the same 100 MB through L2 for 30 MB of operands: 128 x 128 tiles), level or behind on
-  // 7x7 planes.  FLHIP_PW16_PF set lifts the rule (tests).
-  if (!options().pw16_pf && p.P < 64) return -1;
+  // 14x14 and more (both move the same 100 MB through L2 for 30 MB of operands: 128 x 128 tiles); on 7x7 planes ahead
+  // where dy is the large operand (512 -> 2048 channels: 28.6 against 31.2 us), level the other way round.
+  // FLHIP_PW16_PF set lifts the rule (tests).
+  if (!options().pw16_pf && p.P < 64 && g.K < 4 * g.C) return -1;
   const size_t need = p.nsplit > 1 ? (size_t)p.nsplit * ((size_t)p.E + p.Mo) * sizeof(float) : 0;
   if (need && (!ws || ws_bytes < need)) return -1;
   float* out = p.nsplit > 1 ? static_cast<float*>(ws) : dw;
