@@ -20,6 +20,84 @@ struct OpReluBwd {   // (dy, x) -> dy where x > 0
   __device__ float operator()(float dy, float x) const { return x > 0.f ? dy : 0.f; }
 };
 
+// ---- the other element-wise activations of fl::nn (flashlight/fl/nn/modules/Activations.cpp) ----
+// forward y = f(x); backward dx = dy * f'(x) from dy and the forward input.  16-bit storage: fp32 arithmetic,
+// one rounding of the result.
+__device__ __forceinline__ float act_sigmoid(float v) { return 1.f / (1.f + expf(-v)); }
+template <int OP>
+struct OpAct {
+  float a, b;
+  __device__ float operator()(float x, float) const {
+    if (OP == FLHIP_ACT_ELU) return x >= 0.f ? x : a * (expf(x) - 1.f);               // Activations.cpp:136-139
+    if (OP == FLHIP_ACT_CLAMP) return fminf(fmaxf(x, a), b);                          // fl::clip, Functions.cpp:465-466
+    if (OP == FLHIP_ACT_TANH) return tanhf(x);                                        // :454-455
+    if (OP == FLHIP_ACT_LOG) return logf(x);                                          // :403-404
+    if (OP == FLHIP_ACT_SWISH) return x * act_sigmoid(a * x);                         // :498-500
+    return act_sigmoid(x);                                                            // :488-489
+  }
+};
+template <int OP>
+struct OpActBwd {
+  float a, b;
+  __device__ float operator()(float dy, float x) const {
+    if (OP == FLHIP_ACT_ELU) return x >= 0.f ? dy : dy * a * expf(x);
+    if (OP == FLHIP_ACT_CLAMP) return (x > a && x < b) ? dy : 0.f;                    // (result > lo) && (result < hi), :471
+    if (OP == FLHIP_ACT_TANH) {
+      const float t = tanhf(x);
+      return (1.f - t * t) * dy;                                                      // :458-459
+    }
+    if (OP == FLHIP_ACT_LOG) return dy / x;                                           // :408
+    if (OP == FLHIP_ACT_SWISH) {
+      const float sg = act_sigmoid(a * x);
+      return dy * (sg + x * a * sg * (1.f - sg));
+    }
+    const float sg = act_sigmoid(x);
+    return dy * sg * (1.f - sg);                                                      // :492
+  }
+};
+
+// ---- fl::gatedlinearunit (Functions.cpp:1567-1610): the halved dimension's two halves are contiguous blocks of m
+// elements per outer index: y[o][k] = x[o][0][k] * sigmoid(x[o][1][k]) ----
+template <typename T>
+__global__ void __launch_bounds__(256) glu_fwd_kernel(const T* __restrict__ x, T* __restrict__ y, size_t n, size_t m) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    const size_t o = i / m, k = i - o * m;
+    const float a = ld(x, (2 * o) * m + k), g = ld(x, (2 * o + 1) * m + k);
+    st(y, i, a * act_sigmoid(g));
+  }
+}
+// dx first half = sigmoid(b) dy, second half = a sigmoid(b) (1 - sigmoid(b)) dy (:1594-1604)
+template <typename T>
+__global__ void __launch_bounds__(256) glu_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x, T* __restrict__ dx,
+                                                      size_t n, size_t m) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    const size_t o = i / m, k = i - o * m;
+    const float a = ld(x, (2 * o) * m + k), sg = act_sigmoid(ld(x, (2 * o + 1) * m + k)), g = ld(dy, i);
+    st(dx, (2 * o) * m + k, sg * g);
+    st(dx, (2 * o + 1) * m + k, a * sg * (1.f - sg) * g);
+  }
+}
+
+// ---- fl::dropout (Functions.cpp:1777-1785): y = x * keep / (1 - p).  keep(i) is a counter-based function of
+// (seed, i) - two rounds of a 32-bit finaliser, the top 24 bits as a uniform number in [0, 1), kept when >= p - so the
+// backward pass regenerates the mask from the seed instead of storing it (the same function the RNN uses between
+// layers, with the upper half of the element index in the place of the layer) ----
+template <typename T>
+__global__ void __launch_bounds__(256) dropout_kernel(const T* __restrict__ x, T* __restrict__ y, size_t n, uint32_t seed_lo,
+                                                      uint32_t seed_hi, float p, float scale) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    uint32_t h = (uint32_t)i * 0x9E3779B1u ^ seed_lo;
+    h ^= h >> 16; h *= 0x85EBCA6Bu; h ^= h >> 13; h *= 0xC2B2AE35u; h ^= h >> 16;
+    h += seed_hi + (uint32_t)(i >> 32) * 0x632BE5ABu;
+    h ^= h >> 16; h *= 0x85EBCA6Bu; h ^= h >> 13; h *= 0xC2B2AE35u; h ^= h >> 16;
+    const bool keep = (float)(h >> 8) * (1.0f / 16777216.0f) >= p;
+    st(y, i, keep ? ld(x, i) * scale : 0.f);
+  }
+}
+
 // ---- C = op(A) op(B) (+ bias per row), 64 x 64 tiles, 256 threads, 4 x 4 per thread ----
 constexpr int GT = 64, GK = 16;
 
@@ -538,6 +616,90 @@ extern "C" int flhip_relu_bwd(const void* dy, const void* x, void* dx, size_t n,
     launch_elementwise((const T*)dy, (const T*)x, (T*)dx, n, OpReluBwd{}, as_stream(stream));
   });
   return check_launch("relu_bwd");
+}
+
+extern "C" int flhip_act_fwd(int op, const void* x, void* y, size_t n, double a, double b, int dtype, void* stream) {
+  FLHIP_REQUIRE((x && y) || n == 0, "act_fwd: null argument");
+  FLHIP_REQUIRE(dtype_ok(dtype), "act_fwd: unknown dtype");
+  FLHIP_REQUIRE(op >= FLHIP_ACT_ELU && op <= FLHIP_ACT_SIGMOID, "act_fwd: unknown activation");
+  FLHIP_REQUIRE(op != FLHIP_ACT_CLAMP || a <= b, "act_fwd: clamp needs lo <= hi");
+  if (n == 0) return FLHIP_OK;
+  const float fa = (float)a, fb = (float)b;
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    auto go = [&](auto f) { launch_elementwise((const T*)x, (const T*)nullptr, (T*)y, n, f, as_stream(stream)); };
+    switch (op) {
+      case FLHIP_ACT_ELU: go(OpAct<FLHIP_ACT_ELU>{fa, fb}); break;
+      case FLHIP_ACT_CLAMP: go(OpAct<FLHIP_ACT_CLAMP>{fa, fb}); break;
+      case FLHIP_ACT_TANH: go(OpAct<FLHIP_ACT_TANH>{fa, fb}); break;
+      case FLHIP_ACT_LOG: go(OpAct<FLHIP_ACT_LOG>{fa, fb}); break;
+      case FLHIP_ACT_SWISH: go(OpAct<FLHIP_ACT_SWISH>{fa, fb}); break;
+      default: go(OpAct<FLHIP_ACT_SIGMOID>{fa, fb}); break;
+    }
+  });
+  return check_launch("act_fwd");
+}
+
+extern "C" int flhip_act_bwd(int op, const void* dy, const void* x, void* dx, size_t n, double a, double b, int dtype,
+                             void* stream) {
+  FLHIP_REQUIRE((dy && x && dx) || n == 0, "act_bwd: null argument");
+  FLHIP_REQUIRE(dtype_ok(dtype), "act_bwd: unknown dtype");
+  FLHIP_REQUIRE(op >= FLHIP_ACT_ELU && op <= FLHIP_ACT_SIGMOID, "act_bwd: unknown activation");
+  if (n == 0) return FLHIP_OK;
+  const float fa = (float)a, fb = (float)b;
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    auto go = [&](auto f) { launch_elementwise((const T*)dy, (const T*)x, (T*)dx, n, f, as_stream(stream)); };
+    switch (op) {
+      case FLHIP_ACT_ELU: go(OpActBwd<FLHIP_ACT_ELU>{fa, fb}); break;
+      case FLHIP_ACT_CLAMP: go(OpActBwd<FLHIP_ACT_CLAMP>{fa, fb}); break;
+      case FLHIP_ACT_TANH: go(OpActBwd<FLHIP_ACT_TANH>{fa, fb}); break;
+      case FLHIP_ACT_LOG: go(OpActBwd<FLHIP_ACT_LOG>{fa, fb}); break;
+      case FLHIP_ACT_SWISH: go(OpActBwd<FLHIP_ACT_SWISH>{fa, fb}); break;
+      default: go(OpActBwd<FLHIP_ACT_SIGMOID>{fa, fb}); break;
+    }
+  });
+  return check_launch("act_bwd");
+}
+
+extern "C" int flhip_glu_fwd(const void* x, void* y, int64_t outer, int64_t m, int dtype, void* stream) {
+  FLHIP_REQUIRE(x && y, "glu_fwd: null argument");
+  FLHIP_REQUIRE(outer > 0 && m > 0, "glu_fwd: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "glu_fwd: unknown dtype");
+  const size_t n = (size_t)outer * (size_t)m;
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((glu_fwd_kernel<T>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream), (const T*)x, (T*)y, n,
+                       (size_t)m);
+  });
+  return check_launch("glu_fwd");
+}
+
+extern "C" int flhip_glu_bwd(const void* dy, const void* x, void* dx, int64_t outer, int64_t m, int dtype, void* stream) {
+  FLHIP_REQUIRE(dy && x && dx, "glu_bwd: null argument");
+  FLHIP_REQUIRE(outer > 0 && m > 0, "glu_bwd: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "glu_bwd: unknown dtype");
+  const size_t n = (size_t)outer * (size_t)m;
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((glu_bwd_kernel<T>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream), (const T*)dy, (const T*)x,
+                       (T*)dx, n, (size_t)m);
+  });
+  return check_launch("glu_bwd");
+}
+
+extern "C" int flhip_dropout(const void* x, void* y, size_t n, double p, uint32_t seed_lo, uint32_t seed_hi, int dtype,
+                             void* stream) {
+  FLHIP_REQUIRE((x && y) || n == 0, "dropout: null argument");
+  FLHIP_REQUIRE(p >= 0.0 && p < 1.0, "dropout: the probability must be in [0, 1)");
+  FLHIP_REQUIRE(dtype_ok(dtype), "dropout: unknown dtype");
+  if (n == 0) return FLHIP_OK;
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((dropout_kernel<T>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream), (const T*)x, (T*)y, n,
+                       seed_lo, seed_hi, (float)p, (float)(1.0 / (1.0 - p)));
+  });
+  return check_launch("dropout");
 }
 
 extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, int32_t N, int32_t K,

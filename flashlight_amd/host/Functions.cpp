@@ -453,6 +453,96 @@ Variable relu(const Variable& input) {
   return Variable(out, {input}, gradFunc);
 }
 
+namespace {
+// y = f(x) / dx = dy f'(x) through flhip_act_fwd / _bwd; the closure keeps the input (the reference's closures keep
+// the result for tanh, clamp and sigmoid: the same function of the same input)
+Variable activation(const char* name, int op, const Variable& input, double a, double b) {
+  detail::OpScope scope(name);
+  Tensor out(input.shape(), input.type());
+  check(flhip_act_fwd(op, input.tensor().device(), out.device(), (size_t)out.elements(), a, b,
+                      tagOf(input.type(), name), hipBackendStream()));
+  if (scope.on()) scope.done({input.tensor()}, {out});
+  auto gradFunc = [op, a, b, name](std::vector<Variable>& inputs, const Variable& gradOutput) {
+    auto& in = inputs[0];
+    if (!in.isCalcGrad()) return;
+    detail::OpScope scope("activationBackward");
+    Tensor g(in.shape(), gradOutput.type());
+    check(flhip_act_bwd(op, gradOutput.tensor().device(), in.tensor().device(), g.device(), (size_t)g.elements(), a, b,
+                        tagOf(g.type(), name), hipBackendStream()));
+    if (scope.on()) scope.done({gradOutput.tensor(), in.tensor()}, {g});
+    in.addGrad(Variable(g, false));
+  };
+  return Variable(out, {input}, gradFunc);
+}
+}  // namespace
+
+Variable elu(const Variable& input, double alpha) { return activation("elu", FLHIP_ACT_ELU, input, alpha, 0.0); }
+Variable clamp(const Variable& input, double lo, double hi) {
+  if (lo > hi) throw std::invalid_argument("clamp: lo must not exceed hi");
+  return activation("clamp", FLHIP_ACT_CLAMP, input, lo, hi);
+}
+Variable tanh(const Variable& input) { return activation("tanh", FLHIP_ACT_TANH, input, 0.0, 0.0); }
+Variable log(const Variable& input) { return activation("log", FLHIP_ACT_LOG, input, 0.0, 0.0); }
+Variable sigmoid(const Variable& input) { return activation("sigmoid", FLHIP_ACT_SIGMOID, input, 0.0, 0.0); }
+Variable swish(const Variable& input, double beta) { return activation("swish", FLHIP_ACT_SWISH, input, beta, 0.0); }
+
+Variable gatedlinearunit(const Variable& input, int dim) {
+  // Functions.cpp:1567-1579
+  if (dim < 0 || dim >= input.ndim())
+    throw std::invalid_argument("gatedlinearunit - passed dim is great than the number of dimensions of the input.");
+  const Shape& in = input.shape();
+  if (in.dim(dim) % 2 == 1) throw std::invalid_argument("halving dimension must be even for GLU");
+  // column-major: the dimensions before `dim` are the fast ones
+  long long m = in.dim(dim) / 2, outer = 1;
+  for (int i = 0; i < dim; ++i) m *= in.dim(i);
+  for (int i = dim + 1; i < in.ndim(); ++i) outer *= in.dim(i);
+  std::vector<Dim> od = in.get();
+  od[(size_t)dim] /= 2;
+  detail::OpScope scope("gatedlinearunit");
+  Tensor out{Shape(od), input.type()};
+  if (out.elements() > 0)
+    check(flhip_glu_fwd(input.tensor().device(), out.device(), outer, m, tagOf(input.type(), "gatedlinearunit"),
+                        hipBackendStream()));
+  if (scope.on()) scope.done({input.tensor()}, {out});
+  auto gradFunc = [outer, m](std::vector<Variable>& inputs, const Variable& gradOutput) {
+    auto& in = inputs[0];
+    if (!in.isCalcGrad()) return;
+    detail::OpScope scope("gatedlinearunitBackward");
+    Tensor g(in.shape(), gradOutput.type());
+    if (g.elements() > 0)
+      check(flhip_glu_bwd(gradOutput.tensor().device(), in.tensor().device(), g.device(), outer, m,
+                          tagOf(g.type(), "gatedlinearunit"), hipBackendStream()));
+    if (scope.on()) scope.done({gradOutput.tensor(), in.tensor()}, {g});
+    in.addGrad(Variable(g, false));
+  };
+  return Variable(out, {input}, gradFunc);
+}
+
+unsigned long long nextSeed();   // Modules.cpp: the process-wide generator
+
+Variable dropout(const Variable& input, double p) {
+  if (!(p > 0.0)) return input;                                   // Functions.cpp:1778, 1782-1784
+  if (p >= 1.0) throw std::invalid_argument("dropout: the probability must be below 1");
+  const unsigned long long seed = nextSeed();
+  const uint32_t lo = (uint32_t)seed, hi = (uint32_t)(seed >> 32);
+  detail::OpScope scope("dropout");
+  Tensor out(input.shape(), input.type());
+  check(flhip_dropout(input.tensor().device(), out.device(), (size_t)out.elements(), p, lo, hi,
+                      tagOf(input.type(), "dropout"), hipBackendStream()));
+  if (scope.on()) scope.done({input.tensor()}, {out});
+  auto gradFunc = [p, lo, hi](std::vector<Variable>& inputs, const Variable& gradOutput) {
+    auto& in = inputs[0];
+    if (!in.isCalcGrad()) return;
+    detail::OpScope scope("dropoutBackward");
+    Tensor g(in.shape(), gradOutput.type());
+    check(flhip_dropout(gradOutput.tensor().device(), g.device(), (size_t)g.elements(), p, lo, hi,
+                        tagOf(g.type(), "dropout"), hipBackendStream()));
+    if (scope.on()) scope.done({gradOutput.tensor()}, {g});
+    in.addGrad(Variable(g, false));
+  };
+  return Variable(out, {input}, gradFunc);
+}
+
 Variable moddims(const Variable& input, const Shape& dims) {
   // a 0 keeps the input's dimension, one -1 is inferred from the element count
   // (Functions.cpp:969-1008)

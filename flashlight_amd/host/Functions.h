@@ -141,6 +141,21 @@ Variable affine(const Variable& input, const Variable& weight, const Variable& b
 // fl::relu = max(input, 0) (Functions.cpp:329-338, 1787-1789)
 Variable relu(const Variable& input);
 // fl::moddims / View: same data, new shape; one dimension may be -1 (Functions.cpp:790-829)
+// The other element-wise activations (flashlight/fl/autograd/Functions.cpp:403-411 log, :454-463 tanh, :465-475 clamp,
+// :488-496 sigmoid, :498-500 swish; nn/modules/Activations.cpp:136-139 elu).  clamp passes the gradient where
+// lo < result < hi.
+Variable elu(const Variable& input, double alpha = 1.0);
+Variable clamp(const Variable& input, double lo, double hi);
+Variable tanh(const Variable& input);
+Variable log(const Variable& input);
+Variable sigmoid(const Variable& input);
+Variable swish(const Variable& input, double beta);
+// fl::gatedlinearunit (Functions.cpp:1567-1610): first half of dimension `dim` times the sigmoid of the second half
+Variable gatedlinearunit(const Variable& input, int dim);
+// fl::dropout (Functions.cpp:1777-1785): input * mask / (1 - p); p <= 0 returns the input.  The mask is a
+// counter-based function of a seed drawn from the process-wide generator (fl::setSeed), regenerated by the
+// backward pass.
+Variable dropout(const Variable& input, double p);
 Variable moddims(const Variable& input, const Shape& dims);
 // fl::reorder (Functions.cpp:1010-1042): dimension k of the result is dimension dims[k] of the
 // input; the gradient is reordered back with the inverse permutation

@@ -261,6 +261,90 @@ class ReLU : public UnaryModule {          // Activations.cpp:58-70
   std::string prettyString() const override { return "ReLU"; }
 };
 
+// the other element-wise modules of nn/modules/Activations.cpp
+class Log : public UnaryModule {           // :32-34
+ public:
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return log(input); }
+  std::string prettyString() const override { return "Log"; }
+};
+class Tanh : public UnaryModule {          // :46-48
+ public:
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return tanh(input); }
+  std::string prettyString() const override { return "Tanh"; }
+};
+class HardTanh : public UnaryModule {      // :60-62
+ public:
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return clamp(input, -1.0, 1.0); }
+  std::string prettyString() const override { return "HardTanh"; }
+};
+class ReLU6 : public UnaryModule {         // :88-90
+ public:
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return clamp(input, 0.0, 6.0); }
+  std::string prettyString() const override { return "ReLU6"; }
+};
+class ELU : public UnaryModule {           // :132-139
+ public:
+  explicit ELU(double alpha = 1.0) : alpha_(alpha) {}
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return elu(input, alpha_); }
+  std::string prettyString() const override { return "ELU (" + std::to_string(alpha_) + ")"; }
+
+ private:
+  double alpha_;
+};
+class Sigmoid : public UnaryModule {       // :18-20
+ public:
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return sigmoid(input); }
+  std::string prettyString() const override { return "Sigmoid"; }
+};
+class Swish : public UnaryModule {         // :190-196
+ public:
+  explicit Swish(double beta = 1.0) : beta_(beta) {}
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return swish(input, beta_); }
+  std::string prettyString() const override { return "Swish (" + std::to_string(beta_) + ")"; }
+
+ private:
+  double beta_;
+};
+class GatedLinearUnit : public UnaryModule {   // :164-168
+ public:
+  explicit GatedLinearUnit(int dim = 0) : dim_(dim) {}
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return gatedlinearunit(input, dim_); }
+  std::string prettyString() const override { return "GatedLinearUnit (" + std::to_string(dim_) + ")"; }
+
+ private:
+  int dim_;
+};
+// nn/modules/Dropout.cpp:18-24: the identity in eval mode
+class Dropout : public UnaryModule {
+ public:
+  explicit Dropout(double ratio = 0.5) : ratio_(ratio) {}
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return train_ ? dropout(input, ratio_) : input; }
+  std::string prettyString() const override { return "Dropout (" + std::to_string(ratio_) + ")"; }
+
+ private:
+  double ratio_;
+};
+// nn/modules/Reorder.cpp:18-26
+class Reorder : public UnaryModule {
+ public:
+  explicit Reorder(Shape dims) : dims_(std::move(dims)) {}
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return reorder(input, dims_); }
+  std::string prettyString() const override { return "Reorder " + dims_.toString(); }
+
+ private:
+  Shape dims_;
+};
+
 class LogSoftmax : public UnaryModule {    // Activations.cpp:180-192
  public:
   explicit LogSoftmax(int dim = 0) : dim_(dim) {}

@@ -51,10 +51,11 @@ ModulePtr parseLine(const std::string& line) {
   auto I = [&](size_t i) { return toInt(p[i], line); };
   const std::string& op = p[0];
 
-  if (op == "V") {
+  if (op == "V" || op == "RO") {                 // SequentialBuilder.cpp:116-129
     if (n < 2) failParse(line);
     std::vector<Dim> dims;
     for (size_t i = 1; i < n; ++i) dims.push_back(I(i));
+    if (op == "RO") return std::make_shared<Reorder>(Shape(dims));
     return std::make_shared<View>(Shape(dims));
   }
   if (op == "C" || op == "C1") {
@@ -100,6 +101,35 @@ ModulePtr parseLine(const std::string& line) {
     if (n != 2) failParse(line);
     return std::make_shared<LogSoftmax>(I(1));
   }
+  // the other activations (SequentialBuilder.cpp:390-466) and dropout (:360-366)
+  auto F = [&](size_t i) {
+    try {
+      return std::stod(p[i]);
+    } catch (const std::exception&) {
+      failParse(line);
+    }
+    return 0.0;
+  };
+  if (op == "ELU" || op == "R6" || op == "LG" || op == "HT" || op == "T") {
+    if (n != 1) failParse(line);
+    if (op == "ELU") return std::make_shared<ELU>();
+    if (op == "R6") return std::make_shared<ReLU6>();
+    if (op == "LG") return std::make_shared<Log>();
+    if (op == "HT") return std::make_shared<HardTanh>();
+    return std::make_shared<Tanh>();
+  }
+  if (op == "GLU") {
+    if (n != 2) failParse(line);
+    return std::make_shared<GatedLinearUnit>(I(1));
+  }
+  if (op == "SH") {
+    if (!inRange(1, 2)) failParse(line);
+    return std::make_shared<Swish>(n > 1 ? (double)(float)F(1) : 1.0);      // std::stof there
+  }
+  if (op == "DO") {
+    if (n != 2) failParse(line);
+    return std::make_shared<Dropout>(F(1));
+  }
   if (op == "RNN" || op == "GRU" || op == "LSTM") {
     if (n < 3) failParse(line);
     const RnnMode mode = op == "RNN" ? RnnMode::RELU : op == "GRU" ? RnnMode::GRU : RnnMode::LSTM;
@@ -108,9 +138,8 @@ ModulePtr parseLine(const std::string& line) {
     const float dropout = n > 5 ? std::stof(p[5]) : 0.0f;
     return std::make_shared<RNN>(I(1), I(2), layers, mode, bidirectional, dropout);
   }
-  static const char* const absent[] = {"RO", "PD", "TR", "CFR", "POSEMB", "SINPOSEMB", "TDS", "AC", "E", "ADAPTIVEE",
-                                       "WN", "DO", "ELU", "R6", "PR", "LG", "HT", "T", "GLU", "SH", "RES", "SKIP",
-                                       "SKIPL", "SAUG", "PC"};
+  static const char* const absent[] = {"PD", "TR", "CFR", "POSEMB", "SINPOSEMB", "TDS", "AC", "E", "ADAPTIVEE",
+                                       "WN", "PR", "RES", "SKIP", "SKIPL", "SAUG", "PC"};
   for (const char* a : absent)
     if (op == a)
       throw std::invalid_argument("buildSequentialModule: module '" + op +

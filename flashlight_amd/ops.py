@@ -424,6 +424,73 @@ def relu_backward(grad_output, input):
     return dx
 
 
+ACT_ELU, ACT_CLAMP, ACT_TANH, ACT_LOG, ACT_SWISH, ACT_SIGMOID = range(6)
+
+
+def activation(op, input, a=0.0, b=0.0):
+    """flhip_act_fwd: the element-wise activations of nn/modules/Activations.cpp (ELU(a), clamp(a, b) = ReLU6 /
+    HardTanh, tanh, log, swish(a), sigmoid)."""
+    x = _dev(input, "input")
+    y = torch.empty_like(x)
+    capi.check(capi.lib().flhip_act_fwd(int(op), _ptr(x), _ptr(y), x.numel(), float(a), float(b), _dtype_tag(x),
+                                        _stream()))
+    return y
+
+
+def activation_backward(op, grad_output, input, a=0.0, b=0.0):
+    g, x = _dev(grad_output, "gradOutput"), _dev(input, "input")
+    if g.shape != x.shape or g.dtype != x.dtype:
+        raise ValueError("activation backward: gradOutput must match the input")
+    dx = torch.empty_like(x)
+    capi.check(capi.lib().flhip_act_bwd(int(op), _ptr(g), _ptr(x), _ptr(dx), x.numel(), float(a), float(b),
+                                        _dtype_tag(x), _stream()))
+    return dx
+
+
+def _glu_view(shape, dim):
+    """(outer, m) of fl::gatedlinearunit along torch dimension `dim` of a contiguous tensor."""
+    if shape[dim] % 2:
+        raise ValueError("halving dimension must be even for GLU")
+    outer = 1
+    for v in shape[:dim]:
+        outer *= v
+    m = shape[dim] // 2
+    for v in shape[dim + 1:]:
+        m *= v
+    return outer, m
+
+
+def gated_linear_unit(input, dim):
+    """fl::gatedlinearunit (Functions.cpp:1567-1610) along torch dimension `dim`."""
+    x = _dev(input, "input")
+    outer, m = _glu_view(tuple(x.shape), dim)
+    shape = list(x.shape)
+    shape[dim] //= 2
+    y = torch.empty(shape, dtype=x.dtype, device=x.device)
+    capi.check(capi.lib().flhip_glu_fwd(_ptr(x), _ptr(y), outer, m, _dtype_tag(x), _stream()))
+    return y
+
+
+def gated_linear_unit_backward(grad_output, input, dim):
+    g, x = _dev(grad_output, "gradOutput"), _dev(input, "input")
+    outer, m = _glu_view(tuple(x.shape), dim)
+    if g.numel() * 2 != x.numel() or g.dtype != x.dtype:
+        raise ValueError("GLU backward: gradOutput must have half the input's elements")
+    dx = torch.empty_like(x)
+    capi.check(capi.lib().flhip_glu_bwd(_ptr(g), _ptr(x), _ptr(dx), outer, m, _dtype_tag(x), _stream()))
+    return dx
+
+
+def dropout(input, p, seed):
+    """fl::dropout (Functions.cpp:1777-1785) with the counter-based mask of (seed, element index); the backward pass
+    is the same call on the gradient."""
+    x = _dev(input, "input")
+    y = torch.empty_like(x)
+    capi.check(capi.lib().flhip_dropout(_ptr(x), _ptr(y), x.numel(), float(p), int(seed) & 0xffffffff,
+                                        (int(seed) >> 32) & 0xffffffff, _dtype_tag(x), _stream()))
+    return y
+
+
 def linear(input, weight, bias=None):
     """fl::linear (Functions.cpp:1255-1309): input [..., in] (Flashlight [in, ...]), weight
     torch [in, out] (Flashlight [out, in]), bias [out] or None -> [..., out]."""

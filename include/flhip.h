@@ -115,8 +115,9 @@ const char* flhip_last_error(void);
  * compiled against is FLHIP_VERSION; descriptor structs only ever grow at the end, and a caller must
  * refuse to run when flhip_version() / 100 differs from FLHIP_VERSION / 100 (a layout change).
  * 200: flhip_rnn_desc gained dropout, seed_lo, seed_hi; flhip_bn_workspace_bytes never returns less
- * than 32 bytes per feature.  202: the *_plan entry points and FLHIP_DECLINED.  203: FLHIP_F16. */
-#define FLHIP_VERSION 203
+ * than 32 bytes per feature.  202: the *_plan entry points and FLHIP_DECLINED.  203: FLHIP_F16.  204: flhip_act_fwd / _bwd, flhip_glu_fwd / _bwd,
+ * flhip_dropout. */
+#define FLHIP_VERSION 204
 int flhip_version(void);
 const char* flhip_arch(void);
 
@@ -356,6 +357,38 @@ int flhip_add(const void* a, const void* b, void* out, size_t n, int dtype,
 int flhip_relu_fwd(const void* x, void* y, size_t n, int dtype, void* stream);
 int flhip_relu_bwd(const void* dy, const void* x, void* dx, size_t n, int dtype,
                    void* stream);
+
+/* The other element-wise activations of fl::nn (flashlight/fl/nn/modules/Activations.cpp), one entry point:
+ * y = f(x) over n elements, fp32 arithmetic, 16-bit storage rounded once.
+ *   FLHIP_ACT_ELU      a = alpha: x >= 0 ? x : a (exp(x) - 1)                  (Activations.cpp:136-139)
+ *   FLHIP_ACT_CLAMP    a = lo, b = hi: fl::clamp (Functions.cpp:465-475); ReLU6 = clamp(0, 6), HardTanh = clamp(-1, 1)
+ *                      (Activations.cpp:60-62, 88-90)
+ *   FLHIP_ACT_TANH     fl::tanh (Functions.cpp:454-463)      FLHIP_ACT_LOG      fl::log (:403-411)
+ *   FLHIP_ACT_SWISH    a = beta: x * sigmoid(a x) (:498-500)  FLHIP_ACT_SIGMOID  fl::sigmoid (:488-496)
+ * flhip_act_bwd: dx = dy * f'(x) from the gradient and the forward INPUT (clamp passes the gradient where
+ * lo < x < hi, strictly, as the reference's mask on its result does).  y / dx may alias x / dy. */
+#define FLHIP_ACT_ELU 0
+#define FLHIP_ACT_CLAMP 1
+#define FLHIP_ACT_TANH 2
+#define FLHIP_ACT_LOG 3
+#define FLHIP_ACT_SWISH 4
+#define FLHIP_ACT_SIGMOID 5
+int flhip_act_fwd(int op, const void* x, void* y, size_t n, double a, double b, int dtype, void* stream);
+int flhip_act_bwd(int op, const void* dy, const void* x, void* dx, size_t n, double a, double b, int dtype,
+                  void* stream);
+
+/* fl::gatedlinearunit (Functions.cpp:1567-1610) along a dimension whose two halves are contiguous blocks of m
+ * elements per outer index (column-major tensor, halved dimension d: m = half the extent of d times the product of
+ * the extents before it, outer = the product of the extents after it): y[o][k] = x[o][0][k] * sigmoid(x[o][1][k]);
+ * backward dx[o][0][k] = sigmoid(x[o][1][k]) dy, dx[o][1][k] = x[o][0][k] s (1 - s) dy.  dx must not alias x. */
+int flhip_glu_fwd(const void* x, void* y, int64_t outer, int64_t m, int dtype, void* stream);
+int flhip_glu_bwd(const void* dy, const void* x, void* dx, int64_t outer, int64_t m, int dtype, void* stream);
+
+/* fl::dropout (Functions.cpp:1777-1785): y = x * keep / (1 - p) with keep(i) a counter-based function of
+ * (seed, i) - the reference draws fl::rand(...) > p, so masks differ from its generator's while rate and scaling
+ * are the same.  The backward pass is the same call on the gradient with the same seed and p.  y may alias x. */
+int flhip_dropout(const void* x, void* y, size_t n, double p, uint32_t seed_lo, uint32_t seed_hi, int dtype,
+                  void* stream);
 
 /* C (M x N) = op(A) (M x K) * op(B) (K x N), fp32 accumulate; trans_a: A is stored
  * K x M, trans_b: B is stored N x K.  bias_rows (fp32[M], may be NULL) is added to

@@ -401,6 +401,65 @@ void flref_relu_bwd(int64_t n, const float* dy, const float* x, float* dx) {
   for (int64_t i = 0; i < n; ++i) dx[i] = x[i] > 0.f ? dy[i] : 0.f;
 }
 
+/* The element-wise activations of nn/modules/Activations.cpp, in double, rounded once.  op as FLHIP_ACT_*:
+ * 0 ELU (a = alpha; :136-139 there), 1 clamp(a, b) (Functions.cpp:465-475), 2 tanh (:454-463), 3 log (:403-411),
+ * 4 swish (a = beta; :498-500), 5 sigmoid (:488-496). */
+static double act_sigmoid(double v) { return 1.0 / (1.0 + exp(-v)); }
+void flref_act_fwd(int op, int64_t n, const float* x, double a, double b, float* y) {
+  for (int64_t i = 0; i < n; ++i) {
+    const double v = x[i];
+    double r;
+    switch (op) {
+      case 0: r = v >= 0.0 ? v : a * (exp(v) - 1.0); break;
+      case 1: r = v < a ? a : v > b ? b : v; break;
+      case 2: r = tanh(v); break;
+      case 3: r = log(v); break;
+      case 4: r = v * act_sigmoid(a * v); break;
+      default: r = act_sigmoid(v); break;
+    }
+    y[i] = (float)r;
+  }
+}
+/* gradients of the same: the reference's closures (ELU and swish: the chain of their element-wise pieces) */
+void flref_act_bwd(int op, int64_t n, const float* dy, const float* x, double a, double b, float* dx) {
+  for (int64_t i = 0; i < n; ++i) {
+    const double v = x[i], g = dy[i];
+    double r;
+    switch (op) {
+      case 0: r = v >= 0.0 ? g : g * a * exp(v); break;
+      case 1: r = (v > a && v < b) ? g : 0.0; break;          /* (result > lo) && (result < hi), :471 */
+      case 2: { const double t = tanh(v); r = (1.0 - t * t) * g; break; }
+      case 3: r = g / v; break;
+      case 4: { const double sg = act_sigmoid(a * v); r = g * (sg + v * a * sg * (1.0 - sg)); break; }
+      default: { const double sg = act_sigmoid(v); r = g * sg * (1.0 - sg); break; }
+    }
+    dx[i] = (float)r;
+  }
+}
+
+/* fl::gatedlinearunit (Functions.cpp:1567-1610) with the halves as contiguous blocks of m elements per outer index */
+void flref_glu_fwd(int64_t outer, int64_t m, const float* x, float* y) {
+  for (int64_t o = 0; o < outer; ++o)
+    for (int64_t k = 0; k < m; ++k)
+      y[o * m + k] = (float)((double)x[2 * o * m + k] * act_sigmoid(x[(2 * o + 1) * m + k]));
+}
+void flref_glu_bwd(int64_t outer, int64_t m, const float* dy, const float* x, float* dx) {
+  for (int64_t o = 0; o < outer; ++o)
+    for (int64_t k = 0; k < m; ++k) {
+      const double a = x[2 * o * m + k], sg = act_sigmoid(x[(2 * o + 1) * m + k]), g = dy[o * m + k];
+      dx[2 * o * m + k] = (float)(sg * g);                          /* :1598 */
+      dx[(2 * o + 1) * m + k] = (float)(a * sg * (1.0 - sg) * g);   /* :1599-1600 */
+    }
+}
+
+/* fl::dropout (Functions.cpp:1777-1785) with the counter-based mask below in the place of fl::rand(...) > p */
+int flref_dropout_keep(uint32_t seed_lo, uint32_t seed_hi, uint32_t layer, uint32_t index, float dropout);
+void flref_dropout(int64_t n, const float* x, double p, uint32_t seed_lo, uint32_t seed_hi, float* y) {
+  const float scale = (float)(1.0 / (1.0 - p));
+  for (int64_t i = 0; i < n; ++i)
+    y[i] = flref_dropout_keep(seed_lo, seed_hi, (uint32_t)((uint64_t)i >> 32), (uint32_t)i, (float)p) ? x[i] * scale : 0.f;
+}
+
 /* fl::matmul / matmulTN / matmulNT as used by fl::linear (:1264-1265, 1292-1301) */
 void flref_matmul(int M, int N, int K, int ta, int tb, const float* A, const float* B,
                   const float* bias, float* C) {

@@ -100,6 +100,15 @@ void flref_bn_running_update(int64_t C, int64_t M, const float* mean,
 /* max(x, 0) and its mask backward (:329-338, 1787-1789) */
 void flref_relu_fwd(int64_t n, const float* x, float* y);
 void flref_relu_bwd(int64_t n, const float* dy, const float* x, float* dx);
+/* element-wise activations of nn/modules/Activations.cpp: op 0 ELU(a), 1 clamp(a, b), 2 tanh, 3 log, 4 swish(a),
+ * 5 sigmoid; the backward takes the forward input */
+void flref_act_fwd(int op, int64_t n, const float* x, double a, double b, float* y);
+void flref_act_bwd(int op, int64_t n, const float* dy, const float* x, double a, double b, float* dx);
+/* gatedlinearunit (:1567-1610): halves are contiguous blocks of m elements per outer index */
+void flref_glu_fwd(int64_t outer, int64_t m, const float* x, float* y);
+void flref_glu_bwd(int64_t outer, int64_t m, const float* dy, const float* x, float* dx);
+/* dropout (:1777-1785) with the counter-based mask of flref_dropout_keep */
+void flref_dropout(int64_t n, const float* x, double p, uint32_t seed_lo, uint32_t seed_hi, float* y);
 /* C (M x N) = op(A) op(B) + bias[m]; ta: A stored K x M, tb: B stored N x K; double
  * accumulate.  fl::linear (:1255-1309) = (W, X), backward (W^T, dY) and (dY, X^T). */
 void flref_matmul(int M, int N, int K, int ta, int tb, const float* A, const float* B,

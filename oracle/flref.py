@@ -191,6 +191,45 @@ def relu_fwd(x):
     return y
 
 
+ACT_ELU, ACT_CLAMP, ACT_TANH, ACT_LOG, ACT_SWISH, ACT_SIGMOID = range(6)
+
+
+def act_fwd(op, x, a=0.0, b=0.0):
+    x = _f32(x)
+    y = np.empty_like(x)
+    lib().flref_act_fwd(C.c_int(op), _i64(x.size), _p(x), C.c_double(a), C.c_double(b), _p(y))
+    return y
+
+
+def act_bwd(op, dy, x, a=0.0, b=0.0):
+    dy, x = _f32(dy), _f32(x)
+    dx = np.empty_like(x)
+    lib().flref_act_bwd(C.c_int(op), _i64(x.size), _p(dy), _p(x), C.c_double(a), C.c_double(b), _p(dx))
+    return dx
+
+
+def glu_fwd(x, outer, m):
+    """x: any array of outer * 2 * m elements in memory order [outer][2][m]."""
+    x = _f32(x)
+    y = np.empty(outer * m, np.float32)
+    lib().flref_glu_fwd(_i64(outer), _i64(m), _p(x), _p(y))
+    return y
+
+
+def glu_bwd(dy, x, outer, m):
+    dy, x = _f32(dy), _f32(x)
+    dx = np.empty_like(x)
+    lib().flref_glu_bwd(_i64(outer), _i64(m), _p(dy), _p(x), _p(dx))
+    return dx
+
+
+def dropout(x, p, seed_lo, seed_hi):
+    x = _f32(x)
+    y = np.empty_like(x)
+    lib().flref_dropout(_i64(x.size), _p(x), C.c_double(p), C.c_uint32(seed_lo), C.c_uint32(seed_hi), _p(y))
+    return y
+
+
 def relu_bwd(dy, x):
     dy, x = _f32(dy), _f32(x)
     dx = np.empty_like(x)

@@ -957,7 +957,8 @@ static void testArchBuilder() {
   CHECK(one("BN 8 0 1")->prettyString() == BatchNorm(std::vector<int>{0, 1}, 8).prettyString());
   // malformed lines, lines for modules that do not exist here, a missing file
   for (const char* bad : {"C 3 4 5", "C2 3 4 5 6 1", "L 5", "BN 8", "LN", "LN 3", "M 2 2 2", "R 1", "LSM", "GRU 4",
-                          "C 3 x 5 1", "XYZ 1 2", "RO 1 0 2 3", "DO 0.2", "TDS 10 21 80", "RES 2 1 3", "PC f16"})
+                          "C 3 x 5 1", "XYZ 1 2", "RO", "DO", "DO 0.2 1", "GLU", "ELU 1", "SH 1 2", "WN 3 C 1 2 3 4", "PD 0 1 1",
+                          "TDS 10 21 80", "RES 2 1 3", "PC f16"})
     CHECK(throws<std::invalid_argument>([&] { one(bad); }));
   CHECK(throws<std::runtime_error>([] { buildSequentialModule(std::string("/nonexistent/arch.txt"), 1, 1); }));
   // from a file
@@ -971,6 +972,119 @@ static void testArchBuilder() {
     std::remove(path.c_str());
   } else {
     CHECK(false);
+  }
+}
+
+// the element-wise modules of nn/modules/Activations.cpp, GatedLinearUnit, Dropout and Reorder, through their
+// modules and architecture lines, forward and backward against the CPU checker
+static void testActivationModules() {
+  std::printf("activation modules, GLU, dropout, reorder\n");
+  using fl::pkg::runtime::buildSequentialModule;
+  auto one = [](const std::string& l) { return buildSequentialModule(std::vector<std::string>{l}, 1, 1)->module(0); };
+  struct Case { const char* line; int op; double a, b; };
+  const Case cases[] = {{"ELU", 0, 1.0, 0.0}, {"R6", 1, 0.0, 6.0}, {"HT", 1, -1.0, 1.0}, {"T", 2, 0.0, 0.0},
+                        {"LG", 3, 0.0, 0.0}, {"SH", 4, 1.0, 0.0}, {"SH 1.5", 4, 1.5, 0.0}};
+  const Shape shp({9, 5, 4, 3});
+  const size_t n = 9 * 5 * 4 * 3;
+  for (dtype dt : {dtype::f32, dtype::bf16, dtype::f16}) {
+    const double tol = dt == dtype::f32 ? 2e-6 : 4e-3;
+    for (const Case& c : cases) {
+      auto x = randn(n, 700 + c.op, 3.f), dy = randn(n, 701);
+      if (c.op == 3) for (auto& v : x) v = std::fabs(v) + 0.05f;
+      for (auto& v : x) v = roundTo(dt, v);
+      for (auto& v : dy) v = roundTo(dt, v);
+      Variable in(Tensor::fromVector(shp, x).astype(dt), true);
+      auto mod = one(c.line);
+      Variable y = mod->forward({in})[0];
+      y.backward(Variable(Tensor::fromVector(shp, dy).astype(dt), false));
+      std::vector<float> yr(n), dxr(n);
+      flref_act_fwd(c.op, (int64_t)n, x.data(), c.a, c.b, yr.data());
+      flref_act_bwd(c.op, (int64_t)n, dy.data(), x.data(), c.a, c.b, dxr.data());
+      CHECK(y.type() == dt && in.grad().type() == dt);
+      CHECK(relL2(hostOf(y), yr) <= tol);
+      CHECK(relL2(hostOf(in.grad()), dxr) <= tol);
+    }
+    // GLU along each dimension of the column-major shape: memory order [outer][2][m]
+    for (int dim : {0, 1, 2}) {
+      const Shape gs({8, 6, 4, 2});
+      const size_t gn = 8 * 6 * 4 * 2;
+      auto x = randn(gn, 710 + dim), dy = randn(gn / 2, 711);
+      for (auto& v : x) v = roundTo(dt, v);
+      for (auto& v : dy) v = roundTo(dt, v);
+      long long m = gs.dim(dim) / 2, outer = 1;
+      for (int i = 0; i < dim; ++i) m *= gs.dim(i);
+      for (int i = dim + 1; i < 4; ++i) outer *= gs.dim(i);
+      Variable in(Tensor::fromVector(gs, x).astype(dt), true);
+      Variable y = one("GLU " + std::to_string(dim))->forward({in})[0];
+      CHECK(y.shape().dim(dim) == gs.dim(dim) / 2 && (size_t)y.tensor().elements() == gn / 2);
+      y.backward(Variable(Tensor::fromVector(y.shape(), dy).astype(dt), false));
+      std::vector<float> yr(gn / 2), dxr(gn);
+      flref_glu_fwd(outer, m, x.data(), yr.data());
+      flref_glu_bwd(outer, m, dy.data(), x.data(), dxr.data());
+      CHECK(relL2(hostOf(y), yr) <= tol);
+      CHECK(relL2(hostOf(in.grad()), dxr) <= tol);
+    }
+  }
+  CHECK(throws<std::invalid_argument>([&] { gatedlinearunit(Variable(Tensor::fromVector({3, 5}, randn(15, 1)), false), 0); }));
+  CHECK(throws<std::invalid_argument>([&] { gatedlinearunit(Variable(Tensor::fromVector({4, 5}, randn(20, 1)), false), 2); }));
+
+  // dropout: rate, scale, the backward pass uses the forward pass's mask, eval mode is the identity, p = 0 too
+  {
+    const size_t dn = 200000;
+    std::vector<float> ones(dn, 1.f);
+    auto dy = randn(dn, 720);
+    setSeed(5);
+    auto drop = one("DO 0.3");
+    Variable in(Tensor::fromVector({(Dim)dn}, ones), true);
+    Variable y = drop->forward({in})[0];
+    y.backward(Variable(Tensor::fromVector({(Dim)dn}, dy), false));
+    auto yh = hostOf(y), gh = hostOf(in.grad());
+    size_t kept = 0;
+    bool ok = true;
+    for (size_t i = 0; i < dn; ++i) {
+      if (yh[i] != 0.f) {
+        ++kept;
+        ok = ok && std::fabs(yh[i] - 1.f / 0.7f) < 1e-6f && std::fabs(gh[i] - dy[i] * (1.f / 0.7f)) <= 1e-6f * std::fabs(dy[i]) + 1e-12f;
+      } else {
+        ok = ok && gh[i] == 0.f;
+      }
+    }
+    CHECK(ok);
+    CHECK(std::fabs((double)kept / dn - 0.7) < 4 * std::sqrt(0.3 * 0.7 / dn));
+    // another call draws another mask; the same seed draws the same
+    Variable y2 = drop->forward({in})[0];
+    CHECK(hostOf(y2) != yh);
+    setSeed(5);
+    CHECK(hostOf(drop->forward({in})[0]) == yh);
+    drop->eval();
+    CHECK(hostOf(drop->forward({in})[0]) == ones);
+    CHECK(hostOf(dropout(in, 0.0)) == ones);
+    CHECK(throws<std::invalid_argument>([&] { dropout(in, 1.0); }));
+  }
+  // RO: the Reorder module is fl::reorder
+  {
+    auto x = randn(2 * 3 * 4 * 5, 730);
+    Variable a(Tensor::fromVector({2, 3, 4, 5}, x), true), b(Tensor::fromVector({2, 3, 4, 5}, x), true);
+    Variable y1 = one("RO 2 0 3 1")->forward({a})[0], y2 = reorder(b, Shape({2, 0, 3, 1}));
+    CHECK(y1.shape() == Shape({4, 2, 5, 3}) && hostOf(y1) == hostOf(y2));
+    auto dy = randn(x.size(), 731);
+    y1.backward(Variable(Tensor::fromVector(y1.shape(), dy), false));
+    y2.backward(Variable(Tensor::fromVector(y2.shape(), dy), false));
+    CHECK(hostOf(a.grad()) == hostOf(b.grad()));
+  }
+  // a GLU convolution block from text, as in wav2letter's architecture files
+  {
+    setSeed(17);
+    auto net = buildSequentialModule(std::vector<std::string>{"V -1 1 NFEAT 0", "C NFEAT 32 5 1 -1", "GLU 2", "DO 0.2",
+                                                              "C 16 24 3 1 -1", "HT", "RO 2 0 3 1", "V 24 -1", "L 24 NLABEL", "LSM 0"},
+                                     10, 6);
+    CHECK(net->modules().size() == 10);
+    Variable in(Tensor::fromVector({30, 10, 1, 2}, randn(600, 740)), true);
+    Variable y = net->forward(in);
+    CHECK(y.shape() == Shape({6, 60}));
+    y.backward(Variable(Tensor::fromVector(y.shape(), randn(360, 741)), false));
+    CHECK(in.grad().shape() == in.shape());
+    for (const auto& p : net->params()) CHECK(p.isGradAvailable());
   }
 }
 
@@ -1241,6 +1355,7 @@ int main() {
     testSpeechStack(1500, 16);
     testRnn();
     testArchBuilder();
+    testActivationModules();
     testModuleShapesAndBatching();
     testInit();
     testDynamicBenchmark();

@@ -320,3 +320,63 @@ def test_astype_with_f16(src, dst):
     assert torch.equal(got.view(bits)[~nan], ref.view(bits)[~nan])
     many = ops.astype_many([x, x[:5], x[:0]], dst)
     assert torch.equal(many[0].float().nan_to_num(7.0), got.float().nan_to_num(7.0)) and many[2].numel() == 0
+
+
+# ---- activations, gated linear unit, dropout (nn/modules/Activations.cpp, Functions.cpp:1567-1610, 1777-1785) ----
+_ACTS = [(ops.ACT_ELU, 1.0, 0.0), (ops.ACT_ELU, 0.3, 0.0), (ops.ACT_CLAMP, 0.0, 6.0), (ops.ACT_CLAMP, -1.0, 1.0),
+         (ops.ACT_TANH, 0.0, 0.0), (ops.ACT_LOG, 0.0, 0.0), (ops.ACT_SWISH, 1.0, 0.0), (ops.ACT_SWISH, 1.7, 0.0),
+         (ops.ACT_SIGMOID, 0.0, 0.0)]
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("op,a,b", _ACTS)
+@pytest.mark.parametrize("n", [4099, 1 << 18, 3])
+def test_activations(op, a, b, n, dtype):
+    rng = np.random.default_rng(70 + op)
+    x = (rng.standard_normal(n) * 3).astype(np.float32)
+    if op == ops.ACT_LOG:
+        x = np.abs(x) + 0.05
+    if op == ops.ACT_CLAMP and n >= 4:
+        x[:4] = [a, b, np.nextafter(np.float32(a), np.float32(9)), np.nextafter(np.float32(b), np.float32(-9))]
+    x = _round(x, dtype)
+    dy = _round(rng.standard_normal(n).astype(np.float32), dtype)
+    y = host(ops.activation(op, dev(x, dtype), a, b))
+    dx = host(ops.activation_backward(op, dev(dy, dtype), dev(x, dtype), a, b))
+    tol = 2e-6 if dtype == torch.float32 else 4e-3
+    assert rel_l2(y, flref.act_fwd(op, x, a, b)) <= tol
+    assert rel_l2(dx, flref.act_bwd(op, dy, x, a, b)) <= tol
+    if op == ops.ACT_CLAMP:      # selections and copies: exact
+        assert np.array_equal(y, flref.act_fwd(op, x, a, b))
+        assert np.array_equal(dx, flref.act_bwd(op, dy, x, a, b))
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("shape,dim", [((3, 8, 5), 1), ((4, 6), 1), ((10, 7), 0), ((2, 3, 4, 6), 3), ((16, 400, 1, 150), 1)])
+def test_gated_linear_unit(shape, dim, dtype):
+    rng = np.random.default_rng(80 + dim)
+    x = _round(rng.standard_normal(shape).astype(np.float32), dtype)
+    outer = int(np.prod(shape[:dim], dtype=np.int64))
+    m = shape[dim] // 2 * int(np.prod(shape[dim + 1:], dtype=np.int64))
+    y_ref = flref.glu_fwd(x, outer, m)
+    dy = _round(rng.standard_normal(y_ref.shape).astype(np.float32), dtype)
+    tol = 2e-6 if dtype == torch.float32 else 4e-3
+    y = ops.gated_linear_unit(dev(x, dtype), dim)
+    assert tuple(y.shape) == tuple(s // 2 if i == dim else s for i, s in enumerate(shape))
+    assert rel_l2(host(y).ravel(), y_ref) <= tol
+    dx = ops.gated_linear_unit_backward(dev(dy.reshape(y.shape), dtype), dev(x, dtype), dim)
+    assert rel_l2(host(dx).ravel(), flref.glu_bwd(dy, x, outer, m).ravel()) <= tol
+    with pytest.raises(ValueError):
+        ops.gated_linear_unit(dev(np.zeros((3, 5), np.float32), dtype), 1)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("p", [0.0, 0.2, 0.75])
+def test_dropout_mask_matches_the_checker(p, dtype):
+    rng = np.random.default_rng(90)
+    x = _round(rng.standard_normal(100003).astype(np.float32), dtype)
+    seed = (77 << 32) | 12345
+    y = host(ops.dropout(dev(x, dtype), p, seed))
+    ref = flref.dropout(x, p, 12345, 77)
+    assert np.array_equal(y == 0, ref == 0)            # the same mask
+    assert rel_l2(y, ref) <= (1e-6 if dtype == torch.float32 else 4e-3)
+    assert np.array_equal(y, host(ops.dropout(dev(x, dtype), p, seed)))

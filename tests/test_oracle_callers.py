@@ -183,3 +183,70 @@ def test_layer_norm_restated_on_batchnorm_is_layer_norm(whcn, norm, params):
     if params_t:
         assert rel_l2(dw, params_t[0].grad.numpy().reshape(-1)) < 1e-5
         assert rel_l2(db, params_t[1].grad.numpy().reshape(-1)) < 1e-5
+
+
+# ---- the element-wise activations of nn/modules/Activations.cpp, gatedlinearunit, dropout ----
+# (op, a, b, torch function in float64); log gets positive inputs
+_ACTS = [
+    (flref.ACT_ELU, 1.0, 0.0, lambda t: F.elu(t, alpha=1.0)),
+    (flref.ACT_ELU, 0.3, 0.0, lambda t: F.elu(t, alpha=0.3)),
+    (flref.ACT_CLAMP, 0.0, 6.0, lambda t: F.relu6(t)),
+    (flref.ACT_CLAMP, -1.0, 1.0, lambda t: F.hardtanh(t)),
+    (flref.ACT_TANH, 0.0, 0.0, torch.tanh),
+    (flref.ACT_LOG, 0.0, 0.0, torch.log),
+    (flref.ACT_SWISH, 1.0, 0.0, F.silu),
+    (flref.ACT_SWISH, 1.7, 0.0, lambda t: t * torch.sigmoid(1.7 * t)),
+    (flref.ACT_SIGMOID, 0.0, 0.0, torch.sigmoid),
+]
+
+
+@pytest.mark.parametrize("op,a,b,fn", _ACTS)
+def test_activations_against_torch_float64(op, a, b, fn):
+    rng = np.random.default_rng(300 + op)
+    x = (rng.standard_normal(4000) * 3).astype(np.float32)
+    if op == flref.ACT_LOG:
+        x = np.abs(x) + 0.05
+    dy = rng.standard_normal(4000).astype(np.float32)
+    t = torch.from_numpy(x.astype(np.float64)).requires_grad_(True)
+    y = fn(t)
+    y.backward(torch.from_numpy(dy.astype(np.float64)))
+    assert rel_l2(flref.act_fwd(op, x, a, b), y.detach().numpy()) <= 1e-6
+    assert rel_l2(flref.act_bwd(op, dy, x, a, b), t.grad.numpy()) <= 1e-6
+
+
+def test_clamp_passes_the_gradient_strictly_inside():
+    # Functions.cpp:471: (result > lo) && (result < hi) — nothing at the bounds themselves
+    x = np.array([-2.0, -1.0, -0.5, 0.0, 1.0, 1.5, 6.0, 7.0], np.float32)
+    dy = np.arange(1, 9, dtype=np.float32)
+    assert np.array_equal(flref.act_fwd(flref.ACT_CLAMP, x, -1.0, 1.0), np.array([-1, -1, -0.5, 0, 1, 1, 1, 1], np.float32))
+    assert np.array_equal(flref.act_bwd(flref.ACT_CLAMP, dy, x, -1.0, 1.0), np.array([0, 0, 3, 4, 0, 0, 0, 0], np.float32))
+    assert np.array_equal(flref.act_bwd(flref.ACT_CLAMP, dy, x, 0.0, 6.0), np.array([0, 0, 0, 0, 5, 6, 0, 0], np.float32))
+
+
+@pytest.mark.parametrize("shape,dim", [((3, 8, 5), 1), ((4, 6), 1), ((10, 7), 0), ((2, 3, 4, 6), 3), ((2, 4, 3, 5), 1)])
+def test_glu_against_torch_float64(shape, dim):
+    # Functions.cpp:1567-1610; a torch dimension `dim` of a contiguous array: halves are blocks of m per outer index
+    rng = np.random.default_rng(310 + dim)
+    x = rng.standard_normal(shape).astype(np.float32)
+    outer = int(np.prod(shape[:dim], dtype=np.int64))
+    m = shape[dim] // 2 * int(np.prod(shape[dim + 1:], dtype=np.int64))
+    t = torch.from_numpy(x.astype(np.float64)).requires_grad_(True)
+    y = F.glu(t, dim)
+    dy = rng.standard_normal(tuple(y.shape)).astype(np.float32)
+    y.backward(torch.from_numpy(dy.astype(np.float64)))
+    assert rel_l2(flref.glu_fwd(x, outer, m).reshape(y.shape), y.detach().numpy()) <= 1e-6
+    assert rel_l2(flref.glu_bwd(dy, x, outer, m).reshape(shape), t.grad.numpy()) <= 1e-6
+
+
+def test_dropout_mask_rate_scale_and_determinism():
+    # Functions.cpp:1777-1785: zero with probability p, the rest scaled by 1 / (1 - p); the mask is a function of
+    # (seed, index) only
+    x = np.ones(200000, np.float32)
+    for p in (0.2, 0.5, 0.9):
+        y = flref.dropout(x, p, 123, 456)
+        kept = y != 0
+        assert np.allclose(y[kept], 1.0 / (1.0 - p), rtol=1e-6)
+        assert abs(kept.mean() - (1.0 - p)) < 4 * np.sqrt(p * (1 - p) / x.size)
+        assert np.array_equal(y, flref.dropout(x, p, 123, 456))
+        assert not np.array_equal(y, flref.dropout(x, p, 124, 456))
+    assert np.array_equal(flref.dropout(x, 0.0, 1, 2), x)
