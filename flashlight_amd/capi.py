@@ -85,6 +85,11 @@ SYMBOLS = {
     "flhip_glu_fwd": (C.c_int, [_VP, _VP, C.c_int64, C.c_int64, C.c_int, _VP]),
     "flhip_glu_bwd": (C.c_int, [_VP, _VP, _VP, C.c_int64, C.c_int64, C.c_int, _VP]),
     "flhip_dropout": (C.c_int, [_VP, _VP, _SZ, C.c_double, C.c_uint32, C.c_uint32, C.c_int, _VP]),
+    "flhip_rownorm": (C.c_int, [_VP, _VP, C.c_int64, C.c_int64, C.c_int, C.c_int, _VP]),
+    "flhip_weightnorm_fwd": (C.c_int, [_VP, _VP, _VP, C.c_int64, C.c_int64, C.c_int, C.c_int, _VP]),
+    "flhip_weightnorm_bwd": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_int64, C.c_int64, C.c_int, C.c_int, _VP]),
+    "flhip_pad_fwd": (C.c_int, [_VP, _VP, C.POINTER(C.c_int64), C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.c_double, C.c_int, _VP]),
+    "flhip_pad_bwd": (C.c_int, [_VP, _VP, C.POINTER(C.c_int64), C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.c_int, _VP]),
     "flhip_matmul": (C.c_int, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int, C.c_int, _VP,
                                C.c_int, _VP]),
     "flhip_sum_columns": (C.c_int, [_VP, _VP, C.c_int32, C.c_int32, C.c_int, _VP]),

@@ -98,6 +98,119 @@ __global__ void __launch_bounds__(256) dropout_kernel(const T* __restrict__ x, T
   }
 }
 
+// ---- WeightNorm (flashlight/fl/nn/modules/WeightNorm.cpp:45-72): w = v * g[r] / ||v_r|| with one g per index r of the
+// kept dimension; the tensor is a rows x cols matrix whose rows are either contiguous (the kept dimension is the
+// slowest: Conv2D weights, dim 3) or interleaved (it is the fastest: Linear weights, dim 0: element (r, j) at r + j * rows).
+// MODE 0: n[r] = ||v_r|| (the initial g).  MODE 1: w.  MODE 2: dv = (g / n) (dw - c v / n^2), dg[r] = c / n with
+// c = sum_j dw v (the chain of the reference's norm, division, tileAs and product). ----
+template <typename T, int MODE>
+__global__ void __launch_bounds__(256)
+wn_rows_kernel(const T* __restrict__ v, const T* __restrict__ g, const T* __restrict__ dw, T* __restrict__ out,
+               T* __restrict__ dg, long long cols) {
+  __shared__ float red[2][4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const size_t base = (size_t)blockIdx.x * (size_t)cols;
+  float s2 = 0.f, c = 0.f;
+  for (long long j = tid; j < cols; j += 256) {
+    const float x = ld(v, base + j);
+    s2 += x * x;
+    if (MODE == 2) c += ld(dw, base + j) * x;
+  }
+  s2 = wave_sum(s2);
+  if (MODE == 2) c = wave_sum(c);
+  if (lane == 0) {
+    red[0][wave] = s2;
+    red[1][wave] = c;
+  }
+  __syncthreads();
+  s2 = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
+  c = (red[1][0] + red[1][1]) + (red[1][2] + red[1][3]);
+  const float n = sqrtf(s2);
+  if (MODE == 0) {
+    if (tid == 0) st(out, blockIdx.x, n);
+    return;
+  }
+  const float scale = ld(g, blockIdx.x) / n;
+  if (MODE == 1) {
+    for (long long j = tid; j < cols; j += 256) st(out, base + j, ld(v, base + j) * scale);
+  } else {
+    const float k = c / s2;
+    for (long long j = tid; j < cols; j += 256) st(out, base + j, scale * (ld(dw, base + j) - k * ld(v, base + j)));
+    if (tid == 0) st(dg, blockIdx.x, c / n);
+  }
+}
+// interleaved rows: lane = row (64 consecutive rows are contiguous), the four waves split the columns
+template <typename T, int MODE>
+__global__ void __launch_bounds__(256)
+wn_cols_kernel(const T* __restrict__ v, const T* __restrict__ g, const T* __restrict__ dw, T* __restrict__ out,
+               T* __restrict__ dg, long long rows, long long cols) {
+  __shared__ float red[2][4][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const long long r = (long long)blockIdx.x * 64 + lane;
+  const bool rv = r < rows;
+  float s2 = 0.f, c = 0.f;
+  if (rv)
+    for (long long j = wave; j < cols; j += 4) {
+      const size_t e = (size_t)r + (size_t)j * (size_t)rows;
+      const float x = ld(v, e);
+      s2 += x * x;
+      if (MODE == 2) c += ld(dw, e) * x;
+    }
+  red[0][wave][lane] = s2;
+  red[1][wave][lane] = c;
+  __syncthreads();
+  s2 = (red[0][0][lane] + red[0][1][lane]) + (red[0][2][lane] + red[0][3][lane]);
+  c = (red[1][0][lane] + red[1][1][lane]) + (red[1][2][lane] + red[1][3][lane]);
+  if (!rv) return;
+  const float n = sqrtf(s2);
+  if (MODE == 0) {
+    if (wave == 0) st(out, (size_t)r, n);
+    return;
+  }
+  const float scale = ld(g, (size_t)r) / n, k = c / s2;
+  for (long long j = wave; j < cols; j += 4) {
+    const size_t e = (size_t)r + (size_t)j * (size_t)rows;
+    st(out, e, MODE == 1 ? ld(v, e) * scale : scale * (ld(dw, e) - k * ld(v, e)));
+  }
+  if (MODE == 2 && wave == 0) st(dg, (size_t)r, c / n);
+}
+
+// ---- fl::padding (Functions.cpp:1751-1775): the input inside a tensor of `value`; one thread per result element,
+// up to four column-major dimensions; the backward pass copies the inner box back ----
+struct PadGeom {
+  long long od[4], id[4], lo[4];
+};
+template <typename T, bool BWD>
+__global__ void __launch_bounds__(256) pad_kernel(const T* __restrict__ src, T* __restrict__ dst, size_t n, PadGeom g, float value) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    // forward: i walks the padded result; backward: i walks the input-shaped gradient
+    size_t rem = i;
+    long long c[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const long long ext = BWD ? g.id[k] : g.od[k];
+      c[k] = (long long)(rem % (size_t)ext);
+      rem /= (size_t)ext;
+    }
+    if (BWD) {
+      const size_t o = (size_t)(c[0] + g.lo[0]) + (size_t)g.od[0] * ((size_t)(c[1] + g.lo[1]) + (size_t)g.od[1] * ((size_t)(c[2] + g.lo[2]) + (size_t)g.od[2] * (size_t)(c[3] + g.lo[3])));
+      st(dst, i, ld(src, o));
+    } else {
+      bool in = true;
+      size_t e = 0, mul = 1;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const long long q = c[k] - g.lo[k];
+        in = in && q >= 0 && q < g.id[k];
+        e += (size_t)(in ? q : 0) * mul;
+        mul *= (size_t)g.id[k];
+      }
+      st(dst, i, in ? ld(src, e) : value);
+    }
+  }
+}
+
 // ---- C = op(A) op(B) (+ bias per row), 64 x 64 tiles, 256 threads, 4 x 4 per thread ----
 constexpr int GT = 64, GK = 16;
 
@@ -700,6 +813,73 @@ extern "C" int flhip_dropout(const void* x, void* y, size_t n, double p, uint32_
                        seed_lo, seed_hi, (float)p, (float)(1.0 / (1.0 - p)));
   });
   return check_launch("dropout");
+}
+
+template <int MODE>
+static int weightnorm_launch(const char* what, const void* v, const void* g, const void* dw, void* out, void* dg,
+                             int64_t rows, int64_t cols, int rows_fast, int dtype, void* stream) {
+  FLHIP_REQUIRE(v && out && (MODE == 0 || g) && (MODE != 2 || (dw && dg)), "weightnorm: null argument");
+  FLHIP_REQUIRE(rows > 0 && cols > 0, "weightnorm: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "weightnorm: unknown dtype");
+  FLHIP_REQUIRE(rows <= 0x7fffffffll, "weightnorm: too many rows");
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    if (rows_fast)
+      hipLaunchKernelGGL((wn_cols_kernel<T, MODE>), dim3((unsigned)((rows + 63) / 64)), dim3(256), 0, as_stream(stream),
+                         (const T*)v, (const T*)g, (const T*)dw, (T*)out, (T*)dg, (long long)rows, (long long)cols);
+    else
+      hipLaunchKernelGGL((wn_rows_kernel<T, MODE>), dim3((unsigned)rows), dim3(256), 0, as_stream(stream), (const T*)v,
+                         (const T*)g, (const T*)dw, (T*)out, (T*)dg, (long long)cols);
+  });
+  return check_launch(what);
+}
+
+extern "C" int flhip_rownorm(const void* v, void* n, int64_t rows, int64_t cols, int rows_fast, int dtype, void* stream) {
+  return weightnorm_launch<0>("rownorm", v, nullptr, nullptr, n, nullptr, rows, cols, rows_fast, dtype, stream);
+}
+extern "C" int flhip_weightnorm_fwd(const void* v, const void* g, void* w, int64_t rows, int64_t cols, int rows_fast,
+                                    int dtype, void* stream) {
+  return weightnorm_launch<1>("weightnorm_fwd", v, g, nullptr, w, nullptr, rows, cols, rows_fast, dtype, stream);
+}
+extern "C" int flhip_weightnorm_bwd(const void* dw, const void* v, const void* g, void* dv, void* dg, int64_t rows,
+                                    int64_t cols, int rows_fast, int dtype, void* stream) {
+  return weightnorm_launch<2>("weightnorm_bwd", v, g, dw, dv, dg, rows, cols, rows_fast, dtype, stream);
+}
+
+static int pad_launch(bool bwd, const void* src, void* dst, const int64_t* dims, const int32_t* before, const int32_t* after,
+                      double value, int dtype, void* stream) {
+  FLHIP_REQUIRE(src && dst && dims && before && after, "padding: null argument");
+  FLHIP_REQUIRE(dtype_ok(dtype), "padding: unknown dtype");
+  PadGeom g;
+  size_t nin = 1, nout = 1;
+  for (int k = 0; k < 4; ++k) {
+    FLHIP_REQUIRE(dims[k] > 0, "padding: sizes must be positive");
+    FLHIP_REQUIRE(before[k] >= 0 && after[k] >= 0, "padding: widths must not be negative");
+    g.id[k] = dims[k];
+    g.lo[k] = before[k];
+    g.od[k] = dims[k] + before[k] + after[k];
+    nin *= (size_t)g.id[k];
+    nout *= (size_t)g.od[k];
+  }
+  const size_t n = bwd ? nin : nout;
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    if (bwd)
+      hipLaunchKernelGGL((pad_kernel<T, true>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream), (const T*)src, (T*)dst, n,
+                         g, 0.f);
+    else
+      hipLaunchKernelGGL((pad_kernel<T, false>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream), (const T*)src, (T*)dst,
+                         n, g, (float)value);
+  });
+  return check_launch(bwd ? "padding_bwd" : "padding_fwd");
+}
+extern "C" int flhip_pad_fwd(const void* x, void* y, const int64_t* dims, const int32_t* before, const int32_t* after,
+                             double value, int dtype, void* stream) {
+  return pad_launch(false, x, y, dims, before, after, value, dtype, stream);
+}
+extern "C" int flhip_pad_bwd(const void* dy, void* dx, const int64_t* dims, const int32_t* before, const int32_t* after,
+                             int dtype, void* stream) {
+  return pad_launch(true, dy, dx, dims, before, after, 0.0, dtype, stream);
 }
 
 extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, int32_t N, int32_t K,

@@ -543,6 +543,95 @@ Variable dropout(const Variable& input, double p) {
   return Variable(out, {input}, gradFunc);
 }
 
+namespace {
+// rows x cols view of a weight for WeightNorm: the kept dimension first (fastest) or last
+void weightNormView(const Shape& s, int dim, long long* rows, long long* cols, int* rowsFast) {
+  const int nd = s.ndim();
+  if (!(nd >= 1 && (dim == 0 || dim == nd - 1)))
+    throw std::invalid_argument("Wrong dimension for Weight Norm: " + std::to_string(dim));   // WeightNorm.cpp:62-64
+  *rows = s.dim(dim);
+  *cols = s.elements() / std::max<long long>(1, s.dim(dim));
+  // a one-dimensional or single-row weight: either view is the same memory
+  *rowsFast = (dim == 0 && nd > 1) ? 1 : 0;
+  if (*rows <= 0 || *cols <= 0) throw std::invalid_argument("WeightNorm: empty weight");
+}
+}  // namespace
+
+Tensor rowNorm(const Tensor& v, int dim) {
+  long long rows, cols;
+  int fast;
+  weightNormView(v.shape(), dim, &rows, &cols, &fast);
+  std::vector<Dim> gd((size_t)v.ndim(), 1);
+  gd[(size_t)dim] = rows;
+  Tensor n{Shape(gd), v.type()};
+  check(flhip_rownorm(v.device(), n.device(), rows, cols, fast, tagOf(v.type(), "weightNorm"), hipBackendStream()));
+  return n;
+}
+
+Variable weightNorm(const Variable& v, const Variable& g, int dim) {
+  dtypesMatch("weightNorm", {&v, &g});
+  long long rows, cols;
+  int fast;
+  weightNormView(v.shape(), dim, &rows, &cols, &fast);
+  if (g.tensor().elements() != rows) throw std::invalid_argument("weightNorm: g must have one element per index of dim");
+  const int tag = tagOf(v.type(), "weightNorm");
+  detail::OpScope scope("weightNorm");
+  Tensor w(v.shape(), v.type());
+  check(flhip_weightnorm_fwd(v.tensor().device(), g.tensor().device(), w.device(), rows, cols, fast, tag, hipBackendStream()));
+  if (scope.on()) scope.done({v.tensor(), g.tensor()}, {w});
+  auto gradFunc = [rows, cols, fast, tag](std::vector<Variable>& inputs, const Variable& gradOutput) {
+    auto& vv = inputs[0];
+    auto& gg = inputs[1];
+    if (!vv.isCalcGrad() && !gg.isCalcGrad()) return;
+    detail::OpScope scope("weightNormBackward");
+    Tensor dv(vv.shape(), vv.type()), dg(gg.shape(), gg.type());
+    const Tensor go = gradOutput.tensor().type() == vv.type() ? gradOutput.tensor() : gradOutput.tensor().astype(vv.type());
+    check(flhip_weightnorm_bwd(go.device(), vv.tensor().device(), gg.tensor().device(), dv.device(), dg.device(), rows,
+                               cols, fast, tag, hipBackendStream()));
+    if (scope.on()) scope.done({go, vv.tensor(), gg.tensor()}, {dv, dg});
+    if (vv.isCalcGrad()) vv.addGrad(Variable(dv, false));
+    if (gg.isCalcGrad()) gg.addGrad(Variable(dg, false));
+  };
+  return Variable(w, {v, g}, gradFunc);
+}
+
+Variable padding(const Variable& input, const std::vector<std::pair<int, int>>& pad, double val) {
+  const int nd = input.ndim();
+  if ((int)pad.size() > nd)
+    throw std::invalid_argument("padding: number of padding dimensions exceeds number of input dimensions");
+  if (nd > 4) throw std::invalid_argument("padding: at most four dimensions");
+  int64_t dims[4] = {1, 1, 1, 1};
+  int32_t before[4] = {0, 0, 0, 0}, after[4] = {0, 0, 0, 0};
+  std::vector<Dim> od = input.shape().get();
+  for (int i = 0; i < nd; ++i) dims[i] = input.shape().dim(i);
+  for (size_t i = 0; i < pad.size(); ++i) {
+    if (pad[i].first < 0 || pad[i].second < 0) throw std::invalid_argument("padding: widths must not be negative");
+    before[i] = pad[i].first;
+    after[i] = pad[i].second;
+    od[i] += pad[i].first + pad[i].second;
+  }
+  const int tag = tagOf(input.type(), "padding");
+  detail::OpScope scope("padding");
+  Tensor out{Shape(od), input.type()};
+  if (input.tensor().elements() > 0)
+    check(flhip_pad_fwd(input.tensor().device(), out.device(), dims, before, after, val, tag, hipBackendStream()));
+  if (scope.on()) scope.done({input.tensor()}, {out});
+  std::vector<int64_t> dv(dims, dims + 4);
+  std::vector<int32_t> bv(before, before + 4), av(after, after + 4);
+  auto gradFunc = [dv, bv, av, tag](std::vector<Variable>& inputs, const Variable& gradOutput) {
+    auto& in = inputs[0];
+    if (!in.isCalcGrad()) return;
+    detail::OpScope scope("paddingBackward");
+    Tensor g(in.shape(), gradOutput.type());
+    if (g.elements() > 0)
+      check(flhip_pad_bwd(gradOutput.tensor().device(), g.device(), dv.data(), bv.data(), av.data(),
+                          tagOf(g.type(), "padding"), hipBackendStream()));
+    if (scope.on()) scope.done({gradOutput.tensor()}, {g});
+    in.addGrad(Variable(g, false));
+  };
+  return Variable(out, {input}, gradFunc);
+}
+
 Variable moddims(const Variable& input, const Shape& dims) {
   // a 0 keeps the input's dimension, one -1 is inferred from the element count
   // (Functions.cpp:969-1008)

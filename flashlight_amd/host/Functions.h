@@ -11,6 +11,7 @@
 #include <functional>
 #include <memory>
 #include <tuple>
+#include <utility>
 #include <vector>
 
 #include "DynamicBenchmark.h"
@@ -156,6 +157,13 @@ Variable gatedlinearunit(const Variable& input, int dim);
 // counter-based function of a seed drawn from the process-wide generator (fl::setSeed), regenerated by the
 // backward pass.
 Variable dropout(const Variable& input, double p);
+// The weight of fl::WeightNorm (nn/modules/WeightNorm.cpp:45-66): v * tileAs(g / norm(v over all dimensions but
+// `dim`), v); dim is 0 or the last dimension of v (the reference: 0 or 3 of four).  g has one element per index of
+// `dim`.  rowNorm gives those norms with the kept-dimensions shape (the initial g, :68-72).
+Variable weightNorm(const Variable& v, const Variable& g, int dim);
+Tensor rowNorm(const Tensor& v, int dim);
+// fl::padding (Functions.cpp:1751-1775): pad[i] = (before, after) for dimension i, filled with val
+Variable padding(const Variable& input, const std::vector<std::pair<int, int>>& pad, double val);
 Variable moddims(const Variable& input, const Shape& dims);
 // fl::reorder (Functions.cpp:1010-1042): dimension k of the result is dimension dims[k] of the
 // input; the gradient is reordered back with the inverse permutation

@@ -220,6 +220,59 @@ std::string Conv2D::prettyString() const {
   return ss.str();
 }
 
+// ---- Padding, WeightNorm ------------------------------------------------------------------
+std::string Padding::prettyString() const {
+  std::ostringstream ss;
+  ss << "Padding (" << val_ << ", { ";
+  for (const auto& p : pad_) ss << "(" << p.first << ", " << p.second << "), ";
+  ss << "})";
+  return ss.str();
+}
+
+WeightNorm::WeightNorm(ModulePtr module, int dim) : module_(std::move(module)), dim_(dim) {
+  if (!module_) throw std::invalid_argument("WeightNorm: null module");
+  const auto mp = module_->params();
+  if (mp.size() != 1 && mp.size() != 2) throw std::invalid_argument("WeightNorm only supports Linear and Conv2D");
+  const Variable& v = mp[0];
+  if (dim_ < 0 || dim_ > v.ndim()) throw std::invalid_argument("invalid dimension for WeightNorm");   // WeightNorm.cpp:36-38
+  Variable g(rowNorm(v.tensor(), dim_), true);                                                          // :68-72
+  params_ = mp.size() == 2 ? std::vector<Variable>{v, g, mp[1]} : std::vector<Variable>{v, g};
+  computeWeight();
+}
+
+void WeightNorm::computeWeight() { module_->setParams(weightNorm(params_[0], params_[1], dim_), 0); }   // :45-66
+
+void WeightNorm::setParams(const Variable& var, int position) {
+  Module::setParams(var, position);
+  // :84-93: the wrapped module keeps copies, not pointers
+  if (position == 2)
+    module_->setParams(var, 1);
+  else if (position <= 1)
+    computeWeight();
+}
+
+std::vector<Variable> WeightNorm::forward(const std::vector<Variable>& inputs) {
+  if (train_) computeWeight();                                                                         // :95-100
+  return module_->forward(inputs);
+}
+
+void WeightNorm::train() {
+  Module::train();
+  module_->train();
+}
+
+void WeightNorm::eval() {
+  Module::eval();
+  module_->eval();
+  computeWeight();
+}
+
+std::string WeightNorm::prettyString() const {
+  std::ostringstream ss;
+  ss << "WeightNorm (" << module_->prettyString() << ", " << dim_ << ")";
+  return ss.str();
+}
+
 // ---- Pool2D ----------------------------------------------------------------------------
 Pool2D::Pool2D(int wx, int wy, int sx, int sy, IntOrPadMode px, IntOrPadMode py, PoolingMode mode)
     : xFilter_(wx), yFilter_(wy), xStride_(sx), yStride_(sy), xPad_(px.padVal), yPad_(py.padVal),

@@ -345,6 +345,40 @@ class Reorder : public UnaryModule {
   Shape dims_;
 };
 
+// nn/modules/Padding.cpp:14-20
+class Padding : public UnaryModule {
+ public:
+  Padding(std::vector<std::pair<int, int>> padding, double val) : pad_(std::move(padding)), val_(val) {}
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return padding(input, pad_, val_); }
+  std::string prettyString() const override;
+
+ private:
+  std::vector<std::pair<int, int>> pad_;
+  double val_;
+};
+
+// nn/modules/WeightNorm.{h,cpp}: the wrapped module's weight (parameter 0) is v * g / ||v||, the norm over all
+// dimensions but `dim`; parameters {v, g} or {v, g, bias}.  Wraps a Linear or a Conv2D (one or two parameters).
+class WeightNorm : public Module {
+ public:
+  WeightNorm(ModulePtr module, int dim);
+  template <typename T, typename = std::enable_if_t<std::is_base_of_v<Module, std::decay_t<T>>>>
+  WeightNorm(T&& module, int dim) : WeightNorm(ModulePtr(std::make_shared<std::decay_t<T>>(std::forward<T>(module))), dim) {}
+  using Module::forward;
+  std::vector<Variable> forward(const std::vector<Variable>& inputs) override;
+  void setParams(const Variable& var, int position) override;
+  void train() override;
+  void eval() override;
+  ModulePtr module() const { return module_; }
+  std::string prettyString() const override;
+
+ private:
+  void computeWeight();
+  ModulePtr module_;
+  int dim_;
+};
+
 class LogSoftmax : public UnaryModule {    // Activations.cpp:180-192
  public:
   explicit LogSoftmax(int dim = 0) : dim_(dim) {}

@@ -130,6 +130,19 @@ ModulePtr parseLine(const std::string& line) {
     if (n != 2) failParse(line);
     return std::make_shared<Dropout>(F(1));
   }
+  if (op == "PD") {                               // SequentialBuilder.cpp:131-144: a value, then (before, after) pairs
+    if (!inRange(4, 10) || (n & 1)) failParse(line);
+    const double val = F(1);
+    std::vector<std::pair<int, int>> pads(4, {0, 0});
+    for (size_t i = 2; i + 1 < n; i += 2) pads[(i - 2) / 2] = {I(i), I(i + 1)};
+    return std::make_shared<Padding>(pads, val);
+  }
+  if (op == "WN") {                               // :352-359: a dimension, then the line of the wrapped module
+    if (n < 3) failParse(line);
+    std::string child;
+    for (size_t i = 2; i < n; ++i) child += (i > 2 ? " " : "") + p[i];
+    return std::make_shared<WeightNorm>(parseLine(child), I(1));
+  }
   if (op == "RNN" || op == "GRU" || op == "LSTM") {
     if (n < 3) failParse(line);
     const RnnMode mode = op == "RNN" ? RnnMode::RELU : op == "GRU" ? RnnMode::GRU : RnnMode::LSTM;
@@ -138,8 +151,8 @@ ModulePtr parseLine(const std::string& line) {
     const float dropout = n > 5 ? std::stof(p[5]) : 0.0f;
     return std::make_shared<RNN>(I(1), I(2), layers, mode, bidirectional, dropout);
   }
-  static const char* const absent[] = {"PD", "TR", "CFR", "POSEMB", "SINPOSEMB", "TDS", "AC", "E", "ADAPTIVEE",
-                                       "WN", "PR", "RES", "SKIP", "SKIPL", "SAUG", "PC"};
+  static const char* const absent[] = {"TR", "CFR", "POSEMB", "SINPOSEMB", "TDS", "AC", "E", "ADAPTIVEE",
+                                       "PR", "RES", "SKIP", "SKIPL", "SAUG", "PC"};
   for (const char* a : absent)
     if (op == a)
       throw std::invalid_argument("buildSequentialModule: module '" + op +

@@ -491,6 +491,59 @@ def dropout(input, p, seed):
     return y
 
 
+def rownorm(v, rows, cols, rows_fast):
+    """flhip_rownorm: ||v_r|| of a rows x cols view (rows_fast: element (r, j) at r + j * rows)."""
+    x = _dev(v, "v")
+    n = torch.empty(rows, dtype=x.dtype, device=x.device)
+    capi.check(capi.lib().flhip_rownorm(_ptr(x), _ptr(n), rows, cols, int(rows_fast), _dtype_tag(x), _stream()))
+    return n
+
+
+def weightnorm(v, g, rows, cols, rows_fast):
+    """fl::WeightNorm's weight (WeightNorm.cpp:45-66): v * g[r] / ||v_r||."""
+    x, gg = _dev(v, "v"), _dev(g, "g")
+    w = torch.empty_like(x)
+    capi.check(capi.lib().flhip_weightnorm_fwd(_ptr(x), _ptr(gg), _ptr(w), rows, cols, int(rows_fast), _dtype_tag(x),
+                                               _stream()))
+    return w
+
+
+def weightnorm_backward(dw, v, g, rows, cols, rows_fast):
+    d, x, gg = _dev(dw, "dw"), _dev(v, "v"), _dev(g, "g")
+    dv, dg = torch.empty_like(x), torch.empty_like(gg)
+    capi.check(capi.lib().flhip_weightnorm_bwd(_ptr(d), _ptr(x), _ptr(gg), _ptr(dv), _ptr(dg), rows, cols,
+                                               int(rows_fast), _dtype_tag(x), _stream()))
+    return dv, dg
+
+
+def _pad_args(dims, before, after):
+    return ((C.c_int64 * 4)(*dims), (C.c_int32 * 4)(*before), (C.c_int32 * 4)(*after))
+
+
+def padding(input, dims, before, after, value=0.0):
+    """fl::padding (Functions.cpp:1751-1775); dims / before / after: four column-major entries (dims[0] fastest) of a
+    contiguous tensor with prod(dims) elements.  Returns a flat tensor in the padded shape's memory order."""
+    x = _dev(input, "input")
+    d, b, a = _pad_args(dims, before, after)
+    n = 1
+    for k in range(4):
+        n *= dims[k] + before[k] + after[k]
+    y = torch.empty(n, dtype=x.dtype, device=x.device)
+    capi.check(capi.lib().flhip_pad_fwd(_ptr(x), _ptr(y), d, b, a, float(value), _dtype_tag(x), _stream()))
+    return y
+
+
+def padding_backward(grad_output, dims, before, after):
+    g = _dev(grad_output, "gradOutput")
+    d, b, a = _pad_args(dims, before, after)
+    n = 1
+    for k in range(4):
+        n *= dims[k]
+    dx = torch.empty(n, dtype=g.dtype, device=g.device)
+    capi.check(capi.lib().flhip_pad_bwd(_ptr(g), _ptr(dx), d, b, a, _dtype_tag(g), _stream()))
+    return dx
+
+
 def linear(input, weight, bias=None):
     """fl::linear (Functions.cpp:1255-1309): input [..., in] (Flashlight [in, ...]), weight
     torch [in, out] (Flashlight [out, in]), bias [out] or None -> [..., out]."""

@@ -116,7 +116,7 @@ const char* flhip_last_error(void);
  * refuse to run when flhip_version() / 100 differs from FLHIP_VERSION / 100 (a layout change).
  * 200: flhip_rnn_desc gained dropout, seed_lo, seed_hi; flhip_bn_workspace_bytes never returns less
  * than 32 bytes per feature.  202: the *_plan entry points and FLHIP_DECLINED.  203: FLHIP_F16.  204: flhip_act_fwd / _bwd, flhip_glu_fwd / _bwd,
- * flhip_dropout. */
+ * flhip_dropout, flhip_rownorm, flhip_weightnorm_fwd / _bwd, flhip_pad_fwd / _bwd. */
 #define FLHIP_VERSION 204
 int flhip_version(void);
 const char* flhip_arch(void);
@@ -389,6 +389,26 @@ int flhip_glu_bwd(const void* dy, const void* x, void* dx, int64_t outer, int64_
  * are the same.  The backward pass is the same call on the gradient with the same seed and p.  y may alias x. */
 int flhip_dropout(const void* x, void* y, size_t n, double p, uint32_t seed_lo, uint32_t seed_hi, int dtype,
                   void* stream);
+
+/* fl::WeightNorm (flashlight/fl/nn/modules/WeightNorm.cpp:45-72): w = v * g[r] / ||v_r||, one g per index r of the
+ * kept dimension, the norm over all the others.  The tensor is a rows x cols matrix: rows_fast != 0 when the kept
+ * dimension is the tensor's first (element (r, j) at r + j * rows: Linear weights, dim 0), 0 when it is the last
+ * (element (r, j) at r * cols + j: Conv2D weights, dim 3) - the two the reference accepts.  g, n and dg have `rows`
+ * elements of the tensor's dtype.  flhip_rownorm gives ||v_r|| (the initial g, :68-72).  Backward (the chain of the
+ * reference's norm / division / tileAs / product): dv = (g / n) (dw - c v / n^2), dg[r] = c / n, c = sum_j dw v. */
+int flhip_rownorm(const void* v, void* n, int64_t rows, int64_t cols, int rows_fast, int dtype, void* stream);
+int flhip_weightnorm_fwd(const void* v, const void* g, void* w, int64_t rows, int64_t cols, int rows_fast,
+                         int dtype, void* stream);
+int flhip_weightnorm_bwd(const void* dw, const void* v, const void* g, void* dv, void* dg, int64_t rows,
+                         int64_t cols, int rows_fast, int dtype, void* stream);
+
+/* fl::padding (Functions.cpp:1751-1775) of a tensor with the four column-major extents dims[0..3] (pad with 1):
+ * before[k] / after[k] elements of `value` in front of / behind dimension k.  flhip_pad_bwd copies the inner box of
+ * the padded gradient back (dims, before, after as in the forward call).  Buffers must not overlap. */
+int flhip_pad_fwd(const void* x, void* y, const int64_t* dims, const int32_t* before, const int32_t* after,
+                  double value, int dtype, void* stream);
+int flhip_pad_bwd(const void* dy, void* dx, const int64_t* dims, const int32_t* before, const int32_t* after,
+                  int dtype, void* stream);
 
 /* C (M x N) = op(A) (M x K) * op(B) (K x N), fp32 accumulate; trans_a: A is stored
  * K x M, trans_b: B is stored N x K.  bias_rows (fp32[M], may be NULL) is added to

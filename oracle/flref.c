@@ -460,6 +460,74 @@ void flref_dropout(int64_t n, const float* x, double p, uint32_t seed_lo, uint32
     y[i] = flref_dropout_keep(seed_lo, seed_hi, (uint32_t)((uint64_t)i >> 32), (uint32_t)i, (float)p) ? x[i] * scale : 0.f;
 }
 
+/* WeightNorm (nn/modules/WeightNorm.cpp:45-72): w = v g[r] / ||v_r|| over a rows x cols view, element (r, j) at
+ * r + j*rows (rows_fast) or r*cols + j; in double */
+static size_t wn_at(int64_t r, int64_t j, int64_t rows, int64_t cols, int rows_fast) {
+  return rows_fast ? (size_t)r + (size_t)j * (size_t)rows : (size_t)r * (size_t)cols + (size_t)j;
+}
+void flref_rownorm(int64_t rows, int64_t cols, int rows_fast, const float* v, float* n) {
+  for (int64_t r = 0; r < rows; ++r) {
+    double s2 = 0.0;
+    for (int64_t j = 0; j < cols; ++j) { const double x = v[wn_at(r, j, rows, cols, rows_fast)]; s2 += x * x; }
+    n[r] = (float)sqrt(s2);
+  }
+}
+void flref_weightnorm_fwd(int64_t rows, int64_t cols, int rows_fast, const float* v, const float* g, float* w) {
+  for (int64_t r = 0; r < rows; ++r) {
+    double s2 = 0.0;
+    for (int64_t j = 0; j < cols; ++j) { const double x = v[wn_at(r, j, rows, cols, rows_fast)]; s2 += x * x; }
+    const double scale = (double)g[r] / sqrt(s2);
+    for (int64_t j = 0; j < cols; ++j) {
+      const size_t e = wn_at(r, j, rows, cols, rows_fast);
+      w[e] = (float)(v[e] * scale);
+    }
+  }
+}
+/* w = v s, s = g / n: dv = s dw + (dL/ds)(ds/dn)(dn/dv) = s (dw - c v / n^2), dg = c / n, c = sum dw v */
+void flref_weightnorm_bwd(int64_t rows, int64_t cols, int rows_fast, const float* dw, const float* v, const float* g,
+                          float* dv, float* dg) {
+  for (int64_t r = 0; r < rows; ++r) {
+    double s2 = 0.0, c = 0.0;
+    for (int64_t j = 0; j < cols; ++j) {
+      const size_t e = wn_at(r, j, rows, cols, rows_fast);
+      s2 += (double)v[e] * v[e];
+      c += (double)dw[e] * v[e];
+    }
+    const double n = sqrt(s2), scale = (double)g[r] / n;
+    for (int64_t j = 0; j < cols; ++j) {
+      const size_t e = wn_at(r, j, rows, cols, rows_fast);
+      dv[e] = (float)(scale * ((double)dw[e] - c * v[e] / s2));
+    }
+    dg[r] = (float)(c / n);
+  }
+}
+
+/* fl::padding (Functions.cpp:1751-1775), four column-major extents */
+void flref_pad_fwd(const int64_t* dims, const int32_t* before, const int32_t* after, double value, const float* x, float* y) {
+  int64_t od[4];
+  for (int k = 0; k < 4; ++k) od[k] = dims[k] + before[k] + after[k];
+  for (int64_t d = 0; d < od[3]; ++d)
+    for (int64_t c = 0; c < od[2]; ++c)
+      for (int64_t b = 0; b < od[1]; ++b)
+        for (int64_t a = 0; a < od[0]; ++a) {
+          const int64_t q[4] = {a - before[0], b - before[1], c - before[2], d - before[3]};
+          int in = 1;
+          for (int k = 0; k < 4; ++k) in = in && q[k] >= 0 && q[k] < dims[k];
+          y[a + od[0] * (b + od[1] * (c + od[2] * d))] =
+              in ? x[q[0] + dims[0] * (q[1] + dims[1] * (q[2] + dims[2] * q[3]))] : (float)value;
+        }
+}
+void flref_pad_bwd(const int64_t* dims, const int32_t* before, const int32_t* after, const float* dy, float* dx) {
+  int64_t od[4];
+  for (int k = 0; k < 4; ++k) od[k] = dims[k] + before[k] + after[k];
+  for (int64_t d = 0; d < dims[3]; ++d)
+    for (int64_t c = 0; c < dims[2]; ++c)
+      for (int64_t b = 0; b < dims[1]; ++b)
+        for (int64_t a = 0; a < dims[0]; ++a)
+          dx[a + dims[0] * (b + dims[1] * (c + dims[2] * d))] =
+              dy[(a + before[0]) + od[0] * ((b + before[1]) + od[1] * ((c + before[2]) + od[2] * (d + before[3])))];
+}
+
 /* fl::matmul / matmulTN / matmulNT as used by fl::linear (:1264-1265, 1292-1301) */
 void flref_matmul(int M, int N, int K, int ta, int tb, const float* A, const float* B,
                   const float* bias, float* C) {

@@ -109,6 +109,15 @@ void flref_glu_fwd(int64_t outer, int64_t m, const float* x, float* y);
 void flref_glu_bwd(int64_t outer, int64_t m, const float* dy, const float* x, float* dx);
 /* dropout (:1777-1785) with the counter-based mask of flref_dropout_keep */
 void flref_dropout(int64_t n, const float* x, double p, uint32_t seed_lo, uint32_t seed_hi, float* y);
+/* WeightNorm (nn/modules/WeightNorm.cpp:45-72) over a rows x cols view (rows_fast: element (r, j) at r + j*rows,
+ * else r*cols + j): row norms, w = v g / ||v||, and the gradients of v and g */
+void flref_rownorm(int64_t rows, int64_t cols, int rows_fast, const float* v, float* n);
+void flref_weightnorm_fwd(int64_t rows, int64_t cols, int rows_fast, const float* v, const float* g, float* w);
+void flref_weightnorm_bwd(int64_t rows, int64_t cols, int rows_fast, const float* dw, const float* v, const float* g,
+                          float* dv, float* dg);
+/* fl::padding (:1751-1775) over four column-major extents and the slice back */
+void flref_pad_fwd(const int64_t* dims, const int32_t* before, const int32_t* after, double value, const float* x, float* y);
+void flref_pad_bwd(const int64_t* dims, const int32_t* before, const int32_t* after, const float* dy, float* dx);
 /* C (M x N) = op(A) op(B) + bias[m]; ta: A stored K x M, tb: B stored N x K; double
  * accumulate.  fl::linear (:1255-1309) = (W, X), backward (W^T, dY) and (dY, X^T). */
 void flref_matmul(int M, int N, int K, int ta, int tb, const float* A, const float* B,

@@ -230,6 +230,48 @@ def dropout(x, p, seed_lo, seed_hi):
     return y
 
 
+def rownorm(v, rows, cols, rows_fast):
+    v = _f32(v)
+    n = np.empty(rows, np.float32)
+    lib().flref_rownorm(_i64(rows), _i64(cols), C.c_int(int(rows_fast)), _p(v), _p(n))
+    return n
+
+
+def weightnorm_fwd(v, g, rows, cols, rows_fast):
+    v, g = _f32(v), _f32(g)
+    w = np.empty_like(v)
+    lib().flref_weightnorm_fwd(_i64(rows), _i64(cols), C.c_int(int(rows_fast)), _p(v), _p(g), _p(w))
+    return w
+
+
+def weightnorm_bwd(dw, v, g, rows, cols, rows_fast):
+    dw, v, g = _f32(dw), _f32(v), _f32(g)
+    dv, dg = np.empty_like(v), np.empty(rows, np.float32)
+    lib().flref_weightnorm_bwd(_i64(rows), _i64(cols), C.c_int(int(rows_fast)), _p(dw), _p(v), _p(g), _p(dv), _p(dg))
+    return dv, dg
+
+
+def _pad_args(dims, before, after):
+    return ((C.c_int64 * 4)(*dims), (C.c_int32 * 4)(*before), (C.c_int32 * 4)(*after))
+
+
+def pad_fwd(x, dims, before, after, value):
+    """dims / before / after: four column-major entries (dims[0] fastest); x in memory order."""
+    x = _f32(x)
+    d, b, a = _pad_args(dims, before, after)
+    y = np.empty(int(np.prod([dims[k] + before[k] + after[k] for k in range(4)])), np.float32)
+    lib().flref_pad_fwd(d, b, a, C.c_double(value), _p(x), _p(y))
+    return y
+
+
+def pad_bwd(dy, dims, before, after):
+    dy = _f32(dy)
+    d, b, a = _pad_args(dims, before, after)
+    dx = np.empty(int(np.prod(dims)), np.float32)
+    lib().flref_pad_bwd(d, b, a, _p(dy), _p(dx))
+    return dx
+
+
 def relu_bwd(dy, x):
     dy, x = _f32(dy), _f32(x)
     dx = np.empty_like(x)

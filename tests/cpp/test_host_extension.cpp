@@ -957,7 +957,7 @@ static void testArchBuilder() {
   CHECK(one("BN 8 0 1")->prettyString() == BatchNorm(std::vector<int>{0, 1}, 8).prettyString());
   // malformed lines, lines for modules that do not exist here, a missing file
   for (const char* bad : {"C 3 4 5", "C2 3 4 5 6 1", "L 5", "BN 8", "LN", "LN 3", "M 2 2 2", "R 1", "LSM", "GRU 4",
-                          "C 3 x 5 1", "XYZ 1 2", "RO", "DO", "DO 0.2 1", "GLU", "ELU 1", "SH 1 2", "WN 3 C 1 2 3 4", "PD 0 1 1",
+                          "C 3 x 5 1", "XYZ 1 2", "RO", "DO", "DO 0.2 1", "GLU", "ELU 1", "SH 1 2", "WN 3", "WN 1 C 4 4 3 1", "WN 3 R", "PD 0 1", "PD 0 1 1 1",
                           "TDS 10 21 80", "RES 2 1 3", "PC f16"})
     CHECK(throws<std::invalid_argument>([&] { one(bad); }));
   CHECK(throws<std::runtime_error>([] { buildSequentialModule(std::string("/nonexistent/arch.txt"), 1, 1); }));
@@ -1072,13 +1072,76 @@ static void testActivationModules() {
     y2.backward(Variable(Tensor::fromVector(y2.shape(), dy), false));
     CHECK(hostOf(a.grad()) == hostOf(b.grad()));
   }
+  // WN: the wrapped module's weight is v g / ||v||; outputs and gradients against the plain module with that weight
+  // and the checker's chain rule (WeightNorm.cpp:45-72)
+  for (int which = 0; which < 2; ++which) {
+    setSeed(23 + which);
+    auto wn = std::dynamic_pointer_cast<WeightNorm>(one(which == 0 ? "WN 3 C 6 10 5 1 -1" : "WN 0 L 12 7"));
+    CHECK(wn != nullptr);
+    if (!wn) continue;
+    CHECK(wn->params().size() == 3);
+    const Variable v = wn->param(0), g0 = wn->param(1);
+    const int dim = which == 0 ? 3 : 0;
+    const long long rows = v.shape().dim(dim), cols = v.tensor().elements() / rows;
+    const int fast = which == 0 ? 0 : 1;
+    auto vh = hostOf(v);
+    // the initial g is the norm: the initial weight is v itself
+    std::vector<float> nr((size_t)rows);
+    flref_rownorm(rows, cols, fast, vh.data(), nr.data());
+    CHECK(g0.shape().dim(dim) == rows && (long long)g0.tensor().elements() == rows && relL2(hostOf(g0), nr) <= 1e-6);
+    CHECK(relL2(hostOf(wn->module()->param(0)), vh) <= 1e-6);
+    // a g of its own
+    auto gh = randn((size_t)rows, 750 + which, 0.3f, 1.f);
+    wn->setParams(Variable(Tensor::fromVector(g0.shape(), gh), true), 1);
+    std::vector<float> wr(vh.size());
+    flref_weightnorm_fwd(rows, cols, fast, vh.data(), gh.data(), wr.data());
+    CHECK(relL2(hostOf(wn->module()->param(0)), wr) <= 1e-6);
+    const Shape ishape = which == 0 ? Shape({20, 1, 6, 2}) : Shape({12, 5});
+    auto x = randn((size_t)ishape.elements(), 752);
+    Variable in1(Tensor::fromVector(ishape, x), true), in2(Tensor::fromVector(ishape, x), true);
+    Variable y1 = wn->forward({in1})[0];
+    // the same layer with the checker's weight
+    Variable wplain(Tensor::fromVector(v.shape(), wr), true);
+    Variable y2 = which == 0 ? conv2d(in2, wplain, wn->param(2), 1, 1, 2, 0, 1, 1, 1) : linear(in2, wplain, wn->param(2));
+    CHECK(y1.shape() == y2.shape() && relL2(hostOf(y1), hostOf(y2)) <= 1e-6);
+    auto dy = randn((size_t)y1.tensor().elements(), 753);
+    for (const auto& p : wn->params()) Variable(p).zeroGrad();
+    y1.backward(Variable(Tensor::fromVector(y1.shape(), dy), false));
+    y2.backward(Variable(Tensor::fromVector(y2.shape(), dy), false));
+    CHECK(relL2(hostOf(in1.grad()), hostOf(in2.grad())) <= 1e-6);
+    auto dwh = hostOf(wplain.grad());
+    std::vector<float> dvr(vh.size()), dgr((size_t)rows);
+    flref_weightnorm_bwd(rows, cols, fast, dwh.data(), vh.data(), gh.data(), dvr.data(), dgr.data());
+    CHECK(relL2(hostOf(wn->param(0).grad()), dvr) <= 1e-5);
+    CHECK(relL2(hostOf(wn->param(1).grad()), dgr) <= 1e-5);
+    CHECK(wn->prettyString().rfind("WeightNorm (", 0) == 0);
+  }
+  CHECK(throws<std::invalid_argument>([&] { WeightNorm(Conv2D(4, 4, 3, 1), 1).forward({Variable()}); }));
+  // PD: the input inside a tensor of the value, the gradient is the inner box
+  {
+    auto x = randn(5 * 3 * 2 * 2, 760);
+    Variable in(Tensor::fromVector({5, 3, 2, 2}, x), true);
+    Variable y = one("PD -1 2 1 0 0 1 3")->forward({in})[0];
+    CHECK(y.shape() == Shape({8, 3, 6, 2}));
+    const int64_t dims[4] = {5, 3, 2, 2};
+    const int32_t before[4] = {2, 0, 1, 0}, after[4] = {1, 0, 3, 0};
+    std::vector<float> yr(8 * 3 * 6 * 2), dxr(x.size());
+    flref_pad_fwd(dims, before, after, -1.0, x.data(), yr.data());
+    CHECK(hostOf(y) == yr);
+    auto dy = randn(yr.size(), 761);
+    y.backward(Variable(Tensor::fromVector(y.shape(), dy), false));
+    flref_pad_bwd(dims, before, after, dy.data(), dxr.data());
+    CHECK(hostOf(in.grad()) == dxr);
+    CHECK(throws<std::invalid_argument>([&] { padding(Variable(Tensor::fromVector({4, 2}, randn(8, 1)), false), {{1, 1}, {0, 0}, {1, 0}}, 0.0); }));
+  }
   // a GLU convolution block from text, as in wav2letter's architecture files
   {
     setSeed(17);
-    auto net = buildSequentialModule(std::vector<std::string>{"V -1 1 NFEAT 0", "C NFEAT 32 5 1 -1", "GLU 2", "DO 0.2",
-                                                              "C 16 24 3 1 -1", "HT", "RO 2 0 3 1", "V 24 -1", "L 24 NLABEL", "LSM 0"},
+    auto net = buildSequentialModule(std::vector<std::string>{"V -1 1 NFEAT 0", "WN 3 C NFEAT 32 5 1 -1", "GLU 2", "DO 0.2",
+                                                              "PD 0 2 0", "WN 3 C 16 24 3 1", "HT", "RO 2 0 3 1", "V 24 -1",
+                                                              "WN 0 L 24 NLABEL", "LSM 0"},
                                      10, 6);
-    CHECK(net->modules().size() == 10);
+    CHECK(net->modules().size() == 11);
     Variable in(Tensor::fromVector({30, 10, 1, 2}, randn(600, 740)), true);
     Variable y = net->forward(in);
     CHECK(y.shape() == Shape({6, 60}));

@@ -380,3 +380,37 @@ def test_dropout_mask_matches_the_checker(p, dtype):
     assert np.array_equal(y == 0, ref == 0)            # the same mask
     assert rel_l2(y, ref) <= (1e-6 if dtype == torch.float32 else 4e-3)
     assert np.array_equal(y, host(ops.dropout(dev(x, dtype), p, seed)))
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("shape,dim", [((13, 1, 80, 200), 3), ((1816, 30), 0), ((7, 3, 5, 11), 3), ((13, 40), 0), ((70, 2), 0),
+                                       ((1, 1, 300, 3), 3)])
+def test_weightnorm(shape, dim, dtype):
+    # WeightNorm.cpp:45-72 over Conv2D (dim 3) and Linear (dim 0) weights in Flashlight's order
+    rng = np.random.default_rng(100 + dim)
+    rows = shape[dim]
+    cols = int(np.prod(shape)) // rows
+    rows_fast = dim == 0
+    v = _round(rng.standard_normal(int(np.prod(shape))).astype(np.float32), dtype)
+    g = _round((1 + 0.3 * rng.standard_normal(rows)).astype(np.float32), dtype)
+    dw = _round(rng.standard_normal(v.size).astype(np.float32), dtype)
+    tol = 1e-5 if dtype == torch.float32 else 6e-3
+    assert rel_l2(host(ops.rownorm(dev(v, dtype), rows, cols, rows_fast)), flref.rownorm(v, rows, cols, rows_fast)) <= tol
+    assert rel_l2(host(ops.weightnorm(dev(v, dtype), dev(g, dtype), rows, cols, rows_fast)),
+                  flref.weightnorm_fwd(v, g, rows, cols, rows_fast)) <= tol
+    dv, dg = ops.weightnorm_backward(dev(dw, dtype), dev(v, dtype), dev(g, dtype), rows, cols, rows_fast)
+    dv_ref, dg_ref = flref.weightnorm_bwd(dw, v, g, rows, cols, rows_fast)
+    assert rel_l2(host(dv), dv_ref) <= tol
+    assert rel_l2(host(dg), dg_ref) <= (1e-5 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("dims,before,after", [((5, 4, 3, 2), (1, 0, 2, 0), (0, 3, 0, 1)), ((1500, 1, 80, 4), (170, 0, 0, 0), (0, 0, 0, 0)),
+                                               ((7, 1, 1, 1), (2, 0, 0, 0), (5, 0, 0, 0)), ((3, 3, 2, 2), (0, 0, 0, 0), (0, 0, 0, 0))])
+def test_padding(dims, before, after, dtype):
+    rng = np.random.default_rng(110)
+    x = _round(rng.standard_normal(int(np.prod(dims))).astype(np.float32), dtype)
+    y_ref = flref.pad_fwd(x, dims, before, after, 0.25)
+    assert np.array_equal(host(ops.padding(dev(x, dtype), dims, before, after, 0.25)), y_ref)
+    dy = _round(rng.standard_normal(y_ref.size).astype(np.float32), dtype)
+    assert np.array_equal(host(ops.padding_backward(dev(dy, dtype), dims, before, after)), flref.pad_bwd(dy, dims, before, after))

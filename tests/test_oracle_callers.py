@@ -250,3 +250,43 @@ def test_dropout_mask_rate_scale_and_determinism():
         assert np.array_equal(y, flref.dropout(x, p, 123, 456))
         assert not np.array_equal(y, flref.dropout(x, p, 124, 456))
     assert np.array_equal(flref.dropout(x, 0.0, 1, 2), x)
+
+
+@pytest.mark.parametrize("shape,dim", [((7, 3, 5, 11), 3), ((13, 40), 0), ((1, 1, 9, 4), 3), ((64, 3), 0)])
+def test_weightnorm_against_torch_float64(shape, dim):
+    # WeightNorm.cpp:45-72 on a Flashlight (column-major) weight of `shape`: numpy holds it with the shape reversed
+    rng = np.random.default_rng(320 + dim)
+    rows = shape[dim]
+    cols = int(np.prod(shape)) // rows
+    rows_fast = dim == 0
+    v = rng.standard_normal(shape[::-1]).astype(np.float32)          # numpy [d3, d2, d1, d0]
+    g = (1 + 0.3 * rng.standard_normal(rows)).astype(np.float32)
+    dw = rng.standard_normal(v.shape).astype(np.float32)
+    tv = torch.from_numpy(v.astype(np.float64)).requires_grad_(True)
+    tg = torch.from_numpy(g.astype(np.float64)).requires_grad_(True)
+    ax = v.ndim - 1 - dim                                            # the kept numpy axis
+    other = tuple(a for a in range(v.ndim) if a != ax)
+    bshape = [1] * v.ndim
+    bshape[ax] = rows
+    nrm = torch.sqrt((tv * tv).sum(dim=other, keepdim=True))
+    w = tv * (tg.reshape(bshape) / nrm)
+    w.backward(torch.from_numpy(dw.astype(np.float64)))
+    assert rel_l2(flref.rownorm(v, rows, cols, rows_fast), nrm.detach().numpy().ravel()) <= 1e-6
+    assert rel_l2(flref.weightnorm_fwd(v, g, rows, cols, rows_fast), w.detach().numpy()) <= 1e-6
+    dv, dg = flref.weightnorm_bwd(dw, v, g, rows, cols, rows_fast)
+    assert rel_l2(dv, tv.grad.numpy()) <= 1e-6
+    assert rel_l2(dg, tg.grad.numpy()) <= 1e-6
+
+
+@pytest.mark.parametrize("dims,before,after", [((5, 4, 3, 2), (1, 0, 2, 0), (0, 3, 0, 1)), ((7, 1, 1, 1), (2, 0, 0, 0), (5, 0, 0, 0)),
+                                               ((3, 3, 2, 2), (0, 0, 0, 0), (0, 0, 0, 0))])
+def test_padding_against_numpy(dims, before, after):
+    # Functions.cpp:1751-1775: the input inside a tensor of `val`; the gradient is the inner box
+    rng = np.random.default_rng(330)
+    x = rng.standard_normal(dims[::-1]).astype(np.float32)           # numpy [d3, d2, d1, d0]
+    widths = [(before[k], after[k]) for k in (3, 2, 1, 0)]
+    ref = np.pad(x, widths, constant_values=-1.5)
+    assert np.array_equal(flref.pad_fwd(x, dims, before, after, -1.5).reshape(ref.shape), ref)
+    dy = rng.standard_normal(ref.shape).astype(np.float32)
+    sl = tuple(slice(b, b + n) for (b, _), n in zip(widths, x.shape))
+    assert np.array_equal(flref.pad_bwd(dy, dims, before, after).reshape(x.shape), dy[sl])
