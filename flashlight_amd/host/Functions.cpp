@@ -632,6 +632,38 @@ Variable padding(const Variable& input, const std::vector<std::pair<int, int>>& 
   return Variable(out, {input}, gradFunc);
 }
 
+Variable narrow(const Variable& input, int dim, long long start, long long size) {
+  const int nd = input.ndim();
+  if (dim < 0 || dim >= nd || nd > 4) throw std::invalid_argument("narrow: dimension out of range");
+  const long long ext = input.shape().dim(dim);
+  if (start < 0 || size <= 0 || start + size > ext) throw std::invalid_argument("narrow: range outside the dimension");
+  // the slice as the inner box of the input: the kernels of fl::padding with the roles exchanged
+  std::vector<int64_t> dims(4, 1);
+  std::vector<int32_t> before(4, 0), after(4, 0);
+  std::vector<Dim> od = input.shape().get();
+  for (int i = 0; i < nd; ++i) dims[(size_t)i] = input.shape().dim(i);
+  dims[(size_t)dim] = size;
+  before[(size_t)dim] = (int32_t)start;
+  after[(size_t)dim] = (int32_t)(ext - start - size);
+  od[(size_t)dim] = size;
+  detail::OpScope scope("narrow");
+  Tensor out{Shape(od), input.type()};
+  check(flhip_pad_bwd(input.tensor().device(), out.device(), dims.data(), before.data(), after.data(),
+                      tagOf(input.type(), "narrow"), hipBackendStream()));
+  if (scope.on()) scope.done({input.tensor()}, {out});
+  auto gradFunc = [dims, before, after](std::vector<Variable>& inputs, const Variable& gradOutput) {
+    auto& in = inputs[0];
+    if (!in.isCalcGrad()) return;
+    detail::OpScope scope("narrowBackward");
+    Tensor g(in.shape(), gradOutput.type());
+    check(flhip_pad_fwd(gradOutput.tensor().device(), g.device(), dims.data(), before.data(), after.data(), 0.0,
+                        tagOf(g.type(), "narrow"), hipBackendStream()));
+    if (scope.on()) scope.done({gradOutput.tensor()}, {g});
+    in.addGrad(Variable(g, false));
+  };
+  return Variable(out, {input}, gradFunc);
+}
+
 Variable moddims(const Variable& input, const Shape& dims) {
   // a 0 keeps the input's dimension, one -1 is inferred from the element count
   // (Functions.cpp:969-1008)

@@ -164,6 +164,9 @@ Variable weightNorm(const Variable& v, const Variable& g, int dim);
 Tensor rowNorm(const Tensor& v, int dim);
 // fl::padding (Functions.cpp:1751-1775): pad[i] = (before, after) for dimension i, filled with val
 Variable padding(const Variable& input, const std::vector<std::pair<int, int>>& pad, double val);
+// input(range(start, start + size)) along dimension dim, as the reference's indexing of a Variable with a range: the
+// gradient is the incoming one inside zeros
+Variable narrow(const Variable& input, int dim, long long start, long long size);
 Variable moddims(const Variable& input, const Shape& dims);
 // fl::reorder (Functions.cpp:1010-1042): dimension k of the result is dimension dims[k] of the
 // input; the gradient is reordered back with the inverse permutation

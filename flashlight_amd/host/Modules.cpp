@@ -273,6 +273,90 @@ std::string WeightNorm::prettyString() const {
   return ss.str();
 }
 
+// ---- AsymmetricConv1D, TDSBlock (flashlight/fl/contrib/modules) -------------------------
+AsymmetricConv1D::AsymmetricConv1D(int nin, int nout, int wx, int sx, IntOrPadMode px, float futurePart, int dx,
+                                   bool bias, int groups)
+    : Conv2D(nin, nout, wx, 1, sx, 1, px, 0, dx, 1, bias, groups), futurePart_(futurePart) {
+  // AsymmetricConv1D.cpp:16-25
+  if (xPad_ != static_cast<int>(PaddingMode::SAME) && xPad_ != 0)
+    throw std::invalid_argument("AsymmetricConv1D: invalid xPad_, now supports only '0' or 'SAME' ");
+  if (futurePart_ < 0 || futurePart_ > 1)
+    throw std::invalid_argument("AsymmetricConv1D: invalid futurePart_, should be in [0, 1]");
+}
+
+Variable AsymmetricConv1D::forward(const Variable& input) {
+  // AsymmetricConv1D.cpp:64-104
+  const int px = derivePadding((int)input.dim(0), xFilter_, xStride_, xPad_, xDilation_);
+  if (!(px >= 0)) throw std::invalid_argument("invalid padding for AsymmetricConv1D");
+  const int cutPx = (int)(std::abs(2 * (0.5 - futurePart_)) * px);
+  const int asymmetryPx = px + cutPx;
+  Variable output =
+      bias_ ? conv2d(input, params_[0].astype(input.type()), params_[1].astype(input.type()), xStride_, yStride_,
+                     asymmetryPx, 0, xDilation_, yDilation_, groups_, benchmarks_)
+            : conv2d(input, params_[0].astype(input.type()), xStride_, yStride_, asymmetryPx, 0, xDilation_, yDilation_,
+                     groups_, benchmarks_);
+  if (cutPx == 0) return output;
+  if (futurePart_ < 0.5) return narrow(output, 0, 0, output.dim(0) - 2 * cutPx);
+  if (futurePart_ > 0.5) return narrow(output, 0, 2 * cutPx, output.dim(0) - 2 * cutPx);
+  return output;
+}
+
+std::string AsymmetricConv1D::prettyString() const { return "AsymmetricConv1D (" + Conv2D::prettyString() + ")"; }
+
+TDSBlock::TDSBlock(int channels, int kernelSize, int width, double dropout, int innerLinearDim, int rightPadding,
+                   bool lNormIncludeTime) {
+  // TDSBlock.cpp:13-67
+  Sequential conv;
+  int convPadding = static_cast<int>(PaddingMode::SAME);
+  if (rightPadding != -1) {
+    const int totalPadding = kernelSize - 1;
+    if (rightPadding > totalPadding)
+      throw std::invalid_argument("right padding exceeds the 'SAME' padding required for TDSBlock");
+    conv.add(Padding({std::pair<int, int>{totalPadding - rightPadding, rightPadding}}, 0.0));
+    convPadding = 0;
+  }
+  conv.add(Conv2D(channels, channels, kernelSize, 1, 1, 1, convPadding, 0));
+  conv.add(ReLU());
+  conv.add(Dropout(dropout));
+  const int linearDim = channels * width;
+  if (innerLinearDim == 0) innerLinearDim = linearDim;
+  Sequential fc;
+  fc.add(Reorder(Shape({2, 1, 0, 3})));
+  fc.add(View(Shape({linearDim, -1, 1, 0})));
+  fc.add(Linear(linearDim, innerLinearDim));
+  fc.add(ReLU());
+  if (dropout > 0) fc.add(Dropout(dropout));
+  fc.add(Linear(innerLinearDim, linearDim));
+  fc.add(View(Shape({channels, width, -1, 0})));
+  fc.add(Reorder(Shape({2, 1, 0, 3})));
+  if (dropout > 0) fc.add(Dropout(dropout));
+  const std::vector<int> axes = lNormIncludeTime ? std::vector<int>{0, 1, 2} : std::vector<int>{1, 2};
+  add(std::move(conv));
+  add(LayerNorm(axes));
+  add(std::move(fc));
+  add(LayerNorm(axes));
+}
+
+std::vector<Variable> TDSBlock::forward(const std::vector<Variable>& inputs) {
+  // TDSBlock.cpp:69-75
+  if (inputs.size() != 1) throw std::invalid_argument("TDSBlock expects one input");
+  Variable out = inputs[0];
+  out = module(0)->forward({out})[0].astype(out.type()) + out;
+  out = module(1)->forward({out})[0];
+  out = module(2)->forward({out})[0].astype(out.type()) + out;
+  return module(3)->forward({out});
+}
+
+std::string TDSBlock::prettyString() const {
+  // TDSBlock.cpp:77-91
+  std::ostringstream ss;
+  const Variable convW = param(0), linW = param(4);
+  const int kw = (int)convW.dim(0), c = (int)convW.dim(2);
+  const int w = (int)linW.dim(0) / c, l = (int)linW.dim(1), l2 = (int)linW.dim(0);
+  ss << "Time-Depth Separable Block (" << kw << ", " << w << ", " << c << ") [" << l << " -> " << l2 << " -> " << l << "]";
+  return ss.str();
+}
+
 // ---- Pool2D ----------------------------------------------------------------------------
 Pool2D::Pool2D(int wx, int wy, int sx, int sy, IntOrPadMode px, IntOrPadMode py, PoolingMode mode)
     : xFilter_(wx), yFilter_(wy), xStride_(sx), yStride_(sy), xPad_(px.padVal), yPad_(py.padVal),

@@ -142,12 +142,26 @@ class Conv2D : public UnaryModule {
   std::string prettyString() const override;
   std::vector<Variable> castParams() const override { return params_; }
 
- private:
+ protected:
   int nIn_, nOut_, xFilter_, yFilter_, xStride_, yStride_, xPad_, yPad_, xDilation_, yDilation_;
   bool bias_;
   int groups_;
   // the kernel-choice benchmarks of this layer's backward passes (flashlight/fl/nn/modules/Conv2D.h:206)
   std::shared_ptr<detail::ConvBenchmarks> benchmarks_ = std::make_shared<detail::ConvBenchmarks>();
+};
+
+// flashlight/fl/contrib/modules/AsymmetricConv1D.{h,cpp}: a convolution along dimension 0 whose window looks
+// futurePart of its length ahead (0.5: symmetric, 0: causal, 1: only ahead): more padding, then the surplus results cut
+class AsymmetricConv1D : public Conv2D {
+ public:
+  AsymmetricConv1D(int nin, int nout, int wx, int sx = 1, IntOrPadMode px = 0, float futurePart = 0.5f, int dx = 1,
+                   bool bias = true, int groups = 1);
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override;
+  std::string prettyString() const override;
+
+ private:
+  float futurePart_;
 };
 
 // flashlight/fl/nn/modules/Pool2D.cpp:19-52
@@ -377,6 +391,17 @@ class WeightNorm : public Module {
   void computeWeight();
   ModulePtr module_;
   int dim_;
+};
+
+// flashlight/fl/contrib/modules/TDSBlock.{h,cpp}: a time-depth separable block over [T, W, C, B]: convolution along
+// time + ReLU + dropout with a shortcut, layer norm, two linear layers over W * C with a shortcut, layer norm
+class TDSBlock : public Container {
+ public:
+  explicit TDSBlock(int channels, int kernelSize, int width, double dropout = 0, int innerLinearDim = 0,
+                    int rightPadding = -1, bool lNormIncludeTime = true);
+  using Module::forward;
+  std::vector<Variable> forward(const std::vector<Variable>& inputs) override;
+  std::string prettyString() const override;
 };
 
 class LogSoftmax : public UnaryModule {    // Activations.cpp:180-192

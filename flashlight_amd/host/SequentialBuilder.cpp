@@ -50,6 +50,14 @@ ModulePtr parseLine(const std::string& line) {
   auto inRange = [&](size_t a, size_t c) { return a <= n && n <= c; };
   auto I = [&](size_t i) { return toInt(p[i], line); };
   const std::string& op = p[0];
+  auto F = [&](size_t i) {
+    try {
+      return std::stod(p[i]);
+    } catch (const std::exception&) {
+      failParse(line);
+    }
+    return 0.0;
+  };
 
   if (op == "V" || op == "RO") {                 // SequentialBuilder.cpp:116-129
     if (n < 2) failParse(line);
@@ -62,6 +70,19 @@ ModulePtr parseLine(const std::string& line) {
     if (!inRange(5, 7)) failParse(line);
     const int px = n >= 6 ? I(5) : 0, dx = n >= 7 ? I(6) : 1;
     return std::make_shared<Conv2D>(I(1), I(2), I(3), 1, I(4), 1, px, 0, dx, 1);
+  }
+  if (op == "TDS") {                              // SequentialBuilder.cpp:228-243
+    if (!inRange(4, 8)) failParse(line);
+    const double dropprob = n >= 5 ? F(4) : 0.0;
+    const int l2 = n >= 6 ? I(5) : 0, rPad = n >= 7 ? I(6) : -1;
+    const bool lNormIncludeTime = !(n >= 8 && I(7) == 0);
+    return std::make_shared<TDSBlock>(I(1), I(2), I(3), dropprob, l2, rPad, lNormIncludeTime);
+  }
+  if (op == "AC") {                               // :245-258
+    if (!inRange(5, 8)) failParse(line);
+    const int px = n >= 6 ? I(5) : 0, dx = n >= 8 ? I(7) : 1;
+    const float future = n >= 7 ? (float)F(6) : 1.0f;
+    return std::make_shared<AsymmetricConv1D>(I(1), I(2), I(3), I(4), px, future, dx);
   }
   if (op == "C2") {
     if (!inRange(7, 11)) failParse(line);
@@ -102,14 +123,6 @@ ModulePtr parseLine(const std::string& line) {
     return std::make_shared<LogSoftmax>(I(1));
   }
   // the other activations (SequentialBuilder.cpp:390-466) and dropout (:360-366)
-  auto F = [&](size_t i) {
-    try {
-      return std::stod(p[i]);
-    } catch (const std::exception&) {
-      failParse(line);
-    }
-    return 0.0;
-  };
   if (op == "ELU" || op == "R6" || op == "LG" || op == "HT" || op == "T") {
     if (n != 1) failParse(line);
     if (op == "ELU") return std::make_shared<ELU>();
@@ -151,7 +164,7 @@ ModulePtr parseLine(const std::string& line) {
     const float dropout = n > 5 ? std::stof(p[5]) : 0.0f;
     return std::make_shared<RNN>(I(1), I(2), layers, mode, bidirectional, dropout);
   }
-  static const char* const absent[] = {"TR", "CFR", "POSEMB", "SINPOSEMB", "TDS", "AC", "E", "ADAPTIVEE",
+  static const char* const absent[] = {"TR", "CFR", "POSEMB", "SINPOSEMB", "E", "ADAPTIVEE",
                                        "PR", "RES", "SKIP", "SKIPL", "SAUG", "PC"};
   for (const char* a : absent)
     if (op == a)

@@ -958,7 +958,7 @@ static void testArchBuilder() {
   // malformed lines, lines for modules that do not exist here, a missing file
   for (const char* bad : {"C 3 4 5", "C2 3 4 5 6 1", "L 5", "BN 8", "LN", "LN 3", "M 2 2 2", "R 1", "LSM", "GRU 4",
                           "C 3 x 5 1", "XYZ 1 2", "RO", "DO", "DO 0.2 1", "GLU", "ELU 1", "SH 1 2", "WN 3", "WN 1 C 4 4 3 1", "WN 3 R", "PD 0 1", "PD 0 1 1 1",
-                          "TDS 10 21 80", "RES 2 1 3", "PC f16"})
+                          "TDS 10 21", "AC 1 2 3", "RES 2 1 3", "PC f16"})
     CHECK(throws<std::invalid_argument>([&] { one(bad); }));
   CHECK(throws<std::runtime_error>([] { buildSequentialModule(std::string("/nonexistent/arch.txt"), 1, 1); }));
   // from a file
@@ -1134,6 +1134,81 @@ static void testActivationModules() {
     CHECK(hostOf(in.grad()) == dxr);
     CHECK(throws<std::invalid_argument>([&] { padding(Variable(Tensor::fromVector({4, 2}, randn(8, 1)), false), {{1, 1}, {0, 0}, {1, 0}}, 0.0); }));
   }
+  // AC: a window that looks only ahead (future part 1, the line's default) or only back (0): against the checker's
+  // convolution with twice the SAME padding, cut at the front / the back (AsymmetricConv1D.cpp:64-104)
+  for (const char* line : {"AC 4 6 5 1 -1", "AC 4 6 5 1 -1 0", "AC 4 6 5 1 -1 0.5", "AC 4 6 5 1 -1 0.75"}) {
+    setSeed(29);
+    auto ac = one(line);
+    CHECK(ac->prettyString().rfind("AsymmetricConv1D (Conv2D", 0) == 0);
+    const int T = 17, Cc = 4, K = 6, k = 5, B = 3, p0 = 2;
+    const double fut = std::string(line).size() > 13 ? std::stod(std::string(line).substr(14)) : 1.0;
+    const int cut = (int)(std::fabs(2 * (0.5 - fut)) * p0), pad = p0 + cut;
+    auto x = randn((size_t)T * Cc * B, 770), wv = hostOf(ac->param(0)), bv = hostOf(ac->param(1));
+    flref_conv d{B, Cc, 1, T, K, 1, k, 1, 1, 0, pad, 1, 1, 1};
+    int32_t OH, OW;
+    flref_conv_out(&d, &OH, &OW);
+    CHECK(OW == T + 2 * cut);
+    std::vector<float> yfull((size_t)B * K * OW), yr((size_t)B * K * T);
+    flref_conv2d_fwd(&d, x.data(), wv.data(), bv.data(), yfull.data());
+    const int off = fut > 0.5 ? 2 * cut : 0;
+    for (int r = 0; r < B * K; ++r)
+      for (int t = 0; t < T; ++t) yr[(size_t)r * T + t] = yfull[(size_t)r * OW + off + t];
+    Variable in(Tensor::fromVector({T, 1, Cc, B}, x), true);
+    Variable y = ac->forward({in})[0];
+    CHECK(y.shape() == Shape({T, 1, K, B}));
+    CHECK(relL2(hostOf(y), yr) <= 1e-5);
+    // the gradient of the cut: zeros where results were dropped
+    auto dy = randn(yr.size(), 771);
+    std::vector<float> dyfull(yfull.size(), 0.f), dxr(x.size());
+    for (int r = 0; r < B * K; ++r)
+      for (int t = 0; t < T; ++t) dyfull[(size_t)r * OW + off + t] = dy[(size_t)r * T + t];
+    flref_conv2d_bwd_data(&d, dyfull.data(), wv.data(), dxr.data());
+    y.backward(Variable(Tensor::fromVector(y.shape(), dy), false));
+    CHECK(relL2(hostOf(in.grad()), dxr) <= 1e-5);
+  }
+  CHECK(throws<std::invalid_argument>([&] { one("AC 4 6 5 1 2"); }));
+  CHECK(throws<std::invalid_argument>([&] { one("AC 4 6 5 1 -1 1.5"); }));
+  // TDS: the block from its line equals the chain of its parts (TDSBlock.cpp:13-75), with and without dropout-free
+  // right padding and time in the layer norm
+  for (const char* line : {"TDS 3 5 4", "TDS 3 5 4 0 10 1 0"}) {
+    const bool second = std::string(line).size() > 9;
+    setSeed(31);
+    auto tds = std::dynamic_pointer_cast<TDSBlock>(one(line));
+    CHECK(tds != nullptr);
+    if (!tds) continue;
+    setSeed(31);
+    const int C3 = 3, KS = 5, Wd = 4, LD = C3 * Wd, inner = second ? 10 : LD;
+    Sequential conv, fc;
+    if (second) conv.add(Padding({std::pair<int, int>{KS - 1 - 1, 1}}, 0.0));
+    conv.add(Conv2D(C3, C3, KS, 1, 1, 1, second ? IntOrPadMode(0) : IntOrPadMode(PaddingMode::SAME), 0));
+    conv.add(ReLU());
+    fc.add(Reorder(Shape({2, 1, 0, 3})));
+    fc.add(View(Shape({LD, -1, 1, 0})));
+    fc.add(Linear(LD, inner));
+    fc.add(ReLU());
+    fc.add(Linear(inner, LD));
+    fc.add(View(Shape({C3, Wd, -1, 0})));
+    fc.add(Reorder(Shape({2, 1, 0, 3})));
+    const std::vector<int> axes = second ? std::vector<int>{1, 2} : std::vector<int>{0, 1, 2};
+    LayerNorm ln1(axes), ln2(axes);
+    CHECK(tds->params().size() == conv.params().size() + fc.params().size() + ln1.params().size() + ln2.params().size());
+    const int T = 11, B = 2;
+    auto x = randn((size_t)T * Wd * C3 * B, 780);
+    Variable in1(Tensor::fromVector({T, Wd, C3, B}, x), true), in2(Tensor::fromVector({T, Wd, C3, B}, x), true);
+    Variable y1 = tds->forward({in1})[0];
+    Variable h = conv.forward(in2) + in2;
+    h = ln1.forward(h);
+    h = fc.forward(h) + h;
+    Variable y2 = ln2.forward(h);
+    CHECK(y1.shape() == in1.shape() && hostOf(y1) == hostOf(y2));
+    auto dy = randn(x.size(), 781);
+    y1.backward(Variable(Tensor::fromVector(y1.shape(), dy), false));
+    y2.backward(Variable(Tensor::fromVector(y2.shape(), dy), false));
+    CHECK(hostOf(in1.grad()) == hostOf(in2.grad()));
+    CHECK(tds->prettyString() == std::string("Time-Depth Separable Block (5, ") + std::to_string(inner / 3) + ", 3) [12 -> " +
+                                     std::to_string(inner) + " -> 12]");
+  }
+  CHECK(throws<std::invalid_argument>([&] { one("TDS 3 5 4 0 0 9"); }));
   // a GLU convolution block from text, as in wav2letter's architecture files
   {
     setSeed(17);
