@@ -485,6 +485,7 @@ Variable tanh(const Variable& input) { return activation("tanh", FLHIP_ACT_TANH,
 Variable log(const Variable& input) { return activation("log", FLHIP_ACT_LOG, input, 0.0, 0.0); }
 Variable sigmoid(const Variable& input) { return activation("sigmoid", FLHIP_ACT_SIGMOID, input, 0.0, 0.0); }
 Variable swish(const Variable& input, double beta) { return activation("swish", FLHIP_ACT_SWISH, input, beta, 0.0); }
+Variable scale(const Variable& input, double factor) { return activation("scale", FLHIP_ACT_SCALE, input, factor, 0.0); }
 
 Variable gatedlinearunit(const Variable& input, int dim) {
   // Functions.cpp:1567-1579

@@ -151,6 +151,10 @@ Variable tanh(const Variable& input);
 Variable log(const Variable& input);
 Variable sigmoid(const Variable& input);
 Variable swish(const Variable& input, double beta);
+// a Variable times a number (the reference's operator*(Variable, double))
+Variable scale(const Variable& input, double factor);
+inline Variable operator*(const Variable& lhs, double rhs) { return scale(lhs, rhs); }
+inline Variable operator*(double lhs, const Variable& rhs) { return scale(rhs, lhs); }
 // fl::gatedlinearunit (Functions.cpp:1567-1610): first half of dimension `dim` times the sigmoid of the second half
 Variable gatedlinearunit(const Variable& input, int dim);
 // fl::dropout (Functions.cpp:1777-1785): input * mask / (1 - p); p <= 0 returns the input.  The mask is a

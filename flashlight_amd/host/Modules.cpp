@@ -357,6 +357,93 @@ std::string TDSBlock::prettyString() const {
   return ss.str();
 }
 
+// ---- Residual (flashlight/fl/contrib/modules/Residual.cpp) --------------------------------
+void Residual::addScale(int beforeLayer, float scale) {
+  const int nLayers = (int)modules_.size() - (int)projectionsIndices_.size();
+  if (beforeLayer < 1 || beforeLayer > nLayers + 1)
+    throw std::invalid_argument("Residual: invalid layer index " + std::to_string(beforeLayer) +
+                                " before which apply the scaling");
+  if (scales_.find(beforeLayer - 1) != scales_.end())
+    throw std::invalid_argument("Residual: scaling before layer " + std::to_string(beforeLayer) +
+                                " was already added; adding only once is allowed");
+  scales_[beforeLayer - 1] = scale;
+}
+
+void Residual::checkShortcut(int fromLayer, int toLayer) {
+  const int nLayers = (int)modules_.size() - (int)projectionsIndices_.size();
+  if (fromLayer < 0 || fromLayer >= nLayers || toLayer <= 0 || toLayer > nLayers + 2 || toLayer - fromLayer <= 1)
+    throw std::invalid_argument("Residual: invalid skip connection; check fromLayer=" + std::to_string(fromLayer) +
+                                " and toLayer=" + std::to_string(toLayer) +
+                                " parameters. They are out of range of added layers");
+  const auto it = shortcut_.find(toLayer - 1);
+  if (it != shortcut_.end() && it->second.find(fromLayer) != it->second.end())
+    throw std::invalid_argument("Residual: skip connection for fromLayer " + std::to_string(fromLayer) + " to toLayer " +
+                                std::to_string(toLayer) + " is already added");
+}
+
+void Residual::addShortcut(int fromLayer, int toLayer) {
+  checkShortcut(fromLayer, toLayer);
+  shortcut_[toLayer - 1].insert({fromLayer, -1});
+}
+
+void Residual::addShortcut(int fromLayer, int toLayer, ModulePtr projection) {
+  checkShortcut(fromLayer, toLayer);
+  Container::add(std::move(projection));
+  shortcut_[toLayer - 1].insert({fromLayer, (int)modules_.size() - 1});
+  projectionsIndices_.insert((int)modules_.size() - 1);
+}
+
+Variable Residual::applyScale(const Variable& input, int layerIndex) {
+  // Residual.cpp:69-73 multiplies by 1 where no scale was given: the same values
+  const auto it = scales_.find(layerIndex);
+  return it == scales_.end() ? input : input * (double)it->second;
+}
+
+std::vector<Variable> Residual::forward(const std::vector<Variable>& inputs) {
+  if (inputs.size() != 1) throw std::invalid_argument("Residual module expects only one input");
+  return {forward(inputs[0])};
+}
+
+Variable Residual::forward(const Variable& input) {
+  // Residual.cpp:82-124
+  Variable output = input;
+  const int nLayers = (int)modules_.size() - (int)projectionsIndices_.size();
+  std::vector<Variable> outputs((size_t)nLayers + 1);
+  outputs[0] = input;
+  auto addShortcuts = [&](int layerIndex) {
+    const auto it = shortcut_.find(layerIndex);
+    if (it == shortcut_.end()) return;
+    for (const auto& sc : it->second) {
+      Variable connectionOut = outputs[(size_t)sc.first];
+      if (sc.second != -1) connectionOut = modules_[(size_t)sc.second]->forward({outputs[(size_t)sc.first]}).front();
+      output = output + connectionOut.astype(output.type());
+    }
+  };
+  int moduleIndex = 0;
+  for (int layerIndex = 0; layerIndex < nLayers; ++layerIndex, ++moduleIndex) {
+    while (projectionsIndices_.count(moduleIndex)) ++moduleIndex;
+    addShortcuts(layerIndex);
+    output = modules_[(size_t)moduleIndex]->forward({applyScale(output, layerIndex)}).front();
+    outputs[(size_t)layerIndex + 1] = output;
+  }
+  addShortcuts(nLayers);
+  return applyScale(output, nLayers);
+}
+
+std::string Residual::prettyString() const {
+  std::ostringstream ss;
+  const int nLayers = (int)modules_.size() - (int)projectionsIndices_.size();
+  ss << "Residual (" << nLayers << " layers";
+  for (const auto& end : shortcut_)
+    for (const auto& sc : end.second) {
+      ss << "; skip " << sc.first << " -> " << end.first + 1;
+      if (sc.second != -1) ss << " through " << modules_[(size_t)sc.second]->prettyString();
+    }
+  for (const auto& sc : scales_) ss << "; scale " << sc.second << " before " << sc.first + 1;
+  ss << ")";
+  return ss.str();
+}
+
 // ---- Pool2D ----------------------------------------------------------------------------
 Pool2D::Pool2D(int wx, int wy, int sx, int sy, IntOrPadMode px, IntOrPadMode py, PoolingMode mode)
     : xFilter_(wx), yFilter_(wy), xStride_(sx), yStride_(sy), xPad_(px.padVal), yPad_(py.padVal),

@@ -7,8 +7,10 @@
 // operators are not provided.
 #pragma once
 
+#include <map>
 #include <memory>
 #include <string>
+#include <unordered_set>
 #include <vector>
 
 #include "Functions.h"
@@ -402,6 +404,33 @@ class TDSBlock : public Container {
   using Module::forward;
   std::vector<Variable> forward(const std::vector<Variable>& inputs) override;
   std::string prettyString() const override;
+};
+
+// flashlight/fl/contrib/modules/Residual.{h,cpp}: a chain of layers with shortcuts from the output of layer
+// `fromLayer` (0 = the input) to the input of layer `toLayer` (number of layers + 1 = the output), optionally through a
+// projection module, and a scale applied before a layer (or to the output)
+class Residual : public Container {
+ public:
+  Residual() = default;
+  void addScale(int beforeLayer, float scale);
+  void addShortcut(int fromLayer, int toLayer);
+  void addShortcut(int fromLayer, int toLayer, ModulePtr projection);
+  template <typename T, typename = std::enable_if_t<std::is_base_of_v<Module, std::decay_t<T>>>>
+  void addShortcut(int fromLayer, int toLayer, T&& projection) {
+    addShortcut(fromLayer, toLayer, ModulePtr(std::make_shared<std::decay_t<T>>(std::forward<T>(projection))));
+  }
+  std::unordered_set<int> getProjectionsIndices() const { return projectionsIndices_; }
+  using Module::forward;
+  std::vector<Variable> forward(const std::vector<Variable>& inputs) override;
+  Variable forward(const Variable& input);
+  std::string prettyString() const override;
+
+ private:
+  void checkShortcut(int fromLayer, int toLayer);
+  Variable applyScale(const Variable& input, int layerIndex);
+  std::map<int, std::map<int, int>> shortcut_;      // end -> (start -> projection module or -1)
+  std::unordered_set<int> projectionsIndices_;
+  std::map<int, float> scales_;
 };
 
 class LogSoftmax : public UnaryModule {    // Activations.cpp:180-192

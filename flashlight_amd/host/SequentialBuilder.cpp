@@ -164,8 +164,7 @@ ModulePtr parseLine(const std::string& line) {
     const float dropout = n > 5 ? std::stof(p[5]) : 0.0f;
     return std::make_shared<RNN>(I(1), I(2), layers, mode, bidirectional, dropout);
   }
-  static const char* const absent[] = {"TR", "CFR", "POSEMB", "SINPOSEMB", "E", "ADAPTIVEE",
-                                       "PR", "RES", "SKIP", "SKIPL", "SAUG", "PC"};
+  static const char* const absent[] = {"TR", "CFR", "POSEMB", "SINPOSEMB", "E", "ADAPTIVEE", "PR", "SAUG", "PC"};
   for (const char* a : absent)
     if (op == a)
       throw std::invalid_argument("buildSequentialModule: module '" + op +
@@ -173,17 +172,81 @@ ModulePtr parseLine(const std::string& line) {
   failParse(line);
 }
 
+// The module that starts at lines[idx]; *parsed = the lines it took beyond its first (SequentialBuilder.cpp:98-104,
+// 498-566): a residual block "RES layers skips [repeats]" is followed by its layer lines and its "SKIP from to [scale]" /
+// "SKIPL from to projectionLayers [scale]" lines (the latter followed by the lines of the projection).
+ModulePtr parseLines(const std::vector<std::string>& lines, size_t idx, size_t* parsed) {
+  const std::string& line = lines[idx];
+  *parsed = 0;
+  const std::vector<std::string> p = splitOnWhitespace(line);
+  if (p.empty()) failParse(line);
+  if (p[0] == "SKIP" || p[0] == "SKIPL") failParse(line);      // only inside a residual block
+  if (p[0] != "RES") return parseLine(line);
+  if (p.size() <= 3) failParse(line);                          // :500-502: the number of repeats is not optional
+  const int numResLayers = toInt(p[1], line), numSkip = toInt(p[2], line);
+  const int numBlocks = p.size() == 4 ? toInt(p[3], line) : 1;
+  if (numBlocks <= 0) throw std::invalid_argument("Invalid number of residual blocks: " + std::to_string(numBlocks));
+  size_t taken = 0;
+  auto block = [&]() {
+    auto res = std::make_shared<Residual>();
+    size_t projections = 0;
+    for (int i = 1; i <= numResLayers + numSkip; ++i) {
+      const size_t at = idx + (size_t)i + projections;
+      if (at >= lines.size()) throw std::invalid_argument("Failed parsing Residual block");
+      const std::string& rl = lines[at];
+      const std::vector<std::string> q = splitOnWhitespace(rl);
+      if (q.empty()) failParse(rl);
+      if (q[0] == "SKIP") {
+        if (q.size() < 3 || q.size() > 4) failParse(rl);
+        res->addShortcut(toInt(q[1], rl), toInt(q[2], rl));
+        if (q.size() == 4) res->addScale(toInt(q[2], rl), std::stof(q[3]));
+      } else if (q[0] == "SKIPL") {
+        if (q.size() < 4 || q.size() > 5) failParse(rl);
+        const int nproj = toInt(q[3], rl);
+        auto projection = std::make_shared<Sequential>();
+        for (int j = 1; j <= nproj; ++j) {
+          if (at + (size_t)j >= lines.size()) throw std::invalid_argument("Failed parsing Residual block");
+          projection->add(parseLine(lines[at + (size_t)j]));
+        }
+        res->addShortcut(toInt(q[1], rl), toInt(q[2], rl), ModulePtr(projection));
+        if (q.size() == 5) res->addScale(toInt(q[2], rl), std::stof(q[4]));
+        projections += (size_t)nproj;
+      } else {
+        res->add(parseLine(rl));
+      }
+    }
+    taken = (size_t)(numResLayers + numSkip) + projections;
+    return res;
+  };
+  ModulePtr out;
+  if (numBlocks > 1) {
+    auto seq = std::make_shared<Sequential>();
+    for (int b = 0; b < numBlocks; ++b) seq->add(block());     // every repeat reads the same lines
+    out = seq;
+  } else {
+    out = block();
+  }
+  *parsed = taken;
+  return out;
+}
+
 }  // namespace
 
 std::shared_ptr<fl::Sequential> buildSequentialModule(const std::vector<std::string>& lines, int64_t nFeatures,
                                                       int64_t nClasses) {
-  auto net = std::make_shared<fl::Sequential>();
+  std::vector<std::string> layers;
   for (const std::string& raw : lines) {
     std::string l = trim(raw);
     replaceAll(l, "NFEAT", std::to_string(nFeatures));
     replaceAll(l, "NLABEL", std::to_string(nClasses));
     if (l.empty() || l[0] == '#') continue;   // blank lines and comments
-    net->add(parseLine(l));
+    layers.push_back(l);
+  }
+  auto net = std::make_shared<fl::Sequential>();
+  for (size_t i = 0; i < layers.size();) {
+    size_t parsed = 0;
+    net->add(parseLines(layers, i, &parsed));
+    i += parsed + 1;
   }
   return net;
 }

@@ -365,6 +365,7 @@ int flhip_relu_bwd(const void* dy, const void* x, void* dx, size_t n, int dtype,
  *                      (Activations.cpp:60-62, 88-90)
  *   FLHIP_ACT_TANH     fl::tanh (Functions.cpp:454-463)      FLHIP_ACT_LOG      fl::log (:403-411)
  *   FLHIP_ACT_SWISH    a = beta: x * sigmoid(a x) (:498-500)  FLHIP_ACT_SIGMOID  fl::sigmoid (:488-496)
+ *   FLHIP_ACT_SCALE    a x: a Variable times a number (the scales of fl::Residual, contrib/modules/Residual.cpp:69-73)
  * flhip_act_bwd: dx = dy * f'(x) from the gradient and the forward INPUT (clamp passes the gradient where
  * lo < x < hi, strictly, as the reference's mask on its result does).  y / dx may alias x / dy. */
 #define FLHIP_ACT_ELU 0
@@ -373,6 +374,7 @@ int flhip_relu_bwd(const void* dy, const void* x, void* dx, size_t n, int dtype,
 #define FLHIP_ACT_LOG 3
 #define FLHIP_ACT_SWISH 4
 #define FLHIP_ACT_SIGMOID 5
+#define FLHIP_ACT_SCALE 6
 int flhip_act_fwd(int op, const void* x, void* y, size_t n, double a, double b, int dtype, void* stream);
 int flhip_act_bwd(int op, const void* dy, const void* x, void* dx, size_t n, double a, double b, int dtype,
                   void* stream);

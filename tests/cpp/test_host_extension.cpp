@@ -958,7 +958,7 @@ static void testArchBuilder() {
   // malformed lines, lines for modules that do not exist here, a missing file
   for (const char* bad : {"C 3 4 5", "C2 3 4 5 6 1", "L 5", "BN 8", "LN", "LN 3", "M 2 2 2", "R 1", "LSM", "GRU 4",
                           "C 3 x 5 1", "XYZ 1 2", "RO", "DO", "DO 0.2 1", "GLU", "ELU 1", "SH 1 2", "WN 3", "WN 1 C 4 4 3 1", "WN 3 R", "PD 0 1", "PD 0 1 1 1",
-                          "TDS 10 21", "AC 1 2 3", "RES 2 1 3", "PC f16"})
+                          "TDS 10 21", "AC 1 2 3", "RES 2 1", "RES 1 0 1", "SKIP 0 2", "PC f16"})
     CHECK(throws<std::invalid_argument>([&] { one(bad); }));
   CHECK(throws<std::runtime_error>([] { buildSequentialModule(std::string("/nonexistent/arch.txt"), 1, 1); }));
   // from a file
@@ -1209,6 +1209,65 @@ static void testActivationModules() {
                                      std::to_string(inner) + " -> 12]");
   }
   CHECK(throws<std::invalid_argument>([&] { one("TDS 3 5 4 0 0 9"); }));
+  // RES: residual blocks from text against the same network written out (Residual.cpp:82-124; SequentialBuilder.cpp:498-566)
+  {
+    const std::vector<std::string> arch = {
+        "RES 3 2 1",
+        "C 4 4 3 1 -1",
+        "R",
+        "C 4 6 3 1 -1",
+        "SKIP 0 2 0.5",              // the input joins the output of layer 1 in front of layer 2, scaled by 0.5 there
+        "SKIPL 0 4 1 0.25",          // and, through a projection, the block's output
+        "C 4 6 1 1",
+        "T",
+        "RES 1 1 2",                 // two blocks of one layer with an identity shortcut around it
+        "L 6 6",
+        "SKIP 0 2",
+    };
+    setSeed(41);
+    auto net = buildSequentialModule(arch, 1, 1);
+    CHECK(net->modules().size() == 3);
+    auto res = std::dynamic_pointer_cast<Residual>(net->module(0));
+    CHECK(res != nullptr && res->modules().size() == 4 && res->getProjectionsIndices().size() == 1);
+    setSeed(41);
+    Conv2D c1(4, 4, 3, 1, 1, 1, PaddingMode::SAME, 0), c2(4, 6, 3, 1, 1, 1, PaddingMode::SAME, 0), proj(4, 6, 1, 1, 1, 1, 0, 0);
+    ReLU relu1;
+    Tanh tanh1;
+    Linear l1(6, 6), l2(6, 6);
+    const int T = 9, B = 2;
+    auto x = randn((size_t)T * 4 * B, 790);
+    Variable in1(Tensor::fromVector({T, 1, 4, B}, x), true), in2(Tensor::fromVector({T, 1, 4, B}, x), true);
+    Variable y1 = net->module(0)->forward({in1})[0];
+    Variable h = c1.forward(in2);                          // layer 1
+    h = relu1.forward((h + in2) * 0.5);                    // shortcut 0 -> 2, scale before layer 2
+    h = c2.forward(h);                                     // layer 3
+    Variable y2 = (h + proj.forward(in2)) * 0.25;          // shortcut 0 -> 4 through the projection, scale at the output
+    CHECK(y1.shape() == Shape({T, 1, 6, B}) && hostOf(y1) == hostOf(y2));
+    auto dy = randn((size_t)y1.tensor().elements(), 791);
+    y1.backward(Variable(Tensor::fromVector(y1.shape(), dy), false));
+    y2.backward(Variable(Tensor::fromVector(y2.shape(), dy), false));
+    CHECK(hostOf(in1.grad()) == hostOf(in2.grad()));
+    // the rest of the network: tanh, then two residual linear blocks
+    auto z = randn((size_t)6 * 5, 792);
+    Variable zin1(Tensor::fromVector({6, 5}, z), true), zin2(Tensor::fromVector({6, 5}, z), true);
+    Variable z1 = net->module(2)->forward({net->module(1)->forward({zin1})[0]})[0];
+    Variable t = tanh1.forward(zin2);
+    t = l1.forward(t) + t;
+    Variable z2 = l2.forward(t) + t;
+    CHECK(hostOf(z1) == hostOf(z2));
+    // checks of the reference's bookkeeping
+    Residual r;
+    r.add(ReLU());
+    r.add(ReLU());
+    CHECK(throws<std::invalid_argument>([&] { r.addShortcut(0, 1); }));        // to the next layer: no shortcut
+    CHECK(throws<std::invalid_argument>([&] { r.addShortcut(2, 4); }));
+    r.addShortcut(0, 3);
+    CHECK(throws<std::invalid_argument>([&] { r.addShortcut(0, 3); }));
+    r.addScale(3, 0.5f);
+    CHECK(throws<std::invalid_argument>([&] { r.addScale(3, 0.5f); }));
+    CHECK(throws<std::invalid_argument>([&] { r.addScale(4, 0.5f); }));
+    CHECK(throws<std::invalid_argument>([&] { buildSequentialModule(std::vector<std::string>{"RES 2 0 1", "R"}, 1, 1); }));
+  }
   // a GLU convolution block from text, as in wav2letter's architecture files
   {
     setSeed(17);

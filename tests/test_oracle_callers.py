@@ -197,6 +197,7 @@ _ACTS = [
     (flref.ACT_SWISH, 1.0, 0.0, F.silu),
     (flref.ACT_SWISH, 1.7, 0.0, lambda t: t * torch.sigmoid(1.7 * t)),
     (flref.ACT_SIGMOID, 0.0, 0.0, torch.sigmoid),
+    (flref.ACT_SCALE, -0.37, 0.0, lambda t: -0.37 * t),
 ]
 
 
