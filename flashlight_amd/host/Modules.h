@@ -433,6 +433,23 @@ class Residual : public Container {
   std::map<int, float> scales_;
 };
 
+// nn/modules/PrecisionCast.cpp:14-30: every input cast to the target type (the gradient is cast back by astype)
+class PrecisionCast : public Module {
+ public:
+  explicit PrecisionCast(dtype targetType) : targetType_(targetType) {}
+  using Module::forward;
+  std::vector<Variable> forward(const std::vector<Variable>& inputs) override {
+    std::vector<Variable> out;
+    for (const auto& in : inputs) out.push_back(in.astype(targetType_));
+    return out;
+  }
+  Variable forward(const Variable& input) { return input.astype(targetType_); }
+  std::string prettyString() const override { return "PrecisionCast"; }
+
+ private:
+  dtype targetType_;
+};
+
 class LogSoftmax : public UnaryModule {    // Activations.cpp:180-192
  public:
   explicit LogSoftmax(int dim = 0) : dim_(dim) {}

@@ -143,6 +143,13 @@ ModulePtr parseLine(const std::string& line) {
     if (n != 2) failParse(line);
     return std::make_shared<Dropout>(F(1));
   }
+  if (op == "PC") {                               // SequentialBuilder.cpp:583-589; the names of fl::stringToDtype that
+    if (n != 2) failParse(line);                  // this backend converts among, and bf16
+    if (p[1] == "f32") return std::make_shared<PrecisionCast>(dtype::f32);
+    if (p[1] == "f16") return std::make_shared<PrecisionCast>(dtype::f16);
+    if (p[1] == "bf16") return std::make_shared<PrecisionCast>(dtype::bf16);
+    throw std::invalid_argument("stringToDtype: Invalid input type: " + p[1]);
+  }
   if (op == "PD") {                               // SequentialBuilder.cpp:131-144: a value, then (before, after) pairs
     if (!inRange(4, 10) || (n & 1)) failParse(line);
     const double val = F(1);
@@ -164,7 +171,7 @@ ModulePtr parseLine(const std::string& line) {
     const float dropout = n > 5 ? std::stof(p[5]) : 0.0f;
     return std::make_shared<RNN>(I(1), I(2), layers, mode, bidirectional, dropout);
   }
-  static const char* const absent[] = {"TR", "CFR", "POSEMB", "SINPOSEMB", "E", "ADAPTIVEE", "PR", "SAUG", "PC"};
+  static const char* const absent[] = {"TR", "CFR", "POSEMB", "SINPOSEMB", "E", "ADAPTIVEE", "PR", "SAUG"};
   for (const char* a : absent)
     if (op == a)
       throw std::invalid_argument("buildSequentialModule: module '" + op +

@@ -958,7 +958,7 @@ static void testArchBuilder() {
   // malformed lines, lines for modules that do not exist here, a missing file
   for (const char* bad : {"C 3 4 5", "C2 3 4 5 6 1", "L 5", "BN 8", "LN", "LN 3", "M 2 2 2", "R 1", "LSM", "GRU 4",
                           "C 3 x 5 1", "XYZ 1 2", "RO", "DO", "DO 0.2 1", "GLU", "ELU 1", "SH 1 2", "WN 3", "WN 1 C 4 4 3 1", "WN 3 R", "PD 0 1", "PD 0 1 1 1",
-                          "TDS 10 21", "AC 1 2 3", "RES 2 1", "RES 1 0 1", "SKIP 0 2", "PC f16"})
+                          "TDS 10 21", "AC 1 2 3", "RES 2 1", "RES 1 0 1", "SKIP 0 2", "PC", "PC f64", "PR 1", "E 4 5"})
     CHECK(throws<std::invalid_argument>([&] { one(bad); }));
   CHECK(throws<std::runtime_error>([] { buildSequentialModule(std::string("/nonexistent/arch.txt"), 1, 1); }));
   // from a file
@@ -1267,6 +1267,24 @@ static void testActivationModules() {
     CHECK(throws<std::invalid_argument>([&] { r.addScale(3, 0.5f); }));
     CHECK(throws<std::invalid_argument>([&] { r.addScale(4, 0.5f); }));
     CHECK(throws<std::invalid_argument>([&] { buildSequentialModule(std::vector<std::string>{"RES 2 0 1", "R"}, 1, 1); }));
+  }
+  // PC: the cast and the gradient's cast back
+  {
+    auto x = randn(40, 795);
+    Variable in(Tensor::fromVector({8, 5}, x), true);
+    Variable y = one("PC bf16")->forward({in})[0];
+    CHECK(y.type() == dtype::bf16);
+    std::vector<float> xr(x);
+    for (auto& v : xr) v = bf16round(v);
+    CHECK(hostOf(y) == xr);
+    Variable z = one("PC f32")->forward({y})[0];
+    CHECK(z.type() == dtype::f32 && hostOf(z) == xr);
+    auto dy = randn(40, 796);
+    z.backward(Variable(Tensor::fromVector({8, 5}, dy), false));
+    std::vector<float> dr(dy);
+    for (auto& v : dr) v = bf16round(v);
+    CHECK(in.grad().type() == dtype::f32 && hostOf(in.grad()) == dr);
+    CHECK(one("PC f16")->forward({in})[0].type() == dtype::f16);
   }
   // a GLU convolution block from text, as in wav2letter's architecture files
   {
