@@ -53,7 +53,7 @@ def _compile(src):
 HOST = os.path.join(HERE, "host")
 HOST_LIB = os.path.join(LIBDIR, "libflhip_host.so")
 STEP_BENCH = os.path.join(LIBDIR, "flhip_step_bench")
-HOST_SOURCES = ["HipTensor.cpp", "HipAutogradExtension.cpp", "Functions.cpp", "Modules.cpp", "Resnet.cpp",
+HOST_SOURCES = ["HipTensor.cpp", "HipAutogradExtension.cpp", "Functions.cpp", "Modules.cpp", "Optimizers.cpp", "Resnet.cpp",
                 "SequentialBuilder.cpp"]
 TESTS_DIR = os.path.join(ROOT, "tests", "cpp")
 TESTS_BIN = os.path.join(TESTS_DIR, "bin")

@@ -151,6 +151,51 @@ __global__ void __launch_bounds__(256) convert_many_kernel(ConvertMany a) {
   }
 }
 
+// fl::SGDOptimizer::step (flashlight/fl/optim/SGDOptimizer.cpp:38-68) over several parameter tensors in one launch, in
+// place: g = grad + wd w; with momentum v = mu v + g and g = nesterov ? g + mu v : v; w = w - lr g.  The same packing of
+// (tensor, piece) into the grid as convert_many_kernel.
+constexpr int SGD_MAX = 48;
+struct SgdMany {
+  void* w[SGD_MAX];
+  const void* g[SGD_MAX];
+  void* v[SGD_MAX];
+  unsigned first[SGD_MAX + 1];
+  unsigned long long n[SGD_MAX];
+  int count;
+  float lr, mu, wd;
+  int nesterov;
+};
+template <typename T>
+__global__ void __launch_bounds__(256) sgd_many_kernel(SgdMany a) {
+  int lo = 0, hi = a.count;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (a.first[mid] <= blockIdx.x) lo = mid; else hi = mid;
+  }
+  T* w = static_cast<T*>(a.w[lo]);
+  const T* g = static_cast<const T*>(a.g[lo]);
+  T* v = static_cast<T*>(a.v[lo]);
+  const size_t base = (size_t)(blockIdx.x - a.first[lo]) * 2048;
+  const size_t n = a.n[lo];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const size_t i = base + (size_t)k * 256 + threadIdx.x;
+    if (i < n) {
+      const float wi = ld(w, i);
+      float gi = ld(g, i);
+      if (a.wd != 0.f) gi = gi + a.wd * wi;
+      if (a.mu != 0.f) {
+        const float vi = a.mu * ld(v, i) + gi;
+        st(v, i, vi);
+        // the velocity as it is stored (rounded for 16-bit parameters), like the reference's evaluated tensor
+        const float vs = ld(v, i);
+        gi = a.nesterov ? gi + vs * a.mu : vs;
+      }
+      st(w, i, wi - a.lr * gi);
+    }
+  }
+}
+
 template <typename D>
 __global__ void __launch_bounds__(256) fill_kernel(D* __restrict__ dst, float value, size_t n) {
   const size_t stride = (size_t)gridDim.x * 256;
@@ -285,6 +330,42 @@ extern "C" int flhip_convert_many(const void* const* src, void* const* dst, cons
   }
   flush();
   return check_launch("convert_many");
+}
+
+extern "C" int flhip_sgd_many(void* const* params, const void* const* grads, void* const* velocities, const size_t* n,
+                              int count, double lr, double momentum, double weight_decay, int nesterov, int dtype,
+                              void* stream) {
+  FLHIP_REQUIRE(dtype_ok(dtype), "sgd_many: unknown dtype");
+  FLHIP_REQUIRE(count >= 0 && (count == 0 || (params && grads && n)), "sgd_many: null argument");
+  FLHIP_REQUIRE(momentum == 0.0 || velocities, "sgd_many: momentum needs velocity buffers");
+  hipStream_t s = as_stream(stream);
+  SgdMany a{};
+  uint64_t pieces = 0;
+  auto flush = [&]() {
+    if (a.count == 0) return;
+    a.first[a.count] = (unsigned)pieces;
+    a.lr = (float)lr; a.mu = (float)momentum; a.wd = (float)weight_decay; a.nesterov = nesterov != 0;
+    const dim3 grid((unsigned)pieces), block(256);
+    by_dtype(dtype, [&](auto* t_) { hipLaunchKernelGGL((sgd_many_kernel<FLHIP_T_OF(t_)>), grid, block, 0, s, a); });
+    a = SgdMany{};
+    pieces = 0;
+  };
+  for (int i = 0; i < count; ++i) {
+    if (n[i] == 0) continue;
+    FLHIP_REQUIRE(params[i] && grads[i] && (momentum == 0.0 || velocities[i]), "sgd_many: null pointer");
+    FLHIP_REQUIRE(n[i] < (1ull << 40), "sgd_many: tensor too large");
+    const uint64_t mine = (n[i] + 2047) / 2048;
+    if (a.count == SGD_MAX || pieces + mine > convert_many_max_pieces()) flush();
+    a.w[a.count] = params[i];
+    a.g[a.count] = grads[i];
+    a.v[a.count] = momentum != 0.0 ? velocities[i] : nullptr;
+    a.n[a.count] = n[i];
+    a.first[a.count] = (unsigned)pieces;
+    pieces += mine;
+    ++a.count;
+  }
+  flush();
+  return check_launch("sgd_many");
 }
 
 extern "C" int flhip_convert_many_launches(const size_t* n, int count, int* launch_of) {

@@ -5,8 +5,9 @@
 // run, the device time per operation class (HIP events around every operation of the
 // host layer) with the idle gaps between operations.
 //
-// usage: flhip_step_bench resnet50|speech [batch] [steps] [warmup] [f32|bf16] [unfused]
-// ("unfused": BatchNorm, residual add and ReLU as three operations, the reference's composition)
+// usage: flhip_step_bench resnet50|speech [batch] [steps] [warmup] [f32|bf16] [unfused|fused] [sgd]
+// ("unfused": BatchNorm, residual add and ReLU as three operations, the reference's composition; "sgd": the step ends
+// with fl::SGDOptimizer::step - momentum 0.9, weight decay 1e-4 - on the ResNet's parameters)
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -16,6 +17,7 @@
 #include <vector>
 
 #include "OpObserver.h"
+#include "Optimizers.h"
 #include "Resnet.h"
 
 using namespace fl;
@@ -53,6 +55,7 @@ int main(int argc, char** argv) {
     const int warmup = argc > 4 ? std::atoi(argv[4]) : 3;
     const bool half = argc > 5 && std::string(argv[5]) == "bf16";
     const bool unfused = argc > 6 && std::string(argv[6]) == "unfused";
+    const bool sgd = argc > 7 && std::string(argv[7]) == "sgd";
     pkg::vision::setFusedBatchNormRelu(!unfused);
     detail::setFusedGradAdd(!unfused);
     setSeed(3);
@@ -61,6 +64,7 @@ int main(int argc, char** argv) {
     // filled on the device, the loss is read back once after the timed loop), so the host runs ahead of the kernels.
     std::function<Tensor()> step;
     std::shared_ptr<Sequential> net;
+    std::shared_ptr<SGDOptimizer> opt;
     std::vector<Conv2D> convs;
     std::vector<BatchNorm> bns;
     Variable in, target, gradOut;
@@ -73,11 +77,13 @@ int main(int argc, char** argv) {
       std::mt19937 gen(5);
       for (int i = 0; i < B; ++i) labels[i] = (int32_t)(gen() % 1000);
       target = Variable(Tensor::fromHost(Shape({B}), dtype::s32, labels.data()), false);
+      if (sgd) opt = std::make_shared<SGDOptimizer>(net->params(), 0.01f, 0.9f, 1e-4f);
       step = [&]() {
         net->zeroGrad();
         Variable out = logSoftmax(net->forward(in), 0);
         Variable loss = categoricalCrossEntropy(out, target);
         loss.backward(Variable(Tensor::full({1}, 1., dtype::f32), false));
+        if (opt) opt->step();
         return loss.tensor();
       };
     } else if (model == "speech") {
@@ -128,10 +134,10 @@ int main(int argc, char** argv) {
       c.calls += kv.second.calls / psteps;
     }
 
-    std::printf("{\"model\": \"%s\", \"batch\": %d, \"dtype\": \"%s\", \"fused_bn_relu\": %s, \"steps\": %d, \"warmup\": %d, \"ms_per_step\": %.4f, "
+    std::printf("{\"model\": \"%s\", \"batch\": %d, \"dtype\": \"%s\", \"fused_bn_relu\": %s, \"optimizer\": \"%s\", \"steps\": %d, \"warmup\": %d, \"ms_per_step\": %.4f, "
                 "\"samples_per_s\": %.1f, \"loss\": %.5f, \"conv_gflop_per_step\": %.2f, \"device_cache_mb\": %.1f, "
                 "\"breakdown_ms\": {",
-                model.c_str(), B, half ? "bf16" : "f32", unfused ? "false" : "true", steps, warmup, ms, B / ms * 1e3, loss, flop / 1e9,
+                model.c_str(), B, half ? "bf16" : "f32", unfused ? "false" : "true", opt ? "sgd momentum 0.9 weight decay 1e-4" : "none", steps, warmup, ms, B / ms * 1e3, loss, flop / 1e9,
                 deviceCacheBytes() / 1e6);
     bool first = true;
     for (const auto& kv : classes) {

@@ -544,6 +544,22 @@ def padding_backward(grad_output, dims, before, after):
     return dx
 
 
+def sgd_step(params, grads, velocities, lr, momentum=0.0, weight_decay=0.0, nesterov=False):
+    """fl::SGDOptimizer::step (optim/SGDOptimizer.cpp:38-68) over lists of tensors of one dtype, in place."""
+    ps = [_dev(p, "param") for p in params]
+    gs = [_dev(g, "grad") for g in grads]
+    vs = [_dev(v, "velocity") for v in velocities] if velocities is not None else None
+    n = len(ps)
+    if n == 0:
+        return
+    pa = (C.c_void_p * n)(*[p.data_ptr() for p in ps])
+    ga = (C.c_void_p * n)(*[g.data_ptr() for g in gs])
+    va = (C.c_void_p * n)(*[v.data_ptr() for v in vs]) if vs is not None else None
+    cnt = (C.c_size_t * n)(*[p.numel() for p in ps])
+    capi.check(capi.lib().flhip_sgd_many(pa, ga, va, cnt, n, float(lr), float(momentum), float(weight_decay),
+                                         int(bool(nesterov)), _dtype_tag(ps[0]), _stream()))
+
+
 def linear(input, weight, bias=None):
     """fl::linear (Functions.cpp:1255-1309): input [..., in] (Flashlight [in, ...]), weight
     torch [in, out] (Flashlight [out, in]), bias [out] or None -> [..., out]."""

@@ -116,7 +116,7 @@ const char* flhip_last_error(void);
  * refuse to run when flhip_version() / 100 differs from FLHIP_VERSION / 100 (a layout change).
  * 200: flhip_rnn_desc gained dropout, seed_lo, seed_hi; flhip_bn_workspace_bytes never returns less
  * than 32 bytes per feature.  202: the *_plan entry points and FLHIP_DECLINED.  203: FLHIP_F16.  204: flhip_act_fwd / _bwd, flhip_glu_fwd / _bwd,
- * flhip_dropout, flhip_rownorm, flhip_weightnorm_fwd / _bwd, flhip_pad_fwd / _bwd. */
+ * flhip_dropout, flhip_rownorm, flhip_weightnorm_fwd / _bwd, flhip_pad_fwd / _bwd, flhip_sgd_many. */
 #define FLHIP_VERSION 204
 int flhip_version(void);
 const char* flhip_arch(void);
@@ -341,6 +341,13 @@ int flhip_convert_many_launches(const size_t* n, int count, int* launch_of);
  * default running statistics (onednn/BatchNorm.cpp:116-122), enqueued like every other
  * kernel (no host buffer, no synchronisation; safe under graph capture). */
 int flhip_fill(void* dst, double value, size_t n, int dtype, void* stream);
+
+/* fl::SGDOptimizer::step (flashlight/fl/optim/SGDOptimizer.cpp:38-68) over `count` parameter tensors of one dtype,
+ * in place, one launch per 48 tensors: g = grad + weight_decay w; with momentum != 0, v = momentum v + g (stored) and
+ * g = nesterov ? g + momentum v : v; w = w - lr g.  velocities may be NULL when momentum == 0. */
+int flhip_sgd_many(void* const* params, const void* const* grads, void* const* velocities, const size_t* n,
+                   int count, double lr, double momentum, double weight_decay, int nesterov, int dtype,
+                   void* stream);
 
 /* out = a + b over n elements of `dtype` (out may alias a or b): the gradient
  * accumulation of Variable::addGrad (flashlight/fl/autograd/Variable.cpp:185-218). */

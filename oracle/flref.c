@@ -530,6 +530,20 @@ void flref_pad_bwd(const int64_t* dims, const int32_t* before, const int32_t* af
               dy[(a + before[0]) + od[0] * ((b + before[1]) + od[1] * ((c + before[2]) + od[2] * (d + before[3])))];
 }
 
+/* fl::SGDOptimizer::step (flashlight/fl/optim/SGDOptimizer.cpp:38-68) on one tensor, in place, in double with the
+ * stored values rounded to float */
+void flref_sgd(int64_t n, float* w, const float* g, float* v, double lr, double mu, double wd, int nesterov) {
+  for (int64_t i = 0; i < n; ++i) {
+    double gi = g[i];
+    if (wd != 0.0) gi = gi + wd * w[i];
+    if (mu != 0.0) {
+      v[i] = (float)(mu * v[i] + gi);
+      gi = nesterov ? gi + (double)v[i] * mu : (double)v[i];
+    }
+    w[i] = (float)((double)w[i] - lr * gi);
+  }
+}
+
 /* fl::matmul / matmulTN / matmulNT as used by fl::linear (:1264-1265, 1292-1301) */
 void flref_matmul(int M, int N, int K, int ta, int tb, const float* A, const float* B,
                   const float* bias, float* C) {

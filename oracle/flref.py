@@ -272,6 +272,16 @@ def pad_bwd(dy, dims, before, after):
     return dx
 
 
+def sgd(w, g, v, lr, mu, wd, nesterov):
+    """One SGD step; returns (w, v) as new arrays (v None when mu == 0)."""
+    w = _f32(w).copy()
+    g = _f32(g)
+    v = _f32(v).copy() if v is not None else None
+    lib().flref_sgd(_i64(w.size), _p(w), _p(g), _p(v) if v is not None else None, C.c_double(lr), C.c_double(mu),
+                    C.c_double(wd), C.c_int(int(nesterov)))
+    return w, v
+
+
 def relu_bwd(dy, x):
     dy, x = _f32(dy), _f32(x)
     dx = np.empty_like(x)

@@ -26,6 +26,7 @@
 
 #include "Functions.h"
 #include "Modules.h"
+#include "Optimizers.h"
 #include "SequentialBuilder.h"
 #include "HipAutogradExtension.h"
 #include "OpObserver.h"
@@ -1303,6 +1304,68 @@ static void testActivationModules() {
   }
 }
 
+// fl::SGDOptimizer (optim/SGDOptimizer.cpp:38-68): one step against the checker for every variant, parameters without
+// a gradient left alone, and a small network trained on one batch until its loss has fallen
+static void testSgd() {
+  std::printf("SGD optimizer\n");
+  struct Cfg { float mu, wd; bool nest; const char* name; };
+  for (const Cfg& c : {Cfg{0.f, 0.f, false, "SGD"}, Cfg{0.9f, 0.f, false, "SGD (momentum=0.9)"},
+                       Cfg{0.9f, 0.01f, false, "SGD (weight decay=0.01) (momentum=0.9)"},
+                       Cfg{0.8f, 0.005f, true, "SGD (weight decay=0.005) (Nesterov momentum=0.8)"}}) {
+    auto w0 = randn(3000, 800), w1 = randn(17, 801), w2 = randn(5, 802);
+    Variable p0(Tensor::fromVector({30, 100}, w0), true), p1(Tensor::fromVector({17}, w1), true),
+        p2(Tensor::fromVector({5}, w2), true);
+    SGDOptimizer opt({p0, p1, p2}, 0.05f, c.mu, c.wd, c.nest);
+    CHECK(opt.prettyString() == c.name);
+    std::vector<float> v0(w0.size(), 0.f), v1(w1.size(), 0.f);
+    for (int step = 0; step < 3; ++step) {
+      auto g0 = randn(w0.size(), 810 + step), g1 = randn(w1.size(), 820 + step);
+      opt.zeroGrad();
+      p0.addGrad(Variable(Tensor::fromVector({30, 100}, g0), false));
+      p1.addGrad(Variable(Tensor::fromVector({17}, g1), false));     // p2 gets no gradient
+      opt.step();
+      flref_sgd((int64_t)w0.size(), w0.data(), g0.data(), v0.data(), 0.05, c.mu, c.wd, c.nest);
+      flref_sgd((int64_t)w1.size(), w1.data(), g1.data(), v1.data(), 0.05, c.mu, c.wd, c.nest);
+      CHECK(relL2(hostOf(p0), w0) <= 2e-6 && relL2(hostOf(p1), w1) <= 2e-6 && hostOf(p2) == w2);
+    }
+  }
+  // training: a two-layer convolutional classifier on one batch of separable data
+  {
+    using fl::pkg::runtime::buildSequentialModule;
+    setSeed(51);
+    auto net = buildSequentialModule(std::vector<std::string>{"C2 1 8 3 3 1 1 -1 -1", "BN 8 2", "R", "M 2 2 2 2", "C2 8 16 3 3 1 1 -1 -1",
+                                                              "R", "M 2 2 2 2", "V 64 -1", "L 64 4", "LSM 0"}, 1, 4);
+    const int B = 32;
+    std::vector<float> x((size_t)8 * 8 * B);
+    std::vector<int32_t> labels(B);
+    std::mt19937 gen(52);
+    std::normal_distribution<float> nd(0.f, 0.3f);
+    for (int b = 0; b < B; ++b) {
+      labels[b] = b % 4;
+      for (int i = 0; i < 64; ++i) {
+        const int r = i / 8, cidx = i % 8;
+        const bool on = labels[b] == 0 ? r < 4 : labels[b] == 1 ? r >= 4 : labels[b] == 2 ? cidx < 4 : cidx >= 4;
+        x[(size_t)b * 64 + i] = (on ? 1.f : -1.f) + nd(gen);
+      }
+    }
+    Variable in(Tensor::fromVector({8, 8, 1, B}, x), false);
+    Variable target(Tensor::fromHost(Shape({B}), dtype::s32, labels.data()), false);
+    SGDOptimizer opt(net->params(), 0.1f, 0.9f, 1e-4f);
+    float first = 0.f, last = 0.f;
+    for (int step = 0; step < 30; ++step) {
+      opt.zeroGrad();
+      Variable loss = categoricalCrossEntropy(net->forward(in), target);
+      loss.backward(Variable(Tensor::full({1}, 1., dtype::f32), false));
+      opt.step();
+      const float l = hostOf(loss)[0];
+      if (step == 0) first = l;
+      last = l;
+    }
+    std::printf("  loss %.4f -> %.4f over 30 steps\n", first, last);
+    CHECK(first > 1.0f && last < 0.1f * first);
+  }
+}
+
 // rnn / rnnBackward through the closure and the RNN module (flashlight/fl/test/autograd/
 // AutogradRnnTest.cpp:24-90 uses 2 layers, hidden 2, input 2, bidirectional; here against
 // the CPU checker instead of finite differences)
@@ -1571,6 +1634,7 @@ int main() {
     testRnn();
     testArchBuilder();
     testActivationModules();
+    testSgd();
     testModuleShapesAndBatching();
     testInit();
     testDynamicBenchmark();

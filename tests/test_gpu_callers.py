@@ -414,3 +414,28 @@ def test_padding(dims, before, after, dtype):
     assert np.array_equal(host(ops.padding(dev(x, dtype), dims, before, after, 0.25)), y_ref)
     dy = _round(rng.standard_normal(y_ref.size).astype(np.float32), dtype)
     assert np.array_equal(host(ops.padding_backward(dev(dy, dtype), dims, before, after)), flref.pad_bwd(dy, dims, before, after))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("mu,wd,nesterov", [(0.0, 0.0, False), (0.9, 1e-2, False), (0.8, 5e-3, True)])
+def test_sgd_many(mu, wd, nesterov, dtype):
+    # several tensors (more than one launch holds), three steps; fp32 against the checker step by step
+    rng = np.random.default_rng(120)
+    sizes = [1, 5, 2048, 2049, 70001] + [int(rng.integers(1, 3000)) for _ in range(60)]
+    ws = [_round(rng.standard_normal(n).astype(np.float32), dtype) for n in sizes]
+    vs = [np.zeros(n, np.float32) for n in sizes] if mu else None
+    wd_ = [dev(w, dtype) for w in ws]
+    vd_ = [dev(v, dtype) for v in vs] if mu else None
+    for step in range(3):
+        gs = [_round(rng.standard_normal(n).astype(np.float32), dtype) for n in sizes]
+        ops.sgd_step(wd_, [dev(g, dtype) for g in gs], vd_, 0.05, mu, wd, nesterov)
+        for i in range(len(sizes)):
+            ws[i], nv = flref.sgd(ws[i], gs[i], vs[i] if mu else None, 0.05, mu, wd, nesterov)
+            if mu:
+                vs[i] = _round(nv, dtype)
+            ws[i] = _round(ws[i], dtype)
+        tol = 2e-6 if dtype == torch.float32 else 8e-3
+        for i in range(len(sizes)):
+            assert rel_l2(host(wd_[i]), ws[i]) <= tol, (step, i, sizes[i])
+            if mu:
+                assert rel_l2(host(vd_[i]), vs[i]) <= tol, (step, i)

@@ -291,3 +291,19 @@ def test_padding_against_numpy(dims, before, after):
     dy = rng.standard_normal(ref.shape).astype(np.float32)
     sl = tuple(slice(b, b + n) for (b, _), n in zip(widths, x.shape))
     assert np.array_equal(flref.pad_bwd(dy, dims, before, after).reshape(x.shape), dy[sl])
+
+
+@pytest.mark.parametrize("mu,wd,nesterov", [(0.0, 0.0, False), (0.9, 0.0, False), (0.9, 1e-2, False), (0.8, 5e-3, True), (0.0, 1e-2, False)])
+def test_sgd_against_torch_optim(mu, wd, nesterov):
+    # optim/SGDOptimizer.cpp:38-68 is torch.optim.SGD's update (dampening 0): three steps with fresh gradients
+    rng = np.random.default_rng(340)
+    w = rng.standard_normal(500).astype(np.float32)
+    tw = torch.nn.Parameter(torch.from_numpy(w.astype(np.float64)))
+    opt = torch.optim.SGD([tw], lr=0.05, momentum=mu, weight_decay=wd, nesterov=nesterov)
+    v = np.zeros_like(w) if mu else None
+    for step in range(3):
+        g = rng.standard_normal(500).astype(np.float32)
+        tw.grad = torch.from_numpy(g.astype(np.float64))
+        opt.step()
+        w, v = flref.sgd(w, g, v, 0.05, mu, wd, nesterov)
+        assert rel_l2(w, tw.detach().numpy()) <= 1e-6
