@@ -86,6 +86,8 @@ SYMBOLS = {
     "flhip_glu_bwd": (C.c_int, [_VP, _VP, _VP, C.c_int64, C.c_int64, C.c_int, _VP]),
     "flhip_sgd_many": (C.c_int, [C.POINTER(_VP), C.POINTER(_VP), C.POINTER(_VP), C.POINTER(_SZ), C.c_int, C.c_double,
                                  C.c_double, C.c_double, C.c_int, C.c_int, _VP]),
+    "flhip_adam_many": (C.c_int, [C.POINTER(_VP), C.POINTER(_VP), C.POINTER(_VP), C.POINTER(_VP), C.POINTER(_SZ), C.c_int,
+                                  C.c_double, C.c_double, C.c_double, C.c_double, C.c_double, C.c_int64, C.c_int, _VP]),
     "flhip_dropout": (C.c_int, [_VP, _VP, _SZ, C.c_double, C.c_uint32, C.c_uint32, C.c_int, _VP]),
     "flhip_rownorm": (C.c_int, [_VP, _VP, C.c_int64, C.c_int64, C.c_int, C.c_int, _VP]),
     "flhip_weightnorm_fwd": (C.c_int, [_VP, _VP, _VP, C.c_int64, C.c_int64, C.c_int, C.c_int, _VP]),

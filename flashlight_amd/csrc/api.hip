@@ -4,6 +4,8 @@
 
 #include <mutex>
 
+#include <cmath>
+
 #include "common.h"
 
 namespace flhip {
@@ -196,6 +198,47 @@ __global__ void __launch_bounds__(256) sgd_many_kernel(SgdMany a) {
   }
 }
 
+// fl::AdamOptimizer::step (flashlight/fl/optim/AdamOptimizer.cpp:45-79) the same way: w = w - wd lr w (decoupled decay),
+// m = b1 m + (1 - b1) g, v = b2 v + (1 - b2) g g (both stored), w = w - clr m / (sqrt(v) + eps) with the
+// bias-corrected rate clr = lr sqrt(1 - b2^t) / (1 - b1^t) computed on the host.
+constexpr int ADAM_MAX = 32;
+struct AdamMany {
+  void* w[ADAM_MAX];
+  const void* g[ADAM_MAX];
+  void* m[ADAM_MAX];
+  void* v[ADAM_MAX];
+  unsigned first[ADAM_MAX + 1];
+  unsigned long long n[ADAM_MAX];
+  int count;
+  float b1, b2, eps, decay, clr;      // decay = wd * lr
+};
+template <typename T>
+__global__ void __launch_bounds__(256) adam_many_kernel(AdamMany a) {
+  int lo = 0, hi = a.count;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (a.first[mid] <= blockIdx.x) lo = mid; else hi = mid;
+  }
+  T* w = static_cast<T*>(a.w[lo]);
+  const T* g = static_cast<const T*>(a.g[lo]);
+  T* m = static_cast<T*>(a.m[lo]);
+  T* v = static_cast<T*>(a.v[lo]);
+  const size_t base = (size_t)(blockIdx.x - a.first[lo]) * 2048;
+  const size_t n = a.n[lo];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const size_t i = base + (size_t)k * 256 + threadIdx.x;
+    if (i < n) {
+      float wi = ld(w, i);
+      const float gi = ld(g, i);
+      if (a.decay != 0.f) wi = wi - a.decay * wi;
+      st(m, i, a.b1 * ld(m, i) + (1.f - a.b1) * gi);
+      st(v, i, a.b2 * ld(v, i) + (1.f - a.b2) * gi * gi);
+      st(w, i, wi - (a.clr * ld(m, i)) / (sqrtf(ld(v, i)) + a.eps));
+    }
+  }
+}
+
 template <typename D>
 __global__ void __launch_bounds__(256) fill_kernel(D* __restrict__ dst, float value, size_t n) {
   const size_t stride = (size_t)gridDim.x * 256;
@@ -366,6 +409,46 @@ extern "C" int flhip_sgd_many(void* const* params, const void* const* grads, voi
   }
   flush();
   return check_launch("sgd_many");
+}
+
+extern "C" int flhip_adam_many(void* const* params, const void* const* grads, void* const* first, void* const* second,
+                               const size_t* n, int count, double lr, double beta1, double beta2, double epsilon,
+                               double weight_decay, int64_t step, int dtype, void* stream) {
+  FLHIP_REQUIRE(dtype_ok(dtype), "adam_many: unknown dtype");
+  FLHIP_REQUIRE(count >= 0 && (count == 0 || (params && grads && first && second && n)), "adam_many: null argument");
+  FLHIP_REQUIRE(step >= 1, "adam_many: steps count from 1");
+  hipStream_t s = as_stream(stream);
+  // AdamOptimizer.cpp:47-49, in float like the reference
+  const float cb1 = 1.f - std::pow((float)beta1, (float)step), cb2 = 1.f - std::pow((float)beta2, (float)step);
+  const float clr = (float)lr * std::sqrt(cb2) / cb1;
+  AdamMany a{};
+  uint64_t pieces = 0;
+  auto flush = [&]() {
+    if (a.count == 0) return;
+    a.first[a.count] = (unsigned)pieces;
+    a.b1 = (float)beta1; a.b2 = (float)beta2; a.eps = (float)epsilon; a.decay = (float)(weight_decay * lr); a.clr = clr;
+    const dim3 grid((unsigned)pieces), block(256);
+    by_dtype(dtype, [&](auto* t_) { hipLaunchKernelGGL((adam_many_kernel<FLHIP_T_OF(t_)>), grid, block, 0, s, a); });
+    a = AdamMany{};
+    pieces = 0;
+  };
+  for (int i = 0; i < count; ++i) {
+    if (n[i] == 0) continue;
+    FLHIP_REQUIRE(params[i] && grads[i] && first[i] && second[i], "adam_many: null pointer");
+    FLHIP_REQUIRE(n[i] < (1ull << 40), "adam_many: tensor too large");
+    const uint64_t mine = (n[i] + 2047) / 2048;
+    if (a.count == ADAM_MAX || pieces + mine > convert_many_max_pieces()) flush();
+    a.w[a.count] = params[i];
+    a.g[a.count] = grads[i];
+    a.m[a.count] = first[i];
+    a.v[a.count] = second[i];
+    a.n[a.count] = n[i];
+    a.first[a.count] = (unsigned)pieces;
+    pieces += mine;
+    ++a.count;
+  }
+  flush();
+  return check_launch("adam_many");
 }
 
 extern "C" int flhip_convert_many_launches(const size_t* n, int count, int* launch_of) {

@@ -1,7 +1,8 @@
 // First-order optimizers over the host layer's Variables: the interface of
 // flashlight/fl/optim/Optimizers.h:25-75 and fl::SGDOptimizer (optim/SGDOptimizer.{h,cpp}): stochastic gradient
-// descent with weight decay, momentum and Nesterov momentum, the update of every parameter tensor of a step in one
-// launch per 48 tensors (flhip_sgd_many) instead of five tensor expressions per parameter.
+// descent with weight decay, momentum and Nesterov momentum, and fl::AdamOptimizer; the update of every parameter tensor
+// of a step in one launch per 48 / 32 tensors (flhip_sgd_many, flhip_adam_many) instead of several tensor expressions per
+// parameter.
 #pragma once
 
 #include <string>
@@ -39,6 +40,20 @@ class SGDOptimizer : public FirstOrderOptimizer {
   bool useNesterov_;
   float mu_, wd_;
   std::vector<Tensor> velocities_;
+};
+
+// fl::AdamOptimizer (optim/AdamOptimizer.{h,cpp}): Adam with decoupled weight decay and the bias-corrected rate
+class AdamOptimizer : public FirstOrderOptimizer {
+ public:
+  AdamOptimizer(const std::vector<Variable>& parameters, float learningRate, float beta1 = 0.9f, float beta2 = 0.999f,
+                float epsilon = 1e-8f, float weightDecay = 0);
+  void step() override;
+  std::string prettyString() const override;
+
+ private:
+  float beta1_, beta2_, eps_, wd_;
+  int count_ = 0;
+  std::vector<Tensor> biasedFirst_, biasedSecond_;
 };
 
 }  // namespace fl

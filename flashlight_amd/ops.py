@@ -560,6 +560,18 @@ def sgd_step(params, grads, velocities, lr, momentum=0.0, weight_decay=0.0, nest
                                          int(bool(nesterov)), _dtype_tag(ps[0]), _stream()))
 
 
+def adam_step(params, grads, first, second, lr, beta1, beta2, epsilon, weight_decay, step):
+    """fl::AdamOptimizer::step (optim/AdamOptimizer.cpp:45-79) over lists of tensors of one dtype, in place."""
+    lists = [[_dev(t, "tensor") for t in l] for l in (params, grads, first, second)]
+    n = len(lists[0])
+    if n == 0:
+        return
+    arrs = [(C.c_void_p * n)(*[t.data_ptr() for t in l]) for l in lists]
+    cnt = (C.c_size_t * n)(*[t.numel() for t in lists[0]])
+    capi.check(capi.lib().flhip_adam_many(arrs[0], arrs[1], arrs[2], arrs[3], cnt, n, float(lr), float(beta1), float(beta2),
+                                          float(epsilon), float(weight_decay), int(step), _dtype_tag(lists[0][0]), _stream()))
+
+
 def linear(input, weight, bias=None):
     """fl::linear (Functions.cpp:1255-1309): input [..., in] (Flashlight [in, ...]), weight
     torch [in, out] (Flashlight [out, in]), bias [out] or None -> [..., out]."""

@@ -116,7 +116,7 @@ const char* flhip_last_error(void);
  * refuse to run when flhip_version() / 100 differs from FLHIP_VERSION / 100 (a layout change).
  * 200: flhip_rnn_desc gained dropout, seed_lo, seed_hi; flhip_bn_workspace_bytes never returns less
  * than 32 bytes per feature.  202: the *_plan entry points and FLHIP_DECLINED.  203: FLHIP_F16.  204: flhip_act_fwd / _bwd, flhip_glu_fwd / _bwd,
- * flhip_dropout, flhip_rownorm, flhip_weightnorm_fwd / _bwd, flhip_pad_fwd / _bwd, flhip_sgd_many. */
+ * flhip_dropout, flhip_rownorm, flhip_weightnorm_fwd / _bwd, flhip_pad_fwd / _bwd, flhip_sgd_many, flhip_adam_many. */
 #define FLHIP_VERSION 204
 int flhip_version(void);
 const char* flhip_arch(void);
@@ -348,6 +348,13 @@ int flhip_fill(void* dst, double value, size_t n, int dtype, void* stream);
 int flhip_sgd_many(void* const* params, const void* const* grads, void* const* velocities, const size_t* n,
                    int count, double lr, double momentum, double weight_decay, int nesterov, int dtype,
                    void* stream);
+
+/* fl::AdamOptimizer::step (flashlight/fl/optim/AdamOptimizer.cpp:45-79), in place, one launch per 32 tensors:
+ * w = w - weight_decay lr w; first = beta1 first + (1 - beta1) g; second = beta2 second + (1 - beta2) g g;
+ * w = w - clr first / (sqrt(second) + epsilon), clr = lr sqrt(1 - beta2^step) / (1 - beta1^step); step counts from 1. */
+int flhip_adam_many(void* const* params, const void* const* grads, void* const* first, void* const* second,
+                    const size_t* n, int count, double lr, double beta1, double beta2, double epsilon,
+                    double weight_decay, int64_t step, int dtype, void* stream);
 
 /* out = a + b over n elements of `dtype` (out may alias a or b): the gradient
  * accumulation of Variable::addGrad (flashlight/fl/autograd/Variable.cpp:185-218). */

@@ -544,6 +544,21 @@ void flref_sgd(int64_t n, float* w, const float* g, float* v, double lr, double 
   }
 }
 
+/* fl::AdamOptimizer::step (optim/AdamOptimizer.cpp:45-79) on one tensor, in place; the corrected rate in float as there */
+void flref_adam(int64_t n, float* w, const float* g, float* m, float* v, double lr, double b1, double b2, double eps,
+                double wd, int64_t step) {
+  const float cb1 = 1.f - powf((float)b1, (float)step), cb2 = 1.f - powf((float)b2, (float)step);
+  const double clr = (float)lr * sqrtf(cb2) / cb1;
+  for (int64_t i = 0; i < n; ++i) {
+    double wi = w[i];
+    const double gi = g[i];
+    if (wd != 0.0) wi = wi - wd * lr * wi;
+    m[i] = (float)(b1 * m[i] + (1.0 - b1) * gi);
+    v[i] = (float)(b2 * v[i] + (1.0 - b2) * gi * gi);
+    w[i] = (float)(wi - clr * m[i] / (sqrt((double)v[i]) + eps));
+  }
+}
+
 /* fl::matmul / matmulTN / matmulNT as used by fl::linear (:1264-1265, 1292-1301) */
 void flref_matmul(int M, int N, int K, int ta, int tb, const float* A, const float* B,
                   const float* bias, float* C) {

@@ -120,6 +120,9 @@ void flref_pad_fwd(const int64_t* dims, const int32_t* before, const int32_t* af
 void flref_pad_bwd(const int64_t* dims, const int32_t* before, const int32_t* after, const float* dy, float* dx);
 /* SGD with weight decay, momentum and Nesterov momentum (optim/SGDOptimizer.cpp:38-68), in place; v may be NULL when mu == 0 */
 void flref_sgd(int64_t n, float* w, const float* g, float* v, double lr, double mu, double wd, int nesterov);
+/* Adam with decoupled weight decay (optim/AdamOptimizer.cpp:45-79), in place; step counts from 1 */
+void flref_adam(int64_t n, float* w, const float* g, float* m, float* v, double lr, double b1, double b2, double eps,
+                double wd, int64_t step);
 /* C (M x N) = op(A) op(B) + bias[m]; ta: A stored K x M, tb: B stored N x K; double
  * accumulate.  fl::linear (:1255-1309) = (W, X), backward (W^T, dY) and (dY, X^T). */
 void flref_matmul(int M, int N, int K, int ta, int tb, const float* A, const float* B,

@@ -282,6 +282,15 @@ def sgd(w, g, v, lr, mu, wd, nesterov):
     return w, v
 
 
+def adam(w, g, m, v, lr, b1, b2, eps, wd, step):
+    """One Adam step; returns new (w, m, v)."""
+    w, m, v = _f32(w).copy(), _f32(m).copy(), _f32(v).copy()
+    g = _f32(g)
+    lib().flref_adam(_i64(w.size), _p(w), _p(g), _p(m), _p(v), C.c_double(lr), C.c_double(b1), C.c_double(b2),
+                     C.c_double(eps), C.c_double(wd), _i64(step))
+    return w, m, v
+
+
 def relu_bwd(dy, x):
     dy, x = _f32(dy), _f32(x)
     dx = np.empty_like(x)

@@ -1329,6 +1329,22 @@ static void testSgd() {
       CHECK(relL2(hostOf(p0), w0) <= 2e-6 && relL2(hostOf(p1), w1) <= 2e-6 && hostOf(p2) == w2);
     }
   }
+  // Adam (optim/AdamOptimizer.cpp:45-79): three steps against the checker, with and without decay
+  for (float wd : {0.f, 0.05f}) {
+    auto w0 = randn(3000, 830), w2 = randn(5, 832);
+    Variable p0(Tensor::fromVector({30, 100}, w0), true), p2(Tensor::fromVector({5}, w2), true);
+    AdamOptimizer opt({p0, p2}, 0.01f, 0.9f, 0.99f, 1e-6f, wd);
+    CHECK(opt.prettyString() == (wd != 0.f ? "Adam (weight decay=0.05)" : "Adam"));
+    std::vector<float> m0(w0.size(), 0.f), v0(w0.size(), 0.f);
+    for (int step = 1; step <= 3; ++step) {
+      auto g0 = randn(w0.size(), 840 + step);
+      opt.zeroGrad();
+      p0.addGrad(Variable(Tensor::fromVector({30, 100}, g0), false));
+      opt.step();
+      flref_adam((int64_t)w0.size(), w0.data(), g0.data(), m0.data(), v0.data(), 0.01f, 0.9f, 0.99f, 1e-6f, wd, step);
+      CHECK(relL2(hostOf(p0), w0) <= 2e-6 && hostOf(p2) == w2);
+    }
+  }
   // training: a two-layer convolutional classifier on one batch of separable data
   {
     using fl::pkg::runtime::buildSequentialModule;
@@ -1363,6 +1379,23 @@ static void testSgd() {
     }
     std::printf("  loss %.4f -> %.4f over 30 steps\n", first, last);
     CHECK(first > 1.0f && last < 0.1f * first);
+    // the same network trained with Adam from the same initial weights
+    setSeed(51);
+    auto net2 = buildSequentialModule(std::vector<std::string>{"C2 1 8 3 3 1 1 -1 -1", "BN 8 2", "R", "M 2 2 2 2", "C2 8 16 3 3 1 1 -1 -1",
+                                                               "R", "M 2 2 2 2", "V 64 -1", "L 64 4", "LSM 0"}, 1, 4);
+    AdamOptimizer adam(net2->params(), 0.01f);
+    float afirst = 0.f, alast = 0.f;
+    for (int step = 0; step < 30; ++step) {
+      adam.zeroGrad();
+      Variable loss = categoricalCrossEntropy(net2->forward(in), target);
+      loss.backward(Variable(Tensor::full({1}, 1., dtype::f32), false));
+      adam.step();
+      const float l = hostOf(loss)[0];
+      if (step == 0) afirst = l;
+      alast = l;
+    }
+    std::printf("  Adam: loss %.4f -> %.4f over 30 steps\n", afirst, alast);
+    CHECK(afirst == first && alast < 0.1f * afirst);
   }
 }
 

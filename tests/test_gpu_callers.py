@@ -439,3 +439,19 @@ def test_sgd_many(mu, wd, nesterov, dtype):
             assert rel_l2(host(wd_[i]), ws[i]) <= tol, (step, i, sizes[i])
             if mu:
                 assert rel_l2(host(vd_[i]), vs[i]) <= tol, (step, i)
+
+
+@pytest.mark.parametrize("wd", [0.0, 0.05])
+def test_adam_many(wd):
+    rng = np.random.default_rng(130)
+    sizes = [1, 7, 2048, 2049, 50001] + [int(rng.integers(1, 3000)) for _ in range(40)]
+    ws = [rng.standard_normal(n).astype(np.float32) for n in sizes]
+    ms = [np.zeros(n, np.float32) for n in sizes]
+    vs = [np.zeros(n, np.float32) for n in sizes]
+    wd_, md_, vd_ = [dev(w) for w in ws], [dev(m) for m in ms], [dev(v) for v in vs]
+    for t in range(1, 4):
+        gs = [rng.standard_normal(n).astype(np.float32) for n in sizes]
+        ops.adam_step(wd_, [dev(g) for g in gs], md_, vd_, 0.01, 0.9, 0.99, 1e-6, wd, t)
+        for i in range(len(sizes)):
+            ws[i], ms[i], vs[i] = flref.adam(ws[i], gs[i], ms[i], vs[i], 0.01, 0.9, 0.99, 1e-6, wd, t)
+            assert rel_l2(host(wd_[i]), ws[i]) <= 2e-6 and rel_l2(host(md_[i]), ms[i]) <= 2e-6 and rel_l2(host(vd_[i]), vs[i]) <= 2e-6

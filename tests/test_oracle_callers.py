@@ -307,3 +307,26 @@ def test_sgd_against_torch_optim(mu, wd, nesterov):
         opt.step()
         w, v = flref.sgd(w, g, v, 0.05, mu, wd, nesterov)
         assert rel_l2(w, tw.detach().numpy()) <= 1e-6
+
+
+@pytest.mark.parametrize("wd", [0.0, 0.05])
+def test_adam_against_torch_adamw(wd):
+    # optim/AdamOptimizer.cpp:45-79: decoupled decay and lr sqrt(1 - b2^t) / (1 - b1^t) m / (sqrt(v) + eps).  torch's
+    # AdamW divides by sqrt(v) / sqrt(1 - b2^t) + eps', the same update for eps' = eps / sqrt(1 - b2^t): each step is
+    # checked against one step of a torch optimizer given the state before it and that epsilon.
+    rng = np.random.default_rng(350)
+    lr, b1, b2, eps = 0.01, 0.9, 0.99, 1e-6
+    w = rng.standard_normal(400).astype(np.float32)
+    m, v = np.zeros_like(w), np.zeros_like(w)
+    for t in range(1, 5):
+        g = rng.standard_normal(400).astype(np.float32)
+        tw = torch.nn.Parameter(torch.from_numpy(w.astype(np.float64)))
+        opt = torch.optim.AdamW([tw], lr=lr, betas=(b1, b2), eps=eps / np.sqrt(1 - b2 ** t), weight_decay=wd)
+        opt.state[tw] = {"step": torch.tensor(float(t - 1)), "exp_avg": torch.from_numpy(m.astype(np.float64)),
+                         "exp_avg_sq": torch.from_numpy(v.astype(np.float64))}
+        tw.grad = torch.from_numpy(g.astype(np.float64))
+        opt.step()
+        w, m, v = flref.adam(w, g, m, v, lr, b1, b2, eps, wd, t)
+        assert rel_l2(w, tw.detach().numpy()) <= 2e-6
+        assert rel_l2(m, opt.state[tw]["exp_avg"].numpy()) <= 1e-6
+        assert rel_l2(v, opt.state[tw]["exp_avg_sq"].numpy()) <= 1e-6
