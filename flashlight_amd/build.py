@@ -13,7 +13,7 @@ LIB = os.path.join(LIBDIR, "libflhip.so")
 
 SOURCES = ["api.hip", "callers.hip", "rnn.hip", "pool2d.hip", "batchnorm.hip", "conv2d.hip", "conv2d_mfma_gather.hip", "conv2d_mfma_wgrad.hip",
            "conv2d_mfma_slab.hip", "conv2d_mfma_pointwise.hip", "conv2d_mfma_pointwise_bf16.hip", "conv2d_mfma_wgrad_slab.hip", "conv2d_mfma_slab_bf16.hip",
-           "conv2d_mfma_wgrad_slab_bf16.hip", "conv2d_mfma_strip_bf16.hip", "conv2d_mfma_first_bf16.hip",
+           "conv2d_mfma_wgrad_slab_bf16.hip", "conv2d_mfma_strip_bf16.hip", "conv2d_mfma_first_bf16.hip", "conv2d_mfma_cells.hip",
            "conv2d_mfma_pointwise_dma_bf16.hip", "conv2d_mfma_wgrad_dma_bf16.hip", "conv2d_mfma_tap1d.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

@@ -44,6 +44,7 @@ static bool apply_option(Options& o, const char* name, const char* v) {
       if (strstr(v, "pwdma")) m |= Options::SKIP_PWDMA;
       if (strstr(v, "wd32")) m |= Options::SKIP_WD32;
       if (strstr(v, "tap1d")) m |= Options::SKIP_TAP1D;
+      if (strstr(v, "cells")) m |= Options::SKIP_CELLS;
     }
     o.conv_skip = m;
     return true;

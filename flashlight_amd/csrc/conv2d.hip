@@ -271,11 +271,11 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
 // family: the caller times them instead of trusting the rules.
 static const char* const kBwdDataPlans[] = {"bf16 1x1, tiles loaded straight to LDS", "bf16 1x1 / gathered taps", "bf16 3x3 strip",
                                             "bf16 slab", "1x1 GEMM, split contraction", "1x1 GEMM", "slab", "tapped GEMM",
-                                            "gather", "direct", "one-row windows"};
+                                            "gather", "direct", "one-row windows", "stride-2 window over few channels, 2 x 2 cells"};
 static const char* const kBwdFilterPlans[] = {"bf16 3x3 rows straight to LDS, 32 x 32 tiles", "bf16 3x3 rows straight to LDS, 64 x 64 tiles",
                                               "bf16 1x1 / gathered taps", "bf16 first layer", "bf16 3x3 rows", "1x1 GEMM", "row slab",
                                               "tapped GEMM", "gather", "direct", "one-row windows"};
-constexpr int kNumPlans = 11;
+constexpr int kNumDataPlans = 12, kNumFilterPlans = 11;
 
 static int bwd_data_direct(const flhip_conv_desc* d, const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s) {
   const size_t total = (size_t)g.N * g.C * g.H * g.W;
@@ -298,7 +298,7 @@ static int bwd_data_impl(const flhip_conv_desc* d, const void* dy, const void* w
   if (rc != FLHIP_OK) return rc;
   hipStream_t s = as_stream(stream);
   if (plan >= 0) {
-    FLHIP_REQUIRE(plan < kNumPlans, "conv2d_bwd_data: unknown plan");
+    FLHIP_REQUIRE(plan < kNumDataPlans, "conv2d_bwd_data: unknown plan");
     const bool lo = d->dtype == FLHIP_BF16;
     int r = -1;
     switch (plan) {
@@ -312,13 +312,15 @@ static int bwd_data_impl(const flhip_conv_desc* d, const void* dy, const void* w
       case 7: r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes); break;
       case 8: r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s); break;
       case 9: r = bwd_data_direct(d, g, dy, w, dx, s); break;
-      default: r = mfma_tap1d_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
+      case 10: r = mfma_tap1d_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes); break;
+      default: r = mfma_cells_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     }
     return r < 0 ? FLHIP_DECLINED : r;
   }
   if (!force_direct()) {
     int r = -1;
     if (tap1d_on(d->dtype)) r = mfma_tap1d_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
+    if (r < 0 && !skip(Options::SKIP_CELLS)) r = mfma_cells_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pwd16_conv_bwd_data(g, dy, w, nullptr, dx, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
@@ -350,12 +352,14 @@ extern "C" int flhip_conv2d_bwd_data_plan(const flhip_conv_desc* d, const void* 
 }
 
 extern "C" int flhip_conv2d_plan_count(int pass) {
-  return pass == FLHIP_CONV_BWD_DATA || pass == FLHIP_CONV_BWD_FILTER ? kNumPlans : 0;
+  return pass == FLHIP_CONV_BWD_DATA ? kNumDataPlans : pass == FLHIP_CONV_BWD_FILTER ? kNumFilterPlans : 0;
 }
 
 extern "C" const char* flhip_conv2d_plan_name(int pass, int plan) {
-  if (plan < 0 || plan >= kNumPlans) return nullptr;
-  return pass == FLHIP_CONV_BWD_DATA ? kBwdDataPlans[plan] : pass == FLHIP_CONV_BWD_FILTER ? kBwdFilterPlans[plan] : nullptr;
+  if (plan < 0) return nullptr;
+  if (pass == FLHIP_CONV_BWD_DATA) return plan < kNumDataPlans ? kBwdDataPlans[plan] : nullptr;
+  if (pass == FLHIP_CONV_BWD_FILTER) return plan < kNumFilterPlans ? kBwdFilterPlans[plan] : nullptr;
+  return nullptr;
 }
 
 extern "C" int flhip_conv2d_bwd_data_add(const flhip_conv_desc* d, const void* dy, const void* w,
@@ -410,7 +414,7 @@ static int bwd_filter_impl(const flhip_conv_desc* d, const void* x, const void* 
   if (rc != FLHIP_OK) return rc;
   hipStream_t s = as_stream(stream);
   if (plan >= 0) {
-    FLHIP_REQUIRE(plan < kNumPlans, "conv2d_bwd_filter: unknown plan");
+    FLHIP_REQUIRE(plan < kNumFilterPlans, "conv2d_bwd_filter: unknown plan");
     if (plan == 9) return bwd_filter_direct(d, g, x, dy, dw, db, s);
     const size_t need = flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER);
     FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter: workspace too small");

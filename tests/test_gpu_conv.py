@@ -833,6 +833,65 @@ def test_full_size_properties(shape, dtype):
     assert not yi[:, nd:].any()
 
 
+# Backward-data of stride-2 windows over at most 4 input channels (the kernel that works on 2 x 2 cells of the input
+# gradient): the stem's 7x7 / pad 3 with 1 to 4 channels, windows of 3 to 8 rows and columns with every padding that
+# keeps the cell's window within 4 x 4, odd input sizes (a last cell of one row / column), planes narrower and wider
+# than a workgroup's columns (1, 2, 4, 7 column tiles and a ragged last one), more rows than one workgroup's 8,
+# filter counts of 4 to 96, the three storage types.  The last cases are outside it (5 input channels, a window whose
+# parities span 5 rows) and run on the other kernels.
+CELL_CASES = [
+    ((2, 3, 32, 32), (64, 3, 7, 7), (3, 3)),
+    ((1, 3, 70, 230), (32, 3, 7, 7), (3, 3)),
+    ((2, 1, 33, 47), (8, 1, 7, 7), (3, 3)),
+    ((2, 4, 40, 130), (16, 4, 7, 7), (3, 3)),
+    ((2, 2, 21, 19), (4, 2, 3, 3), (1, 1)),
+    ((2, 3, 30, 64), (12, 3, 5, 5), (2, 2)),
+    ((1, 3, 27, 100), (20, 3, 3, 5), (0, 1)),
+    ((2, 3, 24, 40), (96, 3, 6, 4), (2, 0)),
+    ((1, 2, 36, 36), (8, 2, 8, 8), (2, 4)),
+    ((2, 3, 19, 35), (8, 3, 7, 5), (0, 0)),
+    ((2, 3, 32, 32), (8, 3, 4, 7), (3, 1)),
+    ((2, 5, 32, 32), (8, 5, 7, 7), (3, 3)),
+    ((1, 3, 36, 36), (8, 3, 8, 8), (3, 3)),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", CELL_CASES)
+def test_backward_data_of_stride_two_windows_over_few_channels(case, dtype):
+    xs, ws, pd = case
+    rng = np.random.default_rng(83)
+    w = round_to((rng.standard_normal(ws) / np.sqrt(ws[1] * ws[2] * ws[3])).astype(np.float32), dtype)
+    d = flref.conv_desc(xs, ws, (2, 2), pd, (1, 1), 1)
+    ys = flref.conv2d_fwd(d, np.zeros(xs, np.float32), w, None).shape
+    dy = round_to(rng.standard_normal(ys).astype(np.float32), dtype)
+    ref = flref.conv2d_bwd_data(d, dy, w)
+    kw = dict(sx=2, sy=2, px=pd[1], py=pd[0])
+    got = fa.conv2d_backward_data(dev(dy, dtype), xs, dev(w, dtype), **kw)
+    from flashlight_amd import capi
+    capi.set_option("CONV_SKIP", "cells")
+    try:
+        other = fa.conv2d_backward_data(dev(dy, dtype), xs, dev(w, dtype), **kw)
+    finally:
+        capi.set_option("CONV_SKIP", None)
+    torch.cuda.synchronize()
+    tol = F32_TOL if dtype == torch.float32 else 4e-3
+    assert rel_l2(host(got), ref) <= tol, rel_l2(host(got), ref)
+    assert rel_l2(host(other), ref) <= tol
+    # a unit gradient at one position gives that filter's window back, flipped into place: exact in every storage type
+    dy1 = np.zeros(ys, np.float32)
+    k, oh, ow = ys[1] - 1, ys[2] // 2, ys[3] - 1
+    dy1[0, k, oh, ow] = 1.0
+    got1 = host(fa.conv2d_backward_data(dev(dy1, dtype), xs, dev(w, dtype), **kw))
+    exp = np.zeros(xs, np.float32)
+    for r in range(ws[2]):
+        for s in range(ws[3]):
+            ih, iw = 2 * oh - pd[0] + r, 2 * ow - pd[1] + s
+            if 0 <= ih < xs[2] and 0 <= iw < xs[3]:
+                exp[0, :, ih, iw] = w[k, :, r, s]
+    assert np.array_equal(got1, exp)
+
+
 # The backward passes with the kernel family named by the caller (flhip_conv2d_bwd_*_plan): every family either
 # declines a geometry (nothing is written) or produces the result within the stated tolerance; plan -1 is the
 # default entry point bit for bit; numbers outside the list are refused.
@@ -872,13 +931,13 @@ def test_backward_passes_by_plan(shape, dtype):
     S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     P = lambda t: C.c_void_p(t.data_ptr())
     nd = L.flhip_conv2d_plan_count(capi.CONV_BWD_DATA)
-    assert nd == L.flhip_conv2d_plan_count(capi.CONV_BWD_FILTER) >= 2 and L.flhip_conv2d_plan_count(capi.CONV_FWD) == 0
+    assert nd >= 2 and L.flhip_conv2d_plan_count(capi.CONV_BWD_FILTER) >= 2 and L.flhip_conv2d_plan_count(capi.CONV_FWD) == 0
     ran = {capi.CONV_BWD_DATA: [], capi.CONV_BWD_FILTER: []}
     for pas in (capi.CONV_BWD_DATA, capi.CONV_BWD_FILTER):
         nws = L.flhip_conv2d_workspace_bytes(C.byref(cd), pas)
         ws = torch.empty(max(nws, 16), dtype=torch.uint8, device="cuda")
         results = {}
-        for plan in range(-1, nd):
+        for plan in range(-1, L.flhip_conv2d_plan_count(pas)):
             if pas == capi.CONV_BWD_DATA:
                 out = torch.full(xs, 7.0, device="cuda", dtype=dtype)
                 rc = L.flhip_conv2d_bwd_data_plan(C.byref(cd), P(dyd), P(wd), P(out), P(ws), nws, plan, S)
