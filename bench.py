@@ -490,7 +490,6 @@ def plan_sweep(a, fa, torch, tdt):
         return best
 
     layers = RESNET50_LAYERS if a.plans == "resnet50" else SPEECH_LAYERS
-    nplans = L.flhip_conv2d_plan_count(capi.CONV_BWD_DATA)
     print("| input NxCxHxW | K | window | stride | pass | default rule us | fastest plan | us | default / fastest |")
     print("|---|---|---|---|---|---|---|---|---|")
     gain = {"data": [0.0, 0.0], "filter": [0.0, 0.0]}
@@ -510,7 +509,9 @@ def plan_sweep(a, fa, torch, tdt):
             nws = L.flhip_conv2d_workspace_bytes(C.byref(cd), pas)
             ws = torch.empty(max(nws, 16), dtype=torch.uint8, device="cuda")
             times = {}
-            for plan in range(-1, nplans - 1):            # (the direct kernels, the last plan, are never competitive)
+            for plan in range(-1, L.flhip_conv2d_plan_count(pas)):
+                if plan == 9:                             # the direct kernels are never competitive
+                    continue
                 if pas == capi.CONV_BWD_DATA:
                     t = timed(lambda: L.flhip_conv2d_bwd_data_plan(C.byref(cd), P(dy), P(w), P(dx), P(ws), nws, plan, S))
                 else:

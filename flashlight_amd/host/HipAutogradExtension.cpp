@@ -169,7 +169,9 @@ void runPlanned(const std::shared_ptr<DynamicBenchmark>& bench, const flhip_conv
     return;
   }
   bench->audit([&] {
-    const int rc = run(opts->currentOption());
+    // the options list is shared by the two passes; a number past this pass's own list counts as declined
+    const int option = opts->currentOption();
+    const int rc = option < flhip_conv2d_plan_count(pass) ? run(option) : FLHIP_DECLINED;
     if (rc == FLHIP_DECLINED) {
       opts->penalise();
       checkRc(run(-1));
@@ -182,7 +184,8 @@ void runPlanned(const std::shared_ptr<DynamicBenchmark>& bench, const flhip_conv
 
 std::shared_ptr<DynamicBenchmark> HipAutogradExtension::createBenchmarkOptions() {
   std::vector<int> plans{-1};
-  for (int i = 0; i < flhip_conv2d_plan_count(FLHIP_CONV_BWD_DATA); ++i) plans.push_back(i);
+  const int count = std::max(flhip_conv2d_plan_count(FLHIP_CONV_BWD_DATA), flhip_conv2d_plan_count(FLHIP_CONV_BWD_FILTER));
+  for (int i = 0; i < count; ++i) plans.push_back(i);
   return std::make_shared<DynamicBenchmark>(std::make_shared<HipPlanOptions>(std::move(plans), kPlanBenchCount));
 }
 
