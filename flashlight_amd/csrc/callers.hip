@@ -606,6 +606,18 @@ affine_fwd_kernel(const T* __restrict__ x, const T* __restrict__ w, const T* __r
   }
 }
 
+// fl::PReLU (flashlight/fl/nn/modules/Activations.cpp:121-124): y = x where x >= 0, w[m] x elsewhere; the
+// parameter is tiled along the tensor's first dimension (m = e % d0), or is a single element (pstride 0)
+template <typename T>
+__global__ void __launch_bounds__(256)
+prelu_fwd_kernel(const T* __restrict__ x, const T* __restrict__ w, T* __restrict__ y, size_t n, long long d0, int pstride) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < n; e += stride) {
+    const float v = ld(x, e);
+    st(y, e, v >= 0.f ? v : v * ld(w, (size_t)pstride * (e % (size_t)d0)));
+  }
+}
+
 // dst[i0, i1, i2, i3] = src[...] with dst dimension k taken from src dimension perm[k]
 // (column-major, dimension 0 fastest); one thread per dst element, writes coalesced
 struct ReorderGeom {
@@ -627,7 +639,9 @@ reorder_kernel(const T* __restrict__ src, T* __restrict__ dst, size_t n, Reorder
 
 // Backward: dx = w * dy, and per parameter element the partial sums of dy * x and dy
 // over slice blockIdx.y of its elements: part[(m * S + s) * 2 + {0, 1}].
-template <typename T>
+// PRELU: the same walk for fl::PReLU's backward pass: dx = dy where x >= 0 and w[m] dy elsewhere, and the
+// parameter's gradient is the sum of dy x over the elements with x < 0 (the second sum is not used).
+template <typename T, bool PRELU = false>
 __global__ void __launch_bounds__(256)
 affine_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ w,
                   T* __restrict__ dx, float* __restrict__ part, long long per, long long chunk,
@@ -641,6 +655,12 @@ affine_bwd_kernel(const T* __restrict__ dy, const T* __restrict__ x, const T* __
     const long long o = j / inner, i = j - o * inner;
     const size_t e = (size_t)((o * mid + m) * inner + i);
     const float d = ld(dy, e);
+    if (PRELU) {
+      const float v = ld(x, e);
+      if (part && v < 0.f) s1 += d * v;
+      if (dx) st(dx, e, v >= 0.f ? d : wm * d);
+      continue;
+    }
     if (part) {
       s1 += d * ld(x, e);
       s2 += d;
@@ -1090,6 +1110,53 @@ extern "C" int flhip_affine_bwd(const void* dy, const void* x, const void* w, vo
     hipLaunchKernelGGL(affine_fold_kernel, dim3((unsigned)((p.nparam + 255) / 256)), dim3(256), 0,
                        as_stream(stream), part, dw, db, p.nparam, p.S);
     return check_launch("affine_bwd (fold)");
+  }
+  return FLHIP_OK;
+}
+
+extern "C" int flhip_prelu_fwd(const void* x, const void* w, void* y, int64_t outer, int64_t d0, int scalar_param,
+                               int dtype, void* stream) {
+  FLHIP_REQUIRE(x && w && y, "prelu_fwd: null argument");
+  FLHIP_REQUIRE(outer > 0 && d0 > 0, "prelu_fwd: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "prelu_fwd: unknown dtype");
+  const size_t n = (size_t)outer * (size_t)d0;
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((prelu_fwd_kernel<T>), dim3(blocks_for(n)), dim3(256), 0, as_stream(stream), (const T*)x,
+                       (const T*)w, (T*)y, n, (long long)d0, scalar_param ? 0 : 1);
+  });
+  return check_launch("prelu_fwd");
+}
+
+extern "C" size_t flhip_prelu_bwd_workspace_bytes(int64_t outer, int64_t d0, int scalar_param) {
+  return flhip_affine_bwd_workspace_bytes(outer, d0, 1, scalar_param);
+}
+
+extern "C" int flhip_prelu_bwd(const void* dy, const void* x, const void* w, void* dx, float* dw, int64_t outer,
+                               int64_t d0, int scalar_param, int dtype, void* workspace, size_t workspace_bytes,
+                               void* stream) {
+  FLHIP_REQUIRE(dy && x, "prelu_bwd: null argument");
+  FLHIP_REQUIRE(outer > 0 && d0 > 0, "prelu_bwd: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "prelu_bwd: unknown dtype");
+  FLHIP_REQUIRE(!dx || w, "prelu_bwd: dx needs the parameter");
+  if (!dx && !dw) return FLHIP_OK;
+  const AffinePlan p = affine_plan(outer, d0, 1, scalar_param);
+  FLHIP_REQUIRE(p.nparam <= 0x7fffffffLL, "prelu_bwd: too many parameter elements");
+  if (dw)
+    FLHIP_REQUIRE(workspace && workspace_bytes >= (size_t)p.nparam * (size_t)p.S * 2 * sizeof(float),
+                  "prelu_bwd: workspace too small");
+  float* part = dw ? static_cast<float*>(workspace) : nullptr;
+  const dim3 grid((unsigned)p.nparam, (unsigned)p.S);
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((affine_bwd_kernel<T, true>), grid, dim3(256), 0, as_stream(stream), (const T*)dy, (const T*)x,
+                       (const T*)w, (T*)dx, part, p.per, p.chunk, p.mid, p.inner, p.S);
+  });
+  if (const int rc = check_launch("prelu_bwd")) return rc;
+  if (dw) {
+    hipLaunchKernelGGL(affine_fold_kernel, dim3((unsigned)((p.nparam + 255) / 256)), dim3(256), 0, as_stream(stream), part,
+                       dw, (float*)nullptr, p.nparam, p.S);
+    return check_launch("prelu_bwd (fold)");
   }
   return FLHIP_OK;
 }

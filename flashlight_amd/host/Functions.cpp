@@ -433,6 +433,39 @@ Variable detail::affine(const Variable& input, const Variable& weight, const Var
   return Variable(out, {input, weight, bias}, gradFunc);
 }
 
+Variable prelu(const Variable& input, const Variable& weight) {
+  dtypesMatch("prelu", {&input, &weight});
+  if (input.ndim() < 1 || input.elements() == 0) throw std::invalid_argument("prelu: empty input");
+  const Dim d0 = input.dim(0), outer = input.elements() / d0;
+  const bool scalar = weight.elements() == 1;
+  // tileAs (Functions.cpp: tileAs) repeats the parameter along dimension 0; one element or a full set are the cases built
+  if (!scalar && weight.elements() != d0)
+    throw std::invalid_argument("prelu: the parameter has one element, or one per index of the input's first dimension");
+  detail::OpScope scope("prelu");
+  const int tag = tagOf(input.type(), "prelu");
+  Tensor out(input.shape(), input.type());
+  check(flhip_prelu_fwd(input.tensor().device(), weight.tensor().device(), out.device(), outer, d0, scalar ? 1 : 0, tag,
+                        hipBackendStream()));
+  if (scope.on()) scope.done({input.tensor(), weight.tensor()}, {out});
+  auto gradFunc = [outer, d0, scalar, tag](std::vector<Variable>& inputs, const Variable& gradOutput) {
+    auto& x = inputs[0];
+    auto& w = inputs[1];
+    if (!x.isCalcGrad() && !w.isCalcGrad()) return;
+    detail::OpScope scope("preluBackward");
+    Tensor dx = x.isCalcGrad() ? Tensor(x.shape(), x.type()) : Tensor();
+    Tensor dw = w.isCalcGrad() ? Tensor(w.shape(), dtype::f32) : Tensor();
+    const size_t wsBytes = w.isCalcGrad() ? flhip_prelu_bwd_workspace_bytes(outer, d0, scalar ? 1 : 0) : 0;
+    Tensor ws = wsBytes ? Tensor({(Dim)wsBytes}, dtype::u8) : Tensor();
+    check(flhip_prelu_bwd(gradOutput.tensor().device(), x.tensor().device(), w.tensor().device(), dx.device(),
+                          static_cast<float*>(dw.device()), outer, d0, scalar ? 1 : 0, tag, ws.device(), wsBytes,
+                          hipBackendStream()));
+    if (scope.on()) scope.done({gradOutput.tensor(), x.tensor()}, {dx});
+    if (x.isCalcGrad()) x.addGrad(Variable(dx, false));
+    if (w.isCalcGrad()) w.addGrad(Variable(dw.astype(w.type()), false));
+  };
+  return Variable(out, {input, weight}, gradFunc);
+}
+
 Variable relu(const Variable& input) {
   detail::OpScope scope("relu");
   Tensor out(input.shape(), input.type());

@@ -155,6 +155,9 @@ Variable swish(const Variable& input, double beta);
 Variable scale(const Variable& input, double factor);
 inline Variable operator*(const Variable& lhs, double rhs) { return scale(lhs, rhs); }
 inline Variable operator*(double lhs, const Variable& rhs) { return scale(rhs, lhs); }
+// fl::PReLU's forward (nn/modules/Activations.cpp:121-124) as one operator: input where input >= 0, input * weight
+// elsewhere, the weight tiled along dimension 0 (one element, or one per index of dimension 0).  Same dtype for both.
+Variable prelu(const Variable& input, const Variable& weight);
 // fl::gatedlinearunit (Functions.cpp:1567-1610): first half of dimension `dim` times the sigmoid of the second half
 Variable gatedlinearunit(const Variable& input, int dim);
 // fl::dropout (Functions.cpp:1777-1785): input * mask / (1 - p); p <= 0 returns the input.  The mask is a

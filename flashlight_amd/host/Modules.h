@@ -312,6 +312,15 @@ class ELU : public UnaryModule {           // :132-139
  private:
   double alpha_;
 };
+class PReLU : public UnaryModule {         // :114-132: `size` parameters (1, or the extent of dimension 0) of value `value`
+ public:
+  explicit PReLU(int size = 1, double value = 0.25)
+      : UnaryModule({constant(value, Shape({size, 1}), dtype::f32, true)}) {}
+  explicit PReLU(const Variable& w) : UnaryModule({w}) {}
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return prelu(input, params_[0].astype(input.type())); }
+  std::string prettyString() const override { return "PReLU"; }
+};
 class Sigmoid : public UnaryModule {       // :18-20
  public:
   using UnaryModule::forward;

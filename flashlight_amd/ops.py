@@ -719,6 +719,34 @@ def affine_backward(grad_output, input, weight, view):
     return dx, dw, db
 
 
+def prelu(input, weight):
+    """fl::PReLU: `weight` has one element, or as many as the input's fastest (last torch) dimension."""
+    x = _dev(input, "input")
+    w = _dev(weight, "weight").to(x.dtype).contiguous()
+    d0 = x.shape[-1]
+    if w.numel() not in (1, d0):
+        raise ValueError("prelu: the parameter has 1 element or one per index of the first dimension")
+    y = torch.empty_like(x)
+    capi.check(capi.lib().flhip_prelu_fwd(_ptr(x), _ptr(w), _ptr(y), x.numel() // d0, d0, int(w.numel() == 1),
+                                          _dtype_tag(x), _stream()))
+    return y
+
+
+def prelu_backward(grad_output, input, weight):
+    """-> (gradInput, gradWeight fp32) of `prelu`."""
+    g, x = _dev(grad_output, "gradOutput"), _dev(input, "input")
+    w = _dev(weight, "weight").to(x.dtype).contiguous()
+    d0 = x.shape[-1]
+    scalar = int(w.numel() == 1)
+    dx = torch.empty_like(x)
+    dw = torch.empty((w.numel(),), dtype=torch.float32, device=x.device)
+    nws = capi.lib().flhip_prelu_bwd_workspace_bytes(x.numel() // d0, d0, scalar)
+    ws = _ws(nws, x.device)
+    capi.check(capi.lib().flhip_prelu_bwd(_ptr(g), _ptr(x), _ptr(w), _ptr(dx), _ptr(dw), x.numel() // d0, d0, scalar,
+                                          _dtype_tag(x), _ptr(ws), nws, _stream()))
+    return dx, dw
+
+
 def reorder(input, perm_whcn):
     """fl::reorder on the Flashlight view of `input` (torch shape reversed, padded to four
     dimensions): Flashlight dimension k of the result is dimension perm_whcn[k] of the

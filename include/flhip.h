@@ -116,8 +116,8 @@ const char* flhip_last_error(void);
  * refuse to run when flhip_version() / 100 differs from FLHIP_VERSION / 100 (a layout change).
  * 200: flhip_rnn_desc gained dropout, seed_lo, seed_hi; flhip_bn_workspace_bytes never returns less
  * than 32 bytes per feature.  202: the *_plan entry points and FLHIP_DECLINED.  203: FLHIP_F16.  204: flhip_act_fwd / _bwd, flhip_glu_fwd / _bwd,
- * flhip_dropout, flhip_rownorm, flhip_weightnorm_fwd / _bwd, flhip_pad_fwd / _bwd, flhip_sgd_many, flhip_adam_many. */
-#define FLHIP_VERSION 204
+ * flhip_dropout, flhip_rownorm, flhip_weightnorm_fwd / _bwd, flhip_pad_fwd / _bwd, flhip_sgd_many, flhip_adam_many.  205: flhip_prelu_fwd / _bwd. */
+#define FLHIP_VERSION 205
 int flhip_version(void);
 const char* flhip_arch(void);
 
@@ -466,6 +466,18 @@ int flhip_affine_bwd(const void* dy, const void* x, const void* w, void* dx, flo
                      float* db, int64_t outer, int64_t mid, int64_t inner,
                      int scalar_params, int dtype, void* workspace,
                      size_t workspace_bytes, void* stream);
+
+/* fl::PReLU (flashlight/fl/nn/modules/Activations.cpp:116-124): y = x where x >= 0, w[m] x elsewhere, the parameter
+ * tiled along the tensor's first (fastest) dimension of extent d0 (m = element index % d0, `outer` = the product of
+ * the other extents) or a single element (scalar_param != 0).  w has the tensor's dtype.  Backward (the chain of
+ * the reference's mask, products and tileAs): dx = dy where x >= 0, w[m] dy elsewhere (skipped when dx is NULL);
+ * dw[m] (fp32, may be NULL) = the sum of dy x over the elements with x < 0 that share m, two-stage in a fixed
+ * order through the workspace. */
+int flhip_prelu_fwd(const void* x, const void* w, void* y, int64_t outer, int64_t d0, int scalar_param, int dtype,
+                    void* stream);
+size_t flhip_prelu_bwd_workspace_bytes(int64_t outer, int64_t d0, int scalar_param);
+int flhip_prelu_bwd(const void* dy, const void* x, const void* w, void* dx, float* dw, int64_t outer, int64_t d0,
+                    int scalar_param, int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /* fl::logSoftmax over dimension 0 of a classes x cols matrix (Functions.cpp:1044-1070)
  * and its backward dx = dy - exp(y) * sum over classes of dy. */

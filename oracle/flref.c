@@ -454,6 +454,28 @@ void flref_glu_bwd(int64_t outer, int64_t m, const float* dy, const float* x, fl
     }
 }
 
+/* fl::PReLU (nn/modules/Activations.cpp:121-124): (input * mask) + (input * !mask * tileAs(w, input)) with mask =
+ * input >= 0; the parameter has `size` elements tiled along the first dimension (extent d0, size divides d0).
+ * Backward by the chain rule of those operators: dx = dy mask + dy !mask w, dw = sumAs(dy input !mask, w). */
+void flref_prelu_fwd(int64_t n, int64_t d0, int64_t size, const float* x, const float* w, float* y) {
+  for (int64_t i = 0; i < n; ++i) {
+    const double mask = x[i] >= 0.f ? 1.0 : 0.0;
+    y[i] = (float)((double)x[i] * mask + (double)x[i] * (1.0 - mask) * (double)w[(i % d0) % size]);
+  }
+}
+void flref_prelu_bwd(int64_t n, int64_t d0, int64_t size, const float* dy, const float* x, const float* w, float* dx,
+                     float* dw) {
+  double* acc = (double*)calloc((size_t)size, sizeof(double));
+  for (int64_t i = 0; i < n; ++i) {
+    const double mask = x[i] >= 0.f ? 1.0 : 0.0;
+    const int64_t m = (i % d0) % size;
+    dx[i] = (float)((double)dy[i] * mask + (double)dy[i] * (1.0 - mask) * (double)w[m]);
+    acc[m] += (double)dy[i] * (double)x[i] * (1.0 - mask);
+  }
+  for (int64_t m = 0; m < size; ++m) dw[m] = (float)acc[m];
+  free(acc);
+}
+
 /* fl::dropout (Functions.cpp:1777-1785) with the counter-based mask below in the place of fl::rand(...) > p */
 int flref_dropout_keep(uint32_t seed_lo, uint32_t seed_hi, uint32_t layer, uint32_t index, float dropout);
 void flref_dropout(int64_t n, const float* x, double p, uint32_t seed_lo, uint32_t seed_hi, float* y) {

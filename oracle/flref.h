@@ -107,6 +107,9 @@ void flref_act_bwd(int op, int64_t n, const float* dy, const float* x, double a,
 /* gatedlinearunit (:1567-1610): halves are contiguous blocks of m elements per outer index */
 void flref_glu_fwd(int64_t outer, int64_t m, const float* x, float* y);
 void flref_glu_bwd(int64_t outer, int64_t m, const float* dy, const float* x, float* dx);
+void flref_prelu_fwd(int64_t n, int64_t d0, int64_t size, const float* x, const float* w, float* y);
+void flref_prelu_bwd(int64_t n, int64_t d0, int64_t size, const float* dy, const float* x, const float* w, float* dx,
+                     float* dw);
 /* dropout (:1777-1785) with the counter-based mask of flref_dropout_keep */
 void flref_dropout(int64_t n, const float* x, double p, uint32_t seed_lo, uint32_t seed_hi, float* y);
 /* WeightNorm (nn/modules/WeightNorm.cpp:45-72) over a rows x cols view (rows_fast: element (r, j) at r + j*rows,

@@ -223,6 +223,21 @@ def glu_bwd(dy, x, outer, m):
     return dx
 
 
+def prelu_fwd(x, w, d0):
+    """x: any array whose fastest dimension has d0 elements; w: 1-D parameter whose size divides d0."""
+    x, w = _f32(x), _f32(w)
+    y = np.empty_like(x)
+    lib().flref_prelu_fwd(_i64(x.size), _i64(d0), _i64(w.size), _p(x), _p(w), _p(y))
+    return y
+
+
+def prelu_bwd(dy, x, w, d0):
+    dy, x, w = _f32(dy), _f32(x), _f32(w)
+    dx, dw = np.empty_like(x), np.empty_like(w)
+    lib().flref_prelu_bwd(_i64(x.size), _i64(d0), _i64(w.size), _p(dy), _p(x), _p(w), _p(dx), _p(dw))
+    return dx, dw
+
+
 def dropout(x, p, seed_lo, seed_hi):
     x = _f32(x)
     y = np.empty_like(x)

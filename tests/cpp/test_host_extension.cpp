@@ -959,7 +959,7 @@ static void testArchBuilder() {
   // malformed lines, lines for modules that do not exist here, a missing file
   for (const char* bad : {"C 3 4 5", "C2 3 4 5 6 1", "L 5", "BN 8", "LN", "LN 3", "M 2 2 2", "R 1", "LSM", "GRU 4",
                           "C 3 x 5 1", "XYZ 1 2", "RO", "DO", "DO 0.2 1", "GLU", "ELU 1", "SH 1 2", "WN 3", "WN 1 C 4 4 3 1", "WN 3 R", "PD 0 1", "PD 0 1 1 1",
-                          "TDS 10 21", "AC 1 2 3", "RES 2 1", "RES 1 0 1", "SKIP 0 2", "PC", "PC f64", "PR 1", "E 4 5"})
+                          "TDS 10 21", "AC 1 2 3", "RES 2 1", "RES 1 0 1", "SKIP 0 2", "PC", "PC f64", "PR 1 2 3", "PR x", "E 4 5"})
     CHECK(throws<std::invalid_argument>([&] { one(bad); }));
   CHECK(throws<std::runtime_error>([] { buildSequentialModule(std::string("/nonexistent/arch.txt"), 1, 1); }));
   // from a file
@@ -1026,6 +1026,35 @@ static void testActivationModules() {
       CHECK(relL2(hostOf(in.grad()), dxr) <= tol);
     }
   }
+  // PReLU (lines PR, PR n, PR n value): one parameter, or one per index of dimension 0; the parameter's gradient
+  for (dtype dt : {dtype::f32, dtype::bf16}) {
+    const double tol = dt == dtype::f32 ? 2e-6 : 4e-3;
+    for (const char* line : {"PR", "PR 9 0.1", "PR 1 0.5"}) {
+      auto x = randn(n, 730, 2.f), dy = randn(n, 731);
+      for (auto& v : x) v = roundTo(dt, v);
+      for (auto& v : dy) v = roundTo(dt, v);
+      auto mod = one(line);
+      CHECK(mod->prettyString() == "PReLU" && mod->params().size() == 1);
+      const auto w = hostOf(mod->param(0));
+      const size_t size = w.size();
+      CHECK(size == (std::string(line) == "PR 9 0.1" ? 9u : 1u));
+      CHECK(std::fabs(w[0] - (std::string(line) == "PR" ? 0.25f : std::string(line) == "PR 9 0.1" ? 0.1f : 0.5f)) < 1e-7f);
+      Variable in(Tensor::fromVector(shp, x).astype(dt), true);
+      mod->zeroGrad();
+      Variable y = mod->forward({in})[0];
+      y.backward(Variable(Tensor::fromVector(shp, dy).astype(dt), false));
+      std::vector<float> wr = w;
+      for (auto& v : wr) v = roundTo(dt, v);
+      std::vector<float> yr(n), dxr(n), dwr(size);
+      flref_prelu_fwd((int64_t)n, 9, (int64_t)size, x.data(), wr.data(), yr.data());
+      flref_prelu_bwd((int64_t)n, 9, (int64_t)size, dy.data(), x.data(), wr.data(), dxr.data(), dwr.data());
+      CHECK(relL2(hostOf(y), yr) <= tol);
+      CHECK(relL2(hostOf(in.grad()), dxr) <= tol);
+      // (bf16: the gradient passes through the parameter's cast and is rounded to bf16 there, as LayerNorm's is)
+      CHECK(mod->param(0).grad().type() == dtype::f32 && relL2(hostOf(mod->param(0).grad()), dwr) <= (dt == dtype::f32 ? 1e-5 : 4e-3));
+    }
+  }
+  CHECK(throws<std::invalid_argument>([&] { PReLU(4).forward(Variable(Tensor::fromVector({9, 2}, randn(18, 1)), false)); }));
   CHECK(throws<std::invalid_argument>([&] { gatedlinearunit(Variable(Tensor::fromVector({3, 5}, randn(15, 1)), false), 0); }));
   CHECK(throws<std::invalid_argument>([&] { gatedlinearunit(Variable(Tensor::fromVector({4, 5}, randn(20, 1)), false), 2); }));
 

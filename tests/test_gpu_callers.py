@@ -148,6 +148,32 @@ def test_affine(outer, mid, inner, scalar, dtype):
 
 
 @pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("shape,scalar", [((3, 5, 7), True), ((3, 5, 7), False), ((1, 600), False), ((40, 9, 1), True),
+                                          ((64, 3, 56, 56), True), ((8, 250, 1, 300), False), ((300001,), True)])
+def test_prelu(shape, scalar, dtype):
+    """fl::PReLU forward, input gradient and parameter gradient against the checker: a single parameter or one per
+    index of the fastest dimension, sizes from one workgroup's slice to many slices per parameter; exact zeros in x
+    (the mask is x >= 0)."""
+    rng = np.random.default_rng(len(shape) * 100 + shape[-1])
+    x = _round(rng.standard_normal(shape).astype(np.float32), dtype)
+    x.flat[::5] = 0.0
+    dy = _round(rng.standard_normal(shape).astype(np.float32), dtype)
+    d0 = shape[-1]
+    w = _round(rng.uniform(0.05, 0.95, 1 if scalar else d0).astype(np.float32), dtype)
+    tol = _tol(dtype)
+    y = ops.prelu(dev(x, dtype), dev(w, dtype))
+    assert rel_l2(host(y), flref.prelu_fwd(x, w, d0)) <= tol
+    dx, dw = ops.prelu_backward(dev(dy, dtype), dev(x, dtype), dev(w, dtype))
+    rdx, rdw = flref.prelu_bwd(dy, x, w, d0)
+    assert rel_l2(host(dx), rdx) <= tol
+    assert rel_l2(host(dw), rdw) <= 1e-4           # fp32 sums whatever the storage type
+    assert np.array_equal(host(dx).flat[::5], dy.flat[::5])
+    # twice the same call: the same bits (fixed order of the two-stage sum)
+    dx2, dw2 = ops.prelu_backward(dev(dy, dtype), dev(x, dtype), dev(w, dtype))
+    assert torch.equal(dw, dw2) and torch.equal(dx, dx2)
+
+
+@pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("whcn,norm,params", [
     ((6, 5, 4, 3), (0, 1, 2), "per"),        # LayerNorm over {0,1,2} of WHCN
     ((6, 5, 4, 3), (0, 1, 2), "scalar"),

@@ -239,6 +239,30 @@ def test_glu_against_torch_float64(shape, dim):
     assert rel_l2(flref.glu_bwd(dy, x, outer, m).reshape(shape), t.grad.numpy()) <= 1e-6
 
 
+@pytest.mark.parametrize("shape,size", [((4, 3, 10), 1), ((4, 3, 10), 10), ((5, 12), 12), ((2, 3, 4, 6), 1), ((7, 8), 4)])
+def test_prelu_against_torch_float64(shape, size):
+    # nn/modules/Activations.cpp:116-124: the parameter tiled along Flashlight's first dimension = the last one of
+    # the contiguous array.  torch.nn.functional.prelu puts its parameter on dimension 1, so the pin is written with
+    # torch's own operators (where / broadcasting) and autograd in float64; size 4 over extent 8 is tileAs' repeat.
+    rng = np.random.default_rng(320 + size)
+    x = rng.standard_normal(shape).astype(np.float32)
+    x.flat[::7] = 0.0                                  # the mask is x >= 0: a zero passes the gradient whole
+    w = rng.uniform(0.1, 0.9, size).astype(np.float32)
+    d0 = shape[-1]
+    t = torch.from_numpy(x.astype(np.float64)).requires_grad_(True)
+    tw = torch.from_numpy(w.astype(np.float64)).requires_grad_(True)
+    y = torch.where(t >= 0, t, t * tw.repeat(d0 // size))
+    dy = rng.standard_normal(shape).astype(np.float32)
+    y.backward(torch.from_numpy(dy.astype(np.float64)))
+    assert rel_l2(flref.prelu_fwd(x, w, d0), y.detach().numpy()) <= 1e-6
+    dx, dw = flref.prelu_bwd(dy, x, w, d0)
+    assert rel_l2(dx, t.grad.numpy()) <= 1e-6 and rel_l2(dw, tw.grad.numpy()) <= 1e-6
+    if size == 1 and len(shape) == 2:
+        # the one case the library routine states the same way: a single parameter
+        assert rel_l2(flref.prelu_fwd(x, w, d0), F.prelu(torch.from_numpy(x), torch.from_numpy(w)).numpy()) <= 1e-6
+    assert np.array_equal(dx.flat[::7], dy.flat[::7])
+
+
 def test_dropout_mask_rate_scale_and_determinism():
     # Functions.cpp:1777-1785: zero with probability p, the rest scaled by 1 / (1 - p); the mask is a function of
     # (seed, index) only
