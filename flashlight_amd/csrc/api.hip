@@ -45,6 +45,7 @@ static bool apply_option(Options& o, const char* name, const char* v) {
       if (strstr(v, "wd32")) m |= Options::SKIP_WD32;
       if (strstr(v, "tap1d")) m |= Options::SKIP_TAP1D;
       if (strstr(v, "cells")) m |= Options::SKIP_CELLS;
+      if (strstr(v, "tap2d")) m |= Options::SKIP_TAP2D;
     }
     o.conv_skip = m;
     return true;
@@ -84,12 +85,13 @@ static bool apply_option(Options& o, const char* name, const char* v) {
   if (!strcmp(name, "TAPPED_NO_REORDER")) return flag(&o.tapped_no_reorder);
   if (!strcmp(name, "MATMUL_VALU")) return flag(&o.matmul_valu);
   if (!strcmp(name, "RNN_UNFUSED")) return flag(&o.rnn_unfused);
+  if (!strcmp(name, "TAP2D_ALL")) return flag(&o.tap2d_all);
   return false;
 }
 
 static void options_from_environment() {
   static const char* const names[] = {"CONV_ALGO", "CONV_SKIP", "PW_PT", "PW16_PF", "CONV_STACK", "SLAB_WAVES", "BN_ALGO", "PW16_NO_TAPS",
-                                      "TAPPED_NO_REORDER", "MATMUL_VALU", "RNN_UNFUSED"};
+                                      "TAPPED_NO_REORDER", "MATMUL_VALU", "RNN_UNFUSED", "TAP2D_ALL"};
   for (const char* n : names) {
     const std::string var = std::string("FLHIP_") + n;
     if (const char* v = getenv(var.c_str())) apply_option(g_options, n, v);   // unknown values keep the default

@@ -281,9 +281,9 @@ inline void launch_elementwise(const T* a, const T* b, T* out, size_t n, Op op, 
 // flhip_set_option(); no entry point calls getenv on its per-call path.
 struct Options {
   enum { ALGO_AUTO = 0, ALGO_DIRECT, ALGO_GATHER, ALGO_TAPPED, ALGO_CONVERT };
-  enum { SKIP_BF16 = 1, SKIP_GEMM1X1 = 2, SKIP_SLAB = 4, SKIP_TAPPED = 8, SKIP_STRIP = 16, SKIP_FIRST = 32, SKIP_WGRAD128 = 64, SKIP_PWDMA = 128, SKIP_WD32 = 256, SKIP_TAP1D = 512, SKIP_CELLS = 1024 };
+  enum { SKIP_BF16 = 1, SKIP_GEMM1X1 = 2, SKIP_SLAB = 4, SKIP_TAPPED = 8, SKIP_STRIP = 16, SKIP_FIRST = 32, SKIP_WGRAD128 = 64, SKIP_PWDMA = 128, SKIP_WD32 = 256, SKIP_TAP1D = 512, SKIP_CELLS = 1024, SKIP_TAP2D = 2048 };
   int conv_algo = ALGO_AUTO;      // CONV_ALGO = direct | gather | tapped | convert
-  unsigned conv_skip = 0;         // CONV_SKIP = comma list of bf16, gemm1x1, slab, tapped, strip, first, wgrad128, pwdma, wd32, tap1d, cells
+  unsigned conv_skip = 0;         // CONV_SKIP = comma list of bf16, gemm1x1, slab, tapped, strip, first, wgrad128, pwdma, wd32, tap1d, cells, tap2d
   int pw_pt = 2;                  // PW_PT = 2 | 4 | 8: position-tile width of the fp32 1x1 kernels / 32
   int pw16_pf = 0;                // PW16_PF = 1 / 4: one / four chunks (shallow / deep ring) in flight in the bf16 1x1 kernels, 2 / 8: the same with
                                   // tiles of 64 result channels in the direct-to-LDS kernels (0: by grid size)
@@ -293,6 +293,7 @@ struct Options {
   bool tapped_no_reorder = false; // TAPPED_NO_REORDER: tapped kernels read the original weight layout
   bool matmul_valu = false;       // MATMUL_VALU: flhip_matmul stays off the matrix cores
   bool rnn_unfused = false;       // RNN_UNFUSED: two-kernel rnn steps
+  bool tap2d_all = false;         // TAP2D_ALL: the kernel for 3x3 windows over stacked planes takes every geometry it can, not only those of its measured rule
   int bn_algo = 0;                // BN_ALGO = split (1) | resident (2)
 };
 const Options& options();

@@ -125,6 +125,14 @@ int mfma_tap1d_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void*
                         void* ws, size_t ws_bytes);
 int mfma_tap1d_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx, hipStream_t s, void* ws,
                              size_t ws_bytes);
+// 3x3 windows of stride 1 and padding 1 over small planes on the same kernels: every plane of the batch in one
+// sequence (rows followed by a zero column, planes separated by a zero row), 65 to 512 (fp32: 256) contraction channels;
+// operands in mfma_tap2d_conv_ws() bytes of workspace; -1 when the shape is not theirs or the room is missing
+size_t mfma_tap2d_conv_ws(const ConvGeom& g, int dtype, bool bwd);
+int mfma_tap2d_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w, const float* bias, void* y, hipStream_t s,
+                        void* ws, size_t ws_bytes);
+int mfma_tap2d_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx, hipStream_t s, void* ws,
+                             size_t ws_bytes);
 // their filter gradient (6 to 23 taps; bf16: an even number of result positions per row): the channels-last rows and
 // the workgroups' tiles in mfma_tap1d_wgrad_ws() bytes of workspace
 size_t mfma_tap1d_wgrad_ws(const ConvGeom& g, int dtype);

@@ -147,6 +147,16 @@ static bool tap1d_on(int dtype) {
   return dtype == FLHIP_F32 || (dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT));
 }
 
+// 3x3 windows over stacked planes: bf16, planes of at most 64 positions (the 7 x 7 layers) and a sequence of at least
+// 2048 positions.  Measured (batch 64 / 32, forward): 7 x 7 x 512 41.9 / 40.3 us against 62.3 / 54.8 on the slab
+// kernel; 14 x 14 x 256 42.2 / 33.0 against 34.6 / 31.0 and 28 x 28 x 128 41.3 / 32.5 against 25.5 / 19.7, so larger planes
+// stay where they were; fp32 loses at every size (14 x 14 x 256: 221 against 140 us).  TAP2D_ALL lifts the rule.
+static bool tap2d_on(const ConvGeom& g, int dtype) {
+  if (!tap1d_on(dtype) || skip(Options::SKIP_TAP2D)) return false;
+  if (options().tap2d_all) return true;
+  return dtype == FLHIP_BF16 && g.H * g.W <= 64 && (long long)g.N * (g.H + 1) * (g.W + 1) >= 2048;
+}
+
 static bool long_rows(const ConvGeom& g, int dtype, bool bwd, size_t ws_bytes) {
   if (algo_is(Options::ALGO_TAPPED)) return false;
   const size_t need = mfma_tapped_ws(g, dtype, bwd);
@@ -221,7 +231,8 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
     const size_t b = d->dtype == FLHIP_BF16 ? mfma_pointwise16_lattice_ws(g, pass == FLHIP_CONV_BWD_DATA)
                                             : pass == FLHIP_CONV_BWD_DATA ? mfma_pointwise_split_ws(g, d->dtype, true) : 0;
     const size_t c = mfma_tap1d_conv_ws(g, d->dtype, pass == FLHIP_CONV_BWD_DATA);
-    return std::max(a, std::max(b, c));
+    const size_t c2 = tap2d_on(g, d->dtype) ? mfma_tap2d_conv_ws(g, d->dtype, pass == FLHIP_CONV_BWD_DATA) : 0;
+    return std::max(std::max(a, c2), std::max(b, c));
   }
   return 0;
 }
@@ -237,6 +248,7 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
   if (!force_direct()) {
     int r = -1;
     if (tap1d_on(d->dtype)) r = mfma_tap1d_conv_fwd(g, d->dtype, x, w, bias, y, s, ws, ws_bytes);
+    if (r < 0 && tap2d_on(g, d->dtype)) r = mfma_tap2d_conv_fwd(g, d->dtype, x, w, bias, y, s, ws, ws_bytes);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pwd16_conv_fwd(g, x, w, bias, y, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
@@ -271,11 +283,12 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
 // family: the caller times them instead of trusting the rules.
 static const char* const kBwdDataPlans[] = {"bf16 1x1, tiles loaded straight to LDS", "bf16 1x1 / gathered taps", "bf16 3x3 strip",
                                             "bf16 slab", "1x1 GEMM, split contraction", "1x1 GEMM", "slab", "tapped GEMM",
-                                            "gather", "direct", "one-row windows", "stride-2 window over few channels, 2 x 2 cells"};
+                                            "gather", "direct", "one-row windows", "stride-2 window over few channels, 2 x 2 cells",
+                                            "3x3 windows over stacked planes"};
 static const char* const kBwdFilterPlans[] = {"bf16 3x3 rows straight to LDS, 32 x 32 tiles", "bf16 3x3 rows straight to LDS, 64 x 64 tiles",
                                               "bf16 1x1 / gathered taps", "bf16 first layer", "bf16 3x3 rows", "1x1 GEMM", "row slab",
                                               "tapped GEMM", "gather", "direct", "one-row windows"};
-constexpr int kNumDataPlans = 12, kNumFilterPlans = 11;
+constexpr int kNumDataPlans = 13, kNumFilterPlans = 11;
 
 static int bwd_data_direct(const flhip_conv_desc* d, const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s) {
   const size_t total = (size_t)g.N * g.C * g.H * g.W;
@@ -313,13 +326,15 @@ static int bwd_data_impl(const flhip_conv_desc* d, const void* dy, const void* w
       case 8: r = mfma_conv_bwd_data(g, d->dtype, dy, w, dx, s); break;
       case 9: r = bwd_data_direct(d, g, dy, w, dx, s); break;
       case 10: r = mfma_tap1d_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes); break;
-      default: r = mfma_cells_conv_bwd_data(g, d->dtype, dy, w, dx, s);
+      case 11: r = mfma_cells_conv_bwd_data(g, d->dtype, dy, w, dx, s); break;
+      default: r = mfma_tap2d_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
     }
     return r < 0 ? FLHIP_DECLINED : r;
   }
   if (!force_direct()) {
     int r = -1;
     if (tap1d_on(d->dtype)) r = mfma_tap1d_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
+    if (r < 0 && tap2d_on(g, d->dtype)) r = mfma_tap2d_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
     if (r < 0 && !skip(Options::SKIP_CELLS)) r = mfma_cells_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_pwd16_conv_bwd_data(g, dy, w, nullptr, dx, s);

@@ -87,6 +87,9 @@ struct Tap1Params {
   int taps_total;        // ntaps[0] + ntaps[1]
   int ptiles, mtiles;
   unsigned src_bytes, w_bytes, dst_bytes;
+  // two-dimensional windows over stacked planes (tap2d_*): taps per window row, slab rows per window row = the
+  // pitch of a plane's row, and the plane's geometry for the results
+  int tw, tpitch, pW, pH, pN;
 };
 
 // ---- operand passes ------------------------------------------------------------------------
@@ -175,14 +178,44 @@ tap1d_weights_kernel(const T* __restrict__ w, uintx4_t* __restrict__ wf, Tap1Wei
   wf[idx] = *reinterpret_cast<const uintx4_t*>(v);
 }
 
+// The same fragments with the tap as the index that changes fastest after the lane: the four waves of a block then read
+// the same cache lines (a lane's 8 or 4 contraction channels x 9 taps are neighbours in memory), where in the order
+// above - the stage fastest - every line is met once per tap by a different block.
+template <typename T>
+__global__ void __launch_bounds__(256)
+tap_weights_by_tap_kernel(const T* __restrict__ w, uintx4_t* __restrict__ wf, Tap1Weights p) {
+  constexpr int CELL = Tap1Elem<T>::CELL;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  const long long total = (long long)p.mblocks * p.taps_total * p.KS * 64;
+  if (idx >= total) return;
+  const int lane = (int)(idx & 63);
+  const long long st = idx >> 6;
+  const int tap = (int)(st % p.taps_total);
+  const long long r2 = st / p.taps_total;
+  const int ks = (int)(r2 % p.KS), mblk = (int)(r2 / p.KS);
+  const int m = mblk * 32 + (lane & 31), c0 = (2 * ks + (lane >> 5)) * CELL;
+  const int j = p.tapj[tap];
+  __attribute__((aligned(16))) T v[CELL];
+#pragma unroll
+  for (int e = 0; e < CELL; ++e) {
+    const int c = c0 + e;
+    v[e] = T{};
+    if (j >= 0 && m < p.Mo && c < p.Cc)
+      v[e] = w[p.bwd ? ((size_t)c * p.Cw + m) * p.KW + j : ((size_t)m * p.Cw + c) * p.KW + j];
+  }
+  wf[(((long long)mblk * p.taps_total + tap) * p.KS + ks) * 64 + lane] = *reinterpret_cast<const uintx4_t*>(v);
+}
+
 // ---- the convolution ---------------------------------------------------------------------
 // KS stages per tap; DT taps per unrolled group; RW stages between a weight fragment's load and its use (RW divides
 // DT * KS; a bf16 stage is one matrix instruction per block, an fp32 stage four longer ones); SS source stride;
 // NPH phases; NB blocks of 32 positions.
-template <typename T, int KS, int DT, int RW, int SS, int NPH, int NB>
-__global__ void __launch_bounds__(256, 1)
-tap1d_conv_kernel(Tap1Params p, const T* __restrict__ xr, const uintx4_t* __restrict__ wf,
-                  const float* __restrict__ bias, T* __restrict__ dst) {
+// TD: the taps form a two-dimensional window over planes stacked in one sequence (see tap2d_plan); only the slab
+// offset of a tap and the addresses of the results differ.
+template <typename T, int KS, int DT, int RW, int SS, int NPH, int NB, bool TD>
+__device__ __forceinline__ void
+tap_conv_body(const Tap1Params& p, const T* __restrict__ xr, const uintx4_t* __restrict__ wf,
+              const float* __restrict__ bias, T* __restrict__ dst) {
   extern __shared__ uintx4_t t1_slab[];
   constexpr int CELL = Tap1Elem<T>::CELL;
   constexpr int ESZ = (int)sizeof(T);
@@ -250,7 +283,8 @@ tap1d_conv_kernel(Tap1Params p, const T* __restrict__ xr, const uintx4_t* __rest
     // slab offset (cells) of a tap's rows; padding taps read the rows of the last tap that exists: finite values
     // times zero weights
     auto toff_of = [&](int tap) {
-      const int d = dq + min(tap, last);
+      const int tl = min(tap, last);
+      const int d = dq + (TD ? (tl / p.tw) * p.tpitch + tl % p.tw : tl);
       const int trow = SS == 1 ? d : (d & 1) * p.half + (d >> 1);
       return trow * CPR;
     };
@@ -288,6 +322,39 @@ tap1d_conv_kernel(Tap1Params p, const T* __restrict__ xr, const uintx4_t* __rest
 
   // ---- results: element r of block b: result index o0 + 32 b + 8 (r / 4) + 4 fg + r % 4 of channel m
   const int m = mtile * T1_BM + wave * 32 + fr;
+  if constexpr (TD) {
+    // Results through LDS (the slab is done with): every wave parks its 32 channels x 32 NB positions at storage size,
+    // then threads walk positions (consecutive lanes = consecutive positions = consecutive addresses inside a plane's
+    // row, and across row ends too: the zero column has no address) with the position's plane / row / column worked
+    // out once per thread.  Position o of the sequence = row o / pitch (row 0 and every (pH + 1)-th after it are the
+    // zero rows between the planes), column o % pitch (the last one of a row is the zero column).
+    constexpr int TPOS = 32 * NB;
+    constexpr int SPT = TPOS + 4;                 // staging pitch (elements): 8-byte rows, lanes on distinct banks
+    T* const stage = reinterpret_cast<T*>(t1_slab);
+    const float bvt = (bias && m < p.Mo) ? bias[m] : 0.f;
+    __syncthreads();
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; ++g4) {
+        T* const at = stage + (wave * 32 + fr) * SPT + b * 32 + g4 * 8 + fg * 4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) st(at, e, acc[0][b][4 * g4 + e] + bvt);
+      }
+    __syncthreads();
+    if (tid >= 2 * TPOS) return;
+    const int pos = tid % TPOS, cg = tid / TPOS;
+    const int o = o0 + pos;
+    const int P = p.tpitch, H1 = p.pH + 1;
+    const int prow = o / P, col = o - prow * P;
+    const int n = max(prow - 1, 0) / H1, h = max(prow - 1, 0) - n * H1;
+    if (!(prow >= 1 && n < p.pN && h < p.pH && col < p.pW)) return;
+    const int mlim = min(T1_BM, p.Mo - mtile * T1_BM);
+    const size_t plane = (size_t)p.pH * p.pW;
+    T* const out = dst + ((size_t)n * p.Mo + mtile * T1_BM) * plane + (size_t)h * p.pW + col;
+    for (int c = cg; c < mlim; c += 2) out[(size_t)c * plane] = stage[c * SPT + pos];
+    return;
+  }
   if (m >= p.Mo) return;
   const float bv = bias ? bias[m] : 0.f;
   const int n = row / p.H, h = row - n * p.H;
@@ -324,6 +391,61 @@ tap1d_conv_kernel(Tap1Params p, const T* __restrict__ xr, const uintx4_t* __rest
           if (u + e < p.TOu) st(dst, (size_t)(rbase + u + e), v[e]);
       }
     }
+}
+
+template <typename T, int KS, int DT, int RW, int SS, int NPH, int NB>
+__global__ void __launch_bounds__(256, 1)
+tap1d_conv_kernel(Tap1Params p, const T* __restrict__ xr, const uintx4_t* __restrict__ wf,
+                  const float* __restrict__ bias, T* __restrict__ dst) {
+  tap_conv_body<T, KS, DT, RW, SS, NPH, NB, false>(p, xr, wf, bias, dst);
+}
+
+// 3 x 3 windows of stride 1 over small planes (the 14 x 14 and 7 x 7 layers of a residual network): the same loop
+// over a sequence that holds every plane of the batch, rows pH + 1 apart with a zero row between two planes, a row's
+// pW positions followed by one zero column (tap2d_rows_kernel writes it so) - the window's taps are then nine fixed
+// offsets into the sequence, and the zero row / column are the padding.  Results at the zero positions are not stored.
+template <typename T, int KS, int DT, int RW, int NB>
+__global__ void __launch_bounds__(256, 1)
+tap2d_conv_kernel(Tap1Params p, const T* __restrict__ xr, const uintx4_t* __restrict__ wf,
+                  const float* __restrict__ bias, T* __restrict__ dst) {
+  tap_conv_body<T, KS, DT, RW, 1, 1, NB, true>(p, xr, wf, bias, dst);
+}
+
+// x[n][c][h][w] -> xr[position][Cs] with position = ((n (H + 1) + 1 + h) P + w), P = W + 1; the zero rows, the zero
+// column and channels c >= C are written as zeros.  A block transposes 64 channels x 64 positions through LDS.
+template <typename T>
+__global__ void __launch_bounds__(256)
+tap2d_rows_kernel(const T* __restrict__ x, T* __restrict__ xr, int C, int H, int W, int N, int TS, int Cs) {
+  constexpr int CELL = Tap1Elem<T>::CELL;
+  __shared__ T tile[64][sizeof(T) == 2 ? 66 : 65];
+  const int t0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+  const int P = W + 1, H1 = H + 1;
+  {
+    const int tx = threadIdx.x & 63, cy = threadIdx.x >> 6;
+    const int t = t0 + tx;
+    const int prow = t / P, col = t - prow * P;
+    const int n = (prow - 1) / H1, h = (prow - 1) - n * H1;
+    const bool ok = t < TS && prow >= 1 && n < N && h < H && col < W;
+    const size_t at = ok ? ((size_t)n * C * H + h) * W + col : 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int c = c0 + cy + 4 * i;
+      tile[cy + 4 * i][tx] = (ok && c < C) ? x[at + (size_t)c * H * W] : T{};
+    }
+  }
+  __syncthreads();
+  constexpr int CPT = 64 / CELL;
+#pragma unroll
+  for (int i = 0; i < CPT * 64 / 256; ++i) {
+    const int item = threadIdx.x + 256 * i, cell = item % CPT, tl = item / CPT;
+    const int t = t0 + tl, c = c0 + CELL * cell;
+    if (t < TS && c < Cs) {
+      __attribute__((aligned(16))) T v[CELL];
+#pragma unroll
+      for (int e = 0; e < CELL; ++e) v[e] = tile[CELL * cell + e][tl];
+      *reinterpret_cast<uintx4_t*>(xr + (size_t)t * Cs + c) = *reinterpret_cast<const uintx4_t*>(v);
+    }
+  }
 }
 
 // ---- host side ---------------------------------------------------------------------------
@@ -485,6 +607,108 @@ int run_conv(const ConvGeom& g, bool bwd, const void* src, const void* w, const 
       case 16: return launch_conv<T, 16, 1, 4>(pl, xr, wf, bias, out, s);
       default: return launch_conv<T, 32, 1, 4>(pl, xr, wf, bias, out, s);
     }
+  }
+}
+
+// ---- 3 x 3 windows over small planes -------------------------------------------------------
+// The sequence of tap2d_conv_kernel: N planes of H x W, each row followed by one zero column (pitch P = W + 1), one
+// zero row before every plane and one after the last: TS = (N (H + 1) + 1) P positions.  Result position o takes tap
+// (r, s) from position o + (r - 1) P + (s - 1): the slab of a tile starts P + 1 positions before its first result and
+// tap 3 r + s sits r P + s rows into it.  Backward-data is the same walk over dy with the taps in reverse order and
+// the roles of the two channel counts exchanged.  (H + 1)(W + 1) / (H W) of the positions are computed: 1.15 for
+// 14 x 14 planes, 1.31 for 7 x 7.
+bool tap2d_plan(const ConvGeom& g, bool bwd, int esz, Tap1Plan* pl) {
+  if (g.KH != 3 || g.KW != 3 || g.sy != 1 || g.sx != 1 || g.py != 1 || g.px != 1 || g.dly != 1 || g.dlx != 1 || g.groups != 1)
+    return false;
+  const int Cc = bwd ? g.K : g.C, Mo = bwd ? g.C : g.K;
+  // contraction channels padded to a count the two-dimensional kernel is compiled for
+  int Cs = 0;
+  for (int c : {128, 256, 512})
+    if (!Cs && Cc <= c && (esz == 2 || c <= 256)) Cs = c;
+  if (!Cs || Cc <= Cs / 2) return false;
+  const int cell = 16 / esz;
+  const int KS = Cs / (2 * cell), DT = esz == 2 ? dt_of(KS) : 1;
+  Tap1Params& p = pl->p;
+  Tap1Weights& w = pl->w;
+  std::memset(&p, 0, sizeof p);
+  std::memset(&w, 0, sizeof w);
+  const int P = g.W + 1;
+  const long long ts = ((long long)g.N * (g.H + 1) + 1) * P;
+  if (ts >= (1ll << 22) - 256) return false;
+  p.rows = 1; p.H = 1;
+  p.Cs = Cs; p.KS = KS; p.Mo = Mo;
+  p.nph = 1;
+  p.TS = (int)ts; p.TOu = p.TS; p.TO = p.TS;
+  p.nreal[0] = 9;
+  p.ntaps[0] = (9 + DT - 1) / DT * DT;
+  p.taps_total = p.ntaps[0];
+  p.d0[0] = 0;
+  p.smin = -(P + 1);
+  p.tw = 3; p.tpitch = P; p.pW = g.W; p.pH = g.H; p.pN = g.N;
+  for (int i = 0; i < p.ntaps[0]; ++i) w.tapj[i] = (signed char)(i < 9 ? (bwd ? 8 - i : i) : -1);
+  const int CPR = 2 * KS + 1;
+  // three blocks of positions per wave; two where three would leave compute units without a workgroup
+  // (7 x 7 x 512 at batch 64: 172 workgroups of three blocks 43.0 / 40.9 us, 256 of two 41.3 / 39.1)
+  const int mt = (Mo + T1_BM - 1) / T1_BM;
+  pl->SS = 1; pl->DT = DT;
+  pl->NB = (long long)((ts - P + 95) / 96) * mt < mfma_num_cus() ? 2 : 3;
+  p.SR = 32 * pl->NB + 2 * P + 2;
+  p.half = 0;
+  // the slab; the results are staged in the same memory afterwards (128 channels x 100 elements)
+  pl->lds_bytes = std::max((size_t)(((long long)p.SR * CPR + 63) / 64) * 1024, (size_t)T1_BM * (32 * pl->NB + 4) * esz);
+  if (pl->lds_bytes > 160 * 1024) return false;
+  p.ptiles = (p.TS - P + 32 * pl->NB - 1) / (32 * pl->NB);      // (the last zero row holds no result)
+  p.mtiles = (Mo + T1_BM - 1) / T1_BM;
+  const long long rb = ts * Cs * esz;
+  const long long wb = (long long)p.mtiles * (T1_BM / 32) * p.taps_total * KS * 1024;
+  const long long db = (long long)g.N * Mo * g.H * g.W * esz;
+  if (rb >= (1ll << 31) || wb >= (1ll << 31) || db >= (1ll << 31)) return false;
+  p.src_bytes = (unsigned)rb; p.w_bytes = (unsigned)wb; p.dst_bytes = (unsigned)db;
+  pl->rows_bytes = ((size_t)rb + 255) & ~(size_t)255;
+  pl->w_bytes = (size_t)wb;
+  w.Mo = Mo; w.Cc = Cc; w.KS = KS; w.taps_total = p.taps_total; w.bwd = bwd ? 1 : 0;
+  w.Cw = g.C; w.KW = 9; w.mblocks = p.mtiles * (T1_BM / 32);
+  pl->C = Cc; pl->H = g.H; pl->T = g.W;
+  return true;
+}
+
+template <typename T, int KS, int DT, int RW>
+int launch_conv2d(const Tap1Plan& pl, const T* xr, const uintx4_t* wf, const float* bias, T* dst, hipStream_t s) {
+  const dim3 grid((unsigned)pl.p.ptiles, (unsigned)pl.p.mtiles);
+  auto go = [&](auto kernel) {
+    if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), pl.lds_bytes)) return -1;
+    hipLaunchKernelGGL(kernel, grid, dim3(256), pl.lds_bytes, s, pl.p, xr, wf, bias, dst);
+    return check_launch("conv2d (3x3 windows over stacked planes)");
+  };
+  return pl.NB == 2 ? go(tap2d_conv_kernel<T, KS, DT, RW, 2>) : go(tap2d_conv_kernel<T, KS, DT, RW, 3>);
+}
+
+template <typename T>
+int run_conv2d(const ConvGeom& g, bool bwd, const void* src, const void* w, const float* bias, void* dst, hipStream_t s,
+               void* ws, size_t ws_bytes) {
+  Tap1Plan pl;
+  if (!tap2d_plan(g, bwd, (int)sizeof(T), &pl)) return -1;
+  if (!ws || ws_bytes < pl.rows_bytes + pl.w_bytes) return -1;
+  T* xr = static_cast<T*>(ws);
+  uintx4_t* wf = reinterpret_cast<uintx4_t*>(static_cast<char*>(ws) + pl.rows_bytes);
+  {
+    const dim3 grid((unsigned)((pl.p.TS + 63) / 64), (unsigned)((pl.p.Cs + 63) / 64));
+    hipLaunchKernelGGL(tap2d_rows_kernel<T>, grid, dim3(256), 0, s, static_cast<const T*>(src), xr, pl.C, g.H, g.W, g.N, pl.p.TS,
+                       pl.p.Cs);
+    const long long total = (long long)pl.w.mblocks * pl.w.taps_total * pl.w.KS * 64;
+    hipLaunchKernelGGL(tap_weights_by_tap_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+                       static_cast<const T*>(w), wf, pl.w);
+  }
+  if (const int rc = check_launch("conv2d (3x3 windows over stacked planes, operand passes)")) return rc;
+  T* out = static_cast<T*>(dst);
+  if constexpr (sizeof(T) == 2) {
+    switch (pl.p.KS) {
+      case 8: return launch_conv2d<T, 8, 2, 16>(pl, xr, wf, bias, out, s);
+      case 16: return launch_conv2d<T, 16, 1, 16>(pl, xr, wf, bias, out, s);
+      default: return launch_conv2d<T, 32, 1, 16>(pl, xr, wf, bias, out, s);
+    }
+  } else {
+    return pl.p.KS == 16 ? launch_conv2d<T, 16, 1, 4>(pl, xr, wf, bias, out, s) : launch_conv2d<T, 32, 1, 4>(pl, xr, wf, bias, out, s);
   }
 }
 
@@ -794,6 +1018,25 @@ int mfma_tap1d_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const
                              size_t ws_bytes) {
   if (dtype == FLHIP_F32) return run_conv<float>(g, true, dy, w, nullptr, dx, s, ws, ws_bytes);
   if (dtype == FLHIP_BF16) return run_conv<bf16_t>(g, true, dy, w, nullptr, dx, s, ws, ws_bytes);
+  return -1;
+}
+
+size_t mfma_tap2d_conv_ws(const ConvGeom& g, int dtype, bool bwd) {
+  Tap1Plan pl;
+  return esz_of(dtype) && tap2d_plan(g, bwd, esz_of(dtype), &pl) ? pl.rows_bytes + pl.w_bytes : 0;
+}
+
+int mfma_tap2d_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w, const float* bias, void* y, hipStream_t s,
+                        void* ws, size_t ws_bytes) {
+  if (dtype == FLHIP_F32) return run_conv2d<float>(g, false, x, w, bias, y, s, ws, ws_bytes);
+  if (dtype == FLHIP_BF16) return run_conv2d<bf16_t>(g, false, x, w, bias, y, s, ws, ws_bytes);
+  return -1;
+}
+
+int mfma_tap2d_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx, hipStream_t s, void* ws,
+                             size_t ws_bytes) {
+  if (dtype == FLHIP_F32) return run_conv2d<float>(g, true, dy, w, nullptr, dx, s, ws, ws_bytes);
+  if (dtype == FLHIP_BF16) return run_conv2d<bf16_t>(g, true, dy, w, nullptr, dx, s, ws, ws_bytes);
   return -1;
 }
 

@@ -833,6 +833,65 @@ def test_full_size_properties(shape, dtype):
     assert not yi[:, nd:].any()
 
 
+# 3x3 windows (stride 1, padding 1) on the kernels that walk every plane of the batch as one sequence with a zero
+# column after each row and a zero row between planes: the 14x14 and 7x7 layers of ResNet-50 at a small batch, every
+# padded contraction size they are compiled for (128, 256, 512; fp32: 128, 256), channel counts that are not multiples
+# of anything, planes that are not square, a single image, a sequence shorter than one tile, more result channels than
+# one workgroup's 128, planes above the size rule (TAP2D_ALL lifts it).  Forward and backward-data against the checker,
+# and against the kernels they replace.
+STACKED_PLANE_CASES = [
+    ((4, 256, 14, 14), (256, 256, 3, 3)),
+    ((5, 512, 7, 7), (512, 512, 3, 3)),
+    ((2, 128, 14, 14), (128, 128, 3, 3)),
+    ((3, 130, 9, 11), (70, 130, 3, 3)),
+    ((1, 100, 5, 5), (200, 100, 3, 3)),
+    ((2, 300, 6, 13), (150, 300, 3, 3)),
+    ((1, 96, 3, 2), (96, 96, 3, 3)),
+    ((2, 72, 28, 28), (136, 72, 3, 3)),
+    ((7, 256, 1, 1), (256, 256, 3, 3)),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("case", STACKED_PLANE_CASES)
+def test_3x3_windows_over_stacked_planes(case, dtype):
+    from flashlight_amd import capi
+    xs, ws = case
+    lo = dtype == torch.bfloat16
+    if not lo and max(xs[1], ws[0]) > 256:
+        pytest.skip("fp32: at most 256 contraction channels")
+    full = (xs, ws, (1, 1), (1, 1), (1, 1), 1)
+    capi.set_option("TAP2D_ALL", "1")
+    try:
+        res = _run(full, 47, dtype)
+        # the family named as a plan takes these geometries
+        import ctypes as C
+        L = capi.lib()
+        cd = capi.ConvDesc(xs[0], xs[1], xs[2], xs[3], ws[0], 3, 3, 1, 1, 1, 1, 1, 1, 1, capi.BF16 if lo else capi.F32)
+        nws = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_BWD_DATA)
+        wsb = torch.empty(max(nws, 16), dtype=torch.uint8, device="cuda")
+        dyd = torch.zeros((xs[0], ws[0], xs[2], xs[3]), device="cuda", dtype=dtype)
+        wd = torch.zeros(ws, device="cuda", dtype=dtype)
+        out = torch.full(xs, 7.0, device="cuda", dtype=dtype)
+        P = lambda t: C.c_void_p(t.data_ptr())
+        rc = L.flhip_conv2d_bwd_data_plan(C.byref(cd), P(dyd), P(wd), P(out), P(wsb), nws, 12,
+                                          C.c_void_p(torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        assert rc == 0 and bool((out == 0).all())
+    finally:
+        capi.set_option("TAP2D_ALL", None)
+    for name, (got, ref) in res.items():
+        tight = 1e-4 if (name in ("dw", "db") or not lo) else 4e-3
+        assert got.shape == ref.shape and rel_l2(got, ref) <= tight, (name, rel_l2(got, ref))
+    capi.set_option("CONV_SKIP", "tap2d")
+    try:
+        old = _run(full, 47, dtype)
+    finally:
+        capi.set_option("CONV_SKIP", None)
+    for name in ("y", "dx", "y_nobias"):
+        assert rel_l2(res[name][0], old[name][0]) <= (6e-3 if lo else 1e-4), name
+
+
 # Backward-data of stride-2 windows over at most 4 input channels (the kernel that works on 2 x 2 cells of the input
 # gradient): the stem's 7x7 / pad 3 with 1 to 4 channels, windows of 3 to 8 rows and columns with every padding that
 # keeps the cell's window within 4 x 4, odd input sizes (a last cell of one row / column), planes narrower and wider
