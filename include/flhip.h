@@ -126,10 +126,10 @@ const char* flhip_arch(void);
  * (value NULL restores the default; the FLHIP_ prefix on `name` is optional).  Not to be
  * called while another thread is inside the library.  Results stay within the stated
  * tolerances under every setting; the switches only choose between kernels.
- *   CONV_ALGO = direct | gather | tapped | convert | auto    CONV_SKIP = bf16,gemm1x1,slab,tapped,strip,first,wgrad128,pwdma,wd32,tap1d
+ *   CONV_ALGO = direct | gather | tapped | convert | auto    CONV_SKIP = bf16,gemm1x1,slab,tapped,strip,first,wgrad128,pwdma,wd32,tap1d,cells,tap2d
  *   PW_PT = 2 | 4 | 8    PW16_PF = 0 | 1 | 2 | 4 | 8    CONV_STACK = 0 | 1 | 2 | 4 | 8    BN_ALGO = split | resident | auto
  *   SLAB_WAVES = 0 | 4 | 8
- *   PW16_NO_TAPS, TAPPED_NO_REORDER, MATMUL_VALU, RNN_UNFUSED = 1 | 0
+ *   PW16_NO_TAPS, TAPPED_NO_REORDER, MATMUL_VALU, RNN_UNFUSED, TAP2D_ALL = 1 | 0
  * Unknown names or values return FLHIP_INVALID_ARGUMENT.  The nearest thing in the
  * reference is the kernel-choice options object of its cuDNN extension
  * (createBenchmarkOptions, flashlight/fl/autograd/tensor/backend/cudnn/CudnnAutogradExtension.h:25). */
