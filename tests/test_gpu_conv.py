@@ -701,6 +701,44 @@ def test_random_one_row_windows(case):
             assert rel_l2(got, ref) <= lim, (case, dtype, name, rel_l2(got, ref))
 
 
+def _random_new_family_cases(n, seed):
+    """Seeded random geometries of the two newest kernel families: 3x3 / stride 1 / padding 1 over small planes with 65
+    to 512 channels on either side (stacked planes), and stride-2 windows of 3 to 8 rows / columns over 1 to 4 input
+    channels with any padding below the window (2 x 2 cells; paddings that spread a cell's window over 5 rows fall
+    to the other kernels, which the comparison covers as well)."""
+    rng = np.random.default_rng(seed)
+    cases = []
+    for i in range(n):
+        if i % 2 == 0:
+            N, H, W = int(rng.integers(1, 7)), int(rng.integers(1, 16)), int(rng.integers(1, 16))
+            C, K = int(rng.integers(65, 513)), int(rng.integers(1, 300))
+            if i % 4 == 0:
+                C, K = K + 64, C                       # the long side as the result channels (backward: the contraction)
+            cases.append(((N, C, H, W), (K, C, 3, 3), (1, 1), (1, 1), (1, 1), 1))
+        else:
+            kh, kw = int(rng.integers(3, 9)), int(rng.integers(3, 9))
+            py, px = int(rng.integers(0, kh)), int(rng.integers(0, kw))
+            H, W = int(rng.integers(kh, 60)), int(rng.integers(kw, 150))
+            N, C, K = int(rng.integers(1, 4)), int(rng.integers(1, 5)), 4 * int(rng.integers(1, 20))
+            cases.append(((N, C, H, W), (K, C, kh, kw), (2, 2), (py, px), (1, 1), 1))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_new_family_cases(28, 20251127))
+def test_random_stacked_planes_and_cells(case):
+    from flashlight_amd import capi
+    capi.set_option("TAP2D_ALL", "1")
+    try:
+        for dtype in (torch.float32, torch.bfloat16):
+            if dtype == torch.float32 and case[2] == (1, 1) and max(case[0][1], case[1][0]) > 256:
+                continue
+            for name, (got, ref) in _run(case, 59, dtype).items():
+                lim = F32_TOL if dtype == torch.float32 or name in ("dw", "db") else 4e-3
+                assert got.shape == ref.shape and rel_l2(got, ref) <= lim, (case, dtype, name, rel_l2(got, ref))
+    finally:
+        capi.set_option("TAP2D_ALL", None)
+
+
 def test_invalid_arguments_raise():
     x = torch.zeros((1, 4, 8, 8), device="cuda")
     w = torch.zeros((4, 3, 3, 3), device="cuda")
