@@ -144,7 +144,7 @@ static const unsigned SK_BF16 = Options::SKIP_BF16, SK_GEMM = Options::SKIP_GEMM
 // the one-row-window kernels take this storage type (bf16: unless the bf16 families are switched off or converted)
 static bool tap1d_on(int dtype) {
   if (force_direct() || skip(Options::SKIP_TAP1D)) return false;
-  return dtype == FLHIP_F32 || (dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT));
+  return dtype == FLHIP_F32 || ((dtype == FLHIP_BF16 || dtype == FLHIP_F16) && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT));
 }
 
 // 3x3 windows over stacked planes: bf16, planes of at most 64 positions (the 7 x 7 layers) and a sequence of at least
@@ -154,7 +154,7 @@ static bool tap1d_on(int dtype) {
 static bool tap2d_on(const ConvGeom& g, int dtype) {
   if (!tap1d_on(dtype) || skip(Options::SKIP_TAP2D)) return false;
   if (options().tap2d_all) return true;
-  return dtype == FLHIP_BF16 && g.H * g.W <= 64 && (long long)g.N * (g.H + 1) * (g.W + 1) >= 2048;
+  return (dtype == FLHIP_BF16 || dtype == FLHIP_F16) && g.H * g.W <= 64 && (long long)g.N * (g.H + 1) * (g.W + 1) >= 2048;
 }
 
 static bool long_rows(const ConvGeom& g, int dtype, bool bwd, size_t ws_bytes) {

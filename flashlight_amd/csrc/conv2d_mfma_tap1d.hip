@@ -48,6 +48,7 @@ namespace flhip {
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
 #if defined(__HIP_DEVICE_COMPILE__)
 typedef __attribute__((address_space(3))) const uintx4_t* lds_cell_t;
 #else
@@ -61,12 +62,20 @@ constexpr int T1_OOB = (int)0x80000000;
 // element type -> channels per 16-byte cell; a stage is two cells
 template <typename T> struct Tap1Elem;
 template <> struct Tap1Elem<bf16_t> { static constexpr int CELL = 8; };
+template <> struct Tap1Elem<f16_t> { static constexpr int CELL = 8; };
 template <> struct Tap1Elem<float> { static constexpr int CELL = 4; };
 
 // one stage of one block: acc += a (positions x stage channels) * w (stage channels x result channels)
 __device__ __forceinline__ void tap1d_mma(floatx16& acc, const uintx4_t& a, const uintx4_t& w, const bf16_t*) {
   acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, w), acc, 0, 0, 0);
 }
+__device__ __forceinline__ void tap1d_mma(floatx16& acc, const uintx4_t& a, const uintx4_t& w, const f16_t*) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, w), acc, 0, 0, 0);
+}
+// two results rounded to the storage type, the first in the low half
+__device__ __forceinline__ uint32_t tap1d_pack(float a, float b, const bf16_t*) { return pack_bf16(a, b); }
+__device__ __forceinline__ uint32_t tap1d_pack(float a, float b, const f16_t*) { return pack_f16(a, b); }
+__device__ __forceinline__ uint32_t tap1d_pack(float, float, const float*) { return 0u; }   // (fp32 results are not packed)
 __device__ __forceinline__ void tap1d_mma(floatx16& acc, const uintx4_t& a, const uintx4_t& w, const float*) {
 #pragma unroll
   for (int e = 0; e < 4; ++e)
@@ -379,10 +388,12 @@ tap_conv_body(const Tap1Params& p, const T* __restrict__ xr, const uintx4_t* __r
           if (NPH == 2)
             __builtin_amdgcn_raw_buffer_store_b128(uintx4_t{__float_as_uint(v[4]), __float_as_uint(v[5]), __float_as_uint(v[6]), __float_as_uint(v[7])}, drs, at + 16, 0, 0);
         } else if (NPH == 1) {
-          const uintx2_t t = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
+          const T* const tt = nullptr;
+          const uintx2_t t = {tap1d_pack(v[0], v[1], tt), tap1d_pack(v[2], v[3], tt)};
           __builtin_amdgcn_raw_buffer_store_b64(t, drs, at, 0, 0);
         } else {
-          const uintx4_t t = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])};
+          const T* const tt = nullptr;
+          const uintx4_t t = {tap1d_pack(v[0], v[1], tt), tap1d_pack(v[2], v[3], tt), tap1d_pack(v[4], v[5], tt), tap1d_pack(v[6], v[7], tt)};
           __builtin_amdgcn_raw_buffer_store_b128(t, drs, at, 0, 0);
         }
       } else {
@@ -773,7 +784,7 @@ tap1d_wgrad_kernel(Tap1WParams p, const T* __restrict__ xr, const T* __restrict_
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][t][r] = 0.f;
   // a tile of ones for the bias slot
-  const uint32_t one = LO ? 0x3f803f80u : 0x3f800000u;
+  const uint32_t one = !LO ? 0x3f800000u : std::is_same<T, f16_t>::value ? 0x3c003c00u : 0x3f803f80u;
   const uintx4_t ones = {one, one, one, one};
   const int bias_slot = p.KW - wave * TQ;       // this wave's slot index of the bias gradient (outside 0 .. TQ - 1: none)
 
@@ -998,7 +1009,7 @@ int run_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float
   return check_launch("conv2d_bwd_filter (one-row windows, sum)");
 }
 
-int esz_of(int dtype) { return dtype == FLHIP_F32 ? 4 : dtype == FLHIP_BF16 ? 2 : 0; }
+int esz_of(int dtype) { return dtype == FLHIP_F32 ? 4 : dtype == FLHIP_BF16 || dtype == FLHIP_F16 ? 2 : 0; }
 
 }  // namespace
 
@@ -1011,6 +1022,7 @@ int mfma_tap1d_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void*
                         void* ws, size_t ws_bytes) {
   if (dtype == FLHIP_F32) return run_conv<float>(g, false, x, w, bias, y, s, ws, ws_bytes);
   if (dtype == FLHIP_BF16) return run_conv<bf16_t>(g, false, x, w, bias, y, s, ws, ws_bytes);
+  if (dtype == FLHIP_F16) return run_conv<f16_t>(g, false, x, w, bias, y, s, ws, ws_bytes);
   return -1;
 }
 
@@ -1018,6 +1030,7 @@ int mfma_tap1d_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const
                              size_t ws_bytes) {
   if (dtype == FLHIP_F32) return run_conv<float>(g, true, dy, w, nullptr, dx, s, ws, ws_bytes);
   if (dtype == FLHIP_BF16) return run_conv<bf16_t>(g, true, dy, w, nullptr, dx, s, ws, ws_bytes);
+  if (dtype == FLHIP_F16) return run_conv<f16_t>(g, true, dy, w, nullptr, dx, s, ws, ws_bytes);
   return -1;
 }
 
@@ -1030,6 +1043,7 @@ int mfma_tap2d_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void*
                         void* ws, size_t ws_bytes) {
   if (dtype == FLHIP_F32) return run_conv2d<float>(g, false, x, w, bias, y, s, ws, ws_bytes);
   if (dtype == FLHIP_BF16) return run_conv2d<bf16_t>(g, false, x, w, bias, y, s, ws, ws_bytes);
+  if (dtype == FLHIP_F16) return run_conv2d<f16_t>(g, false, x, w, bias, y, s, ws, ws_bytes);
   return -1;
 }
 
@@ -1037,6 +1051,7 @@ int mfma_tap2d_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const
                              size_t ws_bytes) {
   if (dtype == FLHIP_F32) return run_conv2d<float>(g, true, dy, w, nullptr, dx, s, ws, ws_bytes);
   if (dtype == FLHIP_BF16) return run_conv2d<bf16_t>(g, true, dy, w, nullptr, dx, s, ws, ws_bytes);
+  if (dtype == FLHIP_F16) return run_conv2d<f16_t>(g, true, dy, w, nullptr, dx, s, ws, ws_bytes);
   return -1;
 }
 
@@ -1056,6 +1071,7 @@ int mfma_tap1d_wgrad(const ConvGeom& g, int dtype, const void* x, const void* dy
                      hipStream_t s, const void* rows) {
   if (dtype == FLHIP_F32) return run_wgrad<float>(g, x, dy, dw, db, ws, ws_bytes, s, rows);
   if (dtype == FLHIP_BF16) return run_wgrad<bf16_t>(g, x, dy, dw, db, ws, ws_bytes, s, rows);
+  if (dtype == FLHIP_F16) return run_wgrad<f16_t>(g, x, dy, dw, db, ws, ws_bytes, s, rows);
   return -1;
 }
 

@@ -5,7 +5,7 @@
 // run, the device time per operation class (HIP events around every operation of the
 // host layer) with the idle gaps between operations.
 //
-// usage: flhip_step_bench resnet50|speech [batch] [steps] [warmup] [f32|bf16] [unfused|fused] [sgd]
+// usage: flhip_step_bench resnet50|speech [batch] [steps] [warmup] [f32|bf16|f16] [unfused|fused] [sgd]
 // ("unfused": BatchNorm, residual add and ReLU as three operations, the reference's composition; "sgd": the step ends
 // with fl::SGDOptimizer::step - momentum 0.9, weight decay 1e-4 - on the ResNet's parameters)
 #include <chrono>
@@ -53,7 +53,9 @@ int main(int argc, char** argv) {
     const int B = argc > 2 ? std::atoi(argv[2]) : (model == "speech" ? 16 : 64);
     const int steps = argc > 3 ? std::atoi(argv[3]) : 10;
     const int warmup = argc > 4 ? std::atoi(argv[4]) : 3;
-    const bool half = argc > 5 && std::string(argv[5]) == "bf16";
+    const std::string dname = argc > 5 ? argv[5] : "f32";
+    const bool half = dname == "bf16" || dname == "f16";
+    const dtype lowType = dname == "f16" ? dtype::f16 : dtype::bf16;
     const bool unfused = argc > 6 && std::string(argv[6]) == "unfused";
     const bool sgd = argc > 7 && std::string(argv[7]) == "sgd";
     pkg::vision::setFusedBatchNormRelu(!unfused);
@@ -72,7 +74,7 @@ int main(int argc, char** argv) {
     if (model == "resnet50") {
       net = pkg::vision::resnet50();
       Tensor x = Tensor::fromVector({224, 224, 3, B}, randn((size_t)B * 3 * 224 * 224, 1));
-      in = Variable(half ? x.astype(dtype::bf16) : x, false);
+      in = Variable(half ? x.astype(lowType) : x, false);
       std::vector<int32_t> labels(B);
       std::mt19937 gen(5);
       for (int i = 0; i < B; ++i) labels[i] = (int32_t)(gen() % 1000);
@@ -94,9 +96,9 @@ int main(int argc, char** argv) {
         flop += 3.0 * 2.0 * B * chans[l + 1] * (double)(T / strides[l]) * chans[l] * 21;
       }
       Tensor x = Tensor::fromVector({T, 1, 80, B}, randn((size_t)B * 80 * T, 71));
-      in = Variable(half ? x.astype(dtype::bf16) : x, true);
+      in = Variable(half ? x.astype(lowType) : x, true);
       Tensor g = Tensor::fromVector({T / 2, 1, 250, B}, randn((size_t)B * 250 * (T / 2), 72));
-      gradOut = Variable(half ? g.astype(dtype::bf16) : g, false);
+      gradOut = Variable(half ? g.astype(lowType) : g, false);
       step = [&]() {
         for (auto& c : convs) c.zeroGrad();
         for (auto& b : bns) b.zeroGrad();
@@ -137,7 +139,7 @@ int main(int argc, char** argv) {
     std::printf("{\"model\": \"%s\", \"batch\": %d, \"dtype\": \"%s\", \"fused_bn_relu\": %s, \"optimizer\": \"%s\", \"steps\": %d, \"warmup\": %d, \"ms_per_step\": %.4f, "
                 "\"samples_per_s\": %.1f, \"loss\": %.5f, \"conv_gflop_per_step\": %.2f, \"device_cache_mb\": %.1f, "
                 "\"breakdown_ms\": {",
-                model.c_str(), B, half ? "bf16" : "f32", unfused ? "false" : "true", opt ? "sgd momentum 0.9 weight decay 1e-4" : "none", steps, warmup, ms, B / ms * 1e3, loss, flop / 1e9,
+                model.c_str(), B, half ? dname.c_str() : "f32", unfused ? "false" : "true", opt ? "sgd momentum 0.9 weight decay 1e-4" : "none", steps, warmup, ms, B / ms * 1e3, loss, flop / 1e9,
                 deviceCacheBytes() / 1e6);
     bool first = true;
     for (const auto& kv : classes) {

@@ -195,11 +195,11 @@ ONE_ROW_CASES = [
 ]
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 @pytest.mark.parametrize("case", ONE_ROW_CASES)
 def test_conv_one_row_windows(case, dtype):
     from flashlight_amd import capi
-    lo = dtype == torch.bfloat16
+    lo = dtype != torch.float32
     res = _run(case, 38, dtype)
     for name, (got, ref) in res.items():
         tight = 1e-4 if (name in ("dw", "db") or not lo) else 4e-3
@@ -214,8 +214,8 @@ def test_conv_one_row_windows(case, dtype):
         assert rel_l2(res[name][0], old[name][0]) <= (6e-3 if lo else 1e-4), name
 
 
-# f16 storage goes through the kernels that widen their operands to fp32 (the bf16 matrix-core families are
-# not taken): every case once, inputs exact in f16, fp32 sums, results rounded once (2^-12 relative).
+# f16 storage goes through the kernels that widen their operands to fp32 (of the 16-bit matrix-core families only the
+# one-row-window kernels, and their use for 3x3 windows over 7x7 planes, are compiled for it): every case once, inputs exact in f16, fp32 sums, results rounded once (2^-12 relative).
 @pytest.mark.parametrize("case", ALL)
 def test_conv_f16(case):
     for name, (got, ref) in _run(case, 37, torch.float16).items():
@@ -603,7 +603,7 @@ def test_bf16_filter_gradient_from_the_forward_pass_gather(shape, with_bias):
 @pytest.mark.parametrize("shape", [((3, 80, 1, 180), (250, 80, 1, 21), (1, 1), (0, 10)),
                                    ((3, 250, 1, 180), (250, 250, 1, 21), (1, 2), (0, 10)),
                                    ((2, 32, 3, 50), (40, 32, 1, 5), (1, 1), (0, 2))])        # 5 taps: that filter gradient declines
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 def test_one_row_filter_gradient_from_the_forward_pass_rows(shape, dtype):
     """One-row windows: the forward pass leaves its channels-last rows at the start of its workspace; the filter
     gradient computed from them equals the one that makes the rows again, bit for bit."""
@@ -618,7 +618,7 @@ def test_one_row_filter_gradient_from_the_forward_pass_rows(shape, dtype):
         assert rows is None
         return
     cs = 96 if xs[1] == 80 else 256
-    esz = 2 if dtype == torch.bfloat16 else 4
+    esz = 4 if dtype == torch.float32 else 2
     assert rows is not None and rows.numel() >= xs[0] * xs[2] * xs[3] * cs * esz
     # the rows are the input with its channels last, padded with zeros
     r = rows[:xs[0] * xs[2] * xs[3] * cs * esz].view(dtype).view(xs[0], xs[2], xs[3], cs)
@@ -729,7 +729,7 @@ def test_random_stacked_planes_and_cells(case):
     from flashlight_amd import capi
     capi.set_option("TAP2D_ALL", "1")
     try:
-        for dtype in (torch.float32, torch.bfloat16):
+        for dtype in (torch.float32, torch.bfloat16, torch.float16):
             if dtype == torch.float32 and case[2] == (1, 1) and max(case[0][1], case[1][0]) > 256:
                 continue
             for name, (got, ref) in _run(case, 59, dtype).items():
@@ -891,12 +891,12 @@ STACKED_PLANE_CASES = [
 
 
 # (fp32: at most 256 contraction channels)
-@pytest.mark.parametrize("case,dtype", [(c, dt) for c in STACKED_PLANE_CASES for dt in (torch.bfloat16, torch.float32)
-                                        if dt == torch.bfloat16 or max(c[0][1], c[1][0]) <= 256])
+@pytest.mark.parametrize("case,dtype", [(c, dt) for c in STACKED_PLANE_CASES for dt in (torch.bfloat16, torch.float32, torch.float16)
+                                        if dt != torch.float32 or max(c[0][1], c[1][0]) <= 256])
 def test_3x3_windows_over_stacked_planes(case, dtype):
     from flashlight_amd import capi
     xs, ws = case
-    lo = dtype == torch.bfloat16
+    lo = dtype != torch.float32
     full = (xs, ws, (1, 1), (1, 1), (1, 1), 1)
     capi.set_option("TAP2D_ALL", "1")
     try:
@@ -904,7 +904,8 @@ def test_3x3_windows_over_stacked_planes(case, dtype):
         # the family named as a plan takes these geometries
         import ctypes as C
         L = capi.lib()
-        cd = capi.ConvDesc(xs[0], xs[1], xs[2], xs[3], ws[0], 3, 3, 1, 1, 1, 1, 1, 1, 1, capi.BF16 if lo else capi.F32)
+        cd = capi.ConvDesc(xs[0], xs[1], xs[2], xs[3], ws[0], 3, 3, 1, 1, 1, 1, 1, 1, 1,
+                           capi.F32 if not lo else capi.BF16 if dtype == torch.bfloat16 else capi.F16)
         nws = L.flhip_conv2d_workspace_bytes(C.byref(cd), capi.CONV_BWD_DATA)
         wsb = torch.empty(max(nws, 16), dtype=torch.uint8, device="cuda")
         dyd = torch.zeros((xs[0], ws[0], xs[2], xs[3]), device="cuda", dtype=dtype)
