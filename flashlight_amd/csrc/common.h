@@ -302,6 +302,8 @@ inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s);
 
 inline bool dtype_ok(int32_t dt) { return dt == FLHIP_F32 || dt == FLHIP_BF16 || dt == FLHIP_F16; }
 inline size_t dtype_size(int32_t dt) { return dt == FLHIP_F32 ? 4 : 2; }
+// the two 16-bit storage types (bf16 and IEEE half share the 16-bit matrix-core kernels)
+inline bool is_lo16(int32_t dt) { return dt == FLHIP_BF16 || dt == FLHIP_F16; }
 
 // Calls f with a null pointer of the storage type of `dt`:
 //   by_dtype(dt, [&](auto* t) { using T = std::remove_pointer_t<decltype(t)>; return launch<T>(...); })

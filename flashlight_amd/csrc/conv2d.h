@@ -44,15 +44,15 @@ int mfma_pointwise_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, c
 // gradient) and return -1 without it; so do the backward passes of strided windows with 2 to 9
 // taps, which gather the taps next to the channels (bwd = true in the query).
 int mfma_pointwise16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
-                              hipStream_t s, void* ws = nullptr, size_t ws_bytes = 0);
+                              hipStream_t s, void* ws, size_t ws_bytes, int dtype);
 int mfma_pointwise16_conv_bwd_data_add(const ConvGeom& g, const void* dy, const void* w, const void* addend, void* dx,
-                                       hipStream_t s);
+                                       hipStream_t s, int dtype);
 int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s,
-                                   void* ws = nullptr, size_t ws_bytes = 0);
+                                   void* ws, size_t ws_bytes, int dtype);
 size_t mfma_pointwise16_lattice_ws(const ConvGeom& g, bool bwd);
 size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g);
 int mfma_pointwise16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
-                           size_t ws_bytes, hipStream_t s, const void* gathered = nullptr);
+                           size_t ws_bytes, hipStream_t s, const void* gathered, int dtype);
 // bytes of gathered input that the forward pass leaves at the start of its workspace for the filter gradient (0: none)
 size_t mfma_pointwise16_gathered_bytes(const ConvGeom& g);
 // fp32, stride 1, few tiles and a long contraction: the contraction in slices through
@@ -91,10 +91,10 @@ void wgrad_reduce_launch(const float* part, int nsplit, int E, int K, int want_d
 // bf16 forward of a first layer: few input channels, window rows of at most 8 columns, even column stride
 // (conv2d_mfma_first_bf16.hip)
 int mfma_first16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
-                          hipStream_t s);
+                          hipStream_t s, int dtype);
 size_t mfma_first16_wgrad_ws(const ConvGeom& g);
 int mfma_first16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
-                       size_t ws_bytes, hipStream_t s);
+                       size_t ws_bytes, hipStream_t s, int dtype);
 // backward-data of a stride-2 window over at most 4 input channels (the stem), any storage type, as a 4 x 4
 // stride-1 window over the output gradient onto the 2 x 2 cells of the input gradient (conv2d_mfma_cells.hip)
 int mfma_cells_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx, hipStream_t s);
@@ -102,21 +102,23 @@ int mfma_cells_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const
 // bf16 1x1 stride-1 convolutions with operand tiles copied to LDS by the loads themselves
 // (conv2d_mfma_pointwise_dma_bf16.hip); -1 when the shape is not theirs.  addend (or null): added
 // to the rounded input gradient.
-int mfma_pwd16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y, hipStream_t s);
+int mfma_pwd16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y, hipStream_t s,
+                        int dtype = FLHIP_BF16);
 int mfma_pwd16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, const void* addend, void* dx,
-                             hipStream_t s);
+                             hipStream_t s, int dtype);
 // their filter gradient (no bias gradient; at least 128 channels on both sides); partial tiles in ws
 size_t mfma_pwd16_wgrad_ws(const ConvGeom& g);
 // workgroups the bf16 slab kernel's forward pass would launch (0: not its shape)
 long long mfma_slab16_conv_fwd_workgroups(const ConvGeom& g);
-int mfma_pwd16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, void* ws, size_t ws_bytes, hipStream_t s);
+int mfma_pwd16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, void* ws, size_t ws_bytes, hipStream_t s,
+                     int dtype = FLHIP_BF16);
 int mfma_strip16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
-                          hipStream_t s);
-int mfma_strip16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s);
+                          hipStream_t s, int dtype);
+int mfma_strip16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s, int dtype);
 int mfma_slab16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
-                         hipStream_t s);
+                         hipStream_t s, int dtype);
 int mfma_slab16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx,
-                              hipStream_t s);
+                              hipStream_t s, int dtype);
 // windows of one row (KH = 1, 2 to 32 taps, column stride 1 or 2, no groups, 16 to 256 contraction channels) in bf16
 // or fp32 storage through channels-last rows and fragment-ordered weights in mfma_tap1d_conv_ws() bytes of workspace
 // (conv2d_mfma_tap1d.hip); -1 when the shape is not theirs or the room is missing
@@ -145,9 +147,9 @@ size_t mfma_tap1d_rows_bytes(const ConvGeom& g, int dtype);
 size_t mfma_wgrad_dma16_ws(const ConvGeom& g);
 // tile: 0 = by the measured rule, 32 / 64 = that tile side or decline
 int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes,
-                     hipStream_t s, int tile = 0);
+                     hipStream_t s, int tile, int dtype);
 size_t mfma_wgrad16_ws(const ConvGeom& g);
 int mfma_wgrad16(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
-                 size_t ws_bytes, hipStream_t s);
+                 size_t ws_bytes, hipStream_t s, int dtype);
 
 }  // namespace flhip

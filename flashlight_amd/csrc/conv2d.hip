@@ -209,12 +209,12 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
     // the larger of the two filter-gradient plans, so either kernel can run
     size_t a = mfma_conv_bwd_filter_ws(g, d->dtype);
     const size_t b = mfma_slab_wgrad_ws(g, d->dtype);
-    size_t c = d->dtype == FLHIP_BF16 ? mfma_wgrad16_ws(g) : 0;
-    const size_t c2 = d->dtype == FLHIP_BF16 ? mfma_wgrad_dma16_ws(g) : 0;
+    size_t c = is_lo16(d->dtype) ? mfma_wgrad16_ws(g) : 0;
+    const size_t c2 = is_lo16(d->dtype) ? mfma_wgrad_dma16_ws(g) : 0;
     if (c2 > c) c = c2;
     const size_t e = mfma_pointwise_wgrad_ws(g);
-    const size_t f = d->dtype == FLHIP_BF16 ? mfma_pointwise16_wgrad_ws(g) : 0;
-    const size_t h = d->dtype == FLHIP_BF16 ? mfma_first16_wgrad_ws(g) : 0;
+    const size_t f = is_lo16(d->dtype) ? mfma_pointwise16_wgrad_ws(g) : 0;
+    const size_t h = is_lo16(d->dtype) ? mfma_first16_wgrad_ws(g) : 0;
     const size_t t1 = mfma_tap1d_wgrad_ws(g, d->dtype);
     if (h > a) a = h;
     if (t1 > a) a = t1;
@@ -228,7 +228,7 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
   // (bf16: strided 1x1 windows gather the input's lattice points / spread a compact gradient)
   if (pass == FLHIP_CONV_FWD || pass == FLHIP_CONV_BWD_DATA) {
     const size_t a = mfma_tapped_ws(g, d->dtype, pass == FLHIP_CONV_BWD_DATA);
-    const size_t b = d->dtype == FLHIP_BF16 ? mfma_pointwise16_lattice_ws(g, pass == FLHIP_CONV_BWD_DATA)
+    const size_t b = is_lo16(d->dtype) ? mfma_pointwise16_lattice_ws(g, pass == FLHIP_CONV_BWD_DATA)
                                             : pass == FLHIP_CONV_BWD_DATA ? mfma_pointwise_split_ws(g, d->dtype, true) : 0;
     const size_t c = mfma_tap1d_conv_ws(g, d->dtype, pass == FLHIP_CONV_BWD_DATA);
     const size_t c2 = tap2d_on(g, d->dtype) ? mfma_tap2d_conv_ws(g, d->dtype, pass == FLHIP_CONV_BWD_DATA) : 0;
@@ -249,16 +249,16 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
     int r = -1;
     if (tap1d_on(d->dtype)) r = mfma_tap1d_conv_fwd(g, d->dtype, x, w, bias, y, s, ws, ws_bytes);
     if (r < 0 && tap2d_on(g, d->dtype)) r = mfma_tap2d_conv_fwd(g, d->dtype, x, w, bias, y, s, ws, ws_bytes);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_pwd16_conv_fwd(g, x, w, bias, y, s);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_pointwise16_conv_fwd(g, x, w, bias, y, s, ws, ws_bytes);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_FIRST) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_first16_conv_fwd(g, x, w, bias, y, s);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_STRIP) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_strip16_conv_fwd(g, x, w, bias, y, s);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_slab16_conv_fwd(g, x, w, bias, y, s);
+    if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_pwd16_conv_fwd(g, x, w, bias, y, s, d->dtype);
+    if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_pointwise16_conv_fwd(g, x, w, bias, y, s, ws, ws_bytes, d->dtype);
+    if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !skip(Options::SKIP_FIRST) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_first16_conv_fwd(g, x, w, bias, y, s, d->dtype);
+    if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !skip(Options::SKIP_STRIP) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_strip16_conv_fwd(g, x, w, bias, y, s, d->dtype);
+    if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_slab16_conv_fwd(g, x, w, bias, y, s, d->dtype);
     if (r < 0 && !skip(SK_GEMM)) r = mfma_pointwise_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r < 0 && algo_is(Options::ALGO_TAPPED)) r = mfma_tapped_conv_fwd(g, d->dtype, x, w, bias, y, s, ws, ws_bytes);
     if (r < 0 && !skip(SK_SLAB)) r = mfma_slab_conv_fwd(g, d->dtype, x, w, bias, y, s);
@@ -312,13 +312,13 @@ static int bwd_data_impl(const flhip_conv_desc* d, const void* dy, const void* w
   hipStream_t s = as_stream(stream);
   if (plan >= 0) {
     FLHIP_REQUIRE(plan < kNumDataPlans, "conv2d_bwd_data: unknown plan");
-    const bool lo = d->dtype == FLHIP_BF16;
+    const bool lo = is_lo16(d->dtype);
     int r = -1;
     switch (plan) {
-      case 0: if (lo) r = mfma_pwd16_conv_bwd_data(g, dy, w, nullptr, dx, s); break;
-      case 1: if (lo) r = mfma_pointwise16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes); break;
-      case 2: if (lo) r = mfma_strip16_conv_bwd_data(g, dy, w, dx, s); break;
-      case 3: if (lo) r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s); break;
+      case 0: if (lo) r = mfma_pwd16_conv_bwd_data(g, dy, w, nullptr, dx, s, d->dtype); break;
+      case 1: if (lo) r = mfma_pointwise16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes, d->dtype); break;
+      case 2: if (lo) r = mfma_strip16_conv_bwd_data(g, dy, w, dx, s, d->dtype); break;
+      case 3: if (lo) r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s, d->dtype); break;
       case 4: r = mfma_pointwise_conv_split(g, d->dtype, true, dy, w, nullptr, dx, ws, ws_bytes, s); break;
       case 5: r = mfma_pointwise_conv_bwd_data(g, d->dtype, dy, w, dx, s); break;
       case 6: r = mfma_slab_conv_bwd_data(g, d->dtype, dy, w, dx, s); break;
@@ -336,14 +336,14 @@ static int bwd_data_impl(const flhip_conv_desc* d, const void* dy, const void* w
     if (tap1d_on(d->dtype)) r = mfma_tap1d_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
     if (r < 0 && tap2d_on(g, d->dtype)) r = mfma_tap2d_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
     if (r < 0 && !skip(Options::SKIP_CELLS)) r = mfma_cells_conv_bwd_data(g, d->dtype, dy, w, dx, s);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_pwd16_conv_bwd_data(g, dy, w, nullptr, dx, s);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_pointwise16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_STRIP) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_strip16_conv_bwd_data(g, dy, w, dx, s);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s);
+    if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_pwd16_conv_bwd_data(g, dy, w, nullptr, dx, s, d->dtype);
+    if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_pointwise16_conv_bwd_data(g, dy, w, dx, s, ws, ws_bytes, d->dtype);
+    if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !skip(Options::SKIP_STRIP) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_strip16_conv_bwd_data(g, dy, w, dx, s, d->dtype);
+    if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_slab16_conv_bwd_data(g, dy, w, dx, s, d->dtype);
     if (r < 0 && !skip(SK_GEMM)) r = mfma_pointwise_conv_split(g, d->dtype, true, dy, w, nullptr, dx, ws, ws_bytes, s);
     if (r < 0 && !skip(SK_GEMM)) r = mfma_pointwise_conv_bwd_data(g, d->dtype, dy, w, dx, s);
     if (r < 0 && algo_is(Options::ALGO_TAPPED)) r = mfma_tapped_conv_bwd_data(g, d->dtype, dy, w, dx, s, ws, ws_bytes);
@@ -388,9 +388,9 @@ extern "C" int flhip_conv2d_bwd_data_add(const flhip_conv_desc* d, const void* d
   // after another workgroup may have written it (planes that are not a multiple of 8 positions), the others
   // write dx before they read addend
   FLHIP_REQUIRE(dx != addend, "conv2d_bwd_data_add: dx aliases addend");
-  if (!force_direct() && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT)) {
-    int r = skip(Options::SKIP_PWDMA) ? -1 : mfma_pwd16_conv_bwd_data(g, dy, w, addend, dx, s);
-    if (r < 0) r = mfma_pointwise16_conv_bwd_data_add(g, dy, w, addend, dx, s);
+  if (!force_direct() && is_lo16(d->dtype) && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT)) {
+    int r = skip(Options::SKIP_PWDMA) ? -1 : mfma_pwd16_conv_bwd_data(g, dy, w, addend, dx, s, d->dtype);
+    if (r < 0) r = mfma_pointwise16_conv_bwd_data_add(g, dy, w, addend, dx, s, d->dtype);
     if (r >= 0) return r;
   }
   // every other kernel: the plain pass, then the element-wise sum
@@ -433,14 +433,14 @@ static int bwd_filter_impl(const flhip_conv_desc* d, const void* x, const void* 
     if (plan == 9) return bwd_filter_direct(d, g, x, dy, dw, db, s);
     const size_t need = flhip_conv2d_workspace_bytes(d, FLHIP_CONV_BWD_FILTER);
     FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter: workspace too small");
-    const bool lo = d->dtype == FLHIP_BF16;
+    const bool lo = is_lo16(d->dtype);
     int r = -1;
     switch (plan) {
-      case 0: if (lo) r = mfma_wgrad_dma16(g, x, dy, dw, db, ws, ws_bytes, s, 32); break;
-      case 1: if (lo) r = mfma_wgrad_dma16(g, x, dy, dw, db, ws, ws_bytes, s, 64); break;
-      case 2: if (lo) r = mfma_pointwise16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s); break;
-      case 3: if (lo) r = mfma_first16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s); break;
-      case 4: if (lo) r = mfma_wgrad16(g, x, dy, dw, db, ws, ws_bytes, s); break;
+      case 0: if (lo) r = mfma_wgrad_dma16(g, x, dy, dw, db, ws, ws_bytes, s, 32, d->dtype); break;
+      case 1: if (lo) r = mfma_wgrad_dma16(g, x, dy, dw, db, ws, ws_bytes, s, 64, d->dtype); break;
+      case 2: if (lo) r = mfma_pointwise16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s, nullptr, d->dtype); break;
+      case 3: if (lo) r = mfma_first16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s, d->dtype); break;
+      case 4: if (lo) r = mfma_wgrad16(g, x, dy, dw, db, ws, ws_bytes, s, d->dtype); break;
       case 5: r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, false, s); break;
       case 6: r = mfma_slab_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s); break;
       case 7: r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, true, s); break;
@@ -456,14 +456,14 @@ static int bwd_filter_impl(const flhip_conv_desc* d, const void* x, const void* 
     // (3x3 stride 1 with rows copied straight to LDS first: it also takes the 7x7 planes that would otherwise go
     // through gathered taps below)
     if (dw && tap1d_on(d->dtype)) r = mfma_tap1d_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_wgrad_dma16(g, x, dy, dw, db, ws, ws_bytes, s);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_pointwise16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !skip(Options::SKIP_FIRST) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_first16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s);
-    if (r < 0 && d->dtype == FLHIP_BF16 && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
-      r = mfma_wgrad16(g, x, dy, dw, db, ws, ws_bytes, s);
+    if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !skip(Options::SKIP_PWDMA) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_wgrad_dma16(g, x, dy, dw, db, ws, ws_bytes, s, 0, d->dtype);
+    if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_pointwise16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s, nullptr, d->dtype);
+    if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !skip(Options::SKIP_FIRST) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_first16_wgrad(g, x, dy, dw, db, ws, ws_bytes, s, d->dtype);
+    if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))
+      r = mfma_wgrad16(g, x, dy, dw, db, ws, ws_bytes, s, d->dtype);
     if (r < 0 && !skip(SK_GEMM))
       r = mfma_pointwise_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, algo_is(Options::ALGO_TAPPED), s);
     if (r < 0 && !skip(SK_SLAB)) r = mfma_slab_wgrad(g, d->dtype, x, dy, dw, db, ws, ws_bytes, s);
@@ -489,7 +489,7 @@ extern "C" int flhip_conv2d_bwd_filter_plan(const flhip_conv_desc* d, const void
 // its workspace; the filter gradient needs the same copy.  A caller that keeps those bytes passes them here and
 // saves the second gather.
 static bool gathered_path(const flhip_conv_desc* d) {
-  return d->dtype == FLHIP_BF16 && !force_direct() && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT);
+  return is_lo16(d->dtype) && !force_direct() && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT);
 }
 
 extern "C" size_t flhip_conv2d_gathered_bytes(const flhip_conv_desc* d) {
@@ -512,7 +512,7 @@ extern "C" int flhip_conv2d_bwd_filter_gathered(const flhip_conv_desc* d, const 
   FLHIP_REQUIRE(ws_bytes >= need && (ws || need == 0), "conv2d_bwd_filter_gathered: workspace too small");
   const bool one_row = tap1d_on(d->dtype) && mfma_tap1d_conv_ws(g, d->dtype, false) > 0;
   const int r = one_row ? mfma_tap1d_wgrad(g, d->dtype, nullptr, dy, dw, db, ws, ws_bytes, as_stream(stream), gathered)
-                        : mfma_pointwise16_wgrad(g, nullptr, dy, dw, db, ws, ws_bytes, as_stream(stream), gathered);
+                        : mfma_pointwise16_wgrad(g, nullptr, dy, dw, db, ws, ws_bytes, as_stream(stream), gathered, d->dtype);
   if (r < 0) return fail(FLHIP_INVALID_ARGUMENT, "conv2d_bwd_filter_gathered: no kernel takes the gathered input of this geometry");
   return r;
 }

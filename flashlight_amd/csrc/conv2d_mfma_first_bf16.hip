@@ -37,6 +37,7 @@ struct First16Params {
   unsigned src_bytes;
 };
 
+template <typename E>
 __global__ void __launch_bounds__(64 * F1_WAVES, 2)
 first16_conv_kernel(First16Params p, const bf16_t* __restrict__ src, const bf16_t* __restrict__ wgt,
                     const float* __restrict__ bias, bf16_t* __restrict__ dst) {
@@ -142,8 +143,8 @@ first16_conv_kernel(First16Params p, const bf16_t* __restrict__ src, const bf16_
 #pragma unroll
       for (int s = 0; s < F1_NS; ++s) {
         const uint4 av = make_uint4(a[s].x & mk[0], a[s].y & mk[1], a[s].z & mk[2], a[s].w & mk[3]);
-        acc[b][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(av), frag(wf[0][s]), acc[b][0], 0, 0, 0);
-        acc[b][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(av), frag(wf[1][s]), acc[b][1], 0, 0, 0);
+        acc[b][0] = Lo16<E>::mma32(frag(av), frag(wf[0][s]), acc[b][0]);
+        acc[b][1] = Lo16<E>::mma32(frag(av), frag(wf[1][s]), acc[b][1]);
       }
     }
     // ---- results: element r of an accumulator is position b*32 + (r/4)*8 + fh*4 + r%4 of channel
@@ -156,7 +157,7 @@ first16_conv_kernel(First16Params p, const bf16_t* __restrict__ src, const bf16_
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const floatx16& c = acc[b][mb];
-          const uintx2_t v = {pack_bf16(c[4 * g] + bv, c[4 * g + 1] + bv), pack_bf16(c[4 * g + 2] + bv, c[4 * g + 3] + bv)};
+          const uintx2_t v = {Lo16<E>::pack(c[4 * g] + bv, c[4 * g + 1] + bv), Lo16<E>::pack(c[4 * g + 2] + bv, c[4 * g + 3] + bv)};
           *reinterpret_cast<uintx2_t*>(stage + (mb * 32 + fr) * F1_SP + b * 32 + g * 8 + fh * 4) = v;
         }
       }
@@ -205,7 +206,7 @@ struct First16WgradParams {
 
 // KS = steps of 16 positions per result row when known at compile time (the loop is then
 // unrolled and its fragment reads run ahead of the matrix instructions), 0 = any
-template <int KS>
+template <typename E, int KS>
 __global__ void __launch_bounds__(256, 2)
 first16_wgrad_kernel(First16WgradParams p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy,
                      float* __restrict__ partial) {
@@ -218,7 +219,7 @@ first16_wgrad_kernel(First16WgradParams p, const bf16_t* __restrict__ x, const b
   uint16_t* const xs = lds_first;                      // [nrows + 2][2 copies][FW_CP]
   uint16_t* const dys = lds_first + (nrows + 2) * 2 * FW_CP;   // [2][64][FW_DP]
   for (int i = tid; i < 2 * FW_CP; i += 256) {
-    xs[nrows * 2 * FW_CP + i] = 0x3f80;                // 1.0
+    xs[nrows * 2 * FW_CP + i] = (uint16_t)(Lo16<E>::ONE2 & 0xffffu);   // 1.0
     xs[(nrows + 1) * 2 * FW_CP + i] = 0;
   }
 
@@ -328,7 +329,7 @@ first16_wgrad_kernel(First16WgradParams p, const bf16_t* __restrict__ x, const b
 #pragma unroll
         for (int t = 0; t < 3; ++t) {
           const bf16x8 b = bfrag(xs + baddr[t] + r * bstep[t] + 32 * ks);
-          acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[t], 0, 0, 0);
+          acc[t] = Lo16<E>::mma32(a, b, acc[t]);
         }
       };
       if (KS > 0) {
@@ -421,7 +422,7 @@ size_t mfma_first16_wgrad_ws(const ConvGeom& g) {
 }
 
 int mfma_first16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
-                       size_t ws_bytes, hipStream_t s) {
+                       size_t ws_bytes, hipStream_t s, int dtype) {
   First16WgradParams p{};
   int nwg;
   size_t shmem;
@@ -430,11 +431,16 @@ int mfma_first16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* 
   if (reinterpret_cast<uintptr_t>(x) % 4 != 0 || reinterpret_cast<uintptr_t>(dy) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(ws) % 16 != 0 || (g.OH * g.OW) % 8 != 0)
     return -1;
-  auto kernel = g.OW == 112 ? first16_wgrad_kernel<7> : first16_wgrad_kernel<0>;
-  if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
   float* partial = static_cast<float*>(ws);
-  hipLaunchKernelGGL(kernel, dim3((unsigned)nwg, (unsigned)p.mtiles), dim3(256), shmem, s, p,
-                     static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), partial);
+  const int rc = by_lo16(dtype, [&](auto* e_) {
+    using E = FLHIP_T_OF(e_);
+    auto kernel = g.OW == 112 ? first16_wgrad_kernel<E, 7> : first16_wgrad_kernel<E, 0>;
+    if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)nwg, (unsigned)p.mtiles), dim3(256), shmem, s, p,
+                       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), partial);
+    return 0;
+  });
+  if (rc) return rc;
   const int total = g.K * (p.NO * g.KW + 1);
   hipLaunchKernelGGL(first16_wgrad_reduce, dim3((unsigned)((total + 31) / 32)), dim3(256), 0, s, p, partial, nwg, dw, db);
   return check_launch("conv2d_bwd_filter (bf16 mfma first layer)");
@@ -442,7 +448,7 @@ int mfma_first16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* 
 
 
 int mfma_first16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
-                          hipStream_t s) {
+                          hipStream_t s, int dtype) {
   if (g.groups != 1 || g.dly != 1 || g.dlx != 1) return -1;
   const int sh = g.px & 1;
   // every 16-byte read starts on a dword: even column stride, even rows, window inside 8 elements
@@ -464,10 +470,15 @@ int mfma_first16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const
   p.mtiles = (g.K + 63) / 64;
   p.src_bytes = (unsigned)sbytes;
   const size_t shmem = std::max((size_t)64 * p.NO * g.KW, (size_t)F1_WAVES * 64 * F1_SP) * sizeof(uint16_t);
-  if (!mfma_allow_lds(reinterpret_cast<const void*>(first16_conv_kernel), shmem)) return -1;
   const int wgs = std::min((p.total_runs + F1_WAVES - 1) / F1_WAVES, 2 * mfma_num_cus());
-  hipLaunchKernelGGL(first16_conv_kernel, dim3((unsigned)wgs, (unsigned)p.mtiles), dim3(64 * F1_WAVES), shmem, s, p,
-                     static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), bias, static_cast<bf16_t*>(y));
+  const int rc = by_lo16(dtype, [&](auto* e_) {
+    using E = FLHIP_T_OF(e_);
+    if (!mfma_allow_lds(reinterpret_cast<const void*>(first16_conv_kernel<E>), shmem)) return -1;
+    hipLaunchKernelGGL(first16_conv_kernel<E>, dim3((unsigned)wgs, (unsigned)p.mtiles), dim3(64 * F1_WAVES), shmem, s, p,
+                       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), bias, static_cast<bf16_t*>(y));
+    return 0;
+  });
+  if (rc) return rc;
   return check_launch("conv2d (bf16 mfma first layer)");
 }
 

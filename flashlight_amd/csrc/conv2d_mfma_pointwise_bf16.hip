@@ -85,9 +85,9 @@ __device__ __forceinline__ uintx2_t merge_runs(uintx2_t a, uintx2_t b, int rem) 
 
 // a + b on two bf16 values per dword, each sum rounded to bf16 (what an element-wise add of the
 // two tensors would give)
-__device__ __forceinline__ uint32_t add_bf16x2(uint32_t a, uint32_t b) {
-  return pack_bf16(__uint_as_float(a << 16) + __uint_as_float(b << 16),
-                   __uint_as_float(a & 0xffff0000u) + __uint_as_float(b & 0xffff0000u));
+template <typename E>
+__device__ __forceinline__ uint32_t add_x2(uint32_t a, uint32_t b) {
+  return Lo16<E>::pack(Lo16<E>::lo(a) + Lo16<E>::lo(b), Lo16<E>::hi(a) + Lo16<E>::hi(b));
 }
 
 // BWD = false: forward (weights [Mo][Kc]); true: backward-data (weights [Kc][Mo]).
@@ -100,7 +100,7 @@ __device__ __forceinline__ uint32_t add_bf16x2(uint32_t a, uint32_t b) {
 // fills the chip several times over (other workgroups hide the latency), 4 for small grids
 // with long contractions (7x7 planes: about 100 workgroups of up to 64 chunks each, one
 // wave per SIMD), where a chunk otherwise costs one trip to memory.
-template <bool BWD, int MT, bool ODD, int PF>
+template <typename E, bool BWD, int MT, bool ODD, int PF>
 __global__ void __launch_bounds__(256)
 pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __restrict__ wgt,
                  const float* __restrict__ bias, bf16_t* __restrict__ dst, const bf16_t* __restrict__ addend) {
@@ -224,7 +224,7 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
       const bf16x8 b = BWD ? gather8_tr(Wt, PB_WPB, 8 * fg, j * 16, fr)
                            : __builtin_bit_cast(bf16x8, *reinterpret_cast<const uintx4_t*>(&Wt[wslot(j * 16 + fr, fg)]));
 #pragma unroll
-      for (int i = 0; i < 2; ++i) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b, acc[i][j], 0, 0, 0);
+      for (int i = 0; i < 2; ++i) acc[i][j] = Lo16<E>::mma16(a[i], b, acc[i][j]);
     }
   };
 
@@ -287,8 +287,8 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
     for (int j = 0; j < MT; ++j) {
       const int ml = j * 16 + fr;
       const float bv = (!BWD && bias && m0 + ml < p.Mo) ? bias[m0 + ml] : 0.f;
-      const uintx2_t o = {(uint32_t)f32_to_bf16(acc[i][j][0] + bv) | ((uint32_t)f32_to_bf16(acc[i][j][1] + bv) << 16),
-                          (uint32_t)f32_to_bf16(acc[i][j][2] + bv) | ((uint32_t)f32_to_bf16(acc[i][j][3] + bv) << 16)};
+      const uintx2_t o = {(uint32_t)Lo16<E>::narrow(acc[i][j][0] + bv) | ((uint32_t)Lo16<E>::narrow(acc[i][j][1] + bv) << 16),
+                          (uint32_t)Lo16<E>::narrow(acc[i][j][2] + bv) | ((uint32_t)Lo16<E>::narrow(acc[i][j][3] + bv) << 16)};
       *reinterpret_cast<uintx2_t*>(&Ys[ml * YP + wave * 32 + i * 16 + 4 * fg]) = o;
     }
   __syncthreads();
@@ -304,7 +304,7 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
         if (left >= 4) {
           if (addend) {
             const uintx2_t a = load8_any(addend + (dp - dst) + row);
-            v = uintx2_t{add_bf16x2(v.x, a.x), add_bf16x2(v.y, a.y)};
+            v = uintx2_t{add_x2<E>(v.x, a.x), add_x2<E>(v.y, a.y)};
           }
           store8_any(dp + row, v);
         } else {
@@ -313,7 +313,7 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
           for (int e = 0; e < 4; ++e)
             if (qo + e < p.Ptot) {
               bf16_t* o = (e < left ? dp : dp2) + row + e;
-              *o = addend ? f32_to_bf16(bf16_to_f32((bf16_t)e4[e]) + bf16_to_f32(addend[o - dst])) : (bf16_t)e4[e];
+              *o = addend ? Lo16<E>::narrow(Lo16<E>::widen((uint16_t)e4[e]) + Lo16<E>::widen(addend[o - dst])) : (bf16_t)e4[e];
             }
         }
       }
@@ -327,7 +327,7 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
         uintx4_t v = *reinterpret_cast<const uintx4_t*>(&Ys[ml * YP + pc]);
         if (addend) {
           const uintx4_t a = *reinterpret_cast<const uintx4_t*>(addend + (dp - dst) + (size_t)(m0 + ml) * p.P);
-          v = uintx4_t{add_bf16x2(v.x, a.x), add_bf16x2(v.y, a.y), add_bf16x2(v.z, a.z), add_bf16x2(v.w, a.w)};
+          v = uintx4_t{add_x2<E>(v.x, a.x), add_x2<E>(v.y, a.y), add_x2<E>(v.z, a.z), add_x2<E>(v.w, a.w)};
         }
         *reinterpret_cast<uintx4_t*>(dp + (size_t)(m0 + ml) * p.P) = v;
       }
@@ -341,7 +341,7 @@ pw16_conv_kernel(Pw16Params p, const bf16_t* __restrict__ src, const bf16_t* __r
         uintx2_t v = *reinterpret_cast<const uintx2_t*>(&Ys[ml * YP + pc]);
         if (addend) {
           const uintx2_t a = *reinterpret_cast<const uintx2_t*>(addend + (dp - dst) + (size_t)(m0 + ml) * p.P);
-          v = uintx2_t{add_bf16x2(v.x, a.x), add_bf16x2(v.y, a.y)};
+          v = uintx2_t{add_x2<E>(v.x, a.x), add_x2<E>(v.y, a.y)};
         }
         *reinterpret_cast<uintx2_t*>(dp + (size_t)(m0 + ml) * p.P) = v;
       }
@@ -354,7 +354,7 @@ bool pw16_applies(const ConvGeom& g) {
          g.OH == g.H && g.OW == g.W && g.H * g.W >= 4 && g.C % 8 == 0 && g.K % 8 == 0;
 }
 
-template <bool BWD>
+template <typename E, bool BWD>
 int launch_pw16(const ConvGeom& g, const void* src, const void* w, const float* bias, void* dst, hipStream_t s,
                 const void* addend = nullptr) {
   Pw16Params p{};
@@ -380,11 +380,11 @@ int launch_pw16(const ConvGeom& g, const void* src, const void* w, const float* 
                        static_cast<const bf16_t*>(w), bias, static_cast<bf16_t*>(dst), static_cast<const bf16_t*>(addend));
   };
   if (odd) {
-    if (deep) go(pw16_conv_kernel<BWD, 4, true, 4>);
-    else go(pw16_conv_kernel<BWD, 4, true, 1>);
+    if (deep) go(pw16_conv_kernel<E, BWD, 4, true, 4>);
+    else go(pw16_conv_kernel<E, BWD, 4, true, 1>);
   } else {
-    if (deep) go(pw16_conv_kernel<BWD, 4, false, 4>);
-    else go(pw16_conv_kernel<BWD, 4, false, 1>);
+    if (deep) go(pw16_conv_kernel<E, BWD, 4, false, 4>);
+    else go(pw16_conv_kernel<E, BWD, 4, false, 1>);
   }
   return check_launch(BWD ? "conv2d_bwd_data 1x1 (bf16 mfma)" : "conv2d_fwd 1x1 (bf16 mfma)");
 }
@@ -406,7 +406,7 @@ struct Pw16WgradParams {
 // image) of rows t / 16 + 16 g, g = 0..3, of both operands.  out: slice-major partial results
 // [nsplit][E + Mo] (dw tile values, then the bias sums), or dw / db themselves when there
 // is one slice.
-template <bool ODD>
+template <typename E, bool ODD>
 __global__ void __launch_bounds__(256)
 pw16_wgrad_kernel(Pw16WgradParams p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy,
                   float* __restrict__ out, float* __restrict__ db_direct) {
@@ -483,8 +483,8 @@ pw16_wgrad_kernel(Pw16WgradParams p, const bf16_t* __restrict__ x, const bf16_t*
       *reinterpret_cast<uintx2_t*>(&Ds[buf][(lrow + 16 * g) * PG_P + lpos]) = sd[g];
       *reinterpret_cast<uintx2_t*>(&Xs[buf][(lrow + 16 * g) * PG_P + lpos]) = sx[g];
       if (do_bias) {
-        bsum[g] += bf16_to_f32((bf16_t)(sd[g].x & 0xffffu)) + bf16_to_f32((bf16_t)(sd[g].x >> 16));
-        bsum[g] += bf16_to_f32((bf16_t)(sd[g].y & 0xffffu)) + bf16_to_f32((bf16_t)(sd[g].y >> 16));
+        bsum[g] += Lo16<E>::widen((uint16_t)(sd[g].x & 0xffffu)) + Lo16<E>::widen((uint16_t)(sd[g].x >> 16));
+        bsum[g] += Lo16<E>::widen((uint16_t)(sd[g].y & 0xffffu)) + Lo16<E>::widen((uint16_t)(sd[g].y >> 16));
       }
     }
   };
@@ -514,7 +514,7 @@ pw16_wgrad_kernel(Pw16WgradParams p, const bf16_t* __restrict__ x, const bf16_t*
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < 2; ++j) acc[i][j] = Lo16<E>::mma16(a[i], b[j], acc[i][j]);
     }
     if (c + 1 < cend) sstore(buf ^ 1);
     __syncthreads();
@@ -595,6 +595,7 @@ struct Pw16Wgrad2Params {
   unsigned x_bytes, dy_bytes;
 };
 
+template <typename E>
 __global__ void __launch_bounds__(256, 2)
 pw16_wgrad2_kernel(Pw16Wgrad2Params p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy,
                    float* __restrict__ out, float* __restrict__ db_direct) {
@@ -665,7 +666,7 @@ pw16_wgrad2_kernel(Pw16Wgrad2Params p, const bf16_t* __restrict__ x, const bf16_
         const unsigned w4[4] = {sd[g].x, sd[g].y, sd[g].z, sd[g].w};
 #pragma unroll
         for (int d = 0; d < 4; ++d)
-          bsum[g] += bf16_to_f32((bf16_t)(w4[d] & 0xffffu)) + bf16_to_f32((bf16_t)(w4[d] >> 16));
+          bsum[g] += Lo16<E>::widen((uint16_t)(w4[d] & 0xffffu)) + Lo16<E>::widen((uint16_t)(w4[d] >> 16));
       }
     }
   };
@@ -703,7 +704,7 @@ pw16_wgrad2_kernel(Pw16Wgrad2Params p, const bf16_t* __restrict__ x, const bf16_
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < 2; ++j) acc[i][j] = Lo16<E>::mma32(af[i], bf[j], acc[i][j]);
     }
     if (ch + 1 < cend) sstore(buf ^ 1);
     __syncthreads();
@@ -884,7 +885,7 @@ taps_gather_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ xc, ConvGe
 
 // S2: strides 2, no dilation (parity picks the taps that reach an element, no division by a
 // stride); PAIR as above, over the columns of dx
-template <bool S2, bool PAIR>
+template <typename E, bool S2, bool PAIR>
 __global__ void __launch_bounds__(256)
 taps_spread_kernel(const bf16_t* __restrict__ dxc, bf16_t* __restrict__ dx, ConvGeom g) {
   constexpr int V = PAIR ? 2 : 1;
@@ -918,7 +919,7 @@ taps_spread_kernel(const bf16_t* __restrict__ dxc, bf16_t* __restrict__ dx, Conv
 #pragma unroll
         for (int a = 0; a < 2; ++a)
 #pragma unroll
-          for (int b = 0; b < 2; ++b) acc[e] += ok[a][b] ? bf16_to_f32((bf16_t)ld[a][b]) : 0.f;
+          for (int b = 0; b < 2; ++b) acc[e] += ok[a][b] ? Lo16<E>::widen((uint16_t)ld[a][b]) : 0.f;
       } else {
         for (int kh = 0; kh < g.KH; ++kh) {
           const int a = h + g.py - kh * g.dly;
@@ -926,14 +927,14 @@ taps_spread_kernel(const bf16_t* __restrict__ dxc, bf16_t* __restrict__ dx, Conv
           for (int kw = 0; kw < g.KW; ++kw) {
             const int b = w + g.px - kw * g.dlx;
             if (b < 0 || b % g.sx != 0 || b / g.sx >= g.OW) continue;
-            acc[e] += bf16_to_f32(cp[(kh * g.KW + kw) * P + (a / g.sy) * g.OW + b / g.sx]);
+            acc[e] += Lo16<E>::widen(cp[(kh * g.KW + kw) * P + (a / g.sy) * g.OW + b / g.sx]);
           }
         }
       }
     }
     bf16_t* o = dp + h * g.W + w0;
-    if constexpr (PAIR) *reinterpret_cast<uint32_t*>(o) = (uint32_t)f32_to_bf16(acc[0]) | ((uint32_t)f32_to_bf16(acc[1]) << 16);
-    else *o = f32_to_bf16(acc[0]);
+    if constexpr (PAIR) *reinterpret_cast<uint32_t*>(o) = (uint32_t)Lo16<E>::narrow(acc[0]) | ((uint32_t)Lo16<E>::narrow(acc[1]) << 16);
+    else *o = Lo16<E>::narrow(acc[0]);
   }
 }
 
@@ -958,6 +959,7 @@ bool taps_gather(const ConvGeom& g, const void* x, void* xc, hipStream_t s) {
   else hipLaunchKernelGGL(taps_gather_kernel<false>, grid, block, 0, s, static_cast<const bf16_t*>(x), static_cast<bf16_t*>(xc), g);
   return true;
 }
+template <typename E>
 bool taps_spread(const ConvGeom& g, const void* dxc, void* dx, hipStream_t s) {
   const bool pair = g.W % 2 == 0 && ((uintptr_t)dx & 3) == 0;
   const bool s2 = g.sy == 2 && g.sx == 2 && g.dly == 1 && g.dlx == 1 && g.KH <= 4 && g.KW <= 4;
@@ -967,8 +969,8 @@ bool taps_spread(const ConvGeom& g, const void* dxc, void* dx, hipStream_t s) {
   auto go = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, grid, block, 0, s, static_cast<const bf16_t*>(dxc), static_cast<bf16_t*>(dx), g);
   };
-  if (s2) { if (pair) go(taps_spread_kernel<true, true>); else go(taps_spread_kernel<true, false>); }
-  else { if (pair) go(taps_spread_kernel<false, true>); else go(taps_spread_kernel<false, false>); }
+  if (s2) { if (pair) go(taps_spread_kernel<E, true, true>); else go(taps_spread_kernel<E, true, false>); }
+  else { if (pair) go(taps_spread_kernel<E, false, true>); else go(taps_spread_kernel<E, false, false>); }
   return true;
 }
 
@@ -1027,59 +1029,72 @@ size_t mfma_pointwise16_gathered_bytes(const ConvGeom& g) {
 
 // the compact 1x1 problem of a strided layer: on the kernels that load straight to LDS where those
 // are ahead, else on the ones above
-template <bool BWD>
+template <typename E, bool BWD>
 int launch_compact(const ConvGeom& c, const void* src, const void* w, const float* bias, void* dst, hipStream_t s) {
   if (!(options().conv_skip & Options::SKIP_PWDMA)) {
-    const int r = BWD ? mfma_pwd16_conv_bwd_data(c, src, w, nullptr, dst, s) : mfma_pwd16_conv_fwd(c, src, w, bias, dst, s);
+    const int r = BWD ? mfma_pwd16_conv_bwd_data(c, src, w, nullptr, dst, s, Lo16<E>::TAG)
+                      : mfma_pwd16_conv_fwd(c, src, w, bias, dst, s, Lo16<E>::TAG);
     if (r >= 0) return r;
   }
-  return launch_pw16<BWD>(c, src, w, bias, dst, s);
+  return launch_pw16<E, BWD>(c, src, w, bias, dst, s);
 }
 
-int mfma_pointwise16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
-                              hipStream_t s, void* ws, size_t ws_bytes) {
+template <typename E>
+static int pointwise16_conv_fwd_impl(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
+                                     hipStream_t s, void* ws, size_t ws_bytes) {
   ConvGeom c;
   if (pw16_strided_plan(g, &c)) {
     if (!ws || ws_bytes < lattice_bytes(c)) return -1;
     lattice_gather(g, x, ws, s);
-    return launch_compact<false>(c, ws, w, bias, y, s);
+    return launch_compact<E, false>(c, ws, w, bias, y, s);
   }
   if (!options().pw16_no_taps && pw16_taps_plan(g, &c) && pw16_taps_forward(g, c) && ws && ws_bytes >= lattice_bytes(c) &&
       taps_gather(g, x, ws, s))
-    return launch_compact<false>(c, ws, w, bias, y, s);
+    return launch_compact<E, false>(c, ws, w, bias, y, s);
   if (!pw16_applies(g)) return -1;
-  return launch_pw16<false>(g, x, w, bias, y, s);
+  return launch_pw16<E, false>(g, x, w, bias, y, s);
 }
 
-int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s,
-                                   void* ws, size_t ws_bytes) {
+template <typename E>
+static int pointwise16_conv_bwd_data_impl(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s,
+                                          void* ws, size_t ws_bytes) {
   ConvGeom c;
   if (pw16_strided_plan(g, &c)) {
     if (!ws || ws_bytes < lattice_bytes(c)) return -1;
-    const int rc = launch_compact<true>(c, dy, w, nullptr, ws, s);
+    const int rc = launch_compact<E, true>(c, dy, w, nullptr, ws, s);
     if (rc != FLHIP_OK) return rc;
     lattice_scatter(g, ws, dx, s);
     return check_launch("conv2d_bwd_data strided 1x1 (bf16 mfma)");
   }
   if (!options().pw16_no_taps && pw16_taps_plan(g, &c)) {
     if (!ws || ws_bytes < lattice_bytes(c)) return -1;
-    const int rc = launch_compact<true>(c, dy, w, nullptr, ws, s);
+    const int rc = launch_compact<E, true>(c, dy, w, nullptr, ws, s);
     if (rc != FLHIP_OK) return rc;
-    if (!taps_spread(g, ws, dx, s)) return fail(FLHIP_RUNTIME_ERROR, "conv2d_bwd_data: plane too wide for the spread kernel");
+    if (!taps_spread<E>(g, ws, dx, s)) return fail(FLHIP_RUNTIME_ERROR, "conv2d_bwd_data: plane too wide for the spread kernel");
     return check_launch("conv2d_bwd_data strided window (bf16 mfma)");
   }
   if (!pw16_applies(g)) return -1;
-  return launch_pw16<true>(g, dy, w, nullptr, dx, s);
+  return launch_pw16<E, true>(g, dy, w, nullptr, dx, s);
 }
 
 // dx = addend + backward-data, in the kernel's own result pass; -1 when this geometry's
 // backward-data pass is not the plain 1x1 kernel
+int mfma_pointwise16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
+                              hipStream_t s, void* ws, size_t ws_bytes, int dtype) {
+  return by_lo16(dtype, [&](auto* e_) { return pointwise16_conv_fwd_impl<FLHIP_T_OF(e_)>(g, x, w, bias, y, s, ws, ws_bytes); });
+}
+
+int mfma_pointwise16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s,
+                                   void* ws, size_t ws_bytes, int dtype) {
+  return by_lo16(dtype, [&](auto* e_) { return pointwise16_conv_bwd_data_impl<FLHIP_T_OF(e_)>(g, dy, w, dx, s, ws, ws_bytes); });
+}
+
 int mfma_pointwise16_conv_bwd_data_add(const ConvGeom& g, const void* dy, const void* w, const void* addend, void* dx,
-                                       hipStream_t s) {
+                                       hipStream_t s, int dtype) {
   ConvGeom c;
   if (pw16_strided_plan(g, &c) || (!options().pw16_no_taps && pw16_taps_plan(g, &c)) || !pw16_applies(g)) return -1;
   if (reinterpret_cast<uintptr_t>(addend) % 16 != 0) return -1;
-  return launch_pw16<true>(g, dy, w, nullptr, dx, s, addend);
+  return by_lo16(dtype, [&](auto* e_) { return launch_pw16<FLHIP_T_OF(e_), true>(g, dy, w, nullptr, dx, s, addend); });
 }
 
 size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g0) {
@@ -1099,8 +1114,9 @@ size_t mfma_pointwise16_wgrad_ws(const ConvGeom& g0) {
 
 // (gathered: the gathered input a forward pass left behind - mfma_pointwise16_gathered_bytes() of it -, taken in
 // place of x; -1 when this geometry has none)
-int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, float* dw, float* db, void* ws,
-                           size_t ws_bytes, hipStream_t s, const void* gathered) {
+template <typename E>
+static int pointwise16_wgrad_impl(const ConvGeom& g0, const void* x, const void* dy, float* dw, float* db, void* ws,
+                                  size_t ws_bytes, hipStream_t s, const void* gathered) {
   if (!dw) return -1;
   ConvGeom g = g0;
   const bool strided = pw16_strided_plan(g0, &g);
@@ -1122,7 +1138,7 @@ int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, fl
     ws_bytes -= lb;
   }
   if (!db && !(options().conv_skip & Options::SKIP_PWDMA)) {
-    const int r = mfma_pwd16_wgrad(g, x, dy, dw, ws, ws_bytes, s);
+    const int r = mfma_pwd16_wgrad(g, x, dy, dw, ws, ws_bytes, s, Lo16<E>::TAG);
     if (r >= 0) return r;
   }
   Pw16Wgrad2Params p2{};
@@ -1131,9 +1147,9 @@ int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, fl
     p2.want_db = db != nullptr;
     const size_t need2 = p2.nsplit > 1 ? (size_t)p2.nsplit * ((size_t)p2.E + p2.Mo) * sizeof(float) : 0;
     const size_t shmem = (size_t)2 * 2 * PG2_T * PG2_P * sizeof(uint16_t);
-    if ((!need2 || (ws && ws_bytes >= need2)) && mfma_allow_lds(reinterpret_cast<const void*>(pw16_wgrad2_kernel), shmem)) {
+    if ((!need2 || (ws && ws_bytes >= need2)) && mfma_allow_lds(reinterpret_cast<const void*>(pw16_wgrad2_kernel<E>), shmem)) {
       float* out2 = p2.nsplit > 1 ? static_cast<float*>(ws) : dw;
-      hipLaunchKernelGGL(pw16_wgrad2_kernel, dim3((unsigned)p2.nsplit, (unsigned)(p2.ctiles * p2.mtiles)), dim3(256), shmem, s,
+      hipLaunchKernelGGL(pw16_wgrad2_kernel<E>, dim3((unsigned)p2.nsplit, (unsigned)(p2.ctiles * p2.mtiles)), dim3(256), shmem, s,
                          p2, static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), out2, db);
       if (p2.nsplit > 1) wgrad_reduce_launch(static_cast<const float*>(ws), p2.nsplit, p2.E, p2.Mo, p2.want_db, dw, db, s);
       return check_launch("conv2d_bwd_filter 1x1 (bf16 mfma, 128 x 128 tiles)");
@@ -1145,13 +1161,20 @@ int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, fl
   float* out = p.nsplit > 1 ? static_cast<float*>(ws) : dw;
   const dim3 grid((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles));
   if (p.P % 4 == 0)
-    hipLaunchKernelGGL(pw16_wgrad_kernel<false>, grid, dim3(256), 0, s, p, static_cast<const bf16_t*>(x),
+    hipLaunchKernelGGL((pw16_wgrad_kernel<E, false>), grid, dim3(256), 0, s, p, static_cast<const bf16_t*>(x),
                        static_cast<const bf16_t*>(dy), out, db);
   else
-    hipLaunchKernelGGL(pw16_wgrad_kernel<true>, grid, dim3(256), 0, s, p, static_cast<const bf16_t*>(x),
+    hipLaunchKernelGGL((pw16_wgrad_kernel<E, true>), grid, dim3(256), 0, s, p, static_cast<const bf16_t*>(x),
                        static_cast<const bf16_t*>(dy), out, db);
   if (p.nsplit > 1) wgrad_reduce_launch(static_cast<const float*>(ws), p.nsplit, p.E, p.Mo, p.want_db, dw, db, s);
   return check_launch("conv2d_bwd_filter 1x1 (bf16 mfma)");
+}
+
+int mfma_pointwise16_wgrad(const ConvGeom& g0, const void* x, const void* dy, float* dw, float* db, void* ws,
+                           size_t ws_bytes, hipStream_t s, const void* gathered, int dtype) {
+  return by_lo16(dtype, [&](auto* e_) {
+    return pointwise16_wgrad_impl<FLHIP_T_OF(e_)>(g0, x, dy, dw, db, ws, ws_bytes, s, gathered);
+  });
 }
 
 }  // namespace flhip

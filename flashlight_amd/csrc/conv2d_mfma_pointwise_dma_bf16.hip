@@ -80,9 +80,10 @@ __device__ __forceinline__ bf16x8 pd_gather8(const uint16_t* tile, int pitch, in
   return __builtin_bit_cast(bf16x8, v);
 }
 
-__device__ __forceinline__ uint32_t pd_add_bf16x2(uint32_t a, uint32_t b) {
-  return pack_bf16(__uint_as_float(a << 16) + __uint_as_float(b << 16),
-                   __uint_as_float(a & 0xffff0000u) + __uint_as_float(b & 0xffff0000u));
+// two packed elements plus two packed elements, each sum rounded once
+template <typename E>
+__device__ __forceinline__ uint32_t pd_add_x2(uint32_t a, uint32_t b) {
+  return Lo16<E>::pack(Lo16<E>::lo(a) + Lo16<E>::lo(b), Lo16<E>::hi(a) + Lo16<E>::hi(b));
 }
 
 // at most N of this wave's loads outstanding
@@ -100,10 +101,10 @@ __device__ __forceinline__ void pd_wait_loads() {
   if (N == 24) PD_WAIT_VM(24);
 }
 
-template <bool BWD, int PD_NS, int BM>
+template <typename E, bool BWD, int PD_NS, int BM>
 __global__ void __launch_bounds__(256, PD_NS == 4 ? 2 : 1)
-pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __restrict__ wgt,
-                  const float* __restrict__ bias, bf16_t* __restrict__ dst, const bf16_t* __restrict__ addend) {
+pwd16_conv_kernel(PwdParams p, const E* __restrict__ src, const E* __restrict__ wgt,
+                  const float* __restrict__ bias, E* __restrict__ dst, const E* __restrict__ addend) {
   static_assert(BM == 128 || BM == 64, "tile heights in use");
   constexpr int PD_D = PD_NS - 2;
   constexpr int PD_STAGE = pd_stage(BM);
@@ -202,7 +203,7 @@ pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __r
   _Pragma("unroll") for (int ks = 0; ks < 2; ++ks)                                                      \
     _Pragma("unroll") for (int i = 0; i < NA; ++i)                                                      \
       _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                     \
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][ks][i], fb[SET][ks][j], acc[i][j], 0, 0, 0);
+        acc[i][j] = Lo16<E>::mma32(fa[SET][ks][i], fb[SET][ks][j], acc[i][j]);
 
   // stages 0 .. D in flight, stage 0 in registers
 #pragma unroll
@@ -254,8 +255,8 @@ pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __r
     for (int i = 0; i < NA; ++i)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const uintx2_t o = {pack_bf16(acc[i][j][4 * g] + bv, acc[i][j][4 * g + 1] + bv),
-                            pack_bf16(acc[i][j][4 * g + 2] + bv, acc[i][j][4 * g + 3] + bv)};
+        const uintx2_t o = {Lo16<E>::pack(acc[i][j][4 * g] + bv, acc[i][j][4 * g + 1] + bv),
+                            Lo16<E>::pack(acc[i][j][4 * g + 2] + bv, acc[i][j][4 * g + 3] + bv)};
         *reinterpret_cast<uintx2_t*>(&ys[ml * PD_YP + pos0 + i * 32 + g * 8 + fh * 4]) = o;
       }
   }
@@ -272,8 +273,8 @@ pwd16_conv_kernel(PwdParams p, const bf16_t* __restrict__ src, const bf16_t* __r
         const int off = (base + ml * p.P) * 2;
         if (addend) {
           const uintx4_t a = __builtin_amdgcn_raw_buffer_load_b128(ars, off, 0, 0);
-          v = uintx4_t{pd_add_bf16x2(v.x, a.x), pd_add_bf16x2(v.y, a.y), pd_add_bf16x2(v.z, a.z),
-                       pd_add_bf16x2(v.w, a.w)};
+          v = uintx4_t{pd_add_x2<E>(v.x, a.x), pd_add_x2<E>(v.y, a.y), pd_add_x2<E>(v.z, a.z),
+                       pd_add_x2<E>(v.w, a.w)};
         }
         __builtin_amdgcn_raw_buffer_store_b128(v, drs, off, 0, 0);
       }
@@ -294,7 +295,7 @@ bool pwd16_applies(const ConvGeom& g, bool bwd) {
   return options().pw16_pf != 0 || (g.H * g.W <= 1024 && mo > 64);
 }
 
-template <bool BWD>
+template <typename E, bool BWD>
 int launch_pwd16(const ConvGeom& g, const void* src, const void* w, const float* bias, void* dst, const void* addend,
                  hipStream_t s) {
   if (!pwd16_applies(g, BWD)) return -1;
@@ -325,18 +326,17 @@ int launch_pwd16(const ConvGeom& g, const void* src, const void* w, const float*
   const long long grid = (long long)((p.ctiles + 7) / 8) * 8 * p.mtiles;
   if (grid > 0x7fffffffll) return -1;
   auto go = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), 0, s, p, static_cast<const bf16_t*>(src),
-                       static_cast<const bf16_t*>(w), bias, static_cast<bf16_t*>(dst),
-                       static_cast<const bf16_t*>(addend));
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), 0, s, p, static_cast<const E*>(src),
+                       static_cast<const E*>(w), bias, static_cast<E*>(dst), static_cast<const E*>(addend));
   };
   bool deep = (long long)p.ctiles * p.mtiles <= (long long)cus;
   if (pf) deep = pf >= 4;
   if (small) {
-    if (deep) go(pwd16_conv_kernel<BWD, 8, 64>);
-    else go(pwd16_conv_kernel<BWD, 4, 64>);
+    if (deep) go(pwd16_conv_kernel<E, BWD, 8, 64>);
+    else go(pwd16_conv_kernel<E, BWD, 4, 64>);
   } else {
-    if (deep) go(pwd16_conv_kernel<BWD, 8, 128>);
-    else go(pwd16_conv_kernel<BWD, 4, 128>);
+    if (deep) go(pwd16_conv_kernel<E, BWD, 8, 128>);
+    else go(pwd16_conv_kernel<E, BWD, 4, 128>);
   }
   return check_launch(BWD ? "conv2d_bwd_data 1x1 (bf16 mfma, direct-to-LDS)" : "conv2d_fwd 1x1 (bf16 mfma, direct-to-LDS)");
 }
@@ -373,8 +373,9 @@ struct PwdWgradParams {
   unsigned x_bytes, dy_bytes;
 };
 
+template <typename E>
 __global__ void __launch_bounds__(256, 1)
-pwd16_wgrad_kernel(PwdWgradParams p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy, float* __restrict__ out) {
+pwd16_wgrad_kernel(PwdWgradParams p, const E* __restrict__ x, const E* __restrict__ dy, float* __restrict__ out) {
   __shared__ __align__(16) uint4 ring[PWG_NS * PWG_STAGE];
   const int slice = blockIdx.x, mtile = blockIdx.y / p.ctiles, ctile = blockIdx.y - mtile * p.ctiles;
   const int m0 = mtile * PWG_T, c0 = ctile * PWG_T;
@@ -475,7 +476,7 @@ pwd16_wgrad_kernel(PwdWgradParams p, const bf16_t* __restrict__ x, const bf16_t*
   _Pragma("unroll") for (int sk = 0; sk < 4; ++sk)                                                           \
     _Pragma("unroll") for (int i = 0; i < 2; ++i)                                                            \
       _Pragma("unroll") for (int jj = 0; jj < 2; ++jj)                                                       \
-        acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][sk][i], fb[SET][sk][jj], acc[i][jj], 0, 0, 0);
+        acc[i][jj] = Lo16<E>::mma32(fa[SET][sk][i], fb[SET][sk][jj], acc[i][jj]);
 
   // stages 0 .. D in flight; every wave issues 8 loads per stage.  Only the wait and the loads depend on the
   // stage number: the reads of one register set and the matrix instructions on the other are one block of
@@ -561,13 +562,13 @@ bool pwd16_wgrad_plan(const ConvGeom& g, PwdWgradParams* p) {
 
 }  // namespace
 
-int mfma_pwd16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y, hipStream_t s) {
-  return launch_pwd16<false>(g, x, w, bias, y, nullptr, s);
+int mfma_pwd16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y, hipStream_t s, int dtype) {
+  return by_lo16(dtype, [&](auto* e_) { return launch_pwd16<FLHIP_T_OF(e_), false>(g, x, w, bias, y, nullptr, s); });
 }
 
 int mfma_pwd16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, const void* addend, void* dx,
-                             hipStream_t s) {
-  return launch_pwd16<true>(g, dy, w, nullptr, dx, addend, s);
+                             hipStream_t s, int dtype) {
+  return by_lo16(dtype, [&](auto* e_) { return launch_pwd16<FLHIP_T_OF(e_), true>(g, dy, w, nullptr, dx, addend, s); });
 }
 
 }  // namespace flhip
@@ -585,7 +586,8 @@ size_t mfma_pwd16_wgrad_ws(const ConvGeom& g) {
 }
 
 // -1 when the shape (or a bias gradient) is not this kernel's
-int mfma_pwd16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, void* ws, size_t ws_bytes, hipStream_t s) {
+int mfma_pwd16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw, void* ws, size_t ws_bytes, hipStream_t s,
+                     int dtype) {
   PwdWgradParams p{};
   if (!dw || !pwd16_wgrad_plan(g, &p)) return -1;
   // measured on the ResNet-50 layers at batch 64: 7 to 20 % ahead of the kernel with register staging on planes of
@@ -596,8 +598,11 @@ int mfma_pwd16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw
   const size_t need = p.nsplit > 1 ? (size_t)p.nsplit * ((size_t)p.E + p.Mo) * sizeof(float) : 0;
   if (need && (!ws || ws_bytes < need)) return -1;
   float* out = p.nsplit > 1 ? static_cast<float*>(ws) : dw;
-  hipLaunchKernelGGL(pwd16_wgrad_kernel, dim3((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles)), dim3(256), 0, s, p,
-                     static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(dy), out);
+  by_lo16(dtype, [&](auto* e_) {
+    using E = FLHIP_T_OF(e_);
+    hipLaunchKernelGGL(pwd16_wgrad_kernel<E>, dim3((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles)), dim3(256), 0, s, p,
+                       static_cast<const E*>(x), static_cast<const E*>(dy), out);
+  });
   if (p.nsplit > 1) wgrad_reduce_launch(static_cast<const float*>(ws), p.nsplit, p.E, p.Mo, 0, dw, nullptr, s);
   return check_launch("conv2d_bwd_filter 1x1 (bf16 mfma, direct-to-LDS)");
 }

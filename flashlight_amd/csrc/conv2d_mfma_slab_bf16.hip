@@ -72,10 +72,10 @@ struct Slab16Params {
   unsigned src_bytes, wt_bytes;
 };
 
-template <bool BWD>
+template <typename E, bool BWD>
 __global__ void __launch_bounds__(THREADS, 2)
-slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t* __restrict__ wgt,
-                   const float* __restrict__ bias, bf16_t* __restrict__ dst) {
+slab16_conv_kernel(Slab16Params p, const E* __restrict__ src, const E* __restrict__ wgt,
+                   const float* __restrict__ bias, E* __restrict__ dst) {
   extern __shared__ uint4 lds16[];
   uint4* Xs = lds16;                            // [2][x_cells]
   uint4* As = lds16 + 2 * p.x_cells;            // [2][a_cells]
@@ -398,11 +398,11 @@ slab16_conv_kernel(Slab16Params p, const bf16_t* __restrict__ src, const bf16_t*
 
     auto frag = [](uint4 v) { return __builtin_bit_cast(bf16x8, v); };
     auto mma32 = [&](int j, uint4 a, uint4 b) {
-      acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(a), frag(b), acc[j], 0, 0, 0);
+      acc[j] = Lo16<E>::mma32(frag(a), frag(b), acc[j]);
     };
     auto mma16 = [&](uint4 a0, uint4 a1, uint4 b) {
-      acc16[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(a0), frag(b), acc16[0], 0, 0, 0);
-      acc16[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(a1), frag(b), acc16[1], 0, 0, 0);
+      acc16[0] = Lo16<E>::mma16(frag(a0), frag(b), acc16[0]);
+      acc16[1] = Lo16<E>::mma16(frag(a1), frag(b), acc16[1]);
     };
 
     __syncthreads();                             // chunk 0 is in buffer 0
@@ -673,10 +673,10 @@ bool plan(Slab16Params* p, size_t* shmem) {
 // results of the last image that contain it: one thread per result of the box rows
 // [r0, r0+nr) x columns [c0, c0+nc) x the channels of the last group (those results are
 // rounded to bf16 twice).
-template <bool BWD>
+template <typename E, bool BWD>
 __global__ void __launch_bounds__(256)
-slab16_tail_fix(ConvGeom g, const bf16_t* __restrict__ src, const bf16_t* __restrict__ w,
-                bf16_t* __restrict__ dst, int r0, int nr, int c0, int nc) {
+slab16_tail_fix(ConvGeom g, const E* __restrict__ src, const E* __restrict__ w,
+                E* __restrict__ dst, int r0, int nr, int c0, int nc) {
   const int nch = BWD ? g.Cg : g.Kg;
   const int idx = blockIdx.x * 256 + threadIdx.x;
   if (idx >= nch * nr * nc) return;
@@ -703,7 +703,7 @@ slab16_tail_fix(ConvGeom g, const bf16_t* __restrict__ src, const bf16_t* __rest
   st(dst, o, ld(dst, o) + last * wv);
 }
 
-template <bool BWD>
+template <typename E, bool BWD>
 int launch(const ConvGeom& g, Slab16Params& p, const void* src, const void* wgt, const float* bias, void* dst,
            hipStream_t s) {
   const long long sbytes = (long long)p.N * p.SC * p.SH * p.SW * 2;
@@ -721,11 +721,11 @@ int launch(const ConvGeom& g, Slab16Params& p, const void* src, const void* wgt,
     p.wvec = BWD ? (al && p.a_cstride % 8 == 0 && (BM * p.KHW) % 8 == 0 && (BM * p.a_mstride) % 8 == 0)
                  : (al && p.KHW == 9 && p.a_mstride % 8 == 0 && p.SCg % 8 == 0);
   }
-  auto kernel = slab16_conv_kernel<BWD>;
+  auto kernel = slab16_conv_kernel<E, BWD>;
   if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
   const dim3 grid((unsigned)(p.VS > 1 ? (p.N + p.VS - 1) / p.VS : p.N * p.tiles_per_image), (unsigned)(p.mtiles * p.groups));
-  hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const bf16_t*>(src),
-                     static_cast<const bf16_t*>(wgt), bias, static_cast<bf16_t*>(dst));
+  hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const E*>(src),
+                     static_cast<const E*>(wgt), bias, static_cast<E*>(dst));
   if (p.SW & 1) {
     // results of the last image whose window reaches the last source element
     int r0, r1, c0, c1;
@@ -738,9 +738,9 @@ int launch(const ConvGeom& g, Slab16Params& p, const void* src, const void* wgt,
     }
     if (r1 >= r0 && c1 >= c0) {
       const int nr = r1 - r0 + 1, nc = c1 - c0 + 1, total = (BWD ? g.Cg : g.Kg) * nr * nc;
-      hipLaunchKernelGGL((slab16_tail_fix<BWD>), dim3((total + 255) / 256), dim3(256), 0, s, g,
-                         static_cast<const bf16_t*>(src), static_cast<const bf16_t*>(wgt),
-                         static_cast<bf16_t*>(dst), r0, nr, c0, nc);
+      hipLaunchKernelGGL((slab16_tail_fix<E, BWD>), dim3((total + 255) / 256), dim3(256), 0, s, g,
+                         static_cast<const E*>(src), static_cast<const E*>(wgt),
+                         static_cast<E*>(dst), r0, nr, c0, nc);
     }
   }
   return check_launch("conv2d (bf16 mfma slab)");
@@ -781,20 +781,20 @@ long long mfma_slab16_conv_fwd_workgroups(const ConvGeom& g) {
 }
 
 int mfma_slab16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
-                         hipStream_t s) {
+                         hipStream_t s, int dtype) {
   // strides: results step through the slab; 1x1 windows with a stride are left to the GEMM kernels
   if ((g.sy != 1 || g.sx != 1) && g.KH * g.KW == 1) return -1;
   Slab16Params p{};
   fill_fwd(g, &p);
-  return launch<false>(g, p, x, w, bias, y, s);
+  return by_lo16(dtype, [&](auto* e_) { return launch<FLHIP_T_OF(e_), false>(g, p, x, w, bias, y, s); });
 }
 
 int mfma_slab16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx,
-                              hipStream_t s) {
+                              hipStream_t s, int dtype) {
   if (g.sy != 1 || g.sx != 1) return -1;
   Slab16Params p{};
   fill_bwd(g, &p);
-  return launch<true>(g, p, dy, w, nullptr, dx, s);
+  return by_lo16(dtype, [&](auto* e_) { return launch<FLHIP_T_OF(e_), true>(g, p, dy, w, nullptr, dx, s); });
 }
 
 }  // namespace flhip

@@ -62,10 +62,10 @@ struct Strip16Params {
   unsigned src_bytes, wt_bytes;
 };
 
-template <bool BWD, int R>
+template <typename E, bool BWD, int R>
 __global__ void __launch_bounds__(ST_THREADS, 2)
-strip16_conv_kernel(Strip16Params p, const bf16_t* __restrict__ src, const bf16_t* __restrict__ wgt,
-                    const float* __restrict__ bias, bf16_t* __restrict__ dst) {
+strip16_conv_kernel(Strip16Params p, const E* __restrict__ src, const E* __restrict__ wgt,
+                    const float* __restrict__ bias, E* __restrict__ dst) {
   static_assert(R == ST_R, "the slab plane pitch is laid out for ST_R result rows");
   constexpr int RS = R + 2;
   constexpr int OOB = (int)0x80000000;
@@ -266,7 +266,7 @@ strip16_conv_kernel(Strip16Params p, const bf16_t* __restrict__ src, const bf16_
   // part g = the four positions of elements 4g .. 4g+3
   auto stage_part = [&](const floatx16& a, int o, int g) {
     if (blk * 32 + g * 8 + fh * 4 < DW) {
-      const uintx2_t v = {pack_bf16(a[4 * g] + bv, a[4 * g + 1] + bv), pack_bf16(a[4 * g + 2] + bv, a[4 * g + 3] + bv)};
+      const uintx2_t v = {Lo16<E>::pack(a[4 * g] + bv, a[4 * g + 1] + bv), Lo16<E>::pack(a[4 * g + 2] + bv, a[4 * g + 3] + bv)};
       *reinterpret_cast<uintx2_t*>(srow + o * DW + g * 8) = v;
     }
   };
@@ -274,7 +274,7 @@ strip16_conv_kernel(Strip16Params p, const bf16_t* __restrict__ src, const bf16_
   auto mma = [&](int rr, int dr, uint4 f, int j) {
     const int o = rr - dr;
     if (o >= 0 && o < R)
-      acc[o % 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(f), frag(wf[dr * 3 + j % 3][j / 3]), acc[o % 3], 0, 0, 0);
+      acc[o % 3] = Lo16<E>::mma32(frag(f), frag(wf[dr * 3 + j % 3][j / 3]), acc[o % 3]);
   };
 
   // fragment i = (slab row i / 12, contraction step (i % 12) / 3, column shift i % 3); its read
@@ -334,7 +334,7 @@ strip16_conv_kernel(Strip16Params p, const bf16_t* __restrict__ src, const bf16_
   }
 }
 
-template <bool BWD>
+template <typename E, bool BWD>
 int launch(Strip16Params& p, const void* src, const void* wgt, const float* bias, void* dst, hipStream_t s) {
   constexpr int R = ST_R;
   if (p.SCg != 64 || p.DCg % ST_BM != 0 || p.SW % 8 != 0 || p.SW <= 32 || p.SW > 64 || p.SH % R != 0) return -1;
@@ -355,11 +355,11 @@ int launch(Strip16Params& p, const void* src, const void* wgt, const float* bias
   const size_t cells = (size_t)ST_CG * ST_XPL + 8 + (size_t)ST_CG * ST_APL + 8;
   const size_t shmem = cells * 16;
   if ((size_t)ST_BM * p.SPI * 2 > ((size_t)ST_CG * ST_APL + 8) * 16) return -1;
-  auto kernel = strip16_conv_kernel<BWD, R>;
+  auto kernel = strip16_conv_kernel<E, BWD, R>;
   if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
   const dim3 grid((unsigned)(p.SH / R), (unsigned)p.N, (unsigned)(p.mtiles * p.groups));
-  hipLaunchKernelGGL(kernel, grid, dim3(ST_THREADS), shmem, s, p, static_cast<const bf16_t*>(src),
-                     static_cast<const bf16_t*>(wgt), bias, static_cast<bf16_t*>(dst));
+  hipLaunchKernelGGL(kernel, grid, dim3(ST_THREADS), shmem, s, p, static_cast<const E*>(src),
+                     static_cast<const E*>(wgt), bias, static_cast<E*>(dst));
   return check_launch("conv2d (bf16 mfma strip)");
 }
 
@@ -371,22 +371,22 @@ bool strip16_shape(const ConvGeom& g) {
 }  // namespace
 
 int mfma_strip16_conv_fwd(const ConvGeom& g, const void* x, const void* w, const float* bias, void* y,
-                          hipStream_t s) {
+                          hipStream_t s, int dtype) {
   if (!strip16_shape(g)) return -1;
   Strip16Params p{};
   p.N = g.N; p.SC = g.C; p.SH = g.H; p.SW = g.W; p.DC = g.K;
   p.groups = g.groups; p.SCg = g.Cg; p.DCg = g.Kg;
   p.a_mstride = g.Cg * 9; p.a_cstride = 9; p.w_group_stride = g.Kg * g.Cg * 9;
-  return launch<false>(p, x, w, bias, y, s);
+  return by_lo16(dtype, [&](auto* e_) { return launch<FLHIP_T_OF(e_), false>(p, x, w, bias, y, s); });
 }
 
-int mfma_strip16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s) {
+int mfma_strip16_conv_bwd_data(const ConvGeom& g, const void* dy, const void* w, void* dx, hipStream_t s, int dtype) {
   if (!strip16_shape(g)) return -1;
   Strip16Params p{};
   p.N = g.N; p.SC = g.K; p.SH = g.OH; p.SW = g.OW; p.DC = g.C;
   p.groups = g.groups; p.SCg = g.Kg; p.DCg = g.Cg;
   p.a_mstride = 9; p.a_cstride = g.Cg * 9; p.w_group_stride = g.Kg * g.Cg * 9;
-  return launch<true>(p, dy, w, nullptr, dx, s);
+  return by_lo16(dtype, [&](auto* e_) { return launch<FLHIP_T_OF(e_), true>(p, dy, w, nullptr, dx, s); });
 }
 
 }  // namespace flhip

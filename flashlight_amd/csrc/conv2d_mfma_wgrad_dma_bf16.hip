@@ -111,9 +111,9 @@ struct WdStages {
 // the first group of an image needs no stage before it (row -1 is loaded as zeros); after the last group of an
 // image or of the workgroup's range one stage only loads (the rows below the last group).
 constexpr int NW = 8;
-template <int NK16, int G>
+template <typename E, int NK16, int G>
 __global__ void __launch_bounds__(64 * NW, 1)
-wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy, float* __restrict__ out) {
+wgrad_dma_kernel(WdParams p, const E* __restrict__ x, const E* __restrict__ dy, float* __restrict__ out) {
   constexpr bool IMG = G == 0;          // a stage is a whole image
   constexpr bool GRP = G >= 2;          // a stage is a group of G rows
   constexpr int CPR = GRP ? 8 / G : 8;  // cells of a row in a slot
@@ -224,9 +224,9 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
           uint16_t* qd = reinterpret_cast<uint16_t*>(dring + ds * WD_SLOT + (NW * i + wave) * 1024 + lane * 16);
           const int ox = xoff[i] + img * p.C * P * 2, od = doff[i] + img * p.K * P * 2;
           if ((unsigned)ox + 16u > p.x_bytes)
-            for (int e = 0; e < p.keep; ++e) q[e] = x[(ox >> 1) + e];
+            for (int e = 0; e < p.keep; ++e) q[e] = reinterpret_cast<const uint16_t*>(x)[(ox >> 1) + e];
           if ((unsigned)od + 16u > p.dy_bytes)
-            for (int e = 0; e < p.keep; ++e) qd[e] = dy[(od >> 1) + e];
+            for (int e = 0; e < p.keep; ++e) qd[e] = reinterpret_cast<const uint16_t*>(dy)[(od >> 1) + e];
           for (int e = p.keep; e < 8; ++e) q[e] = 0;
         }
       }
@@ -319,8 +319,8 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
         float t = 0.f;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-          t += 2u * k >= sh_skip[i] ? __uint_as_float(w[k] << 16) : 0.f;          // (the tail is masked already)
-          t += 2u * k + 1 >= sh_skip[i] ? __uint_as_float(w[k] & 0xffff0000u) : 0.f;
+          t += 2u * k >= sh_skip[i] ? Lo16<E>::lo(w[k]) : 0.f;                    // (the tail is masked already)
+          t += 2u * k + 1 >= sh_skip[i] ? Lo16<E>::hi(w[k]) : 0.f;
         }
         dbsum[i] += sh_on[i] ? t : 0.f;
       }
@@ -403,7 +403,7 @@ wgrad_dma_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restr
 #define WD_MULT(SET)                                                                                   \
   _Pragma("unroll") for (int kh = 0; kh < 3; ++kh)                                                     \
     _Pragma("unroll") for (int kw = 0; kw < 3; ++kw)                                                   \
-      acc[kh][kw] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SET][kw], fb[SET][kh], acc[kh][kw], 0, 0, 0);
+      acc[kh][kw] = Lo16<E>::mma32(fa[SET][kw], fb[SET][kh], acc[kh][kw]);
     if (IMG || GRP) {
       // the first two stages multiply too: their shifted copies, and the first fragments of stage 0
       __syncthreads();
@@ -646,9 +646,9 @@ __device__ __forceinline__ int4 w3_stage(const WdParams& p, int row_begin, int n
   return make_int4((img * p.C * p.H + ih0) * p.W * 2, ih0, (img * p.K * p.H + max(oh0, 0)) * p.W * 2, oh0);
 }
 
-template <int G>
+template <typename E, int G>
 __global__ void __launch_bounds__(512, 1)
-wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy, float* __restrict__ out) {
+wgrad_dma32_kernel(WdParams p, const E* __restrict__ x, const E* __restrict__ dy, float* __restrict__ out) {
   constexpr bool IMG = G == 0;          // a stage is a whole image
   constexpr bool GRP = G >= 2;          // a stage is a group of G rows
   constexpr int CPR = GRP ? 8 / G : 8;  // cells of a row in a slot
@@ -732,7 +732,7 @@ wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __res
         uint16_t* q = reinterpret_cast<uint16_t*>(cellp);
         const int o = loff + img * (ldx ? p.C : p.K) * P * 2;
         if ((unsigned)o + 16u > (ldx ? p.x_bytes : p.dy_bytes)) {
-          const bf16_t* src = ldx ? x : dy;
+          const uint16_t* src = reinterpret_cast<const uint16_t*>(ldx ? x : dy);
           for (int e = 0; e < p.keep; ++e) q[e] = src[(o >> 1) + e];
         }
         if (ldx)
@@ -828,7 +828,7 @@ wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __res
     uint32_t w[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k)
-      w[k] = ((2 * k >= skip && 2 * k < keep) ? 0x3f80u : 0u) | ((2 * k + 1 >= skip && 2 * k + 1 < keep) ? 0x3f800000u : 0u);
+      w[k] = ((2 * k >= skip && 2 * k < keep) ? (Lo16<E>::ONE2 & 0xffffu) : 0u) | ((2 * k + 1 >= skip && 2 * k + 1 < keep) ? (Lo16<E>::ONE2 & 0xffff0000u) : 0u);
     ones = __builtin_bit_cast(bf16x8, uintx4_t{w[0], w[1], w[2], w[3]});
   }
   floatx16 acc[3][3], accb;
@@ -990,14 +990,14 @@ wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __res
         // the products of stage s; each fragment register is refilled with stage s + 2's as soon as its last reader has issued
         {
 #pragma unroll
-          for (int kw = 0; kw < 3; ++kw) acc[0][kw] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kw], fb[0], acc[0][kw], 0, 0, 0);
+          for (int kw = 0; kw < 3; ++kw) acc[0][kw] = Lo16<E>::mma32(fa[kw], fb[0], acc[0][kw]);
         }
         __builtin_amdgcn_sched_barrier(0);
         load_fb(std::integral_constant<int, S2>{}, I0{});
         __builtin_amdgcn_sched_barrier(0);
         {
 #pragma unroll
-          for (int kw = 0; kw < 3; ++kw) acc[1][kw] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kw], fb[1], acc[1][kw], 0, 0, 0);
+          for (int kw = 0; kw < 3; ++kw) acc[1][kw] = Lo16<E>::mma32(fa[kw], fb[1], acc[1][kw]);
         }
         __builtin_amdgcn_sched_barrier(0);
         load_fb(std::integral_constant<int, S2>{}, I1{});
@@ -1005,8 +1005,8 @@ wgrad_dma32_kernel(WdParams p, const bf16_t* __restrict__ x, const bf16_t* __res
         __builtin_amdgcn_sched_barrier(0);
         {
 #pragma unroll
-          for (int kw = 0; kw < 3; ++kw) acc[2][kw] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kw], fb[2], acc[2][kw], 0, 0, 0);
-          if (do_db) accb = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1], ones, accb, 0, 0, 0);
+          for (int kw = 0; kw < 3; ++kw) acc[2][kw] = Lo16<E>::mma32(fa[kw], fb[2], acc[2][kw]);
+          if (do_db) accb = Lo16<E>::mma32(fa[1], ones, accb);
         }
         __builtin_amdgcn_sched_barrier(0);
         load_fb(std::integral_constant<int, S2>{}, I2{});
@@ -1208,8 +1208,9 @@ size_t mfma_wgrad_dma16_ws(const ConvGeom& g) {
 }
 
 // -1 when the shape is not this kernel's
-int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes,
-                     hipStream_t s, int tile) {
+template <typename E>
+static int wgrad_dma16_run(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes,
+                           hipStream_t s, int tile) {
   WdParams p{};
   if (!dw) return -1;
   const bool t32 = tile == 0 ? wd_use32(g, &p) : tile == W3_T && wd_plan(g, &p, W3_T);
@@ -1218,15 +1219,15 @@ int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw
   if (!ws || ws_bytes < wd_ws_bytes(p) || reinterpret_cast<uintptr_t>(ws) % 16 != 0) return -1;   // (the reduce kernels read 16 bytes at a time)
   p.want_db = db != nullptr;
   float* part = static_cast<float*>(ws);
-  const bf16_t* xp = static_cast<const bf16_t*>(x);
-  const bf16_t* dyp = static_cast<const bf16_t*>(dy);
+  const E* xp = static_cast<const E*>(x);
+  const E* dyp = static_cast<const E*>(dy);
   if (t32) {
     const unsigned wgs = (unsigned)(p.nsplit * p.ctiles * p.mtiles);
     const dim3 grid((wgs + 7) / 8 * 8);
 #define W3_LAUNCH(GR)                                                                                      \
   {                                                                                                        \
-    if (!mfma_allow_lds(reinterpret_cast<const void*>(wgrad_dma32_kernel<GR>), W3_LDS)) return -1;         \
-    hipLaunchKernelGGL((wgrad_dma32_kernel<GR>), grid, dim3(512), W3_LDS, s, p, xp, dyp, part);            \
+    if (!mfma_allow_lds(reinterpret_cast<const void*>(wgrad_dma32_kernel<E, GR>), W3_LDS)) return -1;      \
+    hipLaunchKernelGGL((wgrad_dma32_kernel<E, GR>), grid, dim3(512), W3_LDS, s, p, xp, dyp, part);         \
   }
     if (p.G == 0) W3_LAUNCH(0)
     else if (p.G == 1) W3_LAUNCH(1)
@@ -1240,8 +1241,8 @@ int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw
   const dim3 grid((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles));
 #define WD_LAUNCH(NK, GR)                                                                                      \
   {                                                                                                            \
-    if (!mfma_allow_lds(reinterpret_cast<const void*>(wgrad_dma_kernel<NK, GR>), WD_LDS)) return -1;           \
-    hipLaunchKernelGGL((wgrad_dma_kernel<NK, GR>), grid, dim3(64 * NW), WD_LDS, s, p, xp, dyp, part);          \
+    if (!mfma_allow_lds(reinterpret_cast<const void*>(wgrad_dma_kernel<E, NK, GR>), WD_LDS)) return -1;        \
+    hipLaunchKernelGGL((wgrad_dma_kernel<E, NK, GR>), grid, dim3(64 * NW), WD_LDS, s, p, xp, dyp, part);       \
   }
   if (p.G == 0) WD_LAUNCH(4, 0)
   else if (p.G == 1) WD_LAUNCH(4, 1)
@@ -1262,5 +1263,9 @@ int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw
   return check_launch("conv2d_bwd_filter 3x3 (bf16 mfma, direct-to-LDS)");
 }
 
-}  // namespace flhip
+int mfma_wgrad_dma16(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws, size_t ws_bytes,
+                     hipStream_t s, int tile, int dtype) {
+  return by_lo16(dtype, [&](auto* e_) { return wgrad_dma16_run<FLHIP_T_OF(e_)>(g, x, dy, dw, db, ws, ws_bytes, s, tile); });
+}
 
+}  // namespace flhip

@@ -73,9 +73,9 @@ struct W16Params {
   unsigned x_bytes, dy_bytes;
 };
 
-template <int NXI, int NDI>
+template <typename E, int NXI, int NDI>
 __global__ void __launch_bounds__(THREADS, 2)
-wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy,
+wgrad16_kernel(W16Params p, const E* __restrict__ x, const E* __restrict__ dy,
                float* __restrict__ out, float* __restrict__ db_out) {
   extern __shared__ uint4 lds16[];
   float* lds = reinterpret_cast<float*>(lds16);
@@ -212,7 +212,7 @@ wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restri
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
             const unsigned d = k == 0 ? v.x : k == 1 ? v.y : k == 2 ? v.z : v.w;
-            s += __uint_as_float(d << 16) + __uint_as_float(d & 0xffff0000u);
+            s += Lo16<E>::lo(d) + Lo16<E>::hi(d);
           }
           dbp[i] += s;
         }
@@ -311,14 +311,14 @@ wgrad16_kernel(W16Params p, const bf16_t* __restrict__ x, const bf16_t* __restri
     const uint4 n0 = ap[OFF], n1 = ap[(OFF) + 2];                        \
     const uint4 m0 = aq0[OFF], m1 = aq1[OFF];                            \
     _Pragma("unroll") for (int j = 0; j < NB32; ++j)                     \
-      acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(a[0]), frag(b[j][0]), acc[j], 0, 0, 0); \
+      acc[j] = Lo16<E>::mma32(frag(a[0]), frag(b[j][0]), acc[j]); \
     _Pragma("unroll") for (int j = 0; j < NB32; ++j) {                   \
-      acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag(a[1]), frag(b[j][1]), acc[j], 0, 0, 0); \
+      acc[j] = Lo16<E>::mma32(frag(a[1]), frag(b[j][1]), acc[j]); \
       b[j][0] = bp[j][OFF];                                              \
       b[j][1] = bp[j][(OFF) + 2];                                        \
     }                                                                    \
-    acc16[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(sa0), frag(sb), acc16[0], 0, 0, 0); \
-    acc16[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(frag(sa1), frag(sb), acc16[1], 0, 0, 0); \
+    acc16[0] = Lo16<E>::mma16(frag(sa0), frag(sb), acc16[0]); \
+    acc16[1] = Lo16<E>::mma16(frag(sa1), frag(sb), acc16[1]); \
     sb = bq[OFF];                                                        \
     a[0] = n0;                                                           \
     a[1] = n1;                                                           \
@@ -424,7 +424,7 @@ size_t mfma_wgrad16_ws(const ConvGeom& g) {
 }
 
 int mfma_wgrad16(const ConvGeom& g, const void* x, const void* dy, float* dw, float* db, void* ws,
-                 size_t ws_bytes, hipStream_t s) {
+                 size_t ws_bytes, hipStream_t s, int dtype) {
   if (!dw) return -1;
   W16Params p{};
   if (!plan(g, &p)) return -1;
@@ -443,11 +443,15 @@ int mfma_wgrad16(const ConvGeom& g, const void* x, const void* dy, float* dw, fl
   const size_t shmem = (size_t)3 * p.buf_cells * 16;
   // loader units per thread and step the shape needs (fewer = fewer loader instructions)
   const bool small = CB * 3 <= 2 * 4 * p.RPW && BM <= 4 * p.RPW;
-  auto kernel = small ? wgrad16_kernel<2, 1> : wgrad16_kernel<NXI_MAX, NDI_MAX>;
-  if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
   const dim3 grid(p.nsplit, p.nhalves * p.mtiles, g.groups);
-  hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const bf16_t*>(x),
-                     static_cast<const bf16_t*>(dy), out, db);
+  const int rc = by_lo16(dtype, [&](auto* e_) {
+    using E = FLHIP_T_OF(e_);
+    auto kernel = small ? wgrad16_kernel<E, 2, 1> : wgrad16_kernel<E, NXI_MAX, NDI_MAX>;
+    if (!mfma_allow_lds(reinterpret_cast<const void*>(kernel), shmem)) return -1;
+    hipLaunchKernelGGL(kernel, grid, dim3(THREADS), shmem, s, p, static_cast<const E*>(x), static_cast<const E*>(dy), out, db);
+    return 0;
+  });
+  if (rc) return rc;
   if (p.nsplit > 1)
     wgrad_reduce_launch(static_cast<const float*>(ws), p.nsplit, p.E, p.K, p.want_db, dw, db, s);
   return check_launch("conv2d_bwd_filter (bf16 mfma)");
