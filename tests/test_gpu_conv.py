@@ -787,12 +787,12 @@ FULL = [
 ]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape", FULL)
 def test_full_size_oracle(shape, dtype):
     """y, dx, dw, db of every full-size layer against the CPU checker, whole tensors."""
     xs, ws, st, pd = shape
-    lo = dtype == torch.bfloat16
+    lo = dtype != torch.float32
     for name, (got, ref) in _run((xs, ws, st, pd, (1, 1), 1), 43, dtype).items():
         tol = (1e-4 if name in ("dw", "db") else 4e-3) if lo else F32_TOL
         assert got.shape == ref.shape, name
@@ -1002,29 +1002,29 @@ PLAN_CASES = [
 ]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("shape", PLAN_CASES)
 def test_backward_passes_by_plan(shape, dtype):
     import ctypes as C
     from flashlight_amd import capi
     L = capi.lib()
     xs, ws_, st, pd = shape
-    lo = dtype == torch.bfloat16
+    lo = dtype != torch.float32
     rng = np.random.default_rng(71)
     x = rng.standard_normal(xs).astype(np.float32)
     w = (rng.standard_normal(ws_) / np.sqrt(ws_[1] * ws_[2] * ws_[3])).astype(np.float32)
     if lo:
-        x, w = bf16_round(x), bf16_round(w)
+        x, w = round_to(x, dtype), round_to(w, dtype)
     d = flref.conv_desc(xs, ws_, st, pd, (1, 1), 1)
     y_shape = flref.conv2d_fwd(d, x, w, None).shape
     dy = rng.standard_normal(y_shape).astype(np.float32)
     if lo:
-        dy = bf16_round(dy)
+        dy = round_to(dy, dtype)
     dx_ref = flref.conv2d_bwd_data(d, dy, w)
     dw_ref, db_ref = flref.conv2d_bwd_filter(d, x, dy)
     xd, wd, dyd = dev(x, dtype), dev(w, dtype), dev(dy, dtype)
     cd = capi.ConvDesc(xs[0], xs[1], xs[2], xs[3], ws_[0], ws_[2], ws_[3], st[0], st[1], pd[0], pd[1], 1, 1, 1,
-                       capi.BF16 if lo else capi.F32)
+                       capi.F32 if not lo else capi.BF16 if dtype == torch.bfloat16 else capi.F16)
     S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     P = lambda t: C.c_void_p(t.data_ptr())
     nd = L.flhip_conv2d_plan_count(capi.CONV_BWD_DATA)
