@@ -732,9 +732,11 @@ __device__ __forceinline__ void buf_st8(__amdgpu_buffer_rsrc_t r, int byte_off, 
   const uintx4_t t = {v.x, v.y, v.z, v.w};
   __builtin_amdgcn_raw_buffer_store_b128(t, r, byte_off, 0, 2);
 }
-__device__ __forceinline__ float bf_lo(uint32_t u) { return __uint_as_float(u << 16); }
-__device__ __forceinline__ float bf_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
-__device__ __forceinline__ uint32_t bf_pack(float lo, float hi) {
+// (HALF: the two 16-bit values are IEEE halves, else bf16; the kernels below hold either as raw words)
+template <bool HALF> __device__ __forceinline__ float bf_lo(uint32_t u) { return HALF ? f16lo(u) : __uint_as_float(u << 16); }
+template <bool HALF> __device__ __forceinline__ float bf_hi(uint32_t u) { return HALF ? f16hi(u) : __uint_as_float(u & 0xffff0000u); }
+template <bool HALF> __device__ __forceinline__ uint32_t bf_pack(float lo, float hi) {
+  if (HALF) return pack_f16(lo, hi);
   return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
 }
 // keeps the halves of d whose counterpart in y is a positive bf16 value
@@ -769,7 +771,7 @@ __device__ __forceinline__ float uniform(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
 }
 
-template <int RES_THREADS, int K, int FUSE = 0, bool RES_EARLY = false>
+template <bool HALF, int RES_THREADS, int K, int FUSE = 0, bool RES_EARLY = false>
 __global__ void __launch_bounds__(RES_THREADS)
 bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_t* __restrict__ y,
                    BnTrainArgs a, BnFuseFwd<bf16_t> fu = BnFuseFwd<bf16_t>{nullptr, 0, nullptr}) {
@@ -777,7 +779,7 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
   __shared__ float sh[2];
   const __amdgpu_buffer_rsrc_t xr_ = make_rsrc(x, bytes), yr_ = make_rsrc(y, bytes);
   const long long c = res_feature(g);
-  const float shift = ld(x, (size_t)(c * g.inner));
+  const float shift = HALF ? f16_to_f32(f16_t{x[(size_t)(c * g.inner)]}) : ld(x, (size_t)(c * g.inner));
   // (the kernels that hold 25 vectors per thread have no registers to keep the scalars through the statistics)
   constexpr bool EARLY = K <= 16;
   BnTrainPre pre = EARLY ? bn_preload(a, c) : BnTrainPre{};
@@ -795,7 +797,7 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
     float p1 = 0.f, p2 = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const float t0 = bf_lo(w[j]) - shift, t1 = bf_hi(w[j]) - shift;
+      const float t0 = bf_lo<HALF>(w[j]) - shift, t1 = bf_hi<HALF>(w[j]) - shift;
       p1 += t0 + t1;
       p2 += t0 * t0 + t1 * t1;
     }
@@ -823,30 +825,30 @@ bn_train_resident8(BnGeom g, unsigned bytes, const bf16_t* __restrict__ x, bf16_
       auto pos = [](uint32_t w, unsigned blo, unsigned bhi) {
         return ((int)(w << 16) > 0 ? blo : 0u) | ((int)(w & 0xffff0000u) > 0 ? bhi : 0u);
       };
-      v.x = bf_pack(fmaxf((bf_lo(v.x) - mean) * scale + bt + bf_lo(rv.x), lo), fmaxf((bf_hi(v.x) - mean) * scale + bt + bf_hi(rv.x), lo));
+      v.x = bf_pack<HALF>(fmaxf((bf_lo<HALF>(v.x) - mean) * scale + bt + bf_lo<HALF>(rv.x), lo), fmaxf((bf_hi<HALF>(v.x) - mean) * scale + bt + bf_hi<HALF>(rv.x), lo));
       unsigned bits = pos(v.x, 1u, 2u);
       __builtin_amdgcn_sched_barrier(0);   // one word at a time: the packing temporaries of all four do not fit
-      v.y = bf_pack(fmaxf((bf_lo(v.y) - mean) * scale + bt + bf_lo(rv.y), lo), fmaxf((bf_hi(v.y) - mean) * scale + bt + bf_hi(rv.y), lo));
+      v.y = bf_pack<HALF>(fmaxf((bf_lo<HALF>(v.y) - mean) * scale + bt + bf_lo<HALF>(rv.y), lo), fmaxf((bf_hi<HALF>(v.y) - mean) * scale + bt + bf_hi<HALF>(rv.y), lo));
       bits |= pos(v.y, 4u, 8u);
       __builtin_amdgcn_sched_barrier(0);
-      v.z = bf_pack(fmaxf((bf_lo(v.z) - mean) * scale + bt + bf_lo(rv.z), lo), fmaxf((bf_hi(v.z) - mean) * scale + bt + bf_hi(rv.z), lo));
+      v.z = bf_pack<HALF>(fmaxf((bf_lo<HALF>(v.z) - mean) * scale + bt + bf_lo<HALF>(rv.z), lo), fmaxf((bf_hi<HALF>(v.z) - mean) * scale + bt + bf_hi<HALF>(rv.z), lo));
       bits |= pos(v.z, 0x100u, 0x200u);
       __builtin_amdgcn_sched_barrier(0);
-      v.w = bf_pack(fmaxf((bf_lo(v.w) - mean) * scale + bt + bf_lo(rv.w), lo), fmaxf((bf_hi(v.w) - mean) * scale + bt + bf_hi(rv.w), lo));
+      v.w = bf_pack<HALF>(fmaxf((bf_lo<HALF>(v.w) - mean) * scale + bt + bf_lo<HALF>(rv.w), lo), fmaxf((bf_hi<HALF>(v.w) - mean) * scale + bt + bf_hi<HALF>(rv.w), lo));
       bits |= pos(v.w, 0x400u, 0x800u);
       // two mask bytes per vector (8 elements)
       if (FUSE == 2) __builtin_amdgcn_raw_buffer_store_b16((uint16_t)bits, mr_, mask_off(off, 2), 0, 0);
     } else {
-      v.x = bf_pack((bf_lo(v.x) - mean) * scale + bt, (bf_hi(v.x) - mean) * scale + bt);
-      v.y = bf_pack((bf_lo(v.y) - mean) * scale + bt, (bf_hi(v.y) - mean) * scale + bt);
-      v.z = bf_pack((bf_lo(v.z) - mean) * scale + bt, (bf_hi(v.z) - mean) * scale + bt);
-      v.w = bf_pack((bf_lo(v.w) - mean) * scale + bt, (bf_hi(v.w) - mean) * scale + bt);
+      v.x = bf_pack<HALF>((bf_lo<HALF>(v.x) - mean) * scale + bt, (bf_hi<HALF>(v.x) - mean) * scale + bt);
+      v.y = bf_pack<HALF>((bf_lo<HALF>(v.y) - mean) * scale + bt, (bf_hi<HALF>(v.y) - mean) * scale + bt);
+      v.z = bf_pack<HALF>((bf_lo<HALF>(v.z) - mean) * scale + bt, (bf_hi<HALF>(v.z) - mean) * scale + bt);
+      v.w = bf_pack<HALF>((bf_lo<HALF>(v.w) - mean) * scale + bt, (bf_hi<HALF>(v.w) - mean) * scale + bt);
     }
     buf_st8(yr_, off, v);
   });
 }
 
-template <int RES_THREADS, int K, int FUSE = 0>
+template <bool HALF, int RES_THREADS, int K, int FUSE = 0>
 __global__ void __launch_bounds__(RES_THREADS)
 bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ x, const bf16_t* __restrict__ dy,
                  bf16_t* __restrict__ dx, BnBwdArgs a, BnFuseBwd<bf16_t> fu = BnFuseBwd<bf16_t>{nullptr, nullptr, nullptr}) {
@@ -898,9 +900,9 @@ bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ 
     float p1 = 0.f, p2 = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const float d0 = bf_lo(dw[j]), d1 = bf_hi(dw[j]);
+      const float d0 = bf_lo<HALF>(dw[j]), d1 = bf_hi<HALF>(dw[j]);
       p1 += d0 + d1;
-      p2 += d0 * (bf_lo(xw[j]) - mean) + d1 * (bf_hi(xw[j]) - mean);
+      p2 += d0 * (bf_lo<HALF>(xw[j]) - mean) + d1 * (bf_hi<HALF>(xw[j]) - mean);
     }
     s1 += in ? p1 : 0.f;
     s2 += in ? p2 : 0.f;
@@ -922,8 +924,8 @@ bn_bwd_resident8(BnGeom g, unsigned bytes, int klim, const bf16_t* __restrict__ 
     uint32_t o[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      o[j] = bf_pack(kdy * bf_lo(dw[j]) + (kx * (bf_lo(xw[j]) - mean) + k0),
-                     kdy * bf_hi(dw[j]) + (kx * (bf_hi(xw[j]) - mean) + k0));
+      o[j] = bf_pack<HALF>(kdy * bf_lo<HALF>(dw[j]) + (kx * (bf_lo<HALF>(xw[j]) - mean) + k0),
+                     kdy * bf_hi<HALF>(dw[j]) + (kx * (bf_hi<HALF>(xw[j]) - mean) + k0));
     buf_st8(dxr_, off, make_uint4(o[0], o[1], o[2], o[3]));
     if (FUSE) buf_st8(drr_, off, d);               // no residual branch: the empty range drops the store
   });
@@ -1273,7 +1275,7 @@ static ResPlan resident_plan(const BnGeom& g, int vec, int min_c) {
 static ResPlan resident8_plan(const BnGeom& g, int vec, int dtype, int min_c) {
   ResPlan r{0, 0, 0};
   const int mode = options().bn_algo;
-  if (mode == 1 || vec != 4 || dtype != FLHIP_BF16 || g.inner % 8 != 0) return r;
+  if (mode == 1 || vec != 4 || !is_lo16(dtype) || g.inner % 8 != 0) return r;
   const long long units8 = g.units / 2;
   if (units8 > (long long)RES_KMAX * 1024) return r;
   if (g.outer * g.C * g.inner * 2 >= (1ll << 31)) return r;   // 32-bit buffer offsets
@@ -1293,25 +1295,25 @@ static ResPlan resident8_plan(const BnGeom& g, int vec, int dtype, int min_c) {
   return r;
 }
 
-template <int THREADS, int K, int FUSE>
+template <bool HALF, int THREADS, int K, int FUSE>
 static int launch_train_resident8(const BnGeom& g, const bf16_t* x, bf16_t* y, const BnTrainArgs& a,
                                   const BnFuseFwd<bf16_t>& fu, hipStream_t s) {
   const unsigned bytes = (unsigned)(g.outer * g.C * g.inner * 2);
   if (FUSE && THREADS == 256 && g.C <= 2 * mfma_num_cus())
-    hipLaunchKernelGGL((bn_train_resident8<THREADS, K, FUSE, (FUSE && THREADS == 256)>), dim3((unsigned)g.C), dim3(THREADS), 0, s, g,
+    hipLaunchKernelGGL((bn_train_resident8<HALF, THREADS, K, FUSE, (FUSE && THREADS == 256)>), dim3((unsigned)g.C), dim3(THREADS), 0, s, g,
                        bytes, x, y, a, fu);
   else
-    hipLaunchKernelGGL((bn_train_resident8<THREADS, K, FUSE>), dim3((unsigned)g.C), dim3(THREADS), 0, s, g, bytes, x, y,
+    hipLaunchKernelGGL((bn_train_resident8<HALF, THREADS, K, FUSE>), dim3((unsigned)g.C), dim3(THREADS), 0, s, g, bytes, x, y,
                        a, fu);
   return check_launch("bn_fwd_train (resident, 8-wide)");
 }
 
-template <int THREADS, int K, int FUSE>
+template <bool HALF, int THREADS, int K, int FUSE>
 static int launch_bwd_resident8(const BnGeom& g, int need, const bf16_t* x, const bf16_t* dy, bf16_t* dx,
                                 const BnBwdArgs& a, const BnFuseBwd<bf16_t>& fu, hipStream_t s) {
   constexpr int KL = K < RES_KL ? K : RES_KL;
   constexpr size_t max_shmem = (size_t)KL * THREADS * sizeof(uint4);
-  auto kernel = bn_bwd_resident8<THREADS, K, FUSE>;
+  auto kernel = bn_bwd_resident8<HALF, THREADS, K, FUSE>;
   static const hipError_t attr = hipFuncSetAttribute(
       reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)max_shmem);
   if (attr != hipSuccess)
@@ -1323,23 +1325,23 @@ static int launch_bwd_resident8(const BnGeom& g, int need, const bf16_t* x, cons
   return check_launch("bn_bwd (resident, 8-wide)");
 }
 
-template <int FUSE>
+template <bool HALF, int FUSE>
 static int run_train8(const BnGeom& g, const ResPlan& r, const bf16_t* x, bf16_t* y, const BnTrainArgs& a,
                       const BnFuseFwd<bf16_t>& fu, hipStream_t s) {
-  if (r.threads == 256 && r.k == 8) return launch_train_resident8<256, 8, FUSE>(g, x, y, a, fu, s);
-  if (r.threads == 256) return launch_train_resident8<256, 16, FUSE>(g, x, y, a, fu, s);
-  if (r.k == 8) return launch_train_resident8<1024, 8, FUSE>(g, x, y, a, fu, s);
-  if (r.k == 16) return launch_train_resident8<1024, 16, FUSE>(g, x, y, a, fu, s);
-  return launch_train_resident8<1024, RES_KMAX, FUSE>(g, x, y, a, fu, s);
+  if (r.threads == 256 && r.k == 8) return launch_train_resident8<HALF, 256, 8, FUSE>(g, x, y, a, fu, s);
+  if (r.threads == 256) return launch_train_resident8<HALF, 256, 16, FUSE>(g, x, y, a, fu, s);
+  if (r.k == 8) return launch_train_resident8<HALF, 1024, 8, FUSE>(g, x, y, a, fu, s);
+  if (r.k == 16) return launch_train_resident8<HALF, 1024, 16, FUSE>(g, x, y, a, fu, s);
+  return launch_train_resident8<HALF, 1024, RES_KMAX, FUSE>(g, x, y, a, fu, s);
 }
-template <int FUSE>
+template <bool HALF, int FUSE>
 static int run_bwd8(const BnGeom& g, const ResPlan& r, const bf16_t* x, const bf16_t* dy, bf16_t* dx,
                     const BnBwdArgs& a, const BnFuseBwd<bf16_t>& fu, hipStream_t s) {
-  if (r.threads == 256 && r.k == 8) return launch_bwd_resident8<256, 8, FUSE>(g, r.need, x, dy, dx, a, fu, s);
-  if (r.threads == 256) return launch_bwd_resident8<256, 16, FUSE>(g, r.need, x, dy, dx, a, fu, s);
-  if (r.k == 8) return launch_bwd_resident8<1024, 8, FUSE>(g, r.need, x, dy, dx, a, fu, s);
-  if (r.k == 16) return launch_bwd_resident8<1024, 16, FUSE>(g, r.need, x, dy, dx, a, fu, s);
-  return launch_bwd_resident8<1024, RES_KMAX, FUSE>(g, r.need, x, dy, dx, a, fu, s);
+  if (r.threads == 256 && r.k == 8) return launch_bwd_resident8<HALF, 256, 8, FUSE>(g, r.need, x, dy, dx, a, fu, s);
+  if (r.threads == 256) return launch_bwd_resident8<HALF, 256, 16, FUSE>(g, r.need, x, dy, dx, a, fu, s);
+  if (r.k == 8) return launch_bwd_resident8<HALF, 1024, 8, FUSE>(g, r.need, x, dy, dx, a, fu, s);
+  if (r.k == 16) return launch_bwd_resident8<HALF, 1024, 16, FUSE>(g, r.need, x, dy, dx, a, fu, s);
+  return launch_bwd_resident8<HALF, 1024, RES_KMAX, FUSE>(g, r.need, x, dy, dx, a, fu, s);
 }
 
 template <typename T, int THREADS, int K, int FUSE>
@@ -1383,10 +1385,10 @@ static int run_train(const BnGeom& g, int vec, const void* x, void* y, float* ws
   const T* xp = static_cast<const T*>(x);
   T* yp = static_cast<T*>(y);
   constexpr int F1 = FUSE == 2 ? 1 : FUSE;   // element-wise kernels: no mask-byte form (never asked for: vec == 4 only)
-  if (std::is_same<T, bf16_t>::value) {
+  if (sizeof(T) == 2) {          // (bf16 and f16: the same kernels on raw 16-bit words, the arithmetic by type)
     const ResPlan r8 = resident8_plan(g, vec, FLHIP_BF16, RES_MIN_C_FWD);
     if (r8.threads)
-      return run_train8<FUSE>(g, r8, reinterpret_cast<const bf16_t*>(xp), reinterpret_cast<bf16_t*>(yp), a,
+      return run_train8<std::is_same<T, f16_t>::value, FUSE>(g, r8, reinterpret_cast<const bf16_t*>(xp), reinterpret_cast<bf16_t*>(yp), a,
                               reinterpret_cast<const BnFuseFwd<bf16_t>&>(fu), s);
   }
   {
@@ -1441,10 +1443,10 @@ static int run_bwd(const BnGeom& g, int vec, const void* x, const void* dy, void
   const T* dyp = static_cast<const T*>(dy);
   T* dxp = static_cast<T*>(dx);
   constexpr int F1 = FUSE == 2 ? 1 : FUSE;   // element-wise kernels: no mask-byte form (never asked for: vec == 4 only)
-  if (std::is_same<T, bf16_t>::value) {
+  if (sizeof(T) == 2) {
     const ResPlan r8 = resident8_plan(g, vec, FLHIP_BF16, RES_MIN_C_BWD);
     if (r8.threads)
-      return run_bwd8<FUSE>(g, r8, reinterpret_cast<const bf16_t*>(xp), reinterpret_cast<const bf16_t*>(dyp),
+      return run_bwd8<std::is_same<T, f16_t>::value, FUSE>(g, r8, reinterpret_cast<const bf16_t*>(xp), reinterpret_cast<const bf16_t*>(dyp),
                             reinterpret_cast<bf16_t*>(dxp), a, reinterpret_cast<const BnFuseBwd<bf16_t>&>(fu), s);
   }
   {

@@ -60,9 +60,10 @@ def _data(shape, axes, seed, dtype):
     return outer, C, inner, x, dy, g, b
 
 
-# f16 storage takes the kernels of the other two types with its own loads and stores: the shapes up to 4M elements
+# f16 storage takes the kernels of the other two types with its own loads, stores and conversions (the 8-wide resident
+# kernels hold bf16 and f16 alike as raw words): the shapes up to 20M elements, which reach every vector count of those
 TYPED_CASES = ([(s, a, dt) for s, a in CASES for dt in (torch.float32, torch.bfloat16)] +
-               [(s, a, torch.float16) for s, a in CASES if int(np.prod(s)) <= 4 << 20])
+               [(s, a, torch.float16) for s, a in CASES if int(np.prod(s)) <= 20 << 20])
 
 
 @pytest.mark.parametrize("shape,axes,dtype", TYPED_CASES)
@@ -145,7 +146,7 @@ def test_errors():
         fa.batchnorm(x, torch.zeros(5, device="cuda"), None, None, None, [2], True, 0.0, 1e-5)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 def test_full_size_oracle(dtype):
     """configs[2] at its stated size (56x56x256, batch 32, values N(0.5, 2), gamma N(1, 0.1),
     eps 1e-5, momentum 0.1): y, saved statistics, running statistics, dx, dgamma, dbeta
@@ -156,9 +157,9 @@ def test_full_size_oracle(dtype):
     dy = rng.standard_normal((N, Cc, 56, 56), dtype=np.float32)
     gamma = (1 + 0.1 * rng.standard_normal(Cc)).astype(np.float32)
     beta = np.zeros(Cc, np.float32)
-    lo = dtype == torch.bfloat16
+    lo = dtype != torch.float32
     if lo:
-        x, dy = bf16_round(x), bf16_round(dy)
+        x, dy = round_to(x, dtype), round_to(dy, dtype)
     y_ref, mean, var = flref.bn_fwd_train(N, Cc, HW, x, gamma, beta, 1e-5)
     dx_ref, dg_ref, db_ref = flref.bn_bwd(N, Cc, HW, x, dy, gamma, mean, var, 1e-5)
     rm, rv = torch.zeros(Cc, device="cuda"), torch.ones(Cc, device="cuda")
