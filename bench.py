@@ -43,7 +43,8 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=0, help="timed steps (default 100; 20 for --step)")
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--dtype", choices=["f32", "bf16"], default="f32")
+    ap.add_argument("--dtype", choices=["f32", "bf16", "f16"], default="f32",
+                    help="storage type (f16: with --layers, --plans or --step)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--only", default="", help="comma list of ops to time (debugging/profiling)")
     ap.add_argument("--layers", choices=["resnet50", "speech"], default="",
@@ -80,13 +81,17 @@ def main():
     fa.capi.lib()                      # fails loudly when the HIP library is missing
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    tdt = torch.float32 if a.dtype == "f32" else torch.bfloat16
+    tdt = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[a.dtype]
     if a.layers:
         return layer_sweep(a, fa, torch, tdt)
     if a.plans:
         return plan_sweep(a, fa, torch, tdt)
     if a.rnn:
         return rnn_sweep(a, fa, torch)
+    if a.dtype == "f16":
+        print("bench.py: --dtype f16 goes with --layers, --plans or --step (the bench line is quoted in f32, with bf16 beside it)",
+              file=sys.stderr)
+        return 1
     gen = torch.Generator(device=dev).manual_seed(0)
 
     def randn(*shape, scale=1.0, shift=0.0):
@@ -406,7 +411,7 @@ def layer_sweep(a, fa, torch, tdt):
     a.steps launches after a.warmup); the first layer of a network has no backward-data
     in training (its input needs no gradient), so it is left out of the totals."""
     capi, L = fa.capi, fa.capi.lib()
-    tag = capi.F32 if tdt == torch.float32 else capi.BF16
+    tag = capi.F32 if tdt == torch.float32 else capi.BF16 if tdt == torch.bfloat16 else capi.F16
     S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     P = lambda t: C.c_void_p(t.data_ptr())
 
@@ -466,7 +471,7 @@ def plan_sweep(a, fa, torch, tdt):
     default rule, of the fastest plan, and which plans the library declined.  This is the measurement that
     HipAutogradExtension::createBenchmarkOptions makes per layer at run time in benchmark mode."""
     capi, L = fa.capi, fa.capi.lib()
-    tag = capi.F32 if tdt == torch.float32 else capi.BF16
+    tag = capi.F32 if tdt == torch.float32 else capi.BF16 if tdt == torch.bfloat16 else capi.F16
     S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     P = lambda t: C.c_void_p(t.data_ptr())
     steps = a.steps if a.steps != 100 else 20
