@@ -34,6 +34,8 @@ struct OpAct {
     if (OP == FLHIP_ACT_LOG) return logf(x);                                          // :403-404
     if (OP == FLHIP_ACT_SWISH) return x * act_sigmoid(a * x);                         // :498-500
     if (OP == FLHIP_ACT_SCALE) return a * x;
+    if (OP == FLHIP_ACT_LEAKY) return fmaxf(x, a * x);                                // Activations.cpp:102-104
+    if (OP == FLHIP_ACT_THRESHOLD) return x >= a ? x : 0.f;                           // :151-154
     return act_sigmoid(x);                                                            // :488-489
   }
 };
@@ -53,6 +55,8 @@ struct OpActBwd {
       return dy * (sg + x * a * sg * (1.f - sg));
     }
     if (OP == FLHIP_ACT_SCALE) return a * dy;
+    if (OP == FLHIP_ACT_LEAKY) return x > a * x ? dy : a * dy;                        // fl::max's mask, Functions.cpp:320-324
+    if (OP == FLHIP_ACT_THRESHOLD) return x >= a ? dy : 0.f;
     const float sg = act_sigmoid(x);
     return dy * sg * (1.f - sg);                                                      // :492
   }
@@ -756,7 +760,7 @@ extern "C" int flhip_relu_bwd(const void* dy, const void* x, void* dx, size_t n,
 extern "C" int flhip_act_fwd(int op, const void* x, void* y, size_t n, double a, double b, int dtype, void* stream) {
   FLHIP_REQUIRE((x && y) || n == 0, "act_fwd: null argument");
   FLHIP_REQUIRE(dtype_ok(dtype), "act_fwd: unknown dtype");
-  FLHIP_REQUIRE(op >= FLHIP_ACT_ELU && op <= FLHIP_ACT_SCALE, "act_fwd: unknown activation");
+  FLHIP_REQUIRE(op >= FLHIP_ACT_ELU && op <= FLHIP_ACT_THRESHOLD, "act_fwd: unknown activation");
   FLHIP_REQUIRE(op != FLHIP_ACT_CLAMP || a <= b, "act_fwd: clamp needs lo <= hi");
   if (n == 0) return FLHIP_OK;
   const float fa = (float)a, fb = (float)b;
@@ -770,6 +774,8 @@ extern "C" int flhip_act_fwd(int op, const void* x, void* y, size_t n, double a,
       case FLHIP_ACT_LOG: go(OpAct<FLHIP_ACT_LOG>{fa, fb}); break;
       case FLHIP_ACT_SWISH: go(OpAct<FLHIP_ACT_SWISH>{fa, fb}); break;
       case FLHIP_ACT_SCALE: go(OpAct<FLHIP_ACT_SCALE>{fa, fb}); break;
+      case FLHIP_ACT_LEAKY: go(OpAct<FLHIP_ACT_LEAKY>{fa, fb}); break;
+      case FLHIP_ACT_THRESHOLD: go(OpAct<FLHIP_ACT_THRESHOLD>{fa, fb}); break;
       default: go(OpAct<FLHIP_ACT_SIGMOID>{fa, fb}); break;
     }
   });
@@ -780,7 +786,7 @@ extern "C" int flhip_act_bwd(int op, const void* dy, const void* x, void* dx, si
                              void* stream) {
   FLHIP_REQUIRE((dy && x && dx) || n == 0, "act_bwd: null argument");
   FLHIP_REQUIRE(dtype_ok(dtype), "act_bwd: unknown dtype");
-  FLHIP_REQUIRE(op >= FLHIP_ACT_ELU && op <= FLHIP_ACT_SCALE, "act_bwd: unknown activation");
+  FLHIP_REQUIRE(op >= FLHIP_ACT_ELU && op <= FLHIP_ACT_THRESHOLD, "act_bwd: unknown activation");
   if (n == 0) return FLHIP_OK;
   const float fa = (float)a, fb = (float)b;
   by_dtype(dtype, [&](auto* t_) {
@@ -793,6 +799,8 @@ extern "C" int flhip_act_bwd(int op, const void* dy, const void* x, void* dx, si
       case FLHIP_ACT_LOG: go(OpActBwd<FLHIP_ACT_LOG>{fa, fb}); break;
       case FLHIP_ACT_SWISH: go(OpActBwd<FLHIP_ACT_SWISH>{fa, fb}); break;
       case FLHIP_ACT_SCALE: go(OpActBwd<FLHIP_ACT_SCALE>{fa, fb}); break;
+      case FLHIP_ACT_LEAKY: go(OpActBwd<FLHIP_ACT_LEAKY>{fa, fb}); break;
+      case FLHIP_ACT_THRESHOLD: go(OpActBwd<FLHIP_ACT_THRESHOLD>{fa, fb}); break;
       default: go(OpActBwd<FLHIP_ACT_SIGMOID>{fa, fb}); break;
     }
   });

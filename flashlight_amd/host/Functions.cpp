@@ -519,6 +519,10 @@ Variable log(const Variable& input) { return activation("log", FLHIP_ACT_LOG, in
 Variable sigmoid(const Variable& input) { return activation("sigmoid", FLHIP_ACT_SIGMOID, input, 0.0, 0.0); }
 Variable swish(const Variable& input, double beta) { return activation("swish", FLHIP_ACT_SWISH, input, beta, 0.0); }
 Variable scale(const Variable& input, double factor) { return activation("scale", FLHIP_ACT_SCALE, input, factor, 0.0); }
+Variable leakyRelu(const Variable& input, double slope) { return activation("leakyRelu", FLHIP_ACT_LEAKY, input, slope, 0.0); }
+Variable thresholdRelu(const Variable& input, double threshold) {
+  return activation("thresholdRelu", FLHIP_ACT_THRESHOLD, input, threshold, 0.0);
+}
 
 Variable gatedlinearunit(const Variable& input, int dim) {
   // Functions.cpp:1567-1579

@@ -151,6 +151,10 @@ Variable tanh(const Variable& input);
 Variable log(const Variable& input);
 Variable sigmoid(const Variable& input);
 Variable swish(const Variable& input, double beta);
+// LeakyReLU's max(input, slope * input) and ThresholdReLU's input * (input >= threshold) as one operator each
+// (nn/modules/Activations.cpp:102-104, 151-154; the first with fl::max's gradient mask, Functions.cpp:315-327)
+Variable leakyRelu(const Variable& input, double slope);
+Variable thresholdRelu(const Variable& input, double threshold);
 // a Variable times a number (the reference's operator*(Variable, double))
 Variable scale(const Variable& input, double factor);
 inline Variable operator*(const Variable& lhs, double rhs) { return scale(lhs, rhs); }

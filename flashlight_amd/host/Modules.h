@@ -327,6 +327,32 @@ class Sigmoid : public UnaryModule {       // :18-20
   Variable forward(const Variable& input) override { return sigmoid(input); }
   std::string prettyString() const override { return "Sigmoid"; }
 };
+class LeakyReLU : public UnaryModule {     // :100-112
+ public:
+  explicit LeakyReLU(double slope = 0.0) : slope_(slope) {}
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return leakyRelu(input, slope_); }
+  std::string prettyString() const override { return "LeakyReLU (" + std::to_string(slope_) + ")"; }
+
+ private:
+  double slope_;
+};
+class ThresholdReLU : public UnaryModule { // :149-163
+ public:
+  explicit ThresholdReLU(double threshold = 1.0) : threshold_(threshold) {}
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return thresholdRelu(input, threshold_); }
+  std::string prettyString() const override { return "ThresholdReLU (" + std::to_string(threshold_) + ")"; }
+
+ private:
+  double threshold_;
+};
+// nn/modules/Identity.cpp:12-22: the inputs as they are
+class Identity : public Module {
+ public:
+  std::vector<Variable> forward(const std::vector<Variable>& inputs) override { return inputs; }
+  std::string prettyString() const override { return "Identity"; }
+};
 class Swish : public UnaryModule {         // :190-196
  public:
   explicit Swish(double beta = 1.0) : beta_(beta) {}

@@ -424,7 +424,7 @@ def relu_backward(grad_output, input):
     return dx
 
 
-ACT_ELU, ACT_CLAMP, ACT_TANH, ACT_LOG, ACT_SWISH, ACT_SIGMOID, ACT_SCALE = range(7)
+ACT_ELU, ACT_CLAMP, ACT_TANH, ACT_LOG, ACT_SWISH, ACT_SIGMOID, ACT_SCALE, ACT_LEAKY, ACT_THRESHOLD = range(9)
 
 
 def activation(op, input, a=0.0, b=0.0):

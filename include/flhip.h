@@ -116,7 +116,7 @@ const char* flhip_last_error(void);
  * refuse to run when flhip_version() / 100 differs from FLHIP_VERSION / 100 (a layout change).
  * 200: flhip_rnn_desc gained dropout, seed_lo, seed_hi; flhip_bn_workspace_bytes never returns less
  * than 32 bytes per feature.  202: the *_plan entry points and FLHIP_DECLINED.  203: FLHIP_F16.  204: flhip_act_fwd / _bwd, flhip_glu_fwd / _bwd,
- * flhip_dropout, flhip_rownorm, flhip_weightnorm_fwd / _bwd, flhip_pad_fwd / _bwd, flhip_sgd_many, flhip_adam_many.  205: flhip_prelu_fwd / _bwd. */
+ * flhip_dropout, flhip_rownorm, flhip_weightnorm_fwd / _bwd, flhip_pad_fwd / _bwd, flhip_sgd_many, flhip_adam_many.  205: flhip_prelu_fwd / _bwd, FLHIP_ACT_LEAKY, FLHIP_ACT_THRESHOLD. */
 #define FLHIP_VERSION 205
 int flhip_version(void);
 const char* flhip_arch(void);
@@ -380,6 +380,9 @@ int flhip_relu_bwd(const void* dy, const void* x, void* dx, size_t n, int dtype,
  *   FLHIP_ACT_TANH     fl::tanh (Functions.cpp:454-463)      FLHIP_ACT_LOG      fl::log (:403-411)
  *   FLHIP_ACT_SWISH    a = beta: x * sigmoid(a x) (:498-500)  FLHIP_ACT_SIGMOID  fl::sigmoid (:488-496)
  *   FLHIP_ACT_SCALE    a x: a Variable times a number (the scales of fl::Residual, contrib/modules/Residual.cpp:69-73)
+ *   FLHIP_ACT_LEAKY    a = slope: max(x, a x) (LeakyReLU, Activations.cpp:102-104); the gradient is fl::max's
+ *                      (Functions.cpp:315-327): dy where x > a x, a dy elsewhere
+ *   FLHIP_ACT_THRESHOLD  a = threshold: x where x >= a, else 0 (ThresholdReLU, Activations.cpp:151-154)
  * flhip_act_bwd: dx = dy * f'(x) from the gradient and the forward INPUT (clamp passes the gradient where
  * lo < x < hi, strictly, as the reference's mask on its result does).  y / dx may alias x / dy. */
 #define FLHIP_ACT_ELU 0
@@ -389,6 +392,8 @@ int flhip_relu_bwd(const void* dy, const void* x, void* dx, size_t n, int dtype,
 #define FLHIP_ACT_SWISH 4
 #define FLHIP_ACT_SIGMOID 5
 #define FLHIP_ACT_SCALE 6
+#define FLHIP_ACT_LEAKY 7
+#define FLHIP_ACT_THRESHOLD 8
 int flhip_act_fwd(int op, const void* x, void* y, size_t n, double a, double b, int dtype, void* stream);
 int flhip_act_bwd(int op, const void* dy, const void* x, void* dx, size_t n, double a, double b, int dtype,
                   void* stream);

@@ -403,7 +403,8 @@ void flref_relu_bwd(int64_t n, const float* dy, const float* x, float* dx) {
 
 /* The element-wise activations of nn/modules/Activations.cpp, in double, rounded once.  op as FLHIP_ACT_*:
  * 0 ELU (a = alpha; :136-139 there), 1 clamp(a, b) (Functions.cpp:465-475), 2 tanh (:454-463), 3 log (:403-411),
- * 4 swish (a = beta; :498-500), 5 sigmoid (:488-496), 6 a x. */
+ * 4 swish (a = beta; :498-500), 5 sigmoid (:488-496), 6 a x, 7 LeakyReLU max(x, a x) (:102-104 there, with
+ * fl::max's gradient mask x > a x, Functions.cpp:315-327), 8 ThresholdReLU x * (x >= a) (:151-154). */
 static double act_sigmoid(double v) { return 1.0 / (1.0 + exp(-v)); }
 void flref_act_fwd(int op, int64_t n, const float* x, double a, double b, float* y) {
   for (int64_t i = 0; i < n; ++i) {
@@ -416,6 +417,8 @@ void flref_act_fwd(int op, int64_t n, const float* x, double a, double b, float*
       case 3: r = log(v); break;
       case 4: r = v * act_sigmoid(a * v); break;
       case 6: r = a * v; break;
+      case 7: r = v > a * v ? v : a * v; break;
+      case 8: r = v >= a ? v : 0.0; break;
       default: r = act_sigmoid(v); break;
     }
     y[i] = (float)r;
@@ -433,6 +436,8 @@ void flref_act_bwd(int op, int64_t n, const float* dy, const float* x, double a,
       case 3: r = g / v; break;
       case 4: { const double sg = act_sigmoid(a * v); r = g * (sg + v * a * sg * (1.0 - sg)); break; }
       case 6: r = a * g; break;
+      case 7: r = v > a * v ? g : a * g; break;
+      case 8: r = v >= a ? g : 0.0; break;
       default: { const double sg = act_sigmoid(v); r = g * sg * (1.0 - sg); break; }
     }
     dx[i] = (float)r;

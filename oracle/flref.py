@@ -191,7 +191,7 @@ def relu_fwd(x):
     return y
 
 
-ACT_ELU, ACT_CLAMP, ACT_TANH, ACT_LOG, ACT_SWISH, ACT_SIGMOID, ACT_SCALE = range(7)
+ACT_ELU, ACT_CLAMP, ACT_TANH, ACT_LOG, ACT_SWISH, ACT_SIGMOID, ACT_SCALE, ACT_LEAKY, ACT_THRESHOLD = range(9)
 
 
 def act_fwd(op, x, a=0.0, b=0.0):

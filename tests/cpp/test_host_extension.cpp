@@ -1026,6 +1026,29 @@ static void testActivationModules() {
       CHECK(relL2(hostOf(in.grad()), dxr) <= tol);
     }
   }
+  // LeakyReLU, ThresholdReLU (no architecture line in the reference's builder), Identity
+  for (dtype dt : {dtype::f32, dtype::f16}) {
+    const double tol = dt == dtype::f32 ? 2e-6 : 4e-3;
+    struct MCase { std::shared_ptr<Module> m; int op; double a; const char* pretty; };
+    const MCase mc[] = {{std::make_shared<LeakyReLU>(0.1), 7, 0.1, "LeakyReLU (0.100000)"},
+                        {std::make_shared<ThresholdReLU>(0.5), 8, 0.5, "ThresholdReLU (0.500000)"}};
+    for (const MCase& c : mc) {
+      auto x = randn(n, 740 + c.op, 2.f), dy = randn(n, 741);
+      for (auto& v : x) v = roundTo(dt, v);
+      for (auto& v : dy) v = roundTo(dt, v);
+      Variable in(Tensor::fromVector(shp, x).astype(dt), true);
+      Variable y = c.m->forward({in})[0];
+      y.backward(Variable(Tensor::fromVector(shp, dy).astype(dt), false));
+      std::vector<float> yr(n), dxr(n);
+      flref_act_fwd(c.op, (int64_t)n, x.data(), c.a, 0.0, yr.data());
+      flref_act_bwd(c.op, (int64_t)n, dy.data(), x.data(), c.a, 0.0, dxr.data());
+      CHECK(c.m->prettyString() == c.pretty);
+      CHECK(relL2(hostOf(y), yr) <= tol && relL2(hostOf(in.grad()), dxr) <= tol);
+    }
+    Variable idIn(Tensor::fromVector(shp, randn(n, 742)).astype(dt), false);
+    auto idOut = Identity().forward({idIn, idIn});
+    CHECK(idOut.size() == 2 && idOut[0].tensor().device() == idIn.tensor().device() && Identity().prettyString() == "Identity");
+  }
   // PReLU (lines PR, PR n, PR n value): one parameter, or one per index of dimension 0; the parameter's gradient
   for (dtype dt : {dtype::f32, dtype::bf16}) {
     const double tol = dt == dtype::f32 ? 2e-6 : 4e-3;

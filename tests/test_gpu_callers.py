@@ -351,7 +351,8 @@ def test_astype_with_f16(src, dst):
 # ---- activations, gated linear unit, dropout (nn/modules/Activations.cpp, Functions.cpp:1567-1610, 1777-1785) ----
 _ACTS = [(ops.ACT_ELU, 1.0, 0.0), (ops.ACT_ELU, 0.3, 0.0), (ops.ACT_CLAMP, 0.0, 6.0), (ops.ACT_CLAMP, -1.0, 1.0),
          (ops.ACT_TANH, 0.0, 0.0), (ops.ACT_LOG, 0.0, 0.0), (ops.ACT_SWISH, 1.0, 0.0), (ops.ACT_SWISH, 1.7, 0.0),
-         (ops.ACT_SIGMOID, 0.0, 0.0), (ops.ACT_SCALE, -0.37, 0.0)]
+         (ops.ACT_SIGMOID, 0.0, 0.0), (ops.ACT_SCALE, -0.37, 0.0), (ops.ACT_LEAKY, 0.01, 0.0), (ops.ACT_LEAKY, 1.5, 0.0),
+         (ops.ACT_THRESHOLD, 0.7, 0.0)]
 
 
 @pytest.mark.parametrize("dtype", DT)

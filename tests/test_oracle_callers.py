@@ -198,6 +198,10 @@ _ACTS = [
     (flref.ACT_SWISH, 1.7, 0.0, lambda t: t * torch.sigmoid(1.7 * t)),
     (flref.ACT_SIGMOID, 0.0, 0.0, torch.sigmoid),
     (flref.ACT_SCALE, -0.37, 0.0, lambda t: -0.37 * t),
+    (flref.ACT_LEAKY, 0.01, 0.0, lambda t: F.leaky_relu(t, 0.01)),
+    (flref.ACT_LEAKY, 0.3, 0.0, lambda t: torch.maximum(t, 0.3 * t)),
+    (flref.ACT_LEAKY, 1.5, 0.0, lambda t: torch.where(t > 1.5 * t, t, 1.5 * t)),       # a slope above 1: still max(x, a x)
+    (flref.ACT_THRESHOLD, 0.7, 0.0, lambda t: F.threshold(t, 0.7, 0.0) + 0.0 * t),
 ]
 
 
