@@ -98,6 +98,8 @@ int mfma_first16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* 
 // backward-data of a stride-2 window over at most 4 input channels (the stem), any storage type, as a 4 x 4
 // stride-1 window over the output gradient onto the 2 x 2 cells of the input gradient (conv2d_mfma_cells.hip)
 int mfma_cells_conv_bwd_data(const ConvGeom& g, int dtype, const void* dy, const void* w, void* dx, hipStream_t s);
+// the forward pass of the same layers on the same cells (the window spans at most 4 x 4 cells of the input)
+int mfma_cells_conv_fwd(const ConvGeom& g, int dtype, const void* x, const void* w, const float* bias, void* y, hipStream_t s);
 // bf16 3x3 stride-1 pad-1 over 64 source channels, whole contraction per workgroup (conv2d_mfma_strip_bf16.hip)
 // bf16 1x1 stride-1 convolutions with operand tiles copied to LDS by the loads themselves
 // (conv2d_mfma_pointwise_dma_bf16.hip); -1 when the shape is not theirs.  addend (or null): added

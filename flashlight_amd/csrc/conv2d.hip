@@ -255,6 +255,7 @@ extern "C" int flhip_conv2d_fwd(const flhip_conv_desc* d, const void* x, const v
       r = mfma_pointwise16_conv_fwd(g, x, w, bias, y, s, ws, ws_bytes, d->dtype);
     if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !skip(Options::SKIP_FIRST) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_first16_conv_fwd(g, x, w, bias, y, s, d->dtype);
+    if (r < 0 && !skip(Options::SKIP_CELLS)) r = mfma_cells_conv_fwd(g, d->dtype, x, w, bias, y, s);
     if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !skip(Options::SKIP_STRIP) && !algo_is(Options::ALGO_CONVERT))
       r = mfma_strip16_conv_fwd(g, x, w, bias, y, s, d->dtype);
     if (r < 0 && is_lo16(d->dtype) && !skip(SK_BF16) && !algo_is(Options::ALGO_CONVERT))

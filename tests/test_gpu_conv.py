@@ -955,7 +955,7 @@ CELL_CASES = [
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("case", CELL_CASES)
-def test_backward_data_of_stride_two_windows_over_few_channels(case, dtype):
+def test_stride_two_windows_over_few_channels(case, dtype):
     xs, ws, pd = case
     rng = np.random.default_rng(83)
     w = round_to((rng.standard_normal(ws) / np.sqrt(ws[1] * ws[2] * ws[3])).astype(np.float32), dtype)
@@ -987,6 +987,37 @@ def test_backward_data_of_stride_two_windows_over_few_channels(case, dtype):
             if 0 <= ih < xs[2] and 0 <= iw < xs[3]:
                 exp[0, :, ih, iw] = w[k, :, r, s]
     assert np.array_equal(got1, exp)
+    # the forward pass of the same layers on the same cells (16-bit storage: with the first-layer family, which takes
+    # some of these shapes ahead of it, switched off as well as on), against the checker and the kernels it replaced
+    x = round_to(rng.standard_normal(xs).astype(np.float32), dtype)
+    b = rng.uniform(-1, 1, ws[0]).astype(np.float32)
+    y_ref = flref.conv2d_fwd(d, x, w, b)
+    outs = [fa.conv2d(dev(x, dtype), dev(w, dtype), dev(b), **kw)]
+    for skip_ in ("first", "cells,first"):
+        capi.set_option("CONV_SKIP", skip_)
+        try:
+            outs.append(fa.conv2d(dev(x, dtype), dev(w, dtype), dev(b), **kw))
+        finally:
+            capi.set_option("CONV_SKIP", None)
+    torch.cuda.synchronize()
+    for o in outs:
+        assert o.shape == y_ref.shape and rel_l2(host(o), y_ref) <= tol, rel_l2(host(o), y_ref)
+    # an input of one unit value puts the (flipped) filter taps into the result: exact
+    x1 = np.zeros(xs, np.float32)
+    c1, ih1, iw1 = xs[1] - 1, xs[2] // 2, xs[3] // 2
+    x1[0, c1, ih1, iw1] = 1.0
+    capi.set_option("CONV_SKIP", "first")
+    try:
+        y1 = host(fa.conv2d(dev(x1, dtype), dev(w, dtype), None, **kw))
+    finally:
+        capi.set_option("CONV_SKIP", None)
+    exp1 = np.zeros(y_ref.shape, np.float32)
+    for r in range(ws[2]):
+        for s in range(ws[3]):
+            th, tw = ih1 + pd[0] - r, iw1 + pd[1] - s
+            if th % 2 == 0 and tw % 2 == 0 and 0 <= th // 2 < ys[2] and 0 <= tw // 2 < ys[3]:
+                exp1[0, :, th // 2, tw // 2] = w[:, c1, r, s]
+    assert np.array_equal(y1, exp1)
 
 
 # The backward passes with the kernel family named by the caller (flhip_conv2d_bwd_*_plan): every family either
