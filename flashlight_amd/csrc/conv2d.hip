@@ -231,7 +231,9 @@ extern "C" size_t flhip_conv2d_workspace_bytes(const flhip_conv_desc* d, int pas
     const size_t b = is_lo16(d->dtype) ? mfma_pointwise16_lattice_ws(g, pass == FLHIP_CONV_BWD_DATA)
                                             : pass == FLHIP_CONV_BWD_DATA ? mfma_pointwise_split_ws(g, d->dtype, true) : 0;
     const size_t c = mfma_tap1d_conv_ws(g, d->dtype, pass == FLHIP_CONV_BWD_DATA);
-    const size_t c2 = tap2d_on(g, d->dtype) ? mfma_tap2d_conv_ws(g, d->dtype, pass == FLHIP_CONV_BWD_DATA) : 0;
+    // (the stacked-plane kernels: where their rule takes the geometry, and for every plane of at most 32 x 32 positions so
+    // that a caller can try them by plan number; beyond that their copy of the input is tens of megabytes nobody asked for)
+    const size_t c2 = (tap2d_on(g, d->dtype) || g.H * g.W <= 1024) ? mfma_tap2d_conv_ws(g, d->dtype, pass == FLHIP_CONV_BWD_DATA) : 0;
     return std::max(std::max(a, c2), std::max(b, c));
   }
   return 0;

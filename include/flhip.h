@@ -222,7 +222,8 @@ int flhip_conv2d_bwd_filter_static(const flhip_conv_desc* d, const void* x,
  * points are flhip_conv2d_bwd_data / flhip_conv2d_bwd_filter with one more argument: plan < 0 runs the default
  * rule (identical to the entry points above), plan >= 0 runs that family alone, whatever the rules and
  * switches say, or returns FLHIP_DECLINED without launching anything when the family does not take the
- * geometry or storage type.  Workspace as for the entry points above (their size covers every plan).  Every
+ * geometry or storage type, or when the workspace is too small for it.  Workspace as for the entry points above (their
+ * size covers every plan; the stacked-plane plan of backward-data on planes of at most 32 x 32 positions).  Every
  * plan meets the stated tolerances; results of different plans differ in summation order only. */
 int flhip_conv2d_plan_count(int pass);
 const char* flhip_conv2d_plan_name(int pass, int plan);
