@@ -662,7 +662,7 @@ def _random_cases(n, seed):
 
 @pytest.mark.parametrize("case", _random_cases(40, 20251125))
 def test_random_geometries(case):
-    for dtype, tol, tight_w in ((torch.float32, F32_TOL, 1e-4), (torch.bfloat16, BF16_TOL, 1e-4)):
+    for dtype, tol, tight_w in ((torch.float32, F32_TOL, 1e-4), (torch.bfloat16, BF16_TOL, 1e-4), (torch.float16, BF16_TOL, 1e-4)):
         for name, (got, ref) in _run(case, 3, dtype).items():
             lim = tol if dtype == torch.float32 else (tight_w if name in ("dw", "db") else 4e-3)
             assert rel_l2(got, ref) <= lim, (case, dtype, name, rel_l2(got, ref))
