@@ -944,7 +944,12 @@ extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, in
     }
   }
   // the matrix-core kernels of the 1x1 convolutions take the three products fl::linear
-  // needs; the tiled vector-ALU kernel below covers the rest
+  // needs; the tiled vector-ALU kernel below covers the rest.  16-bit storage: on the 16-bit
+  // matrix instructions where the shape allows (MATMUL_FP32_CORES keeps them on the fp32 ones).
+  if (is_lo16(dtype) && !(trans_a && trans_b) && !options().matmul_valu && !options().matmul_fp32_cores) {
+    const int rc = mfma_gemm16(dtype, trans_a ? 1 : trans_b ? 2 : 0, A, B, C, M, N, K, bias_rows, as_stream(stream));
+    if (rc >= 0) return rc;
+  }
   if (!trans_a && trans_b && !bias_rows && !options().matmul_valu) {
     const int rc = gemm_nt(dtype, A, B, C, M, N, K, 1, as_stream(stream));
     if (rc >= 0) return rc;

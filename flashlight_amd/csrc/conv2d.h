@@ -65,6 +65,9 @@ int mfma_pointwise_conv_split(const ConvGeom& g, int dtype, bool bwd, const void
 int mfma_gemm(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,
               const float* bias_rows, hipStream_t s, int ksplit = 1);
 int mfma_gemm_slices(int K, int ksplit);
+// the same three products in 16-bit storage on the 16-bit matrix instructions (conv2d_mfma_pointwise_dma_bf16.hip)
+int mfma_gemm16(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,
+                const float* bias_rows, hipStream_t s);
 // column-major C = A * B^T on a kernel of its own (both operands contiguous along the
 // surviving dimension); slices > 1 (f32): partial products M * N floats apart
 int gemm_nt(int dtype, const void* A, const void* B, void* C, int M, int N, int K, int slices, hipStream_t s);

@@ -67,6 +67,7 @@ struct PwdParams {
   int ncells;           // cells over the batch
   int nstages, mtiles, ctiles;
   unsigned src_bytes, w_bytes, dst_bytes;
+  const float* pos_bias;   // one value per position, added to every result channel (matrix products: one image), or null
 };
 
 // rows r0 .. r0+7 of column c0 + s of a 16-bit tile stored [row][column] (see the 1x1 kernels
@@ -130,7 +131,7 @@ pwd16_conv_kernel(PwdParams p, const E* __restrict__ src, const E* __restrict__ 
 
   // ---- load roles: instruction ii = wave + 4 n of a stage; lane -> LDS cell ii * 64 + lane.
   // Per instruction, the same for all lanes: descriptor, LDS offset, bytes to advance per stage.
-  int voff[5];
+  int voff[5], klim[5];      // klim: contraction channels from the lane's cell to the end of its row (forward weights)
   intx4_t lrs[5];
   int loff[5], lstep[5];
 #pragma unroll
@@ -141,6 +142,7 @@ pwd16_conv_kernel(PwdParams p, const E* __restrict__ src, const E* __restrict__ 
     loff[n] = (isx ? ii * 64 : PD_XCELLS + (ii - NXI) * 64) * 16;
     lstep[n] = isx ? PD_KC * 2 * p.P : BWD ? PD_KC * 2 * p.Mo : PD_KC * 2;
     voff[n] = (int)0x80000000;      // past every tensor: such a lane fetches nothing and its cell gets zeros
+    klim[n] = 0x7fffffff;
     if (ii < NXI) {
       const int L = ii * 64 + lane, row = L / PD_XC, c = L - row * PD_XC;
       const int cell = cell0 + c;
@@ -156,6 +158,7 @@ pwd16_conv_kernel(PwdParams p, const E* __restrict__ src, const E* __restrict__ 
       } else {
         const int m = L / PD_WC, c = L - m * PD_WC;
         if (c < 4 && m0 + m < p.Mo) voff[n] = ((m0 + m) * p.Kc + 8 * c) * 2;
+        klim[n] = p.Kc - 8 * c;     // a last stage of fewer than 32 channels: the cells past the row's end fetch nothing
       }
     }
   }
@@ -167,9 +170,10 @@ pwd16_conv_kernel(PwdParams p, const E* __restrict__ src, const E* __restrict__ 
     const unsigned base = (unsigned)reinterpret_cast<uintptr_t>((lds_void_t)ring);
     const bool live = t < n;
 #pragma unroll
-    for (int k = 0; k < 3; ++k) pd_load_lds(lrs[k], base + loff[k], live ? voff[k] : (int)0x80000000, t * lstep[k]);
-    if (fourth) pd_load_lds(lrs[3], base + loff[3], live ? voff[3] : (int)0x80000000, t * lstep[3]);
-    if (fifth) pd_load_lds(lrs[4], base + loff[4], live ? voff[4] : (int)0x80000000, t * lstep[4]);
+    for (int k = 0; k < 3; ++k)
+      pd_load_lds(lrs[k], base + loff[k], (live && t * PD_KC < klim[k]) ? voff[k] : (int)0x80000000, t * lstep[k]);
+    if (fourth) pd_load_lds(lrs[3], base + loff[3], (live && t * PD_KC < klim[3]) ? voff[3] : (int)0x80000000, t * lstep[3]);
+    if (fifth) pd_load_lds(lrs[4], base + loff[4], (live && t * PD_KC < klim[4]) ? voff[4] : (int)0x80000000, t * lstep[4]);
   };
 
   // ---- fragments: 128 result channels: wave = (position half, channel half), 2 x 2 blocks of 32 x 32;
@@ -255,6 +259,14 @@ pwd16_conv_kernel(PwdParams p, const E* __restrict__ src, const E* __restrict__ 
     for (int i = 0; i < NA; ++i)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
+        if (p.pos_bias) {      // one image: slot 8 c + e of the tile is position min(8 (cell0 + c), P - 8) + e
+          const int cell = cell0 + (pos0 + i * 32) / 8 + g;
+          if (cell < p.ncells) {
+            const float* pb = p.pos_bias + min(8 * cell, p.P - 8) + fh * 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][4 * g + e] += pb[e];
+          }
+        }
         const uintx2_t o = {Lo16<E>::pack(acc[i][j][4 * g] + bv, acc[i][j][4 * g + 1] + bv),
                             Lo16<E>::pack(acc[i][j][4 * g + 2] + bv, acc[i][j][4 * g + 3] + bv)};
         *reinterpret_cast<uintx2_t*>(&ys[ml * PD_YP + pos0 + i * 32 + g * 8 + fh * 4]) = o;
@@ -295,26 +307,10 @@ bool pwd16_applies(const ConvGeom& g, bool bwd) {
   return options().pw16_pf != 0 || (g.H * g.W <= 1024 && mo > 64);
 }
 
+// grid and kernel variant for a filled-in PwdParams (Kc, Mo, P, Pc, ncells, nstages, ctiles and the byte sizes)
 template <typename E, bool BWD>
-int launch_pwd16(const ConvGeom& g, const void* src, const void* w, const float* bias, void* dst, const void* addend,
-                 hipStream_t s) {
-  if (!pwd16_applies(g, BWD)) return -1;
-  PwdParams p{};
-  p.Kc = BWD ? g.K : g.C;
-  p.Mo = BWD ? g.C : g.K;
-  p.P = g.H * g.W;
-  p.Pc = (p.P + 7) / 8;
-  const long long sb = (long long)g.N * p.Kc * p.P * 2, db = (long long)g.N * p.Mo * p.P * 2;
-  const long long wb = (long long)p.Kc * p.Mo * 2;
-  // 32-bit byte offsets, with room for the rows of a last tile that lie past the tensor
-  if (std::max(sb, db) + (long long)(PD_BM + PD_KC) * p.P * 2 >= (1ll << 31) || wb + PD_BM * p.Kc * 2ll >= (1ll << 31))
-    return -1;
-  p.src_bytes = (unsigned)sb;
-  p.dst_bytes = (unsigned)db;
-  p.w_bytes = (unsigned)wb;
-  p.ncells = g.N * p.Pc;
-  p.nstages = p.Kc / PD_KC;
-  p.ctiles = (p.ncells + PD_CELLS - 1) / PD_CELLS;
+int pwd16_go(PwdParams p, const void* src, const void* w, const float* bias, void* dst, const void* addend,
+             hipStream_t s, const char* what) {
   // tiles of 64 result channels when tiles of 128 would leave half of the CUs without a workgroup (7x7 planes
   // with 512 result channels at batch 64: 112 workgroups of 64 stages); the deep ring for grids of at most one
   // workgroup per CU.  FLHIP_PW16_PF = 1 / 4 forces the shallow / deep ring with tiles of 128, 2 / 8 with tiles of 64.
@@ -338,7 +334,36 @@ int launch_pwd16(const ConvGeom& g, const void* src, const void* w, const float*
     if (deep) go(pwd16_conv_kernel<E, BWD, 8, 128>);
     else go(pwd16_conv_kernel<E, BWD, 4, 128>);
   }
-  return check_launch(BWD ? "conv2d_bwd_data 1x1 (bf16 mfma, direct-to-LDS)" : "conv2d_fwd 1x1 (bf16 mfma, direct-to-LDS)");
+  return check_launch(what);
+}
+
+// byte sizes as 32-bit offsets, with room for the rows of a last tile that lie past the tensor
+bool pwd16_sizes(PwdParams* p, long long images) {
+  const long long sb = images * p->Kc * p->P * 2, db = images * p->Mo * p->P * 2;
+  const long long wb = (long long)p->Kc * p->Mo * 2;
+  if (std::max(sb, db) + (long long)(PD_BM + PD_KC) * p->P * 2 >= (1ll << 31) || wb + PD_BM * p->Kc * 2ll >= (1ll << 31))
+    return false;
+  p->src_bytes = (unsigned)sb;
+  p->dst_bytes = (unsigned)db;
+  p->w_bytes = (unsigned)wb;
+  p->Pc = (p->P + 7) / 8;
+  p->ncells = (int)(images * p->Pc);
+  p->nstages = (p->Kc + PD_KC - 1) / PD_KC;
+  p->ctiles = (p->ncells + PD_CELLS - 1) / PD_CELLS;
+  return images * p->Pc <= 0x7fffffffll;
+}
+
+template <typename E, bool BWD>
+int launch_pwd16(const ConvGeom& g, const void* src, const void* w, const float* bias, void* dst, const void* addend,
+                 hipStream_t s) {
+  if (!pwd16_applies(g, BWD)) return -1;
+  PwdParams p{};
+  p.Kc = BWD ? g.K : g.C;
+  p.Mo = BWD ? g.C : g.K;
+  p.P = g.H * g.W;
+  if (!pwd16_sizes(&p, g.N)) return -1;
+  return pwd16_go<E, BWD>(p, src, w, bias, dst, addend, s,
+                          BWD ? "conv2d_bwd_data 1x1 (bf16 mfma, direct-to-LDS)" : "conv2d_fwd 1x1 (bf16 mfma, direct-to-LDS)");
 }
 
 
@@ -373,9 +398,11 @@ struct PwdWgradParams {
   unsigned x_bytes, dy_bytes;
 };
 
-template <typename E>
+// DIRECT (matrix products: one slice): the tile leaves in the element type, at out16, with bias[column] added
+template <typename E, bool DIRECT>
 __global__ void __launch_bounds__(256, 1)
-pwd16_wgrad_kernel(PwdWgradParams p, const E* __restrict__ x, const E* __restrict__ dy, float* __restrict__ out) {
+pwd16_wgrad_kernel(PwdWgradParams p, const E* __restrict__ x, const E* __restrict__ dy, float* __restrict__ out,
+                   uint16_t* __restrict__ out16, const float* __restrict__ bias) {
   __shared__ __align__(16) uint4 ring[PWG_NS * PWG_STAGE];
   const int slice = blockIdx.x, mtile = blockIdx.y / p.ctiles, ctile = blockIdx.y - mtile * p.ctiles;
   const int m0 = mtile * PWG_T, c0 = ctile * PWG_T;
@@ -522,10 +549,13 @@ pwd16_wgrad_kernel(PwdWgradParams p, const E* __restrict__ x, const E* __restric
     for (int jj = 0; jj < 2; ++jj) {
       const int c = c0 + wn * 64 + jj * 32 + fr;
       if (c >= p.C) continue;
+      const float bv = (DIRECT && bias) ? bias[c] : 0.f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = m0 + wm * 64 + i * 32 + (r >> 2) * 8 + fh * 4 + (r & 3);
-        if (m < p.Mo) o[(size_t)m * p.C + c] = acc[i][jj][r];
+        if (m >= p.Mo) continue;
+        if (DIRECT) out16[(size_t)m * p.C + c] = Lo16<E>::narrow(acc[i][jj][r] + bv);
+        else o[(size_t)m * p.C + c] = acc[i][jj][r];
       }
     }
 }
@@ -600,11 +630,65 @@ int mfma_pwd16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw
   float* out = p.nsplit > 1 ? static_cast<float*>(ws) : dw;
   by_lo16(dtype, [&](auto* e_) {
     using E = FLHIP_T_OF(e_);
-    hipLaunchKernelGGL(pwd16_wgrad_kernel<E>, dim3((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles)), dim3(256), 0, s, p,
-                       static_cast<const E*>(x), static_cast<const E*>(dy), out);
+    hipLaunchKernelGGL((pwd16_wgrad_kernel<E, false>), dim3((unsigned)p.nsplit, (unsigned)(p.ctiles * p.mtiles)), dim3(256), 0,
+                       s, p, static_cast<const E*>(x), static_cast<const E*>(dy), out, (uint16_t*)nullptr, (const float*)nullptr);
   });
   if (p.nsplit > 1) wgrad_reduce_launch(static_cast<const float*>(ws), p.nsplit, p.E, p.Mo, 0, dw, nullptr, s);
   return check_launch("conv2d_bwd_filter 1x1 (bf16 mfma, direct-to-LDS)");
+}
+
+// Column-major matrix products in 16-bit storage on the kernels above (C is M x N, stored [n][m]):
+//   mode 0, C = A B    : A (M x K) is stored [k][m]: the source of a forward 1x1 layer over ONE image whose plane is the
+//                        M rows; B stored [n][k] are its weights; bias_rows (one per row of C) is a bias per position
+//   mode 1, C = A^T B  : A stored [m][k] and B stored [n][k] are both contiguous along the contraction: the filter
+//                        gradient's tile, written in the element type; bias_rows is a bias per column of that tile
+//   mode 2, C = A B^T  : A stored [k][m], B stored [k][n]: a backward-data 1x1 layer with B as the weights
+// One rounding per element, after the fp32 sum (and the bias).  -1 when the shape is not these kernels':
+// fewer than 8 rows (modes 0, 2) or a contraction shorter than 8 (mode 1), a contraction that is not a multiple
+// of 8 in mode 0 (a 16-byte cell of B would straddle two rows), a bias or an odd number of columns in mode 2 (the
+// range check of a buffer load works on 4-byte words: the word that holds the last element of B's last row would
+// lie half past the tensor and come back as zero), operands of 2 GiB.
+int mfma_gemm16(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,
+                const float* bias_rows, hipStream_t s) {
+  if (!is_lo16(dtype) || M <= 0 || N <= 0 || K <= 0) return -1;
+  if (mode == 1) {
+    if (K < 8) return -1;
+    PwdWgradParams p{};
+    p.C = M; p.Mo = N; p.P = K; p.N = 1;
+    p.Pc = (K + 7) / 8;
+    p.dup = (8 - K % 8) % 8;
+    const long long xb = (long long)M * K * 2, db = (long long)N * K * 2;
+    if (xb >= (1ll << 31) || db >= (1ll << 31)) return -1;
+    p.x_bytes = (unsigned)xb;
+    p.dy_bytes = (unsigned)db;
+    p.ncells = p.Pc;
+    p.nstages = (p.ncells + PWG_CH - 1) / PWG_CH;
+    p.ctiles = (M + PWG_T - 1) / PWG_T;
+    p.mtiles = (N + PWG_T - 1) / PWG_T;
+    p.E = 0;
+    p.sps = p.nstages;
+    p.nsplit = 1;
+    if ((long long)p.ctiles * p.mtiles > 65535) return -1;
+    by_lo16(dtype, [&](auto* e_) {
+      using E = FLHIP_T_OF(e_);
+      hipLaunchKernelGGL((pwd16_wgrad_kernel<E, true>), dim3(1u, (unsigned)(p.ctiles * p.mtiles)), dim3(256), 0, s, p,
+                         static_cast<const E*>(A), static_cast<const E*>(B), (float*)nullptr, static_cast<uint16_t*>(C),
+                         bias_rows);
+      return 0;
+    });
+    return check_launch("matmul (A^T * B, 16-bit mfma)");
+  }
+  if (mode != 0 && mode != 2) return -1;
+  if (M < 8 || (mode == 0 && K % 8 != 0) || (mode == 2 && (bias_rows || N % 2 != 0))) return -1;
+  PwdParams p{};
+  p.Kc = K; p.Mo = N; p.P = M;
+  if (!pwd16_sizes(&p, 1)) return -1;
+  p.pos_bias = bias_rows;
+  return by_lo16(dtype, [&](auto* e_) {
+    using E = FLHIP_T_OF(e_);
+    return mode == 0 ? pwd16_go<E, false>(p, A, B, nullptr, C, nullptr, s, "matmul (A * B, 16-bit mfma)")
+                     : pwd16_go<E, true>(p, A, B, nullptr, C, nullptr, s, "matmul (A * B^T, 16-bit mfma)");
+  });
 }
 
 }  // namespace flhip

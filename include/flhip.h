@@ -129,7 +129,7 @@ const char* flhip_arch(void);
  *   CONV_ALGO = direct | gather | tapped | convert | auto    CONV_SKIP = bf16,gemm1x1,slab,tapped,strip,first,wgrad128,pwdma,wd32,tap1d,cells,tap2d
  *   PW_PT = 2 | 4 | 8    PW16_PF = 0 | 1 | 2 | 4 | 8    CONV_STACK = 0 | 1 | 2 | 4 | 8    BN_ALGO = split | resident | auto
  *   SLAB_WAVES = 0 | 4 | 8
- *   PW16_NO_TAPS, TAPPED_NO_REORDER, MATMUL_VALU, RNN_UNFUSED, TAP2D_ALL = 1 | 0
+ *   PW16_NO_TAPS, TAPPED_NO_REORDER, MATMUL_VALU, MATMUL_FP32_CORES, RNN_UNFUSED, TAP2D_ALL = 1 | 0
  * Unknown names or values return FLHIP_INVALID_ARGUMENT.  The nearest thing in the
  * reference is the kernel-choice options object of its cuDNN extension
  * (createBenchmarkOptions, flashlight/fl/autograd/tensor/backend/cudnn/CudnnAutogradExtension.h:25). */
@@ -432,9 +432,10 @@ int flhip_pad_fwd(const void* x, void* y, const int64_t* dims, const int32_t* be
 int flhip_pad_bwd(const void* dy, void* dx, const int64_t* dims, const int32_t* before, const int32_t* after,
                   int dtype, void* stream);
 
-/* C (M x N) = op(A) (M x K) * op(B) (K x N), fp32 accumulate; trans_a: A is stored
- * K x M, trans_b: B is stored N x K.  bias_rows (fp32[M], may be NULL) is added to
- * every column.  Serves fl::linear (Functions.cpp:1255-1309): forward
+/* C (M x N) = op(A) (M x K) * op(B) (K x N), fp32 accumulate, one rounding to the element
+ * type; trans_a: A is stored K x M, trans_b: B is stored N x K.  bias_rows (fp32[M], may be
+ * NULL) is added to every column.  bf16 / f16 products of more than 128 columns run on the
+ * 16-bit matrix instructions (option MATMUL_FP32_CORES: on the fp32 ones).  Serves fl::linear (Functions.cpp:1255-1309): forward
  * matmul(weight, input) + tile(bias), backward matmulTN(weight, gradOutput) and
  * matmulNT(gradOutput, input). */
 int flhip_matmul(const void* A, const void* B, void* C, int32_t M, int32_t N,

@@ -76,6 +76,64 @@ def test_matmul_all_forms_through_the_c_abi(M, N, K, ta, tb, with_bias):
     assert rel_l2(host(Cd), want) <= 1e-5
 
 
+def _matmul_through_c_abi(A, B, M, N, K, ta, tb, bias, dtype):
+    import ctypes as C
+    from flashlight_amd import capi
+    Ad, Bd, Cd = dev(A, dtype), dev(B, dtype), torch.empty(N, M, device="cuda", dtype=dtype)
+    bd = dev(bias) if bias is not None else None
+    P = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None
+    S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    code = {torch.float32: capi.F32, torch.bfloat16: capi.BF16, torch.float16: capi.F16}[dtype]
+    rc = capi.lib().flhip_matmul(P(Ad), P(Bd), P(Cd), M, N, K, int(ta), int(tb), P(bd), code, S)
+    assert rc == 0
+    return host(Cd)
+
+
+# shapes around the edges of the 16-bit matrix-instruction kernels: rows that are no multiple of the 8-row cells
+# (and fewer than 8: another kernel's), columns that are no multiple of the 64/128-column tiles, contractions of
+# a partial last stage (40, 72, 200), of no whole cell (67, 1001: not for A B, which then takes another kernel)
+# and of many stages
+LO16_MATMUL = [(67, 130, 40), (8, 257, 72), (9, 129, 200), (135, 1000, 67), (300, 131, 1001), (5, 300, 64),
+               (128, 256, 32), (257, 513, 1000), (1000, 200, 8), (64, 2000, 96)]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K", LO16_MATMUL)
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True)])
+def test_matmul_in_16_bit_storage(M, N, K, ta, tb, dtype):
+    """The three products fl::linear needs, in 16-bit storage with more than 128 columns: they run on the
+    16-bit matrix instructions.  Every element is compared: one rounding of the exact sum, plus what an fp32
+    accumulation over K terms may add."""
+    rng = np.random.default_rng(M * 1000 + N * 10 + K + int(ta) + 2 * int(tb))
+    A = _round(rng.standard_normal((M, K) if ta else (K, M)).astype(np.float32), dtype)
+    B = _round(rng.standard_normal((K, N) if tb else (N, K)).astype(np.float32), dtype)
+    for bias in ([None] if tb else [None, rng.standard_normal(M).astype(np.float32)]):
+        want = flref.matmul(M, N, K, A, B, ta, tb, bias)
+        got = _matmul_through_c_abi(A, B, M, N, K, ta, tb, bias, dtype)
+        half_ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+        slack = 1.01 * half_ulp * np.abs(want) + 2e-6 * K + (0 if dtype == torch.bfloat16 else 6e-8)
+        bad = np.abs(got.astype(np.float64) - want) > slack
+        assert not bad.any(), (int(bad.sum()), np.argwhere(bad)[:4].tolist())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_matmul_in_16_bit_storage_at_the_size_of_a_speech_model(dtype):
+    """2000 x 2000 weights against 4000 frames, the three products of a layer's step; checked against numpy's
+    float64 product of the same rounded operands (the oracle's loops would take minutes here)."""
+    M, N, K = 2000, 4000, 2000
+    rng = np.random.default_rng(77)
+    half_ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    for ta, tb in [(False, False), (True, False), (False, True)]:
+        A = _round(rng.standard_normal((M, K) if ta else (K, M)).astype(np.float32), dtype)
+        B = _round(rng.standard_normal((K, N) if tb else (N, K)).astype(np.float32), dtype)
+        A64 = A.astype(np.float64) if ta else A.astype(np.float64).T            # M x K
+        B64 = B.astype(np.float64) if tb else B.astype(np.float64).T            # K x N
+        want = (A64 @ B64).T                                                     # stored [n][m]
+        got = _matmul_through_c_abi(A, B, M, N, K, ta, tb, None, dtype)
+        bad = np.abs(got.astype(np.float64) - want) > 1.01 * half_ulp * np.abs(want) + 2e-6 * K
+        assert not bad.any(), (ta, tb, int(bad.sum()), np.argwhere(bad)[:4].tolist())
+
+
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("classes,cols", [(10, 64), (1000, 7), (1, 5), (65, 3)])
 def test_logsoftmax(classes, cols, dtype):
