@@ -60,6 +60,9 @@ def parse():
     ap.add_argument("--repeats", type=int, default=5, help="timed repeats of --steps calls; the median is reported")
     ap.add_argument("--rnn", action="store_true",
                     help="instead of the bench line: time rnn / rnnBackward (LSTM, GRU) at a few sizes")
+    ap.add_argument("--linear", action="store_true",
+                    help="instead of the bench line: time fl::linear's forward product and backward pass (dx, dW, db) "
+                         "at the sizes of a speech model's layers, in --dtype")
     return ap.parse_args()
 
 
@@ -88,6 +91,8 @@ def main():
         return plan_sweep(a, fa, torch, tdt)
     if a.rnn:
         return rnn_sweep(a, fa, torch)
+    if a.linear:
+        return linear_sweep(a, fa, torch)
     if a.dtype == "f16":
         print("bench.py: --dtype f16 goes with --layers, --plans or --step (the bench line is quoted in f32, with bf16 beside it)",
               file=sys.stderr)
@@ -403,6 +408,37 @@ def rnn_sweep(a, fa, torch):
             print("%-4s input %d hidden %d layers %d dirs %d T %d batch %d: fwd %.2f ms (%.1f TFLOP/s)  "
                   "bwd %.2f ms (%.1f TFLOP/s)" % (name, I, H, L, D, T, B, tf, fl / tf / 1e9, tb, 2 * fl / tb / 1e9),
                   flush=True)
+    return 0
+
+
+def linear_sweep(a, fa, torch):
+    """Times of fl::linear's forward product (weight x input + bias) and of its backward pass (input gradient,
+    weight gradient, bias gradient) through the C ABI, by HIP events over a.steps calls after a.warmup; TFLOP/s
+    counts the one product forward and the two backward."""
+    ops = fa.ops
+    tdt = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}[a.dtype]
+    def timed(fn):
+        for _ in range(max(a.warmup, 1)):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(a.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / a.steps * 1e3
+    for (fin, fout, frames) in ((2000, 2000, 4000), (1024, 1024, 12000), (1200, 1200, 3000), (80, 2000, 12000),
+                                (2048, 1000, 256)):
+        x = torch.randn(frames, fin, device="cuda").to(tdt)
+        w = (torch.randn(fin, fout, device="cuda") / fin ** 0.5).to(tdt)
+        b = torch.randn(fout, device="cuda")
+        dy = torch.randn(frames, fout, device="cuda").to(tdt)
+        tf = timed(lambda: ops.linear(x, w, b))
+        tb = timed(lambda: ops.linear_backward(dy, x, w))
+        fl = 2.0 * fin * fout * frames
+        print("%s Linear %d -> %d over %d frames: forward %.1f us (%.0f TFLOP/s)  backward %.1f us (%.0f TFLOP/s)"
+              % (a.dtype, fin, fout, frames, tf, fl / tf / 1e6, tb, 2 * fl / tb / 1e6), flush=True)
     return 0
 
 
