@@ -96,7 +96,12 @@ SYMBOLS = {
     "flhip_pad_bwd": (C.c_int, [_VP, _VP, C.POINTER(C.c_int64), C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.c_int, _VP]),
     "flhip_matmul": (C.c_int, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int, C.c_int, _VP,
                                C.c_int, _VP]),
+    "flhip_matmul_workspace_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int32, C.c_int, C.c_int, C.c_int]),
+    "flhip_matmul_ws": (C.c_int, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int, C.c_int, _VP,
+                                  C.c_int, _VP, C.c_size_t, _VP]),
     "flhip_sum_columns": (C.c_int, [_VP, _VP, C.c_int32, C.c_int32, C.c_int, _VP]),
+    "flhip_sum_columns_workspace_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int]),
+    "flhip_sum_columns_ws": (C.c_int, [_VP, _VP, C.c_int32, C.c_int32, C.c_int, _VP, C.c_size_t, _VP]),
     "flhip_logsoftmax_fwd": (C.c_int, [_VP, _VP, C.c_int32, C.c_int32, C.c_int, _VP]),
     "flhip_logsoftmax_bwd": (C.c_int, [_VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int, _VP]),
     "flhip_cce_fwd": (C.c_int, [_VP, _VP, _VP, _VP, C.c_int32, C.c_int32, C.c_int32, C.c_int, _VP]),

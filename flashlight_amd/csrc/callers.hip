@@ -914,9 +914,54 @@ extern "C" int flhip_pad_bwd(const void* dy, void* dx, const int64_t* dims, cons
   return pad_launch(true, dy, dx, dims, before, after, 0.0, dtype, stream);
 }
 
+namespace {
+
+// slices of the contraction for A * B^T in fp32 (gemm_nt_kernel: 64 x 64 tiles): enough tiles times slices to
+// give every CU a few workgroups, at least eight chunks of 32 per slice
+int nt_slices(int M, int N, int K) {
+  const long long tiles = (long long)((M + 63) / 64) * ((N + 63) / 64), chunks = (K + 31) / 32;
+  long long ns = 1024 / tiles;
+  if (ns > chunks / 8) ns = chunks / 8;
+  if (ns > 16) ns = 16;
+  if (ns < 1) ns = 1;
+  const long long cps = (chunks + ns - 1) / ns;
+  return (int)((chunks + cps - 1) / cps);
+}
+
+__global__ void __launch_bounds__(256) sum_slices_kernel(const float* __restrict__ part, float* __restrict__ out, size_t n,
+                                                         int slices) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+    float v = part[i];
+#pragma unroll 8
+    for (int k = 1; k < slices; ++k) v += part[(size_t)k * n + i];      // loads in flight together, sums in slice order
+    out[i] = v;
+  }
+}
+
+}  // namespace
+
+extern "C" size_t flhip_matmul_workspace_bytes(int32_t M, int32_t N, int32_t K, int trans_a, int trans_b, int dtype) {
+  if (M <= 0 || N <= 0 || K <= 0 || !dtype_ok(dtype) || trans_a || !trans_b) return 0;
+  if (options().matmul_valu) return 0;
+  if (is_lo16(dtype)) return options().matmul_fp32_cores ? 0 : mfma_gemm16_ws_bytes(dtype, 2, M, N, K);
+  if (dtype != FLHIP_F32) return 0;
+  const int ns = nt_slices(M, N, K);
+  return ns > 1 ? (size_t)ns * M * N * sizeof(float) : 0;
+}
+
+extern "C" int flhip_matmul_ws(const void* A, const void* B, void* C, int32_t M, int32_t N, int32_t K,
+                               int trans_a, int trans_b, const float* bias_rows, int dtype, void* ws,
+                               size_t ws_bytes, void* stream);
+
 extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, int32_t N, int32_t K,
                             int trans_a, int trans_b, const float* bias_rows, int dtype,
                             void* stream) {
+  return flhip_matmul_ws(A, B, C, M, N, K, trans_a, trans_b, bias_rows, dtype, nullptr, 0, stream);
+}
+
+extern "C" int flhip_matmul_ws(const void* A, const void* B, void* C, int32_t M, int32_t N, int32_t K,
+                               int trans_a, int trans_b, const float* bias_rows, int dtype, void* ws,
+                               size_t ws_bytes, void* stream) {
   FLHIP_REQUIRE(A && B && C, "matmul: null argument");
   FLHIP_REQUIRE(M > 0 && N > 0 && K > 0, "matmul: sizes must be positive");
   FLHIP_REQUIRE(dtype_ok(dtype), "matmul: unknown dtype");
@@ -947,10 +992,24 @@ extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, in
   // needs; the tiled vector-ALU kernel below covers the rest.  16-bit storage: on the 16-bit
   // matrix instructions where the shape allows (MATMUL_FP32_CORES keeps them on the fp32 ones).
   if (is_lo16(dtype) && !(trans_a && trans_b) && !options().matmul_valu && !options().matmul_fp32_cores) {
-    const int rc = mfma_gemm16(dtype, trans_a ? 1 : trans_b ? 2 : 0, A, B, C, M, N, K, bias_rows, as_stream(stream));
+    const int rc = mfma_gemm16(dtype, trans_a ? 1 : trans_b ? 2 : 0, A, B, C, M, N, K, bias_rows, as_stream(stream),
+                               ws, ws_bytes);
     if (rc >= 0) return rc;
   }
   if (!trans_a && trans_b && !bias_rows && !options().matmul_valu) {
+    // fp32 with a workspace: the contraction in slices (the weight gradient of a layer over many frames is few
+    // tiles over a long contraction), added in slice order
+    const int ns = dtype == FLHIP_F32 && ws ? nt_slices(M, N, K) : 1;
+    if (ns > 1 && ws_bytes >= (size_t)ns * M * N * sizeof(float)) {
+      const int rc = gemm_nt(dtype, A, B, ws, M, N, K, ns, as_stream(stream));
+      if (rc >= 0) {
+        if (rc != 0) return rc;
+        const size_t n = (size_t)M * N;
+        hipLaunchKernelGGL(sum_slices_kernel, dim3((unsigned)std::min<size_t>((n + 255) / 256, 4096)), dim3(256), 0,
+                           as_stream(stream), static_cast<const float*>(ws), static_cast<float*>(C), n, ns);
+        return check_launch("matmul (A * B^T, slices added)");
+      }
+    }
     const int rc = gemm_nt(dtype, A, B, C, M, N, K, 1, as_stream(stream));
     if (rc >= 0) return rc;
   }
@@ -968,6 +1027,94 @@ extern "C" int flhip_matmul(const void* A, const void* B, void* C, int32_t M, in
                        bias_rows);
   });
   return check_launch("matmul");
+}
+
+namespace {
+
+// the value of a 16-bit element given as bits (the pointer selects the type)
+__device__ __forceinline__ float bits_value(const bf16_t*, uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+__device__ __forceinline__ float bits_value(const f16_t*, uint16_t b) { return f16_to_f32(f16_t{b}); }
+__device__ __forceinline__ float bits_value(const float*, uint16_t) { return 0.f; }      // fp32 rows are read one per lane
+
+// Column sums in two passes: pass 1, workgroup (row block, column slice): a wave's lanes are consecutive rows (two each
+// for 16-bit elements when the row count is even: 256 bytes per load instruction), its four waves take alternate
+// columns of the slice, eight loads in flight per lane; the waves' sums meet in LDS and leave as part[slice][row].
+// Pass 2 adds the slices in order.
+template <typename T, int RPL>
+__global__ void __launch_bounds__(256) sum_cols_sliced_kernel(const T* __restrict__ x, float* __restrict__ part, int R,
+                                                              int Cn, int cps) {
+  __shared__ float red[4][64 * RPL];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = (blockIdx.x * 64 + lane) * RPL;
+  const int cbeg = blockIdx.y * cps, cend = min(Cn, cbeg + cps);
+  float s[RPL] = {};
+  if (r < R) {
+    auto add = [&](int c) {
+      if (RPL == 2) {
+        const uint32_t v = *reinterpret_cast<const uint32_t*>(x + (size_t)c * R + r);
+        s[0] += bits_value(x, (uint16_t)(v & 0xffffu));
+        s[RPL - 1] += bits_value(x, (uint16_t)(v >> 16));
+      } else {
+        s[0] += ld(x, (size_t)c * R + r);
+      }
+    };
+    int c = cbeg + wave;
+    for (; c + 28 < cend; c += 32) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) add(c + 4 * u);
+    }
+    for (; c < cend; c += 4) add(c);
+  }
+#pragma unroll
+  for (int e = 0; e < RPL; ++e) red[wave][lane * RPL + e] = s[e];
+  __syncthreads();
+  for (int i = threadIdx.x; i < 64 * RPL; i += 256) {
+    const int row = blockIdx.x * 64 * RPL + i;
+    if (row < R) part[(size_t)blockIdx.y * R + row] = (red[0][i] + red[1][i]) + (red[2][i] + red[3][i]);
+  }
+}
+
+// column slices for rows x cols: enough workgroups for four per CU, at least 64 columns per slice
+int sum_cols_slices(int rows, int cols, int rpl) {
+  if ((long long)rows * cols < (1ll << 21)) return 1;      // a second launch costs more than it saves
+  const long long rb = (rows + 64 * rpl - 1) / (64 * rpl);
+  long long ns = 1024 / rb;
+  if (ns > cols / 64) ns = cols / 64;
+  if (ns > 32) ns = 32;      // the second pass reads them one after the other, one thread per row
+  if (ns < 1) ns = 1;
+  const long long cps = (cols + ns - 1) / ns;
+  return (int)((cols + cps - 1) / cps);
+}
+
+int sum_cols_rpl(int rows, int dtype) { return (is_lo16(dtype) && rows % 2 == 0) ? 2 : 1; }
+
+}  // namespace
+
+extern "C" size_t flhip_sum_columns_workspace_bytes(int32_t rows, int32_t cols, int dtype) {
+  if (rows <= 0 || cols <= 0 || !dtype_ok(dtype)) return 0;
+  const int ns = sum_cols_slices(rows, cols, sum_cols_rpl(rows, dtype));
+  return ns > 1 ? (size_t)ns * rows * sizeof(float) : 0;
+}
+
+extern "C" int flhip_sum_columns_ws(const void* x, float* out, int32_t rows, int32_t cols, int dtype, void* ws,
+                                    size_t ws_bytes, void* stream) {
+  FLHIP_REQUIRE(x && out, "sum_columns: null argument");
+  FLHIP_REQUIRE(rows > 0 && cols > 0, "sum_columns: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "sum_columns: unknown dtype");
+  const int rpl = sum_cols_rpl(rows, dtype), ns = sum_cols_slices(rows, cols, rpl);
+  if (ns <= 1 || !ws || ws_bytes < (size_t)ns * rows * sizeof(float) || ns > 65535)
+    return flhip_sum_columns(x, out, rows, cols, dtype, stream);
+  const int cps = (cols + ns - 1) / ns;
+  const dim3 grid((unsigned)((rows + 64 * rpl - 1) / (64 * rpl)), (unsigned)ns);
+  float* part = static_cast<float*>(ws);
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    if (rpl == 2) hipLaunchKernelGGL((sum_cols_sliced_kernel<T, 2>), grid, dim3(256), 0, as_stream(stream), (const T*)x, part, rows, cols, cps);
+    else hipLaunchKernelGGL((sum_cols_sliced_kernel<T, 1>), grid, dim3(256), 0, as_stream(stream), (const T*)x, part, rows, cols, cps);
+  });
+  hipLaunchKernelGGL(sum_slices_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, as_stream(stream), part, out,
+                     (size_t)rows, ns);
+  return check_launch("sum_columns (sliced)");
 }
 
 extern "C" int flhip_sum_columns(const void* x, float* out, int32_t rows, int32_t cols, int dtype,

@@ -67,7 +67,8 @@ int mfma_gemm(int dtype, int mode, const void* A, const void* B, void* C, int M,
 int mfma_gemm_slices(int K, int ksplit);
 // the same three products in 16-bit storage on the 16-bit matrix instructions (conv2d_mfma_pointwise_dma_bf16.hip)
 int mfma_gemm16(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,
-                const float* bias_rows, hipStream_t s);
+                const float* bias_rows, hipStream_t s, void* ws, size_t ws_bytes);
+size_t mfma_gemm16_ws_bytes(int dtype, int mode, int M, int N, int K);
 // column-major C = A * B^T on a kernel of its own (both operands contiguous along the
 // surviving dimension); slices > 1 (f32): partial products M * N floats apart
 int gemm_nt(int dtype, const void* A, const void* B, void* C, int M, int N, int K, int slices, hipStream_t s);

@@ -68,6 +68,11 @@ struct PwdParams {
   int nstages, mtiles, ctiles;
   unsigned src_bytes, w_bytes, dst_bytes;
   const float* pos_bias;   // one value per position, added to every result channel (matrix products: one image), or null
+  // matrix products with the contraction cut into slices (blockIdx.y): sps stages per slice (nstages: one slice), and
+  // where slice k leaves its fp32 partial product, [result channel][position], Mo * P floats per slice (null: one slice,
+  // results in the element type at dst)
+  int sps;
+  float* part;
 };
 
 // rows r0 .. r0+7 of column c0 + s of a 16-bit tile stored [row][column] (see the 1x1 kernels
@@ -163,17 +168,19 @@ pwd16_conv_kernel(PwdParams p, const E* __restrict__ src, const E* __restrict__ 
     }
   }
   const bool fourth = wave + 12 < NI, fifth = wave + 16 < NI;
-  const int n = p.nstages, n2 = (n + 1) & ~1;
+  const int sbeg = blockIdx.y * p.sps;      // this slice's first stage
+  const int n = min(p.nstages - sbeg, p.sps), n2 = (n + 1) & ~1;
   // stages are multiplied in pairs: with an odd number the stage past the contraction fetches nothing and fills its
   // slot with zeros (both operands: it adds 0)
   auto issue = [&](int t, uint4* ring) {
     const unsigned base = (unsigned)reinterpret_cast<uintptr_t>((lds_void_t)ring);
     const bool live = t < n;
+    const int tg = sbeg + t;
 #pragma unroll
     for (int k = 0; k < 3; ++k)
-      pd_load_lds(lrs[k], base + loff[k], (live && t * PD_KC < klim[k]) ? voff[k] : (int)0x80000000, t * lstep[k]);
-    if (fourth) pd_load_lds(lrs[3], base + loff[3], (live && t * PD_KC < klim[3]) ? voff[3] : (int)0x80000000, t * lstep[3]);
-    if (fifth) pd_load_lds(lrs[4], base + loff[4], (live && t * PD_KC < klim[4]) ? voff[4] : (int)0x80000000, t * lstep[4]);
+      pd_load_lds(lrs[k], base + loff[k], (live && tg * PD_KC < klim[k]) ? voff[k] : (int)0x80000000, tg * lstep[k]);
+    if (fourth) pd_load_lds(lrs[3], base + loff[3], (live && tg * PD_KC < klim[3]) ? voff[3] : (int)0x80000000, tg * lstep[3]);
+    if (fifth) pd_load_lds(lrs[4], base + loff[4], (live && tg * PD_KC < klim[4]) ? voff[4] : (int)0x80000000, tg * lstep[4]);
   };
 
   // ---- fragments: 128 result channels: wave = (position half, channel half), 2 x 2 blocks of 32 x 32;
@@ -248,6 +255,27 @@ pwd16_conv_kernel(PwdParams p, const E* __restrict__ src, const E* __restrict__ 
 #undef PD_MULT
 #undef PD_READ
 
+  if (p.part) {
+    // a slice's partial product leaves in fp32 straight from the accumulators (one image): a lane's four consecutive
+    // positions of a result channel; the positions a plane's last cell repeats are written twice with the same value
+    float* const part = p.part + (size_t)blockIdx.y * p.Mo * p.P;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int ch = m0 + mw0 + j * 32 + fr;
+      if (ch >= p.Mo) continue;
+#pragma unroll
+      for (int i = 0; i < NA; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int cell = cell0 + (pos0 + i * 32) / 8 + g;
+          if (cell >= p.ncells) continue;
+          float* q = part + (size_t)ch * p.P + min(8 * cell, p.P - 8) + fh * 4;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) q[e] = acc[i][j][4 * g + e];
+        }
+    }
+    return;
+  }
   __syncthreads();      // every wave has read its last fragments: the ring becomes the staging tile
   // ---- results: element r of block (i, j): slot pos0 + i*32 + (r/4)*8 + fh*4 + r%4 of channel
   // mw0 + j*32 + fr.  [channel][slot] in LDS, then whole cells to memory.
@@ -307,25 +335,51 @@ bool pwd16_applies(const ConvGeom& g, bool bwd) {
   return options().pw16_pf != 0 || (g.H * g.W <= 1024 && mo > 64);
 }
 
+// slices of the contraction for a matrix product of ctiles x mtiles tiles over nstages stages: as many as it takes to
+// give every CU a workgroup, at least eight stages each; *sps = stages per slice
+int pwd16_slices(int ctiles, int mtiles, int nstages, int* sps, int cap = 32) {
+  long long ns = mfma_num_cus() / std::max(1ll, (long long)ctiles * mtiles);
+  if (ns > nstages / 8) ns = nstages / 8;
+  if (ns > cap) ns = cap;
+  if (ns < 1) ns = 1;
+  *sps = (int)((nstages + ns - 1) / ns);
+  return (*sps > 0) ? (nstages + *sps - 1) / *sps : 1;
+}
+
+// result channels per tile
+int pwd16_bm(const PwdParams& p) {
+  const int pf = options().pw16_pf;
+  bool small = (long long)p.ctiles * ((p.Mo + PD_BM - 1) / PD_BM) <= mfma_num_cus() / 2;
+  if (pf) small = pf == 2 || pf == 8;
+  return small ? 64 : PD_BM;
+}
+
 // grid and kernel variant for a filled-in PwdParams (Kc, Mo, P, Pc, ncells, nstages, ctiles and the byte sizes)
+// slices > 1 (matrix products): the contraction in that many slices at most, their fp32 partial products at p.part
 template <typename E, bool BWD>
 int pwd16_go(PwdParams p, const void* src, const void* w, const float* bias, void* dst, const void* addend,
-             hipStream_t s, const char* what) {
+             hipStream_t s, const char* what, int* slices = nullptr) {
   // tiles of 64 result channels when tiles of 128 would leave half of the CUs without a workgroup (7x7 planes
   // with 512 result channels at batch 64: 112 workgroups of 64 stages); the deep ring for grids of at most one
   // workgroup per CU.  FLHIP_PW16_PF = 1 / 4 forces the shallow / deep ring with tiles of 128, 2 / 8 with tiles of 64.
   const int cus = mfma_num_cus(), pf = options().pw16_pf;
-  bool small = (long long)p.ctiles * ((p.Mo + PD_BM - 1) / PD_BM) <= cus / 2;
-  if (pf) small = pf == 2 || pf == 8;
-  const int bm = small ? 64 : PD_BM;
+  const int bm = pwd16_bm(p);
+  const bool small = bm == 64;
   p.mtiles = (p.Mo + bm - 1) / bm;
   const long long grid = (long long)((p.ctiles + 7) / 8) * 8 * p.mtiles;
   if (grid > 0x7fffffffll) return -1;
+  int ns = 1;
+  p.sps = p.nstages;
+  if (slices) {
+    ns = pwd16_slices(p.ctiles, p.mtiles, p.nstages, &p.sps, *slices);      // at most what the caller's workspace holds
+    *slices = ns;
+    if (ns <= 1) p.part = nullptr;
+  }
   auto go = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), 0, s, p, static_cast<const E*>(src),
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid, (unsigned)ns), dim3(256), 0, s, p, static_cast<const E*>(src),
                        static_cast<const E*>(w), bias, static_cast<E*>(dst), static_cast<const E*>(addend));
   };
-  bool deep = (long long)p.ctiles * p.mtiles <= (long long)cus;
+  bool deep = (long long)p.ctiles * p.mtiles * ns <= (long long)cus;
   if (pf) deep = pf >= 4;
   if (small) {
     if (deep) go(pwd16_conv_kernel<E, BWD, 8, 64>);
@@ -637,6 +691,33 @@ int mfma_pwd16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw
   return check_launch("conv2d_bwd_filter 1x1 (bf16 mfma, direct-to-LDS)");
 }
 
+// out[i] = the sum of `slices` fp32 partial products, n floats apart, added in slice order and rounded once
+template <typename E>
+__global__ void __launch_bounds__(256) gemm16_sum_slices_kernel(const float* __restrict__ part, uint16_t* __restrict__ out,
+                                                                size_t n, int slices) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+    float v = part[i];
+    for (int k = 1; k < slices; ++k) v += part[(size_t)k * n + i];
+    out[i] = Lo16<E>::narrow(v);
+  }
+}
+
+bool gemm16_plan(int mode, int M, int N, int K, const float* bias_rows, PwdParams* p) {
+  if (M < 8 || (mode == 0 && K % 8 != 0) || (mode == 2 && (bias_rows || N % 2 != 0))) return false;
+  p->Kc = K; p->Mo = N; p->P = M;
+  return pwd16_sizes(p, 1);
+}
+
+// bytes of workspace with which A B^T (mode 2) cuts its contraction into slices (0: one slice, or not these kernels')
+size_t mfma_gemm16_ws_bytes(int dtype, int mode, int M, int N, int K) {
+  PwdParams p{};
+  if (!is_lo16(dtype) || mode != 2 || M <= 0 || N <= 0 || K <= 0 || !gemm16_plan(mode, M, N, K, nullptr, &p)) return 0;
+  const int bm = pwd16_bm(p);
+  int sps;
+  const int ns = pwd16_slices(p.ctiles, (N + bm - 1) / bm, p.nstages, &sps);
+  return ns > 1 ? (size_t)ns * M * N * sizeof(float) : 0;
+}
+
 // Column-major matrix products in 16-bit storage on the kernels above (C is M x N, stored [n][m]):
 //   mode 0, C = A B    : A (M x K) is stored [k][m]: the source of a forward 1x1 layer over ONE image whose plane is the
 //                        M rows; B stored [n][k] are its weights; bias_rows (one per row of C) is a bias per position
@@ -648,8 +729,11 @@ int mfma_pwd16_wgrad(const ConvGeom& g, const void* x, const void* dy, float* dw
 // of 8 in mode 0 (a 16-byte cell of B would straddle two rows), a bias or an odd number of columns in mode 2 (the
 // range check of a buffer load works on 4-byte words: the word that holds the last element of B's last row would
 // lie half past the tensor and come back as zero), operands of 2 GiB.
+// With a workspace of mfma_gemm16_ws_bytes, A B^T over a long contraction and few tiles (the weight gradient of a
+// layer over many frames) cuts the contraction into slices, one workgroup per tile and slice; their fp32 partial
+// products are added in slice order.
 int mfma_gemm16(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,
-                const float* bias_rows, hipStream_t s) {
+                const float* bias_rows, hipStream_t s, void* ws, size_t ws_bytes) {
   if (!is_lo16(dtype) || M <= 0 || N <= 0 || K <= 0) return -1;
   if (mode == 1) {
     if (K < 8) return -1;
@@ -679,15 +763,22 @@ int mfma_gemm16(int dtype, int mode, const void* A, const void* B, void* C, int 
     return check_launch("matmul (A^T * B, 16-bit mfma)");
   }
   if (mode != 0 && mode != 2) return -1;
-  if (M < 8 || (mode == 0 && K % 8 != 0) || (mode == 2 && (bias_rows || N % 2 != 0))) return -1;
   PwdParams p{};
-  p.Kc = K; p.Mo = N; p.P = M;
-  if (!pwd16_sizes(&p, 1)) return -1;
+  if (!gemm16_plan(mode, M, N, K, bias_rows, &p)) return -1;
   p.pos_bias = bias_rows;
   return by_lo16(dtype, [&](auto* e_) {
     using E = FLHIP_T_OF(e_);
-    return mode == 0 ? pwd16_go<E, false>(p, A, B, nullptr, C, nullptr, s, "matmul (A * B, 16-bit mfma)")
-                     : pwd16_go<E, true>(p, A, B, nullptr, C, nullptr, s, "matmul (A * B^T, 16-bit mfma)");
+    if (mode == 0) return pwd16_go<E, false>(p, A, B, nullptr, C, nullptr, s, "matmul (A * B, 16-bit mfma)");
+    const size_t per = (size_t)M * N * sizeof(float);
+    int slices = ws ? (int)std::min<size_t>(ws_bytes / per, 32) : 1;
+    if (slices <= 1) return pwd16_go<E, true>(p, A, B, nullptr, C, nullptr, s, "matmul (A * B^T, 16-bit mfma)");
+    p.part = static_cast<float*>(ws);
+    const int rc = pwd16_go<E, true>(p, A, B, nullptr, C, nullptr, s, "matmul (A * B^T, 16-bit mfma)", &slices);
+    if (rc != 0 || slices <= 1) return rc;
+    const size_t n = (size_t)M * N;
+    hipLaunchKernelGGL(gemm16_sum_slices_kernel<E>, dim3((unsigned)std::min<size_t>((n + 255) / 256, 4096)), dim3(256), 0, s,
+                       static_cast<const float*>(ws), static_cast<uint16_t*>(C), n, slices);
+    return check_launch("matmul (A * B^T, 16-bit mfma, slices added)");
   });
 }
 

@@ -804,8 +804,10 @@ Variable linear(const Variable& input, const Variable& weight, const Variable& b
     Tensor dxT, dwT, dbT;
     if (hasBias && inputs[2].isCalcGrad()) {
       Tensor db(inputs[2].shape(), dtype::f32);
-      check(flhip_sum_columns(g, static_cast<float*>(db.device()), (int32_t)out, (int32_t)frames, tag,
-                              hipBackendStream()));
+      const size_t wsBytes = flhip_sum_columns_workspace_bytes((int32_t)out, (int32_t)frames, tag);
+      Tensor ws = wsBytes ? Tensor({(Dim)wsBytes}, dtype::u8) : Tensor();
+      check(flhip_sum_columns_ws(g, static_cast<float*>(db.device()), (int32_t)out, (int32_t)frames, tag, ws.device(),
+                                 wsBytes, hipBackendStream()));
       dbT = db;
     }
     if (x.isCalcGrad()) {
@@ -816,8 +818,11 @@ Variable linear(const Variable& input, const Variable& weight, const Variable& b
     }
     if (wt.isCalcGrad()) {
       Tensor dw(wt.shape(), wt.type());
-      check(flhip_matmul(g, x.tensor().device(), dw.device(), (int32_t)out, (int32_t)in,
-                         (int32_t)frames, 0, 1, nullptr, tag, hipBackendStream()));
+      // few tiles over a long contraction (the frames): with a workspace the library cuts it into slices
+      const size_t wsBytes = flhip_matmul_workspace_bytes((int32_t)out, (int32_t)in, (int32_t)frames, 0, 1, tag);
+      Tensor ws = wsBytes ? Tensor({(Dim)wsBytes}, dtype::u8) : Tensor();
+      check(flhip_matmul_ws(g, x.tensor().device(), dw.device(), (int32_t)out, (int32_t)in,
+                            (int32_t)frames, 0, 1, nullptr, tag, ws.device(), wsBytes, hipBackendStream()));
       dwT = dw;
     }
     // event: inputs {gradOutput, input, weight}, outputs {dx, dw, db (each may be empty)}, ints {out, in, frames}

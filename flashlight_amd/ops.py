@@ -602,12 +602,17 @@ def linear_backward(grad_output, input, weight, want_bias=True):
     capi.check(capi.lib().flhip_matmul(_ptr(w), _ptr(g), _ptr(dx), fin, frames, fout, 1, 0, None, tag,
                                        _stream()))
     dw = torch.empty_like(w)
-    capi.check(capi.lib().flhip_matmul(_ptr(g), _ptr(x), _ptr(dw), fout, fin, frames, 0, 1, None, tag,
-                                       _stream()))
+    nws = capi.lib().flhip_matmul_workspace_bytes(fout, fin, frames, 0, 1, tag)
+    ws = torch.empty((nws,), dtype=torch.uint8, device=x.device) if nws else None
+    capi.check(capi.lib().flhip_matmul_ws(_ptr(g), _ptr(x), _ptr(dw), fout, fin, frames, 0, 1, None, tag,
+                                          _ptr(ws) if nws else None, nws, _stream()))
     db = None
     if want_bias:
         db = torch.empty((fout,), dtype=torch.float32, device=x.device)
-        capi.check(capi.lib().flhip_sum_columns(_ptr(g), _ptr(db), fout, frames, tag, _stream()))
+        nws = capi.lib().flhip_sum_columns_workspace_bytes(fout, frames, tag)
+        ws = torch.empty((nws,), dtype=torch.uint8, device=x.device) if nws else None
+        capi.check(capi.lib().flhip_sum_columns_ws(_ptr(g), _ptr(db), fout, frames, tag, _ptr(ws) if nws else None,
+                                                   nws, _stream()))
     return dx, dw, db
 
 

@@ -117,7 +117,7 @@ const char* flhip_last_error(void);
  * 200: flhip_rnn_desc gained dropout, seed_lo, seed_hi; flhip_bn_workspace_bytes never returns less
  * than 32 bytes per feature.  202: the *_plan entry points and FLHIP_DECLINED.  203: FLHIP_F16.  204: flhip_act_fwd / _bwd, flhip_glu_fwd / _bwd,
  * flhip_dropout, flhip_rownorm, flhip_weightnorm_fwd / _bwd, flhip_pad_fwd / _bwd, flhip_sgd_many, flhip_adam_many.  205: flhip_prelu_fwd / _bwd, FLHIP_ACT_LEAKY, FLHIP_ACT_THRESHOLD. */
-#define FLHIP_VERSION 205
+#define FLHIP_VERSION 206
 int flhip_version(void);
 const char* flhip_arch(void);
 
@@ -441,11 +441,28 @@ int flhip_pad_bwd(const void* dy, void* dx, const int64_t* dims, const int32_t* 
 int flhip_matmul(const void* A, const void* B, void* C, int32_t M, int32_t N,
                  int32_t K, int trans_a, int trans_b, const float* bias_rows,
                  int dtype, void* stream);
+/* The same product with a workspace.  A * B^T with few tiles of C over a long contraction
+ * (matmulNT(gradOutput, input), Functions.cpp:1297-1303, of a layer over many frames) leaves
+ * most of the chip idle; with flhip_matmul_workspace_bytes(...) bytes at ws (0: this product
+ * has no use for one) the contraction is cut into slices, one workgroup per tile and slice,
+ * whose fp32 partial products are added in slice order (the result does not depend on
+ * timing).  ws == NULL or fewer bytes: as flhip_matmul. */
+size_t flhip_matmul_workspace_bytes(int32_t M, int32_t N, int32_t K, int trans_a, int trans_b, int dtype);
+int flhip_matmul_ws(const void* A, const void* B, void* C, int32_t M, int32_t N,
+                    int32_t K, int trans_a, int trans_b, const float* bias_rows,
+                    int dtype, void* ws, size_t ws_bytes, void* stream);
 
 /* out[r] (fp32) = sum over c of x[r, c] for a rows x cols matrix: the bias gradient
  * sumAs(gradOutput, bias) of fl::linear (Functions.cpp:1285-1289). */
 int flhip_sum_columns(const void* x, float* out, int32_t rows, int32_t cols, int dtype,
                       void* stream);
+/* The same sums with a workspace: few rows over many columns (a layer over many frames) are
+ * few workgroups for flhip_sum_columns; with flhip_sum_columns_workspace_bytes(...) bytes at
+ * ws (0: no use for one) the columns are cut into slices whose partial sums are added in
+ * slice order.  ws == NULL or fewer bytes: as flhip_sum_columns. */
+size_t flhip_sum_columns_workspace_bytes(int32_t rows, int32_t cols, int dtype);
+int flhip_sum_columns_ws(const void* x, float* out, int32_t rows, int32_t cols, int dtype,
+                         void* ws, size_t ws_bytes, void* stream);
 
 /* fl::reorder (flashlight/fl/autograd/Functions.cpp:1010-1042) of a tensor with the four
  * column-major extents dims[0..3] (dims[0] fastest; pad with 1): dimension k of dst is

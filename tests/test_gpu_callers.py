@@ -116,6 +116,74 @@ def test_matmul_in_16_bit_storage(M, N, K, ta, tb, dtype):
         assert not bad.any(), (int(bad.sum()), np.argwhere(bad)[:4].tolist())
 
 
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("M,N,K,part", [(128, 80, 5000, 1.0), (2000, 80, 12000, 1.0), (1024, 1024, 12000, 1.0),
+                                        (67, 130, 3001, 1.0), (256, 64, 4096, 0.5), (300, 200, 70, 1.0)])
+def test_matmul_with_a_workspace_cuts_a_long_contraction(M, N, K, part, dtype):
+    """flhip_matmul_ws: A * B^T of few tiles over a long contraction (the weight gradient of a layer over many
+    frames) in slices whose partial products are added in slice order; with part < 1 the caller brings less than
+    flhip_matmul_workspace_bytes asks for (fewer slices, or none).  Checked against numpy's float64 product of the
+    same rounded operands; two calls give the same bits."""
+    import ctypes as C
+    from flashlight_amd import capi
+    rng = np.random.default_rng(M + N + K)
+    A = _round(rng.standard_normal((K, M)).astype(np.float32), dtype)
+    B = _round(rng.standard_normal((K, N)).astype(np.float32), dtype)
+    want = B.astype(np.float64).T @ A.astype(np.float64)                       # stored [n][m]
+    code = {torch.float32: capi.F32, torch.bfloat16: capi.BF16, torch.float16: capi.F16}[dtype]
+    lib = capi.lib()
+    assert lib.flhip_matmul_workspace_bytes(M, N, K, 0, 0, code) == 0          # only A * B^T has a use for one
+    assert lib.flhip_matmul_workspace_bytes(M, N, K, 1, 0, code) == 0
+    need = lib.flhip_matmul_workspace_bytes(M, N, K, 0, 1, code)
+    if K >= 3000 and M * N <= 1024 * 1024 and (dtype == torch.float32 or N % 2 == 0):
+        assert need >= 2 * M * N * 4
+    nws = int(need * part) // 4 * 4
+    ws = torch.full((max(nws, 4),), 0xff, dtype=torch.uint8, device="cuda")
+    Ad, Bd = dev(A, dtype), dev(B, dtype)
+    P = lambda t: C.c_void_p(t.data_ptr())
+    S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    outs = []
+    for _ in range(2):
+        Cd = torch.empty(N, M, device="cuda", dtype=dtype)
+        assert lib.flhip_matmul_ws(P(Ad), P(Bd), P(Cd), M, N, K, 0, 1, None, code, P(ws) if nws else None, nws, S) == 0
+        outs.append(host(Cd))
+    assert np.array_equal(outs[0], outs[1])
+    half_ulp = {torch.float32: 2.0 ** -24, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[dtype]
+    bad = np.abs(outs[0].astype(np.float64) - want) > 1.01 * half_ulp * np.abs(want) + 2e-6 * K
+    assert not bad.any(), (int(bad.sum()), np.argwhere(bad)[:4].tolist())
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("rows,cols,part", [(2000, 12000, 1.0), (80, 12000, 1.0), (67, 5000, 1.0), (129, 333, 1.0), (1, 4096, 1.0),
+                                            (1024, 64, 1.0), (512, 3000, 0.5), (130, 100000, 1.0)])
+def test_sum_columns_with_a_workspace(rows, cols, part, dtype):
+    """flhip_sum_columns_ws (the bias gradient of fl::linear over many frames): the columns in slices, added in slice
+    order; against the oracle's sums (float64 accumulation), two calls bit-equal, and with less workspace than asked
+    for the one-pass kernel's result."""
+    import ctypes as C
+    from flashlight_amd import capi
+    rng = np.random.default_rng(rows + cols)
+    x = _round(rng.standard_normal((cols, rows)).astype(np.float32), dtype)
+    want = flref.sum_columns(rows, cols, x)
+    code = {torch.float32: capi.F32, torch.bfloat16: capi.BF16, torch.float16: capi.F16}[dtype]
+    lib = capi.lib()
+    need = lib.flhip_sum_columns_workspace_bytes(rows, cols, code)
+    if cols >= 3000 and rows * cols >= 1 << 21:
+        assert need >= 2 * rows * 4
+    nws = int(need * part) // 4 * 4
+    ws = torch.full((max(nws, 4),), 0xff, dtype=torch.uint8, device="cuda")
+    xd = dev(x, dtype)
+    P = lambda t: C.c_void_p(t.data_ptr())
+    S = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    outs = []
+    for _ in range(2):
+        out = torch.full((rows,), float("nan"), device="cuda")
+        assert lib.flhip_sum_columns_ws(P(xd), P(out), rows, cols, code, P(ws) if nws else None, nws, S) == 0
+        outs.append(host(out))
+    assert np.array_equal(outs[0], outs[1])
+    assert np.allclose(outs[0], want, rtol=1e-5, atol=2e-6 * cols)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_matmul_in_16_bit_storage_at_the_size_of_a_speech_model(dtype):
     """2000 x 2000 weights against 4000 frames, the three products of a layer's step; checked against numpy's
