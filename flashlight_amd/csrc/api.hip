@@ -85,6 +85,7 @@ static bool apply_option(Options& o, const char* name, const char* v) {
   if (!strcmp(name, "TAPPED_NO_REORDER")) return flag(&o.tapped_no_reorder);
   if (!strcmp(name, "MATMUL_VALU")) return flag(&o.matmul_valu);
   if (!strcmp(name, "MATMUL_FP32_CORES")) return flag(&o.matmul_fp32_cores);
+  if (!strcmp(name, "MATMUL_PLANES")) { o.matmul_planes = v ? atoi(v) : def.matmul_planes; return true; }
   if (!strcmp(name, "RNN_UNFUSED")) return flag(&o.rnn_unfused);
   if (!strcmp(name, "TAP2D_ALL")) return flag(&o.tap2d_all);
   return false;
@@ -92,7 +93,7 @@ static bool apply_option(Options& o, const char* name, const char* v) {
 
 static void options_from_environment() {
   static const char* const names[] = {"CONV_ALGO", "CONV_SKIP", "PW_PT", "PW16_PF", "CONV_STACK", "SLAB_WAVES", "BN_ALGO", "PW16_NO_TAPS",
-                                      "TAPPED_NO_REORDER", "MATMUL_VALU", "MATMUL_FP32_CORES", "RNN_UNFUSED", "TAP2D_ALL"};
+                                      "TAPPED_NO_REORDER", "MATMUL_VALU", "MATMUL_FP32_CORES", "MATMUL_PLANES", "RNN_UNFUSED", "TAP2D_ALL"};
   for (const char* n : names) {
     const std::string var = std::string("FLHIP_") + n;
     if (const char* v = getenv(var.c_str())) apply_option(g_options, n, v);   // unknown values keep the default

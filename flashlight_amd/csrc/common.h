@@ -292,6 +292,8 @@ struct Options {
   bool pw16_no_taps = false;      // PW16_NO_TAPS: bf16 windows with several taps stay off the gathered-taps path
   bool tapped_no_reorder = false; // TAPPED_NO_REORDER: tapped kernels read the original weight layout
   bool matmul_valu = false;       // MATMUL_VALU: flhip_matmul stays off the matrix cores
+  int matmul_planes = -1;         // MATMUL_PLANES: bit m set = fp32 product of mode m (0: A B, 1: A^T B, 2: A B^T) with a
+                                  // matrix as one image's plane whatever its shape; 0: never; -1: by shape
   bool matmul_fp32_cores = false; // MATMUL_FP32_CORES: 16-bit products stay on the fp32 matrix instructions
   bool rnn_unfused = false;       // RNN_UNFUSED: two-kernel rnn steps
   bool tap2d_all = false;         // TAP2D_ALL: the kernel for 3x3 windows over stacked planes takes every geometry it can, not only those of its measured rule

@@ -65,6 +65,8 @@ int mfma_pointwise_conv_split(const ConvGeom& g, int dtype, bool bwd, const void
 int mfma_gemm(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,
               const float* bias_rows, hipStream_t s, int ksplit = 1);
 int mfma_gemm_slices(int K, int ksplit);
+int mfma_gemm_planes(int mode, const void* A, const void* B, void* C, int M, int N, int K, const float* bias_rows,
+                     hipStream_t s);
 // the same three products in 16-bit storage on the 16-bit matrix instructions (conv2d_mfma_pointwise_dma_bf16.hip)
 int mfma_gemm16(int dtype, int mode, const void* A, const void* B, void* C, int M, int N, int K,
                 const float* bias_rows, hipStream_t s, void* ws, size_t ws_bytes);

@@ -1135,6 +1135,45 @@ int mfma_gemm(int dtype, int mode, const void* A, const void* B, void* C, int M,
   return -1;
 }
 
+// C[n][m] += bias[m]
+__global__ void __launch_bounds__(256) add_row_bias_kernel(float* __restrict__ C, const float* __restrict__ bias, int M,
+                                                           size_t n) {
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) C[i] += bias[i % M];
+}
+
+// The same products (fp32) with a matrix as ONE image whose plane is its contiguous dimension, so that the kernels
+// fetch their operand tiles as on the planes of a convolution (positions contiguous) instead of gathering one
+// position per image:
+//   mode 0, C = A B    : forward layer, x = A ([k][m]: K channels over a plane of M), weights B ([n][k]); the bias
+//                        per row of C is a bias per position: added by a pass of its own
+//   mode 1, C = A^T B  : filter gradient, x = A ([m][k]), dy = B ([n][k]), plane = the contraction (one slice)
+//   mode 2, C = A B^T  : backward-data layer, dy = A ([k][m]), weights B ([k][n])
+int mfma_gemm_planes(int mode, const void* A, const void* B, void* C, int M, int N, int K, const float* bias_rows,
+                     hipStream_t s) {
+  ConvGeom g{};
+  g.N = 1;
+  g.H = g.OH = g.KH = g.KW = 1;
+  g.sy = g.sx = g.dly = g.dlx = g.groups = 1;
+  int rc = -1;
+  if (mode == 0) {
+    g.W = g.OW = M; g.C = g.Cg = K; g.K = g.Kg = N;
+    rc = mfma_pointwise_conv_fwd(g, FLHIP_F32, A, B, nullptr, C, s, 1);
+  } else if (mode == 2 && !bias_rows) {
+    g.W = g.OW = M; g.C = g.Cg = N; g.K = g.Kg = K;
+    rc = mfma_pointwise_conv_bwd_data(g, FLHIP_F32, A, B, C, s, nullptr, 1);
+  } else if (mode == 1) {
+    g.W = g.OW = K; g.C = g.Cg = M; g.K = g.Kg = N;
+    const long long tiles = (long long)((M + BM - 1) / BM) * ((N + BM - 1) / BM);
+    if (tiles < 64) return -1;
+    rc = mfma_pointwise_wgrad(g, FLHIP_F32, A, B, static_cast<float*>(C), nullptr, nullptr, 0, false, s, 1);
+  }
+  if (rc != 0 || !bias_rows) return rc;
+  const size_t n = (size_t)M * N;
+  hipLaunchKernelGGL(add_row_bias_kernel, dim3((unsigned)std::min<size_t>((n + 255) / 256, 8192)), dim3(256), 0, s,
+                     static_cast<float*>(C), bias_rows, M, n);
+  return check_launch("matmul (bias)");
+}
+
 // number of partial products mfma_gemm writes for a contraction of length K cut into at
 // most ksplit slices
 int mfma_gemm_slices(int K, int ksplit) {

@@ -130,6 +130,8 @@ const char* flhip_arch(void);
  *   PW_PT = 2 | 4 | 8    PW16_PF = 0 | 1 | 2 | 4 | 8    CONV_STACK = 0 | 1 | 2 | 4 | 8    BN_ALGO = split | resident | auto
  *   SLAB_WAVES = 0 | 4 | 8
  *   PW16_NO_TAPS, TAPPED_NO_REORDER, MATMUL_VALU, MATMUL_FP32_CORES, RNN_UNFUSED, TAP2D_ALL = 1 | 0
+ *   MATMUL_PLANES = 0..7 (bit m: the fp32 product of form m - 0: A B, 1: A^T B, 2: A B^T - takes a matrix as one
+ *                   image's plane whatever its shape; 0: never; unset: by shape)
  * Unknown names or values return FLHIP_INVALID_ARGUMENT.  The nearest thing in the
  * reference is the kernel-choice options object of its cuDNN extension
  * (createBenchmarkOptions, flashlight/fl/autograd/tensor/backend/cudnn/CudnnAutogradExtension.h:25). */

@@ -184,6 +184,45 @@ def test_sum_columns_with_a_workspace(rows, cols, part, dtype):
     assert np.allclose(outs[0], want, rtol=1e-5, atol=2e-6 * cols)
 
 
+@pytest.mark.parametrize("planes", [7, 0, None])
+@pytest.mark.parametrize("M,N,K", LO16_MATMUL + [(256, 200, 64), (512, 4100, 36), (1027, 1030, 130)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True)])
+def test_matmul_fp32_with_a_matrix_as_one_plane(M, N, K, ta, tb, planes):
+    """fp32 products on the 1x1 kernels with a matrix as one image's plane (option MATMUL_PLANES: 7 = whatever the
+    shape, 0 = never, unset = by shape), every element against the oracle."""
+    from flashlight_amd import capi
+    rng = np.random.default_rng(M * 1000 + N * 10 + K + int(ta) + 2 * int(tb))
+    A = rng.standard_normal((M, K) if ta else (K, M)).astype(np.float32)
+    B = rng.standard_normal((K, N) if tb else (N, K)).astype(np.float32)
+    capi.set_option("MATMUL_PLANES", planes)
+    try:
+        for bias in ([None] if tb else [None, rng.standard_normal(M).astype(np.float32)]):
+            want = flref.matmul(M, N, K, A, B, ta, tb, bias)
+            got = _matmul_through_c_abi(A, B, M, N, K, ta, tb, bias, torch.float32)
+            bad = np.abs(got.astype(np.float64) - want) > 1e-5 * np.abs(want) + 2e-6 * K
+            assert not bad.any(), (int(bad.sum()), np.argwhere(bad)[:4].tolist())
+    finally:
+        capi.set_option("MATMUL_PLANES", None)
+
+
+def test_matmul_fp32_at_the_size_of_a_speech_model():
+    """2000 x 2000 weights against 4000 frames in fp32 (the plane mapping by shape), against numpy's float64 product."""
+    M, N, K = 2000, 4000, 2000
+    rng = np.random.default_rng(78)
+    for ta, tb in [(False, False), (True, False), (False, True)]:
+        A = rng.standard_normal((M, K) if ta else (K, M)).astype(np.float32)
+        B = rng.standard_normal((K, N) if tb else (N, K)).astype(np.float32)
+        A64 = A.astype(np.float64) if ta else A.astype(np.float64).T
+        B64 = B.astype(np.float64) if tb else B.astype(np.float64).T
+        want = (A64 @ B64).T
+        bias = rng.standard_normal(M).astype(np.float32) if not (ta or tb) else None
+        if bias is not None:
+            want = want + bias[None, :]
+        got = _matmul_through_c_abi(A, B, M, N, K, ta, tb, bias, torch.float32)
+        bad = np.abs(got.astype(np.float64) - want) > 1e-5 * np.abs(want) + 2e-6 * K
+        assert not bad.any(), (ta, tb, int(bad.sum()), np.argwhere(bad)[:4].tolist())
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_matmul_in_16_bit_storage_at_the_size_of_a_speech_model(dtype):
     """2000 x 2000 weights against 4000 frames, the three products of a layer's step; checked against numpy's
