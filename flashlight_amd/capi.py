@@ -119,6 +119,8 @@ SYMBOLS = {
     "flhip_affine_bwd_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int64, C.c_int64, C.c_int]),
     "flhip_affine_bwd": (C.c_int, [_VP, _VP, _VP, _VP, _VP, _VP, C.c_int64, C.c_int64, C.c_int64, C.c_int,
                                    C.c_int, _VP, C.c_size_t, _VP]),
+    "flhip_embedding_fwd": (C.c_int, [_VP, _VP, _VP, C.c_int64, C.c_int32, C.c_int32, C.c_int, _VP]),
+    "flhip_embedding_bwd": (C.c_int, [_VP, _VP, _VP, C.c_int64, C.c_int32, C.c_int32, C.c_int, _VP]),
     "flhip_prelu_fwd": (C.c_int, [_VP, _VP, _VP, C.c_int64, C.c_int64, C.c_int, C.c_int, _VP]),
     "flhip_prelu_bwd_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int64, C.c_int]),
     "flhip_prelu_bwd": (C.c_int, [_VP, _VP, _VP, _VP, _VP, C.c_int64, C.c_int64, C.c_int, C.c_int, _VP, C.c_size_t,

@@ -1288,6 +1288,92 @@ extern "C" int flhip_affine_bwd(const void* dy, const void* x, const void* w, vo
   return FLHIP_OK;
 }
 
+namespace {
+
+// y[:, i] = w[:, idx[i]]: a workgroup per group of columns, threads along the embedding dimension
+template <typename T>
+__global__ void __launch_bounds__(256) embedding_fwd_kernel(const int32_t* __restrict__ idx, const T* __restrict__ w,
+                                                            T* __restrict__ y, long long n, int dim, int tokens) {
+  for (long long i = blockIdx.x; i < n; i += gridDim.x) {
+    const int t = idx[i];
+    const bool ok = t >= 0 && t < tokens;
+    for (int d = threadIdx.x; d < dim; d += 256) y[i * dim + d] = ok ? w[(size_t)t * dim + d] : T{};
+  }
+}
+
+// dw[:, t] = the sum, in the order of i, of dy[:, i] over the positions i with idx[i] == t.  A workgroup per token:
+// its first wave scans the indices 64 at a time (one ballot) and queues the matching positions in LDS, in order;
+// then all threads add those columns, each thread its own rows of the embedding dimension, so the order of the
+// additions is that of the positions whatever the timing.
+template <typename T>
+__global__ void __launch_bounds__(256) embedding_bwd_kernel(const int32_t* __restrict__ idx, const T* __restrict__ dy,
+                                                            T* __restrict__ dw, long long n, int dim) {
+  __shared__ int queue[64];
+  __shared__ int qn;
+  const int t = blockIdx.x, tid = threadIdx.x;
+  constexpr int DPT = 8;                      // rows of the embedding dimension per thread and pass
+  for (int d0 = 0; d0 < dim; d0 += 256 * DPT) {
+    float acc[DPT];
+#pragma unroll
+    for (int e = 0; e < DPT; ++e) acc[e] = 0.f;
+    for (long long i0 = 0; i0 < n; i0 += 64) {
+      if (tid < 64) {      // the first wave
+        const long long i = i0 + tid;
+        const bool hit = i < n && idx[i] == t;
+        const unsigned long long m = __ballot(hit);
+        if (hit) queue[__popcll(m & ((1ull << tid) - 1ull))] = tid;
+        if (tid == 0) qn = __popcll(m);
+      }
+      __syncthreads();
+      const int q = qn;
+      for (int k = 0; k < q; ++k) {
+        const long long col = i0 + queue[k];
+#pragma unroll
+        for (int e = 0; e < DPT; ++e) {
+          const int d = d0 + e * 256 + tid;
+          if (d < dim) acc[e] += ld(dy, (size_t)col * dim + d);
+        }
+      }
+      __syncthreads();      // every wave is done with the queue and with qn before the first wave writes them again
+    }
+#pragma unroll
+    for (int e = 0; e < DPT; ++e) {
+      const int d = d0 + e * 256 + tid;
+      if (d < dim) st(dw, (size_t)t * dim + d, acc[e]);
+    }
+    __syncthreads();
+  }
+}
+
+}  // namespace
+
+extern "C" int flhip_embedding_fwd(const int32_t* idx, const void* w, void* y, int64_t n, int32_t dim, int32_t tokens,
+                                   int dtype, void* stream) {
+  FLHIP_REQUIRE(idx && w && y, "embedding: null argument");
+  FLHIP_REQUIRE(n > 0 && dim > 0 && tokens > 0, "embedding: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "embedding: unknown dtype");
+  const unsigned grid = (unsigned)std::min<int64_t>(n, 65535 * 16);
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((embedding_fwd_kernel<T>), dim3(grid), dim3(256), 0, as_stream(stream), idx, (const T*)w, (T*)y,
+                       (long long)n, dim, tokens);
+  });
+  return check_launch("embedding");
+}
+
+extern "C" int flhip_embedding_bwd(const int32_t* idx, const void* dy, void* dw, int64_t n, int32_t dim, int32_t tokens,
+                                   int dtype, void* stream) {
+  FLHIP_REQUIRE(idx && dy && dw, "embedding_bwd: null argument");
+  FLHIP_REQUIRE(n > 0 && dim > 0 && tokens > 0, "embedding_bwd: sizes must be positive");
+  FLHIP_REQUIRE(dtype_ok(dtype), "embedding_bwd: unknown dtype");
+  by_dtype(dtype, [&](auto* t_) {
+    using T = FLHIP_T_OF(t_);
+    hipLaunchKernelGGL((embedding_bwd_kernel<T>), dim3((unsigned)tokens), dim3(256), 0, as_stream(stream), idx,
+                       (const T*)dy, (T*)dw, (long long)n, dim);
+  });
+  return check_launch("embedding_bwd");
+}
+
 extern "C" int flhip_prelu_fwd(const void* x, const void* w, void* y, int64_t outer, int64_t d0, int scalar_param,
                                int dtype, void* stream) {
   FLHIP_REQUIRE(x && w && y, "prelu_fwd: null argument");

@@ -433,6 +433,32 @@ Variable detail::affine(const Variable& input, const Variable& weight, const Var
   return Variable(out, {input, weight, bias}, gradFunc);
 }
 
+Variable embedding(const Variable& input, const Variable& embeddings) {
+  if (input.ndim() >= 4) throw std::invalid_argument("embedding input must have 3 or fewer dims");   // as the reference
+  if (input.type() != dtype::s32) throw std::invalid_argument("embedding: indices must be s32 on this backend");
+  if (embeddings.ndim() != 2 || input.elements() == 0) throw std::invalid_argument("embedding: a [dim, tokens] table and at least one index");
+  detail::OpScope scope("embedding");
+  const int tag = tagOf(embeddings.type(), "embedding");
+  const Dim dim = embeddings.dim(0), tokens = embeddings.dim(1), n = input.elements();
+  std::vector<Dim> rDims{dim};
+  for (int i = 0; i < input.ndim(); ++i) rDims.push_back(input.dim(i));
+  Tensor out{Shape(rDims), embeddings.type()};
+  check(flhip_embedding_fwd(static_cast<const int32_t*>(input.tensor().device()), embeddings.tensor().device(), out.device(),
+                            (int64_t)n, (int32_t)dim, (int32_t)tokens, tag, hipBackendStream()));
+  if (scope.on()) scope.done({input.tensor(), embeddings.tensor()}, {out});
+  auto gradFunc = [n, dim, tokens, tag](std::vector<Variable>& inputs, const Variable& gradOutput) {
+    auto& w = inputs[1];
+    if (!w.isCalcGrad()) return;
+    detail::OpScope scope("embeddingBackward");
+    Tensor dw(w.shape(), w.type());
+    check(flhip_embedding_bwd(static_cast<const int32_t*>(inputs[0].tensor().device()), gradOutput.tensor().device(),
+                              dw.device(), (int64_t)n, (int32_t)dim, (int32_t)tokens, tag, hipBackendStream()));
+    if (scope.on()) scope.done({gradOutput.tensor(), inputs[0].tensor()}, {dw});
+    w.addGrad(Variable(dw, false));
+  };
+  return Variable(out, {input, embeddings}, gradFunc);
+}
+
 Variable prelu(const Variable& input, const Variable& weight) {
   dtypesMatch("prelu", {&input, &weight});
   if (input.ndim() < 1 || input.elements() == 0) throw std::invalid_argument("prelu: empty input");

@@ -162,6 +162,9 @@ inline Variable operator*(double lhs, const Variable& rhs) { return scale(rhs, l
 // fl::PReLU's forward (nn/modules/Activations.cpp:121-124) as one operator: input where input >= 0, input * weight
 // elsewhere, the weight tiled along dimension 0 (one element, or one per index of dimension 0).  Same dtype for both.
 Variable prelu(const Variable& input, const Variable& weight);
+// fl::embedding (Functions.cpp:1707-1749): input = s32 indices of at most 3 dims, embeddings [dim, tokens] ->
+// [dim, input dims...]; the gradient goes to the embeddings only
+Variable embedding(const Variable& input, const Variable& embeddings);
 // fl::gatedlinearunit (Functions.cpp:1567-1610): first half of dimension `dim` times the sigmoid of the second half
 Variable gatedlinearunit(const Variable& input, int dim);
 // fl::dropout (Functions.cpp:1777-1785): input * mask / (1 - p); p <= 0 returns the input.  The mask is a

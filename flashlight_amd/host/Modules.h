@@ -7,6 +7,7 @@
 // operators are not provided.
 #pragma once
 
+#include <cmath>
 #include <map>
 #include <memory>
 #include <string>
@@ -320,6 +321,24 @@ class PReLU : public UnaryModule {         // :114-132: `size` parameters (1, or
   using UnaryModule::forward;
   Variable forward(const Variable& input) override { return prelu(input, params_[0].astype(input.type())); }
   std::string prettyString() const override { return "PReLU"; }
+};
+// fl::Embedding (nn/modules/Embedding.cpp:15-56): a [embeddingDim, numEmbeddings] table drawn uniformly from
+// +-sqrt(1 / embeddingDim); forward = fl::embedding of s32 indices
+class Embedding : public UnaryModule {
+ public:
+  Embedding(int embeddingDim, int numEmbeddings)
+      : UnaryModule({uniform(Shape({embeddingDim, numEmbeddings}), -std::sqrt(1.0 / embeddingDim), std::sqrt(1.0 / embeddingDim),
+                             dtype::f32, true)}),
+        embeddingDim_(embeddingDim), numEmbeddings_(numEmbeddings) {}
+  explicit Embedding(const Variable& w) : UnaryModule({w}), embeddingDim_((int)w.dim(0)), numEmbeddings_((int)w.dim(1)) {}
+  using UnaryModule::forward;
+  Variable forward(const Variable& input) override { return embedding(input, params_[0]); }
+  std::string prettyString() const override {
+    return "Embedding (embeddings: " + std::to_string(numEmbeddings_) + ") (dim: " + std::to_string(embeddingDim_) + ")";
+  }
+
+ private:
+  int embeddingDim_, numEmbeddings_;
 };
 class Sigmoid : public UnaryModule {       // :18-20
  public:

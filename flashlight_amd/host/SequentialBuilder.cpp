@@ -131,6 +131,10 @@ ModulePtr parseLine(const std::string& line) {
     if (op == "HT") return std::make_shared<HardTanh>();
     return std::make_shared<Tanh>();
   }
+  if (op == "E") {                                   // :291-298
+    if (n != 3) failParse(line);
+    return std::make_shared<Embedding>(I(1), I(2));
+  }
   if (op == "PR") {                                  // :411-418
     if (n < 1 || n > 3) failParse(line);
     return std::make_shared<PReLU>(n > 1 ? I(1) : 1, n > 2 ? F(2) : 0.25);
@@ -175,7 +179,7 @@ ModulePtr parseLine(const std::string& line) {
     const float dropout = n > 5 ? std::stof(p[5]) : 0.0f;
     return std::make_shared<RNN>(I(1), I(2), layers, mode, bidirectional, dropout);
   }
-  static const char* const absent[] = {"TR", "CFR", "POSEMB", "SINPOSEMB", "E", "ADAPTIVEE", "SAUG"};
+  static const char* const absent[] = {"TR", "CFR", "POSEMB", "SINPOSEMB", "ADAPTIVEE", "SAUG"};
   for (const char* a : absent)
     if (op == a)
       throw std::invalid_argument("buildSequentialModule: module '" + op +

@@ -724,6 +724,28 @@ def affine_backward(grad_output, input, weight, view):
     return dx, dw, db
 
 
+def embedding(indices, table):
+    """fl::embedding: `indices` int32 (any shape), `table` [tokens, dim] -> indices.shape + [dim]."""
+    idx, w = _dev(indices, "indices"), _dev(table, "table")
+    if idx.dtype != torch.int32:
+        raise ValueError("embedding: indices must be int32")
+    tokens, dim = w.shape
+    y = torch.empty(tuple(idx.shape) + (dim,), dtype=w.dtype, device=w.device)
+    capi.check(capi.lib().flhip_embedding_fwd(_ptr(idx), _ptr(w), _ptr(y), idx.numel(), dim, tokens, _dtype_tag(w),
+                                              _stream()))
+    return y
+
+
+def embedding_backward(grad_output, indices, tokens):
+    """-> the gradient of the table, [tokens, dim]."""
+    g, idx = _dev(grad_output, "gradOutput"), _dev(indices, "indices")
+    dim = g.shape[-1]
+    dw = torch.empty((tokens, dim), dtype=g.dtype, device=g.device)
+    capi.check(capi.lib().flhip_embedding_bwd(_ptr(idx), _ptr(g), _ptr(dw), idx.numel(), dim, tokens, _dtype_tag(g),
+                                              _stream()))
+    return dw
+
+
 def prelu(input, weight):
     """fl::PReLU: `weight` has one element, or as many as the input's fastest (last torch) dimension."""
     x = _dev(input, "input")

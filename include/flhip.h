@@ -493,6 +493,15 @@ int flhip_affine_bwd(const void* dy, const void* x, const void* w, void* dx, flo
                      int scalar_params, int dtype, void* workspace,
                      size_t workspace_bytes, void* stream);
 
+/* fl::embedding (Functions.cpp:1707-1749): y[:, i] = w[:, idx[i]] for n indices (s32 on the device) into a
+ * dim x tokens table; an index outside [0, tokens) gives a column of zeros.  Backward (there a CSR matrix of ones
+ * times the transposed deltas): dw[:, t] = the sum of dy[:, i] over idx[i] == t, added in the order of i in fp32 and
+ * rounded once, zeros for tokens that do not occur; every column of dw is written. */
+int flhip_embedding_fwd(const int32_t* idx, const void* w, void* y, int64_t n, int32_t dim, int32_t tokens, int dtype,
+                        void* stream);
+int flhip_embedding_bwd(const int32_t* idx, const void* dy, void* dw, int64_t n, int32_t dim, int32_t tokens, int dtype,
+                        void* stream);
+
 /* fl::PReLU (flashlight/fl/nn/modules/Activations.cpp:116-124): y = x where x >= 0, w[m] x elsewhere, the parameter
  * tiled along the tensor's first (fastest) dimension of extent d0 (m = element index % d0, `outer` = the product of
  * the other extents) or a single element (scalar_param != 0).  w has the tensor's dtype.  Backward (the chain of

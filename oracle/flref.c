@@ -481,6 +481,24 @@ void flref_prelu_bwd(int64_t n, int64_t d0, int64_t size, const float* dy, const
   free(acc);
 }
 
+/* fl::embedding (Functions.cpp:1707-1749): y[:, i] = w[:, idx[i]] (column-major: dim rows per token); the gradient,
+ * there a CSR matrix of ones times the transposed deltas, is dw[:, t] = the sum of dy[:, i] over idx[i] == t, in
+ * double.  Indices outside [0, tokens) give a zero column and no gradient. */
+void flref_embedding_fwd(int64_t n, int64_t dim, int64_t tokens, const int32_t* idx, const float* w, float* y) {
+  for (int64_t i = 0; i < n; ++i)
+    for (int64_t d = 0; d < dim; ++d)
+      y[i * dim + d] = (idx[i] >= 0 && idx[i] < tokens) ? w[(int64_t)idx[i] * dim + d] : 0.f;
+}
+void flref_embedding_bwd(int64_t n, int64_t dim, int64_t tokens, const int32_t* idx, const float* dy, float* dw) {
+  double* acc = (double*)calloc((size_t)(dim * tokens), sizeof(double));
+  for (int64_t i = 0; i < n; ++i) {
+    if (idx[i] < 0 || idx[i] >= tokens) continue;
+    for (int64_t d = 0; d < dim; ++d) acc[(int64_t)idx[i] * dim + d] += (double)dy[i * dim + d];
+  }
+  for (int64_t k = 0; k < dim * tokens; ++k) dw[k] = (float)acc[k];
+  free(acc);
+}
+
 /* fl::dropout (Functions.cpp:1777-1785) with the counter-based mask below in the place of fl::rand(...) > p */
 int flref_dropout_keep(uint32_t seed_lo, uint32_t seed_hi, uint32_t layer, uint32_t index, float dropout);
 void flref_dropout(int64_t n, const float* x, double p, uint32_t seed_lo, uint32_t seed_hi, float* y) {

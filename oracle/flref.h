@@ -107,6 +107,8 @@ void flref_act_bwd(int op, int64_t n, const float* dy, const float* x, double a,
 /* gatedlinearunit (:1567-1610): halves are contiguous blocks of m elements per outer index */
 void flref_glu_fwd(int64_t outer, int64_t m, const float* x, float* y);
 void flref_glu_bwd(int64_t outer, int64_t m, const float* dy, const float* x, float* dx);
+void flref_embedding_fwd(int64_t n, int64_t dim, int64_t tokens, const int32_t* idx, const float* w, float* y);
+void flref_embedding_bwd(int64_t n, int64_t dim, int64_t tokens, const int32_t* idx, const float* dy, float* dw);
 void flref_prelu_fwd(int64_t n, int64_t d0, int64_t size, const float* x, const float* w, float* y);
 void flref_prelu_bwd(int64_t n, int64_t d0, int64_t size, const float* dy, const float* x, const float* w, float* dx,
                      float* dw);

@@ -223,6 +223,21 @@ def glu_bwd(dy, x, outer, m):
     return dx
 
 
+def embedding_fwd(idx, w):
+    """idx: int array of n indices; w: [tokens, dim] (numpy order of the column-major dim x tokens) -> [n, dim]."""
+    idx, w = np.ascontiguousarray(idx, dtype=np.int32).ravel(), _f32(w)
+    y = np.empty((idx.size, w.shape[1]), dtype=np.float32)
+    lib().flref_embedding_fwd(_i64(idx.size), _i64(w.shape[1]), _i64(w.shape[0]), idx.ctypes.data_as(C.c_void_p), _p(w), _p(y))
+    return y
+
+
+def embedding_bwd(idx, dy, tokens):
+    idx, dy = np.ascontiguousarray(idx, dtype=np.int32).ravel(), _f32(dy)
+    dw = np.empty((tokens, dy.shape[1]), dtype=np.float32)
+    lib().flref_embedding_bwd(_i64(idx.size), _i64(dy.shape[1]), _i64(tokens), idx.ctypes.data_as(C.c_void_p), _p(dy), _p(dw))
+    return dw
+
+
 def prelu_fwd(x, w, d0):
     """x: any array whose fastest dimension has d0 elements; w: 1-D parameter whose size divides d0."""
     x, w = _f32(x), _f32(w)

@@ -959,7 +959,7 @@ static void testArchBuilder() {
   // malformed lines, lines for modules that do not exist here, a missing file
   for (const char* bad : {"C 3 4 5", "C2 3 4 5 6 1", "L 5", "BN 8", "LN", "LN 3", "M 2 2 2", "R 1", "LSM", "GRU 4",
                           "C 3 x 5 1", "XYZ 1 2", "RO", "DO", "DO 0.2 1", "GLU", "ELU 1", "SH 1 2", "WN 3", "WN 1 C 4 4 3 1", "WN 3 R", "PD 0 1", "PD 0 1 1 1",
-                          "TDS 10 21", "AC 1 2 3", "RES 2 1", "RES 1 0 1", "SKIP 0 2", "PC", "PC f64", "PR 1 2 3", "PR x", "E 4 5"})
+                          "TDS 10 21", "AC 1 2 3", "RES 2 1", "RES 1 0 1", "SKIP 0 2", "PC", "PC f64", "PR 1 2 3", "PR x", "E 4", "E 4 5 6", "POSEMB 4 5"})
     CHECK(throws<std::invalid_argument>([&] { one(bad); }));
   CHECK(throws<std::runtime_error>([] { buildSequentialModule(std::string("/nonexistent/arch.txt"), 1, 1); }));
   // from a file
@@ -1078,6 +1078,33 @@ static void testActivationModules() {
     }
   }
   CHECK(throws<std::invalid_argument>([&] { PReLU(4).forward(Variable(Tensor::fromVector({9, 2}, randn(18, 1)), false)); }));
+  // Embedding (line E dim tokens): a gather of the table's columns; the gradient adds the deltas of equal indices
+  {
+    setSeed(33);
+    auto emb = one("E 6 5");
+    CHECK(emb->prettyString() == Embedding(6, 5).prettyString() && emb->params().size() == 1);
+    CHECK(emb->param(0).dim(0) == 6 && emb->param(0).dim(1) == 5);
+    const auto table = hostOf(emb->param(0));
+    for (float v : table) CHECK(std::fabs(v) <= std::sqrt(1.0 / 6.0) + 1e-6);
+    const std::vector<int32_t> ids{3, 0, 3, 4, 0, 3, 1};
+    Variable in(Tensor::fromHost(Shape({7}), dtype::s32, ids.data()), false);
+    emb->zeroGrad();
+    auto out = std::static_pointer_cast<UnaryModule>(emb)->forward(in);
+    CHECK(out.ndim() == 2 && out.dim(0) == 6 && out.dim(1) == 7);
+    const auto y = hostOf(out);
+    bool same = true;
+    for (int i = 0; i < 7; ++i)
+      for (int d = 0; d < 6; ++d) same = same && y[i * 6 + d] == table[ids[i] * 6 + d];
+    CHECK(same);
+    const auto g = randn(42, 17);
+    out.backward(Variable(Tensor::fromVector({6, 7}, g), false));
+    std::vector<float> want(30, 0.f);
+    for (int i = 0; i < 7; ++i)
+      for (int d = 0; d < 6; ++d) want[ids[i] * 6 + d] += g[i * 6 + d];
+    CHECK(relL2(hostOf(emb->param(0).grad()), want) <= 1e-6);
+    for (int d = 0; d < 6; ++d) CHECK(hostOf(emb->param(0).grad())[2 * 6 + d] == 0.f);      // token 2 never occurs
+    CHECK(throws<std::invalid_argument>([&] { embedding(Variable(Tensor::fromVector({7}, randn(7, 1)), false), emb->param(0)); }));
+  }
   CHECK(throws<std::invalid_argument>([&] { gatedlinearunit(Variable(Tensor::fromVector({3, 5}, randn(15, 1)), false), 0); }));
   CHECK(throws<std::invalid_argument>([&] { gatedlinearunit(Variable(Tensor::fromVector({4, 5}, randn(20, 1)), false), 2); }));
 

@@ -313,6 +313,33 @@ def test_affine(outer, mid, inner, scalar, dtype):
 
 
 @pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("idx_shape,dim,tokens", [((1,), 1, 1), ((7,), 5, 3), ((50, 4), 16, 9), ((200, 16), 33, 1000),
+                                                  ((64,), 8, 2), ((300, 40), 512, 10000), ((9,), 2500, 5), ((129,), 300, 1)])
+def test_embedding(idx_shape, dim, tokens, dtype):
+    """fl::embedding forward (bit-exact: a gather) and the table's gradient (sums in the order of the positions, fp32,
+    one rounding), with tokens that repeat, tokens that never occur and two indices outside the table."""
+    rng = np.random.default_rng(dim + tokens + len(idx_shape))
+    idx = rng.integers(0, tokens, size=idx_shape).astype(np.int32)
+    if idx.size > 4:
+        idx.ravel()[1] = tokens
+        idx.ravel()[-2] = -3
+    w = _round(rng.standard_normal((tokens, dim)).astype(np.float32), dtype)
+    dy = _round(rng.standard_normal(idx_shape + (dim,)).astype(np.float32), dtype)
+    idx_d = torch.from_numpy(idx).cuda()
+    y = ops.embedding(idx_d, dev(w, dtype))
+    assert tuple(y.shape) == idx_shape + (dim,)
+    assert np.array_equal(host(y).reshape(-1, dim), flref.embedding_fwd(idx, w))
+    dw = ops.embedding_backward(dev(dy, dtype), idx_d, tokens)
+    want = flref.embedding_bwd(idx, dy.reshape(-1, dim), tokens)
+    if dtype == torch.float32:
+        assert np.allclose(host(dw), want, rtol=1e-5, atol=1e-5 * max(1, idx.size / tokens) ** 0.5)
+    else:
+        assert np.allclose(host(dw), want, rtol=2.0 ** -7, atol=1e-3)
+    dw2 = ops.embedding_backward(dev(dy, dtype), idx_d, tokens)
+    assert torch.equal(dw, dw2)
+
+
+@pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("shape,scalar", [((3, 5, 7), True), ((3, 5, 7), False), ((1, 600), False), ((40, 9, 1), True),
                                           ((64, 3, 56, 56), True), ((8, 250, 1, 300), False), ((300001,), True)])
 def test_prelu(shape, scalar, dtype):

@@ -243,6 +243,34 @@ def test_glu_against_torch_float64(shape, dim):
     assert rel_l2(flref.glu_bwd(dy, x, outer, m).reshape(shape), t.grad.numpy()) <= 1e-6
 
 
+@pytest.mark.parametrize("n,dim,tokens", [(1, 1, 1), (7, 5, 3), (50, 16, 9), (200, 33, 1000), (64, 8, 2)])
+def test_embedding_against_torch_float64(n, dim, tokens):
+    """The checker's embedding against torch.nn.functional.embedding, forward and autograd (float64): a gather of
+    table rows and a scatter-add of the deltas; tokens that occur twice and tokens that never occur both appear.
+    Indices outside the table (which torch refuses) give zero columns and take no gradient."""
+    import torch
+    rng = np.random.default_rng(n + dim + tokens)
+    idx = rng.integers(0, tokens, size=n).astype(np.int32)
+    w = rng.standard_normal((tokens, dim)).astype(np.float32)
+    dy = rng.standard_normal((n, dim)).astype(np.float32)
+    wt = torch.tensor(w, dtype=torch.float64, requires_grad=True)
+    yt = torch.nn.functional.embedding(torch.tensor(idx, dtype=torch.int64), wt)
+    yt.backward(torch.tensor(dy, dtype=torch.float64))
+    assert np.array_equal(flref.embedding_fwd(idx, w), yt.detach().numpy().astype(np.float32))
+    assert np.allclose(flref.embedding_bwd(idx, dy, tokens), wt.grad.numpy(), rtol=1e-6, atol=1e-6)
+    # out of range: zeros forward, nothing backward
+    bad = idx.copy()
+    bad[0] = tokens
+    if n > 1:
+        bad[-1] = -1
+    y = flref.embedding_fwd(bad, w)
+    assert not y[0].any() and (n == 1 or not y[-1].any())
+    keep = (bad >= 0) & (bad < tokens)
+    want = np.zeros((tokens, dim))
+    np.add.at(want, bad[keep], dy[keep].astype(np.float64))
+    assert np.allclose(flref.embedding_bwd(bad, dy, tokens), want, rtol=1e-6, atol=1e-6)
+
+
 @pytest.mark.parametrize("shape,size", [((4, 3, 10), 1), ((4, 3, 10), 10), ((5, 12), 12), ((2, 3, 4, 6), 1), ((7, 8), 4)])
 def test_prelu_against_torch_float64(shape, size):
     # nn/modules/Activations.cpp:116-124: the parameter tiled along Flashlight's first dimension = the last one of
